@@ -1,0 +1,59 @@
+// Shared host/device helpers of the aqtx kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "../../include/aqtx.h"
+
+namespace aqtx {
+
+// ---- error reporting -------------------------------------------------------
+int set_error(const char* fmt, ...);
+void clear_error();
+
+#define AQTX_REQUIRE(cond, ...)                 \
+  do {                                          \
+    if (!(cond)) return ::aqtx::set_error(__VA_ARGS__); \
+  } while (0)
+
+#define AQTX_HIP_CHECK_LAUNCH(name)                                            \
+  do {                                                                         \
+    hipError_t e__ = hipGetLastError();                                        \
+    if (e__ != hipSuccess)                                                     \
+      return ::aqtx::set_error("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+  } while (0)
+
+inline bool is_float_dtype(int d) { return d == AQTX_F32 || d == AQTX_BF16; }
+inline size_t dtype_size(int d) {
+  switch (d) {
+    case AQTX_F32: case AQTX_I32: return 4;
+    case AQTX_BF16: return 2;
+    default: return 1;
+  }
+}
+
+// ---- device numerics -------------------------------------------------------
+#if defined(__HIPCC__)
+
+// float -> nearest bf16 (ties to even), returned as float.
+__device__ __forceinline__ float round_bf16(float x) {
+  return (float)(__bf16)x;
+}
+__device__ __forceinline__ uint16_t bf16_bits(float x) {
+  __bf16 h = (__bf16)x;
+  return __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+// Round to the dtype tag (AQTX_BF16 rounds, AQTX_F32 is the identity).
+template <bool kBf16>
+__device__ __forceinline__ float round_to(float x) {
+  if constexpr (kBf16) return round_bf16(x);
+  return x;
+}
+
+#endif  // __HIPCC__
+
+}  // namespace aqtx

@@ -1,0 +1,697 @@
+// Abs-max calibration + quantization kernels (gfx950).
+//
+// One operand of the quantized dot_general goes through
+//   scale = absmax / quant_bound            (calibration.py:117-157)
+//   t     = x * (1 / scale)                 (aqt_tensor.py:125-159)
+//   t     = t + noise; clip; round; cast    (int_numerics.py:81-111,
+//                                            fp8_numerics.py:36-123)
+// with every intermediate rounded to the dtype the reference holds it in.  Two
+// launch shapes cover the layouts:
+//   * "rows": the reduced axis is the contiguous one.  A segment (one row, or one
+//     subchannel group of a row) is loaded once into registers by 16, 64 or 256
+//     lanes, reduced with wavefront shuffles (+LDS across the four waves),
+//     quantized from registers and stored: one HBM read, one write.
+//   * "tile": the reduced axis is the strided one (or the whole tensor).  A
+//     column abs-max pass (atomic max on the float bit pattern) is followed by a
+//     128x64 tile pass that quantizes and, on request, writes the transposed
+//     layout through LDS so that the consumer GEMM finds its contraction axis
+//     contiguous.
+#include "common.h"
+#include "threefry.h"
+
+namespace aqtx {
+namespace {
+
+struct QArgs {
+  const void* x;
+  const float* prescale;
+  void* q;
+  float* scale;
+  uint32_t* ws_absmax;
+  float* ws_inv;
+  int64_t batch, rows, cols;
+  int64_t L;        // rows kernel: segment length
+  int64_t nseg;     // rows kernel: number of segments
+  int64_t G;        // tile kernels: group length along rows
+  int64_t ngroups;  // tile kernels: rows / G
+  int64_t ssb, ssg, ssc;  // tile kernels: scale index strides
+  int64_t nsb, nsr, nsc;  // noise counter strides
+  float quant_bound, clip_bound;
+  BitGen gen;
+  int noise;
+  int ps_mode;
+  int transpose_out;
+  int out_dtype;
+  int cbf;  // compute dtype is bf16
+  int sbf;  // scale dtype is bf16
+  int scale_given;
+};
+
+// ---- typed vector loads ------------------------------------------------------
+template <typename T> struct Loader;
+template <> struct Loader<float> {
+  static __device__ __forceinline__ void load8(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ float load1(const float* p) { return *p; }
+};
+template <> struct Loader<uint16_t> {  // bf16 bit patterns
+  static __device__ __forceinline__ void load8(const uint16_t* p, float* v) {
+    const uint4 a = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xFFFF0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xFFFF0000u);
+    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xFFFF0000u);
+    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xFFFF0000u);
+  }
+  static __device__ __forceinline__ float load1(const uint16_t* p) {
+    return __uint_as_float(((uint32_t)*p) << 16);
+  }
+};
+template <> struct Loader<int8_t> {
+  static __device__ __forceinline__ void load8(const int8_t* p, float* v) {
+    const uint2 a = *reinterpret_cast<const uint2*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = (float)(int8_t)((a.x >> (8 * i)) & 0xFF);
+      v[4 + i] = (float)(int8_t)((a.y >> (8 * i)) & 0xFF);
+    }
+  }
+  static __device__ __forceinline__ float load1(const int8_t* p) { return (float)*p; }
+};
+
+__device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
+
+// scale and reciprocal scale from the abs-max (calibration.py:145-157,
+// aqt_tensor.py:151-155).
+__device__ __forceinline__ void scale_from_absmax(float amax, const QArgs& a, float& scale,
+                                                  float& inv) {
+  if (amax == 0.0f) amax = 1.0f;
+  float s = rnd(amax / a.quant_bound, a.cbf);
+  s = rnd(s, a.sbf);
+  float i = rnd(1.0f / s, a.sbf);
+  if (isinf(i)) i = 1.0f;
+  scale = s;
+  inv = i;
+}
+
+__device__ __forceinline__ float inv_of_scale(float scale, const QArgs& a) {
+  float i = rnd(1.0f / scale, a.sbf);
+  if (isinf(i)) i = 1.0f;
+  return i;
+}
+
+__device__ __forceinline__ float apply_prescale(float v, float ps, const QArgs& a) {
+  // aqt_dot_general.py:714-720: lhs * scale_t.astype(lhs.dtype)
+  return rnd(v * rnd(ps, a.cbf), a.cbf);
+}
+
+// The value after scaling, noise and clipping, still a float.
+__device__ __forceinline__ float scaled_noisy_clipped(float v, float inv, uint64_t ctr,
+                                                      const QArgs& a) {
+  const int tbf = a.cbf & a.sbf;  // promote(x.dtype, scale.dtype)
+  float t = rnd(v * inv, tbf);
+  if (a.noise == AQTX_NOISE_JAX_UNIFORM) {
+    const uint32_t bits = a.gen.draw(ctr);
+    float u = __uint_as_float((bits >> 9) | 0x3F800000u) - 1.0f;
+    u = fmaxf(0.0f, u);
+    t = rnd(t + (u - 0.5f), tbf);
+  } else if (a.noise == AQTX_NOISE_CUSTOM1) {
+    const uint32_t bits = a.gen.draw(ctr);
+    const float f = __uint_as_float((bits << 7) | 0x3F800000u);
+    t = rnd(t + (f - 1.49999237060546875f), tbf);  // 1.5 - 2^-17
+  } else if (a.noise == AQTX_NOISE_FP8_MANTISSA) {
+    const int mant = (a.out_dtype == AQTX_E4M3) ? 3 : 2;
+    const uint32_t bits = a.gen.draw(ctr);
+    if (tbf) {
+      const uint32_t mask = (1u << (7 - mant)) - 1u;
+      uint32_t u = __float_as_uint(t) >> 16;
+      u = ((u + (bits & mask)) & ~mask) & 0xFFFFu;
+      t = __uint_as_float(u << 16);
+    } else {
+      const uint32_t mask = (1u << (23 - mant)) - 1u;
+      uint32_t u = __float_as_uint(t);
+      u = (u + (bits & mask)) & ~mask;
+      t = __uint_as_float(u);
+    }
+  }
+  t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
+  return t;
+}
+
+// float (already clipped) -> output byte
+__device__ __forceinline__ uint32_t to_qbyte(float t, int out_dtype) {
+  if (out_dtype == AQTX_E4M3) {
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(t, t, 0, false) & 0xFFu;
+  } else if (out_dtype == AQTX_E5M2) {
+    return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(t, t, 0, false) & 0xFFu;
+  }
+  return (uint32_t)((int)rintf(t)) & 0xFFu;
+}
+
+template <int LANES>
+__device__ __forceinline__ float segment_max(float v, float* smem) {
+  constexpr int W = LANES < 64 ? LANES : 64;
+#pragma unroll
+  for (int off = W / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, W));
+  if constexpr (LANES == 256) {
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) smem[wave] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3]));
+  }
+  return v;
+}
+
+// ---- rows kernel: reduced axis contiguous -------------------------------------
+template <typename TIn, int LANES, int ITERS>
+__global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
+  constexpr int VEC = 8;
+  constexpr int SEG_PER_BLOCK = 256 / LANES;
+  __shared__ float smem[4];
+  const int tid = threadIdx.x;
+  const int lane = tid % LANES;
+  const int64_t seg = (int64_t)blockIdx.x * SEG_PER_BLOCK + tid / LANES;
+  const bool active = seg < a.nseg;
+  const int64_t segs_per_row = a.cols / a.L;
+  const int64_t grow = active ? seg / segs_per_row : 0;  // b * rows + r
+  const int64_t col0 = active ? (seg % segs_per_row) * a.L : 0;
+  const int64_t b = grow / a.rows, r = grow % a.rows;
+  const TIn* xp = reinterpret_cast<const TIn*>(a.x) + grow * a.cols + col0;
+
+  float row_ps = 1.0f;
+  if (a.ps_mode == AQTX_PRESCALE_PER_ROW) row_ps = a.prescale[r];
+
+  float v[ITERS][VEC];
+  float amax = 0.0f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
+    if (active && j0 < a.L) {
+      Loader<TIn>::load8(xp + j0, v[it]);
+      if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[it][e] = apply_prescale(v[it][e], row_ps, a);
+      } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+        const float4 p0 = *reinterpret_cast<const float4*>(a.prescale + col0 + j0);
+        const float4 p1 = *reinterpret_cast<const float4*>(a.prescale + col0 + j0 + 4);
+        const float ps[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[it][e] = apply_prescale(v[it][e], ps[e], a);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) amax = fmaxf(amax, fabsf(v[it][e]));
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[it][e] = 0.0f;
+    }
+  }
+  amax = segment_max<LANES>(amax, smem);
+
+  float scale, inv;
+  if (a.scale_given) {
+    scale = active ? a.scale[seg] : 1.0f;
+    inv = inv_of_scale(scale, a);
+  } else {
+    scale_from_absmax(amax, a, scale, inv);
+    if (active && lane == 0) a.scale[seg] = scale;
+  }
+
+  uint8_t* qp = reinterpret_cast<uint8_t*>(a.q) + grow * a.cols + col0;
+  const uint64_t ctr_row = (uint64_t)(b * a.nsb + r * a.nsr + col0 * a.nsc);
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
+    if (active && j0 < a.L) {
+      uint32_t w[2] = {0u, 0u};
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float t =
+            scaled_noisy_clipped(v[it][e], inv, ctr_row + (uint64_t)((j0 + e) * a.nsc), a);
+        w[e >> 2] |= to_qbyte(t, a.out_dtype) << (8 * (e & 3));
+      }
+      *reinterpret_cast<uint2*>(qp + j0) = make_uint2(w[0], w[1]);
+    }
+  }
+}
+
+// Generic rows kernel: any segment length / alignment; one wave per segment, two reads.
+template <typename TIn>
+__global__ __launch_bounds__(256) void quant_rows_generic_kernel(const QArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t seg = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (seg >= a.nseg) return;  // the whole wave leaves together; no barrier below
+  const int64_t segs_per_row = a.cols / a.L;
+  const int64_t grow = seg / segs_per_row;
+  const int64_t col0 = (seg % segs_per_row) * a.L;
+  const int64_t b = grow / a.rows, r = grow % a.rows;
+  const TIn* xp = reinterpret_cast<const TIn*>(a.x) + grow * a.cols + col0;
+  auto value = [&](int64_t j) {
+    float v = Loader<TIn>::load1(xp + j);
+    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[r], a);
+    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[col0 + j], a);
+    return v;
+  };
+  float amax = 0.0f;
+  for (int64_t j = lane; j < a.L; j += 64) amax = fmaxf(amax, fabsf(value(j)));
+  amax = segment_max<64>(amax, nullptr);
+  float scale, inv;
+  if (a.scale_given) {
+    scale = a.scale[seg];
+    inv = inv_of_scale(scale, a);
+  } else {
+    scale_from_absmax(amax, a, scale, inv);
+    if (lane == 0) a.scale[seg] = scale;
+  }
+  uint8_t* qp = reinterpret_cast<uint8_t*>(a.q) + grow * a.cols + col0;
+  const uint64_t ctr_row = (uint64_t)(b * a.nsb + r * a.nsr + col0 * a.nsc);
+  for (int64_t j = lane; j < a.L; j += 64) {
+    const float t = scaled_noisy_clipped(value(j), inv, ctr_row + (uint64_t)(j * a.nsc), a);
+    qp[j] = (uint8_t)to_qbyte(t, a.out_dtype);
+  }
+}
+
+// ---- tile kernels: reduced axis strided (or the whole tensor) -------------------
+
+__global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+constexpr int kAbsRowChunk = 64;
+
+// Column abs-max: block = 4 waves x (64 lanes x VEC cols); the waves interleave
+// over the rows of one chunk, partial maxima meet in LDS and leave through one
+// atomic max per column (|x| >= 0, so the float bit pattern orders like a uint).
+template <typename TIn, int VEC>
+__global__ __launch_bounds__(256) void absmax_cols_kernel(const QArgs a) {
+  __shared__ float smem[4][64 * VEC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t c0 = ((int64_t)blockIdx.x * 64 + lane) * VEC;
+  const int64_t chunks_per_group = (a.G + kAbsRowChunk - 1) / kAbsRowChunk;
+  const int64_t g = blockIdx.y / chunks_per_group;
+  const int64_t chunk = blockIdx.y % chunks_per_group;
+  const int64_t b = blockIdx.z;
+  const int64_t r_begin = g * a.G + chunk * kAbsRowChunk;
+  int64_t r_end = r_begin + kAbsRowChunk;
+  if (r_end > (g + 1) * a.G) r_end = (g + 1) * a.G;
+  float m[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) m[e] = 0.0f;
+  if (c0 < a.cols) {
+    float ps[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ps[e] = 1.0f;
+    if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) ps[e] = a.prescale[c0 + e];
+    }
+    const TIn* xb = reinterpret_cast<const TIn*>(a.x) + b * a.rows * a.cols + c0;
+    for (int64_t r = r_begin + wave; r < r_end; r += 4) {
+      float v[VEC];
+      if constexpr (VEC == 8) Loader<TIn>::load8(xb + r * a.cols, v);
+      else v[0] = Loader<TIn>::load1(xb + r * a.cols);
+      if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+        const float rp = a.prescale[r];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = apply_prescale(v[e], rp, a);
+      } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = apply_prescale(v[e], ps[e], a);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) m[e] = fmaxf(m[e], fabsf(v[e]));
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) smem[wave][lane * VEC + e] = m[e];
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * VEC; i += 256) {
+    const int64_t c = (int64_t)blockIdx.x * 64 * VEC + i;
+    if (c < a.cols) {
+      const float mm = fmaxf(fmaxf(smem[0][i], smem[1][i]), fmaxf(smem[2][i], smem[3][i]));
+      atomicMax(a.ws_absmax + b * a.ssb + g * a.ssg + c * a.ssc, __float_as_uint(mm));
+    }
+  }
+}
+
+// Whole-tensor abs-max per batch entry.
+template <typename TIn>
+__global__ __launch_bounds__(256) void absmax_all_kernel(const QArgs a) {
+  __shared__ float smem[4];
+  const int64_t b = blockIdx.y;
+  const int64_t n = a.rows * a.cols;
+  const TIn* xb = reinterpret_cast<const TIn*>(a.x) + b * n;
+  float m = 0.0f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    float v = Loader<TIn>::load1(xb + i);
+    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[i / a.cols], a);
+    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[i % a.cols], a);
+    m = fmaxf(m, fabsf(v));
+  }
+  m = segment_max<256>(m, smem);
+  if (threadIdx.x == 0) atomicMax(a.ws_absmax + b, __float_as_uint(m));
+}
+
+// abs-max bit patterns -> scale (output) and reciprocal scale (workspace).
+__global__ void finalize_scales_kernel(const QArgs a, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float scale, inv;
+  if (a.scale_given) {
+    scale = a.scale[i];
+    inv = inv_of_scale(scale, a);
+  } else {
+    scale_from_absmax(__uint_as_float(a.ws_absmax[i]), a, scale, inv);
+    a.scale[i] = scale;
+  }
+  a.ws_inv[i] = inv;
+}
+
+constexpr int kTileR = 128, kTileC = 64, kTilePad = 132;
+
+// 128x64 tile: thread (rg = tid/8, cc = tid%8) owns rows 4*rg..+3, cols 8*cc..+7.
+template <typename TIn>
+__global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a) {
+  __shared__ uint32_t lds[kTileC * kTilePad / 4];
+  const int tid = threadIdx.x;
+  const int cc = tid & 7, rg = tid >> 3;
+  const int64_t b = blockIdx.z;
+  const int64_t r0 = (int64_t)blockIdx.y * kTileR, c0 = (int64_t)blockIdx.x * kTileC;
+  const TIn* xb = reinterpret_cast<const TIn*>(a.x) + b * a.rows * a.cols;
+  uint8_t* qb = reinterpret_cast<uint8_t*>(a.q) + b * a.rows * a.cols;
+  const bool vec_ok = (a.cols % 8) == 0;
+  const int64_t c = c0 + cc * 8;
+
+  uint32_t packed[8];  // packed[e] = bytes of rows 4*rg..4*rg+3 at col c+e
+#pragma unroll
+  for (int e = 0; e < 8; ++e) packed[e] = 0u;
+
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t r = r0 + rg * 4 + j;
+    if (r < a.rows && c < a.cols) {
+      float v[8];
+      const int nvalid = (a.cols - c) >= 8 ? 8 : (int)(a.cols - c);
+      if (vec_ok) {
+        Loader<TIn>::load8(xb + r * a.cols + c, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          v[e] = e < nvalid ? Loader<TIn>::load1(xb + r * a.cols + c + e) : 0.0f;
+      }
+      const int64_t sbase = b * a.ssb + (r / a.G) * a.ssg;
+      const float rp = (a.ps_mode == AQTX_PRESCALE_PER_ROW) ? a.prescale[r] : 1.0f;
+      uint32_t w[2] = {0u, 0u};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (e < nvalid) {
+          float x = v[e];
+          if (a.ps_mode == AQTX_PRESCALE_PER_ROW) x = apply_prescale(x, rp, a);
+          else if (a.ps_mode == AQTX_PRESCALE_PER_COL) x = apply_prescale(x, a.prescale[c + e], a);
+          const float inv = a.ws_inv[sbase + (c + e) * a.ssc];
+          const uint64_t ctr = (uint64_t)(b * a.nsb + r * a.nsr + (c + e) * a.nsc);
+          const uint32_t qv = to_qbyte(scaled_noisy_clipped(x, inv, ctr, a), a.out_dtype);
+          w[e >> 2] |= qv << (8 * (e & 3));
+          packed[e] |= qv << (8 * j);
+        }
+      }
+      if (!a.transpose_out) {
+        if (vec_ok) {
+          *reinterpret_cast<uint2*>(qb + r * a.cols + c) = make_uint2(w[0], w[1]);
+        } else {
+          for (int e = 0; e < nvalid; ++e)
+            qb[r * a.cols + c + e] = (uint8_t)(w[e >> 2] >> (8 * (e & 3)));
+        }
+      }
+    }
+  }
+  if (!a.transpose_out) return;  // uniform across the block
+
+  // Transposed write: LDS holds the tile as [col][row bytes], row stride 132 B.
+#pragma unroll
+  for (int e = 0; e < 8; ++e) lds[((cc * 8 + e) * kTilePad + rg * 4) / 4] = packed[e];
+  __syncthreads();
+  // thread -> (col = tid/8 + 32*h, 16-byte chunk = tid%8) of the [64][128] byte tile
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int col = (tid >> 3) + 32 * h;
+    const int chunk = tid & 7;
+    const int64_t gc = c0 + col, gr = r0 + chunk * 16;
+    if (gc < a.cols && gr < a.rows) {
+      uint32_t w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = lds[(col * kTilePad + chunk * 16) / 4 + i];
+      uint8_t* dst = qb + gc * a.rows + gr;
+      if ((a.rows % 16) == 0) {
+        *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+      } else {
+        const int nv = (a.rows - gr) >= 16 ? 16 : (int)(a.rows - gr);
+        for (int i = 0; i < nv; ++i) dst[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+      }
+    }
+  }
+}
+
+__global__ void random_bits_kernel(BitGen gen, int64_t n, void* out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t v = gen.draw((uint64_t)i);
+  if (gen.width == 16) reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)v;
+  else reinterpret_cast<uint32_t*>(out)[i] = v;
+}
+
+// ---- host side ---------------------------------------------------------------------
+
+int validate(const aqtx_quant_plan* p) {
+  AQTX_REQUIRE(p != nullptr, "aqtx_quantize: plan is NULL");
+  AQTX_REQUIRE(p->in_dtype == AQTX_F32 || p->in_dtype == AQTX_BF16 || p->in_dtype == AQTX_I8,
+               "aqtx_quantize: unsupported in_dtype %d", p->in_dtype);
+  AQTX_REQUIRE(is_float_dtype(p->compute_dtype),
+               "aqtx_quantize: compute_dtype must be f32 or bf16, got %d", p->compute_dtype);
+  AQTX_REQUIRE(p->in_dtype == AQTX_I8 || p->in_dtype == p->compute_dtype,
+               "aqtx_quantize: float input must be held in compute_dtype (in %d, compute %d)",
+               p->in_dtype, p->compute_dtype);
+  AQTX_REQUIRE(is_float_dtype(p->scale_dtype),
+               "aqtx_quantize: scale_dtype must be f32 or bf16, got %d", p->scale_dtype);
+  AQTX_REQUIRE(p->out_dtype == AQTX_I8 || p->out_dtype == AQTX_I4 || p->out_dtype == AQTX_E4M3 ||
+                   p->out_dtype == AQTX_E5M2,
+               "aqtx_quantize: unsupported out_dtype %d", p->out_dtype);
+  AQTX_REQUIRE(p->batch >= 0 && p->rows >= 0 && p->cols >= 0, "aqtx_quantize: negative shape");
+  AQTX_REQUIRE(p->reduce >= AQTX_REDUCE_COLS && p->reduce <= AQTX_REDUCE_ALL,
+               "aqtx_quantize: unknown reduce mode %d", p->reduce);
+  AQTX_REQUIRE(p->group >= 0, "aqtx_quantize: negative group");
+  if (p->group > 0) {
+    AQTX_REQUIRE(p->reduce != AQTX_REDUCE_ALL, "aqtx_quantize: group with REDUCE_ALL");
+    const int64_t axis = p->reduce == AQTX_REDUCE_COLS ? p->cols : p->rows;
+    AQTX_REQUIRE(axis % p->group == 0,
+                 "aqtx_quantize: group %lld does not divide the reduced axis %lld",
+                 (long long)p->group, (long long)axis);
+  }
+  AQTX_REQUIRE(!(p->transpose_out && p->reduce == AQTX_REDUCE_COLS),
+               "aqtx_quantize: transpose_out is not supported with REDUCE_COLS");
+  AQTX_REQUIRE(p->noise >= AQTX_NOISE_NONE && p->noise <= AQTX_NOISE_FP8_MANTISSA,
+               "aqtx_quantize: unknown noise kind %d", p->noise);
+  const bool fp8 = p->out_dtype == AQTX_E4M3 || p->out_dtype == AQTX_E5M2;
+  AQTX_REQUIRE(!(p->noise == AQTX_NOISE_FP8_MANTISSA && !fp8),
+               "aqtx_quantize: mantissa noise needs an fp8 out_dtype");
+  AQTX_REQUIRE(!((p->noise == AQTX_NOISE_JAX_UNIFORM || p->noise == AQTX_NOISE_CUSTOM1) && fp8),
+               "aqtx_quantize: additive noise needs an integer out_dtype");
+  if (p->noise != AQTX_NOISE_NONE) {
+    AQTX_REQUIRE(p->noise_total > 0 && p->noise_total < (int64_t)0xFFFFFFFFll,
+                 "aqtx_quantize: noise_total %lld out of range (1 .. 2^32-2)",
+                 (long long)p->noise_total);
+  }
+  AQTX_REQUIRE(p->prescale >= AQTX_PRESCALE_NONE && p->prescale <= AQTX_PRESCALE_PER_COL,
+               "aqtx_quantize: unknown prescale mode %d", p->prescale);
+  AQTX_REQUIRE(p->quant_bound > 0.0f && p->clip_bound > 0.0f,
+               "aqtx_quantize: bounds must be positive");
+  return 0;
+}
+
+int64_t scale_count(const aqtx_quant_plan* p) {
+  switch (p->reduce) {
+    case AQTX_REDUCE_COLS: return p->batch * p->rows * (p->group ? p->cols / p->group : 1);
+    case AQTX_REDUCE_ROWS: return p->batch * (p->group ? p->rows / p->group : 1) * p->cols;
+    default: return p->batch;
+  }
+}
+
+int noise_width(const aqtx_quant_plan* p) {
+  if (p->noise == AQTX_NOISE_CUSTOM1) return 16;
+  if (p->noise == AQTX_NOISE_FP8_MANTISSA)
+    return (p->compute_dtype == AQTX_BF16 && p->scale_dtype == AQTX_BF16) ? 16 : 32;
+  return 32;
+}
+
+template <typename TIn>
+int launch_rows(const QArgs& a, hipStream_t st) {
+  const int64_t L = a.L;
+  const bool aligned = (L % 8 == 0) && (a.cols % 8 == 0);
+  if (!aligned || L > 16384) {
+    const int64_t blocks = (a.nseg + 3) / 4;
+    quant_rows_generic_kernel<TIn><<<dim3((unsigned)blocks), 256, 0, st>>>(a);
+    AQTX_HIP_CHECK_LAUNCH("quant_rows_generic_kernel");
+    return 0;
+  }
+#define AQTX_ROWS(LANES, ITERS)                                                      \
+  {                                                                                  \
+    const int64_t blocks = (a.nseg + (256 / LANES) - 1) / (256 / LANES);             \
+    quant_rows_kernel<TIn, LANES, ITERS><<<dim3((unsigned)blocks), 256, 0, st>>>(a); \
+    AQTX_HIP_CHECK_LAUNCH("quant_rows_kernel");                                      \
+    return 0;                                                                        \
+  }
+  if (L <= 128) AQTX_ROWS(16, 1)
+  if (L <= 512) AQTX_ROWS(64, 1)
+  if (L <= 2048) AQTX_ROWS(256, 1)
+  if (L <= 4096) AQTX_ROWS(256, 2)
+  if (L <= 8192) AQTX_ROWS(256, 4)
+  AQTX_ROWS(256, 8)
+#undef AQTX_ROWS
+}
+
+template <typename TIn>
+int launch_tiles(const QArgs& a, int reduce, int64_t nscales, hipStream_t st) {
+  if (!a.scale_given) {
+    fill_u32_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a.ws_absmax, nscales, 0u);
+    AQTX_HIP_CHECK_LAUNCH("fill_u32_kernel");
+    if (reduce == AQTX_REDUCE_ALL) {
+      int64_t nblk = (a.rows * a.cols + 256 * 16 - 1) / (256 * 16);
+      if (nblk > 2048) nblk = 2048;
+      if (nblk < 1) nblk = 1;
+      absmax_all_kernel<TIn><<<dim3((unsigned)nblk, (unsigned)a.batch), 256, 0, st>>>(a);
+      AQTX_HIP_CHECK_LAUNCH("absmax_all_kernel");
+    } else {
+      const int64_t chunks = a.ngroups * ((a.G + kAbsRowChunk - 1) / kAbsRowChunk);
+      if (a.cols % 8 == 0) {
+        dim3 grid((unsigned)((a.cols + 511) / 512), (unsigned)chunks, (unsigned)a.batch);
+        absmax_cols_kernel<TIn, 8><<<grid, 256, 0, st>>>(a);
+      } else {
+        dim3 grid((unsigned)((a.cols + 63) / 64), (unsigned)chunks, (unsigned)a.batch);
+        absmax_cols_kernel<TIn, 1><<<grid, 256, 0, st>>>(a);
+      }
+      AQTX_HIP_CHECK_LAUNCH("absmax_cols_kernel");
+    }
+  }
+  finalize_scales_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a, nscales);
+  AQTX_HIP_CHECK_LAUNCH("finalize_scales_kernel");
+  dim3 grid((unsigned)((a.cols + kTileC - 1) / kTileC), (unsigned)((a.rows + kTileR - 1) / kTileR),
+            (unsigned)a.batch);
+  quant_tile_kernel<TIn><<<grid, 256, 0, st>>>(a);
+  AQTX_HIP_CHECK_LAUNCH("quant_tile_kernel");
+  return 0;
+}
+
+template <typename TIn>
+int dispatch(const QArgs& a, int reduce, int64_t nscales, hipStream_t st) {
+  if (reduce == AQTX_REDUCE_COLS) return launch_rows<TIn>(a, st);
+  return launch_tiles<TIn>(a, reduce, nscales, st);
+}
+
+}  // namespace
+}  // namespace aqtx
+
+using namespace aqtx;
+
+extern "C" size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* p) {
+  if (p == nullptr || p->reduce == AQTX_REDUCE_COLS) return 0;
+  if (p->batch < 0 || p->rows < 0 || p->cols < 0 || p->group < 0) return 0;
+  if (p->reduce != AQTX_REDUCE_ROWS && p->reduce != AQTX_REDUCE_ALL) return 0;
+  if (p->group > 0 && (p->reduce == AQTX_REDUCE_ALL || p->rows % p->group != 0)) return 0;
+  return (size_t)scale_count(p) * 8;
+}
+
+extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const float* prescale,
+                             void* q, float* scale, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  clear_error();
+  if (int rc = validate(p)) return rc;
+  const int64_t total = p->batch * p->rows * p->cols;
+  if (total == 0) return 0;
+  AQTX_REQUIRE(x != nullptr && q != nullptr && scale != nullptr, "aqtx_quantize: NULL buffer");
+  AQTX_REQUIRE((p->prescale == AQTX_PRESCALE_NONE) == (prescale == nullptr),
+               "aqtx_quantize: prescale pointer does not match plan->prescale");
+  AQTX_REQUIRE(p->batch <= 65535, "aqtx_quantize: batch %lld exceeds 65535", (long long)p->batch);
+  const size_t need = aqtx_quantize_workspace_bytes(p);
+  AQTX_REQUIRE(workspace_bytes >= need && (need == 0 || workspace != nullptr),
+               "aqtx_quantize: workspace too small (%zu < %zu)", workspace_bytes, need);
+  AQTX_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)q % 16) == 0 &&
+                   ((uintptr_t)scale % 4) == 0 &&
+                   (prescale == nullptr || ((uintptr_t)prescale % 16) == 0) &&
+                   (workspace == nullptr || ((uintptr_t)workspace % 4) == 0),
+               "aqtx_quantize: x, q and prescale must be 16-byte aligned");
+
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int64_t nscales = scale_count(p);
+  QArgs a{};
+  a.x = x; a.prescale = prescale; a.q = q; a.scale = scale;
+  a.batch = p->batch; a.rows = p->rows; a.cols = p->cols;
+  a.nsb = p->noise_stride_batch; a.nsr = p->noise_stride_row; a.nsc = p->noise_stride_col;
+  a.quant_bound = p->quant_bound; a.clip_bound = p->clip_bound;
+  a.noise = p->noise; a.ps_mode = p->prescale;
+  a.transpose_out = p->transpose_out; a.out_dtype = p->out_dtype;
+  a.cbf = p->compute_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
+  a.scale_given = p->scale_given;
+  if (p->noise != AQTX_NOISE_NONE)
+    a.gen = make_bitgen(p->key, p->noise_total, noise_width(p), p->partitionable);
+  if (p->reduce == AQTX_REDUCE_COLS) {
+    a.L = p->group ? p->group : p->cols;
+    a.nseg = nscales;
+  } else {
+    a.ws_absmax = reinterpret_cast<uint32_t*>(workspace);
+    a.ws_inv = reinterpret_cast<float*>(workspace) + nscales;
+    if (p->reduce == AQTX_REDUCE_ROWS) {
+      a.G = p->group ? p->group : p->rows;
+      a.ngroups = p->rows / a.G;
+      a.ssb = a.ngroups * p->cols; a.ssg = p->cols; a.ssc = 1;
+    } else {
+      a.G = p->rows; a.ngroups = 1;
+      a.ssb = 1; a.ssg = 0; a.ssc = 0;
+    }
+    const int64_t grid_y = p->reduce == AQTX_REDUCE_ALL
+                               ? (p->rows + kTileR - 1) / kTileR
+                               : a.ngroups * ((a.G + kAbsRowChunk - 1) / kAbsRowChunk);
+    AQTX_REQUIRE(grid_y <= 65535 && (p->rows + kTileR - 1) / kTileR <= 65535,
+                 "aqtx_quantize: too many rows for one launch (%lld)", (long long)p->rows);
+  }
+  switch (p->in_dtype) {
+    case AQTX_F32: return dispatch<float>(a, p->reduce, nscales, st);
+    case AQTX_BF16: return dispatch<uint16_t>(a, p->reduce, nscales, st);
+    default: return dispatch<int8_t>(a, p->reduce, nscales, st);
+  }
+}
+
+extern "C" int aqtx_random_bits(const uint32_t key_host[2], int64_t n, int32_t bit_width,
+                                int32_t partitionable, void* out, void* stream) {
+  clear_error();
+  AQTX_REQUIRE(key_host != nullptr, "aqtx_random_bits: key is NULL");
+  AQTX_REQUIRE(bit_width == 16 || bit_width == 32, "aqtx_random_bits: bit_width must be 16 or 32");
+  AQTX_REQUIRE(n >= 0 && n < (int64_t)0xFFFFFFFFll, "aqtx_random_bits: n out of range");
+  if (n == 0) return 0;
+  AQTX_REQUIRE(out != nullptr, "aqtx_random_bits: out is NULL");
+  BitGen gen = make_bitgen(key_host, n, bit_width, partitionable);
+  random_bits_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0,
+                       reinterpret_cast<hipStream_t>(stream)>>>(gen, n, out);
+  AQTX_HIP_CHECK_LAUNCH("random_bits_kernel");
+  return 0;
+}
+
+extern "C" int aqtx_prng_split_host(const uint32_t key_host[2], int32_t num, int32_t partitionable,
+                                    uint32_t* out_host) {
+  clear_error();
+  AQTX_REQUIRE(key_host != nullptr && out_host != nullptr, "aqtx_prng_split_host: NULL argument");
+  AQTX_REQUIRE(num >= 0, "aqtx_prng_split_host: negative num");
+  if (partitionable) {
+    for (int32_t i = 0; i < num; ++i) {
+      U2 b = threefry2x32(key_host[0], key_host[1], 0u, (uint32_t)i);
+      out_host[2 * i] = b.x;
+      out_host[2 * i + 1] = b.y;
+    }
+  } else {
+    BitGen g = make_bitgen(key_host, 2 * (int64_t)num, 32, 0);
+    for (int32_t i = 0; i < 2 * num; ++i) out_host[i] = g.word_original((uint32_t)i);
+  }
+  return 0;
+}

@@ -1,0 +1,185 @@
+"""Tensor-level entry points over the aqtx C-ABI.
+
+torch is used for device memory and the current HIP stream only; all arithmetic
+happens in the HIP kernels.  Every function raises if a tensor is not on a GPU
+or the library is missing -- there is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from aqt_amd import _lib as L
+
+_TORCH_TO_AQTX = {
+    torch.float32: L.F32,
+    torch.bfloat16: L.BF16,
+    torch.int8: L.I8,
+    torch.int32: L.I32,
+}
+_AQTX_TO_TORCH = {L.F32: torch.float32, L.BF16: torch.bfloat16, L.I32: torch.int32}
+
+
+def aqtx_dtype(dt) -> int:
+  if isinstance(dt, int):
+    return dt
+  try:
+    return _TORCH_TO_AQTX[dt]
+  except KeyError:
+    raise TypeError(f'unsupported dtype for the aqtx kernels: {dt}') from None
+
+
+def _ptr(t: Optional[torch.Tensor]):
+  return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+  return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require_gpu(*tensors):
+  for t in tensors:
+    if t is not None and not t.is_cuda:
+      raise RuntimeError('aqt_amd kernels need tensors in GPU memory (got a CPU tensor); '
+                         'there is no CPU fallback')
+
+
+def quantize(
+    x: torch.Tensor,
+    *,
+    reduce: int,
+    out_dtype: int,
+    quant_bound: float,
+    clip_bound: float,
+    compute_dtype=None,
+    scale_dtype=None,
+    group: int = 0,
+    transpose_out: bool = False,
+    noise: int = L.NOISE_NONE,
+    key: Optional[Sequence[int]] = None,
+    partitionable: bool = False,
+    noise_strides: Optional[Sequence[int]] = None,
+    noise_total: Optional[int] = None,
+    prescale: Optional[torch.Tensor] = None,
+    prescale_mode: int = L.PRESCALE_NONE,
+    scale: Optional[torch.Tensor] = None,
+):
+  """Calibrate (abs-max) and quantize a contiguous [batch, rows, cols] tensor.
+
+  Returns (q, scale): q is int8 (or uint8 holding fp8 bytes), shaped
+  [batch, rows, cols] or [batch, cols, rows] with transpose_out; scale is
+  float32, shaped [batch, rows, cols/group] (REDUCE_COLS),
+  [batch, rows/group, cols] (REDUCE_ROWS) or [batch] (REDUCE_ALL).
+  """
+  _require_gpu(x, prescale, scale)
+  assert x.dim() == 3 and x.is_contiguous(), 'x must be a contiguous [batch, rows, cols] tensor'
+  b, r, c = x.shape
+  in_dt = aqtx_dtype(x.dtype)
+  compute_dt = aqtx_dtype(compute_dtype) if compute_dtype is not None else in_dt
+  scale_dt = aqtx_dtype(scale_dtype) if scale_dtype is not None else compute_dt
+  plan = L.QuantPlan()
+  plan.in_dtype, plan.compute_dtype, plan.scale_dtype, plan.out_dtype = in_dt, compute_dt, scale_dt, out_dtype
+  plan.batch, plan.rows, plan.cols = b, r, c
+  plan.reduce, plan.transpose_out, plan.group = reduce, int(transpose_out), group
+  plan.quant_bound, plan.clip_bound = quant_bound, clip_bound
+  plan.noise, plan.partitionable = noise, int(partitionable)
+  if noise != L.NOISE_NONE:
+    assert key is not None, 'noise requested but no PRNG key given'
+    plan.key[0], plan.key[1] = int(key[0]), int(key[1])
+    nsb, nsr, nsc = noise_strides if noise_strides is not None else (r * c, c, 1)
+    plan.noise_stride_batch, plan.noise_stride_row, plan.noise_stride_col = nsb, nsr, nsc
+    plan.noise_total = noise_total if noise_total is not None else b * r * c
+  plan.prescale = prescale_mode
+  plan.scale_given = int(scale is not None)
+
+  if reduce == L.REDUCE_COLS:
+    sshape = (b, r, c // group if group else 1)
+  elif reduce == L.REDUCE_ROWS:
+    sshape = (b, r // group if group else 1, c)
+  else:
+    sshape = (b,)
+  if scale is None:
+    scale = torch.empty(sshape, dtype=torch.float32, device=x.device)
+  else:
+    assert scale.dtype == torch.float32 and scale.is_contiguous() and tuple(scale.shape) == sshape
+  fp8 = out_dtype in (L.E4M3, L.E5M2)
+  qshape = (b, c, r) if transpose_out else (b, r, c)
+  q = torch.empty(qshape, dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
+  if prescale is not None:
+    assert prescale.dtype == torch.float32 and prescale.is_contiguous()
+  lib = L.lib()
+  ws_bytes = lib.aqtx_quantize_workspace_bytes(ctypes.byref(plan))
+  ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=x.device) if ws_bytes else None
+  L.check(lib.aqtx_quantize(ctypes.byref(plan), _ptr(x), _ptr(prescale), _ptr(q), _ptr(scale),
+                            _ptr(ws), ws_bytes, _stream()))
+  return q, scale
+
+
+def gemm(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    *,
+    row_scale: Optional[torch.Tensor],
+    col_scale: Optional[torch.Tensor],
+    out_dtype,
+    dequant_dtype=None,
+    scale_dtype=None,
+    scale_order: int = L.SCALE_ROW_THEN_COL,
+    a_dtype: int = L.I8,
+    b_dtype: int = L.I8,
+    want_acc: bool = False,
+):
+  """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
+
+  int8 operands use the int32 MFMA path, fp8 operands (uint8 tensors holding
+  e4m3fn/e5m2 bytes) the float32 one.  Returns C, or (C, acc) with want_acc.
+  """
+  _require_gpu(a, b, row_scale, col_scale)
+  assert a.dim() == 3 and b.dim() == 3 and a.shape[0] == b.shape[0] and a.shape[2] == b.shape[2]
+  assert a.stride(2) == 1 and b.stride(2) == 1, 'the contraction axis must be contiguous'
+  batch, m, k = a.shape
+  n = b.shape[1]
+  fp8 = a_dtype in (L.E4M3, L.E5M2)
+  out_dt = aqtx_dtype(out_dtype)
+  dq_dt = aqtx_dtype(dequant_dtype) if dequant_dtype is not None else (out_dt if out_dt != L.I32 else L.F32)
+  sc_dt = aqtx_dtype(scale_dtype) if scale_dtype is not None else dq_dt
+  c = torch.empty((batch, m, n), dtype=_AQTX_TO_TORCH[out_dt], device=a.device)
+  acc = None
+  if want_acc:
+    acc = torch.empty((batch, m, n), dtype=torch.float32 if fp8 else torch.int32, device=a.device)
+  plan = L.GemmPlan()
+  plan.batch, plan.m, plan.n, plan.k = batch, m, n, k
+  plan.lda, plan.ldb, plan.ldc = a.stride(1), b.stride(1), n
+  plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), b.stride(0), m * n
+  plan.a_dtype, plan.b_dtype = a_dtype, b_dtype
+  plan.out_dtype, plan.dequant_dtype, plan.scale_dtype = out_dt, dq_dt, sc_dt
+  plan.scale_order = scale_order
+  for s, dim in ((row_scale, m), (col_scale, n)):
+    if s is not None:
+      assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == (batch, dim), (
+          tuple(s.shape), (batch, dim))
+  plan.row_scale_stride_b, plan.col_scale_stride_b = m, n
+  fn = L.lib().aqtx_gemm_fp8 if fp8 else L.lib().aqtx_gemm_i8
+  L.check(fn(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale), _ptr(col_scale), _ptr(c),
+             _ptr(acc), _stream()))
+  return (c, acc) if want_acc else c
+
+
+def prng_split(key, num: int, partitionable: bool = False) -> np.ndarray:
+  """jax.random.split(key, num) on raw uint32[2] key data (host side)."""
+  k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))
+  out = (ctypes.c_uint32 * (2 * num))()
+  L.check(L.lib().aqtx_prng_split_host(k, num, int(partitionable), out))
+  return np.frombuffer(out, dtype=np.uint32).reshape(num, 2).copy()
+
+
+def random_bits(key, n: int, bit_width: int = 32, partitionable: bool = False, device='cuda'):
+  """jax.random.bits(key, (n,), uint{bit_width}) generated on the GPU."""
+  k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))
+  out = torch.empty(n, dtype=torch.int16 if bit_width == 16 else torch.int32, device=device)
+  _require_gpu(out)
+  L.check(L.lib().aqtx_random_bits(k, n, bit_width, int(partitionable), _ptr(out), _stream()))
+  return out

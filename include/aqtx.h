@@ -1,0 +1,211 @@
+/*
+ * aqtx -- C-ABI of the MI355X (gfx950) kernels behind the aqt.jax.v2 quantized
+ * dot_general path.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless
+ *     its name ends in `_host`;
+ *   - the caller owns every buffer (inputs, outputs, workspace); the library
+ *     allocates nothing, frees nothing and never synchronises;
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it;
+ *   - the return value is 0 on success, non-zero otherwise; the message for
+ *     the calling thread's last failure is aqtx_last_error();
+ *   - argument validation happens before any GPU call, so every error path can
+ *     be exercised on a machine without a GPU;
+ *   - scales travel as float32 arrays whose values are already rounded to the
+ *     scale dtype the plan names (a bf16 scale is a bf16-representable float).
+ *
+ * The reference (google/aqt) is pure Python on JAX and has no FFI of its own;
+ * each entry point below names the reference functions whose XLA-emitted
+ * arithmetic it replaces.
+ */
+#ifndef AQTX_H_
+#define AQTX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AQTX_VERSION 1
+
+/* element types */
+enum {
+  AQTX_F32 = 0,
+  AQTX_BF16 = 1,
+  AQTX_I8 = 2,   /* int8 */
+  AQTX_I4 = 3,   /* int4 values in an int8 container (one value per byte) */
+  AQTX_E4M3 = 4, /* float8_e4m3fn (OCP) */
+  AQTX_E5M2 = 5, /* float8_e5m2 (OCP) */
+  AQTX_I32 = 6,
+  AQTX_I4P = 7   /* int4 packed two per byte, low nibble = even index */
+};
+
+/* which axis of the [batch, rows, cols] view shares one scale */
+enum {
+  AQTX_REDUCE_COLS = 0, /* one scale per (batch,row[,group])  -> scale[batch][rows][cols/group] */
+  AQTX_REDUCE_ROWS = 1, /* one scale per (batch[,group],col)  -> scale[batch][rows/group][cols] */
+  AQTX_REDUCE_ALL = 2   /* one scale per batch entry          -> scale[batch]                   */
+};
+
+/* noise added before rounding */
+enum {
+  AQTX_NOISE_NONE = 0,
+  AQTX_NOISE_JAX_UNIFORM = 1,     /* stochastic_rounding.py:36-46  */
+  AQTX_NOISE_CUSTOM1 = 2,         /* stochastic_rounding.py:50-78  */
+  AQTX_NOISE_FP8_MANTISSA = 3     /* numerics/fp8_numerics.py:36-64 */
+};
+
+enum { AQTX_PRESCALE_NONE = 0, AQTX_PRESCALE_PER_ROW = 1, AQTX_PRESCALE_PER_COL = 2 };
+
+/*
+ * Plan of one calibrate+quantize pass over a contiguous tensor viewed as
+ * [batch, rows, cols] (row-major).
+ */
+typedef struct aqtx_quant_plan {
+  int32_t in_dtype;      /* AQTX_F32 | AQTX_BF16 | AQTX_I8 (int8 values read as floats) */
+  int32_t compute_dtype; /* AQTX_F32 | AQTX_BF16: the dtype the reference holds x in   */
+  int32_t scale_dtype;   /* AQTX_F32 | AQTX_BF16: Calibration.dtype or compute_dtype    */
+  int32_t out_dtype;     /* AQTX_I8 | AQTX_I4 | AQTX_E4M3 | AQTX_E5M2                  */
+  int64_t batch, rows, cols;
+  int32_t reduce;        /* AQTX_REDUCE_*                                               */
+  int32_t transpose_out; /* 1: write q as [batch, cols, rows]                           */
+  int64_t group;         /* subchannel size along the reduced axis; 0 = whole axis      */
+  float quant_bound;     /* AqtNumerics.get_quant_bound(): 127.5, 7.5, 448, 57344       */
+  float clip_bound;      /* forward clip bound: 127, 7, 448, 57344                      */
+  int32_t noise;         /* AQTX_NOISE_*                                                */
+  int32_t partitionable; /* jax_threefry_partitionable                                  */
+  uint32_t key[2];       /* raw threefry key data                                       */
+  /* counter of element (b,r,c) in the noise tensor = b*nb + r*nr + c*nc;
+     noise_total = number of elements of the noise tensor */
+  int64_t noise_stride_batch, noise_stride_row, noise_stride_col, noise_total;
+  int32_t prescale;      /* AQTX_PRESCALE_*: x := round(x * cast(v)) first              */
+  int32_t scale_given;   /* 1: `scale` is an input (calibration skipped)                */
+} aqtx_quant_plan;
+
+/*
+ * aqtx_quantize: abs-max calibration + quantization, one launch sequence.
+ * Replaces, for one operand: AbsMaxCalibration.get_scale_and_bias_and_sparsity
+ * (aqt/jax/v2/calibration.py:117-157), QTensor.quant (aqt_tensor.py:125-159),
+ * IntSymmetric.vjp_fwd (numerics/int_numerics.py:81-111), Fp8Numerics.vjp_fwd
+ * (numerics/fp8_numerics.py:88-123), the noise functions
+ * (stochastic_rounding.py:36-78) and the gradient pre-scaling of
+ * _maybe_use_fwd_quant (aqt_dot_general.py:714-720).
+ *   x         in  : [batch, rows, cols] of in_dtype
+ *   prescale  in  : float32 [rows] or [cols] (NULL when plan->prescale == NONE)
+ *   q         out : int8 / fp8 bytes, [batch, rows, cols] or transposed
+ *   scale     out : float32, layout per plan->reduce (input when scale_given)
+ *   workspace     : aqtx_quantize_workspace_bytes(plan) bytes of scratch
+ */
+int aqtx_quantize(const aqtx_quant_plan* plan, const void* x, const float* prescale,
+                  void* q, float* scale, void* workspace, size_t workspace_bytes,
+                  void* stream);
+
+/* Scratch bytes aqtx_quantize needs for `plan` (0 for single-pass plans). */
+size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* plan);
+
+enum { AQTX_SCALE_ROW_THEN_COL = 0, AQTX_SCALE_COL_THEN_ROW = 1 };
+
+/*
+ * Plan of C[b] = dequant(A[b] * B[b]^T): A is [batch, m, k], B is [batch, n, k]
+ * (both with the contraction axis contiguous), C is [batch, m, n].
+ */
+typedef struct aqtx_gemm_plan {
+  int64_t batch, m, n, k;
+  int64_t lda, ldb, ldc;      /* row strides in elements                                    */
+  int64_t stride_a, stride_b, stride_c; /* batch strides in elements                      */
+  int32_t a_dtype, b_dtype;   /* AQTX_I8 | AQTX_I4 (container) | AQTX_E4M3 | AQTX_E5M2       */
+  int32_t out_dtype;          /* AQTX_BF16 | AQTX_F32 | AQTX_I32 (raw accumulator, no scales) */
+  int32_t dequant_dtype;      /* AQTX_BF16 | AQTX_F32: dtype the accumulator is cast to first */
+  int32_t scale_dtype;        /* AQTX_BF16 | AQTX_F32: dtype of the scale arrays             */
+  int32_t scale_order;        /* AQTX_SCALE_*: which scale multiplies first                  */
+  int64_t row_scale_stride_b, col_scale_stride_b; /* batch strides of the scale vectors    */
+} aqtx_gemm_plan;
+
+/*
+ * aqtx_gemm_i8: int8 x int8 -> int32 MFMA contraction with the dequantisation
+ * fused in the epilogue.  Replaces _qtensor_dot_general
+ * (aqt/jax/v2/aqt_dot_general.py:843-958, the lax.dot_general call at :921-927
+ * with preferred_element_type=int32) followed by QTensor.dequant
+ * (aqt_tensor.py:161-200): out = cast(acc) * first_scale * second_scale, each
+ * product rounded to promote(dequant_dtype, scale_dtype), final cast to
+ * out_dtype.
+ *   row_scale : float32 [batch][m] or NULL (= no scale on that side)
+ *   col_scale : float32 [batch][n] or NULL
+ *   acc_out   : optional int32 [batch][m][n] copy of the raw accumulators
+ */
+int aqtx_gemm_i8(const aqtx_gemm_plan* plan, const void* a, const void* b,
+                 const float* row_scale, const float* col_scale, void* c,
+                 int32_t* acc_out, void* stream);
+
+/*
+ * aqtx_gemm_fp8: fp8 x fp8 -> float32 MFMA contraction (a_dtype/b_dtype select
+ * e4m3fn or e5m2 per operand), same epilogue as aqtx_gemm_i8.  Replaces the
+ * same reference lines with preferred_element_type=float32
+ * (aqt_dot_general.py:119-121).
+ */
+int aqtx_gemm_fp8(const aqtx_gemm_plan* plan, const void* a, const void* b,
+                  const float* row_scale, const float* col_scale, void* c,
+                  float* acc_out, void* stream);
+
+/*
+ * Plan of the serving contraction out[m, n] = dequant(quant(x)[m, k] * W[n, k]^T)
+ * with a pre-quantized weight (QTensor: int8 qvalue + per-output-channel scale)
+ * and per-token dynamic int8 quantisation of the activations, m <= 64.
+ */
+typedef struct aqtx_decode_plan {
+  int64_t m, n, k;
+  int32_t x_dtype;        /* AQTX_BF16 | AQTX_F32                       */
+  int32_t x_scale_dtype;  /* dtype the activation scale is rounded to   */
+  int32_t w_scale_dtype;  /* dtype of the weight scale (values in f32)  */
+  int32_t out_dtype;      /* AQTX_BF16 | AQTX_F32                       */
+  float quant_bound, clip_bound; /* of the activation numerics        */
+} aqtx_decode_plan;
+
+/*
+ * aqtx_decode_i8: fused activation quantisation + skinny int8 contraction +
+ * dequantisation for serving (pre-quantized rhs).  Replaces
+ * DotGeneralRaw.__call__ (aqt/jax/v2/aqt_dot_general.py:757-840) called with a
+ * full rhs_qt, i.e. quant() of the lhs only (:598-672), the int32 dot and
+ * QTensor.dequant; the standalone reference equivalents are
+ * pallas/quantizer.py:33-68 and pallas/dot_general.py:57-137.
+ *   x        in  : [m, k] activations
+ *   w        in  : int8 [n, k] (weight stored with the contraction axis contiguous)
+ *   w_scale  in  : float32 [n]
+ *   xq       out : optional int8 [m, k] (the quantized activations), may be NULL
+ *   x_scale  out : float32 [m]
+ *   out      out : [m, n]
+ *   workspace    : aqtx_decode_workspace_bytes(plan) bytes
+ */
+int aqtx_decode_i8(const aqtx_decode_plan* plan, const void* x, const void* w,
+                   const float* w_scale, void* xq, float* x_scale, void* out,
+                   void* workspace, size_t workspace_bytes, void* stream);
+size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* plan);
+
+/*
+ * aqtx_prng_split_host: jax.random.split(key, num) on the host (used by
+ * config.set_context, aqt/jax/v2/config.py:61-90).  out_host: uint32[num][2].
+ */
+int aqtx_prng_split_host(const uint32_t key_host[2], int32_t num, int32_t partitionable,
+                         uint32_t* out_host);
+
+/*
+ * aqtx_random_bits: jax.random.bits(key, [n], uint{bit_width}) on the device,
+ * bit_width in {16, 32}; out is uint16[n] or uint32[n].  Exposes the in-kernel
+ * generator of aqtx_quantize for tests (stochastic_rounding.py:46,65).
+ */
+int aqtx_random_bits(const uint32_t key_host[2], int64_t n, int32_t bit_width,
+                     int32_t partitionable, void* out, void* stream);
+
+/* Message of the calling thread's most recent failure ("" if none). */
+const char* aqtx_last_error(void);
+
+/* AQTX_VERSION the library was built from. */
+int aqtx_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AQTX_H_ */
