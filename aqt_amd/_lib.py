@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libaqtx.so')
 
 # element types (include/aqtx.h)
 F32, BF16, I8, I4, E4M3, E5M2, I32, I4P = range(8)
-REDUCE_COLS, REDUCE_ROWS, REDUCE_ALL = range(3)
+REDUCE_COLS, REDUCE_ROWS, REDUCE_ALL, REDUCE_ALL_BATCH = range(4)
 NOISE_NONE, NOISE_JAX_UNIFORM, NOISE_CUSTOM1, NOISE_FP8_MANTISSA = range(4)
 PRESCALE_NONE, PRESCALE_PER_ROW, PRESCALE_PER_COL = range(3)
 SCALE_ROW_THEN_COL, SCALE_COL_THEN_ROW = range(2)
@@ -29,6 +29,7 @@ class QuantPlan(ctypes.Structure):
       ('noise_stride_batch', ctypes.c_int64), ('noise_stride_row', ctypes.c_int64),
       ('noise_stride_col', ctypes.c_int64), ('noise_total', ctypes.c_int64),
       ('prescale', ctypes.c_int32), ('scale_given', ctypes.c_int32),
+      ('prescale_stride_batch', ctypes.c_int64),
   ]
 
 
@@ -59,6 +60,7 @@ SYMBOLS = {
     'aqtx_quantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp, _vp,
                                      ctypes.c_size_t, _vp]),
     'aqtx_quantize_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(QuantPlan)]),
+    'aqtx_dequantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_fp8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_decode_i8': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp,

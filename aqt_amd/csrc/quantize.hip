@@ -36,6 +36,7 @@ struct QArgs {
   int64_t ngroups;  // tile kernels: rows / G
   int64_t ssb, ssg, ssc;  // tile kernels: scale index strides
   int64_t nsb, nsr, nsc;  // noise counter strides
+  int64_t psb;            // prescale batch stride
   float quant_bound, clip_bound;
   BitGen gen;
   int noise;
@@ -182,7 +183,8 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
   const TIn* xp = reinterpret_cast<const TIn*>(a.x) + grow * a.cols + col0;
 
   float row_ps = 1.0f;
-  if (a.ps_mode == AQTX_PRESCALE_PER_ROW) row_ps = a.prescale[r];
+  const float* psv = a.prescale + b * a.psb;
+  if (a.ps_mode == AQTX_PRESCALE_PER_ROW) row_ps = psv[r];
 
   float v[ITERS][VEC];
   float amax = 0.0f;
@@ -195,8 +197,8 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v[it][e] = apply_prescale(v[it][e], row_ps, a);
       } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
-        const float4 p0 = *reinterpret_cast<const float4*>(a.prescale + col0 + j0);
-        const float4 p1 = *reinterpret_cast<const float4*>(a.prescale + col0 + j0 + 4);
+        const float4 p0 = *reinterpret_cast<const float4*>(psv + col0 + j0);
+        const float4 p1 = *reinterpret_cast<const float4*>(psv + col0 + j0 + 4);
         const float ps[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v[it][e] = apply_prescale(v[it][e], ps[e], a);
@@ -250,8 +252,8 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const QArgs a) 
   const TIn* xp = reinterpret_cast<const TIn*>(a.x) + grow * a.cols + col0;
   auto value = [&](int64_t j) {
     float v = Loader<TIn>::load1(xp + j);
-    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[r], a);
-    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[col0 + j], a);
+    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[b * a.psb + r], a);
+    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[b * a.psb + col0 + j], a);
     return v;
   };
   float amax = 0.0f;
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const QArgs a) {
     for (int e = 0; e < VEC; ++e) ps[e] = 1.0f;
     if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) ps[e] = a.prescale[c0 + e];
+      for (int e = 0; e < VEC; ++e) ps[e] = a.prescale[b * a.psb + c0 + e];
     }
     const TIn* xb = reinterpret_cast<const TIn*>(a.x) + b * a.rows * a.cols + c0;
     for (int64_t r = r_begin + wave; r < r_end; r += 4) {
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const QArgs a) {
       if constexpr (VEC == 8) Loader<TIn>::load8(xb + r * a.cols, v);
       else v[0] = Loader<TIn>::load1(xb + r * a.cols);
       if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
-        const float rp = a.prescale[r];
+        const float rp = a.prescale[b * a.psb + r];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v[e] = apply_prescale(v[e], rp, a);
       } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
@@ -347,12 +349,12 @@ __global__ __launch_bounds__(256) void absmax_all_kernel(const QArgs a) {
   float m = 0.0f;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
     float v = Loader<TIn>::load1(xb + i);
-    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[i / a.cols], a);
-    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[i % a.cols], a);
+    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[b * a.psb + i / a.cols], a);
+    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[b * a.psb + i % a.cols], a);
     m = fmaxf(m, fabsf(v));
   }
   m = segment_max<256>(m, smem);
-  if (threadIdx.x == 0) atomicMax(a.ws_absmax + b, __float_as_uint(m));
+  if (threadIdx.x == 0) atomicMax(a.ws_absmax + b * a.ssb, __float_as_uint(m));
 }
 
 // abs-max bit patterns -> scale (output) and reciprocal scale (workspace).
@@ -403,14 +405,14 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a) {
           v[e] = e < nvalid ? Loader<TIn>::load1(xb + r * a.cols + c + e) : 0.0f;
       }
       const int64_t sbase = b * a.ssb + (r / a.G) * a.ssg;
-      const float rp = (a.ps_mode == AQTX_PRESCALE_PER_ROW) ? a.prescale[r] : 1.0f;
+      const float rp = (a.ps_mode == AQTX_PRESCALE_PER_ROW) ? a.prescale[b * a.psb + r] : 1.0f;
       uint32_t w[2] = {0u, 0u};
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (e < nvalid) {
           float x = v[e];
           if (a.ps_mode == AQTX_PRESCALE_PER_ROW) x = apply_prescale(x, rp, a);
-          else if (a.ps_mode == AQTX_PRESCALE_PER_COL) x = apply_prescale(x, a.prescale[c + e], a);
+          else if (a.ps_mode == AQTX_PRESCALE_PER_COL) x = apply_prescale(x, a.prescale[b * a.psb + c + e], a);
           const float inv = a.ws_inv[sbase + (c + e) * a.ssc];
           const uint64_t ctr = (uint64_t)(b * a.nsb + r * a.nsr + (c + e) * a.nsc);
           const uint32_t qv = to_qbyte(scaled_noisy_clipped(x, inv, ctr, a), a.out_dtype);
@@ -463,6 +465,27 @@ __global__ void random_bits_kernel(BitGen gen, int64_t n, void* out) {
   else reinterpret_cast<uint32_t*>(out)[i] = v;
 }
 
+// out[b, r, c] = cast(q) * scale (aqt_tensor.py:179-183), one thread per element.
+template <typename TOut>
+__global__ void dequant_kernel(const QArgs a, int fp8_kind) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t per_b = a.rows * a.cols;
+  if (i >= a.batch * per_b) return;
+  const int64_t b = i / per_b, rc = i % per_b, r = rc / a.cols, c = rc % a.cols;
+  const uint8_t* qb = reinterpret_cast<const uint8_t*>(a.x) + b * per_b;
+  const uint8_t raw = a.transpose_out ? qb[c * a.rows + r] : qb[rc];
+  float v;
+  if (fp8_kind == AQTX_E4M3) v = __builtin_amdgcn_cvt_f32_fp8((int)raw, 0);
+  else if (fp8_kind == AQTX_E5M2) v = __builtin_amdgcn_cvt_f32_bf8((int)raw, 0);
+  else v = (float)(int8_t)raw;
+  const float s = a.scale[b * a.ssb + (r / a.G) * a.ssg + (c / a.L) * a.ssc];
+  v = rnd(v, a.cbf);
+  v = rnd(v * s, a.cbf & a.sbf);
+  v = rnd(v, a.cbf);
+  if constexpr (sizeof(TOut) == 2) reinterpret_cast<uint16_t*>(a.q)[i] = bf16_bits(v);
+  else reinterpret_cast<float*>(a.q)[i] = v;
+}
+
 // ---- host side ---------------------------------------------------------------------
 
 int validate(const aqtx_quant_plan* p) {
@@ -480,11 +503,12 @@ int validate(const aqtx_quant_plan* p) {
                    p->out_dtype == AQTX_E5M2,
                "aqtx_quantize: unsupported out_dtype %d", p->out_dtype);
   AQTX_REQUIRE(p->batch >= 0 && p->rows >= 0 && p->cols >= 0, "aqtx_quantize: negative shape");
-  AQTX_REQUIRE(p->reduce >= AQTX_REDUCE_COLS && p->reduce <= AQTX_REDUCE_ALL,
+  AQTX_REQUIRE(p->reduce >= AQTX_REDUCE_COLS && p->reduce <= AQTX_REDUCE_ALL_BATCH,
                "aqtx_quantize: unknown reduce mode %d", p->reduce);
   AQTX_REQUIRE(p->group >= 0, "aqtx_quantize: negative group");
   if (p->group > 0) {
-    AQTX_REQUIRE(p->reduce != AQTX_REDUCE_ALL, "aqtx_quantize: group with REDUCE_ALL");
+    AQTX_REQUIRE(p->reduce == AQTX_REDUCE_COLS || p->reduce == AQTX_REDUCE_ROWS,
+                 "aqtx_quantize: group needs REDUCE_COLS or REDUCE_ROWS");
     const int64_t axis = p->reduce == AQTX_REDUCE_COLS ? p->cols : p->rows;
     AQTX_REQUIRE(axis % p->group == 0,
                  "aqtx_quantize: group %lld does not divide the reduced axis %lld",
@@ -515,7 +539,8 @@ int64_t scale_count(const aqtx_quant_plan* p) {
   switch (p->reduce) {
     case AQTX_REDUCE_COLS: return p->batch * p->rows * (p->group ? p->cols / p->group : 1);
     case AQTX_REDUCE_ROWS: return p->batch * (p->group ? p->rows / p->group : 1) * p->cols;
-    default: return p->batch;
+    case AQTX_REDUCE_ALL: return p->batch;
+    default: return 1;
   }
 }
 
@@ -557,7 +582,7 @@ int launch_tiles(const QArgs& a, int reduce, int64_t nscales, hipStream_t st) {
   if (!a.scale_given) {
     fill_u32_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a.ws_absmax, nscales, 0u);
     AQTX_HIP_CHECK_LAUNCH("fill_u32_kernel");
-    if (reduce == AQTX_REDUCE_ALL) {
+    if (reduce == AQTX_REDUCE_ALL || reduce == AQTX_REDUCE_ALL_BATCH) {
       int64_t nblk = (a.rows * a.cols + 256 * 16 - 1) / (256 * 16);
       if (nblk > 2048) nblk = 2048;
       if (nblk < 1) nblk = 1;
@@ -598,8 +623,8 @@ using namespace aqtx;
 extern "C" size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* p) {
   if (p == nullptr || p->reduce == AQTX_REDUCE_COLS) return 0;
   if (p->batch < 0 || p->rows < 0 || p->cols < 0 || p->group < 0) return 0;
-  if (p->reduce != AQTX_REDUCE_ROWS && p->reduce != AQTX_REDUCE_ALL) return 0;
-  if (p->group > 0 && (p->reduce == AQTX_REDUCE_ALL || p->rows % p->group != 0)) return 0;
+  if (p->reduce < AQTX_REDUCE_ROWS || p->reduce > AQTX_REDUCE_ALL_BATCH) return 0;
+  if (p->group > 0 && (p->reduce != AQTX_REDUCE_ROWS || p->rows % p->group != 0)) return 0;
   return (size_t)scale_count(p) * 8;
 }
 
@@ -630,7 +655,7 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
   a.batch = p->batch; a.rows = p->rows; a.cols = p->cols;
   a.nsb = p->noise_stride_batch; a.nsr = p->noise_stride_row; a.nsc = p->noise_stride_col;
   a.quant_bound = p->quant_bound; a.clip_bound = p->clip_bound;
-  a.noise = p->noise; a.ps_mode = p->prescale;
+  a.noise = p->noise; a.ps_mode = p->prescale; a.psb = p->prescale_stride_batch;
   a.transpose_out = p->transpose_out; a.out_dtype = p->out_dtype;
   a.cbf = p->compute_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
   a.scale_given = p->scale_given;
@@ -648,9 +673,9 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
       a.ssb = a.ngroups * p->cols; a.ssg = p->cols; a.ssc = 1;
     } else {
       a.G = p->rows; a.ngroups = 1;
-      a.ssb = 1; a.ssg = 0; a.ssc = 0;
+      a.ssb = p->reduce == AQTX_REDUCE_ALL ? 1 : 0; a.ssg = 0; a.ssc = 0;
     }
-    const int64_t grid_y = p->reduce == AQTX_REDUCE_ALL
+    const int64_t grid_y = p->reduce != AQTX_REDUCE_ROWS
                                ? (p->rows + kTileR - 1) / kTileR
                                : a.ngroups * ((a.G + kAbsRowChunk - 1) / kAbsRowChunk);
     AQTX_REQUIRE(grid_y <= 65535 && (p->rows + kTileR - 1) / kTileR <= 65535,
@@ -661,6 +686,39 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
     case AQTX_BF16: return dispatch<uint16_t>(a, p->reduce, nscales, st);
     default: return dispatch<int8_t>(a, p->reduce, nscales, st);
   }
+}
+
+extern "C" int aqtx_dequantize(const aqtx_quant_plan* p, const void* q, const float* scale,
+                               void* out, void* stream) {
+  clear_error();
+  if (int rc = validate(p)) return rc;
+  AQTX_REQUIRE(p->in_dtype != AQTX_I8, "aqtx_dequantize: in_dtype names the float result dtype");
+  const int64_t total = p->batch * p->rows * p->cols;
+  if (total == 0) return 0;
+  AQTX_REQUIRE(q != nullptr && scale != nullptr && out != nullptr, "aqtx_dequantize: NULL buffer");
+  QArgs a{};
+  a.x = q; a.q = out; a.scale = const_cast<float*>(scale);
+  a.batch = p->batch; a.rows = p->rows; a.cols = p->cols;
+  a.transpose_out = p->transpose_out;
+  a.cbf = p->in_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
+  // scale index = b*ssb + (r/G)*ssg + (c/L)*ssc
+  if (p->reduce == AQTX_REDUCE_COLS) {
+    a.L = p->group ? p->group : p->cols; a.G = 1;
+    const int64_t per_row = p->cols / a.L;
+    a.ssb = p->rows * per_row; a.ssg = per_row; a.ssc = 1;
+  } else if (p->reduce == AQTX_REDUCE_ROWS) {
+    a.G = p->group ? p->group : p->rows; a.L = 1;
+    a.ssb = (p->rows / a.G) * p->cols; a.ssg = p->cols; a.ssc = 1;
+  } else {
+    a.G = p->rows; a.L = p->cols; a.ssb = p->reduce == AQTX_REDUCE_ALL ? 1 : 0; a.ssg = 0; a.ssc = 0;
+  }
+  const int fp8_kind = (p->out_dtype == AQTX_E4M3 || p->out_dtype == AQTX_E5M2) ? p->out_dtype : 0;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (p->in_dtype == AQTX_BF16) dequant_kernel<uint16_t><<<dim3(blocks), 256, 0, st>>>(a, fp8_kind);
+  else dequant_kernel<float><<<dim3(blocks), 256, 0, st>>>(a, fp8_kind);
+  AQTX_HIP_CHECK_LAUNCH("dequant_kernel");
+  return 0;
 }
 
 extern "C" int aqtx_random_bits(const uint32_t key_host[2], int64_t n, int32_t bit_width,

@@ -93,14 +93,18 @@ def quantize(
     plan.noise_stride_batch, plan.noise_stride_row, plan.noise_stride_col = nsb, nsr, nsc
     plan.noise_total = noise_total if noise_total is not None else b * r * c
   plan.prescale = prescale_mode
+  if prescale is not None and prescale.dim() == 2 and prescale.shape[0] == b and b > 1:
+    plan.prescale_stride_batch = prescale.shape[1]
   plan.scale_given = int(scale is not None)
 
   if reduce == L.REDUCE_COLS:
     sshape = (b, r, c // group if group else 1)
   elif reduce == L.REDUCE_ROWS:
     sshape = (b, r // group if group else 1, c)
-  else:
+  elif reduce == L.REDUCE_ALL:
     sshape = (b,)
+  else:
+    sshape = (1,)
   if scale is None:
     scale = torch.empty(sshape, dtype=torch.float32, device=x.device)
   else:
@@ -182,4 +186,27 @@ def random_bits(key, n: int, bit_width: int = 32, partitionable: bool = False, d
   out = torch.empty(n, dtype=torch.int16 if bit_width == 16 else torch.int32, device=device)
   _require_gpu(out)
   L.check(L.lib().aqtx_random_bits(k, n, bit_width, int(partitionable), _ptr(out), _stream()))
+  return out
+
+
+def dequantize(q: torch.Tensor, scale: torch.Tensor, *, reduce: int, q_dtype: int, out_dtype,
+               scale_dtype=None, group: int = 0, transposed: bool = False):
+  """out = cast(q) * scale for q as written by `quantize` (one scale).
+
+  q is [batch, rows, cols] (or [batch, cols, rows] when transposed); the result is
+  [batch, rows, cols] of out_dtype.
+  """
+  _require_gpu(q, scale)
+  assert q.dim() == 3 and q.is_contiguous() and scale.dtype == torch.float32 and scale.is_contiguous()
+  b, r, c = (q.shape[0], q.shape[2], q.shape[1]) if transposed else q.shape
+  out_dt = aqtx_dtype(out_dtype)
+  plan = L.QuantPlan()
+  plan.in_dtype = plan.compute_dtype = out_dt
+  plan.scale_dtype = aqtx_dtype(scale_dtype) if scale_dtype is not None else out_dt
+  plan.out_dtype = q_dtype
+  plan.batch, plan.rows, plan.cols = b, r, c
+  plan.reduce, plan.transpose_out, plan.group = reduce, int(transposed), group
+  plan.quant_bound = plan.clip_bound = 1.0
+  out = torch.empty((b, r, c), dtype=_AQTX_TO_TORCH[out_dt], device=q.device)
+  L.check(L.lib().aqtx_dequantize(ctypes.byref(plan), _ptr(q), _ptr(scale), _ptr(out), _stream()))
   return out

@@ -1,0 +1,727 @@
+"""Quantized dot_general (mirrors aqt/jax/v2/aqt_dot_general.py) on HIP kernels.
+
+Same configuration dataclasses, call signatures and assertion behaviour as the
+reference; the arithmetic of one `DotGeneralRaw.__call__` is lowered to
+  quantize(lhs) , quantize(rhs)  ->  MFMA contraction with fused dequantisation
+(see lowering.py, csrc/quantize.hip, csrc/gemm_i8.hip).  Differentiation uses a
+torch.autograd.Function in place of jax.custom_vjp.
+"""
+from __future__ import annotations
+
+import abc
+import copy
+import dataclasses
+import enum
+import functools
+from typing import Any, Optional, Sequence
+
+import numpy as onp
+import torch
+
+from aqt_amd import _lib as L
+from aqt_amd import ops
+from aqt_amd.v2 import aqt_quantizer
+from aqt_amd.v2 import aqt_tensor
+from aqt_amd.v2 import lowering
+from aqt_amd.v2 import transpose
+from aqt_amd.v2 import utils
+from aqt_amd.v2.numerics import fp8_numerics
+from aqt_amd.v2.numerics import no_numerics
+
+dtypes_allowed_for_int32_accum = [utils.int4, utils.int8]
+
+
+class CalibrationMode(enum.Enum):
+  """aqt_dot_general.py:51-55."""
+  CONTRACTING_AXIS = 1
+  REMAINING_AXIS = 2
+
+
+class DequantMode(enum.Enum):
+  """aqt_dot_general.py:58-70."""
+  OUTPUT = 1
+  THIS_INPUT = 2
+  OTHER_INPUT = 3
+
+
+@dataclasses.dataclass(kw_only=True)
+class Tensor:
+  """Configuration of quantization of one side of the op (aqt_dot_general.py:73-85)."""
+  use_fwd_quant: bool = False
+  dequant_mode: DequantMode = DequantMode.OUTPUT
+  calibration_mode: CalibrationMode = CalibrationMode.CONTRACTING_AXIS
+
+
+@dataclasses.dataclass(kw_only=True)
+class LocalAqt:
+  """aqt_dot_general.py:88-96."""
+  contraction_axis_shard_count: Optional[int] = None
+  contraction_axis_shard_size: Optional[int] = None
+  tile_largest_shape: bool = False
+
+
+def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+  """Float dot_general with lax semantics (output axes: batch, lhs remaining, rhs remaining).
+
+  Stands in for `jax.lax.dot_general` as the default `DotGeneralRaw.dot_general`; a
+  plain library GEMM (rocBLAS/hipBLASLt through torch), used for unquantized sides.
+  """
+  del precision
+  (lca, rca), (lba, rba) = dimension_numbers
+  lca, rca, lba, rba = list(lca), list(rca), list(lba), list(rba)
+  lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
+  rra = utils.get_remaining_axes(rhs.dim(), rca, rba)
+  lt = lhs.permute(*(lba + lra + lca))
+  rt = rhs.permute(*(rba + rca + rra))
+  bshape = [lhs.shape[a] for a in lba]
+  mshape = [lhs.shape[a] for a in lra]
+  nshape = [rhs.shape[a] for a in rra]
+  kdim = 1
+  for a in lca:
+    kdim *= lhs.shape[a]
+  b = 1
+  for s in bshape:
+    b *= s
+  out = torch.matmul(lt.reshape(b, -1, kdim), rt.reshape(b, kdim, -1))
+  out = out.reshape(bshape + mshape + nshape)
+  if preferred_element_type is not None:
+    out = out.to(preferred_element_type)
+  return out
+
+
+class DotGeneralQuantizer(abc.ABC):
+  """Plugin point for operand quantization (aqt_dot_general.py:331-422)."""
+
+  @abc.abstractmethod
+  def init_calibration(self):
+    pass
+
+  @abc.abstractmethod
+  def calibrate(self, lhs, rhs, dimension_numbers, lhs_mode, rhs_mode):
+    pass
+
+  @abc.abstractmethod
+  def calculate_qvalue(self, lhs, lhs_qt, rhs, rhs_qt):
+    pass
+
+  @abc.abstractmethod
+  def swap_lhs_and_rhs(self) -> None:
+    pass
+
+  @abc.abstractmethod
+  def assert_calib_shared_axes_value(self, lhs_val, rhs_val, msg: str) -> None:
+    pass
+
+  @abc.abstractmethod
+  def set_context(self, lhs_context, rhs_context) -> None:
+    pass
+
+  def __call__(self, lhs_quantization_info, rhs_quantization_info):
+    """Calibrate then quantize (aqt_dot_general.py:334-360)."""
+    lhs_input, lhs_ca = lhs_quantization_info
+    rhs_input, rhs_ca = rhs_quantization_info
+    dn = ((lhs_ca, rhs_ca), ((), ())) if lhs_ca is not None else None
+    (lhs, lhs_qt), (rhs, rhs_qt) = self.calibrate(
+        lhs_input, rhs_input, dn, CalibrationMode.CONTRACTING_AXIS, CalibrationMode.CONTRACTING_AXIS)
+    return self.calculate_qvalue(lhs, lhs_qt, rhs, rhs_qt)
+
+
+@dataclasses.dataclass(kw_only=True)
+class DefaultDotGeneralQuantizer(DotGeneralQuantizer):
+  """Default dot_general quantizer (aqt_dot_general.py:427-595)."""
+
+  lhs: aqt_quantizer.Quantizer
+  rhs: aqt_quantizer.Quantizer
+  lhs_mid: aqt_quantizer.Quantizer
+  rhs_mid: aqt_quantizer.Quantizer
+  lhs_mid_alpha: Optional[float] = None
+  rhs_mid_alpha: Optional[float] = None
+  skip_mid_scales: bool = True
+
+  def init_calibration(self):
+    self.lhs.init_calibration()
+    self.rhs.init_calibration()
+    if self.lhs_mid_alpha is not None:
+      self.lhs_mid.init_calibration()
+    if self.rhs_mid_alpha is not None:
+      self.rhs_mid.init_calibration()
+
+  def calibrate(self, lhs, rhs, dimension_numbers, lhs_mode, rhs_mode):
+    """aqt_dot_general.py:464-559 without the mid ("SmoothQuant") scales."""
+    if self.lhs_mid_alpha is not None or self.rhs_mid_alpha is not None:
+      raise NotImplementedError('mid-scale quantization has no HIP path yet')
+    if dimension_numbers is not None:
+      (lhs_ca, rhs_ca), (lhs_ba, rhs_ba) = dimension_numbers
+
+      def axes(mode, ndim, ca, ba):
+        if mode == CalibrationMode.REMAINING_AXIS:
+          return utils.get_remaining_axes(ndim, ca, ba)
+        if mode == CalibrationMode.CONTRACTING_AXIS:
+          return ca
+        raise ValueError(f'Unknown calibration mode: {mode}')
+
+      lhs_axes = axes(lhs_mode, lhs.dim(), lhs_ca, lhs_ba)
+      rhs_axes = axes(rhs_mode, rhs.dim(), rhs_ca, rhs_ba)
+    else:
+      lhs_axes = rhs_axes = None
+    lhs_qt = self.lhs.calibrate(lhs, calibration_axes=lhs_axes)
+    rhs_qt = self.rhs.calibrate(rhs, calibration_axes=rhs_axes)
+    return ((lhs, lhs_qt), (rhs, rhs_qt))
+
+  def calculate_qvalue(self, lhs, lhs_qt, rhs, rhs_qt):
+    """aqt_dot_general.py:561-575."""
+    lhs_qt, lhs_grad = self.lhs.calculate_qvalue(lhs, lhs_qt)
+    rhs_qt, rhs_grad = self.rhs.calculate_qvalue(rhs, rhs_qt)
+    return (lhs_qt, lhs_grad), (rhs_qt, rhs_grad)
+
+  def swap_lhs_and_rhs(self) -> None:
+    self.lhs, self.rhs = self.rhs, self.lhs
+
+  def assert_calib_shared_axes_value(self, lhs_val, rhs_val, msg: str) -> None:
+    assert self.lhs.calib_shared_axes == lhs_val, msg
+    assert self.rhs.calib_shared_axes == rhs_val, msg
+
+  def set_context(self, lhs_context, rhs_context) -> None:
+    self.lhs.context = lhs_context
+    self.rhs.context = rhs_context
+
+
+def dot_general_raw_make(lhs_bits=None, rhs_bits=None, local_aqt=None, jax_scope_name='aqt',
+                         initialize_calibration=True, allow_dummy_gradients=False) -> 'DotGeneralRaw':
+  """aqt_dot_general.py:99-156."""
+  lhs_cfg, rhs_cfg = Tensor(), Tensor()
+  if (isinstance(lhs_bits, int) and 2 <= lhs_bits <= 8 and isinstance(rhs_bits, int)
+      and 2 <= rhs_bits <= 8):
+    dg_accumulator_dtype = utils.int32
+  elif lhs_bits in fp8_numerics.fp8_map and rhs_bits in fp8_numerics.fp8_map:
+    dg_accumulator_dtype = utils.float32
+  else:
+    dg_accumulator_dtype = None
+  mk = functools.partial(aqt_quantizer.quantizer_make, initialize_calibration=initialize_calibration)
+  dg_quantizer = DefaultDotGeneralQuantizer(lhs=mk(lhs_bits), rhs=mk(rhs_bits), lhs_mid=mk(None),
+                                            rhs_mid=mk(None))
+  return DotGeneralRaw(lhs=lhs_cfg, rhs=rhs_cfg, dg_quantizer=dg_quantizer,
+                       dg_accumulator_dtype=dg_accumulator_dtype, local_aqt=local_aqt,
+                       jax_scope_name=jax_scope_name,
+                       allow_dummy_gradient_into_qtensor=allow_dummy_gradients)
+
+
+def dot_general_make(lhs_bits=None, rhs_bits=None, bwd_bits=None, use_fwd_quant: bool = True,
+                     dlhs_local_aqt=None, drhs_local_aqt=None,
+                     allow_dummy_gradients: bool = False) -> 'DotGeneral':
+  """aqt_dot_general.py:161-203."""
+  fwd = dot_general_raw_make(lhs_bits, rhs_bits, jax_scope_name='aqt_fwd',
+                             initialize_calibration=False, allow_dummy_gradients=allow_dummy_gradients)
+  dlhs = dot_general_raw_make(bwd_bits, bwd_bits, local_aqt=dlhs_local_aqt, jax_scope_name='aqt_dlhs',
+                              initialize_calibration=False, allow_dummy_gradients=allow_dummy_gradients)
+  drhs = dot_general_raw_make(bwd_bits, bwd_bits, local_aqt=drhs_local_aqt, jax_scope_name='aqt_drhs',
+                              initialize_calibration=False, allow_dummy_gradients=allow_dummy_gradients)
+  cfg = DotGeneral(fwd=fwd, dlhs=dlhs, drhs=drhs)
+  # Surprising: lhs quantization determines what drhs can do.
+  if lhs_bits is not None:
+    cfg.drhs.rhs.use_fwd_quant = use_fwd_quant
+  if rhs_bits is not None:
+    cfg.dlhs.rhs.use_fwd_quant = use_fwd_quant
+  assert cfg.fwd.local_aqt is None, 'local_aqt is not yet supported in fwd.'
+  return cfg
+
+
+@dataclasses.dataclass(kw_only=True)
+class MultiTensor:
+  """aqt_dot_general.py:209-213."""
+  x: Any
+  qx: aqt_tensor.QTensor
+
+
+@dataclasses.dataclass(kw_only=True)
+class TensorRes:
+  """What the forward pass hands to the backward pass (aqt_dot_general.py:215-220)."""
+  mt: MultiTensor
+  quant_grad: Any
+
+
+@dataclasses.dataclass(kw_only=True)
+class DotGeneralRes:
+  lhs: TensorRes
+  rhs: TensorRes
+
+
+def _parse_einsum(eqn: str):
+  ins, out = eqn.replace(' ', '').split('->')
+  l, r = ins.split(',')
+  return l, r, out
+
+
+def einsum(eqn: str, lhs, rhs, dg=lax_dot_general):
+  """Two-operand einsum through an injectable dot_general (aqt_dot_general.py:229-241).
+
+  Letters shared by both operands and the output are batch axes, letters shared by
+  the operands only are contracted; the dot_general output (batch, lhs free, rhs
+  free) is then permuted to the requested order.  Like jnp.einsum's planner, the
+  operand whose free letters come first in the output stays on the left.
+  """
+  l, r, out = _parse_einsum(eqn)
+  assert len(set(l)) == len(l) and len(set(r)) == len(r), 'repeated indices are not supported'
+  batch = [c for c in l if c in r and c in out]
+  contract = [c for c in l if c in r and c not in out]
+  lfree = [c for c in l if c not in r]
+  rfree = [c for c in r if c not in l]
+  for c in lfree + rfree:
+    assert c in out, 'summing a free index is not supported'
+  dn = ((tuple(l.index(c) for c in contract), tuple(r.index(c) for c in contract)),
+        (tuple(l.index(c) for c in batch), tuple(r.index(c) for c in batch)))
+  res = dg(lhs, rhs, dn, None, None)
+  names = batch + lfree + rfree
+  perm = [names.index(c) for c in out]
+  if perm != list(range(len(perm))):
+    res = res.permute(*perm)
+  return res
+
+
+def _get_scale_t(qt, transpose_fn, dimension_numbers, lhs_shape, rhs_shape):
+  return [transpose_fn(s, dimension_numbers, lhs_shape, rhs_shape) for s in qt.scale]
+
+
+def _apply_local_aqt(local_aqt, lhs, rhs, dimension_numbers):
+  """aqt_dot_general.py:259-328."""
+  def factor_reshape_largest(x, ca, ba):
+    assert local_aqt.contraction_axis_shard_size is not None
+    assert local_aqt.contraction_axis_shard_count is None
+    shard_size = local_aqt.contraction_axis_shard_size
+    ca, ba = list(ca), list(ba)
+    if not ca:
+      return x, ca, ba
+    shape = list(x.shape)
+    max_ca_shape = max(shape[axis] for axis in ca)
+    ax = shape.index(max_ca_shape)
+    ax_ca_idx = ca.index(ax)
+    assert max_ca_shape % shard_size == 0
+    shape[ax] = max_ca_shape // shard_size
+    shape.insert(ax + 1, shard_size)
+    new_ca = [(b + int(b >= ax)) for b in ca]
+    assert new_ca[ax_ca_idx] == ax + 1
+    new_ba = [ax] + [(b + int(b > ax)) for b in ba]
+    return x.reshape(shape), new_ca, new_ba
+
+  def factor_reshape(x, ca, ba):
+    msg = 'You are using the original local aqt. Please only set shard_count.'
+    assert local_aqt.contraction_axis_shard_count is not None, msg
+    assert local_aqt.contraction_axis_shard_size is None, msg
+    factor = local_aqt.contraction_axis_shard_count
+    ca, ba = list(ca), list(ba)
+    if not ca:
+      return x, ca, ba
+    shape = list(x.shape)
+    ax = ca[0]
+    orig_size = shape[ax]
+    assert orig_size % factor == 0
+    shape[ax] = factor
+    shape.insert(ax + 1, orig_size // factor)
+    new_ca = [(b + int(b >= ax)) for b in ca]
+    assert new_ca[0] == ax + 1
+    new_ba = [ax] + [(b + int(b > ax)) for b in ba]
+    return x.reshape(shape), new_ca, new_ba
+
+  (lhs_ca, rhs_ca), (lhs_ba, rhs_ba) = dimension_numbers
+  fn = factor_reshape_largest if local_aqt.tile_largest_shape else factor_reshape
+  lhs, lhs_ca, lhs_ba = fn(lhs, lhs_ca, lhs_ba)
+  rhs, rhs_ca, rhs_ba = fn(rhs, rhs_ca, rhs_ba)
+  return lhs, rhs, ((lhs_ca, rhs_ca), (lhs_ba, rhs_ba))
+
+
+_POISON = ('Poison. Gradients are not generally expected in serving. Please set '
+           'allow_dummy_gradient_into_qtensor to True if this is the intended behavior.')
+
+
+@dataclasses.dataclass(kw_only=True)
+class _Prescaled:
+  """`lhs * scale_t` of _maybe_use_fwd_quant, deferred so the quantize kernel can fuse it."""
+  x: Any
+  scale_t: Any
+
+
+def _maybe_use_fwd_quant(lhs, rhs: MultiTensor, dimension_numbers, use_fwd_quant: bool):
+  """aqt_dot_general.py:675-729.  Returns (lhs | _Prescaled, rhs array)."""
+  scale_count = -1
+  if rhs.qx.scale is not None:
+    scale_count = len(rhs.qx.scale)
+  msg = (f'Found use_fwd_quant is {use_fwd_quant} in bwd. It is supported only if there is '
+         f'exactly one scale in a good shape.\n{scale_count=}')
+  if use_fwd_quant:
+    assert scale_count == 1, msg
+    if rhs.qx.bias:
+      raise NotImplementedError('Quantization biases are not supported in forward quantization.')
+    scale_t = transpose.rhs_scale_transpose_for_lhs_input(rhs.qx.scale[0], dimension_numbers, lhs.shape)
+    lhs = _Prescaled(x=lhs, scale_t=scale_t)
+    # The quantized residual is quantized again; the kernel reads the int8/fp8 values as
+    # floats of the dequant dtype (qvalue.astype(dequant_dtype) in the reference).
+    rhs_arr = rhs.qx
+  else:
+    rhs_arr = rhs.x
+  return lhs, rhs_arr
+
+
+def _canonical_pairs(lhs, rhs, dimension_numbers):
+  """Orders the contraction and batch axis pairs by lhs memory position.
+
+  The pairing is what matters to dot_general; the listed order only fixes the order of
+  batch axes in the output, which the caller restores.
+  """
+  (lca, rca), (lba, rba) = dimension_numbers
+  del rhs
+  order, _ = lowering.memory_rank(lhs)
+  pos = {a: i for i, a in enumerate(order)}
+
+  def sort_pairs(la, ra):
+    pairs = sorted(zip(la, ra), key=lambda p: (pos.get(p[0], 10**6), p[0]))
+    return [p[0] for p in pairs], [p[1] for p in pairs]
+
+  lca2, rca2 = sort_pairs(list(lca), list(rca))
+  lba2, rba2 = sort_pairs(list(lba), list(rba))
+  return ((lca2, rca2), (lba2, rba2))
+
+
+@dataclasses.dataclass(kw_only=True)
+class DotGeneralRaw:
+  """Configuration of quantization of one dot_general without gradient (aqt_dot_general.py:732-749)."""
+
+  lhs: Tensor
+  rhs: Tensor
+  dg_quantizer: DotGeneralQuantizer
+  dg_accumulator_dtype: Any
+  local_aqt: Optional[LocalAqt]
+  jax_scope_name: str
+  allow_dummy_gradient_into_qtensor: bool = False
+  dot_general: Any = lax_dot_general
+
+  @classmethod
+  def make(cls, *args, **kwargs):
+    return dot_general_raw_make(*args, **kwargs)
+
+  # ------------------------------------------------------------------------------
+  def __call__(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers):
+    """A quantized dot_general without custom gradient (aqt_dot_general.py:757-840).
+
+    Returns (out, DotGeneralRes).  `rhs` may be a MultiTensor (bwd calls).
+    """
+    with torch.profiler.record_function(self.jax_scope_name):
+      if isinstance(rhs, MultiTensor):
+        lhs, rhs = _maybe_use_fwd_quant(lhs, rhs, dimension_numbers, self.rhs.use_fwd_quant)
+      if self.local_aqt is not None:
+        raise NotImplementedError('LocalAqt has no HIP path yet')
+      for side, name in ((self.lhs, 'lhs'), (self.rhs, 'rhs')):
+        if side.dequant_mode != DequantMode.OUTPUT or side.calibration_mode != CalibrationMode.CONTRACTING_AXIS:
+          raise NotImplementedError(
+              f'{name}: only DequantMode.OUTPUT with CalibrationMode.CONTRACTING_AXIS has a HIP path')
+      return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers)
+
+  # ------------------------------------------------------------------------------
+  def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers):
+    dq = self.dg_quantizer
+    prescale_t = None
+    if isinstance(lhs, _Prescaled):
+      prescale_t, lhs = lhs.scale_t, lhs.x
+    rhs_is_q = isinstance(rhs, aqt_tensor.QTensor)  # re-quantization of a fwd residual
+    rhs_arr = rhs.qvalue if rhs_is_q else rhs
+    lhs_dtype = lhs.dtype
+    rhs_dtype = rhs.dequant_dtype if rhs_is_q else rhs.dtype
+    dequant_dtype = torch.promote_types(lhs_dtype, rhs_dtype)
+
+    lhs_none = isinstance(dq.lhs.numerics, no_numerics.NoNumerics) if isinstance(
+        dq, DefaultDotGeneralQuantizer) else False
+    rhs_none = isinstance(dq.rhs.numerics, no_numerics.NoNumerics) if isinstance(
+        dq, DefaultDotGeneralQuantizer) else False
+
+    if lhs_none and rhs_none and lhs_qt is None and rhs_qt is None:
+      # Unquantized: QTensors without scales around a plain float contraction
+      # (aqt_quantizer.py:111-120; aqt_dot_general.py:921-927 with float operands).
+      x = lhs
+      if prescale_t is not None:
+        x = x * prescale_t.to(x.dtype)
+      y = rhs_arr.to(rhs_dtype) if rhs_is_q else rhs_arr
+      out = self.dot_general(x, y, dimension_numbers, None, self.dg_accumulator_dtype)
+      out = out.to(dequant_dtype)
+      mk = lambda t: aqt_tensor.QTensor(qvalue=t, scale=[], scale_t=None, bias=[], dequant_dtype=t.dtype)
+      res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=x, qx=mk(x)), quant_grad=None),
+                          rhs=TensorRes(mt=MultiTensor(x=y, qx=mk(y)), quant_grad=None))
+      return out, res
+
+    if not isinstance(dq, DefaultDotGeneralQuantizer) or lhs_none or rhs_none:
+      raise NotImplementedError(
+          'only DefaultDotGeneralQuantizer with both sides quantized (or both unquantized) is lowered')
+    if dq.lhs_mid_alpha is not None or dq.rhs_mid_alpha is not None:
+      raise NotImplementedError('mid-scale quantization has no HIP path yet')
+
+    dn = _canonical_pairs(lhs, rhs_arr, dimension_numbers)
+    (lca, rca), (lba, rba) = dn
+    lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
+    rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
+
+    # ---- lhs ---------------------------------------------------------------------
+    lq, ls, lsdt, lhs_qt_out, lhs_grad = self._quant_side(
+        'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t)
+    # ---- rhs ---------------------------------------------------------------------
+    rq, rs, rsdt, rhs_qt_out, rhs_grad = self._quant_side(
+        'rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, rba, rra, rca, None)
+
+    lkd = aqt_tensor.qvalue_kernel_dtype(lhs_qt_out)
+    rkd = aqt_tensor.qvalue_kernel_dtype(rhs_qt_out)
+    fp8 = lkd in (L.E4M3, L.E5M2)
+    if fp8 != (rkd in (L.E4M3, L.E5M2)):
+      raise NotImplementedError('mixed integer / fp8 operands')
+    acc = self.dg_accumulator_dtype
+    if not fp8:
+      assert acc == utils.int32, (
+          f'Found {self.dg_accumulator_dtype=}: integer operands are contracted with an int32 '
+          'accumulator only')
+    else:
+      assert acc in (utils.float32, None), f'{self.dg_accumulator_dtype=} with fp8 operands'
+
+    B, M, K = lq.shape
+    N = rq.shape[1]
+    assert rq.shape[0] == B and rq.shape[2] == K, (lq.shape, rq.shape)
+    # scales: [B, M] / [B, N] or a single per-tensor value (broadcast here, tiny)
+    def expand(s, n):
+      return s.reshape(1, 1).expand(B, n).contiguous() if s.numel() == 1 and B * n != 1 else s.reshape(B, n)
+    sdt = torch.promote_types(lsdt, rsdt)
+    if self.dot_general is not lax_dot_general:
+      raise NotImplementedError('a custom DotGeneralRaw.dot_general hook is not lowered')
+    out = ops.gemm(lq, rq,
+                   row_scale=expand(ls, M), col_scale=expand(rs, N), out_dtype=dequant_dtype,
+                   dequant_dtype=dequant_dtype, scale_dtype=sdt, a_dtype=lkd, b_dtype=rkd)
+    # [B, M, N] -> (batch..., lhs remaining..., rhs remaining...) in the caller's batch order
+    bdims = [lhs.shape[a] for a in lba]
+    out = out.reshape(bdims + [lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
+    want_lba = list(dimension_numbers[1][0])
+    if want_lba != lba:
+      perm = [lba.index(a) for a in want_lba] + list(range(len(lba), out.dim()))
+      out = out.permute(*perm)
+
+    lhs_mt = MultiTensor(x=lhs, qx=lhs_qt_out)
+    rhs_mt = MultiTensor(x=rhs_arr if not rhs_is_q else rhs.qvalue, qx=rhs_qt_out)
+    res = DotGeneralRes(lhs=TensorRes(mt=lhs_mt, quant_grad=lhs_grad),
+                        rhs=TensorRes(mt=rhs_mt, quant_grad=rhs_grad))
+    return out, res
+
+  def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t):
+    """Quantizes one side; returns (q [B,R,K], scale f32, scale dtype, QTensor, quant_grad)."""
+    if given_qt is not None and given_qt.is_full():
+      # Serving: the provided QTensor replaces the computed one (aqt_dot_general.py:614-635).
+      quant_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
+      assert not given_qt.bias, (
+          f'biases are only supported in fake quant mode, but got a {name} bias')
+      assert len(given_qt.scale) == 1, 'a provided QTensor must carry exactly one scale'
+      v = lowering.view_operand(given_qt.qvalue, ba, ra, ca)
+      q = v.mem if v.k_last else v.mem.transpose(1, 2).contiguous()
+      if q.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        q = q.view(torch.uint8)
+      s = given_qt.scale[0]
+      sv = lowering.view_operand(s, ba, ra, ca)
+      s32 = sv.mem.reshape(-1).float().contiguous()
+      return q, s32, s.dtype, given_qt, quant_grad
+    spec = quantizer.kernel_spec()
+    if spec is None:
+      raise NotImplementedError(f'{name}: numerics/calibration {quantizer.numerics} / '
+                                f'{quantizer.calibration} have no fused HIP kernel')
+    if getattr(quantizer.numerics, 'clip_gradient', False):
+      raise NotImplementedError('clip_gradient is not supported by the fused path')
+    arr = x
+    if x_is_q and arr.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+      raise NotImplementedError('re-quantizing an fp8 residual (use_fwd_quant with fp8 fwd)')
+    v = lowering.view_operand(arr, ba, ra, ca)
+    prescale = None
+    if prescale_t is not None:
+      pv = lowering.view_operand(prescale_t, ba, ra, ca)
+      if pv.R != 1 and v.R != 1:
+        raise NotImplementedError('use_fwd_quant scale that varies along the remaining axes')
+      prescale = pv.mem.reshape(pv.B, -1).float().contiguous()
+      if pv.B == 1 and v.B > 1:
+        prescale = prescale.reshape(-1)
+    scale_in = None
+    if given_qt is not None:  # incomplete QTensor: scale only (aqt_dot_general.py:645-653)
+      assert len(given_qt.scale) == 1
+      sv = lowering.view_operand(given_qt.scale[0], ba, ra, ca)
+      scale_in = sv.mem.reshape(-1).float().contiguous()
+      scale_in = scale_in.reshape(v.B, v.R, 1) if v.k_last else scale_in.reshape(v.B, 1, v.R)
+    q, s32, sdt = quantizer.quant_view(v, dtype, calibration_axes=ca, prescale=prescale, scale=scale_in)
+    qv = lowering.logical_from_brk(aqt_quantizer._typed(q, spec['out_dtype']), v)
+    if given_qt is not None:
+      scale_list = given_qt.scale
+    else:
+      if s32.numel() == 1 and (v.B * v.R) != 1:
+        sc = s32.reshape([1] * len(v.shape))
+      else:
+        sc = lowering.logical_from_brk(s32, v, k_keep=False)
+      scale_list = [sc.to(sdt)]
+    qt = aqt_tensor.QTensor(qvalue=qv, scale=scale_list, scale_t=None, bias=[], dequant_dtype=dtype,
+                            container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
+    quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))
+    return q, s32, sdt, qt, quant_grad
+
+
+def _qtensor_dot_general(lhs_qt, rhs_qt, dimension_numbers, cfg, dequant_dtype):
+  """QTensor x QTensor -> dequantized array (aqt_dot_general.py:843-958 + the dequant).
+
+  The reference returns a QTensor (accumulator + output scales) that the caller
+  dequantizes; here the dequantisation is fused into the contraction kernel, so the
+  dequantized array is returned directly.
+  """
+  raw = copy.copy(cfg)
+  out, _ = DotGeneralRaw._lowered_call(raw, lhs_qt.qvalue, rhs_qt.qvalue, lhs_qt, rhs_qt, dimension_numbers)
+  return out.to(dequant_dtype)
+
+
+@dataclasses.dataclass(kw_only=True)
+class DotGeneral:
+  """Configuration of quantization of dot_general and its gradients (aqt_dot_general.py:961-1078)."""
+
+  fwd: DotGeneralRaw
+  dlhs: DotGeneralRaw
+  drhs: DotGeneralRaw
+  apply_custom_vjp_on_jax: bool = True
+
+  @classmethod
+  def make(cls, *args, **kwargs):
+    return dot_general_make(*args, **kwargs)
+
+  def dg_core(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers):
+    """dot_general with expanded API (aqt_dot_general.py:975-1000)."""
+    msg = 'AQT is not yet optimized to accept quantized types directly. '
+    msg += f'lhs.dtype: {lhs.dtype}, rhs.dtype: {rhs.dtype}'
+    assert lhs.dtype in [utils.bfloat16, utils.float32, utils.float16], msg
+    assert rhs.dtype in [utils.bfloat16, utils.float32, utils.float16], msg
+    self.assert_config_validity()
+    if self.apply_custom_vjp_on_jax and (lhs.requires_grad or rhs.requires_grad):
+      out, lq, rq = _DgCoreFn.apply(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, self)
+      return out, (lq, rq)
+    (out, qret), _ = dg_core_vjp_fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, self)
+    return out, qret
+
+  def __call__(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+    """aqt_dot_general.py:1002-1022."""
+    del preferred_element_type
+    assert precision is None, f'Precision {precision} requested together with quantization.'
+    out, _ = self.dg_core(lhs=lhs, rhs=rhs, lhs_qt=None, rhs_qt=None,
+                          dimension_numbers=dimension_numbers)
+    return out
+
+  def assert_config_validity(self):
+    """aqt_dot_general.py:1024-1078."""
+    expected_fwd_quant = False
+    msg_fwd_quant = (f'use_fwd_quant should be set to {expected_fwd_quant} when remaining axis are '
+                     'used for calibration axis. ')
+    if self.fwd.rhs.calibration_mode == CalibrationMode.REMAINING_AXIS:
+      assert self.dlhs.rhs.use_fwd_quant is expected_fwd_quant, msg_fwd_quant
+    if self.fwd.lhs.calibration_mode == CalibrationMode.REMAINING_AXIS:
+      assert self.drhs.rhs.use_fwd_quant is expected_fwd_quant, msg_fwd_quant
+    unsupported = [(DequantMode.OUTPUT, CalibrationMode.REMAINING_AXIS),
+                   (DequantMode.OTHER_INPUT, CalibrationMode.CONTRACTING_AXIS)]
+    msg = 'Unsupported calibration mode - dequant mode combination '
+    for dequant_mode, calibration_mode in unsupported:
+      assert not (self.fwd.lhs.calibration_mode == calibration_mode
+                  and self.fwd.lhs.dequant_mode == dequant_mode), msg + ' for lhs.'
+      assert not (self.fwd.rhs.calibration_mode == calibration_mode
+                  and self.fwd.rhs.dequant_mode == dequant_mode), msg + ' for rhs.'
+
+
+def _fresh_cfg(cfg: 'DotGeneral') -> 'DotGeneral':
+  """Copy of the config tree down to the quantizers.
+
+  Under jax.custom_vjp the config reaches dg_core_vjp_fwd as a pytree argument, i.e. as a
+  fresh copy on every call, which is why init_calibration() may assert that it runs once;
+  this gives a reused config object the same behaviour.
+  """
+  cfg = copy.copy(cfg)
+  for name in ('fwd', 'dlhs', 'drhs'):
+    raw = copy.copy(getattr(cfg, name))
+    dq = copy.copy(raw.dg_quantizer)
+    for qn in ('lhs', 'rhs', 'lhs_mid', 'rhs_mid'):
+      if hasattr(dq, qn):
+        q = copy.copy(getattr(dq, qn))
+        q._calibrator = None
+        setattr(dq, qn, q)
+    raw.dg_quantizer = dq
+    setattr(cfg, name, raw)
+  return cfg
+
+
+def dg_core_vjp_fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, cfg: DotGeneral):
+  """Forward pass (aqt_dot_general.py:1098-1124)."""
+  assert lhs.dtype == rhs.dtype, f'Unmatched lhs and rhs dtype: {lhs.dtype} vs {rhs.dtype}'
+  cfg = _fresh_cfg(cfg)
+  cfg.fwd.dg_quantizer.init_calibration()
+  cfg.dlhs.dg_quantizer.init_calibration()
+  cfg.drhs.dg_quantizer.init_calibration()
+  ret, res = cfg.fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers)
+  ret = ret.to(lhs.dtype)
+  assert res is not None, 'res cannot be None in fwd pass.'
+  qret = (res.lhs.mt.qx, res.rhs.mt.qx)
+  return ((ret, qret), (res, cfg))
+
+
+def _update_dimension_numbers_for_backward(fwd_dimension_numbers, y_is_lhs, gradient_rank, y_rank):
+  """aqt_dot_general.py:1127-1175."""
+  def ranges_like(*xs):
+    start = 0
+    for x in xs:
+      yield tuple(range(start, start + len(x)))
+      start += len(x)
+
+  (x_ca, y_ca), (x_ba, y_ba) = fwd_dimension_numbers
+  if y_is_lhs:
+    (y_ca, x_ca) = (x_ca, y_ca)
+    (y_ba, x_ba) = (x_ba, y_ba)
+  gradient_rank = gradient_rank - y_rank + len(x_ba) + 2 * len(x_ca)
+  x_ra = tuple(utils.get_remaining_axes(gradient_rank, x_ca, x_ba))
+  y_ra = tuple(utils.get_remaining_axes(y_rank, y_ca, y_ba))
+  if y_is_lhs:
+    g_ba, g_ca, _ = ranges_like(x_ba, y_ra, x_ra)
+  else:
+    g_ba, _, g_ca = ranges_like(x_ba, x_ra, y_ra)
+  dims = ((g_ca, y_ra), (g_ba, tuple(y_ba)))
+  x_ca_sorted_by_y = tuple(int(i) for i in onp.take(x_ca, onp.argsort(y_ca)))
+  out_transpose_axes = tuple(int(i) for i in onp.argsort(tuple(x_ba) + x_ra + x_ca_sorted_by_y))
+  return dims, out_transpose_axes
+
+
+def dg_core_vjp_bwd(fwd_dimension_numbers, res, g):
+  """Backward pass (aqt_dot_general.py:1178-1221). Returns (dlhs, drhs, None, None, None)."""
+  dg_res, cfg = res
+  msg = 'dg_res can only be None in 2nd derivative. It is not yet supported.'
+  assert dg_res is not None, msg
+  g = g[0]
+
+  def grad_dot_general(y_res: TensorRes, quant_grad, dg_raw: DotGeneralRaw, y_is_lhs):
+    dims, out_transpose_axes = _update_dimension_numbers_for_backward(
+        fwd_dimension_numbers, y_is_lhs, g.dim(), y_res.mt.x.dim())
+    out, _ = dg_raw(g, y_res.mt, None, None, dims)
+    transposed_out = out.permute(*out_transpose_axes)
+    if quant_grad is not None:
+      assert not isinstance(quant_grad, str), quant_grad
+      transposed_out = quant_grad(transposed_out)[0]
+    return transposed_out
+
+  dlhs = grad_dot_general(dg_res.rhs, dg_res.lhs.quant_grad, cfg.dlhs, False)
+  drhs = grad_dot_general(dg_res.lhs, dg_res.rhs.quant_grad, cfg.drhs, True)
+  return (dlhs, drhs, None, None, None)
+
+
+class _DgCoreFn(torch.autograd.Function):
+  """torch.autograd stand-in for jax.custom_vjp(_dg_core) (aqt_dot_general.py:993-997)."""
+
+  @staticmethod
+  def forward(ctx, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, cfg):
+    (out, (lq, rq)), (res, cfg) = dg_core_vjp_fwd(lhs.detach(), rhs.detach(), lhs_qt, rhs_qt,
+                                                  dimension_numbers, cfg)
+    ctx.aqt_res = (res, cfg)
+    ctx.dimension_numbers = dimension_numbers
+    ctx.set_materialize_grads(False)
+    # QTensors are plain Python objects to autograd and pass through untouched.
+    return out, lq, rq
+
+  @staticmethod
+  def backward(ctx, g, *_):
+    if g is None:
+      return None, None, None, None, None, None
+    dlhs, drhs, *_ = dg_core_vjp_bwd(ctx.dimension_numbers, ctx.aqt_res, (g.contiguous(), None))
+    return dlhs, drhs, None, None, None, None

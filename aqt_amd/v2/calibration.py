@@ -1,0 +1,75 @@
+"""Scale calibration (mirrors aqt/jax/v2/calibration.py:25-157).
+
+The abs-max reduction runs inside the quantize kernel; these classes carry the
+settings and, when called on their own, run that kernel for the scale only.
+"""
+from __future__ import annotations
+
+import abc
+import dataclasses
+from typing import Any, Optional, Sequence
+
+import torch
+
+from aqt_amd.v2 import utils
+
+
+@dataclasses.dataclass(kw_only=True)
+class Calibration(abc.ABC):
+  """calibration.py:34-64."""
+
+  # dtype of the scale arrays; None = the dtype of the input.
+  dtype: Any = None
+  po2_scale: bool = False
+
+  @abc.abstractmethod
+  def get_scale_and_bias_and_sparsity(self, x, shared_axes, numerics_, context=None):
+    pass
+
+  def init_calibration(self):
+    pass
+
+  def kernel_supported(self) -> bool:
+    """True if the fused abs-max kernel implements exactly this calibration."""
+    return False
+
+
+@dataclasses.dataclass(kw_only=True)
+class AbsMaxCalibration(Calibration):
+  """max(abs(x)) / quant_bound (calibration.py:107-157)."""
+
+  clipping_scale: Optional[float] = None
+
+  def kernel_supported(self) -> bool:
+    return not self.po2_scale and not self.clipping_scale
+
+  def get_scale_and_bias_and_sparsity(self, x, shared_axes, numerics_, context=None):
+    del context
+    msg = ('Perhaps you are using DequantMode.THIS_INPUT (fake_quant) and forgot to set them.')
+    assert shared_axes is not None, msg
+    if not self.kernel_supported():
+      raise NotImplementedError('po2_scale / clipping_scale have no HIP kernel yet')
+    from aqt_amd.v2 import lowering  # local import: lowering imports this module's users
+    scale = lowering.absmax_scale(x, list(shared_axes), numerics_, self.dtype)
+    return [scale], [], None
+
+
+@dataclasses.dataclass(kw_only=True)
+class ConstantCalibration(Calibration):
+  """Constant bound (calibration.py:68-104): scale = bound / quant_bound, no reduction."""
+
+  bound: Any = None
+  bias: Any = None
+
+  def get_scale_and_bias_and_sparsity(self, x, shared_axes, numerics_, context=None):
+    del context
+    if isinstance(self.bound, float) and self.bound <= 0.0:
+      raise ValueError(f'{self.bound=} should be positive.')
+    if self.po2_scale or self.bias is not None:
+      raise NotImplementedError('po2_scale / bias have no HIP kernel yet')
+    dtype = self.dtype if self.dtype is not None else x.dtype
+    shape = [1 if a in list(shared_axes) else s for a, s in enumerate(x.shape)]
+    # bound and quant_bound are host constants; the division happens in x.dtype.
+    bound = torch.full(shape, float(self.bound), dtype=x.dtype, device=x.device)
+    scale = bound / torch.tensor(float(numerics_.get_quant_bound()), dtype=x.dtype, device=x.device)
+    return [scale.to(dtype)], [], None

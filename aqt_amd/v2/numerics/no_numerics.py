@@ -1,0 +1,23 @@
+"""No quantization (mirrors aqt/jax/v2/numerics/no_numerics.py:23-43)."""
+import dataclasses
+from typing import Any
+
+from aqt_amd.v2.numerics import numerics
+
+
+@dataclasses.dataclass(kw_only=True)
+class NoNumerics(numerics.AqtNumerics):
+  noise_fn: Any = None
+  dtype: Any = None
+
+  def get_dtype(self):
+    return None
+
+  def get_quant_bound(self):
+    pass
+
+  def vjp_fwd(self, x, context):
+    pass
+
+  def vjp_bwd(self, res, grad):
+    pass

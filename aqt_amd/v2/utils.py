@@ -1,0 +1,92 @@
+"""Shared helpers and small types (mirrors aqt/jax/v2/utils.py:63-155).
+
+The reference builds its configs from `flax.struct` dataclasses (mutable, slotted,
+keyword-only).  Here they are plain mutable keyword-only dataclasses; "static"
+and "dynamic" fields are the same thing because nothing is traced.
+"""
+from __future__ import annotations
+
+import dataclasses
+import enum
+from typing import Any, Callable, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+AxisIdx = int
+AxisSize = int
+# lax.dot_general-like callables: (lhs, rhs, dimension_numbers, precision=None,
+# preferred_element_type=None) -> array.
+DotGeneralT = Callable[..., Any]
+
+dataclass = dataclasses.dataclass
+flax_slots_dataclass = dataclasses.dataclass
+flax_slots_kw_only_dataclass = lambda cls: dataclasses.dataclass(cls, kw_only=True)  # noqa: E731
+
+
+def static_field(**kwargs):
+  return dataclasses.field(**kwargs)
+
+
+def dynamic_field(**kwargs):
+  return dataclasses.field(**kwargs)
+
+
+class _Int4:
+  """Stands for jnp.int4: 4-bit values kept one per byte in an int8 tensor."""
+
+  def __repr__(self):
+    return 'int4'
+
+
+# dtype names the reference takes from jax.numpy
+int4 = _Int4()
+int8 = torch.int8
+int32 = torch.int32
+bfloat16 = torch.bfloat16
+float32 = torch.float32
+float16 = torch.float16
+float8_e4m3fn = torch.float8_e4m3fn
+float8_e5m2 = torch.float8_e5m2
+
+
+class QuantMode(enum.Enum):
+  """utils.py:85-89."""
+  TRAIN = 1
+  CALIBRATE = 2
+  CONVERT = 3
+  SERVE = 4
+
+
+def infer_dtype_from_bits(bits: int):
+  """utils.py:120-135."""
+  if bits == 4:
+    return int4
+  if 2 <= bits <= 8:
+    return int8
+  return None
+
+
+def get_remaining_axes(rank: int, contraction_axes: Sequence[int], batch_axes: Sequence[int]):
+  """utils.py:138-148."""
+  used = list(contraction_axes) + list(batch_axes)
+  return [i for i in range(rank) if i not in used]
+
+
+@dataclasses.dataclass
+class Context:
+  """utils.py:151-155. `key` is raw threefry key data: uint32[2] (numpy)."""
+  key: Any = None
+  train_step: Optional[int] = None
+  quant_mode: QuantMode = QuantMode.TRAIN
+
+
+# Process-wide switch standing for jax.config.jax_threefry_partitionable: it selects
+# which of the two jax.random counter layouts the noise kernels reproduce.
+threefry_partitionable = False
+
+
+def prng_key(seed: int) -> np.ndarray:
+  """jax.random.PRNGKey(seed) as raw key data."""
+  seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+  return np.array([seed >> 32, seed & 0xFFFFFFFF], dtype=np.uint32)

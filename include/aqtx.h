@@ -47,7 +47,8 @@ enum {
 enum {
   AQTX_REDUCE_COLS = 0, /* one scale per (batch,row[,group])  -> scale[batch][rows][cols/group] */
   AQTX_REDUCE_ROWS = 1, /* one scale per (batch[,group],col)  -> scale[batch][rows/group][cols] */
-  AQTX_REDUCE_ALL = 2   /* one scale per batch entry          -> scale[batch]                   */
+  AQTX_REDUCE_ALL = 2,  /* one scale per batch entry          -> scale[batch]                   */
+  AQTX_REDUCE_ALL_BATCH = 3 /* one scale for the whole tensor  -> scale[1]                       */
 };
 
 /* noise added before rounding */
@@ -83,6 +84,7 @@ typedef struct aqtx_quant_plan {
   int64_t noise_stride_batch, noise_stride_row, noise_stride_col, noise_total;
   int32_t prescale;      /* AQTX_PRESCALE_*: x := round(x * cast(v)) first              */
   int32_t scale_given;   /* 1: `scale` is an input (calibration skipped)                */
+  int64_t prescale_stride_batch; /* prescale vector of batch b starts at b*this (0 = shared)  */
 } aqtx_quant_plan;
 
 /*
@@ -94,7 +96,7 @@ typedef struct aqtx_quant_plan {
  * (stochastic_rounding.py:36-78) and the gradient pre-scaling of
  * _maybe_use_fwd_quant (aqt_dot_general.py:714-720).
  *   x         in  : [batch, rows, cols] of in_dtype
- *   prescale  in  : float32 [rows] or [cols] (NULL when plan->prescale == NONE)
+ *   prescale  in  : float32 [rows] or [cols] per batch entry (NULL when plan->prescale == NONE)
  *   q         out : int8 / fp8 bytes, [batch, rows, cols] or transposed
  *   scale     out : float32, layout per plan->reduce (input when scale_given)
  *   workspace     : aqtx_quantize_workspace_bytes(plan) bytes of scratch
@@ -105,6 +107,19 @@ int aqtx_quantize(const aqtx_quant_plan* plan, const void* x, const float* presc
 
 /* Scratch bytes aqtx_quantize needs for `plan` (0 for single-pass plans). */
 size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* plan);
+
+/*
+ * aqtx_dequantize: out = cast(q) * scale for a quantized tensor with one scale.
+ * Replaces QTensor.dequant (aqt/jax/v2/aqt_tensor.py:161-200) for a tensor
+ * that has not gone through a contraction (fake-quant, checkpoint inspection).
+ * The plan describes q the way aqtx_quantize wrote it: in_dtype is the
+ * dequantized dtype to produce (AQTX_F32 | AQTX_BF16), out_dtype the storage
+ * type of q (AQTX_I8 | AQTX_I4 | AQTX_E4M3 | AQTX_E5M2), reduce/group the scale
+ * layout, transpose_out whether q is stored [batch, cols, rows].  The result is
+ * [batch, rows, cols] of in_dtype.
+ */
+int aqtx_dequantize(const aqtx_quant_plan* plan, const void* q, const float* scale, void* out,
+                    void* stream);
 
 enum { AQTX_SCALE_ROW_THEN_COL = 0, AQTX_SCALE_COL_THEN_ROW = 1 };
 
