@@ -23,6 +23,48 @@ _TORCH_TO_AQTX = {
 _AQTX_TO_TORCH = {L.F32: torch.float32, L.BF16: torch.bfloat16, L.I32: torch.int32}
 
 
+class KernelTimer:
+  """Collects HIP-event pairs around chosen C-ABI launches on the launching stream.
+
+  Used by the benchmark to time one kernel family inside a full step:
+  `with KernelTimer('gemm') as t: ...; t.mean_ms()` after a synchronize.
+  """
+  active = None
+
+  def __init__(self, family: str):
+    self.family = family
+    self.pairs = []
+
+  def __enter__(self):
+    KernelTimer.active = self
+    return self
+
+  def __exit__(self, *exc):
+    KernelTimer.active = None
+    return False
+
+  def mean_ms(self):
+    return sum(a.elapsed_time(b) for a, b in self.pairs) / max(len(self.pairs), 1)
+
+
+class _timed:
+  def __init__(self, family):
+    t = KernelTimer.active
+    self.t = t if (t is not None and t.family == family) else None
+
+  def __enter__(self):
+    if self.t is not None:
+      self.a = torch.cuda.Event(enable_timing=True)
+      self.a.record(torch.cuda.current_stream())
+
+  def __exit__(self, *exc):
+    if self.t is not None:
+      b = torch.cuda.Event(enable_timing=True)
+      b.record(torch.cuda.current_stream())
+      self.t.pairs.append((self.a, b))
+    return False
+
+
 def aqtx_dtype(dt) -> int:
   if isinstance(dt, int):
     return dt
@@ -167,8 +209,9 @@ def gemm(
           tuple(s.shape), (batch, dim))
   plan.row_scale_stride_b, plan.col_scale_stride_b = m, n
   fn = L.lib().aqtx_gemm_fp8 if fp8 else L.lib().aqtx_gemm_i8
-  L.check(fn(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale), _ptr(col_scale), _ptr(c),
-             _ptr(acc), _stream()))
+  with _timed('gemm'):
+    L.check(fn(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale), _ptr(col_scale), _ptr(c),
+               _ptr(acc), _stream()))
   return (c, acc) if want_acc else c
 
 

@@ -1,0 +1,135 @@
+"""Benchmark of the quantized dot_general hot path on one MI355X.
+
+One step = one int8 AqtDotGeneral forward + backward (dlhs, drhs) at the LLM MLP
+shape of BASELINE.json's metric: lhs bf16 [8192, 4096] (0.5% outliers x20), rhs
+bf16 [4096, 14336] ~N(0, 0.02), `fully_quantized(fwd_bits=8, bwd_bits=8)`:
+per-token / per-channel abs-max scales, RTN forward, stochastic rounding from a
+fixed PRNG key in dlhs/drhs, int32 accumulation, bf16 output.  Inputs live in HBM
+before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+M, K, N = 8192, 4096, 14336
+OPS_PER_CONTRACTION = 2.0 * M * N * K          # 9.6207e11
+OPS_PER_STEP = 3.0 * OPS_PER_CONTRACTION       # fwd + dlhs + drhs
+INT8_MFMA_PEAK = 5.0e15                        # MI355X dense int8, published
+MATMUL = (((1,), (0,)), ((), ()))
+
+
+def make_inputs(device):
+  import numpy as np
+  import torch
+  rng = np.random.default_rng(20240607)
+  lhs = rng.standard_normal((M, K), dtype=np.float32)
+  lhs = np.where(rng.random((M, K)) < 0.005, lhs * np.float32(20.0), lhs)
+  rhs = rng.standard_normal((K, N), dtype=np.float32) * np.float32(0.02)
+  g = rng.standard_normal((M, N), dtype=np.float32) * np.float32(1e-3)
+  to = lambda a: torch.from_numpy(a).to(torch.bfloat16).to(device)
+  return to(lhs), to(rhs), to(g)
+
+
+def cpu_baseline(seconds_budget=20.0):
+  """Times the numpy oracle (a port, not the reference) on a bounded sample of the workload."""
+  import numpy as np
+  from oracle import aqt_ref as R
+  from oracle import numerics as nm
+  from oracle import prng
+  m, k, n = 1024, 4096, 1792  # 1/8 of M and N, full K: same row lengths for the fwd quantizers
+  rng = np.random.default_rng(1)
+  lhs = nm.to_bf16(rng.standard_normal((m, k), dtype=np.float32))
+  rhs = nm.to_bf16(rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.02))
+  g = nm.to_bf16(rng.standard_normal((m, n), dtype=np.float32) * np.float32(1e-3))
+  cfg = R.set_context(R.fully_quantized(8, 8), prng.prng_key(42))
+  ops = 3.0 * 2.0 * m * k * n
+  times = []
+  t_start = time.perf_counter()
+  while True:
+    t0 = time.perf_counter()
+    f = R.dg_fwd(lhs, rhs, 'bf16', MATMUL, cfg)
+    R.dg_bwd(g, 'bf16', MATMUL, f, cfg)
+    times.append(time.perf_counter() - t0)
+    if len(times) >= 3 or time.perf_counter() - t_start > seconds_budget:
+      break
+  best = min(times)
+  cores = int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1))
+  return {
+      'value': ops / best / 1e12, 'unit': 'TOPS', 'cores': cores, 'kind': 'port',
+      'sample': f'numpy oracle fwd+bwd at {m}x{k}x{n} (1/64 of the ops of one step), best of '
+                f'{len(times)}; BLAS float64 GEMM on {cores} threads, elementwise single-thread',
+  }
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--gpus', type=int, default=1)
+  ap.add_argument('--steps', type=int, default=20)
+  ap.add_argument('--warmup', type=int, default=3)
+  ap.add_argument('--no-cpu-baseline', action='store_true')
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)',
+          file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+  from aqt_amd import ops
+  from aqt_amd.v2 import config, utils
+
+  if not torch.cuda.is_available():
+    print('bench.py needs a GPU', file=sys.stderr)
+    sys.exit(1)
+  dev = torch.device('cuda:0')
+  lhs, rhs, g = make_inputs(dev)
+  lhs.requires_grad_(True)
+  rhs.requires_grad_(True)
+  cfg = config.set_context(config.fully_quantized(fwd_bits=8, bwd_bits=8), utils.prng_key(42), None)
+
+  def step():
+    lhs.grad = None
+    rhs.grad = None
+    out, _ = cfg.dg_core(lhs, rhs, None, None, MATMUL)
+    out.backward(g)
+    return out
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  with ops.KernelTimer('gemm') as timer:
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+  ms_per_step = elapsed / args.steps * 1e3
+  gemm_ms = timer.mean_ms()
+  achieved = OPS_PER_CONTRACTION / (gemm_ms * 1e-3) / 1e12
+
+  line = {
+      'metric': 'int8 dot_general TOPS @8192x4096x14336 (fwd+bwd)',
+      'value': OPS_PER_STEP / (ms_per_step * 1e-3) / 1e12,
+      'unit': 'TOPS',
+      'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': ms_per_step,
+      'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+      'dtype': 'int8', 'data': 'synthetic',
+      'config': {'workload': 'configs[1]: int8 dot_general fwd+bwd, lhs bf16 [8192,4096] x rhs bf16 '
+                             '[4096,14336], fully_quantized(8,8), SR key 42, bf16 out',
+                 'pct_of_int8_mfma_peak': 100.0 * OPS_PER_STEP / (ms_per_step * 1e-3) / INT8_MFMA_PEAK},
+      'roofline': {'bound': 'mfma', 'kernel': 'gemm_i8_kernel', 'achieved': achieved,
+                   'peak': INT8_MFMA_PEAK / 1e12, 'unit': 'TFLOP/s',
+                   'frac': achieved * 1e12 / INT8_MFMA_PEAK, 'traffic': None,
+                   'launch_ms': gemm_ms, 'launches_timed': len(timer.pairs)},
+  }
+  if not args.no_cpu_baseline:
+    line['cpu_baseline'] = cpu_baseline()
+  print(json.dumps(line))
+
+
+if __name__ == '__main__':
+  main()
