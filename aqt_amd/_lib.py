@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, 'lib', 'libaqtx.so')
+# AQTX_LIB_PATH points at another build of the same C-ABI (kernel experiments).
+LIB_PATH = os.environ.get('AQTX_LIB_PATH') or os.path.join(_HERE, 'lib', 'libaqtx.so')
 
 # element types (include/aqtx.h)
 F32, BF16, I8, I4, E4M3, E5M2, I32, I4P = range(8)

@@ -16,6 +16,8 @@
 // The MFMA "A" operand is fed from the B tile and vice versa, so a lane ends up
 // holding 4 consecutive n for one m; the epilogue converts, scales, packs these
 // and sends them through LDS to leave as full 256-byte row segments.
+#include <type_traits>
+
 #include "common.h"
 
 namespace aqtx {
@@ -42,10 +44,11 @@ struct GemmArgs {
 };
 
 constexpr int BM = 256, BN = 256, BK = 128;
-constexpr int kStageBytes = (BM + BN) * BK;       // 65536
-constexpr int kEpiRowBytes = 256 + 8;             // padded row of one wave's 128-row region
-constexpr int kEpiWaveBytes = 128 * kEpiRowBytes; // 33792
-constexpr int kLdsBytes = 4 * kEpiWaveBytes > 2 * kStageBytes ? 4 * kEpiWaveBytes : 2 * kStageBytes;
+constexpr int kTileBytes = BM * BK;          // one operand tile of one stage: 32 KiB
+constexpr int kStageBytes = 2 * kTileBytes;  // A tile + B tile
+constexpr uint32_t kBufferRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format (gfx9)
+
+#define AQTX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
 
@@ -67,11 +70,20 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tn = in_band / rows_in_band;
 }
 
+// EPI selects the epilogue arithmetic at compile time (run-time flags there turn into
+// thousands of branches): 0 = bf16 out, bf16 scales; 1 = bf16 out, f32 scales; 2 = f32 out,
+// f32 scales; 3 = raw int32 accumulators only.  COL_FIRST: the column scale multiplies first.
+// KTAIL: K is not a multiple of the 128-byte stage, the last stage masks chunks past K.
+template <int EPI, bool COL_FIRST, bool KTAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm_i8_kernel(const GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+  // Two stages in two distinct LDS objects, so that the compiler can tell the stage
+  // being filled by the buffer->LDS loads from the one the MFMA fragments are read from.
+  __shared__ __attribute__((aligned(1024))) uint8_t stage0[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t stage1[kStageBytes];
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int lr = lane & 31, lh = lane >> 5;
 
@@ -79,35 +91,34 @@ void gemm_i8_kernel(const GemmArgs g) {
   tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
   const int64_t bz = blockIdx.y;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-  const int8_t* A = g.a + bz * g.stride_a;
-  const int8_t* B = g.b + bz * g.stride_b;
 
-  // ---- global -> register staging: thread owns chunk (tid&7) of rows (tid>>3)+32*i
-  const int gc = tid & 7, gr = tid >> 3;
-  const int gf0 = (gr ^ (gr >> 3)) & 7;
-  uint4 stage_a[8], stage_b[8];
-
-  auto load_global = [&](int64_t k0) {
-    const int64_t kb = k0 + gc * 16;
-    const bool kok = kb < g.k;
+  // ---- global -> LDS: each wave instruction moves 8 rows x 128 B (1 KiB) straight into LDS.
+  // Lane l fills LDS slot (row l>>3, chunk l&7) of its block and therefore fetches the global
+  // chunk (l&7) ^ f(row), f(row) = (row ^ row>>3) & 7: that is the XOR swizzle the fragment
+  // reads undo.  Rows past the end of the operand fall outside the buffer and read as zero.
+  const int64_t rows_a = (g.m - m0) < BM ? (g.m - m0) : BM;
+  const int64_t rows_b = (g.n - n0) < BN ? (g.n - n0) : BN;
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + g.k), kBufferRsrcWord3);
+  int voff_a[8], voff_b[8], chunk_byte[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = (wave * 8 + i) * 8 + (lane >> 3);
+    chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ i) & 7) * 16;
+    voff_a[i] = row * (int)g.lda + chunk_byte[i];
+    voff_b[i] = row * (int)g.ldb + chunk_byte[i];
+  }
+  auto issue_loads = [&](uint8_t* st, int k0) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int64_t ra = m0 + gr + 32 * i, rb = n0 + gr + 32 * i;
-      stage_a[i] = (kok && ra < g.m) ? *reinterpret_cast<const uint4*>(A + ra * g.lda + kb)
-                                     : make_uint4(0, 0, 0, 0);
-      stage_b[i] = (kok && rb < g.n) ? *reinterpret_cast<const uint4*>(B + rb * g.ldb + kb)
-                                     : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto store_lds = [&](int stage) {
-    uint8_t* sa = lds + stage * kStageBytes;
-    uint8_t* sb = sa + BM * BK;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = gr + 32 * i;
-      const int sw = (gc ^ gf0 ^ (4 * (i & 1))) * 16;
-      *reinterpret_cast<uint4*>(sa + row * BK + sw) = stage_a[i];
-      *reinterpret_cast<uint4*>(sb + row * BK + sw) = stage_b[i];
+      int va = voff_a[i], vb = voff_b[i];
+      if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) va = vb = 0x7FFFFFF0;  // out of range -> zeros
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, AQTX_LDS_PTR(st + (wave * 8 + i) * 1024), 16,
+                                               va, k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_b, AQTX_LDS_PTR(st + kTileBytes + (wave * 8 + i) * 1024), 16, vb, k0, 0, 0);
     }
   };
 
@@ -116,8 +127,8 @@ void gemm_i8_kernel(const GemmArgs g) {
   int frag_off[8];
 #pragma unroll
   for (int cidx = 0; cidx < 8; ++cidx) frag_off[cidx] = lr * BK + ((lh ^ lf0 ^ cidx) * 16);
-  const int a_base = wm * 128 * BK;            // rows of the A tile this wave needs
-  const int b_base = BM * BK + wn * 128 * BK;  // rows of the B tile
+  const int a_base = wm * 128 * BK;                // rows of the A tile this wave needs
+  const int b_base = kTileBytes + wn * 128 * BK;   // rows of the B tile
 
   v16i acc[4][4];
 #pragma unroll
@@ -127,39 +138,88 @@ void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  const int KT = (int)((g.k + BK - 1) / BK);
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-
-  for (int kt = 0; kt < KT; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < KT) load_global((int64_t)(kt + 1) * BK);
-    const uint8_t* st = lds + cur * kStageBytes;
+  auto load_frags = [&](const uint8_t* st, int ks, v4i* fa, v4i* fb) {
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      v4i fa[4], fb[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int cidx = (2 * ks) ^ (4 * (i & 1));
-        fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[cidx]);
-        fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[cidx]);
-      }
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+    for (int i = 0; i < 4; ++i) {
+      const int cidx = (2 * ks) ^ (4 * (i & 1));
+      fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[cidx]);
+      fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[cidx]);
     }
-    if (kt + 1 < KT) store_lds(cur ^ 1);
+  };
+  auto mfma_step = [&](const v4i* fa, const v4i* fb) {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+        acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+  };
+  // Scheduling groups (llvm.amdgcn.sched.group.barrier masks).
+  constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100;
+
+  // Software pipeline.  The fragments of k-step s+1 are requested from LDS while the 16
+  // MFMAs of k-step s issue (one ds_read after each of the first 8 MFMAs), so LDS latency
+  // hides behind 512 MFMA cycles and the matrix pipe never waits for instruction issue.
+  // The workgroup barrier sits before the MFMAs of the LAST k-step of a stage: at that
+  // point the other stage has landed (vmcnt) and every wave holds its last fragments of
+  // this stage in registers, so the refill of this stage (16 buffer->LDS loads) and the
+  // first fragments of the next stage are issued underneath those MFMAs.  No branch
+  // surrounds any MFMA (a conditional stage makes the compiler shuffle all 256
+  // accumulators through VGPRs).
+  v4i fa0[4], fb0[4], fa1[4], fb1[4];
+  auto interleave_ds = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(kMfma, 8, 0);
+  };
+  auto run_stage = [&](const uint8_t* cur, uint8_t* cur_refill, const uint8_t* next, int refill_k0) {
+    load_frags(cur, 1, fa1, fb1);
+    mfma_step(fa0, fb0);
+    interleave_ds();
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(cur, 2, fa0, fb0);
+    mfma_step(fa1, fb1);
+    interleave_ds();
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(cur, 3, fa1, fb1);
+    mfma_step(fa0, fb0);
+    interleave_ds();
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
+    issue_loads(cur_refill, refill_k0);
+    load_frags(next, 0, fa0, fb0);
+    mfma_step(fa1, fb1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(kVmemRead, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(kMfma, 8, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // An odd number of 128-byte K blocks is rounded up: with KTAIL the extra block is masked
+  // to zeros; without it K is a multiple of 256 bytes and no extra block exists.  The two
+  // refills issued past the end of K are never consumed.
+  const int KT2 = (int)((g.k + 2 * BK - 1) / (2 * BK));
+  issue_loads(stage0, 0);
+  __syncthreads();
+  load_frags(stage0, 0, fa0, fb0);
+  issue_loads(stage1, BK);
+  for (int it = 0; it < KT2; ++it) {
+    run_stage(stage0, stage0, stage1, (2 * it + 2) * BK);
+    run_stage(stage1, stage1, stage0, (2 * it + 3) * BK);
   }
+  __syncthreads();  // drains the refills issued past the end
 
   // ---- epilogue ---------------------------------------------------------------
   // lane holds C[m = mrow0 + mi*32 + lr][n = ncol0 + ni*32 + 8*q + 4*lh + e], e = 0..3, reg = 4*q+e
   const int64_t mrow0 = m0 + wm * 128, ncol0 = n0 + wn * 128;
 
-  if (g.acc_out != nullptr || g.out_dtype == AQTX_I32) {
+  if (EPI == 3 || g.acc_out != nullptr) {
     int32_t* dst = g.acc_out != nullptr ? g.acc_out : reinterpret_cast<int32_t*>(g.c);
     dst += bz * g.stride_c;
 #pragma unroll
@@ -173,104 +233,121 @@ void gemm_i8_kernel(const GemmArgs g) {
           if (mm < g.m && nn < g.n) dst[mm * g.ldc + nn] = acc[mi][ni][r];
         }
     }
-    if (g.out_dtype == AQTX_I32) return;
   }
+  if constexpr (EPI != 3) {
+    constexpr bool kOutBf16 = EPI <= 1;
+    constexpr bool kDqBf16 = EPI <= 1;          // dequant dtype == output dtype
+    constexpr bool kProdBf16 = EPI == 0;        // promote(dequant dtype, scale dtype)
+    // A missing scale is a multiplication by 1, which every rounding below leaves alone.
+    const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
+    const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+    float rscale[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      const int64_t mm = mrow0 + mi * 32 + lr;
+      rscale[mi] = (rs != nullptr && mm < g.m) ? rs[mm] : 1.0f;
+    }
+    auto dequant = [&](int accv, float s_row, float s_col) {
+      float f = round_to<kDqBf16>((float)accv);  // int32 -> f32 -> dequant dtype
+      const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
+      f = round_to<kProdBf16>(f * s1);
+      f = round_to<kProdBf16>(f * s2);
+      return round_to<kDqBf16>(f);
+    };
 
-  const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
-  const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
-  const int pbf = g.dq_bf16 & g.sc_bf16;
-  float rscale[4];
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
-    const int64_t mm = mrow0 + mi * 32 + lr;
-    rscale[mi] = (rs && mm < g.m) ? rs[mm] : 1.0f;
-  }
-  auto dequant = [&](int accv, float s_row, float s_col) {
-    float f = rnd((float)accv, g.dq_bf16);
-    if (g.col_first) {
-      if (cs) f = rnd(f * s_col, pbf);
-      if (rs) f = rnd(f * s_row, pbf);
-    } else {
-      if (rs) f = rnd(f * s_row, pbf);
-      if (cs) f = rnd(f * s_col, pbf);
-    }
-    return rnd(f, g.dq_bf16);
-  };
+    // Each wave stages its 128 x 256-byte block in LDS (32 KiB, no padding): the 8-byte
+    // chunk j of row r sits at chunk j ^ (r & 31), so the 32 lanes that write one column
+    // group hit 32 distinct chunks, and a row is read back as 16 aligned 16-byte pairs.
+    uint8_t* region = (wave < 2 ? stage0 : stage1) + (wave & 1) * 32768;
+    // bf16: one pass over the 4 n-tiles (128 cols x 2 B = 256 B rows);
+    // f32 : two passes of 2 n-tiles (64 cols x 4 B = 256 B rows).
+    constexpr int kPasses = kOutBf16 ? 1 : 2;
+    constexpr int kNiPerPass = kOutBf16 ? 4 : 2;
+    constexpr int kEsz = kOutBf16 ? 2 : 4;
+    constexpr int kColsPerPair = 16 / kEsz;
+    uint8_t* cbase = reinterpret_cast<uint8_t*>(g.c) + bz * g.stride_c * kEsz;
+    const bool vec_store = ((g.ldc * kEsz) % 16) == 0 && ((uintptr_t)cbase % 16) == 0;
+    // Tiles that lie wholly inside C and can use 16-byte stores skip every bounds check.
+    const bool interior = vec_store && (m0 + BM <= g.m) && (n0 + BN <= g.n);
 
-  uint8_t* region = lds + wave * kEpiWaveBytes;
-  const bool out_bf16 = g.out_dtype == AQTX_BF16;
-  // bf16: one pass over the 4 n-tiles (128 cols x 2 B = 256 B rows);
-  // f32 : two passes of 2 n-tiles (64 cols x 4 B = 256 B rows).
-  const int npass = out_bf16 ? 1 : 2;
-  const int ni_per_pass = out_bf16 ? 4 : 2;
-  for (int pass = 0; pass < npass; ++pass) {
+    auto epilogue = [&](auto checked_tag) {
+      constexpr bool kChecked = decltype(checked_tag)::value;
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
-      if (nj >= ni_per_pass) continue;
-      // static register indexing: select the tile with a compile-time switch
+      for (int pass = 0; pass < kPasses; ++pass) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int ncol_local = nj * 32 + 8 * q + 4 * lh;  // within the pass
-        float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-        {
-          const int64_t nn = ncol0 + (pass * ni_per_pass) * 32 + ncol_local;
-          if (cs) {
+        for (int nj = 0; nj < kNiPerPass; ++nj) {
+          const int ni = pass * kNiPerPass + nj;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) csv[e] = (nn + e < g.n) ? cs[nn + e] : 1.0f;
+          for (int q = 0; q < 4; ++q) {
+            const int ncol_local = nj * 32 + 8 * q + 4 * lh;  // within the pass
+            const int64_t nn = ncol0 + ni * 32 + 8 * q + 4 * lh;
+            float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if (cs != nullptr) {
+              if constexpr (kChecked) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) csv[e] = (nn + e < g.n) ? cs[nn + e] : 1.0f;
+              } else {
+                const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
+                csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
+              }
+            }
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) {
+              float o[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = dequant(acc[mi][ni][4 * q + e], rscale[mi], csv[e]);
+              const int row = mi * 32 + lr;
+              uint8_t* p = region + row * 256;
+              if constexpr (kOutBf16) {
+                uint2 w;
+                w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+                w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+                const int j = ncol_local >> 2;  // 8-byte chunk index
+                *reinterpret_cast<uint2*>(p + ((j ^ (row & 31)) * 8)) = w;
+              } else {
+                const int j = ncol_local >> 1;  // two 8-byte chunks per 4 floats
+                *reinterpret_cast<float2*>(p + ((j ^ (row & 31)) * 8)) = make_float2(o[0], o[1]);
+                *reinterpret_cast<float2*>(p + (((j + 1) ^ (row & 31)) * 8)) = make_float2(o[2], o[3]);
+              }
+            }
           }
         }
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-          float o[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int av = (pass == 0) ? acc[mi][nj][4 * q + e]
-                                       : acc[mi][(nj + 2) & 3][4 * q + e];
-            o[e] = dequant(av, rscale[mi], csv[e]);
-          }
-          uint8_t* p = region + (mi * 32 + lr) * kEpiRowBytes;
-          if (out_bf16) {
-            uint2 w;
-            w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
-            w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
-            *reinterpret_cast<uint2*>(p + ncol_local * 2) = w;
-          } else {
-            *reinterpret_cast<float2*>(p + ncol_local * 4) = make_float2(o[0], o[1]);
-            *reinterpret_cast<float2*>(p + ncol_local * 4 + 8) = make_float2(o[2], o[3]);
+        __syncthreads();
+        // read back: lane -> 16-byte pair (lane&15) of row (lane>>4) + 4*it
+        const int64_t ncol_pass0 = ncol0 + (int64_t)pass * kNiPerPass * 32;
+        const int pair = lane & 15;
+        const int64_t nn = ncol_pass0 + pair * kColsPerPair;
+        const bool full = vec_store && (nn + kColsPerPair <= g.n);
+        uint8_t* dst0 = cbase + ((mrow0 + (lane >> 4)) * g.ldc + nn) * kEsz;
+#pragma unroll 8
+        for (int it = 0; it < 32; ++it) {
+          const int row = (lane >> 4) + 4 * it;
+          const int sw = row & 31;
+          uint4 v = *reinterpret_cast<const uint4*>(region + row * 256 + ((pair ^ (sw >> 1)) * 16));
+          if (sw & 1) v = make_uint4(v.z, v.w, v.x, v.y);
+          uint8_t* dst = dst0 + (int64_t)it * 4 * g.ldc * kEsz;
+          if constexpr (!kChecked) {
+            *reinterpret_cast<uint4*>(dst) = v;
+          } else if (mrow0 + row < g.m && nn < g.n) {
+            if (full) {
+              *reinterpret_cast<uint4*>(dst) = v;
+            } else {
+              const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+              const int nv = (int)(g.n - nn) < kColsPerPair ? (int)(g.n - nn) : kColsPerPair;
+              for (int e = 0; e < nv; ++e) {
+                if constexpr (kOutBf16)
+                  reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+                else
+                  reinterpret_cast<uint32_t*>(dst)[e] = w[e];
+              }
+            }
           }
         }
+        if (pass + 1 < kPasses) __syncthreads();
       }
-    }
-    __syncthreads();
-    // read back: lane -> 16-byte chunk (lane&15) of row (lane>>4) + 4*it
-    const int esz = out_bf16 ? 2 : 4;
-    const int cols_per_chunk = 16 / esz;
-    const int64_t ncol_pass0 = ncol0 + (int64_t)pass * ni_per_pass * 32;
-    uint8_t* cbase = reinterpret_cast<uint8_t*>(g.c) + bz * g.stride_c * esz;
-    for (int it = 0; it < 32; ++it) {
-      const int row = (lane >> 4) + 4 * it;
-      const int chunk = lane & 15;
-      const int64_t mm = mrow0 + row;
-      const int64_t nn = ncol_pass0 + chunk * cols_per_chunk;
-      const uint2 lo = *reinterpret_cast<const uint2*>(region + row * kEpiRowBytes + chunk * 16);
-      const uint2 hi = *reinterpret_cast<const uint2*>(region + row * kEpiRowBytes + chunk * 16 + 8);
-      if (mm < g.m && nn < g.n) {
-        uint8_t* dst = cbase + (mm * g.ldc + nn) * esz;
-        if (nn + cols_per_chunk <= g.n && ((g.ldc * esz) % 16) == 0) {
-          *reinterpret_cast<uint4*>(dst) = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        } else {
-          const uint32_t w[4] = {lo.x, lo.y, hi.x, hi.y};
-          const int nv = (int)(g.n - nn) < cols_per_chunk ? (int)(g.n - nn) : cols_per_chunk;
-          for (int e = 0; e < nv; ++e) {
-            if (out_bf16)
-              reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
-            else
-              reinterpret_cast<uint32_t*>(dst)[e] = w[e];
-          }
-        }
-      }
-    }
-    __syncthreads();
+    };
+    if (interior && ((uintptr_t)cs % 16) == 0) epilogue(std::false_type{});
+    else epilogue(std::true_type{});
   }
 }
 
@@ -377,10 +454,37 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
     AQTX_HIP_CHECK_LAUNCH("gemm_i8_simple_kernel");
     return 0;
   }
+  AQTX_REQUIRE(p->lda * (int64_t)BM < (1ll << 31) && p->ldb * (int64_t)BN < (1ll << 31),
+               "aqtx_gemm_i8: leading dimension too large for 32-bit tile offsets");
   g.tiles_m = (int)((p->m + BM - 1) / BM);
   g.tiles_n = (int)((p->n + BN - 1) / BN);
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
-  gemm_i8_kernel<<<grid, 256, 0, st>>>(g);
+  int epi;
+  if (p->out_dtype == AQTX_I32) {
+    epi = 3;
+  } else if (p->out_dtype == AQTX_BF16 && p->dequant_dtype == AQTX_BF16) {
+    epi = p->scale_dtype == AQTX_BF16 ? 0 : 1;
+  } else if (p->out_dtype == AQTX_F32 && p->dequant_dtype == AQTX_F32 && p->scale_dtype == AQTX_F32) {
+    epi = 2;
+  } else {
+    return set_error("aqtx_gemm_i8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
+                     p->out_dtype, p->dequant_dtype, p->scale_dtype);
+  }
+  const bool ktail = (p->k % (2 * BK)) != 0;
+#define AQTX_LAUNCH(E, C, T) gemm_i8_kernel<E, C, T><<<grid, 256, 0, st>>>(g)
+#define AQTX_LAUNCH_T(E, C) \
+  do { if (ktail) AQTX_LAUNCH(E, C, true); else AQTX_LAUNCH(E, C, false); } while (0)
+#define AQTX_LAUNCH_C(E) \
+  do { if (g.col_first) AQTX_LAUNCH_T(E, true); else AQTX_LAUNCH_T(E, false); } while (0)
+  switch (epi) {
+    case 0: AQTX_LAUNCH_C(0); break;
+    case 1: AQTX_LAUNCH_C(1); break;
+    case 2: AQTX_LAUNCH_C(2); break;
+    default: AQTX_LAUNCH_T(3, false); break;
+  }
+#undef AQTX_LAUNCH_C
+#undef AQTX_LAUNCH_T
+#undef AQTX_LAUNCH
   AQTX_HIP_CHECK_LAUNCH("gemm_i8_kernel");
   return 0;
 }
