@@ -92,10 +92,14 @@ void gemm_i8_kernel(const GemmArgs g) {
   const int64_t bz = blockIdx.y;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
-  // ---- global -> LDS: each wave instruction moves 8 rows x 128 B (1 KiB) straight into LDS.
-  // Lane l fills LDS slot (row l>>3, chunk l&7) of its block and therefore fetches the global
-  // chunk (l&7) ^ f(row), f(row) = (row ^ row>>3) & 7: that is the XOR swizzle the fragment
-  // reads undo.  Rows past the end of the operand fall outside the buffer and read as zero.
+  // ---- global -> registers -> LDS.  One wave instruction moves 8 rows x 128 B (1 KiB): lane l
+  // handles LDS slot (row l>>3, chunk l&7) of its 8-row block and fetches the global chunk
+  // (l&7) ^ f(row), f(row) = (row ^ row>>3) & 7, which is the XOR swizzle the fragment reads
+  // undo.  Rows past the end of the operand fall outside the buffer and read as zero.
+  // The loads go through registers (not buffer->LDS DMA) on purpose: a stage buffer is only
+  // free for refilling at the very end of a stage, and 64 KiB requested in one burst queue up
+  // in the CU's address unit while the waves that issued them cannot issue MFMAs.  Register
+  // staging lets the 16 loads of a wave spread over the whole stage.
   const int64_t rows_a = (g.m - m0) < BM ? (g.m - m0) : BM;
   const int64_t rows_b = (g.n - n0) < BN ? (g.n - n0) : BN;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
@@ -110,16 +114,17 @@ void gemm_i8_kernel(const GemmArgs g) {
     voff_a[i] = row * (int)g.lda + chunk_byte[i];
     voff_b[i] = row * (int)g.ldb + chunk_byte[i];
   }
-  auto issue_loads = [&](uint8_t* st, int k0) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      int va = voff_a[i], vb = voff_b[i];
-      if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) va = vb = 0x7FFFFFF0;  // out of range -> zeros
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, AQTX_LDS_PTR(st + (wave * 8 + i) * 1024), 16,
-                                               va, k0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc_b, AQTX_LDS_PTR(st + kTileBytes + (wave * 8 + i) * 1024), 16, vb, k0, 0, 0);
-    }
+  v4i stg[16];  // staging registers: stg[2*i] = A block i, stg[2*i+1] = B block i
+  auto load_global = [&](int j, int k0) {  // j = 0..15
+    const int i = j >> 1;
+    int vo = (j & 1) ? voff_b[i] : voff_a[i];
+    if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
+    stg[j] = __builtin_amdgcn_raw_buffer_load_b128((j & 1) ? rsrc_b : rsrc_a, vo, k0, 0);
+  };
+  const int st_off = wave * 8 * 1024 + lane * 16;
+  auto store_lds = [&](uint8_t* st, int j) {
+    const int i = j >> 1;
+    *reinterpret_cast<v4i*>(st + ((j & 1) ? kTileBytes : 0) + st_off + i * 1024) = stg[j];
   };
 
   // ---- per-lane swizzled fragment offsets: chunk (2*ks + lh) ^ f(row)
@@ -154,66 +159,84 @@ void gemm_i8_kernel(const GemmArgs g) {
         acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
   };
   // Scheduling groups (llvm.amdgcn.sched.group.barrier masks).
-  constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100;
+  constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100, kDsWrite = 0x200;
 
-  // Software pipeline.  The fragments of k-step s+1 are requested from LDS while the 16
-  // MFMAs of k-step s issue (one ds_read after each of the first 8 MFMAs), so LDS latency
-  // hides behind 512 MFMA cycles and the matrix pipe never waits for instruction issue.
-  // The workgroup barrier sits before the MFMAs of the LAST k-step of a stage: at that
-  // point the other stage has landed (vmcnt) and every wave holds its last fragments of
-  // this stage in registers, so the refill of this stage (16 buffer->LDS loads) and the
-  // first fragments of the next stage are issued underneath those MFMAs.  No branch
-  // surrounds any MFMA (a conditional stage makes the compiler shuffle all 256
-  // accumulators through VGPRs).
+  // Software pipeline of one stage (4 k-steps of 16 MFMAs):
+  //   k-steps 0..2: fragments of the next k-step are read from LDS (one ds_read after each of
+  //                 the first 8 MFMAs) and the 16 global loads of the block two stages ahead
+  //                 are issued one every third MFMA, into the staging registers;
+  //   barrier     : every wave holds its last fragments of this stage, the buffer is free;
+  //   k-step 3    : the staging registers are written into the freed buffer (one ds_write per
+  //                 MFMA, each waiting only for its own load) and the first fragments of the
+  //                 next stage are read from the other buffer.
+  // The barrier is a bare s_barrier: a __syncthreads() would also wait for the global loads
+  // still in flight.  No branch surrounds any MFMA (a conditional stage makes the compiler
+  // shuffle all 256 accumulators through VGPRs).
   v4i fa0[4], fb0[4], fa1[4], fb1[4];
-  auto interleave_ds = [&]() {
+  auto kstep_sched = [&](auto nloads_tag) {
+    constexpr int kLoads = decltype(nloads_tag)::value;  // 6 or 5 loads in this k-step
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+      if (i < 8) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+      if (kLoads == 6 ? (i % 3 == 0) : (i % 3 == 1)) __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(kMfma, 8, 0);
   };
   auto run_stage = [&](const uint8_t* cur, uint8_t* cur_refill, const uint8_t* next, int refill_k0) {
     load_frags(cur, 1, fa1, fb1);
+#pragma unroll
+    for (int j = 0; j < 6; ++j) load_global(j, refill_k0);
     mfma_step(fa0, fb0);
-    interleave_ds();
+    kstep_sched(std::integral_constant<int, 6>{});
     __builtin_amdgcn_sched_barrier(0);
     load_frags(cur, 2, fa0, fb0);
+#pragma unroll
+    for (int j = 6; j < 11; ++j) load_global(j, refill_k0);
     mfma_step(fa1, fb1);
-    interleave_ds();
+    kstep_sched(std::integral_constant<int, 5>{});
     __builtin_amdgcn_sched_barrier(0);
     load_frags(cur, 3, fa1, fb1);
+#pragma unroll
+    for (int j = 11; j < 16; ++j) load_global(j, refill_k0);
     mfma_step(fa0, fb0);
-    interleave_ds();
+    kstep_sched(std::integral_constant<int, 5>{});
     __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
-    issue_loads(cur_refill, refill_k0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) store_lds(cur_refill, j);
     load_frags(next, 0, fa0, fb0);
     mfma_step(fa1, fb1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(kVmemRead, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(kDsWrite, 1, 0);
+      if (i < 8) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(kMfma, 8, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
   // An odd number of 128-byte K blocks is rounded up: with KTAIL the extra block is masked
-  // to zeros; without it K is a multiple of 256 bytes and no extra block exists.  The two
-  // refills issued past the end of K are never consumed.
+  // to zeros; without it K is a multiple of 256 bytes and no extra block exists.  Blocks
+  // requested past the end of K are never consumed.
   const int KT2 = (int)((g.k + 2 * BK - 1) / (2 * BK));
-  issue_loads(stage0, 0);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) load_global(j, 0);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) store_lds(stage0, j);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) load_global(j, BK);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) store_lds(stage1, j);
   __syncthreads();
   load_frags(stage0, 0, fa0, fb0);
-  issue_loads(stage1, BK);
   for (int it = 0; it < KT2; ++it) {
     run_stage(stage0, stage0, stage1, (2 * it + 2) * BK);
     run_stage(stage1, stage1, stage0, (2 * it + 3) * BK);
   }
-  __syncthreads();  // drains the refills issued past the end
+  __syncthreads();
 
   // ---- epilogue ---------------------------------------------------------------
   // lane holds C[m = mrow0 + mi*32 + lr][n = ncol0 + ni*32 + 8*q + 4*lh + e], e = 0..3, reg = 4*q+e
