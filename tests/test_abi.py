@@ -1,0 +1,145 @@
+"""The C-ABI library: every declared symbol is exported; argument validation needs no GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from aqt_amd import _lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+  text = open(os.path.join(ROOT, 'include', 'aqtx.h')).read()
+  text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+  return sorted(set(re.findall(r'\b(aqtx_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+  lib = L.lib()
+  names = _declared_symbols()
+  assert len(names) >= 10
+  for name in names:
+    assert hasattr(lib, name), f'{name} is declared in include/aqtx.h but not exported'
+    assert name in L.SYMBOLS, f'{name} has no ctypes prototype in aqt_amd/_lib.py'
+  assert lib.aqtx_version() == 1
+
+
+def _err(status):
+  assert status != 0
+  return L.lib().aqtx_last_error().decode()
+
+
+def _qplan(**kw):
+  p = L.QuantPlan()
+  p.in_dtype = p.compute_dtype = p.scale_dtype = L.BF16
+  p.out_dtype = L.I8
+  p.batch, p.rows, p.cols = 1, 4, 64
+  p.reduce = L.REDUCE_COLS
+  p.quant_bound, p.clip_bound = 127.5, 127.0
+  for k, v in kw.items():
+    setattr(p, k, v)
+  return p
+
+
+FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: every call below fails validation first
+
+
+@pytest.mark.parametrize('kw,needle', [
+    (dict(in_dtype=L.I32), 'in_dtype'),
+    (dict(compute_dtype=L.I8), 'compute_dtype'),
+    (dict(in_dtype=L.F32), 'compute_dtype'),
+    (dict(out_dtype=L.F32), 'out_dtype'),
+    (dict(rows=-1), 'negative'),
+    (dict(reduce=7), 'reduce'),
+    (dict(group=48), 'does not divide'),
+    (dict(transpose_out=1), 'transpose_out'),
+    (dict(noise=9), 'noise'),
+    (dict(noise=L.NOISE_FP8_MANTISSA), 'fp8'),
+    (dict(out_dtype=L.E4M3, noise=L.NOISE_JAX_UNIFORM), 'integer'),
+    (dict(noise=L.NOISE_JAX_UNIFORM, noise_total=0), 'noise_total'),
+    (dict(noise=L.NOISE_JAX_UNIFORM, noise_total=1 << 33), 'noise_total'),
+    (dict(prescale=5), 'prescale'),
+    (dict(quant_bound=0.0), 'positive'),
+])
+def test_quantize_plan_validation(kw, needle):
+  lib = L.lib()
+  p = _qplan(**kw)
+  msg = _err(lib.aqtx_quantize(ctypes.byref(p), FAKE, None, FAKE, FAKE, None, 0, None))
+  assert needle in msg, msg
+
+
+def test_quantize_argument_validation():
+  lib = L.lib()
+  assert 'NULL' in _err(lib.aqtx_quantize(None, FAKE, None, FAKE, FAKE, None, 0, None))
+  p = _qplan()
+  assert 'NULL' in _err(lib.aqtx_quantize(ctypes.byref(p), None, None, FAKE, FAKE, None, 0, None))
+  p = _qplan(prescale=L.PRESCALE_PER_COL)
+  assert 'prescale' in _err(lib.aqtx_quantize(ctypes.byref(p), FAKE, None, FAKE, FAKE, None, 0, None))
+  p = _qplan(reduce=L.REDUCE_ROWS)
+  assert lib.aqtx_quantize_workspace_bytes(ctypes.byref(p)) == 64 * 8
+  assert 'workspace' in _err(lib.aqtx_quantize(ctypes.byref(p), FAKE, None, FAKE, FAKE, None, 0, None))
+  p = _qplan()
+  assert 'aligned' in _err(lib.aqtx_quantize(ctypes.byref(p), ctypes.c_void_p(0x1001), None, FAKE, FAKE, None, 0, None))
+  # empty tensors are a no-op, even without a GPU
+  p = _qplan(rows=0)
+  assert lib.aqtx_quantize(ctypes.byref(p), None, None, None, None, None, 0, None) == 0
+  assert lib.aqtx_last_error() == b''
+
+
+def _gplan(**kw):
+  p = L.GemmPlan()
+  p.batch, p.m, p.n, p.k = 1, 64, 64, 64
+  p.lda = p.ldb = p.ldc = 64
+  p.a_dtype = p.b_dtype = L.I8
+  p.out_dtype = p.dequant_dtype = p.scale_dtype = L.BF16
+  for k, v in kw.items():
+    setattr(p, k, v)
+  return p
+
+
+@pytest.mark.parametrize('kw,needle', [
+    (dict(m=-1), 'negative'),
+    (dict(a_dtype=L.F32), 'operands'),
+    (dict(out_dtype=L.I8), 'out_dtype'),
+    (dict(dequant_dtype=L.I8), 'dequant_dtype'),
+    (dict(scale_dtype=L.I32), 'scale_dtype'),
+    (dict(scale_order=3), 'scale_order'),
+    (dict(lda=32), 'leading dimension'),
+    (dict(out_dtype=L.F32, dequant_dtype=L.BF16), 'combination'),
+])
+def test_gemm_plan_validation(kw, needle):
+  p = _gplan(**kw)
+  msg = _err(L.lib().aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
+  assert needle in msg, msg
+
+
+def test_gemm_argument_validation():
+  lib = L.lib()
+  assert 'NULL' in _err(lib.aqtx_gemm_i8(None, FAKE, FAKE, None, None, FAKE, None, None))
+  p = _gplan()
+  assert 'NULL' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), None, FAKE, None, None, FAKE, None, None))
+  p = _gplan(out_dtype=L.I32)
+  assert 'no scales' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, FAKE, None, FAKE, None, None))
+  p = _gplan(m=0)
+  assert lib.aqtx_gemm_i8(ctypes.byref(p), None, None, None, None, None, None, None) == 0
+
+
+def test_prng_split_host_matches_oracle():
+  import numpy as np
+  from aqt_amd import ops
+  from oracle import prng
+  for part in (False, True):
+    for num in (1, 2, 3, 7):
+      np.testing.assert_array_equal(ops.prng_split(prng.prng_key(7), num, part),
+                                    prng.split(prng.prng_key(7), num, part))
+  assert 'NULL' in _err(L.lib().aqtx_prng_split_host(None, 2, 0, None))
+
+
+def test_cpu_tensors_are_rejected():
+  import torch
+  from aqt_amd import ops
+  x = torch.zeros((1, 4, 64), dtype=torch.bfloat16)
+  with pytest.raises(RuntimeError, match='no CPU fallback'):
+    ops.quantize(x, reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0)

@@ -1,0 +1,210 @@
+"""Host-side logic of the aqt_amd.v2 mirror (runs without a GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from aqt_amd.v2 import aqt_dot_general as aqt
+from aqt_amd.v2 import aqt_quantizer
+from aqt_amd.v2 import calibration
+from aqt_amd.v2 import config
+from aqt_amd.v2 import lowering
+from aqt_amd.v2 import stochastic_rounding
+from aqt_amd.v2 import transpose
+from aqt_amd.v2 import utils
+from aqt_amd.v2.numerics import fp8_numerics
+from aqt_amd.v2.numerics import int_numerics
+from aqt_amd.v2.numerics import no_numerics
+from oracle import aqt_ref as R
+from oracle import prng
+
+
+def test_fully_quantized_defaults():
+  """Structure pinned by the reference's config_test.py:56-270 (fully_quantized(8, 8))."""
+  cfg = config.fully_quantized(fwd_bits=8, bwd_bits=8)
+  for raw, scope in ((cfg.fwd, 'aqt_fwd'), (cfg.dlhs, 'aqt_dlhs'), (cfg.drhs, 'aqt_drhs')):
+    assert raw.jax_scope_name == scope
+    assert raw.dg_accumulator_dtype == utils.int32
+    assert raw.local_aqt is None
+    assert raw.lhs.dequant_mode == aqt.DequantMode.OUTPUT
+    assert raw.lhs.calibration_mode == aqt.CalibrationMode.CONTRACTING_AXIS
+    for q in (raw.dg_quantizer.lhs, raw.dg_quantizer.rhs):
+      n = q.numerics
+      assert isinstance(n, int_numerics.IntSymmetric)
+      assert (n.bits, n.preserve_zero, n.preserve_max_val, n.clip, n.clip_gradient, n.round) == (
+          8, True, False, True, False, True)
+      assert n.dtype == utils.int8
+      assert q.calibration is calibration.AbsMaxCalibration
+      assert q.calib_shared_axes is None and q.scale_stop_grad is True and q.scale_dtype is None
+      assert q._calibrator is None  # initialised lazily inside the forward pass
+  assert cfg.dlhs.rhs.use_fwd_quant is True and cfg.drhs.rhs.use_fwd_quant is True
+  assert cfg.fwd.rhs.use_fwd_quant is False
+  # stochastic rounding on both sides of both backward dots, none in the forward
+  assert cfg.fwd.dg_quantizer.lhs.numerics.noise_fn is None
+  for raw in (cfg.dlhs, cfg.drhs):
+    for q in (raw.dg_quantizer.lhs, raw.dg_quantizer.rhs):
+      assert isinstance(q.numerics.noise_fn, stochastic_rounding.JaxUniform)
+  assert cfg.apply_custom_vjp_on_jax is True
+
+
+def test_config_v4_defaults_and_fp8():
+  cfg = config.config_v4()
+  assert isinstance(cfg.drhs.dg_quantizer.lhs.numerics, no_numerics.NoNumerics)
+  assert cfg.drhs.dg_accumulator_dtype is None
+  assert cfg.dlhs.rhs.use_fwd_quant is False and cfg.drhs.rhs.use_fwd_quant is False
+  assert isinstance(cfg.dlhs.dg_quantizer.lhs.numerics.noise_fn, stochastic_rounding.JaxUniform)
+  assert cfg.dlhs.dg_quantizer.rhs.numerics.noise_fn is None
+  f8 = config.config_v4(fwd_bits='e4m3', dlhs_bits='e5m2', drhs_bits='e5m2')
+  n = f8.fwd.dg_quantizer.lhs.numerics
+  assert isinstance(n, fp8_numerics.Fp8Numerics) and n.dtype == utils.float8_e4m3fn
+  assert n.get_quant_bound() == 448.0 and f8.fwd.dg_accumulator_dtype == utils.float32
+  g = f8.dlhs.dg_quantizer.lhs.numerics
+  assert g.dtype == utils.float8_e5m2 and g.stochastic_rounding is True and g.get_quant_bound() == 57344.0
+  assert f8.dlhs.dg_quantizer.rhs.numerics.stochastic_rounding is False
+  fwd8 = config.config_fwd_fp8('e5m2')
+  assert isinstance(fwd8.dlhs.dg_quantizer.lhs.numerics, no_numerics.NoNumerics)
+
+
+def test_fully_quantized_sr_argument_checks():
+  with pytest.raises(AssertionError):
+    config.fully_quantized(use_stochastic_rounding=None, vjp_lhs_stochastic_rounding=True)
+  with pytest.raises(AssertionError):
+    config.fully_quantized(use_stochastic_rounding=True, vjp_lhs_stochastic_rounding=True,
+                           vjp_rhs_stochastic_rounding=False)
+  cfg = config.fully_quantized(use_stochastic_rounding=None, vjp_lhs_stochastic_rounding=True,
+                               vjp_rhs_stochastic_rounding=False)
+  assert cfg.dlhs.dg_quantizer.rhs.numerics.noise_fn is None
+
+
+def test_int_numerics_bounds_table():
+  for pz, pmv, b8 in ((False, False, 128.0), (False, True, 127.5), (True, False, 127.5), (True, True, 127.0)):
+    n = int_numerics.IntSymmetric(bits=8, preserve_zero=pz, preserve_max_val=pmv, clip=True,
+                                  clip_gradient=False, round=True, noise_fn=None, dtype=utils.int8)
+    assert n.get_quant_bound() == b8
+  n4 = config.fully_quantized(fwd_bits=4).fwd.dg_quantizer.lhs.numerics
+  assert n4.dtype is utils.int4 and n4.get_quant_bound() == 7.5 and n4._get_fwd_clip_bound() == 7.0
+
+
+@pytest.mark.parametrize('partitionable', [False, True])
+def test_set_context_key_fanout_matches_oracle(partitionable, monkeypatch):
+  monkeypatch.setattr(utils, 'threefry_partitionable', partitionable)
+  monkeypatch.setattr(R, 'PARTITIONABLE', partitionable)
+  key = prng.prng_key(42)
+  cfg = config.set_context(config.fully_quantized(), key, None)
+  ocfg = R.set_context(R.fully_quantized(), key)
+  for name in ('fwd', 'dlhs', 'drhs'):
+    raw, oraw = getattr(cfg, name), getattr(ocfg, name)
+    np.testing.assert_array_equal(raw.dg_quantizer.lhs.context.key, oraw.lhs.key)
+    np.testing.assert_array_equal(raw.dg_quantizer.rhs.context.key, oraw.rhs.key)
+  # set_context copies: the input config keeps its empty contexts
+  base = config.fully_quantized()
+  config.set_context(base, key, None)
+  assert base.fwd.dg_quantizer.lhs.context.key is None
+
+
+@pytest.mark.parametrize('dn,ls,rs', [
+    ((((1,), (0,)), ((), ())), (5, 7), (7, 3)),
+    ((((2,), (1,)), ((0,), (0,))), (2, 5, 7), (2, 7, 3)),
+    ((((2,), (0,)), ((), ())), (2, 3, 8), (8, 4, 5)),
+    ((((3, 1), (0, 2)), ((0,), (1,))), (2, 4, 5, 6), (6, 2, 4, 3)),
+])
+def test_backward_dimension_numbers_match_oracle(dn, ls, rs):
+  out_rank = len(ls) + len(rs) - 2 * len(dn[0][0]) - len(dn[1][0])
+  for y_is_lhs, y_rank in ((False, len(rs)), (True, len(ls))):
+    got = aqt._update_dimension_numbers_for_backward(dn, y_is_lhs, out_rank, y_rank)
+    want = R.bwd_dimension_numbers(dn, y_is_lhs, out_rank, y_rank)
+    assert got == want
+
+
+def test_matmul_backward_dimension_numbers():
+  dn = (((1,), (0,)), ((), ()))
+  dims, perm = aqt._update_dimension_numbers_for_backward(dn, False, 2, 2)
+  assert dims == (((1,), (1,)), ((), ())) and perm == (0, 1)
+  dims, perm = aqt._update_dimension_numbers_for_backward(dn, True, 2, 2)
+  assert dims == (((0,), (0,)), ((), ())) and perm == (1, 0)
+
+
+def test_view_operand_layouts():
+  x = torch.zeros((6, 10))
+  v = lowering.view_operand(x, [], [0], [1])
+  assert v.k_last and not v.copied and tuple(v.mem.shape) == (1, 6, 10) and v.noise_strides == (0, 10, 1)
+  v = lowering.view_operand(x, [], [1], [0])  # contraction axis strided
+  assert not v.k_last and not v.copied and tuple(v.mem.shape) == (1, 6, 10)
+  assert v.noise_strides == (0, 1, 10)
+  # a [k, n]-shaped view of an [n, k] buffer: memory order decides, noise counters follow the logical shape
+  xt = torch.zeros((10, 6)).t()
+  v = lowering.view_operand(xt, [], [0], [1])
+  assert not v.k_last and not v.copied and tuple(v.mem.shape) == (1, 10, 6)
+  assert v.noise_strides == (0, 10, 1)
+  # batched, and 'bsd,dhk' style merged axes
+  b = torch.zeros((3, 4, 5))
+  v = lowering.view_operand(b, [0], [1], [2])
+  assert v.k_last and tuple(v.mem.shape) == (3, 4, 5) and v.noise_strides == (20, 5, 1)
+  w = torch.zeros((8, 4, 5))
+  v = lowering.view_operand(w, [], [1, 2], [0])
+  assert not v.k_last and not v.copied and tuple(v.mem.shape) == (1, 8, 20)
+  # batch axis in the middle: needs the canonical copy
+  t = torch.zeros((4, 3, 5))
+  v = lowering.view_operand(t, [1], [0], [2])
+  assert v.copied and v.k_last and tuple(v.mem.shape) == (3, 4, 5)
+  assert v.noise_strides == (5, 15, 1)
+
+
+def test_scale_transposes():
+  dn = (((2,), (1,)), ((0,), (0,)))
+  ls, rs = (3, 4, 5), (3, 5, 6)
+  sl, sr = torch.zeros((3, 4, 1)), torch.zeros((3, 1, 6))
+  tl = transpose.lhs_scale_transpose_to_output(sl, dn, ls, rs)
+  tr = transpose.rhs_scale_transpose_to_output(sr, dn, ls, rs)
+  assert tuple(tl.shape) == (3, 4, 1) and tuple(tr.shape) == (3, 1, 6)
+  assert tuple(transpose.lhs_recover_scale_from_scale_t(tl, dn, ls, rs).shape) == (3, 4, 1)
+  assert tuple(transpose.rhs_recover_scale_from_scale_t(tr, dn, ls, rs).shape) == (3, 1, 6)
+  mm = (((1,), (0,)), ((), ()))
+  s = torch.arange(7.0).reshape(1, 7)
+  t = transpose.rhs_scale_transpose_for_lhs_input(s, (((1,), (1,)), ((), ())), (5, 7))
+  assert tuple(t.shape) == (1, 7)
+  t = transpose.rhs_scale_transpose_for_lhs_input(torch.zeros((5, 1)), (((0,), (0,)), ((), ())), (5, 9))
+  assert tuple(t.shape) == (5, 1)
+  assert transpose.lhs_scale_transpose_to_output(None, mm, (2, 3), (3, 4)) is None
+
+
+def test_reference_assertions_fire_before_any_kernel():
+  cfg = config.fully_quantized()
+  mm = (((1,), (0,)), ((), ()))
+  a8 = torch.zeros((4, 8), dtype=torch.int8)
+  with pytest.raises(AssertionError, match='not yet optimized to accept quantized types'):
+    cfg(a8, a8.t(), mm)
+  a = torch.zeros((4, 8), dtype=torch.bfloat16)
+  b = torch.zeros((8, 4), dtype=torch.float32)
+  with pytest.raises(AssertionError, match='Unmatched lhs and rhs dtype'):
+    cfg(a, b, mm)
+  with pytest.raises(AssertionError, match='Precision'):
+    cfg(a, a.t(), mm, precision='highest')
+  bad = config.fully_quantized()
+  bad.fwd.rhs.calibration_mode = aqt.CalibrationMode.REMAINING_AXIS
+  with pytest.raises(AssertionError):
+    bad(a, a.t().contiguous(), mm)
+  q = aqt_quantizer.quantizer_make(8)
+  with pytest.raises(AssertionError, match='second call'):
+    q.init_calibration()
+
+
+def test_no_cpu_fallback():
+  cfg = config.fully_quantized()
+  a = torch.zeros((4, 64), dtype=torch.bfloat16)
+  with pytest.raises(RuntimeError, match='no CPU fallback'):
+    cfg(a, torch.zeros((64, 8), dtype=torch.bfloat16), (((1,), (0,)), ((), ())))
+
+
+def test_einsum_dimension_numbers():
+  seen = {}
+
+  def spy(lhs, rhs, dn, precision=None, preferred_element_type=None):
+    seen['dn'] = dn
+    return aqt.lax_dot_general(lhs, rhs, dn)
+
+  x, w = torch.randn(2, 3, 8), torch.randn(8, 4, 5)
+  out = aqt.einsum('bsd,dhk->bshk', x, w, spy)
+  assert seen['dn'] == (((2,), (0,)), ((), ()))
+  torch.testing.assert_close(out, torch.einsum('bsd,dhk->bshk', x, w))
+  out = aqt.einsum('bqd,bkd->bkq', torch.randn(2, 3, 4), torch.randn(2, 5, 4), spy)
+  assert seen['dn'] == (((2,), (2,)), ((0,), (0,))) and tuple(out.shape) == (2, 5, 3)
