@@ -399,10 +399,14 @@ class DotGeneralRaw:
     return dot_general_raw_make(*args, **kwargs)
 
   # ------------------------------------------------------------------------------
-  def __call__(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers):
+  def __call__(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes=None):
     """A quantized dot_general without custom gradient (aqt_dot_general.py:757-840).
 
     Returns (out, DotGeneralRes).  `rhs` may be a MultiTensor (bwd calls).
+    `_out_transpose_axes` (this build): the caller is going to transpose the result with these
+    axes; when that transpose merely swaps the lhs-remaining and rhs-remaining groups the
+    contraction kernel writes the transposed result directly and `out` comes back already
+    transposed (and contiguous).
     """
     with torch.profiler.record_function(self.jax_scope_name):
       if isinstance(rhs, MultiTensor):
@@ -413,10 +417,10 @@ class DotGeneralRaw:
         if side.dequant_mode != DequantMode.OUTPUT or side.calibration_mode != CalibrationMode.CONTRACTING_AXIS:
           raise NotImplementedError(
               f'{name}: only DequantMode.OUTPUT with CalibrationMode.CONTRACTING_AXIS has a HIP path')
-      return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers)
+      return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes)
 
   # ------------------------------------------------------------------------------
-  def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers):
+  def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None):
     dq = self.dg_quantizer
     prescale_t = None
     if isinstance(lhs, _Prescaled):
@@ -441,6 +445,8 @@ class DotGeneralRaw:
       y = rhs_arr.to(rhs_dtype) if rhs_is_q else rhs_arr
       out = self.dot_general(x, y, dimension_numbers, None, self.dg_accumulator_dtype)
       out = out.to(dequant_dtype)
+      if out_transpose_axes is not None:
+        out = out.permute(*out_transpose_axes)
       mk = lambda t: aqt_tensor.QTensor(qvalue=t, scale=[], scale_t=None, bias=[], dequant_dtype=t.dtype)
       res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=x, qx=mk(x)), quant_grad=None),
                           rhs=TensorRes(mt=MultiTensor(x=y, qx=mk(y)), quant_grad=None))
@@ -486,16 +492,30 @@ class DotGeneralRaw:
     sdt = torch.promote_types(lsdt, rsdt)
     if self.dot_general is not lax_dot_general:
       raise NotImplementedError('a custom DotGeneralRaw.dot_general hook is not lowered')
-    out = ops.gemm(lq, rq,
-                   row_scale=expand(ls, M), col_scale=expand(rs, N), out_dtype=dequant_dtype,
-                   dequant_dtype=dequant_dtype, scale_dtype=sdt, a_dtype=lkd, b_dtype=rkd)
-    # [B, M, N] -> (batch..., lhs remaining..., rhs remaining...) in the caller's batch order
+    nb, nl, nr = len(lba), len(lra), len(rra)
     bdims = [lhs.shape[a] for a in lba]
-    out = out.reshape(bdims + [lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
+    ldims = [lhs.shape[a] for a in lra]
+    rdims = [rhs_arr.shape[a] for a in rra]
     want_lba = list(dimension_numbers[1][0])
-    if want_lba != lba:
-      perm = [lba.index(a) for a in want_lba] + list(range(len(lba), out.dim()))
-      out = out.permute(*perm)
+    swap_perm = list(range(nb)) + list(range(nb + nl, nb + nl + nr)) + list(range(nb, nb + nl))
+    swapped = (out_transpose_axes is not None and list(out_transpose_axes) == swap_perm
+               and want_lba == lba and nl > 0 and nr > 0)
+    common = dict(out_dtype=dequant_dtype, dequant_dtype=dequant_dtype, scale_dtype=sdt)
+    if swapped:
+      # C^T = rhs_q . lhs_q^T; the lhs scale still multiplies first (aqt_tensor.py:182-183)
+      out = ops.gemm(rq, lq, row_scale=expand(rs, N), col_scale=expand(ls, M), a_dtype=rkd, b_dtype=lkd,
+                     scale_order=L.SCALE_COL_THEN_ROW, **common)
+      out = out.reshape(bdims + rdims + ldims)
+    else:
+      out = ops.gemm(lq, rq, row_scale=expand(ls, M), col_scale=expand(rs, N), a_dtype=lkd, b_dtype=rkd,
+                     **common)
+      # [B, M, N] -> (batch..., lhs remaining..., rhs remaining...) in the caller's batch order
+      out = out.reshape(bdims + ldims + rdims)
+      if want_lba != lba:
+        perm = [lba.index(a) for a in want_lba] + list(range(len(lba), out.dim()))
+        out = out.permute(*perm)
+      if out_transpose_axes is not None:
+        out = out.permute(*out_transpose_axes)
 
     lhs_mt = MultiTensor(x=lhs, qx=lhs_qt_out)
     rhs_mt = MultiTensor(x=rhs_arr if not rhs_is_q else rhs.qvalue, qx=rhs_qt_out)
@@ -694,8 +714,7 @@ def dg_core_vjp_bwd(fwd_dimension_numbers, res, g):
   def grad_dot_general(y_res: TensorRes, quant_grad, dg_raw: DotGeneralRaw, y_is_lhs):
     dims, out_transpose_axes = _update_dimension_numbers_for_backward(
         fwd_dimension_numbers, y_is_lhs, g.dim(), y_res.mt.x.dim())
-    out, _ = dg_raw(g, y_res.mt, None, None, dims)
-    transposed_out = out.permute(*out_transpose_axes)
+    transposed_out, _ = dg_raw(g, y_res.mt, None, None, dims, _out_transpose_axes=out_transpose_axes)
     if quant_grad is not None:
       assert not isinstance(quant_grad, str), quant_grad
       transposed_out = quant_grad(transposed_out)[0]
