@@ -152,6 +152,70 @@ __device__ __forceinline__ uint32_t to_qbyte(float t, int out_dtype) {
   return (uint32_t)((int)rintf(t)) & 0xFFu;
 }
 
+// ---- compile-time specialisations of the element pipeline ------------------------------
+// SPEC 0: every flag is read from QArgs at run time (any dtype / numerics).
+// SPEC 1: bf16 values, bf16 scale, int8 out, round to nearest even (the forward operands).
+// SPEC 2: SPEC 1 + jax.random.uniform noise in the original threefry counter layout (the
+//         gradient-side operands).  With PAIR the two elements that share one threefry block
+//         (indices i and i + total/2) are produced by the same thread from a single block.
+template <int SPEC>
+__device__ __forceinline__ float spec_scale(float v, float inv, const QArgs& a) {
+  if constexpr (SPEC == 0) return rnd(v * inv, a.cbf & a.sbf);
+  return round_bf16(v * inv);
+}
+__device__ __forceinline__ float uniform_noise(uint32_t bits) {
+  // jax.random.uniform: mantissa bits -> [1, 2) - 1, then the centring of JaxUniform
+  float u = __uint_as_float((bits >> 9) | 0x3F800000u) - 1.0f;
+  return fmaxf(0.0f, u) - 0.5f;
+}
+template <int SPEC>
+__device__ __forceinline__ uint32_t spec_finish(float t, const QArgs& a) {
+  // clip, round half to even, cast (int_numerics.py:99-110)
+  if constexpr (SPEC == 0) {
+    t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
+    return to_qbyte(t, a.out_dtype);
+  }
+  t = fminf(fmaxf(t, -127.0f), 127.0f);
+  return (uint32_t)((int)rintf(t)) & 0xFFu;
+}
+// scale -> (noise) -> clip/round/cast for one element
+template <int SPEC>
+__device__ __forceinline__ uint32_t spec_quant(float v, float inv, uint64_t ctr, const QArgs& a) {
+  if constexpr (SPEC == 0) {
+    return to_qbyte(scaled_noisy_clipped(v, inv, ctr, a), a.out_dtype);
+  } else {
+    float t = spec_scale<SPEC>(v, inv, a);
+    if constexpr (SPEC == 2) t = round_bf16(t + uniform_noise(a.gen.word_original((uint32_t)ctr)));
+    return spec_finish<SPEC>(t, a);
+  }
+}
+// the pair (i, i + half) from one threefry block (SPEC 2, original layout, i < half)
+__device__ __forceinline__ void pair_quant(float v0, float inv0, float v1, float inv1, uint32_t i,
+                                           const QArgs& a, uint32_t& q0, uint32_t& q1) {
+  const U2 bits = threefry2x32(a.gen.k0, a.gen.k1, i, i + a.gen.half);
+  float t0 = round_bf16(v0 * inv0), t1 = round_bf16(v1 * inv1);
+  t0 = round_bf16(t0 + uniform_noise(bits.x));
+  t1 = round_bf16(t1 + uniform_noise(bits.y));
+  q0 = spec_finish<2>(t0, a);
+  q1 = spec_finish<2>(t1, a);
+}
+template <int SPEC>
+__device__ __forceinline__ float spec_prescale(float v, float ps, const QArgs& a) {
+  if constexpr (SPEC == 0) return apply_prescale(v, ps, a);
+  return round_bf16(v * round_bf16(ps));
+}
+template <int SPEC>
+__device__ __forceinline__ void spec_scale_from_absmax(float amax, const QArgs& a, float& scale, float& inv) {
+  if constexpr (SPEC == 0) {
+    scale_from_absmax(amax, a, scale, inv);
+  } else {
+    if (amax == 0.0f) amax = 1.0f;
+    scale = round_bf16(amax / a.quant_bound);
+    inv = round_bf16(1.0f / scale);
+    if (isinf(inv)) inv = 1.0f;
+  }
+}
+
 template <int LANES>
 __device__ __forceinline__ float segment_max(float v, float* smem) {
   constexpr int W = LANES < 64 ? LANES : 64;
@@ -167,74 +231,101 @@ __device__ __forceinline__ float segment_max(float v, float* smem) {
 }
 
 // ---- rows kernel: reduced axis contiguous -------------------------------------
-template <typename TIn, int LANES, int ITERS>
+// PAIR (SPEC 2 only): the block owns segment s and segment s + nseg/2, whose elements share
+// threefry blocks; requires whole rows as segments and the natural noise layout.
+template <typename TIn, int LANES, int ITERS, int SPEC, bool PAIR>
 __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
   constexpr int VEC = 8;
   constexpr int SEG_PER_BLOCK = 256 / LANES;
-  __shared__ float smem[4];
+  constexpr int NSET = PAIR ? 2 : 1;
+  __shared__ float smem[NSET][4];
   const int tid = threadIdx.x;
   const int lane = tid % LANES;
-  const int64_t seg = (int64_t)blockIdx.x * SEG_PER_BLOCK + tid / LANES;
-  const bool active = seg < a.nseg;
+  const int64_t nseg_grid = PAIR ? a.nseg / 2 : a.nseg;
+  const int64_t seg0 = (int64_t)blockIdx.x * SEG_PER_BLOCK + tid / LANES;
+  const bool active = seg0 < nseg_grid;
   const int64_t segs_per_row = a.cols / a.L;
-  const int64_t grow = active ? seg / segs_per_row : 0;  // b * rows + r
-  const int64_t col0 = active ? (seg % segs_per_row) * a.L : 0;
-  const int64_t b = grow / a.rows, r = grow % a.rows;
-  const TIn* xp = reinterpret_cast<const TIn*>(a.x) + grow * a.cols + col0;
 
-  float row_ps = 1.0f;
-  const float* psv = a.prescale + b * a.psb;
-  if (a.ps_mode == AQTX_PRESCALE_PER_ROW) row_ps = psv[r];
-
-  float v[ITERS][VEC];
-  float amax = 0.0f;
+  float v[NSET][ITERS][VEC];
+  float scale[NSET], inv[NSET];
+  int64_t grow[NSET], col0[NSET];
 #pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
-    if (active && j0 < a.L) {
-      Loader<TIn>::load8(xp + j0, v[it]);
-      if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+  for (int s = 0; s < NSET; ++s) {
+    const int64_t seg = seg0 + (int64_t)s * nseg_grid;
+    grow[s] = active ? seg / segs_per_row : 0;  // b * rows + r
+    col0[s] = active ? (seg % segs_per_row) * a.L : 0;
+    const int64_t b = grow[s] / a.rows, r = grow[s] % a.rows;
+    const TIn* xp = reinterpret_cast<const TIn*>(a.x) + grow[s] * a.cols + col0[s];
+    const float* psv = a.prescale + b * a.psb;
+    float row_ps = 1.0f;
+    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) row_ps = psv[r];
+    float amax = 0.0f;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[it][e] = apply_prescale(v[it][e], row_ps, a);
-      } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
-        const float4 p0 = *reinterpret_cast<const float4*>(psv + col0 + j0);
-        const float4 p1 = *reinterpret_cast<const float4*>(psv + col0 + j0 + 4);
-        const float ps[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+    for (int it = 0; it < ITERS; ++it) {
+      const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
+      if (active && j0 < a.L) {
+        Loader<TIn>::load8(xp + j0, v[s][it]);
+        if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[it][e] = apply_prescale(v[it][e], ps[e], a);
+          for (int e = 0; e < VEC; ++e) v[s][it][e] = spec_prescale<SPEC>(v[s][it][e], row_ps, a);
+        } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+          const float4 p0 = *reinterpret_cast<const float4*>(psv + col0[s] + j0);
+          const float4 p1 = *reinterpret_cast<const float4*>(psv + col0[s] + j0 + 4);
+          const float ps[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) v[s][it][e] = spec_prescale<SPEC>(v[s][it][e], ps[e], a);
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) amax = fmaxf(amax, fabsf(v[s][it][e]));
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[s][it][e] = 0.0f;
       }
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) amax = fmaxf(amax, fabsf(v[it][e]));
+    }
+    amax = segment_max<LANES>(amax, smem[s]);
+    if (a.scale_given) {
+      scale[s] = active ? a.scale[seg] : 1.0f;
+      inv[s] = inv_of_scale(scale[s], a);
     } else {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) v[it][e] = 0.0f;
+      spec_scale_from_absmax<SPEC>(amax, a, scale[s], inv[s]);
+      if (active && lane == 0) a.scale[seg] = scale[s];
     }
   }
-  amax = segment_max<LANES>(amax, smem);
 
-  float scale, inv;
-  if (a.scale_given) {
-    scale = active ? a.scale[seg] : 1.0f;
-    inv = inv_of_scale(scale, a);
-  } else {
-    scale_from_absmax(amax, a, scale, inv);
-    if (active && lane == 0) a.scale[seg] = scale;
-  }
-
-  uint8_t* qp = reinterpret_cast<uint8_t*>(a.q) + grow * a.cols + col0;
-  const uint64_t ctr_row = (uint64_t)(b * a.nsb + r * a.nsr + col0 * a.nsc);
+  uint8_t* qp0 = reinterpret_cast<uint8_t*>(a.q) + grow[0] * a.cols + col0[0];
+  if constexpr (PAIR) {
+    uint8_t* qp1 = reinterpret_cast<uint8_t*>(a.q) + grow[1] * a.cols + col0[1];
+    const uint32_t ctr_row = (uint32_t)(grow[0] * a.cols);  // natural layout: index of (row, 0)
 #pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
-    if (active && j0 < a.L) {
-      uint32_t w[2] = {0u, 0u};
+    for (int it = 0; it < ITERS; ++it) {
+      const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
+      if (active && j0 < a.L) {
+        uint32_t w0[2] = {0u, 0u}, w1[2] = {0u, 0u};
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float t =
-            scaled_noisy_clipped(v[it][e], inv, ctr_row + (uint64_t)((j0 + e) * a.nsc), a);
-        w[e >> 2] |= to_qbyte(t, a.out_dtype) << (8 * (e & 3));
+        for (int e = 0; e < VEC; ++e) {
+          uint32_t q0, q1;
+          pair_quant(v[0][it][e], inv[0], v[1][it][e], inv[1], ctr_row + (uint32_t)(j0 + e), a, q0, q1);
+          w0[e >> 2] |= q0 << (8 * (e & 3));
+          w1[e >> 2] |= q1 << (8 * (e & 3));
+        }
+        *reinterpret_cast<uint2*>(qp0 + j0) = make_uint2(w0[0], w0[1]);
+        *reinterpret_cast<uint2*>(qp1 + j0) = make_uint2(w1[0], w1[1]);
       }
-      *reinterpret_cast<uint2*>(qp + j0) = make_uint2(w[0], w[1]);
+    }
+  } else {
+    const int64_t b = grow[0] / a.rows, r = grow[0] % a.rows;
+    const uint64_t ctr_row = (uint64_t)(b * a.nsb + r * a.nsr + col0[0] * a.nsc);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
+      if (active && j0 < a.L) {
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          w[e >> 2] |= spec_quant<SPEC>(v[0][it][e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a)
+                       << (8 * (e & 3));
+        *reinterpret_cast<uint2*>(qp0 + j0) = make_uint2(w[0], w[1]);
+      }
     }
   }
 }
@@ -375,83 +466,128 @@ __global__ void finalize_scales_kernel(const QArgs a, int64_t n) {
 constexpr int kTileR = 128, kTileC = 64, kTilePad = 132;
 
 // 128x64 tile: thread (rg = tid/8, cc = tid%8) owns rows 4*rg..+3, cols 8*cc..+7.
-template <typename TIn>
+// PAIR (SPEC 2 only): 1 = the block also owns the tile `rows/2` further down (natural noise
+// layout), 2 = the tile `cols/2` further right (noise counters of the transposed tensor); the
+// two tiles' elements share threefry blocks.
+template <typename TIn, int SPEC, int PAIR>
 __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a) {
-  __shared__ uint32_t lds[kTileC * kTilePad / 4];
+  constexpr int NSET = PAIR ? 2 : 1;
+  __shared__ uint32_t lds[NSET][kTileC * kTilePad / 4];
   const int tid = threadIdx.x;
   const int cc = tid & 7, rg = tid >> 3;
   const int64_t b = blockIdx.z;
-  const int64_t r0 = (int64_t)blockIdx.y * kTileR, c0 = (int64_t)blockIdx.x * kTileC;
   const TIn* xb = reinterpret_cast<const TIn*>(a.x) + b * a.rows * a.cols;
   uint8_t* qb = reinterpret_cast<uint8_t*>(a.q) + b * a.rows * a.cols;
   const bool vec_ok = (a.cols % 8) == 0;
-  const int64_t c = c0 + cc * 8;
+  int64_t r0[NSET], c0[NSET];
+  r0[0] = (int64_t)blockIdx.y * kTileR;
+  c0[0] = (int64_t)blockIdx.x * kTileC;
+  // the first tile of a pair stays inside the first half of the paired axis
+  const int64_t row_lim = PAIR == 1 ? a.rows / 2 : a.rows;
+  const int64_t col_lim = PAIR == 2 ? a.cols / 2 : a.cols;
+  if constexpr (PAIR == 1) { r0[1] = r0[0] + a.rows / 2; c0[1] = c0[0]; }
+  if constexpr (PAIR == 2) { r0[1] = r0[0]; c0[1] = c0[0] + a.cols / 2; }
 
-  uint32_t packed[8];  // packed[e] = bytes of rows 4*rg..4*rg+3 at col c+e
+  uint32_t packed[NSET][8];  // packed[s][e] = bytes of rows 4*rg..4*rg+3 at col c+e
 #pragma unroll
-  for (int e = 0; e < 8; ++e) packed[e] = 0u;
+  for (int s = 0; s < NSET; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) packed[s][e] = 0u;
 
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int64_t r = r0 + rg * 4 + j;
-    if (r < a.rows && c < a.cols) {
-      float v[8];
-      const int nvalid = (a.cols - c) >= 8 ? 8 : (int)(a.cols - c);
-      if (vec_ok) {
-        Loader<TIn>::load8(xb + r * a.cols + c, v);
-      } else {
+    const int64_t rl = r0[0] + rg * 4 + j;  // position inside the first tile's half
+    const int64_t cl = c0[0] + cc * 8;
+    if (rl < row_lim && cl < col_lim) {
+      const int nvalid = (col_lim - cl) >= 8 ? 8 : (int)(col_lim - cl);
+      float x[NSET][8], inv[NSET][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          v[e] = e < nvalid ? Loader<TIn>::load1(xb + r * a.cols + c + e) : 0.0f;
+      for (int s = 0; s < NSET; ++s) {
+        const int64_t r = r0[s] + rg * 4 + j, c = c0[s] + cc * 8;
+        if (vec_ok) {
+          Loader<TIn>::load8(xb + r * a.cols + c, x[s]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            x[s][e] = e < nvalid ? Loader<TIn>::load1(xb + r * a.cols + c + e) : 0.0f;
+        }
+        const int64_t sbase = b * a.ssb + (r / a.G) * a.ssg;
+        if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+          const float rp = a.prescale[b * a.psb + r];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[s][e] = spec_prescale<SPEC>(x[s][e], rp, a);
+        } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e < nvalid) x[s][e] = spec_prescale<SPEC>(x[s][e], a.prescale[b * a.psb + c + e], a);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) inv[s][e] = e < nvalid ? a.ws_inv[sbase + (c + e) * a.ssc] : 1.0f;
       }
-      const int64_t sbase = b * a.ssb + (r / a.G) * a.ssg;
-      const float rp = (a.ps_mode == AQTX_PRESCALE_PER_ROW) ? a.prescale[b * a.psb + r] : 1.0f;
-      uint32_t w[2] = {0u, 0u};
+      uint32_t w[NSET][2];
+#pragma unroll
+      for (int s = 0; s < NSET; ++s) w[s][0] = w[s][1] = 0u;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (e < nvalid) {
-          float x = v[e];
-          if (a.ps_mode == AQTX_PRESCALE_PER_ROW) x = apply_prescale(x, rp, a);
-          else if (a.ps_mode == AQTX_PRESCALE_PER_COL) x = apply_prescale(x, a.prescale[b * a.psb + c + e], a);
-          const float inv = a.ws_inv[sbase + (c + e) * a.ssc];
-          const uint64_t ctr = (uint64_t)(b * a.nsb + r * a.nsr + (c + e) * a.nsc);
-          const uint32_t qv = to_qbyte(scaled_noisy_clipped(x, inv, ctr, a), a.out_dtype);
-          w[e >> 2] |= qv << (8 * (e & 3));
-          packed[e] |= qv << (8 * j);
+          uint32_t qv[NSET];
+          if constexpr (PAIR) {
+            const uint32_t i = (uint32_t)((r0[0] + rg * 4 + j) * a.nsr + (c0[0] + cc * 8 + e) * a.nsc);
+            pair_quant(x[0][e], inv[0][e], x[1][e], inv[1][e], i, a, qv[0], qv[1]);
+          } else {
+            const uint64_t ctr = (uint64_t)(b * a.nsb + rl * a.nsr + (cl + e) * a.nsc);
+            qv[0] = spec_quant<SPEC>(x[0][e], inv[0][e], ctr, a);
+          }
+#pragma unroll
+          for (int s = 0; s < NSET; ++s) {
+            w[s][e >> 2] |= qv[s] << (8 * (e & 3));
+            packed[s][e] |= qv[s] << (8 * j);
+          }
         }
       }
       if (!a.transpose_out) {
-        if (vec_ok) {
-          *reinterpret_cast<uint2*>(qb + r * a.cols + c) = make_uint2(w[0], w[1]);
-        } else {
-          for (int e = 0; e < nvalid; ++e)
-            qb[r * a.cols + c + e] = (uint8_t)(w[e >> 2] >> (8 * (e & 3)));
+#pragma unroll
+        for (int s = 0; s < NSET; ++s) {
+          const int64_t r = r0[s] + rg * 4 + j, c = c0[s] + cc * 8;
+          if (vec_ok) {
+            *reinterpret_cast<uint2*>(qb + r * a.cols + c) = make_uint2(w[s][0], w[s][1]);
+          } else {
+            for (int e = 0; e < nvalid; ++e)
+              qb[r * a.cols + c + e] = (uint8_t)(w[s][e >> 2] >> (8 * (e & 3)));
+          }
         }
       }
     }
   }
   if (!a.transpose_out) return;  // uniform across the block
 
-  // Transposed write: LDS holds the tile as [col][row bytes], row stride 132 B.
+  // Transposed write: LDS holds each tile as [col][row bytes], row stride 132 B.
 #pragma unroll
-  for (int e = 0; e < 8; ++e) lds[((cc * 8 + e) * kTilePad + rg * 4) / 4] = packed[e];
+  for (int s = 0; s < NSET; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) lds[s][((cc * 8 + e) * kTilePad + rg * 4) / 4] = packed[s][e];
   __syncthreads();
   // thread -> (col = tid/8 + 32*h, 16-byte chunk = tid%8) of the [64][128] byte tile
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int col = (tid >> 3) + 32 * h;
-    const int chunk = tid & 7;
-    const int64_t gc = c0 + col, gr = r0 + chunk * 16;
-    if (gc < a.cols && gr < a.rows) {
-      uint32_t w[4];
+  for (int s = 0; s < NSET; ++s) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w[i] = lds[(col * kTilePad + chunk * 16) / 4 + i];
-      uint8_t* dst = qb + gc * a.rows + gr;
-      if ((a.rows % 16) == 0) {
-        *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
-      } else {
-        const int nv = (a.rows - gr) >= 16 ? 16 : (int)(a.rows - gr);
-        for (int i = 0; i < nv; ++i) dst[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+    for (int h = 0; h < 2; ++h) {
+      const int col = (tid >> 3) + 32 * h;
+      const int chunk = tid & 7;
+      const int64_t gc_l = c0[0] + col, gr_l = r0[0] + chunk * 16;  // bounds in first-tile terms
+      const int64_t gc = c0[s] + col, gr = r0[s] + chunk * 16;
+      if (gc_l < col_lim && gr_l < row_lim) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = lds[s][(col * kTilePad + chunk * 16) / 4 + i];
+        uint8_t* dst = qb + gc * a.rows + gr;
+        const int64_t lim = row_lim - gr_l;
+        if ((a.rows % 16) == 0 && (PAIR != 1 || ((a.rows / 2) % 16) == 0)) {
+          *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+          const int nv = lim >= 16 ? 16 : (int)lim;
+          for (int i = 0; i < nv; ++i) dst[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+        }
       }
     }
   }
@@ -551,22 +687,25 @@ int noise_width(const aqtx_quant_plan* p) {
   return 32;
 }
 
-template <typename TIn>
-int launch_rows(const QArgs& a, hipStream_t st) {
+// Which compile-time specialisation (see spec_quant) serves this plan.
+int spec_of(const QArgs& a, int partitionable) {
+  if (!(a.cbf && a.sbf && a.out_dtype == AQTX_I8 && !a.scale_given)) return 0;
+  if (a.quant_bound != 127.5f || a.clip_bound != 127.0f) return 0;
+  if (a.noise == AQTX_NOISE_NONE) return 1;
+  if (a.noise == AQTX_NOISE_JAX_UNIFORM && !partitionable) return 2;
+  return 0;
+}
+
+template <typename TIn, int SPEC, bool PAIR>
+int launch_rows_spec(const QArgs& a, hipStream_t st) {
   const int64_t L = a.L;
-  const bool aligned = (L % 8 == 0) && (a.cols % 8 == 0);
-  if (!aligned || L > 16384) {
-    const int64_t blocks = (a.nseg + 3) / 4;
-    quant_rows_generic_kernel<TIn><<<dim3((unsigned)blocks), 256, 0, st>>>(a);
-    AQTX_HIP_CHECK_LAUNCH("quant_rows_generic_kernel");
-    return 0;
-  }
-#define AQTX_ROWS(LANES, ITERS)                                                      \
-  {                                                                                  \
-    const int64_t blocks = (a.nseg + (256 / LANES) - 1) / (256 / LANES);             \
-    quant_rows_kernel<TIn, LANES, ITERS><<<dim3((unsigned)blocks), 256, 0, st>>>(a); \
-    AQTX_HIP_CHECK_LAUNCH("quant_rows_kernel");                                      \
-    return 0;                                                                        \
+  const int64_t nseg = PAIR ? a.nseg / 2 : a.nseg;
+#define AQTX_ROWS(LANES, ITERS)                                                        \
+  {                                                                                    \
+    const int64_t blocks = (nseg + (256 / LANES) - 1) / (256 / LANES);                 \
+    quant_rows_kernel<TIn, LANES, ITERS, SPEC, PAIR><<<dim3((unsigned)blocks), 256, 0, st>>>(a); \
+    AQTX_HIP_CHECK_LAUNCH("quant_rows_kernel");                                        \
+    return 0;                                                                          \
   }
   if (L <= 128) AQTX_ROWS(16, 1)
   if (L <= 512) AQTX_ROWS(64, 1)
@@ -578,7 +717,30 @@ int launch_rows(const QArgs& a, hipStream_t st) {
 }
 
 template <typename TIn>
-int launch_tiles(const QArgs& a, int reduce, int64_t nscales, hipStream_t st) {
+int launch_rows(const QArgs& a, int partitionable, hipStream_t st) {
+  const int64_t L = a.L;
+  const bool aligned = (L % 8 == 0) && (a.cols % 8 == 0);
+  if (!aligned || L > 16384) {
+    const int64_t blocks = (a.nseg + 3) / 4;
+    quant_rows_generic_kernel<TIn><<<dim3((unsigned)blocks), 256, 0, st>>>(a);
+    AQTX_HIP_CHECK_LAUNCH("quant_rows_generic_kernel");
+    return 0;
+  }
+  const int spec = spec_of(a, partitionable);
+  if (spec == 1) return launch_rows_spec<TIn, 1, false>(a, st);
+  if (spec == 2) {
+    // one threefry block serves elements i and i + total/2: pair whole rows when the noise
+    // counters follow the natural [batch*rows, cols] order
+    const bool natural = a.nsc == 1 && a.nsr == a.cols && (a.batch == 1 || a.nsb == a.rows * a.cols) &&
+                         L == a.cols && (a.nseg % 2 == 0);
+    if (natural) return launch_rows_spec<TIn, 2, true>(a, st);
+    return launch_rows_spec<TIn, 2, false>(a, st);
+  }
+  return launch_rows_spec<TIn, 0, false>(a, st);
+}
+
+template <typename TIn>
+int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales, hipStream_t st) {
   if (!a.scale_given) {
     fill_u32_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a.ws_absmax, nscales, 0u);
     AQTX_HIP_CHECK_LAUNCH("fill_u32_kernel");
@@ -602,17 +764,33 @@ int launch_tiles(const QArgs& a, int reduce, int64_t nscales, hipStream_t st) {
   }
   finalize_scales_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a, nscales);
   AQTX_HIP_CHECK_LAUNCH("finalize_scales_kernel");
-  dim3 grid((unsigned)((a.cols + kTileC - 1) / kTileC), (unsigned)((a.rows + kTileR - 1) / kTileR),
-            (unsigned)a.batch);
-  quant_tile_kernel<TIn><<<grid, 256, 0, st>>>(a);
+  const int spec = spec_of(a, partitionable);
+  auto grid_for = [&](int pair) {
+    const int64_t rows = pair == 1 ? a.rows / 2 : a.rows, cols = pair == 2 ? a.cols / 2 : a.cols;
+    return dim3((unsigned)((cols + kTileC - 1) / kTileC), (unsigned)((rows + kTileR - 1) / kTileR),
+                (unsigned)a.batch);
+  };
+  if (spec == 1) {
+    quant_tile_kernel<TIn, 1, 0><<<grid_for(0), 256, 0, st>>>(a);
+  } else if (spec == 2) {
+    // pair the two elements of each threefry block: i and i + total/2 lie rows/2 apart when the
+    // noise counters are row-major over [rows, cols], cols/2 apart when over [cols, rows]
+    const bool natural = a.batch == 1 && a.nsc == 1 && a.nsr == a.cols && (a.rows % 2 == 0);
+    const bool transposed = a.batch == 1 && a.nsr == 1 && a.nsc == a.rows && (a.cols % 16 == 0);
+    if (natural) quant_tile_kernel<TIn, 2, 1><<<grid_for(1), 256, 0, st>>>(a);
+    else if (transposed) quant_tile_kernel<TIn, 2, 2><<<grid_for(2), 256, 0, st>>>(a);
+    else quant_tile_kernel<TIn, 2, 0><<<grid_for(0), 256, 0, st>>>(a);
+  } else {
+    quant_tile_kernel<TIn, 0, 0><<<grid_for(0), 256, 0, st>>>(a);
+  }
   AQTX_HIP_CHECK_LAUNCH("quant_tile_kernel");
   return 0;
 }
 
 template <typename TIn>
-int dispatch(const QArgs& a, int reduce, int64_t nscales, hipStream_t st) {
-  if (reduce == AQTX_REDUCE_COLS) return launch_rows<TIn>(a, st);
-  return launch_tiles<TIn>(a, reduce, nscales, st);
+int dispatch(const QArgs& a, int reduce, int partitionable, int64_t nscales, hipStream_t st) {
+  if (reduce == AQTX_REDUCE_COLS) return launch_rows<TIn>(a, partitionable, st);
+  return launch_tiles<TIn>(a, reduce, partitionable, nscales, st);
 }
 
 }  // namespace
@@ -682,9 +860,9 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
                  "aqtx_quantize: too many rows for one launch (%lld)", (long long)p->rows);
   }
   switch (p->in_dtype) {
-    case AQTX_F32: return dispatch<float>(a, p->reduce, nscales, st);
-    case AQTX_BF16: return dispatch<uint16_t>(a, p->reduce, nscales, st);
-    default: return dispatch<int8_t>(a, p->reduce, nscales, st);
+    case AQTX_F32: return dispatch<float>(a, p->reduce, p->partitionable, nscales, st);
+    case AQTX_BF16: return dispatch<uint16_t>(a, p->reduce, p->partitionable, nscales, st);
+    default: return dispatch<int8_t>(a, p->reduce, p->partitionable, nscales, st);
   }
 }
 
