@@ -1,0 +1,521 @@
+// Tiled MFMA contraction with the dequantisation fused in the epilogue, shared by the
+// int8 and the fp8 entry points (the element type only changes the MFMA instruction,
+// the fragment width and the accumulator type).
+//
+// C[m, n] = dequant( sum_k A[m, k] * B[n, k] ): both operands carry the
+// contraction axis contiguously (the quantize kernels write whichever layout the
+// consumer needs), so every lane feeds the MFMA with 16 (int8) or 32 (fp8)
+// contiguous bytes per operand.
+//
+// Tiling: one workgroup (4 waves, 2x2) owns a 256x256 tile of C; a wave owns
+// 128x128 = 4x4 MFMA tiles (256 accumulator registers).  K advances 128 bytes per
+// stage; two LDS stages of (256+256) rows x 128 B are filled from registers while
+// the MFMAs of the other stage run.  Rows are 128 B apart in LDS, so the 16-byte
+// chunk index is XOR-swizzled with (row ^ row>>3) & 7: the 16-lane groups of a
+// ds_read_b128/ds_write_b128 then touch 64 distinct banks.
+//
+// The MFMA "A" operand is fed from the B tile and vice versa, so a lane ends up
+// holding 4 consecutive n for one m; the epilogue converts, scales, packs these
+// and sends them through LDS to leave as full 256-byte row segments.
+#pragma once
+#include <type_traits>
+
+#include "common.h"
+
+namespace aqtx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// Element traits.  `mma(x, y, c)` computes c += x * y^T for two 32-row fragments; a fragment
+// holds kChunks 16-byte chunks per lane (lane>>5 selects the k half inside one MFMA).
+struct MmaI8 {
+  using Acc = v16i;
+  using AccScalar = int32_t;
+  using Frag = v4i;
+  static constexpr int kChunks = 1;   // v_mfma_i32_32x32x32_i8: 32 k per MFMA, 16 per lane
+  static constexpr bool kIntAcc = true;
+  static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float decode(uint8_t v) { return (float)(int8_t)v; }
+};
+
+// FMT_A / FMT_B: 0 = e4m3fn, 1 = e5m2 for the operand holding the rows of C (A) and the
+// columns of C (B).  v_mfma_scale_f32_32x32x64_f8f6f4 with both block scales at 2^0.
+template <int FMT_A, int FMT_B>
+struct MmaF8 {
+  using Acc = v16f;
+  using AccScalar = float;
+  using Frag = v8i;
+  static constexpr int kChunks = 2;   // 64 k per MFMA, 32 per lane
+  static constexpr bool kIntAcc = false;
+  // x comes from the B tile, y from the A tile (see mfma_step).  Zero scale operands select the
+  // unscaled form of the instruction (v_mfma_f32_32x32x64_f8f6f4).
+  static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, FMT_B, FMT_A, 0, 0, 0, 0);
+  }
+};
+
+struct GemmArgs {
+  const uint8_t* a;
+  const uint8_t* b;
+  const float* row_scale;
+  const float* col_scale;
+  void* c;
+  void* acc_out;   // int32 (int8 operands) or float (fp8 operands)
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc;
+  int64_t stride_a, stride_b, stride_c, stride_rs, stride_cs;
+  int tiles_m, tiles_n;
+  int out_dtype;  // AQTX_BF16 | AQTX_F32 | AQTX_I32
+  int dq_bf16;    // dequant dtype is bf16
+  int sc_bf16;    // scale dtype is bf16
+  int col_first;  // scale order
+};
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int kTileBytes = BM * BK;          // one operand tile of one stage: 32 KiB
+constexpr int kStageBytes = 2 * kTileBytes;  // A tile + B tile
+constexpr uint32_t kBufferRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format (gfx9)
+
+#define AQTX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+__device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
+
+// Workgroup id -> tile, XCD-aware: ids are dealt round-robin to the 8 XCDs, so id%8
+// picks the XCD; each XCD then walks a contiguous range of tiles in bands of 8 tile
+// rows, keeping the operand panels of concurrently running tiles in its own L2.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (total + 7) / 8;
+  int id = (bid % 8) * per_xcd + bid / 8;
+  if (total % 8 != 0) id = bid;  // uneven split: keep the plain order
+  constexpr int kBand = 8;
+  const int band_tiles = kBand * tiles_n;
+  const int band = id / band_tiles;
+  const int first_m = band * kBand;
+  const int rows_in_band = (tiles_m - first_m) < kBand ? (tiles_m - first_m) : kBand;
+  const int in_band = id % band_tiles;
+  tm = first_m + in_band % rows_in_band;
+  tn = in_band / rows_in_band;
+}
+
+// EPI selects the epilogue arithmetic at compile time (run-time flags there turn into
+// thousands of branches): 0 = bf16 out, bf16 scales; 1 = bf16 out, f32 scales; 2 = f32 out,
+// f32 scales; 3 = raw int32 accumulators only.  COL_FIRST: the column scale multiplies first.
+// KTAIL: K is not a multiple of the 128-byte stage, the last stage masks chunks past K.
+template <class MMA, int EPI, bool COL_FIRST, bool KTAIL>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_kernel(const GemmArgs g) {
+  using Acc = typename MMA::Acc;
+  using AccScalar = typename MMA::AccScalar;
+  using Frag = typename MMA::Frag;
+  constexpr int kChunks = MMA::kChunks;
+  constexpr int KS = 4 / kChunks;  // k-steps (rounds of 16 MFMAs) per 128-byte stage
+  // Two stages in two distinct LDS objects, so that the compiler can tell the stage
+  // being filled by the buffer->LDS loads from the one the MFMA fragments are read from.
+  __shared__ __attribute__((aligned(1024))) uint8_t stage0[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t stage1[kStageBytes];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 31, lh = lane >> 5;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const int64_t bz = blockIdx.y;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+  // ---- global -> registers -> LDS.  One wave instruction moves 8 rows x 128 B (1 KiB): lane l
+  // handles LDS slot (row l>>3, chunk l&7) of its 8-row block and fetches the global chunk
+  // (l&7) ^ f(row), f(row) = (row ^ row>>3) & 7, which is the XOR swizzle the fragment reads
+  // undo.  Rows past the end of the operand fall outside the buffer and read as zero.
+  // The loads go through registers (not buffer->LDS DMA) on purpose: a stage buffer is only
+  // free for refilling at the very end of a stage, and 64 KiB requested in one burst queue up
+  // in the CU's address unit while the waves that issued them cannot issue MFMAs.  Register
+  // staging lets the 16 loads of a wave spread over the whole stage.
+  const int64_t rows_a = (g.m - m0) < BM ? (g.m - m0) : BM;
+  const int64_t rows_b = (g.n - n0) < BN ? (g.n - n0) : BN;
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + g.k), kBufferRsrcWord3);
+  int voff_a[8], voff_b[8], chunk_byte[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = (wave * 8 + i) * 8 + (lane >> 3);
+    chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ i) & 7) * 16;
+    voff_a[i] = row * (int)g.lda + chunk_byte[i];
+    voff_b[i] = row * (int)g.ldb + chunk_byte[i];
+  }
+  v4i stg[16];  // staging registers: stg[2*i] = A block i, stg[2*i+1] = B block i
+  auto load_global = [&](int j, int k0) {  // j = 0..15
+    const int i = j >> 1;
+    int vo = (j & 1) ? voff_b[i] : voff_a[i];
+    if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
+    stg[j] = __builtin_amdgcn_raw_buffer_load_b128((j & 1) ? rsrc_b : rsrc_a, vo, k0, 0);
+  };
+  const int st_off = wave * 8 * 1024 + lane * 16;
+  auto store_lds = [&](uint8_t* st, int j) {
+    const int i = j >> 1;
+    *reinterpret_cast<v4i*>(st + ((j & 1) ? kTileBytes : 0) + st_off + i * 1024) = stg[j];
+  };
+
+  // ---- per-lane swizzled fragment offsets: chunk ((2*ks + lh) * kChunks + c) ^ f(row)
+  const int lf0 = (lr ^ (lr >> 3)) & 7;
+  int frag_off[8];
+#pragma unroll
+  for (int cidx = 0; cidx < 8; ++cidx)
+    frag_off[cidx] = lr * BK + (((lh * kChunks) ^ lf0 ^ cidx) * 16);
+  const int a_base = wm * 128 * BK;                // rows of the A tile this wave needs
+  const int b_base = kTileBytes + wn * 128 * BK;   // rows of the B tile
+
+  Acc acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  auto load_frags = [&](const uint8_t* st, int ks, Frag* fa, Frag* fb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (kChunks == 1) {
+        const int cidx = (2 * ks) ^ (4 * (i & 1));
+        fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[cidx]);
+        fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[cidx]);
+      } else {
+        const int c0 = (4 * ks) ^ (4 * (i & 1)), c1 = c0 ^ 1;
+        const v4i a0 = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[c0]);
+        const v4i a1 = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[c1]);
+        const v4i b0 = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c0]);
+        const v4i b1 = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c1]);
+        fa[i] = Frag{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+        fb[i] = Frag{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      }
+    }
+  };
+  auto mfma_step = [&](const Frag* fa, const Frag* fb) {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = MMA::mma(fb[ni], fa[mi], acc[mi][ni]);
+  };
+  // Scheduling groups (llvm.amdgcn.sched.group.barrier masks).
+  constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100, kDsWrite = 0x200;
+
+  // Software pipeline of one stage (KS k-steps of 16 MFMAs):
+  //   k-steps 0..KS-2: fragments of the next k-step are read from LDS (spread over the MFMAs)
+  //                 and the 16 global loads of the block two stages ahead are issued a few
+  //                 MFMAs apart, into the staging registers;
+  //   barrier     : every wave holds its last fragments of this stage, the buffer is free;
+  //   last k-step : the staging registers are written into the freed buffer (one ds_write per
+  //                 MFMA, each waiting only for its own load) and the first fragments of the
+  //                 next stage are read from the other buffer.
+  // The barrier is a bare s_barrier: a __syncthreads() would also wait for the global loads
+  // still in flight.  No branch surrounds any MFMA (a conditional stage makes the compiler
+  // shuffle all 256 accumulators through VGPRs).
+  Frag fa0[4], fb0[4], fa1[4], fb1[4];
+  constexpr int kDsPerStep = 8 * kChunks;  // ds_read_b128 per k-step
+  auto run_stage = [&](const uint8_t* cur, uint8_t* cur_refill, const uint8_t* next, int refill_k0) {
+#pragma unroll
+    for (int ks = 0; ks < KS - 1; ++ks) {
+      // loads [l0, l1) of the 16 go with this k-step
+      const int l0 = (16 * ks + KS - 2) / (KS - 1), l1 = (16 * (ks + 1) + KS - 2) / (KS - 1);
+      if (ks % 2 == 0) load_frags(cur, ks + 1, fa1, fb1); else load_frags(cur, ks + 1, fa0, fb0);
+#pragma unroll
+      for (int j = l0; j < l1; ++j) load_global(j, refill_k0);
+      if (ks % 2 == 0) mfma_step(fa0, fb0); else mfma_step(fa1, fb1);
+      const int nl = l1 - l0;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+        if (i < kDsPerStep) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+        if (nl == 16 || (nl == 6 ? (i % 3 == 0) : (i % 3 == 1)))
+          __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) store_lds(cur_refill, j);
+    // KS is even, so the last k-step always computes from set 1 and refills set 0.
+    load_frags(next, 0, fa0, fb0);
+    mfma_step(fa1, fb1);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(kDsWrite, 1, 0);
+      if (i < kDsPerStep) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // An odd number of 128-byte K blocks is rounded up: with KTAIL the extra block is masked
+  // to zeros; without it K is a multiple of 256 bytes and no extra block exists.  Blocks
+  // requested past the end of K are never consumed.
+  const int KT2 = (int)((g.k + 2 * BK - 1) / (2 * BK));
+#pragma unroll
+  for (int j = 0; j < 16; ++j) load_global(j, 0);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) store_lds(stage0, j);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) load_global(j, BK);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) store_lds(stage1, j);
+  __syncthreads();
+  load_frags(stage0, 0, fa0, fb0);
+  for (int it = 0; it < KT2; ++it) {
+    run_stage(stage0, stage0, stage1, (2 * it + 2) * BK);
+    run_stage(stage1, stage1, stage0, (2 * it + 3) * BK);
+  }
+  __syncthreads();
+
+  // ---- epilogue ---------------------------------------------------------------
+  // lane holds C[m = mrow0 + mi*32 + lr][n = ncol0 + ni*32 + 8*q + 4*lh + e], e = 0..3, reg = 4*q+e
+  const int64_t mrow0 = m0 + wm * 128, ncol0 = n0 + wn * 128;
+
+  if (EPI == 3 || g.acc_out != nullptr) {
+    AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out != nullptr ? g.acc_out : g.c);
+    dst += bz * g.stride_c;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      const int64_t mm = mrow0 + mi * 32 + lr;
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t nn = ncol0 + ni * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (mm < g.m && nn < g.n) dst[mm * g.ldc + nn] = acc[mi][ni][r];
+        }
+    }
+  }
+  if constexpr (EPI != 3) {
+    constexpr bool kOutBf16 = EPI <= 1;
+    constexpr bool kDqBf16 = EPI <= 1;          // dequant dtype == output dtype
+    constexpr bool kProdBf16 = EPI == 0;        // promote(dequant dtype, scale dtype)
+    // A missing scale is a multiplication by 1, which every rounding below leaves alone.
+    const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
+    const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+    float rscale[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      const int64_t mm = mrow0 + mi * 32 + lr;
+      rscale[mi] = (rs != nullptr && mm < g.m) ? rs[mm] : 1.0f;
+    }
+    auto dequant = [&](AccScalar accv, float s_row, float s_col) {
+      float f = round_to<kDqBf16>((float)accv);  // (int32 ->) f32 -> dequant dtype
+      const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
+      f = round_to<kProdBf16>(f * s1);
+      f = round_to<kProdBf16>(f * s2);
+      return round_to<kDqBf16>(f);
+    };
+
+    // Each wave stages its 128 x 256-byte block in LDS (32 KiB, no padding): the 8-byte
+    // chunk j of row r sits at chunk j ^ (r & 31), so the 32 lanes that write one column
+    // group hit 32 distinct chunks, and a row is read back as 16 aligned 16-byte pairs.
+    uint8_t* region = (wave < 2 ? stage0 : stage1) + (wave & 1) * 32768;
+    // bf16: one pass over the 4 n-tiles (128 cols x 2 B = 256 B rows);
+    // f32 : two passes of 2 n-tiles (64 cols x 4 B = 256 B rows).
+    constexpr int kPasses = kOutBf16 ? 1 : 2;
+    constexpr int kNiPerPass = kOutBf16 ? 4 : 2;
+    constexpr int kEsz = kOutBf16 ? 2 : 4;
+    constexpr int kColsPerPair = 16 / kEsz;
+    uint8_t* cbase = reinterpret_cast<uint8_t*>(g.c) + bz * g.stride_c * kEsz;
+    const bool vec_store = ((g.ldc * kEsz) % 16) == 0 && ((uintptr_t)cbase % 16) == 0;
+    // Tiles that lie wholly inside C and can use 16-byte stores skip every bounds check.
+    const bool interior = vec_store && (m0 + BM <= g.m) && (n0 + BN <= g.n);
+
+    auto epilogue = [&](auto checked_tag) {
+      constexpr bool kChecked = decltype(checked_tag)::value;
+#pragma unroll
+      for (int pass = 0; pass < kPasses; ++pass) {
+#pragma unroll
+        for (int nj = 0; nj < kNiPerPass; ++nj) {
+          const int ni = pass * kNiPerPass + nj;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int ncol_local = nj * 32 + 8 * q + 4 * lh;  // within the pass
+            const int64_t nn = ncol0 + ni * 32 + 8 * q + 4 * lh;
+            float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if (cs != nullptr) {
+              if constexpr (kChecked) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) csv[e] = (nn + e < g.n) ? cs[nn + e] : 1.0f;
+              } else {
+                const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
+                csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
+              }
+            }
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) {
+              float o[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = dequant(acc[mi][ni][4 * q + e], rscale[mi], csv[e]);
+              const int row = mi * 32 + lr;
+              uint8_t* p = region + row * 256;
+              if constexpr (kOutBf16) {
+                uint2 w;
+                w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+                w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+                const int j = ncol_local >> 2;  // 8-byte chunk index
+                *reinterpret_cast<uint2*>(p + ((j ^ (row & 31)) * 8)) = w;
+              } else {
+                const int j = ncol_local >> 1;  // two 8-byte chunks per 4 floats
+                *reinterpret_cast<float2*>(p + ((j ^ (row & 31)) * 8)) = make_float2(o[0], o[1]);
+                *reinterpret_cast<float2*>(p + (((j + 1) ^ (row & 31)) * 8)) = make_float2(o[2], o[3]);
+              }
+            }
+          }
+        }
+        __syncthreads();
+        // read back: lane -> 16-byte pair (lane&15) of row (lane>>4) + 4*it
+        const int64_t ncol_pass0 = ncol0 + (int64_t)pass * kNiPerPass * 32;
+        const int pair = lane & 15;
+        const int64_t nn = ncol_pass0 + pair * kColsPerPair;
+        const bool full = vec_store && (nn + kColsPerPair <= g.n);
+        uint8_t* dst0 = cbase + ((mrow0 + (lane >> 4)) * g.ldc + nn) * kEsz;
+#pragma unroll 8
+        for (int it = 0; it < 32; ++it) {
+          const int row = (lane >> 4) + 4 * it;
+          const int sw = row & 31;
+          uint4 v = *reinterpret_cast<const uint4*>(region + row * 256 + ((pair ^ (sw >> 1)) * 16));
+          if (sw & 1) v = make_uint4(v.z, v.w, v.x, v.y);
+          uint8_t* dst = dst0 + (int64_t)it * 4 * g.ldc * kEsz;
+          if constexpr (!kChecked) {
+            *reinterpret_cast<uint4*>(dst) = v;
+          } else if (mrow0 + row < g.m && nn < g.n) {
+            if (full) {
+              *reinterpret_cast<uint4*>(dst) = v;
+            } else {
+              const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+              const int nv = (int)(g.n - nn) < kColsPerPair ? (int)(g.n - nn) : kColsPerPair;
+              for (int e = 0; e < nv; ++e) {
+                if constexpr (kOutBf16)
+                  reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+                else
+                  reinterpret_cast<uint32_t*>(dst)[e] = w[e];
+              }
+            }
+          }
+        }
+        if (pass + 1 < kPasses) __syncthreads();
+      }
+    };
+    if (interior && ((uintptr_t)cs % 16) == 0) epilogue(std::false_type{});
+    else epilogue(std::true_type{});
+  }
+}
+
+// Reference-shaped fallback for operands the MFMA kernel cannot load with 16-byte
+// vectors (contraction length or leading dimension not a multiple of 16, unaligned
+// base).  One thread per output element; correct for any shape.  DEC_A/DEC_B decode one
+// operand byte to a float (exact for int8 and fp8).
+template <class DecA, class DecB, bool INT_ACC>
+__global__ void gemm_simple_kernel(const GemmArgs g) {
+  const int64_t nn = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t mm = blockIdx.y;
+  const int64_t bz = blockIdx.z;
+  if (nn >= g.n) return;
+  const uint8_t* A = g.a + bz * g.stride_a + mm * g.lda;
+  const uint8_t* B = g.b + bz * g.stride_b + nn * g.ldb;
+  const int64_t o = bz * g.stride_c + mm * g.ldc + nn;
+  float facc;
+  if constexpr (INT_ACC) {
+    int acc = 0;
+    for (int64_t kk = 0; kk < g.k; ++kk) acc += (int)(int8_t)A[kk] * (int)(int8_t)B[kk];
+    if (g.acc_out) reinterpret_cast<int32_t*>(g.acc_out)[o] = acc;
+    if (g.out_dtype == AQTX_I32) {
+      reinterpret_cast<int32_t*>(g.c)[o] = acc;
+      return;
+    }
+    facc = (float)acc;
+  } else {
+    facc = 0.0f;
+    for (int64_t kk = 0; kk < g.k; ++kk) facc = fmaf(DecA::decode(A[kk]), DecB::decode(B[kk]), facc);
+    if (g.acc_out) reinterpret_cast<float*>(g.acc_out)[o] = facc;
+  }
+  const int pbf = g.dq_bf16 & g.sc_bf16;
+  float f = rnd(facc, g.dq_bf16);
+  const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
+  const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+  if (g.col_first) {
+    if (cs) f = rnd(f * cs[nn], pbf);
+    if (rs) f = rnd(f * rs[mm], pbf);
+  } else {
+    if (rs) f = rnd(f * rs[mm], pbf);
+    if (cs) f = rnd(f * cs[nn], pbf);
+  }
+  f = rnd(f, g.dq_bf16);
+  if (g.out_dtype == AQTX_BF16) reinterpret_cast<uint16_t*>(g.c)[o] = bf16_bits(f);
+  else reinterpret_cast<float*>(g.c)[o] = f;
+}
+
+struct DecI8 {
+  static __device__ __forceinline__ float decode(uint8_t v) { return (float)(int8_t)v; }
+};
+struct DecE4M3 {  // e4m3fn: bias 7, no infinities
+  static __device__ __forceinline__ float decode(uint8_t v) {
+    const int e = (v >> 3) & 15, m = v & 7;
+    float f = e == 0 ? ldexpf((float)m, -9) : ldexpf((float)(8 + m), e - 10);
+    if (e == 15 && m == 7) f = __builtin_nanf("");
+    return (v & 0x80) ? -f : f;
+  }
+};
+struct DecE5M2 {  // e5m2: bias 15, IEEE-like
+  static __device__ __forceinline__ float decode(uint8_t v) {
+    const int e = (v >> 2) & 31, m = v & 3;
+    float f = e == 0 ? ldexpf((float)m, -16) : ldexpf((float)(4 + m), e - 17);
+    if (e == 31) f = m ? __builtin_nanf("") : __builtin_inff();
+    return (v & 0x80) ? -f : f;
+  }
+};
+
+// Fills GemmArgs from a validated plan.
+inline GemmArgs make_gemm_args(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                               const float* col_scale, void* c, void* acc_out) {
+  GemmArgs g{};
+  g.a = reinterpret_cast<const uint8_t*>(a);
+  g.b = reinterpret_cast<const uint8_t*>(b);
+  g.row_scale = row_scale; g.col_scale = col_scale;
+  g.c = c; g.acc_out = acc_out;
+  g.m = p->m; g.n = p->n; g.k = p->k;
+  g.lda = p->lda; g.ldb = p->ldb; g.ldc = p->ldc;
+  g.stride_a = p->stride_a; g.stride_b = p->stride_b; g.stride_c = p->stride_c;
+  g.stride_rs = p->row_scale_stride_b; g.stride_cs = p->col_scale_stride_b;
+  g.out_dtype = p->out_dtype;
+  g.dq_bf16 = p->dequant_dtype == AQTX_BF16;
+  g.sc_bf16 = p->scale_dtype == AQTX_BF16;
+  g.col_first = p->scale_order == AQTX_SCALE_COL_THEN_ROW;
+  g.tiles_m = (int)((p->m + BM - 1) / BM);
+  g.tiles_n = (int)((p->n + BN - 1) / BN);
+  return g;
+}
+
+inline bool gemm_vector_path_ok(const aqtx_gemm_plan* p, const void* a, const void* b) {
+  return (p->k % 16 == 0) && (p->lda % 16 == 0) && (p->ldb % 16 == 0) && ((uintptr_t)a % 16 == 0) &&
+         ((uintptr_t)b % 16 == 0) && (p->stride_a % 16 == 0) && (p->stride_b % 16 == 0) && p->k > 0;
+}
+
+// Epilogue id for the (out, dequant, scale) dtype triple, or -1.
+inline int gemm_epilogue_id(const aqtx_gemm_plan* p) {
+  if (p->out_dtype == AQTX_I32) return 3;
+  if (p->out_dtype == AQTX_BF16 && p->dequant_dtype == AQTX_BF16) return p->scale_dtype == AQTX_BF16 ? 0 : 1;
+  if (p->out_dtype == AQTX_F32 && p->dequant_dtype == AQTX_F32 && p->scale_dtype == AQTX_F32) return 2;
+  return -1;
+}
+
+}  // namespace
+
+int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8);
+
+}  // namespace aqtx

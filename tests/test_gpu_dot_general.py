@@ -141,3 +141,21 @@ def test_reference_assertions(gpu):
     cfg(a, b, MATMUL)
   with pytest.raises(AssertionError):  # :1011-1013
     cfg(a, a.t(), MATMUL, precision='highest')
+
+
+@pytest.mark.parametrize('fwd,bwd', [('e4m3', 'e5m2'), ('e4m3', 'e4m3')])
+def test_fp8_config(gpu, fwd, bwd):
+  """fp8 fwd + fp8 gradients (config_v4 with fp8 bits).  Quantized values and scales are
+  bit-exact; contractions accumulate in float32 in MFMA order, so outputs are compared to
+  the oracle (exact sum, one rounding) within one bf16 ulp: rtol 2**-7, plus an absolute
+  term for cancelled sums."""
+  dt = 'bf16'
+  lhs, rhs, g = U.rand((96, 256), dt, 1, outliers=True), U.rand((256, 64), dt, 2, 0.02), U.rand((96, 64), dt, 3, 1e-3)
+  cfg = config.config_v4(fwd_bits=fwd, dlhs_bits=bwd, drhs_bits=bwd)
+  ocfg = R.config_v4(fwd, bwd, bwd)
+  got, want = _run_both(lhs, rhs, g, dt, MATMUL, cfg, ocfg, prng.prng_key(5), gpu)
+  for k in ('lq', 'rq', 'ls', 'rs'):
+    np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+  for k in ('out', 'dlhs', 'drhs'):
+    np.testing.assert_allclose(got[k], want[k], rtol=2.0 ** -7, atol=2.0 ** -9 * np.abs(want[k]).max(),
+                               err_msg=k)

@@ -70,3 +70,82 @@ def test_large_accumulators_round_like_xla(gpu):
   c = ops.gemm(torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu), row_scale=None,
                col_scale=None, out_dtype=torch.bfloat16)
   np.testing.assert_array_equal(c.float().cpu().numpy(), want)
+
+
+# ---- fp8 ---------------------------------------------------------------------------------
+_FP8_TORCH = {'e4m3': torch.float8_e4m3fn, 'e5m2': torch.float8_e5m2}
+_FP8_AQTX = {'e4m3': L.E4M3, 'e5m2': L.E5M2}
+
+
+def _fp8_small_ints(shape, seed, kind):
+  """Bytes of small integers (exact in both fp8 formats) and their float values."""
+  v = np.random.default_rng(seed).integers(-4, 5, size=shape).astype(np.float32)
+  b = torch.from_numpy(v).to(_FP8_TORCH[kind]).view(torch.uint8)
+  return b, v
+
+
+def _fp8_random_bytes(shape, seed, kind):
+  """Random finite fp8 bit patterns (|x| <= 16 so that sums stay far from overflow)."""
+  rng = np.random.default_rng(seed)
+  allb = np.arange(256, dtype=np.uint8)
+  vals = U.fp8_bytes_to_float(allb, kind)
+  ok = allb[np.isfinite(vals) & (np.abs(vals) <= 16.0)]
+  b = ok[rng.integers(0, len(ok), size=shape)]
+  return torch.from_numpy(b), U.fp8_bytes_to_float(b, kind)
+
+
+FP8_SHAPES = [(1, 256, 256, 256), (1, 300, 520, 144), (2, 130, 70, 48), (1, 17, 9, 50), (1, 512, 256, 4096)]
+
+
+@pytest.mark.parametrize('ka,kb', [('e4m3', 'e4m3'), ('e4m3', 'e5m2'), ('e5m2', 'e4m3'), ('e5m2', 'e5m2')])
+@pytest.mark.parametrize('batch,m,n,k', FP8_SHAPES)
+def test_fp8_exact_when_sums_are_representable(gpu, batch, m, n, k, ka, kb):
+  """Small-integer operands: every partial sum is exact in float32, so any summation order
+  must give the exact result; a wrong format decode or a dropped k block cannot."""
+  a, av = _fp8_small_ints((batch, m, k), 11, ka)
+  b, bv = _fp8_small_ints((batch, n, k), 12, kb)
+  want = np.einsum('bmk,bnk->bmn', av.astype(np.float64), bv.astype(np.float64))
+  c = ops.gemm(a.to(gpu), b.to(gpu), row_scale=None, col_scale=None, out_dtype=torch.float32,
+               a_dtype=_FP8_AQTX[ka], b_dtype=_FP8_AQTX[kb])
+  np.testing.assert_array_equal(c.cpu().numpy().astype(np.float64), want)
+
+
+@pytest.mark.parametrize('ka,kb', [('e4m3', 'e4m3'), ('e4m3', 'e5m2'), ('e5m2', 'e5m2')])
+@pytest.mark.parametrize('batch,m,n,k', FP8_SHAPES)
+def test_fp8_random_values_within_mfma_accumulation_error(gpu, batch, m, n, k, ka, kb):
+  """Tolerance: |got - exact| <= 2**-10 * sum_k |a_k b_k|.  The fp8 MFMA adds the 64 products
+  of one instruction in a reduced-precision tree: measured on gfx950, a product more than 2**14
+  below the largest product of its 64-long block is dropped, and the block sum is then added
+  to the float32 accumulator with truncation.  The bound is that per-block loss (63 dropped
+  terms of 2**-14 of the block maximum) with a factor 4 of slack; the exact-sum test above
+  pins everything that does not depend on this hardware rounding."""
+  a, av = _fp8_random_bytes((batch, m, k), 13, ka)
+  b, bv = _fp8_random_bytes((batch, n, k), 14, kb)
+  av, bv = av.astype(np.float64), bv.astype(np.float64)
+  want = np.einsum('bmk,bnk->bmn', av, bv)
+  mag = np.einsum('bmk,bnk->bmn', np.abs(av), np.abs(bv))
+  c = ops.gemm(a.to(gpu), b.to(gpu), row_scale=None, col_scale=None, out_dtype=torch.float32,
+               a_dtype=_FP8_AQTX[ka], b_dtype=_FP8_AQTX[kb])
+  err = np.abs(c.cpu().numpy().astype(np.float64) - want)
+  bound = 2.0 ** -10 * mag + 1e-30
+  assert (err <= bound).all(), (err / bound).max()
+
+
+@pytest.mark.parametrize('out,sdt', [('bf16', 'bf16'), ('bf16', 'f32'), ('f32', 'f32')])
+@pytest.mark.parametrize('order', [L.SCALE_ROW_THEN_COL, L.SCALE_COL_THEN_ROW])
+@pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 1024), (2, 100, 72, 160), (1, 33, 20, 23)])
+def test_fp8_dequant_epilogue(gpu, batch, m, n, k, order, sdt, out):
+  """The epilogue is checked bit-exactly on the accumulators the kernel itself reports."""
+  a, _ = _fp8_random_bytes((batch, m, k), 15, 'e4m3')
+  b, _ = _fp8_random_bytes((batch, n, k), 16, 'e5m2')
+  rs = nm.cast(np.abs(U.rand((batch, m), 'f32', 5, 0.03)) + np.float32(1e-3), sdt)
+  cs = nm.cast(np.abs(U.rand((batch, n), 'f32', 6, 6e-4)) + np.float32(1e-5), sdt)
+  c, acc = ops.gemm(a.to(gpu), b.to(gpu), row_scale=torch.from_numpy(rs).to(gpu),
+                    col_scale=torch.from_numpy(cs).to(gpu), out_dtype=U.TORCH_DT[out],
+                    scale_dtype=U.TORCH_DT[sdt], scale_order=order, a_dtype=L.E4M3, b_dtype=L.E5M2,
+                    want_acc=True)
+  s1, s2 = (rs[:, :, None], cs[:, None, :])
+  if order == L.SCALE_COL_THEN_ROW:
+    s1, s2 = s2, s1
+  want = R.dequant(R.QTensor(acc.cpu().numpy(), 'f32', [s1, s2], sdt, out))
+  np.testing.assert_array_equal(c.float().cpu().numpy(), want)
