@@ -21,6 +21,10 @@ OPS_PER_CONTRACTION = 2.0 * M * N * K          # 9.6207e11
 OPS_PER_STEP = 3.0 * OPS_PER_CONTRACTION       # fwd + dlhs + drhs
 INT8_MFMA_PEAK = 5.0e15                        # MI355X dense int8, published
 MATMUL = (((1,), (0,)), ((), ()))
+# HBM bytes per GEMM launch (mean of fwd, dlhs, drhs) from the FETCH_SIZE / WRITE_SIZE counter runs
+# summarised in profiles/bench_int8_fwd_bwd_8192x4096x14336_hbm_traffic.txt; counters cannot be
+# read from inside this process, so the figure is carried here and re-measured when the kernel changes.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 953e6
 
 
 def make_inputs(device):
@@ -72,6 +76,9 @@ def main():
   ap.add_argument('--steps', type=int, default=20)
   ap.add_argument('--warmup', type=int, default=3)
   ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--calibration-copy', action='store_true',
+                  help='also launch one elementwise kernel that reads and writes 256 MiB, as the '
+                       'known-size reference for FETCH_SIZE / WRITE_SIZE counter runs')
   args = ap.parse_args()
   if args.gpus != 1:
     print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)',
@@ -98,6 +105,10 @@ def main():
     out.backward(g)
     return out
 
+  if args.calibration_copy:
+    src = torch.ones(64 << 20, dtype=torch.int32, device=dev)
+    torch.neg(src, out=torch.empty_like(src))  # 256 MiB in, 256 MiB out
+    del src
   for _ in range(args.warmup):
     step()
   torch.cuda.synchronize()
@@ -121,9 +132,9 @@ def main():
       'config': {'workload': 'configs[1]: int8 dot_general fwd+bwd, lhs bf16 [8192,4096] x rhs bf16 '
                              '[4096,14336], fully_quantized(8,8), SR key 42, bf16 out',
                  'pct_of_int8_mfma_peak': 100.0 * OPS_PER_STEP / (ms_per_step * 1e-3) / INT8_MFMA_PEAK},
-      'roofline': {'bound': 'mfma', 'kernel': 'gemm_i8_kernel', 'achieved': achieved,
+      'roofline': {'bound': 'mfma', 'kernel': 'gemm_kernel<MmaI8, ...>', 'achieved': achieved,
                    'peak': INT8_MFMA_PEAK / 1e12, 'unit': 'TFLOP/s',
-                   'frac': achieved * 1e12 / INT8_MFMA_PEAK, 'traffic': None,
+                   'frac': achieved * 1e12 / INT8_MFMA_PEAK, 'traffic': GEMM_TRAFFIC_BYTES_PER_LAUNCH,
                    'launch_ms': gemm_ms, 'launches_timed': len(timer.pairs)},
   }
   if not args.no_cpu_baseline:
