@@ -41,7 +41,8 @@ class GemmPlan(ctypes.Structure):
       ('stride_a', ctypes.c_int64), ('stride_b', ctypes.c_int64), ('stride_c', ctypes.c_int64),
       ('a_dtype', ctypes.c_int32), ('b_dtype', ctypes.c_int32),
       ('out_dtype', ctypes.c_int32), ('dequant_dtype', ctypes.c_int32),
-      ('scale_dtype', ctypes.c_int32), ('scale_order', ctypes.c_int32),
+      ('row_scale_dtype', ctypes.c_int32), ('col_scale_dtype', ctypes.c_int32),
+      ('scale_order', ctypes.c_int32),
       ('row_scale_stride_b', ctypes.c_int64), ('col_scale_stride_b', ctypes.c_int64),
   ]
 

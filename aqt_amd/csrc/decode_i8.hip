@@ -1,8 +1,307 @@
-// Serving-shape contraction (placeholder until the kernel lands).
+// Serving-shape contraction: out[m, n] = dequant( quant(x)[m, :] . W[n, :] ) for m <= 64 rows of
+// activations against a pre-quantized int8 weight stored [n, k] (contraction axis contiguous).
+//
+// The weight is read exactly once and dominates the traffic, so the kernels are built around
+// streaming W from HBM with every lane fetching 16 contiguous bytes straight into the operand
+// registers of v_mfma_i32_16x16x64_i8 (lane -> row lane&15, bytes 16*(lane>>4).. of a 64-byte
+// k step: 16 rows x 64 B per wave instruction, whole 64-byte sectors).  The activations are
+// quantized first by the row kernel of aqtx_quantize (same arithmetic as training), then:
+//   K split : one workgroup per 16 weight rows, its 4 waves split K and meet in LDS; the
+//             quantized activations come from L2 (m <= 16, or a weight with few rows);
+//   whole K : one workgroup per 64 weight rows (16 per wave, whole K); the activations
+//             are staged chunk by chunk in LDS and shared by the waves, the weights are
+//             requested three chunks ahead (16 < m <= 64 and n >= 12288).  K is never split across workgroups: a partial-sum
+//             exchange inside one launch would need device-scope release/acquire, which
+//             flushes and invalidates the per-XCD L2s.
 #include "common.h"
+
+namespace aqtx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kBufferRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format (gfx9)
+constexpr int kOob = 0x7FFFFFF0;                     // offset that is out of range for every buffer
+
+struct DecodeArgs {
+  const int8_t* xq;       // [m][k]
+  const int8_t* w;        // [n][k]
+  const float* x_scale;   // [m]
+  const float* w_scale;   // [n]
+  void* out;              // [m][n]
+  int m, n, k;
+  int out_bf16, xs_bf16, ws_bf16;
+};
+
+__device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
+
+// QTensor.dequant: cast the accumulator, multiply by the lhs scale, then the rhs scale, each
+// product in the promoted dtype of its operands, final cast.
+__device__ __forceinline__ void store_out(const DecodeArgs& d, int mm, int nn, int acc) {
+  float f = rnd((float)acc, d.out_bf16);
+  const int p1 = d.out_bf16 & d.xs_bf16;
+  f = rnd(f * d.x_scale[mm], p1);
+  f = rnd(f * d.w_scale[nn], p1 & d.ws_bf16);
+  f = rnd(f, d.out_bf16);
+  const int64_t o = (int64_t)mm * d.n + nn;
+  if (d.out_bf16) reinterpret_cast<uint16_t*>(d.out)[o] = bf16_bits(f);
+  else reinterpret_cast<float*>(d.out)[o] = f;
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kBufferRsrcWord3);
+}
+
+// ---- K split inside the workgroup ---------------------------------------------------------------
+// One workgroup per 16 weight rows; its 4 waves take a quarter of K each and meet in LDS.  The
+// quantized activations are read straight from L2 as MFMA operands (MB blocks of 16 rows), so
+// the L2 traffic is (1 + MB) times the weight bytes: the shape for m <= 16, and for larger m
+// when the weight has too few rows to fill the chip with whole-K waves.
+template <int MB, int U>  // U: 64-byte k steps in flight per wave
+__global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) {
+  __shared__ int red[4][MB * 16][16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);  // clamped; such columns are never stored
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
+  const int kq = ((d.k + 3) / 4 + 63) / 64 * 64;  // K range of one wave, whole 64-byte steps
+  const int k_lo = wave * kq;
+  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
+  const int wbase = nrow * d.k + c * 16;
+  int xbase[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) xbase[mb] = (mb * 16 + r) < d.m ? (mb * 16 + r) * d.k + c * 16 : kOob;
+
+  v4i acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = v4i{0, 0, 0, 0};
+  for (int kk = k_lo; kk < k_hi; kk += 64 * U) {
+    v4i wf[U], xf[U][MB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ko = kk + u * 64;
+      const bool ok = ko + c * 16 < k_hi;
+      wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? wbase + ko : kOob, 0, 0);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        xf[u][mb] = __builtin_amdgcn_raw_buffer_load_b128(rx, (ok && xbase[mb] != kOob) ? xbase[mb] + ko : kOob, 0, 0);
+    }
+    // Keep every load of the batch in flight before the first MFMA waits for one: left alone,
+    // the scheduler interleaves them to save registers and the wave stalls on memory latency.
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][mb], wf[u], acc[mb], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // lane holds C[m = mb*16 + 4c + e][n = r]
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][mb * 16 + 4 * c + e][r] = acc[mb][e];
+  __syncthreads();
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int mm = mb * 16 + (tid >> 4), nn = n0 + (tid & 15);
+    if (mm < d.m && nn < d.n) {
+      const int s = red[0][mm][tid & 15] + red[1][mm][tid & 15] + red[2][mm][tid & 15] + red[3][mm][tid & 15];
+      store_out(d, mm, nn, s);
+    }
+  }
+}
+
+// ---- 16 < m <= 64 ------------------------------------------------------------------------------
+constexpr int kChunk = 256;  // bytes of K per pipeline step
+constexpr int kAhead = 3;    // weight chunks requested ahead of the one being multiplied
+
+// MB: 16-row blocks of activations, 2 (m <= 32) or 4 (m <= 64).  NWV: waves per workgroup, each
+// owning 16 weight rows over the whole of K (no K split, so no cross-workgroup reduction).
+template <int MB, int NWV>
+__global__ __launch_bounds__(NWV * 64) void decode_block_kernel(const DecodeArgs d) {
+  // Activations of one K chunk, [MB*16 rows][256 B]; the 16-byte piece j of row i sits at
+  // piece j ^ (i & 15), so the 16 lanes of a fragment read (16 rows, one piece) hit 64 banks.
+  __shared__ __attribute__((aligned(16))) uint8_t xbuf[2][MB * 16 * kChunk];
+  constexpr int NT = NWV * 64;
+  constexpr int XP = MB * 16 * 16 / NT;  // 16-byte pieces of a chunk staged per thread
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int n0 = blockIdx.x * (NWV * 16) + wave * 16;
+  const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);  // clamped; such columns are never stored
+  const int nchunks = (d.k + kChunk - 1) / kChunk;
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
+  const int wbase = nrow * d.k + c * 16;
+  // staging of the activations: thread -> (row tid>>4 of a pass of NT/16 rows, piece tid&15)
+  const int xs_row = tid >> 4, xs_piece = tid & 15;
+
+  v4i wreg[kAhead + 1][4], xr[2][XP];  // xr[p]: activations of a chunk of parity p on their way to LDS
+  auto load_w = [&](v4i* dst, int kc) {  // past K every load reads zeros
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int ko = kc + ks * 64;
+      dst[ks] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < d.k) ? wbase + ko : kOob, 0, 0);
+    }
+  };
+  auto load_x = [&](v4i* dst, int kc) {
+#pragma unroll
+    for (int p = 0; p < XP; ++p) {
+      const int row = p * (NT / 16) + xs_row;
+      const int ko = kc + xs_piece * 16;
+      dst[p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (row < d.m && ko < d.k) ? row * d.k + ko : kOob, 0, 0);
+    }
+  };
+  auto store_x = [&](uint8_t* buf, const v4i* src) {
+#pragma unroll
+    for (int p = 0; p < XP; ++p) {
+      const int row = p * (NT / 16) + xs_row;
+      *reinterpret_cast<v4i*>(buf + row * kChunk + ((xs_piece ^ (row & 15)) * 16)) = src[p];
+    }
+  };
+
+  v4i acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = v4i{0, 0, 0, 0};
+
+  load_x(xr[0], 0);
+#pragma unroll
+  for (int j = 0; j < kAhead; ++j) load_w(wreg[j], j * kChunk);
+  store_x(xbuf[0], xr[0]);
+  load_x(xr[1], kChunk);
+  load_x(xr[0], 2 * kChunk);
+  __syncthreads();
+  // One pipeline step: publish the activations of chunk i+1 (requested two steps ago), request
+  // those of chunk i+3 and the weights of chunk i+kAhead, multiply chunk i.  Every load has two
+  // or more steps to arrive, so a step never waits a full memory latency.  The register sets
+  // rotate roles through the unrolled steps (no register copies that would wait for loads).
+  auto step = [&](const v4i* wc, v4i* wfar, v4i* xnext, int i) {
+    store_x(xbuf[(i + 1) & 1], xnext);
+    load_x(xnext, (i + 3) * kChunk);
+    load_w(wfar, (i + kAhead) * kChunk);
+    const uint8_t* buf = xbuf[i & 1];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const v4i xf = *reinterpret_cast<const v4i*>(buf + (mb * 16 + r) * kChunk + (((ks * 4 + c) ^ r) * 16));
+        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf, wc[ks], acc[mb], 0, 0, 0);
+      }
+    // LDS traffic only: a __syncthreads() would also wait for the global loads in flight.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  static_assert(kAhead == 3, "the unrolled rotation below is written for 4 register sets");
+  // Always four steps per trip: steps past the last chunk read zeros everywhere (loads out of
+  // range) and add nothing.  A branch-free body lets the compiler count the loads in flight
+  // exactly instead of draining them at every loop entry.
+  for (int i = 0; i < nchunks; i += 4) {
+    step(wreg[0], wreg[3], xr[1], i);
+    step(wreg[1], wreg[0], xr[0], i + 1);
+    step(wreg[2], wreg[1], xr[1], i + 2);
+    step(wreg[3], wreg[2], xr[0], i + 3);
+  }
+
+  // lane holds C[m = mb*16 + 4c + e][n = n0 + r]
+  const int nn = n0 + r;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int mm = mb * 16 + 4 * c + e;
+      if (mm < d.m && nn < d.n) store_out(d, mm, nn, acc[mb][e]);
+    }
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int validate_decode(const aqtx_decode_plan* p) {
+  AQTX_REQUIRE(p != nullptr, "aqtx_decode_i8: plan is NULL");
+  AQTX_REQUIRE(p->m >= 0 && p->n >= 0 && p->k >= 0, "aqtx_decode_i8: negative shape");
+  AQTX_REQUIRE(p->m <= 64, "aqtx_decode_i8: m = %lld exceeds 64 (use aqtx_quantize + aqtx_gemm_i8)",
+               (long long)p->m);
+  AQTX_REQUIRE(p->k > 0 && p->k % 16 == 0, "aqtx_decode_i8: k = %lld must be a positive multiple of 16",
+               (long long)p->k);
+  AQTX_REQUIRE(p->n * p->k < (1ll << 31) && p->m * p->n < (1ll << 31),
+               "aqtx_decode_i8: weight larger than 2 GiB is not addressable with 32-bit offsets");
+  AQTX_REQUIRE(is_float_dtype(p->x_dtype) && is_float_dtype(p->x_scale_dtype) &&
+                   is_float_dtype(p->w_scale_dtype) && is_float_dtype(p->out_dtype),
+               "aqtx_decode_i8: dtypes must be bf16 or f32");
+  AQTX_REQUIRE(p->quant_bound > 0.0f && p->clip_bound > 0.0f, "aqtx_decode_i8: bounds must be positive");
+  return 0;
+}
+
+}  // namespace
+}  // namespace aqtx
+
 using namespace aqtx;
-extern "C" size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan*) { return 0; }
-extern "C" int aqtx_decode_i8(const aqtx_decode_plan*, const void*, const void*, const float*, void*,
-                              float*, void*, void*, size_t, void*) {
-  return set_error("aqtx_decode_i8: not implemented in this build");
+
+extern "C" size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* p) {
+  if (p == nullptr || p->m < 0 || p->n < 0 || p->k < 0 || p->m > 64) return 0;
+  return align_up((size_t)(p->m * p->k), 256);  // the quantized activations when the caller keeps none
+}
+
+extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const void* w,
+                              const float* w_scale, void* xq, float* x_scale, void* out,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  if (int rc = validate_decode(p)) return rc;
+  if (p->m == 0 || p->n == 0) return 0;
+  AQTX_REQUIRE(x != nullptr && w != nullptr && w_scale != nullptr && x_scale != nullptr && out != nullptr,
+               "aqtx_decode_i8: NULL buffer");
+  const size_t need = xq != nullptr ? 0 : aqtx_decode_workspace_bytes(p);
+  AQTX_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need),
+               "aqtx_decode_i8: workspace too small (%zu < %zu)", workspace_bytes, need);
+  AQTX_REQUIRE(((uintptr_t)w % 16) == 0 && (need == 0 || ((uintptr_t)workspace % 16) == 0) &&
+                   (xq == nullptr || ((uintptr_t)xq % 16) == 0),
+               "aqtx_decode_i8: w, xq and the workspace must be 16-byte aligned");
+  int8_t* xq_buf = reinterpret_cast<int8_t*>(xq != nullptr ? xq : workspace);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+
+  // 1. per-token dynamic quantization of the activations (same kernel as training)
+  aqtx_quant_plan q{};
+  q.in_dtype = q.compute_dtype = p->x_dtype;
+  q.scale_dtype = p->x_scale_dtype;
+  q.out_dtype = AQTX_I8;
+  q.batch = 1; q.rows = p->m; q.cols = p->k;
+  q.reduce = AQTX_REDUCE_COLS;
+  q.quant_bound = p->quant_bound; q.clip_bound = p->clip_bound;
+  q.noise = AQTX_NOISE_NONE;
+  if (int rc = aqtx_quantize(&q, x, nullptr, xq_buf, x_scale, nullptr, 0, stream)) return rc;
+
+  // 2. the contraction with the dequantisation fused
+  DecodeArgs d{};
+  d.xq = xq_buf; d.w = reinterpret_cast<const int8_t*>(w);
+  d.x_scale = x_scale; d.w_scale = w_scale; d.out = out;
+  d.m = (int)p->m; d.n = (int)p->n; d.k = (int)p->k;
+  d.out_bf16 = p->out_dtype == AQTX_BF16;
+  d.xs_bf16 = p->x_scale_dtype == AQTX_BF16;
+  d.ws_bf16 = p->w_scale_dtype == AQTX_BF16;
+
+  const unsigned grid16 = (unsigned)((p->n + 15) / 16);
+  if (p->m <= 16) {
+    decode_ksplit_kernel<1, 16><<<grid16, 256, 0, st>>>(d);
+    AQTX_HIP_CHECK_LAUNCH("decode_ksplit_kernel");
+    return 0;
+  }
+  // Whole-K waves sharing the activations through LDS need n/16 >= a few waves per CU to keep
+  // HBM busy; below that the K-split shape wins although it re-reads the activations.
+  if (p->n < 12288) {
+    if (p->m <= 32) decode_ksplit_kernel<2, 8><<<grid16, 256, 0, st>>>(d);
+    else decode_ksplit_kernel<4, 4><<<grid16, 256, 0, st>>>(d);
+    AQTX_HIP_CHECK_LAUNCH("decode_ksplit_kernel");
+    return 0;
+  }
+  const unsigned grid = (unsigned)((p->n + 63) / 64);
+  if (p->m <= 32) decode_block_kernel<2, 4><<<grid, 256, 0, st>>>(d);
+  else decode_block_kernel<4, 4><<<grid, 256, 0, st>>>(d);
+  AQTX_HIP_CHECK_LAUNCH("decode_block_kernel");
+  return 0;
 }

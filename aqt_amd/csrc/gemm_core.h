@@ -73,7 +73,8 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int out_dtype;  // AQTX_BF16 | AQTX_F32 | AQTX_I32
   int dq_bf16;    // dequant dtype is bf16
-  int sc_bf16;    // scale dtype is bf16
+  int p1_bf16;    // the first product is rounded to bf16
+  int p2_bf16;    // the second product is rounded to bf16
   int col_first;  // scale order
 };
 
@@ -105,17 +106,26 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 }
 
 // EPI selects the epilogue arithmetic at compile time (run-time flags there turn into
-// thousands of branches): 0 = bf16 out, bf16 scales; 1 = bf16 out, f32 scales; 2 = f32 out,
-// f32 scales; 3 = raw int32 accumulators only.  COL_FIRST: the column scale multiplies first.
+// thousands of branches): 0 = bf16 out, bf16 scales; 1 = bf16 out, first scale f32; 2 = f32 out;
+// 3 = raw accumulators only; 4 = bf16 out, first scale bf16, second f32.  COL_FIRST: the column scale multiplies first.
 // KTAIL: K is not a multiple of the 128-byte stage, the last stage masks chunks past K.
-template <class MMA, int EPI, bool COL_FIRST, bool KTAIL>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+// NW: waves per workgroup.  4 = 2x2 waves with 128x128 wave tiles, one wave per SIMD;
+// 8 = 2x4 waves with 128x64 wave tiles, two waves per SIMD, so that one wave's MFMAs fill the
+// issue slots in which the other waits on the memory pipeline.
+template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gemm_kernel(const GemmArgs g) {
+  static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+  constexpr int NI = 16 / NW;       // 32-column MFMA tiles per wave
+  constexpr int WN = NW / 2;        // waves along n
+  constexpr int LPW = 32 / NW;      // 8-row load blocks per wave and operand
+  constexpr int NL = 2 * LPW;       // global loads per wave and stage
+  constexpr int MPK = 4 * NI;       // MFMAs per wave and k-step
   using Acc = typename MMA::Acc;
   using AccScalar = typename MMA::AccScalar;
   using Frag = typename MMA::Frag;
   constexpr int kChunks = MMA::kChunks;
-  constexpr int KS = 4 / kChunks;  // k-steps (rounds of 16 MFMAs) per 128-byte stage
+  constexpr int KS = 4 / kChunks;  // k-steps (rounds of MPK MFMAs) per 128-byte stage
   // Two stages in two distinct LDS objects, so that the compiler can tell the stage
   // being filled by the buffer->LDS loads from the one the MFMA fragments are read from.
   __shared__ __attribute__((aligned(1024))) uint8_t stage0[kStageBytes];
@@ -123,7 +133,7 @@ void gemm_kernel(const GemmArgs g) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int lr = lane & 31, lh = lane >> 5;
 
   int tm, tn;
@@ -145,22 +155,23 @@ void gemm_kernel(const GemmArgs g) {
       (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + g.k), kBufferRsrcWord3);
-  int voff_a[8], voff_b[8], chunk_byte[8];
+  int voff_a[LPW], voff_b[LPW], chunk_byte[LPW];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = (wave * 8 + i) * 8 + (lane >> 3);
-    chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ i) & 7) * 16;
+  for (int i = 0; i < LPW; ++i) {
+    const int blk = wave * LPW + i;
+    const int row = blk * 8 + (lane >> 3);
+    chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ blk) & 7) * 16;
     voff_a[i] = row * (int)g.lda + chunk_byte[i];
     voff_b[i] = row * (int)g.ldb + chunk_byte[i];
   }
-  v4i stg[16];  // staging registers: stg[2*i] = A block i, stg[2*i+1] = B block i
-  auto load_global = [&](int j, int k0) {  // j = 0..15
+  v4i stg[NL];  // staging registers: stg[2*i] = A block i, stg[2*i+1] = B block i
+  auto load_global = [&](int j, int k0) {  // j = 0..NL-1
     const int i = j >> 1;
     int vo = (j & 1) ? voff_b[i] : voff_a[i];
     if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
     stg[j] = __builtin_amdgcn_raw_buffer_load_b128((j & 1) ? rsrc_b : rsrc_a, vo, k0, 0);
   };
-  const int st_off = wave * 8 * 1024 + lane * 16;
+  const int st_off = wave * LPW * 1024 + lane * 16;
   auto store_lds = [&](uint8_t* st, int j) {
     const int i = j >> 1;
     *reinterpret_cast<v4i*>(st + ((j & 1) ? kTileBytes : 0) + st_off + i * 1024) = stg[j];
@@ -173,39 +184,38 @@ void gemm_kernel(const GemmArgs g) {
   for (int cidx = 0; cidx < 8; ++cidx)
     frag_off[cidx] = lr * BK + (((lh * kChunks) ^ lf0 ^ cidx) * 16);
   const int a_base = wm * 128 * BK;                // rows of the A tile this wave needs
-  const int b_base = kTileBytes + wn * 128 * BK;   // rows of the B tile
+  const int b_base = kTileBytes + wn * NI * 32 * BK;   // rows of the B tile
 
-  Acc acc[4][4];
+  Acc acc[4][NI];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
+  auto load_frag = [&](const uint8_t* rows, int ks, int i) -> Frag {
+    if constexpr (kChunks == 1) {
+      return *reinterpret_cast<const v4i*>(rows + i * 32 * BK + frag_off[(2 * ks) ^ (4 * (i & 1))]);
+    } else {
+      const int c0 = (4 * ks) ^ (4 * (i & 1)), c1 = c0 ^ 1;
+      const v4i x0 = *reinterpret_cast<const v4i*>(rows + i * 32 * BK + frag_off[c0]);
+      const v4i x1 = *reinterpret_cast<const v4i*>(rows + i * 32 * BK + frag_off[c1]);
+      return Frag{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+  };
   auto load_frags = [&](const uint8_t* st, int ks, Frag* fa, Frag* fb) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if constexpr (kChunks == 1) {
-        const int cidx = (2 * ks) ^ (4 * (i & 1));
-        fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[cidx]);
-        fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[cidx]);
-      } else {
-        const int c0 = (4 * ks) ^ (4 * (i & 1)), c1 = c0 ^ 1;
-        const v4i a0 = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[c0]);
-        const v4i a1 = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[c1]);
-        const v4i b0 = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c0]);
-        const v4i b1 = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c1]);
-        fa[i] = Frag{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-        fb[i] = Frag{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
-      }
+      fa[i] = load_frag(st + a_base, ks, i);
+      if (i < NI) fb[i] = load_frag(st + b_base, ks, i);
     }
   };
   auto mfma_step = [&](const Frag* fa, const Frag* fb) {
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = MMA::mma(fb[ni], fa[mi], acc[mi][ni]);
+      for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = MMA::mma(fb[ni], fa[mi], acc[mi][ni]);
   };
   // Scheduling groups (llvm.amdgcn.sched.group.barrier masks).
   constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100, kDsWrite = 0x200;
@@ -221,24 +231,26 @@ void gemm_kernel(const GemmArgs g) {
   // The barrier is a bare s_barrier: a __syncthreads() would also wait for the global loads
   // still in flight.  No branch surrounds any MFMA (a conditional stage makes the compiler
   // shuffle all 256 accumulators through VGPRs).
-  Frag fa0[4], fb0[4], fa1[4], fb1[4];
-  constexpr int kDsPerStep = 8 * kChunks;  // ds_read_b128 per k-step
+  Frag fa0[4], fb0[NI], fa1[4], fb1[NI];
+  constexpr int kDsPerStep = (4 + NI) * kChunks;  // ds_read_b128 per k-step
   auto run_stage = [&](const uint8_t* cur, uint8_t* cur_refill, const uint8_t* next, int refill_k0) {
 #pragma unroll
     for (int ks = 0; ks < KS - 1; ++ks) {
       // loads [l0, l1) of the 16 go with this k-step
-      const int l0 = (16 * ks + KS - 2) / (KS - 1), l1 = (16 * (ks + 1) + KS - 2) / (KS - 1);
+      const int l0 = (NL * ks + KS - 2) / (KS - 1), l1 = (NL * (ks + 1) + KS - 2) / (KS - 1);
       if (ks % 2 == 0) load_frags(cur, ks + 1, fa1, fb1); else load_frags(cur, ks + 1, fa0, fb0);
 #pragma unroll
       for (int j = l0; j < l1; ++j) load_global(j, refill_k0);
       if (ks % 2 == 0) mfma_step(fa0, fb0); else mfma_step(fa1, fb1);
       const int nl = l1 - l0;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
+      for (int i = 0; i < MPK; ++i) {
         __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
         if (i < kDsPerStep) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
-        if (nl == 16 || (nl == 6 ? (i % 3 == 0) : (i % 3 == 1)))
-          __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
+        const bool slot = (MPK == 16 && nl == 6) ? (i % 3 == 0)
+                        : (MPK == 16 && nl == 5) ? (i % 3 == 1)
+                        : ((i + 1) * nl / MPK > i * nl / MPK);
+        if (slot) __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -247,12 +259,12 @@ void gemm_kernel(const GemmArgs g) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < 16; ++j) store_lds(cur_refill, j);
+    for (int j = 0; j < NL; ++j) store_lds(cur_refill, j);
     // KS is even, so the last k-step always computes from set 1 and refills set 0.
     load_frags(next, 0, fa0, fb0);
     mfma_step(fa1, fb1);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < MPK; ++i) {
       __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
       __builtin_amdgcn_sched_group_barrier(kDsWrite, 1, 0);
       if (i < kDsPerStep) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
@@ -265,13 +277,13 @@ void gemm_kernel(const GemmArgs g) {
   // requested past the end of K are never consumed.
   const int KT2 = (int)((g.k + 2 * BK - 1) / (2 * BK));
 #pragma unroll
-  for (int j = 0; j < 16; ++j) load_global(j, 0);
+  for (int j = 0; j < NL; ++j) load_global(j, 0);
 #pragma unroll
-  for (int j = 0; j < 16; ++j) store_lds(stage0, j);
+  for (int j = 0; j < NL; ++j) store_lds(stage0, j);
 #pragma unroll
-  for (int j = 0; j < 16; ++j) load_global(j, BK);
+  for (int j = 0; j < NL; ++j) load_global(j, BK);
 #pragma unroll
-  for (int j = 0; j < 16; ++j) store_lds(stage1, j);
+  for (int j = 0; j < NL; ++j) store_lds(stage1, j);
   __syncthreads();
   load_frags(stage0, 0, fa0, fb0);
   for (int it = 0; it < KT2; ++it) {
@@ -282,7 +294,7 @@ void gemm_kernel(const GemmArgs g) {
 
   // ---- epilogue ---------------------------------------------------------------
   // lane holds C[m = mrow0 + mi*32 + lr][n = ncol0 + ni*32 + 8*q + 4*lh + e], e = 0..3, reg = 4*q+e
-  const int64_t mrow0 = m0 + wm * 128, ncol0 = n0 + wn * 128;
+  const int64_t mrow0 = m0 + wm * 128, ncol0 = n0 + wn * NI * 32;
 
   if (EPI == 3 || g.acc_out != nullptr) {
     AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out != nullptr ? g.acc_out : g.c);
@@ -291,7 +303,7 @@ void gemm_kernel(const GemmArgs g) {
     for (int mi = 0; mi < 4; ++mi) {
       const int64_t mm = mrow0 + mi * 32 + lr;
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni)
+      for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int64_t nn = ncol0 + ni * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
@@ -300,9 +312,10 @@ void gemm_kernel(const GemmArgs g) {
     }
   }
   if constexpr (EPI != 3) {
-    constexpr bool kOutBf16 = EPI <= 1;
-    constexpr bool kDqBf16 = EPI <= 1;          // dequant dtype == output dtype
-    constexpr bool kProdBf16 = EPI == 0;        // promote(dequant dtype, scale dtype)
+    constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
+    constexpr bool kDqBf16 = kOutBf16;                    // dequant dtype == output dtype
+    constexpr bool kProd1Bf16 = EPI == 0 || EPI == 4;     // promote(dequant dtype, first scale dtype)
+    constexpr bool kProd2Bf16 = EPI == 0;                 // promote(that, second scale dtype)
     // A missing scale is a multiplication by 1, which every rounding below leaves alone.
     const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
     const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
@@ -315,21 +328,24 @@ void gemm_kernel(const GemmArgs g) {
     auto dequant = [&](AccScalar accv, float s_row, float s_col) {
       float f = round_to<kDqBf16>((float)accv);  // (int32 ->) f32 -> dequant dtype
       const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
-      f = round_to<kProdBf16>(f * s1);
-      f = round_to<kProdBf16>(f * s2);
+      f = round_to<kProd1Bf16>(f * s1);
+      f = round_to<kProd2Bf16>(f * s2);
       return round_to<kDqBf16>(f);
     };
 
-    // Each wave stages its 128 x 256-byte block in LDS (32 KiB, no padding): the 8-byte
-    // chunk j of row r sits at chunk j ^ (r & 31), so the 32 lanes that write one column
-    // group hit 32 distinct chunks, and a row is read back as 16 aligned 16-byte pairs.
-    uint8_t* region = (wave < 2 ? stage0 : stage1) + (wave & 1) * 32768;
-    // bf16: one pass over the 4 n-tiles (128 cols x 2 B = 256 B rows);
-    // f32 : two passes of 2 n-tiles (64 cols x 4 B = 256 B rows).
+    // Each wave stages its 128-row block in LDS, RB = 256 (4 waves) or 128 (8 waves) bytes per
+    // row, no padding: the 8-byte chunk j of row r sits at chunk j ^ sw(r), sw chosen so that
+    // the 32 lanes that write one column group hit 32 distinct bank pairs, and a row is read
+    // back as aligned 16-byte pairs.
+    //   bf16: one pass over the NI n-tiles; f32: two passes of NI/2 n-tiles (same row bytes).
     constexpr int kPasses = kOutBf16 ? 1 : 2;
-    constexpr int kNiPerPass = kOutBf16 ? 4 : 2;
+    constexpr int kNiPerPass = kOutBf16 ? NI : NI / 2;
     constexpr int kEsz = kOutBf16 ? 2 : 4;
+    constexpr int RB = kNiPerPass * 32 * kEsz;
+    static_assert(RB == NI * 64, "row bytes");
     constexpr int kColsPerPair = 16 / kEsz;
+    uint8_t* region = (wave < NW / 2 ? stage0 : stage1) + (wave % (NW / 2)) * (128 * RB);
+    auto sw_of = [](int row) { return RB == 256 ? (row & 31) : ((row >> 1) & 15); };
     uint8_t* cbase = reinterpret_cast<uint8_t*>(g.c) + bz * g.stride_c * kEsz;
     const bool vec_store = ((g.ldc * kEsz) % 16) == 0 && ((uintptr_t)cbase % 16) == 0;
     // Tiles that lie wholly inside C and can use 16-byte stores skip every bounds check.
@@ -362,35 +378,37 @@ void gemm_kernel(const GemmArgs g) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) o[e] = dequant(acc[mi][ni][4 * q + e], rscale[mi], csv[e]);
               const int row = mi * 32 + lr;
-              uint8_t* p = region + row * 256;
+              uint8_t* p = region + row * RB;
+              const int sw = sw_of(row);
               if constexpr (kOutBf16) {
                 uint2 w;
                 w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
                 w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
                 const int j = ncol_local >> 2;  // 8-byte chunk index
-                *reinterpret_cast<uint2*>(p + ((j ^ (row & 31)) * 8)) = w;
+                *reinterpret_cast<uint2*>(p + ((j ^ sw) * 8)) = w;
               } else {
                 const int j = ncol_local >> 1;  // two 8-byte chunks per 4 floats
-                *reinterpret_cast<float2*>(p + ((j ^ (row & 31)) * 8)) = make_float2(o[0], o[1]);
-                *reinterpret_cast<float2*>(p + (((j + 1) ^ (row & 31)) * 8)) = make_float2(o[2], o[3]);
+                *reinterpret_cast<float2*>(p + ((j ^ sw) * 8)) = make_float2(o[0], o[1]);
+                *reinterpret_cast<float2*>(p + (((j + 1) ^ sw) * 8)) = make_float2(o[2], o[3]);
               }
             }
           }
         }
         __syncthreads();
-        // read back: lane -> 16-byte pair (lane&15) of row (lane>>4) + 4*it
+        // read back: lane -> 16-byte pair (lane % LPR) of row (lane / LPR) + RPI*it
+        constexpr int LPR = RB / 16, RPI = 64 / LPR;
         const int64_t ncol_pass0 = ncol0 + (int64_t)pass * kNiPerPass * 32;
-        const int pair = lane & 15;
+        const int pair = lane % LPR, rsub = lane / LPR;
         const int64_t nn = ncol_pass0 + pair * kColsPerPair;
         const bool full = vec_store && (nn + kColsPerPair <= g.n);
-        uint8_t* dst0 = cbase + ((mrow0 + (lane >> 4)) * g.ldc + nn) * kEsz;
+        uint8_t* dst0 = cbase + ((mrow0 + rsub) * g.ldc + nn) * kEsz;
 #pragma unroll 8
-        for (int it = 0; it < 32; ++it) {
-          const int row = (lane >> 4) + 4 * it;
-          const int sw = row & 31;
-          uint4 v = *reinterpret_cast<const uint4*>(region + row * 256 + ((pair ^ (sw >> 1)) * 16));
+        for (int it = 0; it < 128 / RPI; ++it) {
+          const int row = rsub + RPI * it;
+          const int sw = sw_of(row);
+          uint4 v = *reinterpret_cast<const uint4*>(region + row * RB + ((pair ^ (sw >> 1)) * 16));
           if (sw & 1) v = make_uint4(v.z, v.w, v.x, v.y);
-          uint8_t* dst = dst0 + (int64_t)it * 4 * g.ldc * kEsz;
+          uint8_t* dst = dst0 + (int64_t)it * RPI * g.ldc * kEsz;
           if constexpr (!kChecked) {
             *reinterpret_cast<uint4*>(dst) = v;
           } else if (mrow0 + row < g.m && nn < g.n) {
@@ -444,16 +462,15 @@ __global__ void gemm_simple_kernel(const GemmArgs g) {
     for (int64_t kk = 0; kk < g.k; ++kk) facc = fmaf(DecA::decode(A[kk]), DecB::decode(B[kk]), facc);
     if (g.acc_out) reinterpret_cast<float*>(g.acc_out)[o] = facc;
   }
-  const int pbf = g.dq_bf16 & g.sc_bf16;
   float f = rnd(facc, g.dq_bf16);
   const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
   const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
   if (g.col_first) {
-    if (cs) f = rnd(f * cs[nn], pbf);
-    if (rs) f = rnd(f * rs[mm], pbf);
+    if (cs) f = rnd(f * cs[nn], g.p1_bf16);
+    if (rs) f = rnd(f * rs[mm], g.p2_bf16);
   } else {
-    if (rs) f = rnd(f * rs[mm], pbf);
-    if (cs) f = rnd(f * cs[nn], pbf);
+    if (rs) f = rnd(f * rs[mm], g.p1_bf16);
+    if (cs) f = rnd(f * cs[nn], g.p2_bf16);
   }
   f = rnd(f, g.dq_bf16);
   if (g.out_dtype == AQTX_BF16) reinterpret_cast<uint16_t*>(g.c)[o] = bf16_bits(f);
@@ -494,8 +511,16 @@ inline GemmArgs make_gemm_args(const aqtx_gemm_plan* p, const void* a, const voi
   g.stride_rs = p->row_scale_stride_b; g.stride_cs = p->col_scale_stride_b;
   g.out_dtype = p->out_dtype;
   g.dq_bf16 = p->dequant_dtype == AQTX_BF16;
-  g.sc_bf16 = p->scale_dtype == AQTX_BF16;
   g.col_first = p->scale_order == AQTX_SCALE_COL_THEN_ROW;
+  {
+    // jnp promotion, product by product: bf16 * bf16 -> bf16, anything with f32 -> f32 for good.
+    // A missing scale multiplies by 1 and changes nothing, so only its dtype's effect on the
+    // promotion matters; it is taken as given.
+    const bool first_bf = (g.col_first ? p->col_scale_dtype : p->row_scale_dtype) == AQTX_BF16;
+    const bool second_bf = (g.col_first ? p->row_scale_dtype : p->col_scale_dtype) == AQTX_BF16;
+    g.p1_bf16 = g.dq_bf16 && first_bf;
+    g.p2_bf16 = g.p1_bf16 && second_bf;
+  }
   g.tiles_m = (int)((p->m + BM - 1) / BM);
   g.tiles_n = (int)((p->n + BN - 1) / BN);
   return g;
@@ -509,8 +534,10 @@ inline bool gemm_vector_path_ok(const aqtx_gemm_plan* p, const void* a, const vo
 // Epilogue id for the (out, dequant, scale) dtype triple, or -1.
 inline int gemm_epilogue_id(const aqtx_gemm_plan* p) {
   if (p->out_dtype == AQTX_I32) return 3;
-  if (p->out_dtype == AQTX_BF16 && p->dequant_dtype == AQTX_BF16) return p->scale_dtype == AQTX_BF16 ? 0 : 1;
-  if (p->out_dtype == AQTX_F32 && p->dequant_dtype == AQTX_F32 && p->scale_dtype == AQTX_F32) return 2;
+  const bool first_bf = (p->scale_order == AQTX_SCALE_COL_THEN_ROW ? p->col_scale_dtype : p->row_scale_dtype) == AQTX_BF16;
+  const bool second_bf = (p->scale_order == AQTX_SCALE_COL_THEN_ROW ? p->row_scale_dtype : p->col_scale_dtype) == AQTX_BF16;
+  if (p->out_dtype == AQTX_BF16 && p->dequant_dtype == AQTX_BF16) return first_bf ? (second_bf ? 0 : 4) : 1;
+  if (p->out_dtype == AQTX_F32 && p->dequant_dtype == AQTX_F32) return 2;  // f32 * any scale stays f32
   return -1;
 }
 

@@ -10,11 +10,12 @@ namespace {
 template <class MMA>
 int launch_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
   // K tails are always masked here: fewer instantiations, and the mask is one compare per load.
-#define AQTX_LAUNCH(E, C) gemm_kernel<MMA, E, C, true><<<grid, 256, 0, st>>>(g)
+#define AQTX_LAUNCH(E, C) gemm_kernel<MMA, 4, E, C, true><<<grid, 256, 0, st>>>(g)
 #define AQTX_LAUNCH_C(E) do { if (g.col_first) AQTX_LAUNCH(E, true); else AQTX_LAUNCH(E, false); } while (0)
   switch (epi) {
     case 0: AQTX_LAUNCH_C(0); break;
     case 1: AQTX_LAUNCH_C(1); break;
+    case 4: AQTX_LAUNCH_C(4); break;
     default: AQTX_LAUNCH_C(2); break;
   }
 #undef AQTX_LAUNCH_C
@@ -55,7 +56,7 @@ extern "C" int aqtx_gemm_fp8(const aqtx_gemm_plan* p, const void* a, const void*
   const int epi = gemm_epilogue_id(p);
   if (epi < 0 || epi == 3)
     return set_error("aqtx_gemm_fp8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
-                     p->out_dtype, p->dequant_dtype, p->scale_dtype);
+                     p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
   if (!a5 && !b5) return launch_fp8<MmaF8<0, 0>>(g, epi, grid, st);
   if (!a5 && b5) return launch_fp8<MmaF8<0, 1>>(g, epi, grid, st);
   if (a5 && !b5) return launch_fp8<MmaF8<1, 0>>(g, epi, grid, st);

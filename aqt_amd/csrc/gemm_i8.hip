@@ -21,7 +21,8 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
                  "%s: out_dtype must be bf16, f32 or i32, got %d", who, p->out_dtype);
   }
   AQTX_REQUIRE(is_float_dtype(p->dequant_dtype), "%s: dequant_dtype must be bf16 or f32", who);
-  AQTX_REQUIRE(is_float_dtype(p->scale_dtype), "%s: scale_dtype must be bf16 or f32", who);
+  AQTX_REQUIRE(is_float_dtype(p->row_scale_dtype) && is_float_dtype(p->col_scale_dtype),
+               "%s: row_scale_dtype / col_scale_dtype must be bf16 or f32", who);
   AQTX_REQUIRE(p->scale_order == AQTX_SCALE_ROW_THEN_COL || p->scale_order == AQTX_SCALE_COL_THEN_ROW,
                "%s: unknown scale_order %d", who, p->scale_order);
   AQTX_REQUIRE(p->lda >= p->k && p->ldb >= p->k && p->ldc >= p->n,
@@ -62,9 +63,17 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   const int epi = gemm_epilogue_id(p);
   if (epi < 0)
     return set_error("aqtx_gemm_i8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
-                     p->out_dtype, p->dequant_dtype, p->scale_dtype);
+                     p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
   const bool ktail = (p->k % (2 * BK)) != 0;
-#define AQTX_LAUNCH(E, C, T) gemm_kernel<MmaI8, E, C, T><<<grid, 256, 0, st>>>(g)
+  // Two waves per SIMD by default: measured faster on every shape tried (the epilogue of one
+  // wave overlaps the other's work).  AQTX_GEMM_WAVES=4|8 overrides it per call (tests, tuning).
+  const char* waves_env = getenv("AQTX_GEMM_WAVES");
+  const int waves = (waves_env != nullptr && atoi(waves_env) == 4) ? 4 : 8;
+#define AQTX_LAUNCH(E, C, T)                                             \
+  do {                                                                  \
+    if (waves == 8) gemm_kernel<MmaI8, 8, E, C, T><<<grid, 512, 0, st>>>(g); \
+    else gemm_kernel<MmaI8, 4, E, C, T><<<grid, 256, 0, st>>>(g);       \
+  } while (0)
 #define AQTX_LAUNCH_T(E, C) \
   do { if (ktail) AQTX_LAUNCH(E, C, true); else AQTX_LAUNCH(E, C, false); } while (0)
 #define AQTX_LAUNCH_C(E) \
@@ -73,6 +82,7 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
     case 0: AQTX_LAUNCH_C(0); break;
     case 1: AQTX_LAUNCH_C(1); break;
     case 2: AQTX_LAUNCH_C(2); break;
+    case 4: AQTX_LAUNCH_C(4); break;
     default: AQTX_LAUNCH_T(3, false); break;
   }
 #undef AQTX_LAUNCH_C

@@ -173,6 +173,8 @@ def gemm(
     out_dtype,
     dequant_dtype=None,
     scale_dtype=None,
+    row_scale_dtype=None,
+    col_scale_dtype=None,
     scale_order: int = L.SCALE_ROW_THEN_COL,
     a_dtype: int = L.I8,
     b_dtype: int = L.I8,
@@ -181,7 +183,9 @@ def gemm(
   """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
 
   int8 operands use the int32 MFMA path, fp8 operands (uint8 tensors holding
-  e4m3fn/e5m2 bytes) the float32 one.  Returns C, or (C, acc) with want_acc.
+  e4m3fn/e5m2 bytes) the float32 one.  `scale_dtype` names the dtype of both scale
+  vectors; row_scale_dtype / col_scale_dtype override it per side.  Returns C, or
+  (C, acc) with want_acc.
   """
   _require_gpu(a, b, row_scale, col_scale)
   assert a.dim() == 3 and b.dim() == 3 and a.shape[0] == b.shape[0] and a.shape[2] == b.shape[2]
@@ -201,7 +205,9 @@ def gemm(
   plan.lda, plan.ldb, plan.ldc = a.stride(1), b.stride(1), n
   plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), b.stride(0), m * n
   plan.a_dtype, plan.b_dtype = a_dtype, b_dtype
-  plan.out_dtype, plan.dequant_dtype, plan.scale_dtype = out_dt, dq_dt, sc_dt
+  plan.out_dtype, plan.dequant_dtype = out_dt, dq_dt
+  plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else sc_dt
+  plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else sc_dt
   plan.scale_order = scale_order
   for s, dim in ((row_scale, m), (col_scale, n)):
     if s is not None:
@@ -213,6 +219,38 @@ def gemm(
     L.check(fn(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale), _ptr(col_scale), _ptr(c),
                _ptr(acc), _stream()))
   return (c, acc) if want_acc else c
+
+
+def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
+           clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False):
+  """Serving contraction out = dequant(quant(x) @ w_q^T) for x [m <= 64, k], w_q int8 [n, k].
+
+  The activations get per-token dynamic int8 quantisation; `w_scale` is float32 [n] holding
+  values of `w_scale_dtype`.  Returns (out [m, n] of x.dtype, x_scale float32 [m]) and, with
+  want_xq, the quantized activations as a third element.
+  """
+  _require_gpu(x, w_q, w_scale)
+  assert x.dim() == 2 and w_q.dim() == 2 and x.shape[1] == w_q.shape[1], (x.shape, w_q.shape)
+  assert x.is_contiguous() and w_q.is_contiguous() and w_q.dtype == torch.int8
+  m, k = x.shape
+  n = w_q.shape[0]
+  assert w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() == n
+  plan = L.DecodePlan()
+  plan.m, plan.n, plan.k = m, n, k
+  plan.x_dtype = aqtx_dtype(x.dtype)
+  plan.x_scale_dtype = aqtx_dtype(x_scale_dtype if x_scale_dtype is not None else x.dtype)
+  plan.w_scale_dtype = aqtx_dtype(w_scale_dtype)
+  plan.out_dtype = plan.x_dtype
+  plan.quant_bound, plan.clip_bound = float(quant_bound), float(clip_bound)
+  ws_bytes = int(L.lib().aqtx_decode_workspace_bytes(ctypes.byref(plan)))
+  ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
+  out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+  x_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+  xq = torch.empty((m, k), dtype=torch.int8, device=x.device) if want_xq else None
+  with _timed('decode'):
+    L.check(L.lib().aqtx_decode_i8(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(xq),
+                                   _ptr(x_scale), _ptr(out), _ptr(ws), ws_bytes, _stream()))
+  return (out, x_scale, xq) if want_xq else (out, x_scale)
 
 
 def prng_split(key, num: int, partitionable: bool = False) -> np.ndarray:

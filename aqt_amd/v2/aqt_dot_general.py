@@ -463,6 +463,11 @@ class DotGeneralRaw:
     lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
     rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
 
+    served = self._serve_small_batch(lhs, lhs_dtype, dq, lhs_qt, rhs_arr, rhs_qt, dn, prescale_t,
+                                     out_transpose_axes, dequant_dtype, dimension_numbers)
+    if served is not None:
+      return served
+
     # ---- lhs ---------------------------------------------------------------------
     lq, ls, lsdt, lhs_qt_out, lhs_grad = self._quant_side(
         'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t)
@@ -489,7 +494,6 @@ class DotGeneralRaw:
     # scales: [B, M] / [B, N] or a single per-tensor value (broadcast here, tiny)
     def expand(s, n):
       return s.reshape(1, 1).expand(B, n).contiguous() if s.numel() == 1 and B * n != 1 else s.reshape(B, n)
-    sdt = torch.promote_types(lsdt, rsdt)
     if self.dot_general is not lax_dot_general:
       raise NotImplementedError('a custom DotGeneralRaw.dot_general hook is not lowered')
     nb, nl, nr = len(lba), len(lra), len(rra)
@@ -500,15 +504,15 @@ class DotGeneralRaw:
     swap_perm = list(range(nb)) + list(range(nb + nl, nb + nl + nr)) + list(range(nb, nb + nl))
     swapped = (out_transpose_axes is not None and list(out_transpose_axes) == swap_perm
                and want_lba == lba and nl > 0 and nr > 0)
-    common = dict(out_dtype=dequant_dtype, dequant_dtype=dequant_dtype, scale_dtype=sdt)
+    common = dict(out_dtype=dequant_dtype, dequant_dtype=dequant_dtype)
     if swapped:
       # C^T = rhs_q . lhs_q^T; the lhs scale still multiplies first (aqt_tensor.py:182-183)
       out = ops.gemm(rq, lq, row_scale=expand(rs, N), col_scale=expand(ls, M), a_dtype=rkd, b_dtype=lkd,
-                     scale_order=L.SCALE_COL_THEN_ROW, **common)
+                     scale_order=L.SCALE_COL_THEN_ROW, row_scale_dtype=rsdt, col_scale_dtype=lsdt, **common)
       out = out.reshape(bdims + rdims + ldims)
     else:
       out = ops.gemm(lq, rq, row_scale=expand(ls, M), col_scale=expand(rs, N), a_dtype=lkd, b_dtype=rkd,
-                     **common)
+                     row_scale_dtype=lsdt, col_scale_dtype=rsdt, **common)
       # [B, M, N] -> (batch..., lhs remaining..., rhs remaining...) in the caller's batch order
       out = out.reshape(bdims + ldims + rdims)
       if want_lba != lba:
@@ -521,6 +525,52 @@ class DotGeneralRaw:
     rhs_mt = MultiTensor(x=rhs_arr if not rhs_is_q else rhs.qvalue, qx=rhs_qt_out)
     res = DotGeneralRes(lhs=TensorRes(mt=lhs_mt, quant_grad=lhs_grad),
                         rhs=TensorRes(mt=rhs_mt, quant_grad=rhs_grad))
+    return out, res
+
+  def _serve_small_batch(self, lhs, lhs_dtype, dq, lhs_qt, rhs_arr, rhs_qt, dn, prescale_t,
+                         out_transpose_axes, dequant_dtype, dimension_numbers):
+    """Serving with a frozen int8 rhs and at most 64 lhs rows: the fused decode kernel.
+
+    Same arithmetic as the general path (per-token abs-max int8 quantisation of the lhs, int32
+    contraction, QTensor.dequant); returns None when the call does not have that shape.
+    """
+    (lca, rca), (lba, rba) = dn
+    if (rhs_qt is None or not rhs_qt.is_full() or lhs_qt is not None or prescale_t is not None
+        or out_transpose_axes is not None or lba or rba or self.dot_general is not lax_dot_general):
+      return None
+    spec = dq.lhs.kernel_spec()
+    if (spec is None or spec['out_dtype'] != L.I8 or spec['noise'] != L.NOISE_NONE
+        or dq.lhs.calib_shared_axes is not None or getattr(dq.lhs.numerics, 'clip_gradient', False)):
+      return None
+    if (rhs_qt.qvalue.dtype != torch.int8 or len(rhs_qt.scale) != 1 or rhs_qt.bias
+        or rhs_qt.container_dtype is not None or dequant_dtype != lhs.dtype
+        or self.dg_accumulator_dtype != utils.int32):
+      return None
+    lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
+    rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
+    lv = lowering.view_operand(lhs, [], lra, lca)
+    rv = lowering.view_operand(rhs_qt.qvalue, [], rra, rca)
+    if not (lv.k_last and rv.k_last) or lv.copied or rv.copied:
+      return None
+    M, K, N = lv.R, lv.K, rv.R
+    if M == 0 or M > 64 or K == 0 or K % 16 != 0 or N == 0 or N * K >= 2 ** 31:
+      return None
+    w_scale = rhs_qt.scale[0]
+    sv = lowering.view_operand(w_scale, [], rra, rca)
+    if sv.mem.numel() != N:
+      return None
+    sdt = dq.lhs._calibrator.dtype if dq.lhs._calibrator.dtype is not None else lhs_dtype
+    out, xs, xq = ops.decode(lv.mem[0], rv.mem[0], sv.mem.reshape(-1).float().contiguous(),
+                             quant_bound=spec['quant_bound'], clip_bound=spec['clip_bound'],
+                             x_scale_dtype=sdt, w_scale_dtype=w_scale.dtype, want_xq=True)
+    out = out.reshape([lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
+    qv = lowering.logical_from_brk(xq[None], lv)
+    sc = lowering.logical_from_brk(xs.reshape(1, M), lv, k_keep=False).to(sdt)
+    lhs_qt_out = aqt_tensor.QTensor(qvalue=qv, scale=[sc], scale_t=None, bias=[], dequant_dtype=lhs_dtype)
+    lhs_grad = functools.partial(dq.lhs.numerics.vjp_bwd, (None,))
+    rhs_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
+    res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=lhs, qx=lhs_qt_out), quant_grad=lhs_grad),
+                        rhs=TensorRes(mt=MultiTensor(x=rhs_arr, qx=rhs_qt), quant_grad=rhs_grad))
     return out, res
 
   def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t):

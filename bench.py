@@ -70,12 +70,58 @@ def cpu_baseline(seconds_budget=20.0):
   }
 
 
+def decode_bench(dev):
+  """Serving shapes (rhs frozen as int8 + f32 per-channel scale, K = 4096): device time per call of
+  aqtx_decode_i8 (activation quantisation + contraction + dequantisation) and the HBM rate on the
+  algorithmic bytes K*N + 4N + 2MK + 2MN.  Weight copies rotate through >= 1 GiB so that no cache
+  level can hold them; the calls are replayed from a HIP graph so that host launch overhead does
+  not sit between the kernels being timed."""
+  import torch
+  from aqt_amd import ops
+  k = 4096
+  rows = []
+  for n in (4096, 14336):
+    ncopies = (1 << 30) // (n * k) + 1
+    weights = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(ncopies)]
+    w_scale = torch.rand(n, device=dev) * 1e-3 + 1e-5
+    for m in (1, 8, 32, 64):
+      x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+      run = lambda: [ops.decode(x, w, w_scale, quant_bound=127.5, clip_bound=127.0) for w in weights]
+      run()
+      torch.cuda.synchronize()
+      side = torch.cuda.Stream()
+      graph = torch.cuda.CUDAGraph()
+      with torch.cuda.stream(side):
+        run()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+          keep = run()
+      torch.cuda.synchronize()
+      graph.replay()
+      torch.cuda.synchronize()
+      reps = 5
+      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      a.record()
+      for _ in range(reps):
+        graph.replay()
+      b.record()
+      torch.cuda.synchronize()
+      us = a.elapsed_time(b) * 1e3 / (reps * ncopies)
+      nbytes = k * n + 4 * n + 2 * m * k + 2 * m * n
+      rows.append({'n': n, 'm': m, 'us_per_call': round(us, 2), 'GB/s': round(nbytes / us / 1e3, 1),
+                   'frac_of_8TBps': round(nbytes / us / 1e3 / 8000.0, 3)})
+      del graph, keep
+    del weights
+  return rows
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--gpus', type=int, default=1)
   ap.add_argument('--steps', type=int, default=20)
   ap.add_argument('--warmup', type=int, default=3)
   ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--no-decode', action='store_true', help='skip the serving-shape (decode) measurements')
   ap.add_argument('--calibration-copy', action='store_true',
                   help='also launch one elementwise kernel that reads and writes 256 MiB, as the '
                        'known-size reference for FETCH_SIZE / WRITE_SIZE counter runs')
@@ -137,6 +183,9 @@ def main():
                    'frac': achieved * 1e12 / INT8_MFMA_PEAK, 'traffic': GEMM_TRAFFIC_BYTES_PER_LAUNCH,
                    'launch_ms': gemm_ms, 'launches_timed': len(timer.pairs)},
   }
+  if not args.no_decode:
+    line['decode'] = {'kernel': 'aqtx_decode_i8 (quant_rows + decode_ksplit/decode_block)', 'k': 4096,
+                      'timing': 'HIP graph replay, weights rotated through 1 GiB', 'shapes': decode_bench(dev)}
   if not args.no_cpu_baseline:
     line['cpu_baseline'] = cpu_baseline()
   print(json.dumps(line))

@@ -134,7 +134,8 @@ typedef struct aqtx_gemm_plan {
   int32_t a_dtype, b_dtype;   /* AQTX_I8 | AQTX_I4 (container) | AQTX_E4M3 | AQTX_E5M2       */
   int32_t out_dtype;          /* AQTX_BF16 | AQTX_F32 | AQTX_I32 (raw accumulator, no scales) */
   int32_t dequant_dtype;      /* AQTX_BF16 | AQTX_F32: dtype the accumulator is cast to first */
-  int32_t scale_dtype;        /* AQTX_BF16 | AQTX_F32: dtype of the scale arrays             */
+  int32_t row_scale_dtype;    /* AQTX_BF16 | AQTX_F32: dtype of the values in row_scale      */
+  int32_t col_scale_dtype;    /* AQTX_BF16 | AQTX_F32: dtype of the values in col_scale      */
   int32_t scale_order;        /* AQTX_SCALE_*: which scale multiplies first                  */
   int64_t row_scale_stride_b, col_scale_stride_b; /* batch strides of the scale vectors    */
 } aqtx_gemm_plan;
@@ -145,8 +146,9 @@ typedef struct aqtx_gemm_plan {
  * (aqt/jax/v2/aqt_dot_general.py:843-958, the lax.dot_general call at :921-927
  * with preferred_element_type=int32) followed by QTensor.dequant
  * (aqt_tensor.py:161-200): out = cast(acc) * first_scale * second_scale, each
- * product rounded to promote(dequant_dtype, scale_dtype), final cast to
- * out_dtype.
+ * product rounded to the promoted dtype of its two operands (so a bf16 value
+ * times a bf16 scale rounds to bf16, and anything times an f32 scale stays
+ * f32 from then on), final cast to out_dtype.
  *   row_scale : float32 [batch][m] or NULL (= no scale on that side)
  *   col_scale : float32 [batch][n] or NULL
  *   acc_out   : optional int32 [batch][m][n] copy of the raw accumulators

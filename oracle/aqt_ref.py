@@ -265,6 +265,9 @@ class QTensor:
   scale_dtype: Optional[str]
   dequant_dtype: str
   bias: list = dataclasses.field(default_factory=list)
+  # dtype of each scale when they differ (a bf16 activation scale next to an f32 weight scale in
+  # serving); None = all scales have scale_dtype.
+  scale_dtypes: Optional[list] = None
 
 
 def ceil_to_po2(scale, dt):
@@ -344,8 +347,9 @@ def dequant(qt: QTensor):
   else:
     ret = nm.cast(qt.qvalue, dd)
   rdt = dd
-  for s in qt.scale:
-    rdt = nm.promote(rdt, qt.scale_dtype or dd)
+  for i, s in enumerate(qt.scale):
+    sdt = qt.scale_dtypes[i] if qt.scale_dtypes else (qt.scale_dtype or dd)
+    rdt = nm.promote(rdt, sdt)  # jnp promotion of `ret * scale`, product by product
     ret = nm.cast(ret * s, rdt)
   return nm.cast(ret, dd)
 
@@ -486,17 +490,18 @@ def qtensor_dot_general(lhs_qt: QTensor, rhs_qt: QTensor, dn, raw: RawCfg, dequa
       odt = F32 if F32 in fl else BF16
     out = nm.cast(lax_dot_general(lq, rq, dn, np.float32), odt)
 
-  scales = []
-  sdt = None
+  # Each scale keeps its own dtype: dequant multiplies them in one by one and jnp promotes
+  # product by product (a bf16 lhs scale next to an f32 rhs scale rounds the first product only).
+  scales, sdts = [], []
   if raw.lhs_dequant_mode == 'output':
-    for s in lhs_qt.scale:
+    for i, s in enumerate(lhs_qt.scale):
       scales.append(lhs_scale_transpose_to_output(s, dn, lq.shape, rq.shape))
-      sdt = lhs_qt.scale_dtype
+      sdts.append(lhs_qt.scale_dtypes[i] if lhs_qt.scale_dtypes else (lhs_qt.scale_dtype or dequant_dtype))
   if raw.rhs_dequant_mode == 'output':
-    for s in rhs_qt.scale:
+    for i, s in enumerate(rhs_qt.scale):
       scales.append(rhs_scale_transpose_to_output(s, dn, lq.shape, rq.shape))
-      sdt = nm.promote(sdt, rhs_qt.scale_dtype) if sdt else rhs_qt.scale_dtype
-  return QTensor(out, odt, scales, sdt, dequant_dtype)
+      sdts.append(rhs_qt.scale_dtypes[i] if rhs_qt.scale_dtypes else (rhs_qt.scale_dtype or dequant_dtype))
+  return QTensor(out, odt, scales, None, dequant_dtype, scale_dtypes=sdts or None)
 
 
 def _apply_local_aqt(shard_count, lhs, rhs, dn):

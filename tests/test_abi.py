@@ -93,7 +93,7 @@ def _gplan(**kw):
   p.batch, p.m, p.n, p.k = 1, 64, 64, 64
   p.lda = p.ldb = p.ldc = 64
   p.a_dtype = p.b_dtype = L.I8
-  p.out_dtype = p.dequant_dtype = p.scale_dtype = L.BF16
+  p.out_dtype = p.dequant_dtype = p.row_scale_dtype = p.col_scale_dtype = L.BF16
   for k, v in kw.items():
     setattr(p, k, v)
   return p
@@ -104,7 +104,8 @@ def _gplan(**kw):
     (dict(a_dtype=L.F32), 'operands'),
     (dict(out_dtype=L.I8), 'out_dtype'),
     (dict(dequant_dtype=L.I8), 'dequant_dtype'),
-    (dict(scale_dtype=L.I32), 'scale_dtype'),
+    (dict(row_scale_dtype=L.I32), 'row_scale_dtype'),
+    (dict(col_scale_dtype=L.I8), 'col_scale_dtype'),
     (dict(scale_order=3), 'scale_order'),
     (dict(lda=32), 'leading dimension'),
     (dict(out_dtype=L.F32, dequant_dtype=L.BF16), 'combination'),
@@ -143,3 +144,41 @@ def test_cpu_tensors_are_rejected():
   x = torch.zeros((1, 4, 64), dtype=torch.bfloat16)
   with pytest.raises(RuntimeError, match='no CPU fallback'):
     ops.quantize(x, reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0)
+
+
+def _dplan(**kw):
+  p = L.DecodePlan()
+  p.m, p.n, p.k = 8, 256, 512
+  p.x_dtype = p.x_scale_dtype = p.out_dtype = L.BF16
+  p.w_scale_dtype = L.F32
+  p.quant_bound, p.clip_bound = 127.5, 127.0
+  for k, v in kw.items():
+    setattr(p, k, v)
+  return p
+
+
+@pytest.mark.parametrize('kw,needle', [
+    (dict(m=65), 'exceeds 64'),
+    (dict(k=24), 'multiple of 16'),
+    (dict(k=0), 'multiple of 16'),
+    (dict(n=-1), 'negative'),
+    (dict(x_dtype=L.I8), 'dtypes'),
+    (dict(quant_bound=0.0), 'bounds'),
+    (dict(n=1 << 20, k=4096), '2 GiB'),
+])
+def test_decode_plan_validation(kw, needle):
+  p = _dplan(**kw)
+  rc = L.lib().aqtx_decode_i8(ctypes.byref(p), FAKE, FAKE, FAKE, None, FAKE, FAKE, FAKE, 1 << 30, None)
+  msg = _err(rc)
+  assert needle in msg, msg
+
+
+def test_decode_workspace_and_null_checks():
+  p = _dplan()
+  need = L.lib().aqtx_decode_workspace_bytes(ctypes.byref(p))
+  assert need >= 8 * 512 and need % 256 == 0
+  assert L.lib().aqtx_decode_workspace_bytes(ctypes.byref(_dplan(m=65))) == 0
+  assert 'NULL' in _err(L.lib().aqtx_decode_i8(ctypes.byref(p), None, FAKE, FAKE, None, FAKE, FAKE, FAKE, need, None))
+  assert 'workspace' in _err(L.lib().aqtx_decode_i8(ctypes.byref(p), FAKE, FAKE, FAKE, None, FAKE, FAKE, FAKE, 16, None))
+  # empty problems succeed without touching the GPU
+  assert L.lib().aqtx_decode_i8(ctypes.byref(_dplan(m=0)), None, None, None, None, None, None, None, 0, None) == 0

@@ -1,0 +1,82 @@
+"""GPU parity: aqtx_decode_i8 (serving with a frozen int8 weight) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from aqt_amd import ops
+from oracle import aqt_ref as R
+from oracle import numerics as nm
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_decode(x, dt, wq, w_scale, w_sdt):
+  """quant(x) per token, int32 contraction, QTensor.dequant with [x scale, w scale]."""
+  q = R.QuantizerCfg(bits=8)
+  xqt = R.quantize(x, dt, q, calibration_axes=[1])
+  acc = (xqt.qvalue.astype(np.int64) @ wq.astype(np.int64).T).astype(np.int32)
+  xs = xqt.scale[0].reshape(-1, 1)
+  out = R.dequant(R.QTensor(acc, 'i32', [xs, w_scale.reshape(1, -1)], None, dt,
+                            scale_dtypes=[xqt.scale_dtype, w_sdt]))
+  return out, xqt.qvalue.astype(np.int8), xqt.scale[0].reshape(-1)
+
+
+def _weights(n, k, seed, w_sdt):
+  rng = np.random.default_rng(seed)
+  wq = rng.integers(-127, 128, size=(n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(2e-4) + np.float32(1e-5), w_sdt)
+  return wq, ws
+
+
+@pytest.mark.parametrize('m', [1, 3, 8, 16, 17, 32, 40, 64])
+@pytest.mark.parametrize('n,k', [(256, 1024), (200, 464), (4096, 4096)])
+@pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('bf16', 'bf16'), ('f32', 'f32')])
+def test_decode_matches_oracle(gpu, m, n, k, dt, w_sdt):
+  if (n, k) == (4096, 4096) and (dt, w_sdt) != ('bf16', 'f32'):
+    pytest.skip('large shape once')
+  x = U.rand((m, k), dt, 100 + m, outliers=True)
+  wq, ws = _weights(n, k, 7, w_sdt)
+  want, xq_want, xs_want = _oracle_decode(x, dt, wq, ws, w_sdt)
+  out, xs, xq = ops.decode(U.to_dev(x, dt, gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
+                           quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True)
+  np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
+  np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize('m', [20, 64])
+def test_decode_wide_weight(gpu, m):
+  """n >= 12288 takes the 64-rows-per-workgroup shape; k is not a multiple of the 256-byte chunk."""
+  n, k = 12352 + 24, 336
+  x = U.rand((m, k), 'bf16', 5)
+  wq, ws = _weights(n, k, 9, 'f32')
+  want, _, _ = _oracle_decode(x, 'bf16', wq, ws, 'f32')
+  out, _ = ops.decode(U.to_dev(x, 'bf16', gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
+                      quant_bound=127.5, clip_bound=127.0)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+
+
+def test_decode_equals_quantize_plus_gemm(gpu):
+  """Same result as the training-shape kernels on the same operands."""
+  from aqt_amd import _lib as L
+  m, n, k = 64, 512, 4096
+  x = U.to_dev(U.rand((m, k), 'bf16', 3), 'bf16', gpu)
+  wq, ws = _weights(n, k, 4, 'bf16')
+  wq_t, ws_t = torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu)
+  out, xs = ops.decode(x, wq_t, ws_t, quant_bound=127.5, clip_bound=127.0, w_scale_dtype=torch.bfloat16)
+  xq, xs2 = ops.quantize(x[None], reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0)
+  ref = ops.gemm(xq, wq_t[None], row_scale=xs2.reshape(1, m), col_scale=ws_t.reshape(1, n),
+                 out_dtype=torch.bfloat16, scale_dtype=torch.bfloat16)
+  assert torch.equal(xs, xs2.reshape(-1))
+  assert torch.equal(out, ref[0])
+
+
+def test_decode_rejects_bad_plans(gpu):
+  x = torch.zeros((65, 64), dtype=torch.bfloat16, device=gpu)
+  w = torch.zeros((16, 64), dtype=torch.int8, device=gpu)
+  s = torch.ones(16, device=gpu)
+  with pytest.raises(Exception, match='exceeds 64'):
+    ops.decode(x, w, s, quant_bound=127.5, clip_bound=127.0)
+  with pytest.raises(Exception, match='multiple of 16'):
+    ops.decode(x[:4, :24].contiguous(), w[:, :24].contiguous(), s, quant_bound=127.5, clip_bound=127.0)

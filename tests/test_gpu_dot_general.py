@@ -130,6 +130,30 @@ def test_serving_with_frozen_rhs(gpu):
   np.testing.assert_array_equal(_np(out1), f.out)
 
 
+@pytest.mark.parametrize('m', [1, 8, 33, 64, 100])
+@pytest.mark.parametrize('w_sdt', ['bf16', 'f32'])
+def test_serving_scale_dtypes_and_batch_sizes(gpu, m, w_sdt):
+  """Frozen rhs whose scale is bf16 or f32 (jnp promotes product by product in dequant);
+  m <= 64 takes the fused decode kernel, m = 100 the quantize + GEMM kernels."""
+  import dataclasses
+  dt = 'bf16'
+  lhs, rhs = U.rand((m, 512), dt, 1, outliers=True), U.rand((512, 384), dt, 2, 0.02)
+  cfg = config.set_context(config.fully_quantized(), prng.prng_key(0), None)
+  L, Rr = U.to_dev(lhs, dt, gpu), U.to_dev(rhs, dt, gpu)
+  _, (_, rqt) = cfg.dg_core(L, Rr, None, None, MATMUL)
+  rqt = dataclasses.replace(rqt, scale=[rqt.scale[0].to(U.TORCH_DT[w_sdt])])
+  out, (lqt, _) = cfg.dg_core(L, torch.zeros_like(Rr), None, rqt, MATMUL)
+  # oracle: same quantizers, dequant with [lhs scale (bf16), rhs scale (w_sdt)]
+  ocfg = R.fully_quantized()
+  f = R.dg_fwd(lhs, rhs, dt, MATMUL, ocfg)
+  lq, rq = f.lhs_res.qx, f.rhs_res.qx
+  acc = (lq.qvalue.astype(np.int64) @ rq.qvalue.astype(np.int64)).astype(np.int32)
+  want = R.dequant(R.QTensor(acc, 'i32', [lq.scale[0], rq.scale[0]], None, dt, scale_dtypes=['bf16', w_sdt]))
+  np.testing.assert_array_equal(_np(lqt.qvalue), lq.qvalue.astype(np.float32))
+  np.testing.assert_array_equal(_np(lqt.scale[0]), lq.scale[0])
+  np.testing.assert_array_equal(_np(out), want)
+
+
 def test_reference_assertions(gpu):
   cfg = config.fully_quantized()
   L = torch.zeros((4, 8), dtype=torch.int8, device=gpu)

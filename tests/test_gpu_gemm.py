@@ -12,6 +12,13 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=[4, 8], ids=['waves4', 'waves8'])
+def waves(request, monkeypatch):
+  """Both workgroup shapes of the int8 MFMA kernel."""
+  monkeypatch.setenv('AQTX_GEMM_WAVES', str(request.param))
+  return request.param
+
+
 def _ints(shape, seed):
   return np.random.default_rng(seed).integers(-127, 128, size=shape).astype(np.int8)
 
@@ -27,7 +34,7 @@ SHAPES = [
 
 
 @pytest.mark.parametrize('batch,m,n,k', SHAPES)
-def test_raw_accumulators(gpu, batch, m, n, k):
+def test_raw_accumulators(gpu, waves, batch, m, n, k):
   a, b = _ints((batch, m, k), 1), _ints((batch, n, k), 2)
   c = ops.gemm(torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu), row_scale=None,
                col_scale=None, out_dtype=torch.int32)
@@ -38,7 +45,7 @@ def test_raw_accumulators(gpu, batch, m, n, k):
 @pytest.mark.parametrize('sdt', ['bf16', 'f32'])
 @pytest.mark.parametrize('order', [L.SCALE_ROW_THEN_COL, L.SCALE_COL_THEN_ROW])
 @pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 4096), (2, 100, 72, 160), (1, 33, 20, 23)])
-def test_dequant_epilogue(gpu, batch, m, n, k, order, sdt, out):
+def test_dequant_epilogue(gpu, waves, batch, m, n, k, order, sdt, out):
   if out == 'f32' and sdt == 'bf16':
     pytest.skip('scale dtype never narrower than the dequant dtype in the reference')
   a, b = _ints((batch, m, k), 3), _ints((batch, n, k), 4)
@@ -57,7 +64,27 @@ def test_dequant_epilogue(gpu, batch, m, n, k, order, sdt, out):
   np.testing.assert_array_equal(c.float().cpu().numpy(), want)
 
 
-def test_large_accumulators_round_like_xla(gpu):
+@pytest.mark.parametrize('rdt,cdt', [('bf16', 'f32'), ('f32', 'bf16')])
+@pytest.mark.parametrize('order', [L.SCALE_ROW_THEN_COL, L.SCALE_COL_THEN_ROW])
+@pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 512), (2, 100, 72, 160)])
+def test_dequant_epilogue_mixed_scale_dtypes(gpu, batch, m, n, k, order, rdt, cdt):
+  """A bf16 and an f32 scale: only a first product of two bf16 values is rounded to bf16."""
+  a, b = _ints((batch, m, k), 3), _ints((batch, n, k), 4)
+  rs = nm.cast(np.abs(U.rand((batch, m), 'f32', 5, 0.03)) + np.float32(1e-3), rdt)
+  cs = nm.cast(np.abs(U.rand((batch, n), 'f32', 6, 6e-4)) + np.float32(1e-5), cdt)
+  acc = _ref_acc(a, b).astype(np.int32)
+  scales, sdts = [rs[:, :, None], cs[:, None, :]], [rdt, cdt]
+  if order == L.SCALE_COL_THEN_ROW:
+    scales, sdts = scales[::-1], sdts[::-1]
+  want = R.dequant(R.QTensor(acc, 'i32', scales, None, 'bf16', scale_dtypes=sdts))
+  c = ops.gemm(torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu),
+               row_scale=torch.from_numpy(rs).to(gpu), col_scale=torch.from_numpy(cs).to(gpu),
+               out_dtype=torch.bfloat16, row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt],
+               scale_order=order)
+  np.testing.assert_array_equal(c.float().cpu().numpy(), want)
+
+
+def test_large_accumulators_round_like_xla(gpu, waves):
   """|acc| > 2**24: int32 -> f32 -> bf16 double rounding is part of the contract."""
   k = 4096
   a = np.full((1, 256, k), 127, np.int8)
