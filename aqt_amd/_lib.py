@@ -68,6 +68,7 @@ SYMBOLS = {
     'aqtx_decode_i8': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
+    'aqtx_sum_tiles': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),
     'aqtx_prng_split_host': (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint32), ctypes.c_int32,
                                             ctypes.c_int32, ctypes.POINTER(ctypes.c_uint32)]),
     'aqtx_random_bits': (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint32), ctypes.c_int64,

@@ -253,6 +253,17 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   return (out, x_scale, xq) if want_xq else (out, x_scale)
 
 
+def sum_tiles(x: torch.Tensor) -> torch.Tensor:
+  """Sum over the leading axis of a contiguous bf16/f32 tensor: float32 accumulation in index
+  order, one rounding (jnp.sum semantics for the per-tile outputs of a tiled dot_general)."""
+  _require_gpu(x)
+  assert x.is_contiguous() and x.dim() >= 1
+  tiles = x.shape[0]
+  out = torch.empty(x.shape[1:], dtype=x.dtype, device=x.device)
+  L.check(L.lib().aqtx_sum_tiles(_ptr(x), _ptr(out), tiles, out.numel(), aqtx_dtype(x.dtype), _stream()))
+  return out
+
+
 def prng_split(key, num: int, partitionable: bool = False) -> np.ndarray:
   """jax.random.split(key, num) on raw uint32[2] key data (host side)."""
   k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))

@@ -38,6 +38,21 @@ class _Int4:
   def __repr__(self):
     return 'int4'
 
+  # One object stands for the dtype: configurations are deep-copied (set_context), and
+  # `dtype is utils.int4` must keep holding for the copies.
+  def __copy__(self):
+    return self
+
+  def __deepcopy__(self, memo):
+    return self
+
+  def __reduce__(self):
+    return (_int4_singleton, ())
+
+
+def _int4_singleton():
+  return int4
+
 
 # dtype names the reference takes from jax.numpy
 int4 = _Int4()

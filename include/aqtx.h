@@ -168,6 +168,15 @@ int aqtx_gemm_fp8(const aqtx_gemm_plan* plan, const void* a, const void* b,
                   float* acc_out, void* stream);
 
 /*
+ * aqtx_sum_tiles: out[i] = cast(sum over t of x[t][i]) for x [tiles][count] of
+ * bf16 or f32, accumulated in float32 in tile order and rounded once.  Replaces
+ * the sum over the tile-count axes of the per-tile (already dequantized) outputs
+ * in tiled_dot_general (aqt/jax/v2/tiled_dot_general.py:493).
+ */
+int aqtx_sum_tiles(const void* x, void* out, int64_t tiles, int64_t count, int32_t dtype,
+                   void* stream);
+
+/*
  * Plan of the serving contraction out[m, n] = dequant(quant(x)[m, k] * W[n, k]^T)
  * with a pre-quantized weight (QTensor: int8 qvalue + per-output-channel scale)
  * and per-token dynamic int8 quantisation of the activations, m <= 64.

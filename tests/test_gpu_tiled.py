@@ -1,0 +1,68 @@
+"""GPU parity: tiled (subchannel) dot_general through the product kernels against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from aqt_amd import ops
+from aqt_amd.v2 import aqt_dot_general as aqt
+from aqt_amd.v2 import config
+from aqt_amd.v2 import tiled_dot_general as T
+from oracle import aqt_ref as R
+from oracle import numerics as nm
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+MATMUL = (((1,), (0,)), ((), ()))
+
+
+@pytest.mark.parametrize('dt', ['bf16', 'f32'])
+@pytest.mark.parametrize('tiles,count', [(1, 64), (5, 4096), (64, 1000), (3, 1001), (7, 13)])
+def test_sum_tiles(gpu, tiles, count, dt):
+  x = U.rand((tiles, count), dt, 3, scale=3.0)
+  want = np.zeros(count, np.float32)
+  for t in range(tiles):
+    want = want + x[t]
+  want = nm.cast(want, dt)
+  got = ops.sum_tiles(U.to_dev(x, dt, gpu))
+  np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+
+
+def _tiling(ts):
+  return T.Cfg(lhs=T.TensorTiling([T.AxisTiling(axis=1, tile_size=ts)], []),
+               rhs=T.TensorTiling([T.AxisTiling(axis=0, tile_size=ts)], []))
+
+
+@pytest.mark.parametrize('lhs_bits,rhs_bits', [(8, 4), (8, 8)])
+@pytest.mark.parametrize('m,k,n,ts', [(48, 512, 96, 128), (33, 384, 40, 64), (256, 1024, 512, 128)])
+def test_tiled_int_weights(gpu, m, k, n, ts, lhs_bits, rhs_bits):
+  """int4 (or int8) weights with one scale per tile of `ts` along the contraction axis and
+  per-token-per-tile int8 activations (flax/aqt_flax.py:529-561 wiring); the per-tile outputs
+  are rounded to bf16 and summed in float32 in tile order."""
+  dt = 'bf16'
+  lhs, rhs = U.rand((m, k), dt, 1, outliers=True), U.rand((k, n), dt, 2, 0.015)
+  ocfg = R.dot_general_make(lhs_bits, rhs_bits)
+  want, res = R.tiled_dg_fwd(lhs, rhs, dt, ts, ocfg)
+  dg = aqt.dot_general_make(lhs_bits, rhs_bits)
+  dg = config.set_context(dg, None, None)
+  got = T.tiled_dot_general(_tiling(ts), U.to_dev(lhs, dt, gpu), U.to_dev(rhs, dt, gpu), MATMUL,
+                            dot_general=dg)
+  assert got.dtype == torch.bfloat16 and tuple(got.shape) == (m, n)
+  np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+
+
+def test_tiled_qtensors_and_scales(gpu):
+  """The inner dot_general sees tile-count batch axes: one scale per (tile, row) / (tile, column)."""
+  dt = 'bf16'
+  m, k, n, ts = 40, 256, 24, 64
+  lhs, rhs = U.rand((m, k), dt, 5), U.rand((k, n), dt, 6, 0.02)
+  res = R.tiled_dg_fwd(lhs, rhs, dt, ts, R.dot_general_make(8, 4))[1]
+  dg = config.set_context(aqt.dot_general_make(8, 4), None, None)
+  xl, xr = T.generate_tiling_states_for_dot_general(_tiling(ts), torch.empty(m, k), torch.empty(k, n), MATMUL)
+  tl, tr = xl.apply(U.to_dev(lhs, dt, gpu)), xr.apply(U.to_dev(rhs, dt, gpu))
+  assert list(tl.shape) == [m, k // ts, ts] and list(tr.shape) == [k // ts, ts, n]
+  _, (lqt, rqt) = dg.dg_core(tl, tr, None, None, (((2,), (1,)), ((1,), (0,))))
+  np.testing.assert_array_equal(lqt.qvalue.float().cpu().numpy(), res.lhs_res.qx.qvalue.astype(np.float32))
+  np.testing.assert_array_equal(rqt.qvalue.float().cpu().numpy(), res.rhs_res.qx.qvalue.astype(np.float32))
+  np.testing.assert_array_equal(lqt.scale[0].float().cpu().numpy(), res.lhs_res.qx.scale[0])
+  np.testing.assert_array_equal(rqt.scale[0].float().cpu().numpy(), res.rhs_res.qx.scale[0])
+  assert np.abs(rqt.qvalue.float().cpu().numpy()).max() <= 7
