@@ -282,51 +282,76 @@ def _get_scale_t(qt, transpose_fn, dimension_numbers, lhs_shape, rhs_shape):
   return [transpose_fn(s, dimension_numbers, lhs_shape, rhs_shape) for s in qt.scale]
 
 
-def _apply_local_aqt(local_aqt, lhs, rhs, dimension_numbers):
-  """aqt_dot_general.py:259-328."""
-  def factor_reshape_largest(x, ca, ba):
-    assert local_aqt.contraction_axis_shard_size is not None
-    assert local_aqt.contraction_axis_shard_count is None
-    shard_size = local_aqt.contraction_axis_shard_size
-    ca, ba = list(ca), list(ba)
-    if not ca:
-      return x, ca, ba
-    shape = list(x.shape)
-    max_ca_shape = max(shape[axis] for axis in ca)
-    ax = shape.index(max_ca_shape)
-    ax_ca_idx = ca.index(ax)
-    assert max_ca_shape % shard_size == 0
-    shape[ax] = max_ca_shape // shard_size
-    shape.insert(ax + 1, shard_size)
-    new_ca = [(b + int(b >= ax)) for b in ca]
-    assert new_ca[ax_ca_idx] == ax + 1
-    new_ba = [ax] + [(b + int(b > ax)) for b in ba]
-    return x.reshape(shape), new_ca, new_ba
+def _local_aqt_split(local_aqt, shape, ca, ba):
+  """Which contraction axis LocalAqt splits, and into what (aqt_dot_general.py:259-328).
 
-  def factor_reshape(x, ca, ba):
+  Returns (axis, shard_count, shard_size, new_ca, new_ba) or None without contraction axes:
+  the axis becomes (shard_count, shard_size) in place, the shard-count axis is the new leading
+  batch axis and the shard-size axis stays a contraction axis.  With tile_largest_shape the
+  (first) largest contraction axis is split into shards of contraction_axis_shard_size, else
+  the first contraction axis into contraction_axis_shard_count shards.
+  """
+  ca, ba = list(ca), list(ba)
+  if local_aqt.tile_largest_shape:
+    msg = 'When tile_largest_shape is True, must set shard_size.'
+    assert local_aqt.contraction_axis_shard_size is not None, msg
+    assert local_aqt.contraction_axis_shard_count is None, msg
+  else:
     msg = 'You are using the original local aqt. Please only set shard_count.'
     assert local_aqt.contraction_axis_shard_count is not None, msg
     assert local_aqt.contraction_axis_shard_size is None, msg
-    factor = local_aqt.contraction_axis_shard_count
-    ca, ba = list(ca), list(ba)
-    if not ca:
-      return x, ca, ba
-    shape = list(x.shape)
-    ax = ca[0]
-    orig_size = shape[ax]
-    assert orig_size % factor == 0
-    shape[ax] = factor
-    shape.insert(ax + 1, orig_size // factor)
-    new_ca = [(b + int(b >= ax)) for b in ca]
-    assert new_ca[0] == ax + 1
-    new_ba = [ax] + [(b + int(b > ax)) for b in ba]
-    return x.reshape(shape), new_ca, new_ba
+  if not ca:
+    return None
+  if local_aqt.tile_largest_shape:
+    extent = max(shape[a] for a in ca)
+    axis = list(shape).index(extent)   # the reference looks the extent up in the whole shape
+    assert axis in ca, 'the largest contraction extent also occurs on an earlier, non-contraction axis'
+    size = local_aqt.contraction_axis_shard_size
+    assert extent % size == 0
+    count = extent // size
+  else:
+    axis = ca[0]
+    count = local_aqt.contraction_axis_shard_count
+    assert shape[axis] % count == 0
+    size = shape[axis] // count
+  new_ca = [a + (a >= axis) for a in ca]
+  new_ba = [axis] + [a + (a > axis) for a in ba]
+  return axis, count, size, new_ca, new_ba
 
-  (lhs_ca, rhs_ca), (lhs_ba, rhs_ba) = dimension_numbers
-  fn = factor_reshape_largest if local_aqt.tile_largest_shape else factor_reshape
-  lhs, lhs_ca, lhs_ba = fn(lhs, lhs_ca, lhs_ba)
-  rhs, rhs_ca, rhs_ba = fn(rhs, rhs_ca, rhs_ba)
-  return lhs, rhs, ((lhs_ca, rhs_ca), (lhs_ba, rhs_ba))
+
+def _split_axis(x, axis, count, size):
+  """Reshapes axis `axis` of x into (count, size); an extent-1 axis (a keepdims scale) into (1, 1)."""
+  shape = list(x.shape)
+  shape[axis:axis + 1] = [count, size] if shape[axis] != 1 else [1, 1]
+  return x.reshape(shape)
+
+
+def _apply_local_aqt(local_aqt, lhs, rhs, dimension_numbers):
+  """Both operands with the contraction axis sharded, and the matching dimension numbers.
+
+  lhs may be a deferred `g * scale_t` (_Prescaled) and rhs a quantized residual (QTensor):
+  their payloads are reshaped alike.
+  """
+  (lca, rca), (lba, rba) = dimension_numbers
+
+  def one(x, ca, ba):
+    arr = x.x if isinstance(x, _Prescaled) else x.qvalue if isinstance(x, aqt_tensor.QTensor) else x
+    plan = _local_aqt_split(local_aqt, tuple(arr.shape), ca, ba)
+    if plan is None:
+      return x, list(ca), list(ba)
+    axis, count, size, new_ca, new_ba = plan
+    if isinstance(x, _Prescaled):
+      x = _Prescaled(x=_split_axis(x.x, axis, count, size), scale_t=_split_axis(x.scale_t, axis, count, size))
+    elif isinstance(x, aqt_tensor.QTensor):
+      x = x.replace(qvalue=_split_axis(x.qvalue, axis, count, size),
+                    scale=[_split_axis(sc, axis, count, size) for sc in x.scale])
+    else:
+      x = _split_axis(x, axis, count, size)
+    return x, new_ca, new_ba
+
+  lhs, lca, lba = one(lhs, lca, lba)
+  rhs, rca, rba = one(rhs, rca, rba)
+  return lhs, rhs, ((lca, rca), (lba, rba))
 
 
 _POISON = ('Poison. Gradients are not generally expected in serving. Please set '
@@ -411,13 +436,24 @@ class DotGeneralRaw:
     with torch.profiler.record_function(self.jax_scope_name):
       if isinstance(rhs, MultiTensor):
         lhs, rhs = _maybe_use_fwd_quant(lhs, rhs, dimension_numbers, self.rhs.use_fwd_quant)
-      if self.local_aqt is not None:
-        raise NotImplementedError('LocalAqt has no HIP path yet')
       for side, name in ((self.lhs, 'lhs'), (self.rhs, 'rhs')):
         if side.dequant_mode != DequantMode.OUTPUT or side.calibration_mode != CalibrationMode.CONTRACTING_AXIS:
           raise NotImplementedError(
               f'{name}: only DequantMode.OUTPUT with CalibrationMode.CONTRACTING_AXIS has a HIP path')
-      return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes)
+      if self.local_aqt is None:
+        return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes)
+      # LocalAqt (aqt_dot_general.py:773-776, 833-837): every shard of the contraction axis is
+      # calibrated and contracted on its own (the shard axis is a leading batch axis), the
+      # dequantized shard outputs are summed; no residuals come back.
+      n_ca = len(dimension_numbers[0][0])
+      assert n_ca == len(dimension_numbers[0][1])
+      lhs, rhs, dn = _apply_local_aqt(self.local_aqt, lhs, rhs, dimension_numbers)
+      out, _ = self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dn, None)
+      if n_ca > 0:
+        out = ops.sum_tiles(out.contiguous())
+      if _out_transpose_axes is not None:
+        out = out.permute(*_out_transpose_axes)
+      return out, None
 
   # ------------------------------------------------------------------------------
   def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None):

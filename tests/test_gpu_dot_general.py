@@ -183,3 +183,31 @@ def test_fp8_config(gpu, fwd, bwd):
   for k in ('out', 'dlhs', 'drhs'):
     np.testing.assert_allclose(got[k], want[k], rtol=2.0 ** -7, atol=2.0 ** -9 * np.abs(want[k]).max(),
                                err_msg=k)
+
+
+@pytest.mark.parametrize('sr', [False, True])
+@pytest.mark.parametrize('dl,dr', [(2, 4), (1, 8), (4, None)])
+def test_local_aqt_in_backward(gpu, dl, dr, sr):
+  """LocalAqt (aqt_dot_general.py:259-328, 833-837): the bwd contraction axis is split in
+  shards with their own scales; shard outputs are dequantized, then summed in float32."""
+  dt = 'bf16'
+  lhs, rhs, g = U.rand((64, 128), dt, 1, outliers=True), U.rand((128, 96), dt, 2, 0.02), U.rand((64, 96), dt, 3, 1e-3)
+  mk = lambda c: None if c is None else aqt.LocalAqt(contraction_axis_shard_count=c)
+  cfg = config.fully_quantized(use_stochastic_rounding=sr, dlhs_local_aqt=mk(dl), drhs_local_aqt=mk(dr))
+  ocfg = R.fully_quantized(use_stochastic_rounding=sr)
+  ocfg.dlhs.local_aqt_shard_count, ocfg.drhs.local_aqt_shard_count = dl, dr
+  got, want = _run_both(lhs, rhs, g, dt, MATMUL, cfg, ocfg, prng.prng_key(11), gpu)
+  _assert_same(got, want)
+
+
+def test_local_aqt_largest_shape(gpu):
+  """tile_largest_shape picks the largest contraction axis and a shard size
+  (aqt_dot_general.py:279-300); on a matmul that is the same split as shard_count."""
+  dt = 'bf16'
+  lhs, rhs, g = U.rand((64, 128), dt, 1), U.rand((128, 96), dt, 2, 0.02), U.rand((64, 96), dt, 3, 1e-3)
+  la = aqt.LocalAqt(contraction_axis_shard_size=32, tile_largest_shape=True)
+  cfg = config.fully_quantized(use_stochastic_rounding=False, dlhs_local_aqt=la, drhs_local_aqt=la)
+  ocfg = R.fully_quantized(use_stochastic_rounding=False)
+  ocfg.dlhs.local_aqt_shard_count, ocfg.drhs.local_aqt_shard_count = 96 // 32, 64 // 32
+  got, want = _run_both(lhs, rhs, g, dt, MATMUL, cfg, ocfg, prng.prng_key(11), gpu)
+  _assert_same(got, want)
