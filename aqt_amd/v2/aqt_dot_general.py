@@ -257,8 +257,8 @@ def einsum(eqn: str, lhs, rhs, dg=lax_dot_general):
 
   Letters shared by both operands and the output are batch axes, letters shared by
   the operands only are contracted; the dot_general output (batch, lhs free, rhs
-  free) is then permuted to the requested order.  Like jnp.einsum's planner, the
-  operand whose free letters come first in the output stays on the left.
+  free) is then permuted to the requested order.  Like jnp.einsum, the operands are
+  handed over as (rhs, lhs) when the output is exactly (batch, rhs free, lhs free).
   """
   l, r, out = _parse_einsum(eqn)
   assert len(set(l)) == len(l) and len(set(r)) == len(r), 'repeated indices are not supported'
@@ -268,6 +268,12 @@ def einsum(eqn: str, lhs, rhs, dg=lax_dot_general):
   rfree = [c for c in r if c not in l]
   for c in lfree + rfree:
     assert c in out, 'summing a free index is not supported'
+  if batch + rfree + lfree == list(out):
+    # jnp.einsum tries (rhs, lhs) first and keeps that order when it needs no transpose
+    # afterwards; callers (AqtEinsum) mirror the swap in their per-side settings.
+    dn = ((tuple(r.index(c) for c in contract), tuple(l.index(c) for c in contract)),
+          (tuple(r.index(c) for c in batch), tuple(l.index(c) for c in batch)))
+    return dg(rhs, lhs, dn, None, None)
   dn = ((tuple(l.index(c) for c in contract), tuple(r.index(c) for c in contract)),
         (tuple(l.index(c) for c in batch), tuple(r.index(c) for c in batch)))
   res = dg(lhs, rhs, dn, None, None)

@@ -1,0 +1,430 @@
+"""Callers of the quantized dot_general that models plug in: AqtDotGeneral, AqtEinsum.
+
+Counterpart of aqt/jax/v2/flax/aqt_flax.py for torch modules.  What is kept from the
+reference: the call signatures (a dot_general-shaped `__call__(lhs, rhs,
+dimension_numbers, precision, preferred_element_type=None)`, `AqtEinsum(eqn, lhs, rhs)`),
+the field names and defaults, the quant-mode flow (TRAIN / CALIBRATE quantize on the fly,
+CONVERT stores the quantized operand, SERVE reads it back instead of quantizing), both
+freezers, the operand swap of einsum, external QTensor operands, tiling injection and the
+dtype promotion table of aqt_promote_dtype.
+
+What differs: variables live on the module (`variables()` returns the {collection: ...}
+tree a Flax caller would find under `quant_collection`), and PRNG keys come from the
+`rngs` dict given to the module -- Flax's make_rng folds the module path into the key,
+which has no counterpart here; each make_rng call splits the stored key instead.
+"""
+from __future__ import annotations
+
+import copy
+import enum
+import functools
+from typing import Any, Callable, Dict, Optional, Sequence
+
+import torch
+
+from aqt_amd import ops
+from aqt_amd.v2 import aqt_dot_general
+from aqt_amd.v2 import aqt_tensor
+from aqt_amd.v2 import config
+from aqt_amd.v2 import tiled_dot_general
+from aqt_amd.v2 import transpose
+from aqt_amd.v2 import utils
+from aqt_amd.v2.flax import freezer as general_freezer
+
+QuantMode = utils.QuantMode
+
+_QUANT_TO_FREEZER_MODE = {
+    QuantMode.TRAIN: general_freezer.FreezerMode.NONE,
+    QuantMode.CALIBRATE: general_freezer.FreezerMode.NONE,
+    QuantMode.CONVERT: general_freezer.FreezerMode.WRITE,
+    QuantMode.SERVE: general_freezer.FreezerMode.READ,
+}
+
+
+class FreezerMode(enum.Enum):
+  """What a freezer keeps of a QTensor (aqt_flax.py:143-146)."""
+  NONE = 1
+  CALIBRATION = 2
+  CALIBRATION_AND_VALUE = 3
+
+
+_MANUAL = (utils.int4, torch.float8_e4m3fn, torch.float8_e5m2)
+
+
+def promoted_dtype(lhs_dtype, rhs_dtype):
+  """Common dtype of aqt_promote_dtype (aqt_flax.py:102-140; table aqt_flax_test.py:37-79).
+
+  int4 / fp8 pairs of the same type stay; otherwise int4 counts as float32 and fp8 as bfloat16,
+  and the usual promotion follows, with integer results lifted to float32.
+  """
+  if lhs_dtype in _MANUAL and rhs_dtype in _MANUAL and lhs_dtype == rhs_dtype:
+    return lhs_dtype
+  lift = lambda d: (torch.float32 if d is utils.int4 else torch.bfloat16) if d in _MANUAL else d
+  out = torch.promote_types(lift(lhs_dtype), lift(rhs_dtype))
+  return out if out.is_floating_point else torch.float32
+
+
+def aqt_promote_dtype(lhs_in: torch.Tensor, rhs_in: torch.Tensor):
+  dt = promoted_dtype(lhs_in.dtype, rhs_in.dtype)
+  return lhs_in.to(dt), rhs_in.to(dt)
+
+
+class Freezer(torch.nn.Module):
+  """Legacy freezer: qvalue + transposed scale as two variables (aqt_flax.py:149-232).
+
+  get() returns None in TRAIN / CALIBRATE / CONVERT and the stored QTensor (with scale_t
+  only) in SERVE; set() stores in CONVERT and is a no-op otherwise.
+  """
+
+  def __init__(self, *, quant_collection: str, quant_mode: QuantMode, q_shape, q_dtype, q_init=None,
+               s_shape=None, s_init=None, name: Optional[str] = None):
+    super().__init__()
+    self.quant_collection = quant_collection
+    self.quant_mode = quant_mode
+    self.q_shape, self.q_dtype, self.s_shape = tuple(q_shape), q_dtype, tuple(s_shape or ())
+    self.var_name = name
+    self.qvalue = None
+    self.scale_t = None
+    self.container_dtype = None
+
+  def get(self) -> Optional[aqt_tensor.QTensor]:
+    if self.quant_mode in (QuantMode.TRAIN, QuantMode.CALIBRATE, QuantMode.CONVERT):
+      return None
+    if self.quant_mode == QuantMode.SERVE:
+      assert self.qvalue is not None and self.scale_t is not None, (
+          f'freezer {self.var_name!r} is in SERVE mode but holds no converted tensor')
+      return aqt_tensor.QTensor(qvalue=self.qvalue, scale=None, scale_t=[self.scale_t], bias=[],
+                                dequant_dtype=self.scale_t.dtype, container_dtype=self.container_dtype)
+    assert False, 'Unknown quant mode.'
+
+  def set(self, inputs: aqt_tensor.QTensor) -> None:
+    if inputs.bias:
+      raise NotImplementedError('Quantization biases are not supported in AQT Flax Legacy Freezer.')
+    if self.quant_mode in (QuantMode.TRAIN, QuantMode.CALIBRATE, QuantMode.SERVE):
+      return None
+    if self.quant_mode == QuantMode.CONVERT:
+      self.qvalue = inputs.qvalue
+      assert inputs.scale_t is not None and len(inputs.scale_t) == 1
+      self.scale_t = inputs.scale_t[0]
+      self.container_dtype = inputs.container_dtype
+      return None
+    assert False, 'Unknown quant mode.'
+
+  def state(self):
+    if self.qvalue is None:
+      return {}
+    return {self.quant_collection: {'value': self.qvalue, 'scale': self.scale_t}}
+
+  def load_state(self, state) -> None:
+    tree = state.get(self.quant_collection, {})
+    if 'value' in tree:
+      self.qvalue, self.scale_t = tree['value'], tree['scale']
+
+
+def _maybe_recover_scale_from_scale_t(qt, dimension_numbers, is_rhs: bool, lhs_shape, rhs_shape):
+  """aqt_flax.py:235-255."""
+  if qt is None or qt.scale is not None or qt.scale_t is None:
+    return qt
+  fn = transpose.rhs_recover_scale_from_scale_t if is_rhs else transpose.lhs_recover_scale_from_scale_t
+  return qt.replace(scale=[fn(s, dimension_numbers, lhs_shape, rhs_shape) for s in qt.scale_t], scale_t=None)
+
+
+def _populate_scale_t(qt, dimension_numbers, is_rhs: bool, lhs_shape, rhs_shape):
+  """aqt_flax.py:258-275."""
+  if qt.scale is None:
+    return qt
+  fn = transpose.rhs_scale_transpose_to_output if is_rhs else transpose.lhs_scale_transpose_to_output
+  return qt.replace(scale_t=[fn(s, dimension_numbers, lhs_shape, rhs_shape) for s in qt.scale])
+
+
+def _apply_freeze_mode(qt, freeze_mode, apply_quant_mode, quant_mode, side):
+  """What goes into the freezer (aqt_flax.py:466-492)."""
+  if freeze_mode == FreezerMode.NONE:
+    if apply_quant_mode and quant_mode in (QuantMode.CONVERT, QuantMode.SERVE):
+      raise ValueError('Freezer is used with Freezer mode NONE.')
+    return qt
+  if freeze_mode == FreezerMode.CALIBRATION:
+    return qt.without_qvalue()
+  if freeze_mode == FreezerMode.CALIBRATION_AND_VALUE:
+    return qt
+  raise ValueError('Unknown freeze mode: %s' % freeze_mode)
+
+
+class _RngMixin:
+  """`rngs`: {name: uint32[2] key data}.  make_rng hands out a fresh key per call."""
+
+  def make_rng(self, name: str):
+    rngs = getattr(self, 'rngs', None)
+    assert rngs is not None and name in rngs, f'{type(self).__name__} needs an rng named {name!r} (rngs=...)'
+    key, sub = ops.prng_split(rngs[name], 2, utils.threefry_partitionable)
+    rngs[name] = key
+    return sub
+
+
+class AqtDotGeneral(torch.nn.Module, _RngMixin):
+  """A dot_general-shaped callable that quantizes (aqt_flax.py:278-561)."""
+
+  def __init__(self, cfg: Optional[aqt_dot_general.DotGeneral] = None, prng_name: Optional[str] = 'params', *,
+               lhs_quant_mode: QuantMode = QuantMode.TRAIN, lhs_apply_quant_mode: bool = True,
+               lhs_var_name: str = 'qlhs', lhs_qtensor: Optional[aqt_tensor.QTensor] = None,
+               rhs_quant_mode: QuantMode = QuantMode.TRAIN, rhs_apply_quant_mode: bool = True,
+               rhs_var_name: str = 'qrhs', rhs_qtensor: Optional[aqt_tensor.QTensor] = None,
+               lhs_init=None, lhs_scale_init=None, rhs_init=None, rhs_scale_init=None,
+               lhs_axis_metadata_wrapper=None, rhs_axis_metadata_wrapper=None,
+               lhs_freeze_mode: FreezerMode = FreezerMode.NONE, rhs_freeze_mode: FreezerMode = FreezerMode.NONE,
+               quant_collection: str = 'aqt', tiling_cfg: Optional[tiled_dot_general.Cfg] = None,
+               tiling_fn: Optional[Callable] = None, use_legacy_freezer: bool = True,
+               rngs: Optional[Dict[str, Any]] = None):
+    super().__init__()
+    self.cfg, self.prng_name = cfg, prng_name
+    self.lhs_quant_mode, self.lhs_apply_quant_mode = lhs_quant_mode, lhs_apply_quant_mode
+    self.lhs_var_name, self.lhs_qtensor = lhs_var_name, lhs_qtensor
+    self.rhs_quant_mode, self.rhs_apply_quant_mode = rhs_quant_mode, rhs_apply_quant_mode
+    self.rhs_var_name, self.rhs_qtensor = rhs_var_name, rhs_qtensor
+    self.lhs_axis_metadata_wrapper, self.rhs_axis_metadata_wrapper = lhs_axis_metadata_wrapper, rhs_axis_metadata_wrapper
+    self.lhs_freeze_mode, self.rhs_freeze_mode = lhs_freeze_mode, rhs_freeze_mode
+    self.quant_collection = quant_collection
+    self.tiling_cfg, self.tiling_fn = tiling_cfg, tiling_fn
+    self.use_legacy_freezer = use_legacy_freezer
+    self.rngs = rngs
+    self.freezers = torch.nn.ModuleDict()
+
+  # ---- variables --------------------------------------------------------------------------
+  def _freezer(self, name, make):
+    if name not in self.freezers:
+      self.freezers[name] = make()
+    return self.freezers[name]
+
+  def variables(self):
+    """{quant_collection: {var_name: {...}}}: what a checkpoint of this layer holds."""
+    out = {}
+    for name, fr in self.freezers.items():
+      for coll, tree in fr.state().items():
+        out.setdefault(coll, {})[name] = tree
+    return out
+
+  def load_variables(self, variables) -> None:
+    self._pending = variables
+
+  # ---- the quantized dot_general --------------------------------------------------------
+  def make_aqt_dg(self, lhs_shape, rhs_shape, dimension_numbers, lhs_tile_map=None, rhs_tile_map=None):
+    if self.cfg is None:
+      return aqt_dot_general.lax_dot_general
+    cfg = copy.deepcopy(self.cfg)
+    lhs_shape, rhs_shape = tuple(lhs_shape), tuple(rhs_shape)
+    (contr, _) = dimension_numbers
+    ls, rs = list(lhs_shape), list(rhs_shape)
+    for li, ri in zip(*contr):
+      ls[li] = 1
+      rs[ri] = 1
+    lhs_scale_shape = tuple(transpose.lhs_scale_transpose_to_output(
+        torch.zeros(ls, device='meta'), dimension_numbers, lhs_shape, rhs_shape).shape)
+    rhs_scale_shape = tuple(transpose.rhs_scale_transpose_to_output(
+        torch.zeros(rs, device='meta'), dimension_numbers, lhs_shape, rhs_shape).shape)
+    assert isinstance(cfg.fwd.dg_quantizer, aqt_dot_general.DefaultDotGeneralQuantizer)
+    lhs_q_dtype = cfg.fwd.dg_quantizer.lhs.numerics.get_dtype()
+    rhs_q_dtype = cfg.fwd.dg_quantizer.rhs.numerics.get_dtype()
+
+    if self.use_legacy_freezer:
+      lhs_freezer = self._freezer(self.lhs_var_name, lambda: Freezer(
+          name=self.lhs_var_name, quant_mode=self.lhs_quant_mode, q_shape=lhs_shape, q_dtype=lhs_q_dtype,
+          s_shape=lhs_scale_shape, quant_collection=self.quant_collection))
+      rhs_freezer = self._freezer(self.rhs_var_name, lambda: Freezer(
+          name=self.rhs_var_name, quant_mode=self.rhs_quant_mode, q_shape=rhs_shape, q_dtype=rhs_q_dtype,
+          s_shape=rhs_scale_shape, quant_collection=self.quant_collection))
+      lhs_freezer.quant_mode, rhs_freezer.quant_mode = self.lhs_quant_mode, self.rhs_quant_mode
+    else:
+      lhs_freezer = self._freezer(self.lhs_var_name, lambda: general_freezer.Freezer(
+          name=self.lhs_var_name, collection=self.quant_collection,
+          axis_metadata_wrapper=self.lhs_axis_metadata_wrapper))
+      rhs_freezer = self._freezer(self.rhs_var_name, lambda: general_freezer.Freezer(
+          name=self.rhs_var_name, collection=self.quant_collection,
+          axis_metadata_wrapper=self.rhs_axis_metadata_wrapper))
+      lhs_freezer.mode = _QUANT_TO_FREEZER_MODE[self.lhs_quant_mode]
+      rhs_freezer.mode = _QUANT_TO_FREEZER_MODE[self.rhs_quant_mode]
+    pending = getattr(self, '_pending', None)
+    if pending is not None:
+      for name, fr in ((self.lhs_var_name, lhs_freezer), (self.rhs_var_name, rhs_freezer)):
+        fr.load_state({coll: tree[name] for coll, tree in pending.items() if name in tree})
+      self._pending = None
+
+    key = self.make_rng(self.prng_name) if self.prng_name is not None else None
+    cfg = config.set_context(cfg, key, train_step=None, lhs_quant_mode=self.lhs_quant_mode,
+                             rhs_quant_mode=self.rhs_quant_mode)
+
+    def ret_dg(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+      del preferred_element_type
+      assert precision is None, f'Precision {precision} requested together with quantization.'
+      msg = 'AQT is not yet optimized to accept quantized types directly. '
+      msg += f'lhs.dtype: {lhs.dtype}, rhs.dtype: {rhs.dtype}'
+      assert lhs.dtype in [utils.bfloat16, utils.float32, utils.float16], msg
+      assert rhs.dtype in [utils.bfloat16, utils.float32, utils.float16], msg
+      cfg.assert_config_validity()
+
+      lhs_qt = lhs_freezer.get() if self.lhs_apply_quant_mode else self.lhs_qtensor
+      rhs_qt = rhs_freezer.get() if self.rhs_apply_quant_mode else self.rhs_qtensor
+      # A tensor read from the legacy freezer carries scale_t only.
+      lhs_qt = _maybe_recover_scale_from_scale_t(lhs_qt, dimension_numbers, False, lhs_shape, rhs_shape)
+      rhs_qt = _maybe_recover_scale_from_scale_t(rhs_qt, dimension_numbers, True, lhs_shape, rhs_shape)
+
+      out, (out_lhs_qt, out_rhs_qt) = cfg.dg_core(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers)
+
+      out_lhs_qt = _apply_freeze_mode(out_lhs_qt, self.lhs_freeze_mode, self.lhs_apply_quant_mode,
+                                      self.lhs_quant_mode, 'lhs')
+      out_rhs_qt = _apply_freeze_mode(out_rhs_qt, self.rhs_freeze_mode, self.rhs_apply_quant_mode,
+                                      self.rhs_quant_mode, 'rhs')
+      contracting = aqt_dot_general.CalibrationMode.CONTRACTING_AXIS
+      if self.use_legacy_freezer:
+        if cfg.fwd.lhs.calibration_mode == contracting:
+          out_lhs_qt = _populate_scale_t(out_lhs_qt, dimension_numbers, False, lhs_shape, rhs_shape)
+        if cfg.fwd.rhs.calibration_mode == contracting:
+          out_rhs_qt = _populate_scale_t(out_rhs_qt, dimension_numbers, True, lhs_shape, rhs_shape)
+      if self.lhs_apply_quant_mode:
+        lhs_freezer.set(out_lhs_qt)
+      if self.rhs_apply_quant_mode:
+        rhs_freezer.set(out_rhs_qt)
+      return out
+
+    return ret_dg
+
+  def forward(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+    tiling_cfg = self.tiling_cfg
+    if tiling_cfg is None and self.tiling_fn is not None:
+      tiling_cfg = self.tiling_fn(lhs, rhs, dimension_numbers)
+    if tiling_cfg is not None:
+      xlhs, xrhs = tiled_dot_general.generate_tiling_states_for_dot_general(
+          tiling_cfg, lhs, rhs, dimension_numbers)
+      # The freezers observe tiled shapes: record what the inner dot_general is called with.
+      seen = {}
+
+      def probe(l, r, dn, precision=None, preferred_element_type=None):
+        seen['l'], seen['r'], seen['dn'] = tuple(l.shape), tuple(r.shape), dn
+        return aqt_dot_general.lax_dot_general(l, r, dn, precision, preferred_element_type)
+
+      meta = lambda t: torch.empty(t.shape, dtype=torch.float32, device='meta')
+      tiled_dot_general.tiled_dot_general_with_tiling_states(
+          meta(lhs), copy.deepcopy(xlhs), meta(rhs), copy.deepcopy(xrhs), dimension_numbers, dot_general=probe)
+      aqt_dg = self.make_aqt_dg(seen['l'], seen['r'], seen['dn'], lhs_tile_map=xlhs.tile_map,
+                                rhs_tile_map=xrhs.tile_map)
+      ret_dg = functools.partial(tiled_dot_general.tiled_dot_general, tiling_cfg, dot_general=aqt_dg)
+    else:
+      ret_dg = self.make_aqt_dg(lhs.shape, rhs.shape, dimension_numbers)
+    return ret_dg(lhs, rhs, dimension_numbers, precision, preferred_element_type)
+
+
+def einsum_swaps_operands(eqn: str) -> bool:
+  """Whether einsum hands (rhs, lhs) to dot_general for this equation (see aqt_dot_general.einsum)."""
+  order = []
+
+  def probe(l, r, dn, precision=None, preferred_element_type=None):
+    order.append((l.tag, r.tag))
+    raise _ProbeDone()
+
+  class _T:  # the smallest thing einsum needs: a shape and a tag
+    def __init__(self, tag, n):
+      self.tag, self.shape = tag, (1,) * n
+    def dim(self):
+      return len(self.shape)
+
+  l, r, _ = aqt_dot_general._parse_einsum(eqn)
+  try:
+    aqt_dot_general.einsum(eqn, _T('lhs', len(l)), _T('rhs', len(r)), probe)
+  except _ProbeDone:
+    pass
+  assert order and set(order[0]) == {'lhs', 'rhs'}
+  return order[0] == ('rhs', 'lhs')
+
+
+class _ProbeDone(Exception):
+  pass
+
+
+class AqtEinsum(torch.nn.Module, _RngMixin):
+  """Quantized einsum for model injection (aqt_flax.py:564-732)."""
+
+  def __init__(self, cfg: Optional[aqt_dot_general.DotGeneral] = None, prng_name: Optional[str] = 'params', *,
+               lhs_quant_mode: QuantMode = QuantMode.TRAIN, lhs_var_name: str = 'qlhs',
+               rhs_quant_mode: QuantMode = QuantMode.TRAIN, rhs_var_name: str = 'qrhs',
+               lhs_init=None, lhs_scale_init=None, rhs_init=None, rhs_scale_init=None,
+               lhs_axis_metadata_wrapper=None, rhs_axis_metadata_wrapper=None,
+               lhs_freeze_mode: FreezerMode = FreezerMode.NONE, rhs_freeze_mode: FreezerMode = FreezerMode.NONE,
+               quant_collection: str = 'aqt', assert_eqn: Optional[str] = None, assert_lhs_shape=None,
+               assert_rhs_shape=None, tile_sizes=None, tiling_fn=None, use_legacy_freezer: bool = True,
+               rngs: Optional[Dict[str, Any]] = None):
+    super().__init__()
+    self.cfg, self.prng_name = cfg, prng_name
+    self.lhs_quant_mode, self.lhs_var_name = lhs_quant_mode, lhs_var_name
+    self.rhs_quant_mode, self.rhs_var_name = rhs_quant_mode, rhs_var_name
+    self.lhs_axis_metadata_wrapper, self.rhs_axis_metadata_wrapper = lhs_axis_metadata_wrapper, rhs_axis_metadata_wrapper
+    self.lhs_freeze_mode, self.rhs_freeze_mode = lhs_freeze_mode, rhs_freeze_mode
+    self.quant_collection = quant_collection
+    self.assert_eqn, self.assert_lhs_shape, self.assert_rhs_shape = assert_eqn, assert_lhs_shape, assert_rhs_shape
+    self.tile_sizes, self.tiling_fn = tile_sizes, tiling_fn
+    self.use_legacy_freezer = use_legacy_freezer
+    self.rngs = rngs
+    self.dg: Optional[AqtDotGeneral] = None
+
+  def variables(self):
+    return {} if self.dg is None else self.dg.variables()
+
+  def load_variables(self, variables) -> None:
+    self._pending = variables
+
+  def forward(self, eqn, lhs_g, rhs_g):
+    if self.assert_eqn is not None:
+      assert eqn == self.assert_eqn, f'einsum_eqn: {eqn} != {self.assert_eqn}'
+    if self.assert_lhs_shape is not None:
+      utils.assert_shape(lhs_g.shape, self.assert_lhs_shape, 'lhs.shape')
+    if self.assert_rhs_shape is not None:
+      utils.assert_shape(rhs_g.shape, self.assert_rhs_shape, 'rhs.shape')
+    cfg = self.cfg
+    lhs_is_qt = isinstance(lhs_g, aqt_tensor.QTensor)
+    rhs_is_qt = isinstance(rhs_g, aqt_tensor.QTensor)
+    assert not ((lhs_is_qt or rhs_is_qt) and cfg is None), (
+        'Aqt config is None but inputs to AqtEinsum are QTensor.')
+    # A QTensor operand is passed on through lhs_qtensor / rhs_qtensor; the array handed to
+    # einsum in its place only carries shape and dtype.
+    def placeholder(qt):
+      return torch.zeros(tuple(qt.qvalue.shape), dtype=qt.dequant_dtype, device=qt.qvalue.device)
+    lhs_in = placeholder(lhs_g) if lhs_is_qt else lhs_g
+    rhs_in = placeholder(rhs_g) if rhs_is_qt else rhs_g
+    lhs_in, rhs_in = aqt_promote_dtype(lhs_in, rhs_in)
+
+    yes_swap = einsum_swaps_operands(eqn)
+    sides = dict(
+        lhs=dict(quant_mode=self.lhs_quant_mode, var_name=self.lhs_var_name, qtensor=lhs_g if lhs_is_qt else None,
+                 is_qt=lhs_is_qt, wrapper=self.lhs_axis_metadata_wrapper, freeze_mode=self.lhs_freeze_mode),
+        rhs=dict(quant_mode=self.rhs_quant_mode, var_name=self.rhs_var_name, qtensor=rhs_g if rhs_is_qt else None,
+                 is_qt=rhs_is_qt, wrapper=self.rhs_axis_metadata_wrapper, freeze_mode=self.rhs_freeze_mode))
+    tiling_config = None
+    if self.tile_sizes is not None:
+      tiling_config = tiled_dot_general.Cfg.from_einsum(eqn, self.tile_sizes)
+    elif self.tiling_fn is not None:
+      tiling_config = self.tiling_fn(eqn, lhs_in, rhs_in)
+    if yes_swap:
+      # dot_general sees (rhs, lhs): everything said about a side moves with it
+      # (aqt_flax.py:684-704).
+      if cfg is not None:
+        cfg = copy.deepcopy(cfg)
+        cfg.fwd.lhs, cfg.fwd.rhs = cfg.fwd.rhs, cfg.fwd.lhs
+        cfg.fwd.dg_quantizer.swap_lhs_and_rhs()
+        cfg.dlhs, cfg.drhs = cfg.drhs, cfg.dlhs
+      sides['lhs'], sides['rhs'] = sides['rhs'], sides['lhs']
+      if tiling_config is not None:
+        tiling_config = tiled_dot_general.Cfg(lhs=tiling_config.rhs, rhs=tiling_config.lhs)
+    L, R = sides['lhs'], sides['rhs']
+    if self.dg is None:
+      self.dg = AqtDotGeneral(quant_collection=self.quant_collection, use_legacy_freezer=self.use_legacy_freezer)
+      if getattr(self, '_pending', None) is not None:
+        self.dg.load_variables(self._pending)
+        self._pending = None
+    dg = self.dg
+    dg.cfg, dg.prng_name, dg.rngs = cfg, self.prng_name, self.rngs
+    dg.lhs_quant_mode, dg.lhs_apply_quant_mode = L['quant_mode'], not L['is_qt']
+    dg.lhs_var_name, dg.lhs_qtensor = L['var_name'], L['qtensor']
+    dg.lhs_axis_metadata_wrapper, dg.lhs_freeze_mode = L['wrapper'], L['freeze_mode']
+    dg.rhs_quant_mode, dg.rhs_apply_quant_mode = R['quant_mode'], not R['is_qt']
+    dg.rhs_var_name, dg.rhs_qtensor = R['var_name'], R['qtensor']
+    dg.rhs_axis_metadata_wrapper, dg.rhs_freeze_mode = R['wrapper'], R['freeze_mode']
+    dg.tiling_cfg = tiling_config
+    return aqt_dot_general.einsum(eqn, lhs_in, rhs_in, dg)

@@ -65,6 +65,18 @@ float8_e4m3fn = torch.float8_e4m3fn
 float8_e5m2 = torch.float8_e5m2
 
 
+def assert_shape(shape, shape_template, msg: str):
+  """A None entry of the template matches any extent (utils.py:48-55)."""
+  shape, shape_template = list(shape), list(shape_template)
+  assert len(shape) == len(shape_template), msg
+  for got, want in zip(shape, shape_template):
+    assert want is None or got == want, f'{msg}: {shape} does not match {shape_template}'
+
+
+def assert_eq(value, expected, value_name: str):
+  assert value == expected, f'{value_name}={value}, {expected=}'
+
+
 class QuantMode(enum.Enum):
   """utils.py:85-89."""
   TRAIN = 1

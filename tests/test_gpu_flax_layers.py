@@ -1,0 +1,119 @@
+"""GPU: AqtDotGeneral / AqtEinsum modules over the HIP kernels (flows of aqt/jax/v2/flax/aqt_flax_test.py)."""
+import numpy as np
+import pytest
+import torch
+
+from aqt_amd.v2 import aqt_dot_general as aqt
+from aqt_amd.v2 import config
+from aqt_amd.v2 import tiled_dot_general
+from aqt_amd.v2 import utils
+from aqt_amd.v2.flax import aqt_flax
+from oracle import aqt_ref as R
+from oracle import prng
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+QM, FM = utils.QuantMode, aqt_flax.FreezerMode
+MATMUL = (((1,), (0,)), ((), ()))
+
+
+def _rngs():
+  return {'params': utils.prng_key(0)}
+
+
+def test_aqt_einsum_external_qtensors(gpu):
+  """aqt_flax_test.py:81-158: QTensor operands computed outside give the same result."""
+  lhs = torch.rand(3, 4, 5, 6, device=gpu)
+  rhs = torch.rand(2, 5, 6, device=gpu)
+  eqn = 'ijkh,mkh->ijm'
+
+  def run(lhs_ext, rhs_ext, cfg_fn):
+    cfg = cfg_fn()
+    lhs_in, rhs_in = lhs, rhs
+    if lhs_ext or rhs_ext:
+      dgq = cfg_fn().fwd.dg_quantizer
+      dgq.init_calibration()
+      dn = (((2, 3), (1, 2)), ((), ()))
+      (lq, _), (rq, _) = dgq((lhs, dn[0][0]), (rhs, dn[0][1]))
+      if lhs_ext:
+        lhs_in = lq
+      if rhs_ext:
+        rhs_in = rq
+    einsum = aqt_flax.AqtEinsum(cfg=cfg, lhs_freeze_mode=FM.NONE, rhs_freeze_mode=FM.CALIBRATION_AND_VALUE,
+                                rngs=_rngs())
+    return einsum(eqn, lhs_in, rhs_in)
+
+  out_float = run(False, False, lambda: None)
+  out_int8 = run(False, False, config.config_v4)
+  assert torch.equal(out_int8, run(True, False, config.config_v4)), 'lhs external qt failed'
+  assert torch.equal(out_int8, run(False, True, config.config_v4)), 'rhs external qt failed'
+  assert torch.equal(out_int8, run(True, True, config.config_v4)), 'both external qt failed'
+  assert torch.mean((out_int8 - out_float) ** 2) > 0, 'Einsum is not quantized.'
+  assert torch.allclose(out_int8, out_float, rtol=0.05, atol=0.05)
+
+
+@pytest.mark.parametrize('legacy', [True, False])
+def test_convert_then_serve(gpu, legacy):
+  """TRAIN -> CONVERT (weights frozen into the 'aqt' collection) -> SERVE reads them back:
+  the three outputs agree, and serving ignores the float weight it is handed."""
+  dt = 'bf16'
+  x, w = U.to_dev(U.rand((8, 256), dt, 1), dt, gpu), U.to_dev(U.rand((256, 128), dt, 2, 0.02), dt, gpu)
+  cfg = config.fully_quantized(use_stochastic_rounding=False)
+  mk = lambda mode: aqt_flax.AqtDotGeneral(cfg, rhs_quant_mode=mode, rhs_freeze_mode=FM.CALIBRATION_AND_VALUE,
+                                           use_legacy_freezer=legacy, rngs=_rngs())
+  out_train = mk(QM.TRAIN)(x, w, MATMUL, None)
+  conv = mk(QM.CONVERT)
+  out_conv = conv(x, w, MATMUL, None)
+  variables = conv.variables()
+  assert set(variables) == {'aqt'} and set(variables['aqt']) == {'qrhs'}
+  if legacy:
+    assert set(variables['aqt']['qrhs']) == {'value', 'scale'}
+    assert tuple(variables['aqt']['qrhs']['value'].shape) == (256, 128)
+    assert tuple(variables['aqt']['qrhs']['scale'].shape) == (1, 128)
+  else:
+    frozen = variables['aqt']['qrhs']['frozen']
+    assert tuple(frozen.qvalue.shape) == (256, 128) and tuple(frozen.scale[0].shape) == (1, 128)
+  serve = mk(QM.SERVE)
+  serve.load_variables(variables)
+  out_serve = serve(x, torch.zeros_like(w), MATMUL, None)
+  assert torch.equal(out_train, out_conv) and torch.equal(out_train, out_serve)
+  f = R.dg_fwd(U.rand((8, 256), dt, 1), U.rand((256, 128), dt, 2, 0.02), dt, MATMUL, R.fully_quantized())
+  np.testing.assert_array_equal(out_serve.float().cpu().numpy(), f.out)
+
+
+def test_freezer_none_with_convert_raises(gpu):
+  x, w = torch.randn(4, 32, device=gpu), torch.randn(32, 8, device=gpu)
+  dg = aqt_flax.AqtDotGeneral(config.fully_quantized(), rhs_quant_mode=QM.CONVERT, rngs=_rngs())
+  with pytest.raises(ValueError, match='Freezer mode NONE'):
+    dg(x, w, MATMUL, None)
+
+
+def test_einsum_swap_moves_the_side_settings(gpu):
+  """'bc,ab->ac' reaches dot_general as (rhs, lhs); the frozen weight is einsum's lhs (the model's
+  weight in test_einsum_grad_leak, aqt_flax_test.py:160-198) and must land in 'qlhs'."""
+  dt = 'bf16'
+  wgt, x = U.to_dev(U.rand((64, 48), dt, 1, 0.05), dt, gpu), U.to_dev(U.rand((16, 64), dt, 2), dt, gpu)
+  cfg = config.fully_quantized(use_stochastic_rounding=False)
+  conv = aqt_flax.AqtEinsum(cfg, lhs_quant_mode=QM.CONVERT, lhs_freeze_mode=FM.CALIBRATION_AND_VALUE, rngs=_rngs())
+  out = conv('bc,ab->ac', wgt, x)
+  assert tuple(out.shape) == (16, 48)
+  v = conv.variables()
+  assert set(v['aqt']) == {'qlhs'} and tuple(v['aqt']['qlhs']['value'].shape) == (64, 48)
+  ref = aqt.einsum('bc,ab->ac', wgt, x, config.set_context(cfg, utils.prng_key(0), None))
+  assert torch.equal(out, ref)
+
+
+def test_tiling_injection(gpu):
+  """aqt_flax_test.py:381-410: tile sizes by einsum letter; the layer result equals
+  tiled_dot_general around the same quantized dot_general."""
+  dt = 'bf16'
+  lhs, rhs = U.to_dev(U.rand((6, 4, 256), dt, 1), dt, gpu), U.to_dev(U.rand((10, 4, 256), dt, 2, 0.02), dt, gpu)
+  cfg = config.fully_quantized(use_stochastic_rounding=False)
+  layer = aqt_flax.AqtEinsum(cfg, tile_sizes={'d': 64}, rngs=_rngs())
+  out = layer('abd,cbd->ac', lhs, rhs)
+  tcfg = tiled_dot_general.Cfg.from_einsum('abd,cbd->ac', {'d': 64})
+  dg = config.set_context(cfg, utils.prng_key(0), None)
+  want = tiled_dot_general.tiled_dot_general(tcfg, lhs, rhs, (((1, 2), (1, 2)), ((), ())), dot_general=dg)
+  assert tuple(out.shape) == (6, 10) and torch.equal(out, want)
+  untiled = aqt_flax.AqtEinsum(cfg, rngs=_rngs())('abd,cbd->ac', lhs, rhs)
+  assert not torch.equal(out, untiled) and torch.allclose(out.float(), untiled.float(), rtol=0.1, atol=0.05)
