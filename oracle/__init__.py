@@ -29,4 +29,11 @@ Pin status of each part (what fixes it without importing JAX):
   * tiling / LocalAqt .................. reference known-answer tests
   * fp8 SR (fp_mantissa_round) ......... closed form on bit patterns; the random
                                          bits feeding it inherit the PRNG pins
+  * order of float32 sums (over tiles, over LocalAqt shards, inside an fp8
+    contraction) ....................... PARITY UNPINNED (XLA-internal); sums here
+                                         run in index order, fp8 dots are exact in
+                                         float64 and rounded once
+  * dequant with scales of different dtypes
+        ................................ jnp promotion rule, product by product
+                                         (bf16*bf16 -> bf16, anything with f32 -> f32)
 """
