@@ -17,6 +17,8 @@
 //     layout through LDS so that the consumer GEMM finds its contraction axis
 //     contiguous.
 #include "common.h"
+#include <type_traits>
+
 #include "threefry.h"
 
 namespace aqtx {
@@ -155,6 +157,8 @@ __device__ __forceinline__ uint32_t to_qbyte(float t, int out_dtype) {
 // ---- compile-time specialisations of the element pipeline ------------------------------
 // SPEC 0: every flag is read from QArgs at run time (any dtype / numerics).
 // SPEC 1: bf16 values, bf16 scale, int8 out, round to nearest even (the forward operands).
+// SPEC 3: bf16 values, bf16 scale, fp8 out (e4m3fn or e5m2), no noise.
+// SPEC 5: SPEC 3 + fp8 mantissa stochastic rounding, 16-bit draws of the original layout.
 // SPEC 2: SPEC 1 + jax.random.uniform noise in the original threefry counter layout (the
 //         gradient-side operands).  With PAIR the two elements that share one threefry block
 //         (indices i and i + total/2) are produced by the same thread from a single block.
@@ -170,13 +174,20 @@ __device__ __forceinline__ float uniform_noise(uint32_t bits) {
 }
 template <int SPEC>
 __device__ __forceinline__ uint32_t spec_finish(float t, const QArgs& a) {
-  // clip, round half to even, cast (int_numerics.py:99-110)
-  if constexpr (SPEC == 0) {
+  // clip, round half to even, cast (int_numerics.py:99-110; fp8_numerics.py:112-123)
+  if constexpr (SPEC == 0 || SPEC == 3 || SPEC == 5) {
     t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
     return to_qbyte(t, a.out_dtype);
   }
   t = fminf(fmaxf(t, -127.0f), 127.0f);
   return (uint32_t)((int)rintf(t)) & 0xFFu;
+}
+// fp_mantissa_round on a bf16 value (fp8_numerics.py:36-64): add the masked random bits to the
+// bit pattern, clear the low mantissa bits.
+__device__ __forceinline__ float bf16_mantissa_sr(float t, uint32_t bits, uint32_t mask) {
+  uint32_t u = __float_as_uint(t) >> 16;
+  u = ((u + (bits & mask)) & ~mask) & 0xFFFFu;
+  return __uint_as_float(u << 16);
 }
 // scale -> (noise) -> clip/round/cast for one element
 template <int SPEC>
@@ -186,6 +197,10 @@ __device__ __forceinline__ uint32_t spec_quant(float v, float inv, uint64_t ctr,
   } else {
     float t = spec_scale<SPEC>(v, inv, a);
     if constexpr (SPEC == 2) t = round_bf16(t + uniform_noise(a.gen.word_original((uint32_t)ctr)));
+    if constexpr (SPEC == 5) {
+      const uint32_t w = a.gen.word_original((uint32_t)(ctr >> 1));
+      t = bf16_mantissa_sr(t, (ctr & 1) ? (w >> 16) : w, a.out_dtype == AQTX_E4M3 ? 0xFu : 0x1Fu);
+    }
     return spec_finish<SPEC>(t, a);
   }
 }
@@ -494,71 +509,105 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) packed[s][e] = 0u;
 
+  // Tiles that lie wholly inside the tensor (and inside the first half of a paired axis) take a
+  // branch-free path with vector loads of the reciprocal scales and the pre-scale factors.
+  const bool interior = vec_ok && (r0[0] + kTileR <= row_lim) && (c0[0] + kTileC <= col_lim) &&
+                        (a.ssc == 0 || (a.ssc == 1 && a.ssb % 4 == 0 && a.ssg % 4 == 0 &&
+                                        ((uintptr_t)a.ws_inv % 16) == 0)) &&
+                        (a.ps_mode != AQTX_PRESCALE_PER_COL || a.psb % 4 == 0);
+  auto load8f = [](const float* p, float* v) {
+    const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+  };
+  auto rows = [&](auto fast_tag) {
+    constexpr bool FAST = decltype(fast_tag)::value;
+    float ps_col[NSET][8];
+    if constexpr (FAST) {
+      if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t rl = r0[0] + rg * 4 + j;  // position inside the first tile's half
-    const int64_t cl = c0[0] + cc * 8;
-    if (rl < row_lim && cl < col_lim) {
-      const int nvalid = (col_lim - cl) >= 8 ? 8 : (int)(col_lim - cl);
-      float x[NSET][8], inv[NSET][8];
-#pragma unroll
-      for (int s = 0; s < NSET; ++s) {
-        const int64_t r = r0[s] + rg * 4 + j, c = c0[s] + cc * 8;
-        if (vec_ok) {
-          Loader<TIn>::load8(xb + r * a.cols + c, x[s]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            x[s][e] = e < nvalid ? Loader<TIn>::load1(xb + r * a.cols + c + e) : 0.0f;
-        }
-        const int64_t sbase = b * a.ssb + (r / a.G) * a.ssg;
-        if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
-          const float rp = a.prescale[b * a.psb + r];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) x[s][e] = spec_prescale<SPEC>(x[s][e], rp, a);
-        } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (e < nvalid) x[s][e] = spec_prescale<SPEC>(x[s][e], a.prescale[b * a.psb + c + e], a);
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) inv[s][e] = e < nvalid ? a.ws_inv[sbase + (c + e) * a.ssc] : 1.0f;
+        for (int s = 0; s < NSET; ++s) load8f(a.prescale + b * a.psb + c0[s] + cc * 8, ps_col[s]);
       }
-      uint32_t w[NSET][2];
+    }
 #pragma unroll
-      for (int s = 0; s < NSET; ++s) w[s][0] = w[s][1] = 0u;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if (e < nvalid) {
-          uint32_t qv[NSET];
-          if constexpr (PAIR) {
-            const uint32_t i = (uint32_t)((r0[0] + rg * 4 + j) * a.nsr + (c0[0] + cc * 8 + e) * a.nsc);
-            pair_quant(x[0][e], inv[0][e], x[1][e], inv[1][e], i, a, qv[0], qv[1]);
-          } else {
-            const uint64_t ctr = (uint64_t)(b * a.nsb + rl * a.nsr + (cl + e) * a.nsc);
-            qv[0] = spec_quant<SPEC>(x[0][e], inv[0][e], ctr, a);
-          }
-#pragma unroll
-          for (int s = 0; s < NSET; ++s) {
-            w[s][e >> 2] |= qv[s] << (8 * (e & 3));
-            packed[s][e] |= qv[s] << (8 * j);
-          }
-        }
-      }
-      if (!a.transpose_out) {
+    for (int j = 0; j < 4; ++j) {
+      const int64_t rl = r0[0] + rg * 4 + j;  // position inside the first tile's half
+      const int64_t cl = c0[0] + cc * 8;
+      if (FAST || (rl < row_lim && cl < col_lim)) {
+        const int nvalid = FAST ? 8 : ((col_lim - cl) >= 8 ? 8 : (int)(col_lim - cl));
+        float x[NSET][8], inv[NSET][8];
 #pragma unroll
         for (int s = 0; s < NSET; ++s) {
           const int64_t r = r0[s] + rg * 4 + j, c = c0[s] + cc * 8;
-          if (vec_ok) {
-            *reinterpret_cast<uint2*>(qb + r * a.cols + c) = make_uint2(w[s][0], w[s][1]);
+          if (FAST || vec_ok) {
+            Loader<TIn>::load8(xb + r * a.cols + c, x[s]);
           } else {
-            for (int e = 0; e < nvalid; ++e)
-              qb[r * a.cols + c + e] = (uint8_t)(w[s][e >> 2] >> (8 * (e & 3)));
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              x[s][e] = e < nvalid ? Loader<TIn>::load1(xb + r * a.cols + c + e) : 0.0f;
+          }
+          const int64_t sbase = b * a.ssb + (r / a.G) * a.ssg;
+          if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+            const float rp = a.prescale[b * a.psb + r];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[s][e] = spec_prescale<SPEC>(x[s][e], rp, a);
+          } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              if constexpr (FAST) x[s][e] = spec_prescale<SPEC>(x[s][e], ps_col[s][e], a);
+              else if (e < nvalid) x[s][e] = spec_prescale<SPEC>(x[s][e], a.prescale[b * a.psb + c + e], a);
+            }
+          }
+          if constexpr (FAST) {
+            if (a.ssc == 0) {
+              const float v = a.ws_inv[sbase];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) inv[s][e] = v;
+            } else {
+              load8f(a.ws_inv + sbase + c, inv[s]);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) inv[s][e] = e < nvalid ? a.ws_inv[sbase + (c + e) * a.ssc] : 1.0f;
+          }
+        }
+        uint32_t w[NSET][2];
+#pragma unroll
+        for (int s = 0; s < NSET; ++s) w[s][0] = w[s][1] = 0u;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (FAST || e < nvalid) {
+            uint32_t qv[NSET];
+            if constexpr (PAIR) {
+              const uint32_t i = (uint32_t)((r0[0] + rg * 4 + j) * a.nsr + (c0[0] + cc * 8 + e) * a.nsc);
+              pair_quant(x[0][e], inv[0][e], x[1][e], inv[1][e], i, a, qv[0], qv[1]);
+            } else {
+              const uint64_t ctr = (uint64_t)(b * a.nsb + rl * a.nsr + (cl + e) * a.nsc);
+              qv[0] = spec_quant<SPEC>(x[0][e], inv[0][e], ctr, a);
+            }
+#pragma unroll
+            for (int s = 0; s < NSET; ++s) {
+              w[s][e >> 2] |= qv[s] << (8 * (e & 3));
+              packed[s][e] |= qv[s] << (8 * j);
+            }
+          }
+        }
+        if (!a.transpose_out) {
+#pragma unroll
+          for (int s = 0; s < NSET; ++s) {
+            const int64_t r = r0[s] + rg * 4 + j, c = c0[s] + cc * 8;
+            if (FAST || vec_ok) {
+              *reinterpret_cast<uint2*>(qb + r * a.cols + c) = make_uint2(w[s][0], w[s][1]);
+            } else {
+              for (int e = 0; e < nvalid; ++e)
+                qb[r * a.cols + c + e] = (uint8_t)(w[s][e >> 2] >> (8 * (e & 3)));
+            }
           }
         }
       }
     }
-  }
+  };
+  if (interior) rows(std::true_type{});
+  else rows(std::false_type{});
   if (!a.transpose_out) return;  // uniform across the block
 
   // Transposed write: LDS holds each tile as [col][row bytes], row stride 132 B.
@@ -689,6 +738,11 @@ int noise_width(const aqtx_quant_plan* p) {
 
 // Which compile-time specialisation (see spec_quant) serves this plan.
 int spec_of(const QArgs& a, int partitionable) {
+  if (a.cbf && a.sbf && !a.scale_given && (a.out_dtype == AQTX_E4M3 || a.out_dtype == AQTX_E5M2)) {
+    if (a.noise == AQTX_NOISE_NONE) return 3;
+    if (a.noise == AQTX_NOISE_FP8_MANTISSA && !partitionable && a.gen.width == 16) return 5;
+    return 0;
+  }
   if (!(a.cbf && a.sbf && a.out_dtype == AQTX_I8 && !a.scale_given)) return 0;
   if (a.quant_bound != 127.5f || a.clip_bound != 127.0f) return 0;
   if (a.noise == AQTX_NOISE_NONE) return 1;
@@ -728,6 +782,8 @@ int launch_rows(const QArgs& a, int partitionable, hipStream_t st) {
   }
   const int spec = spec_of(a, partitionable);
   if (spec == 1) return launch_rows_spec<TIn, 1, false>(a, st);
+  if (spec == 3) return launch_rows_spec<TIn, 3, false>(a, st);
+  if (spec == 5) return launch_rows_spec<TIn, 5, false>(a, st);
   if (spec == 2) {
     // one threefry block serves elements i and i + total/2: pair whole rows when the noise
     // counters follow the natural [batch*rows, cols] order
@@ -772,6 +828,10 @@ int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales,
   };
   if (spec == 1) {
     quant_tile_kernel<TIn, 1, 0><<<grid_for(0), 256, 0, st>>>(a);
+  } else if (spec == 3) {
+    quant_tile_kernel<TIn, 3, 0><<<grid_for(0), 256, 0, st>>>(a);
+  } else if (spec == 5) {
+    quant_tile_kernel<TIn, 5, 0><<<grid_for(0), 256, 0, st>>>(a);
   } else if (spec == 2) {
     // pair the two elements of each threefry block: i and i + total/2 lie rows/2 apart when the
     // noise counters are row-major over [rows, cols], cols/2 apart when over [cols, rows]
