@@ -453,11 +453,34 @@ __global__ __launch_bounds__(256) void absmax_all_kernel(const QArgs a) {
   const int64_t n = a.rows * a.cols;
   const TIn* xb = reinterpret_cast<const TIn*>(a.x) + b * n;
   float m = 0.0f;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    float v = Loader<TIn>::load1(xb + i);
-    if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[b * a.psb + i / a.cols], a);
-    else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[b * a.psb + i % a.cols], a);
-    m = fmaxf(m, fabsf(v));
+  if (a.cols % 8 == 0 && (a.ps_mode != AQTX_PRESCALE_PER_COL || a.psb % 4 == 0)) {
+    // 8 elements (one row segment) per lane and load
+    const int64_t stride = (int64_t)gridDim.x * 256 * 8;
+#pragma unroll 4
+    for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += stride) {
+      float v[8];
+      Loader<TIn>::load8(xb + i, v);
+      if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+        const float rp = a.prescale[b * a.psb + i / a.cols];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = apply_prescale(v[e], rp, a);
+      } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+        const float* pc = a.prescale + b * a.psb + i % a.cols;
+        const float4 lo = *reinterpret_cast<const float4*>(pc), hi = *reinterpret_cast<const float4*>(pc + 4);
+        const float ps[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = apply_prescale(v[e], ps[e], a);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(v[e]));
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+      float v = Loader<TIn>::load1(xb + i);
+      if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[b * a.psb + i / a.cols], a);
+      else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[b * a.psb + i % a.cols], a);
+      m = fmaxf(m, fabsf(v));
+    }
   }
   m = segment_max<256>(m, smem);
   if (threadIdx.x == 0) atomicMax(a.ws_absmax + b * a.ssb, __float_as_uint(m));
@@ -481,7 +504,7 @@ __global__ void finalize_scales_kernel(const QArgs a, int64_t n) {
 constexpr int kTileR = 128, kTileC = 64, kTilePad = 132;
 
 // 128x64 tile: thread (rg = tid/8, cc = tid%8) owns rows 4*rg..+3, cols 8*cc..+7.
-// PAIR (SPEC 2 only): 1 = the block also owns the tile `rows/2` further down (natural noise
+// PAIR (SPEC 2, and SPEC 5 with value 1): 1 = the block also owns the tile `rows/2` further down (natural noise
 // layout), 2 = the tile `cols/2` further right (noise counters of the transposed tensor); the
 // two tiles' elements share threefry blocks.
 template <typename TIn, int SPEC, int PAIR>
@@ -573,11 +596,31 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a) {
         uint32_t w[NSET][2];
 #pragma unroll
         for (int s = 0; s < NSET; ++s) w[s][0] = w[s][1] = 0u;
+        U2 wbits{0u, 0u};  // SPEC 5: the 32-bit word(s) two neighbouring elements draw their 16 bits from
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           if (FAST || e < nvalid) {
             uint32_t qv[NSET];
-            if constexpr (PAIR) {
+            if constexpr (SPEC == 5) {
+              // 16-bit draws: elements 2w and 2w+1 share word w; with PAIR the block (w, w + half)
+              // also serves the same two elements of the tile rows/2 further down.
+              const uint32_t sr_mask = a.out_dtype == AQTX_E4M3 ? 0xFu : 0x1Fu;
+              const uint64_t ctr = (uint64_t)(b * a.nsb + rl * a.nsr + (cl + e) * a.nsc);
+              if ((e & 1) == 0) {
+                if constexpr (PAIR) {
+                  wbits = threefry2x32(a.gen.k0, a.gen.k1, (uint32_t)(ctr >> 1), (uint32_t)(ctr >> 1) + a.gen.half);
+                } else {
+                  wbits.x = a.gen.word_original((uint32_t)(ctr >> 1));
+                }
+              }
+              const int sh = (e & 1) * 16;
+#pragma unroll
+              for (int s = 0; s < NSET; ++s) {
+                float t = round_bf16(x[s][e] * inv[s][e]);
+                t = bf16_mantissa_sr(t, (s == 0 ? wbits.x : wbits.y) >> sh, sr_mask);
+                qv[s] = spec_finish<5>(t, a);
+              }
+            } else if constexpr (PAIR) {
               const uint32_t i = (uint32_t)((r0[0] + rg * 4 + j) * a.nsr + (c0[0] + cc * 8 + e) * a.nsc);
               pair_quant(x[0][e], inv[0][e], x[1][e], inv[1][e], i, a, qv[0], qv[1]);
             } else {
@@ -740,7 +783,9 @@ int noise_width(const aqtx_quant_plan* p) {
 int spec_of(const QArgs& a, int partitionable) {
   if (a.cbf && a.sbf && !a.scale_given && (a.out_dtype == AQTX_E4M3 || a.out_dtype == AQTX_E5M2)) {
     if (a.noise == AQTX_NOISE_NONE) return 3;
-    if (a.noise == AQTX_NOISE_FP8_MANTISSA && !partitionable && a.gen.width == 16) return 5;
+    if (a.noise == AQTX_NOISE_FP8_MANTISSA && !partitionable && a.gen.width == 16 && a.nsc == 1 &&
+        a.nsr % 2 == 0 && a.nsb % 2 == 0)
+      return 5;  // neighbouring elements draw from one word, starting at an even counter
     return 0;
   }
   if (!(a.cbf && a.sbf && a.out_dtype == AQTX_I8 && !a.scale_given)) return 0;
@@ -831,7 +876,11 @@ int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales,
   } else if (spec == 3) {
     quant_tile_kernel<TIn, 3, 0><<<grid_for(0), 256, 0, st>>>(a);
   } else if (spec == 5) {
-    quant_tile_kernel<TIn, 5, 0><<<grid_for(0), 256, 0, st>>>(a);
+    // half of a threefry block would be thrown away unless the tile rows/2 further down, whose
+    // elements draw from the other half, is quantized by the same workgroup
+    const bool natural = a.batch == 1 && a.nsr == a.cols && (a.rows % 2 == 0) && (a.cols % 8 == 0);
+    if (natural) quant_tile_kernel<TIn, 5, 1><<<grid_for(1), 256, 0, st>>>(a);
+    else quant_tile_kernel<TIn, 5, 0><<<grid_for(0), 256, 0, st>>>(a);
   } else if (spec == 2) {
     // pair the two elements of each threefry block: i and i + total/2 lie rows/2 apart when the
     // noise counters are row-major over [rows, cols], cols/2 apart when over [cols, rows]

@@ -211,3 +211,25 @@ def test_local_aqt_largest_shape(gpu):
   ocfg.dlhs.local_aqt_shard_count, ocfg.drhs.local_aqt_shard_count = 96 // 32, 64 // 32
   got, want = _run_both(lhs, rhs, g, dt, MATMUL, cfg, ocfg, prng.prng_key(11), gpu)
   _assert_same(got, want)
+
+
+def test_fp8_per_tensor_einsum_projection(gpu):
+  """The attention-projection config: 'bsd,dhk->bshk', per-tensor abs-max scales, e4m3 forward,
+  e5m2 gradients with mantissa stochastic rounding on the gradient side.  Quantized values and
+  scales bit-exact; contraction outputs within one bf16 ulp plus an absolute term (the MFMA's
+  f32 summation order is not XLA's)."""
+  dt = 'bf16'
+  dn = (((2,), (0,)), ((), ()))
+  lhs, rhs = U.rand((2, 64, 128), dt, 1, outliers=True), U.rand((128, 4, 32), dt, 2, 0.02)
+  g = U.rand((2, 64, 4, 32), dt, 3, 1e-3)
+  cfg = config.config_v4(fwd_bits='e4m3', dlhs_bits='e5m2', drhs_bits='e5m2')
+  ocfg = R.config_v4('e4m3', 'e5m2', 'e5m2')
+  for raw, oraw in ((cfg.fwd, ocfg.fwd), (cfg.dlhs, ocfg.dlhs), (cfg.drhs, ocfg.drhs)):
+    raw.dg_quantizer.lhs.calib_shared_axes = raw.dg_quantizer.rhs.calib_shared_axes = 'per_tensor'
+    oraw.lhs.calib_shared_axes = oraw.rhs.calib_shared_axes = 'per_tensor'
+  got, want = _run_both(lhs, rhs, g, dt, dn, cfg, ocfg, prng.prng_key(21), gpu)
+  for k in ('lq', 'rq', 'ls', 'rs'):
+    np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+  for k in ('out', 'dlhs', 'drhs'):
+    np.testing.assert_allclose(got[k], want[k], rtol=2.0 ** -7, atol=2.0 ** -9 * np.abs(want[k]).max(),
+                               err_msg=k)
