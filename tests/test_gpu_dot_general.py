@@ -233,3 +233,38 @@ def test_fp8_per_tensor_einsum_projection(gpu):
   for k in ('out', 'dlhs', 'drhs'):
     np.testing.assert_allclose(got[k], want[k], rtol=2.0 ** -7, atol=2.0 ** -9 * np.abs(want[k]).max(),
                                err_msg=k)
+
+
+def test_mlp_block_fp32_full_size(gpu):
+  """The MlpBlock config at its real size: x f32 [4096, 512], Dense 512 -> 2048, ReLU,
+  Dense 2048 -> 512, fully_quantized(8, 8) with stochastic rounding in the backward pass;
+  forward activations, both weight gradients and the input gradient are bit-exact."""
+  dt = 'f32'
+  rng = np.random.default_rng(0)
+  x = U.rand((4096, 512), dt, 1)
+  w1 = (rng.standard_normal((512, 2048)) / np.sqrt(512)).astype(np.float32)
+  w2 = (rng.standard_normal((2048, 512)) / np.sqrt(2048)).astype(np.float32)
+  g = U.rand((4096, 512), dt, 4, 1.0 / (4096 * 512))
+  k1, k2 = prng.prng_key(1), prng.prng_key(2)
+  # product
+  X = U.to_dev(x, dt, gpu).requires_grad_(True)
+  W1 = U.to_dev(w1, dt, gpu).requires_grad_(True)
+  W2 = U.to_dev(w2, dt, gpu).requires_grad_(True)
+  dg1 = config.set_context(config.fully_quantized(fwd_bits=8, bwd_bits=8), k1, None)
+  dg2 = config.set_context(config.fully_quantized(fwd_bits=8, bwd_bits=8), k2, None)
+  h = dg1(X, W1, MATMUL)
+  y = dg2(torch.relu(h), W2, MATMUL)
+  y.backward(U.to_dev(g, dt, gpu))
+  # oracle
+  o1, o2 = R.set_context(R.fully_quantized(8, 8), k1), R.set_context(R.fully_quantized(8, 8), k2)
+  f1 = R.dg_fwd(x, w1, dt, MATMUL, o1)
+  act = np.maximum(f1.out, np.float32(0))
+  f2 = R.dg_fwd(act, w2, dt, MATMUL, o2)
+  dact, dw2 = R.dg_bwd(g, dt, MATMUL, f2, o2)
+  dh = np.where(f1.out > 0, dact, np.float32(0)).astype(np.float32)
+  dx, dw1 = R.dg_bwd(dh, dt, MATMUL, f1, o1)
+  np.testing.assert_array_equal(_np(h), f1.out)
+  np.testing.assert_array_equal(_np(y), f2.out)
+  np.testing.assert_array_equal(_np(W2.grad), dw2)
+  np.testing.assert_array_equal(_np(W1.grad), dw1)
+  np.testing.assert_array_equal(_np(X.grad), dx)
