@@ -47,6 +47,15 @@ class GemmPlan(ctypes.Structure):
   ]
 
 
+class GroupedGemmPlan(ctypes.Structure):
+  _fields_ = [
+      ('m', ctypes.c_int64), ('n', ctypes.c_int64), ('k', ctypes.c_int64), ('group', ctypes.c_int64),
+      ('lda', ctypes.c_int64), ('ldb', ctypes.c_int64), ('ldc', ctypes.c_int64),
+      ('a_dtype', ctypes.c_int32), ('b_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
+      ('row_scale_dtype', ctypes.c_int32), ('col_scale_dtype', ctypes.c_int32),
+  ]
+
+
 class DecodePlan(ctypes.Structure):
   _fields_ = [
       ('m', ctypes.c_int64), ('n', ctypes.c_int64), ('k', ctypes.c_int64),
@@ -68,6 +77,8 @@ SYMBOLS = {
     'aqtx_decode_i8': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
+    'aqtx_gemm_i8_grouped': (ctypes.c_int, [ctypes.POINTER(GroupedGemmPlan), _vp, _vp, _vp, _vp, _vp, _vp]),
+    'aqtx_pack_i4': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, _vp]),
     'aqtx_sum_tiles': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),
     'aqtx_prng_split_host': (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint32), ctypes.c_int32,
                                             ctypes.c_int32, ctypes.POINTER(ctypes.c_uint32)]),

@@ -16,12 +16,15 @@ CSRC = os.path.join(HERE, 'csrc')
 LIB_DIR = os.path.join(HERE, 'lib')
 LIB_PATH = os.path.join(LIB_DIR, 'libaqtx.so')
 
-SOURCES = ['capi.hip', 'quantize.hip', 'gemm_i8.hip', 'gemm_fp8.hip', 'decode_i8.hip', 'reduce.hip']
+SOURCES = ['capi.hip', 'quantize.hip', 'gemm_i8.hip', 'gemm_fp8.hip', 'decode_i8.hip', 'reduce.hip',
+           'gemm_grouped.hip']
 
 HIPCC_FLAGS = [
     '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC',
     # packed-FP32 VALU forms are kept out of generated code on purpose
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+    # every float product and sum of the reference rounds on its own: no fused multiply-add
+    '-ffp-contract=off',
     '-Wno-unused-command-line-argument', '-Wno-pass-failed',
 ]
 

@@ -253,6 +253,42 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   return (out, x_scale, xq) if want_xq else (out, x_scale)
 
 
+def pack_i4(q: torch.Tensor) -> torch.Tensor:
+  """int4 values held one per int8 byte, last axis even -> uint8 tensor with the last axis halved."""
+  _require_gpu(q)
+  assert q.dtype == torch.int8 and q.is_contiguous() and q.shape[-1] % 2 == 0
+  out = torch.empty(q.shape[:-1] + (q.shape[-1] // 2,), dtype=torch.uint8, device=q.device)
+  L.check(L.lib().aqtx_pack_i4(_ptr(q), _ptr(out), q.numel(), _stream()))
+  return out
+
+
+def gemm_grouped(a: torch.Tensor, b: torch.Tensor, *, row_scale: torch.Tensor, col_scale: torch.Tensor,
+                 group: int, out_dtype, row_scale_dtype=None, col_scale_dtype=None, a_dtype: int = L.I8,
+                 b_dtype: int = L.I8):
+  """C = cast(sum_g dequant_g(A_g @ B_g^T)) for A int8 [m, k], B int8 [n, k] (or packed int4
+  uint8 [n, k/2] with b_dtype=I4P), row_scale float32 [k/group, m], col_scale float32 [k/group, n]."""
+  _require_gpu(a, b, row_scale, col_scale)
+  m, k = a.shape
+  n = b.shape[0]
+  packed = b_dtype == L.I4P
+  assert a.stride(1) == 1 and b.stride(1) == 1 and b.shape[1] == (k // 2 if packed else k)
+  groups = k // group
+  for s_, dim in ((row_scale, m), (col_scale, n)):
+    assert s_.dtype == torch.float32 and s_.is_contiguous() and tuple(s_.shape) == (groups, dim), tuple(s_.shape)
+  out_dt = aqtx_dtype(out_dtype)
+  plan = L.GroupedGemmPlan()
+  plan.m, plan.n, plan.k, plan.group = m, n, k, group
+  plan.lda, plan.ldb, plan.ldc = a.stride(0), b.stride(0), n
+  plan.a_dtype, plan.b_dtype, plan.out_dtype = a_dtype, b_dtype, out_dt
+  plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else out_dt
+  plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else out_dt
+  c = torch.empty((m, n), dtype=_AQTX_TO_TORCH[out_dt], device=a.device)
+  with _timed('gemm_grouped'):
+    L.check(L.lib().aqtx_gemm_i8_grouped(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale),
+                                         _ptr(col_scale), _ptr(c), _stream()))
+  return c
+
+
 def sum_tiles(x: torch.Tensor) -> torch.Tensor:
   """Sum over the leading axis of a contiguous bf16/f32 tensor: float32 accumulation in index
   order, one rounding (jnp.sum semantics for the per-tile outputs of a tiled dot_general)."""

@@ -168,6 +168,44 @@ int aqtx_gemm_fp8(const aqtx_gemm_plan* plan, const void* a, const void* b,
                   float* acc_out, void* stream);
 
 /*
+ * Plan of a contraction whose operands carry one scale per `group` consecutive
+ * elements of the contraction axis (subchannel / tiled quantization).
+ */
+typedef struct aqtx_grouped_gemm_plan {
+  int64_t m, n, k;
+  int64_t group;              /* multiple of 128 that divides k                            */
+  int64_t lda, ldb, ldc;      /* row strides in elements (ldb in bytes for AQTX_I4P)        */
+  int32_t a_dtype;            /* AQTX_I8 | AQTX_I4                                          */
+  int32_t b_dtype;            /* AQTX_I8 | AQTX_I4 | AQTX_I4P (packed, low nibble = even k) */
+  int32_t out_dtype;          /* AQTX_BF16 | AQTX_F32: dequant dtype = output dtype         */
+  int32_t row_scale_dtype, col_scale_dtype; /* AQTX_BF16 | AQTX_F32                         */
+} aqtx_grouped_gemm_plan;
+
+/*
+ * aqtx_gemm_i8_grouped: C[m,n] = cast(sum_g dequant_g(sum_{k in g} A[m,k] B[n,k])) with
+ * dequant_g = QTensor.dequant with the scales of group g.  Replaces tiled_dot_general
+ * (aqt/jax/v2/tiled_dot_general.py:407-543) around a quantizing dot_general for a tiled
+ * contraction axis: the inner per-tile contractions (tile-count axis as a batch axis,
+ * :430-435), their dequantisation (aqt_tensor.py:161-200, each tile rounded to the dequant
+ * dtype) and the sum over tiles (:493, float32 accumulation in tile order), without
+ * materialising the per-tile outputs.
+ *   a          : int8 [m][lda]
+ *   b          : int8 [n][ldb], or packed int4 [n][ldb bytes]
+ *   row_scale  : float32 [k/group][m]   (scale of A's row m in group g)
+ *   col_scale  : float32 [k/group][n]
+ *   c          : [m][ldc] of out_dtype
+ */
+int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* plan, const void* a, const void* b,
+                         const float* row_scale, const float* col_scale, void* c, void* stream);
+
+/*
+ * aqtx_pack_i4: `count` int4 values held one per int8 byte -> count/2 bytes, two per byte
+ * (low nibble = even index).  The reference stores jnp.int4 arrays (int_numerics.py:109-110);
+ * the packed layout is this library's storage format for frozen int4 weights.
+ */
+int aqtx_pack_i4(const void* src, void* dst, int64_t count, void* stream);
+
+/*
  * aqtx_sum_tiles: out[i] = cast(sum over t of x[t][i]) for x [tiles][count] of
  * bf16 or f32, accumulated in float32 in tile order and rounded once.  Replaces
  * the sum over the tile-count axes of the per-tile (already dequantized) outputs

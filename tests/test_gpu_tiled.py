@@ -66,3 +66,41 @@ def test_tiled_qtensors_and_scales(gpu):
   np.testing.assert_array_equal(lqt.scale[0].float().cpu().numpy(), res.lhs_res.qx.scale[0])
   np.testing.assert_array_equal(rqt.scale[0].float().cpu().numpy(), res.rhs_res.qx.scale[0])
   assert np.abs(rqt.qvalue.float().cpu().numpy()).max() <= 7
+
+
+# ---- grouped-scale contraction kernel -----------------------------------------------------------
+def _grouped_ref(a, b, rs, cs, group, out, rdt, cdt):
+  """Per group: QTensor.dequant of the group's int32 accumulators, rounded to `out`; float32 sum
+  of the groups in order; one final cast."""
+  m, k = a.shape
+  n = b.shape[0]
+  acc = np.zeros((m, n), np.float32)
+  for g in range(k // group):
+    sl = slice(g * group, (g + 1) * group)
+    part = (a[:, sl].astype(np.int64) @ b[:, sl].astype(np.int64).T).astype(np.int32)
+    dq = R.dequant(R.QTensor(part, 'i32', [rs[g][:, None], cs[g][None, :]], None, out, scale_dtypes=[rdt, cdt]))
+    acc = acc + dq
+  return nm.cast(acc, out)
+
+
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('out,rdt,cdt', [('bf16', 'bf16', 'bf16'), ('bf16', 'bf16', 'f32'), ('f32', 'f32', 'f32')])
+@pytest.mark.parametrize('m,n,k,group', [(128, 256, 256, 128), (200, 300, 512, 128), (64, 520, 1024, 256), (5, 9, 128, 128)])
+def test_grouped_gemm_kernel(gpu, m, n, k, group, out, rdt, cdt, packed):
+  from aqt_amd import _lib as L
+  rng = np.random.default_rng(7)
+  a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+  b = rng.integers(-7, 8, (n, k)).astype(np.int8)
+  groups = k // group
+  rs = nm.cast(np.abs(rng.standard_normal((groups, m)).astype(np.float32)) * np.float32(0.02) + np.float32(1e-3), rdt)
+  cs = nm.cast(np.abs(rng.standard_normal((groups, n)).astype(np.float32)) * np.float32(3e-3) + np.float32(1e-4), cdt)
+  want = _grouped_ref(a, b, rs, cs, group, out, rdt, cdt)
+  bt = torch.from_numpy(b).to(gpu)
+  if packed:
+    bt = ops.pack_i4(bt)
+    np.testing.assert_array_equal(bt.cpu().numpy(), (b[:, 0::2] & 0xF).astype(np.uint8) | ((b[:, 1::2] & 0xF).astype(np.uint8) << 4))
+  got = ops.gemm_grouped(torch.from_numpy(a).to(gpu), bt, row_scale=torch.from_numpy(rs).to(gpu),
+                         col_scale=torch.from_numpy(cs).to(gpu), group=group, out_dtype=U.TORCH_DT[out],
+                         row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt],
+                         b_dtype=L.I4P if packed else L.I4)
+  np.testing.assert_array_equal(got.float().cpu().numpy(), want)
