@@ -156,7 +156,8 @@ __device__ __forceinline__ uint32_t to_qbyte(float t, int out_dtype) {
 
 // ---- compile-time specialisations of the element pipeline ------------------------------
 // SPEC 0: every flag is read from QArgs at run time (any dtype / numerics).
-// SPEC 1: bf16 values, bf16 scale, int8 out, round to nearest even (the forward operands).
+// SPEC 1: bf16 values, bf16 scale, integer out (int8, or int4 in an int8 byte), round to nearest
+//         even (the forward operands).
 // SPEC 3: bf16 values, bf16 scale, fp8 out (e4m3fn or e5m2), no noise.
 // SPEC 5: SPEC 3 + fp8 mantissa stochastic rounding, 16-bit draws of the original layout.
 // SPEC 2: SPEC 1 + jax.random.uniform noise in the original threefry counter layout (the
@@ -179,7 +180,7 @@ __device__ __forceinline__ uint32_t spec_finish(float t, const QArgs& a) {
     t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
     return to_qbyte(t, a.out_dtype);
   }
-  t = fminf(fmaxf(t, -127.0f), 127.0f);
+  t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
   return (uint32_t)((int)rintf(t)) & 0xFFu;
 }
 // fp_mantissa_round on a bf16 value (fp8_numerics.py:36-64): add the masked random bits to the
@@ -788,8 +789,7 @@ int spec_of(const QArgs& a, int partitionable) {
       return 5;  // neighbouring elements draw from one word, starting at an even counter
     return 0;
   }
-  if (!(a.cbf && a.sbf && a.out_dtype == AQTX_I8 && !a.scale_given)) return 0;
-  if (a.quant_bound != 127.5f || a.clip_bound != 127.0f) return 0;
+  if (!(a.cbf && a.sbf && (a.out_dtype == AQTX_I8 || a.out_dtype == AQTX_I4) && !a.scale_given)) return 0;
   if (a.noise == AQTX_NOISE_NONE) return 1;
   if (a.noise == AQTX_NOISE_JAX_UNIFORM && !partitionable) return 2;
   return 0;

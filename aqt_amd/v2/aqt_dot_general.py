@@ -13,6 +13,7 @@ import copy
 import dataclasses
 import enum
 import functools
+import math
 from typing import Any, Optional, Sequence
 
 import numpy as onp
@@ -708,6 +709,68 @@ class DotGeneral:
       return out, (lq, rq)
     (out, qret), _ = dg_core_vjp_fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, self)
     return out, qret
+
+  def fused_tile_sum(self, lhs, rhs, dimension_numbers, n_sum_axes: int):
+    """sum over the leading `n_sum_axes` output axes of self(lhs, rhs, dimension_numbers), fused.
+
+    This is what tiled_dot_general asks of its inner dot_general when the contraction axis is
+    tiled: lhs [..., T, ts] and rhs [T, ts, ...] with the tile-count axis T as the only batch
+    axis, every tile calibrated on its own, tile outputs dequantized and summed.  When the
+    forward quantizers are plain int8/int4 abs-max ones and no gradient is needed, the
+    grouped-scale kernel does all of it without materialising the per-tile outputs.  Returns
+    None when the call does not have that shape (the caller then takes the unfused route).
+    """
+    if n_sum_axes != 1 or torch.is_grad_enabled() and (lhs.requires_grad or rhs.requires_grad):
+      return None
+    (lca, rca), (lba, rba) = dimension_numbers
+    lca, rca, lba, rba = list(lca), list(rca), list(lba), list(rba)
+    cfg = _fresh_cfg(self)   # calibration objects are created per call, as in dg_core_vjp_fwd
+    cfg.fwd.dg_quantizer.init_calibration()
+    raw, dq = cfg.fwd, cfg.fwd.dg_quantizer
+    if (len(lca) != 1 or len(lba) != 1 or lhs.dtype != rhs.dtype or lhs.dtype not in (utils.bfloat16, utils.float32)
+        or not isinstance(dq, DefaultDotGeneralQuantizer) or raw.dg_accumulator_dtype != utils.int32
+        or raw.dot_general is not lax_dot_general or dq.lhs_mid_alpha is not None or dq.rhs_mid_alpha is not None):
+      return None
+    for side in (raw.lhs, raw.rhs):
+      if side.dequant_mode != DequantMode.OUTPUT or side.calibration_mode != CalibrationMode.CONTRACTING_AXIS:
+        return None
+    specs = []
+    for q in (dq.lhs, dq.rhs):
+      spec = q.kernel_spec()
+      if (spec is None or spec['out_dtype'] not in (L.I8, L.I4) or spec['noise'] != L.NOISE_NONE
+          or q.calib_shared_axes is not None or getattr(q.numerics, 'clip_gradient', False)):
+        return None
+      specs.append(spec)
+    nl, nr = lhs.dim(), rhs.dim()
+    # lhs [remaining..., T, ts], rhs [T, ts, remaining...], both dense in that order
+    if not (lba == [nl - 2] and lca == [nl - 1] and rba == [0] and rca == [1] and lhs.is_contiguous()
+            and rhs.is_contiguous()):
+      return None
+    T, ts = lhs.shape[-2], lhs.shape[-1]
+    if ts % 128 != 0 or rhs.shape[0] != T or rhs.shape[1] != ts or nl < 3 or nr < 3:
+      return None
+    self.assert_config_validity()
+    M = int(math.prod(lhs.shape[:-2]))
+    N = int(math.prod(rhs.shape[2:]))
+    if M == 0 or N == 0:
+      return None
+    sdts = []
+    outs = []
+    for x3, q, spec, reduce in ((lhs.reshape(1, M, T * ts), dq.lhs, specs[0], L.REDUCE_COLS),
+                                (rhs.reshape(1, T * ts, N), dq.rhs, specs[1], L.REDUCE_ROWS)):
+      sdt = q._calibrator.dtype if q._calibrator.dtype is not None else lhs.dtype
+      qv, sc = ops.quantize(x3, reduce=reduce, group=ts, transpose_out=reduce == L.REDUCE_ROWS,
+                            out_dtype=spec['out_dtype'], quant_bound=spec['quant_bound'],
+                            clip_bound=spec['clip_bound'], compute_dtype=lhs.dtype, scale_dtype=sdt)
+      outs.append((qv, sc))
+      sdts.append(sdt)
+    (lq, lsc), (rq, rsc) = outs
+    row_scale = lsc.reshape(M, T).t().contiguous()     # [T, M]
+    col_scale = rsc.reshape(T, N)
+    out = ops.gemm_grouped(lq[0], rq[0], row_scale=row_scale, col_scale=col_scale, group=ts,
+                           out_dtype=lhs.dtype, row_scale_dtype=sdts[0], col_scale_dtype=sdts[1],
+                           a_dtype=specs[0]['out_dtype'], b_dtype=specs[1]['out_dtype'])
+    return out.reshape(tuple(lhs.shape[:-2]) + tuple(rhs.shape[2:]))
 
   def __call__(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
     """aqt_dot_general.py:1002-1022."""

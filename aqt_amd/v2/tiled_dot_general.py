@@ -272,7 +272,15 @@ def tiled_dot_general_with_tiling_states(lhs, xlhs: TilingState, rhs, xrhs: Tili
   for ax in tiled_dn[0][1] + tiled_dn[1][1]:
     assert 0 <= ax < tr.dim()
 
-  out = dot_general(tl, tr, tiled_dn, precision, preferred_element_type)
+  # A quantizing dot_general may be able to contract, dequantize and sum the tiles in one kernel.
+  fused = getattr(dot_general, 'fused_tile_sum', None)
+  out = None
+  if fused is not None and l_ca_t and precision is None:
+    summed = fused(tl, tr, tiled_dn, len(l_ca_t))
+    if summed is not None:
+      out = summed.reshape((1,) * len(l_ca_t) + tuple(summed.shape))
+  if out is None:
+    out = dot_general(tl, tr, tiled_dn, precision, preferred_element_type)
 
   ca_t_sh = xlhs.axes_shape(l_ca_t)
   assert ca_t_sh == xrhs.axes_shape(r_ca_t)
@@ -283,13 +291,17 @@ def tiled_dot_general_with_tiling_states(lhs, xlhs: TilingState, rhs, xrhs: Tili
   r_ra_t_sh = xlhs.axes_shape(l_other)
   assert r_ra_t_sh == xrhs.axes_shape(r_ra_t)
   l_ra_sh, r_ra_sh = xlhs.axes_shape(l_ra), xrhs.axes_shape(r_ra)
+  if fused is not None and tuple(out.shape[:len(ca_t_sh)]) == (1,) * len(ca_t_sh) and ca_t_sh != (1,) * len(ca_t_sh):
+    ca_t_sh = (1,) * len(ca_t_sh)   # already summed by the fused kernel
   assert tuple(out.shape) == ca_t_sh + ba_sh + l_ra_t_sh + r_ra_t_sh + l_ra_sh + r_ra_sh, (
       tuple(out.shape), ca_t_sh, ba_sh, l_ra_t_sh, r_ra_t_sh, l_ra_sh, r_ra_sh)
 
   # Sum of the (dequantized) per-tile outputs over the contraction tile counts.  jnp.sum
   # accumulates 16-bit floats in float32 and rounds once; so does this.
   if ca_t_sh:
-    out = _sum_leading(out.reshape((-1,) + tuple(out.shape[len(ca_t_sh):])))
+    rest = tuple(out.shape[len(ca_t_sh):])
+    only_one = all(c == 1 for c in ca_t_sh)   # a single tile, or tiles already summed by the fused kernel
+    out = out.reshape(rest) if only_one else _sum_leading(out.reshape((-1,) + rest))
 
   # (ba, lhs ra counts, rhs ra counts, lhs ra sizes, rhs ra sizes) -> counts next to their sizes
   n0 = len(ba_sh)
