@@ -23,6 +23,21 @@ namespace {
 
 constexpr int GM = 128, GN = 256;  // GK = BK = 128
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// Rounds two floats to bf16 (ties to even) in place: one packed conversion, then one shift and
+// one mask to widen them again.
+template <bool kBf16>
+__device__ __forceinline__ void round_pair(float& a, float& b) {
+  if constexpr (kBf16) {
+    const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
+    const uint32_t w = __builtin_bit_cast(uint32_t, h);
+    a = __uint_as_float(w << 16);
+    b = __uint_as_float(w & 0xFFFF0000u);
+  }
+}
+
 struct GroupedArgs {
   const uint8_t* a;        // int8 [m][lda]
   const uint8_t* b;        // int8 [n][ldb], or packed int4 [n][ldb] with ldb in bytes (= k/2)
@@ -150,6 +165,7 @@ void gemm_grouped_kernel(const GroupedArgs g) {
     for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
       for (int r = 0; r < 16; ++r) { acc[mi][ni][r] = 0; sum[mi][ni][r] = 0.0f; }
+  const v16i kZero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
   const int nstages = g.groups * g.stages_per_group;
   load_stage(0);
@@ -172,11 +188,15 @@ void gemm_grouped_kernel(const GroupedArgs g) {
         fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[c]);
         fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c]);
       }
+      // the first MFMA of a group starts from a zero accumulator operand instead of zeroed registers
+      const bool fresh = ks == 0 && (s % g.stages_per_group) == 0;
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+        for (int ni = 0; ni < 2; ++ni) {
+          if (fresh) acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], kZero, 0, 0, 0);
+          else acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+        }
     }
     if (last_of_group) {
       // lane holds C[m = mi*32 + lr][n = ni*32 + 8q + 4lh + e], register 4q + e
@@ -193,14 +213,19 @@ void gemm_grouped_kernel(const GroupedArgs g) {
 #pragma unroll
           for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
+            for (int e = 0; e < 4; e += 2) {
               // every product and the sum round on their own (the library is built with
-              // floating-point contraction off, so no fused multiply-add appears here)
-              float f = round_to<kOutBf16>((float)acc[mi][ni][4 * q + e]);
-              f = round_to<kP1Bf16>(f * rs[mi]);
-              f = round_to<kP2Bf16>(f * cs[e]);
-              sum[mi][ni][4 * q + e] += round_to<kOutBf16>(f);
-              acc[mi][ni][4 * q + e] = 0;
+              // floating-point contraction off, so no fused multiply-add appears here); values
+              // are rounded two at a time (one packed conversion per pair)
+              float f0 = (float)acc[mi][ni][4 * q + e], f1 = (float)acc[mi][ni][4 * q + e + 1];
+              round_pair<kOutBf16>(f0, f1);
+              f0 *= rs[mi]; f1 *= rs[mi];
+              round_pair<kP1Bf16>(f0, f1);
+              f0 *= cs[e]; f1 *= cs[e + 1];
+              round_pair<kP2Bf16>(f0, f1);
+              if constexpr (kOutBf16 && !kP2Bf16) round_pair<true>(f0, f1);  // final cast of the tile
+              sum[mi][ni][4 * q + e] += f0;
+              sum[mi][ni][4 * q + e + 1] += f1;
             }
         }
     }
