@@ -182,3 +182,46 @@ def test_decode_workspace_and_null_checks():
   assert 'workspace' in _err(L.lib().aqtx_decode_i8(ctypes.byref(p), FAKE, FAKE, FAKE, None, FAKE, FAKE, FAKE, 16, None))
   # empty problems succeed without touching the GPU
   assert L.lib().aqtx_decode_i8(ctypes.byref(_dplan(m=0)), None, None, None, None, None, None, None, 0, None) == 0
+
+
+def _ggplan(**kw):
+  p = L.GroupedGemmPlan()
+  p.m, p.n, p.k, p.group = 64, 128, 512, 128
+  p.lda, p.ldb, p.ldc = 512, 512, 128
+  p.a_dtype, p.b_dtype = L.I8, L.I4
+  p.out_dtype = p.row_scale_dtype = p.col_scale_dtype = L.BF16
+  for k, v in kw.items():
+    setattr(p, k, v)
+  return p
+
+
+@pytest.mark.parametrize('kw,needle', [
+    (dict(group=96), 'multiple of 128'),
+    (dict(k=640, lda=640, ldb=640, group=256), 'divides k'),
+    (dict(b_dtype=L.E4M3), 'b must be'),
+    (dict(a_dtype=L.I4P), 'a must be'),
+    (dict(out_dtype=L.I32), 'dtypes'),
+    (dict(lda=256), 'leading dimension'),
+    (dict(lda=520, ldb=520), '16'),
+    (dict(m=-2), 'bad shape'),
+])
+def test_grouped_gemm_plan_validation(kw, needle):
+  p = _ggplan(**kw)
+  msg = _err(L.lib().aqtx_gemm_i8_grouped(ctypes.byref(p), FAKE, FAKE, FAKE, FAKE, FAKE, None))
+  assert needle in msg, msg
+
+
+def test_grouped_gemm_packed_leading_dimension_is_in_bytes():
+  # packed int4: a row of b holds k/2 bytes, so ldb = k/2 is valid and ldb < k/2 is not
+  assert 'leading dimension' in _err(L.lib().aqtx_gemm_i8_grouped(
+      ctypes.byref(_ggplan(b_dtype=L.I4P, ldb=128)), FAKE, FAKE, FAKE, FAKE, FAKE, None))
+  assert 'NULL' in _err(L.lib().aqtx_gemm_i8_grouped(
+      ctypes.byref(_ggplan(b_dtype=L.I4P, ldb=256)), None, FAKE, FAKE, FAKE, FAKE, None))
+
+
+def test_small_entry_validation():
+  assert 'even' in _err(L.lib().aqtx_pack_i4(FAKE, FAKE, 7, None))
+  assert L.lib().aqtx_pack_i4(None, None, 0, None) == 0
+  assert 'dtype' in _err(L.lib().aqtx_sum_tiles(FAKE, FAKE, 4, 16, L.I8, None))
+  assert 'NULL' in _err(L.lib().aqtx_sum_tiles(None, FAKE, 4, 16, L.BF16, None))
+  assert L.lib().aqtx_sum_tiles(None, None, 4, 0, L.BF16, None) == 0
