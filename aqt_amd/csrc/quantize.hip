@@ -169,9 +169,21 @@ __device__ __forceinline__ float spec_scale(float v, float inv, const QArgs& a) 
   return round_bf16(v * inv);
 }
 __device__ __forceinline__ float uniform_noise(uint32_t bits) {
-  // jax.random.uniform: mantissa bits -> [1, 2) - 1, then the centring of JaxUniform
-  float u = __uint_as_float((bits >> 9) | 0x3F800000u) - 1.0f;
-  return fmaxf(0.0f, u) - 0.5f;
+  // jax.random.uniform: f = bitcast(bits >> 9 | 0x3F800000) in [1, 2), u = f - 1, max(0, u); then
+  // the centring of JaxUniform, u - 0.5.  f - 1 and u - 0.5 are exact (multiples of 2^-23 below 1)
+  // and u >= 0, so the three steps equal the single exact subtraction f - 1.5.  The shift-and-or
+  // is one funnel shift of {0x7F, bits} by 9.
+  const uint32_t f = __builtin_amdgcn_alignbit(0x7Fu, bits, 9);
+  return __uint_as_float(f) - 1.5f;
+}
+// Rounds two floats to bf16 (ties to even) in place with one packed conversion.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void round_bf16_pair(float& a, float& b) {
+  const bf16x2_t h = __builtin_convertvector(f32x2_t{a, b}, bf16x2_t);
+  const uint32_t w = __builtin_bit_cast(uint32_t, h);
+  a = __uint_as_float(w << 16);
+  b = __uint_as_float(w & 0xFFFF0000u);
 }
 template <int SPEC>
 __device__ __forceinline__ uint32_t spec_finish(float t, const QArgs& a) {
@@ -209,9 +221,11 @@ __device__ __forceinline__ uint32_t spec_quant(float v, float inv, uint64_t ctr,
 __device__ __forceinline__ void pair_quant(float v0, float inv0, float v1, float inv1, uint32_t i,
                                            const QArgs& a, uint32_t& q0, uint32_t& q1) {
   const U2 bits = threefry2x32(a.gen.k0, a.gen.k1, i, i + a.gen.half);
-  float t0 = round_bf16(v0 * inv0), t1 = round_bf16(v1 * inv1);
-  t0 = round_bf16(t0 + uniform_noise(bits.x));
-  t1 = round_bf16(t1 + uniform_noise(bits.y));
+  float t0 = v0 * inv0, t1 = v1 * inv1;
+  round_bf16_pair(t0, t1);
+  t0 += uniform_noise(bits.x);
+  t1 += uniform_noise(bits.y);
+  round_bf16_pair(t0, t1);
   q0 = spec_finish<2>(t0, a);
   q1 = spec_finish<2>(t1, a);
 }
