@@ -8,9 +8,10 @@
 // quantized first by the row kernel of aqtx_quantize (same arithmetic as training), then:
 //   K split : one workgroup per 16 weight rows, its 4 waves split K and meet in LDS; the
 //             quantized activations come from L2 (m <= 16, or a weight with few rows);
-//   whole K : one workgroup per 64 weight rows (16 per wave, whole K); the activations
-//             are staged chunk by chunk in LDS and shared by the waves, the weights are
-//             requested three chunks ahead (16 < m <= 64 and n >= 12288).  K is never split across workgroups: a partial-sum
+//   whole K : one workgroup per 64 weight rows; two groups of 4 waves (16 rows per wave) take half
+//             of K each and meet in LDS; the activations are staged chunk by chunk in LDS and
+//             shared by the waves of a group, the weights are requested three chunks ahead
+//             (16 < m <= 64 and n >= 12288).  K is never split across workgroups: a partial-sum
 //             exchange inside one launch would need device-scope release/acquire, which
 //             flushes and invalidates the per-XCD L2s.
 #include "common.h"
@@ -120,21 +121,28 @@ __global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) 
 constexpr int kChunk = 256;  // bytes of K per pipeline step
 constexpr int kAhead = 3;    // weight chunks requested ahead of the one being multiplied
 
-// MB: 16-row blocks of activations, 2 (m <= 32) or 4 (m <= 64).  NWV: waves per workgroup, each
-// owning 16 weight rows over the whole of K (no K split, so no cross-workgroup reduction).
-template <int MB, int NWV>
-__global__ __launch_bounds__(NWV * 64) void decode_block_kernel(const DecodeArgs d) {
-  // Activations of one K chunk, [MB*16 rows][256 B]; the 16-byte piece j of row i sits at
-  // piece j ^ (i & 15), so the 16 lanes of a fragment read (16 rows, one piece) hit 64 banks.
-  __shared__ __attribute__((aligned(16))) uint8_t xbuf[2][MB * 16 * kChunk];
-  constexpr int NT = NWV * 64;
+// MB: 16-row blocks of activations, 2 (m <= 32) or 4 (m <= 64).  NWV waves own 16 weight rows
+// each; KW groups of NWV waves take one K range each (their partial sums meet in LDS at the end),
+// which doubles the waves per SIMD for the same weight rows.  K is not split across workgroups.
+template <int MB, int NWV, int KW>
+__global__ __launch_bounds__(NWV * KW * 64) void decode_block_kernel(const DecodeArgs d) {
+  // Activations of one K chunk per K range, [MB*16 rows][256 B]; the 16-byte piece j of row i sits
+  // at piece j ^ (i & 15), so the 16 lanes of a fragment read (16 rows, one piece) hit 64 banks.
+  __shared__ __attribute__((aligned(16))) uint8_t xbuf[KW][2][MB * 16 * kChunk];
+  __shared__ int red[KW > 1 ? (KW - 1) * NWV * MB * 256 : 1];
+  constexpr int NT = NWV * 64;           // threads of one K range
   constexpr int XP = MB * 16 * 16 / NT;  // 16-byte pieces of a chunk staged per thread
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kw = wave / NWV, wn = wave % NWV;
+  const int tid = threadIdx.x - kw * NT;  // thread index inside the K range
   const int r = lane & 15, c = lane >> 4;
-  const int n0 = blockIdx.x * (NWV * 16) + wave * 16;
+  const int n0 = blockIdx.x * (NWV * 16) + wn * 16;
   const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);  // clamped; such columns are never stored
-  const int nchunks = (d.k + kChunk - 1) / kChunk;
+  const int k_len = ((d.k + KW - 1) / KW + kChunk - 1) / kChunk * kChunk;  // K range, whole chunks
+  const int k_lo = kw * k_len;
+  const int k_hi = (k_lo + k_len) < d.k ? (k_lo + k_len) : d.k;
+  const int nchunks = k_len / kChunk;  // the same for every K range: they share the barriers
 
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
@@ -143,19 +151,30 @@ __global__ __launch_bounds__(NWV * 64) void decode_block_kernel(const DecodeArgs
   const int xs_row = tid >> 4, xs_piece = tid & 15;
 
   v4i wreg[kAhead + 1][4], xr[2][XP];  // xr[p]: activations of a chunk of parity p on their way to LDS
-  auto load_w = [&](v4i* dst, int kc) {  // past K every load reads zeros
+  // Workgroups walk the chunks of their K range in rotated order (integer sums do not care):
+  // otherwise every workgroup of the launch asks the same few L2 channels for the same
+  // activation chunk at the same time.  Step numbers past the range read zeros.
+  const int rot = blockIdx.x % nchunks;
+  auto chunk_start = [&](int step_no) {
+    int j = step_no + rot;
+    j = j >= nchunks ? j - nchunks : j;
+    return step_no < nchunks ? k_lo + j * kChunk : 0x3FFFFF00;
+  };
+  auto load_w = [&](v4i* dst, int step_no) {
+    const int kc = chunk_start(step_no);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int ko = kc + ks * 64;
-      dst[ks] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < d.k) ? wbase + ko : kOob, 0, 0);
+      dst[ks] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < k_hi) ? wbase + ko : kOob, 0, 0);
     }
   };
-  auto load_x = [&](v4i* dst, int kc) {
+  auto load_x = [&](v4i* dst, int step_no) {
+    const int kc = chunk_start(step_no);
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
       const int row = p * (NT / 16) + xs_row;
       const int ko = kc + xs_piece * 16;
-      dst[p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (row < d.m && ko < d.k) ? row * d.k + ko : kOob, 0, 0);
+      dst[p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (row < d.m && ko < k_hi) ? row * d.k + ko : kOob, 0, 0);
     }
   };
   auto store_x = [&](uint8_t* buf, const v4i* src) {
@@ -172,20 +191,20 @@ __global__ __launch_bounds__(NWV * 64) void decode_block_kernel(const DecodeArgs
 
   load_x(xr[0], 0);
 #pragma unroll
-  for (int j = 0; j < kAhead; ++j) load_w(wreg[j], j * kChunk);
-  store_x(xbuf[0], xr[0]);
-  load_x(xr[1], kChunk);
-  load_x(xr[0], 2 * kChunk);
+  for (int j = 0; j < kAhead; ++j) load_w(wreg[j], j);
+  store_x(xbuf[kw][0], xr[0]);
+  load_x(xr[1], 1);
+  load_x(xr[0], 2);
   __syncthreads();
   // One pipeline step: publish the activations of chunk i+1 (requested two steps ago), request
   // those of chunk i+3 and the weights of chunk i+kAhead, multiply chunk i.  Every load has two
   // or more steps to arrive, so a step never waits a full memory latency.  The register sets
   // rotate roles through the unrolled steps (no register copies that would wait for loads).
   auto step = [&](const v4i* wc, v4i* wfar, v4i* xnext, int i) {
-    store_x(xbuf[(i + 1) & 1], xnext);
-    load_x(xnext, (i + 3) * kChunk);
-    load_w(wfar, (i + kAhead) * kChunk);
-    const uint8_t* buf = xbuf[i & 1];
+    store_x(xbuf[kw][(i + 1) & 1], xnext);
+    load_x(xnext, i + 3);
+    load_w(wfar, i + kAhead);
+    const uint8_t* buf = xbuf[kw][i & 1];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
@@ -209,7 +228,23 @@ __global__ __launch_bounds__(NWV * 64) void decode_block_kernel(const DecodeArgs
     step(wreg[3], wreg[2], xr[0], i + 3);
   }
 
-  // lane holds C[m = mb*16 + 4c + e][n = n0 + r]
+  // lane holds C[m = mb*16 + 4c + e][n = n0 + r]; K ranges 1.. hand their sums to range 0
+  if constexpr (KW > 1) {
+    if (kw > 0) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) red[(((kw - 1) * NWV + wn) * MB + mb) * 256 + e * 64 + lane] = acc[mb][e];
+    }
+    __syncthreads();
+    if (kw > 0) return;
+#pragma unroll
+    for (int j = 1; j < KW; ++j)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[mb][e] += red[(((j - 1) * NWV + wn) * MB + mb) * 256 + e * 64 + lane];
+  }
   const int nn = n0 + r;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
@@ -293,15 +328,19 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
   }
   // Whole-K waves sharing the activations through LDS need n/16 >= a few waves per CU to keep
   // HBM busy; below that the K-split shape wins although it re-reads the activations.
-  if (p->n < 12288) {
+  // AQTX_DECODE_SHAPE=ksplit|block overrides the choice (tuning).
+  const char* shape_env = getenv("AQTX_DECODE_SHAPE");
+  const bool force_ksplit = shape_env != nullptr && shape_env[0] == 'k';
+  const bool force_block = shape_env != nullptr && shape_env[0] == 'b';
+  if ((p->n < 12288 && !force_block) || force_ksplit) {
     if (p->m <= 32) decode_ksplit_kernel<2, 8><<<grid16, 256, 0, st>>>(d);
     else decode_ksplit_kernel<4, 4><<<grid16, 256, 0, st>>>(d);
     AQTX_HIP_CHECK_LAUNCH("decode_ksplit_kernel");
     return 0;
   }
   const unsigned grid = (unsigned)((p->n + 63) / 64);
-  if (p->m <= 32) decode_block_kernel<2, 4><<<grid, 256, 0, st>>>(d);
-  else decode_block_kernel<4, 4><<<grid, 256, 0, st>>>(d);
+  if (p->m <= 32) decode_block_kernel<2, 4, 2><<<grid, 512, 0, st>>>(d);
+  else decode_block_kernel<4, 4, 2><<<grid, 512, 0, st>>>(d);
   AQTX_HIP_CHECK_LAUNCH("decode_block_kernel");
   return 0;
 }
