@@ -14,6 +14,7 @@ import dataclasses
 import enum
 import functools
 import math
+import weakref
 from typing import Any, Optional, Sequence
 
 import numpy as onp
@@ -361,6 +362,24 @@ def _apply_local_aqt(local_aqt, lhs, rhs, dimension_numbers):
   return lhs, rhs, ((lca, rca), (lba, rba))
 
 
+# A frozen operand that arrives in another memory order than the kernels read (e.g. a weight
+# restored from a checkpoint in its logical [K, N] order) is re-laid out once, not on every call:
+# the copy is remembered for as long as the frozen tensor itself lives.
+_KERNEL_LAYOUT_CACHE = {}   # id(frozen tensor) -> (key, re-laid-out copy); entries die with the tensor
+
+
+def _kernel_layout_of(qvalue: torch.Tensor, v: 'lowering.OperandView') -> torch.Tensor:
+  key = (tuple(v.b_axes), tuple(v.r_axes), tuple(v.k_axes), qvalue._version)
+  hit = _KERNEL_LAYOUT_CACHE.get(id(qvalue))
+  if hit is not None and hit[0] == key:
+    return hit[1]
+  q = v.mem if v.k_last else v.mem.transpose(1, 2).contiguous()
+  if hit is None:
+    weakref.finalize(qvalue, _KERNEL_LAYOUT_CACHE.pop, id(qvalue), None)
+  _KERNEL_LAYOUT_CACHE[id(qvalue)] = (key, q)
+  return q
+
+
 _POISON = ('Poison. Gradients are not generally expected in serving. Please set '
            'allow_dummy_gradient_into_qtensor to True if this is the intended behavior.')
 
@@ -593,8 +612,9 @@ class DotGeneralRaw:
     rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
     lv = lowering.view_operand(lhs, [], lra, lca)
     rv = lowering.view_operand(rhs_qt.qvalue, [], rra, rca)
-    if not (lv.k_last and rv.k_last) or lv.copied or rv.copied:
+    if not lv.k_last or lv.copied:
       return None
+    rq = rv.mem if rv.k_last and not rv.copied else _kernel_layout_of(rhs_qt.qvalue, rv)
     M, K, N = lv.R, lv.K, rv.R
     if M == 0 or M > 64 or K == 0 or K % 16 != 0 or N == 0 or N * K >= 2 ** 31:
       return None
@@ -603,7 +623,7 @@ class DotGeneralRaw:
     if sv.mem.numel() != N:
       return None
     sdt = dq.lhs._calibrator.dtype if dq.lhs._calibrator.dtype is not None else lhs_dtype
-    out, xs, xq = ops.decode(lv.mem[0], rv.mem[0], sv.mem.reshape(-1).float().contiguous(),
+    out, xs, xq = ops.decode(lv.mem[0], rq[0], sv.mem.reshape(-1).float().contiguous(),
                              quant_bound=spec['quant_bound'], clip_bound=spec['clip_bound'],
                              x_scale_dtype=sdt, w_scale_dtype=w_scale.dtype, want_xq=True)
     out = out.reshape([lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
@@ -625,7 +645,7 @@ class DotGeneralRaw:
           f'biases are only supported in fake quant mode, but got a {name} bias')
       assert len(given_qt.scale) == 1, 'a provided QTensor must carry exactly one scale'
       v = lowering.view_operand(given_qt.qvalue, ba, ra, ca)
-      q = v.mem if v.k_last else v.mem.transpose(1, 2).contiguous()
+      q = v.mem if v.k_last and not v.copied else _kernel_layout_of(given_qt.qvalue, v)
       if q.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
         q = q.view(torch.uint8)
       s = given_qt.scale[0]

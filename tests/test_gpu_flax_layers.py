@@ -117,3 +117,27 @@ def test_tiling_injection(gpu):
   assert tuple(out.shape) == (6, 10) and torch.equal(out, want)
   untiled = aqt_flax.AqtEinsum(cfg, rngs=_rngs())('abd,cbd->ac', lhs, rhs)
   assert not torch.equal(out, untiled) and torch.allclose(out.float(), untiled.float(), rtol=0.1, atol=0.05)
+
+
+def test_serving_from_logical_order_checkpoint(gpu):
+  """A frozen weight restored in its logical [K, N] order (as a checkpoint would hold it) serves the
+  same values as the one the convert step produced, through the decode path and the GEMM path, and
+  is re-laid out for the kernels once, not per call."""
+  from aqt_amd.v2 import aqt_dot_general as adg
+  dt = 'bf16'
+  w = U.to_dev(U.rand((256, 128), dt, 2, 0.02), dt, gpu)
+  cfg = config.fully_quantized(use_stochastic_rounding=False)
+  conv = aqt_flax.AqtDotGeneral(cfg, rhs_quant_mode=QM.CONVERT, rhs_freeze_mode=FM.CALIBRATION_AND_VALUE, rngs=_rngs())
+  x8 = U.to_dev(U.rand((8, 256), dt, 1), dt, gpu)
+  x100 = U.to_dev(U.rand((100, 256), dt, 3), dt, gpu)
+  want8, want100 = conv(x8, w, MATMUL, None), conv(x100, w, MATMUL, None)
+  v = conv.variables()
+  v['aqt']['qrhs']['value'] = v['aqt']['qrhs']['value'].contiguous().clone()   # logical row-major, like a restore
+  assert v['aqt']['qrhs']['value'].stride() == (128, 1)
+  serve = aqt_flax.AqtDotGeneral(cfg, rhs_quant_mode=QM.SERVE, rhs_freeze_mode=FM.CALIBRATION_AND_VALUE, rngs=_rngs())
+  serve.load_variables(v)
+  adg._KERNEL_LAYOUT_CACHE.clear()
+  for _ in range(2):
+    assert torch.equal(serve(x8, torch.zeros_like(w), MATMUL, None), want8)
+    assert torch.equal(serve(x100, torch.zeros_like(w), MATMUL, None), want100)
+  assert len(adg._KERNEL_LAYOUT_CACHE) == 1
