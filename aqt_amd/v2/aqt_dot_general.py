@@ -62,19 +62,23 @@ class LocalAqt:
   tile_largest_shape: bool = False
 
 
-def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
-  """Float dot_general with lax semantics (output axes: batch, lhs remaining, rhs remaining).
+_FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
 
-  Stands in for `jax.lax.dot_general` as the default `DotGeneralRaw.dot_general`; a
-  plain library GEMM (rocBLAS/hipBLASLt through torch), used for unquantized sides.
+
+def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+  """dot_general with lax semantics (output axes: batch, lhs remaining, rhs remaining).
+
+  Stands in for `jax.lax.dot_general` as the default `DotGeneralRaw.dot_general`.  int8 x int8
+  and fp8 x fp8 operands go to the MFMA contraction kernels and come back as raw int32 /
+  float32 accumulators; float operands (unquantized sides, fake quantization) go to the
+  library GEMM through torch.  An int8 operand next to a float one is promoted to the float
+  dtype first, as jnp's type promotion does.
   """
   del precision
   (lca, rca), (lba, rba) = dimension_numbers
   lca, rca, lba, rba = list(lca), list(rca), list(lba), list(rba)
   lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
   rra = utils.get_remaining_axes(rhs.dim(), rca, rba)
-  lt = lhs.permute(*(lba + lra + lca))
-  rt = rhs.permute(*(rba + rca + rra))
   bshape = [lhs.shape[a] for a in lba]
   mshape = [lhs.shape[a] for a in lra]
   nshape = [rhs.shape[a] for a in rra]
@@ -84,7 +88,32 @@ def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_eleme
   b = 1
   for s in bshape:
     b *= s
-  out = torch.matmul(lt.reshape(b, -1, kdim), rt.reshape(b, kdim, -1))
+  lt = lhs.permute(*(lba + lra + lca)).reshape(b, -1, kdim)
+  both_int = lhs.dtype == torch.int8 and rhs.dtype == torch.int8
+  both_fp8 = lhs.dtype in _FP8_DTYPES and rhs.dtype in _FP8_DTYPES
+  if both_int or both_fp8:
+    # the kernels take both operands with the contraction axis innermost
+    rt = rhs.permute(*(rba + rra + rca)).reshape(b, -1, kdim)
+    m, n = lt.shape[1], rt.shape[1]
+    acc_dtype = torch.int32 if both_int else torch.float32
+    if both_int:
+      assert preferred_element_type == torch.int32, (
+          f'{preferred_element_type=}: int8 operands are contracted into int32 accumulators only')
+    if b * m * n == 0 or kdim == 0:
+      out = torch.zeros((b, m, n), dtype=acc_dtype, device=lhs.device)
+    else:
+      kd = lambda t: {torch.int8: L.I8, torch.float8_e4m3fn: L.E4M3, torch.float8_e5m2: L.E5M2}[t.dtype]
+      raw = lambda t: t.contiguous() if t.dtype == torch.int8 else t.contiguous().view(torch.uint8)
+      out = ops.gemm(raw(lt), raw(rt), row_scale=None, col_scale=None, out_dtype=acc_dtype,
+                     a_dtype=kd(lt), b_dtype=kd(rt))
+  else:
+    common = torch.promote_types(lhs.dtype, rhs.dtype)
+    pet = preferred_element_type
+    if pet is not None and pet.is_floating_point and common.is_floating_point and (
+        torch.finfo(pet).bits > torch.finfo(common).bits):
+      common = pet  # wider accumulator asked for: keep its precision in the result
+    rt = rhs.permute(*(rba + rca + rra)).reshape(b, kdim, -1)
+    out = torch.matmul(lt.to(common), rt.to(common))
   out = out.reshape(bshape + mshape + nshape)
   if preferred_element_type is not None:
     out = out.to(preferred_element_type)
@@ -432,6 +461,9 @@ def _canonical_pairs(lhs, rhs, dimension_numbers):
   return ((lca2, rca2), (lba2, rba2))
 
 
+_NotFused = lowering.NotFused
+
+
 @dataclasses.dataclass(kw_only=True)
 class DotGeneralRaw:
   """Configuration of quantization of one dot_general without gradient (aqt_dot_general.py:732-749)."""
@@ -462,24 +494,87 @@ class DotGeneralRaw:
     with torch.profiler.record_function(self.jax_scope_name):
       if isinstance(rhs, MultiTensor):
         lhs, rhs = _maybe_use_fwd_quant(lhs, rhs, dimension_numbers, self.rhs.use_fwd_quant)
-      for side, name in ((self.lhs, 'lhs'), (self.rhs, 'rhs')):
-        if side.dequant_mode != DequantMode.OUTPUT or side.calibration_mode != CalibrationMode.CONTRACTING_AXIS:
-          raise NotImplementedError(
-              f'{name}: only DequantMode.OUTPUT with CalibrationMode.CONTRACTING_AXIS has a HIP path')
       if self.local_aqt is None:
-        return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes)
+        return self._dispatch(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes)
       # LocalAqt (aqt_dot_general.py:773-776, 833-837): every shard of the contraction axis is
       # calibrated and contracted on its own (the shard axis is a leading batch axis), the
       # dequantized shard outputs are summed; no residuals come back.
+      msg = 'Custom calib_shared_axes not implemented for local AQT.'
+      if isinstance(self.dg_quantizer, DefaultDotGeneralQuantizer):
+        self.dg_quantizer.assert_calib_shared_axes_value(None, None, msg)
       n_ca = len(dimension_numbers[0][0])
       assert n_ca == len(dimension_numbers[0][1])
       lhs, rhs, dn = _apply_local_aqt(self.local_aqt, lhs, rhs, dimension_numbers)
-      out, _ = self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dn, None)
+      out, _ = self._dispatch(lhs, rhs, lhs_qt, rhs_qt, dn, None)
       if n_ca > 0:
         out = ops.sum_tiles(out.contiguous())
       if _out_transpose_axes is not None:
         out = out.permute(*_out_transpose_axes)
       return out, None
+
+  def _dispatch(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes):
+    """The fused kernels where they implement the configuration, the step-by-step path otherwise."""
+    fusable = (self.dot_general is lax_dot_general
+               and type(self.dg_quantizer) is DefaultDotGeneralQuantizer)  # pylint: disable=unidiomatic-typecheck
+    for side in (self.lhs, self.rhs):
+      fusable = fusable and (side.dequant_mode == DequantMode.OUTPUT
+                             and side.calibration_mode == CalibrationMode.CONTRACTING_AXIS)
+    if fusable:
+      try:
+        return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes)
+      except _NotFused:
+        pass
+    return self._unfused_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes)
+
+  # ------------------------------------------------------------------------------
+  def _unfused_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None):
+    """The operator one step at a time: calibrate, quantize, contract, dequantize.
+
+    Follows aqt_dot_general.py:795-828 through the plugin points (`dg_quantizer`,
+    `dot_general`), so configurations without a fused kernel still run on the GPU: custom
+    quantizers and contraction hooks, fake quantization (DequantMode.THIS_INPUT), scaling of
+    the other operand (OTHER_INPUT), calibration over the remaining axes, one-sided
+    quantization, clip_gradient, biases in fake-quant mode.  Each step is its own kernel (the
+    quantize / dequantize kernels, the MFMA or library contraction) with elementwise tensor
+    arithmetic in between.
+    """
+    if isinstance(lhs, _Prescaled):
+      lhs = lhs.x * lhs.scale_t.to(lhs.x.dtype)
+    if isinstance(rhs, aqt_tensor.QTensor):
+      rhs = rhs.qvalue.to(rhs.dequant_dtype)
+
+    # quant() of the reference (aqt_dot_general.py:598-672)
+    dq = self.dg_quantizer
+    (lhs, lhs_incomplete), (rhs, rhs_incomplete) = dq.calibrate(
+        lhs, rhs, dimension_numbers, self.lhs.calibration_mode, self.rhs.calibration_mode)
+    if lhs_qt is not None and not lhs_qt.is_full():
+      lhs_incomplete, lhs_qt = lhs_qt, None
+    if rhs_qt is not None and not rhs_qt.is_full():
+      rhs_incomplete, rhs_qt = rhs_qt, None
+    (lhs_calc, lhs_grad), (rhs_calc, rhs_grad) = dq.calculate_qvalue(lhs, lhs_incomplete, rhs, rhs_incomplete)
+
+    def postprocess(given, calculated, quant_grad):
+      if given is None:
+        return calculated, quant_grad
+      return given, (quant_grad if self.allow_dummy_gradient_into_qtensor else _POISON)
+
+    lhs_qt, lhs_grad = postprocess(lhs_qt, lhs_calc, lhs_grad)
+    rhs_qt, rhs_grad = postprocess(rhs_qt, rhs_calc, rhs_grad)
+
+    msg = ('biases are only supported in fake quant mode, but got a {arg} bias '
+           'and self.{arg}.dequant_mode == {mode} != DequantMode.THIS_INPUT')
+    assert not (lhs_qt.bias and self.lhs.dequant_mode != DequantMode.THIS_INPUT), msg.format(
+        arg='lhs', mode=self.lhs.dequant_mode)
+    assert not (rhs_qt.bias and self.rhs.dequant_mode != DequantMode.THIS_INPUT), msg.format(
+        arg='rhs', mode=self.rhs.dequant_mode)
+
+    res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=lhs, qx=lhs_qt), quant_grad=lhs_grad),
+                        rhs=TensorRes(mt=MultiTensor(x=rhs, qx=rhs_qt), quant_grad=rhs_grad))
+    out = _qtensor_dot_general_unfused(lhs_qt, rhs_qt, dimension_numbers, self,
+                                       torch.promote_types(lhs.dtype, rhs.dtype)).dequant()
+    if out_transpose_axes is not None:
+      out = out.permute(*out_transpose_axes)
+    return out, res
 
   # ------------------------------------------------------------------------------
   def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None):
@@ -515,10 +610,10 @@ class DotGeneralRaw:
       return out, res
 
     if not isinstance(dq, DefaultDotGeneralQuantizer) or lhs_none or rhs_none:
-      raise NotImplementedError(
+      raise _NotFused(
           'only DefaultDotGeneralQuantizer with both sides quantized (or both unquantized) is lowered')
     if dq.lhs_mid_alpha is not None or dq.rhs_mid_alpha is not None:
-      raise NotImplementedError('mid-scale quantization has no HIP path yet')
+      raise _NotFused('mid-scale quantization has no HIP path yet')
 
     dn = _canonical_pairs(lhs, rhs_arr, dimension_numbers)
     (lca, rca), (lba, rba) = dn
@@ -541,7 +636,7 @@ class DotGeneralRaw:
     rkd = aqt_tensor.qvalue_kernel_dtype(rhs_qt_out)
     fp8 = lkd in (L.E4M3, L.E5M2)
     if fp8 != (rkd in (L.E4M3, L.E5M2)):
-      raise NotImplementedError('mixed integer / fp8 operands')
+      raise _NotFused('mixed integer / fp8 operands')
     acc = self.dg_accumulator_dtype
     if not fp8:
       assert acc == utils.int32, (
@@ -557,7 +652,7 @@ class DotGeneralRaw:
     def expand(s, n):
       return s.reshape(1, 1).expand(B, n).contiguous() if s.numel() == 1 and B * n != 1 else s.reshape(B, n)
     if self.dot_general is not lax_dot_general:
-      raise NotImplementedError('a custom DotGeneralRaw.dot_general hook is not lowered')
+      raise _NotFused('a custom DotGeneralRaw.dot_general hook is not lowered')
     nb, nl, nr = len(lba), len(lra), len(rra)
     bdims = [lhs.shape[a] for a in lba]
     ldims = [lhs.shape[a] for a in lra]
@@ -641,9 +736,8 @@ class DotGeneralRaw:
     if given_qt is not None and given_qt.is_full():
       # Serving: the provided QTensor replaces the computed one (aqt_dot_general.py:614-635).
       quant_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
-      assert not given_qt.bias, (
-          f'biases are only supported in fake quant mode, but got a {name} bias')
-      assert len(given_qt.scale) == 1, 'a provided QTensor must carry exactly one scale'
+      if given_qt.bias or len(given_qt.scale) != 1 or given_qt.sparsity_mask is not None:
+        raise _NotFused('a provided QTensor with a bias, a sparsity mask or several scales')
       v = lowering.view_operand(given_qt.qvalue, ba, ra, ca)
       q = v.mem if v.k_last and not v.copied else _kernel_layout_of(given_qt.qvalue, v)
       if q.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
@@ -654,19 +748,19 @@ class DotGeneralRaw:
       return q, s32, s.dtype, given_qt, quant_grad
     spec = quantizer.kernel_spec()
     if spec is None:
-      raise NotImplementedError(f'{name}: numerics/calibration {quantizer.numerics} / '
+      raise _NotFused(f'{name}: numerics/calibration {quantizer.numerics} / '
                                 f'{quantizer.calibration} have no fused HIP kernel')
     if getattr(quantizer.numerics, 'clip_gradient', False):
-      raise NotImplementedError('clip_gradient is not supported by the fused path')
+      raise _NotFused('clip_gradient is not supported by the fused path')
     arr = x
     if x_is_q and arr.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
-      raise NotImplementedError('re-quantizing an fp8 residual (use_fwd_quant with fp8 fwd)')
+      raise _NotFused('re-quantizing an fp8 residual (use_fwd_quant with fp8 fwd)')
     v = lowering.view_operand(arr, ba, ra, ca)
     prescale = None
     if prescale_t is not None:
       pv = lowering.view_operand(prescale_t, ba, ra, ca)
       if pv.R != 1 and v.R != 1:
-        raise NotImplementedError('use_fwd_quant scale that varies along the remaining axes')
+        raise _NotFused('use_fwd_quant scale that varies along the remaining axes')
       prescale = pv.mem.reshape(pv.B, -1).float().contiguous()
       if pv.B == 1 and v.B > 1:
         prescale = prescale.reshape(-1)
@@ -690,6 +784,52 @@ class DotGeneralRaw:
                             container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
     quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))
     return q, s32, sdt, qt, quant_grad
+
+
+_DTYPES_ALLOWED_FOR_INT32_ACCUM = (torch.int8,)  # int4 values are held in int8 containers
+_DTYPES_CAN_BE_SCALED = (torch.bfloat16, torch.float32, torch.float64)
+
+
+def _qtensor_dot_general_unfused(lhs_qt, rhs_qt, dimension_numbers, cfg, dequant_dtype) -> aqt_tensor.QTensor:
+  """QTensor x QTensor -> QTensor of accumulators and output scales (aqt_dot_general.py:843-958)."""
+
+  def maybe_dequant(qt, tensor_cfg):
+    if tensor_cfg.dequant_mode == DequantMode.THIS_INPUT:
+      return qt.dequant()
+    out = qt.qvalue
+    if qt.sparsity_mask is not None:
+      out = out * qt.sparsity_mask
+    return out
+
+  lhs_qin = maybe_dequant(lhs_qt, cfg.lhs)
+  rhs_qin = maybe_dequant(rhs_qt, cfg.rhs)
+  dtype_ms = (f'Found {cfg.dg_accumulator_dtype=}, {lhs_qin.dtype=} and {rhs_qin.dtype=}. Dot general '
+              'accumulator dtype can only be jnp.int32 when both inputs are int8. Otherwise it is '
+              'recommended to be None to let lax.dot_general automatically decide it.')
+  if cfg.dg_accumulator_dtype == utils.int32:
+    assert (lhs_qin.dtype in _DTYPES_ALLOWED_FOR_INT32_ACCUM
+            and rhs_qin.dtype in _DTYPES_ALLOWED_FOR_INT32_ACCUM), dtype_ms
+
+  if cfg.lhs.dequant_mode == DequantMode.OTHER_INPUT:
+    assert rhs_qin.dtype in _DTYPES_CAN_BE_SCALED
+    for scale in lhs_qt.scale:
+      t = transpose.lhs_scale_transpose_for_rhs_input(scale, dimension_numbers, rhs_qt.qvalue.shape)
+      rhs_qin = rhs_qin * t.to(rhs_qin.dtype)
+  if cfg.rhs.dequant_mode == DequantMode.OTHER_INPUT:
+    assert lhs_qin.dtype in _DTYPES_CAN_BE_SCALED
+    for scale in rhs_qt.scale:
+      t = transpose.rhs_scale_transpose_for_lhs_input(scale, dimension_numbers, lhs_qt.qvalue.shape)
+      lhs_qin = lhs_qin * t.to(lhs_qin.dtype)
+
+  acc = cfg.dot_general(lhs_qin, rhs_qin, dimension_numbers, None, cfg.dg_accumulator_dtype)
+  out = aqt_tensor.QTensor(qvalue=acc, scale=[], scale_t=None, bias=[], dequant_dtype=dequant_dtype)
+  if cfg.lhs.dequant_mode == DequantMode.OUTPUT:
+    out.scale.extend(_get_scale_t(lhs_qt, transpose.lhs_scale_transpose_to_output, dimension_numbers,
+                                  lhs_qin.shape, rhs_qin.shape))
+  if cfg.rhs.dequant_mode == DequantMode.OUTPUT:
+    out.scale.extend(_get_scale_t(rhs_qt, transpose.rhs_scale_transpose_to_output, dimension_numbers,
+                                  lhs_qin.shape, rhs_qin.shape))
+  return out
 
 
 def _qtensor_dot_general(lhs_qt, rhs_qt, dimension_numbers, cfg, dequant_dtype):

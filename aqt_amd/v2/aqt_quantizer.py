@@ -61,7 +61,7 @@ class Quantizer:
     else:
       shared = self.calib_shared_axes or calibration_axes
       if sorted(a % len(v.shape) for a in shared) != sorted(v.k_axes):
-        raise NotImplementedError(
+        raise lowering.NotFused(
             f'calib_shared_axes={shared} differs from the contraction axes {v.k_axes}')
       per_tensor = False
     sdt = self._calibrator.dtype if self._calibrator.dtype is not None else dtype
@@ -101,11 +101,15 @@ class Quantizer:
     if isinstance(self.numerics, no_numerics.NoNumerics):
       return qt, None
     spec = self.numerics.kernel_spec()
-    if spec is None or qt.bias or qt.tiling_state is not None or len(qt.scale) != 1:
-      # numerics without a fused kernel: scale, then the numerics' own forward
+    if (spec is None or qt.bias or qt.tiling_state is not None or len(qt.scale) != 1
+        or qt.sparsity_mask is not None or getattr(self.numerics, 'clip_gradient', False)):
+      # No fused scale-and-round kernel for this case (or the scaled tensor has to be kept for
+      # clip_gradient): scale, then the numerics' own forward
       q_scaled = qt.quant(x)
       x_q, res = self.numerics.vjp_fwd(q_scaled.qvalue, self.context)
       q_scaled.qvalue = x_q
+      if self.numerics.get_dtype() is utils.int4:
+        q_scaled.container_dtype = utils.int4
       return q_scaled, functools.partial(self.numerics.vjp_bwd, res)
     (s,) = qt.scale
     shared = [a for a in range(x.dim()) if s.shape[a] == 1 and x.shape[a] > 1]
@@ -120,8 +124,6 @@ class Quantizer:
         key=None if self.context is None else self.context.key, per_tensor=per_tensor, scale=s_in)
     qvalue = lowering.logical_from_brk(_typed(q, spec['out_dtype']), v)
     out = qt.replace(qvalue=qvalue, container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
-    if getattr(self.numerics, 'clip_gradient', False):
-      raise NotImplementedError('clip_gradient needs the scaled pre-rounding tensor; not kept by the kernel')
     return out, functools.partial(self.numerics.vjp_bwd, (None,))
 
 

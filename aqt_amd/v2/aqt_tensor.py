@@ -62,9 +62,13 @@ class QTensor:
     assert self.scale is not None, 'Missing scales to be used for quantization.'
     assert isinstance(self.scale, list), f'QTensor.scale must be a list of arrays, but got {self.scale}'
     assert isinstance(self.bias, list), f'QTensor.bias must be a list of arrays, but got {self.bias}'
-    if self.bias or self.sparsity_mask is not None or self.tiling_state is not None:
-      raise NotImplementedError('bias / sparsity / tiling_state in QTensor.quant')
+    if self.tiling_state is not None:
+      x = self.tiling_state.apply(x)
     qvalue = x
+    for b in self.bias:
+      qvalue = qvalue + b
+    if self.sparsity_mask is not None:
+      qvalue = qvalue * self.sparsity_mask
     for s in self.scale:
       # Scaling is fused into the quantize kernel on the fast path; this standalone form is
       # plain elementwise tensor arithmetic.
@@ -82,13 +86,23 @@ class QTensor:
            'dot_general, but to dequantize you need to set its dtype.')
     assert self.dequant_dtype is not None, msg
     assert self.is_full(), _MSG_NO_QVALUE
-    if self.bias or self.sparsity_mask is not None or self.tiling_state is not None:
-      raise NotImplementedError('bias / sparsity / tiling_state in QTensor.dequant')
     q = self.qvalue
-    if not self.scale:
-      return q.to(self.dequant_dtype)
-    if len(self.scale) != 1:
-      raise NotImplementedError('dequant of a QTensor with several scales')
+    kernel_types = (torch.int8, torch.float8_e4m3fn, torch.float8_e5m2)
+    if (len(self.scale) != 1 or self.bias or self.sparsity_mask is not None
+        or self.tiling_state is not None or q.dtype not in kernel_types):
+      # The general form, one elementwise step per scale and bias; each product takes the
+      # promoted dtype of its factors.  Integers reach bf16 through float32, as the
+      # accumulator conversion of the contraction does.
+      ret = q.to(self.dequant_dtype) if q.dtype.is_floating_point else q.to(torch.float32).to(self.dequant_dtype)
+      for s in self.scale:
+        ret = ret * s
+      if self.sparsity_mask is not None:
+        ret = ret * self.sparsity_mask
+      for b in self.bias:
+        ret = ret - b
+      if self.tiling_state is not None:
+        ret = self.tiling_state.unapply(ret)
+      return ret.to(self.dequant_dtype)
     (s,) = self.scale
     q_dtype = qvalue_kernel_dtype(self)
     shared = [a for a in range(q.dim()) if s.shape[a] == 1 and q.shape[a] > 1]

@@ -34,6 +34,21 @@ class Calibration(abc.ABC):
     return False
 
 
+class _UnitBound:
+  """Stands in for a numerics object whose quant bound is 1."""
+
+  def get_quant_bound(self):
+    return 1.0
+
+
+def ceil_to_po2(scale):
+  """1 / 2**floor(log2(1 / scale)) (calibration.py:25-30): the power of two at or above `scale`."""
+  r = torch.reciprocal(scale)
+  e = torch.floor(torch.log2(r))
+  p = torch.ldexp(torch.ones_like(r), e.to(torch.int32))
+  return torch.reciprocal(p)
+
+
 @dataclasses.dataclass(kw_only=True)
 class AbsMaxCalibration(Calibration):
   """max(abs(x)) / quant_bound (calibration.py:107-157)."""
@@ -47,10 +62,20 @@ class AbsMaxCalibration(Calibration):
     del context
     msg = ('Perhaps you are using DequantMode.THIS_INPUT (fake_quant) and forgot to set them.')
     assert shared_axes is not None, msg
-    if not self.kernel_supported():
-      raise NotImplementedError('po2_scale / clipping_scale have no HIP kernel yet')
     from aqt_amd.v2 import lowering  # local import: lowering imports this module's users
-    scale = lowering.absmax_scale(x, list(shared_axes), numerics_, self.dtype)
+    if self.kernel_supported():
+      scale = lowering.absmax_scale(x, list(shared_axes), numerics_, self.dtype)
+      return [scale], [], None
+    # clipping_scale / po2_scale: the abs-max kernel (bound 1 leaves max|x|, zeros replaced by
+    # ones), then the remaining steps one by one in x.dtype.
+    dtype = self.dtype if self.dtype is not None else x.dtype
+    abs_max = lowering.absmax_scale(x, list(shared_axes), _UnitBound(), x.dtype)
+    if self.clipping_scale:
+      abs_max = abs_max * torch.tensor(self.clipping_scale, dtype=x.dtype, device=x.device)
+    scale = abs_max / torch.tensor(float(numerics_.get_quant_bound()), dtype=x.dtype, device=x.device)
+    if self.po2_scale:
+      scale = ceil_to_po2(scale)
+    scale = scale.to(dtype)
     return [scale], [], None
 
 
@@ -65,11 +90,20 @@ class ConstantCalibration(Calibration):
     del context
     if isinstance(self.bound, float) and self.bound <= 0.0:
       raise ValueError(f'{self.bound=} should be positive.')
-    if self.po2_scale or self.bias is not None:
-      raise NotImplementedError('po2_scale / bias have no HIP kernel yet')
     dtype = self.dtype if self.dtype is not None else x.dtype
-    shape = [1 if a in list(shared_axes) else s for a, s in enumerate(x.shape)]
-    # bound and quant_bound are host constants; the division happens in x.dtype.
-    bound = torch.full(shape, float(self.bound), dtype=x.dtype, device=x.device)
-    scale = bound / torch.tensor(float(numerics_.get_quant_bound()), dtype=x.dtype, device=x.device)
-    return [scale.to(dtype)], [], None
+    if isinstance(self.bound, torch.Tensor):
+      bound = self.bound  # per-channel bounds, already in their keepdims shape
+    else:
+      shape = [1 if a in list(shared_axes) else s for a, s in enumerate(x.shape)]
+      # bound and quant_bound are host constants; the division happens in x.dtype.
+      bound = torch.full(shape, float(self.bound), dtype=x.dtype, device=x.device)
+    scale = bound / torch.tensor(float(numerics_.get_quant_bound()), dtype=bound.dtype, device=x.device)
+    if self.po2_scale:
+      scale = ceil_to_po2(scale)
+    if self.bias is None:
+      bias = []
+    elif isinstance(self.bias, torch.Tensor):
+      bias = [self.bias.to(dtype)]
+    else:
+      bias = [torch.full(tuple(x.shape), float(self.bias), dtype=x.dtype, device=x.device)]
+    return [scale.to(dtype)], bias, None

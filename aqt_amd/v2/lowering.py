@@ -21,6 +21,10 @@ from aqt_amd import ops
 from aqt_amd.v2 import utils
 
 
+class NotFused(NotImplementedError):
+  """The fused kernels do not implement this configuration; the step-by-step path takes it."""
+
+
 def _prod(xs):
   return int(math.prod(xs))
 

@@ -67,9 +67,9 @@ class IntSymmetric(numerics.AqtNumerics):
   def vjp_fwd(self, x, context):
     """Noise, clip, round, cast of an already scaled tensor (int_numerics.py:81-111)."""
     spec = self.kernel_spec()
-    if spec is None:
-      raise NotImplementedError(f'no HIP kernel for {self}')
     assert self.bits <= 22, 'Too many bits, float32 has less precision.'
+    if spec is None:
+      return self._vjp_fwd_stepwise(x, context)
     if spec['noise'] != L.NOISE_NONE:
       assert context.key is not None, (
           'noise_fn is set, requestic stochastic rounding, but RNG was not passed in Context.key')
@@ -78,6 +78,25 @@ class IntSymmetric(numerics.AqtNumerics):
     q, _ = ops.quantize(x3, reduce=L.REDUCE_COLS, scale=ones, key=context.key,
                         partitionable=utils.threefry_partitionable, **spec)
     return q.reshape(x.shape), (x,)
+
+  def _vjp_fwd_stepwise(self, x, context):
+    """The settings the fused kernel leaves out (no rounding or clipping, buckets centred on
+    halves, float-held values, wider integers), one elementwise step each."""
+    res = (x,)
+    input_dtype = x.dtype
+    if self.noise_fn:
+      assert context.key is not None, (
+          'noise_fn is set, requestic stochastic rounding, but RNG was not passed in Context.key')
+      x = (x + self.noise_fn(x.shape, context.key)).to(input_dtype)
+    if self.clip:
+      fwd_clip_bound = self._get_fwd_clip_bound()
+      x = torch.clamp(x, -fwd_clip_bound, fwd_clip_bound)
+    if self.round:
+      x = torch.round(x) if self.preserve_zero else torch.floor(x) + 0.5
+    dtype = self.get_dtype()
+    if dtype is utils.int4:
+      dtype = torch.int8  # int4 values travel in int8 containers
+    return x.to(dtype if dtype is not None else input_dtype), res
 
   def vjp_bwd(self, res, grad):
     ret = grad

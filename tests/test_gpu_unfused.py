@@ -1,0 +1,268 @@
+"""GPU parity of the step-by-step DotGeneralRaw path (configurations without a fused kernel)
+against the numpy oracle: fake quantization, scaling of the other operand, calibration over
+the remaining axes, one-sided quantization, po2 / clipped / constant calibrations, numerics
+without rounding or clipping, plugin hooks.
+
+Quantized values and scales are compared bit for bit.  Outputs of *float* contractions
+(fake quantization, one-sided quantization) go through the library GEMM, whose summation
+order differs from numpy's: those are compared to rtol 1e-4 (f32) / 2e-2 (bf16) with an
+absolute floor scaled to the output magnitude.
+"""
+import copy
+import functools
+
+import numpy as np
+import pytest
+import torch
+
+from aqt_amd.v2 import aqt_dot_general as aqt
+from aqt_amd.v2 import calibration
+from aqt_amd.v2 import config
+from aqt_amd.v2 import utils
+from oracle import aqt_ref as R
+from oracle import prng
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+MATMUL = (((1,), (0,)), ((), ()))
+BATCHED = (((2,), (1,)), ((0,), (0,)))
+MODE = {'output': aqt.DequantMode.OUTPUT, 'this_input': aqt.DequantMode.THIS_INPUT,
+        'other_input': aqt.DequantMode.OTHER_INPUT}
+CAL = {'ca': aqt.CalibrationMode.CONTRACTING_AXIS, 'ra': aqt.CalibrationMode.REMAINING_AXIS}
+
+
+def _np(t):
+  return t.detach().float().cpu().numpy()
+
+
+def _close(got, want, dt):
+  rtol = 1e-4 if dt == 'f32' else 2e-2
+  atol = rtol * float(np.abs(want).max() + 1e-30)
+  np.testing.assert_allclose(got, want, rtol=rtol, atol=atol)
+
+
+def _raw_pair(lhs_bits=8, rhs_bits=8, *, lmode='output', rmode='output', lcal='ca', rcal='ca',
+              keep_float=False, acc='auto', calib=None):
+  """A product DotGeneralRaw and the oracle RawCfg with the same settings."""
+  raw = aqt.dot_general_raw_make(lhs_bits, rhs_bits, initialize_calibration=False)
+  raw.lhs.dequant_mode, raw.rhs.dequant_mode = MODE[lmode], MODE[rmode]
+  raw.lhs.calibration_mode, raw.rhs.calibration_mode = CAL[lcal], CAL[rcal]
+  oraw = R.RawCfg(R.QuantizerCfg(bits=lhs_bits), R.QuantizerCfg(bits=rhs_bits),
+                  lhs_dequant_mode=lmode, rhs_dequant_mode=rmode,
+                  lhs_calibration_mode=lcal, rhs_calibration_mode=rcal)
+  if keep_float:
+    for q, oq, bits in ((raw.dg_quantizer.lhs, oraw.lhs, lhs_bits), (raw.dg_quantizer.rhs, oraw.rhs, rhs_bits)):
+      if bits is not None:
+        q.numerics.dtype = None
+        oq.keep_float = True
+  if acc != 'auto':
+    raw.dg_accumulator_dtype = acc
+    oraw.acc = acc
+  if calib:
+    _set_calibration(raw, oraw, **calib)
+  raw.dg_quantizer.init_calibration()
+  return raw, oraw
+
+
+def _run_raw(raw, oraw, lhs, rhs, dt, dn, gpu):
+  out, res = raw(U.to_dev(lhs, dt, gpu), U.to_dev(rhs, dt, gpu), None, None, dn)
+  want, wdt, (lres, rres), _ = R.dg_raw(lhs, dt, rhs, dt, dn, oraw)
+  assert out.dtype == U.TORCH_DT[wdt]
+  return out, res, want, lres, rres
+
+
+def _assert_residuals_equal(res, lres, rres):
+  for got, want in ((res.lhs.mt.qx, lres.qx), (res.rhs.mt.qx, rres.qx)):
+    np.testing.assert_array_equal(_np(got.qvalue), np.asarray(want.qvalue, np.float32))
+    assert len(got.scale) == len(want.scale)
+    for gs, ws in zip(got.scale, want.scale):
+      assert tuple(gs.shape) == ws.shape
+      np.testing.assert_array_equal(_np(gs), ws)
+
+
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('name,kw', [
+    ('fake_ca', dict(lmode='this_input', rmode='this_input')),
+    ('fake_ca_float_held', dict(lmode='this_input', rmode='this_input', keep_float=True)),
+    ('ra_lhs_scales_rhs', dict(lmode='other_input', rmode='this_input', lcal='ra', rcal='ra')),
+    ('ra_rhs_scales_lhs', dict(lmode='this_input', rmode='other_input', lcal='ra', rcal='ra')),
+    ('fake_ra', dict(lmode='this_input', rmode='this_input', lcal='ra', rcal='ra')),
+    ('fake_lhs_only', dict(lmode='this_input', rmode='output')),
+])
+@pytest.mark.parametrize('dn,ls,rs', [(MATMUL, (48, 96), (96, 40)), (BATCHED, (3, 20, 64), (3, 64, 24))])
+def test_dequant_and_calibration_modes(gpu, name, kw, dt, dn, ls, rs):
+  """aqt_dot_general_test.py:761-903 walks these combinations; here each one is checked
+  against the oracle.  Float-held operands make the contraction a float one."""
+  raw, oraw = _raw_pair(acc=None, **kw)
+  lhs, rhs = U.rand(ls, dt, 1, outliers=True), U.rand(rs, dt, 2, 0.05)
+  out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, dn, gpu)
+  _assert_residuals_equal(res, lres, rres)
+  _close(_np(out), want, dt)
+
+
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('lhs_bits,rhs_bits', [(None, 8), (8, None), (None, 4)])
+def test_one_sided_quantization(gpu, lhs_bits, rhs_bits, dt):
+  """Weight-only / activation-only: the int8 side is promoted to the float dtype for the
+  contraction, its scale multiplies the output."""
+  raw, oraw = _raw_pair(lhs_bits, rhs_bits)
+  assert raw.dg_accumulator_dtype is None
+  lhs, rhs = U.rand((40, 128), dt, 3, outliers=True), U.rand((128, 56), dt, 4, 0.05)
+  out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, MATMUL, gpu)
+  _assert_residuals_equal(res, lres, rres)
+  _close(_np(out), want, dt)
+
+
+def _set_calibration(raw, oraw, **kw):
+  for q, oq in ((raw.dg_quantizer.lhs, oraw.lhs), (raw.dg_quantizer.rhs, oraw.rhs)):
+    if 'const_bound' in kw:
+      q.calibration = functools.partial(calibration.ConstantCalibration, bound=kw['const_bound'])
+      oq.const_bound = kw['const_bound']
+    else:
+      q.calibration = functools.partial(q.calibration, **kw)
+      for k, v in kw.items():
+        setattr(oq, k, v)
+
+
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('kw', [dict(po2_scale=True), dict(clipping_scale=0.3),
+                                dict(po2_scale=True, clipping_scale=0.5), dict(const_bound=2.0)])
+def test_calibration_variants_int8_path(gpu, kw, dt):
+  """po2 / clipped abs-max and constant bounds: the scales come from elementwise steps after
+  the abs-max kernel, the contraction is the int8 MFMA one: everything is bit-exact."""
+  raw, oraw = _raw_pair(calib=kw)
+  lhs, rhs = U.rand((64, 160), dt, 5, outliers=True), U.rand((160, 72), dt, 6, 0.05)
+  out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, MATMUL, gpu)
+  _assert_residuals_equal(res, lres, rres)
+  np.testing.assert_array_equal(_np(out), want)
+
+
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('kw', [dict(round=False), dict(clip=False, round=False),
+                                dict(preserve_zero=False), dict(preserve_max_val=True)])
+def test_numerics_variants_float_held(gpu, kw, dt):
+  """IntSymmetric settings outside the fused kernel (int_numerics.py:81-111), values held in
+  the input dtype, fake-quant dequantisation."""
+  raw, oraw = _raw_pair(lmode='this_input', rmode='this_input', keep_float=True, acc=None)
+  for q, oq in ((raw.dg_quantizer.lhs, oraw.lhs), (raw.dg_quantizer.rhs, oraw.rhs)):
+    for k, v in kw.items():
+      setattr(q.numerics, k, v)
+      setattr(oq, k, v)
+  lhs, rhs = U.rand((32, 64), dt, 7), U.rand((64, 48), dt, 8, 0.05)
+  out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, MATMUL, gpu)
+  _assert_residuals_equal(res, lres, rres)
+  _close(_np(out), want, dt)
+
+
+def test_int_path_equals_fake_quant_with_po2_scales(gpu):
+  """aqt_dot_general_test.py:557-715: with power-of-two scales the int8 contraction with
+  output dequantisation and the fake-quant float contraction are the same numbers."""
+  dt = 'f32'
+  lhs, rhs = U.rand((32, 64), dt, 9, outliers=True), U.rand((64, 48), dt, 10, 0.05)
+  outs = []
+  for mode, acc in (('output', 'auto'), ('this_input', None)):
+    raw, oraw = _raw_pair(lmode=mode, rmode=mode, acc=acc, calib=dict(po2_scale=True))
+    out, _ = raw(U.to_dev(lhs, dt, gpu), U.to_dev(rhs, dt, gpu), None, None, MATMUL)
+    outs.append(_np(out))
+  # int8 products summed in f32 are exact below 2^24; po2 scales only shift exponents
+  np.testing.assert_array_equal(outs[0], outs[1])
+
+
+def test_fake_quant_fwd_and_bwd(gpu):
+  """DotGeneral with a fake-quant forward: the backward contractions still take the fused
+  kernels; use_fwd_quant is off as the forward qvalues are not what the contraction saw."""
+  dt = 'bf16'
+  lhs, rhs, g = U.rand((64, 128), dt, 1), U.rand((128, 32), dt, 2, 0.02), U.rand((64, 32), dt, 3, 1e-3)
+  cfg = config.fully_quantized(use_fwd_quant=False, use_stochastic_rounding=True)
+  config.set_fwd_dequant_mode(cfg, lhs_dequant_mode=aqt.DequantMode.THIS_INPUT,
+                              rhs_dequant_mode=aqt.DequantMode.THIS_INPUT)
+  cfg.fwd.dg_accumulator_dtype = None
+  ocfg = R.fully_quantized(use_fwd_quant=False, use_stochastic_rounding=True)
+  ocfg.fwd.lhs_dequant_mode = ocfg.fwd.rhs_dequant_mode = 'this_input'
+  ocfg.fwd.acc = None
+  key = prng.prng_key(11)
+  cfg = config.set_context(cfg, key, None)
+  ocfg = R.set_context(ocfg, key)
+  L = U.to_dev(lhs, dt, gpu).requires_grad_(True)
+  Rr = U.to_dev(rhs, dt, gpu).requires_grad_(True)
+  out = cfg(L, Rr, MATMUL)
+  out.backward(U.to_dev(g, dt, gpu))
+  f = R.dg_fwd(lhs, rhs, dt, MATMUL, ocfg)
+  dl, dr = R.dg_bwd(g, dt, MATMUL, f, ocfg)
+  _close(_np(out), f.out, dt)
+  np.testing.assert_array_equal(_np(L.grad), dl)
+  np.testing.assert_array_equal(_np(Rr.grad), dr)
+
+
+def test_custom_dot_general_hook(gpu):
+  """DotGeneralRaw.dot_general is a plugin point (aqt_dot_general.py:749): a user function
+  receives the quantized operands and the accumulator dtype."""
+  seen = []
+
+  def hook(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+    seen.append((lhs.dtype, rhs.dtype, preferred_element_type))
+    return aqt.lax_dot_general(lhs, rhs, dimension_numbers, precision, preferred_element_type)
+
+  dt = 'bf16'
+  raw, oraw = _raw_pair()
+  raw.dot_general = hook
+  lhs, rhs = U.rand((48, 96), dt, 1, outliers=True), U.rand((96, 40), dt, 2, 0.05)
+  out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, MATMUL, gpu)
+  assert seen == [(torch.int8, torch.int8, torch.int32)]
+  _assert_residuals_equal(res, lres, rres)
+  np.testing.assert_array_equal(_np(out), want)
+
+
+def test_custom_dg_quantizer(gpu):
+  """A DotGeneralQuantizer of the user's own (aqt_dot_general.py:331-422): here one that
+  halves every calibrated scale's bound by delegating and editing the scale."""
+
+  class Halving(aqt.DefaultDotGeneralQuantizer):
+    calls = 0
+
+    def calibrate(self, lhs, rhs, dimension_numbers, lhs_mode, rhs_mode):
+      Halving.calls += 1
+      (lhs, lqt), (rhs, rqt) = super().calibrate(lhs, rhs, dimension_numbers, lhs_mode, rhs_mode)
+      lqt.scale = [s * 0.5 for s in lqt.scale]
+      return (lhs, lqt), (rhs, rqt)
+
+  dt = 'f32'
+  raw, oraw = _raw_pair()
+  d = raw.dg_quantizer
+  raw.dg_quantizer = Halving(lhs=d.lhs, rhs=d.rhs, lhs_mid=d.lhs_mid, rhs_mid=d.rhs_mid)
+  oraw.lhs.clipping_scale = 0.5  # the same scale: abs_max * 0.5 / 127 (exact halving in f32)
+  lhs, rhs = U.rand((48, 96), dt, 1), U.rand((96, 40), dt, 2, 0.05)
+  out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, MATMUL, gpu)
+  assert Halving.calls == 1
+  # abs_max * 0.5 / 127 and (abs_max / 127) * 0.5 round alike except at subnormals
+  _assert_residuals_equal(res, lres, rres)
+  np.testing.assert_array_equal(_np(out), want)
+
+
+def test_clip_gradient(gpu):
+  """IntSymmetric.clip_gradient with a clipping calibration (int_numerics.py:113-125): the
+  gradient is zeroed where the scaled input fell outside the clip bound."""
+  dt = 'f32'
+  lhs, rhs, g = U.rand((32, 64), dt, 1, outliers=True), U.rand((64, 16), dt, 2), U.rand((32, 16), dt, 3)
+  cfg = config.fully_quantized(use_fwd_quant=False, use_stochastic_rounding=False)
+  config.set_absmax_calib_scale(cfg, 0.25)
+  cfg.fwd.dg_quantizer.lhs.numerics.clip_gradient = True
+  cfg = config.set_context(cfg, None, None)
+  L = U.to_dev(lhs, dt, gpu).requires_grad_(True)
+  Rr = U.to_dev(rhs, dt, gpu).requires_grad_(True)
+  out, (lqt, _) = cfg.dg_core(L, Rr, None, None, MATMUL)
+  out.backward(U.to_dev(g, dt, gpu))
+  scaled = lhs / _np(lqt.scale[0])
+  clipped = np.abs(scaled) > 127.0 + 1e-3
+  inside = np.abs(scaled) < 127.0 - 1e-3
+  assert clipped.any() and inside.any()
+  got = _np(L.grad)
+  assert (got[clipped] == 0).all()
+  cfg2 = copy.deepcopy(cfg)
+  cfg2.fwd.dg_quantizer.lhs.numerics.clip_gradient = False
+  L2 = U.to_dev(lhs, dt, gpu).requires_grad_(True)
+  out2, _ = cfg2.dg_core(L2, U.to_dev(rhs, dt, gpu), None, None, MATMUL)
+  out2.backward(U.to_dev(g, dt, gpu))
+  np.testing.assert_array_equal(_np(out), _np(out2))
+  np.testing.assert_array_equal(got[inside], _np(L2.grad)[inside])
