@@ -178,14 +178,16 @@ class DefaultDotGeneralQuantizer(DotGeneralQuantizer):
       self.rhs_mid.init_calibration()
 
   def calibrate(self, lhs, rhs, dimension_numbers, lhs_mode, rhs_mode):
-    """aqt_dot_general.py:464-559 without the mid ("SmoothQuant") scales."""
-    if self.lhs_mid_alpha is not None or self.rhs_mid_alpha is not None:
-      raise NotImplementedError('mid-scale quantization has no HIP path yet')
+    """aqt_dot_general.py:464-559."""
     if dimension_numbers is not None:
       (lhs_ca, rhs_ca), (lhs_ba, rhs_ba) = dimension_numbers
+      lhs_ra = utils.get_remaining_axes(lhs.dim(), lhs_ca, lhs_ba)
+      rhs_ra = utils.get_remaining_axes(rhs.dim(), rhs_ca, rhs_ba)
 
       def axes(mode, ndim, ca, ba):
         if mode == CalibrationMode.REMAINING_AXIS:
+          m = 'mid-quantization is not supported for REMAINING_AXIS mode'
+          assert self.lhs_mid_alpha is None and self.rhs_mid_alpha is None, m
           return utils.get_remaining_axes(ndim, ca, ba)
         if mode == CalibrationMode.CONTRACTING_AXIS:
           return ca
@@ -194,9 +196,44 @@ class DefaultDotGeneralQuantizer(DotGeneralQuantizer):
       lhs_axes = axes(lhs_mode, lhs.dim(), lhs_ca, lhs_ba)
       rhs_axes = axes(rhs_mode, rhs.dim(), rhs_ca, rhs_ba)
     else:
+      lhs_ra = rhs_ra = None
       lhs_axes = rhs_axes = None
-    lhs_qt = self.lhs.calibrate(lhs, calibration_axes=lhs_axes)
-    rhs_qt = self.rhs.calibrate(rhs, calibration_axes=rhs_axes)
+
+    if self.lhs_mid_alpha is None and self.rhs_mid_alpha is None:
+      lhs_qt = self.lhs.calibrate(lhs, calibration_axes=lhs_axes)
+      rhs_qt = self.rhs.calibrate(rhs, calibration_axes=rhs_axes)
+      return ((lhs, lhs_qt), (rhs, rhs_qt))
+
+    # "Middle" scales (SmoothQuant, AWQ): part of each side's per-contraction-channel scale moves
+    # to the other side before the usual calibration.  Elementwise tensor arithmetic around the
+    # abs-max kernel.
+    def dezero(x):
+      return torch.where(x == 0.0, torch.ones_like(x), x)
+
+    def mid(quantizer, x, ra, alpha, transpose_fn, other_shape):
+      if alpha is None:
+        return 1.0, 1.0
+      assert quantizer is not None
+      qt = quantizer.calibrate(x, calibration_axes=ra)
+      assert len(qt.scale) == 1, 'you must set some numerics'
+      scale = dezero(qt.scale[0]) ** alpha
+      return scale, transpose_fn(scale, dimension_numbers, other_shape)
+
+    lhs_mid_scale, lhs_mid_scale_t = mid(self.lhs_mid, lhs, lhs_ra, self.lhs_mid_alpha,
+                                         transpose.lhs_scale_transpose_for_rhs_input, rhs.shape)
+    rhs_mid_scale, rhs_mid_scale_t = mid(self.rhs_mid, rhs, rhs_ra, self.rhs_mid_alpha,
+                                         transpose.rhs_scale_transpose_for_lhs_input, lhs.shape)
+    lhs_mid_scale_combined = lhs_mid_scale / rhs_mid_scale_t
+    rhs_mid_scale_combined = rhs_mid_scale / lhs_mid_scale_t
+    lhs_mid = lhs / lhs_mid_scale_combined
+    rhs_mid = rhs / rhs_mid_scale_combined
+    lhs_qt = self.lhs.calibrate(lhs_mid, calibration_axes=lhs_axes)
+    rhs_qt = self.rhs.calibrate(rhs_mid, calibration_axes=rhs_axes)
+    assert lhs_qt.scale is not None
+    assert rhs_qt.scale is not None
+    if not self.skip_mid_scales:
+      lhs_qt.scale.append(lhs_mid_scale_combined)
+      rhs_qt.scale.append(rhs_mid_scale_combined)
     return ((lhs, lhs_qt), (rhs, rhs_qt))
 
   def calculate_qvalue(self, lhs, lhs_qt, rhs, rhs_qt):
@@ -786,7 +823,6 @@ class DotGeneralRaw:
     return q, s32, sdt, qt, quant_grad
 
 
-_DTYPES_ALLOWED_FOR_INT32_ACCUM = (torch.int8,)  # int4 values are held in int8 containers
 _DTYPES_CAN_BE_SCALED = (torch.bfloat16, torch.float32, torch.float64)
 
 
@@ -807,8 +843,8 @@ def _qtensor_dot_general_unfused(lhs_qt, rhs_qt, dimension_numbers, cfg, dequant
               'accumulator dtype can only be jnp.int32 when both inputs are int8. Otherwise it is '
               'recommended to be None to let lax.dot_general automatically decide it.')
   if cfg.dg_accumulator_dtype == utils.int32:
-    assert (lhs_qin.dtype in _DTYPES_ALLOWED_FOR_INT32_ACCUM
-            and rhs_qin.dtype in _DTYPES_ALLOWED_FOR_INT32_ACCUM), dtype_ms
+    # int4 values travel in int8 containers, so int8 storage covers both allowed types
+    assert lhs_qin.dtype == utils.int8 and rhs_qin.dtype == utils.int8, dtype_ms
 
   if cfg.lhs.dequant_mode == DequantMode.OTHER_INPUT:
     assert rhs_qin.dtype in _DTYPES_CAN_BE_SCALED

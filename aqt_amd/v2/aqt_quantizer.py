@@ -102,7 +102,8 @@ class Quantizer:
       return qt, None
     spec = self.numerics.kernel_spec()
     if (spec is None or qt.bias or qt.tiling_state is not None or len(qt.scale) != 1
-        or qt.sparsity_mask is not None or getattr(self.numerics, 'clip_gradient', False)):
+        or qt.sparsity_mask is not None or getattr(self.numerics, 'clip_gradient', False)
+        or not x.is_floating_point()):
       # No fused scale-and-round kernel for this case (or the scaled tensor has to be kept for
       # clip_gradient): scale, then the numerics' own forward
       q_scaled = qt.quant(x)

@@ -63,13 +63,20 @@ class AbsMaxCalibration(Calibration):
     msg = ('Perhaps you are using DequantMode.THIS_INPUT (fake_quant) and forgot to set them.')
     assert shared_axes is not None, msg
     from aqt_amd.v2 import lowering  # local import: lowering imports this module's users
-    if self.kernel_supported():
-      scale = lowering.absmax_scale(x, list(shared_axes), numerics_, self.dtype)
+    shared_axes = list(shared_axes)
+    if not x.is_floating_point():
+      x = x.to(torch.float32)  # integer input: the bound is a float (type promotion with the divisor)
+    if self.kernel_supported() and shared_axes:
+      scale = lowering.absmax_scale(x, shared_axes, numerics_, self.dtype)
       return [scale], [], None
     # clipping_scale / po2_scale: the abs-max kernel (bound 1 leaves max|x|, zeros replaced by
     # ones), then the remaining steps one by one in x.dtype.
     dtype = self.dtype if self.dtype is not None else x.dtype
-    abs_max = lowering.absmax_scale(x, list(shared_axes), _UnitBound(), x.dtype)
+    if shared_axes:
+      abs_max = lowering.absmax_scale(x, shared_axes, _UnitBound(), x.dtype)
+    else:  # nothing shared: every element is its own bound
+      abs_max = torch.abs(x)
+      abs_max = torch.where(abs_max == 0.0, torch.ones_like(abs_max), abs_max)
     if self.clipping_scale:
       abs_max = abs_max * torch.tensor(self.clipping_scale, dtype=x.dtype, device=x.device)
     scale = abs_max / torch.tensor(float(numerics_.get_quant_bound()), dtype=x.dtype, device=x.device)

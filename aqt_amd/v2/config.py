@@ -160,14 +160,35 @@ def set_use_fwd_quant(cfg: DotGeneral, dlhs_use_fwd_quant, drhs_use_fwd_quant):
     cfg.drhs.rhs.use_fwd_quant = drhs_use_fwd_quant
 
 
+class _MidNumerics(numerics.AqtNumerics):
+  """Numerics of the mid-scale quantizers: a bound of 1, values untouched (config.py:308-323)."""
+
+  def get_quant_bound(self):
+    return 1.0
+
+  def get_dtype(self):
+    assert False, 'Should not request dtype for mid-quantization.'
+
+  def vjp_fwd(self, x, context):
+    return x, ()
+
+  def vjp_bwd(self, res, grad):
+    assert res == ()
+    return grad
+
+
 def set_use_mid_quant(cfg: DotGeneral, fwd_mid_alpha_both, dlhs_mid_alpha_both, drhs_mid_alpha_both):
-  """config.py:287-352 (settings only; the mid-scale arithmetic has no HIP path yet)."""
+  """Enable middle quantization, a variant of SmoothQuant / AWQ (config.py:287-352)."""
+  for raw in (cfg.fwd, cfg.dlhs, cfg.drhs):
+    assert isinstance(raw.dg_quantizer, aqt_dot_general.DefaultDotGeneralQuantizer)
   msg = 'use_fwd_quant is incompatible with use_mid_quant right now.'
   assert not cfg.dlhs.rhs.use_fwd_quant, msg
   assert not cfg.drhs.rhs.use_fwd_quant, msg
   for raw, alpha in ((cfg.fwd, fwd_mid_alpha_both), (cfg.dlhs, dlhs_mid_alpha_both),
                      (cfg.drhs, drhs_mid_alpha_both)):
     if alpha != SKIP:
+      raw.dg_quantizer.lhs_mid.numerics = _MidNumerics()
+      raw.dg_quantizer.rhs_mid.numerics = _MidNumerics()
       raw.dg_quantizer.lhs_mid.calibration = calibration.AbsMaxCalibration
       raw.dg_quantizer.rhs_mid.calibration = calibration.AbsMaxCalibration
       raw.dg_quantizer.lhs_mid_alpha = alpha

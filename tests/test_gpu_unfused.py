@@ -266,3 +266,65 @@ def test_clip_gradient(gpu):
   out2.backward(U.to_dev(g, dt, gpu))
   np.testing.assert_array_equal(_np(out), _np(out2))
   np.testing.assert_array_equal(got[inside], _np(L2.grad)[inside])
+
+
+def test_mid_quantization_known_answer(gpu):
+  """The reference's own vectors (aqt_dot_general_test.py:1169-1208): binary quantization
+  rounds 1, 2, 4 (and 1, 4, 16) to one magnitude; with mid scales of alpha 0.5 and
+  power-of-two scales it becomes lossless."""
+
+  def make_binary_dg(use_mid):
+    mid_alpha = 0.5 if use_mid else config.SKIP
+    dg = config.config_v4(fwd_bits=1, dlhs_bits=1, drhs_bits=1, fwd_mid_alpha_both=mid_alpha,
+                          dlhs_mid_alpha_both=mid_alpha, drhs_mid_alpha_both=mid_alpha)
+    for q in (dg.fwd.dg_quantizer.lhs, dg.fwd.dg_quantizer.rhs):
+      q.numerics.preserve_max_val = True
+      q.calibration = functools.partial(q.calibration, po2_scale=True)
+    return config.set_context(dg, None, None)
+
+  a = torch.tensor([[1.0, 2.0, 4.0], [1.0, 4.0, 16.0]], device=gpu)
+  b = torch.tensor([[4.0, 2.0, 1.0], [16.0, 4.0, 1.0]], device=gpu)
+  dn = (((1,), (1,)), ((0,), (0,)))
+  ret = np.array([4.0, 16.0], np.float32) * 3.0
+  np.testing.assert_array_equal(_np(aqt.lax_dot_general(a, b, dn)), ret)
+  ret_no_mid = np.array([3 * 4.0 ** 2, 3 * 16.0 ** 2], np.float32)
+  np.testing.assert_array_equal(_np(make_binary_dg(False)(a, b, dn)), ret_no_mid)
+  np.testing.assert_array_equal(_np(make_binary_dg(True)(a, b, dn)), ret)
+
+
+def test_quantizer_per_tensor_known_answer(gpu):
+  """aqt_dot_general_test.py:1115-1144: the abs-max over everything is 2**(bits-1) - 0.5,
+  so the single scale is exactly one."""
+  from aqt_amd.v2 import aqt_quantizer
+  bits = 4
+  q = aqt_quantizer.quantizer_make(bits, initialize_calibration=False)
+  q.calib_shared_axes = 'per_tensor'
+  q.context = utils.Context(key=None, train_step=None)
+  q.init_calibration()
+  x = torch.tensor([[1, 2, 3, 4], [5, 6, 7, 2 ** (bits - 1) - 0.5], [3, 5, 1, -1]],
+                   dtype=torch.float32, device=gpu)
+  qx, _ = q.quant(x, calibration_axes=None)
+  assert len(qx.scale) == 1 and tuple(qx.scale[0].shape) == (1, 1)
+  assert float(qx.scale[0]) == 1.0
+
+
+def test_quantizer_per_subchannel_shapes(gpu):
+  """aqt_dot_general_test.py:1146-1167: an integer input, a float32 scale, axis 2 split in
+  tiles of 2; quantize then dequantize through the tiling state."""
+  from aqt_amd.v2 import aqt_quantizer
+  from aqt_amd.v2 import tiled_dot_general
+  q = aqt_quantizer.quantizer_make(4, scale_dtype=torch.float32)
+  q.context = utils.Context(key=None, train_step=None)
+  x = torch.arange(0, 64, device=gpu).reshape(4, 4, 4)
+  ts = tiled_dot_general.generate_tiling_state(x, [tiled_dot_general.AxisTiling(axis=2, tile_size=2)])
+  qx, _ = q.quant(x, calibration_axes=[0, 2], tiling_state=ts)
+  assert tuple(qx.qvalue.shape) == (4, 4, 2, 2)
+  assert tuple(qx.scale[0].shape) == (1, 4, 2, 1)
+  assert qx.scale[0].dtype == torch.float32
+  y = qx.dequant()
+  assert tuple(y.shape) == (4, 4, 4)
+  # int4 with per-(row, tile) scales: within half a step of the input, plus the truncation of
+  # the cast back to the integer input dtype
+  step = _np(qx.scale[0]).max()
+  assert y.dtype == x.dtype
+  assert np.abs(_np(y) - _np(x)).max() <= 0.5 * step + 1.0
