@@ -328,3 +328,46 @@ def test_quantizer_per_subchannel_shapes(gpu):
   step = _np(qx.scale[0]).max()
   assert y.dtype == x.dtype
   assert np.abs(_np(y) - _np(x)).max() <= 0.5 * step + 1.0
+
+
+def _mode_dg(lmode, rmode, lcal='ca', rcal='ca', disable_rounding=False):
+  """The reference test helper `_modify_dg` (aqt_dot_general_test.py:229-309): po2 scales
+  everywhere, the modes on all three contractions, sides in THIS_INPUT mode held in float."""
+  dg = config.fully_quantized(use_fwd_quant=False, use_stochastic_rounding=False)
+  for raw in (dg.fwd, dg.dlhs, dg.drhs):
+    raw.lhs.dequant_mode, raw.rhs.dequant_mode = MODE[lmode], MODE[rmode]
+    raw.lhs.calibration_mode, raw.rhs.calibration_mode = CAL[lcal], CAL[rcal]
+    for q, mode in ((raw.dg_quantizer.lhs, lmode), (raw.dg_quantizer.rhs, rmode)):
+      q.calibration = functools.partial(q.calibration, po2_scale=True)
+      if mode == 'this_input' or disable_rounding:
+        q.numerics.dtype = None
+      if disable_rounding:
+        q.numerics.round = False
+    if 'this_input' in (lmode, rmode) or disable_rounding:
+      raw.dg_accumulator_dtype = None
+  return config.set_context(dg, None, None)
+
+
+@pytest.mark.parametrize('name,kw', [
+    ('CA', dict(lmode='output', rmode='output', disable_rounding=True)),
+    ('CA int8', dict(lmode='output', rmode='output')),
+    ('CA fake', dict(lmode='this_input', rmode='this_input', disable_rounding=True)),
+    ('RA L', dict(lmode='other_input', rmode='this_input', lcal='ra', rcal='ra')),
+    ('RA R', dict(lmode='this_input', rmode='other_input', lcal='ra', rcal='ra')),
+    ('RA fake', dict(lmode='this_input', rmode='this_input', lcal='ra', rcal='ra')),
+])
+def test_equality_between_different_calibration_axes(gpu, name, kw):
+  """aqt_dot_general_test.py:972-1048: on power-of-two data every calibration axis /
+  dequantisation mode gives the float result exactly, forward and both gradients."""
+  rng = np.random.default_rng(0)
+  po2 = lambda shape: np.exp2(np.floor(rng.uniform(-3.0, 3.0, shape) + 3.0)).astype(np.float32)
+  lhs, rhs, g = po2((10, 20)), po2((20, 30)), po2((10, 30))
+  dg = _mode_dg(**kw)
+  dg.assert_config_validity()
+  L = U.to_dev(lhs, 'f32', gpu).requires_grad_(True)
+  Rr = U.to_dev(rhs, 'f32', gpu).requires_grad_(True)
+  out = dg(L, Rr, MATMUL)
+  out.backward(U.to_dev(g, 'f32', gpu))
+  np.testing.assert_array_equal(_np(out), lhs @ rhs)
+  np.testing.assert_array_equal(_np(L.grad), g @ rhs.T)
+  np.testing.assert_array_equal(_np(Rr.grad), lhs.T @ g)

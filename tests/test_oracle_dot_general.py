@@ -176,3 +176,51 @@ def test_sr_noise_depends_on_key_and_is_centered():
   assert (outs[0] != outs[1]).any()
   assert np.abs(outs[0] - rtn).max() <= 1
   assert abs((outs[0] - rtn).mean()) < 0.02
+
+
+def _po2_data(shape, seed):
+  rng = np.random.default_rng(seed)
+  return np.exp2(np.floor(rng.uniform(-3.0, 3.0, shape) + 3.0)).astype(np.float32)
+
+
+def _mode_cfg(lmode, rmode, lcal='ca', rcal='ca', disable_rounding=False):
+  """The reference test helper `_modify_dg` (aqt_dot_general_test.py:229-309) on the oracle's
+  config: po2 scales everywhere, the modes on all three contractions, sides in THIS_INPUT
+  mode held in float, no use_fwd_quant."""
+  cfg = R.fully_quantized(8, 8, use_fwd_quant=False, use_stochastic_rounding=False)
+  _po2(cfg)
+  for raw in (cfg.fwd, cfg.dlhs, cfg.drhs):
+    raw.lhs_dequant_mode, raw.rhs_dequant_mode = lmode, rmode
+    raw.lhs_calibration_mode, raw.rhs_calibration_mode = lcal, rcal
+    for q, mode in ((raw.lhs, lmode), (raw.rhs, rmode)):
+      if mode == 'this_input' or disable_rounding:
+        q.keep_float = True
+      if disable_rounding:
+        q.round = False
+    if 'this_input' in (lmode, rmode) or disable_rounding:
+      raw.acc = None
+  return cfg
+
+
+MODE_CASES = [
+    ('CA', dict(lmode='output', rmode='output', disable_rounding=True)),
+    ('CA fake', dict(lmode='this_input', rmode='this_input', disable_rounding=True)),
+    ('RA L', dict(lmode='other_input', rmode='this_input', lcal='ra', rcal='ra')),
+    ('RA R', dict(lmode='this_input', rmode='other_input', lcal='ra', rcal='ra')),
+    ('RA fake', dict(lmode='this_input', rmode='this_input', lcal='ra', rcal='ra')),
+]
+
+
+def test_equality_between_different_calibration_axes():
+  """aqt_dot_general_test.py:972-1048: on power-of-two data (no quantization loss) calibrating
+  over the contraction axes with output dequantisation, over the remaining axes with the
+  scale moved to the other operand, and the fake-quant forms all give the float result;
+  a wrong scale transpose or calibration axis breaks it."""
+  lhs, rhs, g = _po2_data((10, 20), 1), _po2_data((20, 30), 2), _po2_data((10, 30), 3)
+  want = (lhs @ rhs, g @ rhs.T, lhs.T @ g)
+  for name, kw in MODE_CASES:
+    cfg = _mode_cfg(**kw)
+    f = R.dg_fwd(lhs, rhs, 'f32', MATMUL, cfg)
+    got = (f.out,) + tuple(R.dg_bwd(g, 'f32', MATMUL, f, cfg))
+    for x, y in zip(got, want):
+      np.testing.assert_array_equal(x, y, err_msg=name)
