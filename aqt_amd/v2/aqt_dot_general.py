@@ -216,7 +216,9 @@ class DefaultDotGeneralQuantizer(DotGeneralQuantizer):
       assert quantizer is not None
       qt = quantizer.calibrate(x, calibration_axes=ra)
       assert len(qt.scale) == 1, 'you must set some numerics'
-      scale = dezero(qt.scale[0]) ** alpha
+      scale = dezero(qt.scale[0])
+      # x ** alpha; the two usual exponents avoid the device pow (a few ulp off)
+      scale = scale if alpha == 1.0 else torch.sqrt(scale) if alpha == 0.5 else scale ** alpha
       return scale, transpose_fn(scale, dimension_numbers, other_shape)
 
     lhs_mid_scale, lhs_mid_scale_t = mid(self.lhs_mid, lhs, lhs_ra, self.lhs_mid_alpha,

@@ -104,14 +104,23 @@ class Quantizer:
     if (spec is None or qt.bias or qt.tiling_state is not None or len(qt.scale) != 1
         or qt.sparsity_mask is not None or getattr(self.numerics, 'clip_gradient', False)
         or not x.is_floating_point()):
-      # No fused scale-and-round kernel for this case (or the scaled tensor has to be kept for
-      # clip_gradient): scale, then the numerics' own forward
-      q_scaled = qt.quant(x)
-      x_q, res = self.numerics.vjp_fwd(q_scaled.qvalue, self.context)
-      q_scaled.qvalue = x_q
-      if self.numerics.get_dtype() is utils.int4:
-        q_scaled.container_dtype = utils.int4
-      return q_scaled, functools.partial(self.numerics.vjp_bwd, res)
+      return self._calculate_qvalue_stepwise(x, qt)
+    try:
+      return self._calculate_qvalue_kernel(x, qt, spec)
+    except lowering.NotFused:
+      return self._calculate_qvalue_stepwise(x, qt)
+
+  def _calculate_qvalue_stepwise(self, x, qt: aqt_tensor.QTensor):
+    """No fused scale-and-round kernel for this case (or the scaled tensor has to be kept for
+    clip_gradient): scale, then the numerics' own forward."""
+    q_scaled = qt.quant(x)
+    x_q, res = self.numerics.vjp_fwd(q_scaled.qvalue, self.context)
+    q_scaled.qvalue = x_q
+    if self.numerics.get_dtype() is utils.int4:
+      q_scaled.container_dtype = utils.int4
+    return q_scaled, functools.partial(self.numerics.vjp_bwd, res)
+
+  def _calculate_qvalue_kernel(self, x, qt: aqt_tensor.QTensor, spec):
     (s,) = qt.scale
     shared = [a for a in range(x.dim()) if s.shape[a] == 1 and x.shape[a] > 1]
     rest = [a for a in range(x.dim()) if a not in shared]

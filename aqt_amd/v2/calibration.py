@@ -41,12 +41,30 @@ class _UnitBound:
     return 1.0
 
 
+def _exp2_int(e):
+  """2**e as float32 for an integer tensor e, written into the exponent field (ldexp and pow go
+  through the device's exp2/log2 and can be one ulp off)."""
+  biased = torch.clamp(e.to(torch.int32) + 127, 1, 254)
+  return torch.bitwise_left_shift(biased, 23).view(torch.float32)
+
+
 def ceil_to_po2(scale):
-  """1 / 2**floor(log2(1 / scale)) (calibration.py:25-30): the power of two at or above `scale`."""
-  r = torch.reciprocal(scale)
-  e = torch.floor(torch.log2(r))
-  p = torch.ldexp(torch.ones_like(r), e.to(torch.int32))
-  return torch.reciprocal(p)
+  """1 / 2**floor(log2(1 / scale)) (calibration.py:25-30), each step rounded to scale.dtype.
+
+  The device reciprocal is not correctly rounded: one ulp at a power of two would halve the
+  result or leave it one ulp off a power of two.  In float32 the result is the power of two
+  at or above `scale`, read from the exponent field.  In a narrower dtype the roundings of the
+  intermediate reciprocal and logarithm are part of the result (log2 can round up to the next
+  integer), so those two steps are done in float64 and rounded to the dtype.
+  """
+  if scale.dtype == torch.float32:
+    m, e = torch.frexp(scale)  # scale = m * 2**e with 0.5 <= m < 1
+    e = torch.where(m == 0.5, e - 1, e)
+    return _exp2_int(e)
+  r = torch.reciprocal(scale.double()).to(scale.dtype)
+  l = torch.log2(r.double()).to(scale.dtype)
+  e = torch.floor(l.float()).to(torch.int32)
+  return _exp2_int(-e).to(scale.dtype)
 
 
 @dataclasses.dataclass(kw_only=True)

@@ -158,7 +158,7 @@ def quantize_view(v: OperandView, *, spec: dict, compute_dtype, scale_dtype, key
   if noise != L.NOISE_NONE:
     assert key is not None, 'stochastic rounding requested but Context.key is None'
     if v.noise_strides is None:
-      raise NotImplementedError('noise counters for this axis layout are not supported')
+      raise NotFused('noise counters for this axis layout are not supported')
     nb, nr, nk = v.noise_strides
     kwargs.update(key=key, noise_total=_prod(v.shape),
                   noise_strides=(nb, nr, nk) if v.k_last else (nb, nk, nr))

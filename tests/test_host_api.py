@@ -208,3 +208,21 @@ def test_einsum_dimension_numbers():
   torch.testing.assert_close(out, torch.einsum('bsd,dhk->bshk', x, w))
   out = aqt.einsum('bqd,bkd->bkq', torch.randn(2, 3, 4), torch.randn(2, 5, 4), spy)
   assert seen['dn'] == (((2,), (2,)), ((0,), (0,))) and tuple(out.shape) == (2, 5, 3)
+
+
+def test_ceil_to_po2_matches_oracle_op_by_op():
+  """calibration.py:25-30 in float32 (random scales over 2^-29..2^29) and bfloat16 (every
+  positive normal value away from the exponent limits)."""
+  import numpy as np
+  import torch
+  from aqt_amd.v2 import calibration
+  from oracle import aqt_ref as R
+  v = np.exp(np.random.default_rng(0).uniform(-20, 20, 100000)).astype(np.float32)
+  v = np.concatenate([v, np.exp2(np.arange(-29, 30)).astype(np.float32)])
+  got = calibration.ceil_to_po2(torch.from_numpy(v)).numpy()
+  np.testing.assert_array_equal(got, R.ceil_to_po2(v, 'f32'))
+  assert (got >= v).all() and (got < 2 * v).all()
+  allb = torch.arange(0x0100, 0x7E80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+  got = calibration.ceil_to_po2(allb)
+  assert got.dtype == torch.bfloat16
+  np.testing.assert_array_equal(got.float().numpy(), R.ceil_to_po2(allb.float().numpy(), 'bf16'))
