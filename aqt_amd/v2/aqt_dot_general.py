@@ -88,12 +88,12 @@ def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_eleme
   b = 1
   for s in bshape:
     b *= s
-  lt = lhs.permute(*(lba + lra + lca)).reshape(b, -1, kdim)
+  lt = lhs.permute(tuple(lba + lra + lca)).reshape(b, -1, kdim)
   both_int = lhs.dtype == torch.int8 and rhs.dtype == torch.int8
   both_fp8 = lhs.dtype in _FP8_DTYPES and rhs.dtype in _FP8_DTYPES
   if both_int or both_fp8:
     # the kernels take both operands with the contraction axis innermost
-    rt = rhs.permute(*(rba + rra + rca)).reshape(b, -1, kdim)
+    rt = rhs.permute(tuple(rba + rra + rca)).reshape(b, -1, kdim)
     m, n = lt.shape[1], rt.shape[1]
     acc_dtype = torch.int32 if both_int else torch.float32
     if both_int:
@@ -112,7 +112,7 @@ def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_eleme
     if pet is not None and pet.is_floating_point and common.is_floating_point and (
         torch.finfo(pet).bits > torch.finfo(common).bits):
       common = pet  # wider accumulator asked for: keep its precision in the result
-    rt = rhs.permute(*(rba + rca + rra)).reshape(b, kdim, -1)
+    rt = rhs.permute(tuple(rba + rca + rra)).reshape(b, kdim, -1)
     out = torch.matmul(lt.to(common), rt.to(common))
   out = out.reshape(bshape + mshape + nshape)
   if preferred_element_type is not None:
@@ -350,7 +350,7 @@ def einsum(eqn: str, lhs, rhs, dg=lax_dot_general):
   names = batch + lfree + rfree
   perm = [names.index(c) for c in out]
   if perm != list(range(len(perm))):
-    res = res.permute(*perm)
+    res = res.permute(tuple(perm))
   return res
 
 
@@ -548,7 +548,7 @@ class DotGeneralRaw:
       if n_ca > 0:
         out = ops.sum_tiles(out.contiguous())
       if _out_transpose_axes is not None:
-        out = out.permute(*_out_transpose_axes)
+        out = out.permute(tuple(_out_transpose_axes))
       return out, None
 
   def _dispatch(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes):
@@ -612,7 +612,7 @@ class DotGeneralRaw:
     out = _qtensor_dot_general_unfused(lhs_qt, rhs_qt, dimension_numbers, self,
                                        torch.promote_types(lhs.dtype, rhs.dtype)).dequant()
     if out_transpose_axes is not None:
-      out = out.permute(*out_transpose_axes)
+      out = out.permute(tuple(out_transpose_axes))
     return out, res
 
   # ------------------------------------------------------------------------------
@@ -642,7 +642,7 @@ class DotGeneralRaw:
       out = self.dot_general(x, y, dimension_numbers, None, self.dg_accumulator_dtype)
       out = out.to(dequant_dtype)
       if out_transpose_axes is not None:
-        out = out.permute(*out_transpose_axes)
+        out = out.permute(tuple(out_transpose_axes))
       mk = lambda t: aqt_tensor.QTensor(qvalue=t, scale=[], scale_t=None, bias=[], dequant_dtype=t.dtype)
       res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=x, qx=mk(x)), quant_grad=None),
                           rhs=TensorRes(mt=MultiTensor(x=y, qx=mk(y)), quant_grad=None))
@@ -713,9 +713,9 @@ class DotGeneralRaw:
       out = out.reshape(bdims + ldims + rdims)
       if want_lba != lba:
         perm = [lba.index(a) for a in want_lba] + list(range(len(lba), out.dim()))
-        out = out.permute(*perm)
+        out = out.permute(tuple(perm))
       if out_transpose_axes is not None:
-        out = out.permute(*out_transpose_axes)
+        out = out.permute(tuple(out_transpose_axes))
 
     lhs_mt = MultiTensor(x=lhs, qx=lhs_qt_out)
     rhs_mt = MultiTensor(x=rhs_arr if not rhs_is_q else rhs.qvalue, qx=rhs_qt_out)

@@ -123,7 +123,7 @@ class QTensor:
     inv = [0] * len(axes)
     for pos, a in enumerate(axes):
       inv[a] = pos
-    return out.reshape(dims).permute(*inv)
+    return out.reshape(dims).permute(tuple(inv))
 
   def qvalue_astype(self, dtype):
     assert self.is_full(), _MSG_NO_QVALUE

@@ -109,7 +109,7 @@ def view_operand(x: torch.Tensor, ba: Sequence[int], ra: Sequence[int], ca: Sequ
   elif dense and within_ok and len(set(pattern)) == len(pattern) and is_subseq(pattern, ['b', 'k', 'r']):
     k_last = False
   else:
-    x = x.permute(*(ba + ra + ca)).contiguous()
+    x = x.permute(tuple(ba + ra + ca)).contiguous()
     # after the copy the logical axes are renumbered; keep the caller's numbering for shapes only
     b_n, r_n = len(ba), len(ra)
     mem = x.reshape(_prod(x.shape[:b_n]), _prod(x.shape[b_n:b_n + r_n]), _prod(x.shape[b_n + r_n:]))
@@ -117,7 +117,7 @@ def view_operand(x: torch.Tensor, ba: Sequence[int], ra: Sequence[int], ca: Sequ
     ns = tuple(_merged_stride(shape, g) for g in (ba, ra, ca))
     return OperandView(mem, k_last, ba, ra, ca, shape, None if None in ns else ns, copied)
   perm = ba + (ra + ca if k_last else ca + ra)
-  xp = x.permute(*perm)
+  xp = x.permute(tuple(perm))
   B, R, K = (_prod(shape[a] for a in g) for g in (ba, ra, ca))
   mem = xp.reshape(B, R, K) if k_last else xp.reshape(B, K, R)
   assert mem.is_contiguous()
@@ -137,7 +137,7 @@ def logical_from_brk(t: torch.Tensor, v: OperandView, k_keep: bool = True) -> to
   inv = [0] * len(axes)
   for pos, a in enumerate(axes):
     inv[a] = pos
-  return t.permute(*inv)
+  return t.permute(tuple(inv))
 
 
 _OUT_TORCH = {L.I8: torch.int8, L.I4: torch.int8, L.E4M3: torch.float8_e4m3fn, L.E5M2: torch.float8_e5m2}

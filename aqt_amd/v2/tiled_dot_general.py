@@ -311,7 +311,7 @@ def tiled_dot_general_with_tiling_states(lhs, xlhs: TilingState, rhs, xrhs: Tili
   perm = (list(range(n0))
           + interleave(range(n0, n1), range(n2, n3), xlhs.tile_map, lra)
           + interleave(range(n1, n2), range(n3, n4), xrhs.tile_map, rra))
-  out = out.permute(*perm) if perm else out
+  out = out.permute(tuple(perm)) if perm else out
   l_flat = interleave(l_ra_t_sh, l_ra_sh, xlhs.tile_map, lra, product=True)
   r_flat = interleave(r_ra_t_sh, r_ra_sh, xrhs.tile_map, rra, product=True)
   return out.reshape(list(ba_sh) + l_flat + r_flat)

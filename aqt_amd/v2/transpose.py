@@ -10,7 +10,7 @@ from aqt_amd.v2 import utils
 
 def transpose(t: torch.Tensor, axes: Sequence[int]) -> torch.Tensor:
   """transpose.py:29-95 (a permute; torch views make the reshape shortcut moot)."""
-  return t.permute(*axes)
+  return t.permute(tuple(axes))
 
 
 def _scale_trans(x, ca, ba):

@@ -118,17 +118,29 @@ def _modify_dg(readonly_dg, *, lhs_dequant_mode=OUTPUT, rhs_dequant_mode=OUTPUT,
   return dg
 
 
-def _aqt_dg_full(dequant_mode, *, readonly_dg, dims, **kw):
-  dg = _modify_dg(readonly_dg, lhs_dequant_mode=dequant_mode, rhs_dequant_mode=dequant_mode, **kw)
+def _aqt_dg_full_lr_diff(lhs_dequant_mode, rhs_dequant_mode, lhs_calibration_mode=CA,
+                         rhs_calibration_mode=CA, *, readonly_dg, dims, **kw):
+  dg = _modify_dg(readonly_dg, lhs_dequant_mode=lhs_dequant_mode, rhs_dequant_mode=rhs_dequant_mode,
+                  lhs_calibration_mode=lhs_calibration_mode, rhs_calibration_mode=rhs_calibration_mode, **kw)
   dg = config.set_context(dg, key=KEY, train_step=None)
   return lambda lhs, rhs: dg(lhs, rhs, dims)
 
 
-def _aqt_dg_raw(dequant_mode, *, readonly_dg, dims):
-  dg = _modify_dg(readonly_dg, lhs_dequant_mode=dequant_mode, rhs_dequant_mode=dequant_mode)
+def _aqt_dg_full(dequant_mode, calibration_mode=CA, **kw):
+  return _aqt_dg_full_lr_diff(dequant_mode, dequant_mode, calibration_mode, calibration_mode, **kw)
+
+
+def _aqt_dg_raw_lr_diff(lhs_dequant_mode, rhs_dequant_mode, lhs_calibration_mode=CA,
+                        rhs_calibration_mode=CA, *, readonly_dg, dims):
+  dg = _modify_dg(readonly_dg, lhs_dequant_mode=lhs_dequant_mode, rhs_dequant_mode=rhs_dequant_mode,
+                  lhs_calibration_mode=lhs_calibration_mode, rhs_calibration_mode=rhs_calibration_mode)
   dg = config.set_context(dg, key=KEY, train_step=None)
   dg.fwd.dg_quantizer.init_calibration()
   return lambda lhs, rhs: dg.fwd(lhs, rhs, None, None, dims)[0]
+
+
+def _aqt_dg_raw(dequant_mode, calibration_mode=CA, **kw):
+  return _aqt_dg_raw_lr_diff(dequant_mode, dequant_mode, calibration_mode, calibration_mode, **kw)
 
 
 def _eq(name, a, b, exact=True):
@@ -282,3 +294,109 @@ class _LaxDg(torch.autograd.Function):
       d, out_axes = aqt._update_dimension_numbers_for_backward(ctx.dims, y_is_lhs, g.dim(), y.dim())
       outs.append(aqt.lax_dot_general(g, y, d).permute(*out_axes))
     return outs[0], outs[1], None
+
+
+RA_CASES = [
+    dict(dg=lambda: config.config_v3(fwd_bits=3, dlhs_bits=4, drhs_bits=5, drhs_accumulator_dtype=torch.int32)),
+    dict(dg=lambda: config.dot_general_make(None, None)),
+    dict(dg=lambda: config.dot_general_make(1, 1)),
+    dict(dg=lambda: config.dot_general_make(1, 2)),
+    dict(dg=lambda: config.dot_general_make(2, 1)),
+    dict(dg=lambda: config.dot_general_make(2, 2)),
+    dict(dg=lambda: config.dot_general_make(8, 8)),
+    dict(dg=lambda: config.dot_general_make(8, 8), clip_gradient=True),
+    dict(dg=lambda: config.dot_general_make(8, 8, dlhs_local_aqt=_LOCAL2)),
+    dict(dg=lambda: config.dot_general_make(8, 8, drhs_local_aqt=_LOCAL2)),
+    dict(dg=lambda: config.dot_general_make(2, 2), dtype=torch.bfloat16),
+    dict(dg=lambda: config.dot_general_make(8, 8), dtype=torch.bfloat16),
+    dict(dg=lambda: config.dot_general_make(None, 8)),
+    dict(dg=lambda: config.dot_general_make(8, None)),
+    dict(dg=lambda: config.dot_general_make(2, 2), **_DIMS_5D),
+    *[_fqt(s, False) for s in range(3)],
+]
+
+
+@pytest.mark.parametrize('case', range(len(RA_CASES)))
+def test_dot_general_calibration_with_remaining_axis(gpu, case):
+  """aqt_dot_general_test.py:717-903: calibration over the remaining axes; the scale of one
+  operand is applied to the other operand (OTHER_INPUT) or the operand is fake-quantized; all
+  forms agree exactly, as full calls, raw forward calls and with local AQT in the backward."""
+  p = dict(lhs_maxval=10.0, rhs_maxval=20.0, gra_maxval=30.0, dims=(((1,), (0,)), ((), ())),
+           lhs_shape=(10, 20), rhs_shape=(20, 30), gra_shape=(10, 30), seed=0, dtype=torch.float32,
+           clip_gradient=False)
+  p.update(RA_CASES[case])
+  readonly_dg, dims, dtype = p['dg'](), p['dims'], p['dtype']
+  readonly_dg.drhs.rhs.use_fwd_quant = False
+  readonly_dg.dlhs.rhs.use_fwd_quant = False
+  lhs = _rand_unif(p['lhs_shape'], p['lhs_maxval'], p['seed'], dtype, gpu)
+  rhs = _rand_unif(p['rhs_shape'], p['rhs_maxval'], p['seed'] + 1, dtype, gpu)
+  gra = _rand_unif(p['gra_shape'], p['gra_maxval'], p['seed'] + 2, dtype, gpu)
+  common = dict(readonly_dg=readonly_dg, dims=dims)
+  full = functools.partial(_aqt_dg_full, clip_gradient=p['clip_gradient'], **common)
+  full_lr = functools.partial(_aqt_dg_full_lr_diff, clip_gradient=p['clip_gradient'], **common)
+  raw = functools.partial(_aqt_dg_raw, **common)
+  raw_lr = functools.partial(_aqt_dg_raw_lr_diff, **common)
+  exact = (_quantized(readonly_dg.fwd), _quantized(readonly_dg.dlhs), _quantized(readonly_dg.drhs))
+  check = functools.partial(_check_result_eq, lhs=lhs, rhs=rhs, gra=gra, exact=exact)
+  OTHER, RA = aqt.DequantMode.OTHER_INPUT, aqt.CalibrationMode.REMAINING_AXIS
+  check([
+      ('RA L       ', full_lr(OTHER, THIS_INPUT, RA, RA), dict()),
+      ('RA R       ', full_lr(THIS_INPUT, OTHER, RA, RA), dict()),
+      ('RA fake    ', full(THIS_INPUT, RA), dict()),
+      ('RA L fwd   ', raw_lr(OTHER, THIS_INPUT, RA, RA), dict(test_gradient=False)),
+      ('RA R fwd   ', raw_lr(THIS_INPUT, OTHER, RA, RA), dict(test_gradient=False)),
+      ('RA fake fwd', raw(THIS_INPUT, RA), dict(test_gradient=False)),
+  ])
+  check([
+      ('RA fake    ', full(THIS_INPUT, RA, local_aqt=_LOCAL2), dict()),
+      ('RA L       ', full_lr(OTHER, THIS_INPUT, RA, RA, local_aqt=_LOCAL2), dict()),
+      ('RA R       ', full_lr(THIS_INPUT, OTHER, RA, RA, local_aqt=_LOCAL2), dict()),
+  ])
+
+
+def test_dynamic_context(gpu):
+  """aqt_dot_general_test.py:1050-1058: a rank-1 contraction, value and gradient."""
+  dg = config.set_context(config.dot_general_make(), key=KEY, train_step=None)
+  lhs = torch.tensor([3.0, 4.0], device=gpu, requires_grad=True)
+  rhs = torch.tensor([4.0, 5.0], device=gpu, requires_grad=True)
+  out = dg(lhs, rhs, (((0,), (0,)), ((), ())))
+  out.backward()
+  assert out.item() == 32.0
+  assert lhs.grad.tolist() == [4.0, 5.0] and rhs.grad.tolist() == [3.0, 4.0]
+
+
+def test_hardware_int8(gpu):
+  """aqt_dot_general_test.py:1060-1077: the contraction of an 8-bit config really is
+  int8 x int8 -> int32."""
+  dg_raw = config.dot_general_raw_make(8, 8)
+  seen = []
+
+  def hook(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
+    out = aqt.lax_dot_general(lhs, rhs, dimension_numbers, precision, preferred_element_type)
+    seen.append((lhs.dtype, rhs.dtype, out.dtype))
+    return out
+
+  dg_raw.dot_general = hook
+  lhs = _rand_unif((10, 20), 1.0, 0, torch.float32, gpu)
+  rhs = _rand_unif((20, 30), 1.0, 1, torch.float32, gpu)
+  ret, _ = dg_raw(lhs, rhs, None, None, (((1,), (0,)), ((), ())))
+  assert seen == [(torch.int8, torch.int8, torch.int32)] and ret.dtype == torch.float32
+  assert dg_raw.dg_quantizer.lhs.numerics.get_dtype() == torch.int8
+  assert dg_raw.dg_quantizer.rhs.numerics.get_dtype() == torch.int8
+
+
+@pytest.mark.parametrize('shard_count,expected_product', [(2, 1281280.0), (1, 1280000.0)])
+def test_local_aqt_known_answer(gpu, shard_count, expected_product):
+  """aqt_dot_general_test.py:1079-1113: with two shards the small and the large half of lhs
+  get their own scales in the drhs contraction, with one shard 1270 and 10 round to 0 and 0...
+  the reference's expected gradients."""
+  dg = config.fully_quantized(fwd_bits=8, bwd_bits=8, use_stochastic_rounding=False,
+                              drhs_local_aqt=aqt.LocalAqt(contraction_axis_shard_count=shard_count))
+  for q in (dg.fwd.dg_quantizer.lhs, dg.fwd.dg_quantizer.rhs, dg.drhs.dg_quantizer.lhs, dg.drhs.dg_quantizer.rhs):
+    q.numerics.preserve_max_val = True
+  dg = config.set_context(dg, None, None)
+  lhs = torch.tensor([1270.0, 10.0, 1270000.0, 10000.0], device=gpu, requires_grad=True)
+  rhs = torch.tensor([1.0], device=gpu, requires_grad=True)
+  out = dg(lhs, rhs, (((), ()), ((), ())))
+  out.backward(torch.ones_like(out))
+  assert rhs.grad.item() == expected_product
