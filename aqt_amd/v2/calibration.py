@@ -132,3 +132,87 @@ class ConstantCalibration(Calibration):
     else:
       bias = [torch.full(tuple(x.shape), float(self.bias), dtype=x.dtype, device=x.device)]
     return [scale.to(dtype)], bias, None
+
+
+@dataclasses.dataclass(kw_only=True)
+class AbsMeanCalibration(Calibration):
+  """clipping_scale * mean(abs(x) ** p) ** (1 / p) over the non-zero entries (calibration.py:160-193).
+
+  Reductions and elementwise steps in x.dtype; not a fused kernel (a weight-side calibration).
+  """
+
+  clipping_scale: float = None
+  p: float = None
+
+  def get_scale_and_bias_and_sparsity(self, x, shared_axes, numerics_, context=None):
+    del context
+    assert shared_axes is not None
+    dtype = self.dtype if self.dtype is not None else x.dtype
+    axes = [a % x.dim() for a in shared_axes]
+
+    def total(t):
+      return torch.sum(t, dim=axes, keepdim=True) if axes else t
+
+    powed = torch.abs(x) if self.p == 1.0 else torch.abs(x) ** self.p
+    abs_sum = total(powed)
+    count = total((x != 0.0).to(torch.int32))
+    count = torch.where(count == 0, torch.ones_like(count), count)
+    abs_mean = abs_sum / count.to(x.dtype)
+    if self.p != 1.0:
+      abs_mean = abs_mean ** (1.0 / self.p)
+    abs_mean = abs_mean * torch.tensor(self.clipping_scale, dtype=x.dtype, device=x.device)
+    abs_mean = torch.where(abs_mean == 0.0, torch.ones_like(abs_mean), abs_mean)
+    scale = abs_mean / torch.tensor(float(numerics_.get_quant_bound()), dtype=x.dtype, device=x.device)
+    if self.po2_scale:
+      scale = ceil_to_po2(scale)
+    return [scale.to(dtype)], [], None
+
+
+@dataclasses.dataclass(kw_only=True)
+class SnrBasedAutoCalibration(Calibration):
+  """Per group, the clipping scale out of `auto_clip_search_config` with the highest
+  log(1 + sum(x**2) / sum(err**2)) of the fake-quantized tensor (calibration.py:196-399).
+
+  One quantize / dequantize kernel pair per candidate plus elementwise steps; meant for
+  weights, as in the reference.
+  """
+
+  auto_clip_search_config: Sequence[float] = None
+
+  def get_scale_and_bias_and_sparsity(self, x, shared_axes, numerics_, context=None):
+    from aqt_amd.v2 import aqt_tensor  # local import: aqt_tensor's users import this module
+    from aqt_amd.v2 import lowering
+    dtype = self.dtype if self.dtype is not None else x.dtype
+    axes = [a % x.dim() for a in shared_axes]
+    clip_shape = [1 if a in axes else s for a, s in enumerate(x.shape)]
+    best = torch.ones(clip_shape, dtype=torch.float32, device=x.device)
+    max_snr = torch.zeros(clip_shape, dtype=torch.float32, device=x.device)
+    if axes:
+      abs_max = lowering.absmax_scale(x, axes, _UnitBound(), x.dtype)
+    else:
+      abs_max = torch.abs(x)
+      abs_max = torch.where(abs_max == 0.0, torch.ones_like(abs_max), abs_max)
+    quant_bound = torch.tensor(float(numerics_.get_quant_bound()), dtype=x.dtype, device=x.device)
+
+    def total(t):
+      return torch.sum(t, dim=axes, keepdim=True) if axes else t
+
+    signal = total(x * x)
+    for clip_scale in self.auto_clip_search_config:
+      bound = abs_max * torch.tensor(clip_scale, dtype=x.dtype, device=x.device)
+      scale = (bound / quant_bound).to(dtype)
+      qt = aqt_tensor.QTensor(qvalue=None, scale=[scale], scale_t=None, bias=[], dequant_dtype=x.dtype)
+      qt = qt.quant(x)
+      qt.qvalue, _ = numerics_.vjp_fwd(qt.qvalue, context)
+      if numerics_.get_dtype() is utils.int4:
+        qt.container_dtype = utils.int4
+      err = x - qt.dequant()
+      noise = total(err * err)
+      snr = torch.log(1 + signal / noise)
+      best = torch.where(snr > max_snr, torch.tensor(clip_scale, dtype=torch.float32, device=x.device), best)
+      max_snr = torch.maximum(snr.to(torch.float32), max_snr)
+    # a tensor divisor: division by a Python scalar becomes a multiplication by its reciprocal
+    scale = (abs_max * best) / quant_bound.to(torch.float32)
+    if self.po2_scale:
+      scale = ceil_to_po2(scale)
+    return [scale.to(dtype)], [], None

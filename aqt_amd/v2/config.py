@@ -220,6 +220,18 @@ def _update_calibration_keywords(quantizer: aqt_quantizer.Quantizer, only_cls=No
   return True
 
 
+def set_auto_calib_scale(cfg: DotGeneral, auto_clip_search_config: Sequence[float]) -> None:
+  """The weight-side (rhs) quantizers search their clipping scale by SNR (config.py:375-410)."""
+  for raw in (cfg.fwd, cfg.dlhs, cfg.drhs):
+    assert isinstance(raw.dg_quantizer, aqt_dot_general.DefaultDotGeneralQuantizer)
+    quantizer = raw.dg_quantizer.rhs
+    keywords = {}
+    if isinstance(quantizer.calibration, functools.partial):
+      keywords = dict(quantizer.calibration.keywords)
+    keywords.update(auto_clip_search_config=auto_clip_search_config)
+    quantizer.calibration = functools.partial(calibration.SnrBasedAutoCalibration, **keywords)
+
+
 def set_absmax_calib_scale(cfg: DotGeneral, scale: float):
   """config.py:418-460."""
   for q in _all_quantizers(cfg):

@@ -43,6 +43,8 @@ class QuantizerCfg:
   po2_scale: bool = False
   clipping_scale: Optional[float] = None
   const_bound: Optional[float] = None  # ConstantCalibration(bound=...)
+  abs_mean_p: Optional[float] = None  # AbsMeanCalibration(p=..., clipping_scale=...)
+  auto_clip_search: Optional[Sequence[float]] = None  # SnrBasedAutoCalibration
   preserve_zero: bool = True
   preserve_max_val: bool = False
   clip: bool = True
@@ -279,15 +281,32 @@ def ceil_to_po2(scale, dt):
 
 
 def calibrate(x, dt, shared_axes, q: QuantizerCfg):
-  """AbsMaxCalibration / ConstantCalibration (calibration.py:68-157).
+  """AbsMaxCalibration / ConstantCalibration / AbsMeanCalibration / SnrBasedAutoCalibration
+  (calibration.py:68-399).
 
   Returns (scale float32 array with keepdims shape, scale dtype tag).
   """
   sdt = q.scale_dtype or dt
   axes = tuple(shared_axes)
+  if q.auto_clip_search is not None:
+    return _snr_calibrate(x, dt, axes, q), sdt
+  qb = nm.cast(np.float32(quant_bound(q)), dt)
   if q.const_bound is not None:
     shape = [1 if a in axes else s for a, s in enumerate(x.shape)]
     bound = nm.cast(np.ones(shape, np.float32) * np.float32(q.const_bound), dt)
+  elif q.abs_mean_p is not None:
+    # calibration.py:160-193; sums accumulate in float32 and round once to dt (the order of
+    # the summation inside XLA is not restated: parity unpinned for non-exact sums)
+    p = nm.cast(np.float32(q.abs_mean_p), dt)
+    powed = np.abs(x) if q.abs_mean_p == 1.0 else nm.cast(np.power(np.abs(x), p), dt)
+    abs_sum = nm.cast(np.sum(powed.astype(np.float32), axis=axes, keepdims=True), dt)
+    count = np.sum(x != 0.0, axis=axes, keepdims=True).astype(np.float32)
+    count = np.where(count == 0.0, np.float32(1.0), count)
+    mean = nm.cast(abs_sum / nm.cast(count, dt), dt)
+    inv_p = nm.cast(np.float32(1.0 / q.abs_mean_p), dt)
+    abs_mean = mean if q.abs_mean_p == 1.0 else nm.cast(np.power(mean, inv_p), dt)
+    abs_mean = nm.cast(abs_mean * nm.cast(np.float32(q.clipping_scale), dt), dt)
+    bound = np.where(abs_mean == 0.0, np.float32(1.0), abs_mean)
   else:
     abs_max = np.max(np.abs(x), axis=axes, keepdims=True).astype(np.float32)
     abs_max = np.where(abs_max == 0.0, np.float32(1.0), abs_max)
@@ -295,11 +314,43 @@ def calibrate(x, dt, shared_axes, q: QuantizerCfg):
       bound = nm.cast(abs_max * nm.cast(np.float32(q.clipping_scale), dt), dt)
     else:
       bound = abs_max
-  qb = nm.cast(np.float32(quant_bound(q)), dt)
   scale = nm.cast(bound / qb, dt)
   if q.po2_scale:
     scale = ceil_to_po2(scale, dt)
   return nm.cast(scale, sdt), sdt
+
+
+def _snr_calibrate(x, dt, axes, q: QuantizerCfg):
+  """SnrBasedAutoCalibration (calibration.py:196-399): for every candidate clipping scale the
+  tensor is fake-quantized and log(1 + signal / noise) computed per group; the best candidate
+  per group gives the scale.  The search keeps float32 state; the candidate scales are
+  computed in the input dtype, the final one in float32 (abs_max * float32 clip)."""
+  sdt = q.scale_dtype or dt
+  x = np.asarray(x, np.float32)
+  abs_max = np.max(np.abs(x), axis=axes, keepdims=True).astype(np.float32)
+  abs_max = np.where(abs_max == 0.0, np.float32(1.0), abs_max)
+  best = np.ones(abs_max.shape, np.float32)
+  max_snr = np.zeros(abs_max.shape, np.float32)
+  qbf = np.float32(quant_bound(q))
+  for clip in q.auto_clip_search:
+    # abs_max (dt) * python float stays in dt
+    bound = nm.cast(abs_max * nm.cast(np.float32(clip), dt), dt)
+    scale = nm.cast(nm.cast(bound / nm.cast(qbf, dt), dt), sdt)
+    qt = calculate_qvalue(x, dt, QTensor(None, None, [scale], sdt, dt), q)
+    err = nm.cast(x - dequant(qt), dt)
+    noise = nm.cast(np.sum(nm.cast(err * err, dt).astype(np.float32), axis=axes, keepdims=True), dt)
+    signal = nm.cast(np.sum(nm.cast(x * x, dt).astype(np.float32), axis=axes, keepdims=True), dt)
+    with np.errstate(divide='ignore', invalid='ignore'):
+      ratio = nm.cast(signal / noise, dt)
+      snr = nm.cast(np.log(nm.cast(np.float32(1.0) + ratio, dt)), dt)
+    better = snr > max_snr
+    best = np.where(better, np.float32(clip), best)
+    max_snr = np.maximum(snr, max_snr)
+  bound = abs_max * best  # float32: dt array times a float32 array
+  scale = bound / qbf
+  if q.po2_scale:
+    scale = ceil_to_po2(scale, 'f32')
+  return nm.cast(scale, sdt)
 
 
 def qtensor_quant(x, dt, scales, sdt):

@@ -371,3 +371,52 @@ def test_equality_between_different_calibration_axes(gpu, name, kw):
   np.testing.assert_array_equal(_np(out), lhs @ rhs)
   np.testing.assert_array_equal(_np(L.grad), g @ rhs.T)
   np.testing.assert_array_equal(_np(Rr.grad), lhs.T @ g)
+
+
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('p,clip', [(1.0, 1.0), (1.0, 2.5), (2.0, 1.5)])
+def test_abs_mean_calibration(gpu, p, clip, dt):
+  """AbsMeanCalibration (calibration.py:160-193) on integer-valued data, where the sums are
+  exact whatever their order; p = 2 goes through the device pow (2 ulp allowed there)."""
+  from aqt_amd.v2 import aqt_quantizer
+  rng = np.random.default_rng(3)
+  x = rng.integers(-6, 7, (24, 96)).astype(np.float32)
+  x[5] = 0.0
+  q = aqt_quantizer.quantizer_make(8, initialize_calibration=False)
+  q.calibration = functools.partial(calibration.AbsMeanCalibration, clipping_scale=clip, p=p)
+  q.context = utils.Context(key=None, train_step=None)
+  q.init_calibration()
+  qx, _ = q.quant(U.to_dev(x, dt, gpu), calibration_axes=[1])
+  oq = R.QuantizerCfg(bits=8, abs_mean_p=p, clipping_scale=clip)
+  want = R.quantize(x, dt, oq, [1])
+  if p == 1.0:
+    np.testing.assert_array_equal(_np(qx.scale[0]), want.scale[0])
+    np.testing.assert_array_equal(_np(qx.qvalue), np.asarray(want.qvalue, np.float32))
+  else:
+    np.testing.assert_allclose(_np(qx.scale[0]), want.scale[0], rtol=2.4e-7 if dt == 'f32' else 8e-3)
+
+
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('bits', [4, 8])
+def test_snr_based_auto_calibration(gpu, bits, dt):
+  """SnrBasedAutoCalibration (calibration.py:196-399) through config.set_auto_calib_scale:
+  rows with an outlier pick a smaller clipping scale; scale and quantized weights equal the
+  oracle's."""
+  rng = np.random.default_rng(0)
+  w = rng.standard_normal((1024, 12)).astype(np.float32)
+  w[7, ::2] = 12.0 if bits == 4 else 300.0
+  w = R.nm.cast(w, dt)
+  lhs = U.rand((16, 1024), dt, 1)
+  cands = [1.0, 0.5, 0.25, 0.1, 0.05]
+  dg = config.dot_general_make(bits, bits)
+  config.set_auto_calib_scale(dg, cands)
+  dg = config.set_context(dg, None, None)
+  out, (_, rqt) = dg.dg_core(U.to_dev(lhs, dt, gpu), U.to_dev(w, dt, gpu), None, None, MATMUL)
+  oraw = R.RawCfg(R.QuantizerCfg(bits=bits), R.QuantizerCfg(bits=bits, auto_clip_search=cands))
+  want, _, (_, rres), _ = R.dg_raw(lhs, dt, w, dt, MATMUL, oraw)
+  np.testing.assert_array_equal(_np(rqt.scale[0]), rres.qx.scale[0])
+  np.testing.assert_array_equal(_np(rqt.qvalue), np.asarray(rres.qx.qvalue, np.float32))
+  np.testing.assert_array_equal(_np(out), want)
+  ratio = _np(rqt.scale[0])[0] / (np.abs(w).max(axis=0) / R.quant_bound(oraw.rhs))
+  if bits == 4:  # coarse steps: clipping the outlier pays
+    assert (ratio[::2] < 0.75).all() and len(set(np.round(ratio, 3))) > 1

@@ -224,3 +224,37 @@ def test_equality_between_different_calibration_axes():
     got = (f.out,) + tuple(R.dg_bwd(g, 'f32', MATMUL, f, cfg))
     for x, y in zip(got, want):
       np.testing.assert_array_equal(x, y, err_msg=name)
+
+
+def test_abs_mean_calibration_closed_forms():
+  """calibration.py:160-193: mean over the non-zero entries, p-norm form, clipping scale."""
+  x = np.array([[1.0, -2.0, 0.0, 3.0], [0.0, 0.0, 0.0, 0.0]], np.float32)
+  q = R.QuantizerCfg(bits=8, abs_mean_p=1.0, clipping_scale=1.0)
+  s, sdt = R.calibrate(x, 'f32', [1], q)
+  np.testing.assert_array_equal(s, np.array([[2.0], [1.0]], np.float32) / np.float32(127.5))
+  q = R.QuantizerCfg(bits=8, abs_mean_p=2.0, clipping_scale=3.0)
+  s, _ = R.calibrate(np.array([[3.0, 4.0, 0.0]], np.float32), 'f32', [1], q)
+  np.testing.assert_allclose(s, [[3.0 * np.sqrt(12.5) / 127.5]], rtol=3e-7)
+
+
+def test_snr_calibration_picks_the_brute_force_best_clip():
+  """calibration.py:196-399: with a single candidate 1.0 it is abs-max calibration; with an
+  outlier in a 4-bit row the candidate minimising the float64 squared error wins."""
+  rng = np.random.default_rng(0)
+  x = rng.standard_normal((6, 1024)).astype(np.float32)
+  x[::2, 7] = 12.0  # outliers in every other row
+  only_one = R.QuantizerCfg(bits=4, auto_clip_search=[1.0])
+  s1, _ = R.calibrate(x, 'f32', [1], only_one)
+  s0, _ = R.calibrate(x, 'f32', [1], R.QuantizerCfg(bits=4))
+  np.testing.assert_array_equal(s1, s0)
+  cands = [1.0, 0.5, 0.25, 0.1, 0.05]
+  s, _ = R.calibrate(x, 'f32', [1], R.QuantizerCfg(bits=4, auto_clip_search=cands))
+  amax = np.abs(x).max(axis=1, keepdims=True).astype(np.float64)
+  errs = []
+  for c in cands:
+    sc = amax * c / 7.5
+    deq = np.clip(np.rint(x / sc), -7, 7) * sc
+    errs.append(((x - deq) ** 2).sum(axis=1))
+  best = np.array(cands)[np.argmin(np.stack(errs), axis=0)]
+  np.testing.assert_allclose(s[:, 0], (amax[:, 0] * best / 7.5), rtol=1e-6)
+  assert (best[::2] < best[1::2]).all()  # rows with the outlier clip harder
