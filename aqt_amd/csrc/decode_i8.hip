@@ -32,6 +32,7 @@ struct DecodeArgs {
   void* out;              // [m][n]
   int m, n, k;
   int out_bf16, xs_bf16, ws_bf16;
+  int acc_shift;  // 4 when the weight operand holds 16 * w (unpacked nibbles), else 0
 };
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
@@ -39,7 +40,7 @@ __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x
 // QTensor.dequant: cast the accumulator, multiply by the lhs scale, then the rhs scale, each
 // product in the promoted dtype of its operands, final cast.
 __device__ __forceinline__ void store_out(const DecodeArgs& d, int mm, int nn, int acc) {
-  float f = rnd((float)acc, d.out_bf16);
+  float f = rnd((float)(acc >> d.acc_shift), d.out_bf16);  // exact: acc is a multiple of 16 then
   const int p1 = d.out_bf16 & d.xs_bf16;
   f = rnd(f * d.x_scale[mm], p1);
   f = rnd(f * d.w_scale[nn], p1 & d.ws_bf16);
@@ -115,6 +116,103 @@ __global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) 
       store_out(d, mm, nn, s);
     }
   }
+}
+
+// ---- packed int4 weights -----------------------------------------------------------------------
+// Two int4 per byte, low nibble = even k.  A lane's 16-byte load holds 32 consecutive k of one
+// weight row, the B operands of two MFMAs; the matching 32 activation bytes are the two A
+// operands.  A nibble is moved to the top of its byte, which makes it 16 * w as a signed int8;
+// the factor leaves the accumulator as an exact right shift by 4.  Same workgroup shape as the
+// K-split kernel (weights stream from HBM once; half the bytes of the int8 form).
+__device__ __forceinline__ void unpack_i4x8(uint32_t w, int& lo, int& hi) {
+  const uint32_t ev = (w << 4) & 0xF0F0F0F0u;  // k0 k2 k4 k6
+  const uint32_t od = w & 0xF0F0F0F0u;         // k1 k3 k5 k7
+  lo = (int)__builtin_amdgcn_perm(od, ev, 0x05010400u);  // k0 k1 k2 k3
+  hi = (int)__builtin_amdgcn_perm(od, ev, 0x07030602u);  // k4 k5 k6 k7
+}
+
+// NB: 16-row weight blocks per wave; every activation fragment a wave loads is used NB times,
+// so the L2 traffic for the activations is MB / NB times the int8-equivalent weight bytes.
+template <int MB, int NB, int U>  // U: 128-k steps (16 packed bytes per lane and block) in flight per wave
+__global__ __launch_bounds__(256) void decode_ksplit_i4_kernel(const DecodeArgs d) {
+  __shared__ int red[4][NB][MB * 16][16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int n0 = blockIdx.x * (16 * NB);
+  const int kb = d.k / 2;  // bytes of one packed weight row
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * kb);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
+  const int kq = ((d.k + 3) / 4 + 127) / 128 * 128;  // K range of one wave, whole 128-k steps
+  const int k_lo = wave * kq;
+  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
+  int wbase[NB], xbase[MB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int row = n0 + nb * 16 + r;
+    wbase[nb] = (row < d.n ? row : d.n - 1) * kb + c * 16;  // clamped; such columns are never stored
+  }
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) xbase[mb] = (mb * 16 + r) < d.m ? (mb * 16 + r) * d.k + c * 32 : kOob;
+
+  v4i acc[MB][NB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = v4i{0, 0, 0, 0};
+  for (int kk = k_lo; kk < k_hi; kk += 128 * U) {
+    v4i wf[U][NB], xf[U][MB][2];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ko = kk + u * 128;
+      const bool ok = ko + c * 32 < k_hi;  // k is a multiple of 32: a lane's 32 k are all in or all out
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        wf[u][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? wbase[nb] + ko / 2 : kOob, 0, 0);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int xo = (ok && xbase[mb] != kOob) ? xbase[mb] + ko : kOob;
+        xf[u][mb][0] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
+        xf[u][mb][1] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo == kOob ? kOob : xo + 16, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        int t[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[u][nb][j], t[2 * j], t[2 * j + 1]);
+        const v4i b0 = v4i{t[0], t[1], t[2], t[3]}, b1 = v4i{t[4], t[5], t[6], t[7]};
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][mb][0], b0, acc[mb][nb], 0, 0, 0);
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][mb][1], b1, acc[mb][nb], 0, 0, 0);
+        }
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // lane holds C[m = mb*16 + 4c + e][n = n0 + nb*16 + r]
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave][nb][mb * 16 + 4 * c + e][r] = acc[mb][nb][e];
+  __syncthreads();
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const int mm = mb * 16 + (tid >> 4), nn = n0 + nb * 16 + (tid & 15);
+      if (mm < d.m && nn < d.n) {
+        const int s = red[0][nb][mm][tid & 15] + red[1][nb][mm][tid & 15] + red[2][nb][mm][tid & 15] +
+                      red[3][nb][mm][tid & 15];
+        store_out(d, mm, nn, s);
+      }
+    }
 }
 
 // ---- 16 < m <= 64 ------------------------------------------------------------------------------
@@ -262,8 +360,11 @@ int validate_decode(const aqtx_decode_plan* p) {
   AQTX_REQUIRE(p->m >= 0 && p->n >= 0 && p->k >= 0, "aqtx_decode_i8: negative shape");
   AQTX_REQUIRE(p->m <= 64, "aqtx_decode_i8: m = %lld exceeds 64 (use aqtx_quantize + aqtx_gemm_i8)",
                (long long)p->m);
-  AQTX_REQUIRE(p->k > 0 && p->k % 16 == 0, "aqtx_decode_i8: k = %lld must be a positive multiple of 16",
-               (long long)p->k);
+  AQTX_REQUIRE(p->w_dtype == AQTX_I8 || p->w_dtype == AQTX_I4 || p->w_dtype == AQTX_I4P,
+               "aqtx_decode_i8: w_dtype must be int8, int4 in int8 containers or packed int4");
+  const int64_t kmul = p->w_dtype == AQTX_I4P ? 32 : 16;
+  AQTX_REQUIRE(p->k > 0 && p->k % kmul == 0, "aqtx_decode_i8: k = %lld must be a positive multiple of %lld",
+               (long long)p->k, (long long)kmul);
   AQTX_REQUIRE(p->n * p->k < (1ll << 31) && p->m * p->n < (1ll << 31),
                "aqtx_decode_i8: weight larger than 2 GiB is not addressable with 32-bit offsets");
   AQTX_REQUIRE(is_float_dtype(p->x_dtype) && is_float_dtype(p->x_scale_dtype) &&
@@ -321,6 +422,20 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
   d.ws_bf16 = p->w_scale_dtype == AQTX_BF16;
 
   const unsigned grid16 = (unsigned)((p->n + 15) / 16);
+  if (p->w_dtype == AQTX_I4P) {
+    d.acc_shift = 4;
+    const unsigned grid32 = (unsigned)((p->n + 31) / 32);
+    // two weight blocks per wave halve the activation re-reads; worth it once n / 32 workgroups
+    // still fill the chip
+    const bool wide = p->n >= 8192;
+    if (p->m <= 16) decode_ksplit_i4_kernel<1, 1, 8><<<grid16, 256, 0, st>>>(d);
+    else if (p->m <= 32 && wide) decode_ksplit_i4_kernel<2, 2, 4><<<grid32, 256, 0, st>>>(d);
+    else if (p->m <= 32) decode_ksplit_i4_kernel<2, 1, 4><<<grid16, 256, 0, st>>>(d);
+    else if (wide) decode_ksplit_i4_kernel<4, 2, 2><<<grid32, 256, 0, st>>>(d);
+    else decode_ksplit_i4_kernel<4, 1, 2><<<grid16, 256, 0, st>>>(d);
+    AQTX_HIP_CHECK_LAUNCH("decode_ksplit_i4_kernel");
+    return 0;
+  }
   if (p->m <= 16) {
     decode_ksplit_kernel<1, 16><<<grid16, 256, 0, st>>>(d);
     AQTX_HIP_CHECK_LAUNCH("decode_ksplit_kernel");

@@ -222,16 +222,19 @@ def gemm(
 
 
 def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
-           clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False):
-  """Serving contraction out = dequant(quant(x) @ w_q^T) for x [m <= 64, k], w_q int8 [n, k].
+           clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False,
+           w_dtype: int = L.I8):
+  """Serving contraction out = dequant(quant(x) @ w_q^T) for x [m <= 64, k], w_q int8 [n, k], or
+  uint8 [n, k/2] holding packed int4 (w_dtype=I4P, the pack_i4 layout).
 
   The activations get per-token dynamic int8 quantisation; `w_scale` is float32 [n] holding
   values of `w_scale_dtype`.  Returns (out [m, n] of x.dtype, x_scale float32 [m]) and, with
   want_xq, the quantized activations as a third element.
   """
   _require_gpu(x, w_q, w_scale)
-  assert x.dim() == 2 and w_q.dim() == 2 and x.shape[1] == w_q.shape[1], (x.shape, w_q.shape)
-  assert x.is_contiguous() and w_q.is_contiguous() and w_q.dtype == torch.int8
+  packed = w_dtype == L.I4P
+  assert x.dim() == 2 and w_q.dim() == 2 and x.shape[1] == w_q.shape[1] * (2 if packed else 1), (x.shape, w_q.shape)
+  assert x.is_contiguous() and w_q.is_contiguous() and w_q.dtype == (torch.uint8 if packed else torch.int8)
   m, k = x.shape
   n = w_q.shape[0]
   assert w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() == n
@@ -242,6 +245,7 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   plan.w_scale_dtype = aqtx_dtype(w_scale_dtype)
   plan.out_dtype = plan.x_dtype
   plan.quant_bound, plan.clip_bound = float(quant_bound), float(clip_bound)
+  plan.w_dtype = w_dtype
   ws_bytes = int(L.lib().aqtx_decode_workspace_bytes(ctypes.byref(plan)))
   ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
   out = torch.empty((m, n), dtype=x.dtype, device=x.device)

@@ -436,12 +436,17 @@ def _apply_local_aqt(local_aqt, lhs, rhs, dimension_numbers):
 _KERNEL_LAYOUT_CACHE = {}   # id(frozen tensor) -> (key, re-laid-out copy); entries die with the tensor
 
 
-def _kernel_layout_of(qvalue: torch.Tensor, v: 'lowering.OperandView') -> torch.Tensor:
-  key = (tuple(v.b_axes), tuple(v.r_axes), tuple(v.k_axes), qvalue._version)
+def _kernel_layout_of(qvalue: torch.Tensor, v: 'lowering.OperandView', pack_int4: bool = False) -> torch.Tensor:
+  """The operand as the kernels read it ([B, R, K], contraction axis contiguous); with
+  pack_int4 additionally packed two values per byte ([B, R, K/2] uint8), which halves the bytes
+  a serving call streams from HBM."""
+  key = (tuple(v.b_axes), tuple(v.r_axes), tuple(v.k_axes), qvalue._version, pack_int4)
   hit = _KERNEL_LAYOUT_CACHE.get(id(qvalue))
   if hit is not None and hit[0] == key:
     return hit[1]
   q = v.mem if v.k_last else v.mem.transpose(1, 2).contiguous()
+  if pack_int4:
+    q = ops.pack_i4(q.contiguous())
   if hit is None:
     weakref.finalize(qvalue, _KERNEL_LAYOUT_CACHE.pop, id(qvalue), None)
   _KERNEL_LAYOUT_CACHE[id(qvalue)] = (key, q)
@@ -739,7 +744,7 @@ class DotGeneralRaw:
         or dq.lhs.calib_shared_axes is not None or getattr(dq.lhs.numerics, 'clip_gradient', False)):
       return None
     if (rhs_qt.qvalue.dtype != torch.int8 or len(rhs_qt.scale) != 1 or rhs_qt.bias
-        or rhs_qt.container_dtype is not None or dequant_dtype != lhs.dtype
+        or rhs_qt.container_dtype not in (None, utils.int4) or dequant_dtype != lhs.dtype
         or self.dg_accumulator_dtype != utils.int32):
       return None
     lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
@@ -748,10 +753,15 @@ class DotGeneralRaw:
     rv = lowering.view_operand(rhs_qt.qvalue, [], rra, rca)
     if not lv.k_last or lv.copied:
       return None
-    rq = rv.mem if rv.k_last and not rv.copied else _kernel_layout_of(rhs_qt.qvalue, rv)
     M, K, N = lv.R, lv.K, rv.R
+    # int4 weights are streamed packed two per byte (a copy made once per frozen tensor)
+    packed = rhs_qt.container_dtype is utils.int4 and K % 32 == 0
     if M == 0 or M > 64 or K == 0 or K % 16 != 0 or N == 0 or N * K >= 2 ** 31:
       return None
+    if packed:
+      rq = _kernel_layout_of(rhs_qt.qvalue, rv, pack_int4=True)
+    else:
+      rq = rv.mem if rv.k_last and not rv.copied else _kernel_layout_of(rhs_qt.qvalue, rv)
     w_scale = rhs_qt.scale[0]
     sv = lowering.view_operand(w_scale, [], rra, rca)
     if sv.mem.numel() != N:
@@ -759,7 +769,8 @@ class DotGeneralRaw:
     sdt = dq.lhs._calibrator.dtype if dq.lhs._calibrator.dtype is not None else lhs_dtype
     out, xs, xq = ops.decode(lv.mem[0], rq[0], sv.mem.reshape(-1).float().contiguous(),
                              quant_bound=spec['quant_bound'], clip_bound=spec['clip_bound'],
-                             x_scale_dtype=sdt, w_scale_dtype=w_scale.dtype, want_xq=True)
+                             x_scale_dtype=sdt, w_scale_dtype=w_scale.dtype, want_xq=True,
+                             w_dtype=L.I4P if packed else L.I4 if rhs_qt.container_dtype is utils.int4 else L.I8)
     out = out.reshape([lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
     qv = lowering.logical_from_brk(xq[None], lv)
     sc = lowering.logical_from_brk(xs.reshape(1, M), lv, k_keep=False).to(sdt)

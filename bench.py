@@ -71,47 +71,55 @@ def cpu_baseline(seconds_budget=30.0):
 
 
 def decode_bench(dev):
-  """Serving shapes (rhs frozen as int8 + f32 per-channel scale, K = 4096): device time per call of
-  aqtx_decode_i8 (activation quantisation + contraction + dequantisation) and the HBM rate on the
-  algorithmic bytes K*N + 4N + 2MK + 2MN.  Weight copies rotate through >= 1 GiB so that no cache
+  """Serving shapes (rhs frozen as int8, or as int4 packed two per byte, + f32 per-channel scale,
+  K = 4096): device time per call of aqtx_decode_i8 (activation quantisation + contraction +
+  dequantisation) and the HBM rate on the algorithmic bytes K*N (K*N/2) + 4N + 2MK + 2MN.  Weight copies rotate through >= 1 GiB so that no cache
   level can hold them; the calls are replayed from a HIP graph so that host launch overhead does
   not sit between the kernels being timed."""
   import torch
+  from aqt_amd import _lib as L
   from aqt_amd import ops
   k = 4096
   rows = []
-  for n in (4096, 14336):
-    ncopies = (1 << 30) // (n * k) + 1
-    weights = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(ncopies)]
-    w_scale = torch.rand(n, device=dev) * 1e-3 + 1e-5
-    for m in (1, 8, 32, 64):
-      x = torch.randn(m, k, device=dev).to(torch.bfloat16)
-      run = lambda: [ops.decode(x, w, w_scale, quant_bound=127.5, clip_bound=127.0) for w in weights]
-      run()
-      torch.cuda.synchronize()
-      side = torch.cuda.Stream()
-      graph = torch.cuda.CUDAGraph()
-      with torch.cuda.stream(side):
+  for w_kind in ('int8', 'int4_packed'):
+    packed = w_kind == 'int4_packed'
+    wbytes_per = 0.5 if packed else 1.0
+    for n in (4096, 14336):
+      ncopies = int((1 << 30) // (n * k * wbytes_per)) + 1
+      if packed:
+        weights = [torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev) for _ in range(ncopies)]
+      else:
+        weights = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(ncopies)]
+      w_scale = torch.rand(n, device=dev) * 1e-3 + 1e-5
+      kw = dict(quant_bound=127.5, clip_bound=127.0, w_dtype=L.I4P if packed else L.I8)
+      for m in (1, 8, 32, 64):
+        x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+        run = lambda: [ops.decode(x, w, w_scale, **kw) for w in weights]
         run()
         torch.cuda.synchronize()
-        with torch.cuda.graph(graph, stream=side):
-          keep = run()
-      torch.cuda.synchronize()
-      graph.replay()
-      torch.cuda.synchronize()
-      reps = 5
-      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-      a.record()
-      for _ in range(reps):
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+          run()
+          torch.cuda.synchronize()
+          with torch.cuda.graph(graph, stream=side):
+            keep = run()
+        torch.cuda.synchronize()
         graph.replay()
-      b.record()
-      torch.cuda.synchronize()
-      us = a.elapsed_time(b) * 1e3 / (reps * ncopies)
-      nbytes = k * n + 4 * n + 2 * m * k + 2 * m * n
-      rows.append({'n': n, 'm': m, 'us_per_call': round(us, 2), 'GB/s': round(nbytes / us / 1e3, 1),
-                   'frac_of_8TBps': round(nbytes / us / 1e3 / 8000.0, 3)})
-      del graph, keep
-    del weights
+        torch.cuda.synchronize()
+        reps = 5
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+          graph.replay()
+        b.record()
+        torch.cuda.synchronize()
+        us = a.elapsed_time(b) * 1e3 / (reps * ncopies)
+        nbytes = int(k * n * wbytes_per) + 4 * n + 2 * m * k + 2 * m * n
+        rows.append({'weights': w_kind, 'n': n, 'm': m, 'us_per_call': round(us, 2),
+                     'GB/s': round(nbytes / us / 1e3, 1), 'frac_of_8TBps': round(nbytes / us / 1e3 / 8000.0, 3)})
+        del graph, keep
+      del weights
   return rows
 
 

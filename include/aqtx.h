@@ -226,6 +226,7 @@ typedef struct aqtx_decode_plan {
   int32_t w_scale_dtype;  /* dtype of the weight scale (values in f32)  */
   int32_t out_dtype;      /* AQTX_BF16 | AQTX_F32                       */
   float quant_bound, clip_bound; /* of the activation numerics        */
+  int32_t w_dtype;        /* AQTX_I8 | AQTX_I4 (container) | AQTX_I4P (packed: k multiple of 32) */
 } aqtx_decode_plan;
 
 /*
@@ -236,7 +237,8 @@ typedef struct aqtx_decode_plan {
  * QTensor.dequant; the standalone reference equivalents are
  * pallas/quantizer.py:33-68 and pallas/dot_general.py:57-137.
  *   x        in  : [m, k] activations
- *   w        in  : int8 [n, k] (weight stored with the contraction axis contiguous)
+ *   w        in  : int8 [n, k] (weight stored with the contraction axis contiguous), or
+ *                  uint8 [n, k/2] for AQTX_I4P (aqtx_pack_i4 layout)
  *   w_scale  in  : float32 [n]
  *   xq       out : optional int8 [m, k] (the quantized activations), may be NULL
  *   x_scale  out : float32 [m]

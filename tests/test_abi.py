@@ -38,6 +38,7 @@ def _qplan(**kw):
   p.batch, p.rows, p.cols = 1, 4, 64
   p.reduce = L.REDUCE_COLS
   p.quant_bound, p.clip_bound = 127.5, 127.0
+  p.w_dtype = L.I8
   for k, v in kw.items():
     setattr(p, k, v)
   return p
@@ -152,6 +153,7 @@ def _dplan(**kw):
   p.x_dtype = p.x_scale_dtype = p.out_dtype = L.BF16
   p.w_scale_dtype = L.F32
   p.quant_bound, p.clip_bound = 127.5, 127.0
+  p.w_dtype = L.I8
   for k, v in kw.items():
     setattr(p, k, v)
   return p
@@ -165,6 +167,8 @@ def _dplan(**kw):
     (dict(x_dtype=L.I8), 'dtypes'),
     (dict(quant_bound=0.0), 'bounds'),
     (dict(n=1 << 20, k=4096), '2 GiB'),
+    (dict(w_dtype=L.E4M3), 'w_dtype'),
+    (dict(w_dtype=L.I4P, k=48), 'multiple of 32'),
 ])
 def test_decode_plan_validation(kw, needle):
   p = _dplan(**kw)

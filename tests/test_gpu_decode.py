@@ -80,3 +80,47 @@ def test_decode_rejects_bad_plans(gpu):
     ops.decode(x, w, s, quant_bound=127.5, clip_bound=127.0)
   with pytest.raises(Exception, match='multiple of 16'):
     ops.decode(x[:4, :24].contiguous(), w[:, :24].contiguous(), s, quant_bound=127.5, clip_bound=127.0)
+
+
+@pytest.mark.parametrize('m', [1, 8, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize('n,k', [(256, 1024), (200, 480), (40, 32), (4096, 4096)])
+@pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('bf16', 'bf16'), ('f32', 'f32')])
+def test_decode_packed_int4_matches_oracle(gpu, m, n, k, dt, w_sdt):
+  """int4 weights packed two per byte (aqtx_pack_i4 layout): same numbers as the int8-held
+  form, half the weight bytes."""
+  from aqt_amd import _lib as L
+  if (n, k) == (4096, 4096) and (dt, w_sdt) != ('bf16', 'f32'):
+    pytest.skip('large shape once')
+  x = U.rand((m, k), dt, 200 + m, outliers=True)
+  rng = np.random.default_rng(11)
+  wq = rng.integers(-7, 8, size=(n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(3e-3) + np.float32(1e-4), w_sdt)
+  want, xq_want, xs_want = _oracle_decode(x, dt, wq, ws, w_sdt)
+  wq_t = torch.from_numpy(wq).to(gpu)
+  packed = ops.pack_i4(wq_t)
+  assert packed.shape == (n, k // 2) and packed.dtype == torch.uint8
+  out, xs, xq = ops.decode(U.to_dev(x, dt, gpu), packed, torch.from_numpy(ws).to(gpu), quant_bound=127.5,
+                           clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True, w_dtype=L.I4P)
+  np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
+  np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+  # and the int8-held int4 weight through the int8 kernels gives the same
+  if k % 16 == 0:
+    out8, _ = ops.decode(U.to_dev(x, dt, gpu), wq_t, torch.from_numpy(ws).to(gpu), quant_bound=127.5,
+                         clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], w_dtype=L.I4)
+    assert torch.equal(out, out8)
+
+
+@pytest.mark.parametrize('m', [20, 64])
+def test_decode_packed_int4_wide_weight(gpu, m):
+  """n >= 8192: each wave takes two 16-row weight blocks; n is not a multiple of 32."""
+  from aqt_amd import _lib as L
+  n, k = 8192 + 40, 160
+  x = U.rand((m, k), 'bf16', 6)
+  rng = np.random.default_rng(12)
+  wq = rng.integers(-7, 8, size=(n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(3e-3) + np.float32(1e-4), 'f32')
+  want, _, _ = _oracle_decode(x, 'bf16', wq, ws, 'f32')
+  out, _ = ops.decode(U.to_dev(x, 'bf16', gpu), ops.pack_i4(torch.from_numpy(wq).to(gpu)),
+                      torch.from_numpy(ws).to(gpu), quant_bound=127.5, clip_bound=127.0, w_dtype=L.I4P)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)

@@ -268,3 +268,24 @@ def test_mlp_block_fp32_full_size(gpu):
   np.testing.assert_array_equal(_np(W2.grad), dw2)
   np.testing.assert_array_equal(_np(W1.grad), dw1)
   np.testing.assert_array_equal(_np(X.grad), dx)
+
+
+@pytest.mark.parametrize('m', [1, 16, 40, 64, 100])
+@pytest.mark.parametrize('k', [512, 528])
+def test_serving_int4_weights(gpu, m, k):
+  """W4A8 serving: a frozen int4 rhs (held one value per byte in the QTensor).  With at most 64
+  rows and k a multiple of 32 the decode kernel streams a packed copy made once; k = 528 and
+  m = 100 take the int8-container kernels.  Same numbers either way."""
+  dt = 'bf16'
+  lhs, rhs = U.rand((m, k), dt, 1, outliers=True), U.rand((k, 384), dt, 2, 0.02)
+  cfg = config.set_context(aqt.dot_general_make(8, 4), None, None)
+  L, Rr = U.to_dev(lhs, dt, gpu), U.to_dev(rhs, dt, gpu)
+  out1, (_, rqt) = cfg.dg_core(L, Rr, None, None, MATMUL)
+  assert rqt.container_dtype is utils.int4
+  out2, (lqt, _) = cfg.dg_core(L, torch.zeros_like(Rr), None, rqt, MATMUL)
+  out3, _ = cfg.dg_core(L, torch.zeros_like(Rr), None, rqt, MATMUL)  # the cached packed copy
+  f = R.dg_fwd(lhs, rhs, dt, MATMUL, R.dot_general_make(8, 4))
+  np.testing.assert_array_equal(_np(out1), f.out)
+  np.testing.assert_array_equal(_np(out2), f.out)
+  np.testing.assert_array_equal(_np(out3), f.out)
+  np.testing.assert_array_equal(_np(lqt.qvalue), f.lhs_res.qx.qvalue.astype(np.float32))
