@@ -723,3 +723,43 @@ def tiled_dg_fwd(lhs, rhs, dt, tile_size, cfg: DgCfg):
   # jnp.sum over the tile axis in dtype dt: XLA accumulates bf16 sums in f32
   # and rounds once at the end.
   return nm.cast(_sum_leading(res.out), dt), res
+
+
+# ----------------------------------------------------------------------------
+# ragged_dot (aqt_ragged_dot.py:49-86): forward only.
+
+
+def lax_ragged_dot(lhs, rhs, group_sizes, out_np_dtype):
+  """jax.lax.ragged_dot: consecutive row groups of lhs [m, k] times rhs[g] [k, n]."""
+  m, n = lhs.shape[0], rhs.shape[2]
+  out = np.zeros((m, n), np.float64)
+  start = 0
+  for g, size in enumerate(group_sizes):
+    size = int(size)
+    out[start:start + size] = lhs[start:start + size].astype(np.float64) @ rhs[g].astype(np.float64)
+    start += size
+  if np.issubdtype(out_np_dtype, np.integer):
+    return np.rint(out).astype(out_np_dtype)
+  return out.astype(out_np_dtype)
+
+
+def ragged_dot_fwd(lhs, rhs, dt, group_sizes, raw: RawCfg):
+  """The fwd DotGeneralRaw with `dot_general = RaggedDot(group_sizes)` and
+  dimension_numbers ([1], [0, 1]), ([], []): the rhs scale is shared by all groups."""
+  dn = (((1,), (0, 1)), ((), ()))
+  lhs, rhs = nm.cast(lhs, dt), nm.cast(rhs, dt)
+  lqt = quantize(lhs, dt, raw.lhs, [1])
+  rqt = quantize(rhs, dt, raw.rhs, [0, 1])
+  acc = raw.accumulator()
+  if acc == 'i32':
+    out, odt = lax_ragged_dot(lqt.qvalue, rqt.qvalue, group_sizes, np.int32), 'i32'
+  else:
+    out, odt = nm.cast(lax_ragged_dot(lqt.qvalue, rqt.qvalue, group_sizes, np.float32), dt), dt
+  scales, sdts = [], []
+  for s in lqt.scale:
+    scales.append(lhs_scale_transpose_to_output(s, dn, lhs.shape, rhs.shape))
+    sdts.append(lqt.scale_dtype or dt)
+  for s in rqt.scale:
+    scales.append(rhs_scale_transpose_to_output(s, dn, lhs.shape, rhs.shape))
+    sdts.append(rqt.scale_dtype or dt)
+  return nm.cast(dequant(QTensor(out, odt, scales, None, dt, scale_dtypes=sdts or None)), dt), lqt, rqt
