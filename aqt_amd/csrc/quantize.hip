@@ -260,11 +260,54 @@ __device__ __forceinline__ float segment_max(float v, float* smem) {
   return v;
 }
 
+// Eight row values kept in registers between the abs-max pass and the quantize pass.  bf16
+// inputs of the specialised pipelines stay packed two per register (the prescaled value is
+// rounded to bf16 as well), which halves the registers a row costs and doubles the waves per SIMD.
+template <bool PACKED> struct RowVals;
+template <> struct RowVals<false> {
+  float f[8];
+  __device__ __forceinline__ void put(const float* t) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = t[e];
+  }
+  __device__ __forceinline__ void get(float* t) const {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) t[e] = f[e];
+  }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = 0.0f;
+  }
+};
+template <> struct RowVals<true> {
+  uint32_t w[4];
+  __device__ __forceinline__ void put(const float* t) {  // t[e] are bf16-representable
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = __builtin_amdgcn_perm(__float_as_uint(t[2 * i + 1]), __float_as_uint(t[2 * i]), 0x07060302u);
+  }
+  __device__ __forceinline__ void get(float* t) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      t[2 * i] = __uint_as_float(w[i] << 16);
+      t[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+    }
+  }
+  __device__ __forceinline__ void zero() { w[0] = w[1] = w[2] = w[3] = 0u; }
+};
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+// max of the two bf16 magnitudes of `w` against the running packed maxima: magnitudes of
+// floats order like unsigned integers
+__device__ __forceinline__ uint32_t packed_absmax(uint32_t m, uint32_t w) {
+  const u16x2_t a = __builtin_bit_cast(u16x2_t, m), b = __builtin_bit_cast(u16x2_t, w & 0x7FFF7FFFu);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+
 // ---- rows kernel: reduced axis contiguous -------------------------------------
 // PAIR (SPEC 2 only): the block owns segment s and segment s + nseg/2, whose elements share
 // threefry blocks; requires whole rows as segments and the natural noise layout.
 template <typename TIn, int LANES, int ITERS, int SPEC, bool PAIR>
-__global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
+__global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void quant_rows_kernel(const QArgs a) {
   constexpr int VEC = 8;
   constexpr int SEG_PER_BLOCK = 256 / LANES;
   constexpr int NSET = PAIR ? 2 : 1;
@@ -276,7 +319,8 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
   const bool active = seg0 < nseg_grid;
   const int64_t segs_per_row = a.cols / a.L;
 
-  float v[NSET][ITERS][VEC];
+  constexpr bool PACKED = (sizeof(TIn) == 2) && (SPEC != 0);
+  RowVals<PACKED> v[NSET][ITERS];
   float scale[NSET], inv[NSET];
   int64_t grow[NSET], col0[NSET];
 #pragma unroll
@@ -290,28 +334,44 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
     float row_ps = 1.0f;
     if (a.ps_mode == AQTX_PRESCALE_PER_ROW) row_ps = psv[r];
     float amax = 0.0f;
-#pragma unroll
+    uint32_t amax_packed = 0u;
+#pragma clang loop unroll(full)
     for (int it = 0; it < ITERS; ++it) {
       const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
       if (active && j0 < a.L) {
-        Loader<TIn>::load8(xp + j0, v[s][it]);
-        if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
+        bool stored = false;
+        if constexpr (PACKED) {
+          if (a.ps_mode == AQTX_PRESCALE_NONE) {  // the loaded words are the stored form
+            const uint4 raw = *reinterpret_cast<const uint4*>(xp + j0);
+            v[s][it].w[0] = raw.x; v[s][it].w[1] = raw.y; v[s][it].w[2] = raw.z; v[s][it].w[3] = raw.w;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) v[s][it][e] = spec_prescale<SPEC>(v[s][it][e], row_ps, a);
-        } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
-          const float4 p0 = *reinterpret_cast<const float4*>(psv + col0[s] + j0);
-          const float4 p1 = *reinterpret_cast<const float4*>(psv + col0[s] + j0 + 4);
-          const float ps[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) v[s][it][e] = spec_prescale<SPEC>(v[s][it][e], ps[e], a);
+            for (int i = 0; i < 4; ++i) amax_packed = packed_absmax(amax_packed, v[s][it].w[i]);
+            stored = true;
+          }
         }
+        if (!stored) {
+          float t[VEC];
+          Loader<TIn>::load8(xp + j0, t);
+          if (a.ps_mode == AQTX_PRESCALE_PER_ROW) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) amax = fmaxf(amax, fabsf(v[s][it][e]));
+            for (int e = 0; e < VEC; ++e) t[e] = spec_prescale<SPEC>(t[e], row_ps, a);
+          } else if (a.ps_mode == AQTX_PRESCALE_PER_COL) {
+            const float4 p0 = *reinterpret_cast<const float4*>(psv + col0[s] + j0);
+            const float4 p1 = *reinterpret_cast<const float4*>(psv + col0[s] + j0 + 4);
+            const float ps[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) t[e] = spec_prescale<SPEC>(t[e], ps[e], a);
+          }
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) amax = fmaxf(amax, fabsf(t[e]));
+          v[s][it].put(t);
+        }
       } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) v[s][it][e] = 0.0f;
+        v[s][it].zero();
       }
     }
+    if constexpr (PACKED)
+      amax = fmaxf(amax, fmaxf(__uint_as_float(amax_packed << 16), __uint_as_float(amax_packed & 0xFFFF0000u)));
     amax = segment_max<LANES>(amax, smem[s]);
     if (a.scale_given) {
       scale[s] = active ? a.scale[seg] : 1.0f;
@@ -326,15 +386,18 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
   if constexpr (PAIR) {
     uint8_t* qp1 = reinterpret_cast<uint8_t*>(a.q) + grow[1] * a.cols + col0[1];
     const uint32_t ctr_row = (uint32_t)(grow[0] * a.cols);  // natural layout: index of (row, 0)
-#pragma unroll
+#pragma clang loop unroll(full)
     for (int it = 0; it < ITERS; ++it) {
       const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
       if (active && j0 < a.L) {
         uint32_t w0[2] = {0u, 0u}, w1[2] = {0u, 0u};
+        float t0[VEC], t1[VEC];
+        v[0][it].get(t0);
+        v[1][it].get(t1);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           uint32_t q0, q1;
-          pair_quant(v[0][it][e], inv[0], v[1][it][e], inv[1], ctr_row + (uint32_t)(j0 + e), a, q0, q1);
+          pair_quant(t0[e], inv[0], t1[e], inv[1], ctr_row + (uint32_t)(j0 + e), a, q0, q1);
           w0[e >> 2] |= q0 << (8 * (e & 3));
           w1[e >> 2] |= q1 << (8 * (e & 3));
         }
@@ -345,14 +408,16 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const QArgs a) {
   } else {
     const int64_t b = grow[0] / a.rows, r = grow[0] % a.rows;
     const uint64_t ctr_row = (uint64_t)(b * a.nsb + r * a.nsr + col0[0] * a.nsc);
-#pragma unroll
+#pragma clang loop unroll(full)
     for (int it = 0; it < ITERS; ++it) {
       const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
       if (active && j0 < a.L) {
         uint32_t w[2] = {0u, 0u};
+        float t[VEC];
+        v[0][it].get(t);
 #pragma unroll
         for (int e = 0; e < VEC; ++e)
-          w[e >> 2] |= spec_quant<SPEC>(v[0][it][e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a)
+          w[e >> 2] |= spec_quant<SPEC>(t[e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a)
                        << (8 * (e & 3));
         *reinterpret_cast<uint2*>(qp0 + j0) = make_uint2(w[0], w[1]);
       }
