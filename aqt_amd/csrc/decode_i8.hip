@@ -33,21 +33,30 @@ struct DecodeArgs {
   int m, n, k;
   int out_bf16, xs_bf16, ws_bf16;
   int acc_shift;  // 4 when the weight operand holds 16 * w (unpacked nibbles), else 0
+  // the fused kernel quantizes the activations itself
+  const void* x;          // [m][k] bf16 or f32
+  int8_t* xq_out;         // optional [m][k]
+  float* x_scale_out;     // [m]
+  float quant_bound, clip_bound;
+  int x_bf16;
 };
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
 
 // QTensor.dequant: cast the accumulator, multiply by the lhs scale, then the rhs scale, each
 // product in the promoted dtype of its operands, final cast.
-__device__ __forceinline__ void store_out(const DecodeArgs& d, int mm, int nn, int acc) {
+__device__ __forceinline__ void store_out_scaled(const DecodeArgs& d, int mm, int nn, int acc, float xs) {
   float f = rnd((float)(acc >> d.acc_shift), d.out_bf16);  // exact: acc is a multiple of 16 then
   const int p1 = d.out_bf16 & d.xs_bf16;
-  f = rnd(f * d.x_scale[mm], p1);
+  f = rnd(f * xs, p1);
   f = rnd(f * d.w_scale[nn], p1 & d.ws_bf16);
   f = rnd(f, d.out_bf16);
   const int64_t o = (int64_t)mm * d.n + nn;
   if (d.out_bf16) reinterpret_cast<uint16_t*>(d.out)[o] = bf16_bits(f);
   else reinterpret_cast<float*>(d.out)[o] = f;
+}
+__device__ __forceinline__ void store_out(const DecodeArgs& d, int mm, int nn, int acc) {
+  store_out_scaled(d, mm, nn, acc, d.x_scale[mm]);
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
@@ -115,6 +124,152 @@ __global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) 
       const int s = red[0][mm][tid & 15] + red[1][mm][tid & 15] + red[2][mm][tid & 15] + red[3][mm][tid & 15];
       store_out(d, mm, nn, s);
     }
+  }
+}
+
+// ---- few rows: activation quantisation inside the contraction kernel ------------------------------
+// For a handful of tokens the separate quantize launch costs as much as a third of the call.
+// Here every workgroup quantizes the activations itself (they come from L2: ROWS * k values),
+// keeps the int8 rows in LDS and multiplies them with its 16 weight rows as the K-split kernel
+// does.  The first batch of weight loads is issued before the quantisation so that HBM latency
+// overlaps it.  Same arithmetic as the row kernel of aqtx_quantize: abs-max over the row,
+// scale = dtype(absmax / bound), inv = dtype(1 / scale), q = rint(clip(dtype(x * inv))).
+// Workgroup 0 also writes the scales and, when asked, the quantized activations.
+// LDS rows are k rounded up to 256 bytes long; the 16-byte piece j of row i sits at piece
+// j ^ (i & 15) of its 16-piece group, so the 16 lanes of a fragment read hit all 64 banks.
+template <typename TIn, int ROWS, int PPT, int U>  // PPT: 16-value pieces of one row per thread
+__global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t xlds[];  // [ROWS][kp]
+  __shared__ float smax[ROWS][4];
+  __shared__ float sscale[ROWS];
+  __shared__ int red[4][16][16];
+  constexpr bool XBF = sizeof(TIn) == 2;
+  constexpr int WPP = XBF ? 8 : 16;  // 32-bit words of one 16-value input piece
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);
+  const int kp = (d.k + 255) / 256 * 256;
+  const int pieces = d.k / 16;
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
+  const int kq = ((d.k + 3) / 4 + 63) / 64 * 64;
+  const int k_lo = wave * kq;
+  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
+  const int wbase = nrow * d.k + c * 16;
+
+  // first batch of weights: in flight while the activations are quantized
+  v4i wf[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int ko = k_lo + u * 64;
+    wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < k_hi) ? wbase + ko : kOob, 0, 0);
+  }
+
+  // ---- quantize the activations into LDS
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.x, (int64_t)d.m * d.k * (int64_t)sizeof(TIn));
+  uint32_t raw[ROWS][PPT][WPP];
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int p = tid + 256 * j;
+      const bool ok = i < d.m && p < pieces;
+      const int off = ok ? (i * d.k + p * 16) * (int)sizeof(TIn) : kOob;  // out of range reads give 0
+#pragma unroll
+      for (int q = 0; q < WPP / 4; ++q) {
+        const v4i t = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? off + 16 * q : kOob, 0, 0);
+        raw[i][j][4 * q + 0] = (uint32_t)t[0]; raw[i][j][4 * q + 1] = (uint32_t)t[1];
+        raw[i][j][4 * q + 2] = (uint32_t)t[2]; raw[i][j][4 * q + 3] = (uint32_t)t[3];
+      }
+    }
+  auto value = [&](int i, int j, int e) -> float {
+    if constexpr (XBF) {
+      const uint32_t w = raw[i][j][e >> 1];
+      return __uint_as_float((e & 1) ? (w & 0xFFFF0000u) : (w << 16));
+    } else {
+      return __uint_as_float(raw[i][j][e]);
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PPT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(value(i, j, e)));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    if (lane == 0) smax[i][wave] = amax;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    float amax = fmaxf(fmaxf(smax[i][0], smax[i][1]), fmaxf(smax[i][2], smax[i][3]));
+    if (amax == 0.0f) amax = 1.0f;
+    float sc = rnd(amax / d.quant_bound, d.x_bf16);
+    sc = rnd(sc, d.xs_bf16);
+    float inv = rnd(1.0f / sc, d.xs_bf16);
+    if (isinf(inv)) inv = 1.0f;
+    if (tid == 0) {
+      sscale[i] = sc;
+      if (blockIdx.x == 0 && i < d.m) d.x_scale_out[i] = sc;
+    }
+    const int tbf = d.x_bf16 & d.xs_bf16;
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int p = tid + 256 * j;
+      uint32_t q[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        float t = rnd(value(i, j, e) * inv, tbf);
+        t = fminf(fmaxf(t, -d.clip_bound), d.clip_bound);
+        q[e >> 2] |= ((uint32_t)((int)rintf(t)) & 0xFFu) << (8 * (e & 3));
+      }
+      if (p < pieces) {
+        const int ps = (p & ~15) | ((p & 15) ^ (i & 15));
+        *reinterpret_cast<uint4*>(xlds + (size_t)i * kp + ps * 16) = make_uint4(q[0], q[1], q[2], q[3]);
+        if (blockIdx.x == 0 && d.xq_out != nullptr && i < d.m)
+          *reinterpret_cast<uint4*>(d.xq_out + (size_t)i * d.k + p * 16) = make_uint4(q[0], q[1], q[2], q[3]);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- contraction, weights from HBM, activations from LDS
+  v4i acc = v4i{0, 0, 0, 0};
+  const bool row_ok = r < ROWS && r < d.m;
+  for (int kk = k_lo; kk < k_hi; kk += 64 * U) {
+    if (kk != k_lo) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int ko = kk + u * 64;
+        wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < k_hi) ? wbase + ko : kOob, 0, 0);
+      }
+    }
+    v4i xf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int pj = (kk + u * 64) / 16 + c;
+      xf[u] = v4i{0, 0, 0, 0};
+      if (row_ok && pj < pieces) {
+        const int ps = (pj & ~15) | ((pj & 15) ^ r);
+        xf[u] = *reinterpret_cast<const v4i*>(xlds + (size_t)r * kp + ps * 16);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u], wf[u], acc, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) red[wave][4 * c + e][r] = acc[e];
+  __syncthreads();
+  const int mm = tid >> 4, nn = n0 + (tid & 15);
+  if (mm < d.m && nn < d.n) {
+    const int sum = red[0][mm][tid & 15] + red[1][mm][tid & 15] + red[2][mm][tid & 15] + red[3][mm][tid & 15];
+    store_out_scaled(d, mm, nn, sum, sscale[mm]);
   }
 }
 
@@ -400,6 +555,44 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
                "aqtx_decode_i8: w, xq and the workspace must be 16-byte aligned");
   int8_t* xq_buf = reinterpret_cast<int8_t*>(xq != nullptr ? xq : workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+
+  // 0. a handful of tokens: one kernel quantizes and contracts (AQTX_DECODE_FUSED=0 turns it off)
+  {
+    const bool xbf = p->x_dtype == AQTX_BF16;
+    const int ppt = p->k <= 4096 ? 1 : 2;
+    // Every workgroup repeats the quantisation, so its cost grows with the rows while the launch
+    // it saves does not: measured at k = 4096, one row gains 2.5 us per call, two rows 1 us,
+    // three rows lose.
+    const int64_t max_rows = 2;
+    const char* fused_env = getenv("AQTX_DECODE_FUSED");
+    const bool fused_off = fused_env != nullptr && fused_env[0] == '0';
+    if (!fused_off && p->w_dtype != AQTX_I4P && p->k <= 8192 && p->m <= max_rows && ((uintptr_t)x % 16) == 0) {
+      DecodeArgs d{};
+      d.w = reinterpret_cast<const int8_t*>(w);
+      d.w_scale = w_scale; d.out = out;
+      d.m = (int)p->m; d.n = (int)p->n; d.k = (int)p->k;
+      d.out_bf16 = p->out_dtype == AQTX_BF16;
+      d.xs_bf16 = p->x_scale_dtype == AQTX_BF16;
+      d.ws_bf16 = p->w_scale_dtype == AQTX_BF16;
+      d.x = x; d.xq_out = reinterpret_cast<int8_t*>(xq); d.x_scale_out = x_scale;
+      d.quant_bound = p->quant_bound; d.clip_bound = p->clip_bound; d.x_bf16 = xbf;
+      const unsigned grid = (unsigned)((p->n + 15) / 16);
+      const int rows = (int)p->m;
+      const size_t lds = (size_t)rows * (size_t)((p->k + 255) / 256 * 256);
+#define AQTX_FUSED(T, R, P)                                                   \
+  decode_fused_kernel<T, R, P, 16><<<grid, 256, lds, st>>>(d);
+      if (xbf) {
+        if (ppt == 1) { if (rows == 1) AQTX_FUSED(uint16_t, 1, 1) else AQTX_FUSED(uint16_t, 2, 1) }
+        else { if (rows == 1) AQTX_FUSED(uint16_t, 1, 2) else AQTX_FUSED(uint16_t, 2, 2) }
+      } else {
+        if (ppt == 1) { if (rows == 1) AQTX_FUSED(float, 1, 1) else AQTX_FUSED(float, 2, 1) }
+        else { if (rows == 1) AQTX_FUSED(float, 1, 2) else AQTX_FUSED(float, 2, 2) }
+      }
+#undef AQTX_FUSED
+      AQTX_HIP_CHECK_LAUNCH("decode_fused_kernel");
+      return 0;
+    }
+  }
 
   // 1. per-token dynamic quantization of the activations (same kernel as training)
   aqtx_quant_plan q{};

@@ -29,7 +29,7 @@ def _weights(n, k, seed, w_sdt):
   return wq, ws
 
 
-@pytest.mark.parametrize('m', [1, 3, 8, 16, 17, 32, 40, 64])
+@pytest.mark.parametrize('m', [1, 2, 3, 8, 16, 17, 32, 40, 64])
 @pytest.mark.parametrize('n,k', [(256, 1024), (200, 464), (4096, 4096)])
 @pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('bf16', 'bf16'), ('f32', 'f32')])
 def test_decode_matches_oracle(gpu, m, n, k, dt, w_sdt):
@@ -124,3 +124,24 @@ def test_decode_packed_int4_wide_weight(gpu, m):
   out, _ = ops.decode(U.to_dev(x, 'bf16', gpu), ops.pack_i4(torch.from_numpy(wq).to(gpu)),
                       torch.from_numpy(ws).to(gpu), quant_bound=127.5, clip_bound=127.0, w_dtype=L.I4P)
   np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize('m', [1, 2])
+@pytest.mark.parametrize('k', [4112, 8192, 8208])
+@pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('f32', 'f32'), ('bf16', 'bf16')])
+def test_decode_one_or_two_rows_long_k(gpu, m, k, dt, w_sdt):
+  """One or two tokens take the kernel that quantizes the activations itself; above k = 4096
+  each thread holds two pieces per row, above 8192 the two-kernel path runs.  The quantized
+  activations and scales it writes out are the oracle's."""
+  n = 72
+  x = U.rand((m, k), dt, 300 + m, outliers=True)
+  wq, ws = _weights(n, k, 8, w_sdt)
+  want, xq_want, xs_want = _oracle_decode(x, dt, wq, ws, w_sdt)
+  out, xs, xq = ops.decode(U.to_dev(x, dt, gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
+                           quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True)
+  np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
+  np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+  out2, _ = ops.decode(U.to_dev(x, dt, gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
+                       quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt])
+  assert torch.equal(out, out2)
