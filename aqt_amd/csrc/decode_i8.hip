@@ -127,6 +127,14 @@ __global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) 
   }
 }
 
+// A word of eight packed int4 (low nibble = even k) -> two words of int8 holding 16 * value.
+__device__ __forceinline__ void unpack_i4x8(uint32_t w, int& lo, int& hi) {
+  const uint32_t ev = (w << 4) & 0xF0F0F0F0u;  // k0 k2 k4 k6
+  const uint32_t od = w & 0xF0F0F0F0u;         // k1 k3 k5 k7
+  lo = (int)__builtin_amdgcn_perm(od, ev, 0x05010400u);  // k0 k1 k2 k3
+  hi = (int)__builtin_amdgcn_perm(od, ev, 0x07030602u);  // k4 k5 k6 k7
+}
+
 // ---- few rows: activation quantisation inside the contraction kernel ------------------------------
 // For a handful of tokens the separate quantize launch costs as much as a third of the call.
 // Here every workgroup quantizes the activations itself (they come from L2: ROWS * k values),
@@ -137,7 +145,8 @@ __global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) 
 // Workgroup 0 also writes the scales and, when asked, the quantized activations.
 // LDS rows are k rounded up to 256 bytes long; the 16-byte piece j of row i sits at piece
 // j ^ (i & 15) of its 16-piece group, so the 16 lanes of a fragment read hit all 64 banks.
-template <typename TIn, int ROWS, int PPT, int U>  // PPT: 16-value pieces of one row per thread
+// PACKED: int4 weights two per byte; a lane's 16 bytes are then 32 k, i.e. two MFMA steps.
+template <typename TIn, int ROWS, int PPT, int U, bool PACKED>  // PPT: 16-value pieces of one row per thread
 __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xlds[];  // [ROWS][kp]
   __shared__ float smax[ROWS][4];
@@ -153,19 +162,20 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   const int kp = (d.k + 255) / 256 * 256;
   const int pieces = d.k / 16;
 
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
-  const int kq = ((d.k + 3) / 4 + 63) / 64 * 64;
+  constexpr int KS = PACKED ? 128 : 64;   // k covered by one wave-wide weight load
+  constexpr int KL = KS / 4;              // k covered by one lane's 16 bytes
+  const int kb = PACKED ? d.k / 2 : d.k;  // bytes of one weight row
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * kb);
+  const int kq = ((d.k + 3) / 4 + KS - 1) / KS * KS;
   const int k_lo = wave * kq;
   const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
-  const int wbase = nrow * d.k + c * 16;
+  const int wbase = nrow * kb + c * 16;
+  auto w_offset = [&](int ko) { return (ko + c * KL < k_hi) ? wbase + (PACKED ? ko / 2 : ko) : kOob; };
 
   // first batch of weights: in flight while the activations are quantized
   v4i wf[U];
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int ko = k_lo + u * 64;
-    wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < k_hi) ? wbase + ko : kOob, 0, 0);
-  }
+  for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
 
   // ---- quantize the activations into LDS
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.x, (int64_t)d.m * d.k * (int64_t)sizeof(TIn));
@@ -240,27 +250,37 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   // ---- contraction, weights from HBM, activations from LDS
   v4i acc = v4i{0, 0, 0, 0};
   const bool row_ok = r < ROWS && r < d.m;
-  for (int kk = k_lo; kk < k_hi; kk += 64 * U) {
+  constexpr int XP = PACKED ? 2 : 1;  // activation pieces per weight load
+  for (int kk = k_lo; kk < k_hi; kk += KS * U) {
     if (kk != k_lo) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int ko = kk + u * 64;
-        wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < k_hi) ? wbase + ko : kOob, 0, 0);
-      }
+      for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, 0);
     }
-    v4i xf[U];
+    v4i xf[U][XP];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int pj = (kk + u * 64) / 16 + c;
-      xf[u] = v4i{0, 0, 0, 0};
-      if (row_ok && pj < pieces) {
-        const int ps = (pj & ~15) | ((pj & 15) ^ r);
-        xf[u] = *reinterpret_cast<const v4i*>(xlds + (size_t)r * kp + ps * 16);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int h = 0; h < XP; ++h) {
+        const int pj = (kk + u * KS) / 16 + c * XP + h;
+        xf[u][h] = v4i{0, 0, 0, 0};
+        if (row_ok && pj < pieces) {
+          const int ps = (pj & ~15) | ((pj & 15) ^ r);
+          xf[u][h] = *reinterpret_cast<const v4i*>(xlds + (size_t)r * kp + ps * 16);
+        }
       }
-    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int u = 0; u < U; ++u) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u], wf[u], acc, 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      if constexpr (PACKED) {
+        int t[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[u][j], t[2 * j], t[2 * j + 1]);
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], v4i{t[0], t[1], t[2], t[3]}, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][1], v4i{t[4], t[5], t[6], t[7]}, acc, 0, 0, 0);
+      } else {
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], wf[u], acc, 0, 0, 0);
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
@@ -279,12 +299,6 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
 // operands.  A nibble is moved to the top of its byte, which makes it 16 * w as a signed int8;
 // the factor leaves the accumulator as an exact right shift by 4.  Same workgroup shape as the
 // K-split kernel (weights stream from HBM once; half the bytes of the int8 form).
-__device__ __forceinline__ void unpack_i4x8(uint32_t w, int& lo, int& hi) {
-  const uint32_t ev = (w << 4) & 0xF0F0F0F0u;  // k0 k2 k4 k6
-  const uint32_t od = w & 0xF0F0F0F0u;         // k1 k3 k5 k7
-  lo = (int)__builtin_amdgcn_perm(od, ev, 0x05010400u);  // k0 k1 k2 k3
-  hi = (int)__builtin_amdgcn_perm(od, ev, 0x07030602u);  // k4 k5 k6 k7
-}
 
 // NB: 16-row weight blocks per wave; every activation fragment a wave loads is used NB times,
 // so the L2 traffic for the activations is MB / NB times the int8-equivalent weight bytes.
@@ -566,7 +580,8 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
     const int64_t max_rows = 2;
     const char* fused_env = getenv("AQTX_DECODE_FUSED");
     const bool fused_off = fused_env != nullptr && fused_env[0] == '0';
-    if (!fused_off && p->w_dtype != AQTX_I4P && p->k <= 8192 && p->m <= max_rows && ((uintptr_t)x % 16) == 0) {
+    if (!fused_off && p->k <= 8192 && p->m <= max_rows && ((uintptr_t)x % 16) == 0) {
+      const bool pk = p->w_dtype == AQTX_I4P;
       DecodeArgs d{};
       d.w = reinterpret_cast<const int8_t*>(w);
       d.w_scale = w_scale; d.out = out;
@@ -579,14 +594,16 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
       const unsigned grid = (unsigned)((p->n + 15) / 16);
       const int rows = (int)p->m;
       const size_t lds = (size_t)rows * (size_t)((p->k + 255) / 256 * 256);
+      d.acc_shift = pk ? 4 : 0;
 #define AQTX_FUSED(T, R, P)                                                   \
-  decode_fused_kernel<T, R, P, 16><<<grid, 256, lds, st>>>(d);
+  if (pk) decode_fused_kernel<T, R, P, 8, true><<<grid, 256, lds, st>>>(d);  \
+  else decode_fused_kernel<T, R, P, 16, false><<<grid, 256, lds, st>>>(d);
       if (xbf) {
-        if (ppt == 1) { if (rows == 1) AQTX_FUSED(uint16_t, 1, 1) else AQTX_FUSED(uint16_t, 2, 1) }
-        else { if (rows == 1) AQTX_FUSED(uint16_t, 1, 2) else AQTX_FUSED(uint16_t, 2, 2) }
+        if (ppt == 1) { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 1) } else { AQTX_FUSED(uint16_t, 2, 1) } }
+        else { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 2) } else { AQTX_FUSED(uint16_t, 2, 2) } }
       } else {
-        if (ppt == 1) { if (rows == 1) AQTX_FUSED(float, 1, 1) else AQTX_FUSED(float, 2, 1) }
-        else { if (rows == 1) AQTX_FUSED(float, 1, 2) else AQTX_FUSED(float, 2, 2) }
+        if (ppt == 1) { if (rows == 1) { AQTX_FUSED(float, 1, 1) } else { AQTX_FUSED(float, 2, 1) } }
+        else { if (rows == 1) { AQTX_FUSED(float, 1, 2) } else { AQTX_FUSED(float, 2, 2) } }
       }
 #undef AQTX_FUSED
       AQTX_HIP_CHECK_LAUNCH("decode_fused_kernel");

@@ -82,8 +82,8 @@ def test_decode_rejects_bad_plans(gpu):
     ops.decode(x[:4, :24].contiguous(), w[:, :24].contiguous(), s, quant_bound=127.5, clip_bound=127.0)
 
 
-@pytest.mark.parametrize('m', [1, 8, 16, 17, 32, 33, 64])
-@pytest.mark.parametrize('n,k', [(256, 1024), (200, 480), (40, 32), (4096, 4096)])
+@pytest.mark.parametrize('m', [1, 2, 8, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize('n,k', [(256, 1024), (200, 480), (40, 32), (4096, 4096), (72, 8192)])
 @pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('bf16', 'bf16'), ('f32', 'f32')])
 def test_decode_packed_int4_matches_oracle(gpu, m, n, k, dt, w_sdt):
   """int4 weights packed two per byte (aqtx_pack_i4 layout): same numbers as the int8-held
