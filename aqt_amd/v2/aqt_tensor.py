@@ -47,6 +47,15 @@ class QTensor:
   def replace(self, **kw):
     return dataclasses.replace(self, **kw)
 
+  def _validate_tiling_state(self):
+    """aqt_tensor.py:103-113."""
+    if self.tiling_state is None:
+      return
+    if self.is_full():
+      assert tuple(self.qvalue.shape) == tuple(self.tiling_state.tiled_shape), (
+          'The shape of the qvalue should be the same as the tiled shape of the tiling state. '
+          f'However, {tuple(self.qvalue.shape)=} and {self.tiling_state.tiled_shape=}')
+
   def is_full(self) -> bool:
     return self.qvalue is not None
 
@@ -86,6 +95,7 @@ class QTensor:
            'dot_general, but to dequantize you need to set its dtype.')
     assert self.dequant_dtype is not None, msg
     assert self.is_full(), _MSG_NO_QVALUE
+    self._validate_tiling_state()
     q = self.qvalue
     kernel_types = (torch.int8, torch.float8_e4m3fn, torch.float8_e5m2)
     if (len(self.scale) != 1 or self.bias or self.sparsity_mask is not None
@@ -132,6 +142,7 @@ class QTensor:
   def __getitem__(self, idx):
     assert self.scale_t is None, 'scale_t is not supported in __getitem__'
     assert self.is_full(), _MSG_NO_QVALUE
+    self._validate_tiling_state()
     return QTensor(qvalue=self.qvalue[idx], scale=[s[idx] for s in self.scale], scale_t=self.scale_t,
                    bias=self.bias, dequant_dtype=self.dequant_dtype,
                    container_dtype=self.container_dtype)
@@ -139,11 +150,17 @@ class QTensor:
   @property
   def ndim(self) -> int:
     assert self.is_full(), _MSG_NO_QVALUE
+    self._validate_tiling_state()
+    if self.tiling_state is not None:
+      return len(self.tiling_state.untiled_shape)
     return self.qvalue.dim()
 
   @property
   def shape(self) -> Sequence[int]:
     assert self.is_full(), _MSG_NO_QVALUE
+    self._validate_tiling_state()
+    if self.tiling_state is not None:
+      return tuple(self.tiling_state.untiled_shape)
     return tuple(self.qvalue.shape)
 
   def __len__(self) -> int:

@@ -420,3 +420,40 @@ def test_snr_based_auto_calibration(gpu, bits, dt):
   ratio = _np(rqt.scale[0])[0] / (np.abs(w).max(axis=0) / R.quant_bound(oraw.rhs))
   if bits == 4:  # coarse steps: clipping the outlier pays
     assert (ratio[::2] < 0.75).all() and len(set(np.round(ratio, 3))) > 1
+
+
+def test_qtensor_with_tiling_state(gpu):
+  """aqt_tensor_test.py:122-204: a QTensor quantized through a tiling state reports the
+  untiled shape, holds the tiled qvalue, dequantizes back to the untiled shape, and refuses a
+  tiling state that does not match its qvalue."""
+  from aqt_amd.v2 import aqt_tensor
+  from aqt_amd.v2 import tiled_dot_general as T
+  rng = np.random.default_rng(0)
+  lhs = torch.from_numpy(rng.integers(0, 100, (30, 40, 50)).astype(np.float32)).to(gpu)
+  rhs = torch.from_numpy(rng.integers(0, 100, (40, 50, 60)).astype(np.float32)).to(gpu)
+  cfg = T.Cfg(
+      lhs=T.TensorTiling(contraction_axes=[T.AxisTiling(axis=1, tile_size=10), T.AxisTiling(axis=2, tile_size=25)],
+                         remaining_axes=[]),
+      rhs=T.TensorTiling(contraction_axes=[T.AxisTiling(axis=0, tile_size=10), T.AxisTiling(axis=1, tile_size=25)],
+                         remaining_axes=[]))
+  lhs_ca, rhs_ca = (1, 2), (0, 1)
+  xlhs, xrhs = T.generate_tiling_states_for_dot_general(cfg, lhs, rhs, ((lhs_ca, rhs_ca), ((), ())))
+  qts = []
+  for x, st, ca in ((lhs, xlhs, lhs_ca), (rhs, xrhs, rhs_ca)):
+    _, tca = st.to_tiled_axes_transposed(ca)
+    scale = torch.amax(st.apply(x), dim=list(tca), keepdim=True) / (2.0 ** 7 - 1)
+    qt = aqt_tensor.QTensor(qvalue=None, scale=[scale], scale_t=None, bias=[], dequant_dtype=scale.dtype,
+                            tiling_state=st)
+    qt = qt.quant(x)
+    assert qt.shape == tuple(x.shape) and qt.ndim == x.dim()
+    assert tuple(qt.qvalue.shape) == tuple(st.tiled_shape)
+    deq = qt.dequant()
+    assert tuple(deq.shape) == tuple(x.shape)
+    np.testing.assert_allclose(_np(deq), _np(x), rtol=1e-6)  # no rounding in QTensor.quant
+    qts.append(qt)
+  qlhs, qrhs = qts
+  qlhs.tiling_state.tiled_shape = tuple(qrhs.qvalue.shape)
+  with pytest.raises(AssertionError):
+    qlhs.dequant()
+  with pytest.raises(AssertionError):
+    qlhs.shape  # pylint: disable=pointless-statement
