@@ -31,6 +31,8 @@ class QuantPlan(ctypes.Structure):
       ('noise_stride_col', ctypes.c_int64), ('noise_total', ctypes.c_int64),
       ('prescale', ctypes.c_int32), ('scale_given', ctypes.c_int32),
       ('prescale_stride_batch', ctypes.c_int64),
+      ('scale_typed', ctypes.c_void_p),
+      ('workspace_zeroed', ctypes.c_int32),
   ]
 
 

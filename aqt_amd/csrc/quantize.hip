@@ -29,6 +29,7 @@ struct QArgs {
   const float* prescale;
   void* q;
   float* scale;
+  uint16_t* scale_bf16;  // optional second copy of the computed scales as bf16 elements
   uint32_t* ws_absmax;
   float* ws_inv;
   int64_t batch, rows, cols;
@@ -48,7 +49,15 @@ struct QArgs {
   int cbf;  // compute dtype is bf16
   int sbf;  // scale dtype is bf16
   int scale_given;
+  int ws_zeroed;  // the abs-max words of the workspace are zero on entry
 };
+
+// The computed scale goes out as float32 and, when the caller keeps its scales in bf16, once
+// more as bf16 elements (the value is already rounded to bf16, so the narrowing is exact).
+__device__ __forceinline__ void store_scale(const QArgs& a, int64_t i, float v) {
+  a.scale[i] = v;
+  if (a.scale_bf16 != nullptr) a.scale_bf16[i] = (uint16_t)(__float_as_uint(v) >> 16);
+}
 
 // ---- typed vector loads ------------------------------------------------------
 template <typename T> struct Loader;
@@ -378,7 +387,7 @@ __global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void 
       inv[s] = inv_of_scale(scale[s], a);
     } else {
       spec_scale_from_absmax<SPEC>(amax, a, scale[s], inv[s]);
-      if (active && lane == 0) a.scale[seg] = scale[s];
+      if (active && lane == 0) store_scale(a, seg, scale[s]);
     }
   }
 
@@ -451,7 +460,7 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const QArgs a) 
     inv = inv_of_scale(scale, a);
   } else {
     scale_from_absmax(amax, a, scale, inv);
-    if (lane == 0) a.scale[seg] = scale;
+    if (lane == 0) store_scale(a, seg, scale);
   }
   uint8_t* qp = reinterpret_cast<uint8_t*>(a.q) + grow * a.cols + col0;
   const uint64_t ctr_row = (uint64_t)(b * a.nsb + r * a.nsr + col0 * a.nsc);
@@ -576,7 +585,8 @@ __global__ void finalize_scales_kernel(const QArgs a, int64_t n) {
     inv = inv_of_scale(scale, a);
   } else {
     scale_from_absmax(__uint_as_float(a.ws_absmax[i]), a, scale, inv);
-    a.scale[i] = scale;
+    a.ws_absmax[i] = 0u;  // the abs-max words leave as they have to arrive: zero
+    store_scale(a, i, scale);
   }
   a.ws_inv[i] = inv;
 }
@@ -922,8 +932,10 @@ int launch_rows(const QArgs& a, int partitionable, hipStream_t st) {
 template <typename TIn>
 int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales, hipStream_t st) {
   if (!a.scale_given) {
-    fill_u32_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a.ws_absmax, nscales, 0u);
-    AQTX_HIP_CHECK_LAUNCH("fill_u32_kernel");
+    if (!a.ws_zeroed) {
+      fill_u32_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a.ws_absmax, nscales, 0u);
+      AQTX_HIP_CHECK_LAUNCH("fill_u32_kernel");
+    }
     if (reduce == AQTX_REDUCE_ALL || reduce == AQTX_REDUCE_ALL_BATCH) {
       int64_t nblk = (a.rows * a.cols + 256 * 16 - 1) / (256 * 16);
       if (nblk > 2048) nblk = 2048;
@@ -1018,6 +1030,8 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
   const int64_t nscales = scale_count(p);
   QArgs a{};
   a.x = x; a.prescale = prescale; a.q = q; a.scale = scale;
+  a.scale_bf16 = (p->scale_typed != nullptr && p->scale_dtype == AQTX_BF16 && !p->scale_given)
+                     ? reinterpret_cast<uint16_t*>(p->scale_typed) : nullptr;
   a.batch = p->batch; a.rows = p->rows; a.cols = p->cols;
   a.nsb = p->noise_stride_batch; a.nsr = p->noise_stride_row; a.nsc = p->noise_stride_col;
   a.quant_bound = p->quant_bound; a.clip_bound = p->clip_bound;
@@ -1025,6 +1039,7 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
   a.transpose_out = p->transpose_out; a.out_dtype = p->out_dtype;
   a.cbf = p->compute_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
   a.scale_given = p->scale_given;
+  a.ws_zeroed = p->workspace_zeroed;
   if (p->noise != AQTX_NOISE_NONE)
     a.gen = make_bitgen(p->key, p->noise_total, noise_width(p), p->partitionable);
   if (p->reduce == AQTX_REDUCE_COLS) {
@@ -1032,7 +1047,10 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
     a.nseg = nscales;
   } else {
     a.ws_absmax = reinterpret_cast<uint32_t*>(workspace);
-    a.ws_inv = reinterpret_cast<float*>(workspace) + nscales;
+    // A workspace kept across calls holds the abs-max words (zero between calls) in its first
+    // half and the reciprocal scales in its second, whatever the number of scales of a call.
+    a.ws_inv = reinterpret_cast<float*>(workspace) +
+               (p->workspace_zeroed ? (int64_t)(workspace_bytes / 8) : nscales);
     if (p->reduce == AQTX_REDUCE_ROWS) {
       a.G = p->group ? p->group : p->rows;
       a.ngroups = p->rows / a.G;

@@ -89,6 +89,20 @@ def _require_gpu(*tensors):
                          'there is no CPU fallback')
 
 
+# One abs-max workspace per (device, stream), kept zeroed by the library between calls, so that
+# the column and whole-tensor calibrations do not pay a clearing launch each time.
+_QUANT_WS = {}
+
+
+def _quantize_workspace(nbytes: int, device) -> torch.Tensor:
+  key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+  ws = _QUANT_WS.get(key)
+  if ws is None or ws.numel() < nbytes:
+    ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+    _QUANT_WS[key] = ws
+  return ws
+
+
 def quantize(
     x: torch.Tensor,
     *,
@@ -108,6 +122,7 @@ def quantize(
     prescale: Optional[torch.Tensor] = None,
     prescale_mode: int = L.PRESCALE_NONE,
     scale: Optional[torch.Tensor] = None,
+    want_typed_scale: bool = False,
 ):
   """Calibrate (abs-max) and quantize a contiguous [batch, rows, cols] tensor.
 
@@ -115,6 +130,9 @@ def quantize(
   [batch, rows, cols] or [batch, cols, rows] with transpose_out; scale is
   float32, shaped [batch, rows, cols/group] (REDUCE_COLS),
   [batch, rows/group, cols] (REDUCE_ROWS) or [batch] (REDUCE_ALL).
+  With want_typed_scale a third element: the computed scales once more as a bf16 tensor of
+  the same shape, written by the same kernels (None unless the scale dtype is bf16 and the
+  scale is computed here).
   """
   _require_gpu(x, prescale, scale)
   assert x.dim() == 3 and x.is_contiguous(), 'x must be a contiguous [batch, rows, cols] tensor'
@@ -147,8 +165,12 @@ def quantize(
     sshape = (b,)
   else:
     sshape = (1,)
+  typed = None
   if scale is None:
     scale = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    if want_typed_scale and scale_dt == L.BF16:
+      typed = torch.empty(sshape, dtype=torch.bfloat16, device=x.device)
+      plan.scale_typed = typed.data_ptr()
   else:
     assert scale.dtype == torch.float32 and scale.is_contiguous() and tuple(scale.shape) == sshape
   fp8 = out_dtype in (L.E4M3, L.E5M2)
@@ -158,10 +180,15 @@ def quantize(
     assert prescale.dtype == torch.float32 and prescale.is_contiguous()
   lib = L.lib()
   ws_bytes = lib.aqtx_quantize_workspace_bytes(ctypes.byref(plan))
-  ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=x.device) if ws_bytes else None
-  L.check(lib.aqtx_quantize(ctypes.byref(plan), _ptr(x), _ptr(prescale), _ptr(q), _ptr(scale),
-                            _ptr(ws), ws_bytes, _stream()))
-  return q, scale
+  ws = _quantize_workspace(ws_bytes, x.device) if ws_bytes else None
+  plan.workspace_zeroed = int(ws is not None)
+  try:
+    L.check(lib.aqtx_quantize(ctypes.byref(plan), _ptr(x), _ptr(prescale), _ptr(q), _ptr(scale),
+                              _ptr(ws), ws.numel() if ws is not None else 0, _stream()))
+  except Exception:
+    _QUANT_WS.clear()  # a failed launch sequence may have left abs-max words behind
+    raise
+  return (q, scale, typed) if want_typed_scale else (q, scale)
 
 
 def gemm(

@@ -453,6 +453,25 @@ def _kernel_layout_of(qvalue: torch.Tensor, v: 'lowering.OperandView', pack_int4
   return q
 
 
+def _scale_vector_f32(scale: torch.Tensor, ba, ra, ca) -> torch.Tensor:
+  """A frozen operand's scale as the flat float32 vector the kernels read.  A scale kept in
+  another dtype is converted once per tensor, not on every call."""
+  src = getattr(scale, 'f32_copy', None)
+  if src is None:
+    src = scale
+  if src.dtype != torch.float32:
+    key = ('scale_f32', scale._version)
+    hit = _KERNEL_LAYOUT_CACHE.get(id(scale))
+    if hit is not None and hit[0] == key:
+      src = hit[1]
+    else:
+      src = scale.float()
+      if hit is None:
+        weakref.finalize(scale, _KERNEL_LAYOUT_CACHE.pop, id(scale), None)
+      _KERNEL_LAYOUT_CACHE[id(scale)] = (key, src)
+  return lowering.view_operand(src, ba, ra, ca).mem.reshape(-1).contiguous()
+
+
 _POISON = ('Poison. Gradients are not generally expected in serving. Please set '
            'allow_dummy_gradient_into_qtensor to True if this is the intended behavior.')
 
@@ -475,7 +494,11 @@ def _maybe_use_fwd_quant(lhs, rhs: MultiTensor, dimension_numbers, use_fwd_quant
     assert scale_count == 1, msg
     if rhs.qx.bias:
       raise NotImplementedError('Quantization biases are not supported in forward quantization.')
-    scale_t = transpose.rhs_scale_transpose_for_lhs_input(rhs.qx.scale[0], dimension_numbers, lhs.shape)
+    # the float32 copy of the scale, when the quantizer left one, spares a cast launch
+    scale0 = getattr(rhs.qx.scale[0], 'f32_copy', None)
+    if scale0 is None:
+      scale0 = rhs.qx.scale[0]
+    scale_t = transpose.rhs_scale_transpose_for_lhs_input(scale0, dimension_numbers, lhs.shape)
     lhs = _Prescaled(x=lhs, scale_t=scale_t)
     # The quantized residual is quantized again; the kernel reads the int8/fp8 values as
     # floats of the dequant dtype (qvalue.astype(dequant_dtype) in the reference).
@@ -767,7 +790,7 @@ class DotGeneralRaw:
     if sv.mem.numel() != N:
       return None
     sdt = dq.lhs._calibrator.dtype if dq.lhs._calibrator.dtype is not None else lhs_dtype
-    out, xs, xq = ops.decode(lv.mem[0], rq[0], sv.mem.reshape(-1).float().contiguous(),
+    out, xs, xq = ops.decode(lv.mem[0], rq[0], _scale_vector_f32(w_scale, [], rra, rca),
                              quant_bound=spec['quant_bound'], clip_bound=spec['clip_bound'],
                              x_scale_dtype=sdt, w_scale_dtype=w_scale.dtype, want_xq=True,
                              w_dtype=L.I4P if packed else L.I4 if rhs_qt.container_dtype is utils.int4 else L.I8)
@@ -793,9 +816,7 @@ class DotGeneralRaw:
       if q.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
         q = q.view(torch.uint8)
       s = given_qt.scale[0]
-      sv = lowering.view_operand(s, ba, ra, ca)
-      s32 = sv.mem.reshape(-1).float().contiguous()
-      return q, s32, s.dtype, given_qt, quant_grad
+      return q, _scale_vector_f32(s, ba, ra, ca), s.dtype, given_qt, quant_grad
     spec = quantizer.kernel_spec()
     if spec is None:
       raise _NotFused(f'{name}: numerics/calibration {quantizer.numerics} / '
@@ -825,11 +846,7 @@ class DotGeneralRaw:
     if given_qt is not None:
       scale_list = given_qt.scale
     else:
-      if s32.numel() == 1 and (v.B * v.R) != 1:
-        sc = s32.reshape([1] * len(v.shape))
-      else:
-        sc = lowering.logical_from_brk(s32, v, k_keep=False)
-      scale_list = [sc.to(sdt)]
+      scale_list = [lowering.scale_in_dtype(s32, v, sdt)]
     qt = aqt_tensor.QTensor(qvalue=qv, scale=scale_list, scale_t=None, bias=[], dequant_dtype=dtype,
                             container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
     quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))

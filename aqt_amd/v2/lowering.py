@@ -172,8 +172,13 @@ def quantize_view(v: OperandView, *, spec: dict, compute_dtype, scale_dtype, key
   transpose = not v.k_last
   if reduce == L.REDUCE_COLS and per_tensor is False and transpose:
     raise AssertionError('unreachable')
-  q, s = ops.quantize(v.mem, reduce=reduce, transpose_out=transpose, scale=scale, **kwargs)
-  return q, s.reshape(-1) if per_tensor else s.reshape(v.B, v.R)
+  q, s, typed = ops.quantize(v.mem, reduce=reduce, transpose_out=transpose, scale=scale,
+                             want_typed_scale=True, **kwargs)
+  shape = (-1,) if per_tensor else (v.B, v.R)
+  s = s.reshape(shape)
+  # the same scales as elements of the scale dtype, written by the kernel (saves a cast launch)
+  s.typed = typed.reshape(shape) if typed is not None else None
+  return q, s
 
 
 def absmax_scale(x: torch.Tensor, shared_axes: Sequence[int], numerics_, scale_dtype):
@@ -185,4 +190,20 @@ def absmax_scale(x: torch.Tensor, shared_axes: Sequence[int], numerics_, scale_d
               noise=L.NOISE_NONE)
   sdt = scale_dtype if scale_dtype is not None else x.dtype
   _, s = quantize_view(v, spec=spec, compute_dtype=x.dtype, scale_dtype=sdt)
-  return logical_from_brk(s, v, k_keep=False).to(sdt)
+  return scale_in_dtype(s, v, sdt)
+
+
+def scale_in_dtype(s32: torch.Tensor, v: OperandView, sdt) -> torch.Tensor:
+  """The keepdims scale array of dtype `sdt` from the [B, R] float32 scales of quantize_view."""
+  typed = getattr(s32, 'typed', None)
+  if s32.numel() == 1 and (v.B * v.R) != 1:  # per tensor
+    src = typed if typed is not None and typed.dtype == sdt else s32
+    out = src.reshape([1] * len(v.shape)).to(sdt)
+    f32 = s32.reshape([1] * len(v.shape))
+  else:
+    src = typed if typed is not None and typed.dtype == sdt else s32
+    out = logical_from_brk(src, v, k_keep=False).to(sdt)
+    f32 = logical_from_brk(s32, v, k_keep=False)
+  if sdt != torch.float32:
+    out.f32_copy = f32  # same values, for kernels that take float32 scale vectors
+  return out

@@ -85,6 +85,11 @@ typedef struct aqtx_quant_plan {
   int32_t prescale;      /* AQTX_PRESCALE_*: x := round(x * cast(v)) first              */
   int32_t scale_given;   /* 1: `scale` is an input (calibration skipped)                */
   int64_t prescale_stride_batch; /* prescale vector of batch b starts at b*this (0 = shared)  */
+  void* scale_typed;     /* optional out: the computed scales once more as scale_dtype elements
+                            (written for AQTX_BF16 only; NULL or F32: `scale` is all there is)   */
+  int32_t workspace_zeroed; /* 1: the caller keeps one workspace across calls on one stream, passes its
+                            whole size as workspace_bytes, and its first half is zero on entry;
+                            aqtx_quantize returns it zeroed and skips its own clearing launch      */
 } aqtx_quant_plan;
 
 /*

@@ -200,3 +200,25 @@ def test_fp8_cast_exhaustive(gpu, kind):
   np.testing.assert_array_equal(got, want)
   # signed zero / sign of tiny values must survive as well
   np.testing.assert_array_equal(np.signbit(got), np.signbit(want))
+
+
+def test_workspace_kept_across_calls(gpu):
+  """The abs-max workspace is shared by successive calls and handed back zeroed: calls with
+  many, few, and again many scales, column-wise and per tensor, give what a first call gives."""
+  from aqt_amd import _lib as L
+  rng = np.random.default_rng(5)
+  xs = [torch.from_numpy(rng.standard_normal(s).astype(np.float32)).to(torch.bfloat16).to(gpu)
+        for s in ((1, 96, 4096), (1, 64, 24), (2, 40, 1000), (1, 128, 8192))]
+  kw = dict(out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0)
+  first = {}
+  for rnd in range(3):
+    for i, x in enumerate(xs):
+      for reduce in (L.REDUCE_ROWS, L.REDUCE_ALL_BATCH):
+        q, s = ops.quantize(x, reduce=reduce, **kw)
+        if rnd == 0:
+          amax = x.float().abs().amax(dim=1) if reduce == L.REDUCE_ROWS else x.float().abs().amax().reshape(1)
+          want = (amax / 127.5).to(torch.bfloat16).float()
+          assert torch.equal(s.reshape(-1), want.reshape(-1))
+          first[(i, reduce)] = (q.clone(), s.clone())
+        else:
+          assert torch.equal(q, first[(i, reduce)][0]) and torch.equal(s, first[(i, reduce)][1])
