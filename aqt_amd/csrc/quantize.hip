@@ -201,8 +201,11 @@ __device__ __forceinline__ uint32_t spec_finish(float t, const QArgs& a) {
     t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
     return to_qbyte(t, a.out_dtype);
   }
-  t = fminf(fmaxf(t, -a.clip_bound), a.clip_bound);
-  return (uint32_t)((int)rintf(t)) & 0xFFu;
+  // clip in one median-of-three; round half to even and convert in one addition: after
+  // t + 1.5 * 2^23 the low mantissa bits are the two's complement of the rounded integer
+  // (|t| <= 127 here)
+  t = __builtin_amdgcn_fmed3f(t, -a.clip_bound, a.clip_bound);
+  return __float_as_uint(t + 12582912.0f) & 0xFFu;
 }
 // fp_mantissa_round on a bf16 value (fp8_numerics.py:36-64): add the masked random bits to the
 // bit pattern, clear the low mantissa bits.
