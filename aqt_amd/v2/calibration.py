@@ -14,6 +14,20 @@ import torch
 from aqt_amd.v2 import utils
 
 
+class State(dict):
+  """Statistics of a stateful calibrator: the stand-in for a Flax variable collection.
+
+  A config tree is deep-copied freely (`config.set_context` does it on every step); the
+  statistics must stay the one shared object through those copies, as variables do.
+  """
+
+  def __copy__(self):
+    return self
+
+  def __deepcopy__(self, memo):
+    return self
+
+
 @dataclasses.dataclass(kw_only=True)
 class Calibration(abc.ABC):
   """calibration.py:34-64."""
