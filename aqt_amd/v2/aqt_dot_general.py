@@ -818,9 +818,28 @@ class DotGeneralRaw:
       s = given_qt.scale[0]
       return q, _scale_vector_f32(s, ba, ra, ca), s.dtype, given_qt, quant_grad
     spec = quantizer.kernel_spec()
+    if spec is None and given_qt is None:
+      # The numerics have a kernel but the calibration does not (power-of-two or clipped
+      # scales, constant bounds, static-range and delayed-scaling statistics...): calibrate step
+      # by step, then quantize and contract in the fused kernels with that scale.
+      nspec = None if isinstance(quantizer.numerics, no_numerics.NoNumerics) else quantizer.numerics.kernel_spec()
+      if nspec is None or quantizer._calibrator is None:
+        raise _NotFused(f'{name}: numerics/calibration {quantizer.numerics} / '
+                        f'{quantizer.calibration} have no fused HIP kernel')
+      # the calibrator has to see the tensor the reference hands it: the gradient already
+      # multiplied by the forward scale, the forward residual as values of the float dtype
+      if x_is_q:
+        x, x_is_q = x.to(dtype), False
+      if prescale_t is not None:
+        x, prescale_t = x * prescale_t.to(x.dtype), None
+      given_qt = quantizer.calibrate(x, calibration_axes=ca)
+      if len(given_qt.scale) != 1 or given_qt.bias or given_qt.sparsity_mask is not None:
+        raise _NotFused(f'{name}: calibration with a bias, a sparsity mask or several scales')
+      spec = nspec
+    elif spec is None:
+      spec = None if isinstance(quantizer.numerics, no_numerics.NoNumerics) else quantizer.numerics.kernel_spec()
     if spec is None:
-      raise _NotFused(f'{name}: numerics/calibration {quantizer.numerics} / '
-                                f'{quantizer.calibration} have no fused HIP kernel')
+      raise _NotFused(f'{name}: numerics {quantizer.numerics} have no fused HIP kernel')
     if getattr(quantizer.numerics, 'clip_gradient', False):
       raise _NotFused('clip_gradient is not supported by the fused path')
     arr = x
@@ -835,13 +854,21 @@ class DotGeneralRaw:
       prescale = pv.mem.reshape(pv.B, -1).float().contiguous()
       if pv.B == 1 and v.B > 1:
         prescale = prescale.reshape(-1)
-    scale_in = None
+    scale_in, scale_dtype = None, None
     if given_qt is not None:  # incomplete QTensor: scale only (aqt_dot_general.py:645-653)
       assert len(given_qt.scale) == 1
-      sv = lowering.view_operand(given_qt.scale[0], ba, ra, ca)
-      scale_in = sv.mem.reshape(-1).float().contiguous()
-      scale_in = scale_in.reshape(v.B, v.R, 1) if v.k_last else scale_in.reshape(v.B, 1, v.R)
-    q, s32, sdt = quantizer.quant_view(v, dtype, calibration_axes=ca, prescale=prescale, scale=scale_in)
+      gs = given_qt.scale[0]
+      scale_dtype = gs.dtype
+      if gs.numel() == 1:
+        flat = gs.reshape(1).float().expand(v.B * v.R)
+      else:
+        sv = lowering.view_operand(gs, ba, ra, ca)
+        if sv.K != 1 or sv.mem.numel() != v.B * v.R:
+          raise _NotFused(f'{name}: a scale that is not shared over exactly the contraction axes')
+        flat = sv.mem.reshape(-1).float()
+      scale_in = flat.contiguous().reshape(v.B, v.R, 1) if v.k_last else flat.contiguous().reshape(v.B, 1, v.R)
+    q, s32, sdt = quantizer.quant_view(v, dtype, calibration_axes=ca, prescale=prescale, scale=scale_in,
+                                       scale_dtype=scale_dtype)
     qv = lowering.logical_from_brk(aqt_quantizer._typed(q, spec['out_dtype']), v)
     if given_qt is not None:
       scale_list = given_qt.scale

@@ -49,14 +49,17 @@ class Quantizer:
     return spec
 
   def quant_view(self, v: lowering.OperandView, dtype, *, calibration_axes, prescale=None,
-                 scale: Optional[torch.Tensor] = None):
+                 scale: Optional[torch.Tensor] = None, scale_dtype=None):
     """Calibrate + quantize an operand view in one kernel sequence.
 
-    Returns (q [B,R,K], scale float32 [B,R] or [1], scale dtype).
+    With `scale` (float32, one value per [B, R] entry, holding values of `scale_dtype`) the
+    calibration is skipped.  Returns (q [B,R,K], scale float32 [B,R] or [1], scale dtype).
     """
-    spec = self.kernel_spec()
+    spec = self.kernel_spec() if scale is None else self.numerics.kernel_spec()
     assert spec is not None
-    if self.calib_shared_axes == 'per_tensor':
+    if scale is not None:
+      per_tensor = False
+    elif self.calib_shared_axes == 'per_tensor':
       per_tensor = True
     else:
       shared = self.calib_shared_axes or calibration_axes
@@ -64,7 +67,10 @@ class Quantizer:
         raise lowering.NotFused(
             f'calib_shared_axes={shared} differs from the contraction axes {v.k_axes}')
       per_tensor = False
-    sdt = self._calibrator.dtype if self._calibrator.dtype is not None else dtype
+    if scale_dtype is not None:
+      sdt = scale_dtype
+    else:
+      sdt = self._calibrator.dtype if self._calibrator.dtype is not None else dtype
     q, s = lowering.quantize_view(v, spec=spec, compute_dtype=dtype, scale_dtype=sdt,
                                   key=None if self.context is None else self.context.key,
                                   per_tensor=per_tensor, prescale=prescale, scale=scale)
