@@ -874,14 +874,14 @@ int noise_width(const aqtx_quant_plan* p) {
 
 // Which compile-time specialisation (see spec_quant) serves this plan.
 int spec_of(const QArgs& a, int partitionable) {
-  if (a.cbf && a.sbf && !a.scale_given && (a.out_dtype == AQTX_E4M3 || a.out_dtype == AQTX_E5M2)) {
+  if (a.cbf && a.sbf && (a.out_dtype == AQTX_E4M3 || a.out_dtype == AQTX_E5M2)) {
     if (a.noise == AQTX_NOISE_NONE) return 3;
     if (a.noise == AQTX_NOISE_FP8_MANTISSA && !partitionable && a.gen.width == 16 && a.nsc == 1 &&
         a.nsr % 2 == 0 && a.nsb % 2 == 0)
       return 5;  // neighbouring elements draw from one word, starting at an even counter
     return 0;
   }
-  if (!(a.cbf && a.sbf && (a.out_dtype == AQTX_I8 || a.out_dtype == AQTX_I4) && !a.scale_given)) return 0;
+  if (!(a.cbf && a.sbf && (a.out_dtype == AQTX_I8 || a.out_dtype == AQTX_I4))) return 0;
   if (a.noise == AQTX_NOISE_NONE) return 1;
   if (a.noise == AQTX_NOISE_JAX_UNIFORM && !partitionable) return 2;
   return 0;
