@@ -46,6 +46,7 @@ class GemmPlan(ctypes.Structure):
       ('row_scale_dtype', ctypes.c_int32), ('col_scale_dtype', ctypes.c_int32),
       ('scale_order', ctypes.c_int32),
       ('row_scale_stride_b', ctypes.c_int64), ('col_scale_stride_b', ctypes.c_int64),
+      ('group_offsets', ctypes.c_void_p),
   ]
 
 

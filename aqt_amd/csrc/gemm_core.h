@@ -76,6 +76,9 @@ struct GemmArgs {
   int p1_bf16;    // the first product is rounded to bf16
   int p2_bf16;    // the second product is rounded to bf16
   int col_first;  // scale order
+  // Ragged batches: entry b multiplies rows [group_offsets[b], group_offsets[b+1]) of one flat
+  // A with B[b] into the same rows of one flat C (m is then an upper bound of a group's rows).
+  const int32_t* group_offsets;
 };
 
 constexpr int BM = 256, BN = 256, BK = 128;
@@ -114,8 +117,9 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // issue slots in which the other waits on the memory pipeline.
 template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
-void gemm_kernel(const GemmArgs g) {
+void gemm_kernel(const GemmArgs g_in) {
   static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+  GemmArgs g = g_in;
   constexpr int NI = 16 / NW;       // 32-column MFMA tiles per wave
   constexpr int WN = NW / 2;        // waves along n
   constexpr int LPW = 32 / NW;      // 8-row load blocks per wave and operand
@@ -140,6 +144,19 @@ void gemm_kernel(const GemmArgs g) {
   tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
   const int64_t bz = blockIdx.y;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+  if (g_in.group_offsets != nullptr) {
+    // the group's row range replaces the batch strides of A, C and the row scale; tiles past
+    // the group's last row leave at once (the grid is sized for the largest possible group)
+    const int64_t row0 = g_in.group_offsets[bz];
+    const int64_t rows = g_in.group_offsets[bz + 1] - row0;
+    if (m0 >= rows) return;
+    g.m = rows;
+    g.a += row0 * g.lda;
+    g.c = reinterpret_cast<uint8_t*>(g.c) + row0 * g.ldc * (g.out_dtype == AQTX_BF16 ? 2 : 4);
+    if (g.acc_out != nullptr) g.acc_out = reinterpret_cast<uint8_t*>(g.acc_out) + row0 * g.ldc * 4;
+    if (g.row_scale != nullptr) g.row_scale += row0;
+    g.stride_a = 0; g.stride_c = 0; g.stride_rs = 0;
+  }
 
   // ---- global -> registers -> LDS.  One wave instruction moves 8 rows x 128 B (1 KiB): lane l
   // handles LDS slot (row l>>3, chunk l&7) of its 8-row block and fetches the global chunk
@@ -523,6 +540,7 @@ inline GemmArgs make_gemm_args(const aqtx_gemm_plan* p, const void* a, const voi
   }
   g.tiles_m = (int)((p->m + BM - 1) / BM);
   g.tiles_n = (int)((p->n + BN - 1) / BN);
+  g.group_offsets = p->group_offsets;
   return g;
 }
 

@@ -41,6 +41,7 @@ extern "C" int aqtx_gemm_fp8(const aqtx_gemm_plan* p, const void* a, const void*
   const bool a5 = p->a_dtype == AQTX_E5M2, b5 = p->b_dtype == AQTX_E5M2;
 
   if (!gemm_vector_path_ok(p, a, b)) {
+    AQTX_REQUIRE(p->group_offsets == nullptr, "aqtx_gemm_fp8: ragged batches need aligned operands");
     dim3 grid((unsigned)((p->n + 255) / 256), (unsigned)p->m, (unsigned)p->batch);
     AQTX_REQUIRE(p->m <= 65535, "aqtx_gemm_fp8: m too large for the unaligned path");
     if (!a5 && !b5) gemm_simple_kernel<DecE4M3, DecE4M3, false><<<grid, 256, 0, st>>>(g);

@@ -51,6 +51,9 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
   if (!gemm_vector_path_ok(p, a, b)) {
+    AQTX_REQUIRE(p->group_offsets == nullptr,
+                 "aqtx_gemm_i8: ragged batches need 16-byte aligned operands with k and leading dimensions "
+                 "multiple of 16");
     dim3 grid((unsigned)((p->n + 255) / 256), (unsigned)p->m, (unsigned)p->batch);
     AQTX_REQUIRE(p->m <= 65535, "aqtx_gemm_i8: m too large for the unaligned path");
     gemm_simple_kernel<DecI8, DecI8, true><<<grid, 256, 0, st>>>(g);

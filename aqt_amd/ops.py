@@ -206,8 +206,14 @@ def gemm(
     a_dtype: int = L.I8,
     b_dtype: int = L.I8,
     want_acc: bool = False,
+    group_offsets: Optional[torch.Tensor] = None,
 ):
   """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
+
+  With `group_offsets` (int32 device tensor [groups + 1], ascending): a ragged product.  A is
+  [1, m, k], B [groups, n, k]; group g multiplies rows off[g]:off[g+1] of A with B[g] into the
+  same rows of C [1, m, n], in one launch; rows outside every group are left as allocated
+  (zero-initialised here).
 
   int8 operands use the int32 MFMA path, fp8 operands (uint8 tensors holding
   e4m3fn/e5m2 bytes) the float32 one.  `scale_dtype` names the dtype of both scale
@@ -215,20 +221,26 @@ def gemm(
   (C, acc) with want_acc.
   """
   _require_gpu(a, b, row_scale, col_scale)
-  assert a.dim() == 3 and b.dim() == 3 and a.shape[0] == b.shape[0] and a.shape[2] == b.shape[2]
+  assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == b.shape[2]
+  assert a.shape[0] == b.shape[0] or group_offsets is not None
   assert a.stride(2) == 1 and b.stride(2) == 1, 'the contraction axis must be contiguous'
   batch, m, k = a.shape
   n = b.shape[1]
+  if group_offsets is not None:
+    assert a.shape[0] == 1 and group_offsets.dtype == torch.int32 and group_offsets.is_cuda
+    assert group_offsets.numel() == b.shape[0] + 1 and group_offsets.is_contiguous()
   fp8 = a_dtype in (L.E4M3, L.E5M2)
   out_dt = aqtx_dtype(out_dtype)
   dq_dt = aqtx_dtype(dequant_dtype) if dequant_dtype is not None else (out_dt if out_dt != L.I32 else L.F32)
   sc_dt = aqtx_dtype(scale_dtype) if scale_dtype is not None else dq_dt
-  c = torch.empty((batch, m, n), dtype=_AQTX_TO_TORCH[out_dt], device=a.device)
+  alloc = torch.zeros if group_offsets is not None else torch.empty
+  c = alloc((batch, m, n), dtype=_AQTX_TO_TORCH[out_dt], device=a.device)
   acc = None
   if want_acc:
     acc = torch.empty((batch, m, n), dtype=torch.float32 if fp8 else torch.int32, device=a.device)
   plan = L.GemmPlan()
-  plan.batch, plan.m, plan.n, plan.k = batch, m, n, k
+  plan.batch, plan.m, plan.n, plan.k = (b.shape[0] if group_offsets is not None else batch), m, n, k
+  plan.group_offsets = group_offsets.data_ptr() if group_offsets is not None else None
   plan.lda, plan.ldb, plan.ldc = a.stride(1), b.stride(1), n
   plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), b.stride(0), m * n
   plan.a_dtype, plan.b_dtype = a_dtype, b_dtype
@@ -236,10 +248,9 @@ def gemm(
   plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else sc_dt
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else sc_dt
   plan.scale_order = scale_order
-  for s, dim in ((row_scale, m), (col_scale, n)):
+  for s, shape in ((row_scale, (batch, m)), (col_scale, (b.shape[0], n))):
     if s is not None:
-      assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == (batch, dim), (
-          tuple(s.shape), (batch, dim))
+      assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == shape, (tuple(s.shape), shape)
   plan.row_scale_stride_b, plan.col_scale_stride_b = m, n
   fn = L.lib().aqtx_gemm_fp8 if fp8 else L.lib().aqtx_gemm_i8
   with _timed('gemm'):

@@ -3,8 +3,8 @@
 `lhs` [m, k] holds the rows of `g` groups one after the other, `rhs` [g, k, n] one matrix per
 group, `group_sizes` [g] the row counts: out[rows of group i] = lhs[rows of group i] @ rhs[i].
 The contraction is plugged into `DotGeneralRaw.dot_general`, so calibration, quantization and
-dequantisation are the ordinary ones; the int8 groups run on the MFMA contraction kernel, one
-launch per non-empty group over a row range of the same operand buffers (no copies).
+dequantisation are the ordinary ones; the int8 groups run on the MFMA contraction kernel in one
+launch: every workgroup looks its group's row range up in a device-side offset table.
 """
 from __future__ import annotations
 
@@ -26,25 +26,46 @@ def _host_group_sizes(group_sizes) -> Sequence[int]:
   return [int(v) for v in group_sizes]
 
 
+def _group_offsets(group_sizes, m: int, device) -> torch.Tensor:
+  """[0, s0, s0+s1, ...] as int32 on the device, clamped to the rows there are; computed on the
+  device when the sizes live there (no host round trip)."""
+  sizes = group_sizes if isinstance(group_sizes, torch.Tensor) else torch.tensor(list(group_sizes), dtype=torch.int32)
+  sizes = sizes.to(device=device, dtype=torch.int32)
+  offs = torch.zeros(sizes.numel() + 1, dtype=torch.int32, device=device)
+  offs[1:] = torch.cumsum(sizes, 0)
+  return torch.clamp(offs, max=m)
+
+
 def lax_ragged_dot(lhs, rhs, group_sizes, precision=None, preferred_element_type=None):
-  """jax.lax.ragged_dot on torch tensors: int8 x int8 -> int32 on the MFMA kernel, anything
-  else as float contractions; rows past sum(group_sizes) are zero."""
+  """jax.lax.ragged_dot on torch tensors: int8 x int8 -> int32 on the MFMA kernel (all groups in
+  one launch, row ranges from a device-side offset table), anything else as float contractions;
+  rows past sum(group_sizes) are zero."""
   del precision
   assert lhs.dim() == 2 and rhs.dim() == 3 and lhs.shape[1] == rhs.shape[1], (lhs.shape, rhs.shape)
-  sizes = _host_group_sizes(group_sizes)
-  assert len(sizes) == rhs.shape[0], (len(sizes), rhs.shape)
   m, k = lhs.shape
   n = rhs.shape[2]
-  assert sum(sizes) <= m, f'group sizes {sizes} exceed the {m} rows of lhs'
+  assert len(group_sizes) == rhs.shape[0], (len(group_sizes), rhs.shape)
   both_int = lhs.dtype == torch.int8 and rhs.dtype == torch.int8
   if both_int:
     assert preferred_element_type == torch.int32, (
         f'{preferred_element_type=}: int8 operands are contracted into int32 accumulators only')
-    out = torch.zeros((m, n), dtype=torch.int32, device=lhs.device)
+    if m * n == 0 or k == 0 or rhs.shape[0] == 0:
+      return torch.zeros((m, n), dtype=torch.int32, device=lhs.device)
     a = lhs if lhs.stride(1) == 1 else lhs.contiguous()
     bt = rhs.permute(0, 2, 1)  # [g, n, k]: the quantizer already wrote the weights k-contiguous
     if bt.stride(2) != 1:
       bt = bt.contiguous()
+    aligned = (k % 16 == 0 and a.stride(0) % 16 == 0 and bt.stride(1) % 16 == 0 and bt.stride(0) % 16 == 0
+               and a.data_ptr() % 16 == 0 and bt.data_ptr() % 16 == 0)
+    if aligned:
+      return ops.gemm(a[None], bt, row_scale=None, col_scale=None, out_dtype=torch.int32, a_dtype=L.I8,
+                      b_dtype=L.I8, group_offsets=_group_offsets(group_sizes, m, lhs.device))[0]
+  # one contraction per group on row slices (sizes read on the host: a synchronisation when they
+  # live on the device)
+  sizes = _host_group_sizes(group_sizes)
+  assert sum(sizes) <= m, f'group sizes {sizes} exceed the {m} rows of lhs'
+  if both_int:
+    out = torch.zeros((m, n), dtype=torch.int32, device=lhs.device)
   else:
     common = torch.promote_types(lhs.dtype, rhs.dtype)
     out_dtype = preferred_element_type if preferred_element_type is not None else common
@@ -54,10 +75,10 @@ def lax_ragged_dot(lhs, rhs, group_sizes, precision=None, preferred_element_type
     if size == 0:
       continue
     rows = slice(start, start + size)
-    if both_int and k > 0 and n > 0:
+    if both_int:
       out[rows] = ops.gemm(a[rows][None], bt[g][None], row_scale=None, col_scale=None,
                            out_dtype=torch.int32, a_dtype=L.I8, b_dtype=L.I8)[0]
-    elif not both_int:
+    else:
       out[rows] = torch.matmul(lhs[rows].to(common), rhs[g].to(common)).to(out.dtype)
     start += size
   return out

@@ -143,6 +143,12 @@ typedef struct aqtx_gemm_plan {
   int32_t col_scale_dtype;    /* AQTX_BF16 | AQTX_F32: dtype of the values in col_scale      */
   int32_t scale_order;        /* AQTX_SCALE_*: which scale multiplies first                  */
   int64_t row_scale_stride_b, col_scale_stride_b; /* batch strides of the scale vectors    */
+  /* Ragged batches (jax.lax.ragged_dot, aqt/jax/v2/aqt_ragged_dot.py:22-46): optional DEVICE
+     pointer to batch+1 ascending int32 row offsets.  Entry b multiplies rows
+     [off[b], off[b+1]) of one flat A [m, k] with B[b] into the same rows of one flat C [m, n]
+     (row_scale is flat [m] too); stride_a, stride_c and row_scale_stride_b are ignored.  Rows
+     outside every group are not written.  NULL: ordinary batches.                          */
+  const int32_t* group_offsets;
 } aqtx_gemm_plan;
 
 /*

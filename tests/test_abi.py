@@ -110,6 +110,7 @@ def _gplan(**kw):
     (dict(scale_order=3), 'scale_order'),
     (dict(lda=32), 'leading dimension'),
     (dict(out_dtype=L.F32, dequant_dtype=L.BF16), 'combination'),
+    (dict(group_offsets=FAKE, k=24, lda=24, ldb=24), 'ragged batches'),
 ])
 def test_gemm_plan_validation(kw, needle):
   p = _gplan(**kw)

@@ -58,7 +58,7 @@ def test_oracle_ragged_dot_integer_exact():
 @pytest.mark.gpu
 @pytest.mark.parametrize('dt', ['bf16', 'f32'])
 @pytest.mark.parametrize('balanced', [True, False])
-@pytest.mark.parametrize('shape', [(32, 128, 16, 8), (300, 96, 200, 5)])
+@pytest.mark.parametrize('shape', [(32, 128, 16, 8), (300, 96, 200, 5), (3000, 256, 520, 6), (66, 72, 40, 3)])
 def test_ragged_dot_matches_oracle(gpu, dt, balanced, shape):
   from aqt_amd.v2 import aqt_ragged_dot
   m, k, n, g = shape
@@ -86,3 +86,22 @@ def test_ragged_dot_unquantized_and_precision(gpu):
   np.testing.assert_allclose(out.cpu().numpy(), R.lax_ragged_dot(lhs, rhs, sizes, np.float32), rtol=1e-5)
   with pytest.raises(AssertionError):  # aqt_ragged_dot_test.py:155-166
     aqt_ragged_dot.ragged_dot(L, Rr, sizes, precision='highest')
+
+
+@pytest.mark.gpu
+def test_ragged_gemm_one_launch_against_integer_reference(gpu):
+  """The grouped launch itself: groups that span several 256-row tiles, start in the middle of
+  a tile, are empty, or leave the last rows uncovered; raw int32 accumulators."""
+  from aqt_amd import ops
+  rng = np.random.default_rng(3)
+  m, k, n = 2000, 320, 300
+  sizes = [700, 0, 257, 1, 511, 300]  # sums to 1769 < m
+  a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+  b = rng.integers(-127, 128, (len(sizes), n, k)).astype(np.int8)
+  offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+  out = ops.gemm(torch.from_numpy(a).to(gpu)[None], torch.from_numpy(b).to(gpu), row_scale=None, col_scale=None,
+                 out_dtype=torch.int32, group_offsets=torch.from_numpy(offs).to(gpu))[0].cpu().numpy()
+  want = np.zeros((m, n), np.int64)
+  for g, (lo, hi) in enumerate(zip(offs[:-1], offs[1:])):
+    want[lo:hi] = a[lo:hi].astype(np.int64) @ b[g].astype(np.int64).T
+  np.testing.assert_array_equal(out, want)
