@@ -141,7 +141,14 @@ void gemm_kernel(const GemmArgs g_in) {
   const int lr = lane & 31, lh = lane >> 5;
 
   int tm, tn;
-  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  if (g_in.group_offsets != nullptr) {
+    // Only the first few tile rows of a group hold work; ids run along n first, so that those
+    // rows are dealt round-robin to all XCDs (the banded walk would leave them to one XCD).
+    tm = (int)(blockIdx.x / (unsigned)g.tiles_n);
+    tn = (int)(blockIdx.x % (unsigned)g.tiles_n);
+  } else {
+    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  }
   const int64_t bz = blockIdx.y;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
   if (g_in.group_offsets != nullptr) {
@@ -313,8 +320,8 @@ void gemm_kernel(const GemmArgs g_in) {
   // lane holds C[m = mrow0 + mi*32 + lr][n = ncol0 + ni*32 + 8*q + 4*lh + e], e = 0..3, reg = 4*q+e
   const int64_t mrow0 = m0 + wm * 128, ncol0 = n0 + wn * NI * 32;
 
-  if (EPI == 3 || g.acc_out != nullptr) {
-    AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out != nullptr ? g.acc_out : g.c);
+  if (g.acc_out != nullptr) {  // optional second copy of the raw accumulators (plain stores)
+    AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out);
     dst += bz * g.stride_c;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
@@ -328,7 +335,9 @@ void gemm_kernel(const GemmArgs g_in) {
         }
     }
   }
-  if constexpr (EPI != 3) {
+  {
+    // EPI 3 (raw accumulators as the output) takes the same staged, coalesced store path as the
+    // float outputs: the 32-bit patterns travel through the float slots untouched.
     constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
     constexpr bool kDqBf16 = kOutBf16;                    // dequant dtype == output dtype
     constexpr bool kProd1Bf16 = EPI == 0 || EPI == 4;     // promote(dequant dtype, first scale dtype)
@@ -343,6 +352,7 @@ void gemm_kernel(const GemmArgs g_in) {
       rscale[mi] = (rs != nullptr && mm < g.m) ? rs[mm] : 1.0f;
     }
     auto dequant = [&](AccScalar accv, float s_row, float s_col) {
+      if constexpr (EPI == 3) return __builtin_bit_cast(float, accv);
       float f = round_to<kDqBf16>((float)accv);  // (int32 ->) f32 -> dequant dtype
       const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
       f = round_to<kProd1Bf16>(f * s1);

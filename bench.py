@@ -173,6 +173,31 @@ def other_configs(dev):
 
   ms = timeit(step5)
   out['int4w_int8a_tiled128_fwd'] = {'ms_per_call': round(ms, 3), 'TOPS': round(2 * 2048 * 8192 * 28672 / ms / 1e9, 1)}
+  del lhs, rhs
+  # quantized ragged_dot (mixture of experts): 8192 tokens routed to 8 experts [4096, 14336], uneven groups,
+  # forward, with the expert weights quantized on the fly (the reference's ragged_dot does the same) and
+  # with the contraction alone (operands already int8)
+  from aqt_amd import ops
+  from aqt_amd.v2 import aqt_ragged_dot
+  tokens, experts, kk, nn = 8192, 8, 4096, 14336
+  x = torch.randn(tokens, kk, device=dev).to(torch.bfloat16)
+  w = (torch.randn(experts, kk, nn, device=dev) * 0.02).to(torch.bfloat16)
+  sizes = torch.tensor([1500, 700, 1024, 0, 2100, 900, 1200, 768], dtype=torch.int32, device=dev)
+
+  def step6():
+    with torch.no_grad():
+      aqt_ragged_dot.ragged_dot(x, w, sizes)
+
+  ms = timeit(step6)
+  xq = torch.randint(-127, 128, (1, tokens, kk), dtype=torch.int8, device=dev)
+  wq = torch.randint(-127, 128, (experts, nn, kk), dtype=torch.int8, device=dev)
+  offs = torch.zeros(experts + 1, dtype=torch.int32, device=dev)
+  offs[1:] = torch.cumsum(sizes, 0)
+  ms_gemm = timeit(lambda: ops.gemm(xq, wq, row_scale=None, col_scale=None, out_dtype=torch.int32, group_offsets=offs))
+  gop = 2.0 * tokens * kk * nn / 1e9
+  out['ragged_dot_int8_fwd_8192tok_8experts'] = {
+      'ms_per_call': round(ms, 3), 'TOPS': round(gop / ms, 1),
+      'contraction_only_ms': round(ms_gemm, 3), 'contraction_only_TOPS': round(gop / ms_gemm, 1)}
   return out
 
 
