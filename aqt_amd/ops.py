@@ -259,6 +259,16 @@ def gemm(
   return (c, acc) if want_acc else c
 
 
+def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
+  """[0, s0, s0+s1, ...] as int32 on the device, clamped to the m rows there are; computed on the
+  device when the sizes live there (no host round trip)."""
+  sizes = group_sizes if isinstance(group_sizes, torch.Tensor) else torch.tensor(list(group_sizes), dtype=torch.int32)
+  sizes = sizes.to(device=device, dtype=torch.int32)
+  offs = torch.zeros(sizes.numel() + 1, dtype=torch.int32, device=device)
+  offs[1:] = torch.cumsum(sizes, 0)
+  return torch.clamp(offs, max=m)
+
+
 def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
            clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False,
            w_dtype: int = L.I8):

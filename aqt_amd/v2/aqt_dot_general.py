@@ -531,6 +531,13 @@ def _canonical_pairs(lhs, rhs, dimension_numbers):
 _NotFused = lowering.NotFused
 
 
+def _ragged_sizes(dot_general_hook):
+  """The group sizes of a ragged-contraction hook (aqt_ragged_dot.RaggedDot), else None."""
+  if getattr(dot_general_hook, 'is_ragged_dot', False):
+    return dot_general_hook.group_sizes
+  return None
+
+
 @dataclasses.dataclass(kw_only=True)
 class DotGeneralRaw:
   """Configuration of quantization of one dot_general without gradient (aqt_dot_general.py:732-749)."""
@@ -581,7 +588,8 @@ class DotGeneralRaw:
 
   def _dispatch(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes):
     """The fused kernels where they implement the configuration, the step-by-step path otherwise."""
-    fusable = (self.dot_general is lax_dot_general
+    # a ragged (grouped) contraction hook is lowered too: same kernels, rows looked up per group
+    fusable = ((self.dot_general is lax_dot_general or _ragged_sizes(self.dot_general) is not None)
                and type(self.dg_quantizer) is DefaultDotGeneralQuantizer)  # pylint: disable=unidiomatic-typecheck
     for side in (self.lhs, self.rhs):
       fusable = fusable and (side.dequant_mode == DequantMode.OUTPUT
@@ -682,7 +690,16 @@ class DotGeneralRaw:
     if dq.lhs_mid_alpha is not None or dq.rhs_mid_alpha is not None:
       raise _NotFused('mid-scale quantization has no HIP path yet')
 
-    dn = _canonical_pairs(lhs, rhs_arr, dimension_numbers)
+    ragged = _ragged_sizes(self.dot_general)
+    if ragged is not None:
+      # lhs [m, k] x rhs [g, k, n]; the dimension numbers only say which axes share a scale
+      (lca, rca), (lba, rba) = dimension_numbers
+      if (lhs.dim() != 2 or rhs_arr.dim() != 3 or list(lca) != [1] or list(rca) != [0, 1] or lba or rba
+          or out_transpose_axes is not None or lhs.shape[1] != rhs_arr.shape[1]):
+        raise _NotFused('ragged contraction in another layout')
+      dn = (([1], [0, 1]), ([], []))
+    else:
+      dn = _canonical_pairs(lhs, rhs_arr, dimension_numbers)
     (lca, rca), (lba, rba) = dn
     lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
     rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
@@ -714,12 +731,24 @@ class DotGeneralRaw:
 
     B, M, K = lq.shape
     N = rq.shape[1]
+    if ragged is not None:
+      G = rhs_arr.shape[0]
+      rq3 = rq.reshape(N, G, K).permute(1, 0, 2)  # [g, n, k] view of the quantizer's [n, g*k] rows
+      if not (K % 16 == 0 and lq.data_ptr() % 16 == 0 and rq3.data_ptr() % 16 == 0 and M * N > 0):
+        raise _NotFused('ragged contraction with unaligned operands')
+      out = ops.gemm(lq, rq3, row_scale=ls.reshape(1, M) if ls.numel() == M else ls.reshape(1, 1).expand(1, M).contiguous(),
+                     col_scale=rs.reshape(1, -1).expand(G, N).contiguous(), a_dtype=lkd, b_dtype=rkd,
+                     row_scale_dtype=lsdt, col_scale_dtype=rsdt, out_dtype=dequant_dtype, dequant_dtype=dequant_dtype,
+                     group_offsets=ops.ragged_offsets(ragged, M, lq.device))
+      res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=lhs, qx=lhs_qt_out), quant_grad=lhs_grad),
+                          rhs=TensorRes(mt=MultiTensor(x=rhs_arr, qx=rhs_qt_out), quant_grad=rhs_grad))
+      return out.reshape(M, N), res
     assert rq.shape[0] == B and rq.shape[2] == K, (lq.shape, rq.shape)
     # scales: [B, M] / [B, N] or a single per-tensor value (broadcast here, tiny)
     def expand(s, n):
       return s.reshape(1, 1).expand(B, n).contiguous() if s.numel() == 1 and B * n != 1 else s.reshape(B, n)
     if self.dot_general is not lax_dot_general:
-      raise _NotFused('a custom DotGeneralRaw.dot_general hook is not lowered')
+      raise _NotFused('a custom DotGeneralRaw.dot_general hook is not lowered')  # (ragged hooks returned above)
     nb, nl, nr = len(lba), len(lra), len(rra)
     bdims = [lhs.shape[a] for a in lba]
     ldims = [lhs.shape[a] for a in lra]

@@ -26,16 +26,6 @@ def _host_group_sizes(group_sizes) -> Sequence[int]:
   return [int(v) for v in group_sizes]
 
 
-def _group_offsets(group_sizes, m: int, device) -> torch.Tensor:
-  """[0, s0, s0+s1, ...] as int32 on the device, clamped to the rows there are; computed on the
-  device when the sizes live there (no host round trip)."""
-  sizes = group_sizes if isinstance(group_sizes, torch.Tensor) else torch.tensor(list(group_sizes), dtype=torch.int32)
-  sizes = sizes.to(device=device, dtype=torch.int32)
-  offs = torch.zeros(sizes.numel() + 1, dtype=torch.int32, device=device)
-  offs[1:] = torch.cumsum(sizes, 0)
-  return torch.clamp(offs, max=m)
-
-
 def lax_ragged_dot(lhs, rhs, group_sizes, precision=None, preferred_element_type=None):
   """jax.lax.ragged_dot on torch tensors: int8 x int8 -> int32 on the MFMA kernel (all groups in
   one launch, row ranges from a device-side offset table), anything else as float contractions;
@@ -59,7 +49,7 @@ def lax_ragged_dot(lhs, rhs, group_sizes, precision=None, preferred_element_type
                and a.data_ptr() % 16 == 0 and bt.data_ptr() % 16 == 0)
     if aligned:
       return ops.gemm(a[None], bt, row_scale=None, col_scale=None, out_dtype=torch.int32, a_dtype=L.I8,
-                      b_dtype=L.I8, group_offsets=_group_offsets(group_sizes, m, lhs.device))[0]
+                      b_dtype=L.I8, group_offsets=ops.ragged_offsets(group_sizes, m, lhs.device))[0]
   # one contraction per group on row slices (sizes read on the host: a synchronisation when they
   # live on the device)
   sizes = _host_group_sizes(group_sizes)
@@ -92,6 +82,7 @@ class RaggedDot:
     group_sizes: the sizes of the groups, shape [g].
   """
   group_sizes: Any
+  is_ragged_dot = True  # DotGeneralRaw lowers this hook to the fused kernels when it can
 
   def __call__(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
     del dimension_numbers
