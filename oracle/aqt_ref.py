@@ -763,3 +763,56 @@ def ragged_dot_fwd(lhs, rhs, dt, group_sizes, raw: RawCfg):
     scales.append(rhs_scale_transpose_to_output(s, dn, lhs.shape, rhs.shape))
     sdts.append(rqt.scale_dtype or dt)
   return nm.cast(dequant(QTensor(out, odt, scales, None, dt, scale_dtypes=sdts or None)), dt), lqt, rqt
+
+
+# ----------------------------------------------------------------------------
+# conv_general_dilated (aqt_conv_general.py:33-135), Flax layout, forward.
+
+
+def lax_conv_nhwc(lhs, rhs, strides, padding, rhs_dilation=None):
+  """jax.lax.conv_general_dilated for input N...C, kernel ...IO, output N...C in float64 (exact
+  for the integer-valued operands it is used on here)."""
+  ns = lhs.ndim - 2
+  dil = list(rhs_dilation) if rhs_dilation is not None else [1] * ns
+  kernel = rhs.shape[:ns]
+  eff = [(k - 1) * d + 1 for k, d in zip(kernel, dil)]
+  if isinstance(padding, str):
+    pads = []
+    for size, k, s in zip(lhs.shape[1:1 + ns], eff, strides):
+      if padding.upper() == 'VALID':
+        pads.append((0, 0))
+      else:
+        out = -(-size // s)
+        total = max((out - 1) * s + k - size, 0)
+        pads.append((total // 2, total - total // 2))
+  else:
+    pads = [tuple(p) for p in padding]
+  x = np.pad(lhs.astype(np.float64), [(0, 0)] + pads + [(0, 0)])
+  out_sizes = [(x.shape[1 + d] - eff[d]) // strides[d] + 1 for d in range(ns)]
+  out = np.zeros([lhs.shape[0]] + out_sizes + [rhs.shape[-1]], np.float64)
+  for tap in np.ndindex(*kernel):
+    sl = [slice(None)]
+    for d in range(ns):
+      start = tap[d] * dil[d]
+      sl.append(slice(start, start + (out_sizes[d] - 1) * strides[d] + 1, strides[d]))
+    out += np.tensordot(x[tuple(sl)], rhs[tap].astype(np.float64), axes=([-1], [0]))
+  return out
+
+
+def conv_general_dilated_fwd(lhs, rhs, dt, strides, padding, raw: RawCfg, rhs_dilation=None):
+  """The input shares a scale over all axes but the batch axis, the kernel over all but the
+  output features (aqt_conv_general.py:203-226); the convolution runs on the quantized values
+  held in the float dtype, the result is multiplied by the lhs scale, then the rhs scale."""
+  lhs, rhs = nm.cast(lhs, dt), nm.cast(rhs, dt)
+  rank = lhs.ndim
+  lq = copy.copy(raw.lhs)
+  lq.calib_shared_axes = list(range(1, rank))
+  rq = copy.copy(raw.rhs)
+  rq.calib_shared_axes = list(range(0, rank - 1))
+  lqt = quantize(lhs, dt, lq, None)
+  rqt = quantize(rhs, dt, rq, None)
+  acc = nm.cast(lax_conv_nhwc(np.asarray(lqt.qvalue, np.float32), np.asarray(rqt.qvalue, np.float32), strides,
+                              padding, rhs_dilation).astype(np.float32), dt)
+  sdts = [lqt.scale_dtype or dt] * len(lqt.scale) + [rqt.scale_dtype or dt] * len(rqt.scale)
+  out = dequant(QTensor(acc, dt, list(lqt.scale) + list(rqt.scale), None, dt, scale_dtypes=sdts or None))
+  return nm.cast(out, dt), lqt, rqt

@@ -1,0 +1,191 @@
+"""Quantized conv_general_dilated: oracle pins (CPU) and GPU parity, after aqt_conv_general_test.py."""
+import functools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import aqt_ref as R
+from oracle import numerics as nm
+from tests import gpu_util as U
+
+BITS = [(1, 1), (1, 2), (2, 1), (2, 2), (8, 8), (None, 8), (8, None), (None, None)]  # aqt_conv_general_test.py:53-62
+
+
+def _rand_unif(shape, maxval, seed, dt='f32'):
+  """aqt_conv_general_test.py:26-30."""
+  rng = np.random.default_rng(seed)
+  return nm.cast(rng.uniform(-maxval, maxval, shape).astype(np.float32), dt)
+
+
+def _qcfg(bits, po2=True):
+  # dot_general_raw_make (aqt_dot_general.py:99-156): one bit cannot hold zero, so the value
+  # stays in the float dtype
+  if bits is None:
+    return R.QuantizerCfg(bits=None)
+  return R.QuantizerCfg(bits=bits, po2_scale=po2, preserve_zero=bits != 1, keep_float=bits == 1)
+
+
+def test_oracle_conv_matches_scipy_correlate():
+  """The float convolution behind the oracle against scipy's n-d correlation: SAME and VALID,
+  strides and kernel dilation (a dilated kernel is the kernel with zeros inserted)."""
+  from scipy.signal import correlate
+  rng = np.random.default_rng(0)
+  lhs = rng.standard_normal((2, 7, 6, 3))
+  rhs = rng.standard_normal((3, 2, 3, 4))
+
+  def full(x, w, pads):
+    xp = np.pad(x, [(0, 0)] + pads + [(0, 0)])
+    out = np.zeros((x.shape[0], xp.shape[1] - w.shape[0] + 1, xp.shape[2] - w.shape[1] + 1, w.shape[-1]))
+    for n in range(x.shape[0]):
+      for o in range(w.shape[-1]):
+        out[n, :, :, o] = sum(correlate(xp[n, :, :, c], w[:, :, c, o], mode='valid') for c in range(x.shape[-1]))
+    return out
+
+  np.testing.assert_allclose(R.lax_conv_nhwc(lhs, rhs, (1, 1), 'VALID'), full(lhs, rhs, [(0, 0), (0, 0)]), atol=1e-12)
+  # SAME with an even kernel extent pads the extra element at the high end
+  np.testing.assert_allclose(R.lax_conv_nhwc(lhs, rhs, (1, 1), 'SAME'), full(lhs, rhs, [(1, 1), (0, 1)]), atol=1e-12)
+  np.testing.assert_allclose(R.lax_conv_nhwc(lhs, rhs, (2, 3), 'VALID'), full(lhs, rhs, [(0, 0), (0, 0)])[:, ::2, ::3],
+                             atol=1e-12)
+  np.testing.assert_allclose(R.lax_conv_nhwc(lhs, rhs, (1, 1), [(2, 1), (0, 3)]), full(lhs, rhs, [(2, 1), (0, 3)]),
+                             atol=1e-12)
+  dil = np.zeros((5, 4, 3, 4))
+  dil[::2, ::3] = rhs
+  np.testing.assert_allclose(R.lax_conv_nhwc(lhs, rhs, (1, 1), 'VALID', (2, 3)), full(lhs, dil, [(0, 0), (0, 0)]),
+                             atol=1e-12)
+  # SAME with stride 2 on 7 rows: 4 output rows, total padding (4-1)*2+3-7 = 2
+  got = R.lax_conv_nhwc(lhs, rhs, (2, 1), 'SAME')
+  np.testing.assert_allclose(got, full(lhs, rhs, [(1, 1), (0, 1)])[:, ::2], atol=1e-12)
+
+
+@pytest.mark.parametrize('lhs_bits,rhs_bits', BITS)
+def test_oracle_conv_equals_conv_of_fake_quantized(lhs_bits, rhs_bits):
+  """aqt_conv_general_test.py:63-103: with power-of-two scales the quantized convolution is
+  exactly the float convolution of the fake-quantized operands."""
+  lhs = _rand_unif((10, 4, 5, 20), 10.0, 0)
+  rhs = _rand_unif((3, 3, 20, 30), 20.0, 1)
+  raw = R.RawCfg(_qcfg(lhs_bits), _qcfg(rhs_bits))
+  out, lqt, rqt = R.conv_general_dilated_fwd(lhs, rhs, 'f32', (1, 1), 'SAME', raw)
+  if lhs_bits is not None:
+    assert lqt.scale[0].shape == (10, 1, 1, 1)
+  if rhs_bits is not None:
+    assert rqt.scale[0].shape == (1, 1, 1, 30)
+  fq = R.lax_conv_nhwc(R.dequant(lqt), R.dequant(rqt), (1, 1), 'SAME').astype(np.float32)
+  if lhs_bits is None or rhs_bits is None:
+    # the unquantized side makes the float sums inexact; only their order differs here
+    np.testing.assert_allclose(out, fq, rtol=2e-6, atol=1e-3)
+  else:
+    np.testing.assert_array_equal(out, fq)
+
+
+def _make(lhs_bits, rhs_bits, po2=True):
+  """aqt_conv_general_test.py:33-84: conv_general_dilated_make with power-of-two scales."""
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  raw = aqt_conv.conv_general_dilated_make(2, lhs_bits, rhs_bits, initialize_calibration=False)
+  for present, q in ((raw.lhs, raw.dg_quantizer.lhs), (raw.rhs, raw.dg_quantizer.rhs)):
+    if present:
+      if po2 and q.calibration is not None:
+        q.calibration = functools.partial(q.calibration, po2_scale=True)
+      q.init_calibration()
+  return raw
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('lhs_bits,rhs_bits', BITS)
+def test_conv_general_dilated(gpu, lhs_bits, rhs_bits):
+  """aqt_conv_general_test.py:63-103, and the same numbers as the oracle."""
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  from aqt_amd.v2 import aqt_quantizer
+  raw = _make(lhs_bits, rhs_bits)
+  lhs_np = _rand_unif((10, 4, 5, 20), 10.0, 0)
+  rhs_np = _rand_unif((3, 3, 20, 30), 20.0, 1)
+  lhs, rhs = U.to_dev(lhs_np, 'f32', gpu), U.to_dev(rhs_np, 'f32', gpu)
+  kwargs = dict(window_strides=(1, 1), padding='SAME',
+                dimension_numbers=aqt_conv.flax_conv_dimension_numbers(lhs.shape))
+  lhs_fq = aqt_quantizer.make_fake_quant(raw.dg_quantizer.lhs)(lhs)
+  rhs_fq = aqt_quantizer.make_fake_quant(raw.dg_quantizer.rhs)(rhs)
+  prod_fq = aqt_conv.lax_conv_general_dilated(lhs_fq, rhs_fq, **kwargs)
+  prod_aqt = aqt_conv.make_conv_general_dilated(raw)(lhs, rhs, **kwargs)
+  assert prod_aqt.shape == (10, 4, 5, 30) and prod_aqt.dtype == torch.float32
+  assert (prod_aqt == prod_fq).all()
+  want, _, _ = R.conv_general_dilated_fwd(lhs_np, rhs_np, 'f32', (1, 1), 'SAME',
+                                          R.RawCfg(_qcfg(lhs_bits), _qcfg(rhs_bits)))
+  if lhs_bits is None or rhs_bits is None:
+    np.testing.assert_allclose(prod_aqt.cpu().numpy(), want, rtol=2e-6, atol=1e-3)
+  else:
+    np.testing.assert_array_equal(prod_aqt.cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('lhs_bits,rhs_bits', BITS)
+def test_conv_general_dilated_quantized(gpu, lhs_bits, rhs_bits):
+  """aqt_conv_general_test.py:105-163: operands handed over as QTensors give the same result."""
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  raw = _make(lhs_bits, rhs_bits)
+  lhs = U.to_dev(_rand_unif((10, 4, 5, 20), 10.0, 0), 'f32', gpu)
+  rhs = U.to_dev(_rand_unif((3, 3, 20, 30), 20.0, 1), 'f32', gpu)
+  fn = aqt_conv.make_conv_general_dilated_with_qt(raw)
+  kwargs = dict(window_strides=(1, 1), padding='SAME',
+                dimension_numbers=aqt_conv.flax_conv_dimension_numbers(lhs.shape))
+  lhs_q, _ = raw.dg_quantizer.lhs.quant(lhs, calibration_axes=[0, 1, 2, 3])
+  rhs_q, _ = raw.dg_quantizer.rhs.quant(rhs, calibration_axes=[0, 1, 2])
+  out_no_quant, (lqt, rqt) = fn(lhs, rhs, lhs_qt=None, rhs_qt=None, **kwargs)
+  out_lhs_quant, _ = fn(torch.zeros_like(lhs), rhs, lhs_qt=lhs_q, rhs_qt=None, **kwargs)
+  out_rhs_quant, _ = fn(lhs, torch.zeros_like(rhs), lhs_qt=None, rhs_qt=rhs_q, **kwargs)
+  out_both_quant, _ = fn(torch.zeros_like(lhs), torch.zeros_like(rhs), lhs_qt=lhs_q, rhs_qt=rhs_q, **kwargs)
+  assert (out_no_quant == out_lhs_quant).all()
+  assert (out_no_quant == out_rhs_quant).all()
+  assert (out_no_quant == out_both_quant).all()
+  if lhs_bits is not None:
+    assert tuple(lqt.scale[0].shape) == (10, 1, 1, 1)
+  if rhs_bits is not None:
+    assert tuple(rqt.scale[0].shape) == (1, 1, 1, 30)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+@pytest.mark.parametrize('case', [
+    dict(lhs=(3, 9, 8, 16), rhs=(3, 3, 16, 24), strides=(2, 1), padding='SAME'),
+    dict(lhs=(2, 12, 11, 32), rhs=(2, 3, 32, 40), strides=(1, 2), padding='VALID', dil=(2, 1)),
+    dict(lhs=(4, 33, 48), rhs=(5, 48, 64), strides=(3,), padding=[(2, 1)]),
+    dict(lhs=(2, 5, 6, 4, 16), rhs=(2, 2, 2, 16, 8), strides=(1, 1, 2), padding='SAME'),
+    dict(lhs=(1, 8, 8, 64), rhs=(1, 1, 64, 128), strides=(1, 1), padding='VALID'),
+])
+def test_conv_strides_padding_dilation_rank_match_oracle(gpu, case, dt):
+  """int8 x int8 with ordinary (not power-of-two) abs-max scales: 1-d, 2-d and 3-d windows,
+  strides, explicit padding, kernel dilation, in both float dtypes; bit-exact to the oracle."""
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  ns = len(case['lhs']) - 2
+  raw = aqt_conv.conv_general_dilated_make(ns, 8, 8)
+  lhs_np = _rand_unif(case['lhs'], 3.0, 5, dt)
+  rhs_np = _rand_unif(case['rhs'], 0.5, 6, dt)
+  lhs, rhs = U.to_dev(lhs_np, dt, gpu), U.to_dev(rhs_np, dt, gpu)
+  out = aqt_conv.make_conv_general_dilated(raw)(
+      lhs, rhs, window_strides=case['strides'], padding=case['padding'], rhs_dilation=case.get('dil'),
+      dimension_numbers=aqt_conv.flax_conv_dimension_numbers(lhs.shape))
+  want, _, _ = R.conv_general_dilated_fwd(lhs_np, rhs_np, dt, case['strides'], case['padding'],
+                                          R.RawCfg(_qcfg(8, po2=False), _qcfg(8, po2=False)), case.get('dil'))
+  assert out.dtype == U.TORCH_DT[dt] and tuple(out.shape) == want.shape
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+def test_conv_layout_and_axis_assertions(gpu):
+  """aqt_conv_general.py:57-86: only the Flax layout, and the quantizers must share scales over
+  the axes that layout implies."""
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  lhs = torch.zeros((2, 4, 4, 8), device=gpu)
+  rhs = torch.zeros((3, 3, 8, 8), device=gpu)
+  fn = aqt_conv.make_conv_general_dilated(aqt_conv.conv_general_dilated_make(2, 8, 8))
+  dn = aqt_conv.flax_conv_dimension_numbers(lhs.shape)
+  with pytest.raises(AssertionError, match='Flax-particular layout'):
+    fn(lhs, rhs, (1, 1), 'SAME', dimension_numbers=None)
+  with pytest.raises(AssertionError, match='Flax-particular layout'):
+    fn(lhs, rhs, (1, 1), 'SAME', dimension_numbers=aqt_conv.ConvDimensionNumbers((0, 1, 2, 3), dn.rhs_spec, dn.out_spec))
+  wrong = aqt_conv.make_conv_general_dilated(aqt_conv.conv_general_dilated_make(1, 8, 8))
+  with pytest.raises(AssertionError, match='spatial'):
+    wrong(lhs, rhs, (1, 1), 'SAME', dimension_numbers=dn)
+  with pytest.raises(NotImplementedError):
+    fn(lhs, rhs, (1, 1), 'SAME', dimension_numbers=dn, feature_group_count=2)
+  # all-zero input: scales fall back to one, the output is zero
+  assert (fn(lhs, rhs, (1, 1), 'SAME', dimension_numbers=dn) == 0).all()
