@@ -71,7 +71,18 @@ class DecodePlan(ctypes.Structure):
 
 # name -> (restype, argtypes); every symbol include/aqtx.h declares
 _vp = ctypes.c_void_p
+class FpRoundPlan(ctypes.Structure):
+  _fields_ = [
+      ('count', ctypes.c_int64), ('noise_mod', ctypes.c_int64),
+      ('dtype', ctypes.c_int32), ('nexp', ctypes.c_int32), ('nmant', ctypes.c_int32),
+      ('has_subnormals', ctypes.c_int32), ('mode', ctypes.c_int32), ('partitionable', ctypes.c_int32),
+  ]
+
+
+FP_NEAREST, FP_NOISE_JAX_BITS, FP_NOISE_INDEX = 0, 1, 2
+
 SYMBOLS = {
+    'aqtx_fp_round': (ctypes.c_int, [ctypes.POINTER(FpRoundPlan), _vp, _vp, ctypes.POINTER(ctypes.c_uint32), _vp]),
     'aqtx_quantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp, _vp,
                                      ctypes.c_size_t, _vp]),
     'aqtx_quantize_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(QuantPlan)]),

@@ -352,6 +352,36 @@ def sum_tiles(x: torch.Tensor) -> torch.Tensor:
   return out
 
 
+def fp_round(x: torch.Tensor, *, nexp: int, nmant: int, has_subnormals: bool, key=None,
+             stochastic_rounding: bool = False, noise_mod: Optional[int] = None,
+             partitionable: bool = False) -> torch.Tensor:
+  """x (bf16 or f32, any shape) rounded to an emulated small float in the same dtype.
+
+  Stochastic rounding draws jax.random.bits(key, x.shape, uint16); `noise_mod` replaces the draw
+  by the index along the last axis (which must have that extent).
+  """
+  _require_gpu(x)
+  x = x.contiguous()
+  out = torch.empty_like(x)
+  plan = L.FpRoundPlan()
+  plan.count = x.numel()
+  plan.dtype = aqtx_dtype(x.dtype)
+  plan.nexp, plan.nmant, plan.has_subnormals = int(nexp), int(nmant), int(bool(has_subnormals))
+  plan.partitionable = int(partitionable)
+  k = None
+  if not stochastic_rounding:
+    plan.mode = L.FP_NEAREST
+  elif noise_mod is not None:
+    assert x.dim() >= 1 and x.shape[-1] == noise_mod
+    plan.mode, plan.noise_mod = L.FP_NOISE_INDEX, int(noise_mod)
+  else:
+    assert key is not None, 'stochastic rounding requested but the key is None'
+    plan.mode = L.FP_NOISE_JAX_BITS
+    k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))
+  L.check(L.lib().aqtx_fp_round(ctypes.byref(plan), _ptr(x), _ptr(out), k, _stream()))
+  return out
+
+
 def prng_split(key, num: int, partitionable: bool = False) -> np.ndarray:
   """jax.random.split(key, num) on raw uint32[2] key data (host side)."""
   k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))

@@ -198,6 +198,17 @@ def other_configs(dev):
   out['ragged_dot_int8_fwd_8192tok_8experts'] = {
       'ms_per_call': round(ms, 3), 'TOPS': round(gop / ms, 1),
       'contraction_only_ms': round(ms_gemm, 3), 'contraction_only_TOPS': round(gop / ms_gemm, 1)}
+  del x, w, xq, wq
+  # emulated fp4 (e2m1 with subnormals) in a bf16 container, 8192 x 14336: one read and one write per element
+  from aqt_amd.v2.numerics import fp_numerics
+  t = torch.randn(8192, 14336, device=dev).to(torch.bfloat16)
+  key = utils.prng_key(3)
+  ms_rn = timeit(lambda: fp_numerics.fp_round(t, cfg=fp_numerics.e2m1_ocp, key=None, stochastic_rounding=False))
+  ms_sr = timeit(lambda: fp_numerics.fp_round(t, cfg=fp_numerics.e2m1_ocp, key=key, stochastic_rounding=True))
+  gb = 2 * 2 * t.numel() / 1e9
+  out['fp_round_e2m1_bf16_8192x14336'] = {
+      'nearest_ms': round(ms_rn, 3), 'nearest_GB/s': round(gb / ms_rn * 1e3, 1),
+      'stochastic_ms': round(ms_sr, 3), 'stochastic_GB/s': round(gb / ms_sr * 1e3, 1)}
   return out
 
 

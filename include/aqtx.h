@@ -226,6 +226,34 @@ int aqtx_sum_tiles(const void* x, void* out, int64_t tiles, int64_t count, int32
                    void* stream);
 
 /*
+ * aqtx_fp_round: rounds x[count] (bf16 or f32) to an emulated small float with `nexp`
+ * exponent bits, `nmant` mantissa bits, smallest exponent 0, with or without subnormals, no
+ * NaN/inf codes, and writes the result in the same container dtype.  Replaces
+ * fp_numerics.fp_round for radix 2 (aqt/jax/v2/numerics/fp_numerics.py:279-459), which
+ * FpNumerics.vjp_fwd calls on the bf16 cast of its input (fp_numerics.py:632-640).
+ *   AQTX_FP_NEAREST        : half a truncated ulp is added to the bit pattern
+ *   AQTX_FP_NOISE_JAX_BITS : stochastic rounding with jax.random.bits(key, [count], uint16)
+ *   AQTX_FP_NOISE_INDEX    : stochastic rounding with noise = index % noise_mod, the
+ *                            reference's equi-spaced test noise along the last axis
+ *                            (test_noise_axis, fp_numerics.py:334-340)
+ */
+enum { AQTX_FP_NEAREST = 0, AQTX_FP_NOISE_JAX_BITS = 1, AQTX_FP_NOISE_INDEX = 2 };
+
+typedef struct aqtx_fp_round_plan {
+  int64_t count;
+  int64_t noise_mod;      /* AQTX_FP_NOISE_INDEX only: 1..65536 */
+  int32_t dtype;          /* AQTX_BF16 | AQTX_F32 */
+  int32_t nexp;           /* 0..7 */
+  int32_t nmant;          /* below the container's mantissa width (7 / 23) */
+  int32_t has_subnormals;
+  int32_t mode;
+  int32_t partitionable;  /* jax_threefry_partitionable layout of the random bits */
+} aqtx_fp_round_plan;
+
+int aqtx_fp_round(const aqtx_fp_round_plan* plan, const void* x, void* out,
+                  const uint32_t key_host[2], void* stream);
+
+/*
  * Plan of the serving contraction out[m, n] = dequant(quant(x)[m, k] * W[n, k]^T)
  * with a pre-quantized weight (QTensor: int8 qvalue + per-output-channel scale)
  * and per-token dynamic int8 quantisation of the activations, m <= 64.
