@@ -51,6 +51,10 @@ class QuantizerCfg:
   round: bool = True
   keep_float: bool = False  # numerics.dtype = None: qvalue stays in the input dtype
   key: Optional[np.ndarray] = None  # Context.key
+  # (full shape, per-axis index arrays): the tensor being quantized is the sub-block
+  # full[np.ix_(*indices)] of a larger one and draws that tensor's noise at its own positions
+  # (for checking slices of tensors too large to restate whole; 'jax.uniform' noise only)
+  noise_window: Any = None
 
   def is_int(self):
     return isinstance(self.bits, int)
@@ -190,6 +194,15 @@ def jax_uniform_noise(shape, key, sharing_axes=()):
   return prng.uniform(key, ns, PARTITIONABLE) - np.float32(0.5)
 
 
+def jax_uniform_noise_window(shape, key, window, kind='jax.uniform', sharing_axes=()):
+  """jax_uniform_noise of the enclosing tensor, read at the positions of a sub-block."""
+  assert kind == 'jax.uniform' and not sharing_axes
+  full_shape, indices = window
+  assert tuple(len(i) for i in indices) == tuple(shape)
+  flat = np.ravel_multi_index(np.ix_(*[np.asarray(i, np.int64) for i in indices]), full_shape)
+  return prng.uniform_at(key, int(np.prod(full_shape, dtype=np.int64)), flat, PARTITIONABLE) - np.float32(0.5)
+
+
 def random_centered_uniform_noise(shape, key, sharing_axes=()):
   """stochastic_rounding.py:50-78 ('custom-1')."""
   ns = _noise_shape(shape, sharing_axes)
@@ -207,7 +220,10 @@ def int_vjp_fwd(x, dt, q: QuantizerCfg):
     assert q.key is not None, 'noise_fn is set but no key in Context'
     fn = {'jax.uniform': jax_uniform_noise,
           'custom-1': random_centered_uniform_noise}[q.noise]
-    noise = fn(x.shape, q.key, q.noise_sharing_axes)
+    if q.noise_window is not None:
+      noise = jax_uniform_noise_window(x.shape, q.key, q.noise_window, q.noise, q.noise_sharing_axes)
+    else:
+      noise = fn(x.shape, q.key, q.noise_sharing_axes)
     # x (dt) + noise (f32) promotes to f32; one f32 rounding, then astype(dt).
     x = nm.cast(x.astype(np.float32) + noise, dt)
   if q.clip:

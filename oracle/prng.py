@@ -91,6 +91,33 @@ def random_bits(key, shape, bit_width=32, partitionable=False):
   return parts.reshape(-1)[:size].astype(out_dtype).reshape(shape)
 
 
+def random_bits_at(key, total, idx, partitionable=False):
+  """jax.random.bits(key, (total,), uint32)[idx] without drawing the other elements: word i of
+  the first half of the counters is lane 0 of block (i, i + half), word i of the second half is
+  lane 1 of block (i - half, i); an odd total pads one zero counter (see _threefry_2x32_flat)."""
+  key = np.asarray(key, np.uint32)
+  idx = np.asarray(idx, np.int64)
+  assert idx.size == 0 or (idx.min() >= 0 and idx.max() < total)
+  flat = idx.ravel()
+  if partitionable:
+    b1, b2 = threefry2x32(key[0], key[1], (flat >> 32).astype(np.uint32), (flat & 0xFFFFFFFF).astype(np.uint32))
+    return (b1 ^ b2).reshape(idx.shape)
+  half = (int(total) + 1) // 2
+  first = flat < half
+  c0 = np.where(first, flat, flat - half)
+  c1 = np.where(first, flat + half, flat)
+  c1 = np.where(c1 < total, c1, 0)  # the padded counter of an odd total
+  y0, y1 = threefry2x32(key[0], key[1], c0.astype(np.uint32), c1.astype(np.uint32))
+  return np.where(first, y0, y1).reshape(idx.shape)
+
+
+def uniform_at(key, total, idx, partitionable=False):
+  """jax.random.uniform(key, (total,))[idx]."""
+  bits = random_bits_at(key, total, idx, partitionable)
+  fbits = (bits >> np.uint32(9)) | np.uint32(0x3F800000)
+  return np.maximum(np.float32(0.0), fbits.view(np.float32) - np.float32(1.0))
+
+
 def uniform(key, shape, partitionable=False):
   """jax.random.uniform(key, shape) (float32, [0, 1))."""
   bits = random_bits(key, shape, 32, partitionable)

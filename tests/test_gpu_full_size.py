@@ -1,0 +1,122 @@
+"""The benchmark configuration at its full size (bf16 [8192, 4096] x [4096, 14336], forward and
+backward, int8): the product runs the whole problem, the oracle restates slices of it.
+
+What makes slices exact: the forward quantizes the lhs per row and the rhs per column, so
+out[rows] needs lhs[rows] and the whole rhs only; dlhs[rows] needs g[rows] (quantized per row
+over N) and the whole rhs residual; drhs[:, cols] needs g[:, cols] (quantized per column over M)
+and the whole lhs residual.  Stochastic-rounding noise is drawn for the whole gradient tensor;
+the oracle reads it at the positions of the slice (QuantizerCfg.noise_window).
+"""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import aqt_ref as R
+from oracle import numerics as nm
+from oracle import prng
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+M, K, N = 8192, 4096, 14336
+MATMUL = (((1,), (0,)), ((), ()))
+# tile and half-tensor boundaries (the noise counters pair element i with i + M*N/2) and a random spread
+ROWS = np.unique(np.concatenate([[0, 1, 127, 128, 255, 256, 2047, 4095, 4096, 4097, 8190, 8191],
+                                 np.random.default_rng(1).integers(0, M, 12)]))
+COLS = np.unique(np.concatenate([[0, 1, 63, 64, 255, 256, 7167, 7168, 14334, 14335],
+                                 np.random.default_rng(2).integers(0, N, 14)]))
+
+
+def make_problem():
+  rng = np.random.default_rng(2024)
+
+  def normal_bf16(shape, scale):
+    x = rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)
+    return (x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)  # truncated: representable in bf16
+
+  lhs, rhs, g = normal_bf16((M, K), 1.0), normal_bf16((K, N), 0.02), normal_bf16((M, N), 1e-3)
+  # outliers so that the abs-max is not the same everywhere
+  lhs[ROWS[:3], 5] = nm.cast(lhs[ROWS[:3], 5] * np.float32(30), 'bf16')
+  g[7, COLS[:3]] = nm.cast(g[7, COLS[:3]] * np.float32(50), 'bf16')
+  return lhs, rhs, g
+
+
+@pytest.fixture(scope='module')
+def problem():
+  return make_problem()
+
+
+def _product(problem, gpu, sr, key):
+  from aqt_amd.v2 import config
+  lhs, rhs, g = problem
+  L = U.to_dev(lhs, 'bf16', gpu).requires_grad_(True)
+  Rr = U.to_dev(rhs, 'bf16', gpu).requires_grad_(True)
+  cfg = config.fully_quantized(fwd_bits=8, bwd_bits=8, use_stochastic_rounding=sr)
+  cfg = config.set_context(cfg, key, None)
+  out = cfg(L, Rr, MATMUL)
+  out.backward(U.to_dev(g, 'bf16', gpu))
+  torch.cuda.synchronize()
+  return out.detach(), L.grad, Rr.grad
+
+
+def _one_side(g, fwd, ocfg, lhs_side):
+  """One of the two backward contractions of dg_core_vjp_bwd (aqt_dot_general.py:1178-1221)."""
+  y_res, raw = (fwd.lhs_res, ocfg.drhs) if lhs_side else (fwd.rhs_res, ocfg.dlhs)
+  dims, out_axes = R.bwd_dimension_numbers(MATMUL, lhs_side, g.ndim, y_res.x.ndim)
+  out, _, _, _ = R.dg_raw(g, 'bf16', y_res, None, dims, raw)
+  return np.transpose(out, out_axes)
+
+
+def _check(problem, gpu, sr):
+  lhs, rhs, g = problem
+  key = prng.prng_key(99)
+  out, dlhs, drhs = _product(problem, gpu, sr, key)
+  assert out.shape == (M, N) and dlhs.shape == (M, K) and drhs.shape == (K, N)
+  ocfg = R.set_context(R.fully_quantized(8, 8, use_stochastic_rounding=sr), key if sr else None)
+
+  # rows: forward and dlhs
+  rcfg = copy.deepcopy(ocfg)
+  if sr:
+    rcfg.dlhs.lhs.noise_window = ((M, N), (ROWS, np.arange(N)))
+  f_r = R.dg_fwd(lhs[ROWS], rhs, 'bf16', MATMUL, rcfg)
+  rows_t = torch.from_numpy(ROWS).to(gpu)
+  np.testing.assert_array_equal(out[rows_t].float().cpu().numpy(), f_r.out)
+  np.testing.assert_array_equal(dlhs[rows_t].float().cpu().numpy(), _one_side(g[ROWS], f_r, rcfg, False))
+  del f_r
+
+  # columns: forward and drhs
+  ccfg = copy.deepcopy(ocfg)
+  if sr:
+    ccfg.drhs.lhs.noise_window = ((M, N), (np.arange(M), COLS))
+  f_c = R.dg_fwd(lhs, rhs[:, COLS], 'bf16', MATMUL, ccfg)
+  cols_t = torch.from_numpy(COLS).to(gpu)
+  np.testing.assert_array_equal(out[:, cols_t].float().cpu().numpy(), f_c.out)
+  np.testing.assert_array_equal(drhs[:, cols_t].float().cpu().numpy(), _one_side(g[:, COLS], f_c, ccfg, True))
+
+  # whole-tensor sanity that no slice can give: finite everywhere, and the quantized product
+  # stays within the quantization error of the float one (checksums over all rows and columns; a
+  # misplaced tile or a wrong scale would show as an error of order one)
+  for t in (out, dlhs, drhs):
+    assert torch.isfinite(t).all()
+  L, Rr, G = (U.to_dev(x, 'bf16', gpu).float() for x in (lhs, rhs, g))
+  ones_n = torch.ones(N, device=gpu)
+  want_rowsum = L @ (Rr @ ones_n)
+  got_rowsum = out.float() @ ones_n
+  rel = (got_rowsum - want_rowsum).norm() / want_rowsum.norm()
+  assert rel < 0.06, rel
+  want_dl = G @ (Rr.t() @ torch.ones(K, device=gpu))
+  rel = (dlhs.float() @ torch.ones(K, device=gpu) - want_dl).norm() / want_dl.norm()
+  assert rel < 0.06, rel
+  want_dr = (L.t() @ G) @ ones_n
+  rel = (drhs.float() @ ones_n - want_dr).norm() / want_dr.norm()
+  assert rel < 0.06, rel
+
+
+def test_full_size_round_to_nearest(problem, gpu):
+  _check(problem, gpu, sr=False)
+
+
+def test_full_size_stochastic_rounding(problem, gpu):
+  _check(problem, gpu, sr=True)

@@ -77,3 +77,23 @@ def test_uniform_range_and_mean():
   u = prng.uniform(prng.prng_key(1), (200000,))
   assert u.min() >= 0.0 and u.max() < 1.0
   assert abs(u.mean() - 0.5) < 3e-3
+
+
+@pytest.mark.parametrize('partitionable', [False, True])
+@pytest.mark.parametrize('total', [1, 2, 7, 64, 1001])
+def test_bits_at_positions_match_the_whole_draw(total, partitionable):
+  key = prng.prng_key(11)
+  whole = prng.random_bits(key, (total,), 32, partitionable)
+  idx = np.random.default_rng(total).integers(0, total, size=(3, 5))
+  np.testing.assert_array_equal(prng.random_bits_at(key, total, idx, partitionable), whole[idx])
+  np.testing.assert_array_equal(prng.uniform_at(key, total, np.arange(total), partitionable),
+                                prng.uniform(key, (total,), partitionable))
+
+
+def test_noise_window_is_the_slice_of_the_full_noise():
+  from oracle import aqt_ref as R
+  key = prng.prng_key(5)
+  full = R.jax_uniform_noise((6, 10), key)
+  rows, cols = [4, 1, 5], [0, 9, 3, 2]
+  got = R.jax_uniform_noise_window((3, 4), key, ((6, 10), (rows, cols)))
+  np.testing.assert_array_equal(got, full[np.ix_(rows, cols)])
