@@ -53,7 +53,8 @@ class QuantizerCfg:
   key: Optional[np.ndarray] = None  # Context.key
   # (full shape, per-axis index arrays): the tensor being quantized is the sub-block
   # full[np.ix_(*indices)] of a larger one and draws that tensor's noise at its own positions
-  # (for checking slices of tensors too large to restate whole; 'jax.uniform' noise only)
+  # (for checking slices of tensors too large to restate whole; 'jax.uniform' noise and the fp8
+  # mantissa noise)
   noise_window: Any = None
 
   def is_int(self):
@@ -197,10 +198,8 @@ def jax_uniform_noise(shape, key, sharing_axes=()):
 def jax_uniform_noise_window(shape, key, window, kind='jax.uniform', sharing_axes=()):
   """jax_uniform_noise of the enclosing tensor, read at the positions of a sub-block."""
   assert kind == 'jax.uniform' and not sharing_axes
-  full_shape, indices = window
-  assert tuple(len(i) for i in indices) == tuple(shape)
-  flat = np.ravel_multi_index(np.ix_(*[np.asarray(i, np.int64) for i in indices]), full_shape)
-  return prng.uniform_at(key, int(np.prod(full_shape, dtype=np.int64)), flat, PARTITIONABLE) - np.float32(0.5)
+  total, flat = _window_flat_index(shape, window)
+  return prng.uniform_at(key, total, flat, PARTITIONABLE) - np.float32(0.5)
 
 
 def random_centered_uniform_noise(shape, key, sharing_axes=()):
@@ -240,8 +239,16 @@ def int_vjp_fwd(x, dt, q: QuantizerCfg):
   return x.astype(np.float32), dt
 
 
-def fp_mantissa_round(x, dt, mantissa_bits, key):
-  """fp8_numerics.py:36-64: add masked random bits to the mantissa, truncate."""
+def _window_flat_index(shape, window):
+  full_shape, indices = window
+  assert tuple(len(i) for i in indices) == tuple(shape)
+  flat = np.ravel_multi_index(np.ix_(*[np.asarray(i, np.int64) for i in indices]), full_shape)
+  return int(np.prod(full_shape, dtype=np.int64)), flat
+
+
+def fp_mantissa_round(x, dt, mantissa_bits, key, window=None):
+  """fp8_numerics.py:36-64: add masked random bits to the mantissa, truncate.  `window`: x is a
+  sub-block of a larger tensor and takes that tensor's bits at its own positions."""
   assert dt in (BF16, F32)
   if dt == BF16:
     nmant, width = 7, 16
@@ -251,7 +258,11 @@ def fp_mantissa_round(x, dt, mantissa_bits, key):
     u = np.ascontiguousarray(x, np.float32).view(np.uint32).copy()
   noise_bits = nmant - mantissa_bits
   mask = u.dtype.type((1 << noise_bits) - 1)
-  noise = prng.random_bits(key, x.shape, width, PARTITIONABLE) & mask
+  if window is not None:
+    total, flat = _window_flat_index(x.shape, window)
+    noise = prng.random_bits_at(key, total, flat, PARTITIONABLE, width).astype(u.dtype) & mask
+  else:
+    noise = prng.random_bits(key, x.shape, width, PARTITIONABLE) & mask
   with np.errstate(over='ignore'):
     u = (u + noise) & ~mask
   return nm.from_bf16_bits(u) if dt == BF16 else u.view(np.float32)
@@ -262,7 +273,7 @@ def fp8_vjp_fwd(x, dt, q: QuantizerCfg):
   mant = 3 if q.bits == 'e4m3' else 2
   if q.fp8_sr:
     assert q.key is not None
-    x = fp_mantissa_round(x, dt, mant, q.key)
+    x = fp_mantissa_round(x, dt, mant, q.key, q.noise_window)
   b = np.float32(quant_bound(q))
   x = np.clip(x, -b, b)
   x = nm.to_e4m3fn(x) if q.bits == 'e4m3' else nm.to_e5m2(x)

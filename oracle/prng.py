@@ -91,17 +91,25 @@ def random_bits(key, shape, bit_width=32, partitionable=False):
   return parts.reshape(-1)[:size].astype(out_dtype).reshape(shape)
 
 
-def random_bits_at(key, total, idx, partitionable=False):
-  """jax.random.bits(key, (total,), uint32)[idx] without drawing the other elements: word i of
-  the first half of the counters is lane 0 of block (i, i + half), word i of the second half is
-  lane 1 of block (i - half, i); an odd total pads one zero counter (see _threefry_2x32_flat)."""
+def random_bits_at(key, total, idx, partitionable=False, bit_width=32):
+  """jax.random.bits(key, (total,), uint{bit_width})[idx] without drawing the other elements.
+
+  32 bits: word i of the first half of the counters is lane 0 of block (i, i + half), word i of
+  the second half is lane 1 of block (i - half, i); an odd count pads one zero counter (see
+  _threefry_2x32_flat).  16 bits: element i is the low (even i) or high half of word i // 2 of
+  the ceil(total / 2) words drawn (see random_bits)."""
   key = np.asarray(key, np.uint32)
   idx = np.asarray(idx, np.int64)
+  assert bit_width in (16, 32)
   assert idx.size == 0 or (idx.min() >= 0 and idx.max() < total)
   flat = idx.ravel()
   if partitionable:
     b1, b2 = threefry2x32(key[0], key[1], (flat >> 32).astype(np.uint32), (flat & 0xFFFFFFFF).astype(np.uint32))
-    return (b1 ^ b2).reshape(idx.shape)
+    bits = b1 ^ b2
+    return (bits & np.uint32(0xFFFF) if bit_width == 16 else bits).reshape(idx.shape)
+  if bit_width == 16:
+    words = random_bits_at(key, -(-int(total) // 2), flat // 2, False, 32)
+    return ((words >> (np.uint32(16) * (flat % 2).astype(np.uint32))) & np.uint32(0xFFFF)).reshape(idx.shape)
   half = (int(total) + 1) // 2
   first = flat < half
   c0 = np.where(first, flat, flat - half)

@@ -120,3 +120,86 @@ def test_full_size_round_to_nearest(problem, gpu):
 
 def test_full_size_stochastic_rounding(problem, gpu):
   _check(problem, gpu, sr=True)
+
+
+def _normal_bf16(rng, shape, scale):
+  x = rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)
+  return (x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)
+
+
+def test_full_size_int4_weight_tiled(gpu):
+  """int4 weights [8192, 28672] in groups of 128 along the contraction axis, int8 activations
+  [2048, 8192], forward: lhs scales are per (row, tile), rhs scales per (tile, column), so
+  out[rows, cols] needs those rows and columns only."""
+  from aqt_amd.v2 import aqt_dot_general as aqt
+  from aqt_amd.v2 import config
+  from aqt_amd.v2 import tiled_dot_general as T
+  m, k, n, ts = 2048, 8192, 28672, 128
+  rng = np.random.default_rng(5)
+  lhs, rhs = _normal_bf16(rng, (m, k), 1.0), _normal_bf16(rng, (k, n), 0.015)
+  rows = np.unique(np.concatenate([[0, 1, 127, 128, 2047], rng.integers(0, m, 8)]))
+  cols = np.unique(np.concatenate([[0, 1, 255, 256, 14335, 14336, 28671], rng.integers(0, n, 10)]))
+  dg = config.set_context(aqt.dot_general_make(8, 4), None, None)
+  tcfg = T.Cfg(lhs=T.TensorTiling([T.AxisTiling(axis=1, tile_size=ts)], []),
+               rhs=T.TensorTiling([T.AxisTiling(axis=0, tile_size=ts)], []))
+  with torch.no_grad():
+    out = T.tiled_dot_general(tcfg, U.to_dev(lhs, 'bf16', gpu), U.to_dev(rhs, 'bf16', gpu), MATMUL, dot_general=dg)
+  assert tuple(out.shape) == (m, n) and out.dtype == torch.bfloat16 and torch.isfinite(out).all()
+  want, _ = R.tiled_dg_fwd(lhs[rows], np.ascontiguousarray(rhs[:, cols]), 'bf16', ts, R.dot_general_make(8, 4))
+  got = out[torch.from_numpy(rows).to(gpu)][:, torch.from_numpy(cols).to(gpu)]
+  np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+
+
+def test_full_size_fp8_einsum(gpu):
+  """'bsd,dhk->bshk' with batch 8, sequence 4096, d 4096, 32 heads of 128: e4m3 forward, e5m2
+  gradients with mantissa stochastic rounding, per-tensor scales.  With one scale per tensor the
+  quantization is elementwise, so any block of the three results can be restated from the
+  matching blocks of the operands, provided each block holds its tensor's largest element (the
+  blocks are chosen that way).  Tolerance as for the small fp8 cases: the MFMA sums in float32
+  in its own order."""
+  from aqt_amd.v2 import aqt_dot_general as aqt
+  from aqt_amd.v2 import config
+  b, s, d, h, kh = 8, 4096, 4096, 32, 128
+  bs, hk = b * s, h * kh
+  rng = np.random.default_rng(6)
+  lhs2, rhs2, g2 = _normal_bf16(rng, (bs, d), 1.0), _normal_bf16(rng, (d, hk), 0.02), _normal_bf16(rng, (bs, hk), 1e-3)
+  rl, cl = np.unravel_index(np.abs(lhs2).argmax(), lhs2.shape)
+  rr, cr = np.unravel_index(np.abs(rhs2).argmax(), rhs2.shape)
+  rg, cg = np.unravel_index(np.abs(g2).argmax(), g2.shape)
+  rows = np.unique(np.concatenate([[rl, rg, 0, bs - 1, bs // 2], rng.integers(0, bs, 6)]))
+  dsel = np.unique(np.concatenate([[cl, rr, 0, d - 1], rng.integers(0, d, 8)]))
+  cols = np.unique(np.concatenate([[cr, cg, 0, hk - 1, hk // 2], rng.integers(0, hk, 8)]))
+
+  key = prng.prng_key(17)
+  cfg = config.config_v4(fwd_bits='e4m3', dlhs_bits='e5m2', drhs_bits='e5m2')
+  ocfg = R.config_v4('e4m3', 'e5m2', 'e5m2')
+  for raw, oraw in ((cfg.fwd, ocfg.fwd), (cfg.dlhs, ocfg.dlhs), (cfg.drhs, ocfg.drhs)):
+    raw.dg_quantizer.lhs.calib_shared_axes = raw.dg_quantizer.rhs.calib_shared_axes = 'per_tensor'
+    oraw.lhs.calib_shared_axes = oraw.rhs.calib_shared_axes = 'per_tensor'
+  cfg = config.set_context(cfg, key, None)
+  ocfg = R.set_context(ocfg, key)
+  x = U.to_dev(lhs2, 'bf16', gpu).reshape(b, s, d).requires_grad_(True)
+  w = U.to_dev(rhs2, 'bf16', gpu).reshape(d, h, kh).requires_grad_(True)
+  out = aqt.einsum('bsd,dhk->bshk', x, w, cfg)
+  out.backward(U.to_dev(g2, 'bf16', gpu).reshape(b, s, h, kh))
+  out2, dl2, dr2 = out.detach().reshape(bs, hk), x.grad.reshape(bs, d), w.grad.reshape(d, hk)
+  for t in (out2, dl2, dr2):
+    assert torch.isfinite(t).all()
+  tr, td, tc = (torch.from_numpy(i).to(gpu) for i in (rows, dsel, cols))
+
+  def close(got, want, what):
+    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=2.0 ** -7, atol=2.0 ** -9 * np.abs(want).max(),
+                               err_msg=what)
+
+  f = R.dg_fwd(lhs2[rows], np.ascontiguousarray(rhs2[:, cols]), 'bf16', MATMUL, ocfg)
+  close(out2[tr][:, tc], f.out, 'out')
+  # dlhs[rows, dsel] = g[rows, :] . rhs[dsel, :]^T
+  c1 = copy.deepcopy(ocfg)
+  c1.dlhs.lhs.noise_window = ((bs, hk), (rows, np.arange(hk)))
+  f1 = R.dg_fwd(lhs2[np.ix_(rows, dsel)], rhs2[dsel], 'bf16', MATMUL, c1)
+  close(dl2[tr][:, td], _one_side(g2[rows], f1, c1, False), 'dlhs')
+  # drhs[dsel, cols] = lhs[:, dsel]^T . g[:, cols]
+  c2 = copy.deepcopy(ocfg)
+  c2.drhs.lhs.noise_window = ((bs, hk), (np.arange(bs), cols))
+  f2 = R.dg_fwd(np.ascontiguousarray(lhs2[:, dsel]), rhs2[np.ix_(dsel, cols)], 'bf16', MATMUL, c2)
+  close(dr2[td][:, tc], _one_side(np.ascontiguousarray(g2[:, cols]), f2, c2, True), 'drhs')

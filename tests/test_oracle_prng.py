@@ -88,6 +88,8 @@ def test_bits_at_positions_match_the_whole_draw(total, partitionable):
   np.testing.assert_array_equal(prng.random_bits_at(key, total, idx, partitionable), whole[idx])
   np.testing.assert_array_equal(prng.uniform_at(key, total, np.arange(total), partitionable),
                                 prng.uniform(key, (total,), partitionable))
+  halves = prng.random_bits(key, (total,), 16, partitionable)
+  np.testing.assert_array_equal(prng.random_bits_at(key, total, idx, partitionable, 16), halves[idx])
 
 
 def test_noise_window_is_the_slice_of_the_full_noise():
@@ -97,3 +99,15 @@ def test_noise_window_is_the_slice_of_the_full_noise():
   rows, cols = [4, 1, 5], [0, 9, 3, 2]
   got = R.jax_uniform_noise_window((3, 4), key, ((6, 10), (rows, cols)))
   np.testing.assert_array_equal(got, full[np.ix_(rows, cols)])
+
+
+def test_fp8_mantissa_noise_window_is_the_slice_of_the_full_draw():
+  from oracle import aqt_ref as R
+  from oracle import numerics as nm
+  key = prng.prng_key(8)
+  x = nm.cast(np.random.default_rng(0).standard_normal((7, 9)).astype(np.float32), 'bf16')
+  rows, cols = [6, 0, 3], [8, 1, 2, 5]
+  for dt in ('bf16', 'f32'):
+    full = R.fp_mantissa_round(x, dt, 2, key)
+    got = R.fp_mantissa_round(x[np.ix_(rows, cols)], dt, 2, key, ((7, 9), (rows, cols)))
+    np.testing.assert_array_equal(got, full[np.ix_(rows, cols)])
