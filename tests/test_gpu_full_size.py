@@ -203,3 +203,32 @@ def test_full_size_fp8_einsum(gpu):
   c2.drhs.lhs.noise_window = ((bs, hk), (np.arange(bs), cols))
   f2 = R.dg_fwd(np.ascontiguousarray(lhs2[:, dsel]), rhs2[np.ix_(dsel, cols)], 'bf16', MATMUL, c2)
   close(dr2[td][:, tc], _one_side(np.ascontiguousarray(g2[:, cols]), f2, c2, True), 'drhs')
+
+
+@pytest.mark.parametrize('m', [1, 8, 32, 64])
+@pytest.mark.parametrize('int4', [False, True])
+def test_full_size_serving_weight(gpu, m, int4):
+  """The serving shapes against the 4096 x 14336 weight (held [n, k]; int8, or int4 packed two
+  per byte): per-token activation quantization in the call, per-output-channel weight scales,
+  so the oracle restates a sample of output columns."""
+  from aqt_amd import _lib as L
+  from aqt_amd import ops
+  n, k = 14336, 4096
+  rng = np.random.default_rng(40 + m)
+  x = U.rand((m, k), 'bf16', 300 + m, outliers=True)
+  lim = 7 if int4 else 127
+  wq = rng.integers(-lim, lim + 1, size=(n, k)).astype(np.int8)
+  ws = np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(2e-4) + np.float32(1e-5)
+  cols = np.unique(np.concatenate([[0, 1, 15, 16, 63, 64, n - 65, n - 64, n - 1], rng.integers(0, n, 300)]))
+  xqt = R.quantize(x, 'bf16', R.QuantizerCfg(bits=8), calibration_axes=[1])
+  acc = (xqt.qvalue.astype(np.float64) @ wq[cols].astype(np.float64).T).astype(np.int32)  # exact: |acc| < 2^53
+  want = R.dequant(R.QTensor(acc, 'i32', [xqt.scale[0].reshape(-1, 1), ws[cols].reshape(1, -1)], None, 'bf16',
+                             scale_dtypes=[xqt.scale_dtype, 'f32']))
+  w_t = torch.from_numpy(wq).to(gpu)
+  out, xs, xq = ops.decode(U.to_dev(x, 'bf16', gpu), ops.pack_i4(w_t) if int4 else w_t, torch.from_numpy(ws).to(gpu),
+                           quant_bound=127.5, clip_bound=127.0, w_scale_dtype=torch.float32, want_xq=True,
+                           w_dtype=L.I4P if int4 else L.I8)
+  assert tuple(out.shape) == (m, n) and torch.isfinite(out).all()
+  np.testing.assert_array_equal(xq.cpu().numpy(), xqt.qvalue.astype(np.int8))
+  np.testing.assert_array_equal(xs.cpu().numpy(), xqt.scale[0].reshape(-1))
+  np.testing.assert_array_equal(out[:, torch.from_numpy(cols).to(gpu)].float().cpu().numpy(), want)
