@@ -4,8 +4,10 @@
 // pattern, clear the truncated mantissa bits, clamp the magnitude pattern between the smallest
 // and largest normal value; magnitudes below the smallest normal are rounded linearly
 // (formats with subnormals) or to +-1 (formats without).  One read and one write per element;
-// HBM-bound when deterministic, threefry-bound with random bits (one block per two elements).
+// HBM-bound when deterministic, threefry-bound with random bits (one block per four elements
+// in the paired kernel, per two otherwise).
 #include "common.h"
+#include <type_traits>
 #include "threefry.h"
 
 namespace aqtx {
@@ -147,6 +149,71 @@ __global__ __launch_bounds__(256) void fp_round_kernel(const FpArgs a) {
   }
 }
 
+// jax.random.bits in its original layout: one threefry block yields word w (first half of the words)
+// and word w + half (second half), i.e. the 16-bit draws of elements 2w, 2w + 1 and of the two
+// elements `2 * half` further on.  A lane takes VEC elements from each region so that no output
+// of a block is thrown away.  Needs 2 * half to be a multiple of VEC (16-byte alignment of the
+// second region).
+template <bool BF16, int VEC>
+__global__ __launch_bounds__(256) void fp_round_paired_kernel(const FpArgs a) {
+  using T = typename std::conditional<BF16, uint16_t, uint32_t>::type;
+  const int64_t second = 2 * (int64_t)a.gen.half;
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (i0 >= second) return;
+  const T* x = reinterpret_cast<const T*>(a.x);
+  T* out = reinterpret_cast<T*>(a.out);
+  uint32_t lo[VEC], hi[VEC];
+  const int64_t i1 = i0 + second;
+  const bool full0 = i0 + VEC <= (second < a.count ? second : a.count);
+  const bool full1 = i1 + VEC <= a.count;
+  auto load = [&](int64_t base, bool full, int64_t limit, uint32_t* bits) {
+    if (full) {
+      const uint4 v = *reinterpret_cast<const uint4*>(x + base);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        if constexpr (BF16) bits[e] = (w[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+        else bits[e] = w[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) bits[e] = base + e < limit ? (uint32_t)x[base + e] : 0u;
+    }
+  };
+  load(i0, full0, second < a.count ? second : a.count, lo);
+  load(i1, full1, a.count, hi);
+#pragma unroll
+  for (int e = 0; e < VEC; e += 2) {
+    const uint32_t w = (uint32_t)((i0 + e) >> 1);
+    uint32_t c1 = w + a.gen.half;
+    c1 = c1 < a.gen.nwords ? c1 : 0u;
+    const U2 blk = threefry2x32(a.gen.k0, a.gen.k1, w, c1);
+    lo[e] = round_pattern<BF16>(lo[e], blk.x & 0xFFFFu, a);
+    lo[e + 1] = round_pattern<BF16>(lo[e + 1], blk.x >> 16, a);
+    hi[e] = round_pattern<BF16>(hi[e], blk.y & 0xFFFFu, a);
+    hi[e + 1] = round_pattern<BF16>(hi[e + 1], blk.y >> 16, a);
+  }
+  auto store = [&](int64_t base, bool full, int64_t limit, const uint32_t* bits) {
+    if (full) {
+      uint4 o;
+      if constexpr (BF16) {
+        o = make_uint4(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16), bits[4] | (bits[5] << 16),
+                       bits[6] | (bits[7] << 16));
+      } else {
+        o = make_uint4(bits[0], bits[1], bits[2], bits[3]);
+      }
+      *reinterpret_cast<uint4*>(out + base) = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        if (base + e < limit) out[base + e] = (T)bits[e];
+      }
+    }
+  };
+  store(i0, full0, second < a.count ? second : a.count, lo);
+  store(i1, full1, a.count, hi);
+}
+
 }  // namespace
 }  // namespace aqtx
 
@@ -202,6 +269,13 @@ extern "C" int aqtx_fp_round(const aqtx_fp_round_plan* p, const void* x, void* o
   const int vec = aligned ? (p->dtype == AQTX_BF16 ? 8 : 4) : 2;
   const int64_t blocks = (p->count + 256 * vec - 1) / (256 * vec);
   AQTX_REQUIRE(blocks < (1ll << 31), "aqtx_fp_round: count too large for one launch");
+  if (p->mode == AQTX_FP_NOISE_JAX_BITS && !p->partitionable && aligned && (2 * (int64_t)a.gen.half) % vec == 0) {
+    const int64_t pblocks = (2 * (int64_t)a.gen.half + 256 * vec - 1) / (256 * vec);
+    if (p->dtype == AQTX_BF16) fp_round_paired_kernel<true, 8><<<(unsigned)pblocks, 256, 0, st>>>(a);
+    else fp_round_paired_kernel<false, 4><<<(unsigned)pblocks, 256, 0, st>>>(a);
+    AQTX_HIP_CHECK_LAUNCH("fp_round_paired_kernel");
+    return 0;
+  }
   if (p->dtype == AQTX_BF16) {
     if (aligned) fp_round_kernel<true, 8><<<(unsigned)blocks, 256, 0, st>>>(a);
     else fp_round_kernel<true, 2><<<(unsigned)blocks, 256, 0, st>>>(a);

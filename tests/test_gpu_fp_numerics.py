@@ -211,3 +211,17 @@ def test_fp_numerics_class_and_quantizer(gpu):
   assert vals <= {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0}
   np.testing.assert_array_equal(qt.dequant().float().cpu().numpy(),
                                 nm.cast(qt.qvalue.float().cpu().numpy() * scale, 'bf16'))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dt,count', [('bf16', 16 * 50 + 13), ('bf16', 16 * 50 + 15), ('bf16', 16), ('bf16', 8),
+                                      ('f32', 8 * 33 + 5), ('f32', 8 * 33 + 7), ('f32', 4), ('bf16', 1 << 20)])
+def test_stochastic_rounding_paired_blocks_ragged_ends(gpu, dt, count):
+  """Sizes at which the kernel that uses both words of a threefry block runs with a partly
+  filled last vector in either half of the tensor."""
+  from aqt_amd.v2.numerics import fp_numerics
+  x = U.rand((count,), dt, count % 97, scale=2.0)
+  key = prng.prng_key(count)
+  for name in ('e2m1_ocp', 'e3m0'):
+    got = fp_numerics.fp_round(U.to_dev(x, dt, gpu), cfg=_cfg(name), key=key, stochastic_rounding=True)
+    _eq_outside_nan(got, F.radix2_round(x, dt, F.CONFIGS[name], key, True), x)
