@@ -51,7 +51,9 @@ struct GroupedArgs {
 
 // EPI as in the dense kernel: 0 = bf16 out, both products rounded to bf16; 4 = bf16 out, first
 // product bf16, second f32; 1 = bf16 out, products in f32; 2 = f32 out.
-template <int EPI, bool PACKED>
+// ONE: a group is exactly one 128-byte stage (group = 128), which takes the branches on the
+// position inside a group out of the loop.
+template <int EPI, bool PACKED, bool ONE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_grouped_kernel(const GroupedArgs g) {
   constexpr bool kOutBf16 = EPI != 2;
@@ -82,31 +84,33 @@ void gemm_grouped_kernel(const GroupedArgs g) {
   // B packed: a wave load covers 16 rows x 64 B; two per wave; a lane's 16 bytes become the two
   // neighbouring 16-byte pieces 2p, 2p+1 of its row.
   constexpr int NLA = 2, NLB = PACKED ? 2 : 4;
-  v4i sta[NLA], stb[NLB];
+  // two sets of staging registers: the loads of a stage are issued two stages ahead of its use and
+  // written to LDS one stage ahead, so that a stage never waits for a load issued in it
+  v4i sta[2][NLA], stb[2][NLB];
   auto row_swz = [](int row) { return (row ^ (row >> 3)) & 7; };
-  auto load_stage = [&](int k0) {
+  auto load_stage = [&](const int set, int k0) {
 #pragma unroll
     for (int i = 0; i < NLA; ++i) {
       const int row = (wave * NLA + i) * 8 + (lane >> 3);
       const int cb = (((lane & 7) ^ row_swz(row)) & 7) * 16;
-      sta[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, row * (int)g.lda + cb, k0, 0);
+      sta[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, row * (int)g.lda + cb, k0, 0);
     }
 #pragma unroll
     for (int i = 0; i < NLB; ++i) {
       if constexpr (PACKED) {
         const int row = (wave * NLB + i) * 16 + (lane >> 2);
-        stb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, row * (int)g.ldb + (lane & 3) * 16, k0 / 2, 0);
+        stb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, row * (int)g.ldb + (lane & 3) * 16, k0 / 2, 0);
       } else {
         const int row = (wave * NLB + i) * 8 + (lane >> 3);
         const int cb = (((lane & 7) ^ row_swz(row)) & 7) * 16;
-        stb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, row * (int)g.ldb + cb, k0, 0);
+        stb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, row * (int)g.ldb + cb, k0, 0);
       }
     }
   };
-  auto store_stage = [&](uint8_t* st) {
+  auto store_stage = [&](const int set, uint8_t* st) {
 #pragma unroll
     for (int i = 0; i < NLA; ++i)
-      *reinterpret_cast<v4i*>(st + (wave * NLA + i) * 1024 + lane * 16) = sta[i];
+      *reinterpret_cast<v4i*>(st + (wave * NLA + i) * 1024 + lane * 16) = sta[set][i];
 #pragma unroll
     for (int i = 0; i < NLB; ++i) {
       if constexpr (PACKED) {
@@ -117,7 +121,7 @@ void gemm_grouped_kernel(const GroupedArgs g) {
         v4i lo, hi;
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const uint32_t x = (uint32_t)stb[i][d];
+          const uint32_t x = (uint32_t)stb[set][i][d];
           const uint32_t ev = (x << 4) & 0xF0F0F0F0u, od = x & 0xF0F0F0F0u;
           const uint32_t k03 = __builtin_amdgcn_perm(od, ev, 0x05010400u);  // e0 o0 e1 o1
           const uint32_t k47 = __builtin_amdgcn_perm(od, ev, 0x07030602u);  // e2 o2 e3 o3
@@ -128,7 +132,7 @@ void gemm_grouped_kernel(const GroupedArgs g) {
         *reinterpret_cast<v4i*>(rowp + (((2 * p) ^ row_swz(row)) * 16)) = lo;
         *reinterpret_cast<v4i*>(rowp + (((2 * p + 1) ^ row_swz(row)) * 16)) = hi;
       } else {
-        *reinterpret_cast<v4i*>(st + kATile + (wave * NLB + i) * 1024 + lane * 16) = stb[i];
+        *reinterpret_cast<v4i*>(st + kATile + (wave * NLB + i) * 1024 + lane * 16) = stb[set][i];
       }
     }
   };
@@ -168,16 +172,18 @@ void gemm_grouped_kernel(const GroupedArgs g) {
   const v16i kZero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
   const int nstages = g.groups * g.stages_per_group;
-  load_stage(0);
+  load_stage(0, 0);
   load_scales(0);
-  store_stage(stage_mem[0]);
+  store_stage(0, stage_mem[0]);
   store_scales(0);
+  if (nstages > 1) load_stage(1, BK);  // set 1 holds stage 1, set 0 will take stage 2, ...
   __syncthreads();
-  for (int s = 0; s < nstages; ++s) {
-    const int grp = s / g.stages_per_group;
-    const bool last_of_group = (s + 1) % g.stages_per_group == 0;
+  // one stage; `set` holds the registers of stage s + 1, the other set takes the loads of s + 2
+  auto stage = [&](const int s, const int set) {
+    const int grp = ONE ? s : s / g.stages_per_group;
+    const bool last_of_group = ONE || (s + 1) % g.stages_per_group == 0;
     const uint8_t* st = stage_mem[s & 1];
-    if (s + 1 < nstages) load_stage((s + 1) * BK);
+    if (s + 2 < nstages) load_stage(set ^ 1, (s + 2) * BK);
     if (last_of_group) load_scales(grp + 1);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
@@ -189,7 +195,7 @@ void gemm_grouped_kernel(const GroupedArgs g) {
         fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c]);
       }
       // the first MFMA of a group starts from a zero accumulator operand instead of zeroed registers
-      const bool fresh = ks == 0 && (s % g.stages_per_group) == 0;
+      const bool fresh = ks == 0 && (ONE || (s % g.stages_per_group) == 0);
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
@@ -229,9 +235,17 @@ void gemm_grouped_kernel(const GroupedArgs g) {
             }
         }
     }
-    if (s + 1 < nstages) store_stage(stage_mem[(s + 1) & 1]);
+    // the registers of stage s + 1 (requested a whole stage ago) go to the buffer stage s - 1 left;
+    // the barrier is a bare s_barrier: a __syncthreads() would also wait for the loads of s + 2
+    if (s + 1 < nstages) store_stage(set, stage_mem[(s + 1) & 1]);
     if (last_of_group) store_scales((grp + 1) & 1);
-    __syncthreads();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  for (int s = 0; s < nstages; s += 2) {
+    stage(s, 1);
+    if (s + 1 < nstages) stage(s + 1, 0);
   }
 
   // ---- output --------------------------------------------------------------------------------
@@ -339,10 +353,14 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   else epi = p->col_scale_dtype == AQTX_BF16 ? 0 : 4;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n));
+  // the compile-time form of the one-stage group costs the unpacked variant a few spilled registers
+  const bool one = g.stages_per_group == 1 && packed;
 #define AQTX_LAUNCH(E)                                                       \
   do {                                                                      \
-    if (packed) gemm_grouped_kernel<E, true><<<grid, 512, 0, st>>>(g);      \
-    else gemm_grouped_kernel<E, false><<<grid, 512, 0, st>>>(g);            \
+    if (packed && one) gemm_grouped_kernel<E, true, true><<<grid, 512, 0, st>>>(g);         \
+    else if (packed) gemm_grouped_kernel<E, true, false><<<grid, 512, 0, st>>>(g);          \
+    else if (one) gemm_grouped_kernel<E, false, true><<<grid, 512, 0, st>>>(g);             \
+    else gemm_grouped_kernel<E, false, false><<<grid, 512, 0, st>>>(g);                     \
   } while (0)
   switch (epi) {
     case 0: AQTX_LAUNCH(0); break;
