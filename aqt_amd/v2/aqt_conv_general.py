@@ -5,7 +5,8 @@ The reference quantizes the input per batch element and the kernel per output fe
 Here the convolution is an implicit-GEMM: the (padded, strided, dilated) windows of the
 quantized input are gathered into a [batch * positions, window * features] int8 matrix and
 contracted with the [out features, window * features] kernel matrix on the int8 MFMA kernel
-(exact int32 accumulators); float-held or unquantized operands take a float matrix product.
+(exact int32 accumulators, both scales applied in its epilogue); float-held or unquantized
+operands take a float matrix product.
 Flax layout only (NHWC input, HWIO kernel), as in the reference; no feature / batch groups and
 no input dilation.
 """
@@ -108,6 +109,44 @@ def lax_conv_general_dilated(lhs, rhs, window_strides, padding, lhs_dilation=Non
   return out.reshape([n] + list(out_sizes) + [cout])
 
 
+def _fused_int8_conv(lhs_qt, rhs_qt, out_dtype, window_strides, padding, lhs_dilation, rhs_dilation,
+                     feature_group_count, batch_group_count, preferred_element_type):
+  """int8 x int8 with one scale per batch element and one per output feature: the contraction
+  kernel dequantizes in its epilogue (accumulator -> out dtype, times the lhs scale, times the rhs
+  scale: QTensor.dequant's order, aqt_tensor.py:179-183).  None if the call is not of that form."""
+  lq, rq = lhs_qt.qvalue, rhs_qt.qvalue
+  rank = lq.dim()
+  if not (lq.dtype == torch.int8 and rq.dtype == torch.int8 and len(lhs_qt.scale) == 1 and len(rhs_qt.scale) == 1
+          and not lhs_qt.bias and not rhs_qt.bias and preferred_element_type in (None, out_dtype)
+          and out_dtype in (torch.bfloat16, torch.float32)
+          and feature_group_count == 1 and batch_group_count == 1
+          and (lhs_dilation is None or all(int(d) == 1 for d in lhs_dilation))):
+    return None
+  ls, rs = lhs_qt.scale[0], rhs_qt.scale[0]
+  n, cout = lq.shape[0], rq.shape[-1]
+  if tuple(ls.shape) != (n,) + (1,) * (rank - 1) or tuple(rs.shape) != (1,) * (rank - 1) + (cout,):
+    return None
+  if ls.dtype not in (torch.bfloat16, torch.float32) or rs.dtype not in (torch.bfloat16, torch.float32):
+    return None
+  ns = rank - 2
+  strides = [int(x) for x in window_strides]
+  dilation = [int(d) for d in rhs_dilation] if rhs_dilation is not None else [1] * ns
+  kernel = list(rq.shape[:ns])
+  eff = [(k - 1) * d + 1 for k, d in zip(kernel, dilation)]
+  pads = _explicit_padding(padding, list(lq.shape[1:1 + ns]), eff, strides)
+  a, out_sizes = _windows(lq.contiguous(), kernel, strides, pads, dilation)
+  k = a.shape[1]
+  positions = math.prod(out_sizes)
+  if a.shape[0] * cout == 0 or k == 0:
+    return None
+  b = rq.reshape(k, cout).t().contiguous()
+  row_scale = ls.reshape(n, 1).float().expand(n, positions).reshape(1, n * positions).contiguous()
+  out = ops.gemm(a.contiguous()[None], b[None], row_scale=row_scale, col_scale=rs.reshape(1, cout).float().contiguous(),
+                 out_dtype=out_dtype, dequant_dtype=out_dtype, row_scale_dtype=ls.dtype, col_scale_dtype=rs.dtype,
+                 a_dtype=L.I8, b_dtype=L.I8)[0]
+  return out.reshape([n] + list(out_sizes) + [cout])
+
+
 def make_conv_general_dilated_with_qt(cfg: aqt_dot_general.DotGeneralRaw):
   """Quantized conv_general_dilated that also returns the QTensors (aqt_conv_general.py:33-135)."""
   assert cfg is not None, 'Missing config for make_conv_general_dilated'
@@ -144,6 +183,10 @@ def make_conv_general_dilated_with_qt(cfg: aqt_dot_general.DotGeneralRaw):
     lq, rq = lhs_qt.qvalue, rhs_qt.qvalue
     out_dtype = torch.promote_types(lhs.dtype, rhs.dtype)
     both_int = lq.dtype == torch.int8 and rq.dtype == torch.int8
+    fused = _fused_int8_conv(lhs_qt, rhs_qt, out_dtype, window_strides, padding, lhs_dilation, rhs_dilation,
+                             feature_group_count, batch_group_count, preferred_element_type)
+    if fused is not None:
+      return fused, (lhs_qt, rhs_qt)
     acc = lax_conv_general_dilated(
         lq.contiguous() if both_int else lq.to(lhs.dtype), rq.contiguous() if both_int else rq.to(rhs.dtype),
         window_strides=window_strides, padding=padding, lhs_dilation=lhs_dilation, rhs_dilation=rhs_dilation,
