@@ -141,3 +141,87 @@ def test_serving_from_logical_order_checkpoint(gpu):
     assert torch.equal(serve(x8, torch.zeros_like(w), MATMUL, None), want8)
     assert torch.equal(serve(x100, torch.zeros_like(w), MATMUL, None), want100)
   assert len(adg._KERNEL_LAYOUT_CACHE) == 1
+
+
+@pytest.mark.parametrize('bits', [8, 4])
+def test_e2e_example_head_convert_and_serve(gpu, bits):
+  """The quantized layers of the reference's end-to-end example (examples/flax_e2e_model.py:79-145):
+  Dense 3136 -> 256 and Dense 256 -> 10 with the contraction axis split in two tiles, then the
+  einsum 'bc,ab->ac' against an identity weight with 'b' tiled by 5 and the two sides' quantizers
+  swapped.  After conversion the frozen QTensors have the shapes and dtypes the reference's test
+  lists (examples/flax_e2e_model_test.py:141-196), the serving model reproduces the training-mode
+  logits bit for bit without the float weights, and does use the frozen values
+  (examples/flax_e2e_model_test.py:250-271)."""
+  import copy
+  batch = 4
+  torch.manual_seed(0)
+  x = torch.randn(batch, 3136, device=gpu)
+  w0 = torch.randn(3136, 256, device=gpu) / 56.0
+  w1 = torch.randn(256, 10, device=gpu) / 16.0
+  # The reference's 4-bit case asks for `fwd_accumulator_dtype=None`, with which lax.dot_general
+  # returns the int4 product wrapped to int4 (its expected loss on TPU is ln 10); this build
+  # contracts integers into int32 only and says so when asked otherwise, so both cases keep the
+  # default int32 accumulator here.
+  cfg = config.config_v4(fwd_bits=bits, drhs_bits=8, drhs_accumulator_dtype=utils.int32)
+  with pytest.raises(AssertionError, match='int32 accumulator'):
+    bad = config.set_context(config.config_v4(fwd_bits=bits, fwd_accumulator_dtype=None), None, None)
+    bad(torch.randn(4, 32, device=gpu), torch.randn(32, 8, device=gpu), MATMUL)
+  tiling = tiled_dot_general.Cfg(
+      lhs=tiled_dot_general.TensorTiling(
+          contraction_axes=[tiled_dot_general.AxisTiling(axis=1, tile_count=2, tile_size=None)], remaining_axes=[]),
+      rhs=tiled_dot_general.TensorTiling(
+          contraction_axes=[tiled_dot_general.AxisTiling(axis=0, tile_count=2, tile_size=None)], remaining_axes=[]))
+  cfg_swapped = copy.deepcopy(cfg)
+  cfg_swapped.fwd.dg_quantizer.swap_lhs_and_rhs()
+
+  def build(weights_mode, act_mode):
+    dense = lambda: aqt_flax.AqtDotGeneral(
+        cfg, lhs_quant_mode=act_mode, rhs_quant_mode=weights_mode, tiling_cfg=tiling,
+        lhs_freeze_mode=FM.CALIBRATION, rhs_freeze_mode=FM.CALIBRATION_AND_VALUE, use_legacy_freezer=False,
+        rngs=_rngs())
+    einsum = aqt_flax.AqtEinsum(
+        cfg_swapped, lhs_quant_mode=weights_mode, rhs_quant_mode=act_mode, assert_eqn='bc,ab->ac',
+        assert_lhs_shape=(10, 10), assert_rhs_shape=(None, 10), tile_sizes={'b': 5},
+        lhs_freeze_mode=FM.CALIBRATION_AND_VALUE, rhs_freeze_mode=FM.CALIBRATION, use_legacy_freezer=False,
+        rngs=_rngs())
+    return dense(), dense(), einsum
+
+  def forward(layers, w0_, w1_):
+    d0, d1, es = layers
+    h = torch.relu(d0(x, w0_, MATMUL, None))
+    h = d1(h, w1_, MATMUL, None)
+    return es('bc,ab->ac', torch.eye(10, device=gpu, dtype=h.dtype), h)
+
+  logits_train = forward(build(QM.TRAIN, QM.TRAIN), w0, w1)
+  conv_layers = build(QM.CONVERT, QM.TRAIN)
+  logits_conv = forward(conv_layers, w0, w1)
+  assert torch.equal(logits_train, logits_conv)
+
+  want_dtype = utils.int4 if bits == 4 else utils.int8
+  expected = [('qrhs', (2, 1568, 256), (2, 1, 256)), ('qrhs', (2, 128, 10), (2, 1, 10)), ('qlhs', (2, 5, 10), (2, 1, 10))]
+  saved = []
+  for layer, (side, qshape, sshape) in zip(conv_layers, expected):
+    v = layer.variables()
+    if isinstance(layer, aqt_flax.AqtEinsum):
+      v = v['aqt']['AqtDotGeneral_0'] if 'AqtDotGeneral_0' in v.get('aqt', {}) else v['aqt']
+    else:
+      v = v['aqt']
+    assert set(v) == {side}, (set(v), side)
+    qt = v[side]['frozen']
+    assert tuple(qt.qvalue.shape) == qshape and [tuple(s.shape) for s in qt.scale] == [sshape]
+    assert qt.scale[0].dtype == torch.float32 and qt.scale_t is None and qt.bias == []
+    assert qt.dequant_dtype == torch.float32
+    assert (qt.container_dtype or utils.int8) is want_dtype or qt.qvalue.dtype == want_dtype
+    saved.append(layer.variables())
+
+  serve_layers = build(QM.SERVE, QM.TRAIN)
+  for layer, v in zip(serve_layers, saved):
+    layer.load_variables(v)
+  logits_serve = forward(serve_layers, torch.zeros_like(w0), torch.zeros_like(w1))
+  assert torch.equal(logits_serve, logits_train)
+  # the frozen values are what serving computes from
+  broken = copy.deepcopy(saved[0])
+  node = broken['aqt']['qrhs']['frozen']
+  node.qvalue = torch.zeros_like(node.qvalue)
+  serve_layers[0].load_variables(broken)
+  assert not torch.equal(forward(serve_layers, torch.zeros_like(w0), torch.zeros_like(w1)), logits_train)
