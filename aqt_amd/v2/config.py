@@ -16,6 +16,7 @@ from aqt_amd.v2.numerics import int_numerics
 from aqt_amd.v2.numerics import no_numerics
 from aqt_amd.v2.numerics import numerics
 from aqt_amd.v2.numerics import utils as numerics_utils
+from aqt_amd.v2.aqt_conv_general import conv_general_dilated_make  # re-exported as in config.py:31
 
 # Re-exports, as in the reference (config.py:33-52).
 CalibrationMode = aqt_dot_general.CalibrationMode

@@ -430,3 +430,85 @@ class AqtEinsum(torch.nn.Module, _RngMixin):
     dg.rhs_axis_metadata_wrapper, dg.rhs_freeze_mode = R['wrapper'], R['freeze_mode']
     dg.tiling_cfg = tiling_config
     return aqt_dot_general.einsum(eqn, lhs_in, rhs_in, dg)
+
+
+class AqtConvGeneralDilated(torch.nn.Module, _RngMixin):
+  """A conv_general_dilated-shaped callable that quantizes (aqt_flax.py:735-935): only `cfg.fwd` is
+  used, the operands are frozen through the general Freezer."""
+
+  def __init__(self, cfg: Optional[aqt_dot_general.DotGeneral] = None, prng_name: Optional[str] = 'params', *,
+               lhs_quant_mode: QuantMode = QuantMode.TRAIN, lhs_apply_quant_mode: bool = True,
+               lhs_var_name: str = 'qlhs', lhs_qtensor: Optional[aqt_tensor.QTensor] = None,
+               rhs_quant_mode: QuantMode = QuantMode.TRAIN, rhs_apply_quant_mode: bool = True,
+               rhs_var_name: str = 'qrhs', rhs_qtensor: Optional[aqt_tensor.QTensor] = None,
+               lhs_axis_metadata_wrapper=None, rhs_axis_metadata_wrapper=None,
+               lhs_freeze_mode: FreezerMode = FreezerMode.NONE, rhs_freeze_mode: FreezerMode = FreezerMode.NONE,
+               quant_collection: str = 'aqt', rngs: Optional[Dict[str, Any]] = None):
+    super().__init__()
+    self.cfg, self.prng_name = cfg, prng_name
+    self.lhs_quant_mode, self.lhs_apply_quant_mode = lhs_quant_mode, lhs_apply_quant_mode
+    self.lhs_var_name, self.lhs_qtensor = lhs_var_name, lhs_qtensor
+    self.rhs_quant_mode, self.rhs_apply_quant_mode = rhs_quant_mode, rhs_apply_quant_mode
+    self.rhs_var_name, self.rhs_qtensor = rhs_var_name, rhs_qtensor
+    self.lhs_axis_metadata_wrapper, self.rhs_axis_metadata_wrapper = lhs_axis_metadata_wrapper, rhs_axis_metadata_wrapper
+    self.lhs_freeze_mode, self.rhs_freeze_mode = lhs_freeze_mode, rhs_freeze_mode
+    self.quant_collection = quant_collection
+    self.rngs = rngs
+    self.freezers = torch.nn.ModuleDict()
+
+  _freezer = AqtDotGeneral._freezer
+  variables = AqtDotGeneral.variables
+  load_variables = AqtDotGeneral.load_variables
+
+  def make_aqt_cg(self):
+    from aqt_amd.v2 import aqt_conv_general
+    if self.cfg is None:
+      return aqt_conv_general.lax_conv_general_dilated
+    cfg = copy.deepcopy(self.cfg)
+    assert isinstance(cfg.fwd.dg_quantizer, aqt_dot_general.DefaultDotGeneralQuantizer)
+    lhs_freezer = self._freezer(self.lhs_var_name, lambda: general_freezer.Freezer(
+        name=self.lhs_var_name, collection=self.quant_collection,
+        axis_metadata_wrapper=self.lhs_axis_metadata_wrapper))
+    rhs_freezer = self._freezer(self.rhs_var_name, lambda: general_freezer.Freezer(
+        name=self.rhs_var_name, collection=self.quant_collection,
+        axis_metadata_wrapper=self.rhs_axis_metadata_wrapper))
+    lhs_freezer.mode = _QUANT_TO_FREEZER_MODE[self.lhs_quant_mode]
+    rhs_freezer.mode = _QUANT_TO_FREEZER_MODE[self.rhs_quant_mode]
+    pending = getattr(self, '_pending', None)
+    if pending is not None:
+      for name, fr in ((self.lhs_var_name, lhs_freezer), (self.rhs_var_name, rhs_freezer)):
+        fr.load_state({coll: tree[name] for coll, tree in pending.items() if name in tree})
+      self._pending = None
+    key = self.make_rng(self.prng_name) if self.prng_name is not None else None
+    cfg = config.set_context(cfg, key, train_step=None, lhs_quant_mode=self.lhs_quant_mode,
+                             rhs_quant_mode=self.rhs_quant_mode)
+
+    def ret_cg(lhs, rhs, window_strides, padding, lhs_dilation, rhs_dilation, dimension_numbers,
+               feature_group_count, batch_group_count, precision, preferred_element_type):
+      msg = 'AQT is not yet optimized to accept quantized types directly. '
+      msg += f'lhs.dtype: {lhs.dtype}, rhs.dtype: {rhs.dtype}'
+      assert lhs.dtype in [utils.bfloat16, utils.float32, utils.float16], msg
+      assert rhs.dtype in [utils.bfloat16, utils.float32, utils.float16], msg
+      cfg.assert_config_validity()
+      lhs_qt = lhs_freezer.get() if self.lhs_apply_quant_mode else self.lhs_qtensor
+      rhs_qt = rhs_freezer.get() if self.rhs_apply_quant_mode else self.rhs_qtensor
+      aqt_conv = aqt_conv_general.make_conv_general_dilated_with_qt(cfg.fwd)
+      out, (out_lhs_qt, out_rhs_qt) = aqt_conv(
+          lhs, rhs, window_strides, padding, lhs_qt, rhs_qt, lhs_dilation, rhs_dilation, dimension_numbers,
+          feature_group_count, batch_group_count, precision, preferred_element_type)
+      out_lhs_qt = _apply_freeze_mode(out_lhs_qt, self.lhs_freeze_mode, self.lhs_apply_quant_mode,
+                                      self.lhs_quant_mode, 'lhs')
+      out_rhs_qt = _apply_freeze_mode(out_rhs_qt, self.rhs_freeze_mode, self.rhs_apply_quant_mode,
+                                      self.rhs_quant_mode, 'rhs')
+      if self.lhs_apply_quant_mode:
+        lhs_freezer.set(out_lhs_qt)
+      if self.rhs_apply_quant_mode:
+        rhs_freezer.set(out_rhs_qt)
+      return out
+
+    return ret_cg
+
+  def forward(self, lhs, rhs, window_strides, padding, lhs_dilation=None, rhs_dilation=None, dimension_numbers=None,
+              feature_group_count: int = 1, batch_group_count: int = 1, precision=None, preferred_element_type=None):
+    return self.make_aqt_cg()(lhs, rhs, window_strides, padding, lhs_dilation, rhs_dilation, dimension_numbers,
+                              feature_group_count, batch_group_count, precision, preferred_element_type)
