@@ -256,6 +256,36 @@ class DefaultDotGeneralQuantizer(DotGeneralQuantizer):
     self.rhs.context = rhs_context
 
 
+def _quant(lhs, rhs, lhs_qt, rhs_qt, dg_quantizer, lhs_cfg, rhs_cfg, dimension_numbers,
+           allow_dummy_gradient_into_qtensor):
+  """quant() below, also returning the operands as the quantizer's calibrate step left them."""
+  (lhs, lhs_incomplete), (rhs, rhs_incomplete) = dg_quantizer.calibrate(
+      lhs, rhs, dimension_numbers, lhs_cfg.calibration_mode, rhs_cfg.calibration_mode)
+  if lhs_qt is not None and not lhs_qt.is_full():
+    lhs_incomplete, lhs_qt = lhs_qt, None  # an incomplete QTensor (scales only) was handed in
+  if rhs_qt is not None and not rhs_qt.is_full():
+    rhs_incomplete, rhs_qt = rhs_qt, None
+  (lhs_calc, lhs_grad), (rhs_calc, rhs_grad) = dg_quantizer.calculate_qvalue(lhs, lhs_incomplete, rhs, rhs_incomplete)
+
+  def postprocess(given, calculated, quant_grad):
+    if given is None:
+      return calculated, quant_grad
+    return given, (quant_grad if allow_dummy_gradient_into_qtensor else _POISON)
+
+  return postprocess(lhs_qt, lhs_calc, lhs_grad), postprocess(rhs_qt, rhs_calc, rhs_grad), (lhs, rhs)
+
+
+def quant(lhs, rhs, lhs_qt, rhs_qt, dg_quantizer, lhs_cfg, rhs_cfg, dimension_numbers,
+          allow_dummy_gradient_into_qtensor):
+  """Quantizes lhs and rhs with dg_quantizer (aqt_dot_general.py:598-672): calibrate, take over
+  scales handed in as incomplete QTensors, compute the qvalues, and keep a QTensor that was
+  handed in whole (its gradient function is then poisoned unless dummy gradients are allowed).
+  Returns ((lhs_qt, lhs_quant_grad), (rhs_qt, rhs_quant_grad))."""
+  l, r, _ = _quant(lhs, rhs, lhs_qt, rhs_qt, dg_quantizer, lhs_cfg, rhs_cfg, dimension_numbers,
+                   allow_dummy_gradient_into_qtensor)
+  return l, r
+
+
 def dot_general_raw_make(lhs_bits=None, rhs_bits=None, local_aqt=None, jax_scope_name='aqt',
                          initialize_calibration=True, allow_dummy_gradients=False) -> 'DotGeneralRaw':
   """aqt_dot_general.py:99-156."""
@@ -618,23 +648,9 @@ class DotGeneralRaw:
     if isinstance(rhs, aqt_tensor.QTensor):
       rhs = rhs.qvalue.to(rhs.dequant_dtype)
 
-    # quant() of the reference (aqt_dot_general.py:598-672)
-    dq = self.dg_quantizer
-    (lhs, lhs_incomplete), (rhs, rhs_incomplete) = dq.calibrate(
-        lhs, rhs, dimension_numbers, self.lhs.calibration_mode, self.rhs.calibration_mode)
-    if lhs_qt is not None and not lhs_qt.is_full():
-      lhs_incomplete, lhs_qt = lhs_qt, None
-    if rhs_qt is not None and not rhs_qt.is_full():
-      rhs_incomplete, rhs_qt = rhs_qt, None
-    (lhs_calc, lhs_grad), (rhs_calc, rhs_grad) = dq.calculate_qvalue(lhs, lhs_incomplete, rhs, rhs_incomplete)
-
-    def postprocess(given, calculated, quant_grad):
-      if given is None:
-        return calculated, quant_grad
-      return given, (quant_grad if self.allow_dummy_gradient_into_qtensor else _POISON)
-
-    lhs_qt, lhs_grad = postprocess(lhs_qt, lhs_calc, lhs_grad)
-    rhs_qt, rhs_grad = postprocess(rhs_qt, rhs_calc, rhs_grad)
+    (lhs_qt, lhs_grad), (rhs_qt, rhs_grad), (lhs, rhs) = _quant(
+        lhs, rhs, lhs_qt, rhs_qt, self.dg_quantizer, self.lhs, self.rhs, dimension_numbers,
+        self.allow_dummy_gradient_into_qtensor)
 
     msg = ('biases are only supported in fake quant mode, but got a {arg} bias '
            'and self.{arg}.dequant_mode == {mode} != DequantMode.THIS_INPUT')

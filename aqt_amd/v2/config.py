@@ -89,6 +89,15 @@ def set_numerics(cfg: DotGeneralRaw, lhs_numerics: numerics.AqtNumerics,
     cfg.dg_accumulator_dtype = None
 
 
+def set_fwd_rhs_dtype_int2(cfg: DotGeneral):
+  """A special setter for int2 weights (config.py:142-154).  The reference switches the storage
+  dtype of the 2-bit weight from int8 to jnp.int2 (an XLA casting limitation keeps it out of
+  infer_dtype_from_bits).  torch has no 2-bit dtype: the values stay one per byte in the int8
+  container, which holds the same numbers, so this only checks what the reference checks."""
+  assert isinstance(cfg.fwd.dg_quantizer.rhs.numerics, int_numerics.IntSymmetric)
+  assert cfg.fwd.dg_quantizer.rhs.numerics.bits == 2
+
+
 def set_accumulator_dtype(cfg: DotGeneral, fwd_dtype, dlhs_dtype, drhs_dtype):
   if fwd_dtype != SKIP:
     cfg.fwd.dg_accumulator_dtype = fwd_dtype

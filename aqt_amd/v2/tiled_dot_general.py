@@ -122,6 +122,10 @@ def interleave(tile_count, tile_size, tile_map, remaining_axes, product=False):
   return out
 
 
+def maybe_add_one(i, min_i):
+  """Index i after an axis was inserted at min_i (tiled_dot_general.py:177-178)."""
+  return i + int(i >= min_i)
+
 @dataclasses.dataclass
 class TilingState:
   """Axis bookkeeping of one operand while it is tiled (tiled_dot_general.py:182-294).
@@ -196,7 +200,6 @@ class TilingState:
       sizes.append(where[-1])
     return counts, sizes
 
-
 def generate_tiling_state(tensor, tiled_axes: Iterable[AxisTiling]) -> TilingState:
   """tiled_dot_general.py:320-331."""
   tiled_axes = list(tiled_axes)
@@ -205,7 +208,6 @@ def generate_tiling_state(tensor, tiled_axes: Iterable[AxisTiling]) -> TilingSta
   st = TilingState(untiled_shape=tuple(tensor.shape))
   st.tile_axes(tiled_axes)
   return st
-
 
 def generate_tiling_states_for_dot_general(cfg: Cfg, lhs, rhs, dimension_numbers):
   """Tiling states of both operands, broadcast axes included (tiled_dot_general.py:334-404)."""
@@ -230,7 +232,6 @@ def generate_tiling_states_for_dot_general(cfg: Cfg, lhs, rhs, dimension_numbers
   xlhs.broadcast_to_other(xrhs.axes_shape(r_ra_tiles))
   return xlhs, xrhs
 
-
 def _sum_leading(x):
   """Sum over axis 0 in float32, tile by tile, rounded once to x.dtype."""
   if x.is_cuda and x.dtype in (torch.bfloat16, torch.float32):
@@ -242,11 +243,9 @@ def _sum_leading(x):
     acc = acc + x[t]
   return acc.to(x.dtype)
 
-
 def _default_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
   from aqt_amd.v2 import aqt_dot_general
   return aqt_dot_general.lax_dot_general(lhs, rhs, dimension_numbers, precision, preferred_element_type)
-
 
 def tiled_dot_general_with_tiling_states(lhs, xlhs: TilingState, rhs, xrhs: TilingState,
                                          untiled_dimension_numbers, precision=None,
@@ -316,10 +315,24 @@ def tiled_dot_general_with_tiling_states(lhs, xlhs: TilingState, rhs, xrhs: Tili
   r_flat = interleave(r_ra_t_sh, r_ra_sh, xrhs.tile_map, rra, product=True)
   return out.reshape(list(ba_sh) + l_flat + r_flat)
 
-
 def tiled_dot_general(cfg: Cfg, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None,
                       dot_general=_default_dot_general):
   """dot_general over tiles of the operands (tiled_dot_general.py:546-568)."""
   xlhs, xrhs = generate_tiling_states_for_dot_general(cfg, lhs, rhs, dimension_numbers)
   return tiled_dot_general_with_tiling_states(lhs, xlhs, rhs, xrhs, dimension_numbers, precision,
                                               preferred_element_type, dot_general)
+
+def print_dimension_numbers(dimension_numbers, lhs, rhs, label) -> None:
+  """Logs the dimension numbers before and / or after tiling at debug level
+  (tiled_dot_general.py:297-320)."""
+  import logging
+  (lhs_ca, rhs_ca), (lhs_ba, rhs_ba) = dimension_numbers
+  lhs_ra = get_ra(lhs.dim(), lhs_ca, lhs_ba)
+  rhs_ra = get_ra(rhs.dim(), rhs_ca, rhs_ba)
+  log = logging.getLogger(__name__)
+  log.debug(label)
+  log.debug(' lhs.shape=%s', tuple(lhs.shape))
+  log.debug(' rhs.shape=%s', tuple(rhs.shape))
+  log.debug(' lhs_ca=%s rhs_ca=%s', lhs_ca, rhs_ca)
+  log.debug(' lhs_ba=%s rhs_ba=%s', lhs_ba, rhs_ba)
+  log.debug(' lhs_ra=%s rhs_ra=%s', lhs_ra, rhs_ra)
