@@ -126,6 +126,7 @@ def maybe_add_one(i, min_i):
   """Index i after an axis was inserted at min_i (tiled_dot_general.py:177-178)."""
   return i + int(i >= min_i)
 
+
 @dataclasses.dataclass
 class TilingState:
   """Axis bookkeeping of one operand while it is tiled (tiled_dot_general.py:182-294).
