@@ -1005,7 +1005,35 @@ int dispatch(const QArgs& a, int reduce, int partitionable, int64_t nscales, hip
 
 using namespace aqtx;
 
+// A few very long rows (one scale per image of a convolution's input, say) would leave most of
+// the chip idle in the row kernels, which give a row to one wave or workgroup.  Such a plan is the
+// same computation as one scale per batch entry of [batch * rows][cols / c][c]: the whole-tensor
+// path, which spreads every entry over many workgroups.  Returns true and fills `q` if `p` is
+// such a plan.
+static bool long_rows_as_batches(const aqtx_quant_plan* p, aqtx_quant_plan* q) {
+  if (p->reduce != AQTX_REDUCE_COLS || p->group != 0 || p->transpose_out || p->prescale != AQTX_PRESCALE_NONE)
+    return false;
+  if (p->batch <= 0 || p->rows <= 0 || p->batch * p->rows > 512 || p->cols < 16384) return false;
+  if (p->noise != AQTX_NOISE_NONE && p->batch > 1 && p->noise_stride_batch != p->rows * p->noise_stride_row)
+    return false;
+  int64_t c = 0;
+  for (int64_t cand = 1024; cand >= 64; cand /= 2) {
+    if (p->cols % cand == 0) { c = cand; break; }
+  }
+  if (c == 0) return false;
+  *q = *p;
+  q->batch = p->batch * p->rows;
+  q->rows = p->cols / c;
+  q->cols = c;
+  q->reduce = AQTX_REDUCE_ALL;
+  q->noise_stride_batch = p->noise_stride_row;
+  q->noise_stride_row = c * p->noise_stride_col;
+  return true;
+}
+
 extern "C" size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* p) {
+  aqtx_quant_plan alt;
+  if (p != nullptr && long_rows_as_batches(p, &alt)) return aqtx_quantize_workspace_bytes(&alt);
   if (p == nullptr || p->reduce == AQTX_REDUCE_COLS) return 0;
   if (p->batch < 0 || p->rows < 0 || p->cols < 0 || p->group < 0) return 0;
   if (p->reduce < AQTX_REDUCE_ROWS || p->reduce > AQTX_REDUCE_ALL_BATCH) return 0;
@@ -1018,6 +1046,8 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
                              void* stream) {
   clear_error();
   if (int rc = validate(p)) return rc;
+  aqtx_quant_plan alt;
+  if (long_rows_as_batches(p, &alt)) return aqtx_quantize(&alt, x, prescale, q, scale, workspace, workspace_bytes, stream);
   const int64_t total = p->batch * p->rows * p->cols;
   if (total == 0) return 0;
   AQTX_REQUIRE(x != nullptr && q != nullptr && scale != nullptr, "aqtx_quantize: NULL buffer");

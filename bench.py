@@ -209,6 +209,18 @@ def other_configs(dev):
   out['fp_round_e2m1_bf16_8192x14336'] = {
       'nearest_ms': round(ms_rn, 3), 'nearest_GB/s': round(gb / ms_rn * 1e3, 1),
       'stochastic_ms': round(ms_sr, 3), 'stochastic_GB/s': round(gb / ms_sr * 1e3, 1)}
+  del t
+  # quantized conv_general_dilated forward (NHWC input [32, 56, 56, 128], 3x3 kernel to 128 features, SAME): per
+  # batch-element input scale, per-feature kernel scale, window gather + int8 contraction with fused dequantisation
+  from aqt_amd.v2 import aqt_conv_general
+  xc = torch.randn(32, 56, 56, 128, device=dev).to(torch.bfloat16)
+  kc = (torch.randn(3, 3, 128, 128, device=dev) * 0.05).to(torch.bfloat16)
+  conv = aqt_conv_general.make_conv_general_dilated(aqt_conv_general.conv_general_dilated_make(2, 8, 8))
+  dnc = aqt_conv_general.flax_conv_dimension_numbers(xc.shape)
+  with torch.no_grad():
+    ms = timeit(lambda: conv(xc, kc, (1, 1), 'SAME', dimension_numbers=dnc))
+  out['conv_int8_fwd_32x56x56x128_k3x3_128'] = {
+      'ms_per_call': round(ms, 3), 'TOPS': round(2.0 * 32 * 56 * 56 * 9 * 128 * 128 / ms / 1e9, 1)}
   return out
 
 

@@ -56,6 +56,8 @@ ROW_CASES = [
     # (rows, cols, group)
     (4, 64, 0), (33, 128, 0), (5, 512, 0), (3, 2048, 0), (7, 4096, 0), (2, 8192, 0),
     (2, 14336, 0), (3, 100, 0), (2, 20000, 0), (6, 1024, 128), (3, 96, 32),
+    # few long rows: taken as one scale per batch entry of [batch * rows][cols / c][c]
+    (3, 32768, 0), (5, 16448, 0), (2, 401408, 0), (1, 16384, 0),
 ]
 
 
@@ -222,3 +224,22 @@ def test_workspace_kept_across_calls(gpu):
           first[(i, reduce)] = (q.clone(), s.clone())
         else:
           assert torch.equal(q, first[(i, reduce)][0]) and torch.equal(s, first[(i, reduce)][1])
+
+
+@pytest.mark.parametrize('noise', ['jax.uniform', 'custom-1'])
+@pytest.mark.parametrize('dt', ['bf16', 'f32'])
+@pytest.mark.parametrize('batch,rows,cols', [(1, 4, 32768), (2, 3, 16448), (3, 1, 65536)])
+def test_few_long_rows_stochastic_rounding(gpu, batch, rows, cols, noise, dt):
+  """The few-long-rows form with noise: the counters of [batch, rows, cols] carry over to the
+  per-batch-entry form, and a scale handed in is used the same way."""
+  x = U.rand((batch, rows, cols), dt, seed=cols + rows, scale=0.3)
+  key = prng.prng_key(77)
+  q = R.QuantizerCfg(bits=8, key=key, noise=noise)
+  qt = R.quantize(x, dt, q, [2])
+  qb, cb = U.bounds(q)
+  qg, sg = ops.quantize(U.to_dev(x, dt, gpu), reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=qb, clip_bound=cb,
+                        noise=U.NOISE[noise], key=key)
+  _check(qt, qg.cpu().numpy(), sg.cpu().numpy(), q)
+  qg2, _ = ops.quantize(U.to_dev(x, dt, gpu), reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=qb, clip_bound=cb,
+                        noise=U.NOISE[noise], key=key, scale=sg.clone())
+  assert torch.equal(qg, qg2)
