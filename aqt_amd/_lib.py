@@ -71,6 +71,14 @@ class DecodePlan(ctypes.Structure):
 
 # name -> (restype, argtypes); every symbol include/aqtx.h declares
 _vp = ctypes.c_void_p
+class Im2colPlan(ctypes.Structure):
+  _fields_ = [
+      ('n', ctypes.c_int64), ('c', ctypes.c_int32), ('rank', ctypes.c_int32),
+      ('in_size', ctypes.c_int32 * 3), ('kernel', ctypes.c_int32 * 3), ('stride', ctypes.c_int32 * 3),
+      ('dilation', ctypes.c_int32 * 3), ('pad_lo', ctypes.c_int32 * 3), ('out_size', ctypes.c_int32 * 3),
+  ]
+
+
 class FpRoundPlan(ctypes.Structure):
   _fields_ = [
       ('count', ctypes.c_int64), ('noise_mod', ctypes.c_int64),
@@ -82,6 +90,7 @@ class FpRoundPlan(ctypes.Structure):
 FP_NEAREST, FP_NOISE_JAX_BITS, FP_NOISE_INDEX = 0, 1, 2
 
 SYMBOLS = {
+    'aqtx_im2col_i8': (ctypes.c_int, [ctypes.POINTER(Im2colPlan), _vp, _vp, _vp]),
     'aqtx_fp_round': (ctypes.c_int, [ctypes.POINTER(FpRoundPlan), _vp, _vp, ctypes.POINTER(ctypes.c_uint32), _vp]),
     'aqtx_quantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp, _vp,
                                      ctypes.c_size_t, _vp]),

@@ -7,6 +7,7 @@ or the library is missing -- there is no CPU path.
 from __future__ import annotations
 
 import ctypes
+import math
 from typing import Optional, Sequence
 
 import numpy as np
@@ -350,6 +351,29 @@ def sum_tiles(x: torch.Tensor) -> torch.Tensor:
   out = torch.empty(x.shape[1:], dtype=x.dtype, device=x.device)
   L.check(L.lib().aqtx_sum_tiles(_ptr(x), _ptr(out), tiles, out.numel(), aqtx_dtype(x.dtype), _stream()))
   return out
+
+
+def im2col_i8(x: torch.Tensor, kernel, strides, pads, dilation):
+  """Windows of an int8 tensor [n, *spatial, c] as a matrix [n * positions, taps * c] (zeros in the
+  padding); returns (matrix, output spatial sizes).  `pads` are (low, high) pairs."""
+  _require_gpu(x)
+  assert x.dtype == torch.int8 and x.is_contiguous() and 3 <= x.dim() <= 5
+  rank = x.dim() - 2
+  plan = L.Im2colPlan()
+  plan.n, plan.c, plan.rank = x.shape[0], x.shape[-1], rank
+  out_sizes = []
+  for d in range(rank):
+    eff = (int(kernel[d]) - 1) * int(dilation[d]) + 1
+    span = int(pads[d][0]) + x.shape[1 + d] + int(pads[d][1]) - eff
+    o = span // int(strides[d]) + 1 if span >= 0 else 0
+    out_sizes.append(o)
+    plan.in_size[d], plan.kernel[d], plan.stride[d] = x.shape[1 + d], int(kernel[d]), int(strides[d])
+    plan.dilation[d], plan.pad_lo[d], plan.out_size[d] = int(dilation[d]), int(pads[d][0]), o
+  rows = x.shape[0] * math.prod(out_sizes)
+  k = math.prod(int(t) for t in kernel[:rank]) * x.shape[-1]
+  out = torch.empty((rows, k), dtype=torch.int8, device=x.device)
+  L.check(L.lib().aqtx_im2col_i8(ctypes.byref(plan), _ptr(x), _ptr(out), _stream()))
+  return out, out_sizes
 
 
 def fp_round(x: torch.Tensor, *, nexp: int, nmant: int, has_subnormals: bool, key=None,

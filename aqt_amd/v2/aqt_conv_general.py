@@ -3,7 +3,7 @@
 The reference quantizes the input per batch element and the kernel per output feature, runs
 `lax.conv_general_dilated` on the quantized values and multiplies the result by both scales.
 Here the convolution is an implicit-GEMM: the (padded, strided, dilated) windows of the
-quantized input are gathered into a [batch * positions, window * features] int8 matrix and
+quantized input are gathered (aqtx_im2col_i8) into a [batch * positions, window * features] int8 matrix and
 contracted with the [out features, window * features] kernel matrix on the int8 MFMA kernel
 (exact int32 accumulators, both scales applied in its epilogue); float-held or unquantized
 operands take a float matrix product.
@@ -89,10 +89,13 @@ def lax_conv_general_dilated(lhs, rhs, window_strides, padding, lhs_dilation=Non
   pads = _explicit_padding(padding, list(lhs.shape[1:1 + ns]), eff, strides)
   n, cin, cout = lhs.shape[0], lhs.shape[-1], rhs.shape[-1]
   assert rhs.shape[-2] == cin, (lhs.shape, rhs.shape)
-  a, out_sizes = _windows(lhs, kernel, strides, pads, dilation)  # [N*P, K]
+  both_int = lhs.dtype == torch.int8 and rhs.dtype == torch.int8
+  if both_int and ns <= 3:
+    a, out_sizes = ops.im2col_i8(lhs.contiguous(), kernel, strides, pads, dilation)  # [N*P, K]
+  else:
+    a, out_sizes = _windows(lhs, kernel, strides, pads, dilation)
   k = a.shape[1]
   b = rhs.reshape(k, cout).t().contiguous()  # [O, K]
-  both_int = lhs.dtype == torch.int8 and rhs.dtype == torch.int8
   if both_int:
     if a.shape[0] * cout == 0 or k == 0:
       out = torch.zeros((a.shape[0], cout), dtype=torch.int32, device=lhs.device)
@@ -134,7 +137,9 @@ def _fused_int8_conv(lhs_qt, rhs_qt, out_dtype, window_strides, padding, lhs_dil
   kernel = list(rq.shape[:ns])
   eff = [(k - 1) * d + 1 for k, d in zip(kernel, dilation)]
   pads = _explicit_padding(padding, list(lq.shape[1:1 + ns]), eff, strides)
-  a, out_sizes = _windows(lq.contiguous(), kernel, strides, pads, dilation)
+  if ns > 3:
+    return None
+  a, out_sizes = ops.im2col_i8(lq.contiguous(), kernel, strides, pads, dilation)
   k = a.shape[1]
   positions = math.prod(out_sizes)
   if a.shape[0] * cout == 0 or k == 0:

@@ -226,6 +226,24 @@ int aqtx_sum_tiles(const void* x, void* out, int64_t tiles, int64_t count, int32
                    void* stream);
 
 /*
+ * aqtx_im2col_i8: the windows of a quantized convolution input x [n][spatial...][c] (int8, one to
+ * three spatial axes, features innermost) as rows of out [n * positions][taps * c]: columns in
+ * the kernel's row-major tap order with the features innermost, zeros in the padding.  With it
+ * lax.conv_general_dilated on the quantized values (aqt/jax/v2/aqt_conv_general.py:95-107, Flax
+ * layout) is aqtx_gemm_i8 of out with the kernel reshaped to [features_out][taps * c].
+ * out_size[d] must be the number of window positions along axis d, i.e.
+ * (pad_lo + in_size + pad_hi - ((kernel - 1) * dilation + 1)) / stride + 1.
+ */
+typedef struct aqtx_im2col_plan {
+  int64_t n;            /* images */
+  int32_t c;            /* features */
+  int32_t rank;         /* spatial axes, 1..3 */
+  int32_t in_size[3], kernel[3], stride[3], dilation[3], pad_lo[3], out_size[3];
+} aqtx_im2col_plan;
+
+int aqtx_im2col_i8(const aqtx_im2col_plan* plan, const void* x, void* out, void* stream);
+
+/*
  * aqtx_fp_round: rounds x[count] (bf16 or f32) to an emulated small float with `nexp`
  * exponent bits, `nmant` mantissa bits, smallest exponent 0, with or without subnormals, no
  * NaN/inf codes, and writes the result in the same container dtype.  Replaces

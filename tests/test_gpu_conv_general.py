@@ -230,3 +230,29 @@ def test_conv_layer_train_convert_serve(gpu, bits):
   # an unconfigured layer is the plain convolution
   plain = aqt_flax.AqtConvGeneralDilated(None)(x, k, (1, 1), 'SAME', dimension_numbers=dn)
   np.testing.assert_allclose(plain.cpu().numpy(), R.lax_conv_nhwc(x_np, k_np, (1, 1), 'SAME'), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('case', [
+    dict(x=(2, 7, 6, 16), ker=(3, 2), strides=(1, 1), pads=[(1, 1), (0, 1)], dil=(1, 1)),
+    dict(x=(3, 9, 8, 32), ker=(3, 3), strides=(2, 1), pads=[(1, 1), (1, 1)], dil=(1, 1)),
+    dict(x=(2, 12, 11, 16), ker=(2, 3), strides=(1, 2), pads=[(0, 0), (0, 0)], dil=(2, 1)),
+    dict(x=(4, 33, 48), ker=(5,), strides=(3,), pads=[(2, 1)], dil=(1,)),
+    dict(x=(2, 5, 6, 4, 16), ker=(2, 2, 2), strides=(1, 1, 2), pads=[(0, 1), (1, 0), (0, 1)], dil=(1, 1, 1)),
+    dict(x=(2, 6, 5, 3), ker=(3, 3), strides=(1, 1), pads=[(1, 1), (1, 1)], dil=(1, 1)),   # features not a multiple of 16
+    dict(x=(1, 4, 4, 16), ker=(5, 5), strides=(1, 1), pads=[(0, 0), (0, 0)], dil=(1, 1)),   # window larger than the input
+    dict(x=(0, 4, 4, 16), ker=(3, 3), strides=(1, 1), pads=[(1, 1), (1, 1)], dil=(1, 1)),   # no images
+])
+def test_window_gather_kernel(gpu, case):
+  """aqtx_im2col_i8 against pad + unfold on the same int8 tensor."""
+  from aqt_amd import ops
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  rng = np.random.default_rng(3)
+  x = torch.from_numpy(rng.integers(-127, 128, case['x']).astype(np.int8)).to(gpu)
+  got, out_sizes = ops.im2col_i8(x, case['ker'], case['strides'], case['pads'], case['dil'])
+  if x.shape[0] == 0 or any(o == 0 for o in out_sizes):
+    assert got.shape[0] == 0
+    return
+  want, want_sizes = aqt_conv._windows(x, list(case['ker']), list(case['strides']), case['pads'], list(case['dil']))
+  assert list(out_sizes) == list(want_sizes) and got.shape == want.shape
+  assert torch.equal(got, want.contiguous())
