@@ -230,3 +230,20 @@ def test_small_entry_validation():
   assert 'dtype' in _err(L.lib().aqtx_sum_tiles(FAKE, FAKE, 4, 16, L.I8, None))
   assert 'NULL' in _err(L.lib().aqtx_sum_tiles(None, FAKE, 4, 16, L.BF16, None))
   assert L.lib().aqtx_sum_tiles(None, None, 4, 0, L.BF16, None) == 0
+
+
+def test_im2col_validation():
+  p = L.Im2colPlan()
+  p.n, p.c, p.rank = 2, 16, 2
+  for d in range(2):
+    p.in_size[d], p.kernel[d], p.stride[d], p.dilation[d], p.pad_lo[d], p.out_size[d] = 8, 3, 1, 1, 1, 8
+  assert 'NULL' in _err(L.lib().aqtx_im2col_i8(None, FAKE, FAKE, None))
+  assert 'NULL' in _err(L.lib().aqtx_im2col_i8(ctypes.byref(p), None, FAKE, None))
+  p.rank = 4
+  assert 'rank' in _err(L.lib().aqtx_im2col_i8(ctypes.byref(p), FAKE, FAKE, None))
+  p.rank = 2
+  p.stride[1] = 0
+  assert 'bad extent' in _err(L.lib().aqtx_im2col_i8(ctypes.byref(p), FAKE, FAKE, None))
+  p.stride[1] = 1
+  p.n = 0
+  assert L.lib().aqtx_im2col_i8(ctypes.byref(p), None, None, None) == 0
