@@ -1,6 +1,7 @@
 """fp8 numerics (mirrors aqt/jax/v2/numerics/fp8_numerics.py:25-145)."""
 from __future__ import annotations
 
+import copy
 import dataclasses
 from typing import Any
 
@@ -31,6 +32,13 @@ class Fp8Numerics(numerics.AqtNumerics):
   exponent_bits: int = 4
   mantissa_bits: int = 3
   stochastic_rounding: bool = False
+
+  def __deepcopy__(self, memo):
+    # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
+    # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
+    out = copy.copy(self)
+    memo[id(self)] = out
+    return out
 
   def _get_edge_of_last_fp8_bucket(self):
     return _FINFO_MAX[self.dtype]

@@ -5,6 +5,7 @@ class keep the reference's names.  Radix-4 rounding (fp_numerics.py:653-705) is 
 """
 from __future__ import annotations
 
+import copy
 import dataclasses
 from typing import Any, Optional
 
@@ -112,6 +113,13 @@ class FpNumerics(numerics.AqtNumerics):
   cfg: FpNumericsConfig
   stochastic_rounding: bool = False
   clip_gradient: bool = False
+
+  def __deepcopy__(self, memo):
+    # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
+    # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
+    out = copy.copy(self)
+    memo[id(self)] = out
+    return out
 
   def get_quant_bound(self):
     return fp_largest_representable(cfg=self.cfg)

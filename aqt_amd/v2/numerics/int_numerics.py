@@ -1,6 +1,7 @@
 """Symmetric integer numerics (mirrors aqt/jax/v2/numerics/int_numerics.py:25-125)."""
 from __future__ import annotations
 
+import copy
 import dataclasses
 from typing import Any
 
@@ -24,6 +25,13 @@ class IntSymmetric(numerics.AqtNumerics):
   round: bool
   noise_fn: Any  # None | stochastic_rounding.JaxUniform | RandomCenteredUniform | partial
   dtype: Any = None
+
+  def __deepcopy__(self, memo):
+    # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
+    # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
+    out = copy.copy(self)
+    memo[id(self)] = out
+    return out
 
   def get_edge_of_last_int_bucket(self):
     ret = 2.0 ** (self.bits - 1)

@@ -1,4 +1,5 @@
 """No quantization (mirrors aqt/jax/v2/numerics/no_numerics.py:23-43)."""
+import copy
 import dataclasses
 from typing import Any
 
@@ -7,8 +8,16 @@ from aqt_amd.v2.numerics import numerics
 
 @dataclasses.dataclass(kw_only=True)
 class NoNumerics(numerics.AqtNumerics):
+
   noise_fn: Any = None
   dtype: Any = None
+
+  def __deepcopy__(self, memo):
+    # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
+    # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
+    out = copy.copy(self)
+    memo[id(self)] = out
+    return out
 
   def get_dtype(self):
     return None
