@@ -1,7 +1,7 @@
 """Benchmark of the quantized dot_general hot path on one MI355X.
 
 One step = one int8 AqtDotGeneral forward + backward (dlhs, drhs) at the LLM MLP
-shape of BASELINE.json's metric: lhs bf16 [8192, 4096] (0.5% outliers x20), rhs
+shape the headline metric is quoted on: lhs bf16 [8192, 4096] (0.5% outliers x20), rhs
 bf16 [4096, 14336] ~N(0, 0.02), `fully_quantized(fwd_bits=8, bwd_bits=8)`:
 per-token / per-channel abs-max scales, RTN forward, stochastic rounding from a
 fixed PRNG key in dlhs/drhs, int32 accumulation, bf16 output.  Inputs live in HBM
