@@ -1008,15 +1008,19 @@ class DotGeneral:
     (out, qret), _ = dg_core_vjp_fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, self)
     return out, qret
 
-  def fused_tile_sum(self, lhs, rhs, dimension_numbers, n_sum_axes: int):
+  def fused_tile_sum(self, lhs, rhs, dimension_numbers, n_sum_axes: int, lhs_qt=None, rhs_qt=None,
+                     with_qt: bool = False):
     """sum over the leading `n_sum_axes` output axes of self(lhs, rhs, dimension_numbers), fused.
 
     This is what tiled_dot_general asks of its inner dot_general when the contraction axis is
     tiled: lhs [..., T, ts] and rhs [T, ts, ...] with the tile-count axis T as the only batch
     axis, every tile calibrated on its own, tile outputs dequantized and summed.  When the
     forward quantizers are plain int8/int4 abs-max ones and no gradient is needed, the
-    grouped-scale kernel does all of it without materialising the per-tile outputs.  Returns
-    None when the call does not have that shape (the caller then takes the unfused route).
+    grouped-scale kernel does all of it without materialising the per-tile outputs.  `rhs_qt`
+    may be a frozen weight (the serving case): it is read in the kernel's layout, an int4 one
+    packed two values per byte, both made once per frozen tensor.  Returns None when the call
+    does not have that shape (the caller then takes the unfused route); with `with_qt`,
+    (out, (lhs QTensor, rhs QTensor)) like dg_core.
     """
     if n_sum_axes != 1 or torch.is_grad_enabled() and (lhs.requires_grad or rhs.requires_grad):
       return None
@@ -1047,28 +1051,64 @@ class DotGeneral:
     T, ts = lhs.shape[-2], lhs.shape[-1]
     if ts % 128 != 0 or rhs.shape[0] != T or rhs.shape[1] != ts or nl < 3 or nr < 3:
       return None
-    self.assert_config_validity()
     M = int(math.prod(lhs.shape[:-2]))
     N = int(math.prod(rhs.shape[2:]))
     if M == 0 or N == 0:
       return None
-    sdts = []
-    outs = []
-    for x3, q, spec, reduce in ((lhs.reshape(1, M, T * ts), dq.lhs, specs[0], L.REDUCE_COLS),
-                                (rhs.reshape(1, T * ts, N), dq.rhs, specs[1], L.REDUCE_ROWS)):
-      sdt = q._calibrator.dtype if q._calibrator.dtype is not None else lhs.dtype
-      qv, sc = ops.quantize(x3, reduce=reduce, group=ts, transpose_out=reduce == L.REDUCE_ROWS,
-                            out_dtype=spec['out_dtype'], quant_bound=spec['quant_bound'],
-                            clip_bound=spec['clip_bound'], compute_dtype=lhs.dtype, scale_dtype=sdt)
-      outs.append((qv, sc))
-      sdts.append(sdt)
-    (lq, lsc), (rq, rsc) = outs
+    if lhs_qt is not None:
+      return None  # a quantized activation handed in: the step-by-step route knows what to do
+    frozen = rhs_qt is not None
+    if frozen:
+      sc = rhs_qt.scale[0] if rhs_qt.scale is not None and len(rhs_qt.scale) == 1 else None
+      if (not rhs_qt.is_full() or sc is None or rhs_qt.bias or rhs_qt.qvalue.dtype != torch.int8
+          or rhs_qt.container_dtype not in (None, utils.int4) or tuple(rhs_qt.qvalue.shape) != tuple(rhs.shape)
+          or tuple(sc.shape) != (T, 1) + tuple(rhs.shape[2:]) or sc.dtype not in (utils.bfloat16, utils.float32)
+          or rhs_qt.dequant_dtype not in (None, lhs.dtype)):
+        return None
+    self.assert_config_validity()
+    sdt_l = dq.lhs._calibrator.dtype if dq.lhs._calibrator.dtype is not None else lhs.dtype
+    lq, lsc = ops.quantize(lhs.reshape(1, M, T * ts), reduce=L.REDUCE_COLS, group=ts, out_dtype=specs[0]['out_dtype'],
+                           quant_bound=specs[0]['quant_bound'], clip_bound=specs[0]['clip_bound'],
+                           compute_dtype=lhs.dtype, scale_dtype=sdt_l)
+    rra = list(range(2, nr))
+    if frozen:
+      int4 = rhs_qt.container_dtype is utils.int4
+      rv = lowering.view_operand(rhs_qt.qvalue, [], rra, [0, 1])
+      packed = int4 and (T * ts) % 32 == 0
+      rq = _kernel_layout_of(rhs_qt.qvalue, rv, pack_int4=packed)     # [1, N, T*ts] (or packed)
+      b_dtype = L.I4P if packed else L.I4 if int4 else L.I8
+      sdt_r = sc.dtype
+      src = getattr(sc, 'f32_copy', None)
+      col_scale = (src if src is not None else sc).reshape(T, N).float().contiguous()
+    else:
+      sdt_r = dq.rhs._calibrator.dtype if dq.rhs._calibrator.dtype is not None else lhs.dtype
+      rq, rsc = ops.quantize(rhs.reshape(1, T * ts, N), reduce=L.REDUCE_ROWS, group=ts, transpose_out=True,
+                             out_dtype=specs[1]['out_dtype'], quant_bound=specs[1]['quant_bound'],
+                             clip_bound=specs[1]['clip_bound'], compute_dtype=lhs.dtype, scale_dtype=sdt_r)
+      b_dtype = specs[1]['out_dtype']
+      col_scale = rsc.reshape(T, N)
     row_scale = lsc.reshape(M, T).t().contiguous()     # [T, M]
-    col_scale = rsc.reshape(T, N)
     out = ops.gemm_grouped(lq[0], rq[0], row_scale=row_scale, col_scale=col_scale, group=ts,
-                           out_dtype=lhs.dtype, row_scale_dtype=sdts[0], col_scale_dtype=sdts[1],
-                           a_dtype=specs[0]['out_dtype'], b_dtype=specs[1]['out_dtype'])
-    return out.reshape(tuple(lhs.shape[:-2]) + tuple(rhs.shape[2:]))
+                           out_dtype=lhs.dtype, row_scale_dtype=sdt_l, col_scale_dtype=sdt_r,
+                           a_dtype=specs[0]['out_dtype'], b_dtype=b_dtype)
+    out = out.reshape(tuple(lhs.shape[:-2]) + tuple(rhs.shape[2:]))
+    if not with_qt:
+      return out
+    mk_container = lambda spec: utils.int4 if spec['out_dtype'] == L.I4 else None
+    lhs_qt_out = aqt_tensor.QTensor(
+        qvalue=lq.reshape(lhs.shape), scale=[lsc.reshape(tuple(lhs.shape[:-1]) + (1,)).to(sdt_l)], scale_t=None,
+        bias=[], dequant_dtype=lhs.dtype, container_dtype=mk_container(specs[0]))
+    if frozen:
+      rhs_qt_out = rhs_qt
+    else:
+      rest = tuple(rhs.shape[2:])
+      n_rest = len(rest)
+      # [N, T*ts] as the kernel wrote it -> [T, ts, rest...] (a view)
+      qv = rq.reshape(rest + (T, ts)).permute(tuple([n_rest, n_rest + 1] + list(range(n_rest))))
+      rhs_qt_out = aqt_tensor.QTensor(
+          qvalue=qv, scale=[rsc.reshape((T, 1) + rest).to(sdt_r)], scale_t=None, bias=[],
+          dequant_dtype=rhs.dtype, container_dtype=mk_container(specs[1]))
+    return out, (lhs_qt_out, rhs_qt_out)
 
   def __call__(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
     """aqt_dot_general.py:1002-1022."""

@@ -287,6 +287,28 @@ class AqtDotGeneral(torch.nn.Module, _RngMixin):
         rhs_freezer.set(out_rhs_qt)
       return out
 
+    def fused_tile_sum(tl, tr, tiled_dn, n_sum_axes):
+      """tiled_dot_general's shortcut for a tiled contraction axis (contract, dequantize and sum the
+      tiles in one kernel), with the same freezer traffic as ret_dg; None if it does not apply."""
+      if self.use_legacy_freezer:
+        return None
+      lhs_qt = lhs_freezer.get() if self.lhs_apply_quant_mode else self.lhs_qtensor
+      rhs_qt = rhs_freezer.get() if self.rhs_apply_quant_mode else self.rhs_qtensor
+      res = cfg.fused_tile_sum(tl, tr, tiled_dn, n_sum_axes, lhs_qt=lhs_qt, rhs_qt=rhs_qt, with_qt=True)
+      if res is None:
+        return None
+      out, (out_lhs_qt, out_rhs_qt) = res
+      out_lhs_qt = _apply_freeze_mode(out_lhs_qt, self.lhs_freeze_mode, self.lhs_apply_quant_mode,
+                                      self.lhs_quant_mode, 'lhs')
+      out_rhs_qt = _apply_freeze_mode(out_rhs_qt, self.rhs_freeze_mode, self.rhs_apply_quant_mode,
+                                      self.rhs_quant_mode, 'rhs')
+      if self.lhs_apply_quant_mode:
+        lhs_freezer.set(out_lhs_qt)
+      if self.rhs_apply_quant_mode:
+        rhs_freezer.set(out_rhs_qt)
+      return out
+
+    ret_dg.fused_tile_sum = fused_tile_sum
     return ret_dg
 
   def forward(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
@@ -301,11 +323,14 @@ class AqtDotGeneral(torch.nn.Module, _RngMixin):
 
       def probe(l, r, dn, precision=None, preferred_element_type=None):
         seen['l'], seen['r'], seen['dn'] = tuple(l.shape), tuple(r.shape), dn
-        return aqt_dot_general.lax_dot_general(l, r, dn, precision, preferred_element_type)
+        raise _ProbeDone()  # the shapes are all that is wanted; the tile sums after it cost host time
 
       meta = lambda t: torch.empty(t.shape, dtype=torch.float32, device='meta')
-      tiled_dot_general.tiled_dot_general_with_tiling_states(
-          meta(lhs), copy.deepcopy(xlhs), meta(rhs), copy.deepcopy(xrhs), dimension_numbers, dot_general=probe)
+      try:
+        tiled_dot_general.tiled_dot_general_with_tiling_states(
+            meta(lhs), copy.deepcopy(xlhs), meta(rhs), copy.deepcopy(xrhs), dimension_numbers, dot_general=probe)
+      except _ProbeDone:
+        pass
       aqt_dg = self.make_aqt_dg(seen['l'], seen['r'], seen['dn'], lhs_tile_map=xlhs.tile_map,
                                 rhs_tile_map=xrhs.tile_map)
       ret_dg = functools.partial(tiled_dot_general.tiled_dot_general, tiling_cfg, dot_general=aqt_dg)

@@ -173,6 +173,22 @@ def other_configs(dev):
 
   ms = timeit(step5)
   out['int4w_int8a_tiled128_fwd'] = {'ms_per_call': round(ms, 3), 'TOPS': round(2 * 2048 * 8192 * 28672 / ms / 1e9, 1)}
+  # the same contraction as a serving layer: the int4 weight frozen once (packed two values per byte), only the
+  # activations quantized per call
+  from aqt_amd.v2.flax import aqt_flax
+  mk = lambda mode: aqt_flax.AqtDotGeneral(
+      aqt.dot_general_make(8, 4), rhs_quant_mode=mode, tiling_cfg=tcfg, use_legacy_freezer=False,
+      lhs_freeze_mode=aqt_flax.FreezerMode.CALIBRATION, rhs_freeze_mode=aqt_flax.FreezerMode.CALIBRATION_AND_VALUE,
+      rngs={'params': utils.prng_key(0)})
+  with torch.no_grad():
+    conv = mk(utils.QuantMode.CONVERT)
+    conv(lhs, rhs, MATMUL, None)
+    serve = mk(utils.QuantMode.SERVE)
+    serve.load_variables(conv.variables())
+    ms = timeit(lambda: serve(lhs, rhs, MATMUL, None))
+  out['int4w_packed_frozen_tiled128_serving_fwd'] = {
+      'ms_per_call': round(ms, 3), 'TOPS': round(2 * 2048 * 8192 * 28672 / ms / 1e9, 1)}
+  del conv, serve
   del lhs, rhs
   # quantized ragged_dot (mixture of experts): 8192 tokens routed to 8 experts [4096, 14336], uneven groups,
   # forward, with the expert weights quantized on the fly (the reference's ragged_dot does the same) and

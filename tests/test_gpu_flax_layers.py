@@ -225,3 +225,58 @@ def test_e2e_example_head_convert_and_serve(gpu, bits):
   node.qvalue = torch.zeros_like(node.qvalue)
   serve_layers[0].load_variables(broken)
   assert not torch.equal(forward(serve_layers, torch.zeros_like(w0), torch.zeros_like(w1)), logits_train)
+
+
+@pytest.mark.parametrize('rhs_bits', [8, 4])
+def test_tiled_layer_serves_frozen_weights_through_the_grouped_kernel(gpu, rhs_bits, monkeypatch):
+  """A Dense-like layer with the contraction axis in tiles of 256: training-mode forward (no
+  gradient asked), conversion and serving all run the grouped-scale kernel (one launch instead of
+  one contraction per tile plus a sum), serving reads the frozen weight -- an int4 one packed two
+  per byte -- and all three equal the oracle's tiled dot_general bit for bit."""
+  from aqt_amd import ops
+  dt = 'bf16'
+  m, k, n, tiles = 16, 1024, 384, 4
+  x_np, w_np = U.rand((m, k), dt, 1, outliers=True), U.rand((k, n), dt, 2, 0.02)
+  x, w = U.to_dev(x_np, dt, gpu), U.to_dev(w_np, dt, gpu)
+  cfg = aqt.dot_general_make(8, rhs_bits)
+  tiling = tiled_dot_general.Cfg(
+      lhs=tiled_dot_general.TensorTiling(
+          contraction_axes=[tiled_dot_general.AxisTiling(axis=1, tile_count=tiles, tile_size=None)], remaining_axes=[]),
+      rhs=tiled_dot_general.TensorTiling(
+          contraction_axes=[tiled_dot_general.AxisTiling(axis=0, tile_count=tiles, tile_size=None)], remaining_axes=[]))
+  calls = []
+  real = ops.gemm_grouped
+  monkeypatch.setattr(ops, 'gemm_grouped', lambda *a, **kw: (calls.append(kw.get('b_dtype')), real(*a, **kw))[1])
+  mk = lambda mode: aqt_flax.AqtDotGeneral(
+      cfg, rhs_quant_mode=mode, tiling_cfg=tiling, lhs_freeze_mode=FM.CALIBRATION,
+      rhs_freeze_mode=FM.CALIBRATION_AND_VALUE, use_legacy_freezer=False, rngs=_rngs())
+  want, _ = R.tiled_dg_fwd(x_np, w_np, dt, k // tiles, R.dot_general_make(8, rhs_bits))
+  with torch.no_grad():
+    out_train = mk(QM.TRAIN)(x, w, MATMUL, None)
+    conv = mk(QM.CONVERT)
+    out_conv = conv(x, w, MATMUL, None)
+    v = conv.variables()
+    frozen = v['aqt']['qrhs']['frozen']
+    assert tuple(frozen.qvalue.shape) == (tiles, k // tiles, n) and frozen.qvalue.dtype == torch.int8
+    assert [tuple(s.shape) for s in frozen.scale] == [(tiles, 1, n)]
+    assert (frozen.container_dtype is utils.int4) == (rhs_bits == 4)
+    serve = mk(QM.SERVE)
+    serve.load_variables(v)
+    out_serve = serve(x, torch.zeros_like(w), MATMUL, None)
+    # a checkpoint restore hands the values back in their logical order
+    import copy
+    v2 = copy.deepcopy(v)
+    node = v2['aqt']['qrhs']['frozen']
+    node.qvalue = node.qvalue.contiguous().clone()
+    serve2 = mk(QM.SERVE)
+    serve2.load_variables(v2)
+    out_serve2 = serve2(x, torch.zeros_like(w), MATMUL, None)
+  from aqt_amd import _lib as L
+  assert len(calls) == 4 and calls[2] == calls[3] == (L.I4P if rhs_bits == 4 else L.I8), calls
+  for out in (out_train, out_conv, out_serve, out_serve2):
+    np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+  # with a gradient asked for, the layer takes the per-tile route and gives the same forward values
+  xg = x.clone().requires_grad_(True)
+  out_grad = mk(QM.TRAIN)(xg, w, MATMUL, None)
+  assert len(calls) == 4
+  np.testing.assert_array_equal(out_grad.detach().float().cpu().numpy(), want)
