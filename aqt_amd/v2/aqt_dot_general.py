@@ -912,18 +912,37 @@ class DotGeneralRaw:
           raise _NotFused(f'{name}: a scale that is not shared over exactly the contraction axes')
         flat = sv.mem.reshape(-1).float()
       scale_in = flat.contiguous().reshape(v.B, v.R, 1) if v.k_last else flat.contiguous().reshape(v.B, 1, v.R)
+    # Both gradient contractions calibrate the same gradient; with one scale per tensor and no
+    # forward-scale factor on it the abs-max is the same number, found once per backward pass.
+    memo_key, memo_hit = None, None
+    if (_PER_TENSOR_SCALES is not None and given_qt is None and prescale is None and not x_is_q
+        and quantizer.calib_shared_axes == 'per_tensor' and quantizer.kernel_spec() is not None):
+      memo_key = (arr.data_ptr(), arr._version, tuple(arr.shape), arr.dtype, spec['quant_bound'],
+                  quantizer._calibrator.dtype)
+      memo_hit = _PER_TENSOR_SCALES.get(memo_key)
+      if memo_hit is not None:
+        flat = memo_hit[0].reshape(1).expand(v.B * v.R)
+        scale_in = flat.contiguous().reshape(v.B, v.R, 1) if v.k_last else flat.contiguous().reshape(v.B, 1, v.R)
+        scale_dtype = memo_hit[2]
     q, s32, sdt = quantizer.quant_view(v, dtype, calibration_axes=ca, prescale=prescale, scale=scale_in,
                                        scale_dtype=scale_dtype)
     qv = lowering.logical_from_brk(aqt_quantizer._typed(q, spec['out_dtype']), v)
-    if given_qt is not None:
+    if memo_hit is not None:
+      s32, scale_list = memo_hit[0], memo_hit[1]
+    elif given_qt is not None:
       scale_list = given_qt.scale
     else:
       scale_list = [lowering.scale_in_dtype(s32, v, sdt)]
+      if memo_key is not None:
+        _PER_TENSOR_SCALES[memo_key] = (s32, scale_list, sdt)
     qt = aqt_tensor.QTensor(qvalue=qv, scale=scale_list, scale_t=None, bias=[], dequant_dtype=dtype,
                             container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
     quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))
     return q, s32, sdt, qt, quant_grad
 
+
+# per-tensor scales found during the backward pass in progress (None outside one)
+_PER_TENSOR_SCALES = None
 
 _DTYPES_CAN_BE_SCALED = (torch.bfloat16, torch.float32, torch.float64)
 
@@ -1213,8 +1232,13 @@ def dg_core_vjp_bwd(fwd_dimension_numbers, res, g):
       transposed_out = quant_grad(transposed_out)[0]
     return transposed_out
 
-  dlhs = grad_dot_general(dg_res.rhs, dg_res.lhs.quant_grad, cfg.dlhs, False)
-  drhs = grad_dot_general(dg_res.lhs, dg_res.rhs.quant_grad, cfg.drhs, True)
+  global _PER_TENSOR_SCALES
+  _PER_TENSOR_SCALES = {}
+  try:
+    dlhs = grad_dot_general(dg_res.rhs, dg_res.lhs.quant_grad, cfg.dlhs, False)
+    drhs = grad_dot_general(dg_res.lhs, dg_res.rhs.quant_grad, cfg.drhs, True)
+  finally:
+    _PER_TENSOR_SCALES = None
   return (dlhs, drhs, None, None, None)
 
 
