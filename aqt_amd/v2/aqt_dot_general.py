@@ -9,7 +9,6 @@ torch.autograd.Function in place of jax.custom_vjp.
 from __future__ import annotations
 
 import abc
-import copy
 import dataclasses
 import enum
 import functools
@@ -996,7 +995,7 @@ def _qtensor_dot_general(lhs_qt, rhs_qt, dimension_numbers, cfg, dequant_dtype):
   dequantizes; here the dequantisation is fused into the contraction kernel, so the
   dequantized array is returned directly.
   """
-  raw = copy.copy(cfg)
+  raw = utils.clone_fields(cfg)
   out, _ = DotGeneralRaw._lowered_call(raw, lhs_qt.qvalue, rhs_qt.qvalue, lhs_qt, rhs_qt, dimension_numbers)
   return out.to(dequant_dtype)
 
@@ -1163,13 +1162,13 @@ def _fresh_cfg(cfg: 'DotGeneral') -> 'DotGeneral':
   fresh copy on every call, which is why init_calibration() may assert that it runs once;
   this gives a reused config object the same behaviour.
   """
-  cfg = copy.copy(cfg)
+  cfg = utils.clone_fields(cfg)
   for name in ('fwd', 'dlhs', 'drhs'):
-    raw = copy.copy(getattr(cfg, name))
-    dq = copy.copy(raw.dg_quantizer)
+    raw = utils.clone_fields(getattr(cfg, name))
+    dq = utils.clone_fields(raw.dg_quantizer)
     for qn in ('lhs', 'rhs', 'lhs_mid', 'rhs_mid'):
       if hasattr(dq, qn):
-        q = copy.copy(getattr(dq, qn))
+        q = utils.clone_fields(getattr(dq, qn))
         q._calibrator = None
         setattr(dq, qn, q)
     raw.dg_quantizer = dq

@@ -1,6 +1,7 @@
 """One-tensor quantizer (mirrors aqt/jax/v2/aqt_quantizer.py:38-214)."""
 from __future__ import annotations
 
+import copy
 import dataclasses
 import functools
 from typing import Any, Optional, Sequence
@@ -31,6 +32,19 @@ class Quantizer:
   calibration: Any = None  # class or functools.partial producing a Calibration
   _calibrator: Any = None
   context: utils.Context = None
+
+  def __deepcopy__(self, memo):
+    # Field by field: the flags, dtype tags and the calibration factory (a class or a
+    # functools.partial, never changed in place) are shared, the rest is copied.  Same result as
+    # the generic deep copy; configurations are copied on every layer call.
+    out = utils.clone_fields(self)
+    memo[id(self)] = out
+    out.numerics = copy.deepcopy(self.numerics, memo)
+    if not isinstance(self.calib_shared_axes, (str, type(None))):
+      out.calib_shared_axes = copy.deepcopy(self.calib_shared_axes, memo)
+    out._calibrator = copy.deepcopy(self._calibrator, memo)
+    out.context = copy.deepcopy(self.context, memo)
+    return out
 
   def init_calibration(self):
     assert self._calibrator is None, 'second call to self.init_calibration()'

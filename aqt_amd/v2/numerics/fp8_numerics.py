@@ -1,7 +1,6 @@
 """fp8 numerics (mirrors aqt/jax/v2/numerics/fp8_numerics.py:25-145)."""
 from __future__ import annotations
 
-import copy
 import dataclasses
 from typing import Any
 
@@ -36,7 +35,7 @@ class Fp8Numerics(numerics.AqtNumerics):
   def __deepcopy__(self, memo):
     # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
     # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
-    out = copy.copy(self)
+    out = utils.clone_fields(self)
     memo[id(self)] = out
     return out
 

@@ -5,7 +5,6 @@ class keep the reference's names.  Radix-4 rounding (fp_numerics.py:653-705) is 
 """
 from __future__ import annotations
 
-import copy
 import dataclasses
 from typing import Any, Optional
 
@@ -117,7 +116,7 @@ class FpNumerics(numerics.AqtNumerics):
   def __deepcopy__(self, memo):
     # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
     # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
-    out = copy.copy(self)
+    out = utils.clone_fields(self)
     memo[id(self)] = out
     return out
 

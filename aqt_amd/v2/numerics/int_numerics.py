@@ -1,7 +1,6 @@
 """Symmetric integer numerics (mirrors aqt/jax/v2/numerics/int_numerics.py:25-125)."""
 from __future__ import annotations
 
-import copy
 import dataclasses
 from typing import Any
 
@@ -29,7 +28,7 @@ class IntSymmetric(numerics.AqtNumerics):
   def __deepcopy__(self, memo):
     # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
     # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
-    out = copy.copy(self)
+    out = utils.clone_fields(self)
     memo[id(self)] = out
     return out
 

@@ -1,8 +1,8 @@
 """No quantization (mirrors aqt/jax/v2/numerics/no_numerics.py:23-43)."""
-import copy
 import dataclasses
 from typing import Any
 
+from aqt_amd.v2 import utils
 from aqt_amd.v2.numerics import numerics
 
 
@@ -15,7 +15,7 @@ class NoNumerics(numerics.AqtNumerics):
   def __deepcopy__(self, memo):
     # every field is immutable (numbers, flags, dtype tags, a noise function): a field-wise copy
     # is a deep copy, at a fraction of the cost (configurations are copied on every layer call)
-    out = copy.copy(self)
+    out = utils.clone_fields(self)
     memo[id(self)] = out
     return out
 
