@@ -6,6 +6,7 @@ or the library is missing -- there is no CPU path.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import math
 from typing import Optional, Sequence
@@ -93,6 +94,18 @@ def _require_gpu(*tensors):
 # One abs-max workspace per (device, stream), kept zeroed by the library between calls, so that
 # the column and whole-tensor calibrations do not pay a clearing launch each time.
 _QUANT_WS = {}
+
+
+@contextlib.contextmanager
+def private_workspaces(store: dict):
+  """Calls made inside keep their abs-max workspaces in `store` instead of the process-wide table:
+  a recorded HIP graph owns the workspace its kernels were recorded with."""
+  global _QUANT_WS
+  prev, _QUANT_WS = _QUANT_WS, store
+  try:
+    yield store
+  finally:
+    _QUANT_WS = prev
 
 
 def _quantize_workspace(nbytes: int, device) -> torch.Tensor:

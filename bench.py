@@ -190,6 +190,25 @@ def other_configs(dev):
       'ms_per_call': round(ms, 3), 'TOPS': round(2 * 2048 * 8192 * 28672 / ms / 1e9, 1)}
   del conv, serve
   del lhs, rhs
+  # one decode-sized serving layer call (8 x 4096 against a frozen int8 [4096, 14336] weight): issued from Python
+  # each time, and recorded once into a HIP graph and replayed (host time included in both)
+  from aqt_amd.v2 import hip_graph
+  xs = torch.randn(8, 4096, device=dev).to(torch.bfloat16)
+  ws = (torch.randn(4096, 14336, device=dev) * 0.02).to(torch.bfloat16)
+  mk8 = lambda mode: aqt_flax.AqtDotGeneral(
+      config.fully_quantized(use_stochastic_rounding=False), rhs_quant_mode=mode, use_legacy_freezer=False,
+      rhs_freeze_mode=aqt_flax.FreezerMode.CALIBRATION_AND_VALUE, rngs={'params': utils.prng_key(0)})
+  with torch.no_grad():
+    conv = mk8(utils.QuantMode.CONVERT)
+    conv(xs, ws, MATMUL, None)
+    serve = mk8(utils.QuantMode.SERVE)
+    serve.load_variables(conv.variables())
+    call = lambda a: serve(a, ws, MATMUL, None)
+    graphed = hip_graph.GraphedCall(call, xs)
+    out['int8_frozen_serving_layer_call_m8_4096x14336'] = {
+        'eager_us_per_call': round(timeit(lambda: call(xs), n=100, w=10) * 1e3, 1),
+        'hip_graph_us_per_call': round(timeit(lambda: graphed(xs), n=100, w=10) * 1e3, 1)}
+  del conv, serve, graphed, xs, ws
   # quantized ragged_dot (mixture of experts): 8192 tokens routed to 8 experts [4096, 14336], uneven groups,
   # forward, with the expert weights quantized on the fly (the reference's ragged_dot does the same) and
   # with the contraction alone (operands already int8)

@@ -1,0 +1,120 @@
+"""GPU: serving calls recorded into a HIP graph give the eager call's bits on every replay.
+
+Each graph is replayed several times on fresh inputs, with eager calls of the same layer (and
+synchronisations) between the replays, and every replay is compared with the eager result.
+"""
+import pytest
+import torch
+
+from aqt_amd.v2 import aqt_dot_general as aqt
+from aqt_amd.v2 import config
+from aqt_amd.v2 import hip_graph
+from aqt_amd.v2 import tiled_dot_general
+from aqt_amd.v2 import utils
+from aqt_amd.v2.flax import aqt_flax
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+QM, FM = utils.QuantMode, aqt_flax.FreezerMode
+MATMUL = (((1,), (0,)), ((), ()))
+
+
+def _rngs():
+  return {'params': utils.prng_key(0)}
+
+
+def _serving_layer(cfg, x, w, tiling=None):
+  mk = lambda mode: aqt_flax.AqtDotGeneral(
+      cfg, rhs_quant_mode=mode, tiling_cfg=tiling, lhs_freeze_mode=FM.CALIBRATION,
+      rhs_freeze_mode=FM.CALIBRATION_AND_VALUE, use_legacy_freezer=False, rngs=_rngs())
+  with torch.no_grad():
+    conv = mk(QM.CONVERT)
+    conv(x, w, MATMUL, None)
+    serve = mk(QM.SERVE)
+    serve.load_variables(conv.variables())
+  return serve
+
+
+def _check_replays(graphed, eager, make_input, n=5):
+  for i in range(n):
+    x = make_input(100 + i)
+    got = graphed(x).clone()
+    torch.cuda.synchronize()
+    with torch.no_grad():
+      want = eager(x)
+      eager(make_input(500 + i))  # eager work of the same kernels between replays
+    torch.cuda.synchronize()
+    assert got.dtype == want.dtype and got.shape == want.shape
+    assert torch.equal(got, want), f'replay {i} differs from the eager call'
+
+
+@pytest.mark.parametrize('m', [1, 8, 64, 512])
+def test_int8_serving_layer_replays(gpu, m):
+  """Frozen int8 weight: the small-batch decode kernels (m <= 64) and the dense GEMM (m = 512)."""
+  dt = 'bf16'
+  k, n = 1024, 1536
+  w = U.to_dev(U.rand((k, n), dt, 2, 0.02), dt, gpu)
+  mk = lambda seed: U.to_dev(U.rand((m, k), dt, seed, outliers=True), dt, gpu)
+  serve = _serving_layer(config.fully_quantized(use_stochastic_rounding=False), mk(1), w)
+  call = lambda x: serve(x, w, MATMUL, None)
+  graphed = hip_graph.GraphedCall(call, mk(1))
+  _check_replays(graphed, call, mk)
+
+
+@pytest.mark.parametrize('rhs_bits', [8, 4])
+def test_tiled_serving_layer_replays(gpu, rhs_bits):
+  """Subchannel scales (contraction axis in 4 tiles): the grouped-scale kernel, int4 weight packed."""
+  dt = 'bf16'
+  m, k, n, tiles = 16, 1024, 384, 4
+  w = U.to_dev(U.rand((k, n), dt, 2, 0.02), dt, gpu)
+  mk = lambda seed: U.to_dev(U.rand((m, k), dt, seed, outliers=True), dt, gpu)
+  tiling = tiled_dot_general.Cfg(
+      lhs=tiled_dot_general.TensorTiling(
+          contraction_axes=[tiled_dot_general.AxisTiling(axis=1, tile_count=tiles, tile_size=None)], remaining_axes=[]),
+      rhs=tiled_dot_general.TensorTiling(
+          contraction_axes=[tiled_dot_general.AxisTiling(axis=0, tile_count=tiles, tile_size=None)], remaining_axes=[]))
+  serve = _serving_layer(aqt.dot_general_make(8, rhs_bits), mk(1), w, tiling)
+  call = lambda x: serve(x, w, MATMUL, None)
+  graphed = hip_graph.GraphedCall(call, mk(1))
+  _check_replays(graphed, call, mk)
+
+
+def test_both_operands_quantized_per_call_replays(gpu):
+  """No frozen state: both operands calibrated and quantized inside the recorded call."""
+  dt = 'bf16'
+  m, k, n = 256, 512, 384
+  mk = lambda seed: U.to_dev(U.rand((m, k), dt, seed, outliers=True), dt, gpu)
+  w = U.to_dev(U.rand((k, n), dt, 2, 0.02), dt, gpu)
+  dg = config.config_v4()
+  call = lambda x: dg(x, w, MATMUL)
+  graphed = hip_graph.GraphedCall(call, mk(1))
+  _check_replays(graphed, call, mk)
+
+
+def test_static_argument_is_read_in_place(gpu):
+  dt = 'bf16'
+  x = U.to_dev(U.rand((64, 256), dt, 1), dt, gpu)
+  w = U.to_dev(U.rand((256, 128), dt, 2, 0.02), dt, gpu)
+  dg = config.config_v4()
+  graphed = hip_graph.GraphedCall(lambda a, b: dg(a, b, MATMUL), x, w, static_argnums=(1,))
+  assert graphed.inputs[1] is w and graphed.inputs[0] is not x
+  w2 = U.to_dev(U.rand((256, 128), dt, 3, 0.02), dt, gpu)
+  w.copy_(w2)
+  got = graphed(x, w).clone()
+  with torch.no_grad():
+    assert torch.equal(got, dg(x, w2, MATMUL))
+
+
+def test_argument_checks(gpu):
+  x = torch.zeros(8, 256, device=gpu, dtype=torch.bfloat16)
+  w = torch.ones(256, 128, device=gpu, dtype=torch.bfloat16)
+  dg = config.config_v4()
+  graphed = hip_graph.GraphedCall(lambda a: dg(a, w, MATMUL), x)
+  with pytest.raises(ValueError, match='recorded as'):
+    graphed(torch.zeros(4, 256, device=gpu, dtype=torch.bfloat16))
+  with pytest.raises(ValueError, match='recorded as'):
+    graphed(x.float())
+  with pytest.raises(ValueError, match='arguments'):
+    graphed(x, x)
+  with pytest.raises(ValueError, match='GPU'):
+    hip_graph.GraphedCall(lambda a: a, torch.zeros(4))
