@@ -667,7 +667,10 @@ class DotGeneralRaw:
     return out, res
 
   # ------------------------------------------------------------------------------
-  def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None):
+  def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None,
+                    _dtypes=None):
+    """`_dtypes` = (lhs dtype, rhs dtype, dequant dtype) when `lhs` and `rhs` are the qvalues of
+    the given QTensors and so do not carry the dtypes of the tensors they were quantized from."""
     dq = self.dg_quantizer
     prescale_t = None
     if isinstance(lhs, _Prescaled):
@@ -677,6 +680,8 @@ class DotGeneralRaw:
     lhs_dtype = lhs.dtype
     rhs_dtype = rhs.dequant_dtype if rhs_is_q else rhs.dtype
     dequant_dtype = torch.promote_types(lhs_dtype, rhs_dtype)
+    if _dtypes is not None:
+      lhs_dtype, rhs_dtype, dequant_dtype = _dtypes
 
     lhs_none = isinstance(dq.lhs.numerics, no_numerics.NoNumerics) if isinstance(
         dq, DefaultDotGeneralQuantizer) else False
@@ -996,8 +1001,9 @@ def _qtensor_dot_general(lhs_qt, rhs_qt, dimension_numbers, cfg, dequant_dtype):
   dequantized array is returned directly.
   """
   raw = utils.clone_fields(cfg)
-  out, _ = DotGeneralRaw._lowered_call(raw, lhs_qt.qvalue, rhs_qt.qvalue, lhs_qt, rhs_qt, dimension_numbers)
-  return out.to(dequant_dtype)
+  out, _ = DotGeneralRaw._lowered_call(raw, lhs_qt.qvalue, rhs_qt.qvalue, lhs_qt, rhs_qt, dimension_numbers,
+                                       _dtypes=(lhs_qt.dequant_dtype, rhs_qt.dequant_dtype, dequant_dtype))
+  return out
 
 
 @dataclasses.dataclass(kw_only=True)
