@@ -941,10 +941,14 @@ int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales,
     }
     if (reduce == AQTX_REDUCE_ALL || reduce == AQTX_REDUCE_ALL_BATCH) {
       int64_t nblk = (a.rows * a.cols + 256 * 16 - 1) / (256 * 16);
-      // Every block ends in one atomic max, and atomics on one address take turns (about 10 ns each,
-      // measured): at most 2048 blocks per abs-max word, also when all batch entries share the word.
-      int64_t cap = 2048;
-      if (reduce == AQTX_REDUCE_ALL_BATCH && a.batch > 1) cap = a.batch >= 2048 ? 1 : 2048 / a.batch;
+      // Every block ends in one atomic max.  Atomics on one address take turns (about 10 ns each,
+      // measured), and so do those on the neighbouring words of the batch entries, which share a
+      // cache line: 32 entries x 98 blocks took 31 us for 26 MB.  So the launch as a whole gets at
+      // most one block per 48 KiB of input (the time to stream that much), between 256 and 2048.
+      const int64_t total_bytes = a.batch * a.rows * a.cols * (int64_t)sizeof(TIn);
+      int64_t cap_total = total_bytes / (48 << 10);
+      cap_total = cap_total < 256 ? 256 : cap_total > 2048 ? 2048 : cap_total;
+      const int64_t cap = a.batch >= cap_total ? 1 : cap_total / a.batch;
       if (nblk > cap) nblk = cap;
       if (nblk < 1) nblk = 1;
       absmax_all_kernel<TIn><<<dim3((unsigned)nblk, (unsigned)a.batch), 256, 0, st>>>(a);

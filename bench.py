@@ -253,9 +253,15 @@ def other_configs(dev):
   conv = aqt_conv_general.make_conv_general_dilated(aqt_conv_general.conv_general_dilated_make(2, 8, 8))
   dnc = aqt_conv_general.flax_conv_dimension_numbers(xc.shape)
   with torch.no_grad():
-    ms = timeit(lambda: conv(xc, kc, (1, 1), 'SAME', dimension_numbers=dnc))
+    call = lambda a: conv(a, kc, (1, 1), 'SAME', dimension_numbers=dnc)
+    ms = timeit(lambda: call(xc))
+    graphed = hip_graph.GraphedCall(call, xc)
+    ms_graph = timeit(graphed.replay, n=20, w=3)
+  gop = 2.0 * 32 * 56 * 56 * 9 * 128 * 128 / 1e9
   out['conv_int8_fwd_32x56x56x128_k3x3_128'] = {
-      'ms_per_call': round(ms, 3), 'TOPS': round(2.0 * 32 * 56 * 56 * 9 * 128 * 128 / ms / 1e9, 1)}
+      'ms_per_call': round(ms, 3), 'TOPS': round(gop / ms, 1),
+      'hip_graph_ms_per_call': round(ms_graph, 3), 'hip_graph_TOPS': round(gop / ms_graph, 1)}
+  del graphed
   return out
 
 

@@ -91,6 +91,42 @@ def test_both_operands_quantized_per_call_replays(gpu):
   _check_replays(graphed, call, mk)
 
 
+def test_quantized_convolution_replays(gpu):
+  """conv_general_dilated: per-batch-element abs-max through the kept-zero workspace (owned by the
+  graph), window gather, contraction with both scales in the epilogue."""
+  from aqt_amd.v2 import aqt_conv_general
+  dt = 'bf16'
+  mk = lambda seed: U.to_dev(U.rand((4, 14, 14, 128), dt, seed, outliers=True), dt, gpu)
+  kernel = U.to_dev(U.rand((3, 3, 128, 64), dt, 2, 0.05), dt, gpu)
+  conv = aqt_conv_general.make_conv_general_dilated(aqt_conv_general.conv_general_dilated_make(2, 8, 8))
+  dn = aqt_conv_general.flax_conv_dimension_numbers((4, 14, 14, 128))
+  call = lambda x: conv(x, kernel, (1, 1), 'SAME', dimension_numbers=dn)
+  graphed = hip_graph.GraphedCall(call, mk(1))
+  _check_replays(graphed, call, mk)
+  # a second graph recorded while the first is alive, replayed alternately
+  other = hip_graph.GraphedCall(call, mk(2))
+  for i in range(3):
+    xa, xb = mk(40 + i), mk(60 + i)
+    ya = graphed(xa).clone()
+    yb = other(xb).clone()
+    with torch.no_grad():
+      assert torch.equal(ya, call(xa)) and torch.equal(yb, call(xb))
+
+
+def test_per_tensor_scales_replay(gpu):
+  """Whole-tensor abs-max (atomics into the kept-zero workspace) inside a recording."""
+  dt = 'bf16'
+  mk = lambda seed: U.to_dev(U.rand((512, 1024), dt, seed, outliers=True), dt, gpu)
+  w = U.to_dev(U.rand((1024, 256), dt, 2, 0.02), dt, gpu)
+  dg = config.config_v4()
+  for raw in (dg.fwd,):
+    raw.dg_quantizer.lhs.calib_shared_axes = 'per_tensor'
+    raw.dg_quantizer.rhs.calib_shared_axes = 'per_tensor'
+  call = lambda x: dg(x, w, MATMUL)
+  graphed = hip_graph.GraphedCall(call, mk(1))
+  _check_replays(graphed, call, mk)
+
+
 def test_static_argument_is_read_in_place(gpu):
   dt = 'bf16'
   x = U.to_dev(U.rand((64, 256), dt, 1), dt, gpu)
