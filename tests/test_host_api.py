@@ -226,3 +226,44 @@ def test_ceil_to_po2_matches_oracle_op_by_op():
   got = calibration.ceil_to_po2(allb)
   assert got.dtype == torch.bfloat16
   np.testing.assert_array_equal(got.float().numpy(), R.ceil_to_po2(allb.float().numpy(), 'bf16'))
+
+
+def test_standalone_entry_points_and_graph_wrapper_without_a_gpu():
+  """The reference's `aqt.jax.v2.pallas` names exist under the same path; nothing computes on the
+  CPU: tensors off the GPU are refused, recording a graph needs a GPU."""
+  import aqt_amd.v2.pallas as aqt_pl
+  from aqt_amd.v2 import aqt_tensor, hip_graph
+  for name in ('quant', 'dot_general', 'load_qtensor', 'pallas_call', 'DequantMode'):
+    assert hasattr(aqt_pl, name), name
+  assert aqt_pl.DequantMode is aqt.DequantMode
+  with pytest.raises(NotImplementedError, match='no Pallas'):
+    aqt_pl.pallas_call(lambda: None)
+  qt = aqt_tensor.QTensor(qvalue=torch.zeros(4, 4, dtype=torch.int8), scale=[torch.ones(4, 1)], scale_t=None,
+                          bias=[], dequant_dtype=torch.float32)
+  assert aqt_pl.load_qtensor(qt) is qt
+  with pytest.raises(Exception):  # no CPU path: the quantize kernel refuses a CPU tensor
+    aqt_pl.quant(torch.randn(8, 16), 8, (1,))
+  if not torch.cuda.is_available():
+    with pytest.raises(RuntimeError, match='needs a GPU'):
+      hip_graph.GraphedCall(lambda a: a, torch.zeros(4))
+
+
+def test_deep_copy_of_a_configuration_is_independent_and_equal():
+  """config.set_context copies the configuration on every call (config.py:66-90): the field-wise
+  copies of the quantizer, numerics and context classes must behave like copy.deepcopy."""
+  import copy
+  from aqt_amd.v2 import utils
+  cfg = config.fully_quantized(use_stochastic_rounding=True)
+  assert copy.deepcopy(cfg) == cfg  # (keys are numpy arrays, which dataclass equality cannot compare: none set yet)
+  cfg = config.set_context(cfg, utils.prng_key(3), train_step=7)
+  dup = copy.deepcopy(cfg)
+  for a, b in ((cfg.fwd, dup.fwd), (cfg.dlhs, dup.dlhs), (cfg.drhs, dup.drhs)):
+    for side in ('lhs', 'rhs'):
+      qa, qb = getattr(a.dg_quantizer, side), getattr(b.dg_quantizer, side)
+      assert qa is not qb and qa.numerics is not qb.numerics and qa.context is not qb.context
+      assert qa.calibration is qb.calibration  # the factory is shared, never changed in place
+      if qa.context.key is not None:
+        assert qa.context.key is not qb.context.key and (qa.context.key == qb.context.key).all()
+  dup.fwd.dg_quantizer.lhs.numerics.bits = 4
+  dup.fwd.dg_quantizer.lhs.context.train_step = 99
+  assert cfg.fwd.dg_quantizer.lhs.numerics.bits == 8 and cfg.fwd.dg_quantizer.lhs.context.train_step == 7
