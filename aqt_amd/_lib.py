@@ -65,7 +65,7 @@ class DecodePlan(ctypes.Structure):
       ('x_dtype', ctypes.c_int32), ('x_scale_dtype', ctypes.c_int32),
       ('w_scale_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
       ('quant_bound', ctypes.c_float), ('clip_bound', ctypes.c_float),
-      ('w_dtype', ctypes.c_int32),
+      ('w_dtype', ctypes.c_int32), ('tuning', ctypes.c_int32),
   ]
 
 

@@ -1,19 +1,14 @@
 // Serving-shape contraction: out[m, n] = dequant( quant(x)[m, :] . W[n, :] ) for m <= 64 rows of
-// activations against a pre-quantized int8 weight stored [n, k] (contraction axis contiguous).
+// activations against a pre-quantized int8 weight stored [n, k] (contraction axis contiguous),
+// or an int4 weight packed two values per byte.
 //
 // The weight is read exactly once and dominates the traffic, so the kernels are built around
 // streaming W from HBM with every lane fetching 16 contiguous bytes straight into the operand
 // registers of v_mfma_i32_16x16x64_i8 (lane -> row lane&15, bytes 16*(lane>>4).. of a 64-byte
-// k step: 16 rows x 64 B per wave instruction, whole 64-byte sectors).  The activations are
-// quantized first by the row kernel of aqtx_quantize (same arithmetic as training), then:
-//   K split : one workgroup per 16 weight rows, its 4 waves split K and meet in LDS; the
-//             quantized activations come from L2 (m <= 16, or a weight with few rows);
-//   whole K : one workgroup per 64 weight rows; two groups of 4 waves (16 rows per wave) take half
-//             of K each and meet in LDS; the activations are staged chunk by chunk in LDS and
-//             shared by the waves of a group, the weights are requested three chunks ahead
-//             (16 < m <= 64 and n >= 12288).  K is never split across workgroups: a partial-sum
-//             exchange inside one launch would need device-scope release/acquire, which
-//             flushes and invalidates the per-XCD L2s.
+// k step: 16 rows x 64 B per wave instruction, whole 64-byte sectors).
+//   m <= 2 : one kernel; every workgroup (16 weight rows) quantizes the activations itself.
+//   m >= 3 : a per-token quantize kernel, then a contraction kernel whose workgroups own a tile of
+//            weight rows and one K range; partial sums of the K ranges meet through int32 atomics.
 #include "common.h"
 
 namespace aqtx {
@@ -39,6 +34,19 @@ struct DecodeArgs {
   float* x_scale_out;     // [m]
   float quant_bound, clip_bound;
   int x_bf16;
+  // K split across workgroups (decode_tile_kernel)
+  int k_slice;            // K range of one workgroup (blockIdx.y), a multiple of 4 wave-wide steps
+  int splits;             // gridDim.y
+  int* sums;              // [n tiles][MB*NB*4][64] int32 exchange words, zero on entry (splits > 1)
+  int count_shift;        // bit position of the arrival count inside an exchange word
+  // Quantized activations in MFMA fragment order (written by decode_quant_kernel, read by
+  // decode_tile_kernel): one 1 KiB block per (K step, 16-token block, half h), holding for lane
+  // (r = token in the block, c = k quarter) its 16 operand bytes at c*256 + r*16, so that a
+  // wave's fragment load is one contiguous KiB.  A K step is 64 k (int8 weights, one half) or
+  // 128 k (packed int4 weights: the lane's 32 k are split in two halves of 16).
+  int8_t* xq_frag;
+  int mb_total;           // 16-token blocks
+  int frag_halves;        // 1 | 2
 };
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
@@ -61,70 +69,6 @@ __device__ __forceinline__ void store_out(const DecodeArgs& d, int mm, int nn, i
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kBufferRsrcWord3);
-}
-
-// ---- K split inside the workgroup ---------------------------------------------------------------
-// One workgroup per 16 weight rows; its 4 waves take a quarter of K each and meet in LDS.  The
-// quantized activations are read straight from L2 as MFMA operands (MB blocks of 16 rows), so
-// the L2 traffic is (1 + MB) times the weight bytes: the shape for m <= 16, and for larger m
-// when the weight has too few rows to fill the chip with whole-K waves.
-template <int MB, int U>  // U: 64-byte k steps in flight per wave
-__global__ __launch_bounds__(256) void decode_ksplit_kernel(const DecodeArgs d) {
-  __shared__ int red[4][MB * 16][16];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, c = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);  // clamped; such columns are never stored
-
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
-  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
-  const int kq = ((d.k + 3) / 4 + 63) / 64 * 64;  // K range of one wave, whole 64-byte steps
-  const int k_lo = wave * kq;
-  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
-  const int wbase = nrow * d.k + c * 16;
-  int xbase[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) xbase[mb] = (mb * 16 + r) < d.m ? (mb * 16 + r) * d.k + c * 16 : kOob;
-
-  v4i acc[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) acc[mb] = v4i{0, 0, 0, 0};
-  for (int kk = k_lo; kk < k_hi; kk += 64 * U) {
-    v4i wf[U], xf[U][MB];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int ko = kk + u * 64;
-      const bool ok = ko + c * 16 < k_hi;
-      wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? wbase + ko : kOob, 0, 0);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        xf[u][mb] = __builtin_amdgcn_raw_buffer_load_b128(rx, (ok && xbase[mb] != kOob) ? xbase[mb] + ko : kOob, 0, 0);
-    }
-    // Keep every load of the batch in flight before the first MFMA waits for one: left alone,
-    // the scheduler interleaves them to save registers and the wave stalls on memory latency.
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][mb], wf[u], acc[mb], 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  // lane holds C[m = mb*16 + 4c + e][n = r]
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) red[wave][mb * 16 + 4 * c + e][r] = acc[mb][e];
-  __syncthreads();
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int mm = mb * 16 + (tid >> 4), nn = n0 + (tid & 15);
-    if (mm < d.m && nn < d.n) {
-      const int s = red[0][mm][tid & 15] + red[1][mm][tid & 15] + red[2][mm][tid & 15] + red[3][mm][tid & 15];
-      store_out(d, mm, nn, s);
-    }
-  }
 }
 
 // A word of eight packed int4 (low nibble = even k) -> two words of int8 holding 16 * value.
@@ -293,233 +237,297 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   }
 }
 
-// ---- packed int4 weights -----------------------------------------------------------------------
-// Two int4 per byte, low nibble = even k.  A lane's 16-byte load holds 32 consecutive k of one
-// weight row, the B operands of two MFMAs; the matching 32 activation bytes are the two A
-// operands.  A nibble is moved to the top of its byte, which makes it 16 * w as a signed int8;
-// the factor leaves the accumulator as an exact right shift by 4.  Same workgroup shape as the
-// K-split kernel (weights stream from HBM once; half the bytes of the int8 form).
+// ---- 3 <= m <= 64: K split across workgroups -----------------------------------------------------
+// Phase 1, one workgroup per token: per-token abs-max, scale and int8 values (the arithmetic of the
+// row kernel of aqtx_quantize), the row kept in registers between the two passes (PPT 16-value
+// pieces per thread; PPT = 0 reads the row twice, any length).  The int8 values are written in
+// MFMA fragment order for the contraction kernel (and in plain [m][k] order when the caller asks
+// for them); token rows that only pad the last 16-token block are written as zeros.  Every
+// workgroup of the launch also clears its share of the exchange words the contraction kernel
+// accumulates into, so that no separate clearing launch is needed.
+template <typename TIn, int PPT>
+__global__ __launch_bounds__(256) void decode_quant_kernel(const DecodeArgs d, uint4* clear, int clear_vec16) {
+  __shared__ float smax[4];
+  constexpr bool XBF = sizeof(TIn) == 2;
+  constexpr int WPP = XBF ? 8 : 16;  // 32-bit words of one 16-value input piece
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = blockIdx.x * 256 + tid; i < clear_vec16; i += gridDim.x * 256) clear[i] = make_uint4(0u, 0u, 0u, 0u);
+  const int row = blockIdx.x;
+  if (row >= d.mb_total * 16) return;  // uniform across the workgroup
+  const int pieces = d.k / 16;
+  // piece p of this row inside the fragment-ordered copy
+  auto frag_ptr = [&](int p) {
+    const int step = d.frag_halves == 2 ? p >> 3 : p >> 2;
+    const int c = d.frag_halves == 2 ? (p & 7) >> 1 : p & 3;
+    const int h = d.frag_halves == 2 ? p & 1 : 0;
+    return d.xq_frag + ((int64_t)(step * d.mb_total + (row >> 4)) * d.frag_halves + h) * 1024 + c * 256 + (row & 15) * 16;
+  };
+  if (row >= d.m) {
+    for (int p = tid; p < pieces; p += 256) *reinterpret_cast<uint4*>(frag_ptr(p)) = make_uint4(0u, 0u, 0u, 0u);
+    return;
+  }
+  const TIn* xr = reinterpret_cast<const TIn*>(d.x) + (int64_t)row * d.k;
+  constexpr int NP = PPT > 0 ? PPT : 1;
+  uint32_t raw[NP][WPP];
+  auto load_piece = [&](int p, uint32_t* dst) {
+#pragma unroll
+    for (int q = 0; q < WPP / 4; ++q) {
+      const uint4 t = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(xr) + ((int64_t)p * WPP + 4 * q) * 4);
+      dst[4 * q + 0] = t.x; dst[4 * q + 1] = t.y; dst[4 * q + 2] = t.z; dst[4 * q + 3] = t.w;
+    }
+  };
+  auto value = [&](const uint32_t* w, int e) -> float {
+    if constexpr (XBF) return __uint_as_float((e & 1) ? (w[e >> 1] & 0xFFFF0000u) : (w[e >> 1] << 16));
+    else return __uint_as_float(w[e]);
+  };
+  float amax = 0.0f;
+  if constexpr (PPT > 0) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int p = tid + 256 * j;
+      if (p < pieces) {
+        load_piece(p, raw[j]);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(value(raw[j], e)));
+      }
+    }
+  } else {
+    for (int p = tid; p < pieces; p += 256) {
+      load_piece(p, raw[0]);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(value(raw[0], e)));
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  if (lane == 0) smax[wave] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+  if (amax == 0.0f) amax = 1.0f;
+  float sc = rnd(amax / d.quant_bound, d.x_bf16);
+  sc = rnd(sc, d.xs_bf16);
+  float inv = rnd(1.0f / sc, d.xs_bf16);
+  if (isinf(inv)) inv = 1.0f;
+  if (tid == 0) d.x_scale_out[row] = sc;
+  const int tbf = d.x_bf16 & d.xs_bf16;
+  auto quant_piece = [&](const uint32_t* w, int p) {
+    uint32_t q[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      float t = rnd(value(w, e) * inv, tbf);
+      t = fminf(fmaxf(t, -d.clip_bound), d.clip_bound);
+      q[e >> 2] |= ((uint32_t)((int)rintf(t)) & 0xFFu) << (8 * (e & 3));
+    }
+    const uint4 v = make_uint4(q[0], q[1], q[2], q[3]);
+    *reinterpret_cast<uint4*>(frag_ptr(p)) = v;
+    if (d.xq_out != nullptr) *reinterpret_cast<uint4*>(d.xq_out + (int64_t)row * d.k + (int64_t)p * 16) = v;
+  };
+  if constexpr (PPT > 0) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int p = tid + 256 * j;
+      if (p < pieces) quant_piece(raw[j], p);
+    }
+  } else {
+    for (int p = tid; p < pieces; p += 256) {
+      load_piece(p, raw[0]);
+      quant_piece(raw[0], p);
+    }
+  }
+}
 
-// NB: 16-row weight blocks per wave; every activation fragment a wave loads is used NB times,
-// so the L2 traffic for the activations is MB / NB times the int8-equivalent weight bytes.
-template <int MB, int NB, int U>  // U: 128-k steps (16 packed bytes per lane and block) in flight per wave
-__global__ __launch_bounds__(256) void decode_ksplit_i4_kernel(const DecodeArgs d) {
-  __shared__ int red[4][NB][MB * 16][16];
+// Phase 2.  A workgroup owns 16*NB weight rows, all m <= 16*MB tokens and one K range
+// (blockIdx.y); its four waves take a quarter of that range each.  A wave streams its weight
+// fragments from HBM and its activation fragments (fragment order, contiguous KiB) from L2
+// straight into MFMA operand registers: every weight fragment meets MB activation fragments and
+// every activation fragment NB weight fragments, so the L2 traffic for the activations is
+// MB / NB times the weight bytes.  D k-steps are in flight per wave at any time (a ring of
+// register sets: the loads of step i + D are issued as soon as step i has been multiplied).
+// The weights are the MFMA's row operand, so a lane ends up with four consecutive output
+// columns of one token.  The four waves' accumulators meet in LDS.
+//
+// With one K range per weight tile the workgroup dequantizes and stores.  With several, every
+// thread adds its sums to the tile's exchange words with one int32 atomic each (integer addition
+// is exact in any order).  The same addition counts the arrival: the addend is
+// (1 << count_shift) + sum, and |sum of any subset of the K ranges| < 2^(count_shift - 1), so the
+// value the atomic returns says how many K ranges had been added before.  The thread that finds
+// every other range already there holds the total (returned value + its own) and dequantizes
+// that element.  Device-scope atomic read-modify-writes are carried out at the memory side of the
+// per-XCD L2s, so the exchange needs no fence, no second round trip and no waiting loop.
+// PACKED: int4 weights two per byte; a lane's 16 bytes are 32 k = two MFMA steps.
+template <int MB, int NB, int D, bool PACKED>
+__global__ __launch_bounds__(256, (D * (NB + MB * (PACKED ? 2 : 1)) * 4 + MB * NB * 4 + 48 > 256) ? 1 : 2)
+void decode_tile_kernel(const DecodeArgs d) {
+  constexpr int T = MB * NB;
+  static_assert(T % 4 == 0, "a thread owns whole 16x16 tiles after the reduction");
+  __shared__ v4i red[4][T][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
+  constexpr int KS = PACKED ? 128 : 64;  // k covered by one wave-wide weight load
+  constexpr int KL = KS / 4;             // k covered by one lane's 16 bytes
+  constexpr int XP = PACKED ? 2 : 1;     // activation fragments per weight fragment
   const int n0 = blockIdx.x * (16 * NB);
-  const int kb = d.k / 2;  // bytes of one packed weight row
+  const int kb = PACKED ? d.k / 2 : d.k;  // bytes of one weight row
+  const int s_lo = blockIdx.y * d.k_slice;
+  const int s_hi = (s_lo + d.k_slice) < d.k ? (s_lo + d.k_slice) : d.k;
+  const int kq = d.k_slice / 4;
+  const int k_lo = s_lo + wave * kq;
+  const int k_hi = (k_lo + kq) < s_hi ? (k_lo + kq) : s_hi;
 
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * kb);
-  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
-  const int kq = ((d.k + 3) / 4 + 127) / 128 * 128;  // K range of one wave, whole 128-k steps
-  const int k_lo = wave * kq;
-  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
-  int wbase[NB], xbase[MB];
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq_frag, (int64_t)((d.k + KS - 1) / KS) * d.mb_total * XP * 1024);
+  int wbase[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int row = n0 + nb * 16 + r;
     wbase[nb] = (row < d.n ? row : d.n - 1) * kb + c * 16;  // clamped; such columns are never stored
   }
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) xbase[mb] = (mb * 16 + r) < d.m ? (mb * 16 + r) * d.k + c * 32 : kOob;
 
   v4i acc[MB][NB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = v4i{0, 0, 0, 0};
-  for (int kk = k_lo; kk < k_hi; kk += 128 * U) {
-    v4i wf[U][NB], xf[U][MB][2];
+
+  // The scales of the outputs this thread will dequantize at the end (tiles t = wave + 4*j: weight
+  // block t % NB is the same for all of them), requested now so that they are long there by then.
+  float ws[4], xs[T / 4];
+  {
+    const int nn = n0 + (wave % NB) * 16 + 4 * c;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int ko = kk + u * 128;
-      const bool ok = ko + c * 32 < k_hi;  // k is a multiple of 32: a lane's 32 k are all in or all out
+    for (int e = 0; e < 4; ++e) ws[e] = d.w_scale[(nn + e) < d.n ? (nn + e) : (d.n - 1)];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        wf[u][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? wbase[nb] + ko / 2 : kOob, 0, 0);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const int xo = (ok && xbase[mb] != kOob) ? xbase[mb] + ko : kOob;
-        xf[u][mb][0] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
-        xf[u][mb][1] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo == kOob ? kOob : xo + 16, 0, 0);
-      }
+    for (int j = 0; j < T / 4; ++j) {
+      const int mm = ((wave + 4 * j) / NB) * 16 + r;
+      xs[j] = d.x_scale[mm < d.m ? mm : (d.m - 1)];
     }
-    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  v4i wf[D][NB], xf[D][MB][XP];
+  // Steps past the end of the wave's range, lanes past the end of K and token blocks past m read
+  // zeros: their offsets get the out-of-range bits ORed in (no memory access; no branch, which
+  // would make the compiler drain the loads in flight).
+  unsigned xdead[MB];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+  for (int mb = 0; mb < MB; ++mb) xdead[mb] = mb < d.mb_total ? 0u : (unsigned)kOob;
+  auto issue = [&](int slot, int ko) {
+    const unsigned dead = (ko + c * KL < k_hi) ? 0u : (unsigned)kOob;  // a lane's KL values are all inside or all outside
+    const unsigned wk = (unsigned)(PACKED ? ko / 2 : ko);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
+    for (int nb = 0; nb < NB; ++nb)
+      wf[slot][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)(((unsigned)wbase[nb] + wk) | dead), 0, 0);
+    const unsigned xstep = (unsigned)(ko / KS) * (unsigned)d.mb_total;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int h = 0; h < XP; ++h)
+        xf[slot][mb][h] = __builtin_amdgcn_raw_buffer_load_b128(
+            rx, (int)(((((xstep + mb) * XP + h) << 10) + (unsigned)lane * 16u) | dead | xdead[mb]), 0, 0);
+  };
+  auto multiply = [&](int slot) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      if constexpr (PACKED) {
         int t[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[u][nb][j], t[2 * j], t[2 * j + 1]);
+        for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[slot][nb][j], t[2 * j], t[2 * j + 1]);
         const v4i b0 = v4i{t[0], t[1], t[2], t[3]}, b1 = v4i{t[4], t[5], t[6], t[7]};
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][mb][0], b0, acc[mb][nb], 0, 0, 0);
-          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][mb][1], b1, acc[mb][nb], 0, 0, 0);
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, xf[slot][mb][0], acc[mb][nb], 0, 0, 0);
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, xf[slot][mb][XP - 1], acc[mb][nb], 0, 0, 0);
         }
+      } else {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[slot][nb], xf[slot][mb][0], acc[mb][nb], 0, 0, 0);
       }
-    __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // Workgroups walk the steps of their K range in rotated order (integer sums do not care):
+  // otherwise every workgroup of the launch asks the same L2 channel for the same activation
+  // bytes at the same time.  Workgroup ids are dealt round-robin to the 8 XCDs, so id / 8
+  // spreads the workgroups that share an L2 evenly over the steps.
+  const int nsteps = kq / KS;
+  const int rot = (int)((blockIdx.x / 8 + blockIdx.y) % (unsigned)nsteps);
+  auto step_k = [&](int i) {
+    int j = i + rot;
+    j = j >= nsteps ? j - nsteps : j;
+    return i < nsteps ? k_lo + j * KS : 0x3FFFFF00;
+  };
+#pragma unroll
+  for (int s = 0; s < D; ++s) issue(s, step_k(s));
+  __builtin_amdgcn_sched_barrier(0);
+  for (int i = 0; i < nsteps; i += D) {
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+      multiply(s);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(s, step_k(i + D + s));
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
-  // lane holds C[m = mb*16 + 4c + e][n = n0 + nb*16 + r]
+  // lane holds C[n = n0 + nb*16 + 4c + e][m = mb*16 + r] in acc[mb][nb][e]
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) red[wave][nb][mb * 16 + 4 * c + e][r] = acc[mb][nb][e];
+    for (int nb = 0; nb < NB; ++nb) red[wave][mb * NB + nb][lane] = acc[mb][nb];
   __syncthreads();
+  // thread -> the lane's four words of tiles t = wave + 4*j, j = 0..T/4-1
+  int* tile_sums = d.sums + (int64_t)blockIdx.x * (T * 4 * 64);
+  const int one = 1 << d.count_shift, half = one >> 1;
+  const bool wide_ok = (d.n % 4) == 0;  // 4 consecutive outputs of a row are then 8 / 16-byte aligned
+  const int p1 = d.out_bf16 & d.xs_bf16;
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
+  for (int j = 0; j < T / 4; ++j) {
+    const int t = wave + 4 * j;
+    v4i total = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
+    bool last[4] = {true, true, true, true};
+    if (d.splits > 1) {
+      int before[4];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const int mm = mb * 16 + (tid >> 4), nn = n0 + nb * 16 + (tid & 15);
-      if (mm < d.m && nn < d.n) {
-        const int s = red[0][nb][mm][tid & 15] + red[1][nb][mm][tid & 15] + red[2][nb][mm][tid & 15] +
-                      red[3][nb][mm][tid & 15];
-        store_out(d, mm, nn, s);
+      for (int e = 0; e < 4; ++e)
+        before[e] = __hip_atomic_fetch_add(tile_sums + (t * 4 + e) * 64 + lane, one + total[e], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int arrived = (before[e] + half) >> d.count_shift;  // K ranges added before this one
+        total[e] += before[e] - arrived * one;
+        last[e] = arrived == d.splits - 1;
       }
     }
-}
-
-// ---- 16 < m <= 64 ------------------------------------------------------------------------------
-constexpr int kChunk = 256;  // bytes of K per pipeline step
-constexpr int kAhead = 3;    // weight chunks requested ahead of the one being multiplied
-
-// MB: 16-row blocks of activations, 2 (m <= 32) or 4 (m <= 64).  NWV waves own 16 weight rows
-// each; KW groups of NWV waves take one K range each (their partial sums meet in LDS at the end),
-// which doubles the waves per SIMD for the same weight rows.  K is not split across workgroups.
-template <int MB, int NWV, int KW>
-__global__ __launch_bounds__(NWV * KW * 64) void decode_block_kernel(const DecodeArgs d) {
-  // Activations of one K chunk per K range, [MB*16 rows][256 B]; the 16-byte piece j of row i sits
-  // at piece j ^ (i & 15), so the 16 lanes of a fragment read (16 rows, one piece) hit 64 banks.
-  __shared__ __attribute__((aligned(16))) uint8_t xbuf[KW][2][MB * 16 * kChunk];
-  __shared__ int red[KW > 1 ? (KW - 1) * NWV * MB * 256 : 1];
-  constexpr int NT = NWV * 64;           // threads of one K range
-  constexpr int XP = MB * 16 * 16 / NT;  // 16-byte pieces of a chunk staged per thread
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kw = wave / NWV, wn = wave % NWV;
-  const int tid = threadIdx.x - kw * NT;  // thread index inside the K range
-  const int r = lane & 15, c = lane >> 4;
-  const int n0 = blockIdx.x * (NWV * 16) + wn * 16;
-  const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);  // clamped; such columns are never stored
-  const int k_len = ((d.k + KW - 1) / KW + kChunk - 1) / kChunk * kChunk;  // K range, whole chunks
-  const int k_lo = kw * k_len;
-  const int k_hi = (k_lo + k_len) < d.k ? (k_lo + k_len) : d.k;
-  const int nchunks = k_len / kChunk;  // the same for every K range: they share the barriers
-
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * d.k);
-  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq, (int64_t)d.m * d.k);
-  const int wbase = nrow * d.k + c * 16;
-  // staging of the activations: thread -> (row tid>>4 of a pass of NT/16 rows, piece tid&15)
-  const int xs_row = tid >> 4, xs_piece = tid & 15;
-
-  v4i wreg[kAhead + 1][4], xr[2][XP];  // xr[p]: activations of a chunk of parity p on their way to LDS
-  // Workgroups walk the chunks of their K range in rotated order (integer sums do not care):
-  // otherwise every workgroup of the launch asks the same few L2 channels for the same
-  // activation chunk at the same time.  Step numbers past the range read zeros.
-  const int rot = blockIdx.x % nchunks;
-  auto chunk_start = [&](int step_no) {
-    int j = step_no + rot;
-    j = j >= nchunks ? j - nchunks : j;
-    return step_no < nchunks ? k_lo + j * kChunk : 0x3FFFFF00;
-  };
-  auto load_w = [&](v4i* dst, int step_no) {
-    const int kc = chunk_start(step_no);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int ko = kc + ks * 64;
-      dst[ks] = __builtin_amdgcn_raw_buffer_load_b128(rw, (ko + c * 16 < k_hi) ? wbase + ko : kOob, 0, 0);
-    }
-  };
-  auto load_x = [&](v4i* dst, int step_no) {
-    const int kc = chunk_start(step_no);
-#pragma unroll
-    for (int p = 0; p < XP; ++p) {
-      const int row = p * (NT / 16) + xs_row;
-      const int ko = kc + xs_piece * 16;
-      dst[p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (row < d.m && ko < k_hi) ? row * d.k + ko : kOob, 0, 0);
-    }
-  };
-  auto store_x = [&](uint8_t* buf, const v4i* src) {
-#pragma unroll
-    for (int p = 0; p < XP; ++p) {
-      const int row = p * (NT / 16) + xs_row;
-      *reinterpret_cast<v4i*>(buf + row * kChunk + ((xs_piece ^ (row & 15)) * 16)) = src[p];
-    }
-  };
-
-  v4i acc[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) acc[mb] = v4i{0, 0, 0, 0};
-
-  load_x(xr[0], 0);
-#pragma unroll
-  for (int j = 0; j < kAhead; ++j) load_w(wreg[j], j);
-  store_x(xbuf[kw][0], xr[0]);
-  load_x(xr[1], 1);
-  load_x(xr[0], 2);
-  __syncthreads();
-  // One pipeline step: publish the activations of chunk i+1 (requested two steps ago), request
-  // those of chunk i+3 and the weights of chunk i+kAhead, multiply chunk i.  Every load has two
-  // or more steps to arrive, so a step never waits a full memory latency.  The register sets
-  // rotate roles through the unrolled steps (no register copies that would wait for loads).
-  auto step = [&](const v4i* wc, v4i* wfar, v4i* xnext, int i) {
-    store_x(xbuf[kw][(i + 1) & 1], xnext);
-    load_x(xnext, i + 3);
-    load_w(wfar, i + kAhead);
-    const uint8_t* buf = xbuf[kw][i & 1];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const v4i xf = *reinterpret_cast<const v4i*>(buf + (mb * 16 + r) * kChunk + (((ks * 4 + c) ^ r) * 16));
-        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf, wc[ks], acc[mb], 0, 0, 0);
-      }
-    // LDS traffic only: a __syncthreads() would also wait for the global loads in flight.
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-  };
-  static_assert(kAhead == 3, "the unrolled rotation below is written for 4 register sets");
-  // Always four steps per trip: steps past the last chunk read zeros everywhere (loads out of
-  // range) and add nothing.  A branch-free body lets the compiler count the loads in flight
-  // exactly instead of draining them at every loop entry.
-  for (int i = 0; i < nchunks; i += 4) {
-    step(wreg[0], wreg[3], xr[1], i);
-    step(wreg[1], wreg[0], xr[0], i + 1);
-    step(wreg[2], wreg[1], xr[1], i + 2);
-    step(wreg[3], wreg[2], xr[0], i + 3);
-  }
-
-  // lane holds C[m = mb*16 + 4c + e][n = n0 + r]; K ranges 1.. hand their sums to range 0
-  if constexpr (KW > 1) {
-    if (kw > 0) {
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) red[(((kw - 1) * NWV + wn) * MB + mb) * 256 + e * 64 + lane] = acc[mb][e];
-    }
-    __syncthreads();
-    if (kw > 0) return;
-#pragma unroll
-    for (int j = 1; j < KW; ++j)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[mb][e] += red[(((j - 1) * NWV + wn) * MB + mb) * 256 + e * 64 + lane];
-  }
-  const int nn = n0 + r;
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
+    const int mm = (t / NB) * 16 + r, nn = n0 + (t % NB) * 16 + 4 * c;
+    // QTensor.dequant: cast the accumulator, multiply by the lhs scale, then the rhs scale, each
+    // product in the promoted dtype of its operands, final cast.
+    float f[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int mm = mb * 16 + 4 * c + e;
-      if (mm < d.m && nn < d.n) store_out(d, mm, nn, acc[mb][e]);
+      float v = rnd((float)(total[e] >> d.acc_shift), d.out_bf16);  // exact: a multiple of 16 when shifted
+      v = rnd(v * xs[j], p1);
+      v = rnd(v * ws[e], p1 & d.ws_bf16);
+      f[e] = rnd(v, d.out_bf16);
     }
+    const int64_t o = (int64_t)mm * d.n + nn;
+    const bool inside = mm < d.m && nn < d.n;
+    if (inside && wide_ok && last[0] && last[1] && last[2] && last[3]) {
+      if (d.out_bf16) {
+        uint2 v;
+        v.x = (uint32_t)bf16_bits(f[0]) | ((uint32_t)bf16_bits(f[1]) << 16);
+        v.y = (uint32_t)bf16_bits(f[2]) | ((uint32_t)bf16_bits(f[3]) << 16);
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(d.out) + o) = v;
+      } else {
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(d.out) + o) = make_float4(f[0], f[1], f[2], f[3]);
+      }
+    } else if (inside) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (last[e] && nn + e < d.n) {
+          if (d.out_bf16) reinterpret_cast<uint16_t*>(d.out)[o + e] = bf16_bits(f[e]);
+          else reinterpret_cast<float*>(d.out)[o + e] = f[e];
+        }
+    }
+  }
 }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -534,7 +542,7 @@ int validate_decode(const aqtx_decode_plan* p) {
   const int64_t kmul = p->w_dtype == AQTX_I4P ? 32 : 16;
   AQTX_REQUIRE(p->k > 0 && p->k % kmul == 0, "aqtx_decode_i8: k = %lld must be a positive multiple of %lld",
                (long long)p->k, (long long)kmul);
-  AQTX_REQUIRE(p->n * p->k < (1ll << 31) && p->m * p->n < (1ll << 31),
+  AQTX_REQUIRE(p->n * p->k < (1ll << 31) - 64 && p->m * p->n < (1ll << 31),
                "aqtx_decode_i8: weight larger than 2 GiB is not addressable with 32-bit offsets");
   AQTX_REQUIRE(is_float_dtype(p->x_dtype) && is_float_dtype(p->x_scale_dtype) &&
                    is_float_dtype(p->w_scale_dtype) && is_float_dtype(p->out_dtype),
@@ -548,9 +556,105 @@ int validate_decode(const aqtx_decode_plan* p) {
 
 using namespace aqtx;
 
+// ---- launch shape of the split-K path ------------------------------------------------------------
+namespace {
+
+struct TileShape {
+  int mb, nb, depth;  // template parameters of decode_tile_kernel
+  int ntiles;         // weight tiles of 16*nb rows
+  int splits;         // K ranges (workgroups per weight tile)
+  int k_slice;        // K per range
+  int count_shift;    // arrival count position in an exchange word
+  size_t sums_bytes;  // exchange words actually used (0 when splits == 1)
+};
+
+// plan->tuning, all fields 0 = the library's choice:
+//   bits 0-7 K ranges per weight tile, bits 8-11 nb (2 | 4), bits 12-15 K steps in flight per
+//   wave (2 | 4), bits 16-19 path (1 = never fuse the activation quantisation into the
+//   contraction kernel)
+TileShape choose_tile_shape(const aqtx_decode_plan* p) {
+  TileShape t{};
+  const int tune = p->tuning;
+  const bool packed = p->w_dtype == AQTX_I4P;
+  const int ks = packed ? 128 : 64;
+  t.mb = p->m <= 16 ? 1 : p->m <= 32 ? 2 : 4;
+  // About one workgroup per CU (256): weight tiles of 64 rows when the weight has enough rows for
+  // that, else of 32 rows; whatever is still missing comes from splitting K, which costs
+  // exchange traffic in proportion to m * n * K ranges.
+  t.nb = ((tune >> 8) & 15) ? ((tune >> 8) & 15) : ((p->n + 63) / 64 >= 192 ? 4 : 2);
+  if ((t.nb != 2 && t.nb != 4) || t.mb == 1) t.nb = 4;  // mb * nb must be a multiple of 4
+  t.ntiles = (int)((p->n + 16 * t.nb - 1) / (16 * t.nb));
+  // An exchange word holds count * 2^shift + sum with |sum| <= k * 127 * 128 < 2^(shift - 1).
+  int magnitude_bits = 1;
+  while (((int64_t)1 << magnitude_bits) <= p->k * (int64_t)(127 * 128)) ++magnitude_bits;
+  t.count_shift = magnitude_bits + 1;
+  const int max_by_count = t.count_shift >= 31 ? 1 : (1 << (31 - t.count_shift)) - 1;
+  const int max_by_k = (int)((p->k + 4 * ks - 1) / (4 * ks));  // at least one step per wave
+  int splits = tune & 255;
+  if (splits == 0) splits = (256 + t.ntiles / 2) / t.ntiles;
+  if (splits > max_by_k) splits = max_by_k;
+  if (splits > max_by_count) splits = max_by_count;
+  if (splits < 1) splits = 1;
+  int k_slice = (int)((p->k + splits - 1) / splits);
+  k_slice = (k_slice + 4 * ks - 1) / (4 * ks) * (4 * ks);
+  t.k_slice = k_slice;
+  t.splits = (int)((p->k + k_slice - 1) / k_slice);
+  const int steps = k_slice / (4 * ks);
+  const int loads_per_step = t.nb + t.mb * (packed ? 2 : 1);
+  t.depth = ((tune >> 12) & 15) ? ((tune >> 12) & 15) : ((steps >= 4 && t.mb == 1) ? 4 : 2);
+  if (t.depth != 2 && t.depth != 4) t.depth = 4;
+  while (t.depth > 2 && t.depth * loads_per_step > 64) t.depth /= 2;  // 256 registers of operands in flight
+  if (t.splits > 1) t.sums_bytes = (size_t)t.ntiles * t.mb * t.nb * 1024;
+  return t;
+}
+
+// Upper bound of the exchange words over every launch shape: 64 token rows x (n rounded up to a
+// whole tile) int32 words.
+size_t exchange_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)(p->n + 64) * 4; }
+// The quantized activations in fragment order: 64 token rows x k rounded up to a whole K step.
+size_t fragment_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)((p->k + 127) / 128 * 128); }
+
+template <bool PACKED>
+int launch_tile(const TileShape& t, const DecodeArgs& d, hipStream_t st) {
+  const dim3 grid((unsigned)t.ntiles, (unsigned)t.splits);
+#define AQTX_TILE(MB, NB, D) decode_tile_kernel<MB, NB, D, PACKED><<<grid, 256, 0, st>>>(d)
+#define AQTX_TILE_D(MB, NB)                         \
+  do {                                              \
+    if (t.depth == 2) AQTX_TILE(MB, NB, 2);         \
+    else AQTX_TILE(MB, NB, 4);                      \
+  } while (0)
+#define AQTX_TILE_N(MB) do { if (t.nb == 2) AQTX_TILE_D(MB, 2); else AQTX_TILE_D(MB, 4); } while (0)
+  if (t.mb == 1) AQTX_TILE_D(1, 4);
+  else if (t.mb == 2) AQTX_TILE_N(2);
+  else AQTX_TILE_N(4);
+#undef AQTX_TILE_N
+#undef AQTX_TILE_D
+#undef AQTX_TILE
+  AQTX_HIP_CHECK_LAUNCH("decode_tile_kernel");
+  return 0;
+}
+
+template <typename TIn>
+int launch_decode_quant(const DecodeArgs& d, uint4* clear, int clear_vec16, hipStream_t st) {
+  int clear_blocks = (clear_vec16 + 1023) / 1024;
+  if (clear_blocks > 256) clear_blocks = 256;
+  const int rows = d.mb_total * 16;
+  const unsigned grid = (unsigned)(rows > clear_blocks ? rows : clear_blocks);
+  const int pieces = d.k / 16;
+  if (pieces <= 256) decode_quant_kernel<TIn, 1><<<grid, 256, 0, st>>>(d, clear, clear_vec16);
+  else if (pieces <= 512) decode_quant_kernel<TIn, 2><<<grid, 256, 0, st>>>(d, clear, clear_vec16);
+  else if (pieces <= 1024) decode_quant_kernel<TIn, 4><<<grid, 256, 0, st>>>(d, clear, clear_vec16);
+  else decode_quant_kernel<TIn, 0><<<grid, 256, 0, st>>>(d, clear, clear_vec16);
+  AQTX_HIP_CHECK_LAUNCH("decode_quant_kernel");
+  return 0;
+}
+
+}  // namespace
+
 extern "C" size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* p) {
   if (p == nullptr || p->m < 0 || p->n < 0 || p->k < 0 || p->m > 64) return 0;
-  return align_up((size_t)(p->m * p->k), 256);  // the quantized activations when the caller keeps none
+  // the partial-sum exchange first, then the quantized activations when the caller keeps none
+  return exchange_bytes_bound(p) + fragment_bytes_bound(p);
 }
 
 extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const void* w,
@@ -561,111 +665,70 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
   if (p->m == 0 || p->n == 0) return 0;
   AQTX_REQUIRE(x != nullptr && w != nullptr && w_scale != nullptr && x_scale != nullptr && out != nullptr,
                "aqtx_decode_i8: NULL buffer");
-  const size_t need = xq != nullptr ? 0 : aqtx_decode_workspace_bytes(p);
-  AQTX_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need),
-               "aqtx_decode_i8: workspace too small (%zu < %zu)", workspace_bytes, need);
-  AQTX_REQUIRE(((uintptr_t)w % 16) == 0 && (need == 0 || ((uintptr_t)workspace % 16) == 0) &&
-                   (xq == nullptr || ((uintptr_t)xq % 16) == 0),
-               "aqtx_decode_i8: w, xq and the workspace must be 16-byte aligned");
-  int8_t* xq_buf = reinterpret_cast<int8_t*>(xq != nullptr ? xq : workspace);
+  AQTX_REQUIRE(((uintptr_t)w % 16) == 0 && ((uintptr_t)x % 16) == 0 && (xq == nullptr || ((uintptr_t)xq % 16) == 0),
+               "aqtx_decode_i8: x, w and xq must be 16-byte aligned");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const bool xbf = p->x_dtype == AQTX_BF16;
+  const bool pk = p->w_dtype == AQTX_I4P;
 
-  // 0. a handful of tokens: one kernel quantizes and contracts (AQTX_DECODE_FUSED=0 turns it off)
-  {
-    const bool xbf = p->x_dtype == AQTX_BF16;
-    const int ppt = p->k <= 4096 ? 1 : 2;
-    // Every workgroup repeats the quantisation, so its cost grows with the rows while the launch
-    // it saves does not: measured at k = 4096, one row gains 2.5 us per call, two rows 1 us,
-    // three rows lose.
-    const int64_t max_rows = 2;
-    const char* fused_env = getenv("AQTX_DECODE_FUSED");
-    const bool fused_off = fused_env != nullptr && fused_env[0] == '0';
-    if (!fused_off && p->k <= 8192 && p->m <= max_rows && ((uintptr_t)x % 16) == 0) {
-      const bool pk = p->w_dtype == AQTX_I4P;
-      DecodeArgs d{};
-      d.w = reinterpret_cast<const int8_t*>(w);
-      d.w_scale = w_scale; d.out = out;
-      d.m = (int)p->m; d.n = (int)p->n; d.k = (int)p->k;
-      d.out_bf16 = p->out_dtype == AQTX_BF16;
-      d.xs_bf16 = p->x_scale_dtype == AQTX_BF16;
-      d.ws_bf16 = p->w_scale_dtype == AQTX_BF16;
-      d.x = x; d.xq_out = reinterpret_cast<int8_t*>(xq); d.x_scale_out = x_scale;
-      d.quant_bound = p->quant_bound; d.clip_bound = p->clip_bound; d.x_bf16 = xbf;
-      const unsigned grid = (unsigned)((p->n + 15) / 16);
-      const int rows = (int)p->m;
-      const size_t lds = (size_t)rows * (size_t)((p->k + 255) / 256 * 256);
-      d.acc_shift = pk ? 4 : 0;
-#define AQTX_FUSED(T, R, P)                                                   \
-  if (pk) decode_fused_kernel<T, R, P, 8, true><<<grid, 256, lds, st>>>(d);  \
-  else decode_fused_kernel<T, R, P, 16, false><<<grid, 256, lds, st>>>(d);
-      if (xbf) {
-        if (ppt == 1) { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 1) } else { AQTX_FUSED(uint16_t, 2, 1) } }
-        else { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 2) } else { AQTX_FUSED(uint16_t, 2, 2) } }
-      } else {
-        if (ppt == 1) { if (rows == 1) { AQTX_FUSED(float, 1, 1) } else { AQTX_FUSED(float, 2, 1) } }
-        else { if (rows == 1) { AQTX_FUSED(float, 1, 2) } else { AQTX_FUSED(float, 2, 2) } }
-      }
-#undef AQTX_FUSED
-      AQTX_HIP_CHECK_LAUNCH("decode_fused_kernel");
-      return 0;
-    }
-  }
-
-  // 1. per-token dynamic quantization of the activations (same kernel as training)
-  aqtx_quant_plan q{};
-  q.in_dtype = q.compute_dtype = p->x_dtype;
-  q.scale_dtype = p->x_scale_dtype;
-  q.out_dtype = AQTX_I8;
-  q.batch = 1; q.rows = p->m; q.cols = p->k;
-  q.reduce = AQTX_REDUCE_COLS;
-  q.quant_bound = p->quant_bound; q.clip_bound = p->clip_bound;
-  q.noise = AQTX_NOISE_NONE;
-  if (int rc = aqtx_quantize(&q, x, nullptr, xq_buf, x_scale, nullptr, 0, stream)) return rc;
-
-  // 2. the contraction with the dequantisation fused
   DecodeArgs d{};
-  d.xq = xq_buf; d.w = reinterpret_cast<const int8_t*>(w);
-  d.x_scale = x_scale; d.w_scale = w_scale; d.out = out;
+  d.w = reinterpret_cast<const int8_t*>(w);
+  d.w_scale = w_scale; d.out = out;
   d.m = (int)p->m; d.n = (int)p->n; d.k = (int)p->k;
   d.out_bf16 = p->out_dtype == AQTX_BF16;
   d.xs_bf16 = p->x_scale_dtype == AQTX_BF16;
   d.ws_bf16 = p->w_scale_dtype == AQTX_BF16;
+  d.x = x; d.x_scale_out = x_scale;
+  d.quant_bound = p->quant_bound; d.clip_bound = p->clip_bound; d.x_bf16 = xbf;
+  d.acc_shift = pk ? 4 : 0;
 
-  const unsigned grid16 = (unsigned)((p->n + 15) / 16);
-  if (p->w_dtype == AQTX_I4P) {
-    d.acc_shift = 4;
-    const unsigned grid32 = (unsigned)((p->n + 31) / 32);
-    // two weight blocks per wave halve the activation re-reads; worth it once n / 32 workgroups
-    // still fill the chip
-    const bool wide = p->n >= 8192;
-    if (p->m <= 16) decode_ksplit_i4_kernel<1, 1, 8><<<grid16, 256, 0, st>>>(d);
-    else if (p->m <= 32 && wide) decode_ksplit_i4_kernel<2, 2, 4><<<grid32, 256, 0, st>>>(d);
-    else if (p->m <= 32) decode_ksplit_i4_kernel<2, 1, 4><<<grid16, 256, 0, st>>>(d);
-    else if (wide) decode_ksplit_i4_kernel<4, 2, 2><<<grid32, 256, 0, st>>>(d);
-    else decode_ksplit_i4_kernel<4, 1, 2><<<grid16, 256, 0, st>>>(d);
-    AQTX_HIP_CHECK_LAUNCH("decode_ksplit_i4_kernel");
+  // One or two tokens: one kernel quantizes and contracts.  Every workgroup repeats the
+  // quantisation, so its cost grows with the rows while the launch it saves does not: measured at
+  // k = 4096, one row gains 2.5 us per call, two rows 1 us, three rows lose.
+  const bool never_fuse = ((p->tuning >> 16) & 15) == 1;
+  if (!never_fuse && p->k <= 8192 && p->m <= 2) {
+    d.xq_out = reinterpret_cast<int8_t*>(xq);
+    const int ppt = p->k <= 4096 ? 1 : 2;
+    const unsigned grid = (unsigned)((p->n + 15) / 16);
+    const int rows = (int)p->m;
+    const size_t lds = (size_t)rows * (size_t)((p->k + 255) / 256 * 256);
+#define AQTX_FUSED(T, R, P)                                                   \
+  if (pk) decode_fused_kernel<T, R, P, 8, true><<<grid, 256, lds, st>>>(d);  \
+  else decode_fused_kernel<T, R, P, 16, false><<<grid, 256, lds, st>>>(d);
+    if (xbf) {
+      if (ppt == 1) { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 1) } else { AQTX_FUSED(uint16_t, 2, 1) } }
+      else { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 2) } else { AQTX_FUSED(uint16_t, 2, 2) } }
+    } else {
+      if (ppt == 1) { if (rows == 1) { AQTX_FUSED(float, 1, 1) } else { AQTX_FUSED(float, 2, 1) } }
+      else { if (rows == 1) { AQTX_FUSED(float, 1, 2) } else { AQTX_FUSED(float, 2, 2) } }
+    }
+#undef AQTX_FUSED
+    AQTX_HIP_CHECK_LAUNCH("decode_fused_kernel");
     return 0;
   }
-  if (p->m <= 16) {
-    decode_ksplit_kernel<1, 16><<<grid16, 256, 0, st>>>(d);
-    AQTX_HIP_CHECK_LAUNCH("decode_ksplit_kernel");
-    return 0;
-  }
-  // Whole-K waves sharing the activations through LDS need n/16 >= a few waves per CU to keep
-  // HBM busy; below that the K-split shape wins although it re-reads the activations.
-  // AQTX_DECODE_SHAPE=ksplit|block overrides the choice (tuning).
-  const char* shape_env = getenv("AQTX_DECODE_SHAPE");
-  const bool force_ksplit = shape_env != nullptr && shape_env[0] == 'k';
-  const bool force_block = shape_env != nullptr && shape_env[0] == 'b';
-  if ((p->n < 12288 && !force_block) || force_ksplit) {
-    if (p->m <= 32) decode_ksplit_kernel<2, 8><<<grid16, 256, 0, st>>>(d);
-    else decode_ksplit_kernel<4, 4><<<grid16, 256, 0, st>>>(d);
-    AQTX_HIP_CHECK_LAUNCH("decode_ksplit_kernel");
-    return 0;
-  }
-  const unsigned grid = (unsigned)((p->n + 63) / 64);
-  if (p->m <= 32) decode_block_kernel<2, 4, 2><<<grid, 512, 0, st>>>(d);
-  else decode_block_kernel<4, 4, 2><<<grid, 512, 0, st>>>(d);
-  AQTX_HIP_CHECK_LAUNCH("decode_block_kernel");
-  return 0;
+
+  const TileShape t = choose_tile_shape(p);
+  const size_t exch = t.sums_bytes;
+  const size_t frag_off = exchange_bytes_bound(p);
+  const size_t need = frag_off + fragment_bytes_bound(p);
+  AQTX_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+               "aqtx_decode_i8: workspace too small (%zu < %zu)", workspace_bytes, need);
+  AQTX_REQUIRE(((uintptr_t)workspace % 256) == 0, "aqtx_decode_i8: the workspace must be 256-byte aligned");
+  uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+  d.xq_frag = reinterpret_cast<int8_t*>(ws + frag_off);
+  d.mb_total = (int)((p->m + 15) / 16);
+  d.frag_halves = pk ? 2 : 1;
+
+  // 1. per-token dynamic quantisation of the activations; the same launch clears the exchange words
+  d.xq_out = reinterpret_cast<int8_t*>(xq);
+  if (int rc = xbf ? launch_decode_quant<uint16_t>(d, reinterpret_cast<uint4*>(ws), (int)(exch / 16), st)
+                   : launch_decode_quant<float>(d, reinterpret_cast<uint4*>(ws), (int)(exch / 16), st))
+    return rc;
+
+  // 2. the contraction with the dequantisation fused
+  d.x_scale = x_scale;
+  d.k_slice = t.k_slice; d.splits = t.splits;
+  d.sums = reinterpret_cast<int*>(ws);
+  d.count_shift = t.count_shift;
+  return pk ? launch_tile<true>(t, d, st) : launch_tile<false>(t, d, st);
 }

@@ -297,9 +297,15 @@ void gemm_kernel(const GemmArgs g_in) {
   };
 
   // An odd number of 128-byte K blocks is rounded up: with KTAIL the extra block is masked
-  // to zeros; without it K is a multiple of 256 bytes and no extra block exists.  Blocks
-  // requested past the end of K are never consumed.
+  // to zeros; without it K is a multiple of 256 bytes and no extra block exists.
   const int KT2 = (int)((g.k + 2 * BK - 1) / (2 * BK));
+  // The scalar offset of a buffer load is not part of the hardware's range check, so a block
+  // requested past the end of K would really be fetched (up to 256 bytes past the last row of
+  // the operand).  Without KTAIL the two look-ahead requests of the last trip are redirected to
+  // the last block of K instead (a scalar minimum; their data is never consumed); with KTAIL
+  // the per-chunk mask in load_global already covers them.
+  const int k0_last = KTAIL ? 0x7FFFFF00 : (int)g.k - BK;
+  auto refill_at = [&](int k0) { return k0 < k0_last ? k0 : k0_last; };
 #pragma unroll
   for (int j = 0; j < NL; ++j) load_global(j, 0);
 #pragma unroll
@@ -311,8 +317,8 @@ void gemm_kernel(const GemmArgs g_in) {
   __syncthreads();
   load_frags(stage0, 0, fa0, fb0);
   for (int it = 0; it < KT2; ++it) {
-    run_stage(stage0, stage0, stage1, (2 * it + 2) * BK);
-    run_stage(stage1, stage1, stage0, (2 * it + 3) * BK);
+    run_stage(stage0, stage0, stage1, refill_at((2 * it + 2) * BK));
+    run_stage(stage1, stage1, stage0, refill_at((2 * it + 3) * BK));
   }
   __syncthreads();
 

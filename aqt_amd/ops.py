@@ -285,7 +285,7 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
 
 def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
            clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False,
-           w_dtype: int = L.I8):
+           w_dtype: int = L.I8, tuning: int = 0):
   """Serving contraction out = dequant(quant(x) @ w_q^T) for x [m <= 64, k], w_q int8 [n, k], or
   uint8 [n, k/2] holding packed int4 (w_dtype=I4P, the pack_i4 layout).
 
@@ -308,6 +308,7 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   plan.out_dtype = plan.x_dtype
   plan.quant_bound, plan.clip_bound = float(quant_bound), float(clip_bound)
   plan.w_dtype = w_dtype
+  plan.tuning = tuning  # launch-shape override for measurements; results do not depend on it
   ws_bytes = int(L.lib().aqtx_decode_workspace_bytes(ctypes.byref(plan)))
   ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
   out = torch.empty((m, n), dtype=x.dtype, device=x.device)

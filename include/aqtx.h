@@ -284,6 +284,10 @@ typedef struct aqtx_decode_plan {
   int32_t out_dtype;      /* AQTX_BF16 | AQTX_F32                       */
   float quant_bound, clip_bound; /* of the activation numerics        */
   int32_t w_dtype;        /* AQTX_I8 | AQTX_I4 (container) | AQTX_I4P (packed: k multiple of 32) */
+  int32_t tuning;         /* 0 = the library chooses the launch shape.  Tuning only (results never
+                             depend on it): bits 0-7 K ranges per weight tile, bits 8-11 16-row weight
+                             blocks per wave (2 | 4), bits 12-15 K steps in flight per wave (2 | 4),
+                             bits 16-19 = 1 keeps the one/two-token calls on the two-kernel path   */
 } aqtx_decode_plan;
 
 /*
@@ -300,7 +304,8 @@ typedef struct aqtx_decode_plan {
  *   xq       out : optional int8 [m, k] (the quantized activations), may be NULL
  *   x_scale  out : float32 [m]
  *   out      out : [m, n]
- *   workspace    : aqtx_decode_workspace_bytes(plan) bytes
+ *   workspace    : aqtx_decode_workspace_bytes(plan) bytes, 256-byte aligned, any contents (the
+ *                  partial sums of the K ranges and, when xq is NULL, the quantized activations)
  */
 int aqtx_decode_i8(const aqtx_decode_plan* plan, const void* x, const void* w,
                    const float* w_scale, void* xq, float* x_scale, void* out,
