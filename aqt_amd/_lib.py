@@ -65,7 +65,7 @@ class DecodePlan(ctypes.Structure):
       ('x_dtype', ctypes.c_int32), ('x_scale_dtype', ctypes.c_int32),
       ('w_scale_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
       ('quant_bound', ctypes.c_float), ('clip_bound', ctypes.c_float),
-      ('w_dtype', ctypes.c_int32), ('tuning', ctypes.c_int32),
+      ('w_dtype', ctypes.c_int32), ('tuning', ctypes.c_int32), ('workspace_zeroed', ctypes.c_int32),
   ]
 
 
@@ -101,6 +101,7 @@ SYMBOLS = {
     'aqtx_decode_i8': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
+    'aqtx_decode_exchange_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
     'aqtx_gemm_i8_grouped': (ctypes.c_int, [ctypes.POINTER(GroupedGemmPlan), _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_pack_i4': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, _vp]),
     'aqtx_sum_tiles': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),

@@ -495,6 +495,11 @@ void decode_tile_kernel(const DecodeArgs d) {
         const int arrived = (before[e] + half) >> d.count_shift;  // K ranges added before this one
         total[e] += before[e] - arrived * one;
         last[e] = arrived == d.splits - 1;
+        // Every K range has been added: the word goes back to zero for the next call.  A
+        // read-modify-write like the additions, so that it is carried out at the same place; a
+        // store could sit in this XCD's L2 as part of a line whose other words are still changing.
+        if (last[e])
+          __hip_atomic_fetch_and(tile_sums + (t * 4 + e) * 64 + lane, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
     const int mm = (t / NB) * 16 + r, nn = n0 + (t % NB) * 16 + 4 * c;
@@ -570,8 +575,7 @@ struct TileShape {
 
 // plan->tuning, all fields 0 = the library's choice:
 //   bits 0-7 K ranges per weight tile, bits 8-11 nb (2 | 4), bits 12-15 K steps in flight per
-//   wave (2 | 4), bits 16-19 path (1 = never fuse the activation quantisation into the
-//   contraction kernel)
+//   wave (2 | 4), bits 16-19 path (1 = one or two tokens take the path of three and more)
 TileShape choose_tile_shape(const aqtx_decode_plan* p) {
   TileShape t{};
   const int tune = p->tuning;
@@ -612,7 +616,7 @@ TileShape choose_tile_shape(const aqtx_decode_plan* p) {
 // whole tile) int32 words.
 size_t exchange_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)(p->n + 64) * 4; }
 // The quantized activations in fragment order: 64 token rows x k rounded up to a whole K step.
-size_t fragment_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)((p->k + 127) / 128 * 128); }
+size_t fragment_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)((p->k + 127) / 128 * 128) + 256; }
 
 template <bool PACKED>
 int launch_tile(const TileShape& t, const DecodeArgs& d, hipStream_t st) {
@@ -657,11 +661,15 @@ extern "C" size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* p) {
   return exchange_bytes_bound(p) + fragment_bytes_bound(p);
 }
 
-extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const void* w,
-                              const float* w_scale, void* xq, float* x_scale, void* out,
-                              void* workspace, size_t workspace_bytes, void* stream) {
-  clear_error();
-  if (int rc = validate_decode(p)) return rc;
+extern "C" size_t aqtx_decode_exchange_bytes(const aqtx_decode_plan* p) {
+  if (p == nullptr || p->m < 0 || p->n < 0 || p->k < 0 || p->m > 64) return 0;
+  return exchange_bytes_bound(p);
+}
+
+namespace {
+
+int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const float* w_scale, void* xq,
+                float* x_scale, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   if (p->m == 0 || p->n == 0) return 0;
   AQTX_REQUIRE(x != nullptr && w != nullptr && w_scale != nullptr && x_scale != nullptr && out != nullptr,
                "aqtx_decode_i8: NULL buffer");
@@ -685,7 +693,7 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
   // One or two tokens: one kernel quantizes and contracts.  Every workgroup repeats the
   // quantisation, so its cost grows with the rows while the launch it saves does not: measured at
   // k = 4096, one row gains 2.5 us per call, two rows 1 us, three rows lose.
-  const bool never_fuse = ((p->tuning >> 16) & 15) == 1;
+  const bool never_fuse = ((p->tuning >> 16) & 15) != 0;
   if (!never_fuse && p->k <= 8192 && p->m <= 2) {
     d.xq_out = reinterpret_cast<int8_t*>(xq);
     const int ppt = p->k <= 4096 ? 1 : 2;
@@ -709,26 +717,41 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
 
   const TileShape t = choose_tile_shape(p);
   const size_t exch = t.sums_bytes;
-  const size_t frag_off = exchange_bytes_bound(p);
-  const size_t need = frag_off + fragment_bytes_bound(p);
+  const size_t need = exchange_bytes_bound(p) + fragment_bytes_bound(p);
   AQTX_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                "aqtx_decode_i8: workspace too small (%zu < %zu)", workspace_bytes, need);
   AQTX_REQUIRE(((uintptr_t)workspace % 256) == 0, "aqtx_decode_i8: the workspace must be 256-byte aligned");
   uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+  // exchange words at the start, fragments in the last bytes: in a workspace shared by calls of
+  // different shapes no call's fragments land on words another call expects to be zero
+  const size_t frag_off = (workspace_bytes - fragment_bytes_bound(p)) / 256 * 256;
   d.xq_frag = reinterpret_cast<int8_t*>(ws + frag_off);
   d.mb_total = (int)((p->m + 15) / 16);
   d.frag_halves = pk ? 2 : 1;
 
-  // 1. per-token dynamic quantisation of the activations; the same launch clears the exchange words
   d.xq_out = reinterpret_cast<int8_t*>(xq);
-  if (int rc = xbf ? launch_decode_quant<uint16_t>(d, reinterpret_cast<uint4*>(ws), (int)(exch / 16), st)
-                   : launch_decode_quant<float>(d, reinterpret_cast<uint4*>(ws), (int)(exch / 16), st))
+  d.k_slice = t.k_slice; d.splits = t.splits;
+  d.sums = reinterpret_cast<int*>(ws);
+  d.count_shift = t.count_shift;
+
+  // 1. per-token dynamic quantisation of the activations; the same launch clears the exchange
+  //    words unless the caller vouches for them
+  const int clear16 = p->workspace_zeroed ? 0 : (int)(exch / 16);
+  if (int rc = xbf ? launch_decode_quant<uint16_t>(d, reinterpret_cast<uint4*>(ws), clear16, st)
+                   : launch_decode_quant<float>(d, reinterpret_cast<uint4*>(ws), clear16, st))
     return rc;
 
   // 2. the contraction with the dequantisation fused
   d.x_scale = x_scale;
-  d.k_slice = t.k_slice; d.splits = t.splits;
-  d.sums = reinterpret_cast<int*>(ws);
-  d.count_shift = t.count_shift;
   return pk ? launch_tile<true>(t, d, st) : launch_tile<false>(t, d, st);
+}
+
+}  // namespace
+
+extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const void* w,
+                              const float* w_scale, void* xq, float* x_scale, void* out,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  if (int rc = validate_decode(p)) return rc;
+  return decode_impl(p, x, w, w_scale, xq, x_scale, out, workspace, workspace_bytes, stream);
 }

@@ -117,6 +117,21 @@ def _quantize_workspace(nbytes: int, device) -> torch.Tensor:
   return ws
 
 
+def _decode_workspace(exchange_bytes: int, scratch_bytes: int, device) -> torch.Tensor:
+  """The serving contraction's workspace for the current stream.  Its leading exchange words are
+  zero between calls (the kernels reset what they use); the library keeps its other scratch in
+  the last bytes, so the tensor holds the largest exchange size and the largest scratch size
+  seen so far side by side."""
+  key = ('decode', device.index, torch.cuda.current_stream(device).cuda_stream)
+  ent = _QUANT_WS.get(key)
+  if ent is None or ent[1] < exchange_bytes or ent[2] < scratch_bytes:
+    ex = max(exchange_bytes, ent[1] if ent else 0, 1 << 20)
+    sc = max(scratch_bytes, ent[2] if ent else 0, 1 << 20)
+    ent = (torch.zeros(ex + sc, dtype=torch.uint8, device=device), ex, sc)
+    _QUANT_WS[key] = ent
+  return ent[0]
+
+
 def quantize(
     x: torch.Tensor,
     *,
@@ -310,13 +325,20 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   plan.w_dtype = w_dtype
   plan.tuning = tuning  # launch-shape override for measurements; results do not depend on it
   ws_bytes = int(L.lib().aqtx_decode_workspace_bytes(ctypes.byref(plan)))
-  ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=x.device)
+  ex_bytes = int(L.lib().aqtx_decode_exchange_bytes(ctypes.byref(plan)))
+  # one workspace per (device, stream), zero before its first use and left zero by every call
+  ws = _decode_workspace(ex_bytes, ws_bytes - ex_bytes, x.device)
+  plan.workspace_zeroed = 1
   out = torch.empty((m, n), dtype=x.dtype, device=x.device)
   x_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
   xq = torch.empty((m, k), dtype=torch.int8, device=x.device) if want_xq else None
-  with _timed('decode'):
-    L.check(L.lib().aqtx_decode_i8(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(xq),
-                                   _ptr(x_scale), _ptr(out), _ptr(ws), ws_bytes, _stream()))
+  try:
+    with _timed('decode'):
+      L.check(L.lib().aqtx_decode_i8(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(xq),
+                                     _ptr(x_scale), _ptr(out), _ptr(ws), ws.numel(), _stream()))
+  except Exception:
+    _QUANT_WS.clear()  # a failed launch sequence may have left partial sums behind
+    raise
   return (out, x_scale, xq) if want_xq else (out, x_scale)
 
 

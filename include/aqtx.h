@@ -287,7 +287,14 @@ typedef struct aqtx_decode_plan {
   int32_t tuning;         /* 0 = the library chooses the launch shape.  Tuning only (results never
                              depend on it): bits 0-7 K ranges per weight tile, bits 8-11 16-row weight
                              blocks per wave (2 | 4), bits 12-15 K steps in flight per wave (2 | 4),
-                             bits 16-19 = 1 keeps the one/two-token calls on the two-kernel path   */
+                             bits 16-19 path: 1 = one or two tokens take the path of three and more  */
+  int32_t workspace_zeroed; /* 1: the caller keeps one workspace across calls on one stream and its first
+                             aqtx_decode_exchange_bytes(plan) bytes were zero before the first call.
+                             Every call leaves them zero (the kernels reset the words they use), so
+                             later calls may say 1 again and no call has to clear them.  The rest of
+                             the scratch lives in the LAST bytes of the workspace: one shared by plans
+                             of different shapes must hold the largest exchange size plus the largest
+                             (workspace_bytes - exchange_bytes) of those plans.                      */
 } aqtx_decode_plan;
 
 /*
@@ -311,6 +318,8 @@ int aqtx_decode_i8(const aqtx_decode_plan* plan, const void* x, const void* w,
                    const float* w_scale, void* xq, float* x_scale, void* out,
                    void* workspace, size_t workspace_bytes, void* stream);
 size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* plan);
+/* Leading bytes of the workspace that hold the partial-sum exchange (see workspace_zeroed). */
+size_t aqtx_decode_exchange_bytes(const aqtx_decode_plan* plan);
 
 /*
  * aqtx_prng_split_host: jax.random.split(key, num) on the host (used by
