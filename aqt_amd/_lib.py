@@ -102,6 +102,7 @@ SYMBOLS = {
                                       _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
     'aqtx_decode_exchange_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
+    'aqtx_decode_i8_static': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8_grouped': (ctypes.c_int, [ctypes.POINTER(GroupedGemmPlan), _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_pack_i4': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, _vp]),
     'aqtx_sum_tiles': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),

@@ -11,6 +11,8 @@
 //            weight rows and one K range; partial sums of the K ranges meet through int32 atomics.
 #include "common.h"
 
+#include <mutex>
+
 namespace aqtx {
 namespace {
 
@@ -746,6 +748,38 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
   return pk ? launch_tile<true>(t, d, st) : launch_tile<false>(t, d, st);
 }
 
+// ---- scratch of the entry point that allocates nothing -------------------------------------------
+// Room for the exchange words and the fragment-ordered activations of any call with
+// n <= kStaticMaxN and k <= kStaticMaxK.  Every GPU the library runs on holds its own copy of the
+// array for the life of the process.
+constexpr int64_t kStaticMaxN = 32768, kStaticMaxK = 32768;
+constexpr size_t kStaticScratchBytes =
+    (size_t)64 * (size_t)(kStaticMaxN + 64) * 4 + (size_t)64 * (size_t)kStaticMaxK + 512;  // 10.6 MB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on each GPU, looked up once per device (the array's name is only a
+// host-side handle: it must never reach a kernel or a memset as a pointer).
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error("aqtx_decode_i8_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  AQTX_REQUIRE(dev >= 0 && dev < kMaxDevices, "aqtx_decode_i8_static: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || sym == nullptr)
+      return set_error("aqtx_decode_i8_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = sym;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
 }  // namespace
 
 extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const void* w,
@@ -754,4 +788,23 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
   clear_error();
   if (int rc = validate_decode(p)) return rc;
   return decode_impl(p, x, w, w_scale, xq, x_scale, out, workspace, workspace_bytes, stream);
+}
+
+extern "C" int aqtx_decode_i8_static(const aqtx_decode_plan* p, const void* x, const void* w,
+                                     const float* w_scale, void* xq, float* x_scale, void* out,
+                                     void* stream) {
+  clear_error();
+  if (int rc = validate_decode(p)) return rc;
+  AQTX_REQUIRE(p->n <= kStaticMaxN && p->k <= kStaticMaxK,
+               "aqtx_decode_i8_static: n = %lld, k = %lld exceed the built-in scratch (n <= %lld, k <= %lld); "
+               "use aqtx_decode_i8 with a workspace",
+               (long long)p->n, (long long)p->k, (long long)kStaticMaxN, (long long)kStaticMaxK);
+  if (p->m == 0 || p->n == 0) return 0;
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // The array keeps whatever the last call on this GPU left: the exchange words a call uses are
+  // cleared by its first kernel, never assumed to be zero.
+  aqtx_decode_plan plan = *p;
+  plan.workspace_zeroed = 0;
+  return decode_impl(&plan, x, w, w_scale, xq, x_scale, out, ws, kStaticScratchBytes, stream);
 }

@@ -300,13 +300,15 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
 
 def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
            clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False,
-           w_dtype: int = L.I8, tuning: int = 0):
+           w_dtype: int = L.I8, tuning: int = 0, static_scratch: bool = False):
   """Serving contraction out = dequant(quant(x) @ w_q^T) for x [m <= 64, k], w_q int8 [n, k], or
   uint8 [n, k/2] holding packed int4 (w_dtype=I4P, the pack_i4 layout).
 
   The activations get per-token dynamic int8 quantisation; `w_scale` is float32 [n] holding
   values of `w_scale_dtype`.  Returns (out [m, n] of x.dtype, x_scale float32 [m]) and, with
-  want_xq, the quantized activations as a third element.
+  want_xq, the quantized activations as a third element.  With static_scratch the call goes
+  through aqtx_decode_i8_static: the library's built-in device scratch instead of a workspace
+  tensor (n, k <= 32768; calls on one GPU must not overlap).
   """
   _require_gpu(x, w_q, w_scale)
   packed = w_dtype == L.I4P
@@ -324,6 +326,14 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   plan.quant_bound, plan.clip_bound = float(quant_bound), float(clip_bound)
   plan.w_dtype = w_dtype
   plan.tuning = tuning  # launch-shape override for measurements; results do not depend on it
+  if static_scratch:
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    x_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+    xq = torch.empty((m, k), dtype=torch.int8, device=x.device) if want_xq else None
+    with _timed('decode'):
+      L.check(L.lib().aqtx_decode_i8_static(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(xq),
+                                            _ptr(x_scale), _ptr(out), _stream()))
+    return (out, x_scale, xq) if want_xq else (out, x_scale)
   ws_bytes = int(L.lib().aqtx_decode_workspace_bytes(ctypes.byref(plan)))
   ex_bytes = int(L.lib().aqtx_decode_exchange_bytes(ctypes.byref(plan)))
   # one workspace per (device, stream), zero before its first use and left zero by every call

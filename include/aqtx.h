@@ -322,6 +322,21 @@ size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* plan);
 size_t aqtx_decode_exchange_bytes(const aqtx_decode_plan* plan);
 
 /*
+ * aqtx_decode_i8_static: aqtx_decode_i8 without the workspace argument.  It has no counterpart in
+ * the reference; it is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The partial sums and the
+ * fragment-ordered activations live in a 10.6 MB array built into the library's device code (one
+ * copy per GPU, held until the process ends); the call makes no allocation, copy, memset or
+ * synchronisation.  Limits: n <= 32768 and k <= 32768 (larger plans are rejected with an error;
+ * use aqtx_decode_i8).  plan->workspace_zeroed is ignored.  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (different streams or host threads) race; calls on
+ * one stream are ordered and safe.  The first call on a GPU looks up the array's device address
+ * and must not be made while a stream of that GPU is being captured.
+ */
+int aqtx_decode_i8_static(const aqtx_decode_plan* plan, const void* x, const void* w,
+                          const float* w_scale, void* xq, float* x_scale, void* out, void* stream);
+
+/*
  * aqtx_prng_split_host: jax.random.split(key, num) on the host (used by
  * config.set_context, aqt/jax/v2/config.py:61-90).  out_host: uint32[num][2].
  */
