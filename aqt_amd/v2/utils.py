@@ -37,7 +37,7 @@ class _Int4:
   """Stands for jnp.int4: 4-bit values kept one per byte in an int8 tensor."""
 
   def __repr__(self):
-    return 'int4'
+    return 'torch.int4'  # printed like the torch dtypes it sits next to in configuration trees
 
   # One object stands for the dtype: configurations are deep-copied (set_context), and
   # `dtype is utils.int4` must keep holding for the copies.
@@ -58,6 +58,7 @@ def _int4_singleton():
 # dtype names the reference takes from jax.numpy
 int4 = _Int4()
 int8 = torch.int8
+int16 = torch.int16
 int32 = torch.int32
 bfloat16 = torch.bfloat16
 float32 = torch.float32
