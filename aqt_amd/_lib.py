@@ -47,6 +47,7 @@ class GemmPlan(ctypes.Structure):
       ('scale_order', ctypes.c_int32),
       ('row_scale_stride_b', ctypes.c_int64), ('col_scale_stride_b', ctypes.c_int64),
       ('group_offsets', ctypes.c_void_p),
+      ('tuning', ctypes.c_int32),
   ]
 
 

@@ -69,9 +69,8 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
                      p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
   const bool ktail = (p->k % (2 * BK)) != 0;
   // Two waves per SIMD by default: measured faster on every shape tried (the epilogue of one
-  // wave overlaps the other's work).  AQTX_GEMM_WAVES=4|8 overrides it per call (tests, tuning).
-  const char* waves_env = getenv("AQTX_GEMM_WAVES");
-  const int waves = (waves_env != nullptr && atoi(waves_env) == 4) ? 4 : 8;
+  // wave overlaps the other's work).  plan->tuning = 4 | 8 overrides it (tests, tuning).
+  const int waves = p->tuning == 4 ? 4 : 8;
 #define AQTX_LAUNCH(E, C, T)                                             \
   do {                                                                  \
     if (waves == 8) gemm_kernel<MmaI8, 8, E, C, T><<<grid, 512, 0, st>>>(g); \

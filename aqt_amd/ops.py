@@ -220,6 +220,11 @@ def quantize(
   return (q, scale, typed) if want_typed_scale else (q, scale)
 
 
+# aqtx_gemm_plan.tuning of every gemm() call: 0 = the library's choice; 4 | 8 = waves per workgroup
+# of the int8 kernel (the parity tests run both shapes).
+GEMM_TUNING = 0
+
+
 def gemm(
     a: torch.Tensor,
     b: torch.Tensor,
@@ -277,6 +282,7 @@ def gemm(
   plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else sc_dt
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else sc_dt
   plan.scale_order = scale_order
+  plan.tuning = GEMM_TUNING
   for s, shape in ((row_scale, (batch, m)), (col_scale, (b.shape[0], n))):
     if s is not None:
       assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == shape, (tuple(s.shape), shape)

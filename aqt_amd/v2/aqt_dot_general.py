@@ -16,7 +16,6 @@ import math
 import weakref
 from typing import Any, Optional, Sequence
 
-import numpy as onp
 import torch
 
 from aqt_amd import _lib as L
@@ -585,20 +584,21 @@ class DotGeneralRaw:
     return dot_general_raw_make(*args, **kwargs)
 
   # ------------------------------------------------------------------------------
-  def __call__(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes=None):
+  def __call__(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes=None, _bwd_memo=None):
     """A quantized dot_general without custom gradient (aqt_dot_general.py:757-840).
 
     Returns (out, DotGeneralRes).  `rhs` may be a MultiTensor (bwd calls).
     `_out_transpose_axes` (this build): the caller is going to transpose the result with these
     axes; when that transpose merely swaps the lhs-remaining and rhs-remaining groups the
     contraction kernel writes the transposed result directly and `out` comes back already
-    transposed (and contiguous).
+    transposed (and contiguous).  `_bwd_memo` (this build): a dict owned by one backward pass, in
+    which its two contractions share per-tensor scales of the gradient.
     """
     with torch.profiler.record_function(self.jax_scope_name):
       if isinstance(rhs, MultiTensor):
         lhs, rhs = _maybe_use_fwd_quant(lhs, rhs, dimension_numbers, self.rhs.use_fwd_quant)
       if self.local_aqt is None:
-        return self._dispatch(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes)
+        return self._dispatch(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, _out_transpose_axes, _bwd_memo)
       # LocalAqt (aqt_dot_general.py:773-776, 833-837): every shard of the contraction axis is
       # calibrated and contracted on its own (the shard axis is a leading batch axis), the
       # dequantized shard outputs are summed; no residuals come back.
@@ -608,14 +608,14 @@ class DotGeneralRaw:
       n_ca = len(dimension_numbers[0][0])
       assert n_ca == len(dimension_numbers[0][1])
       lhs, rhs, dn = _apply_local_aqt(self.local_aqt, lhs, rhs, dimension_numbers)
-      out, _ = self._dispatch(lhs, rhs, lhs_qt, rhs_qt, dn, None)
+      out, _ = self._dispatch(lhs, rhs, lhs_qt, rhs_qt, dn, None, _bwd_memo)
       if n_ca > 0:
         out = ops.sum_tiles(out.contiguous())
       if _out_transpose_axes is not None:
         out = out.permute(tuple(_out_transpose_axes))
       return out, None
 
-  def _dispatch(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes):
+  def _dispatch(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes, bwd_memo=None):
     """The fused kernels where they implement the configuration, the step-by-step path otherwise."""
     # a ragged (grouped) contraction hook is lowered too: same kernels, rows looked up per group
     fusable = ((self.dot_general is lax_dot_general or _ragged_sizes(self.dot_general) is not None)
@@ -623,12 +623,17 @@ class DotGeneralRaw:
     for side in (self.lhs, self.rhs):
       fusable = fusable and (side.dequant_mode == DequantMode.OUTPUT
                              and side.calibration_mode == CalibrationMode.CONTRACTING_AXIS)
+    calibrated = {}  # id(quantizer) -> scales found step by step during the fused attempt
     if fusable:
       try:
-        return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes)
+        return self._lowered_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes,
+                                  _bwd_memo=bwd_memo, _calibrated=calibrated)
       except _NotFused:
         pass
-    return self._unfused_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes)
+    # The attempt may have run a calibration before it found out that the call has no fused form
+    # (the reference updates a stateful calibrator once per call): those results are handed over.
+    with aqt_quantizer.replay_calibrations(calibrated):
+      return self._unfused_call(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes)
 
   # ------------------------------------------------------------------------------
   def _unfused_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None):
@@ -668,7 +673,7 @@ class DotGeneralRaw:
 
   # ------------------------------------------------------------------------------
   def _lowered_call(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes=None,
-                    _dtypes=None):
+                    _dtypes=None, _bwd_memo=None, _calibrated=None):
     """`_dtypes` = (lhs dtype, rhs dtype, dequant dtype) when `lhs` and `rhs` are the qvalues of
     the given QTensors and so do not carry the dtypes of the tensors they were quantized from."""
     dq = self.dg_quantizer
@@ -731,10 +736,10 @@ class DotGeneralRaw:
 
     # ---- lhs ---------------------------------------------------------------------
     lq, ls, lsdt, lhs_qt_out, lhs_grad = self._quant_side(
-        'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t)
+        'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t, _bwd_memo, _calibrated)
     # ---- rhs ---------------------------------------------------------------------
     rq, rs, rsdt, rhs_qt_out, rhs_grad = self._quant_side(
-        'rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, rba, rra, rca, None)
+        'rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, rba, rra, rca, None, _bwd_memo, _calibrated)
 
     lkd = aqt_tensor.qvalue_kernel_dtype(lhs_qt_out)
     rkd = aqt_tensor.qvalue_kernel_dtype(rhs_qt_out)
@@ -853,8 +858,11 @@ class DotGeneralRaw:
                         rhs=TensorRes(mt=MultiTensor(x=rhs_arr, qx=rhs_qt), quant_grad=rhs_grad))
     return out, res
 
-  def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t):
-    """Quantizes one side; returns (q [B,R,K], scale f32, scale dtype, QTensor, quant_grad)."""
+  def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t,
+                  bwd_memo=None, calibrated=None):
+    """Quantizes one side; returns (q [B,R,K], scale f32, scale dtype, QTensor, quant_grad).
+    `bwd_memo`: the backward pass's table of per-tensor scales; `calibrated`: where a calibration
+    that runs step by step leaves its result for a later fall-back of the same call."""
     if given_qt is not None and given_qt.is_full():
       # Serving: the provided QTensor replaces the computed one (aqt_dot_general.py:614-635).
       quant_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
@@ -882,6 +890,8 @@ class DotGeneralRaw:
       if prescale_t is not None:
         x, prescale_t = x * prescale_t.to(x.dtype), None
       given_qt = quantizer.calibrate(x, calibration_axes=ca)
+      if calibrated is not None:
+        calibrated[id(quantizer)] = given_qt
       if len(given_qt.scale) != 1 or given_qt.bias or given_qt.sparsity_mask is not None:
         raise _NotFused(f'{name}: calibration with a bias, a sparsity mask or several scales')
       spec = nspec
@@ -919,11 +929,11 @@ class DotGeneralRaw:
     # Both gradient contractions calibrate the same gradient; with one scale per tensor and no
     # forward-scale factor on it the abs-max is the same number, found once per backward pass.
     memo_key, memo_hit = None, None
-    if (_PER_TENSOR_SCALES is not None and given_qt is None and prescale is None and not x_is_q
+    if (bwd_memo is not None and given_qt is None and prescale is None and not x_is_q
         and quantizer.calib_shared_axes == 'per_tensor' and quantizer.kernel_spec() is not None):
       memo_key = (arr.data_ptr(), arr._version, tuple(arr.shape), arr.dtype, spec['quant_bound'],
                   quantizer._calibrator.dtype)
-      memo_hit = _PER_TENSOR_SCALES.get(memo_key)
+      memo_hit = bwd_memo.get(memo_key)
       if memo_hit is not None:
         flat = memo_hit[0].reshape(1).expand(v.B * v.R)
         scale_in = flat.contiguous().reshape(v.B, v.R, 1) if v.k_last else flat.contiguous().reshape(v.B, 1, v.R)
@@ -938,15 +948,12 @@ class DotGeneralRaw:
     else:
       scale_list = [lowering.scale_in_dtype(s32, v, sdt)]
       if memo_key is not None:
-        _PER_TENSOR_SCALES[memo_key] = (s32, scale_list, sdt)
+        bwd_memo[memo_key] = (s32, scale_list, sdt)
     qt = aqt_tensor.QTensor(qvalue=qv, scale=scale_list, scale_t=None, bias=[], dequant_dtype=dtype,
                             container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
     quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))
     return q, s32, sdt, qt, quant_grad
 
-
-# per-tensor scales found during the backward pass in progress (None outside one)
-_PER_TENSOR_SCALES = None
 
 _DTYPES_CAN_BE_SCALED = (torch.bfloat16, torch.float32, torch.float64)
 
@@ -1197,27 +1204,32 @@ def dg_core_vjp_fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, cfg: DotGeneral
 
 
 def _update_dimension_numbers_for_backward(fwd_dimension_numbers, y_is_lhs, gradient_rank, y_rank):
-  """aqt_dot_general.py:1127-1175."""
-  def ranges_like(*xs):
-    start = 0
-    for x in xs:
-      yield tuple(range(start, start + len(x)))
-      start += len(x)
+  """Dimension numbers of the contraction that turns the output gradient g and the operand y into
+  the gradient of the other operand x, and the permutation that brings its result into x's axis
+  order (what aqt_dot_general.py:1127-1175 computes).
 
-  (x_ca, y_ca), (x_ba, y_ba) = fwd_dimension_numbers
+  The forward output, and so g, is laid out (batch, lhs free, rhs free).  The gradient of x
+  contracts g's axes that came from y's free axes with those free axes, batches over the batch
+  axes, and so comes out as (batch, x free, y contraction axes in y's axis order).
+  """
+  (lhs_ca, rhs_ca), (lhs_ba, rhs_ba) = fwd_dimension_numbers
   if y_is_lhs:
-    (y_ca, x_ca) = (x_ca, y_ca)
-    (y_ba, x_ba) = (x_ba, y_ba)
-  gradient_rank = gradient_rank - y_rank + len(x_ba) + 2 * len(x_ca)
-  x_ra = tuple(utils.get_remaining_axes(gradient_rank, x_ca, x_ba))
-  y_ra = tuple(utils.get_remaining_axes(y_rank, y_ca, y_ba))
-  if y_is_lhs:
-    g_ba, g_ca, _ = ranges_like(x_ba, y_ra, x_ra)
+    x_ca, x_ba, y_ca, y_ba = list(rhs_ca), list(rhs_ba), list(lhs_ca), list(lhs_ba)
   else:
-    g_ba, _, g_ca = ranges_like(x_ba, x_ra, y_ra)
-  dims = ((g_ca, y_ra), (g_ba, tuple(y_ba)))
-  x_ca_sorted_by_y = tuple(int(i) for i in onp.take(x_ca, onp.argsort(y_ca)))
-  out_transpose_axes = tuple(int(i) for i in onp.argsort(tuple(x_ba) + x_ra + x_ca_sorted_by_y))
+    x_ca, x_ba, y_ca, y_ba = list(lhs_ca), list(lhs_ba), list(rhs_ca), list(rhs_ba)
+  n_batch = len(x_ba)
+  y_free = [a for a in range(y_rank) if a not in y_ca and a not in y_ba]
+  x_rank = gradient_rank - len(y_free) + len(x_ca)  # g has batch + x free + y free axes
+  x_free = [a for a in range(x_rank) if a not in x_ca and a not in x_ba]
+  # where y's free axes sit in g: straight after the batch axes when y is the lhs, last otherwise
+  first = n_batch if y_is_lhs else n_batch + len(x_free)
+  g_contract = tuple(range(first, first + len(y_free)))
+  dims = ((g_contract, tuple(y_free)), (tuple(range(n_batch)), tuple(y_ba)))
+  # axis of x that each axis of the result stands for; y's surviving (contraction) axes appear in
+  # increasing y order, each paired with its x axis
+  x_ca_in_y_order = [xa for _, xa in sorted(zip(y_ca, x_ca))]
+  result_is_x_axis = x_ba + x_free + x_ca_in_y_order
+  out_transpose_axes = tuple(result_is_x_axis.index(a) for a in range(x_rank))
   return dims, out_transpose_axes
 
 
@@ -1231,19 +1243,18 @@ def dg_core_vjp_bwd(fwd_dimension_numbers, res, g):
   def grad_dot_general(y_res: TensorRes, quant_grad, dg_raw: DotGeneralRaw, y_is_lhs):
     dims, out_transpose_axes = _update_dimension_numbers_for_backward(
         fwd_dimension_numbers, y_is_lhs, g.dim(), y_res.mt.x.dim())
-    transposed_out, _ = dg_raw(g, y_res.mt, None, None, dims, _out_transpose_axes=out_transpose_axes)
+    transposed_out, _ = dg_raw(g, y_res.mt, None, None, dims, _out_transpose_axes=out_transpose_axes,
+                               _bwd_memo=bwd_memo)
     if quant_grad is not None:
       assert not isinstance(quant_grad, str), quant_grad
       transposed_out = quant_grad(transposed_out)[0]
     return transposed_out
 
-  global _PER_TENSOR_SCALES
-  _PER_TENSOR_SCALES = {}
-  try:
-    dlhs = grad_dot_general(dg_res.rhs, dg_res.lhs.quant_grad, cfg.dlhs, False)
-    drhs = grad_dot_general(dg_res.lhs, dg_res.rhs.quant_grad, cfg.drhs, True)
-  finally:
-    _PER_TENSOR_SCALES = None
+  # Both contractions calibrate the same gradient; a scale that is one number per tensor is found
+  # once and shared through this table, which lives as long as this backward pass.
+  bwd_memo = {}
+  dlhs = grad_dot_general(dg_res.rhs, dg_res.lhs.quant_grad, cfg.dlhs, False)
+  drhs = grad_dot_general(dg_res.lhs, dg_res.rhs.quant_grad, cfg.drhs, True)
   return (dlhs, drhs, None, None, None)
 
 

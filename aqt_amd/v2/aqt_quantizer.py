@@ -2,6 +2,8 @@
 from __future__ import annotations
 
 import copy
+import contextlib
+import contextvars
 import dataclasses
 import functools
 from typing import Any, Optional, Sequence
@@ -20,6 +22,22 @@ from aqt_amd.v2.numerics import utils as numerics_utils
 AbstractAqtNumerics = numerics.AqtNumerics
 AbstractAqtCalibration = calibration.Calibration
 
+
+
+# Calibration results of an abandoned fused attempt, handed to the step-by-step path that takes
+# over the same call (id(quantizer) -> incomplete QTensor); None outside such a hand-over.
+_REPLAY: 'contextvars.ContextVar' = contextvars.ContextVar('aqt_calibration_replay', default=None)
+
+
+@contextlib.contextmanager
+def replay_calibrations(done: dict):
+  """Inside, Quantizer.calibrate returns (once) what `done` holds for that quantizer object
+  instead of calibrating again."""
+  token = _REPLAY.set(dict(done))
+  try:
+    yield
+  finally:
+    _REPLAY.reset(token)
 
 @dataclasses.dataclass(kw_only=True)
 class Quantizer:
@@ -98,6 +116,11 @@ class Quantizer:
 
   def calibrate(self, x, *, calibration_axes, tiling_state=None) -> aqt_tensor.QTensor:
     """Incomplete QTensor holding only the scale (aqt_quantizer.py:79-157)."""
+    replay = _REPLAY.get()
+    if replay is not None and id(self) in replay:
+      # this quantizer has calibrated this very tensor a moment ago, in the attempt to run the
+      # call on the fused kernels: a stateful calibrator must see one update per step, not two
+      return replay.pop(id(self))
     if tiling_state is not None:
       x = tiling_state.apply(x)
       _, calibration_axes = tiling_state.to_tiled_axes_transposed(calibration_axes)

@@ -149,6 +149,8 @@ typedef struct aqtx_gemm_plan {
      (row_scale is flat [m] too); stride_a, stride_c and row_scale_stride_b are ignored.  Rows
      outside every group are not written.  NULL: ordinary batches.                          */
   const int32_t* group_offsets;
+  int32_t tuning;             /* 0 = the library chooses the launch shape.  Tuning only (results never
+                                 depend on it): 4 | 8 = waves per workgroup of the int8 kernel            */
 } aqtx_gemm_plan;
 
 /*

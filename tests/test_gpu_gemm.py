@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(params=[4, 8], ids=['waves4', 'waves8'])
 def waves(request, monkeypatch):
   """Both workgroup shapes of the int8 MFMA kernel."""
-  monkeypatch.setenv('AQTX_GEMM_WAVES', str(request.param))
+  monkeypatch.setattr(ops, 'GEMM_TUNING', request.param)
   return request.param
 
 

@@ -110,3 +110,38 @@ def test_dot_general_with_delayed_scaling(gpu):
   ref = a2 @ b2
   # 7 and 6 effective bits (the operands are half and a quarter of the bounds)
   assert (out - ref).abs().max().item() <= 0.05 * ref.abs().max().item()
+
+
+class _CountingAbsMax(calibration.AbsMaxCalibration):
+  """Abs-max calibration that counts its calls and has no fused kernel (a stand-in for any
+  stateful calibrator: every call is a state update)."""
+  calls = 0
+
+  def kernel_supported(self):
+    return False
+
+  def get_scale_and_bias_and_sparsity(self, x, shared_axes, numerics_, context=None):
+    type(self).calls += 1
+    return super().get_scale_and_bias_and_sparsity(x, shared_axes, numerics_, context)
+
+
+def test_fallback_after_a_fused_attempt_calibrates_once(gpu):
+  """The lhs calibrates step by step inside the fused attempt; the rhs (clip_gradient numerics)
+  then turns the call over to the step-by-step path, which must take the lhs scale over
+  instead of calibrating a second time (the reference calibrates once per call)."""
+  dg = aqt.dot_general_raw_make(8, 8)
+  dg.dg_quantizer.lhs.calibration = _CountingAbsMax
+  dg.dg_quantizer.rhs.numerics.clip_gradient = True  # no fused form: found out after the lhs is done
+  dg.dg_quantizer.lhs._calibrator = None
+  dg.dg_quantizer.rhs._calibrator = None
+  dg.dg_quantizer.init_calibration()
+  lhs = torch.randn(32, 64, device=gpu)
+  rhs = torch.randn(64, 48, device=gpu)
+  _CountingAbsMax.calls = 0
+  out, res = dg(lhs, rhs, None, None, (((1,), (0,)), ((), ())))
+  torch.cuda.synchronize()
+  assert _CountingAbsMax.calls == 1
+  assert out.shape == (32, 48) and torch.isfinite(out).all()
+  # and the scale the step-by-step path used is the one that calibration returned
+  want = lhs.abs().amax(dim=1, keepdim=True) / torch.tensor(127.5, device=gpu)  # a tensor divisor rounds correctly
+  torch.testing.assert_close(res.lhs.mt.qx.scale[0], want, rtol=0, atol=0)

@@ -115,6 +115,31 @@ def test_backward_dimension_numbers_match_oracle(dn, ls, rs):
     assert got == want
 
 
+@pytest.mark.parametrize('dn,ls,rs', [
+    ((((1,), (0,)), ((), ())), (5, 7), (7, 3)),
+    ((((2,), (1,)), ((0,), (0,))), (2, 5, 7), (2, 7, 3)),
+    ((((2,), (0,)), ((), ())), (2, 3, 8), (8, 4, 5)),                     # 'bsd,dhk->bshk'
+    ((((3, 1), (0, 2)), ((0,), (1,))), (2, 4, 5, 6), (6, 2, 4, 3)),
+    ((((0, 2), (2, 0)), ((1,), (1,))), (4, 3, 5, 2), (5, 3, 4, 6, 7)),    # contraction pairs out of order
+    ((((), ()), ((), ())), (3, 2), (4,)),                                 # outer product
+])
+def test_backward_dimension_numbers_give_the_autograd_gradients(dn, ls, rs):
+  """Independent of the restated formula: the float contraction run with the derived dimension
+  numbers and output permutation must equal what torch's autograd returns for the forward
+  contraction."""
+  g_ = torch.Generator().manual_seed(0)
+  lhs = torch.randn(ls, generator=g_, dtype=torch.float64, requires_grad=True)
+  rhs = torch.randn(rs, generator=g_, dtype=torch.float64, requires_grad=True)
+  out = aqt.lax_dot_general(lhs, rhs, dn)
+  g = torch.randn(out.shape, generator=g_, dtype=torch.float64)
+  dl_want, dr_want = torch.autograd.grad(out, (lhs, rhs), g)
+  for y, y_is_lhs, want in ((rhs, False, dl_want), (lhs, True, dr_want)):
+    dims, perm = aqt._update_dimension_numbers_for_backward(dn, y_is_lhs, g.dim(), y.dim())
+    got = aqt.lax_dot_general(g, y.detach(), dims).permute(perm)
+    assert got.shape == want.shape
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+
+
 def test_matmul_backward_dimension_numbers():
   dn = (((1,), (0,)), ((), ()))
   dims, perm = aqt._update_dimension_numbers_for_backward(dn, False, 2, 2)
