@@ -33,6 +33,7 @@ class QuantPlan(ctypes.Structure):
       ('prescale_stride_batch', ctypes.c_int64),
       ('scale_typed', ctypes.c_void_p),
       ('workspace_zeroed', ctypes.c_int32),
+      ('key_device', ctypes.c_void_p),
   ]
 
 

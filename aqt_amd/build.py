@@ -44,6 +44,47 @@ def _compile(src, obj):
   return obj
 
 
+FFI_SOURCE = 'aqtx_ffi.cc'
+FFI_LIB_PATH = os.path.join(LIB_DIR, 'libaqtx_ffi.so')
+
+
+def xla_ffi_include_dir():
+  """Directory holding xla/ffi/api/ffi.h, or None.  The headers ship inside jaxlib
+  (jax.ffi.include_dir()); AQTX_XLA_FFI_INCLUDE names another copy."""
+  cands = []
+  if os.environ.get('AQTX_XLA_FFI_INCLUDE'):
+    cands.append(os.environ['AQTX_XLA_FFI_INCLUDE'])
+  try:
+    import jax.ffi  # pylint: disable=import-outside-toplevel
+    cands.append(jax.ffi.include_dir())
+  except Exception:  # jax is absent or too old to have jax.ffi
+    pass
+  for c in cands:
+    if c and os.path.exists(os.path.join(c, 'xla', 'ffi', 'api', 'ffi.h')):
+      return c
+  return None
+
+
+def build_ffi_shim(verbose=True):
+  """Compiles the XLA FFI handlers (csrc/aqtx_ffi.cc) against libaqtx.so into
+  aqt_amd/lib/libaqtx_ffi.so where the XLA FFI headers exist; returns its path, or None (with a
+  message) where they do not.  Nothing stands in for missing headers."""
+  inc = xla_ffi_include_dir()
+  if inc is None:
+    if verbose:
+      print('XLA FFI headers (xla/ffi/api/ffi.h) not found: libaqtx_ffi.so not built '
+            '(install jaxlib or set AQTX_XLA_FFI_INCLUDE)', file=sys.stderr)
+    return None
+  cmd = [_hipcc(), '-x', 'hip', '--offload-arch=gfx950', '-O2', '-std=c++17', '-fPIC', '-shared', '-I', inc,
+         os.path.join(CSRC, FFI_SOURCE), '-L', LIB_DIR, '-laqtx', '-Wl,-rpath,$ORIGIN', '-o', FFI_LIB_PATH]
+  res = subprocess.run(cmd, capture_output=True, text=True)
+  if res.returncode != 0:
+    raise RuntimeError(f'hipcc failed on {FFI_SOURCE}:\n{res.stdout}\n{res.stderr}')
+  if verbose:
+    print(f'built {FFI_LIB_PATH}', file=sys.stderr)
+  return FFI_LIB_PATH
+
+
 def build_library(jobs=4, verbose=True):
   """Compiles every source and links aqt_amd/lib/libaqtx.so. Returns its path."""
   os.makedirs(LIB_DIR, exist_ok=True)
@@ -61,6 +102,7 @@ def build_library(jobs=4, verbose=True):
   os.replace(tmp, LIB_PATH)
   if verbose:
     print(f'built {LIB_PATH} from {len(sources)} sources', file=sys.stderr)
+  build_ffi_shim(verbose)
   return LIB_PATH
 
 

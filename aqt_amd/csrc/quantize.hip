@@ -42,6 +42,7 @@ struct QArgs {
   int64_t psb;            // prescale batch stride
   float quant_bound, clip_bound;
   BitGen gen;
+  const uint32_t* key_dev;  // optional: the two key words in device memory (replace gen.k0 / gen.k1)
   int noise;
   int ps_mode;
   int transpose_out;
@@ -51,6 +52,17 @@ struct QArgs {
   int scale_given;
   int ws_zeroed;  // the abs-max words of the workspace are zero on entry
 };
+
+// Kernel-side copy of the arguments with the PRNG key taken from device memory when the caller
+// passed it there (a traced key under XLA, a key updated on the device between graph replays).
+__device__ __forceinline__ QArgs with_device_key(const QArgs& in) {
+  QArgs a = in;
+  if (in.key_dev != nullptr) {
+    a.gen.k0 = in.key_dev[0];
+    a.gen.k1 = in.key_dev[1];
+  }
+  return a;
+}
 
 // The computed scale goes out as float32 and, when the caller keeps its scales in bf16, once
 // more as bf16 elements (the value is already rounded to bf16, so the narrowing is exact).
@@ -319,7 +331,8 @@ __device__ __forceinline__ uint32_t packed_absmax(uint32_t m, uint32_t w) {
 // PAIR (SPEC 2 only): the block owns segment s and segment s + nseg/2, whose elements share
 // threefry blocks; requires whole rows as segments and the natural noise layout.
 template <typename TIn, int LANES, int ITERS, int SPEC, bool PAIR>
-__global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void quant_rows_kernel(const QArgs a) {
+__global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void quant_rows_kernel(const QArgs a_in) {
+  const QArgs a = with_device_key(a_in);
   constexpr int VEC = 8;
   constexpr int SEG_PER_BLOCK = 256 / LANES;
   constexpr int NSET = PAIR ? 2 : 1;
@@ -439,7 +452,8 @@ __global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void 
 
 // Generic rows kernel: any segment length / alignment; one wave per segment, two reads.
 template <typename TIn>
-__global__ __launch_bounds__(256) void quant_rows_generic_kernel(const QArgs a) {
+__global__ __launch_bounds__(256) void quant_rows_generic_kernel(const QArgs a_in) {
+  const QArgs a = with_device_key(a_in);
   const int lane = threadIdx.x & 63;
   const int64_t seg = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (seg >= a.nseg) return;  // the whole wave leaves together; no barrier below
@@ -601,7 +615,8 @@ constexpr int kTileR = 128, kTileC = 64, kTilePad = 132;
 // layout), 2 = the tile `cols/2` further right (noise counters of the transposed tensor); the
 // two tiles' elements share threefry blocks.
 template <typename TIn, int SPEC, int PAIR>
-__global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a) {
+__global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
+  const QArgs a = with_device_key(a_in);
   constexpr int NSET = PAIR ? 2 : 1;
   __shared__ uint32_t lds[NSET][kTileC * kTilePad / 4];
   const int tid = threadIdx.x;
@@ -1081,8 +1096,11 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
   a.cbf = p->compute_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
   a.scale_given = p->scale_given;
   a.ws_zeroed = p->workspace_zeroed;
-  if (p->noise != AQTX_NOISE_NONE)
+  if (p->noise != AQTX_NOISE_NONE) {
     a.gen = make_bitgen(p->key, p->noise_total, noise_width(p), p->partitionable);
+    a.key_dev = p->key_device;
+    AQTX_REQUIRE(((uintptr_t)p->key_device % 4) == 0, "aqtx_quantize: key_device is not 4-byte aligned");
+  }
   if (p->reduce == AQTX_REDUCE_COLS) {
     a.L = p->group ? p->group : p->cols;
     a.nseg = nscales;

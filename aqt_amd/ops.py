@@ -152,6 +152,7 @@ def quantize(
     prescale_mode: int = L.PRESCALE_NONE,
     scale: Optional[torch.Tensor] = None,
     want_typed_scale: bool = False,
+    key_device: Optional[torch.Tensor] = None,
 ):
   """Calibrate (abs-max) and quantize a contiguous [batch, rows, cols] tensor.
 
@@ -159,6 +160,7 @@ def quantize(
   [batch, rows, cols] or [batch, cols, rows] with transpose_out; scale is
   float32, shaped [batch, rows, cols/group] (REDUCE_COLS),
   [batch, rows/group, cols] (REDUCE_ROWS) or [batch] (REDUCE_ALL).
+  `key_device` (a 2-word device tensor) replaces `key`: the kernels read the key from device memory.
   With want_typed_scale a third element: the computed scales once more as a bf16 tensor of
   the same shape, written by the same kernels (None unless the scale dtype is bf16 and the
   scale is computed here).
@@ -176,8 +178,13 @@ def quantize(
   plan.quant_bound, plan.clip_bound = quant_bound, clip_bound
   plan.noise, plan.partitionable = noise, int(partitionable)
   if noise != L.NOISE_NONE:
-    assert key is not None, 'noise requested but no PRNG key given'
-    plan.key[0], plan.key[1] = int(key[0]), int(key[1])
+    assert key is not None or key_device is not None, 'noise requested but no PRNG key given'
+    if key_device is not None:  # uint32[2] (held as int32) in device memory, read by the kernels
+      _require_gpu(key_device)
+      assert key_device.numel() == 2 and key_device.element_size() == 4 and key_device.is_contiguous()
+      plan.key_device = key_device.data_ptr()
+    else:
+      plan.key[0], plan.key[1] = int(key[0]), int(key[1])
     nsb, nsr, nsc = noise_strides if noise_strides is not None else (r * c, c, 1)
     plan.noise_stride_batch, plan.noise_stride_row, plan.noise_stride_col = nsb, nsr, nsc
     plan.noise_total = noise_total if noise_total is not None else b * r * c

@@ -90,6 +90,9 @@ typedef struct aqtx_quant_plan {
   int32_t workspace_zeroed; /* 1: the caller keeps one workspace across calls on one stream, passes its
                             whole size as workspace_bytes, and its first half is zero on entry;
                             aqtx_quantize returns it zeroed and skips its own clearing launch      */
+  const uint32_t* key_device; /* optional DEVICE pointer to the two key words; when not NULL the kernels
+                            read the key there and `key` above is ignored (a key that is a traced
+                            array under XLA, or one updated on the device between HIP graph replays) */
 } aqtx_quant_plan;
 
 /*

@@ -247,3 +247,27 @@ def test_im2col_validation():
   p.stride[1] = 1
   p.n = 0
   assert L.lib().aqtx_im2col_i8(ctypes.byref(p), None, None, None) == 0
+
+
+def test_ffi_shim_binds_only_declared_entry_points():
+  """csrc/aqtx_ffi.cc (compiled only where the XLA FFI headers exist) calls nothing that
+  include/aqtx.h does not declare, and fills plan fields that exist."""
+  import re
+  here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  src = open(os.path.join(here, 'aqt_amd', 'csrc', 'aqtx_ffi.cc')).read()
+  header = open(os.path.join(here, 'include', 'aqtx.h')).read()
+  called = set(re.findall(r'\b(aqtx_[a-z0-9_]+)\(', src))
+  assert called and called <= set(L.SYMBOLS), called - set(L.SYMBOLS)
+  for field in set(re.findall(r'\bp(?:\.|->)([a-z_0-9]+)\b', src)):
+    assert re.search(r'\b%s\b' % field, header), field
+  handlers = re.findall(r'XLA_FFI_DEFINE_HANDLER_SYMBOL\(\s*(\w+)', src)
+  assert {'AqtxQuantize', 'AqtxGemmI8', 'AqtxGemmFp8', 'AqtxGemmI8Grouped', 'AqtxDecodeI8', 'AqtxDequantize',
+          'AqtxSumTiles'} <= set(handlers)
+
+
+def test_ffi_shim_is_skipped_without_xla_headers(capsys):
+  from aqt_amd import build
+  if build.xla_ffi_include_dir() is not None:
+    pytest.skip('XLA FFI headers are present here')
+  assert build.build_ffi_shim(verbose=True) is None
+  assert 'not built' in capsys.readouterr().err

@@ -61,12 +61,20 @@ def _product(problem, gpu, sr, key):
   return out.detach(), L.grad, Rr.grad
 
 
-def _one_side(g, fwd, ocfg, lhs_side):
-  """One of the two backward contractions of dg_core_vjp_bwd (aqt_dot_general.py:1178-1221)."""
+def _one_side(g, fwd, ocfg, lhs_side, with_abs_dot=False):
+  """One of the two backward contractions of dg_core_vjp_bwd (aqt_dot_general.py:1178-1221).
+  with_abs_dot: also the dequantized sum of |products| of every output element."""
   y_res, raw = (fwd.lhs_res, ocfg.drhs) if lhs_side else (fwd.rhs_res, ocfg.dlhs)
   dims, out_axes = R.bwd_dimension_numbers(MATMUL, lhs_side, g.ndim, y_res.x.ndim)
-  out, _, _, _ = R.dg_raw(g, 'bf16', y_res, None, dims, raw)
-  return np.transpose(out, out_axes)
+  out, _, (g_res, y_res2), _ = R.dg_raw(g, 'bf16', y_res, None, dims, raw)
+  out = np.transpose(out, out_axes)
+  if not with_abs_dot:
+    return out
+  gq, yq = np.abs(g_res.qx.qvalue.astype(np.float64)), np.abs(y_res2.qx.qvalue.astype(np.float64))
+  scales = float(np.asarray(g_res.qx.scale[0]).reshape(-1)[0]) * float(np.asarray(y_res2.qx.scale[0]).reshape(-1)[0])
+  # dlhs contracts g[m, n] with y[k, n] over n -> [m, k]; drhs g[m, n] with y[m, k] over m -> [n, k] -> [k, n]
+  abs_dot = (yq.T @ gq) if lhs_side else (gq @ yq.T)
+  return out, abs_dot * scales
 
 
 def _check(problem, gpu, sr):
@@ -155,8 +163,11 @@ def test_full_size_fp8_einsum(gpu):
   gradients with mantissa stochastic rounding, per-tensor scales.  With one scale per tensor the
   quantization is elementwise, so any block of the three results can be restated from the
   matching blocks of the operands, provided each block holds its tensor's largest element (the
-  blocks are chosen that way).  Tolerance as for the small fp8 cases: the MFMA sums in float32
-  in its own order."""
+  blocks are chosen that way).  Tolerance, element by element: 2^-10 of the dequantized sum of
+  |products| of that element (within one instruction the fp8 MFMA drops products 2^14 below the
+  largest of its 64-long block and truncates the block sum into the float32 accumulator) plus
+  2^-7 of the value (the three bf16 roundings of the dequantisation, here and in the oracle).  fp8
+  outputs are therefore NOT comparable to the reference within one bf16 ulp."""
   from aqt_amd.v2 import aqt_dot_general as aqt
   from aqt_amd.v2 import config
   b, s, d, h, kh = 8, 4096, 4096, 32, 128
@@ -187,22 +198,29 @@ def test_full_size_fp8_einsum(gpu):
     assert torch.isfinite(t).all()
   tr, td, tc = (torch.from_numpy(i).to(gpu) for i in (rows, dsel, cols))
 
-  def close(got, want, what):
-    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=2.0 ** -7, atol=2.0 ** -9 * np.abs(want).max(),
-                               err_msg=what)
+  def close(got, want, abs_dot, what):
+    got = got.float().cpu().numpy().astype(np.float64)
+    err, bound = np.abs(got - want), 2.0 ** -10 * abs_dot + 2.0 ** -7 * np.abs(want)
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert (err <= bound).all(), f'{what}: error {err[worst]} above the bound {bound[worst]} at {worst}'
+
+  def fwd_abs_dot(f):
+    lq, rq = np.abs(f.lhs_res.qx.qvalue.astype(np.float64)), np.abs(f.rhs_res.qx.qvalue.astype(np.float64))
+    return (lq @ rq) * float(np.asarray(f.lhs_res.qx.scale[0]).reshape(-1)[0]) * float(
+        np.asarray(f.rhs_res.qx.scale[0]).reshape(-1)[0])
 
   f = R.dg_fwd(lhs2[rows], np.ascontiguousarray(rhs2[:, cols]), 'bf16', MATMUL, ocfg)
-  close(out2[tr][:, tc], f.out, 'out')
+  close(out2[tr][:, tc], f.out, fwd_abs_dot(f), 'out')
   # dlhs[rows, dsel] = g[rows, :] . rhs[dsel, :]^T
   c1 = copy.deepcopy(ocfg)
   c1.dlhs.lhs.noise_window = ((bs, hk), (rows, np.arange(hk)))
   f1 = R.dg_fwd(lhs2[np.ix_(rows, dsel)], rhs2[dsel], 'bf16', MATMUL, c1)
-  close(dl2[tr][:, td], _one_side(g2[rows], f1, c1, False), 'dlhs')
+  close(dl2[tr][:, td], *_one_side(g2[rows], f1, c1, False, with_abs_dot=True), 'dlhs')
   # drhs[dsel, cols] = lhs[:, dsel]^T . g[:, cols]
   c2 = copy.deepcopy(ocfg)
   c2.drhs.lhs.noise_window = ((bs, hk), (np.arange(bs), cols))
   f2 = R.dg_fwd(np.ascontiguousarray(lhs2[:, dsel]), rhs2[np.ix_(dsel, cols)], 'bf16', MATMUL, c2)
-  close(dr2[td][:, tc], _one_side(np.ascontiguousarray(g2[:, cols]), f2, c2, True), 'drhs')
+  close(dr2[td][:, tc], *_one_side(np.ascontiguousarray(g2[:, cols]), f2, c2, True, with_abs_dot=True), 'drhs')
 
 
 @pytest.mark.parametrize('m', [1, 8, 32, 64])

@@ -243,3 +243,30 @@ def test_few_long_rows_stochastic_rounding(gpu, batch, rows, cols, noise, dt):
   qg2, _ = ops.quantize(U.to_dev(x, dt, gpu), reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=qb, clip_bound=cb,
                         noise=U.NOISE[noise], key=key, scale=sg.clone())
   assert torch.equal(qg, qg2)
+
+
+@pytest.mark.parametrize('reduce,transpose,shape', [
+    (L.REDUCE_COLS, False, (1, 64, 1024)),   # rows kernel, rows paired over one threefry block
+    (L.REDUCE_COLS, False, (2, 9, 1000)),    # rows kernel, plain
+    (L.REDUCE_COLS, False, (1, 5, 1001)),    # generic rows kernel
+    (L.REDUCE_ROWS, True, (1, 256, 192)),    # tile kernel, transposed write
+    (L.REDUCE_ALL, False, (2, 130, 70)),     # tile kernel, one scale per batch entry
+])
+@pytest.mark.parametrize('noise,out', [(L.NOISE_JAX_UNIFORM, L.I8), (L.NOISE_FP8_MANTISSA, L.E5M2)])
+def test_key_in_device_memory_equals_key_in_the_plan(gpu, reduce, transpose, shape, noise, out):
+  """plan.key_device: the kernels read the two key words from device memory (the form a traced
+  jax key arrives in under XLA); same bits as the key given by value."""
+  x = U.to_dev(U.rand(shape, 'bf16', seed=7, scale=0.5), 'bf16', gpu)
+  key = prng.prng_key(4321)
+  qb, cb = (127.5, 127.0) if out == L.I8 else (57344.0, 57344.0)
+  kw = dict(reduce=reduce, out_dtype=out, quant_bound=qb, clip_bound=cb, noise=noise, transpose_out=transpose)
+  q0, s0 = ops.quantize(x, key=key, **kw)
+  kd = torch.tensor([int(key[0]), int(key[1])], dtype=torch.int64).to(torch.int32).to(gpu) if max(key) < 2**31 else \
+      torch.from_numpy(np.asarray(key, dtype=np.uint32).view(np.int32).copy()).to(gpu)
+  q1, s1 = ops.quantize(x, key_device=kd, **kw)
+  assert torch.equal(q0, q1) and torch.equal(s0, s1)
+  # and a different key gives different bits (the device key is really what is read)
+  kd2 = kd.clone()
+  kd2[1] += 1
+  q2, _ = ops.quantize(x, key_device=kd2, **kw)
+  assert not torch.equal(q0, q2)
