@@ -361,7 +361,7 @@ template <int MB, int NB, int D, bool PACKED>
 __global__ __launch_bounds__(256, (D * (NB + MB * (PACKED ? 2 : 1)) * 4 + MB * NB * 4 + 48 > 256) ? 1 : 2)
 void decode_tile_kernel(const DecodeArgs d) {
   constexpr int T = MB * NB;
-  static_assert(T % 4 == 0, "a thread owns whole 16x16 tiles after the reduction");
+  constexpr int TPW = (T + 3) / 4;  // 16x16 tiles a wave owns after the reduction: t = wave + 4*j < T
   __shared__ v4i red[4][T][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -394,13 +394,13 @@ void decode_tile_kernel(const DecodeArgs d) {
 
   // The scales of the outputs this thread will dequantize at the end (tiles t = wave + 4*j: weight
   // block t % NB is the same for all of them), requested now so that they are long there by then.
-  float ws[4], xs[T / 4];
+  float ws[4], xs[TPW];
   {
-    const int nn = n0 + (wave % NB) * 16 + 4 * c;
+    const int nn = n0 + (wave % NB) * 16 + 4 * c;  // (wave + 4*j) % NB == wave % NB: NB divides 4
 #pragma unroll
     for (int e = 0; e < 4; ++e) ws[e] = d.w_scale[(nn + e) < d.n ? (nn + e) : (d.n - 1)];
 #pragma unroll
-    for (int j = 0; j < T / 4; ++j) {
+    for (int j = 0; j < TPW; ++j) {
       const int mm = ((wave + 4 * j) / NB) * 16 + r;
       xs[j] = d.x_scale[mm < d.m ? mm : (d.m - 1)];
     }
@@ -476,14 +476,15 @@ void decode_tile_kernel(const DecodeArgs d) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) red[wave][mb * NB + nb][lane] = acc[mb][nb];
   __syncthreads();
-  // thread -> the lane's four words of tiles t = wave + 4*j, j = 0..T/4-1
+  // thread -> the lane's four words of tiles t = wave + 4*j < T
   int* tile_sums = d.sums + (int64_t)blockIdx.x * (T * 4 * 64);
   const int one = 1 << d.count_shift, half = one >> 1;
   const bool wide_ok = (d.n % 4) == 0;  // 4 consecutive outputs of a row are then 8 / 16-byte aligned
   const int p1 = d.out_bf16 & d.xs_bf16;
 #pragma unroll
-  for (int j = 0; j < T / 4; ++j) {
+  for (int j = 0; j < TPW; ++j) {
     const int t = wave + 4 * j;
+    if (T % 4 != 0 && t >= T) break;  // fewer tiles than waves: the other waves are done (uniform per wave)
     v4i total = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
     bool last[4] = {true, true, true, true};
     if (d.splits > 1) {
@@ -576,19 +577,23 @@ struct TileShape {
 };
 
 // plan->tuning, all fields 0 = the library's choice:
-//   bits 0-7 K ranges per weight tile, bits 8-11 nb (2 | 4), bits 12-15 K steps in flight per
-//   wave (2 | 4), bits 16-19 path (1 = one or two tokens take the path of three and more)
+//   bits 0-7 K ranges per weight tile, bits 8-11 nb (1 | 2 | 4), bits 12-15 K steps in flight
+//   per wave (2 | 4 | 8 | 15 for 16), bits 16-19 path (1 = one or two tokens take the path of three and more)
 TileShape choose_tile_shape(const aqtx_decode_plan* p) {
   TileShape t{};
   const int tune = p->tuning;
   const bool packed = p->w_dtype == AQTX_I4P;
   const int ks = packed ? 128 : 64;
   t.mb = p->m <= 16 ? 1 : p->m <= 32 ? 2 : 4;
-  // About one workgroup per CU (256): weight tiles of 64 rows when the weight has enough rows for
-  // that, else of 32 rows; whatever is still missing comes from splitting K, which costs
-  // exchange traffic in proportion to m * n * K ranges.
-  t.nb = ((tune >> 8) & 15) ? ((tune >> 8) & 15) : ((p->n + 63) / 64 >= 192 ? 4 : 2);
-  if ((t.nb != 2 && t.nb != 4) || t.mb == 1) t.nb = 4;  // mb * nb must be a multiple of 4
+  // About one workgroup per CU (256): the tallest weight tile (64, 32 or 16 rows) that still gives
+  // 192 tiles or more (a taller tile re-reads the activations less often); whatever is then
+  // still missing comes from splitting K, which costs exchange traffic in proportion to
+  // m * n * K ranges.  Measured at k = 4096: n = 4096 is fastest with 16-row tiles and no split,
+  // n = 14336 with 64-row tiles and no split.
+  int nb_auto = 4;
+  while (nb_auto > 1 && (p->n + 16 * nb_auto - 1) / (16 * nb_auto) < 192) nb_auto /= 2;
+  t.nb = ((tune >> 8) & 15) ? ((tune >> 8) & 15) : nb_auto;
+  if (t.nb != 1 && t.nb != 2 && t.nb != 4) t.nb = nb_auto;
   t.ntiles = (int)((p->n + 16 * t.nb - 1) / (16 * t.nb));
   // An exchange word holds count * 2^shift + sum with |sum| <= k * 127 * 128 < 2^(shift - 1).
   int magnitude_bits = 1;
@@ -607,9 +612,11 @@ TileShape choose_tile_shape(const aqtx_decode_plan* p) {
   t.splits = (int)((p->k + k_slice - 1) / k_slice);
   const int steps = k_slice / (4 * ks);
   const int loads_per_step = t.nb + t.mb * (packed ? 2 : 1);
-  t.depth = ((tune >> 12) & 15) ? ((tune >> 12) & 15) : ((steps >= 4 && t.mb == 1) ? 4 : 2);
-  if (t.depth != 2 && t.depth != 4) t.depth = 4;
+  t.depth = ((tune >> 12) & 15) ? ((tune >> 12) & 15) : ((steps >= 4 && (t.mb == 1 || t.nb == 1)) ? 4 : 2);
+  if (t.depth == 15) t.depth = 16;  // the 4-bit field cannot say 16
+  if (t.depth != 2 && t.depth != 4 && t.depth != 8 && t.depth != 16) t.depth = 4;
   while (t.depth > 2 && t.depth * loads_per_step > 64) t.depth /= 2;  // 256 registers of operands in flight
+  while (t.depth > 2 && t.depth > steps) t.depth /= 2;                // steps past the range are wasted issue slots
   if (t.splits > 1) t.sums_bytes = (size_t)t.ntiles * t.mb * t.nb * 1024;
   return t;
 }
@@ -624,13 +631,22 @@ template <bool PACKED>
 int launch_tile(const TileShape& t, const DecodeArgs& d, hipStream_t st) {
   const dim3 grid((unsigned)t.ntiles, (unsigned)t.splits);
 #define AQTX_TILE(MB, NB, D) decode_tile_kernel<MB, NB, D, PACKED><<<grid, 256, 0, st>>>(d)
-#define AQTX_TILE_D(MB, NB)                         \
-  do {                                              \
-    if (t.depth == 2) AQTX_TILE(MB, NB, 2);         \
-    else AQTX_TILE(MB, NB, 4);                      \
+  // depths whose operands in flight fit the register file: (nb + mb * halves) * depth <= 64 loads
+#define AQTX_TILE_D(MB, NB)                                                          \
+  do {                                                                               \
+    constexpr int kLoads = NB + MB * (PACKED ? 2 : 1);                               \
+    if constexpr (kLoads * 16 <= 64) { if (t.depth == 16) { AQTX_TILE(MB, NB, 16); break; } } \
+    if constexpr (kLoads * 8 <= 64) { if (t.depth >= 8) { AQTX_TILE(MB, NB, 8); break; } }    \
+    if (t.depth >= 4 && kLoads * 4 <= 64) { AQTX_TILE(MB, NB, 4); break; }           \
+    AQTX_TILE(MB, NB, 2);                                                            \
   } while (0)
-#define AQTX_TILE_N(MB) do { if (t.nb == 2) AQTX_TILE_D(MB, 2); else AQTX_TILE_D(MB, 4); } while (0)
-  if (t.mb == 1) AQTX_TILE_D(1, 4);
+#define AQTX_TILE_N(MB)                         \
+  do {                                          \
+    if (t.nb == 1) AQTX_TILE_D(MB, 1);          \
+    else if (t.nb == 2) AQTX_TILE_D(MB, 2);     \
+    else AQTX_TILE_D(MB, 4);                    \
+  } while (0)
+  if (t.mb == 1) AQTX_TILE_N(1);
   else if (t.mb == 2) AQTX_TILE_N(2);
   else AQTX_TILE_N(4);
 #undef AQTX_TILE_N

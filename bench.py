@@ -265,6 +265,47 @@ def other_configs(dev):
   return out
 
 
+def gemm_probe(dev, data, reps=10):
+  """The three contractions of a step on their own, on synthetic int8 operands of a chosen value
+  distribution (the MFMA rate of this part depends on the operand values: the chip lowers its
+  clock when more datapath bits toggle), next to the vendor library's int8 GEMM (torch._int_mm,
+  raw int32 output) on the same operands.  For counter runs (rocprofv3 --pmc) and the
+  data-dependence table; prints one JSON line."""
+  import torch
+  from aqt_amd import ops
+  gens = {
+      'zeros': lambda s: torch.zeros(s, dtype=torch.int8, device=dev),
+      'normal25': lambda s: (torch.randn(s, device=dev) * 25).clamp(-127, 127).round().to(torch.int8),
+      'uniform': lambda s: torch.randint(-127, 128, s, dtype=torch.int8, device=dev),
+  }
+  gen = gens[data]
+
+  def timed(f):
+    for _ in range(3):
+      f()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+      f()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+  rows = {}
+  for shape, (m, n, k) in (('fwd', (M, N, K)), ('dlhs', (M, K, N)), ('drhs', (K, N, M))):
+    a, b = gen((1, m, k)), gen((1, n, k))
+    rs, cs = torch.rand(1, m, device=dev), torch.rand(1, n, device=dev)
+    ms = timed(lambda: ops.gemm(a, b, row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16))
+    bt = b[0].t().contiguous()  # the library takes the second operand [k, n]
+    ms_lib = timed(lambda: torch._int_mm(a[0], bt))
+    ops_ = 2.0 * m * n * k
+    rows[shape] = {'m': m, 'n': n, 'k': k, 'aqtx_gemm_i8_us': round(ms * 1e3, 1), 'aqtx_TOPS': round(ops_ / ms / 1e9),
+                   'library_int_mm_us': round(ms_lib * 1e3, 1), 'library_TOPS': round(ops_ / ms_lib / 1e9)}
+    del a, b, bt
+  print(json.dumps({'gemm_probe': data, 'reps': reps, 'shapes': rows}))
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--gpus', type=int, default=1)
@@ -277,6 +318,9 @@ def main():
   ap.add_argument('--calibration-copy', action='store_true',
                   help='also launch one elementwise kernel that reads and writes 256 MiB, as the '
                        'known-size reference for FETCH_SIZE / WRITE_SIZE counter runs')
+  ap.add_argument('--gemm-probe', choices=['zeros', 'normal25', 'uniform'], default=None,
+                  help='only run the three int8 contractions of a step on operands of this value '
+                       'distribution (and the vendor int8 GEMM beside them) and exit')
   args = ap.parse_args()
   if args.gpus != 1:
     print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)',
@@ -291,6 +335,9 @@ def main():
     print('bench.py needs a GPU', file=sys.stderr)
     sys.exit(1)
   dev = torch.device('cuda:0')
+  if args.gemm_probe is not None:
+    gemm_probe(dev, args.gemm_probe)
+    return
   lhs, rhs, g = make_inputs(dev)
   lhs.requires_grad_(True)
   rhs.requires_grad_(True)
@@ -336,7 +383,8 @@ def main():
                    'launch_ms': gemm_ms, 'launches_timed': len(timer.pairs)},
   }
   if not args.no_decode:
-    line['decode'] = {'kernel': 'aqtx_decode_i8 (quant_rows + decode_ksplit/decode_block)', 'k': 4096,
+    line['decode'] = {'kernel': 'aqtx_decode_i8 (m <= 2: decode_fused_kernel; m >= 3: decode_quant_kernel + decode_tile_kernel)',
+                      'k': 4096,
                       'timing': 'HIP graph replay, weights rotated through 1 GiB', 'shapes': decode_bench(dev)}
   if not args.no_other_configs:
     del lhs, rhs, g

@@ -291,7 +291,8 @@ typedef struct aqtx_decode_plan {
   int32_t w_dtype;        /* AQTX_I8 | AQTX_I4 (container) | AQTX_I4P (packed: k multiple of 32) */
   int32_t tuning;         /* 0 = the library chooses the launch shape.  Tuning only (results never
                              depend on it): bits 0-7 K ranges per weight tile, bits 8-11 16-row weight
-                             blocks per wave (2 | 4), bits 12-15 K steps in flight per wave (2 | 4),
+                             blocks per wave (1 | 2 | 4), bits 12-15 K steps in flight per wave (2 | 4 |
+                             8 | 15 = 16; capped by the register file),
                              bits 16-19 path: 1 = one or two tokens take the path of three and more  */
   int32_t workspace_zeroed; /* 1: the caller keeps one workspace across calls on one stream and its first
                              aqtx_decode_exchange_bytes(plan) bytes were zero before the first call.

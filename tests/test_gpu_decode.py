@@ -145,3 +145,92 @@ def test_decode_one_or_two_rows_long_k(gpu, m, k, dt, w_sdt):
   out2, _ = ops.decode(U.to_dev(x, dt, gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
                        quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt])
   assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('m,n,k', [(5, 200, 464 + 16), (24, 1000, 2048), (64, 520, 4096), (40, 4096, 1024)])
+def test_decode_every_launch_shape_gives_the_same_bits(gpu, packed, m, n, k):
+  """plan.tuning only chooses the launch shape (rows per weight tile, K ranges per tile that meet
+  through the int32 atomic exchange, K steps in flight): every choice must return the oracle's
+  bits, and so must the one- and two-token kernel's arithmetic when m <= 2 is sent down the
+  two-kernel path."""
+  from aqt_amd import _lib as L
+  if packed:
+    k = (k + 31) // 32 * 32
+  x = U.rand((m, k), 'bf16', 400 + m, outliers=True)
+  rng = np.random.default_rng(13)
+  lim = 7 if packed else 127
+  wq = rng.integers(-lim, lim + 1, size=(n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(2e-4) + np.float32(1e-5), 'f32')
+  want, xq_want, xs_want = _oracle_decode(x, 'bf16', wq, ws, 'f32')
+  w_t = torch.from_numpy(wq).to(gpu)
+  if packed:
+    w_t = ops.pack_i4(w_t)
+  for splits in (1, 2, 3, 7):
+    for nb in (1, 2, 4):
+      for depth in (2, 4, 15):
+        tuning = splits | (nb << 8) | (depth << 12)
+        out, xs, xq = ops.decode(U.to_dev(x, 'bf16', gpu), w_t, torch.from_numpy(ws).to(gpu), quant_bound=127.5,
+                                 clip_bound=127.0, want_xq=True, w_dtype=L.I4P if packed else L.I8, tuning=tuning)
+        np.testing.assert_array_equal(out.float().cpu().numpy(), want, err_msg=hex(tuning))
+        np.testing.assert_array_equal(xq.cpu().numpy(), xq_want, err_msg=hex(tuning))
+        np.testing.assert_array_equal(xs.cpu().numpy(), xs_want, err_msg=hex(tuning))
+
+
+@pytest.mark.parametrize('m', [1, 2])
+def test_decode_two_kernel_path_for_one_or_two_tokens(gpu, m):
+  n, k = 328, 2048
+  x = U.rand((m, k), 'bf16', 500 + m, outliers=True)
+  wq, ws = _weights(n, k, 14, 'f32')
+  want, xq_want, xs_want = _oracle_decode(x, 'bf16', wq, ws, 'f32')
+  out, xs, xq = ops.decode(U.to_dev(x, 'bf16', gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
+                           quant_bound=127.5, clip_bound=127.0, want_xq=True, tuning=1 << 16)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+  np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
+  np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
+
+
+def test_decode_workspace_contract(gpu):
+  """A caller-owned workspace with arbitrary contents (workspace_zeroed = 0) and one kept zeroed
+  across calls of different shapes (workspace_zeroed = 1) give the same bits; the exchange words
+  are zero again after every call."""
+  import ctypes
+  from aqt_amd import _lib as L
+  shapes = [(64, 4096, 512), (8, 136, 8192), (33, 1000, 1024), (64, 264, 4096)]
+  plans = []
+  for m, n, k in shapes:
+    p = L.DecodePlan()
+    p.m, p.n, p.k = m, n, k
+    p.x_dtype = p.x_scale_dtype = p.out_dtype = L.BF16
+    p.w_scale_dtype = L.F32
+    p.quant_bound, p.clip_bound, p.w_dtype = 127.5, 127.0, L.I8
+    p.tuning = 3 | (2 << 8)  # three K ranges per tile: the exchange is in use for every shape
+    plans.append(p)
+  lib = L.lib()
+  ex = max(int(lib.aqtx_decode_exchange_bytes(ctypes.byref(p))) for p in plans)
+  rest = max(int(lib.aqtx_decode_workspace_bytes(ctypes.byref(p))) - int(lib.aqtx_decode_exchange_bytes(ctypes.byref(p)))
+             for p in plans)
+  kept = torch.zeros(ex + rest, dtype=torch.uint8, device=gpu)
+  ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+  st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+  for p, (m, n, k) in zip(plans, shapes):
+    x = U.to_dev(U.rand((m, k), 'bf16', 600 + m), 'bf16', gpu)
+    wq, ws = _weights(n, k, 15, 'f32')
+    w_t, ws_t = torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu)
+    outs = []
+    for zeroed in (0, 1):
+      p.workspace_zeroed = zeroed
+      if zeroed:
+        wsp = kept
+      else:
+        wsp = torch.randint(0, 256, (int(lib.aqtx_decode_workspace_bytes(ctypes.byref(p))),), dtype=torch.uint8, device=gpu)
+      out = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+      xs = torch.empty(m, dtype=torch.float32, device=gpu)
+      L.check(lib.aqtx_decode_i8(ctypes.byref(p), ptr(x), ptr(w_t), ptr(ws_t), None, ptr(xs), ptr(out), ptr(wsp),
+                                 wsp.numel(), st))
+      outs.append(out)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]), (m, n, k)
+    assert int(kept[:ex].max()) == 0, 'exchange words were left non-zero'
+    want, _, _ = _oracle_decode(U.rand((m, k), 'bf16', 600 + m), 'bf16', wq, ws, 'f32')
+    np.testing.assert_array_equal(outs[1].float().cpu().numpy(), want)
