@@ -15,6 +15,7 @@ REDUCE_COLS, REDUCE_ROWS, REDUCE_ALL, REDUCE_ALL_BATCH = range(4)
 NOISE_NONE, NOISE_JAX_UNIFORM, NOISE_CUSTOM1, NOISE_FP8_MANTISSA = range(4)
 PRESCALE_NONE, PRESCALE_PER_ROW, PRESCALE_PER_COL = range(3)
 SCALE_ROW_THEN_COL, SCALE_COL_THEN_ROW = range(2)
+W_ROWS, W_FRAGMENTS = range(2)
 
 
 class QuantPlan(ctypes.Structure):
@@ -67,7 +68,8 @@ class DecodePlan(ctypes.Structure):
       ('x_dtype', ctypes.c_int32), ('x_scale_dtype', ctypes.c_int32),
       ('w_scale_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
       ('quant_bound', ctypes.c_float), ('clip_bound', ctypes.c_float),
-      ('w_dtype', ctypes.c_int32), ('tuning', ctypes.c_int32), ('workspace_zeroed', ctypes.c_int32),
+      ('w_dtype', ctypes.c_int32), ('tuning', ctypes.c_int32), ('w_layout', ctypes.c_int32),
+      ('workspace_zeroed', ctypes.c_int32),
   ]
 
 
@@ -104,6 +106,8 @@ SYMBOLS = {
                                       _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
     'aqtx_decode_exchange_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
+    'aqtx_tile_weight_bytes': (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int32]),
+    'aqtx_tile_weight': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),
     'aqtx_decode_i8_static': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8_grouped': (ctypes.c_int, [ctypes.POINTER(GroupedGemmPlan), _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_pack_i4': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, _vp]),

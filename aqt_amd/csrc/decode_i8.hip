@@ -49,6 +49,12 @@ struct DecodeArgs {
   int8_t* xq_frag;
   int mb_total;           // 16-token blocks
   int frag_halves;        // 1 | 2
+  // Weight layout.  Rows: [n][k bytes], a wave's load is 16 rows x 64 bytes.  Fragments
+  // (aqtx_tile_weight): [16-row block][64-byte k step][1 KiB], the KiB holding for lane
+  // (r = row in the block, c = 16-byte quarter) its operand bytes at (c*16 + r)*16, so that a
+  // wave's load is one contiguous KiB; rows past n and bytes past the row end are zero.
+  int w_frag;             // 1: fragment order
+  int w_steps;            // fragment order: 64-byte steps of one row block
 };
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
@@ -92,7 +98,9 @@ __device__ __forceinline__ void unpack_i4x8(uint32_t w, int& lo, int& hi) {
 // LDS rows are k rounded up to 256 bytes long; the 16-byte piece j of row i sits at piece
 // j ^ (i & 15) of its 16-piece group, so the 16 lanes of a fragment read hit all 64 banks.
 // PACKED: int4 weights two per byte; a lane's 16 bytes are then 32 k, i.e. two MFMA steps.
-template <typename TIn, int ROWS, int PPT, int U, bool PACKED>  // PPT: 16-value pieces of one row per thread
+// WFRAG: the weight is in fragment order (compile-time here: the offsets of all U loads of a
+// batch are then constants off one base register).
+template <typename TIn, int ROWS, int PPT, int U, bool PACKED, bool WFRAG>  // PPT: 16-value pieces of one row per thread
 __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xlds[];  // [ROWS][kp]
   __shared__ float smax[ROWS][4];
@@ -111,12 +119,14 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   constexpr int KS = PACKED ? 128 : 64;   // k covered by one wave-wide weight load
   constexpr int KL = KS / 4;              // k covered by one lane's 16 bytes
   const int kb = PACKED ? d.k / 2 : d.k;  // bytes of one weight row
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * kb);
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, d.w_frag ? (int64_t)((d.n + 15) / 16) * d.w_steps * 1024 : (int64_t)d.n * kb);
   const int kq = ((d.k + 3) / 4 + KS - 1) / KS * KS;
   const int k_lo = wave * kq;
   const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
-  const int wbase = nrow * kb + c * 16;
-  auto w_offset = [&](int ko) { return (ko + c * KL < k_hi) ? wbase + (PACKED ? ko / 2 : ko) : kOob; };
+  // byte offset of the lane's 16 bytes of k step 0, and what one k step adds to it
+  const int wbase = WFRAG ? (int)blockIdx.x * d.w_steps * 1024 + lane * 16 : nrow * kb + c * 16;
+  constexpr int wstep = WFRAG ? 1024 : 64;
+  auto w_offset = [&](int ko) { return (ko + c * KL < k_hi) ? wbase + (ko / KS) * wstep : kOob; };
 
   // first batch of weights: in flight while the activations are quantized
   v4i wf[U];
@@ -377,13 +387,14 @@ void decode_tile_kernel(const DecodeArgs d) {
   const int k_lo = s_lo + wave * kq;
   const int k_hi = (k_lo + kq) < s_hi ? (k_lo + kq) : s_hi;
 
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, (int64_t)d.n * kb);
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, d.w_frag ? (int64_t)((d.n + 15) / 16) * d.w_steps * 1024 : (int64_t)d.n * kb);
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.xq_frag, (int64_t)((d.k + KS - 1) / KS) * d.mb_total * XP * 1024);
   int wbase[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int row = n0 + nb * 16 + r;
-    wbase[nb] = (row < d.n ? row : d.n - 1) * kb + c * 16;  // clamped; such columns are never stored
+    wbase[nb] = d.w_frag ? (int)(blockIdx.x * NB + nb) * d.w_steps * 1024 + lane * 16  // past n: reads zeros
+                         : (row < d.n ? row : d.n - 1) * kb + c * 16;  // clamped; such columns are never stored
   }
 
   v4i acc[MB][NB];
@@ -406,6 +417,7 @@ void decode_tile_kernel(const DecodeArgs d) {
     }
   }
 
+  const unsigned wstep = d.w_frag ? 1024u : 64u;
   v4i wf[D][NB], xf[D][MB][XP];
   // Steps past the end of the wave's range, lanes past the end of K and token blocks past m read
   // zeros: their offsets get the out-of-range bits ORed in (no memory access; no branch, which
@@ -415,7 +427,7 @@ void decode_tile_kernel(const DecodeArgs d) {
   for (int mb = 0; mb < MB; ++mb) xdead[mb] = mb < d.mb_total ? 0u : (unsigned)kOob;
   auto issue = [&](int slot, int ko) {
     const unsigned dead = (ko + c * KL < k_hi) ? 0u : (unsigned)kOob;  // a lane's KL values are all inside or all outside
-    const unsigned wk = (unsigned)(PACKED ? ko / 2 : ko);
+    const unsigned wk = (unsigned)(ko / KS) * wstep;  // a k step is 64 bytes of a row, or one KiB fragment
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       wf[slot][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)(((unsigned)wbase[nb] + wk) | dead), 0, 0);
@@ -538,6 +550,22 @@ void decode_tile_kernel(const DecodeArgs d) {
   }
 }
 
+// Weight rows -> fragment order (see DecodeArgs): thread -> (16-row block, 64-byte k step, lane).
+__global__ __launch_bounds__(256) void tile_weight_kernel(const uint8_t* src, uint8_t* dst, int n, int kb, int steps) {
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one 16-byte piece each
+  const int64_t frag = id >> 6;
+  const int lane = (int)(id & 63);
+  const int64_t blk = frag / steps;
+  const int step = (int)(frag % steps);
+  if (blk * 16 >= n) return;
+  const int r = lane & 15, c = lane >> 4;
+  const int64_t row = blk * 16 + r;
+  const int byte = step * 64 + c * 16;
+  uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (row < n && byte < kb) v = *reinterpret_cast<const uint4*>(src + row * kb + byte);
+  *reinterpret_cast<uint4*>(dst + id * 16) = v;
+}
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 int validate_decode(const aqtx_decode_plan* p) {
@@ -556,6 +584,10 @@ int validate_decode(const aqtx_decode_plan* p) {
                    is_float_dtype(p->w_scale_dtype) && is_float_dtype(p->out_dtype),
                "aqtx_decode_i8: dtypes must be bf16 or f32");
   AQTX_REQUIRE(p->quant_bound > 0.0f && p->clip_bound > 0.0f, "aqtx_decode_i8: bounds must be positive");
+  AQTX_REQUIRE(p->w_layout == AQTX_W_ROWS || p->w_layout == AQTX_W_FRAGMENTS, "aqtx_decode_i8: unknown w_layout %d",
+               p->w_layout);
+  AQTX_REQUIRE(p->w_layout == AQTX_W_ROWS || (p->n + 15) / 16 * ((p->k + 63) / 64) * 1024 < (1ll << 31) - 64,
+               "aqtx_decode_i8: fragment-ordered weight larger than 2 GiB");
   return 0;
 }
 
@@ -707,6 +739,8 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
   d.x = x; d.x_scale_out = x_scale;
   d.quant_bound = p->quant_bound; d.clip_bound = p->clip_bound; d.x_bf16 = xbf;
   d.acc_shift = pk ? 4 : 0;
+  d.w_frag = p->w_layout == AQTX_W_FRAGMENTS;
+  d.w_steps = (int)(((pk ? p->k / 2 : p->k) + 63) / 64);
 
   // One or two tokens: one kernel quantizes and contracts.  Every workgroup repeats the
   // quantisation, so its cost grows with the rows while the launch it saves does not: measured at
@@ -718,9 +752,14 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
     const unsigned grid = (unsigned)((p->n + 15) / 16);
     const int rows = (int)p->m;
     const size_t lds = (size_t)rows * (size_t)((p->k + 255) / 256 * 256);
-#define AQTX_FUSED(T, R, P)                                                   \
-  if (pk) decode_fused_kernel<T, R, P, 8, true><<<grid, 256, lds, st>>>(d);  \
-  else decode_fused_kernel<T, R, P, 16, false><<<grid, 256, lds, st>>>(d);
+#define AQTX_FUSED(T, R, P)                                                                       \
+  if (d.w_frag) {                                                                                 \
+    if (pk) decode_fused_kernel<T, R, P, 8, true, true><<<grid, 256, lds, st>>>(d);              \
+    else decode_fused_kernel<T, R, P, 16, false, true><<<grid, 256, lds, st>>>(d);               \
+  } else {                                                                                        \
+    if (pk) decode_fused_kernel<T, R, P, 8, true, false><<<grid, 256, lds, st>>>(d);             \
+    else decode_fused_kernel<T, R, P, 16, false, false><<<grid, 256, lds, st>>>(d);              \
+  }
     if (xbf) {
       if (ppt == 1) { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 1) } else { AQTX_FUSED(uint16_t, 2, 1) } }
       else { if (rows == 1) { AQTX_FUSED(uint16_t, 1, 2) } else { AQTX_FUSED(uint16_t, 2, 2) } }
@@ -823,4 +862,30 @@ extern "C" int aqtx_decode_i8_static(const aqtx_decode_plan* p, const void* x, c
   aqtx_decode_plan plan = *p;
   plan.workspace_zeroed = 0;
   return decode_impl(&plan, x, w, w_scale, xq, x_scale, out, ws, kStaticScratchBytes, stream);
+}
+
+extern "C" size_t aqtx_tile_weight_bytes(int64_t n, int64_t k, int32_t w_dtype) {
+  if (n <= 0 || k <= 0) return 0;
+  const int64_t kb = w_dtype == AQTX_I4P ? k / 2 : k;
+  return (size_t)((n + 15) / 16) * (size_t)((kb + 63) / 64) * 1024;
+}
+
+extern "C" int aqtx_tile_weight(const void* src, void* dst, int64_t n, int64_t k, int32_t w_dtype, void* stream) {
+  clear_error();
+  AQTX_REQUIRE(w_dtype == AQTX_I8 || w_dtype == AQTX_I4 || w_dtype == AQTX_I4P,
+               "aqtx_tile_weight: w_dtype must be int8, int4 in int8 containers or packed int4");
+  AQTX_REQUIRE(n >= 0 && k >= 0, "aqtx_tile_weight: negative shape");
+  const int64_t kmul = w_dtype == AQTX_I4P ? 32 : 16;
+  AQTX_REQUIRE(k % kmul == 0, "aqtx_tile_weight: k = %lld must be a multiple of %lld", (long long)k, (long long)kmul);
+  if (n == 0 || k == 0) return 0;
+  AQTX_REQUIRE(src != nullptr && dst != nullptr, "aqtx_tile_weight: NULL buffer");
+  AQTX_REQUIRE(((uintptr_t)src % 16) == 0 && ((uintptr_t)dst % 16) == 0, "aqtx_tile_weight: buffers must be 16-byte aligned");
+  const int64_t kb = w_dtype == AQTX_I4P ? k / 2 : k;
+  const int64_t steps = (kb + 63) / 64;
+  const int64_t pieces = (n + 15) / 16 * steps * 64;
+  AQTX_REQUIRE(pieces / 256 + 1 < (1ll << 31), "aqtx_tile_weight: weight too large for one launch");
+  tile_weight_kernel<<<dim3((unsigned)((pieces + 255) / 256)), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint8_t*>(src), reinterpret_cast<uint8_t*>(dst), (int)n, (int)kb, (int)steps);
+  AQTX_HIP_CHECK_LAUNCH("tile_weight_kernel");
+  return 0;
 }

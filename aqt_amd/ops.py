@@ -313,7 +313,7 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
 
 def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
            clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False,
-           w_dtype: int = L.I8, tuning: int = 0, static_scratch: bool = False):
+           w_dtype: int = L.I8, tuning: int = 0, static_scratch: bool = False, w_layout: int = L.W_ROWS):
   """Serving contraction out = dequant(quant(x) @ w_q^T) for x [m <= 64, k], w_q int8 [n, k], or
   uint8 [n, k/2] holding packed int4 (w_dtype=I4P, the pack_i4 layout).
 
@@ -325,10 +325,15 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   """
   _require_gpu(x, w_q, w_scale)
   packed = w_dtype == L.I4P
-  assert x.dim() == 2 and w_q.dim() == 2 and x.shape[1] == w_q.shape[1] * (2 if packed else 1), (x.shape, w_q.shape)
-  assert x.is_contiguous() and w_q.is_contiguous() and w_q.dtype == (torch.uint8 if packed else torch.int8)
+  assert x.dim() == 2 and x.is_contiguous() and w_q.is_contiguous()
   m, k = x.shape
-  n = w_q.shape[0]
+  if w_layout == L.W_FRAGMENTS:  # the output of tile_weight: a flat buffer; n is the number of scales
+    n = w_scale.numel()
+    assert w_q.numel() * w_q.element_size() == L.lib().aqtx_tile_weight_bytes(n, k, w_dtype), (w_q.shape, n, k)
+  else:
+    assert w_q.dim() == 2 and k == w_q.shape[1] * (2 if packed else 1), (x.shape, w_q.shape)
+    assert w_q.dtype == (torch.uint8 if packed else torch.int8)
+    n = w_q.shape[0]
   assert w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() == n
   plan = L.DecodePlan()
   plan.m, plan.n, plan.k = m, n, k
@@ -339,6 +344,7 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   plan.quant_bound, plan.clip_bound = float(quant_bound), float(clip_bound)
   plan.w_dtype = w_dtype
   plan.tuning = tuning  # launch-shape override for measurements; results do not depend on it
+  plan.w_layout = w_layout
   if static_scratch:
     out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     x_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
@@ -363,6 +369,18 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
     _QUANT_WS.clear()  # a failed launch sequence may have left partial sums behind
     raise
   return (out, x_scale, xq) if want_xq else (out, x_scale)
+
+
+def tile_weight(w_q: torch.Tensor, w_dtype: int = L.I8) -> torch.Tensor:
+  """A frozen weight [n, k] (int8, or packed int4 uint8 [n, k/2]) in MFMA fragment order: the layout
+  decode(..., w_layout=W_FRAGMENTS) streams fastest.  Returns a flat uint8 buffer."""
+  _require_gpu(w_q)
+  packed = w_dtype == L.I4P
+  assert w_q.dim() == 2 and w_q.is_contiguous() and w_q.dtype == (torch.uint8 if packed else torch.int8)
+  n, k = w_q.shape[0], w_q.shape[1] * (2 if packed else 1)
+  out = torch.empty(int(L.lib().aqtx_tile_weight_bytes(n, k, w_dtype)), dtype=torch.uint8, device=w_q.device)
+  L.check(L.lib().aqtx_tile_weight(_ptr(w_q), _ptr(out), n, k, w_dtype, _stream()))
+  return out
 
 
 def pack_i4(q: torch.Tensor) -> torch.Tensor:

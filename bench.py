@@ -81,7 +81,9 @@ def decode_bench(dev):
   from aqt_amd import ops
   k = 4096
   rows = []
-  for w_kind in ('int8', 'int4_packed'):
+  # weights in this library's serving format (MFMA fragment order, what a frozen layer keeps) and,
+  # for int8, also as plain rows [n][k] (what a caller holding the reference's layout passes)
+  for w_kind, layout in (('int8', 'fragments'), ('int4_packed', 'fragments'), ('int8', 'rows')):
     packed = w_kind == 'int4_packed'
     wbytes_per = 0.5 if packed else 1.0
     for n in (4096, 14336):
@@ -92,6 +94,9 @@ def decode_bench(dev):
         weights = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(ncopies)]
       w_scale = torch.rand(n, device=dev) * 1e-3 + 1e-5
       kw = dict(quant_bound=127.5, clip_bound=127.0, w_dtype=L.I4P if packed else L.I8)
+      if layout == 'fragments':
+        weights = [ops.tile_weight(w, kw['w_dtype']) for w in weights]
+        kw['w_layout'] = L.W_FRAGMENTS
       for m in (1, 8, 32, 64):
         x = torch.randn(m, k, device=dev).to(torch.bfloat16)
         run = lambda: [ops.decode(x, w, w_scale, **kw) for w in weights]
@@ -116,7 +121,7 @@ def decode_bench(dev):
         torch.cuda.synchronize()
         us = a.elapsed_time(b) * 1e3 / (reps * ncopies)
         nbytes = int(k * n * wbytes_per) + 4 * n + 2 * m * k + 2 * m * n
-        rows.append({'weights': w_kind, 'n': n, 'm': m, 'us_per_call': round(us, 2),
+        rows.append({'weights': w_kind, 'layout': layout, 'n': n, 'm': m, 'us_per_call': round(us, 2),
                      'GB/s': round(nbytes / us / 1e3, 1), 'frac_of_8TBps': round(nbytes / us / 1e3 / 8000.0, 3)})
         del graph, keep
       del weights

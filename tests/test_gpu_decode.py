@@ -234,3 +234,53 @@ def test_decode_workspace_contract(gpu):
     assert int(kept[:ex].max()) == 0, 'exchange words were left non-zero'
     want, _, _ = _oracle_decode(U.rand((m, k), 'bf16', 600 + m), 'bf16', wq, ws, 'f32')
     np.testing.assert_array_equal(outs[1].float().cpu().numpy(), want)
+
+
+def _fragment_order(w_bytes):
+  """numpy statement of the fragment layout: [16-row block][64-byte step][lane = c*16 + r][16 bytes]
+  with lane (r, c) holding bytes [64*step + 16*c, +16) of row 16*block + r, zeros outside."""
+  n, kb = w_bytes.shape
+  nb, ns = (n + 15) // 16, (kb + 63) // 64
+  padded = np.zeros((nb * 16, ns * 64), dtype=np.uint8)
+  padded[:n, :kb] = w_bytes
+  t = padded.reshape(nb, 16, ns, 4, 16)        # block, r, step, c, byte
+  return np.ascontiguousarray(t.transpose(0, 2, 3, 1, 4)).reshape(-1)  # block, step, c, r, byte
+
+
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('n,k', [(16, 64), (200, 480), (4096, 1024), (72, 8192 + 32)])
+def test_tile_weight_layout(gpu, packed, n, k):
+  from aqt_amd import _lib as L
+  rng = np.random.default_rng(21)
+  w = rng.integers(0, 256, size=(n, k // 2 if packed else k)).astype(np.uint8)
+  src = torch.from_numpy(w).to(gpu)
+  got = ops.tile_weight(src if packed else src.view(torch.int8), L.I4P if packed else L.I8)
+  np.testing.assert_array_equal(got.cpu().numpy(), _fragment_order(w))
+
+
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('m', [1, 2, 3, 16, 33, 64])
+@pytest.mark.parametrize('n,k', [(256, 1024), (200, 480), (4096, 4096), (72, 8192)])
+def test_decode_fragment_ordered_weight(gpu, packed, m, n, k):
+  """The weight in fragment order (aqtx_tile_weight) gives the oracle's bits on every path: the
+  one/two-token kernel, 16/32/64-row tiles, K ranges meeting through the exchange."""
+  from aqt_amd import _lib as L
+  if packed:
+    k = (k + 31) // 32 * 32
+  x = U.rand((m, k), 'bf16', 700 + m, outliers=True)
+  rng = np.random.default_rng(22)
+  lim = 7 if packed else 127
+  wq = rng.integers(-lim, lim + 1, size=(n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(2e-4) + np.float32(1e-5), 'f32')
+  want, xq_want, xs_want = _oracle_decode(x, 'bf16', wq, ws, 'f32')
+  w_t = torch.from_numpy(wq).to(gpu)
+  wd = L.I8
+  if packed:
+    w_t, wd = ops.pack_i4(w_t), L.I4P
+  tiled = ops.tile_weight(w_t, wd)
+  for tuning in (0, 2 | (4 << 8), 3 | (1 << 8) | (4 << 12)):
+    out, xs, xq = ops.decode(U.to_dev(x, 'bf16', gpu), tiled, torch.from_numpy(ws).to(gpu), quant_bound=127.5,
+                             clip_bound=127.0, want_xq=True, w_dtype=wd, w_layout=L.W_FRAGMENTS, tuning=tuning)
+    np.testing.assert_array_equal(out.float().cpu().numpy(), want, err_msg=hex(tuning))
+    np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
+    np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
