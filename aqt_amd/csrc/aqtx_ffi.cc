@@ -204,17 +204,20 @@ ffi::Error GemmI8GroupedImpl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffe
 }
 
 // ---- aqtx_decode_i8 -----------------------------------------------------------------------------
-// x [m, k] bf16/f32, w int8 [n, k] (uint8 [n, k/2] when w_dtype = AQTX_I4P), w_scale f32 [n]
+// x [m, k] bf16/f32, w int8 [n, k] (uint8 [n, k/2] when w_dtype = AQTX_I4P; the flat output of
+// aqtx_tile_weight when w_layout = AQTX_W_FRAGMENTS), w_scale f32 [n]
 // -> out [m, n], x_scale f32 [m], xq int8 [m, k], workspace uint8[aqtx_decode_workspace_bytes].
 ffi::Error DecodeI8Impl(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer w, ffi::Buffer<ffi::F32> w_scale,
                         ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::Buffer<ffi::F32>> x_scale,
                         ffi::Result<ffi::Buffer<ffi::S8>> xq, ffi::Result<ffi::Buffer<ffi::U8>> workspace,
                         float quant_bound, float clip_bound, int32_t x_scale_dtype, int32_t w_scale_dtype,
-                        int32_t w_dtype) {
-  auto xd = x.dimensions(), wd = w.dimensions();
-  if (xd.size() != 2 || wd.size() != 2) return Bad("aqtx_decode_i8: x must be [m, k], w [n, k]");
+                        int32_t w_dtype, int32_t w_layout) {
+  auto xd = x.dimensions();
+  if (xd.size() != 2) return Bad("aqtx_decode_i8: x must be [m, k]");
   aqtx_decode_plan p{};
-  p.m = xd[0]; p.k = xd[1]; p.n = wd[0];
+  p.m = xd[0]; p.k = xd[1];
+  p.n = (int64_t)w_scale.element_count();  // a fragment-ordered weight is a flat buffer: n = number of scales
+  p.w_layout = w_layout;
   p.x_dtype = Dtype(x.element_type());
   p.x_scale_dtype = x_scale_dtype;
   p.w_scale_dtype = w_scale_dtype;
@@ -336,7 +339,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Ret<ffi::Buffer<ffi::S8>>()     // xq
         .Ret<ffi::Buffer<ffi::U8>>()     // workspace
         .Attr<float>("quant_bound").Attr<float>("clip_bound").Attr<int32_t>("x_scale_dtype")
-        .Attr<int32_t>("w_scale_dtype").Attr<int32_t>("w_dtype"));
+        .Attr<int32_t>("w_scale_dtype").Attr<int32_t>("w_dtype").Attr<int32_t>("w_layout"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxSumTiles, SumTilesImpl,

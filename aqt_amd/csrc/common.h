@@ -47,6 +47,18 @@ __device__ __forceinline__ uint16_t bf16_bits(float x) {
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }
+// Running abs-max that keeps a NaN, as jnp.max(jnp.abs(x)) does (aqt/jax/v2/calibration.py:126): a
+// diverged step must show up as a NaN scale and NaN outputs, and v_max_f32 would drop it.  For
+// non-negative floats and NaNs (sign cleared) the unsigned order of the bit patterns is the order
+// wanted: every NaN pattern lies above infinity.
+__device__ __forceinline__ float nanmax(float a, float b) {  // a, b: non-negative or NaN
+  const uint32_t x = __float_as_uint(a), y = __float_as_uint(b);
+  return __uint_as_float(x > y ? x : y);
+}
+__device__ __forceinline__ float absmax_step(float m, float v) {  // max(m, |v|)
+  return nanmax(m, __uint_as_float(__float_as_uint(v) & 0x7FFFFFFFu));
+}
+
 // Round to the dtype tag (AQTX_BF16 rounds, AQTX_F32 is the identity).
 template <bool kBf16>
 __device__ __forceinline__ float round_to(float x) {

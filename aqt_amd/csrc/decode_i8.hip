@@ -164,15 +164,15 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
 #pragma unroll
     for (int j = 0; j < PPT; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(value(i, j, e)));
+      for (int e = 0; e < 16; ++e) amax = absmax_step(amax, value(i, j, e));
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    for (int off = 32; off > 0; off >>= 1) amax = nanmax(amax, __shfl_xor(amax, off, 64));
     if (lane == 0) smax[i][wave] = amax;
   }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) {
-    float amax = fmaxf(fmaxf(smax[i][0], smax[i][1]), fmaxf(smax[i][2], smax[i][3]));
+    float amax = nanmax(nanmax(smax[i][0], smax[i][1]), nanmax(smax[i][2], smax[i][3]));
     if (amax == 0.0f) amax = 1.0f;
     float sc = rnd(amax / d.quant_bound, d.x_bf16);
     sc = rnd(sc, d.xs_bf16);
@@ -300,21 +300,21 @@ __global__ __launch_bounds__(256) void decode_quant_kernel(const DecodeArgs d, u
       if (p < pieces) {
         load_piece(p, raw[j]);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(value(raw[j], e)));
+        for (int e = 0; e < 16; ++e) amax = absmax_step(amax, value(raw[j], e));
       }
     }
   } else {
     for (int p = tid; p < pieces; p += 256) {
       load_piece(p, raw[0]);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(value(raw[0], e)));
+      for (int e = 0; e < 16; ++e) amax = absmax_step(amax, value(raw[0], e));
     }
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  for (int off = 32; off > 0; off >>= 1) amax = nanmax(amax, __shfl_xor(amax, off, 64));
   if (lane == 0) smax[wave] = amax;
   __syncthreads();
-  amax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+  amax = nanmax(nanmax(smax[0], smax[1]), nanmax(smax[2], smax[3]));
   if (amax == 0.0f) amax = 1.0f;
   float sc = rnd(amax / d.quant_bound, d.x_bf16);
   sc = rnd(sc, d.xs_bf16);

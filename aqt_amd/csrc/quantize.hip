@@ -274,12 +274,12 @@ template <int LANES>
 __device__ __forceinline__ float segment_max(float v, float* smem) {
   constexpr int W = LANES < 64 ? LANES : 64;
 #pragma unroll
-  for (int off = W / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, W));
+  for (int off = W / 2; off > 0; off >>= 1) v = nanmax(v, __shfl_xor(v, off, W));
   if constexpr (LANES == 256) {
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) smem[wave] = v;
     __syncthreads();
-    v = fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3]));
+    v = nanmax(nanmax(smem[0], smem[1]), nanmax(smem[2], smem[3]));
   }
   return v;
 }
@@ -387,16 +387,21 @@ __global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void 
 #pragma unroll
             for (int e = 0; e < VEC; ++e) t[e] = spec_prescale<SPEC>(t[e], ps[e], a);
           }
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) amax = fmaxf(amax, fabsf(t[e]));
           v[s][it].put(t);
+          if constexpr (PACKED) {  // the values are bf16 by now: two magnitudes per integer max
+#pragma unroll
+            for (int i = 0; i < 4; ++i) amax_packed = packed_absmax(amax_packed, v[s][it].w[i]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) amax = absmax_step(amax, t[e]);
+          }
         }
       } else {
         v[s][it].zero();
       }
     }
     if constexpr (PACKED)
-      amax = fmaxf(amax, fmaxf(__uint_as_float(amax_packed << 16), __uint_as_float(amax_packed & 0xFFFF0000u)));
+      amax = nanmax(amax, nanmax(__uint_as_float(amax_packed << 16), __uint_as_float(amax_packed & 0xFFFF0000u)));
     amax = segment_max<LANES>(amax, smem[s]);
     if (a.scale_given) {
       scale[s] = active ? a.scale[seg] : 1.0f;
@@ -469,7 +474,7 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const QArgs a_i
     return v;
   };
   float amax = 0.0f;
-  for (int64_t j = lane; j < a.L; j += 64) amax = fmaxf(amax, fabsf(value(j)));
+  for (int64_t j = lane; j < a.L; j += 64) amax = absmax_step(amax, value(j));
   amax = segment_max<64>(amax, nullptr);
   float scale, inv;
   if (a.scale_given) {
@@ -536,7 +541,7 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const QArgs a) {
         for (int e = 0; e < VEC; ++e) v[e] = apply_prescale(v[e], ps[e], a);
       }
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) m[e] = fmaxf(m[e], fabsf(v[e]));
+      for (int e = 0; e < VEC; ++e) m[e] = absmax_step(m[e], v[e]);
     }
   }
 #pragma unroll
@@ -545,7 +550,7 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const QArgs a) {
   for (int i = threadIdx.x; i < 64 * VEC; i += 256) {
     const int64_t c = (int64_t)blockIdx.x * 64 * VEC + i;
     if (c < a.cols) {
-      const float mm = fmaxf(fmaxf(smem[0][i], smem[1][i]), fmaxf(smem[2][i], smem[3][i]));
+      const float mm = nanmax(nanmax(smem[0][i], smem[1][i]), nanmax(smem[2][i], smem[3][i]));
       atomicMax(a.ws_absmax + b * a.ssb + g * a.ssg + c * a.ssc, __float_as_uint(mm));
     }
   }
@@ -578,14 +583,14 @@ __global__ __launch_bounds__(256) void absmax_all_kernel(const QArgs a) {
         for (int e = 0; e < 8; ++e) v[e] = apply_prescale(v[e], ps[e], a);
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(v[e]));
+      for (int e = 0; e < 8; ++e) m = absmax_step(m, v[e]);
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
       float v = Loader<TIn>::load1(xb + i);
       if (a.ps_mode == AQTX_PRESCALE_PER_ROW) v = apply_prescale(v, a.prescale[b * a.psb + i / a.cols], a);
       else if (a.ps_mode == AQTX_PRESCALE_PER_COL) v = apply_prescale(v, a.prescale[b * a.psb + i % a.cols], a);
-      m = fmaxf(m, fabsf(v));
+      m = absmax_step(m, v);
     }
   }
   m = segment_max<256>(m, smem);

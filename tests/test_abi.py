@@ -271,3 +271,45 @@ def test_ffi_shim_is_skipped_without_xla_headers(capsys):
     pytest.skip('XLA FFI headers are present here')
   assert build.build_ffi_shim(verbose=True) is None
   assert 'not built' in capsys.readouterr().err
+
+
+def _gemm_operand_requests(rows, k, ld):
+  """Highest byte offset (exclusive) the MFMA contraction kernel (csrc/gemm_core.h) requests from
+  an operand of `rows` rows, row stride `ld`, contraction length `k`: a model of its load
+  schedule.  A workgroup tile holds 256 rows; a stage is 128 bytes of K; the prologue requests
+  stages 0 and 1, every later stage two ahead.  A 16-byte request of tile row r, chunk c (c = 0,
+  16, .. 112) has buffer offset r*ld + c, range-checked by the hardware against the tile's
+  (rows_in_tile - 1)*ld + k bytes, plus the stage's scalar offset k0, which is NOT range-checked.
+  Without a K tail (k a multiple of 256) k0 is clamped to the last stage; with one, chunks at or
+  past k are masked."""
+  BM, BK = 256, 128
+  ktail = k % (2 * BK) != 0
+  kt2 = (k + 2 * BK - 1) // (2 * BK)
+  stages = [0, BK] + [s for it in range(kt2) for s in ((2 * it + 2) * BK, (2 * it + 3) * BK)]
+  if not ktail:
+    stages = [min(s, k - BK) for s in stages]
+  highest = 0
+  for tile0 in range(0, rows, BM):
+    rows_in_tile = min(BM, rows - tile0)
+    records = (rows_in_tile - 1) * ld + k
+    for k0 in set(stages):
+      for c in range(0, BK, 16):
+        if ktail and k0 + c >= k:
+          continue  # masked
+        # the last row of the tile that passes the range check reaches furthest
+        for r in range(rows_in_tile - 1, -1, -1):
+          if r * ld + c + 16 <= records:
+            highest = max(highest, tile0 * ld + r * ld + c + k0 + 16)
+            break
+  return highest
+
+
+@pytest.mark.parametrize('rows,k,ld', [
+    (8192, 4096, 4096), (256, 256, 256), (300, 512, 512), (17, 1024, 1040), (512, 384, 384), (256, 128, 128),
+    (100, 144, 144), (64, 16, 16), (1000, 2064, 2064), (14336, 8192, 8192),
+])
+def test_gemm_never_requests_bytes_past_an_operand(rows, k, ld):
+  """The scalar offset of a buffer load escapes the hardware range check; the kernel has to keep
+  its look-ahead requests inside the operand by itself (an exactly sized allocation may end on a
+  page boundary)."""
+  assert _gemm_operand_requests(rows, k, ld) <= (rows - 1) * ld + k

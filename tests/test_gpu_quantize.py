@@ -270,3 +270,44 @@ def test_key_in_device_memory_equals_key_in_the_plan(gpu, reduce, transpose, sha
   kd2[1] += 1
   q2, _ = ops.quantize(x, key_device=kd2, **kw)
   assert not torch.equal(q0, q2)
+
+
+@pytest.mark.parametrize('dt', ['bf16', 'f32'])
+@pytest.mark.parametrize('reduce,shape', [
+    (L.REDUCE_COLS, (2, 9, 1024)), (L.REDUCE_COLS, (1, 3, 1001)), (L.REDUCE_ROWS, (1, 200, 96)),
+    (L.REDUCE_ALL, (3, 40, 64)),
+])
+def test_nan_reaches_the_scale(gpu, dt, reduce, shape):
+  """jnp.max(jnp.abs(x)) propagates a NaN into the scale (calibration.py:126-157), which is how a
+  diverged step shows up in the outputs; the kernels' abs-max does the same, and the scales of
+  segments without a NaN are untouched."""
+  x = U.rand(shape, dt, seed=11)
+  x[0, 1, 5] = np.nan
+  q = R.QuantizerCfg(bits=8)
+  axes = {L.REDUCE_COLS: [2], L.REDUCE_ROWS: [1], L.REDUCE_ALL: [1, 2]}[reduce]
+  with np.errstate(invalid='ignore'):
+    want = R.quantize(x, dt, q, axes).scale[0].reshape(-1)
+  _, sg = ops.quantize(U.to_dev(x, dt, gpu), reduce=reduce, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0)
+  got = sg.cpu().numpy().reshape(-1)
+  assert np.isnan(want).sum() == 1
+  np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+  np.testing.assert_array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+
+
+def test_nan_row_gives_nan_outputs(gpu):
+  """End to end: one NaN activation makes exactly that token's outputs NaN (its scale is NaN), in
+  the training-shape path and in the serving kernels."""
+  from aqt_amd.v2 import aqt_dot_general as aqt
+  from aqt_amd.v2 import config
+  lhs = torch.randn(48, 256, device=gpu).to(torch.bfloat16)
+  rhs = (torch.randn(256, 64, device=gpu) * 0.05).to(torch.bfloat16)
+  lhs[7, 100] = float('nan')
+  cfg = config.set_context(config.fully_quantized(fwd_bits=8, bwd_bits=8, use_stochastic_rounding=False), None, None)
+  out, _ = cfg.dg_core(lhs, rhs, None, None, (((1,), (0,)), ((), ())))
+  bad = torch.isnan(out).any(dim=1).cpu().numpy()
+  assert bad[7] and bad.sum() == 1 and bool(torch.isnan(out[7]).all())
+  wq = torch.randint(-127, 128, (64, 256), dtype=torch.int8, device=gpu)
+  ws = torch.rand(64, device=gpu) * 1e-3
+  for m in (2, 48):
+    o, xs = ops.decode(lhs[6:6 + m].contiguous(), wq, ws, quant_bound=127.5, clip_bound=127.0)
+    assert bool(torch.isnan(xs[1])) and bool(torch.isnan(o[1]).all()) and not bool(torch.isnan(o[0]).any())
