@@ -53,10 +53,45 @@ __global__ __launch_bounds__(256) void sum_tiles_kernel(const void* x, void* out
   }
 }
 
+// Reads `bytes` once, 16 bytes per lane and load, PER loads in flight per lane, and writes one
+// word per workgroup: the least any kernel that streams a buffer of this size can take.
+template <int PER>
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4* p, int64_t vecs, uint32_t* out) {
+  uint32_t acc = 0u;
+  const int64_t base = (int64_t)blockIdx.x * 256 * PER + threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int64_t i = base + (int64_t)j * 256;
+    if (i < vecs) {
+      const uint4 v = p[i];
+      acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, 64);
+  if ((threadIdx.x & 63) == 0) atomicXor(out + blockIdx.x, acc);
+}
+
 }  // namespace
 }  // namespace aqtx
 
 using namespace aqtx;
+
+extern "C" int aqtx_read_probe(const void* src, int64_t bytes, void* out_words, int64_t out_count, void* stream) {
+  clear_error();
+  AQTX_REQUIRE(bytes >= 0 && bytes % 16 == 0, "aqtx_read_probe: bytes must be a non-negative multiple of 16");
+  if (bytes == 0) return 0;
+  AQTX_REQUIRE(src != nullptr && out_words != nullptr, "aqtx_read_probe: NULL buffer");
+  AQTX_REQUIRE(((uintptr_t)src % 16) == 0, "aqtx_read_probe: src must be 16-byte aligned");
+  constexpr int kPer = 16;  // 64 KiB per workgroup
+  const int64_t vecs = bytes / 16;
+  const int64_t blocks = (vecs + 256 * kPer - 1) / (256 * kPer);
+  AQTX_REQUIRE(blocks <= out_count && blocks < (1ll << 31), "aqtx_read_probe: out needs %lld words", (long long)blocks);
+  read_probe_kernel<kPer><<<(unsigned)blocks, 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      reinterpret_cast<const uint4*>(src), vecs, reinterpret_cast<uint32_t*>(out_words));
+  AQTX_HIP_CHECK_LAUNCH("read_probe_kernel");
+  return 0;
+}
 
 extern "C" int aqtx_sum_tiles(const void* x, void* out, int64_t tiles, int64_t count, int32_t dtype,
                               void* stream) {

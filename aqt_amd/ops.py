@@ -383,6 +383,19 @@ def tile_weight(w_q: torch.Tensor, w_dtype: int = L.I8) -> torch.Tensor:
   return out
 
 
+def read_probe(buf: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+  """Streams `buf` once through the library's read-only kernel (a measurement aid); returns the
+  per-workgroup checksum words."""
+  _require_gpu(buf)
+  assert buf.is_contiguous()
+  nbytes = buf.numel() * buf.element_size()
+  words = (nbytes + 65535) // 65536
+  if out is None:
+    out = torch.zeros(max(words, 1), dtype=torch.int32, device=buf.device)
+  L.check(L.lib().aqtx_read_probe(_ptr(buf), nbytes, _ptr(out), out.numel(), _stream()))
+  return out
+
+
 def pack_i4(q: torch.Tensor) -> torch.Tensor:
   """int4 values held one per int8 byte, last axis even -> uint8 tensor with the last axis halved."""
   _require_gpu(q)

@@ -24,7 +24,7 @@ MATMUL = (((1,), (0,)), ((), ()))
 # HBM bytes per GEMM launch (mean of fwd, dlhs, drhs) from the FETCH_SIZE / WRITE_SIZE counter runs
 # summarised in profiles/bench_int8_fwd_bwd_8192x4096x14336_hbm_traffic.txt; counters cannot be
 # read from inside this process, so the figure is carried here and re-measured when the kernel changes.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 953e6
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 868e6
 
 
 def make_inputs(device):
@@ -270,6 +270,76 @@ def other_configs(dev):
   return out
 
 
+def read_floor(dev):
+  """What this box's memory system delivers to a kernel that only reads a decode-sized weight once
+  (aqtx_read_probe: coalesced 16 bytes per lane, one checksum word per workgroup, nothing else),
+  measured the way decode_bench measures: the buffers rotate through 1 GiB and the calls are
+  replayed from a HIP graph.  The decode kernels cannot be faster than this; prints one JSON line."""
+  import torch
+  from aqt_amd import ops
+  rows = []
+  for n in (4096, 14336):
+    for scale, what in ((1.0, 'int8'), (0.5, 'packed int4')):
+      nbytes = int(n * 4096 * scale)
+      ncopies = (1 << 30) // nbytes + 1
+      bufs = [torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=dev) for _ in range(ncopies)]
+      out = torch.zeros(nbytes // 65536 + 1, dtype=torch.int32, device=dev)
+      run = lambda: [ops.read_probe(b, out) for b in bufs]
+      run()
+      torch.cuda.synchronize()
+      side = torch.cuda.Stream()
+      graph = torch.cuda.CUDAGraph()
+      with torch.cuda.stream(side):
+        run()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+          run()
+      torch.cuda.synchronize()
+      graph.replay()
+      torch.cuda.synchronize()
+      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      a.record()
+      for _ in range(5):
+        graph.replay()
+      b.record()
+      torch.cuda.synchronize()
+      us = a.elapsed_time(b) * 1e3 / (5 * ncopies)
+      rows.append({'weight': f'{n}x4096 {what}', 'bytes': nbytes, 'us_per_read': round(us, 2),
+                   'GB/s': round(nbytes / us / 1e3, 1)})
+      del graph, bufs
+  print(json.dumps({'read_floor': 'aqtx_read_probe over a buffer of the weight size, HIP graph replay, 1 GiB rotation',
+                    'rows': rows}))
+
+
+def decode_probe(dev, calibration_copy=False):
+  """A few eager serving calls per shape (int8 weight in fragment order, n in {4096, 14336},
+  m in {1, 8, 64}, weights rotated through 1 GiB) for counter and kernel-trace runs of the
+  serving kernels, plus one read of each weight size by aqtx_read_probe."""
+  import torch
+  from aqt_amd import _lib as L
+  from aqt_amd import ops
+  if calibration_copy:
+    src = torch.ones(64 << 20, dtype=torch.int32, device=dev)
+    torch.neg(src, out=torch.empty_like(src))  # 256 MiB in, 256 MiB out
+    del src
+  k = 4096
+  for n in (4096, 14336):
+    ncopies = (1 << 30) // (n * k) + 1
+    raw = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(ncopies)]
+    weights = [ops.tile_weight(w, L.I8) for w in raw]
+    w_scale = torch.rand(n, device=dev) * 1e-3 + 1e-5
+    out = torch.zeros(n * k // 65536 + 1, dtype=torch.int32, device=dev)
+    for w in raw:
+      ops.read_probe(w, out)
+    for m in (1, 8, 64):
+      x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+      for w in weights:
+        ops.decode(x, w, w_scale, quant_bound=127.5, clip_bound=127.0, w_layout=L.W_FRAGMENTS)
+    torch.cuda.synchronize()
+    del raw, weights
+  print(json.dumps({'decode_probe': 'done'}))
+
+
 def gemm_probe(dev, data, reps=10):
   """The three contractions of a step on their own, on synthetic int8 operands of a chosen value
   distribution (the MFMA rate of this part depends on the operand values: the chip lowers its
@@ -326,6 +396,10 @@ def main():
   ap.add_argument('--gemm-probe', choices=['zeros', 'normal25', 'uniform'], default=None,
                   help='only run the three int8 contractions of a step on operands of this value '
                        'distribution (and the vendor int8 GEMM beside them) and exit')
+  ap.add_argument('--decode-probe', action='store_true',
+                  help='only issue a few serving calls per shape (for rocprofv3 runs) and exit')
+  ap.add_argument('--read-floor', action='store_true',
+                  help='only time a pure read of decode-sized buffers (the memory floor of the serving kernels) and exit')
   args = ap.parse_args()
   if args.gpus != 1:
     print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)',
@@ -342,6 +416,12 @@ def main():
   dev = torch.device('cuda:0')
   if args.gemm_probe is not None:
     gemm_probe(dev, args.gemm_probe)
+    return
+  if args.read_floor:
+    read_floor(dev)
+    return
+  if args.decode_probe:
+    decode_probe(dev, args.calibration_copy)
     return
   lhs, rhs, g = make_inputs(dev)
   lhs.requires_grad_(True)

@@ -377,6 +377,14 @@ int aqtx_prng_split_host(const uint32_t key_host[2], int32_t num, int32_t partit
 int aqtx_random_bits(const uint32_t key_host[2], int64_t n, int32_t bit_width,
                      int32_t partitionable, void* out, void* stream);
 
+/*
+ * aqtx_read_probe: a measurement aid with no counterpart in the reference.  Streams `bytes` (a multiple of
+ * 16) from src once, coalesced 16 bytes per lane, 64 KiB per workgroup, and XORs one checksum word per
+ * workgroup into out_words[0 .. ceil(bytes / 65536)): the floor for the device time of any kernel that has
+ * to read a buffer of that size once (the serving kernels are measured against it).
+ */
+int aqtx_read_probe(const void* src, int64_t bytes, void* out_words, int64_t out_count, void* stream);
+
 /* Message of the calling thread's most recent failure ("" if none). */
 const char* aqtx_last_error(void);
 

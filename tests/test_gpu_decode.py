@@ -284,3 +284,12 @@ def test_decode_fragment_ordered_weight(gpu, packed, m, n, k):
     np.testing.assert_array_equal(out.float().cpu().numpy(), want, err_msg=hex(tuning))
     np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
     np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
+
+
+def test_read_probe_reads_every_byte(gpu):
+  """The read-floor kernel's checksum is the XOR of all 32-bit words of its 64 KiB share."""
+  buf = torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * 16384 + 52,), dtype=torch.int32, device=gpu)
+  got = ops.read_probe(buf).cpu().numpy().view(np.uint32)
+  words = buf.cpu().numpy().view(np.uint32)
+  want = [np.bitwise_xor.reduce(words[i:i + 16384]) for i in range(0, len(words), 16384)]
+  np.testing.assert_array_equal(got, np.asarray(want, dtype=np.uint32))
