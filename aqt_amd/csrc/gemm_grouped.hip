@@ -6,35 +6,50 @@
 // a batch axis of the inner call, every tile is dequantized (rounded to the dequant dtype) on its
 // own and the tiles are summed afterwards.  Here the per-group results never leave registers.
 //
-// One workgroup (8 waves, 2x4) owns a 128x256 tile of C, a wave 64x64 = 2x2 MFMA tiles
-// (v_mfma_i32_32x32x32_i8): 64 int32 accumulators of the current group and 64 float32 running
-// sums.  A stage is 128 bytes of K, double-buffered in LDS with the same XOR swizzle as the dense
-// kernel.  The group scales of a stage sit in LDS next to it.  The per-group rescale is ~9 VALU
-// operations per element and group, which bounds this kernel (the MFMAs of one wave run under the
-// rescale of the other wave of its SIMD).
+// The per-group rescale is 7 vector instructions per element and group (int->float, three
+// roundings to bf16, two multiplications, one addition) against one MFMA per 1024 elements and
+// 32 k: with groups of 128 the kernel is bound by the vector ALU, not by the matrix cores.  On
+// this device a wave issues one vector instruction every ~12 cycles however independent its
+// instructions are (measured: 2 waves per SIMD reach 2.7 ns per instruction and SIMD, 4 waves
+// 1.5 ns for add/mul/and and 2.3 ns for the conversions and shifts), so a kernel of this kind
+// wants 4 waves per SIMD, i.e. at most 128 registers per lane, more than it wants large tiles.
+//
+// Two kernels, both with 128-byte K stages double-buffered in LDS, the group scales of a stage
+// next to it in LDS:
+//   gemm_grouped128_kernel  group = 128 (one stage per group).  Workgroup = 8 waves (4 x 2) on a
+//       128 x 128 tile of C, a wave 32 x 64 = two MFMA tiles (v_mfma_i32_32x32x32_i8): 32 int32
+//       accumulators of the current group and 32 float32 running sums; two workgroups per CU.
+//   gemm_grouped_kernel     longer groups.  Workgroup = 8 waves (2 x 4) on 128 x 256, a wave
+//       64 x 64, LDS under the XOR swizzle of the dense kernel; the rescale follows the last
+//       stage of a group.
 //
 // Packed int4 weights (two values per byte, low nibble = even k) are unpacked in registers on their
 // way to LDS: a nibble is moved to the top of its byte (value * 16) and the factor 1/16 is folded,
 // exactly, into the column scale.
+//
+// Not used, measured: accumulating the rounded group results with v_mfma_f32_32x32x16_bf16 against
+// a 0/1 selection matrix (which would save the widening and the addition) is not a correctly
+// rounded float32 addition on this device: 2-10 % of random sums differ in the last bit.
 #include "gemm_core.h"
 
 namespace aqtx {
 namespace {
 
-constexpr int GM = 128, GN = 256;  // GK = BK = 128
+constexpr int GM = 128;  // rows of C per workgroup; a stage is BK = 128 bytes of K
+constexpr int grouped_cols(bool group128) { return group128 ? 128 : 256; }
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-// Rounds two floats to bf16 (ties to even) in place: one packed conversion, then one shift and
-// one mask to widen them again.
+// Rounds a float to bf16 (ties to even) and widens it again in one instruction: the packed
+// conversion of (0, x) leaves bf16(x) in the upper half of the word over a zero lower half.
 template <bool kBf16>
-__device__ __forceinline__ void round_pair(float& a, float& b) {
+__device__ __forceinline__ float round_wide(float x) {
   if constexpr (kBf16) {
-    const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
-    const uint32_t w = __builtin_bit_cast(uint32_t, h);
-    a = __uint_as_float(w << 16);
-    b = __uint_as_float(w & 0xFFFF0000u);
+    const bf16x2 h = __builtin_convertvector(f32x2{0.0f, x}, bf16x2);
+    return __builtin_bit_cast(float, h);
+  } else {
+    return x;
   }
 }
 
@@ -49,16 +64,282 @@ struct GroupedArgs {
   int tiles_m, tiles_n;
 };
 
+__device__ __forceinline__ int row_swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+// 16 bytes of packed int4 (32 values, low nibble = even k) -> 32 bytes of values * 16 in k order.
+// dword d of the load = k 8d..8d+7: even k: (x << 4) & 0xF0F0F0F0, odd k: x & 0xF0F0F0F0; then
+// the bytes are interleaved back to k order.
+__device__ __forceinline__ void unpack_i4x32(const v4i x4, v4i& lo, v4i& hi) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const uint32_t x = (uint32_t)x4[d];
+    const uint32_t ev = (x << 4) & 0xF0F0F0F0u, od = x & 0xF0F0F0F0u;
+    const uint32_t k03 = __builtin_amdgcn_perm(od, ev, 0x05010400u);  // e0 o0 e1 o1
+    const uint32_t k47 = __builtin_amdgcn_perm(od, ev, 0x07030602u);  // e2 o2 e3 o3
+    if (d < 2) { lo[2 * d] = (int)k03; lo[2 * d + 1] = (int)k47; }
+    else { hi[2 * (d - 2)] = (int)k03; hi[2 * (d - 2) + 1] = (int)k47; }
+  }
+}
+
 // EPI as in the dense kernel: 0 = bf16 out, both products rounded to bf16; 4 = bf16 out, first
 // product bf16, second f32; 1 = bf16 out, products in f32; 2 = f32 out.
-// ONE: a group is exactly one 128-byte stage (group = 128), which takes the branches on the
-// position inside a group out of the loop.
-template <int EPI, bool PACKED, bool ONE>
+template <int EPI>
+struct Rescale {
+  static constexpr bool kOutBf16 = EPI != 2;
+  static constexpr bool kP1Bf16 = EPI == 0 || EPI == 4;
+  static constexpr bool kP2Bf16 = EPI == 0;
+  // sum[r] += dequant(acc[r]) for registers r = 4q .. 4q+3 of NT accumulator tiles that share the
+  // four column scales cs (tile t has row scale rs[t]).  Every product and the sum round on their
+  // own (the library is built with floating-point contraction off, so no fused multiply-add
+  // appears here); the elements go through each step together, not one after the other.
+  template <int NT>
+  static __device__ __forceinline__ void quarter(const v16i* const (&acc)[NT], v16f* const (&sum)[NT], const int q,
+                                                 const float (&rs)[NT], const float4 cs4) {
+    const float cs[4] = {cs4.x, cs4.y, cs4.z, cs4.w};
+    float f[4 * NT];
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) f[i] = (float)(*acc[i >> 2])[4 * q + (i & 3)];
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) f[i] = round_wide<kOutBf16>(f[i]);
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) f[i] *= rs[i >> 2];
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) f[i] = round_wide<kP1Bf16>(f[i]);
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) f[i] *= cs[i & 3];
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) f[i] = round_wide<kP2Bf16 || kOutBf16>(f[i]);  // P2 rounding, or the tile's final cast
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) (*sum[i >> 2])[4 * q + (i & 3)] += f[i];
+  }
+};
+
+// Writes registers 4q..4q+3 of a running-sum tile: four consecutive n of row mm.
+template <bool kOutBf16>
+__device__ __forceinline__ void store_out4(const GroupedArgs& g, const v16f& sum, int q, int64_t mm, int64_t nn, bool vec) {
+  constexpr int kEsz = kOutBf16 ? 2 : 4;
+  if (mm >= g.m || nn >= g.n) return;
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = round_to<kOutBf16>(sum[4 * q + e]);
+  uint8_t* dst = reinterpret_cast<uint8_t*>(g.c) + (mm * g.ldc + nn) * kEsz;
+  if (vec && nn + 4 <= g.n) {
+    if constexpr (kOutBf16) {
+      uint2 w;
+      w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+      w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+      *reinterpret_cast<uint2*>(dst) = w;
+    } else {
+      *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+  } else {
+    for (int e = 0; e < 4 && nn + e < g.n; ++e) {
+      if constexpr (kOutBf16) reinterpret_cast<uint16_t*>(dst)[e] = bf16_bits(o[e]);
+      else reinterpret_cast<float*>(dst)[e] = o[e];
+    }
+  }
+}
+
+// The group scale this thread fetches for its workgroup: thread t < GM a row scale, GM <= t <
+// GM + GN a column scale.  The load is unconditional from a clamped address and nothing reads its
+// result before store(): a use next to the load would wait there for every load issued before it.
+template <int GN, bool PACKED>
+struct ScaleFetch {
+  const float* ptr;
+  int64_t len;
+  float reg = 1.0f;
+  bool row, inside, valid = false, active;
+  int groups;
+  __device__ __forceinline__ ScaleFetch(const GroupedArgs& g, int tid, int64_t m0, int64_t n0) {
+    row = tid < GM;
+    active = tid < GM + GN;
+    const int64_t idx = row ? m0 + tid : n0 + (tid - GM);
+    len = row ? g.m : g.n;
+    inside = active && idx < len;
+    ptr = (row ? g.row_scale : g.col_scale) + (inside ? idx : 0);
+    groups = g.groups;
+  }
+  // called for grp = 0, 1, 2, ... in order: the pointer moves on by one group per call and stops
+  // at the last group
+  __device__ __forceinline__ void load(int grp) {
+    valid = inside && grp < groups;
+    if (active) reg = *ptr;
+    if (grp + 1 < groups) ptr += len;
+  }
+  __device__ __forceinline__ void store(int tid, float* srow, float* scol) {
+    asm volatile("" : "+v"(reg));  // keeps the arithmetic on the loaded value down here
+    const float v = valid ? reg * ((PACKED && !row) ? 0.0625f : 1.0f) : 1.0f;
+    if (row) srow[tid] = v;
+    else if (active) scol[tid - GM] = v;
+  }
+};
+
+// ---- group = 128 ---------------------------------------------------------------------------------
+// LDS rows are 144 bytes apart (128 of data, 16 of padding) instead of XOR-swizzled: the 16 lanes
+// of a fragment read still fall into 64 distinct banks, and every address of the loop is one of a
+// few loop-invariant registers plus an immediate, which this kernel needs more than it needs
+// the 12 % of LDS: it has 128 registers per lane.
+//
+// A stage: eight MFMAs (four 32-byte k steps x two column tiles); the staging registers (stage
+// s + 1, requested during stage s - 1) go to LDS, into the buffer stage s - 1 left; the rescale of
+// the group just accumulated, with the global loads of stage s + 2 issued one per quarter of it
+// (issued in one burst, the loads of all waves queue up in the CU's address unit and the waves
+// stand still behind them); the next group's scales go to LDS; barrier.  The other three waves of
+// the SIMD fill the gaps each of these leaves.
+template <int EPI, bool PACKED>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void gemm_grouped128_kernel(const GroupedArgs g) {
+  using R = Rescale<EPI>;
+  constexpr int GN = grouped_cols(true);
+  constexpr int kRow = BK + 16;
+  constexpr int kATile = GM * kRow, kBTile = GN * kRow, kStage = kATile + kBTile;  // 36 KiB
+  __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[2 * kStage];
+  __shared__ __attribute__((aligned(16))) float srow[2][GM];
+  __shared__ __attribute__((aligned(16))) float scol[2][GN];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;  // 32 rows, 64 columns
+  const int lr = lane & 31, lh = lane >> 5;
+  int tm, tn;
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const int64_t m0 = (int64_t)tm * GM, n0 = (int64_t)tn * GN;
+  const int64_t rows_a = (g.m - m0) < GM ? (g.m - m0) : GM;
+  const int64_t rows_b = (g.n - n0) < GN ? (g.n - n0) : GN;
+  const int kb_bytes = PACKED ? (int)(g.k / 2) : (int)g.k;  // bytes of one B row
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + kb_bytes), kBufferRsrcWord3);
+  // group scales: waves 0, 1 fetch the 128 row scales, waves 2, 3 the 128 column scales of the next
+  // group, one per lane, through a buffer whose scalar offset selects the group.  Nothing reads the
+  // result before it goes to LDS at the end of the stage: a use next to the load would wait there
+  // for every load issued before it.
+  const bool sc_row = wave < 2, sc_active = wave < 4;
+  const int sc_idx = (tid & 127);
+  const int64_t sc_len = sc_row ? g.m : g.n, sc_first = sc_row ? m0 : n0;
+  const bool sc_inside = sc_active && sc_first + sc_idx < sc_len;
+  const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)((sc_row ? g.row_scale : g.col_scale) + sc_first), 0, (int)(((int64_t)g.groups * sc_len - sc_first) * 4),
+      kBufferRsrcWord3);
+  const int sc_step = (int)sc_len * 4;  // bytes from one group's scales to the next
+  float sc_reg = 1.0f;
+  auto load_scales = [&](int grp) {  // lanes past the operand read another row's scale or zero; store_scales masks them
+    const int grp_c = grp < g.groups ? grp : g.groups - 1;
+    if (sc_active) sc_reg = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, sc_idx * 4, grp_c * sc_step, 0));
+  };
+  auto store_scales = [&](int grp, int buf) {
+    asm volatile("" : "+v"(sc_reg));  // keeps the arithmetic on the loaded value down here
+    const float v = (sc_inside && grp < g.groups) ? sc_reg * ((PACKED && !sc_row) ? 0.0625f : 1.0f) : 1.0f;
+    if (sc_row) srow[buf][sc_idx] = v;
+    else if (sc_active) scol[buf][sc_idx] = v;
+  };
+
+  // ---- global -> registers -> LDS (rows past the operand read as zero) ----------------------
+  // A: 16 blocks of 8 rows x 128 B, two per wave.  B unpacked: 16 such blocks, two per wave.
+  // B packed: a wave load covers 16 rows x 64 B, one per wave; a lane's 16 bytes become the 32
+  // bytes at 32 * (lane & 3) of its row.  Loads j of one operand differ by a scalar offset.
+  constexpr int NLA = 2, NLB = PACKED ? 1 : 2, NL = NLA + NLB;
+  v4i stg[NL];
+  const int ld_a = (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
+  const int ld_b = PACKED ? (wave * 16 + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
+                          : (wave * 16 + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
+  const int st_a = (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
+  const int st_b = kATile + (PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
+                                    : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
+  auto load_one = [&](const int j, int k0) {
+    if (j < NLA) stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ld_a, k0 + j * 8 * (int)g.lda, 0);
+    else if constexpr (PACKED) stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ld_b, k0 / 2, 0);
+    else stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ld_b, k0 + (j - NLA) * 8 * (int)g.ldb, 0);
+  };
+  auto store_stage = [&](const int stage_base) {
+    uint8_t* st = stage_mem + stage_base;
+#pragma unroll
+    for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
+    if constexpr (PACKED) {
+      v4i lo, hi;
+      unpack_i4x32(stg[NLA], lo, hi);
+      *reinterpret_cast<v4i*>(st + st_b) = lo;
+      *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLB; ++j) *reinterpret_cast<v4i*>(st + st_b + j * 8 * kRow) = stg[NLA + j];
+    }
+  };
+
+  // fragment of k step ks: 16 bytes at 32 ks + 16 lh of row lr of the 32-row block
+  const int a_off = (wm * 32 + lr) * kRow + lh * 16;
+  const int b_off = kATile + (wn * 64 + lr) * kRow + lh * 16;
+  const int rs_off = wm * 32 + lr, cs_off = wn * 64 + 4 * lh;
+
+  v16i acc[2];
+  v16f sum[2];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { acc[0][r] = 0; acc[1][r] = 0; sum[0][r] = 0.0f; sum[1][r] = 0.0f; }
+  const v16i kZero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+  const int nstages = g.groups;
+  for (int j = 0; j < NL; ++j) load_one(j, 0);
+  load_scales(0);
+  store_stage(0);
+  store_scales(0, 0);
+  for (int j = 0; j < NL; ++j) load_one(j, nstages > 1 ? BK : 0);
+  __syncthreads();
+
+  // BUF (compile time) is the LDS buffer of stage s, so that every LDS address is a register plus an immediate
+  auto stage = [&](const int s, auto buf_c) {
+    constexpr int BUF = decltype(buf_c)::value;
+    const uint8_t* st = stage_mem + BUF * kStage;
+    load_scales(s + 1);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const v4i fa = *reinterpret_cast<const v4i*>(st + a_off + ks * 32);
+      const v4i fb0 = *reinterpret_cast<const v4i*>(st + b_off + ks * 32);
+      const v4i fb1 = *reinterpret_cast<const v4i*>(st + b_off + 32 * kRow + ks * 32);
+      // the first MFMA of a group starts from a zero accumulator operand instead of zeroed registers
+      acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb0, fa, ks == 0 ? kZero : acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb1, fa, ks == 0 ? kZero : acc[1], 0, 0, 0);
+    }
+    // Past the last stage the store and the loads are repeated harmlessly (a buffer nobody reads,
+    // k offset 0) rather than branched around.
+    store_stage((1 - BUF) * kStage);
+    const int k_next = s + 2 < nstages ? (s + 2) * BK : 0;
+    // lane holds C[m = wm*32 + lr][n = wn*64 + ni*32 + 8q + 4lh + e], register 4q + e of tile ni
+    const float rs[1] = {srow[BUF][rs_off]};
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (ni * 4 + q < NL) load_one(ni * 4 + q, k_next);
+        const v16i* const a1[1] = {&acc[ni]};
+        v16f* const s1[1] = {&sum[ni]};
+        R::template quarter<1>(a1, s1, q, rs, *reinterpret_cast<const float4*>(&scol[BUF][cs_off + ni * 32 + 8 * q]));
+      }
+    store_scales(s + 1, 1 - BUF);
+    // a bare s_barrier: a __syncthreads() would also wait for the global loads just issued
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  for (int s = 0; s < nstages; s += 2) {
+    stage(s, std::integral_constant<int, 0>{});
+    if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
+  }
+
+  const bool vec = (g.ldc % 4) == 0 && ((uintptr_t)g.c % 16) == 0;
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      store_out4<R::kOutBf16>(g, sum[ni], q, m0 + wm * 32 + lr, n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh, vec);
+}
+
+// ---- groups of 256 and more ------------------------------------------------------------------------
+template <int EPI, bool PACKED>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_grouped_kernel(const GroupedArgs g) {
-  constexpr bool kOutBf16 = EPI != 2;
-  constexpr bool kP1Bf16 = EPI == 0 || EPI == 4;
-  constexpr bool kP2Bf16 = EPI == 0;
+  using R = Rescale<EPI>;
+  constexpr int GN = grouped_cols(false);
   constexpr int kATile = GM * BK, kBTile = GN * BK, kStage = kATile + kBTile;  // 48 KiB
   __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[2][kStage];
   __shared__ __attribute__((aligned(16))) float srow[2][GM];
@@ -66,7 +347,7 @@ void gemm_grouped_kernel(const GroupedArgs g) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave >> 2, wn = wave & 3;  // 64 rows, 64 columns
   const int lr = lane & 31, lh = lane >> 5;
   int tm, tn;
   tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
@@ -81,13 +362,11 @@ void gemm_grouped_kernel(const GroupedArgs g) {
 
   // ---- global -> registers -> LDS (rows past the operand read as zero) ----------------------
   // A: 16 blocks of 8 rows x 128 B, two per wave.  B unpacked: 32 such blocks, four per wave.
-  // B packed: a wave load covers 16 rows x 64 B; two per wave; a lane's 16 bytes become the two
-  // neighbouring 16-byte pieces 2p, 2p+1 of its row.
+  // B packed: a wave load covers 16 rows x 64 B; two per wave.
   constexpr int NLA = 2, NLB = PACKED ? 2 : 4;
-  // two sets of staging registers: the loads of a stage are issued two stages ahead of its use and
-  // written to LDS one stage ahead, so that a stage never waits for a load issued in it
+  // two sets of staging registers: a stage without a rescale is short, so the loads of a stage
+  // are issued two stages ahead of its use and written to LDS one stage ahead
   v4i sta[2][NLA], stb[2][NLB];
-  auto row_swz = [](int row) { return (row ^ (row >> 3)) & 7; };
   auto load_stage = [&](const int set, int k0) {
 #pragma unroll
     for (int i = 0; i < NLA; ++i) {
@@ -114,20 +393,9 @@ void gemm_grouped_kernel(const GroupedArgs g) {
 #pragma unroll
     for (int i = 0; i < NLB; ++i) {
       if constexpr (PACKED) {
-        const int row = (wave * NLB + i) * 16 + (lane >> 2);
-        const int p = lane & 3;
-        // dword d of the load = k 8d..8d+7 of this lane's 32: even k in low nibbles.  Values * 16:
-        // even k: (x << 4) & 0xF0F0F0F0, odd k: x & 0xF0F0F0F0; then bytes interleaved back to k order.
+        const int row = (wave * NLB + i) * 16 + (lane >> 2), p = lane & 3;
         v4i lo, hi;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const uint32_t x = (uint32_t)stb[set][i][d];
-          const uint32_t ev = (x << 4) & 0xF0F0F0F0u, od = x & 0xF0F0F0F0u;
-          const uint32_t k03 = __builtin_amdgcn_perm(od, ev, 0x05010400u);  // e0 o0 e1 o1
-          const uint32_t k47 = __builtin_amdgcn_perm(od, ev, 0x07030602u);  // e2 o2 e3 o3
-          if (d < 2) { lo[2 * d] = (int)k03; lo[2 * d + 1] = (int)k47; }
-          else { hi[2 * (d - 2)] = (int)k03; hi[2 * (d - 2) + 1] = (int)k47; }
-        }
+        unpack_i4x32(stb[set][i], lo, hi);
         uint8_t* rowp = st + kATile + row * BK;
         *reinterpret_cast<v4i*>(rowp + (((2 * p) ^ row_swz(row)) * 16)) = lo;
         *reinterpret_cast<v4i*>(rowp + (((2 * p + 1) ^ row_swz(row)) * 16)) = hi;
@@ -136,33 +404,14 @@ void gemm_grouped_kernel(const GroupedArgs g) {
       }
     }
   };
-  // group scales of the tile: thread t < 128 a row scale, 128 <= t < 384 a column scale
-  float sc_reg = 1.0f;
-  auto load_scales = [&](int grp) {
-    sc_reg = 1.0f;
-    if (grp < g.groups) {
-      if (tid < GM) {
-        if (m0 + tid < g.m) sc_reg = g.row_scale[(int64_t)grp * g.m + m0 + tid];
-      } else if (tid < GM + GN) {
-        const int64_t nn = n0 + (tid - GM);
-        if (nn < g.n) sc_reg = g.col_scale[(int64_t)grp * g.n + nn] * (PACKED ? 0.0625f : 1.0f);
-      }
-    }
-  };
-  auto store_scales = [&](int buf) {
-    if (tid < GM) srow[buf][tid] = sc_reg;
-    else if (tid < GM + GN) scol[buf][tid - GM] = sc_reg;
-  };
+  ScaleFetch<GN, PACKED> sc(g, tid, m0, n0);
 
-  // ---- fragments ---------------------------------------------------------------------------
-  const int lf0 = (lr ^ (lr >> 3)) & 7;
-  int frag_off[8];
-#pragma unroll
-  for (int c = 0; c < 8; ++c) frag_off[c] = lr * BK + ((lh ^ lf0 ^ c) * 16);
+  const int frag_off0 = lr * BK + ((lh ^ ((lr ^ (lr >> 3)) & 7)) * 16);
+  auto frag_off = [&](int c) { return frag_off0 ^ (c * 16); };
   const int a_base = wm * 64 * BK, b_base = kATile + wn * 64 * BK;
 
   v16i acc[2][2];
-  float sum[2][2][16];
+  v16f sum[2][2];
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
@@ -173,29 +422,29 @@ void gemm_grouped_kernel(const GroupedArgs g) {
 
   const int nstages = g.groups * g.stages_per_group;
   load_stage(0, 0);
-  load_scales(0);
+  sc.load(0);
   store_stage(0, stage_mem[0]);
-  store_scales(0);
+  sc.store(tid, srow[0], scol[0]);
   if (nstages > 1) load_stage(1, BK);  // set 1 holds stage 1, set 0 will take stage 2, ...
   __syncthreads();
   // one stage; `set` holds the registers of stage s + 1, the other set takes the loads of s + 2
   auto stage = [&](const int s, const int set) {
-    const int grp = ONE ? s : s / g.stages_per_group;
-    const bool last_of_group = ONE || (s + 1) % g.stages_per_group == 0;
+    const int grp = s / g.stages_per_group, pos = s % g.stages_per_group;
+    const bool last_of_group = pos + 1 == g.stages_per_group;
     const uint8_t* st = stage_mem[s & 1];
     if (s + 2 < nstages) load_stage(set ^ 1, (s + 2) * BK);
-    if (last_of_group) load_scales(grp + 1);
+    if (last_of_group) sc.load(grp + 1);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       v4i fa[2], fb[2];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int c = (2 * ks) ^ (4 * (i & 1));
-        fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off[c]);
-        fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off[c]);
+        fa[i] = *reinterpret_cast<const v4i*>(st + a_base + i * 32 * BK + frag_off(c));
+        fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off(c));
       }
       // the first MFMA of a group starts from a zero accumulator operand instead of zeroed registers
-      const bool fresh = ks == 0 && (ONE || (s % g.stages_per_group) == 0);
+      const bool fresh = ks == 0 && pos == 0;
 #pragma unroll
       for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
@@ -205,40 +454,22 @@ void gemm_grouped_kernel(const GroupedArgs g) {
         }
     }
     if (last_of_group) {
-      // lane holds C[m = mi*32 + lr][n = ni*32 + 8q + 4lh + e], register 4q + e
+      // lane holds C[m = wm*64 + mi*32 + lr][n = wn*64 + ni*32 + 8q + 4lh + e], register 4q + e
       const int buf = grp & 1;
-      float rs[2];
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi) rs[mi] = srow[buf][wm * 64 + mi * 32 + lr];
+      const float rs[2] = {srow[buf][wm * 64 + lr], srow[buf][wm * 64 + 32 + lr]};
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float4 cs4 = *reinterpret_cast<const float4*>(&scol[buf][wn * 64 + ni * 32 + 8 * q + 4 * lh]);
-          const float cs[4] = {cs4.x, cs4.y, cs4.z, cs4.w};
-#pragma unroll
-          for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-            for (int e = 0; e < 4; e += 2) {
-              // every product and the sum round on their own (the library is built with
-              // floating-point contraction off, so no fused multiply-add appears here); values
-              // are rounded two at a time (one packed conversion per pair)
-              float f0 = (float)acc[mi][ni][4 * q + e], f1 = (float)acc[mi][ni][4 * q + e + 1];
-              round_pair<kOutBf16>(f0, f1);
-              f0 *= rs[mi]; f1 *= rs[mi];
-              round_pair<kP1Bf16>(f0, f1);
-              f0 *= cs[e]; f1 *= cs[e + 1];
-              round_pair<kP2Bf16>(f0, f1);
-              if constexpr (kOutBf16 && !kP2Bf16) round_pair<true>(f0, f1);  // final cast of the tile
-              sum[mi][ni][4 * q + e] += f0;
-              sum[mi][ni][4 * q + e + 1] += f1;
-            }
+          const v16i* const a2[2] = {&acc[0][ni], &acc[1][ni]};
+          v16f* const s2[2] = {&sum[0][ni], &sum[1][ni]};
+          R::template quarter<2>(a2, s2, q, rs, *reinterpret_cast<const float4*>(&scol[buf][wn * 64 + ni * 32 + 8 * q + 4 * lh]));
         }
     }
     // the registers of stage s + 1 (requested a whole stage ago) go to the buffer stage s - 1 left;
     // the barrier is a bare s_barrier: a __syncthreads() would also wait for the loads of s + 2
     if (s + 1 < nstages) store_stage(set, stage_mem[(s + 1) & 1]);
-    if (last_of_group) store_scales((grp + 1) & 1);
+    if (last_of_group) sc.store(tid, srow[(grp + 1) & 1], scol[(grp + 1) & 1]);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -248,41 +479,14 @@ void gemm_grouped_kernel(const GroupedArgs g) {
     if (s + 1 < nstages) stage(s + 1, 0);
   }
 
-  // ---- output --------------------------------------------------------------------------------
-  constexpr int kEsz = kOutBf16 ? 2 : 4;
-  uint8_t* cb = reinterpret_cast<uint8_t*>(g.c);
-  const bool vec = (g.ldc % 4) == 0 && ((uintptr_t)cb % 16) == 0;
+  const bool vec = (g.ldc % 4) == 0 && ((uintptr_t)g.c % 16) == 0;
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi) {
-    const int64_t mm = m0 + wm * 64 + mi * 32 + lr;
-    if (mm >= g.m) continue;
+  for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
     for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t nn = n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh;
-        if (nn >= g.n) continue;
-        float o[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = round_to<kOutBf16>(sum[mi][ni][4 * q + e]);
-        uint8_t* dst = cb + (mm * g.ldc + nn) * kEsz;
-        if (vec && nn + 4 <= g.n) {
-          if constexpr (kOutBf16) {
-            uint2 w;
-            w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
-            w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
-            *reinterpret_cast<uint2*>(dst) = w;
-          } else {
-            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-          }
-        } else {
-          for (int e = 0; e < 4 && nn + e < g.n; ++e) {
-            if constexpr (kOutBf16) reinterpret_cast<uint16_t*>(dst)[e] = bf16_bits(o[e]);
-            else reinterpret_cast<float*>(dst)[e] = o[e];
-          }
-        }
-      }
-  }
+      for (int q = 0; q < 4; ++q)
+        store_out4<R::kOutBf16>(g, sum[mi][ni], q, m0 + wm * 64 + mi * 32 + lr, n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh, vec);
 }
 
 // [n][k] int4 values in int8 bytes -> [n][k/2] packed, low nibble = even k.
@@ -333,6 +537,10 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   AQTX_REQUIRE(p->k > 0, "aqtx_gemm_i8_grouped: empty contraction");
   AQTX_REQUIRE((p->lda % 16 == 0) && (p->ldb % 16 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0),
                "aqtx_gemm_i8_grouped: operands must be 16-byte aligned with leading dimensions multiple of 16");
+  const bool group128 = p->group == 128;
+  const int GN = grouped_cols(group128);
+  AQTX_REQUIRE(!group128 || (p->k / 128) * (p->m > p->n ? p->m : p->n) * 4 < (1ll << 31),
+               "aqtx_gemm_i8_grouped: a scale array of more than 2 GiB");
   AQTX_REQUIRE(p->lda * (int64_t)GM < (1ll << 31) && p->ldb * (int64_t)GN < (1ll << 31),
                "aqtx_gemm_i8_grouped: leading dimension too large for 32-bit tile offsets");
   const size_t esz = p->out_dtype == AQTX_BF16 ? 2 : 4;
@@ -353,14 +561,12 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   else epi = p->col_scale_dtype == AQTX_BF16 ? 0 : 4;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n));
-  // the compile-time form of the one-stage group costs the unpacked variant a few spilled registers
-  const bool one = g.stages_per_group == 1 && packed;
-#define AQTX_LAUNCH(E)                                                       \
-  do {                                                                      \
-    if (packed && one) gemm_grouped_kernel<E, true, true><<<grid, 512, 0, st>>>(g);         \
-    else if (packed) gemm_grouped_kernel<E, true, false><<<grid, 512, 0, st>>>(g);          \
-    else if (one) gemm_grouped_kernel<E, false, true><<<grid, 512, 0, st>>>(g);             \
-    else gemm_grouped_kernel<E, false, false><<<grid, 512, 0, st>>>(g);                     \
+#define AQTX_LAUNCH(E)                                                                      \
+  do {                                                                                     \
+    if (packed && group128) gemm_grouped128_kernel<E, true><<<grid, 512, 0, st>>>(g);       \
+    else if (group128) gemm_grouped128_kernel<E, false><<<grid, 512, 0, st>>>(g);           \
+    else if (packed) gemm_grouped_kernel<E, true><<<grid, 512, 0, st>>>(g);                 \
+    else gemm_grouped_kernel<E, false><<<grid, 512, 0, st>>>(g);                            \
   } while (0)
   switch (epi) {
     case 0: AQTX_LAUNCH(0); break;
