@@ -275,11 +275,12 @@ __device__ __forceinline__ float segment_max(float v, float* smem) {
   constexpr int W = LANES < 64 ? LANES : 64;
 #pragma unroll
   for (int off = W / 2; off > 0; off >>= 1) v = nanmax(v, __shfl_xor(v, off, W));
-  if constexpr (LANES == 256) {
+  if constexpr (LANES >= 256) {  // the segment is the whole block
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) smem[wave] = v;
     __syncthreads();
     v = nanmax(nanmax(smem[0], smem[1]), nanmax(smem[2], smem[3]));
+    if constexpr (LANES == 512) v = nanmax(v, nanmax(nanmax(smem[4], smem[5]), nanmax(smem[6], smem[7])));
   }
   return v;
 }
@@ -330,13 +331,18 @@ __device__ __forceinline__ uint32_t packed_absmax(uint32_t m, uint32_t w) {
 // ---- rows kernel: reduced axis contiguous -------------------------------------
 // PAIR (SPEC 2 only): the block owns segment s and segment s + nseg/2, whose elements share
 // threefry blocks; requires whole rows as segments and the natural noise layout.
+// A block is 256 threads, or 512 (LANES = 512: one long segment per block, half the row values per
+// thread, so that six waves fit a SIMD: the stochastic pipeline is bound by vector instruction
+// issue, and a wave issues one such instruction every ~12 cycles at best).
 template <typename TIn, int LANES, int ITERS, int SPEC, bool PAIR>
-__global__ __launch_bounds__(256, (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1) void quant_rows_kernel(const QArgs a_in) {
+__global__ __launch_bounds__(LANES == 512 ? 512 : 256, LANES == 512 ? 3 : (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1)
+void quant_rows_kernel(const QArgs a_in) {
   const QArgs a = with_device_key(a_in);
   constexpr int VEC = 8;
-  constexpr int SEG_PER_BLOCK = 256 / LANES;
+  constexpr int NT = LANES == 512 ? 512 : 256;
+  constexpr int SEG_PER_BLOCK = NT / LANES;
   constexpr int NSET = PAIR ? 2 : 1;
-  __shared__ float smem[NSET][4];
+  __shared__ float smem[NSET][NT / 64];
   const int tid = threadIdx.x;
   const int lane = tid % LANES;
   const int64_t nseg_grid = PAIR ? a.nseg / 2 : a.nseg;
@@ -913,8 +919,9 @@ int launch_rows_spec(const QArgs& a, hipStream_t st) {
   const int64_t nseg = PAIR ? a.nseg / 2 : a.nseg;
 #define AQTX_ROWS(LANES, ITERS)                                                        \
   {                                                                                    \
-    const int64_t blocks = (nseg + (256 / LANES) - 1) / (256 / LANES);                 \
-    quant_rows_kernel<TIn, LANES, ITERS, SPEC, PAIR><<<dim3((unsigned)blocks), 256, 0, st>>>(a); \
+    constexpr int kThreads = LANES == 512 ? 512 : 256;                                 \
+    const int64_t blocks = (nseg + (kThreads / LANES) - 1) / (kThreads / LANES);       \
+    quant_rows_kernel<TIn, LANES, ITERS, SPEC, PAIR><<<dim3((unsigned)blocks), kThreads, 0, st>>>(a); \
     AQTX_HIP_CHECK_LAUNCH("quant_rows_kernel");                                        \
     return 0;                                                                          \
   }
@@ -923,6 +930,7 @@ int launch_rows_spec(const QArgs& a, hipStream_t st) {
   if (L <= 2048) AQTX_ROWS(256, 1)
   if (L <= 4096) AQTX_ROWS(256, 2)
   if (L <= 8192) AQTX_ROWS(256, 4)
+  if (SPEC == 2 && sizeof(TIn) == 2) AQTX_ROWS(512, 4)
   AQTX_ROWS(256, 8)
 #undef AQTX_ROWS
 }
