@@ -16,6 +16,7 @@ NOISE_NONE, NOISE_JAX_UNIFORM, NOISE_CUSTOM1, NOISE_FP8_MANTISSA = range(4)
 PRESCALE_NONE, PRESCALE_PER_ROW, PRESCALE_PER_COL = range(3)
 SCALE_ROW_THEN_COL, SCALE_COL_THEN_ROW = range(2)
 W_ROWS, W_FRAGMENTS = range(2)
+K_NATURAL, K_EVEN_ODD8 = range(2)
 
 
 class QuantPlan(ctypes.Structure):
@@ -35,6 +36,7 @@ class QuantPlan(ctypes.Structure):
       ('scale_typed', ctypes.c_void_p),
       ('workspace_zeroed', ctypes.c_int32),
       ('key_device', ctypes.c_void_p),
+      ('out_k_order', ctypes.c_int32),
   ]
 
 
@@ -59,6 +61,7 @@ class GroupedGemmPlan(ctypes.Structure):
       ('lda', ctypes.c_int64), ('ldb', ctypes.c_int64), ('ldc', ctypes.c_int64),
       ('a_dtype', ctypes.c_int32), ('b_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
       ('row_scale_dtype', ctypes.c_int32), ('col_scale_dtype', ctypes.c_int32),
+      ('a_k_order', ctypes.c_int32), ('row_scale_by_row', ctypes.c_int32),
   ]
 
 

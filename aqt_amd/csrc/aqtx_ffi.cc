@@ -57,8 +57,8 @@ ffi::Error QuantizeCommon(hipStream_t stream, ffi::AnyBuffer x, const float* pre
                           ffi::Result<ffi::Buffer<ffi::U8>> workspace, int32_t compute_dtype, int32_t scale_dtype,
                           int32_t out_dtype, int32_t reduce, int32_t transpose_out, int64_t group, float quant_bound,
                           float clip_bound, int32_t noise, int32_t partitionable, int64_t noise_stride_batch,
-                          int64_t noise_stride_row, int64_t noise_stride_col, int64_t noise_total, int32_t prescale_mode,
-                          int64_t prescale_stride_batch) {
+                          int64_t noise_stride_row, int64_t noise_stride_col, int64_t noise_total, int32_t out_k_order,
+                          int32_t prescale_mode, int64_t prescale_stride_batch) {
   auto dims = x.dimensions();
   if (dims.size() != 3) return Bad("aqtx_quantize: x must be [batch, rows, cols]");
   if (key.element_count() != 2) return Bad("aqtx_quantize: key must be uint32[2]");
@@ -79,6 +79,7 @@ ffi::Error QuantizeCommon(hipStream_t stream, ffi::AnyBuffer x, const float* pre
   p.noise_stride_row = noise_stride_row;
   p.noise_stride_col = noise_stride_col;
   p.noise_total = noise_total;
+  p.out_k_order = out_k_order;
   p.prescale = prescale_mode;
   p.prescale_stride_batch = prescale_stride_batch;
   p.key_device = noise != AQTX_NOISE_NONE ? key.typed_data() : nullptr;
@@ -91,10 +92,10 @@ ffi::Error QuantizeImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi::U
                         int32_t compute_dtype, int32_t scale_dtype, int32_t out_dtype, int32_t reduce,
                         int32_t transpose_out, int64_t group, float quant_bound, float clip_bound, int32_t noise,
                         int32_t partitionable, int64_t noise_stride_batch, int64_t noise_stride_row,
-                        int64_t noise_stride_col, int64_t noise_total) {
+                        int64_t noise_stride_col, int64_t noise_total, int32_t out_k_order) {
   return QuantizeCommon(stream, x, nullptr, key, q, scale, workspace, compute_dtype, scale_dtype, out_dtype, reduce,
                         transpose_out, group, quant_bound, clip_bound, noise, partitionable, noise_stride_batch,
-                        noise_stride_row, noise_stride_col, noise_total, AQTX_PRESCALE_NONE, 0);
+                        noise_stride_row, noise_stride_col, noise_total, out_k_order, AQTX_PRESCALE_NONE, 0);
 }
 
 // The gradient side of a backward contraction: x := x * cast(prescale) first
@@ -106,11 +107,11 @@ ffi::Error QuantizePrescaledImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::Buff
                                  int32_t transpose_out, int64_t group, float quant_bound, float clip_bound,
                                  int32_t noise, int32_t partitionable, int64_t noise_stride_batch,
                                  int64_t noise_stride_row, int64_t noise_stride_col, int64_t noise_total,
-                                 int32_t prescale_mode, int64_t prescale_stride_batch) {
+                                 int32_t out_k_order, int32_t prescale_mode, int64_t prescale_stride_batch) {
   return QuantizeCommon(stream, x, prescale.typed_data(), key, q, scale, workspace, compute_dtype, scale_dtype,
                         out_dtype, reduce, transpose_out, group, quant_bound, clip_bound, noise, partitionable,
-                        noise_stride_batch, noise_stride_row, noise_stride_col, noise_total, prescale_mode,
-                        prescale_stride_batch);
+                        noise_stride_batch, noise_stride_row, noise_stride_col, noise_total, out_k_order,
+                        prescale_mode, prescale_stride_batch);
 }
 
 // ---- aqtx_dequantize ----------------------------------------------------------------------------
@@ -186,10 +187,12 @@ ffi::Error GemmFp8Impl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b, f
 }
 
 // ---- aqtx_gemm_i8_grouped -----------------------------------------------------------------------
-// a int8 [m, k]; b int8 [n, k] or packed int4 uint8 [n, k/2]; scales f32 [k/group, m], [k/group, n].
+// a int8 [m, k]; b int8 [n, k] or packed int4 uint8 [n, k/2]; scales f32 [k/group, m] (or [m, k/group] with
+// row_scale_by_row), [k/group, n].
 ffi::Error GemmI8GroupedImpl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b, ffi::Buffer<ffi::F32> row_scale,
                              ffi::Buffer<ffi::F32> col_scale, ffi::Result<ffi::AnyBuffer> c, int64_t group,
-                             int32_t a_dtype, int32_t b_dtype, int32_t row_scale_dtype, int32_t col_scale_dtype) {
+                             int32_t a_dtype, int32_t b_dtype, int32_t row_scale_dtype, int32_t col_scale_dtype,
+                             int32_t a_k_order, int32_t row_scale_by_row) {
   auto ad = a.dimensions(), bd = b.dimensions();
   if (ad.size() != 2 || bd.size() != 2) return Bad("aqtx_gemm_i8_grouped: operands must be [m, k] and [n, k]");
   aqtx_grouped_gemm_plan p{};
@@ -199,6 +202,7 @@ ffi::Error GemmI8GroupedImpl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffe
   p.a_dtype = a_dtype; p.b_dtype = b_dtype;
   p.out_dtype = Dtype(c->element_type());
   p.row_scale_dtype = row_scale_dtype; p.col_scale_dtype = col_scale_dtype;
+  p.a_k_order = a_k_order; p.row_scale_by_row = row_scale_by_row;
   return Status(aqtx_gemm_i8_grouped(&p, a.untyped_data(), b.untyped_data(), row_scale.typed_data(),
                                      col_scale.typed_data(), c->untyped_data(), stream));
 }
@@ -247,7 +251,7 @@ ffi::Error SumTilesImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::Result<ffi::A
   .Attr<int32_t>("reduce").Attr<int32_t>("transpose_out").Attr<int64_t>("group")                       \
   .Attr<float>("quant_bound").Attr<float>("clip_bound").Attr<int32_t>("noise")                         \
   .Attr<int32_t>("partitionable").Attr<int64_t>("noise_stride_batch").Attr<int64_t>("noise_stride_row") \
-  .Attr<int64_t>("noise_stride_col").Attr<int64_t>("noise_total")
+  .Attr<int64_t>("noise_stride_col").Attr<int64_t>("noise_total").Attr<int32_t>("out_k_order")
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxQuantize, QuantizeImpl,
@@ -325,7 +329,8 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Arg<ffi::Buffer<ffi::F32>>()
         .Ret<ffi::AnyBuffer>()
         .Attr<int64_t>("group").Attr<int32_t>("a_dtype").Attr<int32_t>("b_dtype")
-        .Attr<int32_t>("row_scale_dtype").Attr<int32_t>("col_scale_dtype"));
+        .Attr<int32_t>("row_scale_dtype").Attr<int32_t>("col_scale_dtype")
+        .Attr<int32_t>("a_k_order").Attr<int32_t>("row_scale_by_row"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxDecodeI8, DecodeI8Impl,

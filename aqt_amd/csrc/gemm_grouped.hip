@@ -62,6 +62,8 @@ struct GroupedArgs {
   int64_t m, n, k, lda, ldb, ldc;
   int groups, stages_per_group;
   int tiles_m, tiles_n;
+  int a_even_odd8;   // A's bytes of every 8 k are stored as k 0,2,4,6,1,3,5,7 (packed B only)
+  int rs_by_row;     // row_scale is [m][groups] instead of [groups][m]
 };
 
 __device__ __forceinline__ int row_swz(int row) { return (row ^ (row >> 3)) & 7; }
@@ -69,7 +71,18 @@ __device__ __forceinline__ int row_swz(int row) { return (row ^ (row >> 3)) & 7;
 // 16 bytes of packed int4 (32 values, low nibble = even k) -> 32 bytes of values * 16 in k order.
 // dword d of the load = k 8d..8d+7: even k: (x << 4) & 0xF0F0F0F0, odd k: x & 0xF0F0F0F0; then
 // the bytes are interleaved back to k order.
-__device__ __forceinline__ void unpack_i4x32(const v4i x4, v4i& lo, v4i& hi) {
+// With even_odd8 the other operand stores every 8 k as k 0,2,4,6,1,3,5,7, and the interleaving is left out.
+__device__ __forceinline__ void unpack_i4x32(const v4i x4, v4i& lo, v4i& hi, int even_odd8) {
+  if (even_odd8) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t x = (uint32_t)x4[d];
+      const int ev = (int)((x << 4) & 0xF0F0F0F0u), od = (int)(x & 0xF0F0F0F0u);
+      if (d < 2) { lo[2 * d] = ev; lo[2 * d + 1] = od; }
+      else { hi[2 * (d - 2)] = ev; hi[2 * (d - 2) + 1] = od; }
+    }
+    return;
+  }
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
     const uint32_t x = (uint32_t)x4[d];
@@ -146,7 +159,7 @@ __device__ __forceinline__ void store_out4(const GroupedArgs& g, const v16f& sum
 template <int GN, bool PACKED>
 struct ScaleFetch {
   const float* ptr;
-  int64_t len;
+  int64_t len;  // elements from one group's scale to the next
   float reg = 1.0f;
   bool row, inside, valid = false, active;
   int groups;
@@ -154,9 +167,11 @@ struct ScaleFetch {
     row = tid < GM;
     active = tid < GM + GN;
     const int64_t idx = row ? m0 + tid : n0 + (tid - GM);
-    len = row ? g.m : g.n;
-    inside = active && idx < len;
-    ptr = (row ? g.row_scale : g.col_scale) + (inside ? idx : 0);
+    const int64_t n_idx = row ? g.m : g.n;
+    inside = active && idx < n_idx;
+    const bool by_idx = row && g.rs_by_row;  // [idx][group] instead of [group][idx]
+    ptr = (row ? g.row_scale : g.col_scale) + (inside ? idx : 0) * (by_idx ? g.groups : 1);
+    len = by_idx ? 1 : n_idx;
     groups = g.groups;
   }
   // called for grp = 0, 1, 2, ... in order: the pointer moves on by one group per call and stops
@@ -219,14 +234,17 @@ void gemm_grouped128_kernel(const GroupedArgs g) {
   const int sc_idx = (tid & 127);
   const int64_t sc_len = sc_row ? g.m : g.n, sc_first = sc_row ? m0 : n0;
   const bool sc_inside = sc_active && sc_first + sc_idx < sc_len;
+  const bool sc_by_idx = sc_row && g.rs_by_row;  // [row][group] instead of [group][row]
+  const int64_t sc_skip = sc_first * (sc_by_idx ? g.groups : 1);
   const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)((sc_row ? g.row_scale : g.col_scale) + sc_first), 0, (int)(((int64_t)g.groups * sc_len - sc_first) * 4),
+      (void*)((sc_row ? g.row_scale : g.col_scale) + sc_skip), 0, (int)(((int64_t)g.groups * sc_len - sc_skip) * 4),
       kBufferRsrcWord3);
-  const int sc_step = (int)sc_len * 4;  // bytes from one group's scales to the next
+  const int sc_step = sc_by_idx ? 4 : (int)sc_len * 4;  // bytes from one group's scale to the next
+  const int sc_voff = sc_idx * (sc_by_idx ? g.groups * 4 : 4);
   float sc_reg = 1.0f;
   auto load_scales = [&](int grp) {  // lanes past the operand read another row's scale or zero; store_scales masks them
     const int grp_c = grp < g.groups ? grp : g.groups - 1;
-    if (sc_active) sc_reg = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, sc_idx * 4, grp_c * sc_step, 0));
+    if (sc_active) sc_reg = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, sc_voff, grp_c * sc_step, 0));
   };
   auto store_scales = [&](int grp, int buf) {
     asm volatile("" : "+v"(sc_reg));  // keeps the arithmetic on the loaded value down here
@@ -258,7 +276,7 @@ void gemm_grouped128_kernel(const GroupedArgs g) {
     for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
     if constexpr (PACKED) {
       v4i lo, hi;
-      unpack_i4x32(stg[NLA], lo, hi);
+      unpack_i4x32(stg[NLA], lo, hi, g.a_even_odd8);
       *reinterpret_cast<v4i*>(st + st_b) = lo;
       *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
     } else {
@@ -395,7 +413,7 @@ void gemm_grouped_kernel(const GroupedArgs g) {
       if constexpr (PACKED) {
         const int row = (wave * NLB + i) * 16 + (lane >> 2), p = lane & 3;
         v4i lo, hi;
-        unpack_i4x32(stb[set][i], lo, hi);
+        unpack_i4x32(stb[set][i], lo, hi, g.a_even_odd8);
         uint8_t* rowp = st + kATile + row * BK;
         *reinterpret_cast<v4i*>(rowp + (((2 * p) ^ row_swz(row)) * 16)) = lo;
         *reinterpret_cast<v4i*>(rowp + (((2 * p + 1) ^ row_swz(row)) * 16)) = hi;
@@ -555,6 +573,10 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   g.stages_per_group = (int)(p->group / 128);
   g.tiles_m = (int)((p->m + GM - 1) / GM);
   g.tiles_n = (int)((p->n + GN - 1) / GN);
+  AQTX_REQUIRE(p->a_k_order == AQTX_K_NATURAL || (p->a_k_order == AQTX_K_EVEN_ODD8 && packed),
+               "aqtx_gemm_i8_grouped: a_k_order must be AQTX_K_NATURAL, or AQTX_K_EVEN_ODD8 with a packed int4 b");
+  g.a_even_odd8 = p->a_k_order == AQTX_K_EVEN_ODD8;
+  g.rs_by_row = p->row_scale_by_row != 0;
   int epi;
   if (p->out_dtype == AQTX_F32) epi = 2;
   else if (p->row_scale_dtype != AQTX_BF16) epi = 1;

@@ -51,6 +51,7 @@ struct QArgs {
   int sbf;  // scale dtype is bf16
   int scale_given;
   int ws_zeroed;  // the abs-max words of the workspace are zero on entry
+  int even_odd8;  // rows kernel: bytes of each group of 8 outputs stored as elements 0,2,4,6,1,3,5,7
 };
 
 // Kernel-side copy of the arguments with the PRNG key taken from device memory when the caller
@@ -328,6 +329,13 @@ __device__ __forceinline__ uint32_t packed_absmax(uint32_t m, uint32_t w) {
   return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
 }
 
+// Eight output bytes -> two words, in element order or as elements 0,2,4,6 | 1,3,5,7.
+__device__ __forceinline__ uint2 pack8(const uint32_t (&q)[8], int even_odd8) {
+  if (even_odd8)
+    return make_uint2(q[0] | (q[2] << 8) | (q[4] << 16) | (q[6] << 24), q[1] | (q[3] << 8) | (q[5] << 16) | (q[7] << 24));
+  return make_uint2(q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24), q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24));
+}
+
 // ---- rows kernel: reduced axis contiguous -------------------------------------
 // PAIR (SPEC 2 only): the block owns segment s and segment s + nseg/2, whose elements share
 // threefry blocks; requires whole rows as segments and the natural noise layout.
@@ -426,19 +434,15 @@ void quant_rows_kernel(const QArgs a_in) {
     for (int it = 0; it < ITERS; ++it) {
       const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
       if (active && j0 < a.L) {
-        uint32_t w0[2] = {0u, 0u}, w1[2] = {0u, 0u};
+        uint32_t q0[VEC], q1[VEC];
         float t0[VEC], t1[VEC];
         v[0][it].get(t0);
         v[1][it].get(t1);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          uint32_t q0, q1;
-          pair_quant(t0[e], inv[0], t1[e], inv[1], ctr_row + (uint32_t)(j0 + e), a, q0, q1);
-          w0[e >> 2] |= q0 << (8 * (e & 3));
-          w1[e >> 2] |= q1 << (8 * (e & 3));
-        }
-        *reinterpret_cast<uint2*>(qp0 + j0) = make_uint2(w0[0], w0[1]);
-        *reinterpret_cast<uint2*>(qp1 + j0) = make_uint2(w1[0], w1[1]);
+        for (int e = 0; e < VEC; ++e)
+          pair_quant(t0[e], inv[0], t1[e], inv[1], ctr_row + (uint32_t)(j0 + e), a, q0[e], q1[e]);
+        *reinterpret_cast<uint2*>(qp0 + j0) = pack8(q0, a.even_odd8);
+        *reinterpret_cast<uint2*>(qp1 + j0) = pack8(q1, a.even_odd8);
       }
     }
   } else {
@@ -448,14 +452,12 @@ void quant_rows_kernel(const QArgs a_in) {
     for (int it = 0; it < ITERS; ++it) {
       const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
       if (active && j0 < a.L) {
-        uint32_t w[2] = {0u, 0u};
+        uint32_t q[VEC];
         float t[VEC];
         v[0][it].get(t);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e)
-          w[e >> 2] |= spec_quant<SPEC>(t[e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a)
-                       << (8 * (e & 3));
-        *reinterpret_cast<uint2*>(qp0 + j0) = make_uint2(w[0], w[1]);
+        for (int e = 0; e < VEC; ++e) q[e] = spec_quant<SPEC>(t[e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a);
+        *reinterpret_cast<uint2*>(qp0 + j0) = pack8(q, a.even_odd8);
       }
     }
   }
@@ -940,6 +942,8 @@ int launch_rows(const QArgs& a, int partitionable, hipStream_t st) {
   const int64_t L = a.L;
   const bool aligned = (L % 8 == 0) && (a.cols % 8 == 0);
   if (!aligned || L > 16384) {
+    AQTX_REQUIRE(!a.even_odd8, "aqtx_quantize: out_k_order = EVEN_ODD8 needs cols and group to be multiples of 8 and "
+                 "segments of at most 16384");
     const int64_t blocks = (a.nseg + 3) / 4;
     quant_rows_generic_kernel<TIn><<<dim3((unsigned)blocks), 256, 0, st>>>(a);
     AQTX_HIP_CHECK_LAUNCH("quant_rows_generic_kernel");
@@ -1043,7 +1047,8 @@ using namespace aqtx;
 // path, which spreads every entry over many workgroups.  Returns true and fills `q` if `p` is
 // such a plan.
 static bool long_rows_as_batches(const aqtx_quant_plan* p, aqtx_quant_plan* q) {
-  if (p->reduce != AQTX_REDUCE_COLS || p->group != 0 || p->transpose_out || p->prescale != AQTX_PRESCALE_NONE)
+  if (p->reduce != AQTX_REDUCE_COLS || p->group != 0 || p->transpose_out || p->prescale != AQTX_PRESCALE_NONE ||
+      p->out_k_order != AQTX_K_NATURAL)
     return false;
   if (p->batch <= 0 || p->rows <= 0 || p->batch * p->rows > 512 || p->cols < 16384) return false;
   if (p->noise != AQTX_NOISE_NONE && p->batch > 1 && p->noise_stride_batch != p->rows * p->noise_stride_row)
@@ -1109,6 +1114,14 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
   a.cbf = p->compute_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
   a.scale_given = p->scale_given;
   a.ws_zeroed = p->workspace_zeroed;
+  AQTX_REQUIRE(p->out_k_order == AQTX_K_NATURAL || p->out_k_order == AQTX_K_EVEN_ODD8,
+               "aqtx_quantize: unknown out_k_order %d", p->out_k_order);
+  if (p->out_k_order == AQTX_K_EVEN_ODD8) {
+    AQTX_REQUIRE(p->reduce == AQTX_REDUCE_COLS && !p->transpose_out &&
+                     (p->out_dtype == AQTX_I8 || p->out_dtype == AQTX_I4),
+                 "aqtx_quantize: out_k_order = EVEN_ODD8 needs AQTX_REDUCE_COLS, an integer out_dtype and no transpose_out");
+    a.even_odd8 = 1;
+  }
   if (p->noise != AQTX_NOISE_NONE) {
     a.gen = make_bitgen(p->key, p->noise_total, noise_width(p), p->partitionable);
     a.key_dev = p->key_device;

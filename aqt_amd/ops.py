@@ -153,6 +153,7 @@ def quantize(
     scale: Optional[torch.Tensor] = None,
     want_typed_scale: bool = False,
     key_device: Optional[torch.Tensor] = None,
+    k_order: int = 0,
 ):
   """Calibrate (abs-max) and quantize a contiguous [batch, rows, cols] tensor.
 
@@ -161,6 +162,8 @@ def quantize(
   float32, shaped [batch, rows, cols/group] (REDUCE_COLS),
   [batch, rows/group, cols] (REDUCE_ROWS) or [batch] (REDUCE_ALL).
   `key_device` (a 2-word device tensor) replaces `key`: the kernels read the key from device memory.
+  `k_order` = L.K_EVEN_ODD8 stores every aligned group of 8 values along cols as elements
+  0,2,4,6,1,3,5,7 (the lhs of gemm_grouped against a packed int4 rhs).
   With want_typed_scale a third element: the computed scales once more as a bf16 tensor of
   the same shape, written by the same kernels (None unless the scale dtype is bf16 and the
   scale is computed here).
@@ -192,6 +195,7 @@ def quantize(
   if prescale is not None and prescale.dim() == 2 and prescale.shape[0] == b and b > 1:
     plan.prescale_stride_batch = prescale.shape[1]
   plan.scale_given = int(scale is not None)
+  plan.out_k_order = k_order
 
   if reduce == L.REDUCE_COLS:
     sshape = (b, r, c // group if group else 1)
@@ -407,17 +411,19 @@ def pack_i4(q: torch.Tensor) -> torch.Tensor:
 
 def gemm_grouped(a: torch.Tensor, b: torch.Tensor, *, row_scale: torch.Tensor, col_scale: torch.Tensor,
                  group: int, out_dtype, row_scale_dtype=None, col_scale_dtype=None, a_dtype: int = L.I8,
-                 b_dtype: int = L.I8):
+                 b_dtype: int = L.I8, a_k_order: int = 0, row_scale_by_row: bool = False):
   """C = cast(sum_g dequant_g(A_g @ B_g^T)) for A int8 [m, k], B int8 [n, k] (or packed int4
-  uint8 [n, k/2] with b_dtype=I4P), row_scale float32 [k/group, m], col_scale float32 [k/group, n]."""
+  uint8 [n, k/2] with b_dtype=I4P), row_scale float32 [k/group, m] ([m, k/group] with
+  row_scale_by_row), col_scale float32 [k/group, n].  a_k_order = L.K_EVEN_ODD8: A was written by
+  quantize(k_order=L.K_EVEN_ODD8) (packed rhs only)."""
   _require_gpu(a, b, row_scale, col_scale)
   m, k = a.shape
   n = b.shape[0]
   packed = b_dtype == L.I4P
   assert a.stride(1) == 1 and b.stride(1) == 1 and b.shape[1] == (k // 2 if packed else k)
   groups = k // group
-  for s_, dim in ((row_scale, m), (col_scale, n)):
-    assert s_.dtype == torch.float32 and s_.is_contiguous() and tuple(s_.shape) == (groups, dim), tuple(s_.shape)
+  for s_, shape in ((row_scale, (m, groups) if row_scale_by_row else (groups, m)), (col_scale, (groups, n))):
+    assert s_.dtype == torch.float32 and s_.is_contiguous() and tuple(s_.shape) == shape, tuple(s_.shape)
   out_dt = aqtx_dtype(out_dtype)
   plan = L.GroupedGemmPlan()
   plan.m, plan.n, plan.k, plan.group = m, n, k, group
@@ -425,6 +431,7 @@ def gemm_grouped(a: torch.Tensor, b: torch.Tensor, *, row_scale: torch.Tensor, c
   plan.a_dtype, plan.b_dtype, plan.out_dtype = a_dtype, b_dtype, out_dt
   plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else out_dt
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else out_dt
+  plan.a_k_order, plan.row_scale_by_row = a_k_order, int(row_scale_by_row)
   c = torch.empty((m, n), dtype=_AQTX_TO_TORCH[out_dt], device=a.device)
   with _timed('gemm_grouped'):
     L.check(L.lib().aqtx_gemm_i8_grouped(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale),

@@ -494,9 +494,9 @@ def _kernel_layout_of(qvalue: torch.Tensor, v: 'lowering.OperandView', pack_int4
   return q
 
 
-def _scale_vector_f32(scale: torch.Tensor, ba, ra, ca) -> torch.Tensor:
-  """A frozen operand's scale as the flat float32 vector the kernels read.  A scale kept in
-  another dtype is converted once per tensor, not on every call."""
+def _scale_f32(scale: torch.Tensor) -> torch.Tensor:
+  """A frozen operand's scale in float32, same shape.  A scale kept in another dtype is converted
+  once per tensor, not on every call."""
   src = getattr(scale, 'f32_copy', None)
   if src is None:
     src = scale
@@ -510,7 +510,12 @@ def _scale_vector_f32(scale: torch.Tensor, ba, ra, ca) -> torch.Tensor:
       if hit is None:
         weakref.finalize(scale, _KERNEL_LAYOUT_CACHE.pop, id(scale), None)
       _KERNEL_LAYOUT_CACHE[id(scale)] = (key, src)
-  return lowering.view_operand(src, ba, ra, ca).mem.reshape(-1).contiguous()
+  return src
+
+
+def _scale_vector_f32(scale: torch.Tensor, ba, ra, ca) -> torch.Tensor:
+  """A frozen operand's scale as the flat float32 vector the kernels read."""
+  return lowering.view_operand(_scale_f32(scale), ba, ra, ca).mem.reshape(-1).contiguous()
 
 
 _POISON = ('Poison. Gradients are not generally expected in serving. Please set '
@@ -1053,7 +1058,7 @@ class DotGeneral:
     return out, qret
 
   def fused_tile_sum(self, lhs, rhs, dimension_numbers, n_sum_axes: int, lhs_qt=None, rhs_qt=None,
-                     with_qt: bool = False):
+                     with_qt: bool = False, lhs_qvalue_needed: bool = True):
     """sum over the leading `n_sum_axes` output axes of self(lhs, rhs, dimension_numbers), fused.
 
     This is what tiled_dot_general asks of its inner dot_general when the contraction axis is
@@ -1064,7 +1069,8 @@ class DotGeneral:
     may be a frozen weight (the serving case): it is read in the kernel's layout, an int4 one
     packed two values per byte, both made once per frozen tensor.  Returns None when the call
     does not have that shape (the caller then takes the unfused route); with `with_qt`,
-    (out, (lhs QTensor, rhs QTensor)) like dg_core.
+    (out, (lhs QTensor, rhs QTensor)) like dg_core; a caller that will only look at the lhs
+    QTensor's scales says so with lhs_qvalue_needed=False (it then comes without its qvalue).
     """
     if n_sum_axes != 1 or torch.is_grad_enabled() and (lhs.requires_grad or rhs.requires_grad):
       return None
@@ -1111,19 +1117,22 @@ class DotGeneral:
         return None
     self.assert_config_validity()
     sdt_l = dq.lhs._calibrator.dtype if dq.lhs._calibrator.dtype is not None else lhs.dtype
+    rra = list(range(2, nr))
+    int4 = frozen and rhs_qt.container_dtype is utils.int4
+    packed = int4 and (T * ts) % 32 == 0
+    # Against a packed weight, and when nobody asks for the quantized activation itself, the
+    # activation is written with every 8 k in even-odd order: the kernel then takes the weight's
+    # nibbles as they lie instead of interleaving them again.
+    k_order = L.K_EVEN_ODD8 if packed and not (with_qt and lhs_qvalue_needed) else L.K_NATURAL
     lq, lsc = ops.quantize(lhs.reshape(1, M, T * ts), reduce=L.REDUCE_COLS, group=ts, out_dtype=specs[0]['out_dtype'],
                            quant_bound=specs[0]['quant_bound'], clip_bound=specs[0]['clip_bound'],
-                           compute_dtype=lhs.dtype, scale_dtype=sdt_l)
-    rra = list(range(2, nr))
+                           compute_dtype=lhs.dtype, scale_dtype=sdt_l, k_order=k_order)
     if frozen:
-      int4 = rhs_qt.container_dtype is utils.int4
       rv = lowering.view_operand(rhs_qt.qvalue, [], rra, [0, 1])
-      packed = int4 and (T * ts) % 32 == 0
       rq = _kernel_layout_of(rhs_qt.qvalue, rv, pack_int4=packed)     # [1, N, T*ts] (or packed)
       b_dtype = L.I4P if packed else L.I4 if int4 else L.I8
       sdt_r = sc.dtype
-      src = getattr(sc, 'f32_copy', None)
-      col_scale = (src if src is not None else sc).reshape(T, N).float().contiguous()
+      col_scale = _scale_f32(sc).reshape(T, N).contiguous()
     else:
       sdt_r = dq.rhs._calibrator.dtype if dq.rhs._calibrator.dtype is not None else lhs.dtype
       rq, rsc = ops.quantize(rhs.reshape(1, T * ts, N), reduce=L.REDUCE_ROWS, group=ts, transpose_out=True,
@@ -1131,16 +1140,15 @@ class DotGeneral:
                              clip_bound=specs[1]['clip_bound'], compute_dtype=lhs.dtype, scale_dtype=sdt_r)
       b_dtype = specs[1]['out_dtype']
       col_scale = rsc.reshape(T, N)
-    row_scale = lsc.reshape(M, T).t().contiguous()     # [T, M]
-    out = ops.gemm_grouped(lq[0], rq[0], row_scale=row_scale, col_scale=col_scale, group=ts,
+    out = ops.gemm_grouped(lq[0], rq[0], row_scale=lsc.reshape(M, T), col_scale=col_scale, group=ts,
                            out_dtype=lhs.dtype, row_scale_dtype=sdt_l, col_scale_dtype=sdt_r,
-                           a_dtype=specs[0]['out_dtype'], b_dtype=b_dtype)
+                           a_dtype=specs[0]['out_dtype'], b_dtype=b_dtype, a_k_order=k_order, row_scale_by_row=True)
     out = out.reshape(tuple(lhs.shape[:-2]) + tuple(rhs.shape[2:]))
     if not with_qt:
       return out
     mk_container = lambda spec: utils.int4 if spec['out_dtype'] == L.I4 else None
     lhs_qt_out = aqt_tensor.QTensor(
-        qvalue=lq.reshape(lhs.shape), scale=[lsc.reshape(tuple(lhs.shape[:-1]) + (1,)).to(sdt_l)], scale_t=None,
+        qvalue=lq.reshape(lhs.shape) if k_order == L.K_NATURAL else None, scale=[lsc.reshape(tuple(lhs.shape[:-1]) + (1,)).to(sdt_l)], scale_t=None,
         bias=[], dequant_dtype=lhs.dtype, container_dtype=mk_container(specs[0]))
     if frozen:
       rhs_qt_out = rhs_qt

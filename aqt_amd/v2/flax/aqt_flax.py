@@ -294,7 +294,12 @@ class AqtDotGeneral(torch.nn.Module, _RngMixin):
         return None
       lhs_qt = lhs_freezer.get() if self.lhs_apply_quant_mode else self.lhs_qtensor
       rhs_qt = rhs_freezer.get() if self.rhs_apply_quant_mode else self.rhs_qtensor
-      res = cfg.fused_tile_sum(tl, tr, tiled_dn, n_sum_axes, lhs_qt=lhs_qt, rhs_qt=rhs_qt, with_qt=True)
+      # the quantized lhs values are only looked at when this call freezes them (Freezer.set stores
+      # in CONVERT, and FreezerMode.CALIBRATION keeps the scales alone)
+      lhs_values_kept = (self.lhs_apply_quant_mode and self.lhs_quant_mode == QuantMode.CONVERT
+                         and self.lhs_freeze_mode != FreezerMode.CALIBRATION)
+      res = cfg.fused_tile_sum(tl, tr, tiled_dn, n_sum_axes, lhs_qt=lhs_qt, rhs_qt=rhs_qt, with_qt=True,
+                               lhs_qvalue_needed=lhs_values_kept)
       if res is None:
         return None
       out, (out_lhs_qt, out_rhs_qt) = res

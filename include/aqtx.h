@@ -61,6 +61,12 @@ enum {
 
 enum { AQTX_PRESCALE_NONE = 0, AQTX_PRESCALE_PER_ROW = 1, AQTX_PRESCALE_PER_COL = 2 };
 
+/* Order of the bytes of every aligned group of 8 along the contraction (contiguous) axis of a
+ * quantized int8 operand.  EVEN_ODD8 stores elements 0,2,4,6,1,3,5,7 of the group: the order in
+ * which aqtx_gemm_i8_grouped gets the values of a packed int4 operand out of its nibbles without
+ * interleaving them again, so the other operand is written that way by the quantizer. */
+enum { AQTX_K_NATURAL = 0, AQTX_K_EVEN_ODD8 = 1 };
+
 /*
  * Plan of one calibrate+quantize pass over a contiguous tensor viewed as
  * [batch, rows, cols] (row-major).
@@ -93,6 +99,8 @@ typedef struct aqtx_quant_plan {
   const uint32_t* key_device; /* optional DEVICE pointer to the two key words; when not NULL the kernels
                             read the key there and `key` above is ignored (a key that is a traced
                             array under XLA, or one updated on the device between HIP graph replays) */
+  int32_t out_k_order;   /* AQTX_K_*: byte order of q along cols; EVEN_ODD8 needs AQTX_REDUCE_COLS, an
+                            int8 / int4 out_dtype, no transpose_out, cols and group multiples of 8 */
 } aqtx_quant_plan;
 
 /*
@@ -195,6 +203,9 @@ typedef struct aqtx_grouped_gemm_plan {
   int32_t b_dtype;            /* AQTX_I8 | AQTX_I4 | AQTX_I4P (packed, low nibble = even k) */
   int32_t out_dtype;          /* AQTX_BF16 | AQTX_F32: dequant dtype = output dtype         */
   int32_t row_scale_dtype, col_scale_dtype; /* AQTX_BF16 | AQTX_F32                         */
+  int32_t a_k_order;          /* AQTX_K_*: byte order of a along k; EVEN_ODD8 needs b_dtype AQTX_I4P */
+  int32_t row_scale_by_row;   /* 0: row_scale is [k/group][m]; 1: [m][k/group], as aqtx_quantize
+                                 with AQTX_REDUCE_COLS and a group writes it                  */
 } aqtx_grouped_gemm_plan;
 
 /*
@@ -207,7 +218,7 @@ typedef struct aqtx_grouped_gemm_plan {
  * materialising the per-tile outputs.
  *   a          : int8 [m][lda]
  *   b          : int8 [n][ldb], or packed int4 [n][ldb bytes]
- *   row_scale  : float32 [k/group][m]   (scale of A's row m in group g)
+ *   row_scale  : float32 [k/group][m]   (scale of A's row m in group g), or [m][k/group] with row_scale_by_row
  *   col_scale  : float32 [k/group][n]
  *   c          : [m][ldc] of out_dtype
  */

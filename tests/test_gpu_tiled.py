@@ -104,3 +104,56 @@ def test_grouped_gemm_kernel(gpu, m, n, k, group, out, rdt, cdt, packed):
                          row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt],
                          b_dtype=L.I4P if packed else L.I4)
   np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+
+
+def _even_odd8(a):
+  """Every aligned group of 8 along the last axis as elements 0,2,4,6,1,3,5,7."""
+  g = a.reshape(a.shape[:-1] + (a.shape[-1] // 8, 8))
+  return g[..., [0, 2, 4, 6, 1, 3, 5, 7]].reshape(a.shape)
+
+
+@pytest.mark.parametrize('rows,cols,group', [(64, 1024, 128), (33, 256, 0), (8, 16384, 0)])
+def test_quantize_even_odd_byte_order(gpu, rows, cols, group):
+  """out_k_order = EVEN_ODD8 changes where the bytes of q land and nothing else."""
+  from aqt_amd import _lib as L
+  rng = np.random.default_rng(3)
+  x = torch.from_numpy(rng.standard_normal((1, rows, cols)).astype(np.float32)).to(gpu).to(torch.bfloat16)
+  kw = dict(reduce=L.REDUCE_COLS, group=group, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0)
+  q0, s0 = ops.quantize(x, **kw)
+  q1, s1 = ops.quantize(x, k_order=L.K_EVEN_ODD8, **kw)
+  np.testing.assert_array_equal(s1.cpu().numpy(), s0.cpu().numpy())
+  np.testing.assert_array_equal(q1.cpu().numpy(), _even_odd8(q0.cpu().numpy()))
+
+
+def test_quantize_even_odd_byte_order_rejected_where_unsupported(gpu):
+  from aqt_amd import _lib as L
+  x = torch.zeros((1, 16, 64), device=gpu, dtype=torch.bfloat16)
+  with pytest.raises(RuntimeError, match='EVEN_ODD8'):
+    ops.quantize(x, reduce=L.REDUCE_ROWS, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0, k_order=L.K_EVEN_ODD8)
+  x = torch.zeros((1, 16, 60), device=gpu, dtype=torch.bfloat16)
+  with pytest.raises(RuntimeError, match='EVEN_ODD8'):
+    ops.quantize(x, reduce=L.REDUCE_COLS, out_dtype=L.I8, quant_bound=127.5, clip_bound=127.0, k_order=L.K_EVEN_ODD8)
+
+
+@pytest.mark.parametrize('m,n,k,group', [(128, 256, 256, 128), (200, 300, 512, 128), (64, 520, 1024, 256), (5, 9, 128, 128)])
+def test_grouped_gemm_even_odd_lhs_and_row_major_scales(gpu, m, n, k, group):
+  """A in even-odd byte order against a packed int4 B, row scales as [m][groups]: same result."""
+  from aqt_amd import _lib as L
+  rng = np.random.default_rng(11)
+  a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+  b = rng.integers(-7, 8, (n, k)).astype(np.int8)
+  groups = k // group
+  rs = nm.cast(np.abs(rng.standard_normal((groups, m)).astype(np.float32)) * np.float32(0.02) + np.float32(1e-3), 'bf16')
+  cs = nm.cast(np.abs(rng.standard_normal((groups, n)).astype(np.float32)) * np.float32(3e-3) + np.float32(1e-4), 'bf16')
+  want = _grouped_ref(a, b, rs, cs, group, 'bf16', 'bf16', 'bf16')
+  bt = ops.pack_i4(torch.from_numpy(b).to(gpu))
+  got = ops.gemm_grouped(torch.from_numpy(_even_odd8(a)).to(gpu), bt,
+                         row_scale=torch.from_numpy(np.ascontiguousarray(rs.T)).to(gpu),
+                         col_scale=torch.from_numpy(cs).to(gpu), group=group, out_dtype=torch.bfloat16,
+                         row_scale_dtype=torch.bfloat16, col_scale_dtype=torch.bfloat16, b_dtype=L.I4P,
+                         a_k_order=L.K_EVEN_ODD8, row_scale_by_row=True)
+  np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+  with pytest.raises(RuntimeError, match='a_k_order'):
+    ops.gemm_grouped(torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu), row_scale=torch.from_numpy(rs).to(gpu),
+                     col_scale=torch.from_numpy(cs).to(gpu), group=group, out_dtype=torch.bfloat16, b_dtype=L.I4,
+                     a_k_order=L.K_EVEN_ODD8)
