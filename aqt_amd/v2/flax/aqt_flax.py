@@ -29,7 +29,6 @@ from aqt_amd.v2 import config
 from aqt_amd.v2 import tiled_dot_general
 from aqt_amd.v2 import transpose
 from aqt_amd.v2 import utils
-from aqt_amd.v2.flax import aqt_flax_dg_core
 from aqt_amd.v2.flax import freezer as general_freezer
 
 QuantMode = utils.QuantMode
@@ -268,8 +267,11 @@ class AqtDotGeneral(torch.nn.Module, _RngMixin):
       lhs_qt = _maybe_recover_scale_from_scale_t(lhs_qt, dimension_numbers, False, lhs_shape, rhs_shape)
       rhs_qt = _maybe_recover_scale_from_scale_t(rhs_qt, dimension_numbers, True, lhs_shape, rhs_shape)
 
-      out, (out_lhs_qt, out_rhs_qt) = aqt_flax_dg_core.dg_core_flax_lifted(
-          lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, self, cfg)
+      # aqt_flax_dg_core.py:22-127 wraps this call in flax.linen.custom_vjp so that the custom gradient
+      # survives module lifting; here the custom gradient is the autograd Function behind dg_core and the
+      # layer's variables are buffers outside the graph, so the call itself is all there is
+      out, (out_lhs_qt, out_rhs_qt) = cfg.dg_core(lhs=lhs, rhs=rhs, lhs_qt=lhs_qt, rhs_qt=rhs_qt,
+                                                  dimension_numbers=dimension_numbers)
 
       out_lhs_qt = _apply_freeze_mode(out_lhs_qt, self.lhs_freeze_mode, self.lhs_apply_quant_mode,
                                       self.lhs_quant_mode, 'lhs')
