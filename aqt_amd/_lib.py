@@ -91,6 +91,7 @@ class FpRoundPlan(ctypes.Structure):
       ('count', ctypes.c_int64), ('noise_mod', ctypes.c_int64),
       ('dtype', ctypes.c_int32), ('nexp', ctypes.c_int32), ('nmant', ctypes.c_int32),
       ('has_subnormals', ctypes.c_int32), ('mode', ctypes.c_int32), ('partitionable', ctypes.c_int32),
+      ('radix', ctypes.c_int32),
   ]
 
 

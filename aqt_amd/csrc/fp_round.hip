@@ -1,5 +1,6 @@
 // Rounding to an emulated small float (e2m1, e3m0, the OCP fp4/fp5/fp6 formats ...) held in a
-// bf16 or f32 container: fp_numerics.radix2_round (aqt/jax/v2/numerics/fp_numerics.py:300-459).
+// bf16 or f32 container: fp_numerics.radix2_round (aqt/jax/v2/numerics/fp_numerics.py:300-459),
+// and to the powers of 4 of the RADIX4 format (radix4_round, :661-706; round_radix4 below).
 // Elementwise on the bit patterns: add half a truncated ulp (or masked random bits) to the
 // pattern, clear the truncated mantissa bits, clamp the magnitude pattern between the smallest
 // and largest normal value; magnitudes below the smallest normal are rounded linearly
@@ -19,13 +20,48 @@ struct FpArgs {
   int64_t count;
   int64_t noise_mod;
   uint32_t trunc, trunc_mask, min_repr, max_repr;
-  int32_t nmant, sub, nexp0, mode;
+  int32_t nmant, sub, nexp0, mode, radix4;
   float scale, inv_scale, max_sub, min_float;
   BitGen gen;
 };
 
+// floor(log4(z)) of a non-negative float32 from its exponent field: floor(floor(log2 z) / 2).  Zero and
+// float32 subnormals come out far below the smallest radix-4 value, infinity and NaN far above.
+__device__ __forceinline__ int floor_log4(float z) {
+  return ((int)((__float_as_uint(z) >> 23) & 0xFFu) - 127) >> 1;
+}
+
+// radix4_round (aqt/jax/v2/numerics/fp_numerics.py:661-706) on a bf16 pattern; rnd = 16 random bits.
+__device__ __forceinline__ uint32_t round_radix4(uint32_t ob, uint32_t rnd, const FpArgs& a) {
+  const float x = __uint_as_float(ob << 16);
+  if (x != x) return 0x7FC0u;
+  const float ax = fabsf(x);
+  float z;
+  if (a.mode == AQTX_FP_NEAREST) {
+    z = fabsf(1.6f * x);
+  } else {
+    // the bucket [4^l, 4^(l+1)) that holds |x|, its width times a uniform number in [0, 1) added to |x|
+    float width = 0.0f;
+    if (ax != 0.0f) {
+      if (isinf(ax)) return 0x7FC0u;  // 4^inf - 4^inf in the reference
+      const float lower = ldexpf(1.0f, 2 * floor_log4(ax));
+      width = 4.0f * lower - lower;
+    }
+    const float u = __uint_as_float((rnd << 7) | 0x3F800000u) - 1.0f;
+    z = ax + u * width;
+  }
+  const int ebit = floor_log4(z);
+  if (z == 0.0f || ebit < -3) return 0u;
+  const uint32_t sign = ob & 0x8000u;
+  if (ebit >= 3) return sign | 0x4280u;                       // +-64
+  return sign | (uint32_t)((127 + 2 * ebit) << 7);            // +-4^ebit
+}
+
 template <bool BF16>
 __device__ __forceinline__ uint32_t round_pattern(uint32_t ob, uint32_t rnd, const FpArgs& a) {
+  if constexpr (BF16) {
+    if (a.radix4) return round_radix4(ob, rnd, a);
+  }
   constexpr int CM = BF16 ? 7 : 23;
   constexpr uint32_t WRAP = BF16 ? 0xFFFFu : 0xFFFFFFFFu;
   constexpr uint32_t SIGN = BF16 ? 0x8000u : 0x80000000u;
@@ -225,8 +261,11 @@ extern "C" int aqtx_fp_round(const aqtx_fp_round_plan* p, const void* x, void* o
   AQTX_REQUIRE(p != nullptr, "aqtx_fp_round: plan is NULL");
   AQTX_REQUIRE(is_float_dtype(p->dtype), "aqtx_fp_round: dtype must be bf16 or f32, got %d", p->dtype);
   const int cm = p->dtype == AQTX_BF16 ? 7 : 23;
-  AQTX_REQUIRE(p->nexp >= 0 && p->nexp <= 7, "aqtx_fp_round: nexp %d outside 0..7", p->nexp);
-  AQTX_REQUIRE(p->nmant >= 0 && p->nmant < cm,
+  AQTX_REQUIRE(p->radix == 0 || p->radix == 2 || p->radix == 4, "aqtx_fp_round: radix must be 2 or 4, got %d", p->radix);
+  const bool radix4 = p->radix == 4;
+  AQTX_REQUIRE(!radix4 || p->dtype == AQTX_BF16, "aqtx_fp_round: radix 4 takes bf16 only");
+  AQTX_REQUIRE(radix4 || (p->nexp >= 0 && p->nexp <= 7), "aqtx_fp_round: nexp %d outside 0..7", p->nexp);
+  AQTX_REQUIRE(radix4 || (p->nmant >= 0 && p->nmant < cm),
                "aqtx_fp_round: nmant %d must be below the container's %d mantissa bits", p->nmant, cm);
   AQTX_REQUIRE(p->mode == AQTX_FP_NEAREST || p->mode == AQTX_FP_NOISE_JAX_BITS || p->mode == AQTX_FP_NOISE_INDEX,
                "aqtx_fp_round: unknown mode %d", p->mode);
@@ -247,18 +286,20 @@ extern "C" int aqtx_fp_round(const aqtx_fp_round_plan* p, const void* x, void* o
   a.out = out;
   a.count = p->count;
   a.noise_mod = p->mode == AQTX_FP_NOISE_INDEX ? p->noise_mod : 1;
-  a.trunc = (uint32_t)(cm - p->nmant);
+  a.radix4 = radix4 ? 1 : 0;
+  const int nmant = radix4 ? 0 : p->nmant, nexp = radix4 ? 3 : p->nexp;  // unread by the radix-4 branch
+  a.trunc = (uint32_t)(cm - nmant);
   a.trunc_mask = (1u << a.trunc) - 1u;
   const uint32_t min_exp = 127u - (p->has_subnormals ? 1u : 0u);
-  const uint32_t max_exp = min_exp + (1u << p->nexp) - 1u;
+  const uint32_t max_exp = min_exp + (1u << nexp) - 1u;
   const uint32_t mant_mask = (1u << cm) - 1u;
   a.min_repr = min_exp << cm;
   a.max_repr = (max_exp << cm) + (mant_mask & ~a.trunc_mask);
-  a.nmant = p->nmant;
+  a.nmant = nmant;
   a.sub = p->has_subnormals ? 1 : 0;
-  a.nexp0 = p->nexp == 0;
+  a.nexp0 = nexp == 0;
   a.mode = p->mode;
-  a.scale = (float)(1u << p->nmant);
+  a.scale = (float)(1u << nmant);
   a.inv_scale = 1.0f / a.scale;
   a.max_sub = 1.0f - a.inv_scale;
   a.min_float = p->has_subnormals ? 0.5f : 1.0f;

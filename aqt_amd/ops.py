@@ -475,8 +475,9 @@ def im2col_i8(x: torch.Tensor, kernel, strides, pads, dilation):
 
 def fp_round(x: torch.Tensor, *, nexp: int, nmant: int, has_subnormals: bool, key=None,
              stochastic_rounding: bool = False, noise_mod: Optional[int] = None,
-             partitionable: bool = False) -> torch.Tensor:
-  """x (bf16 or f32, any shape) rounded to an emulated small float in the same dtype.
+             partitionable: bool = False, radix: int = 2) -> torch.Tensor:
+  """x (bf16 or f32, any shape) rounded to an emulated small float in the same dtype
+  (radix = 4: to the powers of 4 from 4^-3 to 4^3, bf16 only; nexp / nmant are then not read).
 
   Stochastic rounding draws jax.random.bits(key, x.shape, uint16); `noise_mod` replaces the draw
   by the index along the last axis (which must have that extent).
@@ -489,6 +490,7 @@ def fp_round(x: torch.Tensor, *, nexp: int, nmant: int, has_subnormals: bool, ke
   plan.dtype = aqtx_dtype(x.dtype)
   plan.nexp, plan.nmant, plan.has_subnormals = int(nexp), int(nmant), int(bool(has_subnormals))
   plan.partitionable = int(partitionable)
+  plan.radix = int(radix)
   k = None
   if not stochastic_rounding:
     plan.mode = L.FP_NEAREST

@@ -64,10 +64,11 @@ RADIX4 = _make(3, 0, True, radix=4)
 
 def fp_round(x: torch.Tensor, *, cfg: FpNumericsConfig, key, stochastic_rounding: bool,
              test_noise_axis: Optional[int] = None) -> torch.Tensor:
-  """fp_numerics.py:279-459 for radix 2: x (bf16 or f32) rounded to `cfg`, same dtype."""
+  """fp_numerics.py:279-459 (radix 2) and :661-706 (radix 4): x (bf16 or f32) rounded to `cfg`, same dtype."""
   assert cfg.radix == 2 or cfg.radix == 4, 'Only radix 2 and 4 are supported.'
   if cfg.radix == 4:
-    raise NotImplementedError('radix-4 rounding is not built')
+    assert cfg == RADIX4
+    assert x.dtype == torch.bfloat16, f'Unsupported dtype for sthochastic rounding: {x.dtype}.'
   assert cfg.minexp == 0, 'minexp not implemented'
   assert not cfg.has_two_nan, 'two_nan not implemented'
   assert not cfg.has_naninf, 'naninf not implemented'
@@ -85,7 +86,7 @@ def fp_round(x: torch.Tensor, *, cfg: FpNumericsConfig, key, stochastic_rounding
     noise_mod = x.shape[-1]
   return ops.fp_round(x, nexp=cfg.nexp, nmant=cfg.nmant, has_subnormals=cfg.has_subnormals, key=key,
                       stochastic_rounding=stochastic_rounding, noise_mod=noise_mod,
-                      partitionable=utils.threefry_partitionable)
+                      partitionable=utils.threefry_partitionable, radix=cfg.radix)
 
 
 def fp_largest_representable(cfg: FpNumericsConfig):

@@ -265,6 +265,12 @@ int aqtx_im2col_i8(const aqtx_im2col_plan* plan, const void* x, void* out, void*
  * NaN/inf codes, and writes the result in the same container dtype.  Replaces
  * fp_numerics.fp_round for radix 2 (aqt/jax/v2/numerics/fp_numerics.py:279-459), which
  * FpNumerics.vjp_fwd calls on the bf16 cast of its input (fp_numerics.py:632-640).
+ * With radix = 4 the result is sign(x) * 4^floor(log4(1.6 |x|)) (nearest), or
+ * sign(x) * 4^floor(log4(|x| + u * (width of x's bucket))) with u in [0, 1) from 16 random bits
+ * (stochastic), zero below 4^-3 and +-64 from 4^3 up.  floor(log4(.)) is taken from the float32
+ * exponent (exact), where the reference divides two float32 logarithms: the two can differ only
+ * where the argument is a power of 4 to within an ulp, points the reference's own test leaves
+ * out (fp_numerics_test.py:364-377).
  *   AQTX_FP_NEAREST        : half a truncated ulp is added to the bit pattern
  *   AQTX_FP_NOISE_JAX_BITS : stochastic rounding with jax.random.bits(key, [count], uint16)
  *   AQTX_FP_NOISE_INDEX    : stochastic rounding with noise = index % noise_mod, the
@@ -282,6 +288,9 @@ typedef struct aqtx_fp_round_plan {
   int32_t has_subnormals;
   int32_t mode;
   int32_t partitionable;  /* jax_threefry_partitionable layout of the random bits */
+  int32_t radix;          /* 0 or 2: the format described by nexp / nmant / has_subnormals; 4: the
+                             reference's RADIX4 format {0, +-4^-3 .. +-4^3} (fp_numerics.py:661-706),
+                             bf16 only; nexp, nmant and has_subnormals are then not read */
 } aqtx_fp_round_plan;
 
 int aqtx_fp_round(const aqtx_fp_round_plan* plan, const void* x, void* out,

@@ -9,8 +9,13 @@ representable values and clamping of overflows (fp_numerics_test.py:296-440); ex
 the mean under equi-spaced noise (fp_numerics_test.py:442-460); the representable-value tables
 (fp_numerics_test.py:169-293).
 
-radix-4 rounding (fp_numerics.py:653-705) is not restated: it goes through log() of the input,
-whose last bit differs between libraries.  Parity unpinned, and not built.
+radix-4 rounding (`radix4_round`, fp_numerics.py:661-706) is restated as written, through float32
+log(): floor(log(z) / log(4)).  Pins: every interior point of every bucket goes to the bucket's
+centre, zero below 4^-3 and +-64 above (the reference's own bucket test, fp_numerics_test.py:330-440,
+with its shifted edge of the lowest bucket, :364-377); the mean under equi-spaced noise.  Where z is
+a power of 4 to within a float32 ulp the result depends on the last bit of the library's log():
+parity unpinned at those arguments (the reference's test leaves the bucket edges out as well);
+`radix4_log_is_safe` says which arguments are clear of them.
 
 Arrays: float32 numpy arrays whose values are representable in the container dtype ('bf16' or
 'f32'), like the rest of the oracle.
@@ -218,6 +223,60 @@ def fp_round_new(x, dt, cfg: FpNumericsConfig, key=None, stochastic_rounding=Fal
     if nexp == 0 and cfg.has_subnormals:
       out = np.clip(out, -max_subnormal, max_subnormal)
   return out.astype(np.float32)
+
+
+RADIX4_VALUES = np.array([0.0] + [4.0**e for e in range(-3, 4)] + [-(4.0**e) for e in range(-3, 4)], np.float32)
+
+
+def _radix4_args(x, key, stochastic_rounding, test_noise_axis, coeff):
+  """The float32 argument whose floor(log4) picks the bucket (fp_numerics.py:679-700)."""
+  x = np.asarray(x, np.float32)
+  f32 = np.float32
+  with np.errstate(divide='ignore', invalid='ignore', over='ignore'):
+    if not stochastic_rounding:
+      return np.abs(f32(coeff) * x)
+    abs_x = np.abs(x)
+    lower_ebit = np.floor(np.log(abs_x) / np.log(f32(4)))
+    lower = np.power(f32(4), lower_ebit, dtype=np.float32)
+    higher = np.power(f32(4), lower_ebit + f32(1), dtype=np.float32)
+    bucket_size = higher - lower
+    if test_noise_axis is not None:
+      assert x.shape[test_noise_axis] == 2**16, 'Input repetition should be consistent with effective noise bits.'
+    rnd = _noise_bits(x.shape, key, test_noise_axis)
+    noise = ((rnd.astype(np.uint32) << np.uint32(7)) | np.uint32(0x3F800000)).view(np.float32) - f32(1.0)
+    return abs_x + noise * bucket_size
+
+
+def radix4_log_is_safe(x, key=None, stochastic_rounding=False, test_noise_axis=None, coeff=1.6):
+  """False where the argument of the logarithm (of either logarithm, with stochastic rounding) lies within four
+  float32 ulps of one of the powers of 4 at which the result changes (4^-4 .. 4^3), i.e. where
+  floor(log(z)/log(4)) hangs on the last bit of log()."""
+  def clear(z):
+    z = np.asarray(z, np.float32).astype(np.float64)
+    ok = np.ones(z.shape, bool)
+    for k in range(-4, 4):
+      p = 4.0**k
+      ok &= ~(np.abs(z - p) <= 4 * float(np.spacing(np.float32(p))))
+    return ok
+  ok = clear(_radix4_args(x, key, stochastic_rounding, test_noise_axis, coeff))
+  if stochastic_rounding:
+    ok &= clear(np.abs(np.asarray(x, np.float32)))
+  return ok
+
+
+def radix4_round(x, dt, key=None, stochastic_rounding=False, test_noise_axis=None, coeff=1.6):
+  """radix4_round (fp_numerics.py:661-706): to the nearest of {0, +-4^-3 .. +-4^3}; bf16 in and out."""
+  assert dt == 'bf16', f'Unsupported dtype for sthochastic rounding: {dt}.'
+  x = np.asarray(x, np.float32)
+  f32 = np.float32
+  z = _radix4_args(x, key, stochastic_rounding, test_noise_axis, coeff)
+  with np.errstate(divide='ignore', invalid='ignore', over='ignore'):
+    ebit = np.floor(np.log(z) / np.log(f32(4)))
+    subnormal = np.zeros_like(x)
+    overflow = np.sign(x) * f32(64)
+    radix4 = np.sign(x) * np.power(f32(4), ebit, dtype=np.float32)
+    ret = np.where(ebit < -3, subnormal, np.where(ebit >= 3, overflow, radix4))
+  return nm.cast(ret.astype(np.float32), 'bf16')
 
 
 def fp_values(cfg: FpNumericsConfig):

@@ -225,3 +225,64 @@ def test_stochastic_rounding_paired_blocks_ragged_ends(gpu, dt, count):
   for name in ('e2m1_ocp', 'e3m0'):
     got = fp_numerics.fp_round(U.to_dev(x, dt, gpu), cfg=_cfg(name), key=key, stochastic_rounding=True)
     _eq_outside_nan(got, F.radix2_round(x, dt, F.CONFIGS[name], key, True), x)
+
+
+# ---- radix 4 (fp_numerics.py:661-706) -------------------------------------------------------------
+@pytest.mark.gpu
+def test_radix4_every_bf16_pattern(gpu):
+  """Round to nearest on all 65536 patterns: equal to the oracle wherever the reference's logarithm
+  is clear of a power of 4, and the mathematical floor(log4) where it is not (1.6 x = 4^n exactly)."""
+  from aqt_amd.v2.numerics import fp_numerics
+  x, t = _all_bf16(gpu)
+  got = fp_numerics.fp_round(t, cfg=fp_numerics.RADIX4, key=None, stochastic_rounding=False)
+  g = got.float().cpu().numpy()
+  want = F.radix4_round(x, 'bf16')
+  safe = F.radix4_log_is_safe(x) & ~np.isnan(x)
+  assert safe.sum() > 65536 - 254 - 20
+  np.testing.assert_array_equal(g[safe].view(np.uint32), want[safe].view(np.uint32))
+  assert np.isnan(g[np.isnan(x)]).all()
+  edge = ~safe & ~np.isnan(x)
+  y = np.abs(np.float32(1.6) * x[edge]).astype(np.float64)
+  exact = np.sign(x[edge]) * 4.0**np.floor(np.log2(y) / 2)
+  exact = np.where(np.abs(exact) < 4.0**-3, 0.0, np.where(np.abs(exact) >= 64, np.sign(x[edge]) * 64, exact))
+  np.testing.assert_array_equal(g[edge], exact.astype(np.float32))
+  assert set(np.unique(np.abs(g[~np.isnan(g)]))) == set(np.abs(F.RADIX4_VALUES))
+
+
+@pytest.mark.gpu
+def test_radix4_stochastic_rounding(gpu):
+  """The 2^16 equi-spaced noise values (test_noise_axis) and jax.random.bits noise against the oracle,
+  and the exact mean."""
+  from aqt_amd.v2.numerics import fp_numerics
+  xs = nm.cast(np.array([0.0, 0.004, 0.02, 0.05, 0.3, 0.9, 1.7, 3.1, 5.0, 12.0, 17.0, 50.0, 300.0, -2.5, -40.0], np.float32), 'bf16')
+  x = np.broadcast_to(xs[:, None], (xs.size, 2**16)).copy()
+  t = U.to_dev(x, 'bf16', gpu)
+  got = fp_numerics.fp_round(t, cfg=fp_numerics.RADIX4, key=None, stochastic_rounding=True, test_noise_axis=1)
+  g = got.float().cpu().numpy()
+  want = F.radix4_round(x, 'bf16', stochastic_rounding=True, test_noise_axis=1)
+  safe = F.radix4_log_is_safe(x, stochastic_rounding=True, test_noise_axis=1)
+  assert safe.mean() > 0.99
+  np.testing.assert_array_equal(g[safe], want[safe])
+  inside = (np.abs(xs) >= 4.0**-3) & (np.abs(xs) < 64)
+  width = 3 * 4.0**np.floor(np.log2(np.abs(xs[inside].astype(np.float64))) / 2)
+  assert np.all(np.abs(g[inside].astype(np.float64).mean(axis=1) - xs[inside]) <= 2.0**-15 * width)
+  key = np.array([7, 11], np.uint32)
+  rng = np.random.default_rng(5)
+  x = nm.cast((rng.standard_normal((257, 1000)) * np.exp(rng.uniform(-5, 5, (257, 1000)))).astype(np.float32), 'bf16')
+  got = fp_numerics.fp_round(U.to_dev(x, 'bf16', gpu), cfg=fp_numerics.RADIX4, key=key, stochastic_rounding=True)
+  want = F.radix4_round(x, 'bf16', key=key, stochastic_rounding=True)
+  safe = F.radix4_log_is_safe(x, key=key, stochastic_rounding=True)
+  assert safe.mean() > 0.99
+  np.testing.assert_array_equal(got.float().cpu().numpy()[safe], want[safe])
+
+
+@pytest.mark.gpu
+def test_radix4_takes_bf16_only(gpu):
+  from aqt_amd.v2.numerics import fp_numerics
+  with pytest.raises(AssertionError, match='Unsupported dtype'):
+    fp_numerics.fp_round(torch.zeros(8, device=gpu), cfg=fp_numerics.RADIX4, key=None, stochastic_rounding=False)
+  p = L.FpRoundPlan()
+  p.count, p.dtype, p.radix, p.mode = 16, L.F32, 4, L.FP_NEAREST
+  fake = ctypes.c_void_p(0x1000)
+  assert L.lib().aqtx_fp_round(ctypes.byref(p), fake, fake, None, None) != 0
+  assert 'bf16' in L.lib().aqtx_last_error().decode()

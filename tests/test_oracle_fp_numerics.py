@@ -164,3 +164,51 @@ def test_largest_representable():
   """fp_numerics.py:594-615 against the enumerated values."""
   for name, cfg in F.CONFIGS.items():
     assert F.fp_largest_representable(cfg) == F.fp_values(cfg).max(), name
+
+
+# ---- radix 4 (fp_numerics.py:661-706) -------------------------------------------------------------
+def _radix4_buckets():
+  """fp_numerics_test.py:342-377 for RADIX4: centres, boundaries halfway between them, except that the
+  edge of the zero bucket is where floor(log4(1.6 x)) turns -3, at (4^-3 + 4^-4) / 2."""
+  centers = np.unique(F.RADIX4_VALUES.astype(np.float64))
+  assert centers[-1] == 64.0
+  bounds = (centers[1:] + centers[:-1]) / 2
+  edge = centers[-1] + (centers[-1] - bounds[-1])
+  bounds = np.concatenate([[-edge], bounds, [edge]])
+  bounds = np.where(np.abs(bounds) == 4.0**-3 / 2, np.sign(bounds) * (4.0**-3 + 4.0**-4) / 2, bounds)
+  return centers, bounds, edge
+
+
+def test_radix4_round_to_nearest_and_overflow():
+  centers, bounds, edge = _radix4_buckets()
+  lower, upper = bounds[:-1], bounds[1:]
+  data = nm.cast(np.linspace(lower, upper, 257, endpoint=True, axis=0).astype(np.float32), 'bf16')
+  interior = (data > lower[None]) & (data < upper[None])
+  assert interior.mean() > 0.9
+  q = F.radix4_round(data, 'bf16')
+  want = np.broadcast_to(centers[None].astype(np.float32), q.shape)
+  np.testing.assert_array_equal(np.where(interior, q, 0), np.where(interior, want, 0))
+  for sign in (-1.0, 1.0):
+    far = nm.cast(np.linspace(sign * edge, sign * 10 * edge, 129).astype(np.float32), 'bf16')
+    far = far[np.abs(far) > edge]
+    np.testing.assert_array_equal(F.radix4_round(far, 'bf16'), np.full_like(far, sign * 64.0))
+  np.testing.assert_array_equal(F.radix4_round(np.array([0.0, -0.0, 1e-30, -1e-30], np.float32), 'bf16'), np.zeros(4, np.float32))
+
+
+def test_radix4_equispaced_noise_gives_exact_mean():
+  """With the 2^16 equi-spaced noise values the mean of the rounded values is the input (to the
+  spacing of the noise), for inputs inside the range of the format: P(up) is the position in the bucket."""
+  xs = nm.cast(np.array([0.02, 0.05, 0.3, 0.9, 1.0, 1.7, 3.1, 5.0, 12.0, 17.0, 50.0, -2.5, -40.0], np.float32), 'bf16')
+  x = np.broadcast_to(xs[:, None], (xs.size, 2**16)).copy()
+  q = F.radix4_round(x, 'bf16', stochastic_rounding=True, test_noise_axis=1)
+  assert set(np.unique(np.abs(q))) <= set(np.abs(F.RADIX4_VALUES))
+  mean = q.astype(np.float64).mean(axis=1)
+  width = 3 * 4.0**np.floor(np.log2(np.abs(xs.astype(np.float64))) / 2)
+  np.testing.assert_allclose(mean, xs.astype(np.float64), rtol=0, atol=2.0**-15 * width.max())
+  assert np.all(np.abs(mean - xs) <= 2.0**-15 * width)
+
+
+def test_radix4_log_safety_mask_flags_the_powers_of_four():
+  x = nm.cast(np.array([10.0, 2.5, 0.625, 40.0, 3.0, 1.0, 0.3], np.float32), 'bf16')  # 1.6 x = 16, 4, 1, 64: edges
+  np.testing.assert_array_equal(F.radix4_log_is_safe(x), [False, False, False, False, True, True, True])
+  np.testing.assert_array_equal(F.radix4_log_is_safe(x, stochastic_rounding=True, test_noise_axis=None, key=np.array([0, 1], np.uint32))[5:6], [False])
