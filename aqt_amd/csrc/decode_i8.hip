@@ -249,6 +249,198 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   }
 }
 
+// ---- a few more rows: the same, on 16 waves --------------------------------------------------------
+// Quantizing ROWS rows in every workgroup is vector work (about 8 instructions per value), and a wave
+// issues a vector instruction only every ~12 cycles: with the four waves of the kernel above it
+// takes longer than the weight stream it is meant to hide under.  Here a workgroup has 16 waves:
+// all of them quantize (a row is shared by 256 threads, four rows at a time), waves 0..3 alone
+// request the weights (before the quantisation) and contract.  Rows are written to LDS as in the
+// kernel above.  k <= 4096 * PPT.  The host uses it for ROWS = 4 only: the work every workgroup
+// repeats grows with the rows, the launch it saves does not.
+typedef unsigned short dq_u16x2 __attribute__((ext_vector_type(2)));
+template <typename TIn, int ROWS, int PPT, int U, bool PACKED, bool WFRAG>
+__global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
+  static_assert(ROWS % 4 == 0 && ROWS <= 16, "rows come in fours");
+  extern __shared__ __attribute__((aligned(16))) uint8_t xlds[];  // [ROWS][kp]
+  __shared__ float smax[ROWS][4];
+  __shared__ float sscale[ROWS];
+  __shared__ int red[4][16][16];
+  constexpr bool XBF = sizeof(TIn) == 2;
+  constexpr int WPP = XBF ? 8 : 16;  // 32-bit words of one 16-value input piece
+  constexpr int PASSES = ROWS / 4;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool contracts = wave < 4;
+  const int r = lane & 15, c = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nrow = (n0 + r) < d.n ? (n0 + r) : (d.n - 1);
+  const int kp = (d.k + 255) / 256 * 256;
+  const int pieces = d.k / 16;
+
+  constexpr int KS = PACKED ? 128 : 64;   // k covered by one wave-wide weight load
+  constexpr int KL = KS / 4;              // k covered by one lane's 16 bytes
+  const int kb = PACKED ? d.k / 2 : d.k;  // bytes of one weight row
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, d.w_frag ? (int64_t)((d.n + 15) / 16) * d.w_steps * 1024 : (int64_t)d.n * kb);
+  const int kq = ((d.k + 3) / 4 + KS - 1) / KS * KS;
+  const int k_lo = (wave & 3) * kq;
+  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
+  const int wbase = WFRAG ? (int)blockIdx.x * d.w_steps * 1024 + lane * 16 : nrow * kb + c * 16;
+  constexpr int wstep = WFRAG ? 1024 : 64;
+  auto w_offset = [&](int ko) { return (ko + c * KL < k_hi) ? wbase + (ko / KS) * wstep : kOob; };
+
+  // first batch of weights: in flight while the activations are quantized
+  v4i wf[U];
+  if (contracts) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
+  }
+
+  // ---- quantize the activations into LDS: thread t works on row 4 * pass + t / 256, pieces t % 256 + 256 j
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.x, (int64_t)d.m * d.k * (int64_t)sizeof(TIn));
+  const int sub = tid >> 8, tt = tid & 255, gw = (tid >> 6) & 3;  // row of the pass, thread and wave inside the row's group
+  uint32_t raw[PASSES][PPT][WPP];
+#pragma unroll
+  for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int i = 4 * ps + sub, p = tt + 256 * j;
+      const bool ok = i < d.m && p < pieces;
+      const int off = ok ? (i * d.k + p * 16) * (int)sizeof(TIn) : kOob;  // out of range reads give 0
+#pragma unroll
+      for (int q = 0; q < WPP / 4; ++q) {
+        const v4i t = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? off + 16 * q : kOob, 0, 0);
+        raw[ps][j][4 * q + 0] = (uint32_t)t[0]; raw[ps][j][4 * q + 1] = (uint32_t)t[1];
+        raw[ps][j][4 * q + 2] = (uint32_t)t[2]; raw[ps][j][4 * q + 3] = (uint32_t)t[3];
+      }
+    }
+  auto value = [&](int ps, int j, int e) -> float {
+    if constexpr (XBF) {
+      const uint32_t w = raw[ps][j][e >> 1];
+      return __uint_as_float((e & 1) ? (w & 0xFFFF0000u) : (w << 16));
+    } else {
+      return __uint_as_float(raw[ps][j][e]);
+    }
+  };
+#pragma unroll
+  for (int ps = 0; ps < PASSES; ++ps) {
+    float amax = 0.0f;
+    if constexpr (XBF) {
+      // two bf16 magnitudes per word: they order like unsigned integers, NaN patterns above infinity
+      uint32_t m2 = 0u;
+#pragma unroll
+      for (int j = 0; j < PPT; ++j)
+#pragma unroll
+        for (int q = 0; q < WPP; ++q) {
+          const dq_u16x2 a2 = __builtin_bit_cast(dq_u16x2, m2), b2 = __builtin_bit_cast(dq_u16x2, raw[ps][j][q] & 0x7FFF7FFFu);
+          m2 = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a2, b2));
+        }
+      amax = nanmax(__uint_as_float(m2 << 16), __uint_as_float(m2 & 0xFFFF0000u));
+    } else {
+#pragma unroll
+      for (int j = 0; j < PPT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) amax = absmax_step(amax, value(ps, j, e));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = nanmax(amax, __shfl_xor(amax, off, 64));
+    if (lane == 0) smax[4 * ps + sub][gw] = amax;
+  }
+  __syncthreads();
+  const int tbf = d.x_bf16 & d.xs_bf16;
+#pragma unroll
+  for (int ps = 0; ps < PASSES; ++ps) {
+    const int i = 4 * ps + sub;
+    float amax = nanmax(nanmax(smax[i][0], smax[i][1]), nanmax(smax[i][2], smax[i][3]));
+    if (amax == 0.0f) amax = 1.0f;
+    float sc = rnd(amax / d.quant_bound, d.x_bf16);
+    sc = rnd(sc, d.xs_bf16);
+    float inv = rnd(1.0f / sc, d.xs_bf16);
+    if (isinf(inv)) inv = 1.0f;
+    if (tt == 0) {
+      sscale[i] = sc;
+      if (blockIdx.x == 0 && i < d.m) d.x_scale_out[i] = sc;
+    }
+    auto quantize_row = [&](auto tbf_c) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int p = tt + 256 * j;
+      uint32_t q[4];
+#pragma unroll
+      for (int w4 = 0; w4 < 4; ++w4) {
+        uint32_t b[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float t = value(ps, j, 4 * w4 + e) * inv;
+          if constexpr (decltype(tbf_c)::value) t = round_bf16(t);
+          // clip, then round half to even and convert in one addition: after t + 1.5 * 2^23 the low
+          // mantissa bits are the two's complement of the rounded integer (|t| <= 127 here)
+          t = __builtin_amdgcn_fmed3f(t, -d.clip_bound, d.clip_bound);
+          b[e] = __float_as_uint(t + 12582912.0f);
+        }
+        const uint32_t lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);   // bytes b0 b1 0 0
+        const uint32_t hi = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);   // bytes 0 0 b2 b3
+        q[w4] = lo | hi;
+      }
+      if (p < pieces) {
+        const int pos = (p & ~15) | ((p & 15) ^ (i & 15));
+        *reinterpret_cast<uint4*>(xlds + (size_t)i * kp + pos * 16) = make_uint4(q[0], q[1], q[2], q[3]);
+        if (blockIdx.x == 0 && d.xq_out != nullptr && i < d.m)
+          *reinterpret_cast<uint4*>(d.xq_out + (size_t)i * d.k + p * 16) = make_uint4(q[0], q[1], q[2], q[3]);
+      }
+    }
+    };
+    if (tbf) quantize_row(std::true_type{}); else quantize_row(std::false_type{});
+  }
+  __syncthreads();
+
+  // ---- contraction (waves 0..3), weights from HBM, activations from LDS
+  if (contracts) {
+    v4i acc = v4i{0, 0, 0, 0};
+    const bool row_ok = r < ROWS && r < d.m;
+    constexpr int XP = PACKED ? 2 : 1;  // activation pieces per weight load
+    for (int kk = k_lo; kk < k_hi; kk += KS * U) {
+      if (kk != k_lo) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, 0);
+      }
+      v4i xf[U][XP];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int h = 0; h < XP; ++h) {
+          const int pj = (kk + u * KS) / 16 + c * XP + h;
+          xf[u][h] = v4i{0, 0, 0, 0};
+          if (row_ok && pj < pieces) {
+            const int pos = (pj & ~15) | ((pj & 15) ^ r);
+            xf[u][h] = *reinterpret_cast<const v4i*>(xlds + (size_t)r * kp + pos * 16);
+          }
+        }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if constexpr (PACKED) {
+          int t[8];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[u][j], t[2 * j], t[2 * j + 1]);
+          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], v4i{t[0], t[1], t[2], t[3]}, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][1], v4i{t[4], t[5], t[6], t[7]}, acc, 0, 0, 0);
+        } else {
+          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], wf[u], acc, 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][4 * c + e][r] = acc[e];
+  }
+  __syncthreads();
+  const int mm = tid >> 4, nn = n0 + (tid & 15);
+  if (tid < 256 && mm < d.m && nn < d.n) {
+    const int sum = red[0][mm][tid & 15] + red[1][mm][tid & 15] + red[2][mm][tid & 15] + red[3][mm][tid & 15];
+    store_out_scaled(d, mm, nn, sum, sscale[mm]);
+  }
+}
+
 // ---- 3 <= m <= 64: K split across workgroups -----------------------------------------------------
 // Phase 1, one workgroup per token: per-token abs-max, scale and int8 values (the arithmetic of the
 // row kernel of aqtx_quantize), the row kept in registers between the two passes (PPT 16-value
@@ -769,6 +961,30 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
     }
 #undef AQTX_FUSED
     AQTX_HIP_CHECK_LAUNCH("decode_fused_kernel");
+    return 0;
+  }
+
+  // Three or four tokens against a weight of at most 256 16-row blocks (one workgroup per CU, so the
+  // quantisation every workgroup repeats is paid once): one kernel again, on 16 waves per workgroup.
+  // Measured at k = 4096, n = 4096: 7.7 us against 9.0-9.2 us for the two kernels below; at 8 tokens
+  // the two are equal, and with several rounds of workgroups (n = 14336) the repeated quantisation
+  // loses by 5-12 us.
+  const unsigned wide_grid = (unsigned)((p->n + 15) / 16);
+  if (!never_fuse && p->m <= 4 && p->k <= 8192 && wide_grid <= 256) {
+    d.xq_out = reinterpret_cast<int8_t*>(xq);
+    const size_t lds = (size_t)4 * (size_t)((p->k + 255) / 256 * 256);
+#define AQTX_WIDE(T, P)                                                                          \
+  if (d.w_frag) {                                                                                \
+    if (pk) decode_wide_kernel<T, 4, P, 4, true, true><<<wide_grid, 1024, lds, st>>>(d);         \
+    else decode_wide_kernel<T, 4, P, 8, false, true><<<wide_grid, 1024, lds, st>>>(d);           \
+  } else {                                                                                       \
+    if (pk) decode_wide_kernel<T, 4, P, 4, true, false><<<wide_grid, 1024, lds, st>>>(d);        \
+    else decode_wide_kernel<T, 4, P, 8, false, false><<<wide_grid, 1024, lds, st>>>(d);          \
+  }
+    if (xbf) { if (p->k <= 4096) { AQTX_WIDE(uint16_t, 1) } else { AQTX_WIDE(uint16_t, 2) } }
+    else { if (p->k <= 4096) { AQTX_WIDE(float, 1) } else { AQTX_WIDE(float, 2) } }
+#undef AQTX_WIDE
+    AQTX_HIP_CHECK_LAUNCH("decode_wide_kernel");
     return 0;
   }
 

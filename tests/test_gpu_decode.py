@@ -177,6 +177,26 @@ def test_decode_every_launch_shape_gives_the_same_bits(gpu, packed, m, n, k):
         np.testing.assert_array_equal(xs.cpu().numpy(), xs_want, err_msg=hex(tuning))
 
 
+@pytest.mark.parametrize('m', [3, 4])
+@pytest.mark.parametrize('k', [480, 4096, 4112, 8192])
+@pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('f32', 'f32'), ('bf16', 'bf16')])
+def test_decode_three_or_four_rows_one_kernel(gpu, m, k, dt, w_sdt):
+  """Three or four tokens against a weight of at most 256 row blocks take the 16-wave kernel that
+  quantizes the activations itself (two pieces per thread above k = 4096); forcing the two-kernel
+  path gives the same bits, and both give the oracle's outputs, scales and quantized activations."""
+  n = 200
+  x = U.rand((m, k), dt, 700 + m, outliers=True)
+  wq, ws = _weights(n, k, 9, w_sdt)
+  want, xq_want, xs_want = _oracle_decode(x, dt, wq, ws, w_sdt)
+  for tuning in (0, 1 << 16):
+    out, xs, xq = ops.decode(U.to_dev(x, dt, gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
+                             quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True,
+                             tuning=tuning)
+    np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
+    np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
+    np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+
+
 @pytest.mark.parametrize('m', [1, 2])
 def test_decode_two_kernel_path_for_one_or_two_tokens(gpu, m):
   n, k = 328, 2048
