@@ -52,6 +52,7 @@ class GemmPlan(ctypes.Structure):
       ('row_scale_stride_b', ctypes.c_int64), ('col_scale_stride_b', ctypes.c_int64),
       ('group_offsets', ctypes.c_void_p),
       ('tuning', ctypes.c_int32),
+      ('a_k_order', ctypes.c_int32),
   ]
 
 

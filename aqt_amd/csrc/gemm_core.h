@@ -79,6 +79,7 @@ struct GemmArgs {
   // Ragged batches: entry b multiplies rows [group_offsets[b], group_offsets[b+1]) of one flat
   // A with B[b] into the same rows of one flat C (m is then an upper bound of a group's rows).
   const int32_t* group_offsets;
+  int a_even_odd8;  // packed int4 B only: A's bytes of every 8 k are stored as k 0,2,4,6,1,3,5,7
 };
 
 constexpr int BM = 256, BN = 256, BK = 128;
@@ -89,6 +90,33 @@ constexpr uint32_t kBufferRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data f
 #define AQTX_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
+
+// 16 bytes of packed int4 (32 values, low nibble = even k) -> 32 bytes of values * 16 in k order.
+// dword d of the load = k 8d..8d+7: even k: (x << 4) & 0xF0F0F0F0, odd k: x & 0xF0F0F0F0; then
+// the bytes are interleaved back to k order.
+// With even_odd8 the other operand stores every 8 k as k 0,2,4,6,1,3,5,7, and the interleaving is left out.
+__device__ __forceinline__ void unpack_i4x32(const v4i x4, v4i& lo, v4i& hi, int even_odd8) {
+  if (even_odd8) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t x = (uint32_t)x4[d];
+      const int ev = (int)((x << 4) & 0xF0F0F0F0u), od = (int)(x & 0xF0F0F0F0u);
+      if (d < 2) { lo[2 * d] = ev; lo[2 * d + 1] = od; }
+      else { hi[2 * (d - 2)] = ev; hi[2 * (d - 2) + 1] = od; }
+    }
+    return;
+  }
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const uint32_t x = (uint32_t)x4[d];
+    const uint32_t ev = (x << 4) & 0xF0F0F0F0u, od = x & 0xF0F0F0F0u;
+    const uint32_t k03 = __builtin_amdgcn_perm(od, ev, 0x05010400u);  // e0 o0 e1 o1
+    const uint32_t k47 = __builtin_amdgcn_perm(od, ev, 0x07030602u);  // e2 o2 e3 o3
+    if (d < 2) { lo[2 * d] = (int)k03; lo[2 * d + 1] = (int)k47; }
+    else { hi[2 * (d - 2)] = (int)k03; hi[2 * (d - 2) + 1] = (int)k47; }
+  }
+}
+
 
 // Workgroup id -> tile, XCD-aware: ids are dealt round-robin to the 8 XCDs, so id%8
 // picks the XCD; each XCD then walks a contiguous range of tiles in bands of 8 tile
@@ -115,15 +143,23 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // NW: waves per workgroup.  4 = 2x2 waves with 128x128 wave tiles, one wave per SIMD;
 // 8 = 2x4 waves with 128x64 wave tiles, two waves per SIMD, so that one wave's MFMAs fill the
 // issue slots in which the other waits on the memory pipeline.
-template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL>
+// BPACK (int8 MFMA only): B holds int4 values packed two per byte ([n][k/2], low nibble = even k; ldb and
+// stride_b in bytes).  A wave load then covers 16 rows x 64 B, and a lane's 16 bytes are unpacked in
+// registers into the two neighbouring 16-byte chunks of its row on their way to LDS: a nibble is
+// moved to the top of its byte (value * 16); the epilogue takes the factor 16 out again, exactly (a
+// power of two commutes with every rounding of the dequantisation).
+template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gemm_kernel(const GemmArgs g_in) {
   static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+  static_assert(!BPACK || MMA::kIntAcc, "packed int4 goes with the int8 MFMA");
   GemmArgs g = g_in;
   constexpr int NI = 16 / NW;       // 32-column MFMA tiles per wave
   constexpr int WN = NW / 2;        // waves along n
   constexpr int LPW = 32 / NW;      // 8-row load blocks per wave and operand
-  constexpr int NL = 2 * LPW;       // global loads per wave and stage
+  constexpr int NL = 2 * LPW;       // LDS stores per wave and stage
+  constexpr int LPB = BPACK ? LPW / 2 : LPW;  // B loads per wave and stage
+  constexpr int NLD = LPW + LPB;    // global loads per wave and stage
   constexpr int MPK = 4 * NI;       // MFMAs per wave and k-step
   using Acc = typename MMA::Acc;
   using AccScalar = typename MMA::AccScalar;
@@ -178,27 +214,67 @@ void gemm_kernel(const GemmArgs g_in) {
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + g.k), kBufferRsrcWord3);
-  int voff_a[LPW], voff_b[LPW], chunk_byte[LPW];
+      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + (BPACK ? g.k / 2 : g.k)),
+      kBufferRsrcWord3);
+  int voff_a[LPW], voff_b[LPB], chunk_byte[LPW];
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
     const int blk = wave * LPW + i;
     const int row = blk * 8 + (lane >> 3);
     chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ blk) & 7) * 16;
     voff_a[i] = row * (int)g.lda + chunk_byte[i];
-    voff_b[i] = row * (int)g.ldb + chunk_byte[i];
+    if constexpr (!BPACK) voff_b[i] = row * (int)g.ldb + chunk_byte[i];
   }
-  v4i stg[NL];  // staging registers: stg[2*i] = A block i, stg[2*i+1] = B block i
-  auto load_global = [&](int j, int k0) {  // j = 0..NL-1
-    const int i = j >> 1;
-    int vo = (j & 1) ? voff_b[i] : voff_a[i];
-    if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
-    stg[j] = __builtin_amdgcn_raw_buffer_load_b128((j & 1) ? rsrc_b : rsrc_a, vo, k0, 0);
+  // packed B: load q of a wave covers rows 16 (wave LPB + q) .. +15, lane -> row lane >> 2, 16 packed bytes
+  // (32 k) at 16 (lane & 3); they become the chunks 2p, 2p + 1 of that row, at positions chunk ^ f(row)
+  int pb_st[LPB];
+  if constexpr (BPACK) {
+#pragma unroll
+    for (int q = 0; q < LPB; ++q) {
+      const int row = (wave * LPB + q) * 16 + (lane >> 2);
+      voff_b[q] = row * (int)g.ldb + (lane & 3) * 16;
+      pb_st[q] = kTileBytes + row * BK + (((2 * (lane & 3)) ^ ((row ^ (row >> 3)) & 7)) * 16);
+    }
+  }
+  // Loads and stores are numbered in the order they are issued.  Unpacked: A block i, B block i alternate
+  // (load j = store j).  Packed: A0 B0 A1 | A2 B1 A3 | ..., and a B load feeds two stores.
+  v4i stga[LPW], stgb[LPB], pb_hi[LPB];
+  auto load_global = [&](int j, int k0) {  // j = 0..NLD-1
+    const bool is_b = BPACK ? (j % 3 == 1) : (j & 1);
+    const int i = BPACK ? (is_b ? j / 3 : j - (j + 1) / 3) : (j >> 1);
+    if (!is_b) {
+      int vo = voff_a[i];
+      if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
+      stga[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, k0, 0);
+    } else if constexpr (BPACK) {
+      int vo = voff_b[i];
+      if (KTAIL && k0 + (lane & 3) * 32 >= (int)g.k) vo = 0x7FFFFFF0;
+      stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 / 2, 0);
+    } else {
+      int vo = voff_b[i];
+      if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;
+      stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0, 0);
+    }
   };
   const int st_off = wave * LPW * 1024 + lane * 16;
-  auto store_lds = [&](uint8_t* st, int j) {
-    const int i = j >> 1;
-    *reinterpret_cast<v4i*>(st + ((j & 1) ? kTileBytes : 0) + st_off + i * 1024) = stg[j];
+  auto store_lds = [&](uint8_t* st, int j) {  // j = 0..NL-1
+    if constexpr (!BPACK) {
+      const int i = j >> 1;
+      *reinterpret_cast<v4i*>(st + ((j & 1) ? kTileBytes : 0) + st_off + i * 1024) = (j & 1) ? stgb[i] : stga[i];
+    } else {
+      // stores in the order of the loads: A0 B0.lo B0.hi A1 | A2 B1.lo B1.hi A3 | ...
+      const int grp = j >> 2, r4 = j & 3;
+      if (r4 == 0 || r4 == 3) {
+        const int i = 2 * grp + (r4 == 3 ? 1 : 0);
+        *reinterpret_cast<v4i*>(st + st_off + i * 1024) = stga[i];
+      } else if (r4 == 1) {
+        v4i lo;
+        unpack_i4x32(stgb[grp], lo, pb_hi[grp], g.a_even_odd8);
+        *reinterpret_cast<v4i*>(st + pb_st[grp]) = lo;
+      } else {
+        *reinterpret_cast<v4i*>(st + (pb_st[grp] ^ 16)) = pb_hi[grp];
+      }
+    }
   };
 
   // ---- per-lane swizzled fragment offsets: chunk ((2*ks + lh) * kChunks + c) ^ f(row)
@@ -261,7 +337,7 @@ void gemm_kernel(const GemmArgs g_in) {
 #pragma unroll
     for (int ks = 0; ks < KS - 1; ++ks) {
       // loads [l0, l1) of the 16 go with this k-step
-      const int l0 = (NL * ks + KS - 2) / (KS - 1), l1 = (NL * (ks + 1) + KS - 2) / (KS - 1);
+      const int l0 = (NLD * ks + KS - 2) / (KS - 1), l1 = (NLD * (ks + 1) + KS - 2) / (KS - 1);
       if (ks % 2 == 0) load_frags(cur, ks + 1, fa1, fb1); else load_frags(cur, ks + 1, fa0, fb0);
 #pragma unroll
       for (int j = l0; j < l1; ++j) load_global(j, refill_k0);
@@ -307,11 +383,11 @@ void gemm_kernel(const GemmArgs g_in) {
   const int k0_last = KTAIL ? 0x7FFFFF00 : (int)g.k - BK;
   auto refill_at = [&](int k0) { return k0 < k0_last ? k0 : k0_last; };
 #pragma unroll
-  for (int j = 0; j < NL; ++j) load_global(j, 0);
+  for (int j = 0; j < NLD; ++j) load_global(j, 0);
 #pragma unroll
   for (int j = 0; j < NL; ++j) store_lds(stage0, j);
 #pragma unroll
-  for (int j = 0; j < NL; ++j) load_global(j, BK);
+  for (int j = 0; j < NLD; ++j) load_global(j, BK);
 #pragma unroll
   for (int j = 0; j < NL; ++j) store_lds(stage1, j);
   __syncthreads();
@@ -337,7 +413,10 @@ void gemm_kernel(const GemmArgs g_in) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int64_t nn = ncol0 + ni * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-          if (mm < g.m && nn < g.n) dst[mm * g.ldc + nn] = acc[mi][ni][r];
+          if (mm < g.m && nn < g.n) {
+            if constexpr (BPACK) dst[mm * g.ldc + nn] = acc[mi][ni][r] >> 4;  // exact: a multiple of 16
+            else dst[mm * g.ldc + nn] = acc[mi][ni][r];
+          }
         }
     }
   }
@@ -358,7 +437,10 @@ void gemm_kernel(const GemmArgs g_in) {
       rscale[mi] = (rs != nullptr && mm < g.m) ? rs[mm] : 1.0f;
     }
     auto dequant = [&](AccScalar accv, float s_row, float s_col) {
-      if constexpr (EPI == 3) return __builtin_bit_cast(float, accv);
+      if constexpr (EPI == 3) {
+        if constexpr (BPACK) return __builtin_bit_cast(float, accv >> 4);
+        else return __builtin_bit_cast(float, accv);
+      }
       float f = round_to<kDqBf16>((float)accv);  // (int32 ->) f32 -> dequant dtype
       const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
       f = round_to<kProd1Bf16>(f * s1);
@@ -404,6 +486,10 @@ void gemm_kernel(const GemmArgs g_in) {
                 const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
                 csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
               }
+            }
+            if constexpr (BPACK) {  // the accumulators hold 16 times the contraction
+#pragma unroll
+              for (int e = 0; e < 4; ++e) csv[e] *= 0.0625f;
             }
 #pragma unroll
             for (int mi = 0; mi < 4; ++mi) {

@@ -68,32 +68,6 @@ struct GroupedArgs {
 
 __device__ __forceinline__ int row_swz(int row) { return (row ^ (row >> 3)) & 7; }
 
-// 16 bytes of packed int4 (32 values, low nibble = even k) -> 32 bytes of values * 16 in k order.
-// dword d of the load = k 8d..8d+7: even k: (x << 4) & 0xF0F0F0F0, odd k: x & 0xF0F0F0F0; then
-// the bytes are interleaved back to k order.
-// With even_odd8 the other operand stores every 8 k as k 0,2,4,6,1,3,5,7, and the interleaving is left out.
-__device__ __forceinline__ void unpack_i4x32(const v4i x4, v4i& lo, v4i& hi, int even_odd8) {
-  if (even_odd8) {
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const uint32_t x = (uint32_t)x4[d];
-      const int ev = (int)((x << 4) & 0xF0F0F0F0u), od = (int)(x & 0xF0F0F0F0u);
-      if (d < 2) { lo[2 * d] = ev; lo[2 * d + 1] = od; }
-      else { hi[2 * (d - 2)] = ev; hi[2 * (d - 2) + 1] = od; }
-    }
-    return;
-  }
-#pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const uint32_t x = (uint32_t)x4[d];
-    const uint32_t ev = (x << 4) & 0xF0F0F0F0u, od = x & 0xF0F0F0F0u;
-    const uint32_t k03 = __builtin_amdgcn_perm(od, ev, 0x05010400u);  // e0 o0 e1 o1
-    const uint32_t k47 = __builtin_amdgcn_perm(od, ev, 0x07030602u);  // e2 o2 e3 o3
-    if (d < 2) { lo[2 * d] = (int)k03; lo[2 * d + 1] = (int)k47; }
-    else { hi[2 * (d - 2)] = (int)k03; hi[2 * (d - 2) + 1] = (int)k47; }
-  }
-}
-
 // EPI as in the dense kernel: 0 = bf16 out, both products rounded to bf16; 4 = bf16 out, first
 // product bf16, second f32; 1 = bf16 out, products in f32; 2 = f32 out.
 template <int EPI>

@@ -15,8 +15,8 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
                  "%s: out_dtype must be bf16 or f32, got %d", who, p->out_dtype);
   } else {
     AQTX_REQUIRE((p->a_dtype == AQTX_I8 || p->a_dtype == AQTX_I4) &&
-                     (p->b_dtype == AQTX_I8 || p->b_dtype == AQTX_I4),
-                 "%s: operands must be int8 containers (got %d, %d)", who, p->a_dtype, p->b_dtype);
+                     (p->b_dtype == AQTX_I8 || p->b_dtype == AQTX_I4 || p->b_dtype == AQTX_I4P),
+                 "%s: operands must be int8 containers, b also packed int4 (got %d, %d)", who, p->a_dtype, p->b_dtype);
     AQTX_REQUIRE(p->out_dtype == AQTX_BF16 || p->out_dtype == AQTX_F32 || p->out_dtype == AQTX_I32,
                  "%s: out_dtype must be bf16, f32 or i32, got %d", who, p->out_dtype);
   }
@@ -25,8 +25,13 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
                "%s: row_scale_dtype / col_scale_dtype must be bf16 or f32", who);
   AQTX_REQUIRE(p->scale_order == AQTX_SCALE_ROW_THEN_COL || p->scale_order == AQTX_SCALE_COL_THEN_ROW,
                "%s: unknown scale_order %d", who, p->scale_order);
-  AQTX_REQUIRE(p->lda >= p->k && p->ldb >= p->k && p->ldc >= p->n,
+  const bool b_packed = !fp8 && p->b_dtype == AQTX_I4P;
+  AQTX_REQUIRE(p->lda >= p->k && p->ldb >= (b_packed ? p->k / 2 : p->k) && p->ldc >= p->n,
                "%s: leading dimension smaller than the row length", who);
+  AQTX_REQUIRE(p->a_k_order == AQTX_K_NATURAL || (p->a_k_order == AQTX_K_EVEN_ODD8 && b_packed),
+               "%s: a_k_order must be AQTX_K_NATURAL, or AQTX_K_EVEN_ODD8 with a packed int4 b", who);
+  AQTX_REQUIRE(!b_packed || (p->k % 32 == 0 && p->k * (int64_t)(127 * 8 * 16) < (1ll << 31)),
+               "%s: a packed int4 b needs k to be a multiple of 32 below 132096, got %lld", who, (long long)p->k);
   AQTX_REQUIRE(p->batch <= 65535 && p->m <= (int64_t)65535 * 256, "%s: shape too large for one launch", who);
   return 0;
 }
@@ -47,10 +52,13 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   const size_t esz = p->out_dtype == AQTX_BF16 ? 2 : 4;
   AQTX_REQUIRE(((uintptr_t)c % esz) == 0, "aqtx_gemm_i8: output is not element aligned");
 
-  const GemmArgs g = make_gemm_args(p, a, b, row_scale, col_scale, c, acc_out);
+  GemmArgs g = make_gemm_args(p, a, b, row_scale, col_scale, c, acc_out);
+  g.a_even_odd8 = p->a_k_order == AQTX_K_EVEN_ODD8;
+  const bool b_packed = p->b_dtype == AQTX_I4P;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
   if (!gemm_vector_path_ok(p, a, b)) {
+    AQTX_REQUIRE(!b_packed, "aqtx_gemm_i8: a packed int4 b needs 16-byte aligned operands and leading dimensions");
     AQTX_REQUIRE(p->group_offsets == nullptr,
                  "aqtx_gemm_i8: ragged batches need 16-byte aligned operands with k and leading dimensions "
                  "multiple of 16");
@@ -71,8 +79,13 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   // Two waves per SIMD by default: measured faster on every shape tried (the epilogue of one
   // wave overlaps the other's work).  plan->tuning = 4 | 8 overrides it (tests, tuning).
   const int waves = p->tuning == 4 ? 4 : 8;
+  AQTX_REQUIRE(!b_packed || !g.col_first, "aqtx_gemm_i8: a packed int4 b takes scale_order = AQTX_SCALE_ROW_THEN_COL");
+  // packed int4 B: the 8-wave kernel, row scale first (a frozen weight is the column operand)
 #define AQTX_LAUNCH(E, C, T)                                             \
   do {                                                                  \
+    if constexpr (!C) {                                                 \
+      if (b_packed) { gemm_kernel<MmaI8, 8, E, false, T, true><<<grid, 512, 0, st>>>(g); break; } \
+    }                                                                   \
     if (waves == 8) gemm_kernel<MmaI8, 8, E, C, T><<<grid, 512, 0, st>>>(g); \
     else gemm_kernel<MmaI8, 4, E, C, T><<<grid, 256, 0, st>>>(g);       \
   } while (0)

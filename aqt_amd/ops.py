@@ -252,8 +252,12 @@ def gemm(
     b_dtype: int = L.I8,
     want_acc: bool = False,
     group_offsets: Optional[torch.Tensor] = None,
+    a_k_order: int = 0,
 ):
   """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
+
+  b_dtype = L.I4P: B is uint8 [batch, n, k/2], int4 values packed two per byte (pack_i4); with
+  a_k_order = L.K_EVEN_ODD8 A was written by quantize(k_order=L.K_EVEN_ODD8).
 
   With `group_offsets` (int32 device tensor [groups + 1], ascending): a ragged product.  A is
   [1, m, k], B [groups, n, k]; group g multiplies rows off[g]:off[g+1] of A with B[g] into the
@@ -266,7 +270,7 @@ def gemm(
   (C, acc) with want_acc.
   """
   _require_gpu(a, b, row_scale, col_scale)
-  assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == b.shape[2]
+  assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == (2 * b.shape[2] if b_dtype == L.I4P else b.shape[2])
   assert a.shape[0] == b.shape[0] or group_offsets is not None
   assert a.stride(2) == 1 and b.stride(2) == 1, 'the contraction axis must be contiguous'
   batch, m, k = a.shape
@@ -294,6 +298,7 @@ def gemm(
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else sc_dt
   plan.scale_order = scale_order
   plan.tuning = GEMM_TUNING
+  plan.a_k_order = a_k_order
   for s, shape in ((row_scale, (batch, m)), (col_scale, (b.shape[0], n))):
     if s is not None:
       assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == shape, (tuple(s.shape), shape)

@@ -801,6 +801,12 @@ class DotGeneralRaw:
     swapped = (out_transpose_axes is not None and list(out_transpose_axes) == swap_perm
                and want_lba == lba and nl > 0 and nr > 0)
     common = dict(out_dtype=dequant_dtype, dequant_dtype=dequant_dtype)
+    if (not swapped and not fp8 and rhs_qt is not None and rhs_qt.is_full() and rhs_qt.container_dtype is utils.int4
+        and rkd == L.I4 and K % 32 == 0 and K < 132096 and rq.dtype == torch.int8):
+      # a frozen int4 weight is read packed two values per byte (half the bytes of a serving call
+      # and of the copy kept per weight; made once per tensor), unpacked in registers by the kernel
+      rq = _kernel_layout_of(rhs_qt.qvalue, lowering.view_operand(rhs_qt.qvalue, rba, rra, rca), pack_int4=True)
+      rkd = L.I4P
     if swapped:
       # C^T = rhs_q . lhs_q^T; the lhs scale still multiplies first (aqt_tensor.py:182-183)
       out = ops.gemm(rq, lq, row_scale=expand(rs, N), col_scale=expand(ls, M), a_dtype=rkd, b_dtype=lkd,

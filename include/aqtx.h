@@ -147,7 +147,10 @@ typedef struct aqtx_gemm_plan {
   int64_t batch, m, n, k;
   int64_t lda, ldb, ldc;      /* row strides in elements                                    */
   int64_t stride_a, stride_b, stride_c; /* batch strides in elements                      */
-  int32_t a_dtype, b_dtype;   /* AQTX_I8 | AQTX_I4 (container) | AQTX_E4M3 | AQTX_E5M2       */
+  int32_t a_dtype, b_dtype;   /* AQTX_I8 | AQTX_I4 (container) | AQTX_E4M3 | AQTX_E5M2; b_dtype of aqtx_gemm_i8
+                                 also AQTX_I4P: int4 packed two per byte ([n][k/2], low nibble = even k, as
+                                 aqtx_pack_i4 writes it; ldb and stride_b in bytes, k a multiple of 32),
+                                 unpacked in registers on the way to LDS                     */
   int32_t out_dtype;          /* AQTX_BF16 | AQTX_F32 | AQTX_I32 (raw accumulator, no scales) */
   int32_t dequant_dtype;      /* AQTX_BF16 | AQTX_F32: dtype the accumulator is cast to first */
   int32_t row_scale_dtype;    /* AQTX_BF16 | AQTX_F32: dtype of the values in row_scale      */
@@ -162,6 +165,8 @@ typedef struct aqtx_gemm_plan {
   const int32_t* group_offsets;
   int32_t tuning;             /* 0 = the library chooses the launch shape.  Tuning only (results never
                                  depend on it): 4 | 8 = waves per workgroup of the int8 kernel            */
+  int32_t a_k_order;          /* AQTX_K_*: byte order of a along k; EVEN_ODD8 (aqtx_gemm_i8 with b_dtype
+                                 AQTX_I4P only) saves the kernel the re-interleaving of the nibbles   */
 } aqtx_gemm_plan;
 
 /*

@@ -274,8 +274,9 @@ def test_mlp_block_fp32_full_size(gpu):
 @pytest.mark.parametrize('k', [512, 528])
 def test_serving_int4_weights(gpu, m, k):
   """W4A8 serving: a frozen int4 rhs (held one value per byte in the QTensor).  With at most 64
-  rows and k a multiple of 32 the decode kernel streams a packed copy made once; k = 528 and
-  m = 100 take the int8-container kernels.  Same numbers either way."""
+  rows and k a multiple of 32 the decode kernel streams a packed copy made once; with m = 100 the
+  dense kernel reads that packed copy and unpacks it in registers; k = 528 takes the
+  int8-container kernels.  Same numbers either way."""
   dt = 'bf16'
   lhs, rhs = U.rand((m, k), dt, 1, outliers=True), U.rand((k, 384), dt, 2, 0.02)
   cfg = config.set_context(aqt.dot_general_make(8, 4), None, None)

@@ -99,6 +99,61 @@ def test_large_accumulators_round_like_xla(gpu, waves):
   np.testing.assert_array_equal(c.float().cpu().numpy(), want)
 
 
+# ---- packed int4 B (two values per byte, unpacked in registers) ---------------------------------
+def _even_odd8(a):
+  g = a.reshape(a.shape[:-1] + (a.shape[-1] // 8, 8))
+  return np.ascontiguousarray(g[..., [0, 2, 4, 6, 1, 3, 5, 7]].reshape(a.shape))
+
+
+@pytest.mark.parametrize('k_order', [L.K_NATURAL, L.K_EVEN_ODD8])
+@pytest.mark.parametrize('batch,m,n,k', [(1, 256, 256, 256), (1, 512, 768, 384), (1, 300, 520, 160), (1, 64, 64, 32),
+                                           (3, 130, 70, 96), (1, 17, 9, 64), (1, 1024, 512, 1056), (1, 100, 4096, 4096)])
+def test_packed_int4_b_raw_accumulators(gpu, batch, m, n, k, k_order):
+  """int32 output and the copy of the accumulators: exact, whatever the byte order of A."""
+  a = _ints((batch, m, k), 11)
+  b = np.random.default_rng(12).integers(-8, 8, size=(batch, n, k)).astype(np.int8)
+  bp = ops.pack_i4(torch.from_numpy(b).to(gpu).reshape(batch * n, k)).reshape(batch, n, k // 2)
+  at = torch.from_numpy(_even_odd8(a) if k_order == L.K_EVEN_ODD8 else a).to(gpu)
+  c = ops.gemm(at, bp, row_scale=None, col_scale=None, out_dtype=torch.int32, b_dtype=L.I4P, a_k_order=k_order)
+  np.testing.assert_array_equal(c.cpu().numpy().astype(np.int64), _ref_acc(a, b))
+
+
+@pytest.mark.parametrize('out,rdt,cdt', [('bf16', 'bf16', 'bf16'), ('bf16', 'bf16', 'f32'), ('bf16', 'f32', 'f32'), ('f32', 'f32', 'f32')])
+@pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 4096), (2, 100, 72, 160), (1, 33, 20, 32)])
+def test_packed_int4_b_dequant_epilogue(gpu, batch, m, n, k, out, rdt, cdt):
+  """Same bits as the same contraction with the int4 values in int8 bytes, and as the oracle's dequant."""
+  a = _ints((batch, m, k), 13)
+  b = np.random.default_rng(14).integers(-8, 8, size=(batch, n, k)).astype(np.int8)
+  rs = nm.cast(np.abs(U.rand((batch, m), 'f32', 5, 0.03)) + np.float32(1e-3), rdt)
+  cs = nm.cast(np.abs(U.rand((batch, n), 'f32', 6, 6e-4)) + np.float32(1e-5), cdt)
+  acc = _ref_acc(a, b).astype(np.int32)
+  want = R.dequant(R.QTensor(acc, 'i32', [rs[:, :, None], cs[:, None, :]], None, out, scale_dtypes=[rdt, cdt]))
+  kw = dict(row_scale=torch.from_numpy(rs).to(gpu), col_scale=torch.from_numpy(cs).to(gpu), out_dtype=U.TORCH_DT[out],
+            row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt], want_acc=True)
+  bt = torch.from_numpy(b).to(gpu)
+  bp = ops.pack_i4(bt.reshape(batch * n, k)).reshape(batch, n, k // 2)
+  c0, acc0 = ops.gemm(torch.from_numpy(a).to(gpu), bt, b_dtype=L.I4, **kw)
+  c1, acc1 = ops.gemm(torch.from_numpy(a).to(gpu), bp, b_dtype=L.I4P, **kw)
+  c2, acc2 = ops.gemm(torch.from_numpy(_even_odd8(a)).to(gpu), bp, b_dtype=L.I4P, a_k_order=L.K_EVEN_ODD8, **kw)
+  np.testing.assert_array_equal(acc1.cpu().numpy(), acc)
+  np.testing.assert_array_equal(acc2.cpu().numpy(), acc)
+  np.testing.assert_array_equal(c1.float().cpu().numpy(), want)
+  assert torch.equal(c0, c1) and torch.equal(c1, c2)
+
+
+def test_packed_int4_b_rejected_where_unsupported(gpu):
+  a = torch.zeros((1, 64, 64), dtype=torch.int8, device=gpu)
+  bp = torch.zeros((1, 64, 32), dtype=torch.uint8, device=gpu)
+  ones = torch.ones((1, 64), device=gpu)
+  with pytest.raises(RuntimeError, match='ROW_THEN_COL'):
+    ops.gemm(a, bp, row_scale=ones, col_scale=ones, out_dtype=torch.bfloat16, b_dtype=L.I4P, scale_order=L.SCALE_COL_THEN_ROW)
+  with pytest.raises(RuntimeError, match='a_k_order'):
+    ops.gemm(a, a, row_scale=ones, col_scale=ones, out_dtype=torch.bfloat16, a_k_order=L.K_EVEN_ODD8)
+  with pytest.raises(RuntimeError, match='multiple of 32'):
+    ops.gemm(a[:, :, :48].contiguous(), bp[:, :, :24].contiguous(), row_scale=ones, col_scale=ones,
+             out_dtype=torch.bfloat16, b_dtype=L.I4P)
+
+
 # ---- fp8 ---------------------------------------------------------------------------------
 _FP8_TORCH = {'e4m3': torch.float8_e4m3fn, 'e5m2': torch.float8_e5m2}
 _FP8_AQTX = {'e4m3': L.E4M3, 'e5m2': L.E5M2}
