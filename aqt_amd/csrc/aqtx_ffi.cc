@@ -138,10 +138,11 @@ int FillGemmPlan(aqtx_gemm_plan* p, const ffi::AnyBuffer& a, const ffi::AnyBuffe
                  int32_t a_dtype, int32_t b_dtype, int32_t dequant_dtype, int32_t row_scale_dtype,
                  int32_t col_scale_dtype, int32_t scale_order) {
   auto ad = a.dimensions(), bd = b.dimensions();
-  if (ad.size() != 3 || bd.size() != 3 || ad[0] != bd[0] || ad[2] != bd[2]) return 1;
+  const bool b_packed = b_dtype == AQTX_I4P;  // b is then uint8 [batch, n, k / 2]
+  if (ad.size() != 3 || bd.size() != 3 || ad[0] != bd[0] || ad[2] != (b_packed ? 2 * bd[2] : bd[2])) return 1;
   p->batch = ad[0]; p->m = ad[1]; p->n = bd[1]; p->k = ad[2];
-  p->lda = p->k; p->ldb = p->k; p->ldc = p->n;
-  p->stride_a = p->m * p->k; p->stride_b = p->n * p->k; p->stride_c = p->m * p->n;
+  p->lda = p->k; p->ldb = bd[2]; p->ldc = p->n;
+  p->stride_a = p->m * p->k; p->stride_b = p->n * bd[2]; p->stride_c = p->m * p->n;
   p->a_dtype = a_dtype; p->b_dtype = b_dtype;
   p->out_dtype = Dtype(c_type);
   p->dequant_dtype = dequant_dtype;
@@ -151,14 +152,17 @@ int FillGemmPlan(aqtx_gemm_plan* p, const ffi::AnyBuffer& a, const ffi::AnyBuffe
   return 0;
 }
 
-// int8 (or int4-in-int8: a_dtype / b_dtype attributes) operands, dequantisation fused.
+// int8 (or int4-in-int8, or b packed int4 as uint8 [batch, n, k / 2]: a_dtype / b_dtype attributes) operands,
+// dequantisation fused.
 ffi::Error GemmI8Impl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b, ffi::Buffer<ffi::F32> row_scale,
                       ffi::Buffer<ffi::F32> col_scale, ffi::Result<ffi::AnyBuffer> c, int32_t a_dtype, int32_t b_dtype,
-                      int32_t dequant_dtype, int32_t row_scale_dtype, int32_t col_scale_dtype, int32_t scale_order) {
+                      int32_t dequant_dtype, int32_t row_scale_dtype, int32_t col_scale_dtype, int32_t scale_order,
+                      int32_t a_k_order) {
   aqtx_gemm_plan p{};
   if (FillGemmPlan(&p, a, b, c->element_type(), a_dtype, b_dtype, dequant_dtype, row_scale_dtype, col_scale_dtype,
                    scale_order))
     return Bad("aqtx_gemm_i8: operands must be [batch, m, k] and [batch, n, k]");
+  p.a_k_order = a_k_order;
   return Status(aqtx_gemm_i8(&p, a.untyped_data(), b.untyped_data(), row_scale.typed_data(), col_scale.typed_data(),
                              c->untyped_data(), nullptr, stream));
 }
@@ -297,7 +301,8 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Arg<ffi::Buffer<ffi::F32>>()    // col scale
         .Ret<ffi::AnyBuffer>()           // c
         .Attr<int32_t>("a_dtype").Attr<int32_t>("b_dtype").Attr<int32_t>("dequant_dtype")
-        .Attr<int32_t>("row_scale_dtype").Attr<int32_t>("col_scale_dtype").Attr<int32_t>("scale_order"));
+        .Attr<int32_t>("row_scale_dtype").Attr<int32_t>("col_scale_dtype").Attr<int32_t>("scale_order")
+        .Attr<int32_t>("a_k_order"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxGemmI8Raw, GemmI8RawImpl,
