@@ -51,6 +51,9 @@ class Tensor:
   dequant_mode: DequantMode = DequantMode.OUTPUT
   calibration_mode: CalibrationMode = CalibrationMode.CONTRACTING_AXIS
 
+  def __deepcopy__(self, memo):
+    return utils.deepcopy_fields(self, memo, shared=('use_fwd_quant', 'dequant_mode', 'calibration_mode'))
+
 
 @dataclasses.dataclass(kw_only=True)
 class LocalAqt:
@@ -58,6 +61,10 @@ class LocalAqt:
   contraction_axis_shard_count: Optional[int] = None
   contraction_axis_shard_size: Optional[int] = None
   tile_largest_shape: bool = False
+
+  def __deepcopy__(self, memo):
+    return utils.deepcopy_fields(self, memo, shared=(
+        'contraction_axis_shard_count', 'contraction_axis_shard_size', 'tile_largest_shape'))
 
 
 _FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
@@ -166,6 +173,9 @@ class DefaultDotGeneralQuantizer(DotGeneralQuantizer):
   lhs_mid_alpha: Optional[float] = None
   rhs_mid_alpha: Optional[float] = None
   skip_mid_scales: bool = True
+
+  def __deepcopy__(self, memo):
+    return utils.deepcopy_fields(self, memo, shared=('lhs_mid_alpha', 'rhs_mid_alpha', 'skip_mid_scales'))
 
   def init_calibration(self):
     self.lhs.init_calibration()
@@ -596,6 +606,11 @@ class DotGeneralRaw:
   jax_scope_name: str
   allow_dummy_gradient_into_qtensor: bool = False
   dot_general: Any = lax_dot_general
+
+  def __deepcopy__(self, memo):
+    # the accumulator dtype tag, the scope name and the inner dot_general (a function) are shared
+    return utils.deepcopy_fields(self, memo, shared=(
+        'dg_accumulator_dtype', 'jax_scope_name', 'allow_dummy_gradient_into_qtensor', 'dot_general'))
 
   @classmethod
   def make(cls, *args, **kwargs):
@@ -1046,6 +1061,9 @@ class DotGeneral:
   drhs: DotGeneralRaw
   apply_custom_vjp_on_jax: bool = True
 
+  def __deepcopy__(self, memo):
+    return utils.deepcopy_fields(self, memo, shared=('apply_custom_vjp_on_jax',))
+
   @classmethod
   def make(cls, *args, **kwargs):
     return dot_general_make(*args, **kwargs)
@@ -1195,13 +1213,10 @@ class DotGeneral:
                   and self.fwd.rhs.dequant_mode == dequant_mode), msg + ' for rhs.'
 
 
-def _fresh_cfg(cfg: 'DotGeneral') -> 'DotGeneral':
-  """Copy of the config tree down to the quantizers.
-
-  Under jax.custom_vjp the config reaches dg_core_vjp_fwd as a pytree argument, i.e. as a
-  fresh copy on every call, which is why init_calibration() may assert that it runs once;
-  this gives a reused config object the same behaviour.
-  """
+def clone_down_to_quantizers(cfg: 'DotGeneral', reset_calibrators: bool = False) -> 'DotGeneral':
+  """New DotGeneral / DotGeneralRaw / dot-general-quantizer / Quantizer objects around the same settings
+  objects (Tensor, LocalAqt, numerics, calibration factories are shared with `cfg`): everything a call
+  writes to (contexts, calibrators) is private to the copy."""
   cfg = utils.clone_fields(cfg)
   for name in ('fwd', 'dlhs', 'drhs'):
     raw = utils.clone_fields(getattr(cfg, name))
@@ -1209,11 +1224,22 @@ def _fresh_cfg(cfg: 'DotGeneral') -> 'DotGeneral':
     for qn in ('lhs', 'rhs', 'lhs_mid', 'rhs_mid'):
       if hasattr(dq, qn):
         q = utils.clone_fields(getattr(dq, qn))
-        q._calibrator = None
+        if reset_calibrators:
+          q._calibrator = None
         setattr(dq, qn, q)
     raw.dg_quantizer = dq
     setattr(cfg, name, raw)
   return cfg
+
+
+def _fresh_cfg(cfg: 'DotGeneral') -> 'DotGeneral':
+  """Copy of the config tree down to the quantizers, calibrators not yet made.
+
+  Under jax.custom_vjp the config reaches dg_core_vjp_fwd as a pytree argument, i.e. as a
+  fresh copy on every call, which is why init_calibration() may assert that it runs once;
+  this gives a reused config object the same behaviour.
+  """
+  return clone_down_to_quantizers(cfg, reset_calibrators=True)
 
 
 def dg_core_vjp_fwd(lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, cfg: DotGeneral):

@@ -42,8 +42,14 @@ def _split_key(key, num_splits: int):
 
 def set_context(cfg: DotGeneral, key, train_step: Optional[int],
                 lhs_quant_mode: utils.QuantMode = utils.QuantMode.TRAIN,
-                rhs_quant_mode: utils.QuantMode = utils.QuantMode.TRAIN):
-  """Fans the PRNG key out to fwd/dlhs/drhs and lhs/rhs (config.py:66-90)."""
+                rhs_quant_mode: utils.QuantMode = utils.QuantMode.TRAIN, *, copy_settings: bool = True):
+  """Fans the PRNG key out to fwd/dlhs/drhs and lhs/rhs (config.py:66-90).
+
+  Returns a deep copy of `cfg` with the contexts set, as the reference does.  With
+  copy_settings=False the copy stops at the quantizers (the objects the contexts are written to)
+  and shares the settings objects below them with `cfg`: for a caller that hands the result to
+  one dot_general call and drops it (the layer modules, on every call), at a fifth of the cost.
+  """
 
   def set_dg_raw_context(cfg_raw: DotGeneralRaw, key):
     key1, key2 = _split_key(key, num_splits=2)
@@ -52,7 +58,13 @@ def set_context(cfg: DotGeneral, key, train_step: Optional[int],
     cfg_raw.dg_quantizer.set_context(lhs_context, rhs_context)
 
   key_fwd, key_dlhs, key_drhs = _split_key(key, num_splits=3)
-  ret_cfg = copy.deepcopy(cfg)
+  plain = type(cfg) is DotGeneral and all(
+      type(raw) is DotGeneralRaw and type(raw.dg_quantizer) is aqt_dot_general.DefaultDotGeneralQuantizer
+      for raw in (cfg.fwd, cfg.dlhs, cfg.drhs))
+  if copy_settings or not plain:
+    ret_cfg = copy.deepcopy(cfg)
+  else:
+    ret_cfg = aqt_dot_general.clone_down_to_quantizers(cfg)
   set_dg_raw_context(ret_cfg.fwd, key_fwd)
   set_dg_raw_context(ret_cfg.dlhs, key_dlhs)
   set_dg_raw_context(ret_cfg.drhs, key_drhs)

@@ -212,20 +212,21 @@ class AqtDotGeneral(torch.nn.Module, _RngMixin):
       return aqt_dot_general.lax_dot_general
     cfg = self.cfg  # read only until config.set_context below makes the per-call copy
     lhs_shape, rhs_shape = tuple(lhs_shape), tuple(rhs_shape)
-    (contr, _) = dimension_numbers
-    ls, rs = list(lhs_shape), list(rhs_shape)
-    for li, ri in zip(*contr):
-      ls[li] = 1
-      rs[ri] = 1
-    lhs_scale_shape = tuple(transpose.lhs_scale_transpose_to_output(
-        torch.zeros(ls, device='meta'), dimension_numbers, lhs_shape, rhs_shape).shape)
-    rhs_scale_shape = tuple(transpose.rhs_scale_transpose_to_output(
-        torch.zeros(rs, device='meta'), dimension_numbers, lhs_shape, rhs_shape).shape)
     assert isinstance(cfg.fwd.dg_quantizer, aqt_dot_general.DefaultDotGeneralQuantizer)
-    lhs_q_dtype = cfg.fwd.dg_quantizer.lhs.numerics.get_dtype()
-    rhs_q_dtype = cfg.fwd.dg_quantizer.rhs.numerics.get_dtype()
 
     if self.use_legacy_freezer:
+      # the legacy freezer's variables have fixed shapes and dtypes: the scales as transposed to the output
+      (contr, _) = dimension_numbers
+      ls, rs = list(lhs_shape), list(rhs_shape)
+      for li, ri in zip(*contr):
+        ls[li] = 1
+        rs[ri] = 1
+      lhs_scale_shape = tuple(transpose.lhs_scale_transpose_to_output(
+          torch.zeros(ls, device='meta'), dimension_numbers, lhs_shape, rhs_shape).shape)
+      rhs_scale_shape = tuple(transpose.rhs_scale_transpose_to_output(
+          torch.zeros(rs, device='meta'), dimension_numbers, lhs_shape, rhs_shape).shape)
+      lhs_q_dtype = cfg.fwd.dg_quantizer.lhs.numerics.get_dtype()
+      rhs_q_dtype = cfg.fwd.dg_quantizer.rhs.numerics.get_dtype()
       lhs_freezer = self._freezer(self.lhs_var_name, lambda: Freezer(
           name=self.lhs_var_name, quant_mode=self.lhs_quant_mode, q_shape=lhs_shape, q_dtype=lhs_q_dtype,
           s_shape=lhs_scale_shape, quant_collection=self.quant_collection))
@@ -250,7 +251,7 @@ class AqtDotGeneral(torch.nn.Module, _RngMixin):
 
     key = self.make_rng(self.prng_name) if self.prng_name is not None else None
     cfg = config.set_context(cfg, key, train_step=None, lhs_quant_mode=self.lhs_quant_mode,
-                             rhs_quant_mode=self.rhs_quant_mode)
+                             rhs_quant_mode=self.rhs_quant_mode, copy_settings=False)
 
     def ret_dg(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
       del preferred_element_type
@@ -513,7 +514,7 @@ class AqtConvGeneralDilated(torch.nn.Module, _RngMixin):
       self._pending = None
     key = self.make_rng(self.prng_name) if self.prng_name is not None else None
     cfg = config.set_context(cfg, key, train_step=None, lhs_quant_mode=self.lhs_quant_mode,
-                             rhs_quant_mode=self.rhs_quant_mode)
+                             rhs_quant_mode=self.rhs_quant_mode, copy_settings=False)
 
     def ret_cg(lhs, rhs, window_strides, padding, lhs_dilation, rhs_dilation, dimension_numbers,
                feature_group_count, batch_group_count, precision, preferred_element_type):

@@ -1,4 +1,6 @@
 """Host-side logic of the aqt_amd.v2 mirror (runs without a GPU)."""
+import dataclasses
+
 import numpy as np
 import pytest
 import torch
@@ -292,3 +294,48 @@ def test_deep_copy_of_a_configuration_is_independent_and_equal():
   dup.fwd.dg_quantizer.lhs.numerics.bits = 4
   dup.fwd.dg_quantizer.lhs.context.train_step = 99
   assert cfg.fwd.dg_quantizer.lhs.numerics.bits == 8 and cfg.fwd.dg_quantizer.lhs.context.train_step == 7
+  # the containers above the quantizers are copied too (their own field-wise deep copies)
+  assert dup.fwd is not cfg.fwd and dup.fwd.lhs is not cfg.fwd.lhs
+  assert cfg.fwd.local_aqt is None or dup.fwd.local_aqt is not cfg.fwd.local_aqt
+  assert dup.fwd.dg_quantizer is not cfg.fwd.dg_quantizer and dup.fwd.dot_general is cfg.fwd.dot_general
+  dup.fwd.lhs.dequant_mode = aqt.DequantMode.THIS_INPUT
+  assert cfg.fwd.lhs.dequant_mode == aqt.DequantMode.OUTPUT
+
+  @dataclasses.dataclass(kw_only=True)
+  class WithTable(aqt.Tensor):  # a field a subclass adds is deep-copied, whatever it holds
+    table: list = dataclasses.field(default_factory=list)
+
+  t = WithTable(table=[[1, 2]])
+  t2 = copy.deepcopy(t)
+  assert t2 == t and t2.table is not t.table and t2.table[0] is not t.table[0]
+
+
+def test_set_context_without_copying_the_settings():
+  """copy_settings=False (what the layer modules pass on every call): the same contexts as the deep copy,
+  written to quantizers of its own, around the settings objects of the configuration it was given."""
+  base = config.fully_quantized(use_stochastic_rounding=True)
+  deep = config.set_context(base, utils.prng_key(3), train_step=7, rhs_quant_mode=utils.QuantMode.SERVE)
+  lean = config.set_context(base, utils.prng_key(3), train_step=7, rhs_quant_mode=utils.QuantMode.SERVE,
+                            copy_settings=False)
+  for name in ('fwd', 'dlhs', 'drhs'):
+    b, d, l = getattr(base, name), getattr(deep, name), getattr(lean, name)
+    assert l is not b and l.dg_quantizer is not b.dg_quantizer
+    assert l.lhs is b.lhs and l.local_aqt is b.local_aqt
+    for side in ('lhs', 'rhs'):
+      qb, qd, ql = (getattr(x.dg_quantizer, side) for x in (b, d, l))
+      assert ql is not qb and ql.numerics is qb.numerics
+      assert qb.context is None or qb.context.key is None  # the configuration handed in is left as it was
+      assert ql.context.quant_mode == qd.context.quant_mode and ql.context.train_step == 7
+      assert (ql.context.key is None) == (qd.context.key is None)
+      if ql.context.key is not None:
+        assert (np.asarray(ql.context.key) == np.asarray(qd.context.key)).all()
+
+  # a dot-general quantizer of another class is deep-copied as before
+  class Mine(aqt.DefaultDotGeneralQuantizer):
+    pass
+
+  other = config.fully_quantized()
+  other.fwd.dg_quantizer = Mine(**{f.name: getattr(other.fwd.dg_quantizer, f.name)
+                                   for f in dataclasses.fields(other.fwd.dg_quantizer)})
+  got = config.set_context(other, None, train_step=None, copy_settings=False)
+  assert got.fwd.lhs is not other.fwd.lhs and got.fwd.dg_quantizer.lhs.numerics is not other.fwd.dg_quantizer.lhs.numerics
