@@ -53,6 +53,8 @@ class GemmPlan(ctypes.Structure):
       ('group_offsets', ctypes.c_void_p),
       ('tuning', ctypes.c_int32),
       ('a_k_order', ctypes.c_int32),
+      ('k_split', ctypes.c_int32),
+      ('k_split_workspace', ctypes.c_void_p), ('k_split_workspace_bytes', ctypes.c_int64),
   ]
 
 
@@ -106,6 +108,7 @@ SYMBOLS = {
     'aqtx_quantize_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(QuantPlan)]),
     'aqtx_dequantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    'aqtx_gemm_i8_k_slices': (ctypes.c_int, [ctypes.POINTER(GemmPlan)]),
     'aqtx_gemm_fp8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_decode_i8': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _vp, ctypes.c_size_t, _vp]),

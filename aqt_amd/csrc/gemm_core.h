@@ -80,6 +80,12 @@ struct GemmArgs {
   // A with B[b] into the same rows of one flat C (m is then an upper bound of a group's rows).
   const int32_t* group_offsets;
   int a_even_odd8;  // packed int4 B only: A's bytes of every 8 k are stored as k 0,2,4,6,1,3,5,7
+  // Split K (gemm_mid_kernel): workgroup z of the grid contracts k in [z * k_chunk, (z + 1) * k_chunk) and
+  // writes its int32 partial sums to slab z of `slabs` ([k_split][batch][m][n]); dequant_slabs_kernel adds
+  // the slabs (integer addition: exact) and dequantizes.
+  int k_split;      // slices (<= 1: none)
+  int64_t k_chunk;  // k per slice, a multiple of 128
+  int32_t* slabs;
 };
 
 constexpr int BM = 256, BN = 256, BK = 128;
@@ -134,6 +140,20 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   const int in_band = id % band_tiles;
   tm = first_m + in_band % rows_in_band;
   tn = in_band / rows_in_band;
+}
+
+// QTensor.dequant of one accumulator for epilogue EPI (see gemm_kernel): cast to the dequant dtype, times
+// the first scale, times the second, each product rounded to the promoted dtype of its operands.
+template <int EPI, bool COL_FIRST, class AccScalar>
+__device__ __forceinline__ float dequant_value(AccScalar accv, float s_row, float s_col) {
+  constexpr bool kDqBf16 = EPI <= 1 || EPI == 4;
+  constexpr bool kProd1Bf16 = EPI == 0 || EPI == 4;     // promote(dequant dtype, first scale dtype)
+  constexpr bool kProd2Bf16 = EPI == 0;                 // promote(that, second scale dtype)
+  float f = round_to<kDqBf16>((float)accv);  // (int32 ->) f32 -> dequant dtype
+  const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
+  f = round_to<kProd1Bf16>(f * s1);
+  f = round_to<kProd2Bf16>(f * s2);
+  return round_to<kDqBf16>(f);
 }
 
 // EPI selects the epilogue arithmetic at compile time (run-time flags there turn into
@@ -423,10 +443,7 @@ void gemm_kernel(const GemmArgs g_in) {
   {
     // EPI 3 (raw accumulators as the output) takes the same staged, coalesced store path as the
     // float outputs: the 32-bit patterns travel through the float slots untouched.
-    constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
-    constexpr bool kDqBf16 = kOutBf16;                    // dequant dtype == output dtype
-    constexpr bool kProd1Bf16 = EPI == 0 || EPI == 4;     // promote(dequant dtype, first scale dtype)
-    constexpr bool kProd2Bf16 = EPI == 0;                 // promote(that, second scale dtype)
+    constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;       // dequant dtype == output dtype
     // A missing scale is a multiplication by 1, which every rounding below leaves alone.
     const float* rs = g.row_scale ? g.row_scale + bz * g.stride_rs : nullptr;
     const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
@@ -441,11 +458,7 @@ void gemm_kernel(const GemmArgs g_in) {
         if constexpr (BPACK) return __builtin_bit_cast(float, accv >> 4);
         else return __builtin_bit_cast(float, accv);
       }
-      float f = round_to<kDqBf16>((float)accv);  // (int32 ->) f32 -> dequant dtype
-      const float s1 = COL_FIRST ? s_col : s_row, s2 = COL_FIRST ? s_row : s_col;
-      f = round_to<kProd1Bf16>(f * s1);
-      f = round_to<kProd2Bf16>(f * s2);
-      return round_to<kDqBf16>(f);
+      return dequant_value<EPI, COL_FIRST>(accv, s_row, s_col);
     };
 
     // Each wave stages its 128-row block in LDS, RB = 256 (4 waves) or 128 (8 waves) bytes per
@@ -553,6 +566,60 @@ void gemm_kernel(const GemmArgs g_in) {
   }
 }
 
+// Second step of a split-K contraction: C = dequant(sum of the k_split int32 slabs [batch][m][n]) with the
+// arithmetic of the fused epilogue EPI (0, 1, 2, 4; 3 = the raw sums); also writes the sums to acc_out when
+// that is given.  One thread per four neighbouring columns.
+template <int EPI, bool COL_FIRST>
+__global__ __launch_bounds__(256) void dequant_slabs_kernel(const GemmArgs g) {
+  constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
+  const int64_t n4 = (int64_t)(blockIdx.x * 256 + threadIdx.x) * 4;
+  const int64_t mm = blockIdx.y, bz = blockIdx.z;
+  if (n4 >= g.n) return;
+  const int nv = (g.n - n4) < 4 ? (int)(g.n - n4) : 4;
+  const int64_t slab = (int64_t)gridDim.z * g.m * g.n;
+  const int64_t so = (bz * g.m + mm) * g.n + n4;
+  int a4[4] = {0, 0, 0, 0};
+  const bool svec = nv == 4 && (g.n % 4) == 0;
+  for (int z = 0; z < g.k_split; ++z) {
+    const int32_t* src = g.slabs + z * slab + so;
+    if (svec) {
+      const int4 t = *reinterpret_cast<const int4*>(src);
+      a4[0] += t.x; a4[1] += t.y; a4[2] += t.z; a4[3] += t.w;
+    } else {
+      for (int e = 0; e < nv; ++e) a4[e] += src[e];
+    }
+  }
+  const int64_t o = bz * g.stride_c + mm * g.ldc + n4;
+  if (g.acc_out != nullptr)
+    for (int e = 0; e < nv; ++e) reinterpret_cast<int32_t*>(g.acc_out)[o + e] = a4[e];
+  if constexpr (EPI == 3) {
+    for (int e = 0; e < nv; ++e) reinterpret_cast<int32_t*>(g.c)[o + e] = a4[e];
+  } else {
+    const float s_row = g.row_scale ? g.row_scale[bz * g.stride_rs + mm] : 1.0f;
+    const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+    float f[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      f[e] = dequant_value<EPI, COL_FIRST>(a4[e], s_row, (cs != nullptr && e < nv) ? cs[n4 + e] : 1.0f);
+    const bool cvec = nv == 4 && (g.ldc % 4) == 0 && (g.stride_c % 4) == 0;
+    if constexpr (kOutBf16) {
+      uint16_t* c = reinterpret_cast<uint16_t*>(g.c) + o;
+      if (cvec && ((uintptr_t)g.c % 8) == 0) {
+        uint2 w;
+        w.x = (uint32_t)bf16_bits(f[0]) | ((uint32_t)bf16_bits(f[1]) << 16);
+        w.y = (uint32_t)bf16_bits(f[2]) | ((uint32_t)bf16_bits(f[3]) << 16);
+        *reinterpret_cast<uint2*>(c) = w;
+      } else {
+        for (int e = 0; e < nv; ++e) c[e] = bf16_bits(f[e]);
+      }
+    } else {
+      float* c = reinterpret_cast<float*>(g.c) + o;
+      if (cvec && ((uintptr_t)g.c % 16) == 0) *reinterpret_cast<float4*>(c) = make_float4(f[0], f[1], f[2], f[3]);
+      else for (int e = 0; e < nv; ++e) c[e] = f[e];
+    }
+  }
+}
+
 // Reference-shaped fallback for operands the MFMA kernel cannot load with 16-byte
 // vectors (contraction length or leading dimension not a multiple of 16, unaligned
 // base).  One thread per output element; correct for any shape.  DEC_A/DEC_B decode one
@@ -646,9 +713,13 @@ inline GemmArgs make_gemm_args(const aqtx_gemm_plan* p, const void* a, const voi
   return g;
 }
 
+inline bool gemm_vector_shape_ok(const aqtx_gemm_plan* p) {
+  return (p->k % 16 == 0) && (p->lda % 16 == 0) && (p->ldb % 16 == 0) && (p->stride_a % 16 == 0) &&
+         (p->stride_b % 16 == 0) && p->k > 0;
+}
+
 inline bool gemm_vector_path_ok(const aqtx_gemm_plan* p, const void* a, const void* b) {
-  return (p->k % 16 == 0) && (p->lda % 16 == 0) && (p->ldb % 16 == 0) && ((uintptr_t)a % 16 == 0) &&
-         ((uintptr_t)b % 16 == 0) && (p->stride_a % 16 == 0) && (p->stride_b % 16 == 0) && p->k > 0;
+  return gemm_vector_shape_ok(p) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0);
 }
 
 // Epilogue id for the (out, dequant, scale) dtype triple, or -1.
@@ -664,5 +735,9 @@ inline int gemm_epilogue_id(const aqtx_gemm_plan* p) {
 }  // namespace
 
 int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8);
+// gemm_mid.hip: 0 = the plan stays with the 256 x 256 kernel, 1 = the 128 x 128 kernel, S > 1 = with K in S slices
+int gemm_mid_k_slices(const aqtx_gemm_plan* p);
+int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                       const float* col_scale, void* c, int32_t* acc_out, int slices, hipStream_t st);
 
 }  // namespace aqtx

@@ -40,6 +40,12 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
 
 using namespace aqtx;
 
+extern "C" int aqtx_gemm_i8_k_slices(const aqtx_gemm_plan* p) {
+  if (p == nullptr || p->k_split < 0 || p->k_split > 64 || p->batch <= 0 || p->m <= 0 || p->n <= 0) return 1;
+  const int s = gemm_mid_k_slices(p);
+  return s > 1 ? s : 1;
+}
+
 extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* b,
                             const float* row_scale, const float* col_scale, void* c,
                             int32_t* acc_out, void* stream) {
@@ -76,6 +82,17 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
     return set_error("aqtx_gemm_i8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
                      p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
   const bool ktail = (p->k % (2 * BK)) != 0;
+
+  // few output tiles: the 128 x 128 kernel, with K in slices where that still leaves CUs idle
+  AQTX_REQUIRE(p->k_split >= 0 && p->k_split <= 64, "aqtx_gemm_i8: k_split must be in 0..64, got %d", p->k_split);
+  if (int slices = gemm_mid_k_slices(p); slices > 0) {
+    // slices the library chose itself are dropped where the caller lent no (or too small a) workspace
+    if (p->k_split == 0 && slices > 1 &&
+        (p->k_split_workspace == nullptr || p->k_split_workspace_bytes < (int64_t)slices * p->batch * p->m * p->n * 4))
+      slices = 1;
+    return launch_gemm_i8_mid(p, a, b, row_scale, col_scale, c, acc_out, slices, st);
+  }
+  AQTX_REQUIRE(p->k_split <= 1, "aqtx_gemm_i8: k_split > 1 with ragged batches, plan->tuning or unaligned operands");
   // Two waves per SIMD by default: measured faster on every shape tried (the epilogue of one
   // wave overlaps the other's work).  plan->tuning = 4 | 8 overrides it (tests, tuning).
   const int waves = p->tuning == 4 ? 4 : 8;

@@ -1,0 +1,304 @@
+// int8 x int8 -> int32 contraction for shapes with few output tiles: the same arithmetic as the
+// 256 x 256 kernel of gemm_core.h on 128 x 128 tiles, optionally with K cut into slices.
+//
+// A 256 x 256 tile keeps one CU busy for all of K whatever the rest of the chip does, so a product
+// of 512 x 4096 (32 such tiles) leaves 224 of the 256 CUs idle.  Here a workgroup of 8 waves (4 x 2)
+// owns 128 x 128 of C, a wave 32 x 64 (two v_mfma_i32_32x32x32_i8 tiles, 32 accumulators), with 128
+// registers per lane and 72 KiB of LDS, so that two workgroups share a CU: four times the workgroups,
+// each a quarter of the work.  When even that leaves CUs idle and K is long, grid.z cuts K into slices
+// whose int32 partial sums go to slabs of a workspace, and dequant_slabs_kernel adds them up (integer
+// sums: exact in any order) and applies the epilogue.
+//
+// LDS rows are 144 bytes apart (128 of data, 16 of padding): the 16 lanes of a fragment read fall into
+// distinct banks and every address of the loop is a loop-invariant register plus an immediate.
+#include "gemm_core.h"
+
+namespace aqtx {
+namespace {
+
+constexpr int TM = 128, TN = 128;
+constexpr int kRow = BK + 16;
+constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile;  // 36 KiB
+
+// EPI, COL_FIRST as in gemm_kernel.  PACKED: B holds int4 values two per byte (see gemm_kernel's BPACK).
+// SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then).
+template <int EPI, bool COL_FIRST, bool PACKED, bool SLAB>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void gemm_mid_kernel(const GemmArgs g_in) {
+  static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
+  GemmArgs g = g_in;
+  __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[2 * kStage];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;  // 32 rows, 64 columns
+  const int lr = lane & 31, lh = lane >> 5;
+  int tm, tn;
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const int64_t bz = blockIdx.y;
+  const int64_t m0 = (int64_t)tm * TM, n0 = (int64_t)tn * TN;
+  if constexpr (SLAB) {  // this workgroup's slice of K
+    const int64_t kb = (int64_t)blockIdx.z * g.k_chunk;
+    g.a += kb;
+    g.b += PACKED ? kb / 2 : kb;
+    g.k = (g.k - kb) < g.k_chunk ? (g.k - kb) : g.k_chunk;
+  }
+  const int64_t rows_a = (g.m - m0) < TM ? (g.m - m0) : TM;
+  const int64_t rows_b = (g.n - n0) < TN ? (g.n - n0) : TN;
+  const int kb_bytes = PACKED ? (int)(g.k / 2) : (int)g.k;  // bytes of one B row (of this slice)
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + kb_bytes), kBufferRsrcWord3);
+
+  // ---- global -> registers -> LDS (rows past the operand read as zero, and so do the 16-byte chunks
+  // past K in the last stage).  A: 16 blocks of 8 rows x 128 B, two per wave.  B unpacked: the same.
+  // B packed: a wave load covers 16 rows x 64 B, one per wave; a lane's 16 bytes become the 32 bytes at
+  // 32 * (lane & 3) of its row.  The row and chunk of a load are in its vector offset, which the buffer's
+  // range check covers; the scalar offset (the stage's k) is not range checked, the mask on K covers it.
+  constexpr int NLA = 2, NLB = PACKED ? 1 : 2, NL = NLA + NLB;
+  constexpr int kOutside = 0x7FFFFFF0;
+  v4i stg[NL];
+  const int ld_a = (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
+  const int ld_b = PACKED ? (wave * 16 + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
+                          : (wave * 16 + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
+  const int kpos_a = (lane & 7) * 16, kpos_b = PACKED ? (lane & 3) * 32 : (lane & 7) * 16;
+  const int st_a = (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
+  const int st_b = kATile + (PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
+                                    : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
+  auto load_one = [&](const int j, int k0) {
+    if (j < NLA) {
+      const int vo = k0 + kpos_a < (int)g.k ? ld_a + j * 8 * (int)g.lda : kOutside;
+      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, k0, 0);
+    } else if constexpr (PACKED) {
+      const int vo = k0 + kpos_b < (int)g.k ? ld_b : kOutside;
+      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 / 2, 0);
+    } else {
+      const int vo = k0 + kpos_b < (int)g.k ? ld_b + (j - NLA) * 8 * (int)g.ldb : kOutside;
+      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0, 0);
+    }
+  };
+  auto store_stage = [&](const int stage_base) {
+    uint8_t* st = stage_mem + stage_base;
+#pragma unroll
+    for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
+    if constexpr (PACKED) {
+      v4i lo, hi;
+      unpack_i4x32(stg[NLA], lo, hi, g.a_even_odd8);
+      *reinterpret_cast<v4i*>(st + st_b) = lo;
+      *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLB; ++j) *reinterpret_cast<v4i*>(st + st_b + j * 8 * kRow) = stg[NLA + j];
+    }
+  };
+
+  // fragment of k step ks: 16 bytes at 32 ks + 16 lh of row lr of the 32-row block
+  const int a_off = (wm * 32 + lr) * kRow + lh * 16;
+  const int b_off = kATile + (wn * 64 + lr) * kRow + lh * 16;
+
+  v16i acc[2];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { acc[0][r] = 0; acc[1][r] = 0; }
+
+  const int nstages = (int)((g.k + BK - 1) / BK);
+#pragma unroll
+  for (int j = 0; j < NL; ++j) load_one(j, 0);
+  store_stage(0);
+#pragma unroll
+  for (int j = 0; j < NL; ++j) load_one(j, nstages > 1 ? BK : 0);
+  __syncthreads();
+
+  // Stage s reads buffer BUF; the staging registers (stage s + 1, requested during stage s - 1) go to the
+  // buffer stage s - 1 left, and the loads of stage s + 2 are issued behind them.  Past the last stage
+  // the store and the loads are repeated harmlessly (a buffer nobody reads, k offset 0) rather than
+  // branched around.
+  auto stage = [&](const int s, auto buf_c) {
+    constexpr int BUF = decltype(buf_c)::value;
+    const uint8_t* st = stage_mem + BUF * kStage;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const v4i fa = *reinterpret_cast<const v4i*>(st + a_off + ks * 32);
+      const v4i fb0 = *reinterpret_cast<const v4i*>(st + b_off + ks * 32);
+      const v4i fb1 = *reinterpret_cast<const v4i*>(st + b_off + 32 * kRow + ks * 32);
+      acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb0, fa, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb1, fa, acc[1], 0, 0, 0);
+    }
+    store_stage((1 - BUF) * kStage);
+    const int k_next = s + 2 < nstages ? (s + 2) * BK : 0;
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(j, k_next);
+    // a bare s_barrier: a __syncthreads() would also wait for the global loads just issued
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  for (int s = 0; s < nstages; s += 2) {
+    stage(s, std::integral_constant<int, 0>{});
+    if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
+  }
+
+  // ---- epilogue: lane holds C[m = wm*32 + lr][n = wn*64 + ni*32 + 8q + 4lh + e], register 4q + e of tile ni
+  const int64_t mm = m0 + wm * 32 + lr;
+  if (mm >= g.m) return;
+  if constexpr (SLAB) {
+    int32_t* dst = g.slabs + (((int64_t)blockIdx.z * gridDim.y + bz) * g.m + mm) * g.n;
+    const bool vec = (g.n % 4) == 0;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t nn = n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh;
+        if (nn >= g.n) continue;
+        int v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[ni][4 * q + e] >> 4 : acc[ni][4 * q + e];  // exact: multiples of 16
+        if (vec) *reinterpret_cast<int4*>(dst + nn) = make_int4(v[0], v[1], v[2], v[3]);
+        else for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[nn + e] = v[e];
+      }
+    return;
+  } else {
+    constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
+    constexpr int kEsz = kOutBf16 ? 2 : 4;
+    const int64_t row_o = bz * g.stride_c + mm * g.ldc;
+    const float s_row = g.row_scale ? g.row_scale[bz * g.stride_rs + mm] : 1.0f;
+    const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+    const bool cs_vec = ((uintptr_t)cs % 16) == 0;
+    const bool acc_vec = (g.ldc % 4) == 0 && (g.stride_c % 4) == 0 && ((uintptr_t)g.acc_out % 16) == 0;
+    const bool c_vec = (g.ldc % 4) == 0 && (g.stride_c % 4) == 0 && ((uintptr_t)g.c % (4 * kEsz)) == 0;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t nn = n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh;
+        if (nn >= g.n) continue;
+        const bool full = nn + 4 <= g.n;
+        int v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[ni][4 * q + e] >> 4 : acc[ni][4 * q + e];
+        if (g.acc_out != nullptr) {
+          int32_t* dst = reinterpret_cast<int32_t*>(g.acc_out) + row_o + nn;
+          if (full && acc_vec) *reinterpret_cast<int4*>(dst) = make_int4(v[0], v[1], v[2], v[3]);
+          else for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[e] = v[e];
+        }
+        uint8_t* dst = reinterpret_cast<uint8_t*>(g.c) + (row_o + nn) * kEsz;
+        if constexpr (EPI == 3) {
+          if (full && c_vec) *reinterpret_cast<int4*>(dst) = make_int4(v[0], v[1], v[2], v[3]);
+          else for (int e = 0; e < 4 && nn + e < g.n; ++e) reinterpret_cast<int32_t*>(dst)[e] = v[e];
+        } else {
+          float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+          if (cs != nullptr) {
+            if (full && cs_vec) {
+              const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
+              csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
+            } else {
+              for (int e = 0; e < 4 && nn + e < g.n; ++e) csv[e] = cs[nn + e];
+            }
+          }
+          float o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = dequant_value<EPI, COL_FIRST>(v[e], s_row, csv[e]);
+          if (full && c_vec) {
+            if constexpr (kOutBf16) {
+              uint2 w;
+              w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+              w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+              *reinterpret_cast<uint2*>(dst) = w;
+            } else {
+              *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+          } else {
+            for (int e = 0; e < 4 && nn + e < g.n; ++e) {
+              if constexpr (kOutBf16) reinterpret_cast<uint16_t*>(dst)[e] = bf16_bits(o[e]);
+              else reinterpret_cast<float*>(dst)[e] = o[e];
+            }
+          }
+        }
+      }
+  }
+}
+
+template <int EPI, bool COL_FIRST>
+void launch_mid(const GemmArgs& g, bool packed, dim3 grid, hipStream_t st) {
+  if constexpr (!COL_FIRST) {
+    if (packed) { gemm_mid_kernel<EPI, false, true, false><<<grid, 512, 0, st>>>(g); return; }
+  }
+  gemm_mid_kernel<EPI, COL_FIRST, false, false><<<grid, 512, 0, st>>>(g);
+}
+
+template <int EPI>
+void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
+  if constexpr (EPI != 3) {
+    if (g.col_first) { dequant_slabs_kernel<EPI, true><<<grid, 256, 0, st>>>(g); return; }
+  }
+  dequant_slabs_kernel<EPI, false><<<grid, 256, 0, st>>>(g);
+}
+
+}  // namespace
+
+// Whether the 128 x 128 kernel takes the plan (0 = no) and in how many slices of K (1 = none).
+int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
+  if (p->group_offsets != nullptr || p->tuning != 0 || !gemm_vector_shape_ok(p)) return 0;
+  if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
+  if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)TN >= (1ll << 31)) return 0;
+  const int64_t tiles256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN) * p->batch;
+  const int64_t tiles128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN) * p->batch;
+  const int64_t max_by_k = (p->k + 2 * BK - 1) / (2 * BK);  // a slice holds at least two stages
+  if (p->k_split > 1) return (int)(p->k_split < max_by_k ? p->k_split : max_by_k);
+  if (tiles256 > 128) return 0;  // the large tiles fill the chip
+  if (p->k_split == 1) return 1;
+  // slices until about 256 workgroups exist (one per CU; two fit), each walking at least 1024 of k; the
+  // slabs they write and the sum kernel reads stay small next to the operands at such tile counts
+  int64_t s = 256 / tiles128;
+  if (s > 8) s = 8;
+  if (s > p->k / 1024) s = p->k / 1024;
+  return s < 1 ? 1 : (int)s;
+}
+
+int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                       const float* col_scale, void* c, int32_t* acc_out, int slices, hipStream_t st) {
+  GemmArgs g = make_gemm_args(p, a, b, row_scale, col_scale, c, acc_out);
+  g.a_even_odd8 = p->a_k_order == AQTX_K_EVEN_ODD8;
+  g.tiles_m = (int)((p->m + TM - 1) / TM);
+  g.tiles_n = (int)((p->n + TN - 1) / TN);
+  const bool packed = p->b_dtype == AQTX_I4P;
+  const int epi = gemm_epilogue_id(p);
+  if (epi < 0)
+    return set_error("aqtx_gemm_i8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
+                     p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
+  dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
+  if (slices > 1) {
+    const int64_t need = (int64_t)slices * p->batch * p->m * p->n * 4;
+    AQTX_REQUIRE(p->k_split_workspace != nullptr && p->k_split_workspace_bytes >= need &&
+                     ((uintptr_t)p->k_split_workspace % 16) == 0,
+                 "aqtx_gemm_i8: %d slices of k need a 16-byte aligned k_split_workspace of %lld bytes", slices,
+                 (long long)need);
+    g.k_split = slices;
+    g.k_chunk = ((p->k + slices - 1) / slices + BK - 1) / BK * BK;
+    g.k_split = (int)((p->k + g.k_chunk - 1) / g.k_chunk);
+    g.slabs = reinterpret_cast<int32_t*>(p->k_split_workspace);
+    grid.z = (unsigned)g.k_split;
+    if (packed) gemm_mid_kernel<3, false, true, true><<<grid, 512, 0, st>>>(g);
+    else gemm_mid_kernel<3, false, false, true><<<grid, 512, 0, st>>>(g);
+    const dim3 egrid((unsigned)((p->n + 1023) / 1024), (unsigned)p->m, (unsigned)p->batch);
+    switch (epi) {
+      case 0: launch_slab_sum<0>(g, egrid, st); break;
+      case 1: launch_slab_sum<1>(g, egrid, st); break;
+      case 2: launch_slab_sum<2>(g, egrid, st); break;
+      case 4: launch_slab_sum<4>(g, egrid, st); break;
+      default: launch_slab_sum<3>(g, egrid, st); break;
+    }
+    AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel, k slices");
+    return 0;
+  }
+  switch (epi) {
+    case 0: if (g.col_first) launch_mid<0, true>(g, packed, grid, st); else launch_mid<0, false>(g, packed, grid, st); break;
+    case 1: if (g.col_first) launch_mid<1, true>(g, packed, grid, st); else launch_mid<1, false>(g, packed, grid, st); break;
+    case 2: if (g.col_first) launch_mid<2, true>(g, packed, grid, st); else launch_mid<2, false>(g, packed, grid, st); break;
+    case 4: if (g.col_first) launch_mid<4, true>(g, packed, grid, st); else launch_mid<4, false>(g, packed, grid, st); break;
+    default: launch_mid<3, false>(g, packed, grid, st); break;
+  }
+  AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel");
+  return 0;
+}
+
+}  // namespace aqtx

@@ -253,8 +253,12 @@ def gemm(
     want_acc: bool = False,
     group_offsets: Optional[torch.Tensor] = None,
     a_k_order: int = 0,
+    k_split: int = 0,
 ):
   """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
+
+  k_split (int8 operands; results do not depend on it): 0 = the library decides whether slices of k go
+  to workgroups of their own (few output tiles, long k), 1 = never, S > 1 = S slices.
 
   b_dtype = L.I4P: B is uint8 [batch, n, k/2], int4 values packed two per byte (pack_i4); with
   a_k_order = L.K_EVEN_ODD8 A was written by quantize(k_order=L.K_EVEN_ODD8).
@@ -299,11 +303,18 @@ def gemm(
   plan.scale_order = scale_order
   plan.tuning = GEMM_TUNING
   plan.a_k_order = a_k_order
+  plan.k_split = 1 if fp8 else k_split
   for s, shape in ((row_scale, (batch, m)), (col_scale, (b.shape[0], n))):
     if s is not None:
       assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == shape, (tuple(s.shape), shape)
   plan.row_scale_stride_b, plan.col_scale_stride_b = m, n
   fn = L.lib().aqtx_gemm_fp8 if fp8 else L.lib().aqtx_gemm_i8
+  slabs = None
+  if not fp8:
+    slices = L.lib().aqtx_gemm_i8_k_slices(ctypes.byref(plan))
+    if slices > 1:  # slices of k leave their partial sums in slabs of a scratch array
+      slabs = torch.empty((slices, batch, m, n), dtype=torch.int32, device=a.device)
+      plan.k_split_workspace, plan.k_split_workspace_bytes = slabs.data_ptr(), slabs.numel() * 4
   with _timed('gemm'):
     L.check(fn(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale), _ptr(col_scale), _ptr(c),
                _ptr(acc), _stream()))

@@ -167,6 +167,15 @@ typedef struct aqtx_gemm_plan {
                                  depend on it): 4 | 8 = waves per workgroup of the int8 kernel            */
   int32_t a_k_order;          /* AQTX_K_*: byte order of a along k; EVEN_ODD8 (aqtx_gemm_i8 with b_dtype
                                  AQTX_I4P only) saves the kernel the re-interleaving of the nibbles   */
+  int32_t k_split;            /* aqtx_gemm_i8 only.  Tuning only (int32 partial sums add up exactly in any
+                                 order): 0 = the library chooses, 1 = one workgroup per output tile walks
+                                 all of k, S > 1 = k is cut into (at most) S slices contracted by
+                                 workgroups of their own, for shapes with few output tiles and a long k.
+                                 Slices write partial sums to k_split_workspace                        */
+  void* k_split_workspace;    /* DEVICE scratch for the slices, 16-byte aligned, at least
+                                 aqtx_gemm_i8_k_slices(plan) * batch * m * n * 4 bytes; NULL: no slices
+                                 unless k_split > 1 asks for them (then an error)                      */
+  int64_t k_split_workspace_bytes;
 } aqtx_gemm_plan;
 
 /*
@@ -185,6 +194,13 @@ typedef struct aqtx_gemm_plan {
 int aqtx_gemm_i8(const aqtx_gemm_plan* plan, const void* a, const void* b,
                  const float* row_scale, const float* col_scale, void* c,
                  int32_t* acc_out, void* stream);
+
+/*
+ * Slices of k aqtx_gemm_i8 takes for `plan` when plan->k_split_workspace is large enough (see
+ * plan->k_split); 1 = none, no workspace needed.  No counterpart in the reference (XLA picks its own
+ * contraction algorithm).
+ */
+int aqtx_gemm_i8_k_slices(const aqtx_gemm_plan* plan);
 
 /*
  * aqtx_gemm_fp8: fp8 x fp8 -> float32 MFMA contraction (a_dtype/b_dtype select

@@ -12,9 +12,17 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[4, 8], ids=['waves4', 'waves8'])
+@pytest.fixture(params=[4, 8, 0], ids=['waves4', 'waves8', 'auto'])
 def waves(request, monkeypatch):
-  """Both workgroup shapes of the int8 MFMA kernel."""
+  """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, and the library's own choice (these
+  shapes have few output tiles: the 128 x 128 kernel, with k in slices where it is long)."""
+  monkeypatch.setattr(ops, 'GEMM_TUNING', request.param)
+  return request.param
+
+
+@pytest.fixture(params=[8, 0], ids=['tiles256', 'auto'])
+def tiles(request, monkeypatch):
+  """The 256 x 256 kernel, and the library's own choice (the 128 x 128 kernel for these shapes)."""
   monkeypatch.setattr(ops, 'GEMM_TUNING', request.param)
   return request.param
 
@@ -67,7 +75,7 @@ def test_dequant_epilogue(gpu, waves, batch, m, n, k, order, sdt, out):
 @pytest.mark.parametrize('rdt,cdt', [('bf16', 'f32'), ('f32', 'bf16')])
 @pytest.mark.parametrize('order', [L.SCALE_ROW_THEN_COL, L.SCALE_COL_THEN_ROW])
 @pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 512), (2, 100, 72, 160)])
-def test_dequant_epilogue_mixed_scale_dtypes(gpu, batch, m, n, k, order, rdt, cdt):
+def test_dequant_epilogue_mixed_scale_dtypes(gpu, tiles, batch, m, n, k, order, rdt, cdt):
   """A bf16 and an f32 scale: only a first product of two bf16 values is rounded to bf16."""
   a, b = _ints((batch, m, k), 3), _ints((batch, n, k), 4)
   rs = nm.cast(np.abs(U.rand((batch, m), 'f32', 5, 0.03)) + np.float32(1e-3), rdt)
@@ -99,6 +107,81 @@ def test_large_accumulators_round_like_xla(gpu, waves):
   np.testing.assert_array_equal(c.float().cpu().numpy(), want)
 
 
+# ---- k in slices (the 128 x 128 kernel writes int32 slabs, a second kernel adds and dequantizes) ----
+@pytest.mark.parametrize('slices', [2, 3, 7])
+@pytest.mark.parametrize('out,sdt,order', [('bf16', 'bf16', L.SCALE_ROW_THEN_COL), ('bf16', 'f32', L.SCALE_COL_THEN_ROW),
+                                           ('f32', 'f32', L.SCALE_ROW_THEN_COL), ('i32', None, None)])
+@pytest.mark.parametrize('batch,m,n,k', [(1, 128, 256, 4096), (2, 100, 72, 1200), (1, 33, 21, 528), (1, 300, 130, 2064)])
+def test_k_slices_give_the_same_bits(gpu, batch, m, n, k, out, sdt, order, slices):
+  a, b = _ints((batch, m, k), 31), _ints((batch, n, k), 32)
+  at, bt = torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu)
+  acc = _ref_acc(a, b).astype(np.int32)
+  if out == 'i32':
+    c = ops.gemm(at, bt, row_scale=None, col_scale=None, out_dtype=torch.int32, k_split=slices)
+    np.testing.assert_array_equal(c.cpu().numpy(), acc)
+    return
+  rs = nm.cast(np.abs(U.rand((batch, m), 'f32', 5, 0.03)) + np.float32(1e-3), sdt)
+  cs = nm.cast(np.abs(U.rand((batch, n), 'f32', 6, 6e-4)) + np.float32(1e-5), sdt)
+  s1, s2 = (rs[:, :, None], cs[:, None, :])
+  if order == L.SCALE_COL_THEN_ROW:
+    s1, s2 = s2, s1
+  want = R.dequant(R.QTensor(acc, 'i32', [s1, s2], sdt, out))
+  kw = dict(row_scale=torch.from_numpy(rs).to(gpu), col_scale=torch.from_numpy(cs).to(gpu),
+            out_dtype=U.TORCH_DT[out], scale_dtype=U.TORCH_DT[sdt], scale_order=order)
+  c, acc_got = ops.gemm(at, bt, want_acc=True, k_split=slices, **kw)
+  np.testing.assert_array_equal(acc_got.cpu().numpy(), acc)
+  np.testing.assert_array_equal(c.float().cpu().numpy(), want)
+  assert torch.equal(c, ops.gemm(at, bt, k_split=1, **kw))
+
+
+def test_k_slices_chosen_by_the_library(gpu):
+  """A long k over few output tiles is cut by default; the plan's answer and the result agree with k_split = 1."""
+  import ctypes
+  m, n, k = 128, 512, 14336
+  a, b = _ints((1, m, k), 33), _ints((1, n, k), 34)
+  at, bt = torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu)
+  plan = L.GemmPlan()
+  plan.batch, plan.m, plan.n, plan.k, plan.lda, plan.ldb, plan.ldc = 1, m, n, k, k, k, n
+  plan.a_dtype = plan.b_dtype = L.I8
+  assert L.lib().aqtx_gemm_i8_k_slices(ctypes.byref(plan)) == 8
+  plan.k_split = 1
+  assert L.lib().aqtx_gemm_i8_k_slices(ctypes.byref(plan)) == 1
+  plan.k_split, plan.m, plan.n = 0, 8192, 14336  # many tiles: never
+  assert L.lib().aqtx_gemm_i8_k_slices(ctypes.byref(plan)) == 1
+  rs = torch.rand(1, m, device=gpu) * 0.01 + 1e-3
+  cs = torch.rand(1, n, device=gpu) * 1e-3 + 1e-5
+  kw = dict(row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16)
+  got, want = ops.gemm(at, bt, **kw), ops.gemm(at, bt, k_split=1, **kw)
+  assert torch.equal(got, want)
+  np.testing.assert_array_equal(ops.gemm(at, bt, row_scale=None, col_scale=None, out_dtype=torch.int32).cpu().numpy(),
+                                _ref_acc(a, b))
+
+
+def test_k_slices_packed_int4_b(gpu):
+  a = _ints((1, 96, 2048), 35)
+  b = np.random.default_rng(36).integers(-8, 8, size=(1, 200, 2048)).astype(np.int8)
+  at, bt = torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu)
+  bp = ops.pack_i4(bt.reshape(200, 2048)).reshape(1, 200, 1024)
+  rs = torch.rand(1, 96, device=gpu) * 0.01 + 1e-3
+  cs = torch.rand(1, 200, device=gpu) * 1e-3 + 1e-5
+  kw = dict(row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16, want_acc=True)
+  c0, acc0 = ops.gemm(at, bt, b_dtype=L.I4, k_split=1, **kw)
+  for a_in, order in ((at, L.K_NATURAL), (torch.from_numpy(_even_odd8(a)).to(gpu), L.K_EVEN_ODD8)):
+    c1, acc1 = ops.gemm(a_in, bp, b_dtype=L.I4P, a_k_order=order, k_split=4, **kw)
+    assert torch.equal(c0, c1) and torch.equal(acc0, acc1)
+  np.testing.assert_array_equal(acc0.cpu().numpy(), _ref_acc(a, b))
+
+
+def test_k_slices_rejected_where_unsupported(gpu):
+  a = torch.zeros((1, 64, 512), dtype=torch.int8, device=gpu)
+  b = torch.zeros((1, 64, 512), dtype=torch.int8, device=gpu)
+  with pytest.raises(RuntimeError, match='k_split must be in 0..64'):
+    ops.gemm(a, b, row_scale=None, col_scale=None, out_dtype=torch.int32, k_split=65)
+  offs = torch.tensor([0, 64], dtype=torch.int32, device=gpu)
+  with pytest.raises(RuntimeError, match='k_split > 1 with ragged batches'):
+    ops.gemm(a, b, row_scale=None, col_scale=None, out_dtype=torch.int32, group_offsets=offs, k_split=2)
+
+
 # ---- packed int4 B (two values per byte, unpacked in registers) ---------------------------------
 def _even_odd8(a):
   g = a.reshape(a.shape[:-1] + (a.shape[-1] // 8, 8))
@@ -108,7 +191,7 @@ def _even_odd8(a):
 @pytest.mark.parametrize('k_order', [L.K_NATURAL, L.K_EVEN_ODD8])
 @pytest.mark.parametrize('batch,m,n,k', [(1, 256, 256, 256), (1, 512, 768, 384), (1, 300, 520, 160), (1, 64, 64, 32),
                                            (3, 130, 70, 96), (1, 17, 9, 64), (1, 1024, 512, 1056), (1, 100, 4096, 4096)])
-def test_packed_int4_b_raw_accumulators(gpu, batch, m, n, k, k_order):
+def test_packed_int4_b_raw_accumulators(gpu, tiles, batch, m, n, k, k_order):
   """int32 output and the copy of the accumulators: exact, whatever the byte order of A."""
   a = _ints((batch, m, k), 11)
   b = np.random.default_rng(12).integers(-8, 8, size=(batch, n, k)).astype(np.int8)
@@ -120,7 +203,7 @@ def test_packed_int4_b_raw_accumulators(gpu, batch, m, n, k, k_order):
 
 @pytest.mark.parametrize('out,rdt,cdt', [('bf16', 'bf16', 'bf16'), ('bf16', 'bf16', 'f32'), ('bf16', 'f32', 'f32'), ('f32', 'f32', 'f32')])
 @pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 4096), (2, 100, 72, 160), (1, 33, 20, 32)])
-def test_packed_int4_b_dequant_epilogue(gpu, batch, m, n, k, out, rdt, cdt):
+def test_packed_int4_b_dequant_epilogue(gpu, tiles, batch, m, n, k, out, rdt, cdt):
   """Same bits as the same contraction with the int4 values in int8 bytes, and as the oracle's dequant."""
   a = _ints((batch, m, k), 13)
   b = np.random.default_rng(14).integers(-8, 8, size=(batch, n, k)).astype(np.int8)
