@@ -153,9 +153,11 @@ int FillGemmPlan(aqtx_gemm_plan* p, const ffi::AnyBuffer& a, const ffi::AnyBuffe
 }
 
 // int8 (or int4-in-int8, or b packed int4 as uint8 [batch, n, k / 2]: a_dtype / b_dtype attributes) operands,
-// dequantisation fused.
+// dequantisation fused.  workspace: uint8 [aqtx_gemm_i8_k_slices(plan) * batch * m * n * 4] when that count is
+// above 1 (few output tiles and a long k: slices of k leave partial sums there), else any small buffer.
 ffi::Error GemmI8Impl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b, ffi::Buffer<ffi::F32> row_scale,
-                      ffi::Buffer<ffi::F32> col_scale, ffi::Result<ffi::AnyBuffer> c, int32_t a_dtype, int32_t b_dtype,
+                      ffi::Buffer<ffi::F32> col_scale, ffi::Result<ffi::AnyBuffer> c,
+                      ffi::Result<ffi::Buffer<ffi::U8>> workspace, int32_t a_dtype, int32_t b_dtype,
                       int32_t dequant_dtype, int32_t row_scale_dtype, int32_t col_scale_dtype, int32_t scale_order,
                       int32_t a_k_order) {
   aqtx_gemm_plan p{};
@@ -163,6 +165,8 @@ ffi::Error GemmI8Impl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b, ff
                    scale_order))
     return Bad("aqtx_gemm_i8: operands must be [batch, m, k] and [batch, n, k]");
   p.a_k_order = a_k_order;
+  p.k_split_workspace = workspace->typed_data();  // too small for the slices: the library takes none
+  p.k_split_workspace_bytes = (int64_t)workspace->size_bytes();
   return Status(aqtx_gemm_i8(&p, a.untyped_data(), b.untyped_data(), row_scale.typed_data(), col_scale.typed_data(),
                              c->untyped_data(), nullptr, stream));
 }
@@ -300,6 +304,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Arg<ffi::Buffer<ffi::F32>>()    // row scale
         .Arg<ffi::Buffer<ffi::F32>>()    // col scale
         .Ret<ffi::AnyBuffer>()           // c
+        .Ret<ffi::Buffer<ffi::U8>>()     // workspace
         .Attr<int32_t>("a_dtype").Attr<int32_t>("b_dtype").Attr<int32_t>("dequant_dtype")
         .Attr<int32_t>("row_scale_dtype").Attr<int32_t>("col_scale_dtype").Attr<int32_t>("scale_order")
         .Attr<int32_t>("a_k_order"));
