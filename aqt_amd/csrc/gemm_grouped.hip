@@ -200,6 +200,13 @@ void gemm_grouped128_kernel(const GroupedArgs g) {
       (void*)(g.a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + kb_bytes), kBufferRsrcWord3);
+  // The second load of an operand (rows 8 further down) has a descriptor of its own, 8 rows in: only the
+  // vector offset of a buffer load is range checked, so those 8 rows cannot travel in the scalar offset
+  // (rows past the operand would really be fetched), and a second vector offset would cost a register.
+  const __amdgpu_buffer_rsrc_t rsrc_a8 = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.a + (m0 + 8) * g.lda), 0, rows_a > 8 ? (int)((rows_a - 9) * g.lda + g.k) : 0, kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_b8 = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(g.b + (n0 + 8) * g.ldb), 0, rows_b > 8 ? (int)((rows_b - 9) * g.ldb + kb_bytes) : 0, kBufferRsrcWord3);
   // group scales: waves 0, 1 fetch the 128 row scales, waves 2, 3 the 128 column scales of the next
   // group, one per lane, through a buffer whose scalar offset selects the group.  Nothing reads the
   // result before it goes to LDS at the end of the stage: a use next to the load would wait there
@@ -214,9 +221,11 @@ void gemm_grouped128_kernel(const GroupedArgs g) {
       (void*)((sc_row ? g.row_scale : g.col_scale) + sc_skip), 0, (int)(((int64_t)g.groups * sc_len - sc_skip) * 4),
       kBufferRsrcWord3);
   const int sc_step = sc_by_idx ? 4 : (int)sc_len * 4;  // bytes from one group's scale to the next
-  const int sc_voff = sc_idx * (sc_by_idx ? g.groups * 4 : 4);
+  // lanes past the operand fetch its last scale (store_scales masks them): no address past the array
+  const int sc_idx_in = sc_first + sc_idx < sc_len ? sc_idx : (int)(sc_len - 1 - sc_first);
+  const int sc_voff = sc_idx_in * (sc_by_idx ? g.groups * 4 : 4);
   float sc_reg = 1.0f;
-  auto load_scales = [&](int grp) {  // lanes past the operand read another row's scale or zero; store_scales masks them
+  auto load_scales = [&](int grp) {
     const int grp_c = grp < g.groups ? grp : g.groups - 1;
     if (sc_active) sc_reg = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, sc_voff, grp_c * sc_step, 0));
   };
@@ -230,7 +239,7 @@ void gemm_grouped128_kernel(const GroupedArgs g) {
   // ---- global -> registers -> LDS (rows past the operand read as zero) ----------------------
   // A: 16 blocks of 8 rows x 128 B, two per wave.  B unpacked: 16 such blocks, two per wave.
   // B packed: a wave load covers 16 rows x 64 B, one per wave; a lane's 16 bytes become the 32
-  // bytes at 32 * (lane & 3) of its row.  Loads j of one operand differ by a scalar offset.
+  // bytes at 32 * (lane & 3) of its row.  The two loads of an operand differ by their descriptor.
   constexpr int NLA = 2, NLB = PACKED ? 1 : 2, NL = NLA + NLB;
   v4i stg[NL];
   const int ld_a = (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
@@ -240,9 +249,9 @@ void gemm_grouped128_kernel(const GroupedArgs g) {
   const int st_b = kATile + (PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
                                     : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
   auto load_one = [&](const int j, int k0) {
-    if (j < NLA) stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ld_a, k0 + j * 8 * (int)g.lda, 0);
+    if (j < NLA) stg[j] = __builtin_amdgcn_raw_buffer_load_b128(j == 0 ? rsrc_a : rsrc_a8, ld_a, k0, 0);
     else if constexpr (PACKED) stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ld_b, k0 / 2, 0);
-    else stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ld_b, k0 + (j - NLA) * 8 * (int)g.ldb, 0);
+    else stg[j] = __builtin_amdgcn_raw_buffer_load_b128(j == NLA ? rsrc_b : rsrc_b8, ld_b, k0, 0);
   };
   auto store_stage = [&](const int stage_base) {
     uint8_t* st = stage_mem + stage_base;
