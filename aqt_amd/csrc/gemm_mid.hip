@@ -237,15 +237,18 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 
 // Whether the 128 x 128 kernel takes the plan (0 = no) and in how many slices of K (1 = none).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
-  if (p->group_offsets != nullptr || p->tuning != 0 || !gemm_vector_shape_ok(p)) return 0;
+  if (p->group_offsets != nullptr || (p->tuning != 0 && p->tuning != 128) || !gemm_vector_shape_ok(p)) return 0;
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
   if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)TN >= (1ll << 31)) return 0;
-  const int64_t tiles256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN) * p->batch;
-  const int64_t tiles128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN) * p->batch;
+  const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);
+  const int64_t pad128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN);
+  const int64_t tiles256 = pad256 * p->batch, tiles128 = pad128 * p->batch;
   const int64_t max_by_k = (p->k + 2 * BK - 1) / (2 * BK);  // a slice holds at least two stages
   if (p->k_split > 1) return (int)(p->k_split < max_by_k ? p->k_split : max_by_k);
-  if (tiles256 > 128) return 0;  // the large tiles fill the chip
-  if (p->k_split == 1) return 1;
+  // the large tiles fill the chip, unless a third of their area or more lies outside C (n or m of 128, say)
+  const bool padded = 4 * pad256 * 2 >= 3 * pad128;
+  if (p->tuning != 128 && tiles256 > 128 && !padded) return 0;
+  if (p->k_split == 1 || tiles256 > 128) return 1;
   // slices until about 256 workgroups exist (one per CU; two fit), each walking at least 1024 of k; the
   // slabs they write and the sum kernel reads stay small next to the operands at such tile counts
   int64_t s = 256 / tiles128;

@@ -12,10 +12,10 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[4, 8, 0], ids=['waves4', 'waves8', 'auto'])
+@pytest.fixture(params=[4, 8, 128, 0], ids=['waves4', 'waves8', 'tiles128', 'auto'])
 def waves(request, monkeypatch):
-  """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, and the library's own choice (these
-  shapes have few output tiles: the 128 x 128 kernel, with k in slices where it is long)."""
+  """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, the 128 x 128 kernel, and the library's own
+  choice (these shapes have few output tiles: the 128 x 128 kernel, with k in slices where it is long)."""
   monkeypatch.setattr(ops, 'GEMM_TUNING', request.param)
   return request.param
 
