@@ -87,6 +87,14 @@ __device__ __forceinline__ void unpack_i4x8(uint32_t w, int& lo, int& hi) {
   hi = (int)__builtin_amdgcn_perm(od, ev, 0x07030602u);  // k4 k5 k6 k7
 }
 
+// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for the global loads
+// in flight (the weights requested ahead of the quantisation).
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // ---- few rows: activation quantisation inside the contraction kernel ------------------------------
 // For a handful of tokens the separate quantize launch costs as much as a third of the call.
 // Here every workgroup quantizes the activations itself (they come from L2: ROWS * k values),
@@ -128,11 +136,6 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   constexpr int wstep = WFRAG ? 1024 : 64;
   auto w_offset = [&](int ko) { return (ko + c * KL < k_hi) ? wbase + (ko / KS) * wstep : kOob; };
 
-  // first batch of weights: in flight while the activations are quantized
-  v4i wf[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
-
   // ---- quantize the activations into LDS
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.x, (int64_t)d.m * d.k * (int64_t)sizeof(TIn));
   uint32_t raw[ROWS][PPT][WPP];
@@ -150,6 +153,11 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
         raw[i][j][4 * q + 2] = (uint32_t)t[2]; raw[i][j][4 * q + 3] = (uint32_t)t[3];
       }
     }
+  // first batch of weights: in flight while the activations are quantized.  Requested after the
+  // activations: loads return in order, so the other way round the quantisation would wait for the weights.
+  v4i wf[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
   auto value = [&](int i, int j, int e) -> float {
     if constexpr (XBF) {
       const uint32_t w = raw[i][j][e >> 1];
@@ -169,7 +177,7 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
     for (int off = 32; off > 0; off >>= 1) amax = nanmax(amax, __shfl_xor(amax, off, 64));
     if (lane == 0) smax[i][wave] = amax;
   }
-  __syncthreads();
+  lds_barrier();
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) {
     float amax = nanmax(nanmax(smax[i][0], smax[i][1]), nanmax(smax[i][2], smax[i][3]));
@@ -201,7 +209,7 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
       }
     }
   }
-  __syncthreads();
+  lds_barrier();
 
   // ---- contraction, weights from HBM, activations from LDS
   v4i acc = v4i{0, 0, 0, 0};
@@ -288,13 +296,6 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
   constexpr int wstep = WFRAG ? 1024 : 64;
   auto w_offset = [&](int ko) { return (ko + c * KL < k_hi) ? wbase + (ko / KS) * wstep : kOob; };
 
-  // first batch of weights: in flight while the activations are quantized
-  v4i wf[U];
-  if (contracts) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
-  }
-
   // ---- quantize the activations into LDS: thread t works on row 4 * pass + t / 256, pieces t % 256 + 256 j
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.x, (int64_t)d.m * d.k * (int64_t)sizeof(TIn));
   const int sub = tid >> 8, tt = tid & 255, gw = (tid >> 6) & 3;  // row of the pass, thread and wave inside the row's group
@@ -313,6 +314,7 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
         raw[ps][j][4 * q + 2] = (uint32_t)t[2]; raw[ps][j][4 * q + 3] = (uint32_t)t[3];
       }
     }
+  v4i wf[U];
   auto value = [&](int ps, int j, int e) -> float {
     if constexpr (XBF) {
       const uint32_t w = raw[ps][j][e >> 1];
@@ -321,6 +323,7 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
       return __uint_as_float(raw[ps][j][e]);
     }
   };
+  auto quantize_rows = [&]() {
 #pragma unroll
   for (int ps = 0; ps < PASSES; ++ps) {
     float amax = 0.0f;
@@ -345,7 +348,7 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
     for (int off = 32; off > 0; off >>= 1) amax = nanmax(amax, __shfl_xor(amax, off, 64));
     if (lane == 0) smax[4 * ps + sub][gw] = amax;
   }
-  __syncthreads();
+  lds_barrier();
   const int tbf = d.x_bf16 & d.xs_bf16;
 #pragma unroll
   for (int ps = 0; ps < PASSES; ++ps) {
@@ -391,7 +394,19 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
     };
     if (tbf) quantize_row(std::true_type{}); else quantize_row(std::false_type{});
   }
-  __syncthreads();
+  };
+  // The waves that contract request their first batch of weights now, after the activations (loads
+  // return in order: the other way round the quantisation would wait for the weights), and quantize
+  // with them in flight.  Two copies of the quantisation, one per kind of wave: after a join the
+  // compiler would make every wave wait as if it had weights outstanding.
+  if (contracts) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
+    quantize_rows();
+  } else {
+    quantize_rows();
+  }
+  lds_barrier();
 
   // ---- contraction (waves 0..3), weights from HBM, activations from LDS
   if (contracts) {
@@ -403,32 +418,37 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
 #pragma unroll
         for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, 0);
       }
-      v4i xf[U][XP];
+      // four weight loads' worth of activation fragments at a time (all U at once would double the registers)
+      constexpr int UC = U < 4 ? U : 4;
 #pragma unroll
-      for (int u = 0; u < U; ++u)
+      for (int u0 = 0; u0 < U; u0 += UC) {
+        v4i xf[UC][XP];
 #pragma unroll
-        for (int h = 0; h < XP; ++h) {
-          const int pj = (kk + u * KS) / 16 + c * XP + h;
-          xf[u][h] = v4i{0, 0, 0, 0};
-          if (row_ok && pj < pieces) {
-            const int pos = (pj & ~15) | ((pj & 15) ^ r);
-            xf[u][h] = *reinterpret_cast<const v4i*>(xlds + (size_t)r * kp + pos * 16);
+        for (int u = 0; u < UC; ++u)
+#pragma unroll
+          for (int h = 0; h < XP; ++h) {
+            const int pj = (kk + (u0 + u) * KS) / 16 + c * XP + h;
+            xf[u][h] = v4i{0, 0, 0, 0};
+            if (row_ok && pj < pieces) {
+              const int pos = (pj & ~15) | ((pj & 15) ^ r);
+              xf[u][h] = *reinterpret_cast<const v4i*>(xlds + (size_t)r * kp + pos * 16);
+            }
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < UC; ++u) {
+          if constexpr (PACKED) {
+            int t[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[u0 + u][j], t[2 * j], t[2 * j + 1]);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], v4i{t[0], t[1], t[2], t[3]}, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][1], v4i{t[4], t[5], t[6], t[7]}, acc, 0, 0, 0);
+          } else {
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], wf[u0 + u], acc, 0, 0, 0);
           }
         }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if constexpr (PACKED) {
-          int t[8];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) unpack_i4x8((uint32_t)wf[u][j], t[2 * j], t[2 * j + 1]);
-          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], v4i{t[0], t[1], t[2], t[3]}, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][1], v4i{t[4], t[5], t[6], t[7]}, acc, 0, 0, 0);
-        } else {
-          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[u][0], wf[u], acc, 0, 0, 0);
-        }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[wave][4 * c + e][r] = acc[e];
@@ -966,9 +986,10 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
 
   // Three or four tokens against a weight of at most 256 16-row blocks (one workgroup per CU, so the
   // quantisation every workgroup repeats is paid once): one kernel again, on 16 waves per workgroup.
-  // Measured at k = 4096, n = 4096: 7.7 us against 9.0-9.2 us for the two kernels below; at 8 tokens
-  // the two are equal, and with several rounds of workgroups (n = 14336) the repeated quantisation
-  // loses by 5-12 us.
+  // Measured at k = 4096, n = 4096: 7.7 us against 9.0-9.2 us for the two kernels below; with 8 rows
+  // per workgroup the two are equal and with 16 this one loses by 3 us (its time grows by 0.37 us per
+  // row, the vector work of quantizing a row on one CU, whatever the weight loads in flight); with
+  // several rounds of workgroups (n = 14336) the repeated quantisation loses by 5-12 us.
   const unsigned wide_grid = (unsigned)((p->n + 15) / 16);
   if (!never_fuse && p->m <= 4 && p->k <= 8192 && wide_grid <= 256) {
     d.xq_out = reinterpret_cast<int8_t*>(xq);
