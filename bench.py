@@ -266,7 +266,27 @@ def other_configs(dev):
   out['conv_int8_fwd_32x56x56x128_k3x3_128'] = {
       'ms_per_call': round(ms, 3), 'TOPS': round(gop / ms, 1),
       'hip_graph_ms_per_call': round(ms_graph, 3), 'hip_graph_TOPS': round(gop / ms_graph, 1)}
-  del graphed
+  del graphed, xc, kc
+  # the reference's own small case: a two-layer MLP block, x f32 [4096, 512], Dense 512 -> 2048, ReLU,
+  # Dense 2048 -> 512, fully_quantized(8, 8) with stochastic rounding in the backward pass, forward + backward
+  # issued from Python (host time included: at this size the step is bound by it, not by the kernels)
+  xm = torch.randn(4096, 512, device=dev, requires_grad=True)
+  w1 = (torch.randn(512, 2048, device=dev) / 512 ** 0.5).requires_grad_(True)
+  w2 = (torch.randn(2048, 512, device=dev) / 2048 ** 0.5).requires_grad_(True)
+  gm = torch.randn(4096, 512, device=dev) / (4096 * 512)
+  mlp_cfg = config.fully_quantized(fwd_bits=8, bwd_bits=8)
+  k1, k2 = utils.prng_key(1), utils.prng_key(2)
+
+  def step_mlp():
+    h = config.set_context(mlp_cfg, k1, None)(xm, w1, MATMUL)
+    y = config.set_context(mlp_cfg, k2, None)(torch.relu(h), w2, MATMUL)
+    y.backward(gm)
+    xm.grad = w1.grad = w2.grad = None
+
+  ms = timeit(step_mlp, n=30, w=5)
+  out['mlp_block_f32_4096x512_2048_512_fwd_bwd'] = {
+      'ms_per_step_from_python': round(ms, 3), 'TOPS': round(3 * 2 * 2 * 4096 * 512 * 2048 / ms / 1e9, 1)}
+  del xm, w1, w2, gm
   return out
 
 

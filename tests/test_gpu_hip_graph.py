@@ -48,11 +48,12 @@ def _check_replays(graphed, eager, make_input, n=5):
     assert torch.equal(got, want), f'replay {i} differs from the eager call'
 
 
-@pytest.mark.parametrize('m', [1, 8, 64, 512])
-def test_int8_serving_layer_replays(gpu, m):
-  """Frozen int8 weight: the small-batch decode kernels (m <= 64) and the dense GEMM (m = 512)."""
+@pytest.mark.parametrize('m,k', [(1, 1024), (8, 1024), (64, 1024), (512, 1024), (96, 4096)])
+def test_int8_serving_layer_replays(gpu, m, k):
+  """Frozen int8 weight: the small-batch decode kernels (m <= 64) and the dense GEMM (m = 512; m = 96 with
+  k = 4096: few output tiles and a long k, contracted in slices of k through a scratch array)."""
   dt = 'bf16'
-  k, n = 1024, 1536
+  n = 1536
   w = U.to_dev(U.rand((k, n), dt, 2, 0.02), dt, gpu)
   mk = lambda seed: U.to_dev(U.rand((m, k), dt, seed, outliers=True), dt, gpu)
   serve = _serving_layer(config.fully_quantized(use_stochastic_rounding=False), mk(1), w)
