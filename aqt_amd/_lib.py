@@ -64,7 +64,7 @@ class GroupedGemmPlan(ctypes.Structure):
       ('lda', ctypes.c_int64), ('ldb', ctypes.c_int64), ('ldc', ctypes.c_int64),
       ('a_dtype', ctypes.c_int32), ('b_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
       ('row_scale_dtype', ctypes.c_int32), ('col_scale_dtype', ctypes.c_int32),
-      ('a_k_order', ctypes.c_int32), ('row_scale_by_row', ctypes.c_int32),
+      ('a_k_order', ctypes.c_int32), ('row_scale_by_row', ctypes.c_int32), ('tuning', ctypes.c_int32),
   ]
 
 

@@ -14,8 +14,8 @@
 // 1.5 ns for add/mul/and and 2.3 ns for the conversions and shifts), so a kernel of this kind
 // wants 4 waves per SIMD, i.e. at most 128 registers per lane, more than it wants large tiles.
 //
-// Two kernels, both with 128-byte K stages double-buffered in LDS, the group scales of a stage
-// next to it in LDS:
+// Two tile kernels, both with 128-byte K stages double-buffered in LDS, the group scales of a stage
+// next to it in LDS (and gemm_grouped_rows_kernel, further down, for at most 64 rows of A):
 //   gemm_grouped128_kernel  group = 128 (one stage per group).  Workgroup = 8 waves (4 x 2) on a
 //       128 x 128 tile of C, a wave 32 x 64 = two MFMA tiles (v_mfma_i32_32x32x32_i8): 32 int32
 //       accumulators of the current group and 32 float32 running sums; two workgroups per CU.
@@ -498,6 +498,161 @@ __global__ void pack_i4_kernel(const int8_t* src, uint8_t* dst, int64_t count2) 
   dst[i] = (uint8_t)(lo | (hi << 4));
 }
 
+// ---- at most 64 rows of A (serving with a frozen subchannel weight) ----------------------------------
+// The tile kernels above rescale a 128-row tile of C per group whatever m is: with a handful of tokens
+// almost all of that vector work is spent on rows that do not exist (measured: 100 us for 1..64 tokens
+// against 2048 x 8192 x 28672's packed weight, 15 % of what the weight stream alone would take).  Here a
+// wave owns 16 rows of B and all tokens (MB blocks of 16) for all of K, in group order, so the running sums
+// add up in the order of the tile kernels: v_mfma_i32_16x16x64_i8 with the activations as the first
+// operand leaves a lane with tokens 4c .. 4c + 3 (c = lane / 16) of column lane % 16, i.e. four row scales
+// and one column scale per lane and group.  A group of 128 k is one 16-byte load per lane of a packed
+// weight row (two of an int8 one), requested U groups ahead, straight from global memory into the MFMA
+// operand.  The activations are shared by the NW waves of a workgroup: chunks of four groups go through
+// LDS, double buffered (two with 64 tokens; every wave reading all of them from L2 instead cost as much again as the weight
+// stream at 8 tokens and eight times that at 64); rows are 528 bytes apart, so that the 16 lanes of one
+// operand read hit distinct banks.  The row scales of all groups sit in LDS, transposed to [group][token].
+constexpr int rows_chunk_groups(int mb) { return mb == 4 ? 2 : 4; }  // 64 tokens: half the chunk, the same LDS
+
+template <int EPI, bool PACKED, int MB, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const GroupedArgs g) {
+  using R = Rescale<EPI>;
+  constexpr int MT = 16 * MB;      // tokens
+  constexpr int CG = rows_chunk_groups(MB);  // groups per activation chunk
+  constexpr int kPitch = CG * 128 + 16;
+  constexpr int NT = NW * 64;
+  constexpr int PPC = CG * 8;           // 16-byte pieces of one token's chunk
+  constexpr int XL = MT * PPC / NT;     // 16-byte activation loads per thread and chunk
+  static_assert(XL >= 1 && MT * PPC % NT == 0, "chunk loads divide among the threads");
+  extern __shared__ __attribute__((aligned(16))) uint8_t rows_lds[];
+  uint8_t* xbuf = rows_lds;                                                  // [2][MT][kPitch]
+  float* srow_all = reinterpret_cast<float*>(rows_lds + 2 * MT * kPitch);    // [groups][MT]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int n0 = ((int)blockIdx.x * NW + wave) * 16;
+  for (int i = tid; i < g.groups * MT; i += NT) {
+    const int grp = i / MT, t = i % MT;
+    float v = 1.0f;
+    if (t < g.m) v = g.rs_by_row ? g.row_scale[(int64_t)t * g.groups + grp] : g.row_scale[(int64_t)grp * g.m + t];
+    srow_all[i] = v;
+  }
+  const int kb = PACKED ? (int)(g.k / 2) : (int)g.k;
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)g.a, 0, (int)((g.m - 1) * g.lda + g.k), kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)g.b, 0, (int)((g.n - 1) * g.ldb + kb), kBufferRsrcWord3);
+  constexpr int kOutside = 0x7FFFFFF0;
+  // lane (r, c): weight row n0 + r, bytes 16 c (packed: k 32 c .. 32 c + 31 of the group) or 32 c (int8:
+  // the same k); the activations of token r, the same k: 32 bytes
+  constexpr int WL = PACKED ? 1 : 2;
+  const int wrow = n0 + r;
+  const int woff = wrow < g.n ? wrow * (int)g.ldb + c * (PACKED ? 16 : 32) : kOutside;
+  const int ncol = wrow < g.n ? wrow : (int)g.n - 1;
+  const float cfold = PACKED ? 0.0625f : 1.0f;  // packed nibbles are unpacked to 16 * value
+  const int nchunks = (g.groups + CG - 1) / CG;
+
+  // activation chunk: load j of a thread is the 16-byte piece (tid + j NT) % PPC of token (tid + j NT) / PPC
+  v4i xs[XL];
+  auto request_x = [&](int ch) {
+#pragma unroll
+    for (int j = 0; j < XL; ++j) {
+      const int id = tid + j * NT, t = id / PPC, piece = id % PPC;
+      const bool ok = t < g.m && ch * CG * 128 + piece * 16 < (int)g.k && ch < nchunks;
+      xs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? t * (int)g.lda + piece * 16 : kOutside,
+                                                    ok ? ch * CG * 128 : 0, 0);
+    }
+  };
+  auto store_x = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < XL; ++j) {
+      const int id = tid + j * NT, t = id / PPC, piece = id % PPC;
+      *reinterpret_cast<v4i*>(xbuf + (buf * MT + t) * kPitch + piece * 16) = xs[j];
+    }
+  };
+  v4i wf[CG][WL];
+  float cs[CG];
+  auto request_w = [&](const int u, int grp) {
+    const int gc = grp < g.groups ? grp : g.groups - 1;  // past the end: the last group again, never used
+#pragma unroll
+    for (int j = 0; j < WL; ++j)
+      wf[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, woff, gc * (PACKED ? 64 : 128) + j * 16, 0);
+    cs[u] = g.col_scale[(int64_t)gc * g.n + ncol];
+  };
+
+  float sum[MB][4];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[mb][e] = 0.0f;
+
+  request_x(0);
+#pragma unroll
+  for (int u = 0; u < CG; ++u) request_w(u, u);
+  store_x(0);
+  request_x(1);
+  __syncthreads();
+  const int x_off = r * kPitch + c * 32;
+  for (int ch = 0; ch < nchunks; ++ch) {
+    const uint8_t* xb = xbuf + (ch & 1) * MT * kPitch + x_off;
+#pragma unroll
+    for (int u = 0; u < CG; ++u) {
+      const int grp = ch * CG + u;
+      v4i wlo, whi;
+      if constexpr (PACKED) {
+        unpack_i4x32(wf[u][0], wlo, whi, g.a_even_odd8);
+      } else {
+        wlo = wf[u][0]; whi = wf[u][1];
+      }
+      const float csv = cs[u] * cfold;
+      request_w(u, grp + CG);  // the registers of this group are free again
+      v4i acc[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const v4i x0 = *reinterpret_cast<const v4i*>(xb + mb * 16 * kPitch + u * 128);
+        const v4i x1 = *reinterpret_cast<const v4i*>(xb + mb * 16 * kPitch + u * 128 + 16);
+        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, wlo, v4i{0, 0, 0, 0}, 0, 0, 0);
+        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, whi, acc[mb], 0, 0, 0);
+      }
+      if (grp < g.groups) {
+        // every product and the sum round on their own, as in Rescale<EPI>::quarter
+        float f[MB][4];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const float4 rs4 = *reinterpret_cast<const float4*>(&srow_all[grp * MT + mb * 16 + 4 * c]);
+          const float rs[4] = {rs4.x, rs4.y, rs4.z, rs4.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f[mb][e] = round_wide<R::kOutBf16>((float)acc[mb][e]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f[mb][e] = round_wide<R::kP1Bf16>(f[mb][e] * rs[e]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f[mb][e] = round_wide<R::kP2Bf16 || R::kOutBf16>(f[mb][e] * csv);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sum[mb][e] += f[mb][e];
+        }
+      }
+    }
+    // chunk ch + 1 (in registers since the last trip) goes to the other buffer, which every wave left
+    // before the barrier that ended chunk ch - 1; chunk ch + 2 is requested behind it
+    store_x((ch + 1) & 1);
+    request_x(ch + 2);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  }
+  if (wrow >= g.n) return;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int t = mb * 16 + 4 * c + e;
+      if (t < g.m) {
+        const float o = round_to<R::kOutBf16>(sum[mb][e]);
+        if constexpr (R::kOutBf16) reinterpret_cast<uint16_t*>(g.c)[(int64_t)t * g.ldc + wrow] = bf16_bits(o);
+        else reinterpret_cast<float*>(g.c)[(int64_t)t * g.ldc + wrow] = o;
+      }
+    }
+}
+
 }  // namespace
 }  // namespace aqtx
 
@@ -565,6 +720,36 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   else if (p->row_scale_dtype != AQTX_BF16) epi = 1;
   else epi = p->col_scale_dtype == AQTX_BF16 ? 0 : 4;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  // a handful of rows: one wave per 16 rows of b, no tile of C padded to 128 rows
+  const int mb = (int)((p->m + 15) / 16), mbt = mb == 3 ? 4 : mb;
+  const size_t rows_lds = (size_t)2 * 16 * mbt * (rows_chunk_groups(mbt) * 128 + 16) + (size_t)g.groups * 16 * mbt * sizeof(float);
+  if (group128 && p->m <= 64 && p->m * p->lda < (1ll << 31) && p->n * p->ldb < (1ll << 31) && rows_lds <= 65536 &&
+      p->tuning != 128) {
+    // 8 waves (128 rows of b) per workgroup where that still gives every CU one, else 4
+    const int nw = (p->n + 127) / 128 >= 200 ? 8 : 4;
+    const dim3 rgrid((unsigned)((p->n + 16 * nw - 1) / (16 * nw)));
+#define AQTX_ROWS_MB(E, P, W)                                                                    \
+  do {                                                                                          \
+    if (mbt == 1) gemm_grouped_rows_kernel<E, P, 1, W><<<rgrid, W * 64, rows_lds, st>>>(g);     \
+    else if (mbt == 2) gemm_grouped_rows_kernel<E, P, 2, W><<<rgrid, W * 64, rows_lds, st>>>(g); \
+    else gemm_grouped_rows_kernel<E, P, 4, W><<<rgrid, W * 64, rows_lds, st>>>(g);              \
+  } while (0)
+#define AQTX_ROWS(E)                                                                            \
+  do {                                                                                          \
+    if (packed) { if (nw == 8) AQTX_ROWS_MB(E, true, 8); else AQTX_ROWS_MB(E, true, 4); }        \
+    else { if (nw == 8) AQTX_ROWS_MB(E, false, 8); else AQTX_ROWS_MB(E, false, 4); }             \
+  } while (0)
+    switch (epi) {
+      case 0: AQTX_ROWS(0); break;
+      case 1: AQTX_ROWS(1); break;
+      case 2: AQTX_ROWS(2); break;
+      default: AQTX_ROWS(4); break;
+    }
+#undef AQTX_ROWS
+#undef AQTX_ROWS_MB
+    AQTX_HIP_CHECK_LAUNCH("gemm_grouped_rows_kernel");
+    return 0;
+  }
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n));
 #define AQTX_LAUNCH(E)                                                                      \
   do {                                                                                     \

@@ -427,7 +427,7 @@ def pack_i4(q: torch.Tensor) -> torch.Tensor:
 
 def gemm_grouped(a: torch.Tensor, b: torch.Tensor, *, row_scale: torch.Tensor, col_scale: torch.Tensor,
                  group: int, out_dtype, row_scale_dtype=None, col_scale_dtype=None, a_dtype: int = L.I8,
-                 b_dtype: int = L.I8, a_k_order: int = 0, row_scale_by_row: bool = False):
+                 b_dtype: int = L.I8, a_k_order: int = 0, row_scale_by_row: bool = False, tuning: int = 0):
   """C = cast(sum_g dequant_g(A_g @ B_g^T)) for A int8 [m, k], B int8 [n, k] (or packed int4
   uint8 [n, k/2] with b_dtype=I4P), row_scale float32 [k/group, m] ([m, k/group] with
   row_scale_by_row), col_scale float32 [k/group, n].  a_k_order = L.K_EVEN_ODD8: A was written by
@@ -448,6 +448,7 @@ def gemm_grouped(a: torch.Tensor, b: torch.Tensor, *, row_scale: torch.Tensor, c
   plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else out_dt
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else out_dt
   plan.a_k_order, plan.row_scale_by_row = a_k_order, int(row_scale_by_row)
+  plan.tuning = tuning  # kernel override for tests and measurements; results do not depend on it
   c = torch.empty((m, n), dtype=_AQTX_TO_TORCH[out_dt], device=a.device)
   with _timed('gemm_grouped'):
     L.check(L.lib().aqtx_gemm_i8_grouped(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(row_scale),

@@ -193,6 +193,18 @@ def other_configs(dev):
     ms = timeit(lambda: serve(lhs, rhs, MATMUL, None))
   out['int4w_packed_frozen_tiled128_serving_fwd'] = {
       'ms_per_call': round(ms, 3), 'TOPS': round(2 * 2048 * 8192 * 28672 / ms / 1e9, 1)}
+  # the same frozen layer with a handful of tokens (one wave per 16 weight rows instead of 128-row tiles of the
+  # output), replayed from a HIP graph: activation quantisation + contraction; GB/s on the packed weight's bytes
+  from aqt_amd.v2 import hip_graph
+  few = {}
+  with torch.no_grad():
+    for m_few in (1, 8, 64):
+      xf = lhs[:m_few].contiguous()
+      graphed = hip_graph.GraphedCall(lambda a: serve(a, rhs, MATMUL, None), xf)
+      us = timeit(graphed.replay, n=20, w=3) * 1e3
+      few[f'm{m_few}'] = {'us_per_call': round(us, 1), 'weight_GB/s': round(8192 * 28672 / 2 / us / 1e3, 1)}
+      del graphed
+  out['int4w_packed_frozen_tiled128_serving_few_tokens'] = few
   del conv, serve
   del lhs, rhs
   # one decode-sized serving layer call (8 x 4096 against a frozen int8 [4096, 14336] weight): issued from Python

@@ -228,6 +228,9 @@ typedef struct aqtx_grouped_gemm_plan {
   int32_t a_k_order;          /* AQTX_K_*: byte order of a along k; EVEN_ODD8 needs b_dtype AQTX_I4P */
   int32_t row_scale_by_row;   /* 0: row_scale is [k/group][m]; 1: [m][k/group], as aqtx_quantize
                                  with AQTX_REDUCE_COLS and a group writes it                  */
+  int32_t tuning;             /* 0 = the library chooses the kernel.  Tuning only (results never depend on
+                                 it): 128 = the tile kernels also for m <= 64 (group 128 otherwise goes to
+                                 a kernel with one wave per 16 rows of b and no padding of m)  */
 } aqtx_grouped_gemm_plan;
 
 /*

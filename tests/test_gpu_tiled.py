@@ -85,8 +85,11 @@ def _grouped_ref(a, b, rs, cs, group, out, rdt, cdt):
 
 @pytest.mark.parametrize('packed', [False, True])
 @pytest.mark.parametrize('out,rdt,cdt', [('bf16', 'bf16', 'bf16'), ('bf16', 'bf16', 'f32'), ('f32', 'f32', 'f32')])
-@pytest.mark.parametrize('m,n,k,group', [(128, 256, 256, 128), (200, 300, 512, 128), (64, 520, 1024, 256), (5, 9, 128, 128)])
+@pytest.mark.parametrize('m,n,k,group', [(128, 256, 256, 128), (200, 300, 512, 128), (64, 520, 1024, 256), (5, 9, 128, 128),
+                                          (1, 200, 1024, 128), (16, 64, 384, 128), (17, 70, 512, 128), (40, 130, 256, 128),
+                                          (64, 1000, 2048, 128)])
 def test_grouped_gemm_kernel(gpu, m, n, k, group, out, rdt, cdt, packed):
+  """The tile kernels and, for at most 64 rows and groups of 128, the kernel with one wave per 16 rows of b."""
   from aqt_amd import _lib as L
   rng = np.random.default_rng(7)
   a = rng.integers(-127, 128, (m, k)).astype(np.int8)
@@ -104,6 +107,18 @@ def test_grouped_gemm_kernel(gpu, m, n, k, group, out, rdt, cdt, packed):
                          row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt],
                          b_dtype=L.I4P if packed else L.I4)
   np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+  if m <= 64 and group == 128:  # the tile kernel on the same call, and the few-rows kernel with row-major scales
+    kw = dict(col_scale=torch.from_numpy(cs).to(gpu), group=group, out_dtype=U.TORCH_DT[out],
+              row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt], b_dtype=L.I4P if packed else L.I4)
+    tiled = ops.gemm_grouped(torch.from_numpy(a).to(gpu), bt, row_scale=torch.from_numpy(rs).to(gpu), tuning=128, **kw)
+    assert torch.equal(tiled, got)
+    by_row = ops.gemm_grouped(torch.from_numpy(a).to(gpu), bt, row_scale=torch.from_numpy(np.ascontiguousarray(rs.T)).to(gpu),
+                              row_scale_by_row=True, **kw)
+    assert torch.equal(by_row, got)
+    if packed:
+      eo = ops.gemm_grouped(torch.from_numpy(np.ascontiguousarray(_even_odd8(a))).to(gpu), bt,
+                            row_scale=torch.from_numpy(rs).to(gpu), a_k_order=L.K_EVEN_ODD8, **kw)
+      assert torch.equal(eo, got)
 
 
 def _even_odd8(a):
