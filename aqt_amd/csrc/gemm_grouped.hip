@@ -510,7 +510,7 @@ __global__ void pack_i4_kernel(const int8_t* src, uint8_t* dst, int64_t count2) 
 // operand.  The activations are shared by the NW waves of a workgroup: chunks of four groups go through
 // LDS, double buffered (two with 64 tokens; every wave reading all of them from L2 instead cost as much again as the weight
 // stream at 8 tokens and eight times that at 64); rows are 528 bytes apart, so that the 16 lanes of one
-// operand read hit distinct banks.  The row scales of all groups sit in LDS, transposed to [group][token].
+// operand read hit distinct banks; the chunk's row scales travel with it, as [group][token].
 constexpr int rows_chunk_groups(int mb) { return mb == 4 ? 2 : 4; }  // 64 tokens: half the chunk, the same LDS
 
 template <int EPI, bool PACKED, int MB, int NW>
@@ -525,17 +525,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
   static_assert(XL >= 1 && MT * PPC % NT == 0, "chunk loads divide among the threads");
   extern __shared__ __attribute__((aligned(16))) uint8_t rows_lds[];
   uint8_t* xbuf = rows_lds;                                                  // [2][MT][kPitch]
-  float* srow_all = reinterpret_cast<float*>(rows_lds + 2 * MT * kPitch);    // [groups][MT]
+  float* srow = reinterpret_cast<float*>(rows_lds + 2 * MT * kPitch);        // [2][CG][MT]
+  static_assert(CG * MT <= NT, "one row scale per thread and chunk");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
   const int n0 = ((int)blockIdx.x * NW + wave) * 16;
-  for (int i = tid; i < g.groups * MT; i += NT) {
-    const int grp = i / MT, t = i % MT;
-    float v = 1.0f;
-    if (t < g.m) v = g.rs_by_row ? g.row_scale[(int64_t)t * g.groups + grp] : g.row_scale[(int64_t)grp * g.m + t];
-    srow_all[i] = v;
-  }
   const int kb = PACKED ? (int)(g.k / 2) : (int)g.k;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)g.a, 0, (int)((g.m - 1) * g.lda + g.k), kBufferRsrcWord3);
@@ -552,8 +547,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
   const int nchunks = (g.groups + CG - 1) / CG;
 
   // activation chunk: load j of a thread is the 16-byte piece (tid + j NT) % PPC of token (tid + j NT) / PPC
+  // and, for the first CG * MT threads, the row scale of token tid % MT in group tid / MT of the chunk
   v4i xs[XL];
+  float rs_reg = 1.0f;
+  bool rs_ok = false;  // applied when the value goes to LDS: a use next to the load would wait for it there
   auto request_x = [&](int ch) {
+    {
+      const int grp = ch * CG + tid / MT, t = tid % MT;
+      rs_ok = tid < CG * MT && t < g.m && grp < g.groups;
+      const int64_t at = g.rs_by_row ? (int64_t)t * g.groups + grp : (int64_t)grp * g.m + t;
+      rs_reg = g.row_scale[rs_ok ? at : 0];
+    }
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
       const int id = tid + j * NT, t = id / PPC, piece = id % PPC;
@@ -563,6 +567,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
     }
   };
   auto store_x = [&](int buf) {
+    if (tid < CG * MT) srow[buf * CG * MT + tid] = rs_ok ? rs_reg : 1.0f;
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
       const int id = tid + j * NT, t = id / PPC, piece = id % PPC;
@@ -618,7 +623,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
         float f[MB][4];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          const float4 rs4 = *reinterpret_cast<const float4*>(&srow_all[grp * MT + mb * 16 + 4 * c]);
+          const float4 rs4 = *reinterpret_cast<const float4*>(&srow[((ch & 1) * CG + u) * MT + mb * 16 + 4 * c]);
           const float rs[4] = {rs4.x, rs4.y, rs4.z, rs4.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) f[mb][e] = round_wide<R::kOutBf16>((float)acc[mb][e]);
@@ -722,9 +727,9 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   // a handful of rows: one wave per 16 rows of b, no tile of C padded to 128 rows
   const int mb = (int)((p->m + 15) / 16), mbt = mb == 3 ? 4 : mb;
-  const size_t rows_lds = (size_t)2 * 16 * mbt * (rows_chunk_groups(mbt) * 128 + 16) + (size_t)g.groups * 16 * mbt * sizeof(float);
-  if (group128 && p->m <= 64 && p->m * p->lda < (1ll << 31) && p->n * p->ldb < (1ll << 31) && rows_lds <= 65536 &&
-      p->tuning != 128) {
+  const size_t rows_lds = (size_t)2 * 16 * mbt * (rows_chunk_groups(mbt) * 128 + 16) +
+                          (size_t)2 * rows_chunk_groups(mbt) * 16 * mbt * sizeof(float);
+  if (group128 && p->m <= 64 && p->m * p->lda < (1ll << 31) && p->n * p->ldb < (1ll << 31) && p->tuning != 128) {
     // 8 waves (128 rows of b) per workgroup where that still gives every CU one, else 4
     const int nw = (p->n + 127) / 128 >= 200 ? 8 : 4;
     const dim3 rgrid((unsigned)((p->n + 16 * nw - 1) / (16 * nw)));

@@ -87,7 +87,7 @@ def _grouped_ref(a, b, rs, cs, group, out, rdt, cdt):
 @pytest.mark.parametrize('out,rdt,cdt', [('bf16', 'bf16', 'bf16'), ('bf16', 'bf16', 'f32'), ('f32', 'f32', 'f32')])
 @pytest.mark.parametrize('m,n,k,group', [(128, 256, 256, 128), (200, 300, 512, 128), (64, 520, 1024, 256), (5, 9, 128, 128),
                                           (1, 200, 1024, 128), (16, 64, 384, 128), (17, 70, 512, 128), (40, 130, 256, 128),
-                                          (64, 1000, 2048, 128)])
+                                          (64, 1000, 2048, 128), (48, 32, 8192 + 128, 128)])
 def test_grouped_gemm_kernel(gpu, m, n, k, group, out, rdt, cdt, packed):
   """The tile kernels and, for at most 64 rows and groups of 128, the kernel with one wave per 16 rows of b."""
   from aqt_amd import _lib as L
