@@ -506,18 +506,20 @@ __global__ void pack_i4_kernel(const int8_t* src, uint8_t* dst, int64_t count2) 
 // add up in the order of the tile kernels: v_mfma_i32_16x16x64_i8 with the activations as the first
 // operand leaves a lane with tokens 4c .. 4c + 3 (c = lane / 16) of column lane % 16, i.e. four row scales
 // and one column scale per lane and group.  A group of 128 k is one 16-byte load per lane of a packed
-// weight row (two of an int8 one), requested U groups ahead, straight from global memory into the MFMA
+// weight row (two of an int8 one), requested eight groups ahead, straight from global memory into the MFMA
 // operand.  The activations are shared by the NW waves of a workgroup: chunks of four groups go through
 // LDS, double buffered (two with 64 tokens; every wave reading all of them from L2 instead cost as much again as the weight
 // stream at 8 tokens and eight times that at 64); rows are 528 bytes apart, so that the 16 lanes of one
 // operand read hit distinct banks; the chunk's row scales travel with it, as [group][token].
 constexpr int rows_chunk_groups(int mb) { return mb == 4 ? 2 : 4; }  // 64 tokens: half the chunk, the same LDS
 
-template <int EPI, bool PACKED, int MB, int NW>
+// MB: token blocks of a wave; TS: waves that share 16 rows of B, each with MB token blocks of its own (more
+// waves per SIMD for the vector work of many tokens, at the price of TS requests per weight fragment).
+template <int EPI, bool PACKED, int MB, int TS, int NW>
 __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const GroupedArgs g) {
   using R = Rescale<EPI>;
-  constexpr int MT = 16 * MB;      // tokens
-  constexpr int CG = rows_chunk_groups(MB);  // groups per activation chunk
+  constexpr int MT = 16 * MB * TS;      // tokens of the workgroup
+  constexpr int CG = rows_chunk_groups(MB * TS);  // groups per activation chunk
   constexpr int kPitch = CG * 128 + 16;
   constexpr int NT = NW * 64;
   constexpr int PPC = CG * 8;           // 16-byte pieces of one token's chunk
@@ -530,7 +532,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
-  const int n0 = ((int)blockIdx.x * NW + wave) * 16;
+  const int n0 = ((int)blockIdx.x * (NW / TS) + wave / TS) * 16;
+  const int tok0 = (wave % TS) * MB * 16;  // first token of this wave
   const int kb = PACKED ? (int)(g.k / 2) : (int)g.k;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)g.a, 0, (int)((g.m - 1) * g.lda + g.k), kBufferRsrcWord3);
@@ -546,36 +549,40 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
   const float cfold = PACKED ? 0.0625f : 1.0f;  // packed nibbles are unpacked to 16 * value
   const int nchunks = (g.groups + CG - 1) / CG;
 
-  // activation chunk: load j of a thread is the 16-byte piece (tid + j NT) % PPC of token (tid + j NT) / PPC
-  // and, for the first CG * MT threads, the row scale of token tid % MT in group tid / MT of the chunk
-  v4i xs[XL];
-  float rs_reg = 1.0f;
-  bool rs_ok = false;  // applied when the value goes to LDS: a use next to the load would wait for it there
-  auto request_x = [&](int ch) {
+  // activation chunk: load j of a thread is the 16-byte piece (tid + j NT) % PPC of token (tid + j NT) / PPC;
+  // and, for the first CG * MT threads, the row scale of token tid % MT in group tid / MT of the chunk.
+  // Chunk j waits in register set j % 2 from its request, two trips ahead of the trip that reads it (one trip is
+  // shorter than a round trip to L2 under load), until the trip before that one stores it to LDS.
+  v4i xs[2][XL];
+  float rs_reg[2] = {1.0f, 1.0f};
+  bool rs_ok[2] = {false, false};  // applied when the value goes to LDS: a use next to the load would wait for it there
+  auto request_x = [&](const int set, int ch) {
     {
       const int grp = ch * CG + tid / MT, t = tid % MT;
-      rs_ok = tid < CG * MT && t < g.m && grp < g.groups;
+      rs_ok[set] = tid < CG * MT && t < g.m && grp < g.groups;
       const int64_t at = g.rs_by_row ? (int64_t)t * g.groups + grp : (int64_t)grp * g.m + t;
-      rs_reg = g.row_scale[rs_ok ? at : 0];
+      rs_reg[set] = g.row_scale[rs_ok[set] ? at : 0];
     }
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
       const int id = tid + j * NT, t = id / PPC, piece = id % PPC;
       const bool ok = t < g.m && ch * CG * 128 + piece * 16 < (int)g.k && ch < nchunks;
-      xs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? t * (int)g.lda + piece * 16 : kOutside,
-                                                    ok ? ch * CG * 128 : 0, 0);
+      xs[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? t * (int)g.lda + piece * 16 : kOutside,
+                                                         ok ? ch * CG * 128 : 0, 0);
     }
   };
-  auto store_x = [&](int buf) {
-    if (tid < CG * MT) srow[buf * CG * MT + tid] = rs_ok ? rs_reg : 1.0f;
+  auto store_x = [&](const int set, const int buf) {
+    if (tid < CG * MT) srow[buf * CG * MT + tid] = rs_ok[set] ? rs_reg[set] : 1.0f;
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
       const int id = tid + j * NT, t = id / PPC, piece = id % PPC;
-      *reinterpret_cast<v4i*>(xbuf + (buf * MT + t) * kPitch + piece * 16) = xs[j];
+      *reinterpret_cast<v4i*>(xbuf + (buf * MT + t) * kPitch + piece * 16) = xs[set][j];
     }
   };
-  v4i wf[CG][WL];
-  float cs[CG];
+  constexpr int WD = 8;  // groups of weights (and column scales) requested ahead: about 2 us of a wave's work
+  static_assert(WD % CG == 0 && (WD / CG) % 2 == 0, "a round of WD groups is an even number of chunks");
+  v4i wf[WD][WL];
+  float cs[WD];
   auto request_w = [&](const int u, int grp) {
     const int gc = grp < g.groups ? grp : g.groups - 1;  // past the end: the last group again, never used
 #pragma unroll
@@ -590,18 +597,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
 #pragma unroll
     for (int e = 0; e < 4; ++e) sum[mb][e] = 0.0f;
 
-  request_x(0);
+  // Chunk 1 is requested ahead of the first weights on purpose: the compiler sizes the wait in front of the
+  // loop's first store of a chunk for the fewest requests that can lie behind that chunk's on any path into
+  // the loop, and with chunk 1 requested last here that wait also covered the weights just requested (one
+  // full memory latency per round of the loop).
+  request_x(0, 0);
+  request_x(1, 1);
 #pragma unroll
-  for (int u = 0; u < CG; ++u) request_w(u, u);
-  store_x(0);
-  request_x(1);
+  for (int u = 0; u < WD; ++u) request_w(u, u);
+  store_x(0, 0);
+  request_x(0, 2);
   __syncthreads();
-  const int x_off = r * kPitch + c * 32;
-  for (int ch = 0; ch < nchunks; ++ch) {
-    const uint8_t* xb = xbuf + (ch & 1) * MT * kPitch + x_off;
+  const int x_off = (tok0 + r) * kPitch + c * 32;
+  // a round = WD groups = WD / CG chunks (an even number: the LDS buffer of a chunk is a compile-time
+  // constant); a last round that is not full runs on clamped requests and skips the sums
+  for (int ch0 = 0; ch0 < nchunks; ch0 += WD / CG) {
 #pragma unroll
-    for (int u = 0; u < CG; ++u) {
-      const int grp = ch * CG + u;
+  for (int cc = 0; cc < WD / CG; ++cc) {
+    const int ch = ch0 + cc;
+    const uint8_t* xb = xbuf + (cc & 1) * MT * kPitch + x_off;
+#pragma unroll
+    for (int uu = 0; uu < CG; ++uu) {
+      const int u = cc * CG + uu;
+      const int grp = ch * CG + uu;
       v4i wlo, whi;
       if constexpr (PACKED) {
         unpack_i4x32(wf[u][0], wlo, whi, g.a_even_odd8);
@@ -609,12 +627,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
         wlo = wf[u][0]; whi = wf[u][1];
       }
       const float csv = cs[u] * cfold;
-      request_w(u, grp + CG);  // the registers of this group are free again
+      request_w(u, grp + WD);  // the registers of this group are free again
       v4i acc[MB];
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const v4i x0 = *reinterpret_cast<const v4i*>(xb + mb * 16 * kPitch + u * 128);
-        const v4i x1 = *reinterpret_cast<const v4i*>(xb + mb * 16 * kPitch + u * 128 + 16);
+        const v4i x0 = *reinterpret_cast<const v4i*>(xb + mb * 16 * kPitch + uu * 128);
+        const v4i x1 = *reinterpret_cast<const v4i*>(xb + mb * 16 * kPitch + uu * 128 + 16);
         acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, wlo, v4i{0, 0, 0, 0}, 0, 0, 0);
         acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, whi, acc[mb], 0, 0, 0);
       }
@@ -623,7 +641,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
         float f[MB][4];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          const float4 rs4 = *reinterpret_cast<const float4*>(&srow[((ch & 1) * CG + u) * MT + mb * 16 + 4 * c]);
+          const float4 rs4 = *reinterpret_cast<const float4*>(&srow[((cc & 1) * CG + uu) * MT + tok0 + mb * 16 + 4 * c]);
           const float rs[4] = {rs4.x, rs4.y, rs4.z, rs4.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) f[mb][e] = round_wide<R::kOutBf16>((float)acc[mb][e]);
@@ -636,20 +654,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_grouped_rows_kernel(const Groupe
         }
       }
     }
-    // chunk ch + 1 (in registers since the last trip) goes to the other buffer, which every wave left
-    // before the barrier that ended chunk ch - 1; chunk ch + 2 is requested behind it
-    store_x((ch + 1) & 1);
-    request_x(ch + 2);
+    // chunk ch + 1 (in registers since the trip before last) goes to the other buffer, which every wave left
+    // before the barrier that ended chunk ch - 1; chunk ch + 3 is requested into the registers it leaves
+    store_x((cc + 1) & 1, (cc + 1) & 1);
+    request_x((cc + 1) & 1, ch + 3);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+  }
   }
   if (wrow >= g.n) return;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int t = mb * 16 + 4 * c + e;
+      const int t = tok0 + mb * 16 + 4 * c + e;
       if (t < g.m) {
         const float o = round_to<R::kOutBf16>(sum[mb][e]);
         if constexpr (R::kOutBf16) reinterpret_cast<uint16_t*>(g.c)[(int64_t)t * g.ldc + wrow] = bf16_bits(o);
@@ -726,18 +745,21 @@ extern "C" int aqtx_gemm_i8_grouped(const aqtx_grouped_gemm_plan* p, const void*
   else epi = p->col_scale_dtype == AQTX_BF16 ? 0 : 4;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   // a handful of rows: one wave per 16 rows of b, no tile of C padded to 128 rows
-  const int mb = (int)((p->m + 15) / 16), mbt = mb == 3 ? 4 : mb;
+  const int mb = (int)((p->m + 15) / 16), mbt = mb == 3 ? 4 : mb;  // token blocks: 1, 2 or 4
   const size_t rows_lds = (size_t)2 * 16 * mbt * (rows_chunk_groups(mbt) * 128 + 16) +
                           (size_t)2 * rows_chunk_groups(mbt) * 16 * mbt * sizeof(float);
   if (group128 && p->m <= 64 && p->m * p->lda < (1ll << 31) && p->n * p->ldb < (1ll << 31) && p->tuning != 128) {
-    // 8 waves (128 rows of b) per workgroup where that still gives every CU one, else 4
-    const int nw = (p->n + 127) / 128 >= 200 ? 8 : 4;
-    const dim3 rgrid((unsigned)((p->n + 16 * nw - 1) / (16 * nw)));
-#define AQTX_ROWS_MB(E, P, W)                                                                    \
-  do {                                                                                          \
-    if (mbt == 1) gemm_grouped_rows_kernel<E, P, 1, W><<<rgrid, W * 64, rows_lds, st>>>(g);     \
-    else if (mbt == 2) gemm_grouped_rows_kernel<E, P, 2, W><<<rgrid, W * 64, rows_lds, st>>>(g); \
-    else gemm_grouped_rows_kernel<E, P, 4, W><<<rgrid, W * 64, rows_lds, st>>>(g);              \
+    // 8 waves per workgroup where that still gives every CU one, else 4; from 17 tokens on two waves share
+    // their 16 rows of b and take half of the token blocks each
+    const int ts = mbt >= 2 ? 2 : 1;
+    const int nw = (p->n * ts + 127) / 128 >= 200 ? 8 : 4;
+    const int rows_per_wg = 16 * nw / ts;
+    const dim3 rgrid((unsigned)((p->n + rows_per_wg - 1) / rows_per_wg));
+#define AQTX_ROWS_MB(E, P, W)                                                                        \
+  do {                                                                                              \
+    if (mbt == 1) gemm_grouped_rows_kernel<E, P, 1, 1, W><<<rgrid, W * 64, rows_lds, st>>>(g);      \
+    else if (mbt == 2) gemm_grouped_rows_kernel<E, P, 1, 2, W><<<rgrid, W * 64, rows_lds, st>>>(g); \
+    else gemm_grouped_rows_kernel<E, P, 2, 2, W><<<rgrid, W * 64, rows_lds, st>>>(g);               \
   } while (0)
 #define AQTX_ROWS(E)                                                                            \
   do {                                                                                          \
