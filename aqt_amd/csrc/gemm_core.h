@@ -739,5 +739,7 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8);
 int gemm_mid_k_slices(const aqtx_gemm_plan* p);
 int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                        const float* col_scale, void* c, int32_t* acc_out, int slices, hipStream_t st);
+int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                        const float* col_scale, void* c, float* acc_out, hipStream_t st);
 
 }  // namespace aqtx

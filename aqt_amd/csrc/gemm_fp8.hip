@@ -51,6 +51,8 @@ extern "C" int aqtx_gemm_fp8(const aqtx_gemm_plan* p, const void* a, const void*
     AQTX_HIP_CHECK_LAUNCH("gemm_simple_kernel");
     return 0;
   }
+  // few output tiles (or tiles that would lie mostly outside C): the 128 x 128 kernel
+  if (p->k_split <= 1 && gemm_mid_k_slices(p) > 0) return launch_gemm_fp8_mid(p, a, b, row_scale, col_scale, c, acc_out, st);
   AQTX_REQUIRE(p->lda * (int64_t)BM < (1ll << 31) && p->ldb * (int64_t)BN < (1ll << 31),
                "aqtx_gemm_fp8: leading dimension too large for 32-bit tile offsets");
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);

@@ -20,12 +20,17 @@ constexpr int TM = 128, TN = 128;
 constexpr int kRow = BK + 16;
 constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile;  // 36 KiB
 
-// EPI, COL_FIRST as in gemm_kernel.  PACKED: B holds int4 values two per byte (see gemm_kernel's BPACK).
-// SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then).
-template <int EPI, bool COL_FIRST, bool PACKED, bool SLAB>
+// MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: B holds int4 values two per byte (see gemm_kernel's BPACK).
+// SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then; integer sums only).
+template <class MMA, int EPI, bool COL_FIRST, bool PACKED, bool SLAB>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void gemm_mid_kernel(const GemmArgs g_in) {
   static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
+  static_assert(MMA::kIntAcc || (!SLAB && !PACKED && EPI != 3), "fp8 operands: float sums, whole K, bytes as they are");
+  using Acc = typename MMA::Acc;
+  using AccScalar = typename MMA::AccScalar;
+  using Frag = typename MMA::Frag;
+  constexpr int kChunks = MMA::kChunks;  // 16-byte chunks a lane holds of one MFMA's k
   GemmArgs g = g_in;
   __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[2 * kStage];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -92,11 +97,19 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     }
   };
 
-  // fragment of k step ks: 16 bytes at 32 ks + 16 lh of row lr of the 32-row block
-  const int a_off = (wm * 32 + lr) * kRow + lh * 16;
-  const int b_off = kATile + (wn * 64 + lr) * kRow + lh * 16;
+  // fragment of k step ks: 16 kChunks bytes at (32 ks + 16 lh) kChunks of row lr of the 32-row block
+  const int a_off = (wm * 32 + lr) * kRow + lh * 16 * kChunks;
+  const int b_off = kATile + (wn * 64 + lr) * kRow + lh * 16 * kChunks;
+  auto frag = [&](const uint8_t* at) -> Frag {
+    if constexpr (kChunks == 1) {
+      return *reinterpret_cast<const v4i*>(at);
+    } else {
+      const v4i x0 = *reinterpret_cast<const v4i*>(at), x1 = *reinterpret_cast<const v4i*>(at + 16);
+      return Frag{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+  };
 
-  v16i acc[2];
+  Acc acc[2];
 #pragma unroll
   for (int r = 0; r < 16; ++r) { acc[0][r] = 0; acc[1][r] = 0; }
 
@@ -116,12 +129,12 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     constexpr int BUF = decltype(buf_c)::value;
     const uint8_t* st = stage_mem + BUF * kStage;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const v4i fa = *reinterpret_cast<const v4i*>(st + a_off + ks * 32);
-      const v4i fb0 = *reinterpret_cast<const v4i*>(st + b_off + ks * 32);
-      const v4i fb1 = *reinterpret_cast<const v4i*>(st + b_off + 32 * kRow + ks * 32);
-      acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb0, fa, acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb1, fa, acc[1], 0, 0, 0);
+    for (int ks = 0; ks < 4 / kChunks; ++ks) {
+      const Frag fa = frag(st + a_off + ks * 32 * kChunks);
+      const Frag fb0 = frag(st + b_off + ks * 32 * kChunks);
+      const Frag fb1 = frag(st + b_off + 32 * kRow + ks * 32 * kChunks);
+      acc[0] = MMA::mma(fb0, fa, acc[0]);
+      acc[1] = MMA::mma(fb1, fa, acc[1]);
     }
     store_stage((1 - BUF) * kStage);
     const int k_next = s + 2 < nstages ? (s + 2) * BK : 0;
@@ -172,13 +185,20 @@ void gemm_mid_kernel(const GemmArgs g_in) {
         const int64_t nn = n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh;
         if (nn >= g.n) continue;
         const bool full = nn + 4 <= g.n;
-        int v[4];
+        AccScalar v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[ni][4 * q + e] >> 4 : acc[ni][4 * q + e];
-        if (g.acc_out != nullptr) {
-          int32_t* dst = reinterpret_cast<int32_t*>(g.acc_out) + row_o + nn;
-          if (full && acc_vec) *reinterpret_cast<int4*>(dst) = make_int4(v[0], v[1], v[2], v[3]);
-          else for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[e] = v[e];
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (PACKED) v[e] = acc[ni][4 * q + e] >> 4;
+          else v[e] = acc[ni][4 * q + e];
+        }
+        if (g.acc_out != nullptr) {  // 32-bit patterns, int32 or float
+          AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out) + row_o + nn;
+          if (full && acc_vec) {
+            *reinterpret_cast<int4*>(dst) = make_int4(__builtin_bit_cast(int, v[0]), __builtin_bit_cast(int, v[1]),
+                                                      __builtin_bit_cast(int, v[2]), __builtin_bit_cast(int, v[3]));
+          } else {
+            for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[e] = v[e];
+          }
         }
         uint8_t* dst = reinterpret_cast<uint8_t*>(g.c) + (row_o + nn) * kEsz;
         if constexpr (EPI == 3) {
@@ -220,9 +240,22 @@ void gemm_mid_kernel(const GemmArgs g_in) {
 template <int EPI, bool COL_FIRST>
 void launch_mid(const GemmArgs& g, bool packed, dim3 grid, hipStream_t st) {
   if constexpr (!COL_FIRST) {
-    if (packed) { gemm_mid_kernel<EPI, false, true, false><<<grid, 512, 0, st>>>(g); return; }
+    if (packed) { gemm_mid_kernel<MmaI8, EPI, false, true, false><<<grid, 512, 0, st>>>(g); return; }
   }
-  gemm_mid_kernel<EPI, COL_FIRST, false, false><<<grid, 512, 0, st>>>(g);
+  gemm_mid_kernel<MmaI8, EPI, COL_FIRST, false, false><<<grid, 512, 0, st>>>(g);
+}
+
+template <class MMA>
+void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
+#define AQTX_MID8(E) do { if (g.col_first) gemm_mid_kernel<MMA, E, true, false, false><<<grid, 512, 0, st>>>(g); \
+                          else gemm_mid_kernel<MMA, E, false, false, false><<<grid, 512, 0, st>>>(g); } while (0)
+  switch (epi) {
+    case 0: AQTX_MID8(0); break;
+    case 1: AQTX_MID8(1); break;
+    case 4: AQTX_MID8(4); break;
+    default: AQTX_MID8(2); break;
+  }
+#undef AQTX_MID8
 }
 
 template <int EPI>
@@ -280,8 +313,8 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     g.k_split = (int)((p->k + g.k_chunk - 1) / g.k_chunk);
     g.slabs = reinterpret_cast<int32_t*>(p->k_split_workspace);
     grid.z = (unsigned)g.k_split;
-    if (packed) gemm_mid_kernel<3, false, true, true><<<grid, 512, 0, st>>>(g);
-    else gemm_mid_kernel<3, false, false, true><<<grid, 512, 0, st>>>(g);
+    if (packed) gemm_mid_kernel<MmaI8, 3, false, true, true><<<grid, 512, 0, st>>>(g);
+    else gemm_mid_kernel<MmaI8, 3, false, false, true><<<grid, 512, 0, st>>>(g);
     const dim3 egrid((unsigned)((p->n + 1023) / 1024), (unsigned)p->m, (unsigned)p->batch);
     switch (epi) {
       case 0: launch_slab_sum<0>(g, egrid, st); break;
@@ -301,6 +334,26 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     default: launch_mid<3, false>(g, packed, grid, st); break;
   }
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel");
+  return 0;
+}
+
+// fp8 operands on the 128 x 128 tiles (float sums: K is never cut).
+int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                        const float* col_scale, void* c, float* acc_out, hipStream_t st) {
+  GemmArgs g = make_gemm_args(p, a, b, row_scale, col_scale, c, acc_out);
+  g.tiles_m = (int)((p->m + TM - 1) / TM);
+  g.tiles_n = (int)((p->n + TN - 1) / TN);
+  const int epi = gemm_epilogue_id(p);
+  if (epi < 0 || epi == 3)
+    return set_error("aqtx_gemm_fp8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
+                     p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
+  const bool a5 = p->a_dtype == AQTX_E5M2, b5 = p->b_dtype == AQTX_E5M2;
+  if (!a5 && !b5) launch_mid_fp8<MmaF8<0, 0>>(g, epi, grid, st);
+  else if (!a5 && b5) launch_mid_fp8<MmaF8<0, 1>>(g, epi, grid, st);
+  else if (a5 && !b5) launch_mid_fp8<MmaF8<1, 0>>(g, epi, grid, st);
+  else launch_mid_fp8<MmaF8<1, 1>>(g, epi, grid, st);
+  AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<fp8>");
   return 0;
 }
 

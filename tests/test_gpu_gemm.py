@@ -264,7 +264,7 @@ FP8_SHAPES = [(1, 256, 256, 256), (1, 300, 520, 144), (2, 130, 70, 48), (1, 17, 
 
 @pytest.mark.parametrize('ka,kb', [('e4m3', 'e4m3'), ('e4m3', 'e5m2'), ('e5m2', 'e4m3'), ('e5m2', 'e5m2')])
 @pytest.mark.parametrize('batch,m,n,k', FP8_SHAPES)
-def test_fp8_exact_when_sums_are_representable(gpu, batch, m, n, k, ka, kb):
+def test_fp8_exact_when_sums_are_representable(gpu, tiles, batch, m, n, k, ka, kb):
   """Small-integer operands: every partial sum is exact in float32, so any summation order
   must give the exact result; a wrong format decode or a dropped k block cannot."""
   a, av = _fp8_small_ints((batch, m, k), 11, ka)
@@ -277,7 +277,7 @@ def test_fp8_exact_when_sums_are_representable(gpu, batch, m, n, k, ka, kb):
 
 @pytest.mark.parametrize('ka,kb', [('e4m3', 'e4m3'), ('e4m3', 'e5m2'), ('e5m2', 'e5m2')])
 @pytest.mark.parametrize('batch,m,n,k', FP8_SHAPES)
-def test_fp8_random_values_within_mfma_accumulation_error(gpu, batch, m, n, k, ka, kb):
+def test_fp8_random_values_within_mfma_accumulation_error(gpu, tiles, batch, m, n, k, ka, kb):
   """Tolerance: |got - exact| <= 2**-10 * sum_k |a_k b_k|.  The fp8 MFMA adds the 64 products
   of one instruction in a reduced-precision tree: measured on gfx950, a product more than 2**14
   below the largest product of its 64-long block is dropped, and the block sum is then added
@@ -299,7 +299,7 @@ def test_fp8_random_values_within_mfma_accumulation_error(gpu, batch, m, n, k, k
 @pytest.mark.parametrize('out,sdt', [('bf16', 'bf16'), ('bf16', 'f32'), ('f32', 'f32')])
 @pytest.mark.parametrize('order', [L.SCALE_ROW_THEN_COL, L.SCALE_COL_THEN_ROW])
 @pytest.mark.parametrize('batch,m,n,k', [(1, 256, 512, 1024), (2, 100, 72, 160), (1, 33, 20, 23)])
-def test_fp8_dequant_epilogue(gpu, batch, m, n, k, order, sdt, out):
+def test_fp8_dequant_epilogue(gpu, tiles, batch, m, n, k, order, sdt, out):
   """The epilogue is checked bit-exactly on the accumulators the kernel itself reports."""
   a, _ = _fp8_random_bytes((batch, m, k), 15, 'e4m3')
   b, _ = _fp8_random_bytes((batch, n, k), 16, 'e5m2')
@@ -314,3 +314,15 @@ def test_fp8_dequant_epilogue(gpu, batch, m, n, k, order, sdt, out):
     s1, s2 = s2, s1
   want = R.dequant(R.QTensor(acc.cpu().numpy(), 'f32', [s1, s2], sdt, out))
   np.testing.assert_array_equal(c.float().cpu().numpy(), want)
+
+
+def test_fp8_tile_sizes_give_the_same_bits(gpu, monkeypatch):
+  """Both tile sizes walk k in the same order with the same instruction: the float sums agree bit for bit."""
+  a, _ = _fp8_random_bytes((1, 300, 2048), 17, 'e4m3')
+  b, _ = _fp8_random_bytes((1, 520, 2048), 18, 'e5m2')
+  outs = []
+  for tuning in (8, 128):
+    monkeypatch.setattr(ops, 'GEMM_TUNING', tuning)
+    outs.append(ops.gemm(a.to(gpu), b.to(gpu), row_scale=None, col_scale=None, out_dtype=torch.float32,
+                         a_dtype=L.E4M3, b_dtype=L.E5M2))
+  assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32))
