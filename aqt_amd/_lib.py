@@ -102,6 +102,7 @@ FP_NEAREST, FP_NOISE_JAX_BITS, FP_NOISE_INDEX = 0, 1, 2
 
 SYMBOLS = {
     'aqtx_im2col_i8': (ctypes.c_int, [ctypes.POINTER(Im2colPlan), _vp, _vp, _vp]),
+    'aqtx_conv_i8': (ctypes.c_int, [ctypes.POINTER(Im2colPlan), ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_fp_round': (ctypes.c_int, [ctypes.POINTER(FpRoundPlan), _vp, _vp, ctypes.POINTER(ctypes.c_uint32), _vp]),
     'aqtx_quantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp, _vp,
                                      ctypes.c_size_t, _vp]),

@@ -86,6 +86,14 @@ struct GemmArgs {
   int k_split;      // slices (<= 1: none)
   int64_t k_chunk;  // k per slice, a multiple of 128
   int32_t* slabs;
+  // Convolution (gemm_mid_kernel<..., CONV>): A is not a matrix but the int8 input [images][spatial...][c]; row
+  // r of the contraction is output position r, k runs over the kernel window in tap order with the features
+  // innermost, and what lies in the padding reads as zero.  Up to three spatial axes, missing leading ones 1.
+  struct {
+    int32_t c;
+    int32_t in[3], ker[3], str[3], dil[3], pad[3], osz[3];
+    int64_t x_bytes;
+  } conv;
 };
 
 constexpr int BM = 256, BN = 256, BK = 128;
@@ -739,6 +747,8 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8);
 int gemm_mid_k_slices(const aqtx_gemm_plan* p);
 int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                        const float* col_scale, void* c, int32_t* acc_out, int slices, hipStream_t st);
+int launch_conv_i8_mid(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, const void* x, const void* b,
+                       const float* row_scale, const float* col_scale, void* c, hipStream_t st);
 int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                         const float* col_scale, void* c, float* acc_out, hipStream_t st);
 

@@ -123,3 +123,35 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   AQTX_HIP_CHECK_LAUNCH("gemm_kernel<int8>");
   return 0;
 }
+
+extern "C" int aqtx_conv_i8(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, const void* x, const void* b,
+                            const float* row_scale, const float* col_scale, void* c, void* stream) {
+  clear_error();
+  AQTX_REQUIRE(w != nullptr, "aqtx_conv_i8: window plan is NULL");
+  if (int rc = validate_gemm_plan(p, "aqtx_conv_i8", false)) return rc;
+  AQTX_REQUIRE(w->rank >= 1 && w->rank <= 3, "aqtx_conv_i8: spatial rank %d outside 1..3", w->rank);
+  AQTX_REQUIRE(w->n >= 0 && w->c >= 0, "aqtx_conv_i8: negative shape");
+  int64_t positions = 1, taps = 1, in_elems = 1;
+  for (int d = 0; d < w->rank; ++d) {
+    AQTX_REQUIRE(w->in_size[d] >= 0 && w->kernel[d] >= 1 && w->stride[d] >= 1 && w->dilation[d] >= 1 &&
+                     w->pad_lo[d] >= 0 && w->out_size[d] >= 0,
+                 "aqtx_conv_i8: bad extent on spatial axis %d", d);
+    positions *= w->out_size[d];
+    taps *= w->kernel[d];
+    in_elems *= w->in_size[d];
+  }
+  AQTX_REQUIRE(p->batch == 1 && p->m == w->n * positions && p->k == taps * w->c && p->group_offsets == nullptr,
+               "aqtx_conv_i8: the contraction plan must be batch 1, m = images * positions, k = taps * features");
+  AQTX_REQUIRE(p->a_dtype != AQTX_I4P && p->b_dtype != AQTX_I4P && p->out_dtype != AQTX_I32 && p->k_split <= 1,
+               "aqtx_conv_i8: int8 containers, a float output and no k slices");
+  if (p->m == 0 || p->n == 0) return 0;
+  AQTX_REQUIRE(x != nullptr && b != nullptr && c != nullptr, "aqtx_conv_i8: NULL buffer");
+  AQTX_REQUIRE(w->c > 0 && w->c % 128 == 0, "aqtx_conv_i8: features (%d) must be a positive multiple of 128 "
+               "(other inputs go through aqtx_im2col_i8 + aqtx_gemm_i8)", w->c);
+  AQTX_REQUIRE(w->n * in_elems * w->c < (1ll << 31), "aqtx_conv_i8: input of 2 GiB or more");
+  AQTX_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)b % 16) == 0 && p->ldb % 16 == 0 && p->ldb * (int64_t)128 < (1ll << 31),
+               "aqtx_conv_i8: operands must be 16-byte aligned, ldb a multiple of 16");
+  const size_t esz = p->out_dtype == AQTX_BF16 ? 2 : 4;
+  AQTX_REQUIRE(((uintptr_t)c % esz) == 0, "aqtx_conv_i8: output is not element aligned");
+  return launch_conv_i8_mid(w, p, x, b, row_scale, col_scale, c, reinterpret_cast<hipStream_t>(stream));
+}

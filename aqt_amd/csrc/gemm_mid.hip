@@ -22,10 +22,13 @@ constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile; 
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: B holds int4 values two per byte (see gemm_kernel's BPACK).
 // SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then; integer sums only).
-template <class MMA, int EPI, bool COL_FIRST, bool PACKED, bool SLAB>
+// CONV: A is a convolution input read in place (GemmArgs::conv): the window gather that would otherwise be
+// materialised (features % 128 == 0, so a 128-byte stage lies inside one tap).
+template <class MMA, int EPI, bool COL_FIRST, bool PACKED, bool SLAB, bool CONV = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void gemm_mid_kernel(const GemmArgs g_in) {
   static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
+  static_assert(!CONV || (MMA::kIntAcc && !PACKED && !SLAB), "the convolution reads int8 bytes, whole K");
   static_assert(MMA::kIntAcc || (!SLAB && !PACKED && EPI != 3), "fp8 operands: float sums, whole K, bytes as they are");
   using Acc = typename MMA::Acc;
   using AccScalar = typename MMA::AccScalar;
@@ -50,8 +53,10 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   const int64_t rows_a = (g.m - m0) < TM ? (g.m - m0) : TM;
   const int64_t rows_b = (g.n - n0) < TN ? (g.n - n0) : TN;
   const int kb_bytes = PACKED ? (int)(g.k / 2) : (int)g.k;  // bytes of one B row (of this slice)
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+  const __amdgpu_buffer_rsrc_t rsrc_a = CONV
+      ? __builtin_amdgcn_make_buffer_rsrc((void*)g.a, 0, (int)g.conv.x_bytes, kBufferRsrcWord3)
+      : __builtin_amdgcn_make_buffer_rsrc((void*)(g.a + bz * g.stride_a + m0 * g.lda), 0,
+                                          (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + kb_bytes), kBufferRsrcWord3);
 
@@ -70,7 +75,43 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   const int st_a = (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
   const int st_b = kATile + (PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
                                     : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
+  // CONV: position of this lane's two rows (first corner of their windows, in input coordinates) and the tap
+  // the next request belongs to, advanced one stage per request (requests come in stage order)
+  int cpix[NLA] = {0, 0}, ci0[NLA] = {0, 0}, ci1[NLA] = {0, 0}, ci2[NLA] = {0, 0};
+  int ct0 = 0, ct1 = 0, ct2 = 0, cch = 0;  // wave-uniform
+  if constexpr (CONV) {
+#pragma unroll
+    for (int j = 0; j < NLA; ++j) {
+      int64_t row = m0 + wave * 16 + (lane >> 3) + j * 8;
+      const bool in = row < g.m;
+      if (!in) row = 0;
+      const int o2 = (int)(row % g.conv.osz[2]); row /= g.conv.osz[2];
+      const int o1 = (int)(row % g.conv.osz[1]); row /= g.conv.osz[1];
+      const int o0 = (int)(row % g.conv.osz[0]); row /= g.conv.osz[0];
+      ci0[j] = in ? o0 * g.conv.str[0] - g.conv.pad[0] : -(1 << 28);  // rows past m: outside for every tap
+      ci1[j] = o1 * g.conv.str[1] - g.conv.pad[1];
+      ci2[j] = o2 * g.conv.str[2] - g.conv.pad[2];
+      cpix[j] = in ? (int)((((row * g.conv.in[0] + ci0[j]) * g.conv.in[1] + ci1[j]) * g.conv.in[2] + ci2[j]) * g.conv.c) : 0;
+    }
+  }
+  auto conv_advance = [&]() {
+    cch += BK;
+    if (cch >= g.conv.c) {
+      cch = 0;
+      if (++ct2 == g.conv.ker[2]) { ct2 = 0; if (++ct1 == g.conv.ker[1]) { ct1 = 0; ++ct0; } }
+    }
+  };
   auto load_one = [&](const int j, int k0) {
+    if constexpr (CONV) {
+      if (j < NLA) {
+        const int d0 = ct0 * g.conv.dil[0], d1 = ct1 * g.conv.dil[1], d2 = ct2 * g.conv.dil[2];
+        const bool in = (unsigned)(ci0[j] + d0) < (unsigned)g.conv.in[0] && (unsigned)(ci1[j] + d1) < (unsigned)g.conv.in[1] &&
+                        (unsigned)(ci2[j] + d2) < (unsigned)g.conv.in[2] && ct0 < g.conv.ker[0];
+        const int tap = ((d0 * g.conv.in[1] + d1) * g.conv.in[2] + d2) * g.conv.c + cch;
+        stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, in ? cpix[j] + tap + kpos_a : kOutside, 0, 0);
+        return;
+      }
+    }
     if (j < NLA) {
       const int vo = k0 + kpos_a < (int)g.k ? ld_a + j * 8 * (int)g.lda : kOutside;
       stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, k0, 0);
@@ -116,9 +157,11 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   const int nstages = (int)((g.k + BK - 1) / BK);
 #pragma unroll
   for (int j = 0; j < NL; ++j) load_one(j, 0);
+  if constexpr (CONV) conv_advance();
   store_stage(0);
 #pragma unroll
   for (int j = 0; j < NL; ++j) load_one(j, nstages > 1 ? BK : 0);
+  if constexpr (CONV) conv_advance();
   __syncthreads();
 
   // Stage s reads buffer BUF; the staging registers (stage s + 1, requested during stage s - 1) go to the
@@ -140,6 +183,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     const int k_next = s + 2 < nstages ? (s + 2) * BK : 0;
 #pragma unroll
     for (int j = 0; j < NL; ++j) load_one(j, k_next);
+    if constexpr (CONV) conv_advance();  // past the last stage the tap leaves the window: zeros nobody reads
     // a bare s_barrier: a __syncthreads() would also wait for the global loads just issued
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -334,6 +378,44 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     default: launch_mid<3, false>(g, packed, grid, st); break;
   }
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel");
+  return 0;
+}
+
+// Convolution of int8 operands without the window matrix: `w` describes the windows, `p` the contraction
+// they amount to (m = images * positions, n = output features, k = taps * features).
+int launch_conv_i8_mid(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, const void* x, const void* b,
+                       const float* row_scale, const float* col_scale, void* c, hipStream_t st) {
+  GemmArgs g = make_gemm_args(p, x, b, row_scale, col_scale, c, nullptr);
+  g.tiles_m = (int)((p->m + TM - 1) / TM);
+  g.tiles_n = (int)((p->n + TN - 1) / TN);
+  g.conv.c = w->c;
+  int64_t in_elems = 1;
+  for (int d = 0; d < 3; ++d) {
+    const int s = d - (3 - w->rank);  // missing leading axes have extent 1
+    g.conv.in[d] = s < 0 ? 1 : w->in_size[s];
+    g.conv.ker[d] = s < 0 ? 1 : w->kernel[s];
+    g.conv.str[d] = s < 0 ? 1 : w->stride[s];
+    g.conv.dil[d] = s < 0 ? 1 : w->dilation[s];
+    g.conv.pad[d] = s < 0 ? 0 : w->pad_lo[s];
+    g.conv.osz[d] = s < 0 ? 1 : w->out_size[s];
+    in_elems *= g.conv.in[d];
+  }
+  g.conv.x_bytes = w->n * in_elems * w->c;
+  const int epi = gemm_epilogue_id(p);
+  if (epi < 0 || epi == 3)
+    return set_error("aqtx_conv_i8: unsupported out/dequant/scale dtype combination (%d, %d, %d)", p->out_dtype,
+                     p->dequant_dtype, p->row_scale_dtype);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1);
+#define AQTX_CONV(E) do { if (g.col_first) gemm_mid_kernel<MmaI8, E, true, false, false, true><<<grid, 512, 0, st>>>(g); \
+                          else gemm_mid_kernel<MmaI8, E, false, false, false, true><<<grid, 512, 0, st>>>(g); } while (0)
+  switch (epi) {
+    case 0: AQTX_CONV(0); break;
+    case 1: AQTX_CONV(1); break;
+    case 4: AQTX_CONV(4); break;
+    default: AQTX_CONV(2); break;
+  }
+#undef AQTX_CONV
+  AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<conv>");
   return 0;
 }
 

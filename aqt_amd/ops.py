@@ -467,11 +467,8 @@ def sum_tiles(x: torch.Tensor) -> torch.Tensor:
   return out
 
 
-def im2col_i8(x: torch.Tensor, kernel, strides, pads, dilation):
-  """Windows of an int8 tensor [n, *spatial, c] as a matrix [n * positions, taps * c] (zeros in the
-  padding); returns (matrix, output spatial sizes).  `pads` are (low, high) pairs."""
-  _require_gpu(x)
-  assert x.dtype == torch.int8 and x.is_contiguous() and 3 <= x.dim() <= 5
+def _window_plan(x: torch.Tensor, kernel, strides, pads, dilation):
+  """aqtx_im2col_plan of the windows of x [n, *spatial, c]; returns (plan, output spatial sizes)."""
   rank = x.dim() - 2
   plan = L.Im2colPlan()
   plan.n, plan.c, plan.rank = x.shape[0], x.shape[-1], rank
@@ -483,11 +480,60 @@ def im2col_i8(x: torch.Tensor, kernel, strides, pads, dilation):
     out_sizes.append(o)
     plan.in_size[d], plan.kernel[d], plan.stride[d] = x.shape[1 + d], int(kernel[d]), int(strides[d])
     plan.dilation[d], plan.pad_lo[d], plan.out_size[d] = int(dilation[d]), int(pads[d][0]), o
+  return plan, out_sizes
+
+
+def im2col_i8(x: torch.Tensor, kernel, strides, pads, dilation):
+  """Windows of an int8 tensor [n, *spatial, c] as a matrix [n * positions, taps * c] (zeros in the
+  padding); returns (matrix, output spatial sizes).  `pads` are (low, high) pairs."""
+  _require_gpu(x)
+  assert x.dtype == torch.int8 and x.is_contiguous() and 3 <= x.dim() <= 5
+  rank = x.dim() - 2
+  plan, out_sizes = _window_plan(x, kernel, strides, pads, dilation)
   rows = x.shape[0] * math.prod(out_sizes)
   k = math.prod(int(t) for t in kernel[:rank]) * x.shape[-1]
   out = torch.empty((rows, k), dtype=torch.int8, device=x.device)
   L.check(L.lib().aqtx_im2col_i8(ctypes.byref(plan), _ptr(x), _ptr(out), _stream()))
   return out, out_sizes
+
+
+def conv_i8_supported(x: torch.Tensor) -> bool:
+  """Whether conv_i8 takes this input: features a multiple of 128, less than 2 GiB."""
+  return x.shape[-1] > 0 and x.shape[-1] % 128 == 0 and x.numel() < 2 ** 31
+
+
+def conv_i8(x: torch.Tensor, w: torch.Tensor, kernel, strides, pads, dilation, *, row_scale, col_scale, out_dtype,
+            row_scale_dtype=None, col_scale_dtype=None, scale_order: int = L.SCALE_ROW_THEN_COL):
+  """dequant(windows(x) @ w^T) in one launch, the windows read in place: x int8 [n, *spatial, c], w int8
+  [features_out, taps * c] (tap order row-major, features innermost), row_scale float32 [n * positions],
+  col_scale float32 [features_out].  Same bits as im2col_i8 + gemm.  Returns ([n * positions, features_out],
+  output spatial sizes)."""
+  _require_gpu(x, w, row_scale, col_scale)
+  assert x.dtype == torch.int8 and w.dtype == torch.int8 and x.is_contiguous() and 3 <= x.dim() <= 5
+  assert w.dim() == 2 and w.stride(1) == 1 and conv_i8_supported(x)
+  rank = x.dim() - 2
+  win, out_sizes = _window_plan(x, kernel, strides, pads, dilation)
+  m = x.shape[0] * math.prod(out_sizes)
+  k = math.prod(int(t) for t in kernel[:rank]) * x.shape[-1]
+  n = w.shape[0]
+  assert w.shape[1] == k
+  out_dt = aqtx_dtype(out_dtype)
+  plan = L.GemmPlan()
+  plan.batch, plan.m, plan.n, plan.k = 1, m, n, k
+  plan.lda, plan.ldb, plan.ldc = k, w.stride(0), n
+  plan.a_dtype = plan.b_dtype = L.I8
+  plan.out_dtype = plan.dequant_dtype = out_dt
+  plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else out_dt
+  plan.col_scale_dtype = aqtx_dtype(col_scale_dtype) if col_scale_dtype is not None else out_dt
+  plan.scale_order = scale_order
+  plan.k_split = 1
+  for s_, shape in ((row_scale, (m,)), (col_scale, (n,))):
+    if s_ is not None:
+      assert s_.dtype == torch.float32 and s_.is_contiguous() and tuple(s_.shape) == shape, (tuple(s_.shape), shape)
+  c = torch.empty((m, n), dtype=_AQTX_TO_TORCH[out_dt], device=x.device)
+  L.check(L.lib().aqtx_conv_i8(ctypes.byref(win), ctypes.byref(plan), _ptr(x), _ptr(w), _ptr(row_scale),
+                               _ptr(col_scale), _ptr(c), _stream()))
+  return c, out_sizes
 
 
 def fp_round(x: torch.Tensor, *, nexp: int, nmant: int, has_subnormals: bool, key=None,

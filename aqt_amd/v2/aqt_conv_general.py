@@ -34,6 +34,12 @@ def flax_conv_dimension_numbers(input_shape) -> ConvDimensionNumbers:
   return ConvDimensionNumbers(lhs_spec, rhs_spec, lhs_spec)
 
 
+def _conv_weight_matrix(rq, k, cout):
+  """The quantized kernel [*window, features_in, features_out] as the contraction's column operand
+  [features_out, window * features_in] (k contiguous)."""
+  return rq.reshape(k, cout).t().contiguous()
+
+
 def _explicit_padding(padding, in_sizes, eff_kernel, strides):
   if isinstance(padding, str):
     if padding.upper() == 'VALID':
@@ -139,12 +145,25 @@ def _fused_int8_conv(lhs_qt, rhs_qt, out_dtype, window_strides, padding, lhs_dil
   pads = _explicit_padding(padding, list(lq.shape[1:1 + ns]), eff, strides)
   if ns > 3:
     return None
-  a, out_sizes = ops.im2col_i8(lq.contiguous(), kernel, strides, pads, dilation)
+  lq = lq.contiguous()
+  if ops.conv_i8_supported(lq) and lq.shape[0] * cout > 0:
+    # features in multiples of 128: one kernel reads the windows in place, no window matrix
+    k = math.prod(kernel) * lq.shape[-1]
+    _, out_sizes = ops._window_plan(lq, kernel, strides, pads, dilation)  # pylint: disable=protected-access
+    positions = math.prod(out_sizes)
+    if positions > 0:
+      b = _conv_weight_matrix(rq, k, cout)
+      row_scale = ls.reshape(n, 1).float().expand(n, positions).reshape(n * positions).contiguous()
+      out, out_sizes = ops.conv_i8(lq, b, kernel, strides, pads, dilation, row_scale=row_scale,
+                                   col_scale=rs.reshape(cout).float().contiguous(), out_dtype=out_dtype,
+                                   row_scale_dtype=ls.dtype, col_scale_dtype=rs.dtype)
+      return out.reshape([n] + list(out_sizes) + [cout])
+  a, out_sizes = ops.im2col_i8(lq, kernel, strides, pads, dilation)
   k = a.shape[1]
   positions = math.prod(out_sizes)
   if a.shape[0] * cout == 0 or k == 0:
     return None
-  b = rq.reshape(k, cout).t().contiguous()
+  b = _conv_weight_matrix(rq, k, cout)
   row_scale = ls.reshape(n, 1).float().expand(n, positions).reshape(1, n * positions).contiguous()
   out = ops.gemm(a.contiguous()[None], b[None], row_scale=row_scale, col_scale=rs.reshape(1, cout).float().contiguous(),
                  out_dtype=out_dtype, dequant_dtype=out_dtype, row_scale_dtype=ls.dtype, col_scale_dtype=rs.dtype,

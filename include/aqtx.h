@@ -285,6 +285,18 @@ typedef struct aqtx_im2col_plan {
 int aqtx_im2col_i8(const aqtx_im2col_plan* plan, const void* x, void* out, void* stream);
 
 /*
+ * aqtx_conv_i8: the same convolution in one launch, the windows read in place instead of gathered:
+ * C[images * positions][n] = dequant(windows(x) * B^T), i.e. aqtx_im2col_i8(window, x) followed by
+ * aqtx_gemm_i8(plan, ., b, ...) without the [images * positions][taps * c] matrix in between (same bits).
+ * Replaces the same reference lines (aqt/jax/v2/aqt_conv_general.py:95-107).  `plan` describes the
+ * contraction (batch 1, m = images * positions, n, k = taps * c, ldb, ldc, dtypes, scale order; lda is not
+ * read); features must be a multiple of 128 and x smaller than 2 GiB, other inputs take the two calls.
+ *   x : int8 [images][spatial...][c];  b : int8 [n][ldb];  row_scale float32 [m], col_scale float32 [n]
+ */
+int aqtx_conv_i8(const aqtx_im2col_plan* window, const aqtx_gemm_plan* plan, const void* x, const void* b,
+                 const float* row_scale, const float* col_scale, void* c, void* stream);
+
+/*
  * aqtx_fp_round: rounds x[count] (bf16 or f32) to an emulated small float with `nexp`
  * exponent bits, `nmant` mantissa bits, smallest exponent 0, with or without subnormals, no
  * NaN/inf codes, and writes the result in the same container dtype.  Replaces

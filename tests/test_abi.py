@@ -338,3 +338,21 @@ def test_gemm_k_slices_choice_is_a_host_decision():
   assert 'k_split must be in 0..64' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
   p = _gplan(m=128, n=4096, k=14336, lda=14336, ldb=14336, ldc=4096, k_split=4)
   assert 'k_split_workspace' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
+
+
+def test_conv_validation():
+  lib = L.lib()
+  w = L.Im2colPlan()
+  w.n, w.c, w.rank = 2, 128, 2
+  for d in range(2):
+    w.in_size[d], w.kernel[d], w.stride[d], w.dilation[d], w.pad_lo[d], w.out_size[d] = 8, 3, 1, 1, 1, 8
+  good = dict(m=2 * 64, n=32, k=9 * 128, lda=9 * 128, ldb=9 * 128, ldc=32)
+  call = lambda wp, gp, x=FAKE: lib.aqtx_conv_i8(ctypes.byref(wp), ctypes.byref(gp), x, FAKE, None, None, FAKE, None)
+  assert 'm = images * positions' in _err(call(w, _gplan(**dict(good, m=100))))
+  assert 'k = taps * features' in _err(call(w, _gplan(**dict(good, k=1024, lda=1024, ldb=1024))))
+  assert 'no k slices' in _err(call(w, _gplan(k_split=2, **good)))
+  assert 'NULL' in _err(call(w, _gplan(**good), None))
+  w.c = 64
+  assert 'multiple of 128' in _err(call(w, _gplan(**dict(good, k=9 * 64, lda=9 * 64, ldb=9 * 64))))
+  w.c, w.rank = 128, 4
+  assert 'rank' in _err(call(w, _gplan(**good)))

@@ -256,3 +256,56 @@ def test_window_gather_kernel(gpu, case):
   want, want_sizes = aqt_conv._windows(x, list(case['ker']), list(case['strides']), case['pads'], list(case['dil']))
   assert list(out_sizes) == list(want_sizes) and got.shape == want.shape
   assert torch.equal(got, want.contiguous())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('out,rdt,cdt', [('bf16', 'bf16', 'bf16'), ('bf16', 'f32', 'f32'), ('f32', 'f32', 'f32')])
+@pytest.mark.parametrize('case', [
+    dict(x=(2, 9, 8, 128), ker=(3, 3), strides=(1, 1), pads=[(1, 1), (1, 1)], dil=(1, 1), n=64),
+    dict(x=(3, 12, 11, 256), ker=(3, 2), strides=(2, 1), pads=[(1, 0), (0, 1)], dil=(1, 2), n=200),
+    dict(x=(5, 37, 128), ker=(5,), strides=(3,), pads=[(2, 1)], dil=(1,), n=130),
+    dict(x=(2, 5, 6, 4, 128), ker=(2, 2, 2), strides=(1, 1, 2), pads=[(0, 1), (1, 0), (0, 1)], dil=(1, 1, 1), n=48),
+    dict(x=(1, 4, 4, 128), ker=(5, 5), strides=(1, 1), pads=[(0, 0), (0, 0)], dil=(1, 1), n=16),   # no position at all
+    dict(x=(2, 30, 30, 128), ker=(1, 1), strides=(1, 1), pads=[(0, 0), (0, 0)], dil=(1, 1), n=256),  # one tap = one stage
+])
+def test_convolution_without_the_window_matrix(gpu, case, out, rdt, cdt):
+  """aqtx_conv_i8 (the windows read in place by the contraction kernel) against aqtx_im2col_i8 + aqtx_gemm_i8:
+  the same bits, for strides, dilations, uneven padding, one to three spatial axes."""
+  from aqt_amd import ops
+  rng = np.random.default_rng(5)
+  x = torch.from_numpy(rng.integers(-127, 128, case['x']).astype(np.int8)).to(gpu)
+  taps = int(np.prod(case['ker']))
+  k, n = taps * case['x'][-1], case['n']
+  w = torch.from_numpy(rng.integers(-127, 128, (n, k)).astype(np.int8)).to(gpu)
+  a, out_sizes = ops.im2col_i8(x, case['ker'], case['strides'], case['pads'], case['dil'])
+  m = a.shape[0]
+  if m == 0:
+    return
+  rs = torch.from_numpy(nm.cast(np.abs(rng.standard_normal(m).astype(np.float32)) * np.float32(0.02) + np.float32(1e-3), rdt)).to(gpu)
+  cs = torch.from_numpy(nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(3e-3) + np.float32(1e-4), cdt)).to(gpu)
+  kw = dict(out_dtype=U.TORCH_DT[out], row_scale_dtype=U.TORCH_DT[rdt], col_scale_dtype=U.TORCH_DT[cdt])
+  want = ops.gemm(a[None], w[None], row_scale=rs[None], col_scale=cs[None], **kw)[0]
+  got, got_sizes = ops.conv_i8(x, w, case['ker'], case['strides'], case['pads'], case['dil'], row_scale=rs, col_scale=cs, **kw)
+  assert list(got_sizes) == list(out_sizes)
+  assert torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_conv_layer_with_128_features_matches_oracle(gpu):
+  """A quantized convolution whose input has 128 features takes the one-kernel path (strides, dilation and
+  uneven padding included); bit-exact to the oracle."""
+  from aqt_amd.v2 import aqt_conv_general as aqt_conv
+  dt = 'bf16'
+  for case in (dict(lhs=(2, 10, 9, 128), rhs=(3, 3, 128, 40), strides=(1, 1), padding='SAME'),
+               dict(lhs=(2, 13, 12, 256), rhs=(3, 2, 256, 130), strides=(2, 1), padding=[(1, 0), (0, 2)], dil=(1, 2))):
+    raw = aqt_conv.conv_general_dilated_make(2, 8, 8)
+    lhs_np = _rand_unif(case['lhs'], 3.0, 5, dt)
+    rhs_np = _rand_unif(case['rhs'], 0.5, 6, dt)
+    lhs, rhs = U.to_dev(lhs_np, dt, gpu), U.to_dev(rhs_np, dt, gpu)
+    out = aqt_conv.make_conv_general_dilated(raw)(
+        lhs, rhs, window_strides=case['strides'], padding=case['padding'], rhs_dilation=case.get('dil'),
+        dimension_numbers=aqt_conv.flax_conv_dimension_numbers(lhs.shape))
+    want, _, _ = R.conv_general_dilated_fwd(lhs_np, rhs_np, dt, case['strides'], case['padding'],
+                                            R.RawCfg(_qcfg(8, po2=False), _qcfg(8, po2=False)), case.get('dil'))
+    assert tuple(out.shape) == want.shape
+    np.testing.assert_array_equal(out.float().cpu().numpy(), want)
