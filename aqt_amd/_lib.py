@@ -123,6 +123,7 @@ SYMBOLS = {
     'aqtx_sum_tiles': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),
     'aqtx_prng_split_host': (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint32), ctypes.c_int32,
                                             ctypes.c_int32, ctypes.POINTER(ctypes.c_uint32)]),
+    'aqtx_prng_split': (ctypes.c_int, [_vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp]),
     'aqtx_random_bits': (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint32), ctypes.c_int64,
                                         ctypes.c_int32, ctypes.c_int32, _vp, _vp]),
     'aqtx_read_probe': (ctypes.c_int, [_vp, ctypes.c_int64, _vp, ctypes.c_int64, _vp]),

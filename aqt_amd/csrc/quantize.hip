@@ -1205,6 +1205,39 @@ extern "C" int aqtx_random_bits(const uint32_t key_host[2], int64_t n, int32_t b
   return 0;
 }
 
+namespace aqtx {
+namespace {
+__global__ __launch_bounds__(256) void prng_split_kernel(const uint32_t* __restrict__ key, int num, int partitionable,
+                                                         uint32_t* __restrict__ out) {
+  const int i = (int)(blockIdx.x * 256 + threadIdx.x);  // word i of the 2 * num
+  if (i >= 2 * num) return;
+  const uint32_t k0 = key[0], k1 = key[1];
+  if (partitionable) {
+    const U2 b = threefry2x32(k0, k1, 0u, (uint32_t)(i >> 1));
+    out[i] = (i & 1) ? b.y : b.x;
+  } else {
+    BitGen g;
+    g.k0 = k0; g.k1 = k1;
+    g.nwords = 2u * (uint32_t)num; g.half = (uint32_t)num;
+    g.partitionable = 0; g.width = 32;
+    out[i] = g.word_original((uint32_t)i);
+  }
+}
+}  // namespace
+}  // namespace aqtx
+
+extern "C" int aqtx_prng_split(const uint32_t* key_device, int32_t num, int32_t partitionable, uint32_t* out_device,
+                               void* stream) {
+  clear_error();
+  AQTX_REQUIRE(num >= 0 && num <= (1 << 20), "aqtx_prng_split: num outside 0..2^20");
+  if (num == 0) return 0;
+  AQTX_REQUIRE(key_device != nullptr && out_device != nullptr, "aqtx_prng_split: NULL argument");
+  prng_split_kernel<<<(unsigned)((2 * num + 255) / 256), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
+      key_device, num, partitionable, out_device);
+  AQTX_HIP_CHECK_LAUNCH("prng_split_kernel");
+  return 0;
+}
+
 extern "C" int aqtx_prng_split_host(const uint32_t key_host[2], int32_t num, int32_t partitionable,
                                     uint32_t* out_host) {
   clear_error();

@@ -161,7 +161,8 @@ def quantize(
   [batch, rows, cols] or [batch, cols, rows] with transpose_out; scale is
   float32, shaped [batch, rows, cols/group] (REDUCE_COLS),
   [batch, rows/group, cols] (REDUCE_ROWS) or [batch] (REDUCE_ALL).
-  `key_device` (a 2-word device tensor) replaces `key`: the kernels read the key from device memory.
+  `key_device` (a 2-word device tensor, or such a tensor passed as `key`) replaces `key`: the kernels read
+  the key from device memory.
   `k_order` = L.K_EVEN_ODD8 stores every aligned group of 8 values along cols as elements
   0,2,4,6,1,3,5,7 (the lhs of gemm_grouped against a packed int4 rhs).
   With want_typed_scale a third element: the computed scales once more as a bf16 tensor of
@@ -180,6 +181,8 @@ def quantize(
   plan.reduce, plan.transpose_out, plan.group = reduce, int(transpose_out), group
   plan.quant_bound, plan.clip_bound = quant_bound, clip_bound
   plan.noise, plan.partitionable = noise, int(partitionable)
+  if isinstance(key, torch.Tensor):  # a key held on the device (prng_split of a device key gives such keys)
+    key_device, key = key, None
   if noise != L.NOISE_NONE:
     assert key is not None or key_device is not None, 'noise requested but no PRNG key given'
     if key_device is not None:  # uint32[2] (held as int32) in device memory, read by the kernels
@@ -562,22 +565,38 @@ def fp_round(x: torch.Tensor, *, nexp: int, nmant: int, has_subnormals: bool, ke
     plan.mode, plan.noise_mod = L.FP_NOISE_INDEX, int(noise_mod)
   else:
     assert key is not None, 'stochastic rounding requested but the key is None'
+    key = _host_key(key, 'fp_round')
     plan.mode = L.FP_NOISE_JAX_BITS
     k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))
   L.check(L.lib().aqtx_fp_round(ctypes.byref(plan), _ptr(x), _ptr(out), k, _stream()))
   return out
 
 
-def prng_split(key, num: int, partitionable: bool = False) -> np.ndarray:
-  """jax.random.split(key, num) on raw uint32[2] key data (host side)."""
+def prng_split(key, num: int, partitionable: bool = False):
+  """jax.random.split(key, num) on raw uint32[2] key data: on the host for a numpy key (returns numpy
+  [num, 2]); for a key that is a 2-word device tensor, by a kernel, into a device tensor [num, 2] (no host
+  round trip: the split can be recorded into a HIP graph and follows the key's value on every replay)."""
+  if isinstance(key, torch.Tensor):
+    _require_gpu(key)
+    assert key.numel() == 2 and key.element_size() == 4 and key.is_contiguous()
+    out = torch.empty((num, 2), dtype=key.dtype, device=key.device)
+    L.check(L.lib().aqtx_prng_split(_ptr(key), num, int(partitionable), _ptr(out), _stream()))
+    return out
   k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))
   out = (ctypes.c_uint32 * (2 * num))()
   L.check(L.lib().aqtx_prng_split_host(k, num, int(partitionable), out))
   return np.frombuffer(out, dtype=np.uint32).reshape(num, 2).copy()
 
 
+def _host_key(key, who: str):
+  if isinstance(key, torch.Tensor):
+    raise TypeError(f'{who}: a PRNG key held on the device is only read by the fused quantize kernels; pass a host key')
+  return key
+
+
 def random_bits(key, n: int, bit_width: int = 32, partitionable: bool = False, device='cuda'):
   """jax.random.bits(key, (n,), uint{bit_width}) generated on the GPU."""
+  key = _host_key(key, 'random_bits')
   k = (ctypes.c_uint32 * 2)(int(key[0]), int(key[1]))
   out = torch.empty(n, dtype=torch.int16 if bit_width == 16 else torch.int32, device=device)
   _require_gpu(out)

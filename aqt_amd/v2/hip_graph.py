@@ -7,9 +7,12 @@ for small-batch serving costs ten times the kernels' own time.  `GraphedCall` re
 of one call, made on fixed-shape inputs, into a HIP graph; a replay is one launch.
 
 What a recorded call may do: launch kernels of this library and torch device ops on the current
-stream.  What it may not: read device data on the host, change Python-side state that later calls
-depend on (calibration statistics, freezing: record serving calls, not training or conversion
-calls), or draw fresh noise (a key is a kernel argument fixed at recording time; serving uses none).
+stream.  What it may not: read device data on the host, or change Python-side state that later calls
+depend on (calibration statistics, freezing: no conversion calls, no stateful calibrators).  A key
+given as host data is a kernel argument fixed at recording time; a key held in a device tensor
+(`config.set_context(cfg, key_tensor, ...)`: the fan-out runs as a kernel, the quantizers read their keys
+from device memory) is read anew by every replay, which is how a training step with stochastic
+rounding is recorded: `GraphedStep`.
 """
 from __future__ import annotations
 
@@ -102,3 +105,34 @@ class GraphedCall:
         if d.data_ptr() != s.data_ptr():
           d.copy_(s)
     return self.replay()
+
+
+class GraphedStep:
+  """`fn()` as a HIP graph, recorded with gradients enabled: a forward + backward pass over tensors the
+  caller keeps (inputs, parameters, the output gradient, a PRNG key in a device tensor).  The caller
+  refills those tensors in place and calls `replay()`; what `fn` returned (and the `.grad` tensors its
+  backward pass created) are overwritten by every replay.  Before recording, set the `.grad` of the
+  leaves to None so that the backward pass writes, not accumulates."""
+
+  def __init__(self, fn: Callable, warmup: int = 3):
+    if not torch.cuda.is_available():
+      raise RuntimeError('GraphedStep needs a GPU')
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), ops.private_workspaces({}):
+      for _ in range(max(1, warmup)):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    self._workspaces = {}
+    self._graph = torch.cuda.CUDAGraph()
+    with ops.private_workspaces(self._workspaces), torch.cuda.graph(self._graph):
+      self._outputs = fn()
+
+  @property
+  def outputs(self):
+    return self._outputs
+
+  def replay(self):
+    self._graph.replay()
+    return self._outputs

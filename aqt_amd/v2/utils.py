@@ -104,7 +104,8 @@ def get_remaining_axes(rank: int, contraction_axes: Sequence[int], batch_axes: S
 
 @dataclasses.dataclass
 class Context:
-  """utils.py:151-155. `key` is raw threefry key data: uint32[2] (numpy)."""
+  """utils.py:151-155. `key` is raw threefry key data: uint32[2], numpy, or a 2-word device tensor
+  (read by the kernels where it lies: a key that changes between replays of a recorded step)."""
   key: Any = None
   train_step: Optional[int] = None
   quant_mode: QuantMode = QuantMode.TRAIN
@@ -112,8 +113,8 @@ class Context:
   def __deepcopy__(self, memo):
     out = clone_fields(self)
     memo[id(self)] = out
-    if out.key is not None:
-      out.key = copy.deepcopy(self.key, memo)
+    if out.key is not None and not isinstance(out.key, torch.Tensor):
+      out.key = copy.deepcopy(self.key, memo)  # (a key in a device tensor is a handle: shared)
     return out
 
 

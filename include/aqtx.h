@@ -427,6 +427,14 @@ int aqtx_prng_split_host(const uint32_t key_host[2], int32_t num, int32_t partit
                          uint32_t* out_host);
 
 /*
+ * aqtx_prng_split: the same split of a key held in DEVICE memory, by a kernel: key_device uint32[2],
+ * out_device uint32[num][2].  For keys that are traced arrays under XLA or change between replays of a
+ * HIP graph (aqtx_quant_plan.key_device reads the results).
+ */
+int aqtx_prng_split(const uint32_t* key_device, int32_t num, int32_t partitionable, uint32_t* out_device,
+                    void* stream);
+
+/*
  * aqtx_random_bits: jax.random.bits(key, [n], uint{bit_width}) on the device,
  * bit_width in {16, 32}; out is uint16[n] or uint32[n].  Exposes the in-kernel
  * generator of aqtx_quantize for tests (stochastic_rounding.py:46,65).

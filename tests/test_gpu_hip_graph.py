@@ -155,3 +155,51 @@ def test_argument_checks(gpu):
     graphed(x, x)
   with pytest.raises(ValueError, match='GPU'):
     hip_graph.GraphedCall(lambda a: a, torch.zeros(4))
+
+
+def test_training_step_with_a_key_on_the_device_replays(gpu):
+  """Forward + backward with stochastic rounding, the PRNG key in a device tensor: the key fan-out of
+  set_context runs as a kernel and the quantizers read their keys from device memory, so a recorded step
+  draws the noise of whatever key the tensor holds at replay time.  Every replay equals the eager step with
+  the same key given as host data."""
+  import numpy as np
+  dt = 'bf16'
+  base = config.fully_quantized(fwd_bits=8, bwd_bits=8)
+  x_np, w_np = U.rand((256, 512), dt, 1, outliers=True), U.rand((512, 384), dt, 2, 0.02)
+  g = U.to_dev(U.rand((256, 384), dt, 3, 1e-3), dt, gpu)
+
+  def eager(key):
+    x = U.to_dev(x_np, dt, gpu).requires_grad_(True)
+    w = U.to_dev(w_np, dt, gpu).requires_grad_(True)
+    y = config.set_context(base, key, None)(x, w, MATMUL)
+    y.backward(g)
+    return y.detach(), x.grad, w.grad
+
+  def on_device(key):
+    return torch.from_numpy(np.asarray(key, dtype=np.uint32).view(np.int32).copy()).to(gpu)
+
+  k1, k2, k3 = utils.prng_key(11), utils.prng_key(12), utils.prng_key(13)
+  want1 = eager(k1)
+  got1 = eager(on_device(k1))
+  assert all(torch.equal(a, b) for a, b in zip(got1, want1)), 'device key differs from the host key (eager)'
+  assert not torch.equal(want1[1], eager(k2)[1]), 'the gradient does not depend on the key'
+
+  key_dev = on_device(k1)
+  x = U.to_dev(x_np, dt, gpu).requires_grad_(True)
+  w = U.to_dev(w_np, dt, gpu).requires_grad_(True)
+
+  def step():
+    x.grad = w.grad = None
+    y = config.set_context(base, key_dev, None)(x, w, MATMUL)
+    y.backward(g)
+    return y, x.grad, w.grad
+
+  graphed = hip_graph.GraphedStep(step)
+  for key in (k2, k3, k1, k2):
+    key_dev.copy_(on_device(key))
+    got = [t.detach().clone() for t in graphed.replay()]
+    torch.cuda.synchronize()
+    want = eager(key)   # eager work of the same kernels between the replays
+    torch.cuda.synchronize()
+    for name, a, b in zip(('out', 'dlhs', 'drhs'), got, want):
+      assert torch.equal(a, b), f'{name} of the replay differs from the eager step'
