@@ -69,6 +69,25 @@ class LocalAqt:
 
 _FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
 
+# Weight-only quantization (a float lhs against an int8 / fp8 rhs) promotes the rhs to the float dtype on
+# every call; for a frozen weight that is the same conversion every time, so large converted copies are
+# kept for as long as the quantized tensor lives and stays unchanged (its version counter).
+_PROMOTED_RHS = {}  # id(rhs) -> (key, promoted [b, k, n] copy)
+
+
+def _promoted_rhs(rhs, perm, shape, common):
+  if rhs.dtype == common or rhs.numel() < (1 << 20) or rhs.requires_grad:
+    return rhs.permute(perm).reshape(shape).to(common)
+  key = (perm, tuple(rhs.shape), common, rhs._version)
+  hit = _PROMOTED_RHS.get(id(rhs))
+  if hit is not None and hit[0] == key:
+    return hit[1]
+  out = rhs.permute(perm).reshape(shape).to(common)
+  if hit is None:
+    weakref.finalize(rhs, _PROMOTED_RHS.pop, id(rhs), None)
+  _PROMOTED_RHS[id(rhs)] = (key, out)
+  return out
+
 
 def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None):
   """dot_general with lax semantics (output axes: batch, lhs remaining, rhs remaining).
@@ -117,8 +136,8 @@ def lax_dot_general(lhs, rhs, dimension_numbers, precision=None, preferred_eleme
     if pet is not None and pet.is_floating_point and common.is_floating_point and (
         torch.finfo(pet).bits > torch.finfo(common).bits):
       common = pet  # wider accumulator asked for: keep its precision in the result
-    rt = rhs.permute(tuple(rba + rca + rra)).reshape(b, kdim, -1)
-    out = torch.matmul(lt.to(common), rt.to(common))
+    rt = _promoted_rhs(rhs, tuple(rba + rca + rra), (b, kdim, -1), common)
+    out = torch.matmul(lt.to(common), rt)
   out = out.reshape(bshape + mshape + nshape)
   if preferred_element_type is not None:
     out = out.to(preferred_element_type)

@@ -114,6 +114,31 @@ def test_one_sided_quantization(gpu, lhs_bits, rhs_bits, dt):
   _close(_np(out), want, dt)
 
 
+def test_weight_only_serving_keeps_the_promoted_weight(gpu):
+  """A frozen int8 weight next to a float lhs is promoted to the float dtype once, not on every call; a change
+  of the weight in place is noticed (version counter)."""
+  from aqt_amd.v2 import aqt_dot_general as adg
+  dt = 'bf16'
+  cfg = config.set_context(aqt.dot_general_make(None, 8), None, None)
+  x1, x2 = U.to_dev(U.rand((8, 1024), dt, 1), dt, gpu), U.to_dev(U.rand((8, 1024), dt, 2), dt, gpu)
+  w = U.to_dev(U.rand((1024, 1024), dt, 3, 0.05), dt, gpu)
+  _, (_, wq) = cfg.dg_core(x1, w, None, None, MATMUL)
+  assert wq.qvalue.dtype == torch.int8
+  serve = lambda x: cfg.dg_core(x, torch.zeros_like(w), None, wq, MATMUL)[0]
+  adg._PROMOTED_RHS.clear()
+  a1, a2 = serve(x1), serve(x2)
+  assert list(adg._PROMOTED_RHS) == [id(wq.qvalue)]
+  kept = adg._PROMOTED_RHS[id(wq.qvalue)][1]
+  b1 = serve(x1)
+  assert adg._PROMOTED_RHS[id(wq.qvalue)][1] is kept and torch.equal(a1, b1) and not torch.equal(a1, a2)
+  want = (x1.float() @ (wq.qvalue.float() * wq.scale[0].float())).to(torch.bfloat16)
+  np.testing.assert_allclose(a1.float().cpu().numpy(), want.float().cpu().numpy(), rtol=2e-2, atol=2e-2)
+  wq.qvalue.neg_()   # in place: the kept copy is stale
+  c1 = serve(x1)
+  assert adg._PROMOTED_RHS[id(wq.qvalue)][1] is not kept
+  assert torch.equal(c1, -a1)
+
+
 def _set_calibration(raw, oraw, **kw):
   for q, oq in ((raw.dg_quantizer.lhs, oraw.lhs), (raw.dg_quantizer.rhs, oraw.rhs)):
     if 'const_bound' in kw:
