@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, 'csrc')
 LIB_DIR = os.path.join(HERE, 'lib')
 LIB_PATH = os.path.join(LIB_DIR, 'libaqtx.so')
 
-SOURCES = ['capi.hip', 'quantize.hip', 'gemm_i8.hip', 'gemm_mid.hip', 'gemm_fp8.hip', 'decode_i8.hip', 'reduce.hip',
+SOURCES = ['capi.hip', 'quantize.hip', 'gemm_i8.hip', 'gemm_mid.hip', 'gemm_fp8.hip', 'decode_i8.hip', 'decode_wo.hip', 'reduce.hip',
            'gemm_grouped.hip', 'fp_round.hip', 'im2col.hip']
 
 HIPCC_FLAGS = [

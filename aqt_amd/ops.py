@@ -334,6 +334,37 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
   return torch.clamp(offs, max=m)
 
 
+def decode_weight_only(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, w_scale_dtype=torch.float32,
+                       w_dtype: int = L.I8, w_layout: int = L.W_ROWS, out_dtype=None, tuning: int = 0):
+  """Weight-only serving contraction out = dequant(x @ float(w_q)^T) for bf16 x [m <= 64, k] that stays
+  unquantized and w_q int8 [n, k] (or packed int4 uint8 [n, k/2], or either re-laid by tile_weight);
+  `w_scale` is float32 [n] holding values of `w_scale_dtype`.  float32 sums."""
+  _require_gpu(x, w_q, w_scale)
+  packed = w_dtype == L.I4P
+  assert x.dim() == 2 and x.is_contiguous() and w_q.is_contiguous() and x.dtype == torch.bfloat16
+  m, k = x.shape
+  if w_layout == L.W_FRAGMENTS:
+    n = w_scale.numel()
+    assert w_q.numel() * w_q.element_size() == L.lib().aqtx_tile_weight_bytes(n, k, w_dtype), (w_q.shape, n, k)
+  else:
+    assert w_q.dim() == 2 and k == w_q.shape[1] * (2 if packed else 1), (x.shape, w_q.shape)
+    n = w_q.shape[0]
+  assert w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() == n
+  out_dtype = out_dtype if out_dtype is not None else x.dtype
+  plan = L.DecodePlan()
+  plan.m, plan.n, plan.k = m, n, k
+  plan.x_dtype = aqtx_dtype(x.dtype)
+  plan.x_scale_dtype = plan.x_dtype
+  plan.w_scale_dtype = aqtx_dtype(w_scale_dtype)
+  plan.out_dtype = aqtx_dtype(out_dtype)
+  plan.quant_bound = plan.clip_bound = 1.0
+  plan.w_dtype, plan.w_layout, plan.tuning = w_dtype, w_layout, tuning
+  out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+  with _timed('decode'):
+    L.check(L.lib().aqtx_decode_weight_only(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(out), _stream()))
+  return out
+
+
 def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_bound: float,
            clip_bound: float, x_scale_dtype=None, w_scale_dtype=torch.float32, want_xq: bool = False,
            w_dtype: int = L.I8, tuning: int = 0, static_scratch: bool = False, w_layout: int = L.W_ROWS):

@@ -761,6 +761,11 @@ class DotGeneralRaw:
                           rhs=TensorRes(mt=MultiTensor(x=y, qx=mk(y)), quant_grad=None))
       return out, res
 
+    if isinstance(dq, DefaultDotGeneralQuantizer) and lhs_none and not rhs_none:
+      served = self._serve_weight_only(lhs, dq, lhs_qt, rhs_arr, rhs_qt, dimension_numbers, prescale_t,
+                                       out_transpose_axes, dequant_dtype)
+      if served is not None:
+        return served
     if not isinstance(dq, DefaultDotGeneralQuantizer) or lhs_none or rhs_none:
       raise _NotFused(
           'only DefaultDotGeneralQuantizer with both sides quantized (or both unquantized) is lowered')
@@ -913,6 +918,49 @@ class DotGeneralRaw:
     lhs_grad = functools.partial(dq.lhs.numerics.vjp_bwd, (None,))
     rhs_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
     res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=lhs, qx=lhs_qt_out), quant_grad=lhs_grad),
+                        rhs=TensorRes(mt=MultiTensor(x=rhs_arr, qx=rhs_qt), quant_grad=rhs_grad))
+    return out, res
+
+  def _serve_weight_only(self, lhs, dq, lhs_qt, rhs_arr, rhs_qt, dimension_numbers, prescale_t, out_transpose_axes,
+                         dequant_dtype):
+    """Serving with an unquantized bf16 lhs of at most 64 rows and a frozen int8 / int4 rhs with one scale per
+    output channel: the weight-only kernel (the weight streamed once, converted to bf16 in registers; the
+    reference promotes the whole weight to bf16 and contracts in float, aqt_dot_general.py:843-958).  Returns
+    None when the call does not have that shape."""
+    if (rhs_qt is None or not rhs_qt.is_full() or lhs_qt is not None or prescale_t is not None
+        or out_transpose_axes is not None or self.dot_general is not lax_dot_general or self.local_aqt is not None
+        or self.rhs.dequant_mode != DequantMode.OUTPUT or lhs.dtype != torch.bfloat16
+        or dequant_dtype != torch.bfloat16 or (lhs.requires_grad and torch.is_grad_enabled())):
+      return None
+    if (rhs_qt.qvalue.dtype != torch.int8 or len(rhs_qt.scale) != 1 or rhs_qt.bias or rhs_qt.sparsity_mask is not None
+        or rhs_qt.container_dtype not in (None, utils.int4)
+        or rhs_qt.scale[0].dtype not in (torch.bfloat16, torch.float32)):
+      return None
+    dn = _canonical_pairs(lhs, rhs_arr, dimension_numbers)
+    (lca, rca), (lba, rba) = dn
+    if lba or rba:
+      return None
+    lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
+    rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
+    lv = lowering.view_operand(lhs, [], lra, lca)
+    rv = lowering.view_operand(rhs_qt.qvalue, [], rra, rca)
+    if not lv.k_last or lv.copied:
+      return None
+    M, K, N = lv.R, lv.K, rv.R
+    packed = rhs_qt.container_dtype is utils.int4 and K % 32 == 0
+    if M == 0 or M > 64 or K == 0 or K % 16 != 0 or N == 0 or N * K >= 2 ** 31:
+      return None
+    w_scale = rhs_qt.scale[0]
+    if lowering.view_operand(w_scale, [], rra, rca).mem.numel() != N:
+      return None
+    w_fragments = _kernel_layout_of(rhs_qt.qvalue, rv, pack_int4=packed, fragments=True)
+    out = ops.decode_weight_only(
+        lv.mem[0], w_fragments, _scale_vector_f32(w_scale, [], rra, rca), w_scale_dtype=w_scale.dtype,
+        w_dtype=L.I4P if packed else L.I4 if rhs_qt.container_dtype is utils.int4 else L.I8, w_layout=L.W_FRAGMENTS)
+    out = out.reshape([lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
+    lhs_qt_out = aqt_tensor.QTensor(qvalue=lhs, scale=[], scale_t=None, bias=[], dequant_dtype=lhs.dtype)
+    rhs_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
+    res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=lhs, qx=lhs_qt_out), quant_grad=None),
                         rhs=TensorRes(mt=MultiTensor(x=rhs_arr, qx=rhs_qt), quant_grad=rhs_grad))
     return out, res
 

@@ -225,7 +225,31 @@ def other_configs(dev):
     out['int8_frozen_serving_layer_call_m8_4096x14336'] = {
         'eager_us_per_call': round(timeit(lambda: call(xs), n=100, w=10) * 1e3, 1),
         'hip_graph_us_per_call': round(timeit(lambda: graphed(xs), n=100, w=10) * 1e3, 1)}
-  del conv, serve, graphed, xs, ws
+  del conv, serve, graphed
+  # weight-only serving (the lhs stays bf16, frozen int8 / int4 rhs [4096, 14336]): ten layer calls recorded
+  # into one HIP graph, so the figure is the call's device time (the weight streamed once and converted
+  # to bf16 in registers), not the gap between graph launches
+  from aqt_amd.v2 import aqt_dot_general
+  wo = {}
+  with torch.no_grad():
+    for bits in (8, 4):
+      cfg = config.set_context(aqt_dot_general.dot_general_make(None, bits), None, None)
+      _, (_, wq) = cfg.dg_core(xs, ws, None, None, MATMUL)
+      for m_few in (1, 8, 64):
+        xf = torch.randn(m_few, 4096, device=dev).to(torch.bfloat16)
+
+        def ten(a):
+          for _ in range(9):
+            cfg.dg_core(a, ws, None, wq, MATMUL)
+          return cfg.dg_core(a, ws, None, wq, MATMUL)[0]
+
+        graphed = hip_graph.GraphedCall(ten, xf)
+        us = timeit(graphed.replay, n=10, w=3) * 1e3 / 10
+        wo[f'int{bits}_m{m_few}'] = {'us_per_call': round(us, 1), 'weight_GB/s': round(4096 * 14336 * bits / 8 / us / 1e3, 1)}
+        del graphed
+      del wq
+  out['weight_only_frozen_serving_few_tokens_4096x14336'] = wo
+  del xs, ws
   # quantized ragged_dot (mixture of experts): 8192 tokens routed to 8 experts [4096, 14336], uneven groups,
   # forward, with the expert weights quantized on the fly (the reference's ragged_dot does the same) and
   # with the contraction alone (operands already int8)

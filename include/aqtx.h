@@ -420,6 +420,20 @@ int aqtx_decode_i8_static(const aqtx_decode_plan* plan, const void* x, const voi
                           const float* w_scale, void* xq, float* x_scale, void* out, void* stream);
 
 /*
+ * aqtx_decode_weight_only: out[m, n] = dequant(x[m, :] . float(w[n, :])) for m <= 64 bf16 activations that are
+ * NOT quantized and a frozen int8 / int4 weight with one scale per output channel.  Replaces
+ * _qtensor_dot_general with an unquantized lhs (aqt/jax/v2/aqt_dot_general.py:843-958: the quantized rhs is
+ * promoted to the lhs dtype, lax.dot_general contracts in float, the rhs scale multiplies the output) followed
+ * by QTensor.dequant (aqt_tensor.py:161-200), for a provided rhs QTensor (:614-635).  The weight is streamed
+ * once and converted to bf16 in registers; sums are float32, so the result agrees with the reference's float
+ * contraction to summation order, not bit for bit.  Of the plan: m, n, k, x_dtype (AQTX_BF16), w_dtype,
+ * w_layout, w_scale_dtype, out_dtype and tuning (low three bits 1 / 2 / 4: weight rows per workgroup in
+ * sixteens; 0 = the library chooses) are read.  k must be a multiple of 16 (32 for packed int4).  No workspace.
+ */
+int aqtx_decode_weight_only(const aqtx_decode_plan* plan, const void* x, const void* w, const float* w_scale,
+                            void* out, void* stream);
+
+/*
  * aqtx_prng_split_host: jax.random.split(key, num) on the host (used by
  * config.set_context, aqt/jax/v2/config.py:61-90).  out_host: uint32[num][2].
  */

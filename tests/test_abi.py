@@ -189,6 +189,28 @@ def test_decode_workspace_and_null_checks():
   assert L.lib().aqtx_decode_i8(ctypes.byref(_dplan(m=0)), None, None, None, None, None, None, None, 0, None) == 0
 
 
+@pytest.mark.parametrize('kw,needle', [
+    (dict(m=65), 'exceeds 64'),
+    (dict(k=24), 'multiple of 16'),
+    (dict(w_dtype=L.I4P, k=48), 'multiple of 32'),
+    (dict(x_dtype=L.F32), 'must be bf16'),
+    (dict(out_dtype=L.I32), 'dtypes'),
+    (dict(w_dtype=L.E5M2), 'w_dtype'),
+    (dict(n=1 << 20, k=4096), '2 GiB'),
+    (dict(w_layout=7), 'w_layout'),
+])
+def test_weight_only_decode_plan_validation(kw, needle):
+  p = _dplan(**kw)
+  msg = _err(L.lib().aqtx_decode_weight_only(ctypes.byref(p), FAKE, FAKE, FAKE, FAKE, None))
+  assert needle in msg, msg
+
+
+def test_weight_only_decode_null_and_empty():
+  assert 'NULL' in _err(L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan()), None, FAKE, FAKE, FAKE, None))
+  assert 'plan is NULL' in _err(L.lib().aqtx_decode_weight_only(None, FAKE, FAKE, FAKE, FAKE, None))
+  assert L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan(n=0)), None, None, None, None, None) == 0
+
+
 def _ggplan(**kw):
   p = L.GroupedGemmPlan()
   p.m, p.n, p.k, p.group = 64, 128, 512, 128

@@ -313,3 +313,75 @@ def test_read_probe_reads_every_byte(gpu):
   words = buf.cpu().numpy().view(np.uint32)
   want = [np.bitwise_xor.reduce(words[i:i + 16384]) for i in range(0, len(words), 16384)]
   np.testing.assert_array_equal(got, np.asarray(want, dtype=np.uint32))
+
+
+# ---- weight-only serving (the lhs stays bf16; float32 sums: tolerance, not bits) ----------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize('layout', ['rows', 'fragments'])
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('w_sdt', ['bf16', 'f32'])
+@pytest.mark.parametrize('m,n,k', [(1, 200, 4096), (5, 16, 64), (16, 1024, 528 + 16 * 31), (17, 72, 2048), (33, 4096, 1024),
+                                   (64, 300, 4096)])
+def test_weight_only_decode_within_float_summation_error(gpu, m, n, k, w_sdt, packed, layout):
+  """out = bf16(bf16(sum_k x w) * scale) with the sum in float32 in the kernel's own order.  Tolerance, stated:
+  against the sum taken exactly (float64; every product of a bf16 and an int8 is exact), a float32 sum in any
+  order is off by less than d = k * 2^-24 * sum_k |x w|.  Every later step (the two roundings, the product with
+  a positive scale) is monotone, so each output must lie between the same steps applied to exact - d and to
+  exact + d; where the terms cancel that is many ulps of a small result, elsewhere less than one.  99 % of the
+  outputs must equal the steps applied to the exact sum."""
+  from aqt_amd import _lib as L
+  if packed and k % 32 != 0:
+    pytest.skip('packed int4 needs k % 32 == 0')
+  rng = np.random.default_rng(41)
+  x = nm.to_bf16(rng.standard_normal((m, k), dtype=np.float32))
+  lo, hi = (-8, 8) if packed else (-127, 128)
+  w = rng.integers(lo, hi, (n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal(n).astype(np.float32)) * np.float32(2e-3) + np.float32(1e-4), w_sdt)
+  exact = x.astype(np.float64) @ w.astype(np.float64).T
+  slack = k * 2.0 ** -24 * (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T)
+
+  def later_steps(total):
+    prod = nm.to_bf16(total.astype(np.float32)).astype(np.float64) * ws.astype(np.float64)[None, :]
+    prod = nm.cast(prod.astype(np.float32), w_sdt)
+    return nm.to_bf16(prod).astype(np.float64)
+
+  want, low, high = later_steps(exact), later_steps(exact - slack), later_steps(exact + slack)
+  wt = torch.from_numpy(w).to(gpu)
+  w_dtype = L.I8
+  if packed:
+    wt, w_dtype = ops.pack_i4(wt), L.I4P
+  w_layout = L.W_ROWS
+  if layout == 'fragments':
+    wt, w_layout = ops.tile_weight(wt, w_dtype), L.W_FRAGMENTS
+  got = ops.decode_weight_only(torch.from_numpy(x).to(torch.bfloat16).to(gpu), wt, torch.from_numpy(ws.astype(np.float32)).to(gpu),
+                               w_scale_dtype=U.TORCH_DT[w_sdt], w_dtype=w_dtype, w_layout=w_layout)
+  got = got.float().cpu().numpy().astype(np.float64)
+  assert ((low <= got) & (got <= high)).all(), np.argwhere((got < low) | (got > high))[:8]
+  assert (got == want).mean() >= 0.99
+
+
+@pytest.mark.gpu
+def test_weight_only_serving_takes_the_kernel(gpu):
+  """A float lhs of at most 64 rows against a frozen int8 rhs goes to the weight-only kernel; more rows (and
+  anything else) take the float product on the promoted weight.  Same numbers to float summation order."""
+  from aqt_amd.v2 import aqt_dot_general as aqt, config
+  dt = 'bf16'
+  MATMUL = (((1,), (0,)), ((), ()))
+  cfg = config.set_context(aqt.dot_general_make(None, 8), None, None)
+  w = U.to_dev(U.rand((1024, 520), dt, 3, 0.05), dt, gpu)
+  x_small, x_large = U.to_dev(U.rand((24, 1024), dt, 1), dt, gpu), U.to_dev(U.rand((80, 1024), dt, 2), dt, gpu)
+  with torch.no_grad():
+    _, (_, wq) = cfg.dg_core(x_small, w, None, None, MATMUL)
+    calls = []
+    real = ops.decode_weight_only
+    ops.decode_weight_only = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+      out_small, (lqt, _) = cfg.dg_core(x_small, torch.zeros_like(w), None, wq, MATMUL)
+      out_large, _ = cfg.dg_core(x_large, torch.zeros_like(w), None, wq, MATMUL)
+    finally:
+      ops.decode_weight_only = real
+  assert len(calls) == 1 and lqt.qvalue is x_small and lqt.scale == []
+  wf = wq.qvalue.float() * wq.scale[0].float()
+  for out, x in ((out_small, x_small), (out_large, x_large)):
+    want = (x.float() @ wf).cpu().numpy()
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2.0 ** -6, atol=2.0 ** -6 * np.abs(want).max())

@@ -115,12 +115,13 @@ def test_one_sided_quantization(gpu, lhs_bits, rhs_bits, dt):
 
 
 def test_weight_only_serving_keeps_the_promoted_weight(gpu):
-  """A frozen int8 weight next to a float lhs is promoted to the float dtype once, not on every call; a change
-  of the weight in place is noticed (version counter)."""
+  """A frozen int8 weight next to a float lhs of more than 64 rows (fewer go to the weight-only kernel) is
+  promoted to the float dtype once, not on every call; a change of the weight in place is noticed (version
+  counter)."""
   from aqt_amd.v2 import aqt_dot_general as adg
   dt = 'bf16'
   cfg = config.set_context(aqt.dot_general_make(None, 8), None, None)
-  x1, x2 = U.to_dev(U.rand((8, 1024), dt, 1), dt, gpu), U.to_dev(U.rand((8, 1024), dt, 2), dt, gpu)
+  x1, x2 = U.to_dev(U.rand((72, 1024), dt, 1), dt, gpu), U.to_dev(U.rand((72, 1024), dt, 2), dt, gpu)
   w = U.to_dev(U.rand((1024, 1024), dt, 3, 0.05), dt, gpu)
   _, (_, wq) = cfg.dg_core(x1, w, None, None, MATMUL)
   assert wq.qvalue.dtype == torch.int8
