@@ -1005,8 +1005,6 @@ class DotGeneralRaw:
       spec = None if isinstance(quantizer.numerics, no_numerics.NoNumerics) else quantizer.numerics.kernel_spec()
     if spec is None:
       raise _NotFused(f'{name}: numerics {quantizer.numerics} have no fused HIP kernel')
-    if getattr(quantizer.numerics, 'clip_gradient', False):
-      raise _NotFused('clip_gradient is not supported by the fused path')
     arr = x
     if x_is_q and arr.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
       raise _NotFused('re-quantizing an fp8 residual (use_fwd_quant with fp8 fwd)')
@@ -1057,7 +1055,10 @@ class DotGeneralRaw:
         bwd_memo[memo_key] = (s32, scale_list, sdt)
     qt = aqt_tensor.QTensor(qvalue=qv, scale=scale_list, scale_t=None, bias=[], dequant_dtype=dtype,
                             container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
-    quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))
+    if getattr(quantizer.numerics, 'clip_gradient', False):
+      quant_grad = aqt_quantizer.clip_gradient_later(quantizer.numerics, x, scale_list)
+    else:
+      quant_grad = functools.partial(quantizer.numerics.vjp_bwd, (None,))
     return q, s32, sdt, qt, quant_grad
 
 

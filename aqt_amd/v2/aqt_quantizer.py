@@ -145,17 +145,18 @@ class Quantizer:
       return qt, None
     spec = self.numerics.kernel_spec()
     if (spec is None or qt.bias or qt.tiling_state is not None or len(qt.scale) != 1
-        or qt.sparsity_mask is not None or getattr(self.numerics, 'clip_gradient', False)
-        or not x.is_floating_point()):
+        or qt.sparsity_mask is not None or not x.is_floating_point()):
       return self._calculate_qvalue_stepwise(x, qt)
     try:
-      return self._calculate_qvalue_kernel(x, qt, spec)
+      out, quant_grad = self._calculate_qvalue_kernel(x, qt, spec)
     except lowering.NotFused:
       return self._calculate_qvalue_stepwise(x, qt)
+    if getattr(self.numerics, 'clip_gradient', False):
+      quant_grad = clip_gradient_later(self.numerics, x, qt.scale)
+    return out, quant_grad
 
   def _calculate_qvalue_stepwise(self, x, qt: aqt_tensor.QTensor):
-    """No fused scale-and-round kernel for this case (or the scaled tensor has to be kept for
-    clip_gradient): scale, then the numerics' own forward."""
+    """No fused scale-and-round kernel for this case: scale, then the numerics' own forward."""
     q_scaled = qt.quant(x)
     x_q, res = self.numerics.vjp_fwd(q_scaled.qvalue, self.context)
     q_scaled.qvalue = x_q
@@ -178,6 +179,18 @@ class Quantizer:
     qvalue = lowering.logical_from_brk(_typed(q, spec['out_dtype']), v)
     out = qt.replace(qvalue=qvalue, container_dtype=utils.int4 if spec['out_dtype'] == L.I4 else None)
     return out, functools.partial(self.numerics.vjp_bwd, (None,))
+
+
+def clip_gradient_later(numerics, x, scale_list):
+  """The gradient function of a numerics with clip_gradient for an input the fused kernel quantized:
+  the kernel keeps no scaled copy of x (the residual the reference's vjp_bwd reads,
+  numerics/int_numerics.py:113-125), so the scaled input is recomputed from x and the scale
+  when the backward pass asks, with QTensor.quant's own arithmetic (aqt_tensor.py:125-159)."""
+  def quant_grad(grad):
+    scaled = aqt_tensor.QTensor(qvalue=None, scale=scale_list, scale_t=None, bias=[],
+                                dequant_dtype=x.dtype).quant(x.detach()).qvalue
+    return numerics.vjp_bwd((scaled,), grad)
+  return quant_grad
 
 
 def _typed(q: torch.Tensor, out_dtype: int) -> torch.Tensor:

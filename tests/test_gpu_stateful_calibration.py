@@ -126,12 +126,12 @@ class _CountingAbsMax(calibration.AbsMaxCalibration):
 
 
 def test_fallback_after_a_fused_attempt_calibrates_once(gpu):
-  """The lhs calibrates step by step inside the fused attempt; the rhs (clip_gradient numerics)
+  """The lhs calibrates step by step inside the fused attempt; the rhs (numerics without the clip)
   then turns the call over to the step-by-step path, which must take the lhs scale over
   instead of calibrating a second time (the reference calibrates once per call)."""
   dg = aqt.dot_general_raw_make(8, 8)
   dg.dg_quantizer.lhs.calibration = _CountingAbsMax
-  dg.dg_quantizer.rhs.numerics.clip_gradient = True  # no fused form: found out after the lhs is done
+  dg.dg_quantizer.rhs.numerics.clip = False  # no fused form: found out after the lhs is done
   dg.dg_quantizer.lhs._calibrator = None
   dg.dg_quantizer.rhs._calibrator = None
   dg.dg_quantizer.init_calibration()

@@ -20,6 +20,7 @@ from aqt_amd.v2 import calibration
 from aqt_amd.v2 import config
 from aqt_amd.v2 import utils
 from oracle import aqt_ref as R
+from oracle import numerics as nm
 from oracle import prng
 from tests import gpu_util as U
 
@@ -266,32 +267,39 @@ def test_custom_dg_quantizer(gpu):
   np.testing.assert_array_equal(_np(out), want)
 
 
-def test_clip_gradient(gpu):
+@pytest.mark.parametrize('dt', ['f32', 'bf16'])
+def test_clip_gradient(gpu, dt, monkeypatch):
   """IntSymmetric.clip_gradient with a clipping calibration (int_numerics.py:113-125): the
-  gradient is zeroed where the scaled input fell outside the clip bound."""
-  dt = 'f32'
+  gradient is the unclipped one times the mask of scaled inputs inside the clip bound, the scaled
+  input being x * (1 / scale) in x's dtype (aqt_tensor.py:151-155).  The call stays on the fused
+  quantize and contraction kernels; the mask is made in the backward pass."""
   lhs, rhs, g = U.rand((32, 64), dt, 1, outliers=True), U.rand((64, 16), dt, 2), U.rand((32, 16), dt, 3)
   cfg = config.fully_quantized(use_fwd_quant=False, use_stochastic_rounding=False)
   config.set_absmax_calib_scale(cfg, 0.25)
-  cfg.fwd.dg_quantizer.lhs.numerics.clip_gradient = True
+  assert cfg.fwd.dg_quantizer.lhs.numerics.clip_gradient and cfg.fwd.dg_quantizer.rhs.numerics.clip_gradient
   cfg = config.set_context(cfg, None, None)
-  L = U.to_dev(lhs, dt, gpu).requires_grad_(True)
-  Rr = U.to_dev(rhs, dt, gpu).requires_grad_(True)
-  out, (lqt, _) = cfg.dg_core(L, Rr, None, None, MATMUL)
+
+  def no_step_by_step(self, *a, **k):
+    raise AssertionError('the step-by-step path was taken')
+  monkeypatch.setattr(aqt.DotGeneralRaw, '_unfused_call', no_step_by_step)
+  Lh = U.to_dev(lhs, dt, gpu).requires_grad_(True)
+  Rh = U.to_dev(rhs, dt, gpu).requires_grad_(True)
+  out, (lqt, rqt) = cfg.dg_core(Lh, Rh, None, None, MATMUL)
   out.backward(U.to_dev(g, dt, gpu))
-  scaled = lhs / _np(lqt.scale[0])
-  clipped = np.abs(scaled) > 127.0 + 1e-3
-  inside = np.abs(scaled) < 127.0 - 1e-3
-  assert clipped.any() and inside.any()
-  got = _np(L.grad)
-  assert (got[clipped] == 0).all()
   cfg2 = copy.deepcopy(cfg)
-  cfg2.fwd.dg_quantizer.lhs.numerics.clip_gradient = False
+  for q in (cfg2.fwd.dg_quantizer.lhs, cfg2.fwd.dg_quantizer.rhs):
+    q.numerics.clip_gradient = False
   L2 = U.to_dev(lhs, dt, gpu).requires_grad_(True)
-  out2, _ = cfg2.dg_core(L2, U.to_dev(rhs, dt, gpu), None, None, MATMUL)
+  R2 = U.to_dev(rhs, dt, gpu).requires_grad_(True)
+  out2, _ = cfg2.dg_core(L2, R2, None, None, MATMUL)
   out2.backward(U.to_dev(g, dt, gpu))
   np.testing.assert_array_equal(_np(out), _np(out2))
-  np.testing.assert_array_equal(got[inside], _np(L2.grad)[inside])
+  for x, qt, got, plain in ((lhs, lqt, Lh.grad, L2.grad), (rhs, rqt, Rh.grad, R2.grad)):
+    inv = nm.cast(np.float32(1.0) / _np(qt.scale[0]), dt)
+    scaled = nm.cast(nm.cast(x, dt) * inv, dt)
+    inside = np.abs(scaled) <= 127.0
+    assert (~inside).any() and inside.any()
+    np.testing.assert_array_equal(_np(got), _np(plain) * inside)
 
 
 def test_mid_quantization_known_answer(gpu):
