@@ -111,6 +111,7 @@ SYMBOLS = {
     'aqtx_gemm_i8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8_k_slices': (ctypes.c_int, [ctypes.POINTER(GemmPlan)]),
     'aqtx_gemm_fp8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    'aqtx_gemm_weight_only': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp]),
     'aqtx_decode_i8': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp,
                                       _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),

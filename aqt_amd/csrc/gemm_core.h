@@ -38,6 +38,7 @@ struct MmaI8 {
   using Frag = v4i;
   static constexpr int kChunks = 1;   // v_mfma_i32_32x32x32_i8: 32 k per MFMA, 16 per lane
   static constexpr bool kIntAcc = true;
+  static constexpr bool kWidenB = false;
   static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, c, 0, 0, 0);
   }
@@ -53,12 +54,42 @@ struct MmaF8 {
   using Frag = v8i;
   static constexpr int kChunks = 2;   // 64 k per MFMA, 32 per lane
   static constexpr bool kIntAcc = false;
+  static constexpr bool kWidenB = false;
   // x comes from the B tile, y from the A tile (see mfma_step).  Zero scale operands select the
   // unscaled form of the instruction (v_mfma_f32_32x32x64_f8f6f4).
   static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, FMT_B, FMT_A, 0, 0, 0, 0);
   }
 };
+
+// Weight-only contraction: A holds bf16 values, B int8 values that are widened to bf16 (exactly) on their
+// way to LDS, where both tiles then hold 16-byte chunks of 8 bf16.  v_mfma_f32_32x32x16_bf16, float sums.
+struct MmaBf16W8 {
+  typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+  using Acc = v16f;
+  using AccScalar = float;
+  using Frag = v4i;
+  static constexpr int kChunks = 1;   // 16 k per MFMA, 8 per lane: 16 bytes
+  static constexpr bool kIntAcc = false;
+  static constexpr bool kWidenB = true;
+  static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, x), __builtin_bit_cast(v8bf, y), c, 0, 0, 0);
+  }
+};
+
+// 16 int8 values (k order) -> 16 bf16 values in two 16-byte chunks.  Every int8 value is a bf16 value, so
+// the upper half of its float32 form is the result.
+__device__ __forceinline__ void widen_i8x16_bf16(const v4i x4, v4i& lo, v4i& hi) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int x = x4[d];
+    const uint32_t f0 = __float_as_uint((float)(int8_t)x), f1 = __float_as_uint((float)(int8_t)(x >> 8));
+    const uint32_t f2 = __float_as_uint((float)(int8_t)(x >> 16)), f3 = __float_as_uint((float)(x >> 24));
+    const int w0 = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u), w1 = (int)__builtin_amdgcn_perm(f3, f2, 0x07060302u);
+    if (d < 2) { lo[2 * d] = w0; lo[2 * d + 1] = w1; }
+    else { hi[2 * (d - 2)] = w0; hi[2 * (d - 2) + 1] = w1; }
+  }
+}
 
 struct GemmArgs {
   const uint8_t* a;
@@ -751,5 +782,7 @@ int launch_conv_i8_mid(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, const
                        const float* row_scale, const float* col_scale, void* c, hipStream_t st);
 int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                         const float* col_scale, void* c, float* acc_out, hipStream_t st);
+int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* col_scale, void* c,
+                                hipStream_t st);
 
 }  // namespace aqtx

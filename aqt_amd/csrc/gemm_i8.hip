@@ -155,3 +155,27 @@ extern "C" int aqtx_conv_i8(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, 
   AQTX_REQUIRE(((uintptr_t)c % esz) == 0, "aqtx_conv_i8: output is not element aligned");
   return launch_conv_i8_mid(w, p, x, b, row_scale, col_scale, c, reinterpret_cast<hipStream_t>(stream));
 }
+
+extern "C" int aqtx_gemm_weight_only(const aqtx_gemm_plan* p, const void* a, const void* b, const float* col_scale,
+                                     void* c, void* stream) {
+  clear_error();
+  const char* who = "aqtx_gemm_weight_only";
+  AQTX_REQUIRE(p != nullptr, "%s: plan is NULL", who);
+  AQTX_REQUIRE(p->batch >= 0 && p->m >= 0 && p->n >= 0 && p->k >= 0, "%s: negative shape", who);
+  AQTX_REQUIRE(p->a_dtype == AQTX_BF16 && (p->b_dtype == AQTX_I8 || p->b_dtype == AQTX_I4),
+               "%s: a must be bf16 and b int8 containers (got %d, %d)", who, p->a_dtype, p->b_dtype);
+  AQTX_REQUIRE(p->out_dtype == AQTX_BF16 && p->dequant_dtype == AQTX_BF16, "%s: out_dtype and dequant_dtype must be bf16", who);
+  AQTX_REQUIRE(is_float_dtype(p->col_scale_dtype), "%s: col_scale_dtype must be bf16 or f32", who);
+  AQTX_REQUIRE(p->group_offsets == nullptr && p->k_split <= 1, "%s: no ragged batches, no slices of k", who);
+  AQTX_REQUIRE(p->lda >= p->k && p->ldb >= p->k && p->ldc >= p->n, "%s: leading dimension smaller than the row length", who);
+  AQTX_REQUIRE(p->k > 0 && p->k % 16 == 0, "%s: k = %lld must be a positive multiple of 16", who, (long long)p->k);
+  AQTX_REQUIRE(p->lda % 8 == 0 && p->stride_a % 8 == 0 && p->ldb % 16 == 0 && p->stride_b % 16 == 0,
+               "%s: rows of a and b must start 16-byte aligned", who);
+  AQTX_REQUIRE(p->batch <= 65535 && p->m <= (int64_t)65535 * 128 && (p->m + 127) / 128 * ((p->n + 127) / 128) < (1ll << 31),
+               "%s: shape too large for one launch", who);
+  AQTX_REQUIRE(p->lda * 256 < (1ll << 31) && p->ldb * 128 < (1ll << 31), "%s: leading dimension too large for 32-bit tile offsets", who);
+  if (p->batch == 0 || p->m == 0 || p->n == 0) return 0;
+  AQTX_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "%s: NULL buffer", who);
+  AQTX_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 2) == 0, "%s: a and b must be 16-byte aligned", who);
+  return launch_gemm_weight_only_mid(p, a, b, col_scale, c, reinterpret_cast<hipStream_t>(stream));
+}

@@ -20,7 +20,9 @@ constexpr int TM = 128, TN = 128;
 constexpr int kRow = BK + 16;
 constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile;  // 36 KiB
 
-// MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: B holds int4 values two per byte (see gemm_kernel's BPACK).
+// MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
+// int4 values two per byte (see gemm_kernel's BPACK), or, with MmaBf16W8, int8 values that become bf16 (A then
+// holds bf16 values, and GemmArgs::k, lda and stride_a count its bytes).
 // SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then; integer sums only).
 // CONV: A is a convolution input read in place (GemmArgs::conv): the window gather that would otherwise be
 // materialised (features % 128 == 0, so a 128-byte stage lies inside one tap).
@@ -29,7 +31,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void gemm_mid_kernel(const GemmArgs g_in) {
   static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
   static_assert(!CONV || (MMA::kIntAcc && !PACKED && !SLAB), "the convolution reads int8 bytes, whole K");
-  static_assert(MMA::kIntAcc || (!SLAB && !PACKED && EPI != 3), "fp8 operands: float sums, whole K, bytes as they are");
+  static_assert(MMA::kIntAcc || (!SLAB && PACKED == MMA::kWidenB && EPI != 3), "float sums: whole K; fp8 bytes as they are");
   using Acc = typename MMA::Acc;
   using AccScalar = typename MMA::AccScalar;
   using Frag = typename MMA::Frag;
@@ -129,7 +131,8 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
     if constexpr (PACKED) {
       v4i lo, hi;
-      unpack_i4x32(stg[NLA], lo, hi, g.a_even_odd8);
+      if constexpr (MMA::kWidenB) widen_i8x16_bf16(stg[NLA], lo, hi);
+      else unpack_i4x32(stg[NLA], lo, hi, g.a_even_odd8);
       *reinterpret_cast<v4i*>(st + st_b) = lo;
       *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
     } else {
@@ -208,7 +211,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
         if (nn >= g.n) continue;
         int v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[ni][4 * q + e] >> 4 : acc[ni][4 * q + e];  // exact: multiples of 16
+        for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[ni][4 * q + e] >> 4 : acc[ni][4 * q + e];  // exact: multiples of 16 (SLAB: int4)
         if (vec) *reinterpret_cast<int4*>(dst + nn) = make_int4(v[0], v[1], v[2], v[3]);
         else for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[nn + e] = v[e];
       }
@@ -232,7 +235,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
         AccScalar v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if constexpr (PACKED) v[e] = acc[ni][4 * q + e] >> 4;
+          if constexpr (PACKED && MMA::kIntAcc) v[e] = acc[ni][4 * q + e] >> 4;
           else v[e] = acc[ni][4 * q + e];
         }
         if (g.acc_out != nullptr) {  // 32-bit patterns, int32 or float
@@ -436,6 +439,23 @@ int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, c
   else if (a5 && !b5) launch_mid_fp8<MmaF8<1, 0>>(g, epi, grid, st);
   else launch_mid_fp8<MmaF8<1, 1>>(g, epi, grid, st);
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<fp8>");
+  return 0;
+}
+
+// Weight-only contraction (bf16 A, int8 B widened in registers, float sums) on the 128 x 128 tiles.  The
+// epilogue is QTensor.dequant with the rhs scale alone: the sum in bf16, times the column scale in the
+// promoted dtype, cast to bf16 (a missing row scale multiplies by one and rounds nothing).
+int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* col_scale, void* c,
+                                hipStream_t st) {
+  GemmArgs g = make_gemm_args(p, a, b, nullptr, col_scale, c, nullptr);
+  g.k *= 2; g.lda *= 2; g.stride_a *= 2;  // A in bytes
+  g.col_first = 0;
+  g.tiles_m = (int)((p->m + TM - 1) / TM);
+  g.tiles_n = (int)((p->n + TN - 1) / TN);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
+  if (p->col_scale_dtype == AQTX_BF16) gemm_mid_kernel<MmaBf16W8, 0, false, true, false><<<grid, 512, 0, st>>>(g);
+  else gemm_mid_kernel<MmaBf16W8, 4, false, true, false><<<grid, 512, 0, st>>>(g);
+  AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<weight only>");
   return 0;
 }
 

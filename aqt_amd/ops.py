@@ -334,6 +334,31 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
   return torch.clamp(offs, max=m)
 
 
+def gemm_weight_only(a: torch.Tensor, b: torch.Tensor, col_scale: torch.Tensor, *, col_scale_dtype=torch.float32,
+                     b_dtype: int = L.I8):
+  """Weight-only contraction C[b] = bf16(bf16(A[b] @ float(B[b])^T) * col_scale[b]) for bf16 A [batch, m, k] that
+  stays unquantized and int8 B [batch, n, k] (k contiguous in both), any m; `col_scale` is float32 [batch, n]
+  holding values of `col_scale_dtype`.  float32 sums; the weight is never copied as bf16."""
+  _require_gpu(a, b, col_scale)
+  assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == b.shape[2] and a.shape[0] == b.shape[0]
+  assert a.dtype == torch.bfloat16 and b.dtype == torch.int8 and a.stride(2) == 1 and b.stride(2) == 1
+  batch, m, k = a.shape
+  n = b.shape[1]
+  assert col_scale.dtype == torch.float32 and col_scale.is_contiguous() and tuple(col_scale.shape) == (batch, n)
+  c = torch.empty((batch, m, n), dtype=torch.bfloat16, device=a.device)
+  plan = L.GemmPlan()
+  plan.batch, plan.m, plan.n, plan.k = batch, m, n, k
+  plan.lda, plan.ldb, plan.ldc = a.stride(1), b.stride(1), n
+  plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), b.stride(0), m * n
+  plan.a_dtype, plan.b_dtype = L.BF16, b_dtype
+  plan.out_dtype = plan.dequant_dtype = plan.row_scale_dtype = L.BF16
+  plan.col_scale_dtype = aqtx_dtype(col_scale_dtype)
+  plan.col_scale_stride_b = n
+  with _timed('gemm'):
+    L.check(L.lib().aqtx_gemm_weight_only(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(col_scale), _ptr(c), _stream()))
+  return c
+
+
 def decode_weight_only(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, w_scale_dtype=torch.float32,
                        w_dtype: int = L.I8, w_layout: int = L.W_ROWS, out_dtype=None, tuning: int = 0):
   """Weight-only serving contraction out = dequant(x @ float(w_q)^T) for bf16 x [m <= 64, k] that stays

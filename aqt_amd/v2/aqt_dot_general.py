@@ -74,6 +74,11 @@ _FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
 # kept for as long as the quantized tensor lives and stays unchanged (its version counter).
 _PROMOTED_RHS = {}  # id(rhs) -> (key, promoted [b, k, n] copy)
 
+# Weight-only serving above 64 lhs rows: True = the library's bf16 product on the kept float copy of the
+# weight (2 bytes per weight element more, the faster of the two on most shapes); False = the weight-only
+# contraction kernel, which widens the int8 bytes in registers and keeps no float copy.
+WEIGHT_ONLY_FLOAT_COPY = True
+
 
 def _promoted_rhs(rhs, perm, shape, common):
   if rhs.dtype == common or rhs.numel() < (1 << 20) or rhs.requires_grad:
@@ -923,10 +928,11 @@ class DotGeneralRaw:
 
   def _serve_weight_only(self, lhs, dq, lhs_qt, rhs_arr, rhs_qt, dimension_numbers, prescale_t, out_transpose_axes,
                          dequant_dtype):
-    """Serving with an unquantized bf16 lhs of at most 64 rows and a frozen int8 / int4 rhs with one scale per
-    output channel: the weight-only kernel (the weight streamed once, converted to bf16 in registers; the
-    reference promotes the whole weight to bf16 and contracts in float, aqt_dot_general.py:843-958).  Returns
-    None when the call does not have that shape."""
+    """Serving with an unquantized bf16 lhs and a frozen int8 / int4 rhs with one scale per output channel:
+    the weight-only kernels (the weight converted to bf16 in registers; the reference promotes the whole
+    weight to bf16 and contracts in float, aqt_dot_general.py:843-958): the streaming kernel up to 64 lhs
+    rows, above that the tiled one unless WEIGHT_ONLY_FLOAT_COPY.  Returns None when the call does not
+    have that shape."""
     if (rhs_qt is None or not rhs_qt.is_full() or lhs_qt is not None or prescale_t is not None
         or out_transpose_axes is not None or self.dot_general is not lax_dot_general or self.local_aqt is not None
         or self.rhs.dequant_mode != DequantMode.OUTPUT or lhs.dtype != torch.bfloat16
@@ -948,15 +954,20 @@ class DotGeneralRaw:
       return None
     M, K, N = lv.R, lv.K, rv.R
     packed = rhs_qt.container_dtype is utils.int4 and K % 32 == 0
-    if M == 0 or M > 64 or K == 0 or K % 16 != 0 or N == 0 or N * K >= 2 ** 31:
+    if M == 0 or (M > 64 and WEIGHT_ONLY_FLOAT_COPY) or K == 0 or K % 16 != 0 or N == 0 or N * K >= 2 ** 31:
       return None
     w_scale = rhs_qt.scale[0]
     if lowering.view_operand(w_scale, [], rra, rca).mem.numel() != N:
       return None
-    w_fragments = _kernel_layout_of(rhs_qt.qvalue, rv, pack_int4=packed, fragments=True)
-    out = ops.decode_weight_only(
-        lv.mem[0], w_fragments, _scale_vector_f32(w_scale, [], rra, rca), w_scale_dtype=w_scale.dtype,
-        w_dtype=L.I4P if packed else L.I4 if rhs_qt.container_dtype is utils.int4 else L.I8, w_layout=L.W_FRAGMENTS)
+    if M <= 64:
+      w_fragments = _kernel_layout_of(rhs_qt.qvalue, rv, pack_int4=packed, fragments=True)
+      out = ops.decode_weight_only(
+          lv.mem[0], w_fragments, _scale_vector_f32(w_scale, [], rra, rca), w_scale_dtype=w_scale.dtype,
+          w_dtype=L.I4P if packed else L.I4 if rhs_qt.container_dtype is utils.int4 else L.I8, w_layout=L.W_FRAGMENTS)
+    else:
+      w_rows = rv.mem if rv.k_last and not rv.copied else _kernel_layout_of(rhs_qt.qvalue, rv)
+      out = ops.gemm_weight_only(lv.mem, w_rows, _scale_vector_f32(w_scale, [], rra, rca).reshape(1, N),
+                                 col_scale_dtype=w_scale.dtype)
     out = out.reshape([lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
     lhs_qt_out = aqt_tensor.QTensor(qvalue=lhs, scale=[], scale_t=None, bias=[], dequant_dtype=lhs.dtype)
     rhs_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON

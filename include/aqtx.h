@@ -204,6 +204,21 @@ int aqtx_gemm_i8(const aqtx_gemm_plan* plan, const void* a, const void* b,
 int aqtx_gemm_i8_k_slices(const aqtx_gemm_plan* plan);
 
 /*
+ * aqtx_gemm_weight_only: c[m, n] = bf16(bf16(sum_k a[m, k] * float(b[n, k])) * col_scale[n]) for bf16
+ * activations that are NOT quantized and an int8 (or int4 in int8 containers) weight, any m.  Replaces
+ * _qtensor_dot_general with an unquantized lhs (aqt/jax/v2/aqt_dot_general.py:843-958: the quantized rhs is
+ * promoted to bf16, lax.dot_general contracts in float) followed by QTensor.dequant with the rhs scale
+ * (aqt_tensor.py:161-200), without the bf16 copy of the weight: the int8 bytes are widened (exactly) on their
+ * way into v_mfma_f32_32x32x16_bf16.  Float32 sums: agrees with the reference's float contraction to summation
+ * order, not bit for bit.  Of the plan: batch, m, n, k, lda, ldb (elements), ldc, strides, a_dtype (AQTX_BF16),
+ * b_dtype (AQTX_I8 | AQTX_I4), out_dtype = dequant_dtype = AQTX_BF16, col_scale_dtype, col_scale_stride_b are
+ * read.  k % 16 == 0, lda % 8 == 0, ldb % 16 == 0, a and b 16-byte aligned.  For m <= 64 aqtx_decode_weight_only
+ * streams the weight faster.
+ */
+int aqtx_gemm_weight_only(const aqtx_gemm_plan* plan, const void* a, const void* b, const float* col_scale,
+                          void* c, void* stream);
+
+/*
  * aqtx_gemm_fp8: fp8 x fp8 -> float32 MFMA contraction (a_dtype/b_dtype select
  * e4m3fn or e5m2 per operand), same epilogue as aqtx_gemm_i8.  Replaces the
  * same reference lines with preferred_element_type=float32

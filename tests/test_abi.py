@@ -211,6 +211,40 @@ def test_weight_only_decode_null_and_empty():
   assert L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan(n=0)), None, None, None, None, None) == 0
 
 
+def _woplan(**kw):
+  p = L.GemmPlan()
+  p.batch, p.m, p.n, p.k = 1, 256, 256, 512
+  p.lda = p.ldb = 512
+  p.ldc = 256
+  p.a_dtype, p.b_dtype = L.BF16, L.I8
+  p.out_dtype = p.dequant_dtype = p.row_scale_dtype = L.BF16
+  p.col_scale_dtype = L.F32
+  for k, v in kw.items():
+    setattr(p, k, v)
+  return p
+
+
+@pytest.mark.parametrize('kw,needle', [
+    (dict(a_dtype=L.I8), 'a must be bf16'),
+    (dict(b_dtype=L.I4P), 'a must be bf16'),
+    (dict(out_dtype=L.F32), 'must be bf16'),
+    (dict(k=520, lda=520, ldb=528), 'multiple of 16'),
+    (dict(lda=516), '16-byte aligned'),
+    (dict(ldb=256), 'leading dimension'),
+    (dict(k_split=2), 'slices'),
+    (dict(m=-1), 'negative'),
+])
+def test_weight_only_gemm_plan_validation(kw, needle):
+  msg = _err(L.lib().aqtx_gemm_weight_only(ctypes.byref(_woplan(**kw)), FAKE, FAKE, FAKE, FAKE, None))
+  assert needle in msg, msg
+
+
+def test_weight_only_gemm_null_and_empty():
+  assert 'NULL' in _err(L.lib().aqtx_gemm_weight_only(ctypes.byref(_woplan()), None, FAKE, FAKE, FAKE, None))
+  assert 'plan is NULL' in _err(L.lib().aqtx_gemm_weight_only(None, FAKE, FAKE, FAKE, FAKE, None))
+  assert L.lib().aqtx_gemm_weight_only(ctypes.byref(_woplan(m=0)), None, None, None, None, None) == 0
+
+
 def _ggplan(**kw):
   p = L.GroupedGemmPlan()
   p.m, p.n, p.k, p.group = 64, 128, 512, 128

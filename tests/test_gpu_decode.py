@@ -361,27 +361,30 @@ def test_weight_only_decode_within_float_summation_error(gpu, m, n, k, w_sdt, pa
 
 
 @pytest.mark.gpu
-def test_weight_only_serving_takes_the_kernel(gpu):
-  """A float lhs of at most 64 rows against a frozen int8 rhs goes to the weight-only kernel; more rows (and
-  anything else) take the float product on the promoted weight.  Same numbers to float summation order."""
+def test_weight_only_serving_takes_the_kernel(gpu, monkeypatch):
+  """A float lhs of at most 64 rows against a frozen int8 rhs goes to the streaming weight-only kernel; more rows
+  take the float product on the promoted weight, or, with WEIGHT_ONLY_FLOAT_COPY off, the tiled weight-only
+  kernel.  Same numbers to float summation order."""
   from aqt_amd.v2 import aqt_dot_general as aqt, config
   dt = 'bf16'
   MATMUL = (((1,), (0,)), ((), ()))
   cfg = config.set_context(aqt.dot_general_make(None, 8), None, None)
   w = U.to_dev(U.rand((1024, 520), dt, 3, 0.05), dt, gpu)
   x_small, x_large = U.to_dev(U.rand((24, 1024), dt, 1), dt, gpu), U.to_dev(U.rand((80, 1024), dt, 2), dt, gpu)
+  calls = []
+  for name in ('decode_weight_only', 'gemm_weight_only'):
+    real = getattr(ops, name)
+    monkeypatch.setattr(ops, name, lambda *a, _real=real, _name=name, **k: (calls.append(_name), _real(*a, **k))[1])
   with torch.no_grad():
     _, (_, wq) = cfg.dg_core(x_small, w, None, None, MATMUL)
-    calls = []
-    real = ops.decode_weight_only
-    ops.decode_weight_only = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
-    try:
-      out_small, (lqt, _) = cfg.dg_core(x_small, torch.zeros_like(w), None, wq, MATMUL)
-      out_large, _ = cfg.dg_core(x_large, torch.zeros_like(w), None, wq, MATMUL)
-    finally:
-      ops.decode_weight_only = real
-  assert len(calls) == 1 and lqt.qvalue is x_small and lqt.scale == []
+    out_small, (lqt, _) = cfg.dg_core(x_small, torch.zeros_like(w), None, wq, MATMUL)
+    out_large, _ = cfg.dg_core(x_large, torch.zeros_like(w), None, wq, MATMUL)
+    assert calls == ['decode_weight_only'] and lqt.qvalue is x_small and lqt.scale == []
+    monkeypatch.setattr(aqt, 'WEIGHT_ONLY_FLOAT_COPY', False)
+    out_large_kernel, _ = cfg.dg_core(x_large, torch.zeros_like(w), None, wq, MATMUL)
+    assert calls == ['decode_weight_only', 'gemm_weight_only']
   wf = wq.qvalue.float() * wq.scale[0].float()
-  for out, x in ((out_small, x_small), (out_large, x_large)):
+  for out, x in ((out_small, x_small), (out_large, x_large), (out_large_kernel, x_large)):
     want = (x.float() @ wf).cpu().numpy()
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2.0 ** -6, atol=2.0 ** -6 * np.abs(want).max())
+  assert (out_large_kernel != out_large).float().mean() < 0.02  # both round a float32 sum to bf16

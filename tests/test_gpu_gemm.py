@@ -326,3 +326,50 @@ def test_fp8_tile_sizes_give_the_same_bits(gpu, monkeypatch):
     outs.append(ops.gemm(a.to(gpu), b.to(gpu), row_scale=None, col_scale=None, out_dtype=torch.float32,
                          a_dtype=L.E4M3, b_dtype=L.E5M2))
   assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32))
+
+
+# ---- weight-only contraction (bf16 lhs, int8 rhs widened in registers; float32 sums: tolerance, not bits) ----
+@pytest.mark.gpu
+@pytest.mark.parametrize('w_sdt', ['bf16', 'f32'])
+@pytest.mark.parametrize('batch,m,n,k', [(1, 65, 128, 64), (1, 200, 328, 1040), (2, 129, 130, 272), (1, 1024, 512, 4096),
+                                         (1, 3, 5, 16)])
+def test_weight_only_gemm_within_float_summation_error(gpu, batch, m, n, k, w_sdt):
+  """c = bf16(bf16(sum_k a b) * scale), float32 sums in the kernel's own order.  Tolerance, stated: against
+  the exact sum (float64; a bf16 times an int8 is exact), a float32 sum in any order is off by less than
+  d = k * 2^-24 * sum_k |a b|; the later steps are monotone (positive scales), so every output lies between
+  those steps applied to exact - d and exact + d, and 99 % of the outputs equal them applied to the exact sum.
+  A transposed operand, a dropped k chunk or a wrong scale index fails both."""
+  rng = np.random.default_rng(7)
+  a = nm.to_bf16(rng.standard_normal((batch, m, k), dtype=np.float32))
+  b = rng.integers(-127, 128, (batch, n, k)).astype(np.int8)
+  ws = nm.cast(np.abs(rng.standard_normal((batch, n)).astype(np.float32)) * np.float32(2e-3) + np.float32(1e-4), w_sdt)
+  exact = np.einsum('bmk,bnk->bmn', a.astype(np.float64), b.astype(np.float64))
+  slack = k * 2.0 ** -24 * np.einsum('bmk,bnk->bmn', np.abs(a).astype(np.float64), np.abs(b).astype(np.float64))
+
+  def later_steps(total):
+    prod = nm.to_bf16(total.astype(np.float32)).astype(np.float64) * ws.astype(np.float64)[:, None, :]
+    return nm.to_bf16(nm.cast(prod.astype(np.float32), w_sdt)).astype(np.float64)
+
+  want, low, high = later_steps(exact), later_steps(exact - slack), later_steps(exact + slack)
+  got = ops.gemm_weight_only(torch.from_numpy(a).to(torch.bfloat16).to(gpu), torch.from_numpy(b).to(gpu),
+                             torch.from_numpy(ws.astype(np.float32)).to(gpu), col_scale_dtype=U.TORCH_DT[w_sdt])
+  got = got.float().cpu().numpy().astype(np.float64)
+  assert ((low <= got) & (got <= high)).all(), np.argwhere((got < low) | (got > high))[:8]
+  assert (got == want).mean() >= 0.99
+
+
+@pytest.mark.gpu
+def test_weight_only_gemm_strided_operands(gpu):
+  """Rows of a and b further apart than k (views into wider tensors) and the few-rows kernel's answer:
+  both kernels round alike except for summation order."""
+  rng = np.random.default_rng(8)
+  m, n, k = 48, 272, 528
+  a_wide = torch.from_numpy(nm.to_bf16(rng.standard_normal((1, m, k + 24), dtype=np.float32))).to(torch.bfloat16).to(gpu)
+  b_wide = torch.from_numpy(rng.integers(-127, 128, (1, n, k + 48)).astype(np.int8)).to(gpu)
+  a, b = a_wide[:, :, 8:8 + k], b_wide[:, :, 16:16 + k]
+  ws = torch.rand(1, n, device=gpu) * 0.01 + 1e-4
+  got = ops.gemm_weight_only(a, b, ws)
+  other = ops.decode_weight_only(a[0].contiguous(), b[0].contiguous(), ws[0].contiguous())
+  ref = (a[0].float() @ b[0].float().T).to(torch.bfloat16).float() * ws[0]
+  assert torch.equal(got[0], other) or (got[0] != other).float().mean() < 0.01
+  torch.testing.assert_close(got[0].float(), ref, rtol=2.0 ** -7, atol=1e-6)
