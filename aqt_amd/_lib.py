@@ -55,6 +55,7 @@ class GemmPlan(ctypes.Structure):
       ('a_k_order', ctypes.c_int32),
       ('k_split', ctypes.c_int32),
       ('k_split_workspace', ctypes.c_void_p), ('k_split_workspace_bytes', ctypes.c_int64),
+      ('b_layout', ctypes.c_int32),
   ]
 
 

@@ -111,6 +111,10 @@ struct GemmArgs {
   // A with B[b] into the same rows of one flat C (m is then an upper bound of a group's rows).
   const int32_t* group_offsets;
   int a_even_odd8;  // packed int4 B only: A's bytes of every 8 k are stored as k 0,2,4,6,1,3,5,7
+  // B in the fragment order of aqtx_tile_weight (batch 1): blocks of 16 rows, b_steps KiB each, a KiB holding
+  // 64 bytes of each of the 16 rows (lane r + 16 c of the KiB = bytes 16 c .. 16 c + 15 of row r); rows past n
+  // and bytes past the row's end are zeros there.
+  int b_frag, b_steps;
   // Split K (gemm_mid_kernel): workgroup z of the grid contracts k in [z * k_chunk, (z + 1) * k_chunk) and
   // writes its int32 partial sums to slab z of `slabs` ([k_split][batch][m][n]); dequant_slabs_kernel adds
   // the slabs (integer addition: exact) and dequantizes.

@@ -26,13 +26,19 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
   AQTX_REQUIRE(p->scale_order == AQTX_SCALE_ROW_THEN_COL || p->scale_order == AQTX_SCALE_COL_THEN_ROW,
                "%s: unknown scale_order %d", who, p->scale_order);
   const bool b_packed = !fp8 && p->b_dtype == AQTX_I4P;
-  AQTX_REQUIRE(p->lda >= p->k && p->ldb >= (b_packed ? p->k / 2 : p->k) && p->ldc >= p->n,
+  AQTX_REQUIRE(p->lda >= p->k && (p->b_layout == AQTX_W_FRAGMENTS || p->ldb >= (b_packed ? p->k / 2 : p->k)) && p->ldc >= p->n,
                "%s: leading dimension smaller than the row length", who);
   AQTX_REQUIRE(p->a_k_order == AQTX_K_NATURAL || (p->a_k_order == AQTX_K_EVEN_ODD8 && b_packed),
                "%s: a_k_order must be AQTX_K_NATURAL, or AQTX_K_EVEN_ODD8 with a packed int4 b", who);
   AQTX_REQUIRE(!b_packed || (p->k % 32 == 0 && p->k * (int64_t)(127 * 8 * 16) < (1ll << 31)),
                "%s: a packed int4 b needs k to be a multiple of 32 below 132096, got %lld", who, (long long)p->k);
   AQTX_REQUIRE(p->batch <= 65535 && p->m <= (int64_t)65535 * 256, "%s: shape too large for one launch", who);
+  AQTX_REQUIRE(p->b_layout == AQTX_W_ROWS || (p->b_layout == AQTX_W_FRAGMENTS && !fp8 && p->batch <= 1 &&
+                                              p->group_offsets == nullptr && p->k > 0 && p->k % (b_packed ? 32 : 16) == 0),
+               "%s: b_layout must be AQTX_W_ROWS, or AQTX_W_FRAGMENTS for one int8 / packed int4 weight (batch 1, no "
+               "ragged batches, k a multiple of 16 / 32)", who);
+  AQTX_REQUIRE(p->b_layout == AQTX_W_ROWS || ((p->n + 15) / 16) * (((b_packed ? p->k / 2 : p->k) + 63) / 64) * 1024 < (1ll << 31),
+               "%s: fragment-ordered weight larger than 2 GiB", who);
   return 0;
 }
 
@@ -63,8 +69,10 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   const bool b_packed = p->b_dtype == AQTX_I4P;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
+  const bool b_frag = p->b_layout == AQTX_W_FRAGMENTS;
   if (!gemm_vector_path_ok(p, a, b)) {
-    AQTX_REQUIRE(!b_packed, "aqtx_gemm_i8: a packed int4 b needs 16-byte aligned operands and leading dimensions");
+    AQTX_REQUIRE(!b_packed && !b_frag,
+                 "aqtx_gemm_i8: a packed int4 or fragment-ordered b needs 16-byte aligned operands and leading dimensions");
     AQTX_REQUIRE(p->group_offsets == nullptr,
                  "aqtx_gemm_i8: ragged batches need 16-byte aligned operands with k and leading dimensions "
                  "multiple of 16");
@@ -85,7 +93,14 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
 
   // few output tiles: the 128 x 128 kernel, with K in slices where that still leaves CUs idle
   AQTX_REQUIRE(p->k_split >= 0 && p->k_split <= 64, "aqtx_gemm_i8: k_split must be in 0..64, got %d", p->k_split);
-  if (int slices = gemm_mid_k_slices(p); slices > 0) {
+  int mid_slices = gemm_mid_k_slices(p);
+  if (b_frag && mid_slices == 0) {
+    // the 256 x 256 kernel reads rows only
+    AQTX_REQUIRE(p->tuning == 0 && (!b_packed || !g.col_first) && p->lda * (int64_t)128 < (1ll << 31),
+                 "aqtx_gemm_i8: a fragment-ordered b takes tuning 0 | 128 (and AQTX_SCALE_ROW_THEN_COL when packed)");
+    mid_slices = 1;
+  }
+  if (int slices = mid_slices; slices > 0) {
     // slices the library chose itself are dropped where the caller lent no (or too small a) workspace
     if (p->k_split == 0 && slices > 1 &&
         (p->k_split_workspace == nullptr || p->k_split_workspace_bytes < (int64_t)slices * p->batch * p->m * p->n * 4))
@@ -167,13 +182,16 @@ extern "C" int aqtx_gemm_weight_only(const aqtx_gemm_plan* p, const void* a, con
   AQTX_REQUIRE(p->out_dtype == AQTX_BF16 && p->dequant_dtype == AQTX_BF16, "%s: out_dtype and dequant_dtype must be bf16", who);
   AQTX_REQUIRE(is_float_dtype(p->col_scale_dtype), "%s: col_scale_dtype must be bf16 or f32", who);
   AQTX_REQUIRE(p->group_offsets == nullptr && p->k_split <= 1, "%s: no ragged batches, no slices of k", who);
-  AQTX_REQUIRE(p->lda >= p->k && p->ldb >= p->k && p->ldc >= p->n, "%s: leading dimension smaller than the row length", who);
+  const bool b_frag = p->b_layout == AQTX_W_FRAGMENTS;
+  AQTX_REQUIRE(p->b_layout == AQTX_W_ROWS || (b_frag && p->batch <= 1), "%s: b_layout must be AQTX_W_ROWS, or AQTX_W_FRAGMENTS with batch 1", who);
+  AQTX_REQUIRE(!b_frag || ((p->n + 15) / 16) * ((p->k + 63) / 64) * 1024 < (1ll << 31), "%s: fragment-ordered weight larger than 2 GiB", who);
+  AQTX_REQUIRE(p->lda >= p->k && (b_frag || p->ldb >= p->k) && p->ldc >= p->n, "%s: leading dimension smaller than the row length", who);
   AQTX_REQUIRE(p->k > 0 && p->k % 16 == 0, "%s: k = %lld must be a positive multiple of 16", who, (long long)p->k);
-  AQTX_REQUIRE(p->lda % 8 == 0 && p->stride_a % 8 == 0 && p->ldb % 16 == 0 && p->stride_b % 16 == 0,
+  AQTX_REQUIRE(p->lda % 8 == 0 && p->stride_a % 8 == 0 && (b_frag || (p->ldb % 16 == 0 && p->stride_b % 16 == 0)),
                "%s: rows of a and b must start 16-byte aligned", who);
   AQTX_REQUIRE(p->batch <= 65535 && p->m <= (int64_t)65535 * 128 && (p->m + 127) / 128 * ((p->n + 127) / 128) < (1ll << 31),
                "%s: shape too large for one launch", who);
-  AQTX_REQUIRE(p->lda * 256 < (1ll << 31) && p->ldb * 128 < (1ll << 31), "%s: leading dimension too large for 32-bit tile offsets", who);
+  AQTX_REQUIRE(p->lda * 256 < (1ll << 31) && (b_frag || p->ldb * 128 < (1ll << 31)), "%s: leading dimension too large for 32-bit tile offsets", who);
   if (p->batch == 0 || p->m == 0 || p->n == 0) return 0;
   AQTX_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "%s: NULL buffer", who);
   AQTX_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 2) == 0, "%s: a and b must be 16-byte aligned", who);

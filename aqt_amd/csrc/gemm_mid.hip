@@ -49,7 +49,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   if constexpr (SLAB) {  // this workgroup's slice of K
     const int64_t kb = (int64_t)blockIdx.z * g.k_chunk;
     g.a += kb;
-    g.b += PACKED ? kb / 2 : kb;
+    g.b += g.b_frag ? (PACKED ? kb / 2 : kb) * 16 : (PACKED ? kb / 2 : kb);  // 64 bytes of a row = one KiB step
     g.k = (g.k - kb) < g.k_chunk ? (g.k - kb) : g.k_chunk;
   }
   const int64_t rows_a = (g.m - m0) < TM ? (g.m - m0) : TM;
@@ -59,8 +59,12 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       ? __builtin_amdgcn_make_buffer_rsrc((void*)g.a, 0, (int)g.conv.x_bytes, kBufferRsrcWord3)
       : __builtin_amdgcn_make_buffer_rsrc((void*)(g.a + bz * g.stride_a + m0 * g.lda), 0,
                                           (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + kb_bytes), kBufferRsrcWord3);
+  const int64_t blocks_b = (rows_b + 15) / 16;  // fragment order: the tile's 16-row blocks, whole
+  const __amdgpu_buffer_rsrc_t rsrc_b = g.b_frag
+      ? __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (n0 / 16) * (int64_t)g.b_steps * 1024), 0,
+                                          (int)(blocks_b * g.b_steps * 1024), kBufferRsrcWord3)
+      : __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0,
+                                          (int)((rows_b - 1) * g.ldb + kb_bytes), kBufferRsrcWord3);
 
   // ---- global -> registers -> LDS (rows past the operand read as zero, and so do the 16-byte chunks
   // past K in the last stage).  A: 16 blocks of 8 rows x 128 B, two per wave.  B unpacked: the same.
@@ -71,12 +75,22 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   constexpr int kOutside = 0x7FFFFFF0;
   v4i stg[NL];
   const int ld_a = (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
-  const int ld_b = PACKED ? (wave * 16 + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
+  // B in fragment order: a wave load is one KiB = 64 bytes of 16 rows (lane -> row lane & 15, bytes 16 (lane >> 4));
+  // unpacked, the wave's two loads are the two KiB of a stage (the second 64 bytes further in LDS), and the
+  // scalar offset advances one KiB per 64 row bytes
+  const int ld_b = g.b_frag ? wave * g.b_steps * 1024 + lane * 16
+                 : PACKED ? (wave * 16 + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
                           : (wave * 16 + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
-  const int kpos_a = (lane & 7) * 16, kpos_b = PACKED ? (lane & 3) * 32 : (lane & 7) * 16;
+  const int ld_b_next = g.b_frag ? 1024 : 8 * (int)g.ldb;  // the wave's second load (unpacked)
+  const int kpos_a = (lane & 7) * 16;
+  const int kpos_b = g.b_frag ? (lane >> 4) * (PACKED ? 32 : 16) : PACKED ? (lane & 3) * 32 : (lane & 7) * 16;
+  const int kpos_b_next = g.b_frag ? 64 : 0;
   const int st_a = (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
-  const int st_b = kATile + (PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
-                                    : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
+  const int st_b = kATile + (g.b_frag ? (wave * 16 + (lane & 15)) * kRow + (lane >> 4) * (PACKED ? 32 : 16)
+                             : PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
+                                      : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
+  const int st_b_next = g.b_frag ? 64 : 8 * kRow;
+  const int ksh_b = g.b_frag ? 4 : 0;  // scalar offset of B = row bytes << ksh_b
   // CONV: position of this lane's two rows (first corner of their windows, in input coordinates) and the tap
   // the next request belongs to, advanced one stage per request (requests come in stage order)
   int cpix[NLA] = {0, 0}, ci0[NLA] = {0, 0}, ci1[NLA] = {0, 0}, ci2[NLA] = {0, 0};
@@ -119,10 +133,10 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, k0, 0);
     } else if constexpr (PACKED) {
       const int vo = k0 + kpos_b < (int)g.k ? ld_b : kOutside;
-      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 / 2, 0);
+      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, (k0 / 2) << ksh_b, 0);
     } else {
-      const int vo = k0 + kpos_b < (int)g.k ? ld_b + (j - NLA) * 8 * (int)g.ldb : kOutside;
-      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0, 0);
+      const int vo = k0 + kpos_b + (j - NLA) * kpos_b_next < (int)g.k ? ld_b + (j - NLA) * ld_b_next : kOutside;
+      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 << ksh_b, 0);
     }
   };
   auto store_stage = [&](const int stage_base) {
@@ -137,7 +151,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
     } else {
 #pragma unroll
-      for (int j = 0; j < NLB; ++j) *reinterpret_cast<v4i*>(st + st_b + j * 8 * kRow) = stg[NLA + j];
+      for (int j = 0; j < NLB; ++j) *reinterpret_cast<v4i*>(st + st_b + j * st_b_next) = stg[NLA + j];
     }
   };
 
@@ -344,6 +358,8 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
   g.tiles_m = (int)((p->m + TM - 1) / TM);
   g.tiles_n = (int)((p->n + TN - 1) / TN);
   const bool packed = p->b_dtype == AQTX_I4P;
+  g.b_frag = p->b_layout == AQTX_W_FRAGMENTS;
+  g.b_steps = (int)(((packed ? p->k / 2 : p->k) + 63) / 64);
   const int epi = gemm_epilogue_id(p);
   if (epi < 0)
     return set_error("aqtx_gemm_i8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
@@ -450,6 +466,8 @@ int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const vo
   GemmArgs g = make_gemm_args(p, a, b, nullptr, col_scale, c, nullptr);
   g.k *= 2; g.lda *= 2; g.stride_a *= 2;  // A in bytes
   g.col_first = 0;
+  g.b_frag = p->b_layout == AQTX_W_FRAGMENTS;
+  g.b_steps = (int)((p->k + 63) / 64);
   g.tiles_m = (int)((p->m + TM - 1) / TM);
   g.tiles_n = (int)((p->n + TN - 1) / TN);
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);

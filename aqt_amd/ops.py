@@ -257,8 +257,12 @@ def gemm(
     group_offsets: Optional[torch.Tensor] = None,
     a_k_order: int = 0,
     k_split: int = 0,
+    b_layout: int = L.W_ROWS,
 ):
   """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
+
+  b_layout = L.W_FRAGMENTS (int8 operands, batch 1): B is the flat buffer tile_weight made of one weight
+  [n, k] (or of its packed int4 form), the copy the serving kernels stream; n is then col_scale's length.
 
   k_split (int8 operands; results do not depend on it): 0 = the library decides whether slices of k go
   to workgroups of their own (few output tiles, long k), 1 = never, S > 1 = S slices.
@@ -277,11 +281,18 @@ def gemm(
   (C, acc) with want_acc.
   """
   _require_gpu(a, b, row_scale, col_scale)
-  assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == (2 * b.shape[2] if b_dtype == L.I4P else b.shape[2])
-  assert a.shape[0] == b.shape[0] or group_offsets is not None
-  assert a.stride(2) == 1 and b.stride(2) == 1, 'the contraction axis must be contiguous'
   batch, m, k = a.shape
-  n = b.shape[1]
+  if b_layout == L.W_FRAGMENTS:
+    assert batch == 1 and group_offsets is None and col_scale is not None and b.is_contiguous() and a.stride(2) == 1
+    n = col_scale.shape[-1]
+    assert b.numel() * b.element_size() == L.lib().aqtx_tile_weight_bytes(n, k, b_dtype), (b.shape, n, k)
+    b_batches, ldb, stride_b = 1, 0, 0
+  else:
+    assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == (2 * b.shape[2] if b_dtype == L.I4P else b.shape[2])
+    assert a.shape[0] == b.shape[0] or group_offsets is not None
+    assert a.stride(2) == 1 and b.stride(2) == 1, 'the contraction axis must be contiguous'
+    n = b.shape[1]
+    b_batches, ldb, stride_b = b.shape[0], b.stride(1), b.stride(0)
   if group_offsets is not None:
     assert a.shape[0] == 1 and group_offsets.dtype == torch.int32 and group_offsets.is_cuda
     assert group_offsets.numel() == b.shape[0] + 1 and group_offsets.is_contiguous()
@@ -295,10 +306,11 @@ def gemm(
   if want_acc:
     acc = torch.empty((batch, m, n), dtype=torch.float32 if fp8 else torch.int32, device=a.device)
   plan = L.GemmPlan()
-  plan.batch, plan.m, plan.n, plan.k = (b.shape[0] if group_offsets is not None else batch), m, n, k
+  plan.batch, plan.m, plan.n, plan.k = (b_batches if group_offsets is not None else batch), m, n, k
   plan.group_offsets = group_offsets.data_ptr() if group_offsets is not None else None
-  plan.lda, plan.ldb, plan.ldc = a.stride(1), b.stride(1), n
-  plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), b.stride(0), m * n
+  plan.lda, plan.ldb, plan.ldc = a.stride(1), ldb, n
+  plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), stride_b, m * n
+  plan.b_layout = b_layout
   plan.a_dtype, plan.b_dtype = a_dtype, b_dtype
   plan.out_dtype, plan.dequant_dtype = out_dt, dq_dt
   plan.row_scale_dtype = aqtx_dtype(row_scale_dtype) if row_scale_dtype is not None else sc_dt
@@ -307,7 +319,7 @@ def gemm(
   plan.tuning = GEMM_TUNING
   plan.a_k_order = a_k_order
   plan.k_split = 1 if fp8 else k_split
-  for s, shape in ((row_scale, (batch, m)), (col_scale, (b.shape[0], n))):
+  for s, shape in ((row_scale, (batch, m)), (col_scale, (b_batches, n))):
     if s is not None:
       assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == shape, (tuple(s.shape), shape)
   plan.row_scale_stride_b, plan.col_scale_stride_b = m, n
@@ -335,21 +347,27 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
 
 
 def gemm_weight_only(a: torch.Tensor, b: torch.Tensor, col_scale: torch.Tensor, *, col_scale_dtype=torch.float32,
-                     b_dtype: int = L.I8):
+                     b_dtype: int = L.I8, b_layout: int = L.W_ROWS):
   """Weight-only contraction C[b] = bf16(bf16(A[b] @ float(B[b])^T) * col_scale[b]) for bf16 A [batch, m, k] that
   stays unquantized and int8 B [batch, n, k] (k contiguous in both), any m; `col_scale` is float32 [batch, n]
   holding values of `col_scale_dtype`.  float32 sums; the weight is never copied as bf16."""
   _require_gpu(a, b, col_scale)
-  assert a.dim() == 3 and b.dim() == 3 and a.shape[2] == b.shape[2] and a.shape[0] == b.shape[0]
-  assert a.dtype == torch.bfloat16 and b.dtype == torch.int8 and a.stride(2) == 1 and b.stride(2) == 1
+  assert a.dim() == 3 and a.dtype == torch.bfloat16 and a.stride(2) == 1
   batch, m, k = a.shape
-  n = b.shape[1]
+  if b_layout == L.W_FRAGMENTS:  # the flat buffer tile_weight made of one int8 weight [n, k]
+    n = col_scale.shape[-1]
+    assert batch == 1 and b.is_contiguous() and b.numel() * b.element_size() == L.lib().aqtx_tile_weight_bytes(n, k, L.I8)
+    ldb = stride_b = 0
+  else:
+    assert b.dim() == 3 and a.shape[2] == b.shape[2] and a.shape[0] == b.shape[0] and b.dtype == torch.int8 and b.stride(2) == 1
+    n, ldb, stride_b = b.shape[1], b.stride(1), b.stride(0)
   assert col_scale.dtype == torch.float32 and col_scale.is_contiguous() and tuple(col_scale.shape) == (batch, n)
   c = torch.empty((batch, m, n), dtype=torch.bfloat16, device=a.device)
   plan = L.GemmPlan()
   plan.batch, plan.m, plan.n, plan.k = batch, m, n, k
-  plan.lda, plan.ldb, plan.ldc = a.stride(1), b.stride(1), n
-  plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), b.stride(0), m * n
+  plan.lda, plan.ldb, plan.ldc = a.stride(1), ldb, n
+  plan.stride_a, plan.stride_b, plan.stride_c = a.stride(0), stride_b, m * n
+  plan.b_layout = b_layout
   plan.a_dtype, plan.b_dtype = L.BF16, b_dtype
   plan.out_dtype = plan.dequant_dtype = plan.row_scale_dtype = L.BF16
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype)

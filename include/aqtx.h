@@ -177,6 +177,10 @@ typedef struct aqtx_gemm_plan {
                                  aqtx_gemm_i8_k_slices(plan) * batch * m * n * 4 bytes; NULL: no slices
                                  unless k_split > 1 asks for them (then an error)                      */
   int64_t k_split_workspace_bytes;
+  int32_t b_layout;           /* aqtx_gemm_i8 and aqtx_gemm_weight_only.  AQTX_W_ROWS (0): b is [batch][n][k] rows.
+                                 AQTX_W_FRAGMENTS: b is one weight (batch 1; int8, or AQTX_I4P) re-laid by
+                                 aqtx_tile_weight, the copy the serving kernels stream; ldb and stride_b are
+                                 ignored.  Same results                                                 */
 } aqtx_gemm_plan;
 
 /*

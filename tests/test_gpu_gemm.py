@@ -373,3 +373,44 @@ def test_weight_only_gemm_strided_operands(gpu):
   ref = (a[0].float() @ b[0].float().T).to(torch.bfloat16).float() * ws[0]
   assert torch.equal(got[0], other) or (got[0] != other).float().mean() < 0.01
   torch.testing.assert_close(got[0].float(), ref, rtol=2.0 ** -7, atol=1e-6)
+
+
+# ---- B in the serving kernels' fragment order: the same results as from rows ----------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('m,n,k,k_split', [(65, 128, 64, 0), (130, 200, 1056, 0), (256, 1024, 4096, 0), (96, 136, 4096, 4),
+                                           (512, 72, 2080, 1), (2048, 2048, 512, 0), (300, 4100, 320, 0)])
+def test_fragment_ordered_b_equals_rows(gpu, m, n, k, k_split, packed):
+  """aqtx_gemm_i8 with b_layout = AQTX_W_FRAGMENTS (the buffer aqtx_tile_weight writes for the serving kernels)
+  against the same call on the rows: integer sums, so bit for bit, outputs and raw accumulators, with and
+  without slices of k, with n and k that end inside a 16-row block / a 64-byte step."""
+  if packed and k % 32 != 0:
+    pytest.skip('packed int4 needs k % 32 == 0')
+  torch.manual_seed(5)
+  lo, hi = (-8, 8) if packed else (-127, 128)
+  a = torch.randint(-127, 128, (1, m, k), dtype=torch.int8, device=gpu)
+  b = torch.randint(lo, hi, (1, n, k), dtype=torch.int8, device=gpu)
+  rs, cs = torch.rand(1, m, device=gpu) + 0.5, torch.rand(1, n, device=gpu) + 0.5
+  b_rows, b_dtype = b, L.I8
+  if packed:
+    b_rows, b_dtype = ops.pack_i4(b.reshape(n, k)).reshape(1, n, k // 2), L.I4P
+  frags = ops.tile_weight(b_rows[0].contiguous(), b_dtype)
+  kw = dict(row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16, scale_dtype=torch.float32, b_dtype=b_dtype, k_split=k_split)
+  want, want_acc = ops.gemm(a, b_rows, want_acc=True, **kw)
+  got, got_acc = ops.gemm(a, frags, want_acc=True, b_layout=L.W_FRAGMENTS, **kw)
+  assert torch.equal(got_acc, want_acc)
+  assert torch.equal(got, want)
+  ref = (a[0].cpu().to(torch.int64) @ b[0].cpu().to(torch.int64).T).to(torch.int32)
+  assert torch.equal(got_acc[0].cpu(), ref)
+
+
+@pytest.mark.gpu
+def test_weight_only_gemm_fragment_ordered_b(gpu):
+  torch.manual_seed(6)
+  m, n, k = 200, 328, 1040
+  a = torch.randn(1, m, k, device=gpu).to(torch.bfloat16)
+  b = torch.randint(-127, 128, (1, n, k), dtype=torch.int8, device=gpu)
+  cs = torch.rand(1, n, device=gpu) * 0.01 + 1e-4
+  want = ops.gemm_weight_only(a, b, cs)
+  got = ops.gemm_weight_only(a, ops.tile_weight(b[0], L.I8), cs, b_layout=L.W_FRAGMENTS)
+  assert torch.equal(got, want)  # the same products added in the same order
