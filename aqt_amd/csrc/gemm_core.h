@@ -211,10 +211,11 @@ __device__ __forceinline__ float dequant_value(AccScalar accv, float s_row, floa
 // registers into the two neighbouring 16-byte chunks of its row on their way to LDS: a nibble is
 // moved to the top of its byte (value * 16); the epilogue takes the factor 16 out again, exactly (a
 // power of two commutes with every rounding of the dequantisation).
-template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = false>
+template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = false, bool BFRAG = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gemm_kernel(const GemmArgs g_in) {
   static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+  static_assert(!BFRAG || MMA::kIntAcc, "the fragment order is that of int8 / packed int4 weights");
   static_assert(!BPACK || MMA::kIntAcc, "packed int4 goes with the int8 MFMA");
   GemmArgs g = g_in;
   constexpr int NI = 16 / NW;       // 32-column MFMA tiles per wave
@@ -276,9 +277,15 @@ void gemm_kernel(const GemmArgs g_in) {
   const int64_t rows_b = (g.n - n0) < BN ? (g.n - n0) : BN;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0, (int)((rows_b - 1) * g.ldb + (BPACK ? g.k / 2 : g.k)),
-      kBufferRsrcWord3);
+  // BFRAG, B in fragment order (GemmArgs::b_frag): the tile's 16-row blocks follow one another, b_steps KiB
+  // each; the piece (row r, 16 bytes at 16 c of a 64-byte step) is lane r % 16 + 16 c of its KiB, and the scalar
+  // offset of a stage is its row bytes times 16.
+  const __amdgpu_buffer_rsrc_t rsrc_b = BFRAG
+      ? __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (n0 / 16) * (int64_t)g.b_steps * 1024), 0,
+                                          (int)((rows_b + 15) / 16 * g.b_steps * 1024), kBufferRsrcWord3)
+      : __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0,
+                                          (int)((rows_b - 1) * g.ldb + (BPACK ? g.k / 2 : g.k)), kBufferRsrcWord3);
+  constexpr int ksh_b = BFRAG ? 4 : 0;
   int voff_a[LPW], voff_b[LPB], chunk_byte[LPW];
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
@@ -286,7 +293,11 @@ void gemm_kernel(const GemmArgs g_in) {
     const int row = blk * 8 + (lane >> 3);
     chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ blk) & 7) * 16;
     voff_a[i] = row * (int)g.lda + chunk_byte[i];
-    if constexpr (!BPACK) voff_b[i] = row * (int)g.ldb + chunk_byte[i];
+    if constexpr (!BPACK) {
+      const int cb = chunk_byte[i] >> 4;  // chunk 0..7 of the 128-byte stage: KiB cb >> 2 of the stage's two
+      voff_b[i] = BFRAG ? ((row >> 4) * g.b_steps + (cb >> 2)) * 1024 + ((cb & 3) * 16 + (row & 15)) * 16
+                        : row * (int)g.ldb + chunk_byte[i];
+    }
   }
   // packed B: load q of a wave covers rows 16 (wave LPB + q) .. +15, lane -> row lane >> 2, 16 packed bytes
   // (32 k) at 16 (lane & 3); they become the chunks 2p, 2p + 1 of that row, at positions chunk ^ f(row)
@@ -295,7 +306,8 @@ void gemm_kernel(const GemmArgs g_in) {
 #pragma unroll
     for (int q = 0; q < LPB; ++q) {
       const int row = (wave * LPB + q) * 16 + (lane >> 2);
-      voff_b[q] = row * (int)g.ldb + (lane & 3) * 16;
+      voff_b[q] = BFRAG ? (wave * LPB + q) * g.b_steps * 1024 + ((lane & 3) * 16 + (lane >> 2)) * 16
+                        : row * (int)g.ldb + (lane & 3) * 16;
       pb_st[q] = kTileBytes + row * BK + (((2 * (lane & 3)) ^ ((row ^ (row >> 3)) & 7)) * 16);
     }
   }
@@ -312,11 +324,11 @@ void gemm_kernel(const GemmArgs g_in) {
     } else if constexpr (BPACK) {
       int vo = voff_b[i];
       if (KTAIL && k0 + (lane & 3) * 32 >= (int)g.k) vo = 0x7FFFFFF0;
-      stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 / 2, 0);
+      stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, (k0 / 2) << ksh_b, 0);
     } else {
       int vo = voff_b[i];
       if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;
-      stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0, 0);
+      stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 << ksh_b, 0);
     }
   };
   const int st_off = wave * LPW * 1024 + lane * 16;
@@ -786,6 +798,9 @@ int launch_conv_i8_mid(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, const
                        const float* row_scale, const float* col_scale, void* c, hipStream_t st);
 int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                         const float* col_scale, void* c, float* acc_out, hipStream_t st);
+// gemm_i8_frag.hip: the 256 x 256 kernel (8 waves, row scale first) on a fragment-ordered b
+int launch_gemm_i8_frag(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                        const float* col_scale, void* c, int32_t* acc_out, hipStream_t st);
 int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* col_scale, void* c,
                                 hipStream_t st);
 

@@ -67,6 +67,8 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   GemmArgs g = make_gemm_args(p, a, b, row_scale, col_scale, c, acc_out);
   g.a_even_odd8 = p->a_k_order == AQTX_K_EVEN_ODD8;
   const bool b_packed = p->b_dtype == AQTX_I4P;
+  g.b_frag = p->b_layout == AQTX_W_FRAGMENTS;
+  g.b_steps = (int)(((b_packed ? p->k / 2 : p->k) + 63) / 64);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
   const bool b_frag = p->b_layout == AQTX_W_FRAGMENTS;
@@ -93,14 +95,7 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
 
   // few output tiles: the 128 x 128 kernel, with K in slices where that still leaves CUs idle
   AQTX_REQUIRE(p->k_split >= 0 && p->k_split <= 64, "aqtx_gemm_i8: k_split must be in 0..64, got %d", p->k_split);
-  int mid_slices = gemm_mid_k_slices(p);
-  if (b_frag && mid_slices == 0) {
-    // the 256 x 256 kernel reads rows only
-    AQTX_REQUIRE(p->tuning == 0 && (!b_packed || !g.col_first) && p->lda * (int64_t)128 < (1ll << 31),
-                 "aqtx_gemm_i8: a fragment-ordered b takes tuning 0 | 128 (and AQTX_SCALE_ROW_THEN_COL when packed)");
-    mid_slices = 1;
-  }
-  if (int slices = mid_slices; slices > 0) {
+  if (int slices = gemm_mid_k_slices(p); slices > 0) {
     // slices the library chose itself are dropped where the caller lent no (or too small a) workspace
     if (p->k_split == 0 && slices > 1 &&
         (p->k_split_workspace == nullptr || p->k_split_workspace_bytes < (int64_t)slices * p->batch * p->m * p->n * 4))
@@ -110,6 +105,11 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   AQTX_REQUIRE(p->k_split <= 1, "aqtx_gemm_i8: k_split > 1 with ragged batches, plan->tuning or unaligned operands");
   // Two waves per SIMD by default: measured faster on every shape tried (the epilogue of one
   // wave overlaps the other's work).  plan->tuning = 4 | 8 overrides it (tests, tuning).
+  if (b_frag) {
+    AQTX_REQUIRE((p->tuning == 0 || p->tuning == 8) && !g.col_first,
+                 "aqtx_gemm_i8: a fragment-ordered b takes scale_order AQTX_SCALE_ROW_THEN_COL and tuning 0, 8 or 128");
+    return launch_gemm_i8_frag(p, a, b, row_scale, col_scale, c, acc_out, st);
+  }
   const int waves = p->tuning == 4 ? 4 : 8;
   AQTX_REQUIRE(!b_packed || !g.col_first, "aqtx_gemm_i8: a packed int4 b takes scale_order = AQTX_SCALE_ROW_THEN_COL");
   // packed int4 B: the 8-wave kernel, row scale first (a frozen weight is the column operand)

@@ -510,14 +510,18 @@ def _kernel_layout_of(qvalue: torch.Tensor, v: 'lowering.OperandView', pack_int4
   hit = _KERNEL_LAYOUT_CACHE.get(id(qvalue))
   if hit is not None and hit[0] == key and slot in hit[1]:
     return hit[1][slot]
+  def rows():
+    r = v.mem if v.k_last else v.mem.transpose(1, 2).contiguous()
+    return ops.pack_i4(r.contiguous()) if pack_int4 else r
   if fragments:
-    base = _kernel_layout_of(qvalue, v, pack_int4=pack_int4)
+    # from the rows copy if one is kept already, else from a passing one: the fragment order is then the
+    # only copy of the weight next to the caller's own
+    base = hit[1].get((pack_int4, False)) if hit is not None and hit[0] == key else None
+    base = base if base is not None else rows()
     assert base.shape[0] == 1
     q = ops.tile_weight(base[0].contiguous(), L.I4P if pack_int4 else L.I8)
   else:
-    q = v.mem if v.k_last else v.mem.transpose(1, 2).contiguous()
-    if pack_int4:
-      q = ops.pack_i4(q.contiguous())
+    q = rows()
   hit = _KERNEL_LAYOUT_CACHE.get(id(qvalue))
   if hit is None:
     weakref.finalize(qvalue, _KERNEL_LAYOUT_CACHE.pop, id(qvalue), None)
@@ -801,7 +805,13 @@ class DotGeneralRaw:
         'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t, _bwd_memo, _calibrated)
     # ---- rhs ---------------------------------------------------------------------
     rq, rs, rsdt, rhs_qt_out, rhs_grad = self._quant_side(
-        'rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, rba, rra, rca, None, _bwd_memo, _calibrated)
+        'rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, rba, rra, rca, None, _bwd_memo, _calibrated,
+        layout_later=rhs_qt is not None and rhs_qt.qvalue is not None and rhs_qt.qvalue.dtype == torch.int8)
+    rv_later = None  # a frozen int8 rhs that is not laid out for the kernels as the caller holds it
+    if rq is None:
+      rv_later = lowering.view_operand(rhs_qt.qvalue, rba, rra, rca)
+      if ragged is not None:
+        rq, rv_later = _kernel_layout_of(rhs_qt.qvalue, rv_later), None
 
     lkd = aqt_tensor.qvalue_kernel_dtype(lhs_qt_out)
     rkd = aqt_tensor.qvalue_kernel_dtype(rhs_qt_out)
@@ -817,7 +827,7 @@ class DotGeneralRaw:
       assert acc in (utils.float32, None), f'{self.dg_accumulator_dtype=} with fp8 operands'
 
     B, M, K = lq.shape
-    N = rq.shape[1]
+    N = rq.shape[1] if rq is not None else rv_later.R
     if ragged is not None:
       G = rhs_arr.shape[0]
       rq3 = rq.reshape(N, G, K).permute(1, 0, 2)  # [g, n, k] view of the quantizer's [n, g*k] rows
@@ -830,7 +840,10 @@ class DotGeneralRaw:
       res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=lhs, qx=lhs_qt_out), quant_grad=lhs_grad),
                           rhs=TensorRes(mt=MultiTensor(x=rhs_arr, qx=rhs_qt_out), quant_grad=rhs_grad))
       return out.reshape(M, N), res
-    assert rq.shape[0] == B and rq.shape[2] == K, (lq.shape, rq.shape)
+    if rq is not None:
+      assert rq.shape[0] == B and rq.shape[2] == K, (lq.shape, rq.shape)
+    else:
+      assert rv_later.B == B and rv_later.K == K, (lq.shape, rv_later.B, rv_later.R, rv_later.K)
     # scales: [B, M] / [B, N] or a single per-tensor value (broadcast here, tiny)
     def expand(s, n):
       return s.reshape(1, 1).expand(B, n).contiguous() if s.numel() == 1 and B * n != 1 else s.reshape(B, n)
@@ -845,10 +858,20 @@ class DotGeneralRaw:
     swapped = (out_transpose_axes is not None and list(out_transpose_axes) == swap_perm
                and want_lba == lba and nl > 0 and nr > 0)
     common = dict(out_dtype=dequant_dtype, dequant_dtype=dequant_dtype)
-    if (not swapped and not fp8 and rhs_qt is not None and rhs_qt.is_full() and rhs_qt.container_dtype is utils.int4
-        and rkd == L.I4 and K % 32 == 0 and K < 132096 and rq.dtype == torch.int8):
-      # a frozen int4 weight is read packed two values per byte (half the bytes of a serving call
-      # and of the copy kept per weight; made once per tensor), unpacked in registers by the kernel
+    # a frozen int4 weight is read packed two values per byte (half the bytes of a serving call
+    # and of the copy kept per weight; made once per tensor), unpacked in registers by the kernel
+    pack = (not swapped and not fp8 and rhs_qt is not None and rhs_qt.is_full() and rhs_qt.container_dtype is utils.int4
+            and rkd == L.I4 and K % 32 == 0 and K < 132096 and (rq is None or rq.dtype == torch.int8))
+    b_layout = L.W_ROWS
+    if rv_later is not None:
+      # the copy the serving kernels stream (fragment order) serves the contraction kernels too, so a weight
+      # used with few and with many lhs rows is kept once; the swapped product reads the weight as rows
+      frag = (not swapped and not fp8 and B == 1 and K % 16 == 0 and N * K < 2 ** 31 and lq.stride(1) % 16 == 0
+              and lq.data_ptr() % 16 == 0 and ops.GEMM_TUNING in (0, 8, 128))
+      rq = _kernel_layout_of(rhs_qt.qvalue, rv_later, pack_int4=pack, fragments=frag)
+      b_layout = L.W_FRAGMENTS if frag else L.W_ROWS
+      rkd = L.I4P if pack else rkd
+    elif pack:
       rq = _kernel_layout_of(rhs_qt.qvalue, lowering.view_operand(rhs_qt.qvalue, rba, rra, rca), pack_int4=True)
       rkd = L.I4P
     if swapped:
@@ -858,7 +881,7 @@ class DotGeneralRaw:
       out = out.reshape(bdims + rdims + ldims)
     else:
       out = ops.gemm(lq, rq, row_scale=expand(ls, M), col_scale=expand(rs, N), a_dtype=lkd, b_dtype=rkd,
-                     row_scale_dtype=lsdt, col_scale_dtype=rsdt, **common)
+                     row_scale_dtype=lsdt, col_scale_dtype=rsdt, b_layout=b_layout, **common)
       # [B, M, N] -> (batch..., lhs remaining..., rhs remaining...) in the caller's batch order
       out = out.reshape(bdims + ldims + rdims)
       if want_lba != lba:
@@ -965,9 +988,12 @@ class DotGeneralRaw:
           lv.mem[0], w_fragments, _scale_vector_f32(w_scale, [], rra, rca), w_scale_dtype=w_scale.dtype,
           w_dtype=L.I4P if packed else L.I4 if rhs_qt.container_dtype is utils.int4 else L.I8, w_layout=L.W_FRAGMENTS)
     else:
-      w_rows = rv.mem if rv.k_last and not rv.copied else _kernel_layout_of(rhs_qt.qvalue, rv)
-      out = ops.gemm_weight_only(lv.mem, w_rows, _scale_vector_f32(w_scale, [], rra, rca).reshape(1, N),
-                                 col_scale_dtype=w_scale.dtype)
+      if rv.k_last and not rv.copied:
+        w, w_layout = rv.mem, L.W_ROWS
+      else:
+        w, w_layout = _kernel_layout_of(rhs_qt.qvalue, rv, fragments=True), L.W_FRAGMENTS
+      out = ops.gemm_weight_only(lv.mem, w, _scale_vector_f32(w_scale, [], rra, rca).reshape(1, N),
+                                 col_scale_dtype=w_scale.dtype, b_layout=w_layout)
     out = out.reshape([lhs.shape[a] for a in lra] + [rhs_arr.shape[a] for a in rra])
     lhs_qt_out = aqt_tensor.QTensor(qvalue=lhs, scale=[], scale_t=None, bias=[], dequant_dtype=lhs.dtype)
     rhs_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
@@ -976,7 +1002,7 @@ class DotGeneralRaw:
     return out, res
 
   def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t,
-                  bwd_memo=None, calibrated=None):
+                  bwd_memo=None, calibrated=None, layout_later=False):
     """Quantizes one side; returns (q [B,R,K], scale f32, scale dtype, QTensor, quant_grad).
     `bwd_memo`: the backward pass's table of per-tensor scales; `calibrated`: where a calibration
     that runs step by step leaves its result for a later fall-back of the same call."""
@@ -986,8 +1012,13 @@ class DotGeneralRaw:
       if given_qt.bias or len(given_qt.scale) != 1 or given_qt.sparsity_mask is not None:
         raise _NotFused('a provided QTensor with a bias, a sparsity mask or several scales')
       v = lowering.view_operand(given_qt.qvalue, ba, ra, ca)
-      q = v.mem if v.k_last and not v.copied else _kernel_layout_of(given_qt.qvalue, v)
-      if q.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+      if v.k_last and not v.copied:
+        q = v.mem
+      elif layout_later:
+        q = None  # the caller picks rows or the serving kernels' fragment order (one copy kept per weight)
+      else:
+        q = _kernel_layout_of(given_qt.qvalue, v)
+      if q is not None and q.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
         q = q.view(torch.uint8)
       s = given_qt.scale[0]
       return q, _scale_vector_f32(s, ba, ra, ca), s.dtype, given_qt, quant_grad

@@ -122,7 +122,8 @@ def test_tiling_injection(gpu):
 def test_serving_from_logical_order_checkpoint(gpu):
   """A frozen weight restored in its logical [K, N] order (as a checkpoint would hold it) serves the
   same values as the one the convert step produced, through the decode path and the GEMM path, and
-  is re-laid out for the kernels once, not per call."""
+  is re-laid out for the kernels once, not per call: one copy, in the serving kernels' fragment order,
+  which the contraction kernels read as well."""
   from aqt_amd.v2 import aqt_dot_general as adg
   dt = 'bf16'
   w = U.to_dev(U.rand((256, 128), dt, 2, 0.02), dt, gpu)
@@ -141,6 +142,9 @@ def test_serving_from_logical_order_checkpoint(gpu):
     assert torch.equal(serve(x8, torch.zeros_like(w), MATMUL, None), want8)
     assert torch.equal(serve(x100, torch.zeros_like(w), MATMUL, None), want100)
   assert len(adg._KERNEL_LAYOUT_CACHE) == 1
+  (_, copies), = adg._KERNEL_LAYOUT_CACHE.values()
+  assert list(copies) == [(False, True)]  # (packed int4, fragment order)
+  assert copies[(False, True)].numel() == 256 * 128
 
 
 @pytest.mark.parametrize('bits', [8, 4])
