@@ -15,6 +15,12 @@
 // (packed) of the step, i.e. two (four) MFMA operands of 8 bf16 after conversion, and reads the same k of
 // token r: 32 (64) contiguous bytes.  The weight is the MFMA's first operand, so a lane ends with four
 // consecutive outputs n of one token.
+//
+// Every workgroup reads all of its tokens' activations (from L2), so with many tokens and a narrow weight
+// (few 64-row tiles) the activation traffic of 16-row tiles is a multiple of the weight's.  Given a workspace,
+// such calls keep the 64-row tiles and cut K into slices instead (grid.y): a workgroup leaves its float32
+// partial sums in slab s of the workspace, and decode_wo_sum_kernel adds the slabs in slice order and applies
+// the epilogue: still one fixed summation order.
 #include "common.h"
 
 namespace aqtx {
@@ -37,6 +43,8 @@ struct WoArgs {
   int m, n, k;
   int out_bf16, ws_bf16;
   int w_frag, w_steps;
+  int splits, k_slice;   // slices of K (grid.y) and their length, a multiple of four weight fragment steps
+  float* slabs;          // [splits][m][n] partial sums when splits > 1
 };
 
 __device__ __forceinline__ float rnd(float v, int bf) { return bf ? round_bf16(v) : v; }
@@ -82,6 +90,37 @@ __device__ __forceinline__ void weight_operands(const v4i w, v8bf (&op)[PACKED ?
   }
 }
 
+// The contraction's result in the activation dtype, times the rhs scale in the promoted dtype, final cast;
+// four consecutive outputs n of token mm.
+__device__ __forceinline__ void wo_store(const WoArgs& d, int mm, int nn, const v4f total, bool wide_ok) {
+  float f[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float ws = d.w_scale[(nn + e) < d.n ? (nn + e) : (d.n - 1)];
+    float v = round_bf16(total[e]);
+    v = rnd(v * ws, d.ws_bf16);
+    f[e] = rnd(v, d.out_bf16);
+  }
+  const int64_t o = (int64_t)mm * d.n + nn;
+  if (wide_ok) {
+    if (d.out_bf16) {
+      uint2 v;
+      v.x = (uint32_t)bf16_bits(f[0]) | ((uint32_t)bf16_bits(f[1]) << 16);
+      v.y = (uint32_t)bf16_bits(f[2]) | ((uint32_t)bf16_bits(f[3]) << 16);
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(d.out) + o) = v;
+    } else {
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(d.out) + o) = make_float4(f[0], f[1], f[2], f[3]);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (nn + e < d.n) {
+        if (d.out_bf16) reinterpret_cast<uint16_t*>(d.out)[o + e] = bf16_bits(f[e]);
+        else reinterpret_cast<float*>(d.out)[o + e] = f[e];
+      }
+  }
+}
+
 template <int MB, int NB, int D, bool PACKED>
 __global__ __launch_bounds__(256) void decode_wo_kernel(const WoArgs d) {
   constexpr int T = MB * NB;             // output tiles of 16 x 16 per workgroup
@@ -95,9 +134,11 @@ __global__ __launch_bounds__(256) void decode_wo_kernel(const WoArgs d) {
   const int r = lane & 15, c = lane >> 4;
   const int n0 = (int)blockIdx.x * 16 * NB;
   const int kb = PACKED ? d.k / 2 : d.k;  // bytes of one weight row
-  const int kq = ((d.k + 3) / 4 + KS - 1) / KS * KS;
-  const int k_lo = wave * kq;
-  const int k_hi = (k_lo + kq) < d.k ? (k_lo + kq) : d.k;
+  const int s_lo = (int)blockIdx.y * d.k_slice;
+  const int s_hi = (s_lo + d.k_slice) < d.k ? (s_lo + d.k_slice) : d.k;
+  const int kq = d.k_slice / 4;
+  const int k_lo = s_lo + wave * kq;
+  const int k_hi = (k_lo + kq) < s_hi ? (k_lo + kq) : s_hi;
 
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(d.w, d.w_frag ? (int64_t)((d.n + 15) / 16) * d.w_steps * 1024 : (int64_t)d.n * kb);
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(d.x, (int64_t)d.m * d.k * 2);
@@ -179,50 +220,75 @@ __global__ __launch_bounds__(256) void decode_wo_kernel(const WoArgs d) {
     const v4f total = ((red[0][t][lane] + red[1][t][lane]) + red[2][t][lane]) + red[3][t][lane];
     const int mm = (t / NB) * 16 + r, nn = n0 + (t % NB) * 16 + 4 * c;
     if (mm >= d.m || nn >= d.n) continue;
-    // the contraction's result in the activation dtype, times the rhs scale in the promoted dtype, final cast
-    float f[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float ws = d.w_scale[(nn + e) < d.n ? (nn + e) : (d.n - 1)];
-      float v = round_bf16(total[e]);
-      v = rnd(v * ws, d.ws_bf16);
-      f[e] = rnd(v, d.out_bf16);
+    if (d.splits > 1) {
+      float* dst = d.slabs + ((int64_t)blockIdx.y * d.m + mm) * d.n + nn;
+      if (wide_ok) *reinterpret_cast<float4*>(dst) = make_float4(total[0], total[1], total[2], total[3]);
+      else for (int e = 0; e < 4 && nn + e < d.n; ++e) dst[e] = total[e];
+      continue;
     }
-    const int64_t o = (int64_t)mm * d.n + nn;
-    if (wide_ok) {
-      if (d.out_bf16) {
-        uint2 v;
-        v.x = (uint32_t)bf16_bits(f[0]) | ((uint32_t)bf16_bits(f[1]) << 16);
-        v.y = (uint32_t)bf16_bits(f[2]) | ((uint32_t)bf16_bits(f[3]) << 16);
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(d.out) + o) = v;
-      } else {
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(d.out) + o) = make_float4(f[0], f[1], f[2], f[3]);
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (nn + e < d.n) {
-          if (d.out_bf16) reinterpret_cast<uint16_t*>(d.out)[o + e] = bf16_bits(f[e]);
-          else reinterpret_cast<float*>(d.out)[o + e] = f[e];
-        }
-    }
+    wo_store(d, mm, nn, total, wide_ok);
   }
 }
 
+// out = epilogue(slab 0 + slab 1 + ...), the slabs added in slice order; thread -> four consecutive n of one token
+__global__ __launch_bounds__(256) void decode_wo_sum_kernel(const WoArgs d) {
+  const int64_t quads = (d.n + 3) / 4;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= quads * d.m) return;
+  const int mm = (int)(id / quads), nn = (int)(id % quads) * 4;
+  const bool wide_ok = (d.n % 4) == 0;
+  v4f total = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int sl = 0; sl < d.splits; ++sl) {
+    const float* src = d.slabs + ((int64_t)sl * d.m + mm) * d.n + nn;
+    v4f part = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    if (wide_ok) {
+      const float4 t = *reinterpret_cast<const float4*>(src);
+      part = v4f{t.x, t.y, t.z, t.w};
+    } else {
+      for (int e = 0; e < 4 && nn + e < d.n; ++e) part[e] = src[e];
+    }
+    total = sl == 0 ? part : total + part;
+  }
+  wo_store(d, mm, nn, total, wide_ok);
+}
+
 template <int MB, int NB, int D>
-void launch_wo(const WoArgs& d, bool packed, unsigned grid, hipStream_t st) {
+void launch_wo(const WoArgs& d, bool packed, dim3 grid, hipStream_t st) {
   if (packed) decode_wo_kernel<MB, NB, D, true><<<grid, 256, 0, st>>>(d);
   else decode_wo_kernel<MB, NB, D, false><<<grid, 256, 0, st>>>(d);
 }
 
-}  // namespace
-}  // namespace aqtx
+// Launch shape for a plan: token blocks, weight blocks per workgroup, slices of K and their length.
+struct WoShape { int mb, nb, splits, k_slice; };
 
-using namespace aqtx;
+WoShape wo_shape(const aqtx_decode_plan* p, bool with_workspace) {
+  const bool pk = p->w_dtype == AQTX_I4P;
+  const int ks = pk ? 128 : 64;
+  WoShape s;
+  s.mb = p->m <= 16 ? 1 : p->m <= 32 ? 2 : 4;
+  // the tallest weight tile of 64 / 32 / 16 rows that still gives most CUs a workgroup
+  s.nb = 4;
+  while (s.nb > 1 && (p->n + 16 * s.nb - 1) / (16 * s.nb) < 192) s.nb /= 2;
+  s.splits = 1;
+  const int64_t tiles64 = (p->n + 63) / 64;
+  if (with_workspace && s.nb < 4 && (p->m > 32 || (p->m > 16 && s.nb == 1 && p->k >= 8192))) {
+    // many tokens against a narrow weight: 64-row tiles (a quarter of the activation reads of 16-row tiles)
+    // and slices of K until about 256 workgroups exist, each slice at least 1024 of k.  Measured: it pays
+    // from 33 tokens on, and from 17 where 16-row tiles would walk a long k (the second launch costs 2 us)
+    int64_t want = (256 + tiles64 - 1) / tiles64;
+    want = want > 8 ? 8 : want;
+    want = want > p->k / 1024 ? p->k / 1024 : want;
+    if (want >= 2) { s.nb = 4; s.splits = (int)want; }
+  }
+  if (const int t = p->tuning & 7; t == 1 || t == 2 || t == 4) s.nb = t;
+  if (const int t = (p->tuning >> 4) & 15; with_workspace && t >= 1 && t <= 8 && t <= p->k / (4 * ks)) s.splits = t;
+  const int64_t per = (p->k + s.splits - 1) / s.splits;
+  s.k_slice = (int)((per + 4 * ks - 1) / (4 * ks) * (4 * ks));
+  s.splits = (int)((p->k + s.k_slice - 1) / s.k_slice);
+  return s;
+}
 
-extern "C" int aqtx_decode_weight_only(const aqtx_decode_plan* p, const void* x, const void* w, const float* w_scale,
-                                       void* out, void* stream) {
-  clear_error();
+int validate_wo(const aqtx_decode_plan* p) {
   AQTX_REQUIRE(p != nullptr, "aqtx_decode_weight_only: plan is NULL");
   AQTX_REQUIRE(p->m >= 0 && p->n >= 0 && p->k >= 0, "aqtx_decode_weight_only: negative shape");
   AQTX_REQUIRE(p->m <= 64, "aqtx_decode_weight_only: m = %lld exceeds 64", (long long)p->m);
@@ -241,11 +307,35 @@ extern "C" int aqtx_decode_weight_only(const aqtx_decode_plan* p, const void* x,
                "aqtx_decode_weight_only: unknown w_layout %d", p->w_layout);
   AQTX_REQUIRE(p->w_layout == AQTX_W_ROWS || (p->n + 15) / 16 * ((p->k + 63) / 64) * 1024 < (1ll << 31) - 64,
                "aqtx_decode_weight_only: fragment-ordered weight larger than 2 GiB");
+  return 0;
+}
+
+}  // namespace
+}  // namespace aqtx
+
+using namespace aqtx;
+
+extern "C" size_t aqtx_decode_weight_only_workspace_bytes(const aqtx_decode_plan* p) {
+  clear_error();
+  if (validate_wo(p) != 0 || p->m == 0 || p->n == 0) return 0;
+  const WoShape s = wo_shape(p, true);
+  return s.splits > 1 ? (size_t)s.splits * (size_t)p->m * (size_t)p->n * 4 : 0;
+}
+
+extern "C" int aqtx_decode_weight_only(const aqtx_decode_plan* p, const void* x, const void* w, const float* w_scale,
+                                       void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  if (int rc = validate_wo(p)) return rc;
+  const bool pk = p->w_dtype == AQTX_I4P;
   if (p->m == 0 || p->n == 0) return 0;
   AQTX_REQUIRE(x != nullptr && w != nullptr && w_scale != nullptr && out != nullptr, "aqtx_decode_weight_only: NULL buffer");
   AQTX_REQUIRE(((uintptr_t)w % 16) == 0 && ((uintptr_t)x % 16) == 0, "aqtx_decode_weight_only: x and w must be 16-byte aligned");
   const size_t esz = p->out_dtype == AQTX_BF16 ? 2 : 4;
   AQTX_REQUIRE(((uintptr_t)out % (4 * esz)) == 0 || p->n % 4 != 0, "aqtx_decode_weight_only: out must be aligned to four elements");
+  // slices of K only with a workspace that holds their partial sums (the call works without one)
+  WoShape s = wo_shape(p, workspace != nullptr);
+  if (s.splits > 1 && (workspace_bytes < (size_t)s.splits * p->m * p->n * 4 || ((uintptr_t)workspace % 16) != 0))
+    s = wo_shape(p, false);
 
   WoArgs d{};
   d.x = reinterpret_cast<const uint8_t*>(x);
@@ -256,12 +346,10 @@ extern "C" int aqtx_decode_weight_only(const aqtx_decode_plan* p, const void* x,
   d.ws_bf16 = p->w_scale_dtype == AQTX_BF16;
   d.w_frag = p->w_layout == AQTX_W_FRAGMENTS;
   d.w_steps = (int)(((pk ? p->k / 2 : p->k) + 63) / 64);
-  // the tallest weight tile of 64 / 32 / 16 rows that still gives most CUs a workgroup
-  const int mb = p->m <= 16 ? 1 : p->m <= 32 ? 2 : 4;
-  int nb = 4;
-  while (nb > 1 && (p->n + 16 * nb - 1) / (16 * nb) < 192) nb /= 2;
-  if (const int t = p->tuning & 7; t == 1 || t == 2 || t == 4) nb = t;
-  const unsigned grid = (unsigned)((p->n + 16 * nb - 1) / (16 * nb));
+  d.splits = s.splits; d.k_slice = s.k_slice;
+  d.slabs = reinterpret_cast<float*>(workspace);
+  const int nb = s.nb;
+  const dim3 grid((unsigned)((p->n + 16 * nb - 1) / (16 * nb)), (unsigned)s.splits);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define AQTX_WO(M)                                                \
   do {                                                            \
@@ -269,8 +357,13 @@ extern "C" int aqtx_decode_weight_only(const aqtx_decode_plan* p, const void* x,
     else if (nb == 2) launch_wo<M, 2, 4>(d, pk, grid, st);        \
     else launch_wo<M, 1, 4>(d, pk, grid, st);                     \
   } while (0)
-  if (mb == 1) AQTX_WO(1); else if (mb == 2) AQTX_WO(2); else AQTX_WO(4);
+  if (s.mb == 1) AQTX_WO(1); else if (s.mb == 2) AQTX_WO(2); else AQTX_WO(4);
 #undef AQTX_WO
   AQTX_HIP_CHECK_LAUNCH("decode_wo_kernel");
+  if (s.splits > 1) {
+    const int64_t quads = (int64_t)((p->n + 3) / 4) * p->m;
+    decode_wo_sum_kernel<<<dim3((unsigned)((quads + 255) / 256)), 256, 0, st>>>(d);
+    AQTX_HIP_CHECK_LAUNCH("decode_wo_sum_kernel");
+  }
   return 0;
 }

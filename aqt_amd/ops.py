@@ -403,8 +403,11 @@ def decode_weight_only(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor
   plan.quant_bound = plan.clip_bound = 1.0
   plan.w_dtype, plan.w_layout, plan.tuning = w_dtype, w_layout, tuning
   out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+  need = L.lib().aqtx_decode_weight_only_workspace_bytes(ctypes.byref(plan))
+  ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
   with _timed('decode'):
-    L.check(L.lib().aqtx_decode_weight_only(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(out), _stream()))
+    L.check(L.lib().aqtx_decode_weight_only(ctypes.byref(plan), _ptr(x), _ptr(w_q), _ptr(w_scale), _ptr(out),
+                                            _ptr(ws) if ws is not None else None, need, _stream()))
   return out
 
 

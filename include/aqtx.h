@@ -447,10 +447,15 @@ int aqtx_decode_i8_static(const aqtx_decode_plan* plan, const void* x, const voi
  * once and converted to bf16 in registers; sums are float32, so the result agrees with the reference's float
  * contraction to summation order, not bit for bit.  Of the plan: m, n, k, x_dtype (AQTX_BF16), w_dtype,
  * w_layout, w_scale_dtype, out_dtype and tuning (low three bits 1 / 2 / 4: weight rows per workgroup in
- * sixteens; 0 = the library chooses) are read.  k must be a multiple of 16 (32 for packed int4).  No workspace.
+ * sixteens, bits 4-7: slices of k; 0 = the library chooses) are read.  k must be a multiple of 16 (32 for
+ * packed int4).
  */
 int aqtx_decode_weight_only(const aqtx_decode_plan* plan, const void* x, const void* w, const float* w_scale,
-                            void* out, void* stream);
+                            void* out, void* workspace, size_t workspace_bytes, void* stream);
+/* Scratch bytes with which aqtx_decode_weight_only cuts k into slices for `plan` (more than 16 tokens against a
+   weight of few rows; float32 partial sums, added in slice order); 0 = it would not.  The workspace is optional:
+   without it (NULL) the call walks all of k per workgroup. */
+size_t aqtx_decode_weight_only_workspace_bytes(const aqtx_decode_plan* plan);
 
 /*
  * aqtx_prng_split_host: jax.random.split(key, num) on the host (used by

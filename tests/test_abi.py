@@ -201,14 +201,26 @@ def test_decode_workspace_and_null_checks():
 ])
 def test_weight_only_decode_plan_validation(kw, needle):
   p = _dplan(**kw)
-  msg = _err(L.lib().aqtx_decode_weight_only(ctypes.byref(p), FAKE, FAKE, FAKE, FAKE, None))
+  msg = _err(L.lib().aqtx_decode_weight_only(ctypes.byref(p), FAKE, FAKE, FAKE, FAKE, None, 0, None))
   assert needle in msg, msg
 
 
 def test_weight_only_decode_null_and_empty():
-  assert 'NULL' in _err(L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan()), None, FAKE, FAKE, FAKE, None))
-  assert 'plan is NULL' in _err(L.lib().aqtx_decode_weight_only(None, FAKE, FAKE, FAKE, FAKE, None))
-  assert L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan(n=0)), None, None, None, None, None) == 0
+  assert 'NULL' in _err(L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan()), None, FAKE, FAKE, FAKE, None, 0, None))
+  assert 'plan is NULL' in _err(L.lib().aqtx_decode_weight_only(None, FAKE, FAKE, FAKE, FAKE, None, 0, None))
+  assert L.lib().aqtx_decode_weight_only(ctypes.byref(_dplan(n=0)), None, None, None, None, None, 0, None) == 0
+
+
+def test_weight_only_decode_workspace_bytes():
+  """Slices of k (and so a workspace) only for more than 16 tokens against a weight of few rows and a long k."""
+  need = lambda **kw: L.lib().aqtx_decode_weight_only_workspace_bytes(ctypes.byref(_dplan(**kw)))
+  assert need(m=64, n=4096, k=14336) == 4 * 64 * 4096 * 4     # 64 tiles of 64 rows -> 4 slices
+  assert need(m=8, n=4096, k=14336) == 0
+  assert need(m=24, n=4096, k=14336) == 4 * 24 * 4096 * 4
+  assert need(m=24, n=4096, k=4096) == 0 and need(m=40, n=4096, k=4096) == 4 * 40 * 4096 * 4
+  assert need(m=64, n=14336, k=4096) == 0                      # 224 tiles of 64 rows fill the chip
+  assert need(m=64, n=4096, k=1024) == 0                       # k too short to cut
+  assert need(m=65, n=4096, k=14336) == 0                      # not a valid plan
 
 
 def _woplan(**kw):

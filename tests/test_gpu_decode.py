@@ -317,18 +317,20 @@ def test_read_probe_reads_every_byte(gpu):
 
 # ---- weight-only serving (the lhs stays bf16; float32 sums: tolerance, not bits) ----------------------------
 @pytest.mark.gpu
+@pytest.mark.parametrize('tuning', [0, 3 << 4, (8 << 4) | 1])  # the library's choice; 3 slices of k; 8 slices, 16-row tiles
 @pytest.mark.parametrize('layout', ['rows', 'fragments'])
 @pytest.mark.parametrize('packed', [False, True])
 @pytest.mark.parametrize('w_sdt', ['bf16', 'f32'])
 @pytest.mark.parametrize('m,n,k', [(1, 200, 4096), (5, 16, 64), (16, 1024, 528 + 16 * 31), (17, 72, 2048), (33, 4096, 1024),
                                    (64, 300, 4096)])
-def test_weight_only_decode_within_float_summation_error(gpu, m, n, k, w_sdt, packed, layout):
+def test_weight_only_decode_within_float_summation_error(gpu, m, n, k, w_sdt, packed, layout, tuning):
   """out = bf16(bf16(sum_k x w) * scale) with the sum in float32 in the kernel's own order.  Tolerance, stated:
   against the sum taken exactly (float64; every product of a bf16 and an int8 is exact), a float32 sum in any
   order is off by less than d = k * 2^-24 * sum_k |x w|.  Every later step (the two roundings, the product with
   a positive scale) is monotone, so each output must lie between the same steps applied to exact - d and to
   exact + d; where the terms cancel that is many ulps of a small result, elsewhere less than one.  99 % of the
-  outputs must equal the steps applied to the exact sum."""
+  outputs must equal the steps applied to the exact sum.  With slices of k (forced through `tuning`, or chosen
+  for the last two shapes) the partial sums are added in slice order: the same bound."""
   from aqt_amd import _lib as L
   if packed and k % 32 != 0:
     pytest.skip('packed int4 needs k % 32 == 0')
@@ -354,7 +356,7 @@ def test_weight_only_decode_within_float_summation_error(gpu, m, n, k, w_sdt, pa
   if layout == 'fragments':
     wt, w_layout = ops.tile_weight(wt, w_dtype), L.W_FRAGMENTS
   got = ops.decode_weight_only(torch.from_numpy(x).to(torch.bfloat16).to(gpu), wt, torch.from_numpy(ws.astype(np.float32)).to(gpu),
-                               w_scale_dtype=U.TORCH_DT[w_sdt], w_dtype=w_dtype, w_layout=w_layout)
+                               w_scale_dtype=U.TORCH_DT[w_sdt], w_dtype=w_dtype, w_layout=w_layout, tuning=tuning)
   got = got.float().cpu().numpy().astype(np.float64)
   assert ((low <= got) & (got <= high)).all(), np.argwhere((got < low) | (got > high))[:8]
   assert (got == want).mean() >= 0.99
