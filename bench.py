@@ -248,6 +248,21 @@ def other_configs(dev):
         wo[f'int{bits}_m{m_few}'] = {'us_per_call': round(us, 1), 'weight_GB/s': round(4096 * 14336 * bits / 8 / us / 1e3, 1)}
         del graphed
       del wq
+    # the narrow weight of the same block (14336 -> 4096) against 64 tokens: 64-row tiles with k in slices
+    wn = (torch.randn(14336, 4096, device=dev) * 0.02).to(torch.bfloat16)
+    cfg = config.set_context(aqt_dot_general.dot_general_make(None, 8), None, None)
+    xn = torch.randn(64, 14336, device=dev).to(torch.bfloat16)
+    _, (_, wq) = cfg.dg_core(xn, wn, None, None, MATMUL)
+
+    def ten_narrow(a):
+      for _ in range(9):
+        cfg.dg_core(a, wn, None, wq, MATMUL)
+      return cfg.dg_core(a, wn, None, wq, MATMUL)[0]
+
+    graphed = hip_graph.GraphedCall(ten_narrow, xn)
+    us = timeit(graphed.replay, n=10, w=3) * 1e3 / 10
+    wo['int8_m64_14336x4096'] = {'us_per_call': round(us, 1), 'weight_GB/s': round(4096 * 14336 / us / 1e3, 1)}
+    del graphed, wq, wn, xn
   out['weight_only_frozen_serving_few_tokens_4096x14336'] = wo
   del xs, ws
   # quantized ragged_dot (mixture of experts): 8192 tokens routed to 8 experts [4096, 14336], uneven groups,
