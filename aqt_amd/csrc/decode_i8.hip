@@ -9,6 +9,8 @@
 //   m <= 2 : one kernel; every workgroup (16 weight rows) quantizes the activations itself.
 //   m >= 3 : a per-token quantize kernel, then a contraction kernel whose workgroups own a tile of
 //            weight rows and one K range; partial sums of the K ranges meet through int32 atomics.
+#include <type_traits>
+
 #include "common.h"
 
 #include <mutex>
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   // activations: loads return in order, so the other way round the quantisation would wait for the weights.
   v4i wf[U];
 #pragma unroll
-  for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
+  for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, WFRAG ? kStreamOnce : 0);
   auto value = [&](int i, int j, int e) -> float {
     if constexpr (XBF) {
       const uint32_t w = raw[i][j][e >> 1];
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
   for (int kk = k_lo; kk < k_hi; kk += KS * U) {
     if (kk != k_lo) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, 0);
+      for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, WFRAG ? kStreamOnce : 0);
     }
     v4i xf[U][XP];
 #pragma unroll
@@ -401,7 +403,7 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
   // compiler would make every wave wait as if it had weights outstanding.
   if (contracts) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, 0);
+    for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(k_lo + u * KS), 0, WFRAG ? kStreamOnce : 0);
     quantize_rows();
   } else {
     quantize_rows();
@@ -416,7 +418,7 @@ __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
     for (int kk = k_lo; kk < k_hi; kk += KS * U) {
       if (kk != k_lo) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, 0);
+        for (int u = 0; u < U; ++u) wf[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_offset(kk + u * KS), 0, WFRAG ? kStreamOnce : 0);
       }
       // four weight loads' worth of activation fragments at a time (all U at once would double the registers)
       constexpr int UC = U < 4 ? U : 4;
@@ -637,12 +639,13 @@ void decode_tile_kernel(const DecodeArgs d) {
   unsigned xdead[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) xdead[mb] = mb < d.mb_total ? 0u : (unsigned)kOob;
-  auto issue = [&](int slot, int ko) {
+  auto issue = [&](auto stream_c, int slot, int ko) {
+    constexpr int kPolicy = decltype(stream_c)::value ? kStreamOnce : 0;
     const unsigned dead = (ko + c * KL < k_hi) ? 0u : (unsigned)kOob;  // a lane's KL values are all inside or all outside
     const unsigned wk = (unsigned)(ko / KS) * wstep;  // a k step is 64 bytes of a row, or one KiB fragment
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
-      wf[slot][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)(((unsigned)wbase[nb] + wk) | dead), 0, 0);
+      wf[slot][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)(((unsigned)wbase[nb] + wk) | dead), 0, kPolicy);
     const unsigned xstep = (unsigned)(ko / KS) * (unsigned)d.mb_total;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -682,18 +685,23 @@ void decode_tile_kernel(const DecodeArgs d) {
     j = j >= nsteps ? j - nsteps : j;
     return i < nsteps ? k_lo + j * KS : 0x3FFFFF00;
   };
+  // The weight loads carry the streaming hint when a wave load is a whole KiB fragment; the choice is made
+  // once, outside the loop (a branch around a load would make the compiler drain the loads in flight).
+  auto walk = [&](auto stream_c) {
 #pragma unroll
-  for (int s = 0; s < D; ++s) issue(s, step_k(s));
-  __builtin_amdgcn_sched_barrier(0);
-  for (int i = 0; i < nsteps; i += D) {
+    for (int s = 0; s < D; ++s) issue(stream_c, s, step_k(s));
+    __builtin_amdgcn_sched_barrier(0);
+    for (int i = 0; i < nsteps; i += D) {
 #pragma unroll
-    for (int s = 0; s < D; ++s) {
-      multiply(s);
-      __builtin_amdgcn_sched_barrier(0);
-      issue(s, step_k(i + D + s));
-      __builtin_amdgcn_sched_barrier(0);
+      for (int s = 0; s < D; ++s) {
+        multiply(s);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(stream_c, s, step_k(i + D + s));
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-  }
+  };
+  if (d.w_frag) walk(std::true_type{}); else walk(std::false_type{});
   // lane holds C[n = n0 + nb*16 + 4c + e][m = mb*16 + r] in acc[mb][nb][e]
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
