@@ -53,8 +53,9 @@ __global__ __launch_bounds__(256) void sum_tiles_kernel(const void* x, void* out
   }
 }
 
-// Reads `bytes` once, 16 bytes per lane and load, PER loads in flight per lane, and writes one
-// word per workgroup: the least any kernel that streams a buffer of this size can take.
+// Reads `bytes` once, 16 bytes per lane and load (with the non-temporal hint the serving kernels give
+// their weight loads), PER loads in flight per lane, and writes one word per workgroup: the least any
+// kernel that streams a buffer of this size can take.
 template <int PER>
 __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* p, int64_t vecs, uint32_t* out) {
   uint32_t acc = 0u;
@@ -63,8 +64,9 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* p, int64_t
   for (int j = 0; j < PER; ++j) {
     const int64_t i = base + (int64_t)j * 256;
     if (i < vecs) {
-      const uint4 v = p[i];
-      acc ^= v.x ^ v.y ^ v.z ^ v.w;
+      typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+      const v4u v = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p + i));
+      acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
     }
   }
 #pragma unroll
