@@ -390,3 +390,29 @@ def test_weight_only_serving_takes_the_kernel(gpu, monkeypatch):
     want = (x.float() @ wf).cpu().numpy()
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2.0 ** -6, atol=2.0 ** -6 * np.abs(want).max())
   assert (out_large_kernel != out_large).float().mean() < 0.02  # both round a float32 sum to bf16
+
+
+@pytest.mark.gpu
+def test_weight_only_serving_many_tokens_narrow_weight(gpu):
+  """48 tokens against a frozen int8 weight of 512 rows and k = 8192: the layer call goes to the weight-only kernel
+  with k in slices (a workspace is asked for and lent), and agrees with the float product on the dequantized
+  weight to float32 summation order."""
+  from aqt_amd import _lib as L
+  from aqt_amd.v2 import aqt_dot_general as aqt, config
+  import ctypes
+  dt = 'bf16'
+  MATMUL = (((1,), (0,)), ((), ()))
+  plan = L.DecodePlan()
+  plan.m, plan.n, plan.k = 48, 512, 8192
+  plan.x_dtype = plan.x_scale_dtype = plan.out_dtype = plan.w_scale_dtype = L.BF16
+  plan.quant_bound = plan.clip_bound = 1.0
+  plan.w_dtype, plan.w_layout = L.I8, L.W_FRAGMENTS
+  assert L.lib().aqtx_decode_weight_only_workspace_bytes(ctypes.byref(plan)) == 8 * 48 * 512 * 4
+  cfg = config.set_context(aqt.dot_general_make(None, 8), None, None)
+  w = U.to_dev(U.rand((8192, 512), dt, 3, 0.05), dt, gpu)
+  x = U.to_dev(U.rand((48, 8192), dt, 1), dt, gpu)
+  with torch.no_grad():
+    _, (_, wq) = cfg.dg_core(x, w, None, None, MATMUL)
+    out, _ = cfg.dg_core(x, torch.zeros_like(w), None, wq, MATMUL)
+  want = (x.float() @ (wq.qvalue.float() * wq.scale[0].float())).cpu().numpy()
+  np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2.0 ** -6, atol=2.0 ** -6 * np.abs(want).max())
