@@ -10,7 +10,7 @@ namespace {
 template <class MMA>
 int launch_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
   // K tails are always masked here: fewer instantiations, and the mask is one compare per load.
-#define AQTX_LAUNCH(E, C) gemm_kernel<MMA, 4, E, C, true><<<grid, 256, 0, st>>>(g)
+#define AQTX_LAUNCH(E, C) gemm_kernel<MMA, 8, E, C, true><<<grid, 512, 0, st>>>(g)
 #define AQTX_LAUNCH_C(E) do { if (g.col_first) AQTX_LAUNCH(E, true); else AQTX_LAUNCH(E, false); } while (0)
   switch (epi) {
     case 0: AQTX_LAUNCH_C(0); break;
