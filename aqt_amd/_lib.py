@@ -17,6 +17,7 @@ PRESCALE_NONE, PRESCALE_PER_ROW, PRESCALE_PER_COL = range(3)
 SCALE_ROW_THEN_COL, SCALE_COL_THEN_ROW = range(2)
 W_ROWS, W_FRAGMENTS = range(2)
 K_NATURAL, K_EVEN_ODD8 = range(2)
+ACC_FAST, ACC_F32 = range(2)
 
 
 class QuantPlan(ctypes.Structure):
@@ -56,6 +57,7 @@ class GemmPlan(ctypes.Structure):
       ('k_split', ctypes.c_int32),
       ('k_split_workspace', ctypes.c_void_p), ('k_split_workspace_bytes', ctypes.c_int64),
       ('b_layout', ctypes.c_int32),
+      ('accumulate', ctypes.c_int32),
   ]
 
 

@@ -38,7 +38,7 @@ struct MmaI8 {
   using Frag = v4i;
   static constexpr int kChunks = 1;   // v_mfma_i32_32x32x32_i8: 32 k per MFMA, 16 per lane
   static constexpr bool kIntAcc = true;
-  static constexpr bool kWidenB = false;
+  static constexpr bool kWidenA = false, kWidenB = false;
   static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, c, 0, 0, 0);
   }
@@ -54,7 +54,7 @@ struct MmaF8 {
   using Frag = v8i;
   static constexpr int kChunks = 2;   // 64 k per MFMA, 32 per lane
   static constexpr bool kIntAcc = false;
-  static constexpr bool kWidenB = false;
+  static constexpr bool kWidenA = false, kWidenB = false;
   // x comes from the B tile, y from the A tile (see mfma_step).  Zero scale operands select the
   // unscaled form of the instruction (v_mfma_f32_32x32x64_f8f6f4).
   static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
@@ -71,25 +71,65 @@ struct MmaBf16W8 {
   using Frag = v4i;
   static constexpr int kChunks = 1;   // 16 k per MFMA, 8 per lane: 16 bytes
   static constexpr bool kIntAcc = false;
-  static constexpr bool kWidenB = true;
+  static constexpr bool kWidenA = false, kWidenB = true;
   static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, x), __builtin_bit_cast(v8bf, y), c, 0, 0, 0);
   }
+  // 16 int8 values (k order) -> 16 bf16 values in two 16-byte chunks.  Every int8 value is a bf16 value, so
+  // the upper half of its float32 form is the result.
+  static __device__ __forceinline__ void widen_b(const v4i x4, v4i& lo, v4i& hi) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int x = x4[d];
+      const uint32_t f0 = __float_as_uint((float)(int8_t)x), f1 = __float_as_uint((float)(int8_t)(x >> 8));
+      const uint32_t f2 = __float_as_uint((float)(int8_t)(x >> 16)), f3 = __float_as_uint((float)(x >> 24));
+      const int w0 = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u), w1 = (int)__builtin_amdgcn_perm(f3, f2, 0x07060302u);
+      if (d < 2) { lo[2 * d] = w0; lo[2 * d + 1] = w1; }
+      else { hi[2 * (d - 2)] = w0; hi[2 * (d - 2) + 1] = w1; }
+    }
+  }
 };
 
-// 16 int8 values (k order) -> 16 bf16 values in two 16-byte chunks.  Every int8 value is a bf16 value, so
-// the upper half of its float32 form is the result.
-__device__ __forceinline__ void widen_i8x16_bf16(const v4i x4, v4i& lo, v4i& hi) {
+// 16 fp8 bytes (FMT 0 = e4m3fn, 1 = e5m2; k order) -> 16 bf16 values in two 16-byte chunks.  Every fp8 value,
+// subnormals included, is a bf16 value (3 or 2 mantissa bits against 7, a narrower exponent range), so the upper
+// half of its float32 form is the result; a NaN byte stays a NaN.
+template <int FMT>
+__device__ __forceinline__ void widen_f8x16_bf16(const v4i x4, v4i& lo, v4i& hi) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
     const int x = x4[d];
-    const uint32_t f0 = __float_as_uint((float)(int8_t)x), f1 = __float_as_uint((float)(int8_t)(x >> 8));
-    const uint32_t f2 = __float_as_uint((float)(int8_t)(x >> 16)), f3 = __float_as_uint((float)(x >> 24));
-    const int w0 = (int)__builtin_amdgcn_perm(f1, f0, 0x07060302u), w1 = (int)__builtin_amdgcn_perm(f3, f2, 0x07060302u);
+    const v2f p0 = FMT ? __builtin_amdgcn_cvt_pk_f32_bf8(x, false) : __builtin_amdgcn_cvt_pk_f32_fp8(x, false);
+    const v2f p1 = FMT ? __builtin_amdgcn_cvt_pk_f32_bf8(x, true) : __builtin_amdgcn_cvt_pk_f32_fp8(x, true);
+    const int w0 = (int)__builtin_amdgcn_perm(__float_as_uint(p0[1]), __float_as_uint(p0[0]), 0x07060302u);
+    const int w1 = (int)__builtin_amdgcn_perm(__float_as_uint(p1[1]), __float_as_uint(p1[0]), 0x07060302u);
     if (d < 2) { lo[2 * d] = w0; lo[2 * d + 1] = w1; }
     else { hi[2 * (d - 2)] = w0; hi[2 * (d - 2) + 1] = w1; }
   }
 }
+
+// fp8 x fp8 with float32-like sums (aqtx_gemm_plan.accumulate = AQTX_ACC_F32): both operands' bytes are widened
+// to bf16, exactly, on their way to LDS and contracted by v_mfma_f32_32x32x16_bf16.  Measured on gfx950: that
+// instruction keeps every product bit down to 2^-24 of the largest term of its 16-long k block and rounds the
+// block sum plus accumulator to nearest even, so a contraction stays within the error bound of a float32
+// summation; the fp8 MFMA forms (v_mfma_f32_32x32x16_fp8_fp8 and v_mfma_scale_f32_32x32x64_f8f6f4 alike) align
+// the products of every 8 consecutive k to the largest of them and cut each off 2^-13 below it.  Half the
+// matrix-core rate and twice the LDS bytes of the fp8 form.
+template <int FMT_A, int FMT_B>
+struct MmaBf16F8 {
+  typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+  using Acc = v16f;
+  using AccScalar = float;
+  using Frag = v4i;
+  static constexpr int kChunks = 1;
+  static constexpr bool kIntAcc = false;
+  static constexpr bool kWidenA = true, kWidenB = true;
+  static __device__ __forceinline__ Acc mma(const Frag& x, const Frag& y, const Acc& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, x), __builtin_bit_cast(v8bf, y), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void widen_a(const v4i x4, v4i& lo, v4i& hi) { widen_f8x16_bf16<FMT_A>(x4, lo, hi); }
+  static __device__ __forceinline__ void widen_b(const v4i x4, v4i& lo, v4i& hi) { widen_f8x16_bf16<FMT_B>(x4, lo, hi); }
+};
 
 struct GemmArgs {
   const uint8_t* a;
@@ -801,6 +841,9 @@ int launch_conv_i8_mid(const aqtx_im2col_plan* w, const aqtx_gemm_plan* p, const
                        const float* row_scale, const float* col_scale, void* c, hipStream_t st);
 int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                         const float* col_scale, void* c, float* acc_out, hipStream_t st);
+// the same plan contracted through bf16 (plan->accumulate == AQTX_ACC_F32)
+int launch_gemm_fp8_f32sum_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                               const float* col_scale, void* c, float* acc_out, hipStream_t st);
 // gemm_i8_frag.hip: the 256 x 256 kernel (8 waves, row scale first) on a fragment-ordered b
 int launch_gemm_i8_frag(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                         const float* col_scale, void* c, int32_t* acc_out, hipStream_t st);

@@ -1,6 +1,7 @@
 // fp8 x fp8 -> float32 contraction on gfx950 MFMA (v_mfma_scale_f32_32x32x64_f8f6f4 with
 // unit block scales) with the dequantisation fused in the epilogue; the kernel lives in
-// gemm_core.h.  Each operand is e4m3fn or e5m2 independently.
+// gemm_core.h.  Each operand is e4m3fn or e5m2 independently.  plan->accumulate == AQTX_ACC_F32
+// sends the plan through bf16 instead (gemm_mid.hip, MmaBf16F8).
 #include "gemm_core.h"
 
 using namespace aqtx;
@@ -51,6 +52,7 @@ extern "C" int aqtx_gemm_fp8(const aqtx_gemm_plan* p, const void* a, const void*
     AQTX_HIP_CHECK_LAUNCH("gemm_simple_kernel");
     return 0;
   }
+  if (p->accumulate == AQTX_ACC_F32) return launch_gemm_fp8_f32sum_mid(p, a, b, row_scale, col_scale, c, acc_out, st);
   // few output tiles (or tiles that would lie mostly outside C): the 128 x 128 kernel
   if (p->k_split <= 1 && gemm_mid_k_slices(p) > 0) return launch_gemm_fp8_mid(p, a, b, row_scale, col_scale, c, acc_out, st);
   AQTX_REQUIRE(p->lda * (int64_t)BM < (1ll << 31) && p->ldb * (int64_t)BN < (1ll << 31),

@@ -20,6 +20,8 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
     AQTX_REQUIRE(p->out_dtype == AQTX_BF16 || p->out_dtype == AQTX_F32 || p->out_dtype == AQTX_I32,
                  "%s: out_dtype must be bf16, f32 or i32, got %d", who, p->out_dtype);
   }
+  AQTX_REQUIRE(p->accumulate == AQTX_ACC_FAST || (fp8 && p->accumulate == AQTX_ACC_F32 && p->group_offsets == nullptr),
+               "%s: accumulate must be AQTX_ACC_FAST, or AQTX_ACC_F32 for fp8 operands without ragged batches", who);
   AQTX_REQUIRE(is_float_dtype(p->dequant_dtype), "%s: dequant_dtype must be bf16 or f32", who);
   AQTX_REQUIRE(is_float_dtype(p->row_scale_dtype) && is_float_dtype(p->col_scale_dtype),
                "%s: row_scale_dtype / col_scale_dtype must be bf16 or f32", who);

@@ -22,7 +22,9 @@ constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile; 
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
 // int4 values two per byte (see gemm_kernel's BPACK), or, with MmaBf16W8, int8 values that become bf16 (A then
-// holds bf16 values, and GemmArgs::k, lda and stride_a count its bytes).
+// holds bf16 values, and GemmArgs::k, lda and stride_a count its bytes), or, with MmaBf16F8, fp8 bytes that become
+// bf16; A's rows are then widened the same way (MMA::kWidenA: GemmArgs::k counts the bf16 bytes of a row in LDS,
+// twice the fp8 bytes in memory, while lda and stride_a count those).
 // SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then; integer sums only).
 // CONV: A is a convolution input read in place (GemmArgs::conv): the window gather that would otherwise be
 // materialised (features % 128 == 0, so a 128-byte stage lies inside one tap).
@@ -32,6 +34,8 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
   static_assert(!CONV || (MMA::kIntAcc && !PACKED && !SLAB), "the convolution reads int8 bytes, whole K");
   static_assert(MMA::kIntAcc || (!SLAB && PACKED == MMA::kWidenB && EPI != 3), "float sums: whole K; fp8 bytes as they are");
+  constexpr bool WIDEN_A = MMA::kWidenA;
+  static_assert(!WIDEN_A || (PACKED && !CONV), "a widened A goes with a widened B");
   using Acc = typename MMA::Acc;
   using AccScalar = typename MMA::AccScalar;
   using Frag = typename MMA::Frag;
@@ -58,7 +62,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   const __amdgpu_buffer_rsrc_t rsrc_a = CONV
       ? __builtin_amdgcn_make_buffer_rsrc((void*)g.a, 0, (int)g.conv.x_bytes, kBufferRsrcWord3)
       : __builtin_amdgcn_make_buffer_rsrc((void*)(g.a + bz * g.stride_a + m0 * g.lda), 0,
-                                          (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+                                          (int)((rows_a - 1) * g.lda + (WIDEN_A ? g.k / 2 : g.k)), kBufferRsrcWord3);
   const int64_t blocks_b = (rows_b + 15) / 16;  // fragment order: the tile's 16-row blocks, whole
   const __amdgpu_buffer_rsrc_t rsrc_b = g.b_frag
       ? __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (n0 / 16) * (int64_t)g.b_steps * 1024), 0,
@@ -71,10 +75,11 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   // B packed: a wave load covers 16 rows x 64 B, one per wave; a lane's 16 bytes become the 32 bytes at
   // 32 * (lane & 3) of its row.  The row and chunk of a load are in its vector offset, which the buffer's
   // range check covers; the scalar offset (the stage's k) is not range checked, the mask on K covers it.
-  constexpr int NLA = 2, NLB = PACKED ? 1 : 2, NL = NLA + NLB;
+  constexpr int NLA = WIDEN_A ? 1 : 2, NLB = PACKED ? 1 : 2, NL = NLA + NLB;
   constexpr int kOutside = 0x7FFFFFF0;
   v4i stg[NL];
-  const int ld_a = (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
+  const int ld_a = WIDEN_A ? (wave * 16 + (lane >> 2)) * (int)g.lda + (lane & 3) * 16
+                           : (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
   // B in fragment order: a wave load is one KiB = 64 bytes of 16 rows (lane -> row lane & 15, bytes 16 (lane >> 4));
   // unpacked, the wave's two loads are the two KiB of a stage (the second 64 bytes further in LDS), and the
   // scalar offset advances one KiB per 64 row bytes
@@ -82,10 +87,11 @@ void gemm_mid_kernel(const GemmArgs g_in) {
                  : PACKED ? (wave * 16 + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
                           : (wave * 16 + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
   const int ld_b_next = g.b_frag ? 1024 : 8 * (int)g.ldb;  // the wave's second load (unpacked)
-  const int kpos_a = (lane & 7) * 16;
+  const int kpos_a = WIDEN_A ? (lane & 3) * 32 : (lane & 7) * 16;
   const int kpos_b = g.b_frag ? (lane >> 4) * (PACKED ? 32 : 16) : PACKED ? (lane & 3) * 32 : (lane & 7) * 16;
   const int kpos_b_next = g.b_frag ? 64 : 0;
-  const int st_a = (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
+  const int st_a = WIDEN_A ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
+                           : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
   const int st_b = kATile + (g.b_frag ? (wave * 16 + (lane & 15)) * kRow + (lane >> 4) * (PACKED ? 32 : 16)
                              : PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
                                       : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
@@ -93,7 +99,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   const int ksh_b = g.b_frag ? 4 : 0;  // scalar offset of B = row bytes << ksh_b
   // CONV: position of this lane's two rows (first corner of their windows, in input coordinates) and the tap
   // the next request belongs to, advanced one stage per request (requests come in stage order)
-  int cpix[NLA] = {0, 0}, ci0[NLA] = {0, 0}, ci1[NLA] = {0, 0}, ci2[NLA] = {0, 0};
+  int cpix[2] = {0, 0}, ci0[2] = {0, 0}, ci1[2] = {0, 0}, ci2[2] = {0, 0};
   int ct0 = 0, ct1 = 0, ct2 = 0, cch = 0;  // wave-uniform
   if constexpr (CONV) {
 #pragma unroll
@@ -130,7 +136,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     }
     if (j < NLA) {
       const int vo = k0 + kpos_a < (int)g.k ? ld_a + j * 8 * (int)g.lda : kOutside;
-      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, k0, 0);
+      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, WIDEN_A ? k0 / 2 : k0, 0);
     } else if constexpr (PACKED) {
       const int vo = k0 + kpos_b < (int)g.k ? ld_b : kOutside;
       stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, (k0 / 2) << ksh_b, 0);
@@ -141,11 +147,18 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   };
   auto store_stage = [&](const int stage_base) {
     uint8_t* st = stage_mem + stage_base;
+    if constexpr (WIDEN_A) {
+      v4i lo, hi;
+      MMA::widen_a(stg[0], lo, hi);
+      *reinterpret_cast<v4i*>(st + st_a) = lo;
+      *reinterpret_cast<v4i*>(st + st_a + 16) = hi;
+    } else {
 #pragma unroll
-    for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
+      for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
+    }
     if constexpr (PACKED) {
       v4i lo, hi;
-      if constexpr (MMA::kWidenB) widen_i8x16_bf16(stg[NLA], lo, hi);
+      if constexpr (MMA::kWidenB) MMA::widen_b(stg[NLA], lo, hi);
       else unpack_i4x32(stg[NLA], lo, hi, g.a_even_odd8);
       *reinterpret_cast<v4i*>(st + st_b) = lo;
       *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
@@ -306,10 +319,10 @@ void launch_mid(const GemmArgs& g, bool packed, dim3 grid, hipStream_t st) {
   gemm_mid_kernel<MmaI8, EPI, COL_FIRST, false, false><<<grid, 512, 0, st>>>(g);
 }
 
-template <class MMA>
+template <class MMA, bool WIDENED = false>
 void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
-#define AQTX_MID8(E) do { if (g.col_first) gemm_mid_kernel<MMA, E, true, false, false><<<grid, 512, 0, st>>>(g); \
-                          else gemm_mid_kernel<MMA, E, false, false, false><<<grid, 512, 0, st>>>(g); } while (0)
+#define AQTX_MID8(E) do { if (g.col_first) gemm_mid_kernel<MMA, E, true, WIDENED, false><<<grid, 512, 0, st>>>(g); \
+                          else gemm_mid_kernel<MMA, E, false, WIDENED, false><<<grid, 512, 0, st>>>(g); } while (0)
   switch (epi) {
     case 0: AQTX_MID8(0); break;
     case 1: AQTX_MID8(1); break;
@@ -371,6 +384,8 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
                      ((uintptr_t)p->k_split_workspace % 16) == 0,
                  "aqtx_gemm_i8: %d slices of k need a 16-byte aligned k_split_workspace of %lld bytes", slices,
                  (long long)need);
+    AQTX_REQUIRE(p->m <= 65535, "aqtx_gemm_i8: slices of k take at most 65535 rows (m = %lld); set k_split = 1",
+                 (long long)p->m);
     g.k_split = slices;
     g.k_chunk = ((p->k + slices - 1) / slices + BK - 1) / BK * BK;
     g.k_split = (int)((p->k + g.k_chunk - 1) / g.k_chunk);
@@ -455,6 +470,30 @@ int launch_gemm_fp8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, c
   else if (a5 && !b5) launch_mid_fp8<MmaF8<1, 0>>(g, epi, grid, st);
   else launch_mid_fp8<MmaF8<1, 1>>(g, epi, grid, st);
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<fp8>");
+  return 0;
+}
+
+// fp8 operands contracted through bf16 (both widened in registers, float32-like sums) on the 128 x 128 tiles,
+// whatever the number of tiles.
+int launch_gemm_fp8_f32sum_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
+                               const float* col_scale, void* c, float* acc_out, hipStream_t st) {
+  GemmArgs g = make_gemm_args(p, a, b, row_scale, col_scale, c, acc_out);
+  g.k *= 2;  // bf16 bytes of a row in LDS; lda, ldb and the batch strides stay in fp8 bytes
+  g.tiles_m = (int)((p->m + TM - 1) / TM);
+  g.tiles_n = (int)((p->n + TN - 1) / TN);
+  const int epi = gemm_epilogue_id(p);
+  if (epi < 0 || epi == 3)
+    return set_error("aqtx_gemm_fp8: unsupported out/dequant/scale dtype combination (%d, %d, %d)",
+                     p->out_dtype, p->dequant_dtype, p->row_scale_dtype);
+  AQTX_REQUIRE(p->lda * (int64_t)TM < (1ll << 31) && p->ldb * (int64_t)TN < (1ll << 31) && p->k < (1ll << 29),
+               "aqtx_gemm_fp8: leading dimension or k too large for 32-bit tile offsets");
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
+  const bool a5 = p->a_dtype == AQTX_E5M2, b5 = p->b_dtype == AQTX_E5M2;
+  if (!a5 && !b5) launch_mid_fp8<MmaBf16F8<0, 0>, true>(g, epi, grid, st);
+  else if (!a5 && b5) launch_mid_fp8<MmaBf16F8<0, 1>, true>(g, epi, grid, st);
+  else if (a5 && !b5) launch_mid_fp8<MmaBf16F8<1, 0>, true>(g, epi, grid, st);
+  else launch_mid_fp8<MmaBf16F8<1, 1>, true>(g, epi, grid, st);
+  AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<fp8 through bf16>");
   return 0;
 }
 

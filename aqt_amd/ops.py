@@ -9,6 +9,7 @@ from __future__ import annotations
 import contextlib
 import ctypes
 import math
+import os
 from typing import Optional, Sequence
 
 import numpy as np
@@ -238,6 +239,12 @@ def quantize(
 # of the int8 kernel on 256 x 256 tiles, 128 = the kernel on 128 x 128 tiles (the parity tests run all three).
 GEMM_TUNING = 0
 
+# aqtx_gemm_plan.accumulate of fp8 gemm() calls that do not say: L.ACC_FAST = the fp8 matrix instruction (products
+# of every 8 consecutive k aligned to the largest of them and cut off 2^-13 below it), L.ACC_F32 = both operands
+# widened to bf16 on their way to the matrix cores, sums within the error bound of a float32 summation at half the
+# rate.  AQTX_FP8_ACCUMULATE=f32 in the environment selects the latter for a whole process.
+FP8_ACCUMULATE = L.ACC_F32 if os.environ.get('AQTX_FP8_ACCUMULATE', '').lower() == 'f32' else L.ACC_FAST
+
 
 def gemm(
     a: torch.Tensor,
@@ -258,8 +265,12 @@ def gemm(
     a_k_order: int = 0,
     k_split: int = 0,
     b_layout: int = L.W_ROWS,
+    accumulate: Optional[int] = None,
 ):
   """C[b] = dequant(A[b] @ B[b]^T) for A [batch, m, k], B [batch, n, k] (k contiguous).
+
+  accumulate (fp8 operands only; None = FP8_ACCUMULATE): L.ACC_FAST contracts with the fp8 matrix
+  instruction, L.ACC_F32 through bf16 with float32-like sums at half the rate.
 
   b_layout = L.W_FRAGMENTS (int8 operands, batch 1): B is the flat buffer tile_weight made of one weight
   [n, k] (or of its packed int4 form), the copy the serving kernels stream; n is then col_scale's length.
@@ -319,6 +330,7 @@ def gemm(
   plan.tuning = GEMM_TUNING
   plan.a_k_order = a_k_order
   plan.k_split = 1 if fp8 else k_split
+  plan.accumulate = (FP8_ACCUMULATE if accumulate is None else accumulate) if fp8 else L.ACC_FAST
   for s, shape in ((row_scale, (batch, m)), (col_scale, (b_batches, n))):
     if s is not None:
       assert s.dtype == torch.float32 and s.is_contiguous() and tuple(s.shape) == shape, (tuple(s.shape), shape)

@@ -163,6 +163,16 @@ def other_configs(dev):
 
   ms = timeit(step4)
   out['fp8_einsum_bsd_dhk_fwd_bwd'] = {'ms_per_step': round(ms, 3), 'TFLOP/s': round(3 * 2 * 32768 * 4096 * 4096 / ms / 1e9, 1)}
+  # the same step with the three contractions through bf16 (float32-like sums, aqtx_gemm_plan.accumulate = AQTX_ACC_F32)
+  from aqt_amd import _lib as L
+  from aqt_amd import ops
+  fast = ops.FP8_ACCUMULATE
+  try:
+    ops.FP8_ACCUMULATE = L.ACC_F32
+    ms = timeit(step4)
+  finally:
+    ops.FP8_ACCUMULATE = fast
+  out['fp8_einsum_bsd_dhk_fwd_bwd_f32_sums'] = {'ms_per_step': round(ms, 3), 'TFLOP/s': round(3 * 2 * 32768 * 4096 * 4096 / ms / 1e9, 1)}
   del x, w, g
   # int4 weights / int8 activations, groups of 128 along K (tiled dot_general), forward
   lhs = torch.randn(2048, 8192, device=dev).to(torch.bfloat16)
