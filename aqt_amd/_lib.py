@@ -132,7 +132,8 @@ SYMBOLS = {
     'aqtx_prng_split': (ctypes.c_int, [_vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp]),
     'aqtx_random_bits': (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint32), ctypes.c_int64,
                                         ctypes.c_int32, ctypes.c_int32, _vp, _vp]),
-    'aqtx_read_probe': (ctypes.c_int, [_vp, ctypes.c_int64, _vp, ctypes.c_int64, _vp]),
+    'aqtx_read_probe': (ctypes.c_int, [_vp, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _vp, _vp,
+                                       ctypes.POINTER(ctypes.c_int32), _vp]),
     'aqtx_last_error': (ctypes.c_char_p, []),
     'aqtx_version': (ctypes.c_int, []),
 }

@@ -53,25 +53,48 @@ __global__ __launch_bounds__(256) void sum_tiles_kernel(const void* x, void* out
   }
 }
 
-// Reads `bytes` once, 16 bytes per lane and load (with the non-temporal hint the serving kernels give
-// their weight loads), PER loads in flight per lane, and writes one word per workgroup: the least any
-// kernel that streams a buffer of this size can take.
-template <int PER>
-__global__ __launch_bounds__(256) void read_probe_kernel(const uint4* p, int64_t vecs, uint32_t* out) {
-  uint32_t acc = 0u;
-  const int64_t base = (int64_t)blockIdx.x * 256 * PER + threadIdx.x;
+// Reads `bytes` once and does nothing else.  A workgroup of 256 lanes takes chunks of 256 * U * 16 bytes, chunk
+// c = blockIdx.x + i * gridDim.x (a grid of as many workgroups as chunks reads one chunk each), U loads of 16
+// bytes per lane in flight, each wave load one contiguous KiB; POLICY is the cache policy of the buffer loads
+// (bit 1 = the non-temporal hint the serving kernels give their weight loads).  One checksum word per
+// workgroup leaves, and, where asked for, the workgroup's first and last reading of the device's constant-rate
+// clock, from which the host takes the span of the launch without the time to launch it.
+template <int U, int POLICY>
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint8_t* src, uint32_t bytes, int nchunks, uint32_t* out,
+                                                         unsigned long long* stamps) {
+  typedef int v4i __attribute__((ext_vector_type(4)));
+  const int tid = threadIdx.x;
+  unsigned long long t0 = 0;
+  if (stamps != nullptr && tid == 0) t0 = wall_clock64();
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, (int)bytes, 0x00020000u);
+  v4i acc = {0, 0, 0, 0};
+  for (int c = blockIdx.x; c < nchunks; c += gridDim.x) {
+    const uint32_t cb = (uint32_t)c * (256u * U * 16u);
+    v4i v[U];
 #pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    const int64_t i = base + (int64_t)j * 256;
-    if (i < vecs) {
-      typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-      const v4u v = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p + i));
-      acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
-    }
+    for (int u = 0; u < U; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, tid * 16 + u * 4096, cb, POLICY);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u];
   }
+  uint32_t x = (uint32_t)(acc[0] ^ acc[1] ^ acc[2] ^ acc[3]);
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, 64);
-  if ((threadIdx.x & 63) == 0) atomicXor(out + blockIdx.x, acc);
+  for (int off = 32; off > 0; off >>= 1) x ^= __shfl_xor(x, off, 64);
+  if ((tid & 63) == 0) atomicXor(out + blockIdx.x, x);
+  if (stamps != nullptr && tid == 0) {
+    stamps[2 * blockIdx.x] = t0;
+    stamps[2 * blockIdx.x + 1] = wall_clock64();
+  }
+}
+
+template <int POLICY>
+void launch_read_probe(int loads, dim3 grid, hipStream_t st, const uint8_t* src, uint32_t bytes, int nchunks, uint32_t* out,
+                       unsigned long long* stamps) {
+  switch (loads) {
+    case 2: read_probe_kernel<2, POLICY><<<grid, 256, 0, st>>>(src, bytes, nchunks, out, stamps); break;
+    case 4: read_probe_kernel<4, POLICY><<<grid, 256, 0, st>>>(src, bytes, nchunks, out, stamps); break;
+    case 8: read_probe_kernel<8, POLICY><<<grid, 256, 0, st>>>(src, bytes, nchunks, out, stamps); break;
+    default: read_probe_kernel<16, POLICY><<<grid, 256, 0, st>>>(src, bytes, nchunks, out, stamps); break;
+  }
 }
 
 }  // namespace
@@ -79,18 +102,40 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* p, int64_t
 
 using namespace aqtx;
 
-extern "C" int aqtx_read_probe(const void* src, int64_t bytes, void* out_words, int64_t out_count, void* stream) {
+extern "C" int aqtx_read_probe(const void* src, int64_t bytes, int32_t workgroups, int32_t loads_in_flight,
+                               int32_t cache_policy, void* out_words, uint64_t* stamps, int32_t* wall_clock_khz,
+                               void* stream) {
   clear_error();
-  AQTX_REQUIRE(bytes >= 0 && bytes % 16 == 0, "aqtx_read_probe: bytes must be a non-negative multiple of 16");
+  AQTX_REQUIRE(bytes >= 0 && bytes % 16 == 0 && bytes < (1ll << 31), "aqtx_read_probe: bytes must be a multiple of 16 below 2 GiB");
+  AQTX_REQUIRE(loads_in_flight == 2 || loads_in_flight == 4 || loads_in_flight == 8 || loads_in_flight == 16,
+               "aqtx_read_probe: loads_in_flight must be 2, 4, 8 or 16");
+  AQTX_REQUIRE(cache_policy >= 0 && cache_policy <= 3, "aqtx_read_probe: cache_policy must be 0..3");
+  AQTX_REQUIRE(workgroups >= 0 && workgroups <= 65536, "aqtx_read_probe: at most 65536 workgroups");
+  if (wall_clock_khz != nullptr) {
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess)
+      return set_error("aqtx_read_probe: the device does not report its wall clock rate");
+    *wall_clock_khz = khz;
+  }
   if (bytes == 0) return 0;
   AQTX_REQUIRE(src != nullptr && out_words != nullptr, "aqtx_read_probe: NULL buffer");
   AQTX_REQUIRE(((uintptr_t)src % 16) == 0, "aqtx_read_probe: src must be 16-byte aligned");
-  constexpr int kPer = 16;  // 64 KiB per workgroup
-  const int64_t vecs = bytes / 16;
-  const int64_t blocks = (vecs + 256 * kPer - 1) / (256 * kPer);
-  AQTX_REQUIRE(blocks <= out_count && blocks < (1ll << 31), "aqtx_read_probe: out needs %lld words", (long long)blocks);
-  read_probe_kernel<kPer><<<(unsigned)blocks, 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
-      reinterpret_cast<const uint4*>(src), vecs, reinterpret_cast<uint32_t*>(out_words));
+  const int64_t chunk = 256ll * loads_in_flight * 16;
+  const int64_t nchunks = (bytes + chunk - 1) / chunk;
+  int64_t grid = workgroups == 0 ? nchunks : workgroups;
+  if (grid > nchunks) grid = nchunks;
+  AQTX_REQUIRE(grid <= 65536, "aqtx_read_probe: %lld chunks need a workgroup count (at most 65536 workgroups write words)",
+               (long long)nchunks);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const uint8_t* p = reinterpret_cast<const uint8_t*>(src);
+  uint32_t* out = reinterpret_cast<uint32_t*>(out_words);
+  unsigned long long* ts = reinterpret_cast<unsigned long long*>(stamps);
+  switch (cache_policy) {
+    case 0: launch_read_probe<0>(loads_in_flight, dim3((unsigned)grid), st, p, (uint32_t)bytes, (int)nchunks, out, ts); break;
+    case 1: launch_read_probe<1>(loads_in_flight, dim3((unsigned)grid), st, p, (uint32_t)bytes, (int)nchunks, out, ts); break;
+    case 2: launch_read_probe<2>(loads_in_flight, dim3((unsigned)grid), st, p, (uint32_t)bytes, (int)nchunks, out, ts); break;
+    default: launch_read_probe<3>(loads_in_flight, dim3((unsigned)grid), st, p, (uint32_t)bytes, (int)nchunks, out, ts); break;
+  }
   AQTX_HIP_CHECK_LAUNCH("read_probe_kernel");
   return 0;
 }

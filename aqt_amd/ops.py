@@ -495,17 +495,35 @@ def tile_weight(w_q: torch.Tensor, w_dtype: int = L.I8) -> torch.Tensor:
   return out
 
 
-def read_probe(buf: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-  """Streams `buf` once through the library's read-only kernel (a measurement aid); returns the
-  per-workgroup checksum words."""
+def read_probe(buf: torch.Tensor, out: Optional[torch.Tensor] = None, *, workgroups: int = 512, loads_in_flight: int = 4,
+               cache_policy: int = 2, stamps: Optional[torch.Tensor] = None) -> torch.Tensor:
+  """Streams `buf` once through the library's read-only kernel (a measurement aid, not part of any product
+  path); returns the checksum words, one per workgroup.  workgroups = 0: one workgroup per chunk of
+  256 * loads_in_flight * 16 bytes; otherwise that many workgroups walk the chunks round-robin.  `stamps`
+  (int64 [2 * workgroups]) receives every workgroup's first and last device-clock reading (read_probe_span_us)."""
   _require_gpu(buf)
   assert buf.is_contiguous()
   nbytes = buf.numel() * buf.element_size()
-  words = (nbytes + 65535) // 65536
   if out is None:
-    out = torch.zeros(max(words, 1), dtype=torch.int32, device=buf.device)
-  L.check(L.lib().aqtx_read_probe(_ptr(buf), nbytes, _ptr(out), out.numel(), _stream()))
+    out = torch.zeros(65536, dtype=torch.int32, device=buf.device)
+  assert out.numel() >= 65536 and (stamps is None or (stamps.dtype == torch.int64 and stamps.numel() >= 2 * 65536))
+  L.check(L.lib().aqtx_read_probe(_ptr(buf), nbytes, workgroups, loads_in_flight, cache_policy, _ptr(out), _ptr(stamps),
+                                  None, _stream()))
   return out
+
+
+def read_probe_workgroups(nbytes: int, workgroups: int, loads_in_flight: int) -> int:
+  """Workgroups a read_probe launch has (it never has more than chunks)."""
+  nchunks = -(-nbytes // (256 * loads_in_flight * 16))
+  return nchunks if workgroups == 0 else min(workgroups, nchunks)
+
+
+def read_probe_span_us(stamps: torch.Tensor, workgroups: int) -> float:
+  """Span of the read_probe launch that wrote `stamps`: last workgroup's end minus first workgroup's start."""
+  khz = ctypes.c_int32(0)
+  L.check(L.lib().aqtx_read_probe(None, 0, 0, 4, 0, None, None, ctypes.byref(khz), None))
+  s = stamps[:2 * workgroups].cpu().numpy().reshape(-1, 2)
+  return float(int(s[:, 1].max()) - int(s[:, 0].min())) * 1e3 / khz.value
 
 
 def pack_i4(q: torch.Tensor) -> torch.Tensor:

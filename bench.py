@@ -81,6 +81,9 @@ def decode_bench(dev):
   from aqt_amd import ops
   k = 4096
   rows = []
+  # the pure reader on the same bytes, the same way (HIP graph replay, 1 GiB rotation): what "as fast as the
+  # memory system reads this weight once" means on this box
+  ceiling, _ = read_ceiling(dev, sizes=[4096 * k // 2, 4096 * k, 14336 * k // 2, 14336 * k])
   # weights in this library's serving format (MFMA fragment order, what a frozen layer keeps) and,
   # for int8, also as plain rows [n][k] (what a caller holding the reference's layout passes)
   for w_kind, layout in (('int8', 'fragments'), ('int4_packed', 'fragments'), ('int8', 'rows')):
@@ -99,31 +102,12 @@ def decode_bench(dev):
         kw['w_layout'] = L.W_FRAGMENTS
       for m in (1, 8, 32, 64):
         x = torch.randn(m, k, device=dev).to(torch.bfloat16)
-        run = lambda: [ops.decode(x, w, w_scale, **kw) for w in weights]
-        run()
-        torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-          run()
-          torch.cuda.synchronize()
-          with torch.cuda.graph(graph, stream=side):
-            keep = run()
-        torch.cuda.synchronize()
-        graph.replay()
-        torch.cuda.synchronize()
-        reps = 5
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(reps):
-          graph.replay()
-        b.record()
-        torch.cuda.synchronize()
-        us = a.elapsed_time(b) * 1e3 / (reps * ncopies)
+        us = _graph_replay_us(lambda: [ops.decode(x, w, w_scale, **kw) for w in weights], ncopies)
         nbytes = int(k * n * wbytes_per) + 4 * n + 2 * m * k + 2 * m * n
         rows.append({'weights': w_kind, 'layout': layout, 'n': n, 'm': m, 'us_per_call': round(us, 2),
-                     'GB/s': round(nbytes / us / 1e3, 1), 'frac_of_8TBps': round(nbytes / us / 1e3 / 8000.0, 3)})
-        del graph, keep
+                     'GB/s': round(nbytes / us / 1e3, 1), 'frac_of_8TBps': round(nbytes / us / 1e3 / 8000.0, 3),
+                     'pure_read_of_the_weight_us': ceiling[int(k * n * wbytes_per)]['us_per_read'],
+                     'frac_of_pure_read': round(ceiling[int(k * n * wbytes_per)]['us_per_read'] / us, 3)})
       del weights
   return rows
 
@@ -368,45 +352,82 @@ def other_configs(dev):
   return out
 
 
-def read_floor(dev):
-  """What this box's memory system delivers to a kernel that only reads a decode-sized weight once
-  (aqtx_read_probe: coalesced 16 bytes per lane, one checksum word per workgroup, nothing else),
-  measured the way decode_bench measures: the buffers rotate through 1 GiB and the calls are
-  replayed from a HIP graph.  The decode kernels cannot be faster than this; prints one JSON line."""
+def _graph_replay_us(run, ncalls, reps=5):
+  """Device time per call of the `ncalls` launches `run` makes, replayed `reps` times from one HIP graph."""
+  import torch
+  run()
+  torch.cuda.synchronize()
+  side = torch.cuda.Stream()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.stream(side):
+    run()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+      keep = run()
+  torch.cuda.synchronize()
+  graph.replay()
+  torch.cuda.synchronize()
+  a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  a.record()
+  for _ in range(reps):
+    graph.replay()
+  b.record()
+  torch.cuda.synchronize()
+  us = a.elapsed_time(b) * 1e3 / (reps * ncalls)
+  del graph, keep
+  return us
+
+
+# launch shapes of the pure reader that came out on top of the full sweep (read_ceiling(full=True)) at the
+# serving weights' sizes: (workgroups, 16-byte loads in flight per lane, cache policy)
+_READER_SHAPES = ((512, 4, 2), (512, 4, 3), (1024, 2, 2), (512, 8, 2), (256, 8, 2), (1024, 4, 2))
+
+
+def read_ceiling(dev, full=False, sizes=None):
+  """What this box's memory system delivers to a kernel that only reads a buffer once (aqtx_read_probe: each
+  wave load one contiguous KiB, one checksum word per workgroup, nothing else).  Two figures per launch shape:
+  'span_us' = last workgroup's end minus first workgroup's start on the device clock (median of 7 launches, no
+  launch overhead in it), and 'us_per_read' = back-to-back launches replayed from a HIP graph, the way
+  decode_bench times the serving calls; buffers rotate through >= 1 GiB either way.  full: the sweep over
+  sizes (the two int8 serving weights, 256 MiB, 1 GiB), workgroups per CU (one chunk per workgroup, or 1 / 2 / 4 /
+  8 / 16 persistent ones), loads in flight per lane (2..16 x 16 bytes) and cache policy; otherwise the few shapes
+  that won that sweep, at the given sizes.  Returns {bytes: best row} and all rows."""
   import torch
   from aqt_amd import ops
-  rows = []
-  for n in (4096, 14336):
-    for scale, what in ((1.0, 'int8'), (0.5, 'packed int4')):
-      nbytes = int(n * 4096 * scale)
-      ncopies = (1 << 30) // nbytes + 1
-      bufs = [torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device=dev) for _ in range(ncopies)]
-      out = torch.zeros(nbytes // 65536 + 1, dtype=torch.int32, device=dev)
-      run = lambda: [ops.read_probe(b, out) for b in bufs]
-      run()
-      torch.cuda.synchronize()
-      side = torch.cuda.Stream()
-      graph = torch.cuda.CUDAGraph()
-      with torch.cuda.stream(side):
-        run()
+  cus = torch.cuda.get_device_properties(dev).multi_processor_count
+  if sizes is None:
+    sizes = [4096 * 4096, 14336 * 4096, 256 << 20, 1 << 30] if full else [4096 * 4096, 14336 * 4096]
+  if full:
+    shapes = [(w * cus if w else 0, u, pol) for pol in (0, 2, 3) for u in (2, 4, 8, 16) for w in (0, 1, 2, 4, 8, 16)]
+  else:
+    shapes = list(_READER_SHAPES)
+  out_words = torch.zeros(65536, dtype=torch.int32, device=dev)
+  stamps = torch.zeros(2 * 65536, dtype=torch.int64, device=dev)
+  rows, best = [], {}
+  for nbytes in sizes:
+    ncopies = max(2, (1 << 30) // nbytes + 1)
+    pool = torch.randint(-128, 128, (ncopies * nbytes,), dtype=torch.int8, device=dev)
+    bufs = [pool[i * nbytes:(i + 1) * nbytes] for i in range(ncopies)]
+    for wg, u, pol in shapes:
+      nwg = ops.read_probe_workgroups(nbytes, wg, u)
+      if nwg > 65536 or (wg and nwg < wg):
+        continue
+      kw = dict(workgroups=wg, loads_in_flight=u, cache_policy=pol)
+      spans = []
+      for i in range(8):
+        ops.read_probe(bufs[i % ncopies], out_words, stamps=stamps, **kw)
         torch.cuda.synchronize()
-        with torch.cuda.graph(graph, stream=side):
-          run()
-      torch.cuda.synchronize()
-      graph.replay()
-      torch.cuda.synchronize()
-      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-      a.record()
-      for _ in range(5):
-        graph.replay()
-      b.record()
-      torch.cuda.synchronize()
-      us = a.elapsed_time(b) * 1e3 / (5 * ncopies)
-      rows.append({'weight': f'{n}x4096 {what}', 'bytes': nbytes, 'us_per_read': round(us, 2),
-                   'GB/s': round(nbytes / us / 1e3, 1)})
-      del graph, bufs
-  print(json.dumps({'read_floor': 'aqtx_read_probe over a buffer of the weight size, HIP graph replay, 1 GiB rotation',
-                    'rows': rows}))
+        spans.append(ops.read_probe_span_us(stamps, nwg))
+      span = sorted(spans[1:])[3]
+      us = _graph_replay_us(lambda: [ops.read_probe(b, out_words, **kw) for b in bufs], ncopies, reps=3)
+      row = {'bytes': nbytes, 'workgroups': nwg, 'per_cu': round(nwg / cus, 2) if wg else 'one chunk each',
+             'loads_in_flight': u, 'cache_policy': pol, 'span_us': round(span, 2), 'span_TB/s': round(nbytes / span / 1e6, 2),
+             'us_per_read': round(us, 2), 'TB/s': round(nbytes / us / 1e6, 2)}
+      rows.append(row)
+      if nbytes not in best or us < best[nbytes]['us_per_read']:
+        best[nbytes] = row
+    del bufs, pool
+  return best, rows
 
 
 def decode_probe(dev, calibration_copy=False):
@@ -426,9 +447,8 @@ def decode_probe(dev, calibration_copy=False):
     raw = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(ncopies)]
     weights = [ops.tile_weight(w, L.I8) for w in raw]
     w_scale = torch.rand(n, device=dev) * 1e-3 + 1e-5
-    out = torch.zeros(n * k // 65536 + 1, dtype=torch.int32, device=dev)
     for w in raw:
-      ops.read_probe(w, out)
+      ops.read_probe(w)
     for m in (1, 8, 64):
       x = torch.randn(m, k, device=dev).to(torch.bfloat16)
       for w in weights:
@@ -496,8 +516,9 @@ def main():
                        'distribution (and the vendor int8 GEMM beside them) and exit')
   ap.add_argument('--decode-probe', action='store_true',
                   help='only issue a few serving calls per shape (for rocprofv3 runs) and exit')
-  ap.add_argument('--read-floor', action='store_true',
-                  help='only time a pure read of decode-sized buffers (the memory floor of the serving kernels) and exit')
+  ap.add_argument('--read-ceiling', action='store_true',
+                  help='only sweep a pure reader over buffer sizes and launch shapes (what the memory system delivers '
+                       'to a single pass over the serving weights and over 256 MiB / 1 GiB) and exit')
   args = ap.parse_args()
   if args.gpus != 1:
     print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)',
@@ -515,8 +536,12 @@ def main():
   if args.gemm_probe is not None:
     gemm_probe(dev, args.gemm_probe)
     return
-  if args.read_floor:
-    read_floor(dev)
+  if args.read_ceiling:
+    best, rows = read_ceiling(dev, full=True)
+    for r in rows:
+      print(json.dumps(r))
+    print(json.dumps({'read_ceiling': 'best launch shape per size (back-to-back launches from a HIP graph, 1 GiB rotation)',
+                      'best': [best[b] for b in sorted(best)]}))
     return
   if args.decode_probe:
     decode_probe(dev, args.calibration_copy)

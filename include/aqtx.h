@@ -493,12 +493,19 @@ int aqtx_random_bits(const uint32_t key_host[2], int64_t n, int32_t bit_width,
                      int32_t partitionable, void* out, void* stream);
 
 /*
- * aqtx_read_probe: a measurement aid with no counterpart in the reference.  Streams `bytes` (a multiple of
- * 16) from src once, coalesced 16 bytes per lane, 64 KiB per workgroup, and XORs one checksum word per
- * workgroup into out_words[0 .. ceil(bytes / 65536)): the floor for the device time of any kernel that has
- * to read a buffer of that size once (the serving kernels are measured against it).
+ * aqtx_read_probe: a measurement aid with no counterpart in the reference and no use in the product path.
+ * Streams `bytes` (a multiple of 16, below 2 GiB) from src once and does nothing else, so that the serving
+ * kernels can be set against what the memory system delivers to a pure reader of the same bytes.  The launch
+ * shape is the caller's: `workgroups` of 256 lanes walk chunks of 256 * loads_in_flight * 16 bytes round-robin
+ * (0 = one workgroup per chunk), loads_in_flight (2 | 4 | 8 | 16) loads of 16 bytes per lane are in flight, a
+ * wave load is one contiguous KiB, cache_policy (0..3) is the cache-policy field of the buffer loads (bit 1 =
+ * non-temporal).  out_words: uint32 [65536] DEVICE, one checksum word per workgroup XORed in.  stamps: optional
+ * uint64 [2 * workgroups] DEVICE: every workgroup's first and last reading of the constant-rate device clock,
+ * whose rate in kHz goes to *wall_clock_khz (optional, HOST): max(last) - min(first) is the span of the launch.
  */
-int aqtx_read_probe(const void* src, int64_t bytes, void* out_words, int64_t out_count, void* stream);
+int aqtx_read_probe(const void* src, int64_t bytes, int32_t workgroups, int32_t loads_in_flight,
+                    int32_t cache_policy, void* out_words, uint64_t* stamps, int32_t* wall_clock_khz,
+                    void* stream);
 
 /* Message of the calling thread's most recent failure ("" if none). */
 const char* aqtx_last_error(void);

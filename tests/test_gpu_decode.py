@@ -306,13 +306,21 @@ def test_decode_fragment_ordered_weight(gpu, packed, m, n, k):
     np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
 
 
-def test_read_probe_reads_every_byte(gpu):
-  """The read-floor kernel's checksum is the XOR of all 32-bit words of its 64 KiB share."""
-  buf = torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * 16384 + 52,), dtype=torch.int32, device=gpu)
-  got = ops.read_probe(buf).cpu().numpy().view(np.uint32)
+@pytest.mark.parametrize('workgroups,loads,policy', [(0, 16, 2), (0, 2, 0), (3, 4, 2), (512, 8, 3), (7, 16, 1)])
+def test_read_probe_reads_every_byte(gpu, workgroups, loads, policy):
+  """The read-only kernel's checksum words: workgroup w holds the XOR of all 32-bit words of the chunks
+  w, w + workgroups, ... (chunks of 256 * loads * 16 bytes; the last one ragged)."""
+  buf = torch.randint(-2 ** 31, 2 ** 31 - 1, (11 * 16384 + 52,), dtype=torch.int32, device=gpu)
+  stamps = torch.zeros(2 * 65536, dtype=torch.int64, device=gpu)
+  got = ops.read_probe(buf, workgroups=workgroups, loads_in_flight=loads, cache_policy=policy, stamps=stamps)
   words = buf.cpu().numpy().view(np.uint32)
-  want = [np.bitwise_xor.reduce(words[i:i + 16384]) for i in range(0, len(words), 16384)]
-  np.testing.assert_array_equal(got, np.asarray(want, dtype=np.uint32))
+  cw = 256 * loads * 4
+  chunks = [np.bitwise_xor.reduce(words[i:i + cw]) for i in range(0, len(words), cw)]
+  nwg = ops.read_probe_workgroups(buf.numel() * 4, workgroups, loads)
+  want = [np.bitwise_xor.reduce(np.asarray(chunks[w::nwg], dtype=np.uint32)) for w in range(nwg)]
+  np.testing.assert_array_equal(got.cpu().numpy().view(np.uint32)[:nwg], np.asarray(want, dtype=np.uint32))
+  assert not got[nwg:].any()
+  assert 0.0 < ops.read_probe_span_us(stamps, nwg) < 1e4
 
 
 # ---- weight-only serving (the lhs stays bf16; float32 sums: tolerance, not bits) ----------------------------
