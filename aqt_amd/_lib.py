@@ -121,6 +121,7 @@ SYMBOLS = {
     'aqtx_decode_exchange_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),
     'aqtx_tile_weight_bytes': (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int32]),
     'aqtx_tile_weight': (ctypes.c_int, [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, _vp]),
+    'aqtx_decode_i8_check': (ctypes.c_int, [_vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_i8_static': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_decode_weight_only': (ctypes.c_int, [ctypes.POINTER(DecodePlan), _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     'aqtx_decode_weight_only_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(DecodePlan)]),

@@ -19,6 +19,7 @@ namespace aqtx {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned short dq_u16x2 __attribute__((ext_vector_type(2)));
 
 constexpr uint32_t kBufferRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format (gfx9)
 constexpr int kOob = 0x7FFFFFF0;                     // offset that is out of range for every buffer
@@ -57,7 +58,26 @@ struct DecodeArgs {
   // wave's load is one contiguous KiB; rows past n and bytes past the row end are zero.
   int w_frag;             // 1: fragment order
   int w_steps;            // fragment order: 64-byte steps of one row block
+  // Activation quantisation inside the contraction launch (decode_tile_kernel): the first `nprod` workgroups of
+  // grid row 0 quantize one token each (quant_token_publish) and count themselves in each of kWaitGroups arrival
+  // words.  The other workgroups start their weight stream, wait until the arrival word of their group
+  // (workgroup number % kWaitGroups) reaches wait_target (at most wait_ticks of the 100 MHz device clock), and
+  // count themselves out in their group's departure word when they are done; the last of a group clears the
+  // group's two words.  The words lie 128 bytes apart: read-modify-writes on one line take turns at the memory
+  // side, about 10 ns each, which hundreds of workgroups on one word would turn into microseconds.  ctrl[1]
+  // collects expired waits.
+  int nprod;              // 0: the activations were quantized by decode_quant_kernel before this launch
+  int prod_per_token;     // 1: a producer quantizes a whole token; 4: a quarter of each of its 16-value pieces
+  int* ctrl;              // kControlBytes, zero on entry and (no wait having expired) on exit
+  int wait_target;        // nprod (a test makes it unreachable)
+  unsigned wait_ticks;
 };
+
+constexpr int kWaitGroups = 16;
+constexpr int kLineWords = 32;  // 128 bytes
+constexpr size_t kControlBytes = (size_t)(1 + 2 * kWaitGroups) * kLineWords * 4 + 128;  // 4352: a multiple of 256
+__device__ __forceinline__ int* wait_flag(int* ctrl, int g) { return ctrl + (1 + 2 * g) * kLineWords; }
+__device__ __forceinline__ int* departures(int* ctrl, int g) { return ctrl + (2 + 2 * g) * kLineWords; }
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
 
@@ -267,7 +287,6 @@ __global__ __launch_bounds__(256) void decode_fused_kernel(const DecodeArgs d) {
 // request the weights (before the quantisation) and contract.  Rows are written to LDS as in the
 // kernel above.  k <= 4096 * PPT.  The host uses it for ROWS = 4 only: the work every workgroup
 // repeats grows with the rows, the launch it saves does not.
-typedef unsigned short dq_u16x2 __attribute__((ext_vector_type(2)));
 template <typename TIn, int ROWS, int PPT, int U, bool PACKED, bool WFRAG>
 __global__ __launch_bounds__(1024) void decode_wide_kernel(const DecodeArgs d) {
   static_assert(ROWS % 4 == 0 && ROWS <= 16, "rows come in fours");
@@ -562,6 +581,173 @@ __global__ __launch_bounds__(256) void decode_quant_kernel(const DecodeArgs d, u
   }
 }
 
+// Quantisation of a token inside the contraction launch, by one workgroup or by four (d.prod_per_token): each
+// finds the row's abs-max (the whole row: 16 values per thread and pass); one quantizes every 16-value piece,
+// of four each quantizes a quarter of every piece, four values per thread (fewer instructions between the
+// arrival of the row and its stores, but four times the workgroups: for few tokens).  The arithmetic is that of decode_quant_kernel: scale = dtype(absmax / bound),
+// inv = dtype(1 / scale), q = rint(clip(dtype(x * inv))) (clip with one v_med3, round to nearest even and
+// convert with one addition of 1.5 * 2^23: |t| <= 127 there).  The int8 values go to the fragment-ordered copy.
+// The workgroups that read them run on other XCDs, whose L2s this one's stores do not reach on their own: scale
+// and fragments leave with device scope (written through to memory), the workgroup waits until all of them are
+// complete, and only then counts itself in the readers' arrival words with device-scope read-modify-writes.
+// Readers touch the copy only after they have seen every producer counted, so no L2 can hold a line of it from
+// before.  Up to two 16-value pieces per thread stay in registers between the passes; longer rows are read twice.
+__device__ __forceinline__ void quant_token_publish(const DecodeArgs& d, const int row, const int quarter) {
+  __shared__ float smax[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int pieces = d.k / 16;
+  const int pw = d.x_bf16 ? 8 : 16;  // 32-bit words of one 16-value input piece
+  const uint8_t* xr = reinterpret_cast<const uint8_t*>(d.x) + (int64_t)row * d.k * (d.x_bf16 ? 2 : 4);
+  const __amdgpu_buffer_rsrc_t rf = make_rsrc(d.xq_frag, (int64_t)((d.k + 127) / 128) * 2 * d.mb_total * 1024);
+  auto frag_off = [&](int p) __attribute__((always_inline)) {
+    const int step = d.frag_halves == 2 ? p >> 3 : p >> 2;
+    const int c = d.frag_halves == 2 ? (p & 7) >> 1 : p & 3;
+    const int h = d.frag_halves == 2 ? p & 1 : 0;
+    return (((step * d.mb_total + (row >> 4)) * d.frag_halves + h) << 10) + c * 256 + (row & 15) * 16;
+  };
+  auto load_piece = [&](int p, uint32_t* dst) __attribute__((always_inline)) {
+    const uint4 t0 = *reinterpret_cast<const uint4*>(xr + (int64_t)p * pw * 4);
+    const uint4 t1 = *reinterpret_cast<const uint4*>(xr + (int64_t)p * pw * 4 + 16);
+    dst[0] = t0.x; dst[1] = t0.y; dst[2] = t0.z; dst[3] = t0.w; dst[4] = t1.x; dst[5] = t1.y; dst[6] = t1.z; dst[7] = t1.w;
+    if (!d.x_bf16) {
+      const uint4 t2 = *reinterpret_cast<const uint4*>(xr + (int64_t)p * pw * 4 + 32);
+      const uint4 t3 = *reinterpret_cast<const uint4*>(xr + (int64_t)p * pw * 4 + 48);
+      dst[8] = t2.x; dst[9] = t2.y; dst[10] = t2.z; dst[11] = t2.w; dst[12] = t3.x; dst[13] = t3.y; dst[14] = t3.z; dst[15] = t3.w;
+    }
+  };
+  auto piece_absmax = [&](const uint32_t* w, float amax) __attribute__((always_inline)) -> float {
+    if (d.x_bf16) {
+      // two bf16 magnitudes per word: they order like unsigned integers, NaN patterns above infinity
+      uint32_t m2 = 0u;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const dq_u16x2 a2 = __builtin_bit_cast(dq_u16x2, m2), b2 = __builtin_bit_cast(dq_u16x2, w[q] & 0x7FFF7FFFu);
+        m2 = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a2, b2));
+      }
+      return nanmax(amax, nanmax(__uint_as_float(m2 << 16), __uint_as_float(m2 & 0xFFFF0000u)));
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) amax = absmax_step(amax, __uint_as_float(w[e]));
+    return amax;
+  };
+  const bool held = pieces <= 512;
+  uint32_t raw[2][16];
+  float amax = 0.0f;
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int p = tid + 256 * j;
+      if (p < pieces) {
+        load_piece(p, raw[j]);
+        amax = piece_absmax(raw[j], amax);
+      }
+    }
+  } else {
+    for (int p = tid; p < pieces; p += 256) {
+      load_piece(p, raw[0]);
+      amax = piece_absmax(raw[0], amax);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) amax = nanmax(amax, __shfl_xor(amax, off, 64));
+  if (lane == 0) smax[wave] = amax;
+  __syncthreads();
+  amax = nanmax(nanmax(smax[0], smax[1]), nanmax(smax[2], smax[3]));
+  if (amax == 0.0f) amax = 1.0f;
+  float sc = rnd(amax / d.quant_bound, d.x_bf16);
+  sc = rnd(sc, d.xs_bf16);
+  float inv = rnd(1.0f / sc, d.xs_bf16);
+  if (isinf(inv)) inv = 1.0f;
+  if (tid == 0 && quarter == 0) __hip_atomic_store(d.x_scale_out + row, sc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const int tbf = d.x_bf16 & d.xs_bf16;
+  constexpr int kDeviceScope = 16;  // the sc1 bit of the store's cache policy: written through to memory
+  // values 4 * quarter .. + 3 of piece p -> one word of the fragment-ordered copy
+  auto quant_quarter = [&](const uint32_t* w, int p) __attribute__((always_inline)) {
+    // the quarter's four values as float32 patterns: every word is read into a scalar of its own first (a
+    // choice between array elements would become a computed address and send the array to scratch memory)
+    uint32_t f4[4];
+    if (d.x_bf16) {
+      const uint32_t a0 = w[0], a1 = w[1], a2 = w[2], a3 = w[3], a4 = w[4], a5 = w[5], a6 = w[6], a7 = w[7];
+      const uint32_t lo = quarter == 0 ? a0 : quarter == 1 ? a2 : quarter == 2 ? a4 : a6;
+      const uint32_t hi = quarter == 0 ? a1 : quarter == 1 ? a3 : quarter == 2 ? a5 : a7;
+      f4[0] = lo << 16; f4[1] = lo & 0xFFFF0000u; f4[2] = hi << 16; f4[3] = hi & 0xFFFF0000u;
+    } else {
+      const uint32_t a0 = w[0], a1 = w[1], a2 = w[2], a3 = w[3], a4 = w[4], a5 = w[5], a6 = w[6], a7 = w[7];
+      const uint32_t a8 = w[8], a9 = w[9], a10 = w[10], a11 = w[11], a12 = w[12], a13 = w[13], a14 = w[14], a15 = w[15];
+      f4[0] = quarter == 0 ? a0 : quarter == 1 ? a4 : quarter == 2 ? a8 : a12;
+      f4[1] = quarter == 0 ? a1 : quarter == 1 ? a5 : quarter == 2 ? a9 : a13;
+      f4[2] = quarter == 0 ? a2 : quarter == 1 ? a6 : quarter == 2 ? a10 : a14;
+      f4[3] = quarter == 0 ? a3 : quarter == 1 ? a7 : quarter == 2 ? a11 : a15;
+    }
+    uint32_t b[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v = __uint_as_float(f4[e]);
+      float t = rnd(v * inv, tbf);
+      t = __builtin_amdgcn_fmed3f(t, -d.clip_bound, d.clip_bound);
+      b[e] = __float_as_uint(t + 12582912.0f);
+    }
+    const uint32_t lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);   // bytes b0 b1 0 0
+    const uint32_t hi = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);   // bytes 0 0 b2 b3
+    const uint32_t q = lo | hi;
+    __builtin_amdgcn_raw_buffer_store_b32((int)q, rf, frag_off(p) + 4 * quarter, 0, kDeviceScope);
+    if (d.xq_out != nullptr) *reinterpret_cast<uint32_t*>(d.xq_out + (int64_t)row * d.k + (int64_t)p * 16 + 4 * quarter) = q;
+  };
+  // a whole piece: sixteen values, one 16-byte store
+  auto quant_piece = [&](const uint32_t* w, int p) __attribute__((always_inline)) {
+    uint32_t q[4];
+#pragma unroll
+    for (int w4 = 0; w4 < 4; ++w4) {
+      uint32_t b[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * w4 + e;
+        const float v = d.x_bf16 ? __uint_as_float((i & 1) ? (w[i >> 1] & 0xFFFF0000u) : (w[i >> 1] << 16)) : __uint_as_float(w[i]);
+        float t = rnd(v * inv, tbf);
+        t = __builtin_amdgcn_fmed3f(t, -d.clip_bound, d.clip_bound);
+        b[e] = __float_as_uint(t + 12582912.0f);
+      }
+      q[w4] = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u) | __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(v4i{(int)q[0], (int)q[1], (int)q[2], (int)q[3]}, rf, frag_off(p), 0, kDeviceScope);
+    if (d.xq_out != nullptr)
+      *reinterpret_cast<uint4*>(d.xq_out + (int64_t)row * d.k + (int64_t)p * 16) = make_uint4(q[0], q[1], q[2], q[3]);
+  };
+  if (d.prod_per_token == 1) {
+    if (held) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int p = tid + 256 * j;
+        if (p < pieces) quant_piece(raw[j], p);
+      }
+    } else {
+      for (int p = tid; p < pieces; p += 256) {
+        load_piece(p, raw[0]);
+        quant_piece(raw[0], p);
+      }
+    }
+  } else if (held) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int p = tid + 256 * j;
+      if (p < pieces) quant_quarter(raw[j], p);
+    }
+  } else {
+    for (int p = tid; p < pieces; p += 256) {
+      load_piece(p, raw[0]);
+      quant_quarter(raw[0], p);
+    }
+  }
+  // every store of every thread complete (vmcnt counts stores too on this target), then the count
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  // one count per group of waiting workgroups, lane g the count of group g (nothing comes back: the lanes'
+  // additions travel together); only groups that have a member: a count nobody waits for would have nobody to clear it
+  const int waiting = ((int)gridDim.x - d.nprod) * (int)gridDim.y;
+  if (tid < kWaitGroups && tid < waiting)
+    __hip_atomic_fetch_add(wait_flag(d.ctrl, tid), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Phase 2.  A workgroup owns 16*NB weight rows, all m <= 16*MB tokens and one K range
 // (blockIdx.y); its four waves take a quarter of that range each.  A wave streams its weight
 // fragments from HBM and its activation fragments (fragment order, contiguous KiB) from L2
@@ -581,19 +767,42 @@ __global__ __launch_bounds__(256) void decode_quant_kernel(const DecodeArgs d, u
 // that element.  Device-scope atomic read-modify-writes are carried out at the memory side of the
 // per-XCD L2s, so the exchange needs no fence, no second round trip and no waiting loop.
 // PACKED: int4 weights two per byte; a lane's 16 bytes are 32 k = two MFMA steps.
-template <int MB, int NB, int D, bool PACKED>
-__global__ __launch_bounds__(256, (D * (NB + MB * (PACKED ? 2 : 1)) * 4 + MB * NB * 4 + 48 > 256) ? 1 : 2)
+//
+// With d.nprod the launch quantizes the activations itself (DecodeArgs::nprod): the first nprod workgroups are
+// producers and leave after quant_token_publish; the others request their first D steps of weights, wait for
+// the producers' count behind a bounded loop (one wave polls with a device-scope read-modify-write, the
+// workgroup leaves with ctrl[2] set if the wait expires: every wave reaches its end whatever happens to a
+// producer), and only then ask for scales and activation fragments.  The producers have the lowest workgroup
+// ids, so they are resident before any workgroup that waits for them.
+// DX: K steps of activation fragments in flight per wave (D: of weights).  DX < D is for the launches with
+// producers: the weights of D steps are requested before the wait and are there when it ends, the activations
+// come from the L2 afterwards and need little in flight; loads return in the order they were requested, so in
+// the steady state a wave never has more than DX steps of weights outstanding behind a fragment it waits for.
+// PROD: the launch has producers (d.nprod > 0); a template parameter, so that the launches without them keep the
+// registers and the instruction stream they had before producers existed.
+template <int MB, int NB, int D, bool PACKED, int DX = D, bool PROD = false>
+__global__ __launch_bounds__(256, (D * NB * 4 + DX * MB * (PACKED ? 2 : 1) * 4 + MB * NB * 4 + 48 > 256) ? 1 : 2)
 void decode_tile_kernel(const DecodeArgs d) {
+  static_assert(D % DX == 0, "the fragment ring divides the weight ring");
   constexpr int T = MB * NB;
   constexpr int TPW = (T + 3) / 4;  // 16x16 tiles a wave owns after the reduction: t = wave + 4*j < T
   __shared__ v4i red[4][T][64];
+  __shared__ int tokens_ready;
+  int bx = (int)blockIdx.x;
+  if constexpr (PROD) {
+    if (bx < d.nprod) {
+      if (blockIdx.y == 0) quant_token_publish(d, bx / d.prod_per_token, bx % d.prod_per_token);
+      return;
+    }
+    bx -= d.nprod;
+  }
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
   constexpr int KS = PACKED ? 128 : 64;  // k covered by one wave-wide weight load
   constexpr int KL = KS / 4;             // k covered by one lane's 16 bytes
   constexpr int XP = PACKED ? 2 : 1;     // activation fragments per weight fragment
-  const int n0 = blockIdx.x * (16 * NB);
+  const int n0 = bx * (16 * NB);
   const int kb = PACKED ? d.k / 2 : d.k;  // bytes of one weight row
   const int s_lo = blockIdx.y * d.k_slice;
   const int s_hi = (s_lo + d.k_slice) < d.k ? (s_lo + d.k_slice) : d.k;
@@ -607,7 +816,7 @@ void decode_tile_kernel(const DecodeArgs d) {
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int row = n0 + nb * 16 + r;
-    wbase[nb] = d.w_frag ? (int)(blockIdx.x * NB + nb) * d.w_steps * 1024 + lane * 16  // past n: reads zeros
+    wbase[nb] = d.w_frag ? (int)(bx * NB + nb) * d.w_steps * 1024 + lane * 16  // past n: reads zeros
                          : (row < d.n ? row : d.n - 1) * kb + c * 16;  // clamped; such columns are never stored
   }
 
@@ -624,28 +833,35 @@ void decode_tile_kernel(const DecodeArgs d) {
     const int nn = n0 + (wave % NB) * 16 + 4 * c;  // (wave + 4*j) % NB == wave % NB: NB divides 4
 #pragma unroll
     for (int e = 0; e < 4; ++e) ws[e] = d.w_scale[(nn + e) < d.n ? (nn + e) : (d.n - 1)];
+  }
+  auto load_token_scales = [&]() {
 #pragma unroll
     for (int j = 0; j < TPW; ++j) {
       const int mm = ((wave + 4 * j) / NB) * 16 + r;
       xs[j] = d.x_scale[mm < d.m ? mm : (d.m - 1)];
     }
-  }
+  };
+  if constexpr (!PROD) load_token_scales();  // otherwise behind the wait: the producers write them
 
   const unsigned wstep = d.w_frag ? 1024u : 64u;
-  v4i wf[D][NB], xf[D][MB][XP];
+  v4i wf[D][NB], xf[DX][MB][XP];
   // Steps past the end of the wave's range, lanes past the end of K and token blocks past m read
   // zeros: their offsets get the out-of-range bits ORed in (no memory access; no branch, which
   // would make the compiler drain the loads in flight).
+  // (with producers nobody writes the rows that pad the last 16-token block: their lanes read zeros too)
   unsigned xdead[MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) xdead[mb] = mb < d.mb_total ? 0u : (unsigned)kOob;
-  auto issue = [&](auto stream_c, int slot, int ko) {
+  for (int mb = 0; mb < MB; ++mb) xdead[mb] = (PROD ? mb * 16 + r < d.m : mb < d.mb_total) ? 0u : (unsigned)kOob;
+  auto issue_w = [&](auto stream_c, int slot, int ko) {
     constexpr int kPolicy = decltype(stream_c)::value ? kStreamOnce : 0;
     const unsigned dead = (ko + c * KL < k_hi) ? 0u : (unsigned)kOob;  // a lane's KL values are all inside or all outside
     const unsigned wk = (unsigned)(ko / KS) * wstep;  // a k step is 64 bytes of a row, or one KiB fragment
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       wf[slot][nb] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)(((unsigned)wbase[nb] + wk) | dead), 0, kPolicy);
+  };
+  auto issue_x = [&](int slot, int ko) {
+    const unsigned dead = (ko + c * KL < k_hi) ? 0u : (unsigned)kOob;
     const unsigned xstep = (unsigned)(ko / KS) * (unsigned)d.mb_total;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -654,7 +870,46 @@ void decode_tile_kernel(const DecodeArgs d) {
         xf[slot][mb][h] = __builtin_amdgcn_raw_buffer_load_b128(
             rx, (int)(((((xstep + mb) * XP + h) << 10) + (unsigned)lane * 16u) | dead | xdead[mb]), 0, 0);
   };
-  auto multiply = [&](int slot) {
+  auto issue = [&](auto stream_c, int slot, int ko) {
+    issue_w(stream_c, slot, ko);
+    issue_x(slot, ko);
+  };
+  // The bounded wait for the producers (see the kernel's header).  Returns whether the tokens are there.
+  const int wg_id = bx + (int)blockIdx.y * ((int)gridDim.x - d.nprod);
+  const int wgroup = wg_id % kWaitGroups;
+  auto wait_for_tokens = [&]() -> bool {
+    if (wave == 0) {
+      const unsigned long long t0 = wall_clock64();
+      int flag = 0;
+      for (;;) {
+        if (lane == 0) flag = __hip_atomic_load(wait_flag(d.ctrl, wgroup), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        flag = __builtin_amdgcn_readfirstlane(flag);
+        if (flag >= d.wait_target || wall_clock64() - t0 > d.wait_ticks) break;
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (lane == 0) {
+        if (flag < d.wait_target) __hip_atomic_fetch_or(d.ctrl + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        tokens_ready = flag >= d.wait_target ? 1 : 0;
+      }
+    }
+    lds_barrier();
+    return tokens_ready != 0;
+  };
+  // Counted out of the group; the last one out clears the group's words for the next call.  The count is asked
+  // for when the contraction is done and looked at after the outputs have left: nothing waits for it.
+  int left_before = 0;
+  auto depart = [&]() {
+    if (PROD && tid == 0)
+      left_before = __hip_atomic_fetch_add(departures(d.ctrl, wgroup), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  auto departed = [&]() {
+    const int total = ((int)gridDim.x - d.nprod) * (int)gridDim.y;
+    if (PROD && tid == 0 && left_before == (total - wgroup + kWaitGroups - 1) / kWaitGroups - 1) {
+      __hip_atomic_fetch_and(wait_flag(d.ctrl, wgroup), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_and(departures(d.ctrl, wgroup), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  auto multiply = [&](int slot, int xslot) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if constexpr (PACKED) {
@@ -664,13 +919,13 @@ void decode_tile_kernel(const DecodeArgs d) {
         const v4i b0 = v4i{t[0], t[1], t[2], t[3]}, b1 = v4i{t[4], t[5], t[6], t[7]};
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, xf[slot][mb][0], acc[mb][nb], 0, 0, 0);
-          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, xf[slot][mb][XP - 1], acc[mb][nb], 0, 0, 0);
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b0, xf[xslot][mb][0], acc[mb][nb], 0, 0, 0);
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b1, xf[xslot][mb][XP - 1], acc[mb][nb], 0, 0, 0);
         }
       } else {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[slot][nb], xf[slot][mb][0], acc[mb][nb], 0, 0, 0);
+          acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[slot][nb], xf[xslot][mb][0], acc[mb][nb], 0, 0, 0);
       }
     }
   };
@@ -679,7 +934,7 @@ void decode_tile_kernel(const DecodeArgs d) {
   // bytes at the same time.  Workgroup ids are dealt round-robin to the 8 XCDs, so id / 8
   // spreads the workgroups that share an L2 evenly over the steps.
   const int nsteps = kq / KS;
-  const int rot = (int)((blockIdx.x / 8 + blockIdx.y) % (unsigned)nsteps);
+  const int rot = (int)(((unsigned)bx / 8 + blockIdx.y) % (unsigned)nsteps);
   auto step_k = [&](int i) {
     int j = i + rot;
     j = j >= nsteps ? j - nsteps : j;
@@ -687,21 +942,47 @@ void decode_tile_kernel(const DecodeArgs d) {
   };
   // The weight loads carry the streaming hint when a wave load is a whole KiB fragment; the choice is made
   // once, outside the loop (a branch around a load would make the compiler drain the loads in flight).
-  auto walk = [&](auto stream_c) {
+  auto walk = [&](auto stream_c) -> bool {
+    if constexpr (PROD) {
 #pragma unroll
-    for (int s = 0; s < D; ++s) issue(stream_c, s, step_k(s));
+      for (int s = 0; s < D; ++s) issue_w(stream_c, s, step_k(s));
+      __builtin_amdgcn_sched_barrier(0);
+      if (!wait_for_tokens()) return false;
+#pragma unroll
+      for (int s = 0; s < DX; ++s) issue_x(s, step_k(s));
+      load_token_scales();  // behind the fragments: loads return in order, and these come from further away
+    } else if constexpr (DX == D) {
+#pragma unroll
+      for (int s = 0; s < D; ++s) issue(stream_c, s, step_k(s));
+    } else {
+#pragma unroll
+      for (int s = 0; s < D; ++s) issue_w(stream_c, s, step_k(s));
+#pragma unroll
+      for (int s = 0; s < DX; ++s) issue_x(s, step_k(s));
+    }
     __builtin_amdgcn_sched_barrier(0);
     for (int i = 0; i < nsteps; i += D) {
 #pragma unroll
       for (int s = 0; s < D; ++s) {
-        multiply(s);
+        multiply(s, s % DX);
         __builtin_amdgcn_sched_barrier(0);
-        issue(stream_c, s, step_k(i + D + s));
+        if constexpr (DX == D) {
+          issue(stream_c, s, step_k(i + D + s));
+        } else {
+          issue_x(s % DX, step_k(i + DX + s));
+          issue_w(stream_c, s, step_k(i + D + s));
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    return true;
   };
-  if (d.w_frag) walk(std::true_type{}); else walk(std::false_type{});
+  const bool walked = d.w_frag ? walk(std::true_type{}) : walk(std::false_type{});
+  depart();
+  if (!walked) {  // the wait expired (ctrl[1] says so): nothing is written
+    departed();
+    return;
+  }
   // lane holds C[n = n0 + nb*16 + 4c + e][m = mb*16 + r] in acc[mb][nb][e]
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
@@ -709,7 +990,7 @@ void decode_tile_kernel(const DecodeArgs d) {
     for (int nb = 0; nb < NB; ++nb) red[wave][mb * NB + nb][lane] = acc[mb][nb];
   __syncthreads();
   // thread -> the lane's four words of tiles t = wave + 4*j < T
-  int* tile_sums = d.sums + (int64_t)blockIdx.x * (T * 4 * 64);
+  int* tile_sums = d.sums + (int64_t)bx * (T * 4 * 64);
   const int one = 1 << d.count_shift, half = one >> 1;
   const bool wide_ok = (d.n % 4) == 0;  // 4 consecutive outputs of a row are then 8 / 16-byte aligned
   const int p1 = d.out_bf16 & d.xs_bf16;
@@ -768,6 +1049,7 @@ void decode_tile_kernel(const DecodeArgs d) {
         }
     }
   }
+  departed();
 }
 
 // Weight rows -> fragment order (see DecodeArgs): thread -> (16-row block, 64-byte k step, lane).
@@ -875,13 +1157,15 @@ TileShape choose_tile_shape(const aqtx_decode_plan* p) {
 
 // Upper bound of the exchange words over every launch shape: 64 token rows x (n rounded up to a
 // whole tile) int32 words.
-size_t exchange_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)(p->n + 64) * 4; }
+// Before them, in the first kControlBytes of a workspace, the control words of the launches that quantize the
+// activations themselves.
+size_t exchange_bytes_bound(const aqtx_decode_plan* p) { return kControlBytes + (size_t)64 * (size_t)(p->n + 64) * 4; }
 // The quantized activations in fragment order: 64 token rows x k rounded up to a whole K step.
 size_t fragment_bytes_bound(const aqtx_decode_plan* p) { return (size_t)64 * (size_t)((p->k + 127) / 128 * 128) + 256; }
 
 template <bool PACKED>
 int launch_tile(const TileShape& t, const DecodeArgs& d, hipStream_t st) {
-  const dim3 grid((unsigned)t.ntiles, (unsigned)t.splits);
+  const dim3 grid((unsigned)(t.ntiles + d.nprod), (unsigned)t.splits);
 #define AQTX_TILE(MB, NB, D) decode_tile_kernel<MB, NB, D, PACKED><<<grid, 256, 0, st>>>(d)
   // depths whose operands in flight fit the register file: (nb + mb * halves) * depth <= 64 loads
 #define AQTX_TILE_D(MB, NB)                                                          \
@@ -898,9 +1182,25 @@ int launch_tile(const TileShape& t, const DecodeArgs& d, hipStream_t st) {
     else if (t.nb == 2) AQTX_TILE_D(MB, 2);     \
     else AQTX_TILE_D(MB, 4);                    \
   } while (0)
-  if (t.mb == 1) AQTX_TILE_N(1);
+  // With producers: all (or as many as the registers hold) of a wave's weight steps are requested before the
+  // wait, few steps of fragments are in flight (see DX): one shape per (mb, nb).
+#define AQTX_TILE_P(MB, NB, DW, DXV) \
+  decode_tile_kernel<MB, NB, (PACKED ? DW / 2 : DW), PACKED, (PACKED && DXV > 2 ? DXV / 2 : DXV), true><<<grid, 256, 0, st>>>(d)
+#define AQTX_TILE_PN(MB, D4, X1, X2, X4)            \
+  do {                                              \
+    if (t.nb == 1) AQTX_TILE_P(MB, 1, 16, X1);      \
+    else if (t.nb == 2) AQTX_TILE_P(MB, 2, 16, X2); \
+    else AQTX_TILE_P(MB, 4, D4, X4);                \
+  } while (0)
+  if (d.nprod) {
+    if (t.mb == 1) AQTX_TILE_PN(1, 8, 16, 8, 8);
+    else if (t.mb == 2) AQTX_TILE_PN(2, 8, 8, 4, 4);
+    else AQTX_TILE_PN(4, 4, 4, 2, 4);
+  } else if (t.mb == 1) AQTX_TILE_N(1);
   else if (t.mb == 2) AQTX_TILE_N(2);
   else AQTX_TILE_N(4);
+#undef AQTX_TILE_PN
+#undef AQTX_TILE_P
 #undef AQTX_TILE_N
 #undef AQTX_TILE_D
 #undef AQTX_TILE
@@ -1033,14 +1333,39 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
 
   d.xq_out = reinterpret_cast<int8_t*>(xq);
   d.k_slice = t.k_slice; d.splits = t.splits;
-  d.sums = reinterpret_cast<int*>(ws);
+  d.sums = reinterpret_cast<int*>(ws + kControlBytes);
   d.count_shift = t.count_shift;
+
+  // One launch: the first workgroups quantize a token each while the others already stream their weights
+  // (decode_tile_kernel with producers).  It counts in control words that must be zero on entry, so it is for
+  // callers that vouch for their workspace; the others get the two launches below, the first of which clears.
+  // Between the start of the launch and the first matrix instruction lie the row's load, the write-through of its
+  // int8 values, the count, the poll that sees it and the first fragment load: five trips to memory, about a
+  // microsecond each, against two for the weights.  Measured (k = 4096, HIP-graph replay): against the 58.7 MB
+  // weight the one launch takes 13.5 / 13.8 / 15.0 us for 8 / 16 / 32 tokens where the two take 15.0 / 15.0 / 15.5
+  // (packed int4: 9.9 / 10.4 against 10.4 / 10.6 for 8 / 16); with 64 tokens, or against the 16.8 MB weight, whose
+  // stream is over before the chain is, the two launches are as fast or faster (8.5 against 9.2 us at 8 tokens).
+  const int path = (p->tuning >> 16) & 15;
+  const int64_t w_bytes = p->n * (pk ? p->k / 2 : p->k);
+  const bool pays = path == 1 || (w_bytes >= (24ll << 20) && p->m <= (pk ? 16 : 32));
+  if (p->workspace_zeroed && path != 2 && pays) {
+    // one producer per token: four (a quarter of every piece each) measured 0.1-0.4 us slower up to 8 tokens and
+    // 2-4 us slower from 32 on, where their workgroups delay the readers' start
+    d.prod_per_token = ((p->tuning >> 24) & 15) == 4 ? 4 : 1;
+    d.nprod = (int)p->m * d.prod_per_token;
+    d.ctrl = reinterpret_cast<int*>(ws);
+    const bool expire = ((p->tuning >> 20) & 15) == 1;  // test hook: a count that never comes, a wait of a microsecond
+    d.wait_target = expire ? d.nprod + 1 : d.nprod;
+    d.wait_ticks = expire ? 100u : 20000000u;  // 0.2 s of the 100 MHz clock
+    d.x_scale = x_scale;
+    return pk ? launch_tile<true>(t, d, st) : launch_tile<false>(t, d, st);
+  }
 
   // 1. per-token dynamic quantisation of the activations; the same launch clears the exchange
   //    words unless the caller vouches for them
   const int clear16 = p->workspace_zeroed ? 0 : (int)(exch / 16);
-  if (int rc = xbf ? launch_decode_quant<uint16_t>(d, reinterpret_cast<uint4*>(ws), clear16, st)
-                   : launch_decode_quant<float>(d, reinterpret_cast<uint4*>(ws), clear16, st))
+  if (int rc = xbf ? launch_decode_quant<uint16_t>(d, reinterpret_cast<uint4*>(d.sums), clear16, st)
+                   : launch_decode_quant<float>(d, reinterpret_cast<uint4*>(d.sums), clear16, st))
     return rc;
 
   // 2. the contraction with the dequantisation fused
@@ -1054,7 +1379,7 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
 // array for the life of the process.
 constexpr int64_t kStaticMaxN = 32768, kStaticMaxK = 32768;
 constexpr size_t kStaticScratchBytes =
-    (size_t)64 * (size_t)(kStaticMaxN + 64) * 4 + (size_t)64 * (size_t)kStaticMaxK + 512;  // 10.6 MB
+    kControlBytes + (size_t)64 * (size_t)(kStaticMaxN + 64) * 4 + (size_t)64 * (size_t)kStaticMaxK + 512;  // 10.6 MB
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Device address of `scratch` on each GPU, looked up once per device (the array's name is only a
@@ -1088,6 +1413,23 @@ extern "C" int aqtx_decode_i8(const aqtx_decode_plan* p, const void* x, const vo
   clear_error();
   if (int rc = validate_decode(p)) return rc;
   return decode_impl(p, x, w, w_scale, xq, x_scale, out, workspace, workspace_bytes, stream);
+}
+
+extern "C" int aqtx_decode_i8_check(void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  AQTX_REQUIRE(workspace != nullptr && workspace_bytes >= kControlBytes, "aqtx_decode_i8_check: workspace too small");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  int* ctrl = reinterpret_cast<int*>(workspace);
+  int words[2] = {0, 0};
+  hipError_t e = hipMemcpyAsync(words, ctrl, sizeof words, hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return set_error("aqtx_decode_i8_check: reading the control words failed: %s", hipGetErrorString(e));
+  if (words[1] == 0) return 0;
+  e = hipMemsetAsync(ctrl, 0, kControlBytes, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  return set_error("aqtx_decode_i8: a wait for the quantized activations expired in an earlier call on this workspace "
+                   "(mark %d); its outputs are incomplete%s", words[1],
+                   e == hipSuccess ? "; the control words have been cleared" : "");
 }
 
 extern "C" int aqtx_decode_i8_static(const aqtx_decode_plan* p, const void* x, const void* w,

@@ -483,6 +483,21 @@ def decode(x: torch.Tensor, w_q: torch.Tensor, w_scale: torch.Tensor, *, quant_b
   return (out, x_scale, xq) if want_xq else (out, x_scale)
 
 
+def decode_check(device=None) -> None:
+  """Raises if a serving call on this stream's workspace gave up waiting for its quantized activations (which
+  leaves that call's outputs unwritten).  Synchronizes the stream: for the points where a caller synchronizes
+  anyway; the workspace is dropped after an error, so the next call starts from a clean one."""
+  device = torch.device('cuda', torch.cuda.current_device()) if device is None else torch.device(device)
+  ent = _QUANT_WS.get(('decode', device.index, torch.cuda.current_stream(device).cuda_stream))
+  if ent is None:
+    return
+  try:
+    L.check(L.lib().aqtx_decode_i8_check(_ptr(ent[0]), ent[0].numel(), _stream()))
+  except Exception:
+    _QUANT_WS.clear()
+    raise
+
+
 def tile_weight(w_q: torch.Tensor, w_dtype: int = L.I8) -> torch.Tensor:
   """A frozen weight [n, k] (int8, or packed int4 uint8 [n, k/2]) in MFMA fragment order: the layout
   decode(..., w_layout=W_FRAGMENTS) streams fastest.  Returns a flat uint8 buffer."""

@@ -390,7 +390,11 @@ typedef struct aqtx_decode_plan {
                              depend on it): bits 0-7 K ranges per weight tile, bits 8-11 16-row weight
                              blocks per wave (1 | 2 | 4), bits 12-15 K steps in flight per wave (2 | 4 |
                              8 | 15 = 16; capped by the register file),
-                             bits 16-19 path: 1 = one or two tokens take the path of three and more  */
+                             bits 16-19 path: 1 = few tokens take the path of many as well (no kernel in
+                             which every workgroup quantizes the activations itself), 2 = that, with
+                             the activations quantized by a launch of their own.  Bits 20-23: 1 = the
+                             wait of aqtx_decode_i8_check's description expires at once (error-path tests).
+                             Bits 24-27: 4 = four quantizing workgroups per token instead of one          */
   int32_t w_layout;       /* AQTX_W_ROWS | AQTX_W_FRAGMENTS */
   int32_t workspace_zeroed; /* 1: the caller keeps one workspace across calls on one stream and its first
                              aqtx_decode_exchange_bytes(plan) bytes were zero before the first call.
@@ -423,8 +427,18 @@ int aqtx_decode_i8(const aqtx_decode_plan* plan, const void* x, const void* w,
                    const float* w_scale, void* xq, float* x_scale, void* out,
                    void* workspace, size_t workspace_bytes, void* stream);
 size_t aqtx_decode_workspace_bytes(const aqtx_decode_plan* plan);
-/* Leading bytes of the workspace that hold the partial-sum exchange (see workspace_zeroed). */
+/* Leading bytes of the workspace that hold the partial-sum exchange and the control words (see workspace_zeroed). */
 size_t aqtx_decode_exchange_bytes(const aqtx_decode_plan* plan);
+/*
+ * aqtx_decode_i8_check: with plan->workspace_zeroed, three to 32 tokens and a weight of 24 MiB or more,
+ * aqtx_decode_i8 is one launch in which the first m workgroups quantize a token each while the others already
+ * stream their weights and then wait for those tokens behind a bounded loop (0.2 s).  A wait that expires (it never should: the quantizing
+ * workgroups are resident first) leaves the call's outputs unwritten and a mark in the workspace; no kernel
+ * hangs.  This function reads the mark (it synchronizes the stream: call it where the caller synchronizes anyway,
+ * not under graph capture), returns 0 if no wait has expired since the workspace was zeroed or last checked, and
+ * otherwise an error after clearing the control words.  No counterpart in the reference.
+ */
+int aqtx_decode_i8_check(void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * aqtx_tile_weight: a frozen weight [n][k] (int8, or packed int4 as uint8 [n][k/2]) -> AQTX_W_FRAGMENTS order,

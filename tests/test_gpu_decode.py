@@ -29,20 +29,46 @@ def _weights(n, k, seed, w_sdt):
   return wq, ws
 
 
+# aqtx_decode_plan.tuning bits 16-19: the library's choice of kernels; the many-token kernel for every m, its first
+# workgroups quantizing the tokens (one per token, or four); the same with the quantisation in a launch of its own
+PATHS = pytest.mark.parametrize('path', [0, 1 << 16, (1 << 16) | (4 << 24), 2 << 16],
+                                ids=['auto', 'producers', 'producers4', 'two_launches'])
+
+
+@PATHS
 @pytest.mark.parametrize('m', [1, 2, 3, 8, 16, 17, 32, 40, 64])
-@pytest.mark.parametrize('n,k', [(256, 1024), (200, 464), (4096, 4096)])
+@pytest.mark.parametrize('n,k', [(256, 1024), (200, 464), (4096, 4096), (24, 8192 + 4096)])
 @pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('bf16', 'bf16'), ('f32', 'f32')])
-def test_decode_matches_oracle(gpu, m, n, k, dt, w_sdt):
+def test_decode_matches_oracle(gpu, m, n, k, dt, w_sdt, path):
   if (n, k) == (4096, 4096) and (dt, w_sdt) != ('bf16', 'f32'):
     pytest.skip('large shape once')
   x = U.rand((m, k), dt, 100 + m, outliers=True)
   wq, ws = _weights(n, k, 7, w_sdt)
   want, xq_want, xs_want = _oracle_decode(x, dt, wq, ws, w_sdt)
   out, xs, xq = ops.decode(U.to_dev(x, dt, gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu),
-                           quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True)
+                           quant_bound=127.5, clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True, tuning=path)
   np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
   np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
   np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+  ops.decode_check()
+
+
+def test_decode_wait_that_expires_is_reported_and_nothing_hangs(gpu):
+  """Error path of the launch whose first workgroups quantize the tokens, forced from the host: the workgroups
+  that contract are told to wait for one token more than there are, for a microsecond.  Every kernel ends
+  normally, decode_check reports the expired wait, and the next call (on a fresh workspace) is right again."""
+  m, n, k = 8, 512, 1024
+  x = U.rand((m, k), 'bf16', 77)
+  wq, ws = _weights(n, k, 8, 'f32')
+  args = (U.to_dev(x, 'bf16', gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(ws).to(gpu))
+  ops.decode(*args, quant_bound=127.5, clip_bound=127.0, tuning=(1 << 16) | (1 << 20))
+  with pytest.raises(RuntimeError, match='expired'):
+    ops.decode_check()
+  ops.decode_check()  # the mark is gone with the workspace
+  want, _, _ = _oracle_decode(x, 'bf16', wq, ws, 'f32')
+  out, _ = ops.decode(*args, quant_bound=127.5, clip_bound=127.0, tuning=1 << 16)
+  np.testing.assert_array_equal(out.float().cpu().numpy(), want)
+  ops.decode_check()
 
 
 @pytest.mark.parametrize('m', [20, 64])
@@ -82,10 +108,11 @@ def test_decode_rejects_bad_plans(gpu):
     ops.decode(x[:4, :24].contiguous(), w[:, :24].contiguous(), s, quant_bound=127.5, clip_bound=127.0)
 
 
+@PATHS
 @pytest.mark.parametrize('m', [1, 2, 8, 16, 17, 32, 33, 64])
 @pytest.mark.parametrize('n,k', [(256, 1024), (200, 480), (40, 32), (4096, 4096), (72, 8192)])
 @pytest.mark.parametrize('dt,w_sdt', [('bf16', 'f32'), ('bf16', 'bf16'), ('f32', 'f32')])
-def test_decode_packed_int4_matches_oracle(gpu, m, n, k, dt, w_sdt):
+def test_decode_packed_int4_matches_oracle(gpu, m, n, k, dt, w_sdt, path):
   """int4 weights packed two per byte (aqtx_pack_i4 layout): same numbers as the int8-held
   form, half the weight bytes."""
   from aqt_amd import _lib as L
@@ -100,7 +127,7 @@ def test_decode_packed_int4_matches_oracle(gpu, m, n, k, dt, w_sdt):
   packed = ops.pack_i4(wq_t)
   assert packed.shape == (n, k // 2) and packed.dtype == torch.uint8
   out, xs, xq = ops.decode(U.to_dev(x, dt, gpu), packed, torch.from_numpy(ws).to(gpu), quant_bound=127.5,
-                           clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True, w_dtype=L.I4P)
+                           clip_bound=127.0, w_scale_dtype=U.TORCH_DT[w_sdt], want_xq=True, w_dtype=L.I4P, tuning=path)
   np.testing.assert_array_equal(xq.cpu().numpy(), xq_want)
   np.testing.assert_array_equal(xs.cpu().numpy(), xs_want)
   np.testing.assert_array_equal(out.float().cpu().numpy(), want)
@@ -224,7 +251,9 @@ def test_decode_workspace_contract(gpu):
     p.x_dtype = p.x_scale_dtype = p.out_dtype = L.BF16
     p.w_scale_dtype = L.F32
     p.quant_bound, p.clip_bound, p.w_dtype = 127.5, 127.0, L.I8
-    p.tuning = 3 | (2 << 8)  # three K ranges per tile: the exchange is in use for every shape
+    # three K ranges per tile: the exchange is in use for every shape; the many-token kernel for every m, so that the
+    # calls on the kept workspace have their first workgroups quantize the tokens (control words in use as well)
+    p.tuning = 3 | (2 << 8) | (1 << 16)
     plans.append(p)
   lib = L.lib()
   ex = max(int(lib.aqtx_decode_exchange_bytes(ctypes.byref(p))) for p in plans)
