@@ -251,7 +251,11 @@ __device__ __forceinline__ float dequant_value(AccScalar accv, float s_row, floa
 // registers into the two neighbouring 16-byte chunks of its row on their way to LDS: a nibble is
 // moved to the top of its byte (value * 16); the epilogue takes the factor 16 out again, exactly (a
 // power of two commutes with every rounding of the dequantisation).
-template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = false, bool BFRAG = false>
+// PERSIST: the grid has one workgroup per CU (or fewer) and a workgroup walks tiles blockIdx.x, + gridDim.x, ...
+// (the XCD-aware order of tile_of_block continues: a workgroup stays on its XCD's range).  Between two tiles no
+// workgroup has to be launched, and the first stage of the next tile is requested before the epilogue of this one
+// (the staging registers are free then), so its latency passes under the stores.  Plain batches only.
+template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = false, bool BFRAG = false, bool PERSIST = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gemm_kernel(const GemmArgs g_in) {
   static_assert(NW == 4 || NW == 8, "4 or 8 waves");
@@ -290,7 +294,7 @@ void gemm_kernel(const GemmArgs g_in) {
     tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
   }
   const int64_t bz = blockIdx.y;
-  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+  int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
   if (g_in.group_offsets != nullptr) {
     // the group's row range replaces the batch strides of A, C and the row scale; tiles past
     // the group's last row leave at once (the grid is sized for the largest possible group)
@@ -313,18 +317,22 @@ void gemm_kernel(const GemmArgs g_in) {
   // free for refilling at the very end of a stage, and 64 KiB requested in one burst queue up
   // in the CU's address unit while the waves that issued them cannot issue MFMAs.  Register
   // staging lets the 16 loads of a wave spread over the whole stage.
-  const int64_t rows_a = (g.m - m0) < BM ? (g.m - m0) : BM;
-  const int64_t rows_b = (g.n - n0) < BN ? (g.n - n0) : BN;
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.a + bz * g.stride_a + m0 * g.lda), 0, (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
   // BFRAG, B in fragment order (GemmArgs::b_frag): the tile's 16-row blocks follow one another, b_steps KiB
   // each; the piece (row r, 16 bytes at 16 c of a 64-byte step) is lane r % 16 + 16 c of its KiB, and the scalar
   // offset of a stage is its row bytes times 16.
-  const __amdgpu_buffer_rsrc_t rsrc_b = BFRAG
-      ? __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (n0 / 16) * (int64_t)g.b_steps * 1024), 0,
-                                          (int)((rows_b + 15) / 16 * g.b_steps * 1024), kBufferRsrcWord3)
-      : __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + bz * g.stride_b + n0 * g.ldb), 0,
-                                          (int)((rows_b - 1) * g.ldb + (BPACK ? g.k / 2 : g.k)), kBufferRsrcWord3);
+  auto rsrc_a_of = [&](int64_t tm0) {
+    const int64_t rows_a = (g.m - tm0) < BM ? (g.m - tm0) : BM;
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(g.a + bz * g.stride_a + tm0 * g.lda), 0,
+                                             (int)((rows_a - 1) * g.lda + g.k), kBufferRsrcWord3);
+  };
+  auto rsrc_b_of = [&](int64_t tn0) {
+    const int64_t rows_b = (g.n - tn0) < BN ? (g.n - tn0) : BN;
+    return BFRAG ? __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (tn0 / 16) * (int64_t)g.b_steps * 1024), 0,
+                                                     (int)((rows_b + 15) / 16 * g.b_steps * 1024), kBufferRsrcWord3)
+                 : __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + bz * g.stride_b + tn0 * g.ldb), 0,
+                                                     (int)((rows_b - 1) * g.ldb + (BPACK ? g.k / 2 : g.k)), kBufferRsrcWord3);
+  };
+  __amdgpu_buffer_rsrc_t rsrc_a = rsrc_a_of(m0), rsrc_b = rsrc_b_of(n0);
   constexpr int ksh_b = BFRAG ? 4 : 0;
   int voff_a[LPW], voff_b[LPB], chunk_byte[LPW];
 #pragma unroll
@@ -402,12 +410,6 @@ void gemm_kernel(const GemmArgs g_in) {
   const int b_base = kTileBytes + wn * NI * 32 * BK;   // rows of the B tile
 
   Acc acc[4][NI];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < NI; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   auto load_frag = [&](const uint8_t* rows, int ks, int i) -> Frag {
     if constexpr (kChunks == 1) {
@@ -499,6 +501,14 @@ void gemm_kernel(const GemmArgs g_in) {
   auto refill_at = [&](int k0) { return k0 < k0_last ? k0 : k0_last; };
 #pragma unroll
   for (int j = 0; j < NLD; ++j) load_global(j, 0);
+  int tile = (int)blockIdx.x;
+  for (;;) {  // one trip per tile (one trip unless PERSIST)
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 #pragma unroll
   for (int j = 0; j < NL; ++j) store_lds(stage0, j);
 #pragma unroll
@@ -515,7 +525,22 @@ void gemm_kernel(const GemmArgs g_in) {
 
   // ---- epilogue ---------------------------------------------------------------
   // lane holds C[m = mrow0 + mi*32 + lr][n = ncol0 + ni*32 + 8*q + 4*lh + e], e = 0..3, reg = 4*q+e
-  const int64_t mrow0 = m0 + wm * 128, ncol0 = n0 + wn * NI * 32;
+  const int64_t em0 = m0, en0 = n0;  // this tile's corner: m0, n0 move on to the next tile below
+  const int64_t mrow0 = em0 + wm * 128, ncol0 = en0 + wn * NI * 32;
+  bool more = false;
+  if constexpr (PERSIST) {
+    // the next tile's first stage is requested now: the staging registers are free, and the epilogue's stores
+    // hide the latency
+    tile += (int)gridDim.x;
+    more = tile < g.tiles_m * g.tiles_n;
+    if (more) {
+      tile_of_block(tile, g.tiles_m, g.tiles_n, tm, tn);
+      m0 = (int64_t)tm * BM; n0 = (int64_t)tn * BN;
+      rsrc_a = rsrc_a_of(m0); rsrc_b = rsrc_b_of(n0);
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) load_global(j, 0);
+    }
+  }
 
   if (g.acc_out != nullptr) {  // optional second copy of the raw accumulators (plain stores)
     AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out);
@@ -572,7 +597,7 @@ void gemm_kernel(const GemmArgs g_in) {
     uint8_t* cbase = reinterpret_cast<uint8_t*>(g.c) + bz * g.stride_c * kEsz;
     const bool vec_store = ((g.ldc * kEsz) % 16) == 0 && ((uintptr_t)cbase % 16) == 0;
     // Tiles that lie wholly inside C and can use 16-byte stores skip every bounds check.
-    const bool interior = vec_store && (m0 + BM <= g.m) && (n0 + BN <= g.n);
+    const bool interior = vec_store && (em0 + BM <= g.m) && (en0 + BN <= g.n);
 
     auto epilogue = [&](auto checked_tag) {
       constexpr bool kChecked = decltype(checked_tag)::value;
@@ -661,6 +686,9 @@ void gemm_kernel(const GemmArgs g_in) {
     };
     if (interior && ((uintptr_t)cs % 16) == 0) epilogue(std::false_type{});
     else epilogue(std::true_type{});
+  }
+  if (!more) break;
+  __syncthreads();  // the staging rows of the epilogue have been read: the next tile may fill the stages
   }
 }
 

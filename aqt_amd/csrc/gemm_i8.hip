@@ -1,5 +1,7 @@
 // int8 x int8 -> int32 contraction on gfx950 MFMA (v_mfma_i32_32x32x32_i8) with the
 // dequantisation fused in the epilogue; the kernel lives in gemm_core.h.
+#include <atomic>
+
 #include "gemm_core.h"
 
 namespace aqtx {
@@ -47,6 +49,21 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
 }  // namespace aqtx
 
 using namespace aqtx;
+
+namespace {
+// CUs of the current device, asked once per device.
+int compute_units() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+}  // namespace
 
 extern "C" int aqtx_gemm_i8_k_slices(const aqtx_gemm_plan* p) {
   if (p == nullptr || p->k_split < 0 || p->k_split > 64 || p->batch <= 0 || p->m <= 0 || p->n <= 0) return 1;
@@ -114,11 +131,21 @@ extern "C" int aqtx_gemm_i8(const aqtx_gemm_plan* p, const void* a, const void* 
   }
   const int waves = p->tuning == 4 ? 4 : 8;
   AQTX_REQUIRE(!b_packed || !g.col_first, "aqtx_gemm_i8: a packed int4 b takes scale_order = AQTX_SCALE_ROW_THEN_COL");
+  // One workgroup per CU that walks the tiles (gemm_kernel's PERSIST) where there are at least two rounds of them:
+  // no workgroup launch between two tiles, and the next tile's first loads pass under the epilogue's stores.
+  const int cus = compute_units();
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  const bool persist = waves == 8 && !b_packed && !ktail && p->batch == 1 && p->group_offsets == nullptr && cus > 0 &&
+                       (p->tuning == 16 || (p->tuning == 0 && tiles >= 2 * cus));
+  const dim3 pgrid((unsigned)(tiles < cus ? tiles : cus), 1);
   // packed int4 B: the 8-wave kernel, row scale first (a frozen weight is the column operand)
 #define AQTX_LAUNCH(E, C, T)                                             \
   do {                                                                  \
     if constexpr (!C) {                                                 \
       if (b_packed) { gemm_kernel<MmaI8, 8, E, false, T, true><<<grid, 512, 0, st>>>(g); break; } \
+    }                                                                   \
+    if constexpr (!T) {                                                 \
+      if (persist) { gemm_kernel<MmaI8, 8, E, C, false, false, false, true><<<pgrid, 512, 0, st>>>(g); break; } \
     }                                                                   \
     if (waves == 8) gemm_kernel<MmaI8, 8, E, C, T><<<grid, 512, 0, st>>>(g); \
     else gemm_kernel<MmaI8, 4, E, C, T><<<grid, 256, 0, st>>>(g);       \

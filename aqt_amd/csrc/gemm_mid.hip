@@ -344,7 +344,7 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 
 // Whether the 128 x 128 kernel takes the plan (0 = no) and in how many slices of K (1 = none).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
-  if (p->group_offsets != nullptr || (p->tuning != 0 && p->tuning != 128) || !gemm_vector_shape_ok(p)) return 0;
+  if (p->group_offsets != nullptr || (p->tuning != 0 && p->tuning != 128) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
   if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)TN >= (1ll << 31)) return 0;
   const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);

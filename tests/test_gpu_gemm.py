@@ -12,7 +12,7 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[4, 8, 128, 0], ids=['waves4', 'waves8', 'tiles128', 'auto'])
+@pytest.fixture(params=[4, 8, 16, 128, 0], ids=['waves4', 'waves8', 'persistent', 'tiles128', 'auto'])
 def waves(request, monkeypatch):
   """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, the 128 x 128 kernel, and the library's own
   choice (these shapes have few output tiles: the 128 x 128 kernel, with k in slices where it is long)."""
