@@ -102,7 +102,12 @@ def build_library(jobs=4, verbose=True):
   os.replace(tmp, LIB_PATH)
   if verbose:
     print(f'built {LIB_PATH} from {len(sources)} sources', file=sys.stderr)
-  build_ffi_shim(verbose)
+  try:
+    build_ffi_shim(verbose)
+  except RuntimeError as e:
+    # the shim has never met a compiler where this library is developed (no XLA headers there): a failure to
+    # build it must not take the library, which is complete without it, down with it
+    print(f'warning: the XLA FFI shim did not build; libaqtx.so is unaffected\n{e}', file=sys.stderr)
   return LIB_PATH
 
 

@@ -72,7 +72,14 @@ _FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
 # Weight-only quantization (a float lhs against an int8 / fp8 rhs) promotes the rhs to the float dtype on
 # every call; for a frozen weight that is the same conversion every time, so large converted copies are
 # kept for as long as the quantized tensor lives and stays unchanged (its version counter).
-_PROMOTED_RHS = {}  # id(rhs) -> (key, promoted [b, k, n] copy)
+_PROMOTED_RHS = {}  # id(rhs) -> (key, promoted [b, k, n] copy), oldest first
+# The copies cost 2 (bf16) or 4 bytes per weight element on top of the quantized tensor; together they are kept
+# below this many bytes (the oldest go first), and none is made while gradients are being recorded (a quantized
+# residual of a training step is not a frozen weight).
+PROMOTED_RHS_MAX_BYTES = 8 << 30
+# Longest tile for which the activation quantizer writes every 8 k in even-odd order (the row kernels hold a
+# segment in registers up to this length).
+_EVEN_ODD8_MAX_GROUP = 16384
 
 # Weight-only serving above 64 lhs rows: True = the library's bf16 product on the kept float copy of the
 # weight (2 bytes per weight element more, the faster of the two on most shapes); False = the weight-only
@@ -81,16 +88,25 @@ WEIGHT_ONLY_FLOAT_COPY = True
 
 
 def _promoted_rhs(rhs, perm, shape, common):
-  if rhs.dtype == common or rhs.numel() < (1 << 20) or rhs.requires_grad:
+  if rhs.dtype == common or rhs.numel() < (1 << 20) or rhs.requires_grad or torch.is_grad_enabled():
     return rhs.permute(perm).reshape(shape).to(common)
-  key = (perm, tuple(rhs.shape), common, rhs._version)
+  # the storage address is part of the key: writes through .data or set_() do not move the version counter
+  key = (perm, tuple(rhs.shape), common, rhs._version, rhs.data_ptr())
   hit = _PROMOTED_RHS.get(id(rhs))
   if hit is not None and hit[0] == key:
     return hit[1]
   out = rhs.permute(perm).reshape(shape).to(common)
   if hit is None:
     weakref.finalize(rhs, _PROMOTED_RHS.pop, id(rhs), None)
-  _PROMOTED_RHS[id(rhs)] = (key, out)
+  _PROMOTED_RHS.pop(id(rhs), None)
+  nbytes = lambda t: t.numel() * t.element_size()
+  total = sum(nbytes(v[1]) for v in _PROMOTED_RHS.values()) + nbytes(out)
+  for old in list(_PROMOTED_RHS):
+    if total <= PROMOTED_RHS_MAX_BYTES:
+      break
+    total -= nbytes(_PROMOTED_RHS.pop(old)[1])
+  if nbytes(out) <= PROMOTED_RHS_MAX_BYTES:
+    _PROMOTED_RHS[id(rhs)] = (key, out)
   return out
 
 
@@ -1257,7 +1273,9 @@ class DotGeneral:
     # Against a packed weight, and when nobody asks for the quantized activation itself, the
     # activation is written with every 8 k in even-odd order: the kernel then takes the weight's
     # nibbles as they lie instead of interleaving them again.
-    k_order = L.K_EVEN_ODD8 if packed and not (with_qt and lhs_qvalue_needed) else L.K_NATURAL
+    # (aqtx_quantize writes that order for groups of up to _EVEN_ODD8_MAX_GROUP values; longer tiles stay in k order)
+    k_order = (L.K_EVEN_ODD8 if packed and ts <= _EVEN_ODD8_MAX_GROUP and not (with_qt and lhs_qvalue_needed)
+               else L.K_NATURAL)
     lq, lsc = ops.quantize(lhs.reshape(1, M, T * ts), reduce=L.REDUCE_COLS, group=ts, out_dtype=specs[0]['out_dtype'],
                            quant_bound=specs[0]['quant_bound'], clip_bound=specs[0]['clip_bound'],
                            compute_dtype=lhs.dtype, scale_dtype=sdt_l, k_order=k_order)

@@ -89,6 +89,15 @@ def test_quantize_argument_validation():
   assert lib.aqtx_last_error() == b''
 
 
+def test_even_odd_k_order_has_a_longest_group_and_the_host_knows_it():
+  """aqtx_quantize writes every 8 k in even-odd order only for segments its row kernels hold in registers; the
+  tiled dot_general asks for that order up to the same length and falls back to k order beyond it."""
+  from aqt_amd.v2 import aqt_dot_general
+  longest = aqt_dot_general._EVEN_ODD8_MAX_GROUP
+  p = _qplan(rows=2, cols=2 * (longest + 8), group=longest + 8, out_k_order=L.K_EVEN_ODD8)
+  assert 'segments of at most %d' % longest in _err(L.lib().aqtx_quantize(ctypes.byref(p), FAKE, None, FAKE, FAKE, None, 0, None))
+
+
 def _gplan(**kw):
   p = L.GemmPlan()
   p.batch, p.m, p.n, p.k = 1, 64, 64, 64
@@ -406,6 +415,15 @@ def test_gemm_k_slices_choice_is_a_host_decision():
   assert 'k_split must be in 0..64' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
   p = _gplan(m=128, n=4096, k=14336, lda=14336, ldb=14336, ldc=4096, k_split=4)
   assert 'k_split_workspace' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
+  # the kernel that adds the slices up takes a row per grid row: more than 65535 rows are refused in words
+  p = _gplan(m=70000, n=128, k=4096, lda=4096, ldb=4096, ldc=128, k_split=2, k_split_workspace=0x1000,
+             k_split_workspace_bytes=1 << 40)
+  assert 'at most 65535 rows' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
+  # fp8: sums through bf16 are a choice of aqtx_gemm_fp8 alone
+  p = _gplan(accumulate=L.ACC_F32)
+  assert 'accumulate' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
+  p = _gplan(accumulate=5, a_dtype=L.E4M3, b_dtype=L.E4M3)
+  assert 'accumulate' in _err(lib.aqtx_gemm_fp8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
 
 
 def test_conv_validation():
