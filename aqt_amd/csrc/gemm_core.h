@@ -259,8 +259,11 @@ template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = f
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gemm_kernel(const GemmArgs g_in) {
   static_assert(NW == 4 || NW == 8, "4 or 8 waves");
-  static_assert(!BFRAG || MMA::kIntAcc, "the fragment order is that of int8 / packed int4 weights");
-  static_assert(!BPACK || MMA::kIntAcc, "packed int4 goes with the int8 MFMA");
+  static_assert(!BFRAG || MMA::kIntAcc || MMA::kWidenB, "the fragment order is that of int8 / packed int4 weights");
+  static_assert(!BPACK || MMA::kIntAcc || MMA::kWidenB, "packed int4 goes with the int8 MFMA, int8 to widen with a bf16 one");
+  static_assert(BPACK || !MMA::kWidenB, "a B that is widened on its way to LDS takes the packed loads");
+  // the nibbles of a packed int4 B sit at the top of their bytes: the accumulators hold 16 times the contraction
+  constexpr bool kTimes16 = BPACK && MMA::kIntAcc;
   GemmArgs g = g_in;
   constexpr int NI = 16 / NW;       // 32-column MFMA tiles per wave
   constexpr int WN = NW / 2;        // waves along n
@@ -392,7 +395,8 @@ void gemm_kernel(const GemmArgs g_in) {
         *reinterpret_cast<v4i*>(st + st_off + i * 1024) = stga[i];
       } else if (r4 == 1) {
         v4i lo;
-        unpack_i4x32(stgb[grp], lo, pb_hi[grp], g.a_even_odd8);
+        if constexpr (MMA::kWidenB) MMA::widen_b(stgb[grp], lo, pb_hi[grp]);
+        else unpack_i4x32(stgb[grp], lo, pb_hi[grp], g.a_even_odd8);
         *reinterpret_cast<v4i*>(st + pb_st[grp]) = lo;
       } else {
         *reinterpret_cast<v4i*>(st + (pb_st[grp] ^ 16)) = pb_hi[grp];
@@ -554,7 +558,7 @@ void gemm_kernel(const GemmArgs g_in) {
         for (int r = 0; r < 16; ++r) {
           const int64_t nn = ncol0 + ni * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
           if (mm < g.m && nn < g.n) {
-            if constexpr (BPACK) dst[mm * g.ldc + nn] = acc[mi][ni][r] >> 4;  // exact: a multiple of 16
+            if constexpr (kTimes16) dst[mm * g.ldc + nn] = acc[mi][ni][r] >> 4;  // exact: a multiple of 16
             else dst[mm * g.ldc + nn] = acc[mi][ni][r];
           }
         }
@@ -575,7 +579,7 @@ void gemm_kernel(const GemmArgs g_in) {
     }
     auto dequant = [&](AccScalar accv, float s_row, float s_col) {
       if constexpr (EPI == 3) {
-        if constexpr (BPACK) return __builtin_bit_cast(float, accv >> 4);
+        if constexpr (kTimes16) return __builtin_bit_cast(float, accv >> 4);
         else return __builtin_bit_cast(float, accv);
       }
       return dequant_value<EPI, COL_FIRST>(accv, s_row, s_col);
@@ -620,7 +624,7 @@ void gemm_kernel(const GemmArgs g_in) {
                 csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
               }
             }
-            if constexpr (BPACK) {  // the accumulators hold 16 times the contraction
+            if constexpr (kTimes16) {  // the accumulators hold 16 times the contraction
 #pragma unroll
               for (int e = 0; e < 4; ++e) csv[e] *= 0.0625f;
             }
@@ -877,5 +881,8 @@ int launch_gemm_i8_frag(const aqtx_gemm_plan* p, const void* a, const void* b, c
                         const float* col_scale, void* c, int32_t* acc_out, hipStream_t st);
 int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* col_scale, void* c,
                                 hipStream_t st);
+// gemm_wo.hip: the same contraction on 256 x 256 tiles; `workgroups` > 0: that many workgroups walk the tiles
+int launch_gemm_weight_only_large(const aqtx_gemm_plan* p, const void* a, const void* b, const float* col_scale, void* c,
+                                  int workgroups, hipStream_t st);
 
 }  // namespace aqtx

@@ -224,5 +224,15 @@ extern "C" int aqtx_gemm_weight_only(const aqtx_gemm_plan* p, const void* a, con
   if (p->batch == 0 || p->m == 0 || p->n == 0) return 0;
   AQTX_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "%s: NULL buffer", who);
   AQTX_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 2) == 0, "%s: a and b must be 16-byte aligned", who);
+  // 256 x 256 tiles where they fill the chip (the rule of aqtx_gemm_i8), walked by one workgroup per CU from two
+  // rounds of them on; plan->tuning: 128 = the 128 x 128 tiles, 8 = the large ones with a workgroup per tile
+  const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN), pad128 = ((p->m + 127) / 128) * ((p->n + 127) / 128);
+  const bool large = p->tuning == 8 || p->tuning == 16 ||
+                     (p->tuning == 0 && pad256 * p->batch > 128 && 4 * pad256 * 2 < 3 * pad128);
+  if (large && p->lda * (int64_t)(2 * BM) < (1ll << 31) && (b_frag || p->ldb * (int64_t)BN < (1ll << 31))) {
+    const int cus = compute_units();
+    const int workgroups = (p->tuning == 16 || (p->tuning == 0 && pad256 >= 2 * cus)) ? cus : 0;
+    return launch_gemm_weight_only_large(p, a, b, col_scale, c, workgroups, reinterpret_cast<hipStream_t>(stream));
+  }
   return launch_gemm_weight_only_mid(p, a, b, col_scale, c, reinterpret_cast<hipStream_t>(stream));
 }

@@ -359,10 +359,12 @@ def ragged_offsets(group_sizes, m: int, device) -> torch.Tensor:
 
 
 def gemm_weight_only(a: torch.Tensor, b: torch.Tensor, col_scale: torch.Tensor, *, col_scale_dtype=torch.float32,
-                     b_dtype: int = L.I8, b_layout: int = L.W_ROWS):
+                     b_dtype: int = L.I8, b_layout: int = L.W_ROWS, tuning: Optional[int] = None):
   """Weight-only contraction C[b] = bf16(bf16(A[b] @ float(B[b])^T) * col_scale[b]) for bf16 A [batch, m, k] that
   stays unquantized and int8 B [batch, n, k] (k contiguous in both), any m; `col_scale` is float32 [batch, n]
-  holding values of `col_scale_dtype`.  float32 sums; the weight is never copied as bf16."""
+  holding values of `col_scale_dtype`.  float32 sums; the weight is never copied as bf16.  tuning (None =
+  GEMM_TUNING): 128 = 128 x 128 tiles, 8 = 256 x 256 tiles, 16 = those walked by one workgroup per CU; every
+  choice sums k in the same order, so the results do not depend on it."""
   _require_gpu(a, b, col_scale)
   assert a.dim() == 3 and a.dtype == torch.bfloat16 and a.stride(2) == 1
   batch, m, k = a.shape
@@ -384,6 +386,9 @@ def gemm_weight_only(a: torch.Tensor, b: torch.Tensor, col_scale: torch.Tensor, 
   plan.out_dtype = plan.dequant_dtype = plan.row_scale_dtype = L.BF16
   plan.col_scale_dtype = aqtx_dtype(col_scale_dtype)
   plan.col_scale_stride_b = n
+  plan.tuning = GEMM_TUNING if tuning is None else tuning
+  if plan.tuning == 4:
+    plan.tuning = 8  # the weight-only kernel has one workgroup shape on the large tiles
   with _timed('gemm'):
     L.check(L.lib().aqtx_gemm_weight_only(ctypes.byref(plan), _ptr(a), _ptr(b), _ptr(col_scale), _ptr(c), _stream()))
   return c

@@ -499,6 +499,85 @@ def gemm_probe(dev, data, reps=10):
   print(json.dumps({'gemm_probe': data, 'reps': reps, 'shapes': rows}))
 
 
+def power_probe(dev, seconds=8.0):
+  """Socket power and shader clock, sampled from the box's SMI tool (amd-smi) by a thread of this
+  process while the forward contraction (8192 x 14336 x 4096) runs back to back for `seconds` per operand value
+  distribution: the evidence behind 'the clock falls with the operand values under the power cap'.  Prints one
+  JSON line; where no tool answers an ordinary user, the samples are empty and the line says so."""
+  import re
+  import shutil
+  import subprocess
+  import threading
+  import torch
+  from aqt_amd import ops
+  tool = shutil.which('amd-smi') or '/opt/rocm/bin/amd-smi'
+  cap = None
+
+  def sample():
+    """(watts, mean MHz over the XCDs) or None."""
+    try:
+      out = subprocess.run([tool, 'metric', '-g', '0', '-p', '-c', '--json'], capture_output=True, text=True, timeout=10).stdout
+      card = json.loads(out)
+      card = (card['gpu_data'] if isinstance(card, dict) else card)[0]
+      watts = card['power']['socket_power']['value']
+      clks = [v['clk']['value'] for k, v in card['clock'].items() if k.startswith('gfx_') and isinstance(v['clk']['value'], (int, float))]
+      return (float(watts) if isinstance(watts, (int, float)) else None), (sum(clks) / len(clks) if clks else None)
+    except Exception:
+      return None
+
+  try:  # the package power limit, from the older tool (it answers an ordinary user)
+    out = subprocess.run([shutil.which('rocm-smi') or '/opt/rocm/bin/rocm-smi', '-d', '0', '--showmaxpower', '--json'],
+                         capture_output=True, text=True, timeout=10).stdout
+    cap = next((float(v) for k, v in next(iter(json.loads(out).values())).items() if re.match(r'^[0-9.]+$', str(v))), None)
+  except Exception:
+    pass
+  gens = {
+      'zeros': lambda s: torch.zeros(s, dtype=torch.int8, device=dev),
+      'normal25': lambda s: (torch.randn(s, device=dev) * 25).clamp(-127, 127).round().to(torch.int8),
+  }
+  rows = {'idle': {'samples': [sample() for _ in range(3)]}}
+  for kind, gen in gens.items():
+    a, b = gen((1, M, K)), gen((1, N, K))
+    rs, cs = torch.rand(1, M, device=dev), torch.rand(1, N, device=dev)
+    f = lambda: ops.gemm(a, b, row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16)
+    for _ in range(5):
+      f()
+    torch.cuda.synchronize()
+    samples, stop = [], threading.Event()
+
+    def poll():
+      while not stop.is_set():
+        r = sample()
+        if r is not None:
+          samples.append(r)
+
+    th = threading.Thread(target=poll)
+    th.start()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0, calls = time.perf_counter(), 0
+    e0.record()
+    while time.perf_counter() - t0 < seconds:
+      for _ in range(50):
+        f()
+      calls += 50
+      torch.cuda.synchronize()
+    e1.record()
+    torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    us = e0.elapsed_time(e1) * 1e3 / calls
+    watts = [w for w, _ in samples if w is not None]
+    mhz = [c for _, c in samples if c is not None]
+    rows[kind] = {'us_per_launch': round(us, 1), 'TOPS': round(2.0 * M * N * K / us / 1e6), 'samples': len(samples),
+                  'socket_power_W_mean': round(sum(watts) / len(watts), 1) if watts else None,
+                  'socket_power_W_max': max(watts) if watts else None,
+                  'sclk_MHz_mean': round(sum(mhz) / len(mhz)) if mhz else None,
+                  'sclk_MHz_min': min(mhz) if mhz else None, 'sclk_MHz_max': max(mhz) if mhz else None}
+    del a, b
+  print(json.dumps({'power_probe': 'aqtx_gemm_i8 8192x14336x4096 back to back, SMI samples from a thread', 'tool': tool,
+                    'power_cap_W': cap, 'rows': rows}))
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--gpus', type=int, default=1)
@@ -516,6 +595,9 @@ def main():
                        'distribution (and the vendor int8 GEMM beside them) and exit')
   ap.add_argument('--decode-probe', action='store_true',
                   help='only issue a few serving calls per shape (for rocprofv3 runs) and exit')
+  ap.add_argument('--power-probe', action='store_true',
+                  help='only run the forward contraction back to back on all-zero and on quantized-normal operands while '
+                       'sampling socket power and shader clock from the SMI tool, and exit')
   ap.add_argument('--read-ceiling', action='store_true',
                   help='only sweep a pure reader over buffer sizes and launch shapes (what the memory system delivers '
                        'to a single pass over the serving weights and over 256 MiB / 1 GiB) and exit')
@@ -535,6 +617,9 @@ def main():
   dev = torch.device('cuda:0')
   if args.gemm_probe is not None:
     gemm_probe(dev, args.gemm_probe)
+    return
+  if args.power_probe:
+    power_probe(dev)
     return
   if args.read_ceiling:
     best, rows = read_ceiling(dev, full=True)

@@ -391,6 +391,26 @@ def test_weight_only_gemm_within_float_summation_error(gpu, batch, m, n, k, w_sd
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('layout', ['rows', 'fragments'])
+@pytest.mark.parametrize('w_sdt', ['bf16', 'f32'])
+@pytest.mark.parametrize('m,n,k', [(300, 520, 144), (256, 256, 128), (1024, 768, 4096), (130, 72, 1040), (2304, 4100, 320)])
+def test_weight_only_gemm_tile_sizes_give_the_same_bits(gpu, m, n, k, w_sdt, layout):
+  """The 128 x 128 kernel, the 256 x 256 kernel with a workgroup per tile and the same walked by one workgroup
+  per CU sum k in the same order with the same instruction: bit for bit the same float sums (the tolerance
+  test above, which the library's own choice of kernel runs through, therefore covers all three)."""
+  torch.manual_seed(11)
+  a = torch.randn(1, m, k, device=gpu).to(torch.bfloat16)
+  b = torch.randint(-127, 128, (1, n, k), dtype=torch.int8, device=gpu)
+  cs = (torch.rand(1, n, device=gpu) * 0.01 + 1e-4).to(U.TORCH_DT[w_sdt]).float()
+  kw = dict(col_scale_dtype=U.TORCH_DT[w_sdt])
+  if layout == 'fragments':
+    b, kw['b_layout'] = ops.tile_weight(b[0], L.I8), L.W_FRAGMENTS
+  outs = [ops.gemm_weight_only(a, b, cs, tuning=t, **kw) for t in (128, 8, 16, 0)]
+  for o in outs[1:]:
+    assert torch.equal(o.view(torch.int16), outs[0].view(torch.int16))
+
+
+@pytest.mark.gpu
 def test_weight_only_gemm_strided_operands(gpu):
   """Rows of a and b further apart than k (views into wider tensors) and the few-rows kernel's answer:
   both kernels round alike except for summation order."""
