@@ -13,6 +13,7 @@ import dataclasses
 import enum
 import functools
 import math
+import os
 import weakref
 from typing import Any, Optional, Sequence
 
@@ -81,10 +82,13 @@ PROMOTED_RHS_MAX_BYTES = 8 << 30
 # segment in registers up to this length).
 _EVEN_ODD8_MAX_GROUP = 16384
 
-# Weight-only serving above 64 lhs rows: True = the library's bf16 product on the kept float copy of the
-# weight (2 bytes per weight element more, the faster of the two on most shapes); False = the weight-only
-# contraction kernel, which widens the int8 bytes in registers and keeps no float copy.
-WEIGHT_ONLY_FLOAT_COPY = True
+# Weight-only serving above 64 lhs rows: False (the default) = this library's weight-only contraction kernel,
+# which widens the int8 bytes in registers and keeps no float copy of the weight (1090-1170 TFLOP/s from 1024
+# rows on against a 4096 x 14336 weight); True = the vendor library's bf16 product on a float copy of the weight
+# kept next to the quantized tensor (2 bytes per weight element more; 1320-1490 TFLOP/s on the same shapes): a
+# trade of weight memory for 20-25 % of prefill time that the caller has to ask for
+# (AQTX_WEIGHT_ONLY_FLOAT_COPY=1 in the environment does so for a whole process).
+WEIGHT_ONLY_FLOAT_COPY = os.environ.get('AQTX_WEIGHT_ONLY_FLOAT_COPY', '') == '1'
 
 
 def _promoted_rhs(rhs, perm, shape, common):

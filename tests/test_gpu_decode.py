@@ -402,8 +402,8 @@ def test_weight_only_decode_within_float_summation_error(gpu, m, n, k, w_sdt, pa
 @pytest.mark.gpu
 def test_weight_only_serving_takes_the_kernel(gpu, monkeypatch):
   """A float lhs of at most 64 rows against a frozen int8 rhs goes to the streaming weight-only kernel; more rows
-  take the float product on the promoted weight, or, with WEIGHT_ONLY_FLOAT_COPY off, the tiled weight-only
-  kernel.  Same numbers to float summation order."""
+  take the tiled weight-only kernel, or, with WEIGHT_ONLY_FLOAT_COPY on, the float product on the promoted
+  weight.  Same numbers to float summation order."""
   from aqt_amd.v2 import aqt_dot_general as aqt, config
   dt = 'bf16'
   MATMUL = (((1,), (0,)), ((), ()))
@@ -415,6 +415,7 @@ def test_weight_only_serving_takes_the_kernel(gpu, monkeypatch):
     real = getattr(ops, name)
     monkeypatch.setattr(ops, name, lambda *a, _real=real, _name=name, **k: (calls.append(_name), _real(*a, **k))[1])
   with torch.no_grad():
+    monkeypatch.setattr(aqt, 'WEIGHT_ONLY_FLOAT_COPY', True)
     _, (_, wq) = cfg.dg_core(x_small, w, None, None, MATMUL)
     out_small, (lqt, _) = cfg.dg_core(x_small, torch.zeros_like(w), None, wq, MATMUL)
     out_large, _ = cfg.dg_core(x_large, torch.zeros_like(w), None, wq, MATMUL)

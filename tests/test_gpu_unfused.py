@@ -115,19 +115,26 @@ def test_one_sided_quantization(gpu, lhs_bits, rhs_bits, dt):
   _close(_np(out), want, dt)
 
 
-def test_weight_only_serving_keeps_the_promoted_weight(gpu):
-  """A frozen int8 weight next to a float lhs of more than 64 rows (fewer go to the weight-only kernel) is
-  promoted to the float dtype once, not on every call; a change of the weight in place is noticed (version
-  counter)."""
+def test_weight_only_serving_keeps_the_promoted_weight(gpu, monkeypatch):
+  """With WEIGHT_ONLY_FLOAT_COPY on, a frozen int8 weight next to a float lhs of more than 64 rows (fewer go to
+  the weight-only kernel) is promoted to the float dtype once, not on every call; a change of the weight in place
+  is noticed (version counter); while gradients are recorded no copy is kept."""
   from aqt_amd.v2 import aqt_dot_general as adg
+  monkeypatch.setattr(adg, 'WEIGHT_ONLY_FLOAT_COPY', True)
   dt = 'bf16'
   cfg = config.set_context(aqt.dot_general_make(None, 8), None, None)
   x1, x2 = U.to_dev(U.rand((72, 1024), dt, 1), dt, gpu), U.to_dev(U.rand((72, 1024), dt, 2), dt, gpu)
   w = U.to_dev(U.rand((1024, 1024), dt, 3, 0.05), dt, gpu)
   _, (_, wq) = cfg.dg_core(x1, w, None, None, MATMUL)
   assert wq.qvalue.dtype == torch.int8
-  serve = lambda x: cfg.dg_core(x, torch.zeros_like(w), None, wq, MATMUL)[0]
+
+  def serve(x):
+    with torch.no_grad():
+      return cfg.dg_core(x, torch.zeros_like(w), None, wq, MATMUL)[0]
+
   adg._PROMOTED_RHS.clear()
+  cfg.dg_core(x1, torch.zeros_like(w), None, wq, MATMUL)
+  assert not adg._PROMOTED_RHS  # gradients were being recorded
   a1, a2 = serve(x1), serve(x2)
   assert list(adg._PROMOTED_RHS) == [id(wq.qvalue)]
   kept = adg._PROMOTED_RHS[id(wq.qvalue)][1]
