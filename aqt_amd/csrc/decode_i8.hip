@@ -67,7 +67,6 @@ struct DecodeArgs {
   // side, about 10 ns each, which hundreds of workgroups on one word would turn into microseconds.  ctrl[1]
   // collects expired waits.
   int nprod;              // 0: the activations were quantized by decode_quant_kernel before this launch
-  int prod_per_token;     // 1: a producer quantizes a whole token; 4: a quarter of each of its 16-value pieces
   int* ctrl;              // kControlBytes, zero on entry and (no wait having expired) on exit
   int wait_target;        // nprod (a test makes it unreachable)
   unsigned wait_ticks;
@@ -581,10 +580,7 @@ __global__ __launch_bounds__(256) void decode_quant_kernel(const DecodeArgs d, u
   }
 }
 
-// Quantisation of a token inside the contraction launch, by one workgroup or by four (d.prod_per_token): each
-// finds the row's abs-max (the whole row: 16 values per thread and pass); one quantizes every 16-value piece,
-// of four each quantizes a quarter of every piece, four values per thread (fewer instructions between the
-// arrival of the row and its stores, but four times the workgroups: for few tokens).  The arithmetic is that of decode_quant_kernel: scale = dtype(absmax / bound),
+// Quantisation of token `row` by one workgroup inside the contraction launch.  The arithmetic is that of decode_quant_kernel: scale = dtype(absmax / bound),
 // inv = dtype(1 / scale), q = rint(clip(dtype(x * inv))) (clip with one v_med3, round to nearest even and
 // convert with one addition of 1.5 * 2^23: |t| <= 127 there).  The int8 values go to the fragment-ordered copy.
 // The workgroups that read them run on other XCDs, whose L2s this one's stores do not reach on their own: scale
@@ -592,7 +588,7 @@ __global__ __launch_bounds__(256) void decode_quant_kernel(const DecodeArgs d, u
 // complete, and only then counts itself in the readers' arrival words with device-scope read-modify-writes.
 // Readers touch the copy only after they have seen every producer counted, so no L2 can hold a line of it from
 // before.  Up to two 16-value pieces per thread stay in registers between the passes; longer rows are read twice.
-__device__ __forceinline__ void quant_token_publish(const DecodeArgs& d, const int row, const int quarter) {
+__device__ __forceinline__ void quant_token_publish(const DecodeArgs& d, const int row) {
   __shared__ float smax[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int pieces = d.k / 16;
@@ -658,41 +654,9 @@ __device__ __forceinline__ void quant_token_publish(const DecodeArgs& d, const i
   sc = rnd(sc, d.xs_bf16);
   float inv = rnd(1.0f / sc, d.xs_bf16);
   if (isinf(inv)) inv = 1.0f;
-  if (tid == 0 && quarter == 0) __hip_atomic_store(d.x_scale_out + row, sc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) __hip_atomic_store(d.x_scale_out + row, sc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const int tbf = d.x_bf16 & d.xs_bf16;
   constexpr int kDeviceScope = 16;  // the sc1 bit of the store's cache policy: written through to memory
-  // values 4 * quarter .. + 3 of piece p -> one word of the fragment-ordered copy
-  auto quant_quarter = [&](const uint32_t* w, int p) __attribute__((always_inline)) {
-    // the quarter's four values as float32 patterns: every word is read into a scalar of its own first (a
-    // choice between array elements would become a computed address and send the array to scratch memory)
-    uint32_t f4[4];
-    if (d.x_bf16) {
-      const uint32_t a0 = w[0], a1 = w[1], a2 = w[2], a3 = w[3], a4 = w[4], a5 = w[5], a6 = w[6], a7 = w[7];
-      const uint32_t lo = quarter == 0 ? a0 : quarter == 1 ? a2 : quarter == 2 ? a4 : a6;
-      const uint32_t hi = quarter == 0 ? a1 : quarter == 1 ? a3 : quarter == 2 ? a5 : a7;
-      f4[0] = lo << 16; f4[1] = lo & 0xFFFF0000u; f4[2] = hi << 16; f4[3] = hi & 0xFFFF0000u;
-    } else {
-      const uint32_t a0 = w[0], a1 = w[1], a2 = w[2], a3 = w[3], a4 = w[4], a5 = w[5], a6 = w[6], a7 = w[7];
-      const uint32_t a8 = w[8], a9 = w[9], a10 = w[10], a11 = w[11], a12 = w[12], a13 = w[13], a14 = w[14], a15 = w[15];
-      f4[0] = quarter == 0 ? a0 : quarter == 1 ? a4 : quarter == 2 ? a8 : a12;
-      f4[1] = quarter == 0 ? a1 : quarter == 1 ? a5 : quarter == 2 ? a9 : a13;
-      f4[2] = quarter == 0 ? a2 : quarter == 1 ? a6 : quarter == 2 ? a10 : a14;
-      f4[3] = quarter == 0 ? a3 : quarter == 1 ? a7 : quarter == 2 ? a11 : a15;
-    }
-    uint32_t b[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float v = __uint_as_float(f4[e]);
-      float t = rnd(v * inv, tbf);
-      t = __builtin_amdgcn_fmed3f(t, -d.clip_bound, d.clip_bound);
-      b[e] = __float_as_uint(t + 12582912.0f);
-    }
-    const uint32_t lo = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);   // bytes b0 b1 0 0
-    const uint32_t hi = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);   // bytes 0 0 b2 b3
-    const uint32_t q = lo | hi;
-    __builtin_amdgcn_raw_buffer_store_b32((int)q, rf, frag_off(p) + 4 * quarter, 0, kDeviceScope);
-    if (d.xq_out != nullptr) *reinterpret_cast<uint32_t*>(d.xq_out + (int64_t)row * d.k + (int64_t)p * 16 + 4 * quarter) = q;
-  };
   // a whole piece: sixteen values, one 16-byte store
   auto quant_piece = [&](const uint32_t* w, int p) __attribute__((always_inline)) {
     uint32_t q[4];
@@ -713,29 +677,16 @@ __device__ __forceinline__ void quant_token_publish(const DecodeArgs& d, const i
     if (d.xq_out != nullptr)
       *reinterpret_cast<uint4*>(d.xq_out + (int64_t)row * d.k + (int64_t)p * 16) = make_uint4(q[0], q[1], q[2], q[3]);
   };
-  if (d.prod_per_token == 1) {
-    if (held) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int p = tid + 256 * j;
-        if (p < pieces) quant_piece(raw[j], p);
-      }
-    } else {
-      for (int p = tid; p < pieces; p += 256) {
-        load_piece(p, raw[0]);
-        quant_piece(raw[0], p);
-      }
-    }
-  } else if (held) {
+  if (held) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int p = tid + 256 * j;
-      if (p < pieces) quant_quarter(raw[j], p);
+      if (p < pieces) quant_piece(raw[j], p);
     }
   } else {
     for (int p = tid; p < pieces; p += 256) {
       load_piece(p, raw[0]);
-      quant_quarter(raw[0], p);
+      quant_piece(raw[0], p);
     }
   }
   // every store of every thread complete (vmcnt counts stores too on this target), then the count
@@ -791,7 +742,7 @@ void decode_tile_kernel(const DecodeArgs d) {
   int bx = (int)blockIdx.x;
   if constexpr (PROD) {
     if (bx < d.nprod) {
-      if (blockIdx.y == 0) quant_token_publish(d, bx / d.prod_per_token, bx % d.prod_per_token);
+      if (blockIdx.y == 0) quant_token_publish(d, bx);
       return;
     }
     bx -= d.nprod;
@@ -1349,10 +1300,10 @@ int decode_impl(const aqtx_decode_plan* p, const void* x, const void* w, const f
   const int64_t w_bytes = p->n * (pk ? p->k / 2 : p->k);
   const bool pays = path == 1 || (w_bytes >= (24ll << 20) && p->m <= (pk ? 16 : 32));
   if (p->workspace_zeroed && path != 2 && pays) {
-    // one producer per token: four (a quarter of every piece each) measured 0.1-0.4 us slower up to 8 tokens and
-    // 2-4 us slower from 32 on, where their workgroups delay the readers' start
-    d.prod_per_token = ((p->tuning >> 24) & 15) == 4 ? 4 : 1;
-    d.nprod = (int)p->m * d.prod_per_token;
+    // (four producers per token, a quarter of every piece each, measured 0.1-0.4 us slower up to 8 tokens and 2-4 us
+    // slower from 32 on, where their workgroups delay the readers' start; so did four workgroups per token in the
+    // quantize launch of the two-launch form)
+    d.nprod = (int)p->m;
     d.ctrl = reinterpret_cast<int*>(ws);
     const bool expire = ((p->tuning >> 20) & 15) == 1;  // test hook: a count that never comes, a wait of a microsecond
     d.wait_target = expire ? d.nprod + 1 : d.nprod;

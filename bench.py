@@ -676,7 +676,7 @@ def main():
                    'launch_ms': gemm_ms, 'launches_timed': len(timer.pairs)},
   }
   if not args.no_decode:
-    line['decode'] = {'kernel': 'aqtx_decode_i8 (m <= 2: decode_fused_kernel; m >= 3: decode_quant_kernel + decode_tile_kernel)',
+    line['decode'] = {'kernel': 'aqtx_decode_i8 (m <= 2: decode_fused_kernel; m >= 3: decode_tile_kernel, its first workgroups quantizing the tokens against a weight of 24 MiB or more and up to 32 tokens, else behind decode_quant_kernel)',
                       'k': 4096,
                       'timing': 'HIP graph replay, weights rotated through 1 GiB', 'shapes': decode_bench(dev)}
   if not args.no_other_configs:

@@ -394,8 +394,7 @@ typedef struct aqtx_decode_plan {
                              bits 16-19 path: 1 = few tokens take the path of many as well (no kernel in
                              which every workgroup quantizes the activations itself), 2 = that, with
                              the activations quantized by a launch of their own.  Bits 20-23: 1 = the
-                             wait of aqtx_decode_i8_check's description expires at once (error-path tests).
-                             Bits 24-27: 4 = four quantizing workgroups per token instead of one          */
+                             wait of aqtx_decode_i8_check's description expires at once (error-path tests)  */
   int32_t w_layout;       /* AQTX_W_ROWS | AQTX_W_FRAGMENTS */
   int32_t workspace_zeroed; /* 1: the caller keeps one workspace across calls on one stream and its first
                              aqtx_decode_exchange_bytes(plan) bytes were zero before the first call.

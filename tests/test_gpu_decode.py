@@ -30,9 +30,8 @@ def _weights(n, k, seed, w_sdt):
 
 
 # aqtx_decode_plan.tuning bits 16-19: the library's choice of kernels; the many-token kernel for every m, its first
-# workgroups quantizing the tokens (one per token, or four); the same with the quantisation in a launch of its own
-PATHS = pytest.mark.parametrize('path', [0, 1 << 16, (1 << 16) | (4 << 24), 2 << 16],
-                                ids=['auto', 'producers', 'producers4', 'two_launches'])
+# workgroups quantizing the tokens; the same with the quantisation in a launch of its own
+PATHS = pytest.mark.parametrize('path', [0, 1 << 16, 2 << 16], ids=['auto', 'producers', 'two_launches'])
 
 
 @PATHS
