@@ -18,6 +18,7 @@ SCALE_ROW_THEN_COL, SCALE_COL_THEN_ROW = range(2)
 W_ROWS, W_FRAGMENTS = range(2)
 K_NATURAL, K_EVEN_ODD8 = range(2)
 ACC_FAST, ACC_F32 = range(2)
+FACTOR_ROWS, FACTOR_COLS = range(2)
 
 
 class QuantPlan(ctypes.Structure):
@@ -38,6 +39,17 @@ class QuantPlan(ctypes.Structure):
       ('workspace_zeroed', ctypes.c_int32),
       ('key_device', ctypes.c_void_p),
       ('out_k_order', ctypes.c_int32),
+  ]
+
+
+class ScalePlan(ctypes.Structure):
+  _fields_ = [
+      ('in_dtype', ctypes.c_int32), ('out_dtype', ctypes.c_int32),
+      ('batch', ctypes.c_int64), ('rows', ctypes.c_int64), ('cols', ctypes.c_int64),
+      ('factors', ctypes.c_int32),
+      ('factor_axis', ctypes.c_int32 * 2), ('factor_dtype', ctypes.c_int32 * 2),
+      ('factor_recast', ctypes.c_int32 * 2),
+      ('factor_stride_b', ctypes.c_int64 * 2),
   ]
 
 
@@ -111,6 +123,7 @@ SYMBOLS = {
                                      ctypes.c_size_t, _vp]),
     'aqtx_quantize_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(QuantPlan)]),
     'aqtx_dequantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp]),
+    'aqtx_scale_cast': (ctypes.c_int, [ctypes.POINTER(ScalePlan), _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8_k_slices': (ctypes.c_int, [ctypes.POINTER(GemmPlan)]),
     'aqtx_gemm_fp8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -17,7 +17,7 @@ LIB_DIR = os.path.join(HERE, 'lib')
 LIB_PATH = os.path.join(LIB_DIR, 'libaqtx.so')
 
 SOURCES = ['capi.hip', 'quantize.hip', 'gemm_i8.hip', 'gemm_mid.hip', 'gemm_fp8.hip', 'decode_i8.hip', 'decode_wo.hip', 'reduce.hip',
-           'gemm_i8_frag.hip', 'gemm_wo.hip', 'gemm_grouped.hip', 'fp_round.hip', 'im2col.hip']
+           'gemm_i8_frag.hip', 'gemm_wo.hip', 'gemm_grouped.hip', 'fp_round.hip', 'im2col.hip', 'scale_cast.hip']
 
 HIPCC_FLAGS = [
     '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC',

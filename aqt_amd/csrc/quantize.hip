@@ -1165,6 +1165,23 @@ extern "C" int aqtx_dequantize(const aqtx_quant_plan* p, const void* q, const fl
   const int64_t total = p->batch * p->rows * p->cols;
   if (total == 0) return 0;
   AQTX_REQUIRE(q != nullptr && scale != nullptr && out != nullptr, "aqtx_dequantize: NULL buffer");
+  if (!p->transpose_out && p->group == 0) {
+    // q in the order of the result and one scale per row, per column or per (batch) tensor: the
+    // 16-columns-per-lane kernel of aqtx_scale_cast, same arithmetic
+    aqtx_scale_plan sp{};
+    sp.in_dtype = p->out_dtype; sp.out_dtype = p->in_dtype;
+    sp.batch = p->batch; sp.rows = p->rows; sp.cols = p->cols;
+    sp.factors = 1; sp.factor_dtype[0] = p->scale_dtype;
+    if (p->reduce == AQTX_REDUCE_COLS) {
+      sp.factor_axis[0] = AQTX_FACTOR_ROWS; sp.factor_stride_b[0] = p->rows;
+    } else if (p->reduce == AQTX_REDUCE_ROWS) {
+      sp.factor_axis[0] = AQTX_FACTOR_COLS; sp.factor_stride_b[0] = p->cols;
+    } else {
+      sp.rows = 1; sp.cols = p->rows * p->cols;
+      sp.factor_axis[0] = AQTX_FACTOR_ROWS; sp.factor_stride_b[0] = p->reduce == AQTX_REDUCE_ALL ? 1 : 0;
+    }
+    return aqtx_scale_cast(&sp, q, scale, nullptr, out, stream);
+  }
   QArgs a{};
   a.x = q; a.q = out; a.scale = const_cast<float*>(scale);
   a.batch = p->batch; a.rows = p->rows; a.cols = p->cols;

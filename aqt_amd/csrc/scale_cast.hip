@@ -1,0 +1,203 @@
+// aqtx_scale_cast: one elementwise pass from a quantized (or float) tensor to the operand of a float
+// contraction, or from the result of one to the dequantized output: cast, then up to two factors that
+// have one value per row or per column.  HBM-bound: 16 consecutive columns per lane, read and written
+// with 16-byte accesses; a scalar kernel takes shapes whose rows are not multiples of 16 columns or
+// whose buffers are not 16-byte aligned.
+#include "common.h"
+
+namespace aqtx {
+namespace {
+
+struct ScaleArgs {
+  const void* x;
+  void* out;
+  const float* f[2];
+  int64_t rows, cols, total;   // rows of one batch entry, columns, elements of the whole tensor
+  int64_t fsb[2];              // batch stride of each factor
+  int32_t nf;
+  int32_t fcols[2];            // 1: one value per column, 0: one value per row
+  int32_t fbf[2];              // 1: the factor's values are bf16 values
+  int32_t recast[2];
+  int32_t in_dtype;
+  int32_t out_bf;
+};
+
+__device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
+
+// the products of one element; `vbf` follows the dtype jnp's promotion gives the running value
+__device__ __forceinline__ float apply(float v, const ScaleArgs& a, float f0, float f1) {
+  int vbf = a.out_bf;
+  v = rnd(v, vbf);
+  if (a.nf > 0) {
+    if (a.recast[0]) { v = rnd(v, a.out_bf); vbf = a.out_bf; }
+    v = v * f0;
+    vbf &= a.fbf[0];
+    v = rnd(v, vbf);
+  }
+  if (a.nf > 1) {
+    if (a.recast[1]) { v = rnd(v, a.out_bf); vbf = a.out_bf; }
+    v = v * f1;
+    vbf &= a.fbf[1];
+    v = rnd(v, vbf);
+  }
+  return rnd(v, a.out_bf);
+}
+
+__device__ __forceinline__ float decode_byte(uint32_t byte, int in_dtype) {
+  if (in_dtype == AQTX_E4M3) return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0);
+  if (in_dtype == AQTX_E5M2) return __builtin_amdgcn_cvt_f32_bf8((int)byte, 0);
+  return (float)(int8_t)byte;
+}
+
+// IN: bytes per input element (1, 2 or 4).  One lane = 16 consecutive columns of one row.
+template <int IN, bool OUT_BF>
+__global__ __launch_bounds__(256) void scale_cast_vec_kernel(const ScaleArgs a) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 16;
+  if (i0 >= a.total) return;
+  const int64_t row = i0 / a.cols;          // row of the flattened [batch * rows, cols] matrix
+  const int64_t c0 = i0 - row * a.cols;
+  const int64_t b = row / a.rows, r = row - b * a.rows;
+
+  float v[16];
+  if constexpr (IN == 1) {
+    const uint4 w = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.x) + i0);
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = decode_byte((words[j >> 2] >> (8 * (j & 3))) & 0xFFu, a.in_dtype);
+  } else if constexpr (IN == 2) {
+    const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.x) + i0);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint4 w = p[h];
+      const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[8 * h + j] = bf16_bits_to_float((uint16_t)(words[j >> 1] >> (16 * (j & 1))));
+    }
+  } else {
+    const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.x) + i0);
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const float4 w = p[h];
+      v[4 * h] = w.x; v[4 * h + 1] = w.y; v[4 * h + 2] = w.z; v[4 * h + 3] = w.w;
+    }
+  }
+
+  float f[2][16];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    if (i < a.nf) {
+      if (a.fcols[i]) {
+        const float4* p = reinterpret_cast<const float4*>(a.f[i] + b * a.fsb[i] + c0);
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          const float4 w = p[h];
+          f[i][4 * h] = w.x; f[i][4 * h + 1] = w.y; f[i][4 * h + 2] = w.z; f[i][4 * h + 3] = w.w;
+        }
+      } else {
+        const float s = a.f[i][b * a.fsb[i] + r];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) f[i][j] = s;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) f[i][j] = 1.0f;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 16; ++j) v[j] = apply(v[j], a, f[0][j], f[1][j]);
+
+  if constexpr (OUT_BF) {
+    uint4* o = reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.out) + i0);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        w[j] = (uint32_t)bf16_bits(v[8 * h + 2 * j]) | ((uint32_t)bf16_bits(v[8 * h + 2 * j + 1]) << 16);
+      o[h] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  } else {
+    float4* o = reinterpret_cast<float4*>(reinterpret_cast<float*>(a.out) + i0);
+#pragma unroll
+    for (int h = 0; h < 4; ++h) o[h] = make_float4(v[4 * h], v[4 * h + 1], v[4 * h + 2], v[4 * h + 3]);
+  }
+}
+
+// one element per lane: any shape, any alignment
+__global__ __launch_bounds__(256) void scale_cast_scalar_kernel(const ScaleArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.total) return;
+  const int64_t row = i / a.cols, c = i - row * a.cols;
+  const int64_t b = row / a.rows, r = row - b * a.rows;
+  float v;
+  if (a.in_dtype == AQTX_F32) v = reinterpret_cast<const float*>(a.x)[i];
+  else if (a.in_dtype == AQTX_BF16) v = bf16_bits_to_float(reinterpret_cast<const uint16_t*>(a.x)[i]);
+  else v = decode_byte(reinterpret_cast<const uint8_t*>(a.x)[i], a.in_dtype);
+  float f[2] = {1.0f, 1.0f};
+  for (int k = 0; k < a.nf; ++k) f[k] = a.f[k][b * a.fsb[k] + (a.fcols[k] ? c : r)];
+  v = apply(v, a, f[0], f[1]);
+  if (a.out_bf) reinterpret_cast<uint16_t*>(a.out)[i] = bf16_bits(v);
+  else reinterpret_cast<float*>(a.out)[i] = v;
+}
+
+}  // namespace
+}  // namespace aqtx
+
+using namespace aqtx;
+
+extern "C" int aqtx_scale_cast(const aqtx_scale_plan* p, const void* x, const float* f0, const float* f1,
+                               void* out, void* stream) {
+  clear_error();
+  AQTX_REQUIRE(p != nullptr, "aqtx_scale_cast: plan is NULL");
+  const bool in_byte = p->in_dtype == AQTX_I8 || p->in_dtype == AQTX_I4 || p->in_dtype == AQTX_E4M3 ||
+                       p->in_dtype == AQTX_E5M2;
+  AQTX_REQUIRE(in_byte || is_float_dtype(p->in_dtype), "aqtx_scale_cast: unsupported in_dtype %d", p->in_dtype);
+  AQTX_REQUIRE(is_float_dtype(p->out_dtype), "aqtx_scale_cast: out_dtype must be f32 or bf16, got %d", p->out_dtype);
+  AQTX_REQUIRE(p->batch >= 0 && p->rows >= 0 && p->cols >= 0, "aqtx_scale_cast: negative shape");
+  AQTX_REQUIRE(p->factors >= 0 && p->factors <= 2, "aqtx_scale_cast: factors must be 0, 1 or 2, got %d", p->factors);
+  const float* fs[2] = {f0, f1};
+  ScaleArgs a{};
+  for (int i = 0; i < p->factors; ++i) {
+    AQTX_REQUIRE(p->factor_axis[i] == AQTX_FACTOR_ROWS || p->factor_axis[i] == AQTX_FACTOR_COLS,
+                 "aqtx_scale_cast: unknown factor_axis %d", p->factor_axis[i]);
+    AQTX_REQUIRE(is_float_dtype(p->factor_dtype[i]), "aqtx_scale_cast: factor_dtype must be f32 or bf16, got %d",
+                 p->factor_dtype[i]);
+    AQTX_REQUIRE(p->factor_stride_b[i] >= 0, "aqtx_scale_cast: negative factor stride");
+    a.f[i] = fs[i];
+    a.fsb[i] = p->factor_stride_b[i];
+    a.fcols[i] = p->factor_axis[i] == AQTX_FACTOR_COLS;
+    a.fbf[i] = p->factor_dtype[i] == AQTX_BF16;
+    a.recast[i] = p->factor_recast[i] != 0;
+  }
+  const int64_t total = p->batch * p->rows * p->cols;
+  if (total == 0) return 0;
+  AQTX_REQUIRE(x != nullptr && out != nullptr, "aqtx_scale_cast: NULL buffer");
+  for (int i = 0; i < p->factors; ++i)
+    AQTX_REQUIRE(fs[i] != nullptr && ((uintptr_t)fs[i] % 4) == 0, "aqtx_scale_cast: factor %d is NULL or unaligned", i);
+  const size_t isz = dtype_size(p->in_dtype), osz = dtype_size(p->out_dtype);
+  AQTX_REQUIRE(((uintptr_t)x % isz) == 0 && ((uintptr_t)out % osz) == 0, "aqtx_scale_cast: buffer not element aligned");
+  a.x = x; a.out = out;
+  a.rows = p->rows; a.cols = p->cols; a.total = total;
+  a.nf = p->factors; a.in_dtype = p->in_dtype; a.out_bf = p->out_dtype == AQTX_BF16;
+
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  bool vec = p->cols % 16 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  for (int i = 0; i < p->factors; ++i)
+    if (a.fcols[i]) vec = vec && ((uintptr_t)fs[i] % 16) == 0 && a.fsb[i] % 4 == 0;
+  if (vec) {
+    const int64_t blocks = (total / 16 + 255) / 256;
+    AQTX_REQUIRE(blocks < (1ll << 31), "aqtx_scale_cast: tensor too large for one launch");
+    const dim3 grid((unsigned)blocks);
+#define AQTX_SC(IN) do { if (a.out_bf) scale_cast_vec_kernel<IN, true><<<grid, 256, 0, st>>>(a); \
+                         else scale_cast_vec_kernel<IN, false><<<grid, 256, 0, st>>>(a); } while (0)
+    if (isz == 1) AQTX_SC(1); else if (isz == 2) AQTX_SC(2); else AQTX_SC(4);
+#undef AQTX_SC
+    AQTX_HIP_CHECK_LAUNCH("scale_cast_vec_kernel");
+  } else {
+    const int64_t blocks = (total + 255) / 256;
+    AQTX_REQUIRE(blocks < (1ll << 31), "aqtx_scale_cast: tensor too large for one launch");
+    scale_cast_scalar_kernel<<<dim3((unsigned)blocks), 256, 0, st>>>(a);
+    AQTX_HIP_CHECK_LAUNCH("scale_cast_scalar_kernel");
+  }
+  return 0;
+}

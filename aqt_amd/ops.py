@@ -731,6 +731,36 @@ def random_bits(key, n: int, bit_width: int = 32, partitionable: bool = False, d
   return out
 
 
+def scale_cast(x: torch.Tensor, factors=(), *, out_dtype, in_dtype=None) -> torch.Tensor:
+  """out = cast(x) times up to two factors, each with one value per (batch, row) or per (batch, column).
+
+  x is [batch, rows, cols], contiguous: int8 / fp8 bytes (`in_dtype` says which: I8, I4, E4M3, E5M2; default
+  from x.dtype) or bf16 / f32.  `factors`: tuples (vector, axis, dtype, recast) with vector float32 [batch, rows]
+  / [batch, cols] (or [rows] / [cols], shared between the batch entries), axis L.FACTOR_ROWS | L.FACTOR_COLS,
+  dtype the dtype its values are held in, recast whether the running value is cast to out_dtype first.
+  """
+  _require_gpu(x)
+  assert x.dim() == 3 and x.is_contiguous() and len(factors) <= 2
+  b, r, c = x.shape
+  plan = L.ScalePlan()
+  if in_dtype is None:
+    in_dtype = L.I8 if x.dtype in (torch.int8, torch.uint8) else aqtx_dtype(x.dtype)
+  plan.in_dtype, plan.out_dtype = in_dtype, aqtx_dtype(out_dtype)
+  plan.batch, plan.rows, plan.cols = b, r, c
+  plan.factors = len(factors)
+  ptrs = [None, None]
+  for i, (vec, axis, dt, recast) in enumerate(factors):
+    n = r if axis == L.FACTOR_ROWS else c
+    assert vec.dtype == torch.float32 and vec.is_contiguous() and vec.numel() in (n, b * n), (vec.shape, axis, x.shape)
+    _require_gpu(vec)
+    plan.factor_axis[i], plan.factor_dtype[i], plan.factor_recast[i] = axis, aqtx_dtype(dt), int(bool(recast))
+    plan.factor_stride_b[i] = n if vec.numel() == b * n and b > 1 else 0
+    ptrs[i] = _ptr(vec)
+  out = torch.empty((b, r, c), dtype=_AQTX_TO_TORCH[plan.out_dtype], device=x.device)
+  L.check(L.lib().aqtx_scale_cast(ctypes.byref(plan), _ptr(x), ptrs[0], ptrs[1], _ptr(out), _stream()))
+  return out
+
+
 def dequantize(q: torch.Tensor, scale: torch.Tensor, *, reduce: int, q_dtype: int, out_dtype,
                scale_dtype=None, group: int = 0, transposed: bool = False):
   """out = cast(q) * scale for q as written by `quantize` (one scale).

@@ -27,6 +27,7 @@ from aqt_amd.v2 import lowering
 from aqt_amd.v2 import transpose
 from aqt_amd.v2 import utils
 from aqt_amd.v2.numerics import fp8_numerics
+from aqt_amd.v2.numerics import int_numerics
 from aqt_amd.v2.numerics import no_numerics
 
 dtypes_allowed_for_int32_accum = [utils.int4, utils.int8]
@@ -697,13 +698,12 @@ class DotGeneralRaw:
       return out, None
 
   def _dispatch(self, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, out_transpose_axes, bwd_memo=None):
-    """The fused kernels where they implement the configuration, the step-by-step path otherwise."""
+    """The lowered paths where they implement the configuration (_lowered_call: the int8 / fp8 kernels for
+    the default modes, _float_contraction for the modes that contract in float), the step-by-step path
+    otherwise."""
     # a ragged (grouped) contraction hook is lowered too: same kernels, rows looked up per group
     fusable = ((self.dot_general is lax_dot_general or _ragged_sizes(self.dot_general) is not None)
                and type(self.dg_quantizer) is DefaultDotGeneralQuantizer)  # pylint: disable=unidiomatic-typecheck
-    for side in (self.lhs, self.rhs):
-      fusable = fusable and (side.dequant_mode == DequantMode.OUTPUT
-                             and side.calibration_mode == CalibrationMode.CONTRACTING_AXIS)
     calibrated = {}  # id(quantizer) -> scales found step by step during the fused attempt
     if fusable:
       try:
@@ -721,12 +721,11 @@ class DotGeneralRaw:
     """The operator one step at a time: calibrate, quantize, contract, dequantize.
 
     Follows aqt_dot_general.py:795-828 through the plugin points (`dg_quantizer`,
-    `dot_general`), so configurations without a fused kernel still run on the GPU: custom
-    quantizers and contraction hooks, fake quantization (DequantMode.THIS_INPUT), scaling of
-    the other operand (OTHER_INPUT), calibration over the remaining axes, one-sided
-    quantization, clip_gradient, biases in fake-quant mode.  Each step is its own kernel (the
-    quantize / dequantize kernels, the MFMA or library contraction) with elementwise tensor
-    arithmetic in between.
+    `dot_general`), so what the lowered paths leave out still runs on the GPU: quantizers,
+    numerics and contraction hooks of the user's own, numerics whose results are not integers
+    (no rounding, no clipping, buckets centred off zero), mid scales, biases, sparsity masks and
+    several scales per tensor.  Each step is its own kernel (the quantize and scale-and-cast
+    kernels, the MFMA or library contraction) with elementwise tensor arithmetic in between.
     """
     if isinstance(lhs, _Prescaled):
       lhs = lhs.x * lhs.scale_t.to(lhs.x.dtype)
@@ -795,11 +794,20 @@ class DotGeneralRaw:
                                        out_transpose_axes, dequant_dtype)
       if served is not None:
         return served
-    if not isinstance(dq, DefaultDotGeneralQuantizer) or lhs_none or rhs_none:
-      raise _NotFused(
-          'only DefaultDotGeneralQuantizer with both sides quantized (or both unquantized) is lowered')
+    if not isinstance(dq, DefaultDotGeneralQuantizer):
+      raise _NotFused('only DefaultDotGeneralQuantizer is lowered')
     if dq.lhs_mid_alpha is not None or dq.rhs_mid_alpha is not None:
       raise _NotFused('mid-scale quantization has no HIP path yet')
+    default_modes = all(side.dequant_mode == DequantMode.OUTPUT
+                        and side.calibration_mode == CalibrationMode.CONTRACTING_AXIS for side in (self.lhs, self.rhs))
+    held_float = any(isinstance(q.numerics, int_numerics.IntSymmetric) and q.numerics.dtype is None
+                     for q in (dq.lhs, dq.rhs))
+    given_float = any(qt is not None and qt.is_full() and qt.qvalue.is_floating_point()
+                      and qt.qvalue.dtype not in _FP8_DTYPES for qt in (lhs_qt, rhs_qt))
+    if lhs_none or rhs_none or not default_modes or held_float or given_float:
+      return self._float_contraction(lhs, rhs_arr, rhs_is_q, lhs_dtype, rhs_dtype, dequant_dtype, lhs_qt, rhs_qt,
+                                     dimension_numbers, prescale_t, out_transpose_axes, lhs_none, rhs_none,
+                                     _bwd_memo, _calibrated)
 
     ragged = _ragged_sizes(self.dot_general)
     if ragged is not None:
@@ -916,6 +924,183 @@ class DotGeneralRaw:
                         rhs=TensorRes(mt=rhs_mt, quant_grad=rhs_grad))
     return out, res
 
+  def _float_contraction(self, lhs, rhs_arr, rhs_is_q, lhs_dtype, rhs_dtype, dequant_dtype, lhs_qt, rhs_qt,
+                         dimension_numbers, prescale_t, out_transpose_axes, lhs_none, rhs_none,
+                         bwd_memo, calibrated):
+    """The configurations whose contraction is a float one (aqt_dot_general.py:843-958): fake quantization
+    (DequantMode.THIS_INPUT), the scale of one operand multiplied into the other (OTHER_INPUT), calibration
+    over the remaining axes, one side left unquantized.
+
+    Per quantized side one calibrate-and-quantize kernel sequence (the residual the backward pass needs) and
+    one pass of the scale-and-cast kernel that makes the side's contraction operand (its own scale and / or
+    the other side's; a bare cast for an integer side next to a float one); the library's float product; one
+    more scale-and-cast pass over the result when a side is dequantized there (DequantMode.OUTPUT).
+    """
+    dq = self.dg_quantizer
+    if self.dot_general is not lax_dot_general:
+      raise _NotFused('a custom DotGeneralRaw.dot_general hook is not lowered')
+    dn = _canonical_pairs(lhs, rhs_arr, dimension_numbers)
+    (lca, rca), (lba, rba) = dn
+    lra = utils.get_remaining_axes(lhs.dim(), lca, lba)
+    rra = utils.get_remaining_axes(rhs_arr.dim(), rca, rba)
+
+    class Side:
+      pass
+
+    def make(name, x, dtype, x_is_q, quantizer, given, cfg, ba, ra, ca, none, prescale):
+      sd = Side()
+      sd.cfg, sd.none = cfg, none
+      sd.by_k = cfg.calibration_mode == CalibrationMode.REMAINING_AXIS  # one scale per (batch, contraction index)
+      if none:
+        if given is not None or x_is_q:
+          raise _NotFused(f'{name}: a provided QTensor next to NoNumerics')
+        if prescale is not None:
+          x = x * prescale.to(x.dtype)
+        sd.v = lowering.view_operand(x, ba, ra, ca)
+        sd.mem, sd.x, sd.grad, sd.s32, sd.sdt = sd.v.mem, x, None, None, None
+        sd.k_inner = sd.v.k_last  # mem is [B, R, K] (else [B, K, R])
+        sd.qt = aqt_tensor.QTensor(qvalue=x, scale=[], scale_t=None, bias=[], dequant_dtype=x.dtype)
+        sd.kdt = sd.held = None
+        return sd
+      # the quantizer's view: the axes that share a scale take the place of the contraction axes
+      va, vk = (ca, ra) if sd.by_k else (ra, ca)
+      if x_is_q and x.is_floating_point() and x.dtype not in _FP8_DTYPES:
+        x, x_is_q = x.to(dtype), False  # a residual held in a float dtype: qvalue.astype(dequant_dtype)
+      q, s32, sdt, qt, grad = self._quant_side(name, x, dtype, x_is_q, quantizer, given, ba, va, vk, prescale,
+                                               bwd_memo, calibrated, held_float=True)
+      given_full = given is not None and given.is_full()
+      sd.v = lowering.view_operand(qt.qvalue if given_full else x, ba, va, vk)
+      n = sd.v.B * sd.v.R
+      if s32.numel() not in (1, n):
+        raise _NotFused(f'{name}: a scale that is not shared over exactly the calibration axes')
+      sd.s32 = s32.reshape(-1).expand(n).contiguous() if s32.numel() == 1 and n != 1 else s32.reshape(-1)
+      if qt.dequant_dtype is None:
+        raise _NotFused(f'{name}: a QTensor without a dequant_dtype')
+      sd.held = None  # the quantized values as the float tensor the reference holds, [B, R, K] of the view
+      if not given_full and getattr(quantizer.numerics, 'dtype', 0) is None:
+        # numerics that keep their integers in the float dtype (the usual fake-quant setting): the kernel
+        # wrote them as int8, which holds the same values; the residual is their cast
+        held_dt = torch.promote_types(dtype, sdt)
+        sd.held = (ops.scale_cast(q, [], out_dtype=held_dt) if q.numel()
+                   else torch.empty(q.shape, dtype=held_dt, device=q.device))
+        qt = qt.replace(qvalue=lowering.logical_from_brk(sd.held, sd.v), container_dtype=None)
+      elif qt.qvalue.dtype.is_floating_point and qt.qvalue.dtype not in _FP8_DTYPES:
+        sd.held = q
+      elif qt.qvalue.dtype != torch.int8 and qt.qvalue.dtype not in _FP8_DTYPES:
+        raise _NotFused(f'{name}: quantized values held in {qt.qvalue.dtype}')
+      sd.mem, sd.x, sd.grad, sd.sdt, sd.qt = q, x, grad, sdt, qt
+      sd.k_inner = not sd.by_k  # q is [B, R, K] with contraction-axis scales, [B, K, R] with remaining-axis ones
+      sd.kdt = None if q.is_floating_point() and q.dtype not in _FP8_DTYPES else (
+          L.I8 if q.dtype == torch.int8 and sd.held is not None else aqt_tensor.qvalue_kernel_dtype(qt))
+      return sd
+
+    L_ = make('lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, self.lhs, lba, lra, lca, lhs_none, prescale_t)
+    R_ = make('rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, self.rhs, rba, rra, rca, rhs_none, None)
+
+    msg = ('biases are only supported in fake quant mode, but got a {arg} bias '
+           'and self.{arg}.dequant_mode == {mode} != DequantMode.THIS_INPUT')
+    for arg, sd in (('lhs', L_), ('rhs', R_)):
+      assert not (sd.qt.bias and sd.cfg.dequant_mode != DequantMode.THIS_INPUT), msg.format(
+          arg=arg, mode=sd.cfg.dequant_mode)
+      if sd.qt.bias or sd.qt.sparsity_mask is not None or (not sd.none and len(sd.qt.scale) != 1):
+        raise _NotFused('a bias, a sparsity mask or several scales')
+
+    # dtypes of the two operands of the reference's lax.dot_general call
+    def qin_dtype(sd, dtype):
+      if sd.none or sd.cfg.dequant_mode == DequantMode.THIS_INPUT:
+        return sd.qt.dequant_dtype if not sd.none else sd.x.dtype
+      return sd.qt.qvalue.dtype
+    ldt, rdt = qin_dtype(L_, lhs_dtype), qin_dtype(R_, rhs_dtype)
+    if self.dg_accumulator_dtype == utils.int32:
+      assert ldt == utils.int8 and rdt == utils.int8, (
+          f'Found {self.dg_accumulator_dtype=}, lhs_qin.dtype={ldt} and rhs_qin.dtype={rdt}. Dot general '
+          'accumulator dtype can only be jnp.int32 when both inputs are int8. Otherwise it is '
+          'recommended to be None to let lax.dot_general automatically decide it.')
+    if L_.cfg.dequant_mode == DequantMode.OTHER_INPUT and not L_.none:
+      assert rdt in _DTYPES_CAN_BE_SCALED
+    if R_.cfg.dequant_mode == DequantMode.OTHER_INPUT and not R_.none:
+      assert ldt in _DTYPES_CAN_BE_SCALED
+    if not ldt.is_floating_point and not rdt.is_floating_point or ldt in _FP8_DTYPES or rdt in _FP8_DTYPES:
+      raise _NotFused('an integer or fp8 contraction outside the default modes')
+    common = torch.promote_types(ldt, rdt)
+    if common not in (torch.bfloat16, torch.float32):
+      raise _NotFused(f'a contraction in {common}')
+
+    def operand(sd, other, qdt):
+      """This side's operand of the float product, in the layout of sd.mem; qdt: the dtype the reference holds
+      it in when it reaches lax.dot_general."""
+      factors = []
+      if not sd.none and sd.cfg.dequant_mode == DequantMode.THIS_INPUT:
+        factors.append((sd.s32, L.FACTOR_ROWS, sd.sdt, False))  # QTensor.dequant
+      if not other.none and other.cfg.dequant_mode == DequantMode.OTHER_INPUT:
+        if not other.by_k:
+          raise _NotFused('DequantMode.OTHER_INPUT with a scale that varies along the remaining axes')
+        k_count = sd.v.R if (not sd.none and sd.by_k) else sd.v.K
+        if other.s32.numel() != sd.v.B * k_count:
+          raise _NotFused('a scale that does not fit the other operand')
+        # the scale is cast to the dtype of the operand it multiplies (aqt_dot_general.py:893, 902)
+        t = other.s32 if qdt == torch.float32 or other.sdt == qdt else other.s32.to(qdt).float()
+        factors.append((t, L.FACTOR_COLS if sd.k_inner else L.FACTOR_ROWS, qdt, True))
+      if not factors:
+        if sd.held is not None:
+          return sd.held if sd.held.dtype == common else sd.held.to(common)
+        if sd.mem.dtype == common:
+          return sd.mem
+        if sd.mem.is_floating_point() and sd.mem.dtype not in _FP8_DTYPES or sd.mem.numel() == 0:
+          return sd.mem.to(common)
+        qdt = common  # an integer operand next to a float one: jnp's type promotion casts it
+      mem = sd.mem.view(torch.uint8) if sd.mem.dtype in _FP8_DTYPES else sd.mem
+      if mem.numel() == 0:
+        return torch.empty(mem.shape, dtype=common, device=mem.device)
+      out = ops.scale_cast(mem.contiguous(), factors, out_dtype=qdt, in_dtype=sd.kdt)
+      return out if out.dtype == common else out.to(common)
+
+    def logical(t, sd):
+      """The [B, R, K] or [B, K, R] operand indexed like the tensor it was made from."""
+      if sd.none and not sd.k_inner:
+        # mem is [B, K, R] of the caller's own view
+        v = sd.v
+        dims = [v.shape[a] for a in v.b_axes + v.k_axes + v.r_axes]
+        axes = v.b_axes + v.k_axes + v.r_axes
+        inv = [0] * len(axes)
+        for pos, a in enumerate(axes):
+          inv[a] = pos
+        return t.reshape(dims).permute(tuple(inv))
+      return lowering.logical_from_brk(t, sd.v)
+
+    lop = logical(operand(L_, R_, ldt), L_)
+    if (WEIGHT_ONLY_FLOAT_COPY and rhs_qt is not None and rhs_qt.is_full() and not rdt.is_floating_point
+        and L_.cfg.dequant_mode != DequantMode.OTHER_INPUT):
+      rop = R_.qt.qvalue  # a frozen weight: lax_dot_general keeps its float copy between calls
+    else:
+      rop = logical(operand(R_, L_, rdt), R_)
+    out = lax_dot_general(lop, rop, dn, None, self.dg_accumulator_dtype)  # (batch..., lhs remaining..., rhs remaining...)
+
+    nb = len(lba)
+    bdims = [lhs.shape[a] for a in lba]
+    ldims = [lhs.shape[a] for a in lra]
+    rdims = [rhs_arr.shape[a] for a in rra]
+    B, M, N = math.prod(bdims), math.prod(ldims), math.prod(rdims)
+    factors = []
+    for sd, axis, count in ((L_, L.FACTOR_ROWS, M), (R_, L.FACTOR_COLS, N)):
+      if sd.none or sd.cfg.dequant_mode != DequantMode.OUTPUT:
+        continue
+      if sd.by_k or sd.s32.numel() != B * count:
+        raise _NotFused('DequantMode.OUTPUT with a scale along the contraction axes')
+      factors.append((sd.s32, axis, sd.sdt, False))
+    if factors and out.numel():
+      out = ops.scale_cast(out.reshape(B, M, N).contiguous(), factors, out_dtype=dequant_dtype)
+    out = out.to(dequant_dtype).reshape(bdims + ldims + rdims)
+    want_lba = list(dimension_numbers[1][0])
+    if want_lba != lba:
+      perm = [lba.index(a) for a in want_lba] + list(range(nb, out.dim()))
+      out = out.permute(tuple(perm))
+    if out_transpose_axes is not None:
+      out = out.permute(tuple(out_transpose_axes))
+    res = DotGeneralRes(lhs=TensorRes(mt=MultiTensor(x=L_.x, qx=L_.qt), quant_grad=L_.grad),
+                        rhs=TensorRes(mt=MultiTensor(x=R_.x, qx=R_.qt), quant_grad=R_.grad))
+    return out, res
+
   def _serve_small_batch(self, lhs, lhs_dtype, dq, lhs_qt, rhs_arr, rhs_qt, dn, prescale_t,
                          out_transpose_axes, dequant_dtype, dimension_numbers):
     """Serving with a frozen int8 rhs and at most 64 lhs rows: the fused decode kernel.
@@ -1022,10 +1207,16 @@ class DotGeneralRaw:
     return out, res
 
   def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t,
-                  bwd_memo=None, calibrated=None, layout_later=False):
+                  bwd_memo=None, calibrated=None, layout_later=False, held_float=False):
     """Quantizes one side; returns (q [B,R,K], scale f32, scale dtype, QTensor, quant_grad).
     `bwd_memo`: the backward pass's table of per-tensor scales; `calibrated`: where a calibration
-    that runs step by step leaves its result for a later fall-back of the same call."""
+    that runs step by step leaves its result for a later fall-back of the same call; `held_float`:
+    numerics that keep their integers in the float dtype are taken too (q and the QTensor come back
+    as int8, the caller casts)."""
+    def numerics_spec():
+      if isinstance(quantizer.numerics, no_numerics.NoNumerics):
+        return None
+      return quantizer.numerics.kernel_spec(True) if held_float else quantizer.numerics.kernel_spec()
     if given_qt is not None and given_qt.is_full():
       # Serving: the provided QTensor replaces the computed one (aqt_dot_general.py:614-635).
       quant_grad = None if self.allow_dummy_gradient_into_qtensor else _POISON
@@ -1042,12 +1233,12 @@ class DotGeneralRaw:
         q = q.view(torch.uint8)
       s = given_qt.scale[0]
       return q, _scale_vector_f32(s, ba, ra, ca), s.dtype, given_qt, quant_grad
-    spec = quantizer.kernel_spec()
+    spec = quantizer.kernel_spec(held_float)
     if spec is None and given_qt is None:
       # The numerics have a kernel but the calibration does not (power-of-two or clipped
       # scales, constant bounds, static-range and delayed-scaling statistics...): calibrate step
       # by step, then quantize and contract in the fused kernels with that scale.
-      nspec = None if isinstance(quantizer.numerics, no_numerics.NoNumerics) else quantizer.numerics.kernel_spec()
+      nspec = numerics_spec()
       if nspec is None or quantizer._calibrator is None:
         raise _NotFused(f'{name}: numerics/calibration {quantizer.numerics} / '
                         f'{quantizer.calibration} have no fused HIP kernel')
@@ -1064,7 +1255,7 @@ class DotGeneralRaw:
         raise _NotFused(f'{name}: calibration with a bias, a sparsity mask or several scales')
       spec = nspec
     elif spec is None:
-      spec = None if isinstance(quantizer.numerics, no_numerics.NoNumerics) else quantizer.numerics.kernel_spec()
+      spec = numerics_spec()
     if spec is None:
       raise _NotFused(f'{name}: numerics {quantizer.numerics} have no fused HIP kernel')
     arr = x
@@ -1096,7 +1287,7 @@ class DotGeneralRaw:
     # forward-scale factor on it the abs-max is the same number, found once per backward pass.
     memo_key, memo_hit = None, None
     if (bwd_memo is not None and given_qt is None and prescale is None and not x_is_q
-        and quantizer.calib_shared_axes == 'per_tensor' and quantizer.kernel_spec() is not None):
+        and quantizer.calib_shared_axes == 'per_tensor' and quantizer.kernel_spec(held_float) is not None):
       memo_key = (arr.data_ptr(), arr._version, tuple(arr.shape), arr.dtype, spec['quant_bound'],
                   quantizer._calibrator.dtype)
       memo_hit = bwd_memo.get(memo_key)
@@ -1105,7 +1296,7 @@ class DotGeneralRaw:
         scale_in = flat.contiguous().reshape(v.B, v.R, 1) if v.k_last else flat.contiguous().reshape(v.B, 1, v.R)
         scale_dtype = memo_hit[2]
     q, s32, sdt = quantizer.quant_view(v, dtype, calibration_axes=ca, prescale=prescale, scale=scale_in,
-                                       scale_dtype=scale_dtype)
+                                       scale_dtype=scale_dtype, held_float=held_float)
     qv = lowering.logical_from_brk(aqt_quantizer._typed(q, spec['out_dtype']), v)
     if memo_hit is not None:
       s32, scale_list = memo_hit[0], memo_hit[1]

@@ -71,23 +71,27 @@ class Quantizer:
       self._calibrator.init_calibration()
 
   # ---- fused lowering (this build) ----------------------------------------------
-  def kernel_spec(self):
+  def kernel_spec(self, held_float: bool = False):
     """Plan fields if numerics + calibration are covered by the fused kernel, else None."""
     if isinstance(self.numerics, no_numerics.NoNumerics):
       return None
-    spec = self.numerics.kernel_spec()
+    # (a numerics class of the user's own may define kernel_spec() without the argument)
+    spec = self.numerics.kernel_spec(True) if held_float else self.numerics.kernel_spec()
     if spec is None or self._calibrator is None or not self._calibrator.kernel_supported():
       return None
     return spec
 
   def quant_view(self, v: lowering.OperandView, dtype, *, calibration_axes, prescale=None,
-                 scale: Optional[torch.Tensor] = None, scale_dtype=None):
+                 scale: Optional[torch.Tensor] = None, scale_dtype=None, held_float: bool = False):
     """Calibrate + quantize an operand view in one kernel sequence.
 
     With `scale` (float32, one value per [B, R] entry, holding values of `scale_dtype`) the
     calibration is skipped.  Returns (q [B,R,K], scale float32 [B,R] or [1], scale dtype).
     """
-    spec = self.kernel_spec() if scale is None else self.numerics.kernel_spec()
+    if scale is None:
+      spec = self.kernel_spec(held_float)
+    else:
+      spec = self.numerics.kernel_spec(True) if held_float else self.numerics.kernel_spec()
     assert spec is not None
     if scale is not None:
       per_tensor = False

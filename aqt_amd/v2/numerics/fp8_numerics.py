@@ -48,7 +48,7 @@ class Fp8Numerics(numerics.AqtNumerics):
   def get_quant_bound(self):
     return self._get_edge_of_last_fp8_bucket()
 
-  def kernel_spec(self):
+  def kernel_spec(self, held_float: bool = False):
     if self.dtype == utils.float8_e4m3fn:
       assert (self.exponent_bits, self.mantissa_bits) == (4, 3)
       out = L.E4M3

@@ -55,21 +55,31 @@ class IntSymmetric(numerics.AqtNumerics):
   def get_dtype(self):
     return self.dtype
 
-  def kernel_spec(self):
-    """Fields of the quantize plan, or None if the kernels do not cover this setting."""
+  def kernel_spec(self, held_float: bool = False):
+    """Fields of the quantize plan, or None if the kernels do not cover this setting.
+
+    held_float: the caller also takes numerics that keep the rounded values in the float dtype
+    (dtype None, the usual setting of fake quantization) when they fit an int8: the kernel then
+    writes int8 and the caller casts, which gives the same values; the plan says so in 'held_float'."""
     if not (self.clip and self.round and self.preserve_zero):
       return None
+    held = False
     if self.dtype is utils.int8:
       out = L.I8
     elif self.dtype is utils.int4:
       out = L.I4
+    elif self.dtype is None and held_float and self.bits <= 8:
+      out, held = L.I8, True
     else:
       return None
     noise, sharing = _noise_kind(self.noise_fn)
     if noise is None or sharing:
       return None
-    return dict(out_dtype=out, quant_bound=float(self.get_quant_bound()),
+    spec = dict(out_dtype=out, quant_bound=float(self.get_quant_bound()),
                 clip_bound=float(self._get_fwd_clip_bound()), noise=noise)
+    if held:
+      spec['held_float'] = True
+    return spec
 
   def vjp_fwd(self, x, context):
     """Noise, clip, round, cast of an already scaled tensor (int_numerics.py:81-111)."""

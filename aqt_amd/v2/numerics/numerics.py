@@ -25,5 +25,5 @@ class AqtNumerics(abc.ABC):
   def vjp_bwd(self, res, grad):
     pass
 
-  def kernel_spec(self):
+  def kernel_spec(self, held_float: bool = False):
     return None

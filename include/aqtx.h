@@ -137,6 +137,49 @@ size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* plan);
 int aqtx_dequantize(const aqtx_quant_plan* plan, const void* q, const float* scale, void* out,
                     void* stream);
 
+/*
+ * Plan of aqtx_scale_cast: one elementwise pass that turns a quantized (or float) tensor into the
+ * operand of a FLOAT contraction, or scales the result of one.  x is [batch, rows, cols], row-major;
+ * the result has the same shape in out_dtype:
+ *     v = cast(x[b, r, c]) rounded to out_dtype
+ *     for each factor i < factors, in order:
+ *        if factor_recast[i]: v is rounded to out_dtype (and is held in out_dtype from here on)
+ *        v = v * f_i[...]  in the promoted dtype of v and factor_dtype[i] (bf16 x bf16 rounds to bf16;
+ *                          anything with a float32 side is a float32 product and v stays float32)
+ *     out[b, r, c] = v rounded to out_dtype
+ * A factor has one value per (batch, row) (AQTX_FACTOR_ROWS: f_i[b * factor_stride_b[i] + r]) or per
+ * (batch, col) (AQTX_FACTOR_COLS: f_i[b * factor_stride_b[i] + c]); stride 0 shares it between the batch
+ * entries.  The values are float32 words holding values of factor_dtype[i].
+ */
+enum { AQTX_FACTOR_ROWS = 0, AQTX_FACTOR_COLS = 1 };
+
+typedef struct aqtx_scale_plan {
+  int32_t in_dtype;           /* AQTX_I8 | AQTX_I4 (container) | AQTX_E4M3 | AQTX_E5M2 | AQTX_BF16 | AQTX_F32 */
+  int32_t out_dtype;          /* AQTX_BF16 | AQTX_F32                                              */
+  int64_t batch, rows, cols;
+  int32_t factors;            /* 0, 1 or 2                                                         */
+  int32_t factor_axis[2];     /* AQTX_FACTOR_*                                                     */
+  int32_t factor_dtype[2];    /* AQTX_BF16 | AQTX_F32: the dtype the factor's values are held in    */
+  int32_t factor_recast[2];   /* 1: v is cast to out_dtype before this factor multiplies           */
+  int64_t factor_stride_b[2]; /* batch stride of the factor vector, in elements                    */
+} aqtx_scale_plan;
+
+/*
+ * aqtx_scale_cast replaces, for the configurations whose contraction is a float one:
+ * QTensor.dequant of one operand before the contraction (DequantMode.THIS_INPUT, _maybe_dequant,
+ * aqt/jax/v2/aqt_dot_general.py:853-866, with aqt_tensor.py:161-200: one factor, the operand's own scale),
+ * the multiplication by the OTHER operand's transposed scale (DequantMode.OTHER_INPUT,
+ * aqt_dot_general.py:887-903: a second factor with factor_recast = 1, or the only one next to a bare cast),
+ * the cast of an integer operand that meets a float one in lax.dot_general (no factor), and QTensor.dequant of
+ * the contraction's result by the scales of the operands in DequantMode.OUTPUT (aqt_dot_general.py:929-958
+ * with aqt_tensor.py:161-200: x float, one factor per such operand).
+ *   x   in  : [batch, rows, cols] of in_dtype
+ *   f0, f1  : float32 factor vectors (NULL beyond plan->factors)
+ *   out out : [batch, rows, cols] of out_dtype (may not alias x unless the dtypes have the same size)
+ */
+int aqtx_scale_cast(const aqtx_scale_plan* plan, const void* x, const float* f0, const float* f1,
+                    void* out, void* stream);
+
 enum { AQTX_SCALE_ROW_THEN_COL = 0, AQTX_SCALE_COL_THEN_ROW = 1 };
 
 /*

@@ -442,3 +442,18 @@ def test_conv_validation():
   assert 'multiple of 128' in _err(call(w, _gplan(**dict(good, k=9 * 64, lda=9 * 64, ldb=9 * 64))))
   w.c, w.rank = 128, 4
   assert 'rank' in _err(call(w, _gplan(**good)))
+
+
+def test_scale_cast_rejects_bad_plans():
+  plan = L.ScalePlan()
+  plan.in_dtype, plan.out_dtype = L.I8, L.I8
+  plan.batch, plan.rows, plan.cols = 1, 4, 16
+  rc = L.lib().aqtx_scale_cast(ctypes.byref(plan), None, None, None, None, None)
+  assert rc != 0 and b'out_dtype must be f32 or bf16' in L.lib().aqtx_last_error()
+  plan.out_dtype, plan.factors = L.BF16, 3
+  rc = L.lib().aqtx_scale_cast(ctypes.byref(plan), None, None, None, None, None)
+  assert rc != 0 and b'factors must be 0, 1 or 2' in L.lib().aqtx_last_error()
+  plan.factors = 1
+  plan.factor_axis[0], plan.factor_dtype[0] = 5, L.F32
+  rc = L.lib().aqtx_scale_cast(ctypes.byref(plan), None, None, None, None, None)
+  assert rc != 0 and b'unknown factor_axis' in L.lib().aqtx_last_error()

@@ -43,6 +43,14 @@ def _close(got, want, dt):
   np.testing.assert_allclose(got, want, rtol=rtol, atol=atol)
 
 
+@pytest.fixture
+def lowered_only(monkeypatch):
+  """The call has to stay on the lowered kernels: the step-by-step path raises."""
+  def no_step_by_step(self, *a, **k):
+    raise AssertionError('the step-by-step path was taken')
+  monkeypatch.setattr(aqt.DotGeneralRaw, '_unfused_call', no_step_by_step)
+
+
 def _raw_pair(lhs_bits=8, rhs_bits=8, *, lmode='output', rmode='output', lcal='ca', rcal='ca',
               keep_float=False, acc='auto', calib=None):
   """A product DotGeneralRaw and the oracle RawCfg with the same settings."""
@@ -92,9 +100,10 @@ def _assert_residuals_equal(res, lres, rres):
     ('fake_lhs_only', dict(lmode='this_input', rmode='output')),
 ])
 @pytest.mark.parametrize('dn,ls,rs', [(MATMUL, (48, 96), (96, 40)), (BATCHED, (3, 20, 64), (3, 64, 24))])
-def test_dequant_and_calibration_modes(gpu, name, kw, dt, dn, ls, rs):
+def test_dequant_and_calibration_modes(gpu, name, kw, dt, dn, ls, rs, lowered_only):
   """aqt_dot_general_test.py:761-903 walks these combinations; here each one is checked
-  against the oracle.  Float-held operands make the contraction a float one."""
+  against the oracle.  Float-held operands make the contraction a float one.  All of them run on the
+  lowered path: quantize kernels, one scale-and-cast pass per operand, the library's float product."""
   raw, oraw = _raw_pair(acc=None, **kw)
   lhs, rhs = U.rand(ls, dt, 1, outliers=True), U.rand(rs, dt, 2, 0.05)
   out, res, want, lres, rres = _run_raw(raw, oraw, lhs, rhs, dt, dn, gpu)
@@ -104,7 +113,7 @@ def test_dequant_and_calibration_modes(gpu, name, kw, dt, dn, ls, rs):
 
 @pytest.mark.parametrize('dt', ['f32', 'bf16'])
 @pytest.mark.parametrize('lhs_bits,rhs_bits', [(None, 8), (8, None), (None, 4)])
-def test_one_sided_quantization(gpu, lhs_bits, rhs_bits, dt):
+def test_one_sided_quantization(gpu, lhs_bits, rhs_bits, dt, lowered_only):
   """Weight-only / activation-only: the int8 side is promoted to the float dtype for the
   contraction, its scale multiplies the output."""
   raw, oraw = _raw_pair(lhs_bits, rhs_bits)
