@@ -132,6 +132,29 @@ ffi::Error DequantizeImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::Buffer<ffi:
   return Status(aqtx_dequantize(&p, q.untyped_data(), scale.typed_data(), out->untyped_data(), stream));
 }
 
+// ---- aqtx_scale_cast ----------------------------------------------------------------------------
+// x [batch, rows, cols] -> out of the same shape; f0 / f1 f32 factor vectors (a one-element dummy for a factor
+// the plan does not use).  in_dtype is an attribute for the same reason as out_dtype above.
+ffi::Error ScaleCastImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi::F32> f0, ffi::Buffer<ffi::F32> f1,
+                         ffi::Result<ffi::AnyBuffer> out, int32_t in_dtype, int32_t factors, int32_t factor0_axis,
+                         int32_t factor0_dtype, int32_t factor0_recast, int64_t factor0_stride_b,
+                         int32_t factor1_axis, int32_t factor1_dtype, int32_t factor1_recast,
+                         int64_t factor1_stride_b) {
+  auto dims = out->dimensions();
+  if (dims.size() != 3) return Bad("aqtx_scale_cast: out must be [batch, rows, cols]");
+  aqtx_scale_plan p{};
+  p.in_dtype = in_dtype;
+  p.out_dtype = Dtype(out->element_type());
+  p.batch = dims[0]; p.rows = dims[1]; p.cols = dims[2];
+  p.factors = factors;
+  p.factor_axis[0] = factor0_axis; p.factor_dtype[0] = factor0_dtype;
+  p.factor_recast[0] = factor0_recast; p.factor_stride_b[0] = factor0_stride_b;
+  p.factor_axis[1] = factor1_axis; p.factor_dtype[1] = factor1_dtype;
+  p.factor_recast[1] = factor1_recast; p.factor_stride_b[1] = factor1_stride_b;
+  return Status(aqtx_scale_cast(&p, x.untyped_data(), factors > 0 ? f0.typed_data() : nullptr,
+                                factors > 1 ? f1.typed_data() : nullptr, out->untyped_data(), stream));
+}
+
 // ---- aqtx_gemm_i8 / aqtx_gemm_fp8 ---------------------------------------------------------------
 // a [batch, m, k], b [batch, n, k] -> c [batch, m, n]; scales f32 [batch, m] / [batch, n].
 int FillGemmPlan(aqtx_gemm_plan* p, const ffi::AnyBuffer& a, const ffi::AnyBuffer& b, ffi::DataType c_type,
@@ -185,11 +208,12 @@ ffi::Error GemmI8RawImpl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b,
 // fp8 operands: e4m3fn / e5m2 per operand from the buffers' element types.
 ffi::Error GemmFp8Impl(hipStream_t stream, ffi::AnyBuffer a, ffi::AnyBuffer b, ffi::Buffer<ffi::F32> row_scale,
                        ffi::Buffer<ffi::F32> col_scale, ffi::Result<ffi::AnyBuffer> c, int32_t dequant_dtype,
-                       int32_t row_scale_dtype, int32_t col_scale_dtype, int32_t scale_order) {
+                       int32_t row_scale_dtype, int32_t col_scale_dtype, int32_t scale_order, int32_t accumulate) {
   aqtx_gemm_plan p{};
   if (FillGemmPlan(&p, a, b, c->element_type(), Dtype(a.element_type()), Dtype(b.element_type()), dequant_dtype,
                    row_scale_dtype, col_scale_dtype, scale_order))
     return Bad("aqtx_gemm_fp8: operands must be [batch, m, k] and [batch, n, k]");
+  p.accumulate = accumulate;
   return Status(aqtx_gemm_fp8(&p, a.untyped_data(), b.untyped_data(), row_scale.typed_data(), col_scale.typed_data(),
                               c->untyped_data(), nullptr, stream));
 }
@@ -296,6 +320,20 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Attr<int64_t>("group").Attr<int32_t>("transposed"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
+    AqtxScaleCast, ScaleCastImpl,
+    ffi::Ffi::Bind()
+        .Ctx<ffi::PlatformStream<hipStream_t>>()
+        .Arg<ffi::AnyBuffer>()
+        .Arg<ffi::Buffer<ffi::F32>>()
+        .Arg<ffi::Buffer<ffi::F32>>()
+        .Ret<ffi::AnyBuffer>()
+        .Attr<int32_t>("in_dtype").Attr<int32_t>("factors")
+        .Attr<int32_t>("factor0_axis").Attr<int32_t>("factor0_dtype").Attr<int32_t>("factor0_recast")
+        .Attr<int64_t>("factor0_stride_b")
+        .Attr<int32_t>("factor1_axis").Attr<int32_t>("factor1_dtype").Attr<int32_t>("factor1_recast")
+        .Attr<int64_t>("factor1_stride_b"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxGemmI8, GemmI8Impl,
     ffi::Ffi::Bind()
         .Ctx<ffi::PlatformStream<hipStream_t>>()
@@ -327,7 +365,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Arg<ffi::Buffer<ffi::F32>>()
         .Ret<ffi::AnyBuffer>()
         .Attr<int32_t>("dequant_dtype").Attr<int32_t>("row_scale_dtype").Attr<int32_t>("col_scale_dtype")
-        .Attr<int32_t>("scale_order"));
+        .Attr<int32_t>("scale_order").Attr<int32_t>("accumulate"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxGemmI8Grouped, GemmI8GroupedImpl,

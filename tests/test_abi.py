@@ -339,7 +339,7 @@ def test_ffi_shim_binds_only_declared_entry_points():
     assert re.search(r'\b%s\b' % field, header), field
   handlers = re.findall(r'XLA_FFI_DEFINE_HANDLER_SYMBOL\(\s*(\w+)', src)
   assert {'AqtxQuantize', 'AqtxGemmI8', 'AqtxGemmFp8', 'AqtxGemmI8Grouped', 'AqtxDecodeI8', 'AqtxDequantize',
-          'AqtxSumTiles'} <= set(handlers)
+          'AqtxSumTiles', 'AqtxScaleCast'} <= set(handlers)
 
 
 def test_ffi_shim_is_skipped_without_xla_headers(capsys):
