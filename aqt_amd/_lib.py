@@ -50,6 +50,8 @@ class ScalePlan(ctypes.Structure):
       ('factor_axis', ctypes.c_int32 * 2), ('factor_dtype', ctypes.c_int32 * 2),
       ('factor_recast', ctypes.c_int32 * 2),
       ('factor_stride_b', ctypes.c_int64 * 2),
+      ('factor_reciprocal', ctypes.c_int32 * 2),
+      ('finish_clip', ctypes.c_float), ('finish_round', ctypes.c_int32),
   ]
 
 

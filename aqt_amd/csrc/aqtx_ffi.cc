@@ -139,7 +139,8 @@ ffi::Error ScaleCastImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi::
                          ffi::Result<ffi::AnyBuffer> out, int32_t in_dtype, int32_t factors, int32_t factor0_axis,
                          int32_t factor0_dtype, int32_t factor0_recast, int64_t factor0_stride_b,
                          int32_t factor1_axis, int32_t factor1_dtype, int32_t factor1_recast,
-                         int64_t factor1_stride_b) {
+                         int64_t factor1_stride_b, int32_t factor0_reciprocal, int32_t factor1_reciprocal,
+                         float finish_clip, int32_t finish_round) {
   auto dims = out->dimensions();
   if (dims.size() != 3) return Bad("aqtx_scale_cast: out must be [batch, rows, cols]");
   aqtx_scale_plan p{};
@@ -151,6 +152,8 @@ ffi::Error ScaleCastImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::Buffer<ffi::
   p.factor_recast[0] = factor0_recast; p.factor_stride_b[0] = factor0_stride_b;
   p.factor_axis[1] = factor1_axis; p.factor_dtype[1] = factor1_dtype;
   p.factor_recast[1] = factor1_recast; p.factor_stride_b[1] = factor1_stride_b;
+  p.factor_reciprocal[0] = factor0_reciprocal; p.factor_reciprocal[1] = factor1_reciprocal;
+  p.finish_clip = finish_clip; p.finish_round = finish_round;
   return Status(aqtx_scale_cast(&p, x.untyped_data(), factors > 0 ? f0.typed_data() : nullptr,
                                 factors > 1 ? f1.typed_data() : nullptr, out->untyped_data(), stream));
 }
@@ -331,7 +334,9 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Attr<int32_t>("factor0_axis").Attr<int32_t>("factor0_dtype").Attr<int32_t>("factor0_recast")
         .Attr<int64_t>("factor0_stride_b")
         .Attr<int32_t>("factor1_axis").Attr<int32_t>("factor1_dtype").Attr<int32_t>("factor1_recast")
-        .Attr<int64_t>("factor1_stride_b"));
+        .Attr<int64_t>("factor1_stride_b")
+        .Attr<int32_t>("factor0_reciprocal").Attr<int32_t>("factor1_reciprocal")
+        .Attr<float>("finish_clip").Attr<int32_t>("finish_round"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(
     AqtxGemmI8, GemmI8Impl,

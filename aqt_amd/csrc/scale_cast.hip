@@ -18,11 +18,22 @@ struct ScaleArgs {
   int32_t fcols[2];            // 1: one value per column, 0: one value per row
   int32_t fbf[2];              // 1: the factor's values are bf16 values
   int32_t recast[2];
+  int32_t recip[2];
   int32_t in_dtype;
   int32_t out_bf;
+  float clip;                  // 0: none
+  int32_t round;               // 0: none, 1: half to even, 2: floor + 0.5
 };
 
 __device__ __forceinline__ float rnd(float x, int bf) { return bf ? round_bf16(x) : x; }
+
+// a factor as it multiplies: itself, or its reciprocal in its own dtype, 1 where that is infinite
+__device__ __forceinline__ float factor_value(float f, int recip, int fbf) {
+  if (!recip) return f;
+  float i = rnd(1.0f / f, fbf);
+  if (isinf(i)) i = 1.0f;
+  return i;
+}
 
 // the products of one element; `vbf` follows the dtype jnp's promotion gives the running value
 __device__ __forceinline__ float apply(float v, const ScaleArgs& a, float f0, float f1) {
@@ -30,17 +41,21 @@ __device__ __forceinline__ float apply(float v, const ScaleArgs& a, float f0, fl
   v = rnd(v, vbf);
   if (a.nf > 0) {
     if (a.recast[0]) { v = rnd(v, a.out_bf); vbf = a.out_bf; }
-    v = v * f0;
+    v = v * factor_value(f0, a.recip[0], a.fbf[0]);
     vbf &= a.fbf[0];
     v = rnd(v, vbf);
   }
   if (a.nf > 1) {
     if (a.recast[1]) { v = rnd(v, a.out_bf); vbf = a.out_bf; }
-    v = v * f1;
+    v = v * factor_value(f1, a.recip[1], a.fbf[1]);
     vbf &= a.fbf[1];
     v = rnd(v, vbf);
   }
-  return rnd(v, a.out_bf);
+  v = rnd(v, a.out_bf);
+  if (a.clip > 0.0f) v = v < -a.clip ? -a.clip : (v > a.clip ? a.clip : v);  // a NaN stays one, as in jnp.clip
+  if (a.round == 1) v = rintf(v);
+  else if (a.round == 2) v = rnd(floorf(v) + 0.5f, a.out_bf);
+  return v;
 }
 
 __device__ __forceinline__ float decode_byte(uint32_t byte, int in_dtype) {
@@ -168,7 +183,12 @@ extern "C" int aqtx_scale_cast(const aqtx_scale_plan* p, const void* x, const fl
     a.fcols[i] = p->factor_axis[i] == AQTX_FACTOR_COLS;
     a.fbf[i] = p->factor_dtype[i] == AQTX_BF16;
     a.recast[i] = p->factor_recast[i] != 0;
+    a.recip[i] = p->factor_reciprocal[i] != 0;
   }
+  AQTX_REQUIRE(p->finish_clip >= 0.0f, "aqtx_scale_cast: negative finish_clip");
+  AQTX_REQUIRE(p->finish_round >= 0 && p->finish_round <= 2, "aqtx_scale_cast: finish_round must be 0, 1 or 2, got %d",
+               p->finish_round);
+  a.clip = p->finish_clip; a.round = p->finish_round;
   const int64_t total = p->batch * p->rows * p->cols;
   if (total == 0) return 0;
   AQTX_REQUIRE(x != nullptr && out != nullptr, "aqtx_scale_cast: NULL buffer");

@@ -731,13 +731,16 @@ def random_bits(key, n: int, bit_width: int = 32, partitionable: bool = False, d
   return out
 
 
-def scale_cast(x: torch.Tensor, factors=(), *, out_dtype, in_dtype=None) -> torch.Tensor:
+def scale_cast(x: torch.Tensor, factors=(), *, out_dtype, in_dtype=None, finish_clip=None,
+               finish_round: int = 0) -> torch.Tensor:
   """out = cast(x) times up to two factors, each with one value per (batch, row) or per (batch, column).
 
   x is [batch, rows, cols], contiguous: int8 / fp8 bytes (`in_dtype` says which: I8, I4, E4M3, E5M2; default
-  from x.dtype) or bf16 / f32.  `factors`: tuples (vector, axis, dtype, recast) with vector float32 [batch, rows]
-  / [batch, cols] (or [rows] / [cols], shared between the batch entries), axis L.FACTOR_ROWS | L.FACTOR_COLS,
-  dtype the dtype its values are held in, recast whether the running value is cast to out_dtype first.
+  from x.dtype) or bf16 / f32.  `factors`: tuples (vector, axis, dtype, recast[, reciprocal]) with vector float32
+  [batch, rows] / [batch, cols] (or [rows] / [cols], shared between the batch entries), axis L.FACTOR_ROWS |
+  L.FACTOR_COLS, dtype the dtype its values are held in, recast whether the running value is cast to out_dtype
+  first, reciprocal whether the factor divides (QTensor.quant).  finish_clip / finish_round (1: half to even,
+  2: floor + 0.5): the clipping and rounding of integer numerics on the result, which stays a float.
   """
   _require_gpu(x)
   assert x.dim() == 3 and x.is_contiguous() and len(factors) <= 2
@@ -749,7 +752,10 @@ def scale_cast(x: torch.Tensor, factors=(), *, out_dtype, in_dtype=None) -> torc
   plan.batch, plan.rows, plan.cols = b, r, c
   plan.factors = len(factors)
   ptrs = [None, None]
-  for i, (vec, axis, dt, recast) in enumerate(factors):
+  plan.finish_clip = float(finish_clip) if finish_clip else 0.0
+  plan.finish_round = finish_round
+  for i, (vec, axis, dt, recast, *more) in enumerate(factors):
+    plan.factor_reciprocal[i] = int(bool(more and more[0]))
     n = r if axis == L.FACTOR_ROWS else c
     assert vec.dtype == torch.float32 and vec.is_contiguous() and vec.numel() in (n, b * n), (vec.shape, axis, x.shape)
     _require_gpu(vec)

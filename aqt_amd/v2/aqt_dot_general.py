@@ -722,10 +722,10 @@ class DotGeneralRaw:
 
     Follows aqt_dot_general.py:795-828 through the plugin points (`dg_quantizer`,
     `dot_general`), so what the lowered paths leave out still runs on the GPU: quantizers,
-    numerics and contraction hooks of the user's own, numerics whose results are not integers
-    (no rounding, no clipping, buckets centred off zero), mid scales, biases, sparsity masks and
-    several scales per tensor.  Each step is its own kernel (the quantize and scale-and-cast
-    kernels, the MFMA or library contraction) with elementwise tensor arithmetic in between.
+    numerics and contraction hooks of the user's own, biases, sparsity masks and several scales
+    per tensor (mid scales kept in the QTensors).  Each step is its own kernel (the quantize and
+    scale-and-cast kernels, the MFMA or library contraction) with elementwise tensor arithmetic
+    in between.
     """
     if isinstance(lhs, _Prescaled):
       lhs = lhs.x * lhs.scale_t.to(lhs.x.dtype)
@@ -797,7 +797,21 @@ class DotGeneralRaw:
     if not isinstance(dq, DefaultDotGeneralQuantizer):
       raise _NotFused('only DefaultDotGeneralQuantizer is lowered')
     if dq.lhs_mid_alpha is not None or dq.rhs_mid_alpha is not None:
-      raise _NotFused('mid-scale quantization has no HIP path yet')
+      # Mid scales (aqt_dot_general.py:504-554): the calibration runs step by step (abs-max kernels over the
+      # remaining axes and arithmetic on the per-channel vectors, one elementwise division per operand); with
+      # skip_mid_scales, the reference's default, each side is left with one scale, and the quantize and
+      # contraction kernels take it from there as they take any given scale.
+      if lhs_qt is not None or rhs_qt is not None or rhs_is_q or lhs_none or rhs_none:
+        raise _NotFused('mid scales next to a provided QTensor, a forward residual or an unquantized side')
+      if prescale_t is not None:
+        lhs, prescale_t = lhs * prescale_t.to(lhs.dtype), None
+      record = {} if _calibrated is None else _calibrated
+      with aqt_quantizer.record_calibrations(record):
+        (_, lhs_qt), (_, rhs_qt) = dq.calibrate(lhs, rhs_arr, dimension_numbers, self.lhs.calibration_mode,
+                                                self.rhs.calibration_mode)
+      for qt in (lhs_qt, rhs_qt):
+        if len(qt.scale) != 1 or qt.bias or qt.sparsity_mask is not None:
+          raise _NotFused('mid scales kept in the QTensors (skip_mid_scales = False), a bias or a sparsity mask')
     default_modes = all(side.dequant_mode == DequantMode.OUTPUT
                         and side.calibration_mode == CalibrationMode.CONTRACTING_AXIS for side in (self.lhs, self.rhs))
     held_float = any(isinstance(q.numerics, int_numerics.IntSymmetric) and q.numerics.dtype is None
@@ -947,6 +961,16 @@ class DotGeneralRaw:
     class Side:
       pass
 
+    def mem_to_logical(t, v, rk):
+      """A [B, R', K'] (rk) or [B, K', R'] tensor of the view v, indexed like the tensor the view was made from."""
+      if rk:
+        return lowering.logical_from_brk(t, v)
+      axes = v.b_axes + v.k_axes + v.r_axes
+      inv = [0] * len(axes)
+      for pos, a in enumerate(axes):
+        inv[a] = pos
+      return t.reshape([v.shape[a] for a in axes]).permute(tuple(inv))
+
     def make(name, x, dtype, x_is_q, quantizer, given, cfg, ba, ra, ca, none, prescale):
       sd = Side()
       sd.cfg, sd.none = cfg, none
@@ -958,7 +982,7 @@ class DotGeneralRaw:
           x = x * prescale.to(x.dtype)
         sd.v = lowering.view_operand(x, ba, ra, ca)
         sd.mem, sd.x, sd.grad, sd.s32, sd.sdt = sd.v.mem, x, None, None, None
-        sd.k_inner = sd.v.k_last  # mem is [B, R, K] (else [B, K, R])
+        sd.rk = sd.k_inner = sd.v.k_last  # mem is [B, R, K] (else [B, K, R])
         sd.qt = aqt_tensor.QTensor(qvalue=x, scale=[], scale_t=None, bias=[], dequant_dtype=x.dtype)
         sd.kdt = sd.held = None
         return sd
@@ -966,6 +990,45 @@ class DotGeneralRaw:
       va, vk = (ca, ra) if sd.by_k else (ra, ca)
       if x_is_q and x.is_floating_point() and x.dtype not in _FP8_DTYPES:
         x, x_is_q = x.to(dtype), False  # a residual held in a float dtype: qvalue.astype(dequant_dtype)
+      num = quantizer.numerics
+      if ((given is None or not given.is_full()) and isinstance(num, int_numerics.IntSymmetric) and num.dtype is None
+          and num.noise_fn is None and num.kernel_spec(True) is None and not x_is_q and x.is_floating_point()):
+        # Results that are not integers (no rounding, no clipping, buckets centred off zero) and stay in the float
+        # dtype: the calibration as usual, then one scale-and-cast pass with the reciprocal scale and the
+        # numerics' clipping and rounding (aqt_tensor.py:125-159, int_numerics.py:81-111), in x's own layout.
+        if prescale is not None:
+          x = x * prescale.to(x.dtype)
+        if given is not None:
+          inc = given  # an incomplete QTensor: the scale is there already (aqt_dot_general.py:645-653)
+        else:
+          inc = quantizer.calibrate(x, calibration_axes=vk)
+          if calibrated is not None:
+            calibrated[id(quantizer)] = inc
+        if len(inc.scale) != 1 or inc.bias or inc.sparsity_mask is not None:
+          raise _NotFused(f'{name}: calibration with a bias, a sparsity mask or several scales')
+        scale = inc.scale[0]
+        sd.v = lowering.view_operand(x, ba, va, vk)
+        n = sd.v.B * sd.v.R
+        s32 = _scale_vector_f32(scale, ba, va, vk)
+        if s32.numel() not in (1, n):
+          raise _NotFused(f'{name}: a scale that is not shared over exactly the calibration axes')
+        sd.s32 = s32.reshape(-1).expand(n).contiguous() if s32.numel() == 1 and n != 1 else s32.reshape(-1)
+        sd.sdt, sd.rk = scale.dtype, sd.v.k_last
+        held_dt = torch.promote_types(dtype, sd.sdt)
+        if sd.v.mem.numel():
+          sd.held = ops.scale_cast(
+              sd.v.mem, [(sd.s32, L.FACTOR_ROWS if sd.rk else L.FACTOR_COLS, sd.sdt, False, True)], out_dtype=held_dt,
+              finish_clip=num._get_fwd_clip_bound() if num.clip else None,
+              finish_round=0 if not num.round else 1 if num.preserve_zero else 2)
+        else:
+          sd.held = torch.empty(sd.v.mem.shape, dtype=held_dt, device=x.device)
+        sd.mem, sd.x, sd.kdt = sd.held, x, None
+        sd.k_inner = sd.rk != sd.by_k
+        sd.qt = aqt_tensor.QTensor(qvalue=mem_to_logical(sd.held, sd.v, sd.rk), scale=[scale], scale_t=None, bias=[],
+                                   dequant_dtype=dtype)
+        sd.grad = (aqt_quantizer.clip_gradient_later(num, x, [scale]) if num.clip_gradient
+                   else functools.partial(num.vjp_bwd, (None,)))
+        return sd
       q, s32, sdt, qt, grad = self._quant_side(name, x, dtype, x_is_q, quantizer, given, ba, va, vk, prescale,
                                                bwd_memo, calibrated, held_float=True)
       given_full = given is not None and given.is_full()
@@ -989,7 +1052,8 @@ class DotGeneralRaw:
       elif qt.qvalue.dtype != torch.int8 and qt.qvalue.dtype not in _FP8_DTYPES:
         raise _NotFused(f'{name}: quantized values held in {qt.qvalue.dtype}')
       sd.mem, sd.x, sd.grad, sd.sdt, sd.qt = q, x, grad, sdt, qt
-      sd.k_inner = not sd.by_k  # q is [B, R, K] with contraction-axis scales, [B, K, R] with remaining-axis ones
+      sd.rk = True  # the quantize kernel writes [B, R', K'] of its view
+      sd.k_inner = not sd.by_k  # that is [B, R, K] with contraction-axis scales, [B, K, R] with remaining-axis ones
       sd.kdt = None if q.is_floating_point() and q.dtype not in _FP8_DTYPES else (
           L.I8 if q.dtype == torch.int8 and sd.held is not None else aqt_tensor.qvalue_kernel_dtype(qt))
       return sd
@@ -1031,7 +1095,7 @@ class DotGeneralRaw:
       it in when it reaches lax.dot_general."""
       factors = []
       if not sd.none and sd.cfg.dequant_mode == DequantMode.THIS_INPUT:
-        factors.append((sd.s32, L.FACTOR_ROWS, sd.sdt, False))  # QTensor.dequant
+        factors.append((sd.s32, L.FACTOR_ROWS if sd.rk else L.FACTOR_COLS, sd.sdt, False))  # QTensor.dequant
       if not other.none and other.cfg.dequant_mode == DequantMode.OTHER_INPUT:
         if not other.by_k:
           raise _NotFused('DequantMode.OTHER_INPUT with a scale that varies along the remaining axes')
@@ -1056,17 +1120,7 @@ class DotGeneralRaw:
       return out if out.dtype == common else out.to(common)
 
     def logical(t, sd):
-      """The [B, R, K] or [B, K, R] operand indexed like the tensor it was made from."""
-      if sd.none and not sd.k_inner:
-        # mem is [B, K, R] of the caller's own view
-        v = sd.v
-        dims = [v.shape[a] for a in v.b_axes + v.k_axes + v.r_axes]
-        axes = v.b_axes + v.k_axes + v.r_axes
-        inv = [0] * len(axes)
-        for pos, a in enumerate(axes):
-          inv[a] = pos
-        return t.reshape(dims).permute(tuple(inv))
-      return lowering.logical_from_brk(t, sd.v)
+      return mem_to_logical(t, sd.v, sd.rk)
 
     lop = logical(operand(L_, R_, ldt), L_)
     if (WEIGHT_ONLY_FLOAT_COPY and rhs_qt is not None and rhs_qt.is_full() and not rdt.is_floating_point

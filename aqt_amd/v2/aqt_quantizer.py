@@ -29,6 +29,21 @@ AbstractAqtCalibration = calibration.Calibration
 _REPLAY: 'contextvars.ContextVar' = contextvars.ContextVar('aqt_calibration_replay', default=None)
 
 
+# Where Quantizer.calibrate leaves its results while a lowered attempt runs a whole DotGeneralQuantizer.calibrate
+# step by step (id(quantizer) -> incomplete QTensor), so that a fall-back of the same call can replay them.
+_RECORD: 'contextvars.ContextVar' = contextvars.ContextVar('aqt_calibration_record', default=None)
+
+
+@contextlib.contextmanager
+def record_calibrations(into: dict):
+  """Inside, every Quantizer.calibrate also stores its result in `into` under the quantizer object's id."""
+  token = _RECORD.set(into)
+  try:
+    yield
+  finally:
+    _RECORD.reset(token)
+
+
 @contextlib.contextmanager
 def replay_calibrations(done: dict):
   """Inside, Quantizer.calibrate returns (once) what `done` holds for that quantizer object
@@ -140,8 +155,12 @@ class Quantizer:
     assert self._calibrator is not None, 'forgot self.init_calibration()?'
     scale, bias, sparsity_mask = self._calibrator.get_scale_and_bias_and_sparsity(
         x, shared_axes, self.numerics, self.context)
-    return aqt_tensor.QTensor(qvalue=None, sparsity_mask=sparsity_mask, scale=scale, scale_t=None,
-                              bias=bias, dequant_dtype=x.dtype, tiling_state=tiling_state)
+    out = aqt_tensor.QTensor(qvalue=None, sparsity_mask=sparsity_mask, scale=scale, scale_t=None,
+                             bias=bias, dequant_dtype=x.dtype, tiling_state=tiling_state)
+    record = _RECORD.get()
+    if record is not None:
+      record[id(self)] = out
+    return out
 
   def calculate_qvalue(self, x, qt: aqt_tensor.QTensor):
     """Quantize x with the scale in qt (aqt_quantizer.py:159-176)."""

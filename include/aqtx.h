@@ -144,9 +144,14 @@ int aqtx_dequantize(const aqtx_quant_plan* plan, const void* q, const float* sca
  *     v = cast(x[b, r, c]) rounded to out_dtype
  *     for each factor i < factors, in order:
  *        if factor_recast[i]: v is rounded to out_dtype (and is held in out_dtype from here on)
- *        v = v * f_i[...]  in the promoted dtype of v and factor_dtype[i] (bf16 x bf16 rounds to bf16;
+ *        f = f_i[...], or with factor_reciprocal[i] its reciprocal in factor_dtype[i], 1 where that is infinite
+ *            (the reciprocal of QTensor.quant, aqt_tensor.py:151-155)
+ *        v = v * f         in the promoted dtype of v and factor_dtype[i] (bf16 x bf16 rounds to bf16;
  *                          anything with a float32 side is a float32 product and v stays float32)
- *     out[b, r, c] = v rounded to out_dtype
+ *     v is rounded to out_dtype; then, in out_dtype:
+ *        finish_clip > 0:  v = clip(v, -finish_clip, finish_clip)
+ *        finish_round 1:   v = round half to even;  2: v = floor(v) + 0.5
+ *     out[b, r, c] = v
  * A factor has one value per (batch, row) (AQTX_FACTOR_ROWS: f_i[b * factor_stride_b[i] + r]) or per
  * (batch, col) (AQTX_FACTOR_COLS: f_i[b * factor_stride_b[i] + c]); stride 0 shares it between the batch
  * entries.  The values are float32 words holding values of factor_dtype[i].
@@ -162,6 +167,9 @@ typedef struct aqtx_scale_plan {
   int32_t factor_dtype[2];    /* AQTX_BF16 | AQTX_F32: the dtype the factor's values are held in    */
   int32_t factor_recast[2];   /* 1: v is cast to out_dtype before this factor multiplies           */
   int64_t factor_stride_b[2]; /* batch stride of the factor vector, in elements                    */
+  int32_t factor_reciprocal[2]; /* 1: the factor multiplies by its reciprocal (a scale that divides)  */
+  float finish_clip;          /* > 0: clip bound applied to the result; 0: none                    */
+  int32_t finish_round;       /* 0: none, 1: half to even, 2: floor + 0.5                          */
 } aqtx_scale_plan;
 
 /*
@@ -172,7 +180,10 @@ typedef struct aqtx_scale_plan {
  * aqt_dot_general.py:887-903: a second factor with factor_recast = 1, or the only one next to a bare cast),
  * the cast of an integer operand that meets a float one in lax.dot_general (no factor), and QTensor.dequant of
  * the contraction's result by the scales of the operands in DequantMode.OUTPUT (aqt_dot_general.py:929-958
- * with aqt_tensor.py:161-200: x float, one factor per such operand).
+ * with aqt_tensor.py:161-200: x float, one factor per such operand); and, with reciprocal factors and the
+ * finishing step, QTensor.quant + IntSymmetric.vjp_fwd for numerics whose results stay in the float dtype
+ * and need not be integers (round = False, clip = False, preserve_zero = False: aqt_tensor.py:125-159,
+ * numerics/int_numerics.py:81-111, without noise).
  *   x   in  : [batch, rows, cols] of in_dtype
  *   f0, f1  : float32 factor vectors (NULL beyond plan->factors)
  *   out out : [batch, rows, cols] of out_dtype (may not alias x unless the dtypes have the same size)

@@ -121,3 +121,33 @@ def test_dequantize_entry_point_takes_the_same_kernel(gpu):
       got = ops.dequantize(make(gpu), torch.from_numpy(f).to(gpu), reduce=reduce, q_dtype=L.I8, out_dtype=TORCH_DT[dd],
                            scale_dtype=TORCH_DT[sdt])
       np.testing.assert_array_equal(got.float().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize('shape', [(2, 24, 80), (1, 7, 40)])
+@pytest.mark.parametrize('axis', ['rows', 'cols'])
+@pytest.mark.parametrize('dt,sdt', [('bf16', 'bf16'), ('bf16', 'f32'), ('f32', 'f32'), ('f32', 'bf16')])
+@pytest.mark.parametrize('kw', [dict(round=False), dict(clip=False), dict(clip=False, round=False),
+                                dict(preserve_zero=False), dict(bits=1, preserve_zero=False),
+                                dict(preserve_zero=False, round=False), dict()])
+def test_reciprocal_factor_and_finish_are_quant_and_int_numerics(gpu, kw, dt, sdt, axis, shape):
+  """QTensor.quant (multiply by the reciprocal scale, 1 where it is infinite) followed by IntSymmetric.vjp_fwd
+  without noise and with the values kept in the float dtype, against the oracle's two functions: settings whose
+  results are not integers included.  One scale per row or per column; a zero and a tiny scale reach the
+  infinite-reciprocal rule."""
+  b, r, c = shape
+  q = R.QuantizerCfg(**{'bits': 8, 'keep_float': True, **kw})
+  rng = np.random.default_rng(7)
+  x = nm.cast(rng.standard_normal(shape).astype(np.float32) * np.float32(40.0), dt)
+  n = r if axis == 'rows' else c
+  s = _factor(rng, b * n, sdt) * np.float32(20.0)
+  s[0], s[1] = np.float32(0.0), nm.cast(np.float32(1e-39), sdt)
+  sc = s.reshape(b, n, 1) if axis == 'rows' else s.reshape(b, 1, n)
+  with np.errstate(over='ignore', divide='ignore'):
+    v, vdt = R.qtensor_quant(x, dt, [sc], sdt)
+  want, wdt = R.int_vjp_fwd(v, vdt, q)
+  assert wdt == vdt
+  got = ops.scale_cast(U.to_dev(x, dt, gpu), [(torch.from_numpy(s).to(gpu), L.FACTOR_ROWS if axis == 'rows' else L.FACTOR_COLS,
+                                               TORCH_DT[sdt], False, True)],
+                       out_dtype=TORCH_DT[vdt], finish_clip=R.int_clip_bound(q) if q.clip else None,
+                       finish_round=0 if not q.round else 1 if q.preserve_zero else 2)
+  np.testing.assert_array_equal(got.float().cpu().numpy(), want)

@@ -184,8 +184,8 @@ def test_calibration_variants_int8_path(gpu, kw, dt):
 @pytest.mark.parametrize('dt', ['f32', 'bf16'])
 @pytest.mark.parametrize('kw', [dict(round=False), dict(clip=False, round=False),
                                 dict(preserve_zero=False), dict(preserve_max_val=True)])
-def test_numerics_variants_float_held(gpu, kw, dt):
-  """IntSymmetric settings outside the fused kernel (int_numerics.py:81-111), values held in
+def test_numerics_variants_float_held(gpu, kw, dt, lowered_only):
+  """IntSymmetric settings whose results are not integers (int_numerics.py:81-111), values held in
   the input dtype, fake-quant dequantisation."""
   raw, oraw = _raw_pair(lmode='this_input', rmode='this_input', keep_float=True, acc=None)
   for q, oq in ((raw.dg_quantizer.lhs, oraw.lhs), (raw.dg_quantizer.rhs, oraw.rhs)):
@@ -318,7 +318,7 @@ def test_clip_gradient(gpu, dt, monkeypatch):
     np.testing.assert_array_equal(_np(got), _np(plain) * inside)
 
 
-def test_mid_quantization_known_answer(gpu):
+def test_mid_quantization_known_answer(gpu, lowered_only):
   """The reference's own vectors (aqt_dot_general_test.py:1169-1208): binary quantization
   rounds 1, 2, 4 (and 1, 4, 16) to one magnitude; with mid scales of alpha 0.5 and
   power-of-two scales it becomes lossless."""
