@@ -349,7 +349,59 @@ def other_configs(dev):
       'ms_per_step_from_python': round(ms, 3), 'TOPS': round(mlp_gop / ms, 1),
       'hip_graph_ms_per_step': round(ms_graph, 3), 'hip_graph_TOPS': round(mlp_gop / ms_graph, 1)}
   del graphed, xm, w1, w2, gm
+  # the configurations whose contraction is a float one, forward call at 4096^3 bf16, ms per call from Python
+  out['float_contraction_modes_fwd_4096x4096x4096_ms'] = float_modes(dev)
   return out
+
+
+def float_modes(dev, calls=10, warm=3, only=None):
+  """Forward calls of the configurations that contract in float (aqt_dot_general.py:843-958) at 4096 x 4096 x 4096,
+  bf16, int8 numerics, issued from Python: fake quantization with contraction-axis and with remaining-axis
+  calibration, a fake-quantized lhs against an int8 rhs dequantized at the output, the lhs scale applied to the
+  rhs (OTHER_INPUT), integers held in the float dtype, an unquantized lhs against a freshly quantized rhs; the
+  default int8 path beside them.  Returns {name: ms per call}."""
+  import torch
+  from aqt_amd.v2 import aqt_dot_general as aqt
+  m = k = n = 4096
+  lhs = torch.randn(m, k, device=dev).to(torch.bfloat16)
+  rhs = (torch.randn(k, n, device=dev) * 0.02).to(torch.bfloat16)
+  out_m, this_m, other_m = aqt.DequantMode.OUTPUT, aqt.DequantMode.THIS_INPUT, aqt.DequantMode.OTHER_INPUT
+  ca, ra = aqt.CalibrationMode.CONTRACTING_AXIS, aqt.CalibrationMode.REMAINING_AXIS
+
+  def make(lbits=8, rbits=8, lmode=out_m, rmode=out_m, lcal=ca, rcal=ca, held=False):
+    raw = aqt.dot_general_raw_make(lbits, rbits, initialize_calibration=False)
+    raw.lhs.dequant_mode, raw.rhs.dequant_mode = lmode, rmode
+    raw.lhs.calibration_mode, raw.rhs.calibration_mode = lcal, rcal
+    if (lmode, rmode) != (out_m, out_m) or held:
+      raw.dg_accumulator_dtype = None
+    if held:
+      raw.dg_quantizer.lhs.numerics.dtype = raw.dg_quantizer.rhs.numerics.dtype = None
+    raw.dg_quantizer.init_calibration()
+    return raw
+
+  cfgs = {
+      'int8_default': make(),
+      'fake_quant': make(lmode=this_m, rmode=this_m),
+      'fake_quant_float_held': make(lmode=this_m, rmode=this_m, held=True),
+      'fake_quant_remaining_axis': make(lmode=this_m, rmode=this_m, lcal=ra, rcal=ra),
+      'lhs_scale_into_rhs': make(lmode=other_m, rmode=this_m, lcal=ra, rcal=ra),
+      'fake_quant_lhs_int8_rhs': make(lmode=this_m),
+      'float_lhs_int8_rhs': make(lbits=None),
+  }
+  res = {}
+  with torch.no_grad():
+    for name, raw in cfgs.items():
+      if only is not None and name != only:
+        continue
+      for _ in range(warm):
+        raw(lhs, rhs, None, None, MATMUL)
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      for _ in range(calls):
+        raw(lhs, rhs, None, None, MATMUL)
+      torch.cuda.synchronize()
+      res[name] = round((time.perf_counter() - t0) / calls * 1e3, 3)
+  return res
 
 
 def _graph_replay_us(run, ncalls, reps=5):
@@ -598,6 +650,9 @@ def main():
   ap.add_argument('--power-probe', action='store_true',
                   help='only run the forward contraction back to back on all-zero and on quantized-normal operands while '
                        'sampling socket power and shader clock from the SMI tool, and exit')
+  ap.add_argument('--float-modes-probe', default=None, metavar='NAME',
+                  help="only issue 13 forward calls of one float-contraction configuration (a key of float_modes(), or "
+                       "'all') at 4096^3 bf16, print ms per call, and exit (for rocprofv3 runs)")
   ap.add_argument('--read-ceiling', action='store_true',
                   help='only sweep a pure reader over buffer sizes and launch shapes (what the memory system delivers '
                        'to a single pass over the serving weights and over 256 MiB / 1 GiB) and exit')
@@ -620,6 +675,9 @@ def main():
     return
   if args.power_probe:
     power_probe(dev)
+    return
+  if args.float_modes_probe is not None:
+    print(json.dumps(float_modes(dev, only=None if args.float_modes_probe == 'all' else args.float_modes_probe)))
     return
   if args.read_ceiling:
     best, rows = read_ceiling(dev, full=True)

@@ -140,7 +140,7 @@ def test_reciprocal_factor_and_finish_are_quant_and_int_numerics(gpu, kw, dt, sd
   x = nm.cast(rng.standard_normal(shape).astype(np.float32) * np.float32(40.0), dt)
   n = r if axis == 'rows' else c
   s = _factor(rng, b * n, sdt) * np.float32(20.0)
-  s[0], s[1] = np.float32(0.0), nm.cast(np.float32(1e-39), sdt)
+  s[0], s[1] = np.float32(0.0), nm.cast(np.full(1, 1e-39, np.float32), sdt)[0]
   sc = s.reshape(b, n, 1) if axis == 'rows' else s.reshape(b, 1, n)
   with np.errstate(over='ignore', divide='ignore'):
     v, vdt = R.qtensor_quant(x, dt, [sc], sdt)
