@@ -39,6 +39,8 @@ class QuantPlan(ctypes.Structure):
       ('workspace_zeroed', ctypes.c_int32),
       ('key_device', ctypes.c_void_p),
       ('out_k_order', ctypes.c_int32),
+      ('other_axis_absmax', ctypes.c_void_p),
+      ('absmax_partials', ctypes.c_void_p), ('absmax_parts', ctypes.c_int64),
   ]
 
 
@@ -124,6 +126,7 @@ SYMBOLS = {
     'aqtx_quantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp, _vp,
                                      ctypes.c_size_t, _vp]),
     'aqtx_quantize_workspace_bytes': (ctypes.c_size_t, [ctypes.POINTER(QuantPlan)]),
+    'aqtx_quantize_other_axis_parts': (ctypes.c_int64, [ctypes.POINTER(QuantPlan)]),
     'aqtx_dequantize': (ctypes.c_int, [ctypes.POINTER(QuantPlan), _vp, _vp, _vp, _vp]),
     'aqtx_scale_cast': (ctypes.c_int, [ctypes.POINTER(ScalePlan), _vp, _vp, _vp, _vp, _vp]),
     'aqtx_gemm_i8': (ctypes.c_int, [ctypes.POINTER(GemmPlan), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -52,6 +52,12 @@ struct QArgs {
   int scale_given;
   int ws_zeroed;  // the abs-max words of the workspace are zero on entry
   int even_odd8;  // rows kernel: bytes of each group of 8 outputs stored as elements 0,2,4,6,1,3,5,7
+  // Partial maxima of |q| along the axis that carries the scales, one byte per position of the reduced axis and
+  // part (aqtx_quant_plan::other_axis_absmax): written by a launch (oa_out), or read in place of an abs-max pass
+  // over this input (oa_in).
+  uint8_t* oa_out;
+  const uint8_t* oa_in;
+  int64_t oa_in_parts;
 };
 
 // Kernel-side copy of the arguments with the PRNG key taken from device memory when the caller
@@ -242,6 +248,20 @@ __device__ __forceinline__ uint32_t spec_quant(float v, float inv, uint64_t ctr,
     return spec_finish<SPEC>(t, a);
   }
 }
+// The same for the noiseless integer pipelines (SPEC 0 with integer out, SPEC 1), which also hands out the clipped
+// value before rounding: |q| = rint(|t|) and rint is monotonic, so a maximum of |q| can be kept as a maximum of
+// |t| (one instruction per element) and rounded once at the end.
+template <int SPEC>
+__device__ __forceinline__ uint32_t spec_quant_mag(float v, float inv, uint64_t ctr, const QArgs& a, float& t_clipped) {
+  static_assert(SPEC == 0 || SPEC == 1, "noiseless integer pipelines");
+  if constexpr (SPEC == 0) {
+    t_clipped = scaled_noisy_clipped(v, inv, ctr, a);
+    return to_qbyte(t_clipped, a.out_dtype);
+  } else {
+    t_clipped = __builtin_amdgcn_fmed3f(spec_scale<1>(v, inv, a), -a.clip_bound, a.clip_bound);
+    return __float_as_uint(t_clipped + 12582912.0f) & 0xFFu;
+  }
+}
 // the pair (i, i + half) from one threefry block (SPEC 2, original layout, i < half)
 __device__ __forceinline__ void pair_quant(float v0, float inv0, float v1, float inv1, uint32_t i,
                                            const QArgs& a, uint32_t& q0, uint32_t& q1) {
@@ -342,19 +362,36 @@ __device__ __forceinline__ uint2 pack8(const uint32_t (&q)[8], int even_odd8) {
 // A block is 256 threads, or 512 (LANES = 512: one long segment per block, half the row values per
 // thread, so that six waves fit a SIMD: the stochastic pipeline is bound by vector instruction
 // issue, and a wave issues one such instruction every ~12 cycles at best).
-template <typename TIn, int LANES, int ITERS, int SPEC, bool PAIR>
-__global__ __launch_bounds__(LANES == 512 ? 512 : 256, LANES == 512 ? 3 : (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1)
+// COLMAX (whole rows as segments, one per block, no PAIR): the grid is smaller than the number of rows, a block
+// walks rows blockIdx.x, + gridDim.x, ... and keeps, per column it owns, the largest |q| it wrote; at the end it
+// stores them as row blockIdx.x of QArgs::oa_out ([gridDim.x][cols] bytes): what a later pass that calibrates the
+// quantized values over the rows needs instead of reading them again.
+template <typename TIn, int LANES, int ITERS, int SPEC, bool PAIR, bool COLMAX = false>
+__global__ __launch_bounds__(LANES == 512 ? 512 : 256,
+                             (COLMAX && ITERS <= 2 && SPEC != 0) ? 7 : LANES == 512 ? 3 : (sizeof(TIn) == 2 && SPEC != 0) ? 4 : 1)
 void quant_rows_kernel(const QArgs a_in) {
   const QArgs a = with_device_key(a_in);
   constexpr int VEC = 8;
   constexpr int NT = LANES == 512 ? 512 : 256;
   constexpr int SEG_PER_BLOCK = NT / LANES;
   constexpr int NSET = PAIR ? 2 : 1;
+  static_assert(!COLMAX || (!PAIR && SEG_PER_BLOCK == 1), "column maxima: one whole row per block");
   __shared__ float smem[NSET][NT / 64];
   const int tid = threadIdx.x;
   const int lane = tid % LANES;
   const int64_t nseg_grid = PAIR ? a.nseg / 2 : a.nseg;
-  const int64_t seg0 = (int64_t)blockIdx.x * SEG_PER_BLOCK + tid / LANES;
+  float colmax[COLMAX ? ITERS : 1][VEC];  // largest clipped |x / scale| per column (rounded at the end)
+  if constexpr (COLMAX) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) colmax[it][e] = 0.0f;
+  }
+  for (int64_t blk = blockIdx.x;; blk += gridDim.x) {
+  if constexpr (COLMAX) {
+    if (blk >= nseg_grid) break;  // uniform over the block
+  }
+  const int64_t seg0 = blk * SEG_PER_BLOCK + tid / LANES;
   const bool active = seg0 < nseg_grid;
   const int64_t segs_per_row = a.cols / a.L;
 
@@ -456,8 +493,31 @@ void quant_rows_kernel(const QArgs a_in) {
         float t[VEC];
         v[0][it].get(t);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) q[e] = spec_quant<SPEC>(t[e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a);
+        for (int e = 0; e < VEC; ++e) {
+          if constexpr (COLMAX) {
+            float tc;
+            q[e] = spec_quant_mag<SPEC>(t[e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a, tc);
+            colmax[it][e] = fmaxf(colmax[it][e], fabsf(tc));
+          } else {
+            q[e] = spec_quant<SPEC>(t[e], inv[0], ctr_row + (uint64_t)((j0 + e) * a.nsc), a);
+          }
+        }
         *reinterpret_cast<uint2*>(qp0 + j0) = pack8(q, a.even_odd8);
+      }
+    }
+  }
+  if constexpr (!COLMAX) break;
+  __syncthreads();  // the next row's abs-max goes through the same LDS words
+  }
+  if constexpr (COLMAX) {
+#pragma clang loop unroll(full)
+    for (int it = 0; it < ITERS; ++it) {
+      const int64_t j0 = (int64_t)(it * LANES + lane) * VEC;
+      if (j0 < a.L) {
+        uint32_t m[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) m[e] = (uint32_t)(int)rintf(colmax[it][e]);
+        *reinterpret_cast<uint2*>(a.oa_out + (int64_t)blockIdx.x * a.cols + j0) = pack8(m, 0);
       }
     }
   }
@@ -621,14 +681,66 @@ __global__ void finalize_scales_kernel(const QArgs a, int64_t n) {
   a.ws_inv[i] = inv;
 }
 
+// Partial maxima of |x| (bytes, [parts][n], written by an earlier launch next to the int8 values this one reads)
+// -> scale (output) and reciprocal scale (workspace), in place of the abs-max pass and finalize_scales_kernel.
+// A block takes 16 scales: thread t folds the 16 bytes of parts t, t + 256, ... (as eight pairs of 16-bit lanes,
+// two maxima per instruction), the threads meet through wave shuffles and LDS.  (64 scales per block, whose loads
+// use whole 64-byte sectors, leave 64 blocks for 4096 scales and measured slower: 11.6 against 8.1 us on average
+// over 1792 and 224 parts.)
+typedef unsigned short u16x2_max_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t x, uint32_t y) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_max_t, x),
+                                                                __builtin_bit_cast(u16x2_max_t, y)));
+}
+__global__ __launch_bounds__(256) void finalize_partials_kernel(const QArgs a, int64_t n) {
+  __shared__ uint32_t smax[4][8];
+  const int64_t c0 = (int64_t)blockIdx.x * 16;  // n is a multiple of 16 here
+  uint32_t m[8];  // m[2 i] = bytes 0 and 2 of word i in 16-bit lanes, m[2 i + 1] = bytes 1 and 3
+#pragma unroll
+  for (int i = 0; i < 8; ++i) m[i] = 0u;
+  for (int64_t p = threadIdx.x; p < a.oa_in_parts; p += 256) {
+    const uint4 w = *reinterpret_cast<const uint4*>(a.oa_in + p * n + c0);
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      m[2 * i] = pk_max_u16(m[2 * i], ww[i] & 0x00FF00FFu);
+      m[2 * i + 1] = pk_max_u16(m[2 * i + 1], (ww[i] >> 8) & 0x00FF00FFu);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m[i] = pk_max_u16(m[i], (uint32_t)__shfl_xor((int)m[i], off, 64));
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) smax[wave][i] = m[i];
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    // column c0 + t is byte t % 4 of word t / 4: lane (t % 4) / 2 of m[2 (t / 4) + t % 2]
+    const int t = threadIdx.x, i = 2 * (t >> 2) + (t & 1), hi = (t >> 1) & 1;
+    uint32_t v = pk_max_u16(pk_max_u16(smax[0][i], smax[1][i]), pk_max_u16(smax[2][i], smax[3][i]));
+    v = hi ? v >> 16 : v & 0xFFFFu;
+    float scale, inv;
+    scale_from_absmax((float)v, a, scale, inv);
+    store_scale(a, c0 + t, scale);
+    a.ws_inv[c0 + t] = inv;
+  }
+}
+
 constexpr int kTileR = 128, kTileC = 64, kTilePad = 132;
 
 // 128x64 tile: thread (rg = tid/8, cc = tid%8) owns rows 4*rg..+3, cols 8*cc..+7.
 // PAIR (SPEC 2, and SPEC 5 with value 1): 1 = the block also owns the tile `rows/2` further down (natural noise
 // layout), 2 = the tile `cols/2` further right (noise counters of the transposed tensor); the
 // two tiles' elements share threefry blocks.
-template <typename TIn, int SPEC, int PAIR>
+// ROWMAX (no PAIR; every tile interior): the block also finds, for each of its 128 rows, the largest |q| among its 64
+// columns, and stores them as bytes rows r0.. of row blockIdx.x of QArgs::oa_out ([column tiles][rows]).
+template <typename TIn, int SPEC, int PAIR, bool ROWMAX = false>
 __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
+  static_assert(!ROWMAX || PAIR == 0, "row maxima: one tile per block");
   const QArgs a = with_device_key(a_in);
   constexpr int NSET = PAIR ? 2 : 1;
   __shared__ uint32_t lds[NSET][kTileC * kTilePad / 4];
@@ -663,6 +775,7 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
     const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
     v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
   };
+  uint32_t rowmax = 0u;  // ROWMAX: byte j = largest |q| of row r0 + 4 * rg + j among the tile's 64 columns
   auto rows = [&](auto fast_tag) {
     constexpr bool FAST = decltype(fast_tag)::value;
     float ps_col[NSET][8];
@@ -718,6 +831,7 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
 #pragma unroll
         for (int s = 0; s < NSET; ++s) w[s][0] = w[s][1] = 0u;
         U2 wbits{0u, 0u};  // SPEC 5: the 32-bit word(s) two neighbouring elements draw their 16 bits from
+        float rm = 0.0f;   // ROWMAX: largest clipped |x / scale| of this row among this thread's 8 columns
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           if (FAST || e < nvalid) {
@@ -744,6 +858,10 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
             } else if constexpr (PAIR) {
               const uint32_t i = (uint32_t)((r0[0] + rg * 4 + j) * a.nsr + (c0[0] + cc * 8 + e) * a.nsc);
               pair_quant(x[0][e], inv[0][e], x[1][e], inv[1][e], i, a, qv[0], qv[1]);
+            } else if constexpr (ROWMAX) {
+              float tc;
+              qv[0] = spec_quant_mag<SPEC>(x[0][e], inv[0][e], 0, a, tc);
+              rm = fmaxf(rm, fabsf(tc));
             } else {
               const uint64_t ctr = (uint64_t)(b * a.nsb + rl * a.nsr + (cl + e) * a.nsc);
               qv[0] = spec_quant<SPEC>(x[0][e], inv[0][e], ctr, a);
@@ -754,6 +872,13 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
               packed[s][e] |= qv[s] << (8 * j);
             }
           }
+        }
+        if constexpr (ROWMAX) {
+          // every tile is interior here, so all lanes are in this branch: the 8 threads of a row (consecutive lanes)
+          // meet by shuffles; rint(max |t|) = max |q|
+#pragma unroll
+          for (int off = 1; off < 8; off <<= 1) rm = fmaxf(rm, __shfl_xor(rm, off, 64));
+          rowmax |= (uint32_t)(int)rintf(rm) << (8 * j);
         }
         if (!a.transpose_out) {
 #pragma unroll
@@ -772,6 +897,10 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(const QArgs a_in) {
   };
   if (interior) rows(std::true_type{});
   else rows(std::false_type{});
+  if constexpr (ROWMAX) {
+    if (cc == 0)
+      *reinterpret_cast<uint32_t*>(a.oa_out + ((int64_t)blockIdx.x * a.rows + r0[0] + rg * 4)) = rowmax;
+  }
   if (!a.transpose_out) return;  // uniform across the block
 
   // Transposed write: LDS holds each tile as [col][row bytes], row stride 132 B.
@@ -915,6 +1044,35 @@ int spec_of(const QArgs& a, int partitionable) {
   return 0;
 }
 
+// Blocks of the row kernel that also writes column maxima, each walking rows: seven per CU of the largest part, as
+// many as its registers (67 with 16 running maxima) let a CU hold (measured on 8192 rows of 4096 bf16 values, 21 us
+// without the maxima: 62 us with 256 blocks, 40 with 512, 30 with 1024).
+constexpr int64_t kColmaxBlocks = 7 * 256;
+
+// Whether the row kernels can leave column maxima of |q| behind for this plan: whole rows of 520 to 8192
+// aligned values as segments, one batch entry, integer values rounded to nearest.
+bool rows_colmax_ok(const aqtx_quant_plan* p) {
+  return p->reduce == AQTX_REDUCE_COLS && p->batch == 1 && p->group == 0 && !p->transpose_out &&
+         p->noise == AQTX_NOISE_NONE && (p->out_dtype == AQTX_I8 || p->out_dtype == AQTX_I4) &&
+         p->out_k_order == AQTX_K_NATURAL && p->cols % 8 == 0 && p->cols > 512 && p->cols <= 8192 && p->rows > 0;
+}
+
+template <typename TIn, int SPEC>
+int launch_rows_colmax(const QArgs& a, hipStream_t st) {
+  const int64_t L = a.L;
+  const int64_t blocks = a.nseg < kColmaxBlocks ? a.nseg : kColmaxBlocks;  // = aqtx_quantize_other_axis_parts: rows of oa_out
+#define AQTX_ROWS_CM(ITERS)                                                                                  \
+  {                                                                                                          \
+    quant_rows_kernel<TIn, 256, ITERS, SPEC, false, true><<<dim3((unsigned)blocks), 256, 0, st>>>(a);        \
+    AQTX_HIP_CHECK_LAUNCH("quant_rows_kernel, column maxima");                                               \
+    return 0;                                                                                                \
+  }
+  if (L <= 2048) AQTX_ROWS_CM(1)
+  if (L <= 4096) AQTX_ROWS_CM(2)
+  AQTX_ROWS_CM(4)
+#undef AQTX_ROWS_CM
+}
+
 template <typename TIn, int SPEC, bool PAIR>
 int launch_rows_spec(const QArgs& a, hipStream_t st) {
   const int64_t L = a.L;
@@ -950,6 +1108,10 @@ int launch_rows(const QArgs& a, int partitionable, hipStream_t st) {
     return 0;
   }
   const int spec = spec_of(a, partitionable);
+  if (a.oa_out != nullptr) {  // (the caller has checked rows_colmax_ok: noise none, so spec is 1 or 0)
+    if (spec == 1) return launch_rows_colmax<TIn, 1>(a, st);
+    return launch_rows_colmax<TIn, 0>(a, st);
+  }
   if (spec == 1) return launch_rows_spec<TIn, 1, false>(a, st);
   if (spec == 3) return launch_rows_spec<TIn, 3, false>(a, st);
   if (spec == 5) return launch_rows_spec<TIn, 5, false>(a, st);
@@ -964,8 +1126,20 @@ int launch_rows(const QArgs& a, int partitionable, hipStream_t st) {
   return launch_rows_spec<TIn, 0, false>(a, st);
 }
 
+// Whether the tile kernel can leave row maxima of |q| behind for this plan: one scale per column over whole
+// columns, every 128 x 64 tile inside the tensor, one batch entry, integer values rounded to nearest.
+bool tiles_rowmax_ok(const aqtx_quant_plan* p) {
+  return p->reduce == AQTX_REDUCE_ROWS && p->batch == 1 && p->group == 0 && p->noise == AQTX_NOISE_NONE &&
+         (p->out_dtype == AQTX_I8 || p->out_dtype == AQTX_I4) && p->rows > 0 && p->cols > 0 &&
+         p->rows % kTileR == 0 && p->cols % kTileC == 0;
+}
+
 template <typename TIn>
 int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales, hipStream_t st) {
+  if (a.oa_in != nullptr) {
+    finalize_partials_kernel<<<dim3((unsigned)(nscales / 16)), 256, 0, st>>>(a, nscales);
+    AQTX_HIP_CHECK_LAUNCH("finalize_partials_kernel");
+  } else {
   if (!a.scale_given) {
     if (!a.ws_zeroed) {
       fill_u32_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a.ws_absmax, nscales, 0u);
@@ -999,13 +1173,17 @@ int launch_tiles(const QArgs& a, int reduce, int partitionable, int64_t nscales,
   }
   finalize_scales_kernel<<<dim3((unsigned)((nscales + 255) / 256)), 256, 0, st>>>(a, nscales);
   AQTX_HIP_CHECK_LAUNCH("finalize_scales_kernel");
+  }
   const int spec = spec_of(a, partitionable);
   auto grid_for = [&](int pair) {
     const int64_t rows = pair == 1 ? a.rows / 2 : a.rows, cols = pair == 2 ? a.cols / 2 : a.cols;
     return dim3((unsigned)((cols + kTileC - 1) / kTileC), (unsigned)((rows + kTileR - 1) / kTileR),
                 (unsigned)a.batch);
   };
-  if (spec == 1) {
+  if (a.oa_out != nullptr) {  // (the caller has checked tiles_rowmax_ok: noise none, so spec is 1 or 0)
+    if (spec == 1) quant_tile_kernel<TIn, 1, 0, true><<<grid_for(0), 256, 0, st>>>(a);
+    else quant_tile_kernel<TIn, 0, 0, true><<<grid_for(0), 256, 0, st>>>(a);
+  } else if (spec == 1) {
     quant_tile_kernel<TIn, 1, 0><<<grid_for(0), 256, 0, st>>>(a);
   } else if (spec == 3) {
     quant_tile_kernel<TIn, 3, 0><<<grid_for(0), 256, 0, st>>>(a);
@@ -1068,6 +1246,16 @@ static bool long_rows_as_batches(const aqtx_quant_plan* p, aqtx_quant_plan* q) {
   return true;
 }
 
+static bool long_rows_as_batches(const aqtx_quant_plan* p, aqtx_quant_plan* q);
+
+extern "C" int64_t aqtx_quantize_other_axis_parts(const aqtx_quant_plan* p) {
+  aqtx_quant_plan alt;
+  if (p == nullptr || p->scale_given || long_rows_as_batches(p, &alt)) return 0;
+  if (rows_colmax_ok(p)) return p->rows < kColmaxBlocks ? p->rows : kColmaxBlocks;
+  if (tiles_rowmax_ok(p)) return p->cols / kTileC;
+  return 0;
+}
+
 extern "C" size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* p) {
   aqtx_quant_plan alt;
   if (p != nullptr && long_rows_as_batches(p, &alt)) return aqtx_quantize_workspace_bytes(&alt);
@@ -1114,6 +1302,21 @@ extern "C" int aqtx_quantize(const aqtx_quant_plan* p, const void* x, const floa
   a.cbf = p->compute_dtype == AQTX_BF16; a.sbf = p->scale_dtype == AQTX_BF16;
   a.scale_given = p->scale_given;
   a.ws_zeroed = p->workspace_zeroed;
+  if (p->other_axis_absmax != nullptr) {
+    AQTX_REQUIRE(aqtx_quantize_other_axis_parts(p) > 0,
+                 "aqtx_quantize: this plan cannot write other_axis_absmax (aqtx_quantize_other_axis_parts is 0)");
+    AQTX_REQUIRE(((uintptr_t)p->other_axis_absmax % 8) == 0, "aqtx_quantize: other_axis_absmax must be 8-byte aligned");
+    a.oa_out = reinterpret_cast<uint8_t*>(p->other_axis_absmax);
+  }
+  if (p->absmax_partials != nullptr) {
+    AQTX_REQUIRE(p->in_dtype == AQTX_I8 && p->reduce == AQTX_REDUCE_ROWS && p->group == 0 && p->batch == 1 &&
+                     !p->scale_given && p->prescale == AQTX_PRESCALE_NONE && p->absmax_parts > 0 && p->cols % 16 == 0 &&
+                     ((uintptr_t)p->absmax_partials % 16) == 0,
+                 "aqtx_quantize: absmax_partials (16-byte aligned) go with int8 input, AQTX_REDUCE_ROWS over whole columns (a "
+                 "multiple of 16 of them), one batch entry, no prescale and no given scale");
+    a.oa_in = reinterpret_cast<const uint8_t*>(p->absmax_partials);
+    a.oa_in_parts = p->absmax_parts;
+  }
   AQTX_REQUIRE(p->out_k_order == AQTX_K_NATURAL || p->out_k_order == AQTX_K_EVEN_ODD8,
                "aqtx_quantize: unknown out_k_order %d", p->out_k_order);
   if (p->out_k_order == AQTX_K_EVEN_ODD8) {

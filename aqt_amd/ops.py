@@ -155,6 +155,8 @@ def quantize(
     want_typed_scale: bool = False,
     key_device: Optional[torch.Tensor] = None,
     k_order: int = 0,
+    want_other_axis_absmax: bool = False,
+    absmax_partials: Optional[torch.Tensor] = None,
 ):
   """Calibrate (abs-max) and quantize a contiguous [batch, rows, cols] tensor.
 
@@ -169,6 +171,10 @@ def quantize(
   With want_typed_scale a third element: the computed scales once more as a bf16 tensor of
   the same shape, written by the same kernels (None unless the scale dtype is bf16 and the
   scale is computed here).
+  want_other_axis_absmax: where the plan allows it, the kernels also leave partial maxima of |q| along the axis
+  that carries the scales (uint8 [parts, cols] for REDUCE_COLS, [parts, rows] for REDUCE_ROWS) in
+  `q.other_axis_absmax`: what a later quantization of q over that axis takes as `absmax_partials` instead of
+  reading q for its abs-max (the backward pass re-quantizes the forward residuals that way).
   """
   _require_gpu(x, prescale, scale)
   assert x.dim() == 3 and x.is_contiguous(), 'x must be a contiguous [batch, rows, cols] tensor'
@@ -223,6 +229,17 @@ def quantize(
   if prescale is not None:
     assert prescale.dtype == torch.float32 and prescale.is_contiguous()
   lib = L.lib()
+  other = None
+  if want_other_axis_absmax:
+    parts = int(lib.aqtx_quantize_other_axis_parts(ctypes.byref(plan)))
+    if parts > 0:
+      other = torch.empty((parts, c if reduce == L.REDUCE_COLS else r), dtype=torch.uint8, device=x.device)
+      plan.other_axis_absmax = other.data_ptr()
+  if absmax_partials is not None:
+    _require_gpu(absmax_partials)
+    assert (absmax_partials.dtype == torch.uint8 and absmax_partials.is_contiguous() and absmax_partials.dim() == 2
+            and absmax_partials.shape[1] == c and not plan.scale_given), (absmax_partials.shape, x.shape)
+    plan.absmax_partials, plan.absmax_parts = absmax_partials.data_ptr(), absmax_partials.shape[0]
   ws_bytes = lib.aqtx_quantize_workspace_bytes(ctypes.byref(plan))
   ws = _quantize_workspace(ws_bytes, x.device) if ws_bytes else None
   plan.workspace_zeroed = int(ws is not None)
@@ -232,6 +249,8 @@ def quantize(
   except Exception:
     _QUANT_WS.clear()  # a failed launch sequence may have left abs-max words behind
     raise
+  if other is not None:
+    q.other_axis_absmax = other
   return (q, scale, typed) if want_typed_scale else (q, scale)
 
 

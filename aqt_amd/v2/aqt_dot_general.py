@@ -9,6 +9,7 @@ torch.autograd.Function in place of jax.custom_vjp.
 from __future__ import annotations
 
 import abc
+import contextvars
 import dataclasses
 import enum
 import functools
@@ -635,6 +636,13 @@ def _canonical_pairs(lhs, rhs, dimension_numbers):
 
 _NotFused = lowering.NotFused
 
+# (lhs, rhs): whether the forward quantizers of this call should leave, next to the values they write, the partial
+# maxima with which the backward pass calibrates those values over the other axis (DotGeneralRaw._quant_side); set
+# by the differentiable entry point for the operands whose residual a backward contraction re-quantizes.
+_RESIDUAL_ABSMAX: 'contextvars.ContextVar' = contextvars.ContextVar('aqt_residual_absmax', default=(False, False))
+# False (AQTX_RESIDUAL_ABSMAX=0 in the environment): the backward pass reads the residuals for their abs-max; same results
+RESIDUAL_ABSMAX = os.environ.get('AQTX_RESIDUAL_ABSMAX', '1') != '0'
+
 
 def _ragged_sizes(dot_general_hook):
   """The group sizes of a ragged-contraction hook (aqt_ragged_dot.RaggedDot), else None."""
@@ -843,12 +851,15 @@ class DotGeneralRaw:
       return served
 
     # ---- lhs ---------------------------------------------------------------------
+    want_l, want_r = _RESIDUAL_ABSMAX.get()
     lq, ls, lsdt, lhs_qt_out, lhs_grad = self._quant_side(
-        'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t, _bwd_memo, _calibrated)
+        'lhs', lhs, lhs_dtype, False, dq.lhs, lhs_qt, lba, lra, lca, prescale_t, _bwd_memo, _calibrated,
+        want_other_axis_absmax=want_l)
     # ---- rhs ---------------------------------------------------------------------
     rq, rs, rsdt, rhs_qt_out, rhs_grad = self._quant_side(
         'rhs', rhs_arr, rhs_dtype, rhs_is_q, dq.rhs, rhs_qt, rba, rra, rca, None, _bwd_memo, _calibrated,
-        layout_later=rhs_qt is not None and rhs_qt.qvalue is not None and rhs_qt.qvalue.dtype == torch.int8)
+        layout_later=rhs_qt is not None and rhs_qt.qvalue is not None and rhs_qt.qvalue.dtype == torch.int8,
+        want_other_axis_absmax=want_r)
     rv_later = None  # a frozen int8 rhs that is not laid out for the kernels as the caller holds it
     if rq is None:
       rv_later = lowering.view_operand(rhs_qt.qvalue, rba, rra, rca)
@@ -1261,12 +1272,16 @@ class DotGeneralRaw:
     return out, res
 
   def _quant_side(self, name, x, dtype, x_is_q, quantizer, given_qt, ba, ra, ca, prescale_t,
-                  bwd_memo=None, calibrated=None, layout_later=False, held_float=False):
+                  bwd_memo=None, calibrated=None, layout_later=False, held_float=False,
+                  want_other_axis_absmax=False):
     """Quantizes one side; returns (q [B,R,K], scale f32, scale dtype, QTensor, quant_grad).
     `bwd_memo`: the backward pass's table of per-tensor scales; `calibrated`: where a calibration
     that runs step by step leaves its result for a later fall-back of the same call; `held_float`:
     numerics that keep their integers in the float dtype are taken too (q and the QTensor come back
-    as int8, the caller casts)."""
+    as int8, the caller casts); `want_other_axis_absmax`: the backward pass is going to quantize the
+    values written here once more over the other axis (_maybe_use_fwd_quant), so the kernels leave
+    the partial maxima that calibration needs with the quantized tensor (ops.quantize), and the
+    call that finds them there (`x_is_q`) skips its abs-max pass."""
     def numerics_spec():
       if isinstance(quantizer.numerics, no_numerics.NoNumerics):
         return None
@@ -1349,9 +1364,19 @@ class DotGeneralRaw:
         flat = memo_hit[0].reshape(1).expand(v.B * v.R)
         scale_in = flat.contiguous().reshape(v.B, v.R, 1) if v.k_last else flat.contiguous().reshape(v.B, 1, v.R)
         scale_dtype = memo_hit[2]
+    partials = None
+    if (x_is_q and scale_in is None and prescale is None and arr.dim() == 2 and arr.dtype == torch.int8
+        and not v.k_last and not v.copied and quantizer.kernel_spec(held_float) is not None):
+      left = getattr(arr, 'other_axis_absmax', None)  # (partial maxima, version of the tensor they describe)
+      if left is not None and left[1] == arr._version and left[0].shape[1] == v.R and v.R % 16 == 0:
+        partials = left[0]
     q, s32, sdt = quantizer.quant_view(v, dtype, calibration_axes=ca, prescale=prescale, scale=scale_in,
-                                       scale_dtype=scale_dtype, held_float=held_float)
+                                       scale_dtype=scale_dtype, held_float=held_float,
+                                       want_other_axis_absmax=want_other_axis_absmax and arr.dim() == 2,
+                                       absmax_partials=partials)
     qv = lowering.logical_from_brk(aqt_quantizer._typed(q, spec['out_dtype']), v)
+    if getattr(q, 'other_axis_absmax', None) is not None:
+      qv.other_axis_absmax = (q.other_axis_absmax, qv._version)
     if memo_hit is not None:
       s32, scale_list = memo_hit[0], memo_hit[1]
     elif given_qt is not None:
@@ -1693,8 +1718,16 @@ class _DgCoreFn(torch.autograd.Function):
 
   @staticmethod
   def forward(ctx, lhs, rhs, lhs_qt, rhs_qt, dimension_numbers, cfg):
-    (out, (lq, rq)), (res, cfg) = dg_core_vjp_fwd(lhs.detach(), rhs.detach(), lhs_qt, rhs_qt,
-                                                  dimension_numbers, cfg)
+    # drhs re-quantizes the lhs residual, dlhs the rhs residual, when they reuse the forward quantization
+    need_l, need_r = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+    token = _RESIDUAL_ABSMAX.set(
+        (bool(RESIDUAL_ABSMAX and need_r and cfg.drhs.rhs.use_fwd_quant and cfg.drhs.local_aqt is None),
+         bool(RESIDUAL_ABSMAX and need_l and cfg.dlhs.rhs.use_fwd_quant and cfg.dlhs.local_aqt is None)))
+    try:
+      (out, (lq, rq)), (res, cfg) = dg_core_vjp_fwd(lhs.detach(), rhs.detach(), lhs_qt, rhs_qt,
+                                                    dimension_numbers, cfg)
+    finally:
+      _RESIDUAL_ABSMAX.reset(token)
     ctx.aqt_res = (res, cfg)
     ctx.dimension_numbers = dimension_numbers
     ctx.set_materialize_grads(False)

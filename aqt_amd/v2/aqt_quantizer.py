@@ -97,7 +97,8 @@ class Quantizer:
     return spec
 
   def quant_view(self, v: lowering.OperandView, dtype, *, calibration_axes, prescale=None,
-                 scale: Optional[torch.Tensor] = None, scale_dtype=None, held_float: bool = False):
+                 scale: Optional[torch.Tensor] = None, scale_dtype=None, held_float: bool = False,
+                 want_other_axis_absmax: bool = False, absmax_partials: Optional[torch.Tensor] = None):
     """Calibrate + quantize an operand view in one kernel sequence.
 
     With `scale` (float32, one value per [B, R] entry, holding values of `scale_dtype`) the
@@ -124,7 +125,9 @@ class Quantizer:
       sdt = self._calibrator.dtype if self._calibrator.dtype is not None else dtype
     q, s = lowering.quantize_view(v, spec=spec, compute_dtype=dtype, scale_dtype=sdt,
                                   key=None if self.context is None else self.context.key,
-                                  per_tensor=per_tensor, prescale=prescale, scale=scale)
+                                  per_tensor=per_tensor, prescale=prescale, scale=scale,
+                                  want_other_axis_absmax=want_other_axis_absmax and not per_tensor,
+                                  absmax_partials=None if per_tensor else absmax_partials)
     return q, s, sdt
 
   # ---- reference-shaped API -------------------------------------------------------

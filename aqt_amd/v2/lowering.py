@@ -145,7 +145,8 @@ _OUT_TORCH = {L.I8: torch.int8, L.I4: torch.int8, L.E4M3: torch.float8_e4m3fn, L
 
 def quantize_view(v: OperandView, *, spec: dict, compute_dtype, scale_dtype, key=None,
                   per_tensor: bool = False, prescale: Optional[torch.Tensor] = None,
-                  scale: Optional[torch.Tensor] = None):
+                  scale: Optional[torch.Tensor] = None, want_other_axis_absmax: bool = False,
+                  absmax_partials: Optional[torch.Tensor] = None):
   """Runs the quantize kernel on a view.
 
   Returns (q [B, R, K] int8/uint8, scale float32 [B, R] (or [1] per tensor)).
@@ -173,7 +174,8 @@ def quantize_view(v: OperandView, *, spec: dict, compute_dtype, scale_dtype, key
   if reduce == L.REDUCE_COLS and per_tensor is False and transpose:
     raise AssertionError('unreachable')
   q, s, typed = ops.quantize(v.mem, reduce=reduce, transpose_out=transpose, scale=scale,
-                             want_typed_scale=True, **kwargs)
+                             want_typed_scale=True, want_other_axis_absmax=want_other_axis_absmax,
+                             absmax_partials=absmax_partials, **kwargs)
   shape = (-1,) if per_tensor else (v.B, v.R)
   s = s.reshape(shape)
   # the same scales as elements of the scale dtype, written by the kernel (saves a cast launch)

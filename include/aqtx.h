@@ -101,6 +101,19 @@ typedef struct aqtx_quant_plan {
                             array under XLA, or one updated on the device between HIP graph replays) */
   int32_t out_k_order;   /* AQTX_K_*: byte order of q along cols; EVEN_ODD8 needs AQTX_REDUCE_COLS, an
                             int8 / int4 out_dtype, no transpose_out, cols and group multiples of 8 */
+  /* The backward pass quantizes the int8 values a forward quantizer wrote once more, with scales along the other
+     axis (_maybe_use_fwd_quant, aqt/jax/v2/aqt_dot_general.py:675-729), and would read them twice for it (abs-max,
+     then quantize).  A forward plan can leave what that abs-max needs behind instead:
+     other_axis_absmax: optional out, uint8 [parts][len], parts = aqtx_quantize_other_axis_parts(plan) (0: this plan
+     cannot write them), len = the length of the axis this plan reduces over (cols for AQTX_REDUCE_COLS, rows for
+     AQTX_REDUCE_ROWS): entry [p][i] = the largest |q| among part p of the values that share position i.
+     absmax_partials / absmax_parts: optional in, such an array for THIS plan's input (in_dtype AQTX_I8,
+     AQTX_REDUCE_ROWS over whole columns, cols a multiple of 16, batch 1, no prescale, no given scale; [parts][cols],
+     16-byte aligned): the abs-max pass
+     is skipped and the scales come from the maxima over the parts.  Same results either way. */
+  void* other_axis_absmax;
+  const void* absmax_partials;
+  int64_t absmax_parts;
 } aqtx_quant_plan;
 
 /*
@@ -123,6 +136,9 @@ int aqtx_quantize(const aqtx_quant_plan* plan, const void* x, const float* presc
 
 /* Scratch bytes aqtx_quantize needs for `plan` (0 for single-pass plans). */
 size_t aqtx_quantize_workspace_bytes(const aqtx_quant_plan* plan);
+
+/* Rows of the plan->other_axis_absmax array this plan would write (0: it cannot; leave the pointer NULL). */
+int64_t aqtx_quantize_other_axis_parts(const aqtx_quant_plan* plan);
 
 /*
  * aqtx_dequantize: out = cast(q) * scale for a quantized tensor with one scale.

@@ -457,3 +457,33 @@ def test_scale_cast_rejects_bad_plans():
   plan.factor_axis[0], plan.factor_dtype[0] = 5, L.F32
   rc = L.lib().aqtx_scale_cast(ctypes.byref(plan), None, None, None, None, None)
   assert rc != 0 and b'unknown factor_axis' in L.lib().aqtx_last_error()
+
+
+def test_quantize_partial_maxima_plans_are_validated():
+  """other_axis_absmax on a plan that cannot write it, absmax_partials on a plan that cannot take them."""
+  lib = L.lib()
+  p = L.QuantPlan()
+  p.in_dtype = p.compute_dtype = p.scale_dtype = L.BF16
+  p.out_dtype = L.I8
+  p.batch, p.rows, p.cols = 1, 64, 4096
+  p.reduce = L.REDUCE_COLS
+  p.quant_bound, p.clip_bound = 127.5, 127.0
+  assert lib.aqtx_quantize_other_axis_parts(ctypes.byref(p)) == 64
+  p.rows = 5000
+  assert lib.aqtx_quantize_other_axis_parts(ctypes.byref(p)) == 1792
+  p.noise = L.NOISE_JAX_UNIFORM
+  p.noise_total, p.noise_stride_row, p.noise_stride_col = 5000 * 4096, 4096, 1
+  assert lib.aqtx_quantize_other_axis_parts(ctypes.byref(p)) == 0
+  p.other_axis_absmax = 4096
+  assert 'other_axis_absmax' in _err(lib.aqtx_quantize(ctypes.byref(p), FAKE, None, FAKE, FAKE, None, 0, None))
+  p.other_axis_absmax = None
+  p.noise = L.NOISE_NONE
+  p.reduce, p.transpose_out, p.rows, p.cols = L.REDUCE_ROWS, 1, 4096, 14336
+  assert lib.aqtx_quantize_other_axis_parts(ctypes.byref(p)) == 14336 // 64
+  p.cols = 14336 + 8
+  assert lib.aqtx_quantize_other_axis_parts(ctypes.byref(p)) == 0
+  p.cols = 14336
+  p.absmax_partials, p.absmax_parts = 4096, 16  # a bf16 input: the maxima describe int8 values
+  ws = lib.aqtx_quantize_workspace_bytes(ctypes.byref(p))
+  assert 'absmax_partials' in _err(lib.aqtx_quantize(ctypes.byref(p), FAKE, None, FAKE, FAKE, FAKE, ws, None))
+
