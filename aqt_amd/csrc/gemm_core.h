@@ -866,6 +866,7 @@ inline int gemm_epilogue_id(const aqtx_gemm_plan* p) {
 
 int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8);
 // gemm_mid.hip: 0 = the plan stays with the 256 x 256 kernel, 1 = the 128 x 128 kernel, S > 1 = with K in S slices
+int compute_units();  // CUs of the current device (0 if it cannot be asked)
 int gemm_mid_k_slices(const aqtx_gemm_plan* p);
 int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, const float* row_scale,
                        const float* col_scale, void* c, int32_t* acc_out, int slices, hipStream_t st);

@@ -48,9 +48,7 @@ int validate_gemm_plan(const aqtx_gemm_plan* p, const char* who, bool fp8) {
 
 }  // namespace aqtx
 
-using namespace aqtx;
-
-namespace {
+namespace aqtx {
 // CUs of the current device, asked once per device.
 int compute_units() {
   static std::atomic<int> cached[64];
@@ -63,7 +61,10 @@ int compute_units() {
   }
   return n;
 }
-}  // namespace
+}  // namespace aqtx
+
+using namespace aqtx;
+
 
 extern "C" int aqtx_gemm_i8_k_slices(const aqtx_gemm_plan* p) {
   if (p == nullptr || p->k_split < 0 || p->k_split > 64 || p->batch <= 0 || p->m <= 0 || p->n <= 0) return 1;

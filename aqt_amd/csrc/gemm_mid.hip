@@ -18,7 +18,25 @@ namespace {
 
 constexpr int TM = 128, TN = 128;
 constexpr int kRow = BK + 16;
-constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile;  // 36 KiB
+
+// Tile of a workgroup and how its waves share it: WM x WN waves, each (TM / WM) x (TN / WN) of C in 32 x 32
+// matrix-instruction tiles.  A wave fetches TM / waves rows of A and TN / waves rows of B per stage.
+template <int TM_, int TN_, int WM_, int WN_, int OCC_ = 4, bool RING_ = false, int GROUP_ = 1>
+struct MidShape {
+  static constexpr int kOcc = OCC_;      // waves per SIMD the registers are budgeted for
+  static constexpr bool kRing = RING_;   // three LDS buffers and three stages in flight in registers (see the kernel)
+  static constexpr int kGroup = GROUP_;  // ring schedule: k steps whose fragments are read together
+  static constexpr int kTM = TM_, kTN = TN_, kWM = WM_, kWN = WN_, kWaves = WM_ * WN_, kThreads = 64 * kWaves;
+  static constexpr int kIM = TM_ / WM_ / 32, kIN = TN_ / WN_ / 32;  // 32 x 32 tiles of a wave
+  static constexpr int kRA = TM_ / kWaves, kRB = TN_ / kWaves;        // rows a wave fetches per stage
+  static constexpr int kATile = TM_ * kRow, kBTile = TN_ * kRow, kStage = kATile + kBTile;
+  static_assert(kIM >= 1 && kIN >= 1 && kRA % 16 == 0 && kRB % 16 == 0, "whole 32 x 32 tiles, whole 16-row load blocks");
+};
+using Mid128 = MidShape<128, 128, 4, 2>;  // 8 waves of 32 x 64, 36 KiB a stage, two workgroups a CU
+// One workgroup a CU (or several small ones), for launches of at most one workgroup per CU: the ring schedule.
+using Ring128 = MidShape<128, 128, 4, 2, 2, true, 2>;
+using Ring64x128 = MidShape<64, 128, 2, 2, 2, true, 2>;
+using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2>;
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
 // int4 values two per byte (see gemm_kernel's BPACK), or, with MmaBf16W8, int8 values that become bf16 (A then
@@ -28,9 +46,14 @@ constexpr int kATile = TM * kRow, kBTile = TN * kRow, kStage = kATile + kBTile; 
 // SLAB: this launch writes raw partial sums of a K slice to its slab (EPI is 3 then; integer sums only).
 // CONV: A is a convolution input read in place (GemmArgs::conv): the window gather that would otherwise be
 // materialised (features % 128 == 0, so a 128-byte stage lies inside one tap).
-template <class MMA, int EPI, bool COL_FIRST, bool PACKED, bool SLAB, bool CONV = false>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+template <class MMA, int EPI, bool COL_FIRST, bool PACKED, bool SLAB, bool CONV = false, class S = Mid128>
+__global__ __launch_bounds__(S::kThreads) __attribute__((amdgpu_waves_per_eu(S::kOcc, S::kOcc)))
 void gemm_mid_kernel(const GemmArgs g_in) {
+  constexpr int TM = S::kTM, TN = S::kTN, kATile = S::kATile, kStage = S::kStage;
+  constexpr int IM = S::kIM, IN = S::kIN, RA = S::kRA, RB = S::kRB;
+  constexpr bool RING = S::kRing;
+  constexpr int NSETS = RING ? 3 : 1, NBUF = RING ? 3 : 2;
+  static_assert(!CONV || (TM == 128 && S::kWaves == 8), "the window gather is written for two loads of A per wave");
   static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
   static_assert(!CONV || (MMA::kIntAcc && !PACKED && !SLAB), "the convolution reads int8 bytes, whole K");
   static_assert(MMA::kIntAcc || (!SLAB && PACKED == MMA::kWidenB && EPI != 3), "float sums: whole K; fp8 bytes as they are");
@@ -41,10 +64,10 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   using Frag = typename MMA::Frag;
   constexpr int kChunks = MMA::kChunks;  // 16-byte chunks a lane holds of one MFMA's k
   GemmArgs g = g_in;
-  __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[2 * kStage];
+  __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[NBUF * kStage];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;  // 32 rows, 64 columns
+  const int wm = wave / S::kWN, wn = wave % S::kWN;
   const int lr = lane & 31, lh = lane >> 5;
   int tm, tn;
   tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
@@ -75,27 +98,37 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   // B packed: a wave load covers 16 rows x 64 B, one per wave; a lane's 16 bytes become the 32 bytes at
   // 32 * (lane & 3) of its row.  The row and chunk of a load are in its vector offset, which the buffer's
   // range check covers; the scalar offset (the stage's k) is not range checked, the mask on K covers it.
-  constexpr int NLA = WIDEN_A ? 1 : 2, NLB = PACKED ? 1 : 2, NL = NLA + NLB;
+  constexpr int NLA = WIDEN_A ? RA / 16 : RA / 8, NLB = PACKED ? RB / 16 : RB / 8, NL = NLA + NLB;
   constexpr int kOutside = 0x7FFFFFF0;
-  v4i stg[NL];
-  const int ld_a = WIDEN_A ? (wave * 16 + (lane >> 2)) * (int)g.lda + (lane & 3) * 16
-                           : (wave * 16 + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
+  v4i stg[NSETS][NL];
+  // A: load j of a wave covers 8 rows x 128 B (16 rows x 64 B of memory where A is widened)
+  const int ld_a = WIDEN_A ? (wave * RA + (lane >> 2)) * (int)g.lda + (lane & 3) * 16
+                           : (wave * RA + (lane >> 3)) * (int)g.lda + (lane & 7) * 16;
+  const int ld_a_next = (WIDEN_A ? 16 : 8) * (int)g.lda;
   // B in fragment order: a wave load is one KiB = 64 bytes of 16 rows (lane -> row lane & 15, bytes 16 (lane >> 4));
-  // unpacked, the wave's two loads are the two KiB of a stage (the second 64 bytes further in LDS), and the
+  // unpacked, two loads are the two KiB of a 16-row block's stage (the second 64 bytes further in LDS), and the
   // scalar offset advances one KiB per 64 row bytes
-  const int ld_b = g.b_frag ? wave * g.b_steps * 1024 + lane * 16
-                 : PACKED ? (wave * 16 + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
-                          : (wave * 16 + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
-  const int ld_b_next = g.b_frag ? 1024 : 8 * (int)g.ldb;  // the wave's second load (unpacked)
+  const int ld_b = g.b_frag ? wave * (RB / 16) * g.b_steps * 1024 + lane * 16
+                 : PACKED ? (wave * RB + (lane >> 2)) * (int)g.ldb + (lane & 3) * 16
+                          : (wave * RB + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
   const int kpos_a = WIDEN_A ? (lane & 3) * 32 : (lane & 7) * 16;
   const int kpos_b = g.b_frag ? (lane >> 4) * (PACKED ? 32 : 16) : PACKED ? (lane & 3) * 32 : (lane & 7) * 16;
-  const int kpos_b_next = g.b_frag ? 64 : 0;
-  const int st_a = WIDEN_A ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
-                           : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16;
-  const int st_b = kATile + (g.b_frag ? (wave * 16 + (lane & 15)) * kRow + (lane >> 4) * (PACKED ? 32 : 16)
-                             : PACKED ? (wave * 16 + (lane >> 2)) * kRow + (lane & 3) * 32
-                                      : (wave * 16 + (lane >> 3)) * kRow + (lane & 7) * 16);
-  const int st_b_next = g.b_frag ? 64 : 8 * kRow;
+  const int st_a = WIDEN_A ? (wave * RA + (lane >> 2)) * kRow + (lane & 3) * 32
+                           : (wave * RA + (lane >> 3)) * kRow + (lane & 7) * 16;
+  const int st_a_next = (WIDEN_A ? 16 : 8) * kRow;
+  const int st_b = kATile + (g.b_frag ? (wave * RB + (lane & 15)) * kRow + (lane >> 4) * (PACKED ? 32 : 16)
+                             : PACKED ? (wave * RB + (lane >> 2)) * kRow + (lane & 3) * 32
+                                      : (wave * RB + (lane >> 3)) * kRow + (lane & 7) * 16);
+  // load jj of B past the wave's first: memory offset, LDS offset, position along k (jj is a constant where used)
+  auto b_mem_next = [&](const int jj) -> int {
+    if constexpr (PACKED) return g.b_frag ? jj * g.b_steps * 1024 : jj * 16 * (int)g.ldb;
+    else return g.b_frag ? (jj >> 1) * g.b_steps * 1024 + (jj & 1) * 1024 : jj * 8 * (int)g.ldb;
+  };
+  auto b_lds_next = [&](const int jj) -> int {
+    if constexpr (PACKED) return jj * 16 * kRow;
+    else return g.b_frag ? (jj >> 1) * 16 * kRow + (jj & 1) * 64 : jj * 8 * kRow;
+  };
+  auto b_kpos_next = [&](const int jj) -> int { return (!PACKED && g.b_frag) ? (jj & 1) * 64 : 0; };
   const int ksh_b = g.b_frag ? 4 : 0;  // scalar offset of B = row bytes << ksh_b
   // CONV: position of this lane's two rows (first corner of their windows, in input coordinates) and the tap
   // the next request belongs to, advanced one stage per request (requests come in stage order)
@@ -123,54 +156,83 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       if (++ct2 == g.conv.ker[2]) { ct2 = 0; if (++ct1 == g.conv.ker[1]) { ct1 = 0; ++ct0; } }
     }
   };
-  auto load_one = [&](const int j, int k0) {
+  auto load_one = [&](const int set, const int j, int k0) {
     if constexpr (CONV) {
       if (j < NLA) {
         const int d0 = ct0 * g.conv.dil[0], d1 = ct1 * g.conv.dil[1], d2 = ct2 * g.conv.dil[2];
         const bool in = (unsigned)(ci0[j] + d0) < (unsigned)g.conv.in[0] && (unsigned)(ci1[j] + d1) < (unsigned)g.conv.in[1] &&
                         (unsigned)(ci2[j] + d2) < (unsigned)g.conv.in[2] && ct0 < g.conv.ker[0];
         const int tap = ((d0 * g.conv.in[1] + d1) * g.conv.in[2] + d2) * g.conv.c + cch;
-        stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, in ? cpix[j] + tap + kpos_a : kOutside, 0, 0);
+        stg[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, in ? cpix[j] + tap + kpos_a : kOutside, 0, 0);
         return;
       }
     }
     if (j < NLA) {
-      const int vo = k0 + kpos_a < (int)g.k ? ld_a + j * 8 * (int)g.lda : kOutside;
-      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, WIDEN_A ? k0 / 2 : k0, 0);
+      const int vo = k0 + kpos_a < (int)g.k ? ld_a + j * ld_a_next : kOutside;
+      stg[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo, WIDEN_A ? k0 / 2 : k0, 0);
     } else if constexpr (PACKED) {
-      const int vo = k0 + kpos_b < (int)g.k ? ld_b : kOutside;
-      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, (k0 / 2) << ksh_b, 0);
+      const int vo = k0 + kpos_b < (int)g.k ? ld_b + b_mem_next(j - NLA) : kOutside;
+      stg[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, (k0 / 2) << ksh_b, 0);
     } else {
-      const int vo = k0 + kpos_b + (j - NLA) * kpos_b_next < (int)g.k ? ld_b + (j - NLA) * ld_b_next : kOutside;
-      stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 << ksh_b, 0);
+      const int vo = k0 + kpos_b + b_kpos_next(j - NLA) < (int)g.k ? ld_b + b_mem_next(j - NLA) : kOutside;
+      stg[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 << ksh_b, 0);
     }
   };
-  auto store_stage = [&](const int stage_base) {
+  auto store_piece = [&](const int set, const int stage_base, const int jj) {
     uint8_t* st = stage_mem + stage_base;
-    if constexpr (WIDEN_A) {
-      v4i lo, hi;
-      MMA::widen_a(stg[0], lo, hi);
-      *reinterpret_cast<v4i*>(st + st_a) = lo;
-      *reinterpret_cast<v4i*>(st + st_a + 16) = hi;
+    if (jj < NLA) {
+      const int j = jj;
+      if constexpr (WIDEN_A) {
+        v4i lo, hi;
+        MMA::widen_a(stg[set][j], lo, hi);
+        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = lo;
+        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next + 16) = hi;
+      } else {
+        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = stg[set][j];
+      }
     } else {
-#pragma unroll
-      for (int j = 0; j < NLA; ++j) *reinterpret_cast<v4i*>(st + st_a + j * 8 * kRow) = stg[j];
+      const int j = jj - NLA;
+      if constexpr (PACKED) {
+        v4i lo, hi;
+        if constexpr (MMA::kWidenB) MMA::widen_b(stg[set][NLA + j], lo, hi);
+        else unpack_i4x32(stg[set][NLA + j], lo, hi, g.a_even_odd8);
+        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = lo;
+        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j) + 16) = hi;
+      } else {
+        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = stg[set][NLA + j];
+      }
     }
-    if constexpr (PACKED) {
-      v4i lo, hi;
-      if constexpr (MMA::kWidenB) MMA::widen_b(stg[NLA], lo, hi);
-      else unpack_i4x32(stg[NLA], lo, hi, g.a_even_odd8);
-      *reinterpret_cast<v4i*>(st + st_b) = lo;
-      *reinterpret_cast<v4i*>(st + st_b + 16) = hi;
-    } else {
+  };
+  auto store_stage = [&](const int set, const int stage_base) {
+    uint8_t* st = stage_mem + stage_base;
 #pragma unroll
-      for (int j = 0; j < NLB; ++j) *reinterpret_cast<v4i*>(st + st_b + j * st_b_next) = stg[NLA + j];
+    for (int j = 0; j < NLA; ++j) {
+      if constexpr (WIDEN_A) {
+        v4i lo, hi;
+        MMA::widen_a(stg[set][j], lo, hi);
+        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = lo;
+        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next + 16) = hi;
+      } else {
+        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = stg[set][j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NLB; ++j) {
+      if constexpr (PACKED) {
+        v4i lo, hi;
+        if constexpr (MMA::kWidenB) MMA::widen_b(stg[set][NLA + j], lo, hi);
+        else unpack_i4x32(stg[set][NLA + j], lo, hi, g.a_even_odd8);
+        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = lo;
+        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j) + 16) = hi;
+      } else {
+        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = stg[set][NLA + j];
+      }
     }
   };
 
   // fragment of k step ks: 16 kChunks bytes at (32 ks + 16 lh) kChunks of row lr of the 32-row block
-  const int a_off = (wm * 32 + lr) * kRow + lh * 16 * kChunks;
-  const int b_off = kATile + (wn * 64 + lr) * kRow + lh * 16 * kChunks;
+  const int a_off = (wm * 32 * IM + lr) * kRow + lh * 16 * kChunks;
+  const int b_off = kATile + (wn * 32 * IN + lr) * kRow + lh * 16 * kChunks;
   auto frag = [&](const uint8_t* at) -> Frag {
     if constexpr (kChunks == 1) {
       return *reinterpret_cast<const v4i*>(at);
@@ -180,143 +242,326 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     }
   };
 
-  Acc acc[2];
+  Acc acc[IM][IN];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) { acc[0][r] = 0; acc[1][r] = 0; }
+  for (int im = 0; im < IM; ++im)
+#pragma unroll
+    for (int in = 0; in < IN; ++in)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[im][in][r] = 0;
 
   const int nstages = (int)((g.k + BK - 1) / BK);
-#pragma unroll
-  for (int j = 0; j < NL; ++j) load_one(j, 0);
-  if constexpr (CONV) conv_advance();
-  store_stage(0);
-#pragma unroll
-  for (int j = 0; j < NL; ++j) load_one(j, nstages > 1 ? BK : 0);
-  if constexpr (CONV) conv_advance();
-  __syncthreads();
-
-  // Stage s reads buffer BUF; the staging registers (stage s + 1, requested during stage s - 1) go to the
-  // buffer stage s - 1 left, and the loads of stage s + 2 are issued behind them.  Past the last stage
-  // the store and the loads are repeated harmlessly (a buffer nobody reads, k offset 0) rather than
-  // branched around.
-  auto stage = [&](const int s, auto buf_c) {
-    constexpr int BUF = decltype(buf_c)::value;
-    const uint8_t* st = stage_mem + BUF * kStage;
-#pragma unroll
-    for (int ks = 0; ks < 4 / kChunks; ++ks) {
-      const Frag fa = frag(st + a_off + ks * 32 * kChunks);
-      const Frag fb0 = frag(st + b_off + ks * 32 * kChunks);
-      const Frag fb1 = frag(st + b_off + 32 * kRow + ks * 32 * kChunks);
-      acc[0] = MMA::mma(fb0, fa, acc[0]);
-      acc[1] = MMA::mma(fb1, fa, acc[1]);
-    }
-    store_stage((1 - BUF) * kStage);
-    const int k_next = s + 2 < nstages ? (s + 2) * BK : 0;
-#pragma unroll
-    for (int j = 0; j < NL; ++j) load_one(j, k_next);
-    if constexpr (CONV) conv_advance();  // past the last stage the tap leaves the window: zeros nobody reads
-    // a bare s_barrier: a __syncthreads() would also wait for the global loads just issued
+  auto lds_barrier = [&]() {  // a bare s_barrier: a __syncthreads() would also wait for the global loads in flight
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  for (int s = 0; s < nstages; s += 2) {
-    stage(s, std::integral_constant<int, 0>{});
-    if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
+  if constexpr (!RING) {
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(0, j, 0);
+    if constexpr (CONV) conv_advance();
+    store_stage(0, 0);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(0, j, nstages > 1 ? BK : 0);
+    if constexpr (CONV) conv_advance();
+    __syncthreads();
+
+    // Stage s reads buffer BUF; the staging registers (stage s + 1, requested during stage s - 1) go to the
+    // buffer stage s - 1 left, and the loads of stage s + 2 are issued behind them.  Past the last stage
+    // the store and the loads are repeated harmlessly (a buffer nobody reads, k offset 0) rather than
+    // branched around.
+    auto stage = [&](const int s, auto buf_c) {
+      constexpr int BUF = decltype(buf_c)::value;
+      const uint8_t* st = stage_mem + BUF * kStage;
+#pragma unroll
+      for (int ks = 0; ks < 4 / kChunks; ++ks) {
+        Frag fa[IM], fb[IN];
+#pragma unroll
+        for (int im = 0; im < IM; ++im) fa[im] = frag(st + a_off + im * 32 * kRow + ks * 32 * kChunks);
+#pragma unroll
+        for (int in = 0; in < IN; ++in) fb[in] = frag(st + b_off + in * 32 * kRow + ks * 32 * kChunks);
+#pragma unroll
+        for (int im = 0; im < IM; ++im)
+#pragma unroll
+          for (int in = 0; in < IN; ++in) acc[im][in] = MMA::mma(fb[in], fa[im], acc[im][in]);
+      }
+      store_stage(0, (1 - BUF) * kStage);
+      const int k_next = s + 2 < nstages ? (s + 2) * BK : 0;
+#pragma unroll
+      for (int j = 0; j < NL; ++j) load_one(0, j, k_next);
+      if constexpr (CONV) conv_advance();  // past the last stage the tap leaves the window: zeros nobody reads
+      lds_barrier();
+    };
+    for (int s = 0; s < nstages; s += 2) {
+      stage(s, std::integral_constant<int, 0>{});
+      if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
+    }
+  } else {
+    // Ring schedule: three LDS buffers, three staging sets.  Stage s computes from buffer s % 3, group by group
+    // (a group = kGroup k steps whose fragments are read together, one group ahead of the matrix instructions
+    // that use them).  Its share of every group: a piece of stage s + 2 goes from staging set (s + 2) % 3 to
+    // buffer (s + 2) % 3 (free since the barrier of stage s - 1: it held stage s - 1) and the same piece of stage
+    // s + 5 is requested into the registers just emptied, so that LDS writes and memory requests are spread over
+    // the stage and a request has three stages to arrive.  The barrier stands before the last group: every wave
+    // then holds its last fragments of stage s, and everything of stage s + 1 (written during stage s - 1) is
+    // published, so the first fragments of stage s + 1 are read under the last group's matrix instructions.
+    constexpr int KS = 4 / kChunks, G = S::kGroup, NG = KS / G;
+    static_assert(NG >= 2 && NG % 2 == 0, "the last group computes from fragment set 1");
+    static_assert(!CONV, "requests would have to advance the window tap piece by piece");
+    auto k_of = [&](const int s) -> int { return s < nstages ? s * BK : 0; };
+    Frag fa[2][G][IM], fb[2][G][IN];
+    auto load_frags = [&](const uint8_t* st, const int gi, const int fs) {
+#pragma unroll
+      for (int q = 0; q < G; ++q) {
+#pragma unroll
+        for (int im = 0; im < IM; ++im) fa[fs][q][im] = frag(st + a_off + im * 32 * kRow + (gi * G + q) * 32 * kChunks);
+#pragma unroll
+        for (int in = 0; in < IN; ++in) fb[fs][q][in] = frag(st + b_off + in * 32 * kRow + (gi * G + q) * 32 * kChunks);
+      }
+    };
+    auto mfma_group = [&](const int fs) {
+#pragma unroll
+      for (int q = 0; q < G; ++q)
+#pragma unroll
+        for (int im = 0; im < IM; ++im)
+#pragma unroll
+          for (int in = 0; in < IN; ++in) acc[im][in] = MMA::mma(fb[fs][q][in], fa[fs][q][im], acc[im][in]);
+    };
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(0, j, k_of(0));
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(1, j, k_of(1));
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(2, j, k_of(2));
+    store_stage(0, 0);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(0, j, k_of(3));
+    store_stage(1, kStage);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_one(1, j, k_of(4));
+    lds_barrier();
+    load_frags(stage_mem, 0, 0);
+    auto stage = [&](const int s, auto buf_c) {
+      constexpr int BUF = decltype(buf_c)::value, W = (BUF + 2) % 3, NXT = (BUF + 1) % 3;
+      const uint8_t* cur = stage_mem + BUF * kStage;
+      const uint8_t* next = stage_mem + NXT * kStage;
+      const int k_req = k_of(s + 5);
+      auto refill = [&](const int gi) {
+#pragma unroll
+        for (int j = gi * NL / NG; j < (gi + 1) * NL / NG; ++j) {
+          store_piece(W, W * kStage, j);
+          load_one(W, j, k_req);
+        }
+      };
+#pragma unroll
+      for (int gi = 0; gi < NG - 1; ++gi) {
+        load_frags(cur, gi + 1, (gi + 1) & 1);
+        refill(gi);
+        mfma_group(gi & 1);
+      }
+      lds_barrier();
+      mfma_group(1);
+      load_frags(next, 0, 0);
+      refill(NG - 1);
+    };
+    for (int s = 0; s < nstages; s += 3) {
+      stage(s, std::integral_constant<int, 0>{});
+      if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
+      if (s + 2 < nstages) stage(s + 2, std::integral_constant<int, 2>{});
+    }
   }
 
-  // ---- epilogue: lane holds C[m = wm*32 + lr][n = wn*64 + ni*32 + 8q + 4lh + e], register 4q + e of tile ni
-  const int64_t mm = m0 + wm * 32 + lr;
-  if (mm >= g.m) return;
-  if constexpr (SLAB) {
-    int32_t* dst = g.slabs + (((int64_t)blockIdx.z * gridDim.y + bz) * g.m + mm) * g.n;
-    const bool vec = (g.n % 4) == 0;
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t nn = n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh;
-        if (nn >= g.n) continue;
-        int v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[ni][4 * q + e] >> 4 : acc[ni][4 * q + e];  // exact: multiples of 16 (SLAB: int4)
-        if (vec) *reinterpret_cast<int4*>(dst + nn) = make_int4(v[0], v[1], v[2], v[3]);
-        else for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[nn + e] = v[e];
-      }
-    return;
-  } else {
+  // ---- epilogue: lane holds C[m = wm*32*IM + im*32 + lr][n = wn*32*IN + ni*32 + 8q + 4lh + e], register 4q + e of tile (im, ni)
+  // Where rows of C start 16-byte aligned, a wave passes its part of the tile through LDS (a region of its own
+  // in the stage buffers, which nobody reads any more) so that the stores are 16 bytes a lane along whole row
+  // segments: straight from the accumulator layout a store instruction touches 16 bytes in each of 32 rows.
+  if constexpr (!SLAB) {
     constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
     constexpr int kEsz = kOutBf16 ? 2 : 4;
-    const int64_t row_o = bz * g.stride_c + mm * g.ldc;
-    const float s_row = g.row_scale ? g.row_scale[bz * g.stride_rs + mm] : 1.0f;
-    const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
-    const bool cs_vec = ((uintptr_t)cs % 16) == 0;
-    const bool acc_vec = (g.ldc % 4) == 0 && (g.stride_c % 4) == 0 && ((uintptr_t)g.acc_out % 16) == 0;
-    const bool c_vec = (g.ldc % 4) == 0 && (g.stride_c % 4) == 0 && ((uintptr_t)g.c % (4 * kEsz)) == 0;
+    constexpr int kRowBytes = 32 * IN * kEsz, kPitch = kRowBytes + 16, kWaveBytes = 32 * IM * kPitch;
+    static_assert(S::kWaves * kWaveBytes <= NBUF * kStage, "the staged tile fits the stage buffers");
+    const bool staged = g.acc_out == nullptr && ((g.ldc * kEsz) % 16) == 0 && ((g.stride_c * kEsz) % 16) == 0 &&
+                        ((uintptr_t)g.c % 16) == 0 && ((n0 * kEsz) % 16) == 0;
+    if (staged) {
+      lds_barrier();
+      uint8_t* mine = stage_mem + wave * kWaveBytes;
+      const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+      const bool cs_vec = ((uintptr_t)cs % 16) == 0;
 #pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
+      for (int im = 0; im < IM; ++im) {
+        const int64_t mm = m0 + wm * 32 * IM + im * 32 + lr;
+        const float s_row = (g.row_scale && mm < g.m) ? g.row_scale[bz * g.stride_rs + mm] : 1.0f;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t nn = n0 + wn * 64 + ni * 32 + 8 * q + 4 * lh;
-        if (nn >= g.n) continue;
-        const bool full = nn + 4 <= g.n;
-        AccScalar v[4];
+        for (int ni = 0; ni < IN; ++ni)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (PACKED && MMA::kIntAcc) v[e] = acc[ni][4 * q + e] >> 4;
-          else v[e] = acc[ni][4 * q + e];
-        }
-        if (g.acc_out != nullptr) {  // 32-bit patterns, int32 or float
-          AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out) + row_o + nn;
-          if (full && acc_vec) {
-            *reinterpret_cast<int4*>(dst) = make_int4(__builtin_bit_cast(int, v[0]), __builtin_bit_cast(int, v[1]),
-                                                      __builtin_bit_cast(int, v[2]), __builtin_bit_cast(int, v[3]));
-          } else {
-            for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[e] = v[e];
+          for (int q = 0; q < 4; ++q) {
+            const int col = ni * 32 + 8 * q + 4 * lh;
+            const int64_t nn = n0 + wn * 32 * IN + col;
+            AccScalar v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if constexpr (PACKED && MMA::kIntAcc) v[e] = acc[im][ni][4 * q + e] >> 4;
+              else v[e] = acc[im][ni][4 * q + e];
+            }
+            uint8_t* at = mine + (im * 32 + lr) * kPitch + col * kEsz;
+            if constexpr (EPI == 3) {
+              *reinterpret_cast<int4*>(at) = make_int4(v[0], v[1], v[2], v[3]);
+            } else {
+              float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+              if (cs != nullptr) {
+                if (nn + 4 <= g.n && cs_vec) {
+                  const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
+                  csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
+                } else {
+                  for (int e = 0; e < 4 && nn + e < g.n; ++e) csv[e] = cs[nn + e];
+                }
+              }
+              float o[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = dequant_value<EPI, COL_FIRST>(v[e], s_row, csv[e]);
+              if constexpr (kOutBf16) {
+                uint2 w;
+                w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+                w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+                *reinterpret_cast<uint2*>(at) = w;
+              } else {
+                *reinterpret_cast<float4*>(at) = make_float4(o[0], o[1], o[2], o[3]);
+              }
+            }
           }
-        }
-        uint8_t* dst = reinterpret_cast<uint8_t*>(g.c) + (row_o + nn) * kEsz;
-        if constexpr (EPI == 3) {
-          if (full && c_vec) *reinterpret_cast<int4*>(dst) = make_int4(v[0], v[1], v[2], v[3]);
-          else for (int e = 0; e < 4 && nn + e < g.n; ++e) reinterpret_cast<int32_t*>(dst)[e] = v[e];
+      }
+      // the wave's own stores, in order with its reads below: no barrier
+      constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerPass = 64 / kLanesPerRow, kPerLane = 16 / kEsz;
+      const int pr = lane / kLanesPerRow, pc = lane % kLanesPerRow;
+#pragma unroll
+      for (int it = 0; it < 32 * IM / kRowsPerPass; ++it) {
+        const int r = it * kRowsPerPass + pr;
+        const v4i val = *reinterpret_cast<const v4i*>(mine + r * kPitch + pc * 16);
+        const int64_t mm = m0 + wm * 32 * IM + r;
+        const int64_t nn = n0 + wn * 32 * IN + pc * kPerLane;
+        if (mm >= g.m || nn >= g.n) continue;
+        uint8_t* dst = reinterpret_cast<uint8_t*>(g.c) + (bz * g.stride_c + mm * g.ldc + nn) * kEsz;
+        if (nn + kPerLane <= g.n) {
+          *reinterpret_cast<v4i*>(dst) = val;
         } else {
-          float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-          if (cs != nullptr) {
-            if (full && cs_vec) {
-              const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
-              csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
-            } else {
-              for (int e = 0; e < 4 && nn + e < g.n; ++e) csv[e] = cs[nn + e];
-            }
-          }
-          float o[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = dequant_value<EPI, COL_FIRST>(v[e], s_row, csv[e]);
-          if (full && c_vec) {
-            if constexpr (kOutBf16) {
-              uint2 w;
-              w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
-              w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
-              *reinterpret_cast<uint2*>(dst) = w;
-            } else {
-              *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-            }
-          } else {
-            for (int e = 0; e < 4 && nn + e < g.n; ++e) {
-              if constexpr (kOutBf16) reinterpret_cast<uint16_t*>(dst)[e] = bf16_bits(o[e]);
-              else reinterpret_cast<float*>(dst)[e] = o[e];
-            }
+          for (int e = 0; e < kPerLane && nn + e < g.n; ++e) {
+            if constexpr (kEsz == 2) reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)((uint32_t)val[e >> 1] >> (16 * (e & 1)));
+            else reinterpret_cast<int32_t*>(dst)[e] = val[e];
           }
         }
       }
+      return;
+    }
+  }
+#pragma unroll
+  for (int im = 0; im < IM; ++im) {
+    const int64_t mm = m0 + wm * 32 * IM + im * 32 + lr;
+    if (mm >= g.m) continue;
+    if constexpr (SLAB) {
+      int32_t* dst = g.slabs + (((int64_t)blockIdx.z * gridDim.y + bz) * g.m + mm) * g.n;
+      const bool vec = (g.n % 4) == 0;
+#pragma unroll
+      for (int ni = 0; ni < IN; ++ni)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t nn = n0 + wn * 32 * IN + ni * 32 + 8 * q + 4 * lh;
+          if (nn >= g.n) continue;
+          int v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = PACKED ? acc[im][ni][4 * q + e] >> 4 : acc[im][ni][4 * q + e];  // exact: multiples of 16 (SLAB: int4)
+          if (vec) *reinterpret_cast<int4*>(dst + nn) = make_int4(v[0], v[1], v[2], v[3]);
+          else for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[nn + e] = v[e];
+        }
+    } else {
+      constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
+      constexpr int kEsz = kOutBf16 ? 2 : 4;
+      const int64_t row_o = bz * g.stride_c + mm * g.ldc;
+      const float s_row = g.row_scale ? g.row_scale[bz * g.stride_rs + mm] : 1.0f;
+      const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
+      const bool cs_vec = ((uintptr_t)cs % 16) == 0;
+      const bool acc_vec = (g.ldc % 4) == 0 && (g.stride_c % 4) == 0 && ((uintptr_t)g.acc_out % 16) == 0;
+      const bool c_vec = (g.ldc % 4) == 0 && (g.stride_c % 4) == 0 && ((uintptr_t)g.c % (4 * kEsz)) == 0;
+#pragma unroll
+      for (int ni = 0; ni < IN; ++ni)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t nn = n0 + wn * 32 * IN + ni * 32 + 8 * q + 4 * lh;
+          if (nn >= g.n) continue;
+          const bool full = nn + 4 <= g.n;
+          AccScalar v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (PACKED && MMA::kIntAcc) v[e] = acc[im][ni][4 * q + e] >> 4;
+            else v[e] = acc[im][ni][4 * q + e];
+          }
+          if (g.acc_out != nullptr) {  // 32-bit patterns, int32 or float
+            AccScalar* dst = reinterpret_cast<AccScalar*>(g.acc_out) + row_o + nn;
+            if (full && acc_vec) {
+              *reinterpret_cast<int4*>(dst) = make_int4(__builtin_bit_cast(int, v[0]), __builtin_bit_cast(int, v[1]),
+                                                        __builtin_bit_cast(int, v[2]), __builtin_bit_cast(int, v[3]));
+            } else {
+              for (int e = 0; e < 4 && nn + e < g.n; ++e) dst[e] = v[e];
+            }
+          }
+          uint8_t* dst = reinterpret_cast<uint8_t*>(g.c) + (row_o + nn) * kEsz;
+          if constexpr (EPI == 3) {
+            if (full && c_vec) *reinterpret_cast<int4*>(dst) = make_int4(v[0], v[1], v[2], v[3]);
+            else for (int e = 0; e < 4 && nn + e < g.n; ++e) reinterpret_cast<int32_t*>(dst)[e] = v[e];
+          } else {
+            float csv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if (cs != nullptr) {
+              if (full && cs_vec) {
+                const float4 c4 = *reinterpret_cast<const float4*>(cs + nn);
+                csv[0] = c4.x; csv[1] = c4.y; csv[2] = c4.z; csv[3] = c4.w;
+              } else {
+                for (int e = 0; e < 4 && nn + e < g.n; ++e) csv[e] = cs[nn + e];
+              }
+            }
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = dequant_value<EPI, COL_FIRST>(v[e], s_row, csv[e]);
+            if (full && c_vec) {
+              if constexpr (kOutBf16) {
+                uint2 w;
+                w.x = (uint32_t)bf16_bits(o[0]) | ((uint32_t)bf16_bits(o[1]) << 16);
+                w.y = (uint32_t)bf16_bits(o[2]) | ((uint32_t)bf16_bits(o[3]) << 16);
+                *reinterpret_cast<uint2*>(dst) = w;
+              } else {
+                *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+              }
+            } else {
+              for (int e = 0; e < 4 && nn + e < g.n; ++e) {
+                if constexpr (kOutBf16) reinterpret_cast<uint16_t*>(dst)[e] = bf16_bits(o[e]);
+                else reinterpret_cast<float*>(dst)[e] = o[e];
+              }
+            }
+          }
+        }
+    }
   }
 }
 
-template <int EPI, bool COL_FIRST>
+template <int EPI, bool COL_FIRST, class S = Mid128>
 void launch_mid(const GemmArgs& g, bool packed, dim3 grid, hipStream_t st) {
   if constexpr (!COL_FIRST) {
-    if (packed) { gemm_mid_kernel<MmaI8, EPI, false, true, false><<<grid, 512, 0, st>>>(g); return; }
+    if (packed) { gemm_mid_kernel<MmaI8, EPI, false, true, false, false, S><<<grid, S::kThreads, 0, st>>>(g); return; }
   }
-  gemm_mid_kernel<MmaI8, EPI, COL_FIRST, false, false><<<grid, 512, 0, st>>>(g);
+  gemm_mid_kernel<MmaI8, EPI, COL_FIRST, false, false, false, S><<<grid, S::kThreads, 0, st>>>(g);
+}
+
+// Every epilogue of the int8 contraction on tile shape S.
+template <class S>
+void launch_mid_shape(GemmArgs g, const aqtx_gemm_plan* p, int epi, bool packed, hipStream_t st) {
+  g.tiles_m = (int)((p->m + S::kTM - 1) / S::kTM);
+  g.tiles_n = (int)((p->n + S::kTN - 1) / S::kTN);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
+  switch (epi) {
+    case 0: if (g.col_first) launch_mid<0, true, S>(g, packed, grid, st); else launch_mid<0, false, S>(g, packed, grid, st); break;
+    case 1: if (g.col_first) launch_mid<1, true, S>(g, packed, grid, st); else launch_mid<1, false, S>(g, packed, grid, st); break;
+    case 2: if (g.col_first) launch_mid<2, true, S>(g, packed, grid, st); else launch_mid<2, false, S>(g, packed, grid, st); break;
+    case 4: if (g.col_first) launch_mid<4, true, S>(g, packed, grid, st); else launch_mid<4, false, S>(g, packed, grid, st); break;
+    default: launch_mid<3, false, S>(g, packed, grid, st); break;
+  }
 }
 
 template <class MMA, bool WIDENED = false>
@@ -342,22 +587,29 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
-// Whether the 128 x 128 kernel takes the plan (0 = no) and in how many slices of K (1 = none).
+// Whether the kernel of this file takes the plan (0 = no) and in how many slices of K (1 = none).
+// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 = the ring schedule on
+// 128 x 128 | 64 x 128 | 64 x 64 tiles (never in slices).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
-  if (p->group_offsets != nullptr || (p->tuning != 0 && p->tuning != 128) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
+  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 131)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
   if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)TN >= (1ll << 31)) return 0;
   const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);
   const int64_t pad128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN);
   const int64_t tiles256 = pad256 * p->batch, tiles128 = pad128 * p->batch;
   const int64_t max_by_k = (p->k + 2 * BK - 1) / (2 * BK);  // a slice holds at least two stages
+  if (p->tuning > 128) return 1;
   if (p->k_split > 1) return (int)(p->k_split < max_by_k ? p->k_split : max_by_k);
   // the large tiles fill the chip, unless a third of their area or more lies outside C (n or m of 128, say)
   const bool padded = 4 * pad256 * 2 >= 3 * pad128;
-  if (p->tuning != 128 && tiles256 > 128 && !padded) return 0;
+  if (p->tuning < 128 && tiles256 > 128 && !padded) return 0;
   if (p->k_split == 1 || tiles256 > 128) return 1;
-  // slices until about 256 workgroups exist (one per CU; two fit), each walking at least 1024 of k; the
-  // slabs they write and the sum kernel reads stay small next to the operands at such tile counts
+  // A long k over few tiles (a quarter of the CUs or fewer): slices until about 256 workgroups exist, each
+  // walking at least 1024 of k; the slabs they write and the sum kernel reads stay small next to the operands
+  // at such tile counts.  Measured at 4096 columns: k = 14336 in 23 us (128 rows) and 32 us (256 rows) against
+  // 35 and 36 us for the smaller tiles of the ring schedule on all of k; k = 4096 in 17.5 and 20 us against 11
+  // and 12 us, so a k below 8192 is never cut.
+  if (p->k < 8192 || 4 * tiles128 > 256) return 1;
   int64_t s = 256 / tiles128;
   if (s > 8) s = 8;
   if (s > p->k / 1024) s = p->k / 1024;
@@ -404,12 +656,17 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel, k slices");
     return 0;
   }
-  switch (epi) {
-    case 0: if (g.col_first) launch_mid<0, true>(g, packed, grid, st); else launch_mid<0, false>(g, packed, grid, st); break;
-    case 1: if (g.col_first) launch_mid<1, true>(g, packed, grid, st); else launch_mid<1, false>(g, packed, grid, st); break;
-    case 2: if (g.col_first) launch_mid<2, true>(g, packed, grid, st); else launch_mid<2, false>(g, packed, grid, st); break;
-    case 4: if (g.col_first) launch_mid<4, true>(g, packed, grid, st); else launch_mid<4, false>(g, packed, grid, st); break;
-    default: launch_mid<3, false>(g, packed, grid, st); break;
+  // Tile shape: plan->tuning 128 .. 131 names one (tests, measurements); otherwise, where the 128 x 128 tiles
+  // number at most one per CU, the ring schedule on the largest of its tiles that still gives every CU one
+  // (a workgroup alone on its CU has nobody to overlap its waits with: the ring hides them itself)
+  const int64_t tiles128 = (int64_t)g.tiles_m * g.tiles_n * p->batch;
+  const int cus = compute_units();
+  int shape = p->tuning >= 128 ? p->tuning : tiles128 > cus ? 128 : 4 * tiles128 <= cus ? 131 : 2 * tiles128 <= cus ? 130 : 129;
+  switch (shape) {
+    case 129: launch_mid_shape<Ring128>(g, p, epi, packed, st); break;
+    case 130: launch_mid_shape<Ring64x128>(g, p, epi, packed, st); break;
+    case 131: launch_mid_shape<Ring64>(g, p, epi, packed, st); break;
+    default: launch_mid_shape<Mid128>(g, p, epi, packed, st); break;
   }
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel");
   return 0;

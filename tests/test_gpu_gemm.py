@@ -12,10 +12,12 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[4, 8, 16, 128, 0], ids=['waves4', 'waves8', 'persistent', 'tiles128', 'auto'])
+@pytest.fixture(params=[4, 8, 16, 128, 129, 130, 131, 0],
+                ids=['waves4', 'waves8', 'persistent', 'tiles128', 'ring128', 'ring64x128', 'ring64', 'auto'])
 def waves(request, monkeypatch):
-  """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, the 128 x 128 kernel, and the library's own
-  choice (these shapes have few output tiles: the 128 x 128 kernel, with k in slices where it is long)."""
+  """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, the kernel for few output tiles on each of its
+  tile shapes and schedules, and the library's own choice (these shapes have few output tiles: the smaller
+  tiles, with k in slices where it is long)."""
   monkeypatch.setattr(ops, 'GEMM_TUNING', request.param)
   return request.param
 
@@ -182,6 +184,53 @@ def test_k_slices_rejected_where_unsupported(gpu):
   offs = torch.tensor([0, 64], dtype=torch.int32, device=gpu)
   with pytest.raises(RuntimeError, match='k_split > 1 with ragged batches'):
     ops.gemm(a, b, row_scale=None, col_scale=None, out_dtype=torch.int32, group_offsets=offs, k_split=2)
+
+
+# ---- every tile shape and schedule of the kernel for few output tiles gives the bits of the large tiles ----
+@pytest.mark.parametrize('b_kind', ['rows', 'fragments', 'packed', 'packed_fragments'])
+@pytest.mark.parametrize('batch,m,n,k,out,sdt', [
+    (1, 200, 328, 4160, 'bf16', 'bf16'),   # ragged m and n, a k tail of 64
+    (1, 130, 201, 1056, 'bf16', 'f32'),    # rows of C not 16-byte aligned: the stores straight from the accumulators
+    (2, 129, 136, 384, 'f32', 'f32'),      # batches, three stages: as many as the ring has buffers
+    (1, 64, 72, 128, 'bf16', 'bf16'),      # one stage
+    (1, 512, 1024, 256, 'i32', None),      # raw sums, two stages
+    (1, 96, 4096, 2048, 'f32', 'f32'),
+])
+def test_few_tiles_kernel_shapes_give_the_same_bits(gpu, monkeypatch, batch, m, n, k, out, sdt, b_kind):
+  """plan->tuning 128 (128 x 128 tiles, plain schedule) and 129 | 130 | 131 (the ring schedule on 128 x 128,
+  64 x 128 and 64 x 64 tiles) against the 256 x 256 kernel on the same operands: integer sums, the same
+  epilogue arithmetic, so bit for bit, outputs and raw accumulators, for rows and the fragment order of b,
+  int8 and packed int4."""
+  packed, frag = b_kind.startswith('packed'), b_kind.endswith('fragments')
+  if frag and (batch > 1 or out == 'i32'):
+    pytest.skip('the fragment order holds one weight, whose column count the binding reads off the column scale')
+  torch.manual_seed(11)
+  lo, hi = (-8, 8) if packed else (-127, 128)
+  a = torch.randint(-127, 128, (batch, m, k), dtype=torch.int8, device=gpu)
+  b = torch.randint(lo, hi, (batch, n, k), dtype=torch.int8, device=gpu)
+  b_arg, b_dtype = b, L.I8
+  if packed:
+    b_arg, b_dtype = ops.pack_i4(b.reshape(batch * n, k)).reshape(batch, n, k // 2), L.I4P
+  kw = dict(b_dtype=b_dtype, want_acc=True, k_split=1)
+  if out == 'i32':
+    kw.update(row_scale=None, col_scale=None, out_dtype=torch.int32)
+  else:
+    kw.update(row_scale=torch.rand(batch, m, device=gpu) + 0.5, col_scale=torch.rand(batch, n, device=gpu) * 0.01 + 1e-4,
+              out_dtype=U.TORCH_DT[out], scale_dtype=U.TORCH_DT[sdt])
+  monkeypatch.setattr(ops, 'GEMM_TUNING', 8)
+  want, want_acc = ops.gemm(a, b_arg, **kw)
+  ref = torch.einsum('bmk,bnk->bmn', a.cpu().to(torch.int64), b.cpu().to(torch.int64)).to(torch.int32)
+  assert torch.equal(want_acc.cpu(), ref)
+  if frag:
+    b_arg, kw['b_layout'] = ops.tile_weight(b_arg[0].contiguous(), b_dtype), L.W_FRAGMENTS
+  for tuning in (128, 129, 130, 131, 0):
+    monkeypatch.setattr(ops, 'GEMM_TUNING', tuning)
+    got, got_acc = ops.gemm(a, b_arg, **kw)
+    alone = ops.gemm(a, b_arg, **dict(kw, want_acc=False))  # without the copy of the sums the tile leaves through LDS
+    bits = torch.int16 if out == 'bf16' else torch.int32
+    assert torch.equal(got_acc, want_acc), tuning
+    assert torch.equal(got.view(bits), want.view(bits)), tuning
+    assert torch.equal(alone.view(bits), want.view(bits)), tuning
 
 
 # ---- packed int4 B (two values per byte, unpacked in registers) ---------------------------------
