@@ -1,13 +1,15 @@
 // int8 x int8 -> int32 contraction for shapes with few output tiles: the same arithmetic as the
-// 256 x 256 kernel of gemm_core.h on 128 x 128 tiles, optionally with K cut into slices.
+// 256 x 256 kernel of gemm_core.h on smaller tiles, optionally with K cut into slices.
 //
 // A 256 x 256 tile keeps one CU busy for all of K whatever the rest of the chip does, so a product
-// of 512 x 4096 (32 such tiles) leaves 224 of the 256 CUs idle.  Here a workgroup of 8 waves (4 x 2)
-// owns 128 x 128 of C, a wave 32 x 64 (two v_mfma_i32_32x32x32_i8 tiles, 32 accumulators), with 128
-// registers per lane and 72 KiB of LDS, so that two workgroups share a CU: four times the workgroups,
-// each a quarter of the work.  When even that leaves CUs idle and K is long, grid.z cuts K into slices
-// whose int32 partial sums go to slabs of a workspace, and dequant_slabs_kernel adds them up (integer
-// sums: exact in any order) and applies the epilogue.
+// of 512 x 4096 (32 such tiles) leaves 224 of the 256 CUs idle.  Here a workgroup owns a tile of 128 x 128
+// (8 waves of 32 x 64: two v_mfma_i32_32x32x32_i8 tiles, 32 accumulators), 64 x 128 or 64 x 64 (4 waves) of C:
+// MidShape.  Two schedules.  Plain: two LDS buffers (72 KiB) and under 128 registers, so that two workgroups
+// share a CU and fill each other's waits; for launches with more tiles than CUs.  Ring: three LDS buffers,
+// three stages in flight in registers, LDS writes and memory requests spread over the stage, for launches of
+// at most one workgroup per CU, which has nobody to overlap its waits with.  When even the small tiles leave
+// CUs idle and K is long, grid.z cuts K into slices whose int32 partial sums go to slabs of a workspace, and
+// dequant_slabs_kernel adds them up (integer sums: exact in any order) and applies the epilogue.
 //
 // LDS rows are 144 bytes apart (128 of data, 16 of padding): the 16 lanes of a fragment read fall into
 // distinct banks and every address of the loop is a loop-invariant register plus an immediate.
@@ -577,6 +579,23 @@ void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
 #undef AQTX_MID8
 }
 
+// Tile shape for a launch of `tiles128` 128 x 128 tiles on `cus` CUs (plan->tuning values): more tiles than CUs
+// share the CUs two workgroups each on the plain schedule; otherwise the ring schedule on the largest of its
+// tiles that still gives every CU one (a workgroup alone on its CU has nobody to overlap its waits with: the
+// ring hides them itself).
+inline int mid_shape_for(int64_t tiles128, int cus) {
+  return tiles128 > cus ? 128 : 4 * tiles128 <= cus ? 131 : 2 * tiles128 <= cus ? 130 : 129;
+}
+
+template <class S>
+void launch_weight_only_shape(GemmArgs g, const aqtx_gemm_plan* p, hipStream_t st) {
+  g.tiles_m = (int)((p->m + S::kTM - 1) / S::kTM);
+  g.tiles_n = (int)((p->n + S::kTN - 1) / S::kTN);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
+  if (p->col_scale_dtype == AQTX_BF16) gemm_mid_kernel<MmaBf16W8, 0, false, true, false, false, S><<<grid, S::kThreads, 0, st>>>(g);
+  else gemm_mid_kernel<MmaBf16W8, 4, false, true, false, false, S><<<grid, S::kThreads, 0, st>>>(g);
+}
+
 template <int EPI>
 void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
   if constexpr (EPI != 3) {
@@ -656,12 +675,10 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel, k slices");
     return 0;
   }
-  // Tile shape: plan->tuning 128 .. 131 names one (tests, measurements); otherwise, where the 128 x 128 tiles
-  // number at most one per CU, the ring schedule on the largest of its tiles that still gives every CU one
-  // (a workgroup alone on its CU has nobody to overlap its waits with: the ring hides them itself)
+  // tile shape: plan->tuning 128 .. 131 names one (tests, measurements)
   const int64_t tiles128 = (int64_t)g.tiles_m * g.tiles_n * p->batch;
   const int cus = compute_units();
-  int shape = p->tuning >= 128 ? p->tuning : tiles128 > cus ? 128 : 4 * tiles128 <= cus ? 131 : 2 * tiles128 <= cus ? 130 : 129;
+  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(tiles128, cus);
   switch (shape) {
     case 129: launch_mid_shape<Ring128>(g, p, epi, packed, st); break;
     case 130: launch_mid_shape<Ring64x128>(g, p, epi, packed, st); break;
@@ -764,11 +781,15 @@ int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const vo
   g.col_first = 0;
   g.b_frag = p->b_layout == AQTX_W_FRAGMENTS;
   g.b_steps = (int)((p->k + 63) / 64);
-  g.tiles_m = (int)((p->m + TM - 1) / TM);
-  g.tiles_n = (int)((p->n + TN - 1) / TN);
-  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch);
-  if (p->col_scale_dtype == AQTX_BF16) gemm_mid_kernel<MmaBf16W8, 0, false, true, false><<<grid, 512, 0, st>>>(g);
-  else gemm_mid_kernel<MmaBf16W8, 4, false, true, false><<<grid, 512, 0, st>>>(g);
+  const int64_t tiles128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN) * p->batch;
+  const int cus = compute_units();
+  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(tiles128, cus);
+  switch (shape) {
+    case 129: launch_weight_only_shape<Ring128>(g, p, st); break;
+    case 130: launch_weight_only_shape<Ring64x128>(g, p, st); break;
+    case 131: launch_weight_only_shape<Ring64>(g, p, st); break;
+    default: launch_weight_only_shape<Mid128>(g, p, st); break;
+  }
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<weight only>");
   return 0;
 }

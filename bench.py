@@ -542,13 +542,63 @@ def gemm_probe(dev, data, reps=10):
     a, b = gen((1, m, k)), gen((1, n, k))
     rs, cs = torch.rand(1, m, device=dev), torch.rand(1, n, device=dev)
     ms = timed(lambda: ops.gemm(a, b, row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16))
-    bt = b[0].t().contiguous()  # the library takes the second operand [k, n]
-    ms_lib = timed(lambda: torch._int_mm(a[0], bt))
+    # the library takes the second operand [k, n]: the rows of b viewed transposed (k contiguous in both
+    # operands, as this library reads them), and a [k, n] copy
+    ms_lib = timed(lambda: torch._int_mm(a[0], b[0].t()))
+    bt = b[0].t().contiguous()
+    ms_lib_kn = timed(lambda: torch._int_mm(a[0], bt))
     ops_ = 2.0 * m * n * k
     rows[shape] = {'m': m, 'n': n, 'k': k, 'aqtx_gemm_i8_us': round(ms * 1e3, 1), 'aqtx_TOPS': round(ops_ / ms / 1e9),
-                   'library_int_mm_us': round(ms_lib * 1e3, 1), 'library_TOPS': round(ops_ / ms_lib / 1e9)}
+                   'library_int_mm_us': round(ms_lib * 1e3, 1), 'library_TOPS': round(ops_ / ms_lib / 1e9),
+                   'library_int_mm_kn_copy_us': round(ms_lib_kn * 1e3, 1), 'library_kn_copy_TOPS': round(ops_ / ms_lib_kn / 1e9)}
     del a, b, bt
   print(json.dumps({'gemm_probe': data, 'reps': reps, 'shapes': rows}))
+
+
+def prefill_probe(dev, shapes=False):
+  """Contractions of prefill-sized serving calls (128..4096 rows against the 4096 x 14336 MLP weights and a
+  4096 x 4096 one), device time per call replayed from a HIP graph, microseconds: aqtx_gemm_i8 (int8 operands
+  drawn from round(25 * normal), bf16 output with both scales fused, the library's own choice of kernel) next to
+  the vendor int8 GEMM (torch._int_mm, raw int32 output), and aqtx_gemm_weight_only (bf16 rows, int8 weight)
+  next to the vendor bf16 product on a bf16 copy of the weight.  With `shapes`, also every tile shape of the
+  kernel for few output tiles forced through plan->tuning (their results are compared bit for bit with the
+  library's choice).  Prints one JSON line per shape."""
+  import torch
+  from aqt_amd import ops
+
+  def t(f, calls=10):
+    return round(_graph_replay_us(lambda: [f() for _ in range(calls)], calls, reps=3), 1)
+
+  def ints(shape):
+    return (torch.randn(shape, device=dev) * 25).clamp(-127, 127).round().to(torch.int8)
+
+  forced = (('tiles128', 128), ('ring128', 129), ('ring64x128', 130), ('ring64', 131)) if shapes else ()
+  saved = ops.GEMM_TUNING
+  for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
+    b = ints((1, n, k))
+    bt = b[0].t()  # the vendor int8 GEMM takes the second operand [k, n]: the same rows, viewed transposed
+    bf = b[0].to(torch.bfloat16)
+    cs = torch.rand(1, n, device=dev) * 0.01 + 1e-4
+    for m in (128, 256, 512, 1024, 2048, 4096):
+      a = ints((1, m, k))
+      x = torch.randn(1, m, k, device=dev).to(torch.bfloat16)
+      rs = torch.rand(1, m, device=dev) * 0.01 + 1e-4
+      kw = dict(row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16, scale_dtype=torch.bfloat16)
+      ops.GEMM_TUNING = saved
+      ref = ops.gemm(a, b, **kw)
+      row = {'prefill_probe': 'us per call', 'm': m, 'n': n, 'k': k, 'aqtx_gemm_i8': t(lambda: ops.gemm(a, b, **kw)),
+             'vendor_int_mm': t(lambda: torch._int_mm(a[0], bt))}
+      for name, tuning in forced:
+        ops.GEMM_TUNING = tuning
+        out = ops.gemm(a, b, k_split=1, **kw)
+        assert torch.equal(out, ref), (name, m, n, k)
+        row[name] = t(lambda: ops.gemm(a, b, k_split=1, **kw))
+      ops.GEMM_TUNING = saved
+      row['aqtx_gemm_weight_only'] = t(lambda: ops.gemm_weight_only(x, b, cs))
+      row['vendor_bf16_on_a_copy'] = t(lambda: torch.matmul(x[0], bf.t()))
+      print(json.dumps(row), flush=True)
+      del a, x
+    del b, bt, bf
 
 
 def power_probe(dev, seconds=8.0):
@@ -647,6 +697,9 @@ def main():
                        'distribution (and the vendor int8 GEMM beside them) and exit')
   ap.add_argument('--decode-probe', action='store_true',
                   help='only issue a few serving calls per shape (for rocprofv3 runs) and exit')
+  ap.add_argument('--prefill-probe', choices=['library', 'shapes'], default=None,
+                  help='only time prefill-sized contractions (128..4096 rows against the MLP weights) next to the vendor '
+                       "GEMMs and exit; 'shapes' adds every tile shape of the kernel for few output tiles")
   ap.add_argument('--power-probe', action='store_true',
                   help='only run the forward contraction back to back on all-zero and on quantized-normal operands while '
                        'sampling socket power and shader clock from the SMI tool, and exit')
@@ -672,6 +725,9 @@ def main():
   dev = torch.device('cuda:0')
   if args.gemm_probe is not None:
     gemm_probe(dev, args.gemm_probe)
+    return
+  if args.prefill_probe is not None:
+    prefill_probe(dev, shapes=args.prefill_probe == 'shapes')
     return
   if args.power_probe:
     power_probe(dev)
