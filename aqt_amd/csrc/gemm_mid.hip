@@ -19,12 +19,16 @@ namespace aqtx {
 namespace {
 
 constexpr int TM = 128, TN = 128;
-constexpr int kRow = BK + 16;
 
 // Tile of a workgroup and how its waves share it: WM x WN waves, each (TM / WM) x (TN / WN) of C in 32 x 32
 // matrix-instruction tiles.  A wave fetches TM / waves rows of A and TN / waves rows of B per stage.
-template <int TM_, int TN_, int WM_, int WN_, int OCC_ = 4, bool RING_ = false, int GROUP_ = 1>
+template <int TM_, int TN_, int WM_, int WN_, int OCC_ = 4, bool RING_ = false, int GROUP_ = 1, bool SWIZZLE_ = false>
 struct MidShape {
+  // LDS rows: 128 bytes of data and 16 of padding, or (kSwizzle) 128 bytes with the 16-byte chunks of a row
+  // exchanged among themselves by an XOR with a function of the row, which spreads the 16 rows of a fragment
+  // read over the banks just as well and fits three buffers of a 128 x 256 tile into the 160 KiB of a CU
+  static constexpr bool kSwizzle = SWIZZLE_;
+  static constexpr int kRow = SWIZZLE_ ? BK : BK + 16;
   static constexpr int kOcc = OCC_;      // waves per SIMD the registers are budgeted for
   static constexpr bool kRing = RING_;   // three LDS buffers and three stages in flight in registers (see the kernel)
   static constexpr int kGroup = GROUP_;  // ring schedule: k steps whose fragments are read together
@@ -39,6 +43,7 @@ using Mid128 = MidShape<128, 128, 4, 2>;  // 8 waves of 32 x 64, 36 KiB a stage,
 using Ring128 = MidShape<128, 128, 4, 2, 2, true, 2>;
 using Ring64x128 = MidShape<64, 128, 2, 2, 2, true, 2>;
 using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2>;
+using Ring128x256 = MidShape<128, 256, 2, 4, 2, true, 1, true>;  // 8 waves of 64 x 64, 144 KiB of LDS
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
 // int4 values two per byte (see gemm_kernel's BPACK), or, with MmaBf16W8, int8 values that become bf16 (A then
@@ -51,7 +56,8 @@ using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2>;
 template <class MMA, int EPI, bool COL_FIRST, bool PACKED, bool SLAB, bool CONV = false, class S = Mid128>
 __global__ __launch_bounds__(S::kThreads) __attribute__((amdgpu_waves_per_eu(S::kOcc, S::kOcc)))
 void gemm_mid_kernel(const GemmArgs g_in) {
-  constexpr int TM = S::kTM, TN = S::kTN, kATile = S::kATile, kStage = S::kStage;
+  constexpr int TM = S::kTM, TN = S::kTN, kATile = S::kATile, kStage = S::kStage, kRow = S::kRow;
+  constexpr bool SW = S::kSwizzle;
   constexpr int IM = S::kIM, IN = S::kIN, RA = S::kRA, RB = S::kRB;
   constexpr bool RING = S::kRing;
   constexpr int NSETS = RING ? 3 : 1, NBUF = RING ? 3 : 2;
@@ -115,20 +121,36 @@ void gemm_mid_kernel(const GemmArgs g_in) {
                           : (wave * RB + (lane >> 3)) * (int)g.ldb + (lane & 7) * 16;
   const int kpos_a = WIDEN_A ? (lane & 3) * 32 : (lane & 7) * 16;
   const int kpos_b = g.b_frag ? (lane >> 4) * (PACKED ? 32 : 16) : PACKED ? (lane & 3) * 32 : (lane & 7) * 16;
-  const int st_a = WIDEN_A ? (wave * RA + (lane >> 2)) * kRow + (lane & 3) * 32
-                           : (wave * RA + (lane >> 3)) * kRow + (lane & 7) * 16;
-  const int st_a_next = (WIDEN_A ? 16 : 8) * kRow;
-  const int st_b = kATile + (g.b_frag ? (wave * RB + (lane & 15)) * kRow + (lane >> 4) * (PACKED ? 32 : 16)
-                             : PACKED ? (wave * RB + (lane >> 2)) * kRow + (lane & 3) * 32
-                                      : (wave * RB + (lane >> 3)) * kRow + (lane & 7) * 16);
+  // byte offset, within a tile, of 16-byte chunk `chunk` of row `row`
+  auto lds_pos = [&](const int row, const int chunk) -> int {
+    if constexpr (SW) {
+      const int r = row & 31;
+      return row * kRow + ((chunk ^ ((r ^ (r >> 3)) & 7)) << 4);
+    } else {
+      return row * kRow + chunk * 16;
+    }
+  };
+  // where piece j of a stage goes in LDS (the first of its two chunks where a piece is widened to 32 bytes;
+  // the second follows it, or, swizzled, is its neighbour under XOR 16)
+  int st_off[NL];
+#pragma unroll
+  for (int j = 0; j < NLA; ++j)
+    st_off[j] = WIDEN_A ? lds_pos(wave * RA + j * 16 + (lane >> 2), 2 * (lane & 3))
+                        : lds_pos(wave * RA + j * 8 + (lane >> 3), lane & 7);
+#pragma unroll
+  for (int j = 0; j < NLB; ++j) {
+    if constexpr (PACKED)
+      st_off[NLA + j] = kATile + (g.b_frag ? lds_pos(wave * RB + j * 16 + (lane & 15), 2 * (lane >> 4))
+                                           : lds_pos(wave * RB + j * 16 + (lane >> 2), 2 * (lane & 3)));
+    else
+      st_off[NLA + j] = kATile + (g.b_frag ? lds_pos(wave * RB + (j >> 1) * 16 + (lane & 15), (lane >> 4) + 4 * (j & 1))
+                                           : lds_pos(wave * RB + j * 8 + (lane >> 3), lane & 7));
+  }
+  constexpr int kSecond = 16;  // second chunk of a widened piece: + 16, or ^ 16 when swizzled
   // load jj of B past the wave's first: memory offset, LDS offset, position along k (jj is a constant where used)
   auto b_mem_next = [&](const int jj) -> int {
     if constexpr (PACKED) return g.b_frag ? jj * g.b_steps * 1024 : jj * 16 * (int)g.ldb;
     else return g.b_frag ? (jj >> 1) * g.b_steps * 1024 + (jj & 1) * 1024 : jj * 8 * (int)g.ldb;
-  };
-  auto b_lds_next = [&](const int jj) -> int {
-    if constexpr (PACKED) return jj * 16 * kRow;
-    else return g.b_frag ? (jj >> 1) * 16 * kRow + (jj & 1) * 64 : jj * 8 * kRow;
   };
   auto b_kpos_next = [&](const int jj) -> int { return (!PACKED && g.b_frag) ? (jj & 1) * 64 : 0; };
   const int ksh_b = g.b_frag ? 4 : 0;  // scalar offset of B = row bytes << ksh_b
@@ -182,64 +204,45 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   };
   auto store_piece = [&](const int set, const int stage_base, const int jj) {
     uint8_t* st = stage_mem + stage_base;
+    const int second = SW ? (st_off[jj] ^ kSecond) : st_off[jj] + kSecond;
     if (jj < NLA) {
-      const int j = jj;
       if constexpr (WIDEN_A) {
         v4i lo, hi;
-        MMA::widen_a(stg[set][j], lo, hi);
-        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = lo;
-        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next + 16) = hi;
+        MMA::widen_a(stg[set][jj], lo, hi);
+        *reinterpret_cast<v4i*>(st + st_off[jj]) = lo;
+        *reinterpret_cast<v4i*>(st + second) = hi;
       } else {
-        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = stg[set][j];
+        *reinterpret_cast<v4i*>(st + st_off[jj]) = stg[set][jj];
       }
     } else {
-      const int j = jj - NLA;
       if constexpr (PACKED) {
         v4i lo, hi;
-        if constexpr (MMA::kWidenB) MMA::widen_b(stg[set][NLA + j], lo, hi);
-        else unpack_i4x32(stg[set][NLA + j], lo, hi, g.a_even_odd8);
-        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = lo;
-        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j) + 16) = hi;
+        if constexpr (MMA::kWidenB) MMA::widen_b(stg[set][jj], lo, hi);
+        else unpack_i4x32(stg[set][jj], lo, hi, g.a_even_odd8);
+        *reinterpret_cast<v4i*>(st + st_off[jj]) = lo;
+        *reinterpret_cast<v4i*>(st + second) = hi;
       } else {
-        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = stg[set][NLA + j];
+        *reinterpret_cast<v4i*>(st + st_off[jj]) = stg[set][jj];
       }
     }
   };
   auto store_stage = [&](const int set, const int stage_base) {
-    uint8_t* st = stage_mem + stage_base;
 #pragma unroll
-    for (int j = 0; j < NLA; ++j) {
-      if constexpr (WIDEN_A) {
-        v4i lo, hi;
-        MMA::widen_a(stg[set][j], lo, hi);
-        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = lo;
-        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next + 16) = hi;
-      } else {
-        *reinterpret_cast<v4i*>(st + st_a + j * st_a_next) = stg[set][j];
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < NLB; ++j) {
-      if constexpr (PACKED) {
-        v4i lo, hi;
-        if constexpr (MMA::kWidenB) MMA::widen_b(stg[set][NLA + j], lo, hi);
-        else unpack_i4x32(stg[set][NLA + j], lo, hi, g.a_even_odd8);
-        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = lo;
-        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j) + 16) = hi;
-      } else {
-        *reinterpret_cast<v4i*>(st + st_b + b_lds_next(j)) = stg[set][NLA + j];
-      }
-    }
+    for (int j = 0; j < NL; ++j) store_piece(set, stage_base, j);
   };
 
-  // fragment of k step ks: 16 kChunks bytes at (32 ks + 16 lh) kChunks of row lr of the 32-row block
-  const int a_off = (wm * 32 * IM + lr) * kRow + lh * 16 * kChunks;
-  const int b_off = kATile + (wn * 32 * IN + lr) * kRow + lh * 16 * kChunks;
-  auto frag = [&](const uint8_t* at) -> Frag {
+  // fragment of k step ks of a 32-row block: the kChunks chunks from (2 ks + lh) kChunks on of row lr; their
+  // offsets within the block are the same for every block (the swizzle looks at the row modulo 32 only)
+  constexpr int KS = 4 / kChunks;
+  int fo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) fo[i] = lds_pos(lr, (2 * (i / kChunks) + lh) * kChunks + i % kChunks);
+  const int a_blk = wm * 32 * IM * kRow, b_blk = kATile + wn * 32 * IN * kRow;
+  auto frag = [&](const uint8_t* blk, const int ks) -> Frag {
     if constexpr (kChunks == 1) {
-      return *reinterpret_cast<const v4i*>(at);
+      return *reinterpret_cast<const v4i*>(blk + fo[ks]);
     } else {
-      const v4i x0 = *reinterpret_cast<const v4i*>(at), x1 = *reinterpret_cast<const v4i*>(at + 16);
+      const v4i x0 = *reinterpret_cast<const v4i*>(blk + fo[2 * ks]), x1 = *reinterpret_cast<const v4i*>(blk + fo[2 * ks + 1]);
       return Frag{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
     }
   };
@@ -276,12 +279,12 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       constexpr int BUF = decltype(buf_c)::value;
       const uint8_t* st = stage_mem + BUF * kStage;
 #pragma unroll
-      for (int ks = 0; ks < 4 / kChunks; ++ks) {
+      for (int ks = 0; ks < KS; ++ks) {
         Frag fa[IM], fb[IN];
 #pragma unroll
-        for (int im = 0; im < IM; ++im) fa[im] = frag(st + a_off + im * 32 * kRow + ks * 32 * kChunks);
+        for (int im = 0; im < IM; ++im) fa[im] = frag(st + a_blk + im * 32 * kRow, ks);
 #pragma unroll
-        for (int in = 0; in < IN; ++in) fb[in] = frag(st + b_off + in * 32 * kRow + ks * 32 * kChunks);
+        for (int in = 0; in < IN; ++in) fb[in] = frag(st + b_blk + in * 32 * kRow, ks);
 #pragma unroll
         for (int im = 0; im < IM; ++im)
 #pragma unroll
@@ -307,7 +310,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     // the stage and a request has three stages to arrive.  The barrier stands before the last group: every wave
     // then holds its last fragments of stage s, and everything of stage s + 1 (written during stage s - 1) is
     // published, so the first fragments of stage s + 1 are read under the last group's matrix instructions.
-    constexpr int KS = 4 / kChunks, G = S::kGroup, NG = KS / G;
+    constexpr int G = S::kGroup, NG = KS / G;
     static_assert(NG >= 2 && NG % 2 == 0, "the last group computes from fragment set 1");
     static_assert(!CONV, "requests would have to advance the window tap piece by piece");
     auto k_of = [&](const int s) -> int { return s < nstages ? s * BK : 0; };
@@ -316,9 +319,9 @@ void gemm_mid_kernel(const GemmArgs g_in) {
 #pragma unroll
       for (int q = 0; q < G; ++q) {
 #pragma unroll
-        for (int im = 0; im < IM; ++im) fa[fs][q][im] = frag(st + a_off + im * 32 * kRow + (gi * G + q) * 32 * kChunks);
+        for (int im = 0; im < IM; ++im) fa[fs][q][im] = frag(st + a_blk + im * 32 * kRow, gi * G + q);
 #pragma unroll
-        for (int in = 0; in < IN; ++in) fb[fs][q][in] = frag(st + b_off + in * 32 * kRow + (gi * G + q) * 32 * kChunks);
+        for (int in = 0; in < IN; ++in) fb[fs][q][in] = frag(st + b_blk + in * 32 * kRow, gi * G + q);
       }
     };
     auto mfma_group = [&](const int fs) {
@@ -579,12 +582,15 @@ void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
 #undef AQTX_MID8
 }
 
-// Tile shape for a launch of `tiles128` 128 x 128 tiles on `cus` CUs (plan->tuning values): more tiles than CUs
-// share the CUs two workgroups each on the plain schedule; otherwise the ring schedule on the largest of its
-// tiles that still gives every CU one (a workgroup alone on its CU has nobody to overlap its waits with: the
-// ring hides them itself).
-inline int mid_shape_for(int64_t tiles128, int cus) {
-  return tiles128 > cus ? 128 : 4 * tiles128 <= cus ? 131 : 2 * tiles128 <= cus ? 130 : 129;
+// Tile shape for a plan on `cus` CUs (plan->tuning values).  At most one 128 x 128 tile per CU: the ring
+// schedule on the largest of its tiles that still gives every CU one (a workgroup alone on its CU has nobody to
+// overlap its waits with: the ring hides them itself).  More than that but at most one 128 x 256 tile per CU:
+// the ring on those.  Beyond: 128 x 128 tiles on the plain schedule, two workgroups a CU.
+inline int mid_shape_for(const aqtx_gemm_plan* p, int cus) {
+  const int64_t tiles128 = ((p->m + 127) / 128) * ((p->n + 127) / 128) * p->batch;
+  const int64_t tiles256 = ((p->m + 127) / 128) * ((p->n + 255) / 256) * p->batch;
+  if (tiles128 > cus) return tiles256 <= cus ? 132 : 128;
+  return 4 * tiles128 <= cus ? 131 : 2 * tiles128 <= cus ? 130 : 129;
 }
 
 template <class S>
@@ -607,10 +613,10 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 }  // namespace
 
 // Whether the kernel of this file takes the plan (0 = no) and in how many slices of K (1 = none).
-// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 = the ring schedule on
-// 128 x 128 | 64 x 128 | 64 x 64 tiles (never in slices).
+// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 | 132 = the ring schedule on
+// 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 tiles (never in slices).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
-  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 131)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
+  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 132)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
   if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)TN >= (1ll << 31)) return 0;
   const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);
@@ -676,10 +682,9 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     return 0;
   }
   // tile shape: plan->tuning 128 .. 131 names one (tests, measurements)
-  const int64_t tiles128 = (int64_t)g.tiles_m * g.tiles_n * p->batch;
-  const int cus = compute_units();
-  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(tiles128, cus);
+  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(p, compute_units());
   switch (shape) {
+    case 132: launch_mid_shape<Ring128x256>(g, p, epi, packed, st); break;
     case 129: launch_mid_shape<Ring128>(g, p, epi, packed, st); break;
     case 130: launch_mid_shape<Ring64x128>(g, p, epi, packed, st); break;
     case 131: launch_mid_shape<Ring64>(g, p, epi, packed, st); break;
@@ -781,10 +786,9 @@ int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const vo
   g.col_first = 0;
   g.b_frag = p->b_layout == AQTX_W_FRAGMENTS;
   g.b_steps = (int)((p->k + 63) / 64);
-  const int64_t tiles128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN) * p->batch;
-  const int cus = compute_units();
-  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(tiles128, cus);
+  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(p, compute_units());
   switch (shape) {
+    case 132: launch_weight_only_shape<Ring128x256>(g, p, st); break;
     case 129: launch_weight_only_shape<Ring128>(g, p, st); break;
     case 130: launch_weight_only_shape<Ring64x128>(g, p, st); break;
     case 131: launch_weight_only_shape<Ring64>(g, p, st); break;
