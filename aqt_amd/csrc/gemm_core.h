@@ -650,7 +650,7 @@ void gemm_kernel(const GemmArgs g_in) {
             }
           }
         }
-        __syncthreads();
+        // (no barrier: the region is this wave's own, and a wave's LDS accesses complete in order)
         // read back: lane -> 16-byte pair (lane % LPR) of row (lane / LPR) + RPI*it
         constexpr int LPR = RB / 16, RPI = 64 / LPR;
         const int64_t ncol_pass0 = ncol0 + (int64_t)pass * kNiPerPass * 32;
@@ -685,7 +685,6 @@ void gemm_kernel(const GemmArgs g_in) {
             }
           }
         }
-        if (pass + 1 < kPasses) __syncthreads();
       }
     };
     if (interior && ((uintptr_t)cs % 16) == 0) epilogue(std::false_type{});
