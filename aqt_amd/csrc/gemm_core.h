@@ -312,14 +312,15 @@ void gemm_kernel(const GemmArgs g_in) {
     g.stride_a = 0; g.stride_c = 0; g.stride_rs = 0;
   }
 
-  // ---- global -> registers -> LDS.  One wave instruction moves 8 rows x 128 B (1 KiB): lane l
-  // handles LDS slot (row l>>3, chunk l&7) of its 8-row block and fetches the global chunk
-  // (l&7) ^ f(row), f(row) = (row ^ row>>3) & 7, which is the XOR swizzle the fragment reads
-  // undo.  Rows past the end of the operand fall outside the buffer and read as zero.
-  // The loads go through registers (not buffer->LDS DMA) on purpose: a stage buffer is only
-  // free for refilling at the very end of a stage, and 64 KiB requested in one burst queue up
-  // in the CU's address unit while the waves that issued them cannot issue MFMAs.  Register
-  // staging lets the 16 loads of a wave spread over the whole stage.
+  // ---- global -> LDS.  One wave instruction moves 8 rows x 128 B (1 KiB): lane l handles LDS slot
+  // (row l>>3, chunk l&7) of its 8-row block and fetches the global chunk (l&7) ^ f(row),
+  // f(row) = (row ^ row>>3) & 7, which is the XOR swizzle the fragment reads undo.  Rows past the end of
+  // the operand fall outside the buffer and read as zero.  A stage buffer is only free for refilling at the
+  // end of a stage (behind the barrier that stands before the last k step).  Unpacked operands are requested
+  // there straight into it (buffer load to LDS, one request per matrix instruction of that k step; the same
+  // 64 KiB requested in one burst right behind the barrier queued up in the CU's address unit while the waves
+  // that issued them could not issue MFMAs).  Packed operands, and the first stage of a tile, go through
+  // registers: requested a few MFMAs apart over the stage, written to the freed buffer with ds_write.
   // BFRAG, B in fragment order (GemmArgs::b_frag): the tile's 16-row blocks follow one another, b_steps KiB
   // each; the piece (row r, 16 bytes at 16 c of a 64-byte step) is lane r % 16 + 16 c of its KiB, and the scalar
   // offset of a stage is its row bytes times 16.
@@ -383,6 +384,21 @@ void gemm_kernel(const GemmArgs g_in) {
     }
   };
   const int st_off = wave * LPW * 1024 + lane * 16;
+  // Unpacked operands refill a stage buffer straight from memory (buffer load to LDS: lane i's 16 bytes land at
+  // base + 16 i, which is the layout above), one request per matrix instruction of the stage's last k step,
+  // with no ds_write: a stage's 64 ds_write_b128 (8 cycles each) added their 470 cycles to the 2070 the stage
+  // takes without them, wherever in the stage they stood (clock stamps: 2550 cycles a stage through registers,
+  // 2220-2300 this way).  Packed operands are unpacked in registers and keep that path.
+  constexpr bool kDirect = !BPACK;
+  auto load_direct = [&](uint8_t* st, int j, int k0) {  // piece j (the numbering of load_global) of the stage at k0
+    const bool is_b = j & 1;
+    const int i = j >> 1;
+    int vo = is_b ? voff_b[i] : voff_a[i];
+    if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
+    uint8_t* at = st + (is_b ? kTileBytes : 0) + wave * LPW * 1024 + i * 1024;  // wave-uniform
+    if (!is_b) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)at, 16, vo, k0, 0, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)at, 16, vo, k0 << ksh_b, 0, 0);
+  };
   auto store_lds = [&](uint8_t* st, int j) {  // j = 0..NL-1
     if constexpr (!BPACK) {
       const int i = j >> 1;
@@ -442,13 +458,14 @@ void gemm_kernel(const GemmArgs g_in) {
   constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100, kDsWrite = 0x200;
 
   // Software pipeline of one stage (KS k-steps of 16 MFMAs):
-  //   k-steps 0..KS-2: fragments of the next k-step are read from LDS (spread over the MFMAs)
-  //                 and the 16 global loads of the block two stages ahead are issued a few
+  //   k-steps 0..KS-2: fragments of the next k-step are read from LDS (spread over the MFMAs);
+  //                 packed operands: the global loads of the block two stages ahead are issued a few
   //                 MFMAs apart, into the staging registers;
-  //   barrier     : every wave holds its last fragments of this stage, the buffer is free;
-  //   last k-step : the staging registers are written into the freed buffer (one ds_write per
-  //                 MFMA, each waiting only for its own load) and the first fragments of the
-  //                 next stage are read from the other buffer.
+  //   barrier     : every wave holds its last fragments of this stage, the buffer is free; with direct
+  //                 refills each wave has first waited for its own requests into the other buffer;
+  //   last k-step : the freed buffer is refilled with the block two stages ahead, one request (direct) or
+  //                 one ds_write from the staging registers (packed, each waiting only for its own load)
+  //                 per MFMA, and the first fragments of the next stage are read from the other buffer.
   // The barrier is a bare s_barrier: a __syncthreads() would also wait for the global loads
   // still in flight.  No branch surrounds any MFMA (a conditional stage makes the compiler
   // shuffle all 256 accumulators through VGPRs).
@@ -460,10 +477,12 @@ void gemm_kernel(const GemmArgs g_in) {
       // loads [l0, l1) of the 16 go with this k-step
       const int l0 = (NLD * ks + KS - 2) / (KS - 1), l1 = (NLD * (ks + 1) + KS - 2) / (KS - 1);
       if (ks % 2 == 0) load_frags(cur, ks + 1, fa1, fb1); else load_frags(cur, ks + 1, fa0, fb0);
+      if constexpr (!kDirect) {
 #pragma unroll
-      for (int j = l0; j < l1; ++j) load_global(j, refill_k0);
+        for (int j = l0; j < l1; ++j) load_global(j, refill_k0);
+      }
       if (ks % 2 == 0) mfma_step(fa0, fb0); else mfma_step(fa1, fb1);
-      const int nl = l1 - l0;
+      const int nl = kDirect ? 0 : l1 - l0;
 #pragma unroll
       for (int i = 0; i < MPK; ++i) {
         __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
@@ -475,19 +494,28 @@ void gemm_kernel(const GemmArgs g_in) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // direct refills: this wave's pieces of the other buffer (requested a stage ago) have landed, and after the
+    // barrier so have everybody's
+    if constexpr (kDirect) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kDirect) {
 #pragma unroll
-    for (int j = 0; j < NL; ++j) store_lds(cur_refill, j);
+      for (int j = 0; j < NL; ++j) load_direct(cur_refill, j, refill_k0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NL; ++j) store_lds(cur_refill, j);
+    }
     // KS is even, so the last k-step always computes from set 1 and refills set 0.
     load_frags(next, 0, fa0, fb0);
     mfma_step(fa1, fb1);
 #pragma unroll
     for (int i = 0; i < MPK; ++i) {
       __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(kDsWrite, 1, 0);
+      if (kDirect) __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
+      else __builtin_amdgcn_sched_group_barrier(kDsWrite, 1, 0);
       if (i < kDsPerStep) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -515,16 +543,25 @@ void gemm_kernel(const GemmArgs g_in) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 #pragma unroll
   for (int j = 0; j < NL; ++j) store_lds(stage0, j);
+  if constexpr (kDirect) {
 #pragma unroll
-  for (int j = 0; j < NLD; ++j) load_global(j, BK);
+    for (int j = 0; j < NL; ++j) load_direct(stage1, j, BK);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
 #pragma unroll
-  for (int j = 0; j < NL; ++j) store_lds(stage1, j);
+    for (int j = 0; j < NLD; ++j) load_global(j, BK);
+#pragma unroll
+    for (int j = 0; j < NL; ++j) store_lds(stage1, j);
+  }
   __syncthreads();
   load_frags(stage0, 0, fa0, fb0);
   for (int it = 0; it < KT2; ++it) {
     run_stage(stage0, stage0, stage1, refill_at((2 * it + 2) * BK));
     run_stage(stage1, stage1, stage0, refill_at((2 * it + 3) * BK));
   }
+  // (direct refills requested past the end of k re-read its last block: they have to land before the epilogue
+  // stages the output in the same buffers)
+  if constexpr (kDirect) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   // ---- epilogue ---------------------------------------------------------------
