@@ -22,8 +22,12 @@ constexpr int TM = 128, TN = 128;
 
 // Tile of a workgroup and how its waves share it: WM x WN waves, each (TM / WM) x (TN / WN) of C in 32 x 32
 // matrix-instruction tiles.  A wave fetches TM / waves rows of A and TN / waves rows of B per stage.
-template <int TM_, int TN_, int WM_, int WN_, int OCC_ = 4, bool RING_ = false, int GROUP_ = 1, bool SWIZZLE_ = false>
+template <int TM_, int TN_, int WM_, int WN_, int OCC_ = 4, bool RING_ = false, int GROUP_ = 1, bool SWIZZLE_ = false,
+          int BUFFERS_ = 0>
 struct MidShape {
+  // > 0 (ring, swizzled rows): operands that need no unpacking are requested straight into this many LDS
+  // buffers (see the kernel); packed operands keep three buffers and the staging registers
+  static constexpr int kBuffers = BUFFERS_;
   // LDS rows: 128 bytes of data and 16 of padding, or (kSwizzle) 128 bytes with the 16-byte chunks of a row
   // exchanged among themselves by an XOR with a function of the row, which spreads the 16 rows of a fragment
   // read over the banks just as well and fits three buffers of a 128 x 256 tile into the 160 KiB of a CU
@@ -40,10 +44,12 @@ struct MidShape {
 };
 using Mid128 = MidShape<128, 128, 4, 2>;  // 8 waves of 32 x 64, 36 KiB a stage, two workgroups a CU
 // One workgroup a CU (or several small ones), for launches of at most one workgroup per CU: the ring schedule.
-using Ring128 = MidShape<128, 128, 4, 2, 2, true, 2>;
-using Ring64x128 = MidShape<64, 128, 2, 2, 2, true, 2>;
-using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2>;
-using Ring128x256 = MidShape<128, 256, 2, 4, 2, true, 1, true>;  // 8 waves of 64 x 64, 144 KiB of LDS
+// (four buffers each: six for the 64 x 64 tile, one workgroup a CU then, measured 23 us where two workgroups a CU
+// on four take 16 (512 x 4096 x 4096); five for the others changed nothing)
+using Ring128 = MidShape<128, 128, 4, 2, 2, true, 2, true, 4>;
+using Ring64x128 = MidShape<64, 128, 2, 2, 2, true, 2, true, 4>;
+using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2, true, 4>;
+using Ring128x256 = MidShape<128, 256, 2, 4, 2, true, 1, true, 3>;  // 8 waves of 64 x 64, 144 KiB of LDS
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
 // int4 values two per byte (see gemm_kernel's BPACK), or, with MmaBf16W8, int8 values that become bf16 (A then
@@ -60,7 +66,10 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   constexpr bool SW = S::kSwizzle;
   constexpr int IM = S::kIM, IN = S::kIN, RA = S::kRA, RB = S::kRB;
   constexpr bool RING = S::kRing;
-  constexpr int NSETS = RING ? 3 : 1, NBUF = RING ? 3 : 2;
+  // ring, swizzled rows, nothing to unpack: pieces go from memory straight into LDS
+  constexpr bool DIRECT = RING && SW && !PACKED && !MMA::kWidenA && !CONV && !SLAB && S::kBuffers >= 3;
+  constexpr int NB = DIRECT ? S::kBuffers : 0;
+  constexpr int NSETS = DIRECT ? 1 : RING ? 3 : 1, NBUF = RING ? 3 : 2;
   static_assert(!CONV || (TM == 128 && S::kWaves == 8), "the window gather is written for two loads of A per wave");
   static_assert(!SLAB || EPI == 3, "a K slice leaves raw sums");
   static_assert(!CONV || (MMA::kIntAcc && !PACKED && !SLAB), "the convolution reads int8 bytes, whole K");
@@ -72,7 +81,19 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   using Frag = typename MMA::Frag;
   constexpr int kChunks = MMA::kChunks;  // 16-byte chunks a lane holds of one MFMA's k
   GemmArgs g = g_in;
-  __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[NBUF * kStage];
+  __shared__ __attribute__((aligned(1024))) uint8_t stage_mem[DIRECT ? 16 : NBUF * kStage];
+  // the direct ring's buffers are objects of their own, so that the compiler can tell a fragment read of one from
+  // a request in flight into another
+  __shared__ __attribute__((aligned(1024))) uint8_t ring0[DIRECT ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring1[DIRECT ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring2[DIRECT ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring3[DIRECT && NB > 3 ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring4[DIRECT && NB > 4 ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring5[DIRECT && NB > 5 ? kStage : 16];
+  static_assert(NB <= 6, "six ring buffers at most");
+  auto ring = [&](const int b) -> uint8_t* {
+    return b == 0 ? ring0 : b == 1 ? ring1 : b == 2 ? ring2 : b == 3 ? ring3 : b == 4 ? ring4 : ring5;
+  };
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / S::kWN, wn = wave % S::kWN;
@@ -301,6 +322,106 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       stage(s, std::integral_constant<int, 0>{});
       if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
     }
+  } else if constexpr (DIRECT) {
+    // Direct ring: NB LDS buffers, no staging registers and no ds_write (a stage's ds_write_b128, 8 cycles each on
+    // the CU's one LDS pipe, added their time whole to the stage).  A piece = 8 rows x 128 B of a wave's share of
+    // A or B; lane l asks for the chunk that belongs at position l & 7 of row l >> 3 (chunk (l & 7) ^ f(row)), and
+    // the buffer load to LDS puts lane l's 16 bytes at base + 16 l.  Stage s computes from buffer s % NB as in the
+    // ring below and, group by group, requests the pieces of stage s + NB - 1 into the buffer stage s - 1 left at
+    // its barrier.  Requests complete in order, so before its barrier a wave waits until all but the requests
+    // issued after those of stage s + 1 have landed, and behind the barrier everybody's have.
+    constexpr int G = S::kGroup, NG = KS / G, D = NB - 1;
+    static_assert(NG >= 2 && NG % 2 == 0, "the last group computes from fragment set 1");
+    static_assert(NLA == RA / 8 && NLB == RB / 8, "pieces of 8 rows");
+    auto k_of = [&](const int s) -> int { return s < nstages ? s * BK : 0; };
+    int dvo[NL], dkp[NL];  // vector offset of a piece's request and its position along k (for the mask on K)
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      const bool is_b = j >= NLA;
+      const int row = is_b ? wave * RB + (j - NLA) * 8 + (lane >> 3) : wave * RA + j * 8 + (lane >> 3);
+      const int r = row & 31;
+      const int c = (lane & 7) ^ ((r ^ (r >> 3)) & 7);
+      dkp[j] = c * 16;
+      dvo[j] = !is_b ? row * (int)g.lda + c * 16
+             : g.b_frag ? ((row >> 4) * g.b_steps + (c >> 2)) * 1024 + ((c & 3) * 16 + (row & 15)) * 16
+                        : row * (int)g.ldb + c * 16;
+    }
+    auto request = [&](uint8_t* buf, const int j, const int k0) {
+      const int vo = k0 + dkp[j] < (int)g.k ? dvo[j] : kOutside;
+      if (j < NLA)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(buf + (wave * RA + j * 8) * kRow), 16, vo, k0, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(buf + kATile + (wave * RB + (j - NLA) * 8) * kRow), 16, vo, k0 << ksh_b, 0, 0);
+    };
+    Frag fa[2][G][IM], fb[2][G][IN];
+    auto load_frags = [&](const uint8_t* st, const int gi, const int fs) {
+#pragma unroll
+      for (int q = 0; q < G; ++q) {
+#pragma unroll
+        for (int im = 0; im < IM; ++im) fa[fs][q][im] = frag(st + a_blk + im * 32 * kRow, gi * G + q);
+#pragma unroll
+        for (int in = 0; in < IN; ++in) fb[fs][q][in] = frag(st + b_blk + in * 32 * kRow, gi * G + q);
+      }
+    };
+    auto mfma_group = [&](const int fs) {
+#pragma unroll
+      for (int q = 0; q < G; ++q)
+#pragma unroll
+        for (int im = 0; im < IM; ++im)
+#pragma unroll
+          for (int in = 0; in < IN; ++in) acc[im][in] = MMA::mma(fb[fs][q][in], fa[fs][q][im], acc[im][in]);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+#pragma unroll
+      for (int j = 0; j < NL; ++j) request(ring(d), j, k_of(d));
+    // stage 0 has landed when at most the requests of stages 1 .. D - 1 are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D - 1) * NL) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    load_frags(ring0, 0, 0);
+    constexpr int kBefore = (NG - 1) * NL / NG;              // pieces a stage requests before its barrier
+    constexpr int kAfterNext = (D - 2) * NL + kBefore;       // requests issued after those of the next stage
+    static_assert(kAfterNext <= 63, "vmcnt");
+    auto stage = [&](const int s, auto buf_c) {
+      constexpr int BUF = decltype(buf_c)::value, W = (BUF + D) % NB, NXT = (BUF + 1) % NB;
+      const uint8_t* cur = ring(BUF);
+      const uint8_t* next = ring(NXT);
+      const int k_req = k_of(s + D);
+      auto refill = [&](const int gi) {
+#pragma unroll
+        for (int j = gi * NL / NG; j < (gi + 1) * NL / NG; ++j) request(ring(W), j, k_req);
+      };
+#pragma unroll
+      for (int gi = 0; gi < NG - 1; ++gi) {
+        load_frags(cur, gi + 1, (gi + 1) & 1);
+        refill(gi);
+        mfma_group(gi & 1);
+      }
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kAfterNext) : "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      mfma_group(1);
+      load_frags(next, 0, 0);
+      refill(NG - 1);
+    };
+    for (int s = 0; s < nstages; s += NB) {
+      stage(s, std::integral_constant<int, 0>{});
+      if (s + 1 < nstages) stage(s + 1, std::integral_constant<int, 1>{});
+      if (s + 2 < nstages) stage(s + 2, std::integral_constant<int, 2>{});
+      if constexpr (NB > 3) {
+        if (s + 3 < nstages) stage(s + 3, std::integral_constant<int, 3>{});
+      }
+      if constexpr (NB > 4) {
+        if (s + 4 < nstages) stage(s + 4, std::integral_constant<int, 4>{});
+      }
+      if constexpr (NB > 5) {
+        if (s + 5 < nstages) stage(s + 5, std::integral_constant<int, 5>{});
+      }
+    }
+    // requests past the end of k (they repeat stage 0) have to land before the epilogue stages the output in the
+    // same buffers
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   } else {
     // Ring schedule: three LDS buffers, three staging sets.  Stage s computes from buffer s % 3, group by group
     // (a group = kGroup k steps whose fragments are read together, one group ahead of the matrix instructions
@@ -384,12 +505,15 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     constexpr bool kOutBf16 = EPI <= 1 || EPI == 4;
     constexpr int kEsz = kOutBf16 ? 2 : 4;
     constexpr int kRowBytes = 32 * IN * kEsz, kPitch = kRowBytes + 16, kWaveBytes = 32 * IM * kPitch;
-    static_assert(S::kWaves * kWaveBytes <= NBUF * kStage, "the staged tile fits the stage buffers");
-    const bool staged = g.acc_out == nullptr && ((g.ldc * kEsz) % 16) == 0 && ((g.stride_c * kEsz) % 16) == 0 &&
+    // (direct ring: the waves share out its buffers, wave w in buffer w % NB)
+    constexpr bool kStagedFits = DIRECT ? ((S::kWaves + NB - 1) / (DIRECT ? NB : 1)) * kWaveBytes <= kStage
+                                        : S::kWaves * kWaveBytes <= NBUF * kStage;
+    static_assert(DIRECT || kStagedFits, "the staged tile fits the stage buffers");
+    const bool staged = kStagedFits && g.acc_out == nullptr && ((g.ldc * kEsz) % 16) == 0 && ((g.stride_c * kEsz) % 16) == 0 &&
                         ((uintptr_t)g.c % 16) == 0 && ((n0 * kEsz) % 16) == 0;
     if (staged) {
       lds_barrier();
-      uint8_t* mine = stage_mem + wave * kWaveBytes;
+      uint8_t* mine = DIRECT ? ring(wave % (DIRECT ? NB : 1)) + (wave / (DIRECT ? NB : 1)) * kWaveBytes : stage_mem + wave * kWaveBytes;
       const float* cs = g.col_scale ? g.col_scale + bz * g.stride_cs : nullptr;
       const bool cs_vec = ((uintptr_t)cs % 16) == 0;
 #pragma unroll
@@ -583,16 +707,18 @@ void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
 }
 
 // Tile shape for a plan on `cus` CUs (plan->tuning values).  At most one 128 x 128 tile per CU: the ring
-// schedule on the largest of its tiles that still gives every CU one (a workgroup alone on its CU has nobody to
-// overlap its waits with: the ring hides them itself).  More than that but at most one 128 x 256 tile per CU:
-// the ring on those.  Beyond: 128 x 128 tiles on the plain schedule, two workgroups a CU.
+// schedule (a workgroup alone on its CU has nobody to overlap its waits with: the ring hides them itself), on
+// 64 x 64 tiles up to half a 128 x 128 tile per CU (two of its workgroups fit a CU; measured ahead of 64 x 128
+// at 64-128 tiles: 15.8 against 17.7 us at 512 x 4096 x 4096, 17.5 against 19.0 at 128 x 14336 x 4096), on
+// 128 x 128 tiles beyond.  More than one 128 x 128 tile but at most one 128 x 256 tile per CU: the ring on
+// those.  Beyond: 128 x 128 tiles on the plain schedule, two workgroups a CU.
 inline int mid_shape_for(const aqtx_gemm_plan* p, int cus) {
   const int64_t tiles128 = ((p->m + 127) / 128) * ((p->n + 127) / 128) * p->batch;
   const int64_t tiles256 = ((p->m + 127) / 128) * ((p->n + 255) / 256) * p->batch;
   // (not for a k of fewer than eight stages: the ring's five stages of lead are most of such a tile;
   // 4096 x 2048 x 512 measured 15.5 us on it against 13.9 us on the plain schedule)
   if (tiles128 > cus) return (tiles256 <= cus && p->k >= 1024) ? 132 : 128;
-  return 4 * tiles128 <= cus ? 131 : 2 * tiles128 <= cus ? 130 : 129;
+  return 2 * tiles128 <= cus ? 131 : 129;
 }
 
 template <class S>
