@@ -5,14 +5,17 @@
 // of 512 x 4096 (32 such tiles) leaves 224 of the 256 CUs idle.  Here a workgroup owns a tile of 128 x 128
 // (8 waves of 32 x 64: two v_mfma_i32_32x32x32_i8 tiles, 32 accumulators), 64 x 128 or 64 x 64 (4 waves) of C:
 // MidShape.  Two schedules.  Plain: two LDS buffers (72 KiB) and under 128 registers, so that two workgroups
-// share a CU and fill each other's waits; for launches with more tiles than CUs.  Ring: three LDS buffers,
-// three stages in flight in registers, LDS writes and memory requests spread over the stage, for launches of
-// at most one workgroup per CU, which has nobody to overlap its waits with.  When even the small tiles leave
+// share a CU and fill each other's waits; for launches with more tiles than CUs.  Ring: three or four LDS
+// buffers refilled group by group over the stage (unpacked operands by buffer loads straight into LDS, packed
+// ones through three stages' worth of staging registers), for launches of at most one workgroup per CU, which
+// has nobody to overlap its waits with.  When even the small tiles leave
 // CUs idle and K is long, grid.z cuts K into slices whose int32 partial sums go to slabs of a workspace, and
 // dequant_slabs_kernel adds them up (integer sums: exact in any order) and applies the epilogue.
 //
-// LDS rows are 144 bytes apart (128 of data, 16 of padding): the 16 lanes of a fragment read fall into
-// distinct banks and every address of the loop is a loop-invariant register plus an immediate.
+// LDS rows of the plain schedule are 144 bytes apart (128 of data, 16 of padding): the 16 lanes of a fragment
+// read fall into distinct banks and every address of the loop is a loop-invariant register plus an immediate.
+// The ring shapes keep 128-byte rows with their 16-byte chunks swizzled instead, so that 8 rows are 1 KiB of
+// consecutive LDS, which is what a buffer load straight into LDS fills.
 #include "gemm_core.h"
 
 namespace aqtx {
