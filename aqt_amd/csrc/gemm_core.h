@@ -254,7 +254,7 @@ __device__ __forceinline__ float dequant_value(AccScalar accv, float s_row, floa
 // PERSIST: the grid has one workgroup per CU (or fewer) and a workgroup walks tiles blockIdx.x, + gridDim.x, ...
 // (the XCD-aware order of tile_of_block continues: a workgroup stays on its XCD's range).  Between two tiles no
 // workgroup has to be launched, and the first stage of the next tile is requested before the epilogue of this one
-// (the staging registers are free then), so its latency passes under the stores.  Plain batches only.
+// (packed operands: the staging registers are free then), so its latency passes under the stores.  Plain batches only.
 template <class MMA, int NW, int EPI, bool COL_FIRST, bool KTAIL, bool BPACK = false, bool BFRAG = false, bool PERSIST = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void gemm_kernel(const GemmArgs g_in) {
@@ -531,8 +531,10 @@ void gemm_kernel(const GemmArgs g_in) {
   // the per-chunk mask in load_global already covers them.
   const int k0_last = KTAIL ? 0x7FFFFF00 : (int)g.k - BK;
   auto refill_at = [&](int k0) { return k0 < k0_last ? k0 : k0_last; };
+  if constexpr (!kDirect) {
 #pragma unroll
-  for (int j = 0; j < NLD; ++j) load_global(j, 0);
+    for (int j = 0; j < NLD; ++j) load_global(j, 0);
+  }
   int tile = (int)blockIdx.x;
   for (;;) {  // one trip per tile (one trip unless PERSIST)
 #pragma unroll
@@ -541,13 +543,17 @@ void gemm_kernel(const GemmArgs g_in) {
     for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-#pragma unroll
-  for (int j = 0; j < NL; ++j) store_lds(stage0, j);
   if constexpr (kDirect) {
+    // (both stages straight into LDS: asking for the first one before the previous tile's epilogue, into
+    // registers, saved a thousand cycles a tile and cost ten spilled registers; measured level or 1 % behind)
+#pragma unroll
+    for (int j = 0; j < NL; ++j) load_direct(stage0, j, 0);
 #pragma unroll
     for (int j = 0; j < NL; ++j) load_direct(stage1, j, BK);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   } else {
+#pragma unroll
+    for (int j = 0; j < NL; ++j) store_lds(stage0, j);
 #pragma unroll
     for (int j = 0; j < NLD; ++j) load_global(j, BK);
 #pragma unroll
@@ -570,16 +576,18 @@ void gemm_kernel(const GemmArgs g_in) {
   const int64_t mrow0 = em0 + wm * 128, ncol0 = en0 + wn * NI * 32;
   bool more = false;
   if constexpr (PERSIST) {
-    // the next tile's first stage is requested now: the staging registers are free, and the epilogue's stores
-    // hide the latency
+    // packed operands: the next tile's first stage is requested now: the staging registers are free, and the
+    // epilogue's stores hide the latency
     tile += (int)gridDim.x;
     more = tile < g.tiles_m * g.tiles_n;
     if (more) {
       tile_of_block(tile, g.tiles_m, g.tiles_n, tm, tn);
       m0 = (int64_t)tm * BM; n0 = (int64_t)tn * BN;
       rsrc_a = rsrc_a_of(m0); rsrc_b = rsrc_b_of(n0);
+      if constexpr (!kDirect) {
 #pragma unroll
-      for (int j = 0; j < NLD; ++j) load_global(j, 0);
+        for (int j = 0; j < NLD; ++j) load_global(j, 0);
+      }
     }
   }
 
