@@ -221,7 +221,7 @@ extern "C" int aqtx_gemm_weight_only(const aqtx_gemm_plan* p, const void* a, con
                "%s: rows of a and b must start 16-byte aligned", who);
   AQTX_REQUIRE(p->batch <= 65535 && p->m <= (int64_t)65535 * 128 && (p->m + 127) / 128 * ((p->n + 127) / 128) < (1ll << 31),
                "%s: shape too large for one launch", who);
-  AQTX_REQUIRE(p->lda * 256 < (1ll << 31) && (b_frag || p->ldb * 128 < (1ll << 31)), "%s: leading dimension too large for 32-bit tile offsets", who);
+  AQTX_REQUIRE(p->lda * 256 < (1ll << 31) && (b_frag || p->ldb * 256 < (1ll << 31)), "%s: leading dimension too large for 32-bit tile offsets", who);
   if (p->batch == 0 || p->m == 0 || p->n == 0) return 0;
   AQTX_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "%s: NULL buffer", who);
   AQTX_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)c % 2) == 0, "%s: a and b must be 16-byte aligned", who);

@@ -749,7 +749,7 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
   if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 132)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
-  if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)TN >= (1ll << 31)) return 0;
+  if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)(2 * TN) >= (1ll << 31)) return 0;  // 32-bit offsets within a tile of up to 128 x 256
   const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);
   const int64_t pad128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN);
   const int64_t tiles256 = pad256 * p->batch, tiles128 = pad128 * p->batch;
