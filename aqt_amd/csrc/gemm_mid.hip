@@ -52,6 +52,10 @@ using Mid128 = MidShape<128, 128, 4, 2>;  // 8 waves of 32 x 64, 36 KiB a stage,
 using Ring128 = MidShape<128, 128, 4, 2, 2, true, 2, true, 4>;
 using Ring64x128 = MidShape<64, 128, 2, 2, 2, true, 2, true, 4>;
 using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2, true, 4>;
+// eight buffers where a 64 x 64 workgroup has its CU to itself: seven stages (112 KiB) on their way per workgroup.
+// Against weights that come from HBM (a different weight every call) 128 and 256 rows x 4096 x 4096 take 16.8 us
+// instead of 19.8; against a weight that stays in the memory-side cache nothing changes (10-11 us)
+using Ring64Deep = MidShape<64, 64, 2, 2, 2, true, 2, true, 8>;
 using Ring128x256 = MidShape<128, 256, 2, 4, 2, true, 1, true, 3>;  // 8 waves of 64 x 64, 144 KiB of LDS
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
@@ -93,9 +97,11 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   __shared__ __attribute__((aligned(1024))) uint8_t ring3[DIRECT && NB > 3 ? kStage : 16];
   __shared__ __attribute__((aligned(1024))) uint8_t ring4[DIRECT && NB > 4 ? kStage : 16];
   __shared__ __attribute__((aligned(1024))) uint8_t ring5[DIRECT && NB > 5 ? kStage : 16];
-  static_assert(NB <= 6, "six ring buffers at most");
+  __shared__ __attribute__((aligned(1024))) uint8_t ring6[DIRECT && NB > 6 ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring7[DIRECT && NB > 7 ? kStage : 16];
+  static_assert(NB <= 8, "eight ring buffers at most");
   auto ring = [&](const int b) -> uint8_t* {
-    return b == 0 ? ring0 : b == 1 ? ring1 : b == 2 ? ring2 : b == 3 ? ring3 : b == 4 ? ring4 : ring5;
+    return b == 0 ? ring0 : b == 1 ? ring1 : b == 2 ? ring2 : b == 3 ? ring3 : b == 4 ? ring4 : b == 5 ? ring5 : b == 6 ? ring6 : ring7;
   };
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -421,6 +427,12 @@ void gemm_mid_kernel(const GemmArgs g_in) {
       if constexpr (NB > 5) {
         if (s + 5 < nstages) stage(s + 5, std::integral_constant<int, 5>{});
       }
+      if constexpr (NB > 6) {
+        if (s + 6 < nstages) stage(s + 6, std::integral_constant<int, 6>{});
+      }
+      if constexpr (NB > 7) {
+        if (s + 7 < nstages) stage(s + 7, std::integral_constant<int, 7>{});
+      }
     }
     // requests past the end of k (they repeat stage 0) have to land before the epilogue stages the output in the
     // same buffers
@@ -711,7 +723,8 @@ void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
 
 // Tile shape for a plan on `cus` CUs (plan->tuning values).  At most one 128 x 128 tile per CU: the ring
 // schedule (a workgroup alone on its CU has nobody to overlap its waits with: the ring hides them itself), on
-// 64 x 64 tiles up to half a 128 x 128 tile per CU (two of its workgroups fit a CU; measured ahead of 64 x 128
+// 64 x 64 tiles up to half a 128 x 128 tile per CU (on eight buffers while every workgroup has a CU to itself, on
+// four beyond, when two of its workgroups fit a CU; measured ahead of 64 x 128
 // at 64-128 tiles: 15.8 against 17.7 us at 512 x 4096 x 4096, 17.5 against 19.0 at 128 x 14336 x 4096), on
 // 128 x 128 tiles beyond.  More than one 128 x 128 tile but at most one 128 x 256 tile per CU: the ring on
 // those.  Beyond: 128 x 128 tiles on the plain schedule, two workgroups a CU.
@@ -721,7 +734,8 @@ inline int mid_shape_for(const aqtx_gemm_plan* p, int cus) {
   // (not for a k of fewer than eight stages: the ring's five stages of lead are most of such a tile;
   // 4096 x 2048 x 512 measured 15.5 us on it against 13.9 us on the plain schedule)
   if (tiles128 > cus) return (tiles256 <= cus && p->k >= 1024) ? 132 : 128;
-  return 2 * tiles128 <= cus ? 131 : 129;
+  const int64_t tiles64 = ((p->m + 63) / 64) * ((p->n + 63) / 64) * p->batch;
+  return tiles64 <= cus ? 133 : 2 * tiles128 <= cus ? 131 : 129;
 }
 
 template <class S>
@@ -744,10 +758,10 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 }  // namespace
 
 // Whether the kernel of this file takes the plan (0 = no) and in how many slices of K (1 = none).
-// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 | 132 = the ring schedule on
-// 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 tiles (never in slices).
+// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 | 132 | 133 = the ring schedule on
+// 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 | 64 x 64 (eight buffers) tiles (never in slices).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
-  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 132)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
+  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 133)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
   if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)(2 * TN) >= (1ll << 31)) return 0;  // 32-bit offsets within a tile of up to 128 x 256
   const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);
@@ -760,12 +774,13 @@ int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
   const bool padded = 4 * pad256 * 2 >= 3 * pad128;
   if (p->tuning < 128 && tiles256 > 128 && !padded) return 0;
   if (p->k_split == 1 || tiles256 > 128) return 1;
-  // A long k over few tiles (a quarter of the CUs or fewer): slices until about 256 workgroups exist, each
+  // A long k over few tiles (half the CUs or fewer): slices until about 256 workgroups exist, each
   // walking at least 1024 of k; the slabs they write and the sum kernel reads stay small next to the operands
   // at such tile counts.  Measured at 4096 columns: k = 14336 in 23 us (128 rows) and 32 us (256 rows) against
-  // 35 and 36 us for the smaller tiles of the ring schedule on all of k; k = 4096 in 17.5 and 20 us against 11
-  // and 12 us, so a k below 8192 is never cut.
-  if (p->k < 8192 || 4 * tiles128 > 256) return 1;
+  // 35 and 36 us for the smaller tiles of the ring schedule on all of k, and at 512 rows two slices in 50.5 us
+  // against 51 (58 against 74 us when the weight comes from HBM); k = 4096 in 17.5 and 20 us against 10 and 11 us
+  // (19.5 and 21 against 17 from HBM), so a k below 8192 is never cut.
+  if (p->k < 8192 || 2 * tiles128 > 256) return 1;
   int64_t s = 256 / tiles128;
   if (s > 8) s = 8;
   if (s > p->k / 1024) s = p->k / 1024;
@@ -816,6 +831,7 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
   const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(p, compute_units());
   switch (shape) {
     case 132: launch_mid_shape<Ring128x256>(g, p, epi, packed, st); break;
+    case 133: launch_mid_shape<Ring64Deep>(g, p, epi, packed, st); break;
     case 129: launch_mid_shape<Ring128>(g, p, epi, packed, st); break;
     case 130: launch_mid_shape<Ring64x128>(g, p, epi, packed, st); break;
     case 131: launch_mid_shape<Ring64>(g, p, epi, packed, st); break;
@@ -922,7 +938,7 @@ int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const vo
     case 132: launch_weight_only_shape<Ring128x256>(g, p, st); break;
     case 129: launch_weight_only_shape<Ring128>(g, p, st); break;
     case 130: launch_weight_only_shape<Ring64x128>(g, p, st); break;
-    case 131: launch_weight_only_shape<Ring64>(g, p, st); break;
+    case 131: case 133: launch_weight_only_shape<Ring64>(g, p, st); break;  // (the deeper ring is for operands requested straight into LDS)
     default: launch_weight_only_shape<Mid128>(g, p, st); break;
   }
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<weight only>");

@@ -555,6 +555,37 @@ def gemm_probe(dev, data, reps=10):
   print(json.dumps({'gemm_probe': data, 'reps': reps, 'shapes': rows}))
 
 
+def prefill_probe_cold(dev):
+  """prefill_probe's two int8 columns with a different weight every call: the calls of one HIP-graph replay walk
+  through about 1 GiB of distinct weights (24 or 18 of them), so that every weight comes from HBM, as the
+  weights of successive layers do, next to the same calls against one weight that stays in the memory-side cache."""
+  import torch
+  from aqt_amd import ops
+
+  def t(f, calls):
+    return round(_graph_replay_us(f, calls, reps=3), 1)
+
+  def ints(shape):
+    return (torch.randn(shape, device=dev) * 25).clamp(-127, 127).round().to(torch.int8)
+
+  for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
+    nw = min(24, max(2, (1 << 30) // (n * k)))
+    ws = [ints((1, n, k)) for _ in range(nw)]
+    cs = torch.rand(1, n, device=dev) * 0.01 + 1e-4
+    for m in (128, 256, 512, 1024, 2048):
+      a = ints((1, m, k))
+      rs = torch.rand(1, m, device=dev) * 0.01 + 1e-4
+      kw = dict(row_scale=rs, col_scale=cs, out_dtype=torch.bfloat16, scale_dtype=torch.bfloat16)
+      print(json.dumps({
+          'prefill_probe_cold': 'us per call', 'm': m, 'n': n, 'k': k, 'weights_walked': nw,
+          'aqtx_gemm_i8_from_hbm': t(lambda: [ops.gemm(a, w, **kw) for w in ws], nw),
+          'vendor_int_mm_from_hbm': t(lambda: [torch._int_mm(a[0], w[0].t()) for w in ws], nw),
+          'aqtx_gemm_i8_one_weight': t(lambda: [ops.gemm(a, ws[0], **kw) for _ in range(10)], 10),
+          'vendor_int_mm_one_weight': t(lambda: [torch._int_mm(a[0], ws[0][0].t()) for _ in range(10)], 10)}), flush=True)
+      del a
+    del ws
+
+
 def prefill_probe(dev, shapes=False):
   """Contractions of prefill-sized serving calls (128..4096 rows against the 4096 x 14336 MLP weights and a
   4096 x 4096 one), device time per call replayed from a HIP graph, microseconds: aqtx_gemm_i8 (int8 operands
@@ -572,7 +603,7 @@ def prefill_probe(dev, shapes=False):
   def ints(shape):
     return (torch.randn(shape, device=dev) * 25).clamp(-127, 127).round().to(torch.int8)
 
-  forced = (('tiles128', 128), ('ring128', 129), ('ring64x128', 130), ('ring64', 131), ('ring128x256', 132)) if shapes else ()
+  forced = (('tiles128', 128), ('ring128', 129), ('ring64x128', 130), ('ring64', 131), ('ring128x256', 132), ('ring64deep', 133)) if shapes else ()
   saved = ops.GEMM_TUNING
   for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
     b = ints((1, n, k))
@@ -697,9 +728,10 @@ def main():
                        'distribution (and the vendor int8 GEMM beside them) and exit')
   ap.add_argument('--decode-probe', action='store_true',
                   help='only issue a few serving calls per shape (for rocprofv3 runs) and exit')
-  ap.add_argument('--prefill-probe', choices=['library', 'shapes'], default=None,
+  ap.add_argument('--prefill-probe', choices=['library', 'shapes', 'cold'], default=None,
                   help='only time prefill-sized contractions (128..4096 rows against the MLP weights) next to the vendor '
-                       "GEMMs and exit; 'shapes' adds every tile shape of the kernel for few output tiles")
+                       "GEMMs and exit; 'shapes' adds every tile shape of the kernel for few output tiles, 'cold' walks "
+                       "through 1 GiB of distinct weights instead")
   ap.add_argument('--power-probe', action='store_true',
                   help='only run the forward contraction back to back on all-zero and on quantized-normal operands while '
                        'sampling socket power and shader clock from the SMI tool, and exit')
@@ -725,6 +757,9 @@ def main():
   dev = torch.device('cuda:0')
   if args.gemm_probe is not None:
     gemm_probe(dev, args.gemm_probe)
+    return
+  if args.prefill_probe == 'cold':
+    prefill_probe_cold(dev)
     return
   if args.prefill_probe is not None:
     prefill_probe(dev, shapes=args.prefill_probe == 'shapes')

@@ -405,14 +405,15 @@ def test_gemm_k_slices_choice_is_a_host_decision():
   assert slices(256, 4096, 14336) == 4         # 64 tiles
   assert slices(128, 4096, 8192) == 8
   assert slices(128, 4096, 4096) == 1          # a k below 8192 is never cut: smaller tiles instead
-  assert slices(512, 4096, 14336) == 1         # 128 tiles: 64 x 128 tiles instead
+  assert slices(512, 4096, 14336) == 2         # 128 tiles
+  assert slices(1024, 4096, 14336) == 1        # 256 tiles: one per CU already
   assert slices(1024, 4096, 4096) == 1         # 256 tiles: one per CU already
   assert slices(8192, 14336, 4096) == 1        # the large tiles fill the chip
   assert slices(128, 4096, 14336, k_split=1) == 1
   assert slices(128, 4096, 14336, k_split=3) == 3
   assert slices(128, 4096, 512, k_split=16) == 2   # a slice holds at least 256 of k
   assert slices(128, 4096, 14336, tuning=8) == 1   # the 256 x 256 kernel was asked for
-  assert slices(128, 4096, 14336, tuning=132) == 1  # a tile shape of the ring schedule was asked for
+  assert slices(128, 4096, 14336, tuning=133) == 1  # a tile shape of the ring schedule was asked for
   assert slices(100, 72, 24) == 1                  # not the vector path
   p = _gplan(m=128, n=4096, k=14336, lda=14336, ldb=14336, ldc=4096, k_split=65)
   assert 'k_split must be in 0..64' in _err(lib.aqtx_gemm_i8(ctypes.byref(p), FAKE, FAKE, None, None, FAKE, None, None))
