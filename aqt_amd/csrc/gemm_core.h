@@ -338,6 +338,12 @@ void gemm_kernel(const GemmArgs g_in) {
   };
   __amdgpu_buffer_rsrc_t rsrc_a = rsrc_a_of(m0), rsrc_b = rsrc_b_of(n0);
   constexpr int ksh_b = BFRAG ? 4 : 0;
+  // Unpacked B in fragment order keeps that order in LDS: KiB blk of the B tile's stage is half blk & 1 of 16-row
+  // block blk >> 1, as it lies in memory, so that a wave's request is one contiguous KiB (asking for the pieces
+  // the swizzled row layout wants, 16 bytes from each of 64 places of two KiB, cost 146 against 129 us on
+  // 2048 x 4096 x 14336).
+  constexpr bool kFragLds = BFRAG && !BPACK;
+  static_assert(!kFragLds || MMA::kChunks == 1, "fragment order: 16 bytes of a row per lane and k step");
   int voff_a[LPW], voff_b[LPB], chunk_byte[LPW];
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
@@ -345,12 +351,11 @@ void gemm_kernel(const GemmArgs g_in) {
     const int row = blk * 8 + (lane >> 3);
     chunk_byte[i] = (((lane & 7) ^ (lane >> 3) ^ blk) & 7) * 16;
     voff_a[i] = row * (int)g.lda + chunk_byte[i];
-    if constexpr (!BPACK) {
-      const int cb = chunk_byte[i] >> 4;  // chunk 0..7 of the 128-byte stage: KiB cb >> 2 of the stage's two
-      voff_b[i] = BFRAG ? ((row >> 4) * g.b_steps + (cb >> 2)) * 1024 + ((cb & 3) * 16 + (row & 15)) * 16
-                        : row * (int)g.ldb + chunk_byte[i];
-    }
+    if constexpr (kFragLds) voff_b[i] = ((blk >> 1) * g.b_steps + (blk & 1)) * 1024 + lane * 16;
+    else if constexpr (!BPACK) voff_b[i] = row * (int)g.ldb + chunk_byte[i];
   }
+  // position along k of lane's 16 bytes of B piece i (for the mask on K)
+  auto kpos_b = [&](int i) -> int { return kFragLds ? ((wave * LPW + i) & 1) * 64 + (lane >> 4) * 16 : chunk_byte[i]; };
   // packed B: load q of a wave covers rows 16 (wave LPB + q) .. +15, lane -> row lane >> 2, 16 packed bytes
   // (32 k) at 16 (lane & 3); they become the chunks 2p, 2p + 1 of that row, at positions chunk ^ f(row)
   int pb_st[LPB];
@@ -379,7 +384,7 @@ void gemm_kernel(const GemmArgs g_in) {
       stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, (k0 / 2) << ksh_b, 0);
     } else {
       int vo = voff_b[i];
-      if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;
+      if (KTAIL && k0 + kpos_b(i) >= (int)g.k) vo = 0x7FFFFFF0;
       stgb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo, k0 << ksh_b, 0);
     }
   };
@@ -394,7 +399,7 @@ void gemm_kernel(const GemmArgs g_in) {
     const bool is_b = j & 1;
     const int i = j >> 1;
     int vo = is_b ? voff_b[i] : voff_a[i];
-    if (KTAIL && k0 + chunk_byte[i] >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
+    if (KTAIL && k0 + (is_b ? kpos_b(i) : chunk_byte[i]) >= (int)g.k) vo = 0x7FFFFFF0;  // out of range -> zeros
     uint8_t* at = st + (is_b ? kTileBytes : 0) + wave * LPW * 1024 + i * 1024;  // wave-uniform
     if (!is_b) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)at, 16, vo, k0, 0, 0);
     else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)at, 16, vo, k0 << ksh_b, 0, 0);
@@ -426,6 +431,14 @@ void gemm_kernel(const GemmArgs g_in) {
 #pragma unroll
   for (int cidx = 0; cidx < 8; ++cidx)
     frag_off[cidx] = lr * BK + (((lh * kChunks) ^ lf0 ^ cidx) * 16);
+  // B kept in fragment order: chunk q = 2 ks + lh of row r of a 32-row block lies at
+  // (2 (r >> 4) + (q >> 2)) KiB + 16 (16 (q & 3) + (r & 15)); the 16 rows of a read are consecutive
+  int frag_off_b[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    const int q = 2 * ks + lh;
+    frag_off_b[ks] = (2 * (lr >> 4) + (q >> 2)) * 1024 + (16 * (q & 3) + (lr & 15)) * 16;
+  }
   const int a_base = wm * 128 * BK;                // rows of the A tile this wave needs
   const int b_base = kTileBytes + wn * NI * 32 * BK;   // rows of the B tile
 
@@ -445,7 +458,11 @@ void gemm_kernel(const GemmArgs g_in) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       fa[i] = load_frag(st + a_base, ks, i);
-      if (i < NI) fb[i] = load_frag(st + b_base, ks, i);
+      if constexpr (kFragLds) {
+        if (i < NI) fb[i] = *reinterpret_cast<const v4i*>(st + b_base + i * 32 * BK + frag_off_b[ks]);
+      } else {
+        if (i < NI) fb[i] = load_frag(st + b_base, ks, i);
+      }
     }
   };
   auto mfma_step = [&](const Frag* fa, const Frag* fb) {

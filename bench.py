@@ -558,9 +558,11 @@ def gemm_probe(dev, data, reps=10):
 def prefill_probe_cold(dev):
   """prefill_probe's two int8 columns with a different weight every call: the calls of one HIP-graph replay walk
   through about 1 GiB of distinct weights (24 or 18 of them), so that every weight comes from HBM, as the
-  weights of successive layers do, next to the same calls against one weight that stays in the memory-side cache."""
+  weights of successive layers do, next to the same calls against one weight that stays in the memory-side cache.
+  The `fragments` columns read the weight in the serving kernels' fragment order (aqtx_tile_weight), which is what
+  a frozen weight of the layer API is kept in."""
   import torch
-  from aqt_amd import ops
+  from aqt_amd import ops, _lib as L
 
   def t(f, calls):
     return round(_graph_replay_us(f, calls, reps=3), 1)
@@ -571,6 +573,7 @@ def prefill_probe_cold(dev):
   for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
     nw = min(24, max(2, (1 << 30) // (n * k)))
     ws = [ints((1, n, k)) for _ in range(nw)]
+    frs = [ops.tile_weight(w[0], L.I8) for w in ws]
     cs = torch.rand(1, n, device=dev) * 0.01 + 1e-4
     for m in (128, 256, 512, 1024, 2048):
       a = ints((1, m, k))
@@ -579,11 +582,13 @@ def prefill_probe_cold(dev):
       print(json.dumps({
           'prefill_probe_cold': 'us per call', 'm': m, 'n': n, 'k': k, 'weights_walked': nw,
           'aqtx_gemm_i8_from_hbm': t(lambda: [ops.gemm(a, w, **kw) for w in ws], nw),
+          'aqtx_gemm_i8_fragments_from_hbm': t(lambda: [ops.gemm(a, f, b_layout=L.W_FRAGMENTS, **kw) for f in frs], nw),
           'vendor_int_mm_from_hbm': t(lambda: [torch._int_mm(a[0], w[0].t()) for w in ws], nw),
           'aqtx_gemm_i8_one_weight': t(lambda: [ops.gemm(a, ws[0], **kw) for _ in range(10)], 10),
+          'aqtx_gemm_i8_fragments_one_weight': t(lambda: [ops.gemm(a, frs[0], b_layout=L.W_FRAGMENTS, **kw) for _ in range(10)], 10),
           'vendor_int_mm_one_weight': t(lambda: [torch._int_mm(a[0], ws[0][0].t()) for _ in range(10)], 10)}), flush=True)
       del a
-    del ws
+    del ws, frs
 
 
 def prefill_probe(dev, shapes=False):

@@ -481,12 +481,13 @@ def test_weight_only_gemm_strided_operands(gpu):
 @pytest.mark.parametrize('packed', [False, True])
 @pytest.mark.parametrize('m,n,k,k_split', [(65, 128, 64, 0), (130, 200, 1056, 0), (256, 1024, 4096, 0), (96, 136, 4096, 4),
                                            (512, 72, 2080, 1), (2048, 2048, 512, 0), (300, 4100, 320, 0),
-                                           (2048, 4608, 1024, 0), (2048, 4608, 1056, 0), (2304, 4100, 320, 0)])
+                                           (2048, 4608, 1024, 0), (2048, 4608, 1056, 0), (2304, 4100, 320, 0),
+                                           (130, 200, 1120, 0), (2048, 4608, 1120, 0), (64 + 8, 4096, 4000, 0)])
 def test_fragment_ordered_b_equals_rows(gpu, m, n, k, k_split, packed):
   """aqtx_gemm_i8 with b_layout = AQTX_W_FRAGMENTS (the buffer aqtx_tile_weight writes for the serving kernels)
   against the same call on the rows: integer sums, so bit for bit, outputs and raw accumulators, with and
-  without slices of k, with n and k that end inside a 16-row block / a 64-byte step; the last three shapes
-  have enough output tiles for the 256 x 256 kernel."""
+  without slices of k, with n and k that end inside a 16-row block / in either 64-byte step of a 128-byte
+  stage; shapes with 2048 rows or more have enough output tiles for the 256 x 256 kernel."""
   if packed and k % 32 != 0:
     pytest.skip('packed int4 needs k % 32 == 0')
   torch.manual_seed(5)
