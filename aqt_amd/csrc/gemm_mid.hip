@@ -26,8 +26,10 @@ constexpr int TM = 128, TN = 128;
 // Tile of a workgroup and how its waves share it: WM x WN waves, each (TM / WM) x (TN / WN) of C in 32 x 32
 // matrix-instruction tiles.  A wave fetches TM / waves rows of A and TN / waves rows of B per stage.
 template <int TM_, int TN_, int WM_, int WN_, int OCC_ = 4, bool RING_ = false, int GROUP_ = 1, bool SWIZZLE_ = false,
-          int BUFFERS_ = 0>
+          int BUFFERS_ = 0, bool PAIR_ = false>
 struct MidShape {
+  // direct ring: one barrier for every two stages (see the kernel)
+  static constexpr bool kPair = PAIR_;
   // > 0 (ring, swizzled rows): operands that need no unpacking are requested straight into this many LDS
   // buffers (see the kernel); packed operands keep three buffers and the staging registers
   static constexpr int kBuffers = BUFFERS_;
@@ -52,10 +54,11 @@ using Mid128 = MidShape<128, 128, 4, 2>;  // 8 waves of 32 x 64, 36 KiB a stage,
 using Ring128 = MidShape<128, 128, 4, 2, 2, true, 2, true, 4>;
 using Ring64x128 = MidShape<64, 128, 2, 2, 2, true, 2, true, 4>;
 using Ring64 = MidShape<64, 64, 2, 2, 2, true, 2, true, 4>;
-// eight buffers where a 64 x 64 workgroup has its CU to itself: seven stages (112 KiB) on their way per workgroup.
-// Against weights that come from HBM (a different weight every call) 128 and 256 rows x 4096 x 4096 take 16.8 us
-// instead of 19.8; against a weight that stays in the memory-side cache nothing changes (10-11 us)
-using Ring64Deep = MidShape<64, 64, 2, 2, 2, true, 2, true, 8>;
+// Eight (six) buffers where a workgroup has its CU to itself, and one barrier per two stages: six (four) stages on
+// their way per workgroup.  128 x 4096 x 4096, rows, weight cached / from HBM (a different weight every call):
+// 10.0 / 19.8 us on four buffers, 10.3 / 17.1 on eight, 9.4 / 15.6 with the barrier per pair.
+using Ring64Pair = MidShape<64, 64, 2, 2, 2, true, 2, true, 8, true>;
+using Ring64x128Pair = MidShape<64, 128, 2, 2, 2, true, 2, true, 6, true>;
 using Ring128x256 = MidShape<128, 256, 2, 4, 2, true, 1, true, 3>;  // 8 waves of 64 x 64, 144 KiB of LDS
 
 // MMA, EPI, COL_FIRST as in gemm_kernel.  PACKED: a row of B has half the bytes in memory that it has in LDS:
@@ -397,6 +400,60 @@ void gemm_mid_kernel(const GemmArgs g_in) {
 #pragma unroll
           for (int in = 0; in < IN; ++in) acc[im][in] = MMA::mma(fb[fs][q][in], fa[fs][q][im], acc[im][in]);
     };
+    if constexpr (S::kPair) {
+      // Two stages per barrier.  A 64 x 64 tile gives each of its four waves four matrix instructions a stage, and
+      // the wait, the barrier and the latency of the first fragment reads behind it cost more than those; here a
+      // wave waits and meets the others once per 256 bytes of k.  Stages 2 S and 2 S + 1 are computed group by
+      // group as one stage of 2 NG groups, and their share of the requests is the two stages NB - 2 ahead, into
+      // the two buffers that the previous pair left at its barrier.  Stages past the end of k are requested like
+      // any other: the mask on k makes them zeros, so an odd stage count needs no special case.
+      static_assert(NB % 2 == 0 && NB >= 6, "pairs of buffers, and a pair's requests have a pair to land");
+      constexpr int D2 = NB - 2, NG2 = 2 * NG, NL2 = 2 * NL;
+      auto k_at = [&](const int s) -> int { return s * BK; };
+#pragma unroll
+      for (int d = 0; d < D2; ++d)
+#pragma unroll
+        for (int j = 0; j < NL; ++j) request(ring(d), j, k_at(d));
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D2 - 2) * NL) : "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      load_frags(ring0, 0, 0);
+      constexpr int kBefore2 = (NG2 - 1) * NL2 / NG2;
+      constexpr int kAfterNext2 = (D2 - 4) * NL + kBefore2;  // requests issued after those of the next pair
+      static_assert(kAfterNext2 <= 63, "vmcnt");
+      auto pair_stage = [&](const int s, auto buf_c) {
+        constexpr int B0 = decltype(buf_c)::value, W0 = (B0 + D2) % NB, N0 = (B0 + 2) % NB;
+        const int k_req0 = k_at(s + D2), k_req1 = k_at(s + D2 + 1);
+        auto refill = [&](const int gi) {
+#pragma unroll
+          for (int j = gi * NL2 / NG2; j < (gi + 1) * NL2 / NG2; ++j) {
+            if (j < NL) request(ring(W0), j, k_req0);
+            else request(ring(W0 + 1), j - NL, k_req1);
+          }
+        };
+#pragma unroll
+        for (int gi = 0; gi < NG2 - 1; ++gi) {
+          load_frags(ring(B0 + (gi + 1) / NG), (gi + 1) % NG, (gi + 1) & 1);
+          refill(gi);
+          mfma_group(gi & 1);
+        }
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kAfterNext2) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        mfma_group(1);
+        load_frags(ring(N0), 0, 0);
+        refill(NG2 - 1);
+      };
+      for (int s = 0; s < nstages; s += NB) {
+        pair_stage(s, std::integral_constant<int, 0>{});
+        if (s + 2 < nstages) pair_stage(s + 2, std::integral_constant<int, 2>{});
+        if (s + 4 < nstages) pair_stage(s + 4, std::integral_constant<int, 4>{});
+        if constexpr (NB > 6) {
+          if (s + 6 < nstages) pair_stage(s + 6, std::integral_constant<int, 6>{});
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
 #pragma unroll
     for (int d = 0; d < D; ++d)
 #pragma unroll
@@ -454,6 +511,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
     // requests past the end of k (they repeat stage 0) have to land before the epilogue stages the output in the
     // same buffers
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
   } else {
     // Ring schedule: three LDS buffers, three staging sets.  Stage s computes from buffer s % 3, group by group
     // (a group = kGroup k steps whose fragments are read together, one group ahead of the matrix instructions
@@ -740,10 +798,9 @@ void launch_mid_fp8(const GemmArgs& g, int epi, dim3 grid, hipStream_t st) {
 
 // Tile shape for a plan on `cus` CUs (plan->tuning values).  At most one 128 x 128 tile per CU: the ring
 // schedule (a workgroup alone on its CU has nobody to overlap its waits with: the ring hides them itself), on
-// 64 x 64 tiles up to half a 128 x 128 tile per CU (on eight buffers while every workgroup has a CU to itself, on
-// four beyond, when two of its workgroups fit a CU; measured ahead of 64 x 128
-// at 64-128 tiles: 15.8 against 17.7 us at 512 x 4096 x 4096, 17.5 against 19.0 at 128 x 14336 x 4096), on
-// 128 x 128 tiles beyond.  More than one 128 x 128 tile but at most one 128 x 256 tile per CU: the ring on
+// the smallest tiles that still give every workgroup a CU to itself: 64 x 64 on eight buffers, else 64 x 128 on
+// six, both with one barrier per two stages (512 x 4096 x 4096, weight cached / from HBM: 16.6 / 20.5 us on the
+// latter against 16.6 / 22.4 on 64 x 64 tiles, four buffers, two workgroups a CU), on 128 x 128 tiles beyond.  More than one 128 x 128 tile but at most one 128 x 256 tile per CU: the ring on
 // those.  Beyond: 128 x 128 tiles on the plain schedule, two workgroups a CU.
 inline int mid_shape_for(const aqtx_gemm_plan* p, int cus) {
   const int64_t tiles128 = ((p->m + 127) / 128) * ((p->n + 127) / 128) * p->batch;
@@ -752,7 +809,8 @@ inline int mid_shape_for(const aqtx_gemm_plan* p, int cus) {
   // 4096 x 2048 x 512 measured 15.5 us on it against 13.9 us on the plain schedule)
   if (tiles128 > cus) return (tiles256 <= cus && p->k >= 1024) ? 132 : 128;
   const int64_t tiles64 = ((p->m + 63) / 64) * ((p->n + 63) / 64) * p->batch;
-  return tiles64 <= cus ? 133 : 2 * tiles128 <= cus ? 131 : 129;
+  const int64_t tiles64x128 = ((p->m + 63) / 64) * ((p->n + 127) / 128) * p->batch;
+  return tiles64 <= cus ? 133 : tiles64x128 <= cus ? 134 : 129;
 }
 
 template <class S>
@@ -775,10 +833,11 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 }  // namespace
 
 // Whether the kernel of this file takes the plan (0 = no) and in how many slices of K (1 = none).
-// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 | 132 | 133 = the ring schedule on
-// 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 | 64 x 64 (eight buffers) tiles (never in slices).
+// plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 | 132 | 133 | 134 = the ring schedule
+// on 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 | 64 x 64 (eight buffers, a barrier per two stages) | 64 x 128 (six
+// buffers, the same) tiles (never in slices).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
-  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 133)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
+  if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 134)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
   if (p->lda * (int64_t)TM >= (1ll << 31) || p->ldb * (int64_t)(2 * TN) >= (1ll << 31)) return 0;  // 32-bit offsets within a tile of up to 128 x 256
   const int64_t pad256 = ((p->m + BM - 1) / BM) * ((p->n + BN - 1) / BN);
@@ -848,7 +907,8 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
   const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(p, compute_units());
   switch (shape) {
     case 132: launch_mid_shape<Ring128x256>(g, p, epi, packed, st); break;
-    case 133: launch_mid_shape<Ring64Deep>(g, p, epi, packed, st); break;
+    case 133: launch_mid_shape<Ring64Pair>(g, p, epi, packed, st); break;
+    case 134: launch_mid_shape<Ring64x128Pair>(g, p, epi, packed, st); break;
     case 129: launch_mid_shape<Ring128>(g, p, epi, packed, st); break;
     case 130: launch_mid_shape<Ring64x128>(g, p, epi, packed, st); break;
     case 131: launch_mid_shape<Ring64>(g, p, epi, packed, st); break;
@@ -950,12 +1010,18 @@ int launch_gemm_weight_only_mid(const aqtx_gemm_plan* p, const void* a, const vo
   g.col_first = 0;
   g.b_frag = p->b_layout == AQTX_W_FRAGMENTS;
   g.b_steps = (int)((p->k + 63) / 64);
-  const int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(p, compute_units());
+  // (the widened weight goes through registers, where the deeper rings change nothing: their tile counts choose
+  // the same tiles on the three-buffer ring, 64 x 64 up to half a 128 x 128 tile per CU)
+  int shape = p->tuning >= 128 ? p->tuning : mid_shape_for(p, compute_units());
+  if (p->tuning == 0 && shape == 134) {
+    const int64_t tiles128 = ((p->m + 127) / 128) * ((p->n + 127) / 128) * p->batch;
+    shape = 2 * tiles128 <= compute_units() ? 131 : 129;
+  }
   switch (shape) {
     case 132: launch_weight_only_shape<Ring128x256>(g, p, st); break;
     case 129: launch_weight_only_shape<Ring128>(g, p, st); break;
-    case 130: launch_weight_only_shape<Ring64x128>(g, p, st); break;
-    case 131: case 133: launch_weight_only_shape<Ring64>(g, p, st); break;  // (the deeper ring is for operands requested straight into LDS)
+    case 130: case 134: launch_weight_only_shape<Ring64x128>(g, p, st); break;
+    case 131: case 133: launch_weight_only_shape<Ring64>(g, p, st); break;
     default: launch_weight_only_shape<Mid128>(g, p, st); break;
   }
   AQTX_HIP_CHECK_LAUNCH("gemm_mid_kernel<weight only>");

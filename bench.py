@@ -608,7 +608,7 @@ def prefill_probe(dev, shapes=False):
   def ints(shape):
     return (torch.randn(shape, device=dev) * 25).clamp(-127, 127).round().to(torch.int8)
 
-  forced = (('tiles128', 128), ('ring128', 129), ('ring64x128', 130), ('ring64', 131), ('ring128x256', 132), ('ring64deep', 133)) if shapes else ()
+  forced = (('tiles128', 128), ('ring128', 129), ('ring64x128', 130), ('ring64', 131), ('ring128x256', 132), ('ring64pair', 133), ('ring64x128pair', 134)) if shapes else ()
   saved = ops.GEMM_TUNING
   for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
     b = ints((1, n, k))

@@ -240,9 +240,10 @@ typedef struct aqtx_gemm_plan {
                                  depend on it): 4 | 8 = waves per workgroup of the int8 kernel on
                                  256 x 256 tiles, one workgroup per tile; 16 = 8 waves, one workgroup per CU
                                  walking the tiles; 128 = the int8 kernel on 128 x 128 tiles, two workgroups a
-                                 CU; 129 | 130 | 131 | 132 | 133 = its schedule for launches of at most one
-                                 workgroup per CU, on 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 | 64 x 64 (deeper
-                                 ring) tiles                                                              */
+                                 CU; 129 | 130 | 131 | 132 = its schedule for launches of at most one
+                                 workgroup per CU, on 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 tiles;
+                                 133 | 134 = that schedule on 64 x 64 | 64 x 128 tiles with a deeper ring and
+                                 one barrier per two stages                                               */
   int32_t a_k_order;          /* AQTX_K_*: byte order of a along k; EVEN_ODD8 (aqtx_gemm_i8 with b_dtype
                                  AQTX_I4P only) saves the kernel the re-interleaving of the nibbles   */
   int32_t k_split;            /* aqtx_gemm_i8 only.  Tuning only (int32 partial sums add up exactly in any

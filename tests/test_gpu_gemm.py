@@ -12,8 +12,8 @@ from tests import gpu_util as U
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[4, 8, 16, 128, 129, 130, 131, 132, 133, 0],
-                ids=['waves4', 'waves8', 'persistent', 'tiles128', 'ring128', 'ring64x128', 'ring64', 'ring128x256', 'ring64deep', 'auto'])
+@pytest.fixture(params=[4, 8, 16, 128, 129, 130, 131, 132, 133, 134, 0],
+                ids=['waves4', 'waves8', 'persistent', 'tiles128', 'ring128', 'ring64x128', 'ring64', 'ring128x256', 'ring64pair', 'ring64x128pair', 'auto'])
 def waves(request, monkeypatch):
   """Both workgroup shapes of the 256 x 256 int8 MFMA kernel, the kernel for few output tiles on each of its
   tile shapes and schedules, and the library's own choice (these shapes have few output tiles: the smaller
@@ -197,8 +197,8 @@ def test_k_slices_rejected_where_unsupported(gpu):
     (1, 96, 4096, 2048, 'f32', 'f32'),
 ])
 def test_few_tiles_kernel_shapes_give_the_same_bits(gpu, monkeypatch, batch, m, n, k, out, sdt, b_kind):
-  """plan->tuning 128 (128 x 128 tiles, plain schedule) and 129 .. 133 (the ring schedule on 128 x 128,
-  64 x 128, 64 x 64, 128 x 256 and, with eight buffers, 64 x 64 tiles) against the 256 x 256 kernel on the same operands: integer sums, the same
+  """plan->tuning 128 (128 x 128 tiles, plain schedule) and 129 .. 134 (the ring schedule on 128 x 128,
+  64 x 128, 64 x 64 and 128 x 256 tiles and, with a barrier per two stages, on 64 x 64 and 64 x 128) against the 256 x 256 kernel on the same operands: integer sums, the same
   epilogue arithmetic, so bit for bit, outputs and raw accumulators, for rows and the fragment order of b,
   int8 and packed int4."""
   packed, frag = b_kind.startswith('packed'), b_kind.endswith('fragments')
@@ -223,7 +223,7 @@ def test_few_tiles_kernel_shapes_give_the_same_bits(gpu, monkeypatch, batch, m, 
   assert torch.equal(want_acc.cpu(), ref)
   if frag:
     b_arg, kw['b_layout'] = ops.tile_weight(b_arg[0].contiguous(), b_dtype), L.W_FRAGMENTS
-  for tuning in (128, 129, 130, 131, 132, 133, 0):
+  for tuning in (128, 129, 130, 131, 132, 133, 134, 0):
     monkeypatch.setattr(ops, 'GEMM_TUNING', tuning)
     got, got_acc = ops.gemm(a, b_arg, **kw)
     alone = ops.gemm(a, b_arg, **dict(kw, want_acc=False))  # without the copy of the sums the tile leaves through LDS
@@ -454,7 +454,7 @@ def test_weight_only_gemm_tile_sizes_give_the_same_bits(gpu, m, n, k, w_sdt, lay
   kw = dict(col_scale_dtype=U.TORCH_DT[w_sdt])
   if layout == 'fragments':
     b, kw['b_layout'] = ops.tile_weight(b[0], L.I8), L.W_FRAGMENTS
-  outs = [ops.gemm_weight_only(a, b, cs, tuning=t, **kw) for t in (128, 129, 130, 131, 132, 133, 8, 16, 0)]
+  outs = [ops.gemm_weight_only(a, b, cs, tuning=t, **kw) for t in (128, 129, 130, 131, 132, 133, 134, 8, 16, 0)]
   for o in outs[1:]:
     assert torch.equal(o.view(torch.int16), outs[0].view(torch.int16))
 
