@@ -857,6 +857,16 @@ int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
   // against 51 (58 against 74 us when the weight comes from HBM); k = 4096 in 17.5 and 20 us against 10 and 11 us
   // (19.5 and 21 against 17 from HBM), so a k below 8192 is never cut.
   if (p->k < 8192 || 2 * tiles128 > 256) return 1;
+  // Unpacked operands, k below 10240, and the ring's deep shapes (64 x 64 tiles, or 64 x 128 beyond 256 of those)
+  // would put a workgroup on more than half of 256 CUs: no slices.  Measured at 4096 columns, k = 8192, weight
+  // cached / from HBM: 256 rows 18.7 / 25.2 us against 23.9 / 27.0 in four slices, 512 rows 28.0 / 36.6 against
+  // 35.0 / 37.6 in two; but 128 rows (128 tiles) 17.7 / 24.9 against 19.0 / 20.7 in eight, and at k = 11008 and
+  // beyond the slices are ahead from HBM (256 rows: 30.9 against 33.1 us; k = 14336: 34.9 against 41.5).
+  if (p->k < 10240 && p->b_dtype != AQTX_I4P) {
+    const int64_t tiles64 = ((p->m + 63) / 64) * ((p->n + 63) / 64) * p->batch;
+    const int64_t ring_tiles = tiles64 <= 256 ? tiles64 : ((p->m + 63) / 64) * ((p->n + 127) / 128) * p->batch;
+    if (ring_tiles <= 256 && 2 * ring_tiles > 256) return 1;
+  }
   int64_t s = 256 / tiles128;
   if (s > 8) s = 8;
   if (s > p->k / 1024) s = p->k / 1024;

@@ -404,6 +404,9 @@ def test_gemm_k_slices_choice_is_a_host_decision():
   assert slices(128, 4096, 14336) == 8         # 32 tiles of 128 x 128
   assert slices(256, 4096, 14336) == 4         # 64 tiles
   assert slices(128, 4096, 8192) == 8
+  assert slices(256, 4096, 8192) == 1          # 256 tiles of 64 x 64 and a k below 10240: the deep ring on all of k
+  assert slices(512, 4096, 8192) == 1          # 256 tiles of 64 x 128
+  assert slices(256, 4096, 8192, b_dtype=L.I4P) == 4  # packed operands go through registers: slices as before
   assert slices(128, 4096, 4096) == 1          # a k below 8192 is never cut: smaller tiles instead
   assert slices(512, 4096, 14336) == 2         # 128 tiles
   assert slices(1024, 4096, 14336) == 1        # 256 tiles: one per CU already
