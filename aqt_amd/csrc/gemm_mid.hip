@@ -77,7 +77,7 @@ void gemm_mid_kernel(const GemmArgs g_in) {
   constexpr int IM = S::kIM, IN = S::kIN, RA = S::kRA, RB = S::kRB;
   constexpr bool RING = S::kRing;
   // ring, swizzled rows, nothing to unpack: pieces go from memory straight into LDS
-  constexpr bool DIRECT = RING && SW && !PACKED && !MMA::kWidenA && !CONV && !SLAB && S::kBuffers >= 3;
+  constexpr bool DIRECT = RING && SW && !PACKED && !MMA::kWidenA && !CONV && S::kBuffers >= 3;
   constexpr int NB = DIRECT ? S::kBuffers : 0;
   constexpr int NSETS = DIRECT ? 1 : RING ? 3 : 1, NBUF = RING ? 3 : 2;
   static_assert(!CONV || (TM == 128 && S::kWaves == 8), "the window gather is written for two loads of A per wave");
@@ -835,7 +835,7 @@ void launch_slab_sum(const GemmArgs& g, dim3 grid, hipStream_t st) {
 // Whether the kernel of this file takes the plan (0 = no) and in how many slices of K (1 = none).
 // plan->tuning: 128 = the 128 x 128 tiles on the plain schedule, 129 | 130 | 131 | 132 | 133 | 134 = the ring schedule
 // on 128 x 128 | 64 x 128 | 64 x 64 | 128 x 256 | 64 x 64 (eight buffers, a barrier per two stages) | 64 x 128 (six
-// buffers, the same) tiles (never in slices).
+// buffers, the same) tiles (in slices only where plan->k_split asks for them, and only unpacked operands).
 int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
   if (p->group_offsets != nullptr || (p->tuning != 0 && (p->tuning < 128 || p->tuning > 134)) || !gemm_vector_shape_ok(p)) return 0;  // 4, 8, 16: the large tiles
   if (p->b_dtype == AQTX_I4P && p->scale_order != AQTX_SCALE_ROW_THEN_COL) return 0;
@@ -844,7 +844,7 @@ int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
   const int64_t pad128 = ((p->m + TM - 1) / TM) * ((p->n + TN - 1) / TN);
   const int64_t tiles256 = pad256 * p->batch, tiles128 = pad128 * p->batch;
   const int64_t max_by_k = (p->k + 2 * BK - 1) / (2 * BK);  // a slice holds at least two stages
-  if (p->tuning > 128) return 1;
+  if (p->tuning > 128 && !(p->k_split > 1 && p->b_dtype != AQTX_I4P)) return 1;
   if (p->k_split > 1) return (int)(p->k_split < max_by_k ? p->k_split : max_by_k);
   // the large tiles fill the chip, unless a third of their area or more lies outside C (n or m of 128, say)
   const bool padded = 4 * pad256 * 2 >= 3 * pad128;
@@ -869,6 +869,11 @@ int gemm_mid_k_slices(const aqtx_gemm_plan* p) {
   }
   int64_t s = 256 / tiles128;
   if (s > 8) s = 8;
+  // unpacked operands, up to 64 tiles of 64 x 128: the slices run on those, e.g. four instead of eight on
+  // 128 x 128 (128 x 4096 x 14336, weight cached / from HBM: 20.8 / 26.8 us against 23.3 / 26.7; k = 8192:
+  // 16.3 / 19.2 against 18.9 / 20.8)
+  const int64_t tiles64x128 = ((p->m + 63) / 64) * ((p->n + 127) / 128) * p->batch;
+  if (p->b_dtype != AQTX_I4P && 4 * tiles64x128 <= 256) s = 256 / tiles64x128 < 8 ? 256 / tiles64x128 : 8;
   if (s > p->k / 1024) s = p->k / 1024;
   return s < 1 ? 1 : (int)s;
 }
@@ -900,7 +905,27 @@ int launch_gemm_i8_mid(const aqtx_gemm_plan* p, const void* a, const void* b, co
     g.k_split = (int)((p->k + g.k_chunk - 1) / g.k_chunk);
     g.slabs = reinterpret_cast<int32_t*>(p->k_split_workspace);
     grid.z = (unsigned)g.k_split;
+    auto ring_slices = [&](auto shape_tag) {
+      using SH = decltype(shape_tag);
+      g.tiles_m = (int)((p->m + SH::kTM - 1) / SH::kTM);
+      g.tiles_n = (int)((p->n + SH::kTN - 1) / SH::kTN);
+      const dim3 rgrid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)p->batch, (unsigned)g.k_split);
+      gemm_mid_kernel<MmaI8, 3, false, false, true, false, SH><<<rgrid, SH::kThreads, 0, st>>>(g);
+    };
+    // Unpacked operands: the slices run on the ring, its pieces requested straight into LDS, wherever that puts at
+    // most one workgroup on a CU (the plain schedule alone on its CU spends 1300 cycles on a stage's 512 cycles of
+    // matrix instructions): 64 x 128 tiles while they fit, else 128 x 128.  512 x 4096 x 14336 in two slices, weight
+    // cached / from HBM: 45.4 / 54.3 us against 49.8 / 57.5 on the plain schedule; 256 rows in four: 29.1 / 34.8
+    // against 31.2 / 35.2.
+    const int cus = compute_units();
+    const int64_t wg64x128 = ((p->m + 63) / 64) * ((p->n + 127) / 128) * p->batch * g.k_split;
+    const int64_t wg128 = (int64_t)g.tiles_m * g.tiles_n * p->batch * g.k_split;
     if (packed) gemm_mid_kernel<MmaI8, 3, false, true, true><<<grid, 512, 0, st>>>(g);
+    else if (p->tuning == 129) ring_slices(Ring128{});
+    else if (p->tuning == 133) ring_slices(Ring64Pair{});
+    else if (p->tuning == 134) ring_slices(Ring64x128Pair{});
+    else if (p->tuning == 0 && wg64x128 <= cus) ring_slices(Ring64x128Pair{});
+    else if (p->tuning == 0 && wg128 <= cus) ring_slices(Ring128{});
     else gemm_mid_kernel<MmaI8, 3, false, false, true><<<grid, 512, 0, st>>>(g);
     const dim3 egrid((unsigned)((p->n + 1023) / 1024), (unsigned)p->m, (unsigned)p->batch);
     switch (epi) {

@@ -401,9 +401,10 @@ def test_gemm_k_slices_choice_is_a_host_decision():
     p = _gplan(m=m, n=n, k=k, lda=k, ldb=k, ldc=n, **kw)
     return lib.aqtx_gemm_i8_k_slices(ctypes.byref(p))
 
-  assert slices(128, 4096, 14336) == 8         # 32 tiles of 128 x 128
+  assert slices(128, 4096, 14336) == 4         # 64 tiles of 64 x 128
+  assert slices(128, 4096, 14336, b_dtype=L.I4P) == 8  # packed operands: 32 tiles of 128 x 128
   assert slices(256, 4096, 14336) == 4         # 64 tiles
-  assert slices(128, 4096, 8192) == 8
+  assert slices(128, 4096, 8192) == 4
   assert slices(256, 4096, 8192) == 1          # 256 tiles of 64 x 64 and a k below 10240: the deep ring on all of k
   assert slices(512, 4096, 8192) == 1          # 256 tiles of 64 x 128
   assert slices(256, 4096, 8192, b_dtype=L.I4P) == 4  # packed operands go through registers: slices as before

@@ -231,6 +231,12 @@ def test_few_tiles_kernel_shapes_give_the_same_bits(gpu, monkeypatch, batch, m, 
     assert torch.equal(got_acc, want_acc), tuning
     assert torch.equal(got.view(bits), want.view(bits)), tuning
     assert torch.equal(alone.view(bits), want.view(bits)), tuning
+  # k in slices on request: on the plain schedule and on the ring shapes that take slices (unpacked operands)
+  for tuning in (0, 128, 129, 133, 134):
+    monkeypatch.setattr(ops, 'GEMM_TUNING', tuning)
+    got, got_acc = ops.gemm(a, b_arg, **dict(kw, k_split=3))
+    assert torch.equal(got_acc, want_acc), ('slices', tuning)
+    assert torch.equal(got.view(bits), want.view(bits)), ('slices', tuning)
 
 
 # ---- packed int4 B (two values per byte, unpacked in registers) ---------------------------------
