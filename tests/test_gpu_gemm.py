@@ -239,6 +239,31 @@ def test_few_tiles_kernel_shapes_give_the_same_bits(gpu, monkeypatch, batch, m, 
     assert torch.equal(got.view(bits), want.view(bits)), ('slices', tuning)
 
 
+@pytest.mark.gpu
+def test_library_choice_on_random_shapes_gives_the_bits_of_the_large_tiles(gpu, monkeypatch):
+  """Forty seeded shapes with m up to 700, n up to 4500 and k up to 16500 (ragged in all three, so that the tile
+  shape, the slices of k and the tails the library picks vary), b as rows and in fragment order: outputs and raw
+  sums equal those of the 256 x 256 kernel bit for bit."""
+  rng = np.random.default_rng(20250607)
+  for case in range(40):
+    m = int(rng.integers(65, 700))
+    n = int(rng.choice([rng.integers(16, 600), rng.integers(600, 4500)]))
+    k = int(rng.choice([rng.integers(1, 40) * 16, rng.integers(40, 520) * 32]))
+    torch.manual_seed(case)
+    a = torch.randint(-127, 128, (1, m, k), dtype=torch.int8, device=gpu)
+    b = torch.randint(-127, 128, (1, n, k), dtype=torch.int8, device=gpu)
+    kw = dict(row_scale=torch.rand(1, m, device=gpu) + 0.5, col_scale=torch.rand(1, n, device=gpu) * 0.01 + 1e-4,
+              out_dtype=torch.bfloat16, want_acc=True)
+    monkeypatch.setattr(ops, 'GEMM_TUNING', 8)
+    want, want_acc = ops.gemm(a, b, **kw)
+    monkeypatch.setattr(ops, 'GEMM_TUNING', 0)
+    got, got_acc = ops.gemm(a, b, **kw)
+    assert torch.equal(got_acc, want_acc) and torch.equal(got.view(torch.int16), want.view(torch.int16)), (case, m, n, k, 'rows')
+    frags = ops.tile_weight(b[0].contiguous(), L.I8)
+    got, got_acc = ops.gemm(a, frags, b_layout=L.W_FRAGMENTS, **kw)
+    assert torch.equal(got_acc, want_acc) and torch.equal(got.view(torch.int16), want.view(torch.int16)), (case, m, n, k, 'fragments')
+
+
 # ---- packed int4 B (two values per byte, unpacked in registers) ---------------------------------
 def _even_odd8(a):
   g = a.reshape(a.shape[:-1] + (a.shape[-1] // 8, 8))
